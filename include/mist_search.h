@@ -1,0 +1,183 @@
+/*
+ * C ABI of the MI355X configuration-search library (libmist_search.so).
+ *
+ * Plain pointers and sizes only.  Every pointer named `d_*` is DEVICE memory owned by the
+ * caller (the python host side allocates it with torch); `problem` and `tables` are small HOST
+ * structs that are copied into the kernel arguments.  Nothing here allocates or frees device
+ * memory.  All work is enqueued on the `stream` argument (a hipStream_t passed as
+ * void*) and is asynchronous with respect to the host.  Return value: 0 on success, a
+ * negative MIST_E_* code otherwise; mist_last_error() gives the message of the calling
+ * thread's last failure.
+ *
+ * The reference implements this path in python/numpy/numba; the reference interface each
+ * entry point replaces is cited per function (paths relative to the reference repository).
+ */
+#ifndef MIST_SEARCH_H
+#define MIST_SEARCH_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MIST_MAX_PAR 64     /* parallelism rows (b, dp, tp, ZeRO flags) per group */
+#define MIST_MAX_RATIOS 32  /* values per offload-ratio list */
+#define MIST_MAX_PAIRS (MIST_MAX_RATIOS * MIST_MAX_RATIOS)
+#define MIST_PAR_FIELDS 20
+#define MIST_ROW_TERMS 34   /* doubles per candidate row produced by mist_row_terms */
+#define MIST_LC_TILE 256    /* (layers, ckpt) pairs per workgroup of the reduce kernel */
+#define MIST_P_TILE 8       /* pre-saved micro-batch values per thread of the reduce kernel */
+#define MIST_MAX_MESH 16    /* device-mesh candidates of the inter-stage DP */
+
+#define MIST_E_INVALID (-1) /* argument / shape check failed, nothing was launched */
+#define MIST_E_HIP (-2)     /* a HIP runtime call failed */
+
+/* Indices into MistGroupDesc.par[i][...] (all float64). */
+enum {
+  MIST_PAR_B = 0, MIST_PAR_DP, MIST_PAR_TP, MIST_PAR_WRE, MIST_PAR_GRE, MIST_PAR_ORE,
+  MIST_PAR_W,        /* full weights of one block layer at this tp, MB */
+  MIST_PAR_G,        /* full grads, MB */
+  MIST_PAR_O,        /* full optimizer states, MB */
+  MIST_PAR_RAW_CK,   /* saved activations of a checkpointed layer, MB */
+  MIST_PAR_RAW_NOCK, /* saved activations without checkpointing, MB */
+  MIST_PAR_FWD_PEAK, /* forward peak without checkpointing, MB */
+  MIST_PAR_BWD_PEAK, /* backward peak, MB */
+  MIST_PAR_OUT,      /* layer output, MB */
+  MIST_PAR_GCB,      /* attention score buffer when flash attention is off, MB (else 0) */
+  MIST_PAR_EXEC_FWD, MIST_PAR_EXEC_BWD, MIST_PAR_EXTRA_FWD, MIST_PAR_EXTRA_BWD, /* seconds */
+  MIST_PAR_RESERVED
+};
+
+/* Indices into one candidate row of the row-term workspace (all float64). */
+enum {
+  MIST_T_S_LAYER_CK = 0, MIST_T_S_LAYER_NOCK, MIST_T_S_FIRST_CK, MIST_T_S_FIRST_NOCK,
+  MIST_T_S_LAST_CK, MIST_T_S_LAST_NOCK,
+  MIST_T_D_LAYER_CK, MIST_T_D_LAYER_NOCK, MIST_T_D_FIRST_CK, MIST_T_D_FIRST_NOCK,
+  MIST_T_D_LAST_CK, MIST_T_D_LAST_NOCK,
+  MIST_T_FWD_STATES0, /* 2*(Wbuf+Gbuf) + O // ore_size */
+  MIST_T_BWD_STATES0, /* 2*(Wbuf+Gbuf) */
+  MIST_T_PWG,         /* partial weights + partial grads */
+  MIST_T_PO,          /* partial optimizer states */
+  MIST_T_PWGO,        /* (pW + pG) + pO */
+  MIST_T_S_CK, MIST_T_S_NOCK, MIST_T_D_CK, MIST_T_D_NOCK,
+  MIST_T_MF_BASE,     /* memory_factor_for_pp + 0.01 */
+  MIST_T_MF_PP,       /* memory_factor + 0.025 */
+  MIST_T_MF,          /* memory_factor */
+  MIST_T_FWD_PEAK, MIST_T_BWD_PEAK, MIST_T_OUT, MIST_T_GCB,
+  MIST_T_NAG_CK, MIST_T_NAG_NOCK, MIST_T_NRS_CK, MIST_T_NRS_NOCK,
+  MIST_T_OPB,         /* max(post_bwd - extra_pre_bwd_not_last_ck, 0) */
+  MIST_T_RD           /* raw_saved_nock - saved_nock */
+};
+
+/* Problem-wide constants (one tuner call = one tp candidate over all (G, mesh) groups). */
+typedef struct MistProblem {
+  double gpu_gpu[32];      /* hardware.gpu_gpu_comm_params: [inter 1,2,4,8][intra 1,2,4,8](k GB/s, b s) */
+  double cpu_gpu[2];       /* hardware.cpu_gpu_comm_params (k, b): CPU -> GPU */
+  double gpu_cpu[2];       /* hardware.gpu_cpu_comm_params (k, b): GPU -> CPU */
+  double interf_factor[11][4]; /* per mask (4-way, 4x 3-way, 6x 2-way): factor per resource, 1 outside the mask */
+  double mem_cap_mb;       /* hardware.memory_capacity(*0.88) * GB / MB */
+  double frag_factor;      /* fragmentation term of the memory factor */
+  int32_t num_layers;      /* L: layer candidates 1..L, ckpt candidates 0..L */
+  int32_t p_dim;           /* P+1: extent of the pre-saved-micro-batch axis of the tables */
+  int32_t sample_size;     /* S: extent of the trailing sample axis of the tables */
+  int32_t num_grad_accum;  /* extent of the g axis */
+  int32_t num_mesh;        /* extent of the q axis */
+  int32_t adv_first_block; /* enable_advanced_opt_in_first_block */
+  int32_t reserved[2];
+} MistProblem;
+
+/* One (gradient-accumulation steps, device mesh) group = one call of the reference's
+ * batched_tune_best_latency_for_stage (mist/analyzer/batched_module_analyzer.py:581-684).
+ * Candidate rows are never materialised: row r decodes as
+ *   par = r / n_off,  off = r % n_off,  pair = off / (n_oo*n_ao),
+ *   oo  = (off / n_ao) % n_oo,  ao = off % n_ao,  (wo, go) = (pair_wo[pair], pair_go[pair]),
+ * i.e. itertools.product(wo, go, oo, ao) minus (wo > 0 and go == 0), parallelism-major
+ * (batched_module_analyzer.py:490-534). */
+typedef struct MistGroupDesc {
+  int32_t g_index, q_index;     /* position in the (g, q) axes of the output tables */
+  int32_t num_nodes, num_gpus_per_node; /* stage mesh (n, m) */
+  int32_t grad_accum;           /* G */
+  int32_t num_p;                /* pre-saved micro-batch candidates 0..num_p-1 */
+  int32_t n_par, n_pair, n_oo, n_ao, n_off;
+  int32_t pp_wre, pp_gre;       /* ZeRO flags of the pre/post layer strategy */
+  int32_t rows_per_chunk, n_chunks, n_lc_tiles, n_p_tiles; /* decomposition of the reduce kernel */
+  int32_t reserved0;
+  int64_t n_rows;               /* n_par * n_off */
+  int64_t row_offset;           /* first row of this group in the row-term workspace */
+  double par[MIST_MAX_PAR][MIST_PAR_FIELDS];
+  double wo[MIST_MAX_RATIOS], go[MIST_MAX_RATIOS], oo[MIST_MAX_RATIOS], ao[MIST_MAX_RATIOS];
+  uint8_t pair_wo[MIST_MAX_PAIRS], pair_go[MIST_MAX_PAIRS];
+  /* pre / post layer scalars (batched_module_analyzer.py:777-1138) */
+  double pre_full_w, pre_full_g, post_full_w, post_full_g;      /* MB */
+  double pre_states, pre_saved, pre_states_and_saved;            /* MB */
+  double post_states, post_fwd_peak, post_bwd_peak, post_output; /* MB */
+  double pre_fwd, pre_bwd, post_fwd, post_bwd;                   /* s */
+  double pre_ag, pre_rs, post_ag, post_rs;                       /* s, 0 when the pre/post dp size is 1 */
+} MistGroupDesc;
+
+/* Output tables of one tuner call, float64 costs and int32 row indices, laid out like the
+ * reference's IntraStageTuner tables (mist/analyzer/intra_tuning.py:127-166):
+ *   base, with_pre : [g][q][p_dim][L][L+1][S]
+ *   with_post      : [g][q][L][L+1][S]
+ *   no_pp          : [g][q][L+1][S]
+ * The caller pre-fills costs with +inf and indices with -1; only the cells the reference
+ * writes are written. */
+typedef struct MistOutTables {
+  double *stable[4], *delta[4];
+  int32_t *index[4];
+} MistOutTables;
+
+/* Library identification and error text. */
+const char *mist_version(void);
+const char *mist_last_error(void);
+int mist_sizeof_problem(void);
+int mist_sizeof_group(void);
+
+/* Row-invariant terms of every candidate row: decodes the row index, evaluates the alpha-beta
+ * communication terms, the 36 interference evaluations and the memory pieces that do not
+ * depend on (layers, ckpt, pre-saved micro-batches).
+ * Replaces batched_stage_analyze lines 1144-2162 of mist/analyzer/batched_module_analyzer.py
+ * (with predict_gpu_gpu_comm_latency / predict_cpu_gpu_comm_latency /
+ * interference_estimate_for_one_group of mist/tools/optimize.py:201-303,459-470,1012-1122).
+ * d_block_prefix[n_groups+1]: first workgroup of each group, 256 rows per workgroup.
+ * d_row_terms: [total_rows][MIST_ROW_TERMS] float64. */
+int mist_row_terms(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,
+                   const int32_t *d_block_prefix, int n_blocks, double *d_row_terms,
+                   void *stream);
+
+/* Per (group, row chunk, (l, c) tile, p tile): evaluates latency and memory per cell, applies
+ * the memory mask and keeps the running lexicographic (cost, row) minimum per bucket.
+ * Replaces the two hot loops of batched_stage_analyze (batched_module_analyzer.py:2218-3106)
+ * and compute_indices (mist/utils/pareto.py:124-144) for one ratio r = alpha/(1-alpha).
+ * d_block_prefix[n_groups+1]: first workgroup of each group; a group owns
+ * n_lc_tiles*n_p_tiles*n_chunks workgroups ordered (lc_tile, p_tile, chunk), chunk fastest.
+ * d_partial_cost / d_partial_index: [n_blocks][2*MIST_P_TILE+2][MIST_LC_TILE]. */
+int mist_eval_reduce(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,
+                     const int32_t *d_block_prefix, int n_blocks, const double *d_row_terms,
+                     double ratio, double *d_partial_cost, int32_t *d_partial_index,
+                     void *stream);
+
+/* Combines the per-chunk partial minima in chunk order (strict <, so the first row wins ties),
+ * recomputes stable / delta of the winning row and scatters into the output tables at sample
+ * position `sample_index`, reproducing which cells the reference leaves unwritten
+ * (batched_module_analyzer.py:2819-2834, 2915-2923, 3021-3033, 3103-3106). */
+int mist_finalize(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,
+                  const int32_t *d_block_prefix, const double *d_row_terms,
+                  const double *d_partial_cost, const int32_t *d_partial_index,
+                  int sample_index, const MistOutTables *tables, void *stream);
+
+/* mist_row_terms (when `compute_terms` != 0) + mist_eval_reduce + mist_finalize for one ratio:
+ * the device side of IntraStageTuner.tune (mist/analyzer/intra_tuning.py:169-282) for one tp
+ * candidate and one sample. */
+int mist_intra_stage_eval(const MistProblem *problem, const MistGroupDesc *d_groups,
+                          int n_groups, const int32_t *d_terms_block_prefix, int n_terms_blocks,
+                          const int32_t *d_reduce_block_prefix, int n_reduce_blocks,
+                          double *d_row_terms, double *d_partial_cost, int32_t *d_partial_index,
+                          double ratio, int sample_index, int compute_terms,
+                          const MistOutTables *tables, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MIST_SEARCH_H */

@@ -1,0 +1,160 @@
+"""ctypes binding of libmist_search.so (declarations in include/mist_search.h).
+
+There is no CPU fallback: if the shared library is missing or a call fails, this raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+import numpy as np
+
+LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libmist_search.so")
+
+MAX_PAR = 64
+MAX_RATIOS = 32
+MAX_PAIRS = MAX_RATIOS * MAX_RATIOS
+PAR_FIELDS = 20
+ROW_TERMS = 34
+LC_TILE = 256
+P_TILE = 8
+SLOTS = 2 * P_TILE + 2
+STAGE_ROWS = 32
+TERMS_BLOCK = 256
+MAX_MESH = 16
+
+PAR_NAMES = (
+    "b", "dp", "tp", "wre", "gre", "ore", "W", "G", "O", "raw_ck", "raw_nock", "fwd_peak",
+    "bwd_peak", "out", "gcb", "exec_fwd", "exec_bwd", "extra_fwd", "extra_bwd", "reserved",
+)
+PAR = {name: i for i, name in enumerate(PAR_NAMES)}
+TERM_NAMES = (
+    "s_layer_ck", "s_layer_nock", "s_first_ck", "s_first_nock", "s_last_ck", "s_last_nock",
+    "d_layer_ck", "d_layer_nock", "d_first_ck", "d_first_nock", "d_last_ck", "d_last_nock",
+    "fwd_states0", "bwd_states0", "pWG", "pO", "pWGO", "S_ck", "S_nock", "D_ck", "D_nock",
+    "mf_base", "mf_pp", "mf", "fwd_peak", "bwd_peak", "out", "gcb",
+    "nAG_ck", "nAG_nock", "nRS_ck", "nRS_nock", "opb", "RD",
+)
+TERM = {name: i for i, name in enumerate(TERM_NAMES)}
+assert len(TERM_NAMES) == ROW_TERMS and len(PAR_NAMES) == PAR_FIELDS
+
+PROBLEM_DTYPE = np.dtype(
+    [
+        ("gpu_gpu", "<f8", (32,)),
+        ("cpu_gpu", "<f8", (2,)),
+        ("gpu_cpu", "<f8", (2,)),
+        ("interf_factor", "<f8", (11, 4)),
+        ("mem_cap_mb", "<f8"),
+        ("frag_factor", "<f8"),
+        ("num_layers", "<i4"),
+        ("p_dim", "<i4"),
+        ("sample_size", "<i4"),
+        ("num_grad_accum", "<i4"),
+        ("num_mesh", "<i4"),
+        ("adv_first_block", "<i4"),
+        ("reserved", "<i4", (2,)),
+    ],
+    align=True,
+)
+
+GROUP_DTYPE = np.dtype(
+    [
+        ("g_index", "<i4"), ("q_index", "<i4"),
+        ("num_nodes", "<i4"), ("num_gpus_per_node", "<i4"),
+        ("grad_accum", "<i4"), ("num_p", "<i4"),
+        ("n_par", "<i4"), ("n_pair", "<i4"), ("n_oo", "<i4"), ("n_ao", "<i4"), ("n_off", "<i4"),
+        ("pp_wre", "<i4"), ("pp_gre", "<i4"),
+        ("rows_per_chunk", "<i4"), ("n_chunks", "<i4"), ("n_lc_tiles", "<i4"),
+        ("n_p_tiles", "<i4"), ("reserved0", "<i4"),
+        ("n_rows", "<i8"), ("row_offset", "<i8"),
+        ("par", "<f8", (MAX_PAR, PAR_FIELDS)),
+        ("wo", "<f8", (MAX_RATIOS,)), ("go", "<f8", (MAX_RATIOS,)),
+        ("oo", "<f8", (MAX_RATIOS,)), ("ao", "<f8", (MAX_RATIOS,)),
+        ("pair_wo", "u1", (MAX_PAIRS,)), ("pair_go", "u1", (MAX_PAIRS,)),
+        ("pre_full_w", "<f8"), ("pre_full_g", "<f8"), ("post_full_w", "<f8"), ("post_full_g", "<f8"),
+        ("pre_states", "<f8"), ("pre_saved", "<f8"), ("pre_states_and_saved", "<f8"),
+        ("post_states", "<f8"), ("post_fwd_peak", "<f8"), ("post_bwd_peak", "<f8"),
+        ("post_output", "<f8"),
+        ("pre_fwd", "<f8"), ("pre_bwd", "<f8"), ("post_fwd", "<f8"), ("post_bwd", "<f8"),
+        ("pre_ag", "<f8"), ("pre_rs", "<f8"), ("post_ag", "<f8"), ("post_rs", "<f8"),
+    ],
+    align=True,
+)
+
+
+class OutTables(ctypes.Structure):
+    _fields_ = [
+        ("stable", ctypes.c_void_p * 4),
+        ("delta", ctypes.c_void_p * 4),
+        ("index", ctypes.c_void_p * 4),
+    ]
+
+
+class MistLibraryError(RuntimeError):
+    pass
+
+
+_LIB = None
+
+_VP = ctypes.c_void_p
+_SIGNATURES = {
+    "mist_version": (ctypes.c_char_p, []),
+    "mist_last_error": (ctypes.c_char_p, []),
+    "mist_sizeof_problem": (ctypes.c_int, []),
+    "mist_sizeof_group": (ctypes.c_int, []),
+    "mist_row_terms": (ctypes.c_int, [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, _VP]),
+    "mist_eval_reduce": (
+        ctypes.c_int,
+        [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, ctypes.c_double, _VP, _VP, _VP],
+    ),
+    "mist_finalize": (
+        ctypes.c_int,
+        [_VP, _VP, ctypes.c_int, _VP, _VP, _VP, _VP, ctypes.c_int, ctypes.POINTER(OutTables), _VP],
+    ),
+    "mist_intra_stage_eval": (
+        ctypes.c_int,
+        [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, _VP, _VP,
+         ctypes.c_double, ctypes.c_int, ctypes.c_int, ctypes.POINTER(OutTables), _VP],
+    ),
+}
+
+
+def exported_symbols():
+    """Names every entry point declared in include/mist_search.h and include/mist_dp.h."""
+    return tuple(_SIGNATURES) + tuple(_DP_SIGNATURES)
+
+
+_DP_SIGNATURES = {}
+
+
+def load():
+    """Loads the shared library once; raises if it has not been built."""
+    global _LIB
+    if _LIB is not None:
+        return _LIB
+    if not os.path.exists(LIB_PATH):
+        raise MistLibraryError(
+            f"{LIB_PATH} is missing: build it with `python -m mist_amd.build` "
+            "(there is no CPU fallback for the search kernels)"
+        )
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (restype, argtypes) in {**_SIGNATURES, **_DP_SIGNATURES}.items():
+        fn = getattr(lib, name)
+        fn.restype = restype
+        fn.argtypes = argtypes
+    if lib.mist_sizeof_problem() != PROBLEM_DTYPE.itemsize:
+        raise MistLibraryError(
+            f"MistProblem layout mismatch: C {lib.mist_sizeof_problem()} vs numpy {PROBLEM_DTYPE.itemsize}"
+        )
+    if lib.mist_sizeof_group() != GROUP_DTYPE.itemsize:
+        raise MistLibraryError(
+            f"MistGroupDesc layout mismatch: C {lib.mist_sizeof_group()} vs numpy {GROUP_DTYPE.itemsize}"
+        )
+    _LIB = lib
+    return lib
+
+
+def check(rc: int, what: str):
+    if rc != 0:
+        msg = load().mist_last_error().decode(errors="replace")
+        raise MistLibraryError(f"{what} failed with code {rc}: {msg}")

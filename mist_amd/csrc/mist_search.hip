@@ -1,0 +1,708 @@
+// Intra-stage configuration search on MI355X (gfx950): row terms, fused evaluate+mask+argmin,
+// finalize.  Everything is float64 VALU work with float32 rounding points where the reference
+// has them; there is no dense contraction here, so no MFMA.
+//
+// Bit-exactness rules for this file (results must equal the numpy formulation operation for
+// operation): compile with -ffp-contract=off, keep the operand order of every sum exactly as
+// written, use true divisions, and never reassociate.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "mist_search.h"
+
+namespace {
+
+thread_local char g_last_error[512] = "";
+
+int fail(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+#define MIST_HIP_CHECK(expr)                                                              \
+  do {                                                                                    \
+    hipError_t err__ = (expr);                                                            \
+    if (err__ != hipSuccess)                                                              \
+      return fail(MIST_E_HIP, "%s failed: %s", #expr, hipGetErrorString(err__));          \
+  } while (0)
+
+constexpr int kTermsBlock = 256;  // rows per workgroup of the row-term kernel
+constexpr int kStageRows = 32;    // rows staged through LDS per step of the reduce kernel
+constexpr int kSlots = 2 * MIST_P_TILE + 2;  // per-thread running minima: base, with_pre, post, no_pp
+
+// ------------------------------------------------------------------------------------------
+// Communication models (mist/tools/optimize.py:257-303, 459-470).
+// ------------------------------------------------------------------------------------------
+__device__ __forceinline__ int size_index(double s) {
+  return s == 1.0 ? 0 : (s == 2.0 ? 1 : (s == 4.0 ? 2 : 3));
+}
+
+__device__ __forceinline__ double gpu_gpu_latency(const double *gg, double mbytes, double inter,
+                                                  double intra, double factor) {
+  const double gbytes = mbytes / 1024.0;
+  const double ngpu = intra * inter;
+  double lat = 0.0;
+  if (!(gbytes < 1e-5 || ngpu == 1.0)) {
+    const double *cell = gg + (size_index(inter) * 4 + size_index(intra)) * 2;
+    lat = gbytes / cell[0] * (ngpu - 1.0) / ngpu + cell[1];
+  }
+  return lat * factor;
+}
+
+__device__ __forceinline__ double host_link_latency(const double *kb, double mbytes) {
+  const double gbytes = mbytes / 1024.0;
+  const double lat = gbytes / kb[0] + kb[1];
+  return gbytes == 0.0 ? 0.0 : lat;
+}
+
+// numpy's float64 floor_divide (npy_divmod), for a >= 0 and b > 0 as well as the general case.
+__device__ __forceinline__ double np_floor_divide(double a, double b) {
+  if (b == 0.0) return a / b;
+  double mod = fmod(a, b);
+  double div = (a - mod) / b;
+  if (mod != 0.0) {
+    if ((b < 0.0) != (mod < 0.0)) div -= 1.0;
+  }
+  double floordiv;
+  if (div != 0.0) {
+    floordiv = floor(div);
+    if (div - floordiv > 0.5) floordiv += 1.0;
+  } else {
+    floordiv = copysign(0.0, a / b);
+  }
+  return floordiv;
+}
+
+// ------------------------------------------------------------------------------------------
+// Four-resource interference model (mist/tools/optimize.py:1012-1122).  X = [C, G2G, C2G, G2C].
+// Masks in evaluation order: 4-way, four 3-way, six 2-way; bit j set = resource j in the mask.
+// ------------------------------------------------------------------------------------------
+__constant__ unsigned char kMaskBits[11] = {
+    0xF,
+    0x7, 0xB, 0xD, 0xE,
+    0x3, 0x5, 0x9, 0x6, 0xA, 0xC,
+};
+
+struct Interference {
+  const double (*factor)[4];
+
+  // Arguments in the order of the reference's get_layer_critical_latency
+  // (batched_module_analyzer.py:1413-1422): exec, gpu<->gpu, gpu->cpu, cpu->gpu.
+  __device__ __noinline__ double operator()(double exec, double g2g, double g2c, double c2g) const {
+    double x0 = exec, x1 = g2g, x2 = c2g, x3 = g2c;
+    double out = 0.0;
+#pragma unroll 1
+    for (int m = 0; m < 11; ++m) {
+      // "not isclose(x, 0)" with numpy's default tolerances: |x| > 1e-8 (NaN counts as non-zero).
+      const unsigned nz = (!(fabs(x0) <= 1e-8) ? 1u : 0u) | (!(fabs(x1) <= 1e-8) ? 2u : 0u) |
+                          (!(fabs(x2) <= 1e-8) ? 4u : 0u) | (!(fabs(x3) <= 1e-8) ? 8u : 0u);
+      const unsigned mask = kMaskBits[m];
+      if (nz != mask) continue;
+      const double f0 = factor[m][0], f1 = factor[m][1], f2 = factor[m][2], f3 = factor[m][3];
+      const double s0 = x0 * f0, s1 = x1 * f1, s2 = x2 * f2, s3 = x3 * f3;
+      double ov = INFINITY;
+      if (mask & 1u) ov = fmin(ov, s0);
+      if (mask & 2u) ov = fmin(ov, s1);
+      if (mask & 4u) ov = fmin(ov, s2);
+      if (mask & 8u) ov = fmin(ov, s3);
+      if (mask & 1u) x0 = (s0 - ov) / f0 * 1.0;
+      if (mask & 2u) x1 = (s1 - ov) / f1 * 1.0;
+      if (mask & 4u) x2 = (s2 - ov) / f2 * 1.0;
+      if (mask & 8u) x3 = (s3 - ov) / f3 * 1.0;
+      out = out + ov;
+    }
+    return out + (((x0 + x1) + x2) + x3);
+  }
+};
+
+struct Family {
+  double layer, first, last, extra_pre, extra_post;
+};
+
+__device__ __forceinline__ const MistGroupDesc *find_group(const MistGroupDesc *groups,
+                                                           const int32_t *prefix, int n_groups,
+                                                           int block, int *local) {
+  int lo = 0, hi = n_groups;  // prefix[lo] <= block < prefix[hi]
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (prefix[mid] <= block) lo = mid; else hi = mid;
+  }
+  *local = block - prefix[lo];
+  return groups + lo;
+}
+
+// ------------------------------------------------------------------------------------------
+// Kernel 1: row-invariant terms.  One thread per candidate row.
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kTermsBlock) void row_terms_kernel(
+    const MistProblem prob, const MistGroupDesc *__restrict__ groups, int n_groups,
+    const int32_t *__restrict__ block_prefix, double *__restrict__ row_terms) {
+  int local_block;
+  const MistGroupDesc *g = find_group(groups, block_prefix, n_groups, blockIdx.x, &local_block);
+  const int64_t row = (int64_t)local_block * kTermsBlock + threadIdx.x;
+  if (row >= g->n_rows) return;
+
+  // ---- index decomposition (batched_module_analyzer.py:490-534) ----
+  const int par_i = (int)(row / g->n_off);
+  const int off = (int)(row % g->n_off);
+  const int n_tail = g->n_oo * g->n_ao;
+  const int pair = off / n_tail;
+  const int oo_i = (off / g->n_ao) % g->n_oo;
+  const int ao_i = off % g->n_ao;
+  const double wo = g->wo[g->pair_wo[pair]];
+  const double go = g->go[g->pair_go[pair]];
+  const double oo = g->oo[oo_i];
+  const double ao = g->ao[ao_i];
+
+  const double *par = g->par[par_i];
+  const double b = par[MIST_PAR_B], dp = par[MIST_PAR_DP], tp = par[MIST_PAR_TP];
+  const double wre = par[MIST_PAR_WRE], gre = par[MIST_PAR_GRE], ore = par[MIST_PAR_ORE];
+  const double W = par[MIST_PAR_W], Gr = par[MIST_PAR_G], O = par[MIST_PAR_O];
+  const double raw_ck = par[MIST_PAR_RAW_CK], raw_nock = par[MIST_PAR_RAW_NOCK];
+  const double exec_fwd = par[MIST_PAR_EXEC_FWD], exec_bwd_nock = par[MIST_PAR_EXEC_BWD];
+  const double extra_fwd = par[MIST_PAR_EXTRA_FWD], extra_bwd = par[MIST_PAR_EXTRA_BWD];
+  const double wre_size = wre == 1.0 ? dp : 1.0;
+  const double gre_size = gre == 1.0 ? dp : 1.0;
+  const double ore_size = ore == 1.0 ? dp : 1.0;
+
+  // ---- memory factor (:1181-1199) ----
+  double mf = 1.0;
+  mf += prob.frag_factor;
+  mf += wo > 0.0 ? 0.025 : 0.0;
+  mf += go > 0.0 ? 0.025 : 0.0;
+  mf += oo > 0.0 ? 0.03 : 0.0;
+  mf += ao > 0.0 ? 0.04 : 0.0;
+  mf += wre != 0.0 ? 0.025 : 0.0;
+  mf += gre != 0.0 ? 0.025 : 0.0;
+  mf += tp > 1.0 ? 0.04 : 0.0;
+  mf += b >= 4.0 ? 0.01 : 0.0;
+  const double mf_pp = mf + 0.025;
+
+  // ---- memory pieces (:1216-1272, 2091-2162) ----
+  const double pW = W / wre_size * (1.0 - wo);
+  const double pG = Gr / gre_size * (1.0 - go);
+  const double pO = O / ore_size * (1.0 - oo);
+  const double S_ck = raw_ck * (1.0 - ao), D_ck = raw_ck * ao;
+  const double S_nock = raw_nock * (1.0 - ao), D_nock = raw_nock * ao;
+  const bool wbuf_on = wre_size > 1.0 || g->pp_wre == 1 || wo > 0.0;
+  const bool gbuf_on = gre_size > 1.0 || g->pp_gre == 1 || go > 0.0;
+  const double Wbuf = wbuf_on ? fmax(fmax(g->pre_full_w, g->post_full_w), W) : 0.0;
+  const double Gbuf = gbuf_on ? fmax(fmax(g->pre_full_g, g->post_full_g), Gr) : 0.0;
+  const double two_buf = 2.0 * (Wbuf + Gbuf);
+
+  // ---- swap and collective latencies (:1362-1408) ----
+  const double so_W = host_link_latency(prob.gpu_cpu, W / wre_size * wo);
+  const double si_W = host_link_latency(prob.cpu_gpu, W / wre_size * wo);
+  const double so_G = host_link_latency(prob.gpu_cpu, Gr / gre_size * go);
+  const double si_G = host_link_latency(prob.cpu_gpu, Gr / gre_size * go);
+  const double so_O = host_link_latency(prob.gpu_cpu, O / ore_size * oo);
+  const double si_O = host_link_latency(prob.cpu_gpu, O / ore_size * oo);
+  const double so_A_ck = host_link_latency(prob.gpu_cpu, raw_ck * ao);
+  const double si_A_ck = host_link_latency(prob.cpu_gpu, raw_ck * ao);
+  const double so_A_nock = host_link_latency(prob.gpu_cpu, raw_nock * ao);
+  const double si_A_nock = host_link_latency(prob.cpu_gpu, raw_nock * ao);
+  const double n_nodes = (double)g->num_nodes;
+  const double dp_inter = dp > n_nodes ? n_nodes : dp;
+  const double dp_intra = dp > n_nodes ? floor(dp / n_nodes) : 1.0;
+  const double AG_w = gpu_gpu_latency(prob.gpu_gpu, W, dp_inter, dp_intra, 1.0);
+  const double RS_g = gpu_gpu_latency(prob.gpu_gpu, Gr, dp_inter, dp_intra, 1.1);
+  const double AR_g = gpu_gpu_latency(prob.gpu_gpu, Gr, dp_inter, dp_intra, 2.1);
+
+  const Interference I{prob.interf_factor};
+  const bool adv = prob.adv_first_block != 0;
+
+  // ---- forward phases (:1432-1621): index 0 = first micro-batch, 1 = not first ----
+  const double g2c_F[2] = {so_O + so_W, 0.0};
+  const double c2g_F[2] = {si_O + si_G, si_W};
+  const double g2g_F[2] = {AG_w * ore, AG_w * wre};
+  const double E_f = exec_fwd - extra_fwd;
+  Family fwd[2][2];  // [phase][0 = nock, 1 = ck]
+#pragma unroll
+  for (int ph = 0; ph < 2; ++ph) {
+    const double pre_g2g = (ph == 0 || adv) ? g2g_F[ph] : 0.0;
+    const double pre_c2g = adv ? c2g_F[ph] : 0.0;
+    const double first = I(E_f, g2g_F[ph], 0.0, c2g_F[ph]) + extra_fwd;
+    const double extra_pre = I(0.0, pre_g2g, 0.0, pre_c2g);
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const double g2c = g2c_F[ph] + (k ? so_A_ck : so_A_nock);
+      fwd[ph][k].layer = I(E_f, g2g_F[ph], g2c, c2g_F[ph]) + extra_fwd;
+      fwd[ph][k].first = first;
+      fwd[ph][k].last = I(E_f, 0.0, g2c, 0.0) + extra_fwd;
+      fwd[ph][k].extra_pre = extra_pre;
+      fwd[ph][k].extra_post = I(0.0, 0.0, g2c, 0.0);
+    }
+  }
+
+  // ---- backward phases (:1646-1902): index 0 = last micro-batch, 1 = not last ----
+  const double g2c_B = so_G;
+  const double c2g_B = si_W + si_G;
+  const double ag_wre = AG_w * wre;
+  const double g2g_B[2] = {ag_wre + RS_g * ore + AR_g * (1.0 - ore), ag_wre + RS_g * gre};
+  const double extra_fb = extra_fwd + extra_bwd;
+  const double exec_bwd_ck = exec_fwd + exec_bwd_nock;
+  const double first_g2c = adv ? g2c_B : 0.0;
+  Family bwd[2][2];
+#pragma unroll
+  for (int ph = 0; ph < 2; ++ph) {
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const double E = k ? exec_bwd_ck - extra_fb : exec_bwd_nock - extra_bwd;
+      const double extra = k ? extra_fb : extra_bwd;
+      const double c2g = c2g_B + (k ? si_A_ck : si_A_nock);
+      double red;
+      if (ph == 0) red = k ? (ore == 1.0 ? RS_g : AR_g) : RS_g * ore + AR_g * (1.0 - ore);
+      else red = RS_g * gre;
+      // With checkpointing the reference adds the (always zero) all-gather of saved tensors.
+      const double g2g_layer = k ? g2g_B[ph] + 0.0 : g2g_B[ph];
+      bwd[ph][k].layer = I(E, g2g_layer, g2c_B, c2g) + extra;
+      bwd[ph][k].last = I(E, ag_wre, 0.0, c2g) + extra;
+      bwd[ph][k].first = I(E, red, first_g2c, 0.0) + extra;
+      bwd[ph][k].extra_pre = I(0.0, ag_wre, 0.0, c2g);
+      bwd[ph][k].extra_post = I(0.0, red, first_g2c, 0.0);
+    }
+  }
+
+  // ---- stable / delta families (:1910-2028) ----
+  double *t = row_terms + (g->row_offset + row) * MIST_ROW_TERMS;
+  const int st = g->grad_accum == 1 ? 0 : 1;  // phase index that forms the stable part
+#pragma unroll
+  for (int k = 0; k < 2; ++k) {
+    const Family &f = fwd[st][k], &w = bwd[st][k];
+    const double s_layer = f.layer + w.layer;
+    const double s_first = f.extra_pre + w.extra_post + f.first + w.first;
+    const double s_last = f.extra_post + w.extra_pre + f.last + w.last;
+    double d_layer = 0.0, d_first = 0.0, d_last = 0.0;
+    if (st == 1) {
+      const Family &f1 = fwd[0][k], &w1 = bwd[0][k];
+      d_layer = f1.layer + w1.layer - s_layer;
+      d_first = f1.extra_pre + w1.extra_post + f1.first + w1.first - s_first;
+      d_last = f1.extra_post + w1.extra_pre + f1.last + w1.last - s_last;
+    }
+    // k == 1 is "with ckpt": the *_CK slot precedes the *_NOCK slot.
+    t[MIST_T_S_LAYER_CK + (1 - k)] = s_layer;
+    t[MIST_T_S_FIRST_CK + (1 - k)] = s_first;
+    t[MIST_T_S_LAST_CK + (1 - k)] = s_last;
+    t[MIST_T_D_LAYER_CK + (1 - k)] = d_layer;
+    t[MIST_T_D_FIRST_CK + (1 - k)] = d_first;
+    t[MIST_T_D_LAST_CK + (1 - k)] = d_last;
+  }
+
+  t[MIST_T_FWD_STATES0] = two_buf + np_floor_divide(O, ore_size);
+  t[MIST_T_BWD_STATES0] = two_buf;
+  t[MIST_T_PWG] = pW + pG;
+  t[MIST_T_PO] = pO;
+  t[MIST_T_PWGO] = pW + pG + pO;
+  t[MIST_T_S_CK] = S_ck;
+  t[MIST_T_S_NOCK] = S_nock;
+  t[MIST_T_D_CK] = D_ck;
+  t[MIST_T_D_NOCK] = D_nock;
+  t[MIST_T_MF_BASE] = mf_pp + 0.01;
+  t[MIST_T_MF_PP] = mf_pp;
+  t[MIST_T_MF] = mf;
+  t[MIST_T_FWD_PEAK] = par[MIST_PAR_FWD_PEAK];
+  t[MIST_T_BWD_PEAK] = par[MIST_PAR_BWD_PEAK];
+  t[MIST_T_OUT] = par[MIST_PAR_OUT];
+  t[MIST_T_GCB] = par[MIST_PAR_GCB];
+
+  // ---- post-layer overlap pieces (:2251-2292) ----
+  const double ovw_ck = fmax(exec_fwd - 0.0 - so_A_ck, 0.0);
+  const double ovw_nock = fmax(exec_fwd - 0.0 - so_A_nock, 0.0);
+  t[MIST_T_NAG_CK] = fmax(g->post_ag - ovw_ck, 0.0);
+  t[MIST_T_NAG_NOCK] = fmax(g->post_ag - ovw_nock, 0.0);
+  const double ovg_ck = fmax(exec_bwd_ck - ag_wre - c2g_B - si_A_ck, 0.0);
+  const double ovg_nock = fmax(exec_bwd_nock - ag_wre - c2g_B - si_A_nock, 0.0);
+  t[MIST_T_NRS_CK] = fmax(g->post_rs - ovg_ck, 0.0);
+  t[MIST_T_NRS_NOCK] = fmax(g->post_rs - ovg_nock, 0.0);
+  t[MIST_T_OPB] = fmax(g->post_bwd - bwd[1][1].extra_pre, 0.0);
+  t[MIST_T_RD] = raw_nock - S_nock;
+}
+
+// ------------------------------------------------------------------------------------------
+// Per-cell evaluation shared by the reduce and finalize kernels.
+// ------------------------------------------------------------------------------------------
+struct PairIndex {
+  int l, c;  // layers in the stage (1..L), checkpointed layers (0..l)
+};
+
+// Valid (l, c <= l) pairs are numbered l-major: index(l, c) = l*(l+1)/2 - 1 + c.
+__device__ __forceinline__ PairIndex decode_pair(int idx) {
+  int l = (int)((sqrt(8.0 * (double)idx + 9.0) - 1.0) * 0.5);
+  while (l * (l + 1) / 2 - 1 > idx) --l;
+  while ((l + 1) * (l + 2) / 2 - 1 <= idx) ++l;
+  return PairIndex{l, idx - (l * (l + 1) / 2 - 1)};
+}
+
+struct CellLatency {
+  float x, d;           // stable, delta rounded to float32 (batched_module_analyzer.py:2212-2213)
+  double sp, dpre;      // with_pre stable / delta (float64)
+  double spost, dpost;  // with_post
+  double spp, dpp;      // pre_and_post (no_pp)
+};
+
+struct GroupConsts {
+  double pre_fwd, pre_bwd, post_fwd;
+  double w1, w2, w1d, w2d;  // pre-layer all-gather / reduce-scatter split into stable / delta
+  bool pp_wre, pp_gre;
+};
+
+__device__ __forceinline__ GroupConsts group_consts(const MistGroupDesc *g) {
+  GroupConsts k;
+  k.pre_fwd = g->pre_fwd;
+  k.pre_bwd = g->pre_bwd;
+  k.post_fwd = g->post_fwd;
+  k.pp_wre = g->pp_wre == 1;
+  k.pp_gre = g->pp_gre == 1;
+  k.w1 = k.pp_wre ? g->pre_ag : 0.0;
+  k.w2 = k.pp_gre ? g->pre_rs : 0.0;
+  k.w1d = k.pp_wre ? 0.0 : g->pre_ag;
+  k.w2d = k.pp_gre ? 0.0 : g->pre_rs;
+  return k;
+}
+
+// get_latencies (:2165-2216) and the pre / post additions (:2233-2351) for one row and (l, c).
+template <bool kWithPost>
+__device__ __forceinline__ CellLatency cell_latency(const double *__restrict__ t, int l, int c,
+                                                    const GroupConsts &k) {
+  const int lm2 = max(l - 2, 0);
+  const int n_ck = min(max(c - 1, 0), lm2);
+  const int n_nock = lm2 - n_ck;
+  const bool all_ck = c == l, no_ck = c == 0;
+  const double stable = (double)n_ck * t[MIST_T_S_LAYER_CK] + (double)n_nock * t[MIST_T_S_LAYER_NOCK] +
+                        (all_ck ? t[MIST_T_S_FIRST_CK] : t[MIST_T_S_FIRST_NOCK]) +
+                        (no_ck ? t[MIST_T_S_LAST_NOCK] : t[MIST_T_S_LAST_CK]);
+  const double delta = (double)n_ck * t[MIST_T_D_LAYER_CK] + (double)n_nock * t[MIST_T_D_LAYER_NOCK] +
+                       (all_ck ? t[MIST_T_D_FIRST_CK] : t[MIST_T_D_FIRST_NOCK]) +
+                       (no_ck ? t[MIST_T_D_LAST_NOCK] : t[MIST_T_D_LAST_CK]);
+  CellLatency r;
+  r.x = (float)stable;
+  r.d = (float)delta;
+  const double x = (double)r.x, d = (double)r.d;
+  r.sp = x + k.pre_fwd + k.pre_bwd + k.w1 + k.w2;
+  r.dpre = d + k.w1d + k.w2d;
+  if (kWithPost) {
+    const double nag = c > 0 ? t[MIST_T_NAG_CK] : t[MIST_T_NAG_NOCK];
+    const double nrs = c > 0 ? t[MIST_T_NRS_CK] : t[MIST_T_NRS_NOCK];
+    const double ps1 = k.pp_wre ? nag : 0.0, ps2 = k.pp_gre ? nrs : 0.0;
+    const double pd1 = k.pp_wre ? 0.0 : nag, pd2 = k.pp_gre ? 0.0 : nrs;
+    const double opb = t[MIST_T_OPB];
+    r.spost = x + k.post_fwd + opb + ps1 + ps2;
+    r.dpost = d + pd1 + pd2;
+    r.spp = x + k.pre_fwd + k.pre_bwd + k.post_fwd + opb + k.w1 + k.w2 + ps1 + ps2;
+    r.dpp = d + k.w1d + k.w2d + pd1 + pd2;
+  } else {
+    r.spost = r.dpost = r.spp = r.dpp = 0.0;
+  }
+  return r;
+}
+
+// Lexicographic running minimum: strictly smaller cost wins; rows arrive in ascending order so
+// the first row keeps ties, exactly like the strict "<" scan of mist/utils/pareto.py:134-142.
+__device__ __forceinline__ void take_min(double &best, int32_t &best_row, bool feasible,
+                                         double cost, int32_t row) {
+  const bool better = feasible && cost < best;
+  best = better ? cost : best;
+  best_row = better ? row : best_row;
+}
+
+// ------------------------------------------------------------------------------------------
+// Kernel 2: evaluate + mask + running argmin.
+// Workgroup = 256 threads = one tile of (l, c) pairs; it streams one chunk of candidate rows
+// through LDS (every lane reads the same row: broadcast reads, no bank conflicts) and each
+// thread keeps the minima of MIST_P_TILE pre-saved micro-batch values for its own (l, c).
+// No cross-lane reduction is needed: the reduction axis (rows) is the loop, not the lanes.
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(MIST_LC_TILE) void eval_reduce_kernel(
+    const MistProblem prob, const MistGroupDesc *__restrict__ groups, int n_groups,
+    const int32_t *__restrict__ block_prefix, const double *__restrict__ row_terms, double ratio,
+    double *__restrict__ partial_cost, int32_t *__restrict__ partial_index) {
+  __shared__ double lds_terms[kStageRows * MIST_ROW_TERMS];
+
+  int local_block;
+  const MistGroupDesc *g = find_group(groups, block_prefix, n_groups, blockIdx.x, &local_block);
+  const int chunk = local_block % g->n_chunks;
+  const int tile = local_block / g->n_chunks;
+  const int p_tile = tile % g->n_p_tiles;
+  const int lc_tile = tile / g->n_p_tiles;
+
+  const int L = prob.num_layers;
+  const int n_pairs = L * (L + 1) / 2 + L;  // sum over l = 1..L of (l + 1)
+  const int pair_idx = lc_tile * MIST_LC_TILE + threadIdx.x;
+  const bool active = pair_idx < n_pairs;
+  const PairIndex pc = decode_pair(active ? pair_idx : 0);
+  const int l = pc.l, c = pc.c;
+
+  const int p0 = p_tile * MIST_P_TILE;
+  const int num_p = g->num_p;
+  const bool first_p_tile = p_tile == 0;
+  const bool do_nopp = first_p_tile && l == L;
+  const GroupConsts k = group_consts(g);
+  const double cap = prob.mem_cap_mb;
+  const double G64 = (double)g->grad_accum;
+  const float G32 = (float)g->grad_accum;
+  const double pre_saved = g->pre_saved, pre_sas = g->pre_states_and_saved;
+  const double pre_states = g->pre_states;
+  const double post_states = g->post_states, post_fwd_peak = g->post_fwd_peak;
+  const double post_bwd_peak = g->post_bwd_peak, post_output = g->post_output;
+
+  double best[kSlots];
+  int32_t best_row[kSlots];
+#pragma unroll
+  for (int s = 0; s < kSlots; ++s) {
+    best[s] = INFINITY;
+    best_row[s] = -1;
+  }
+
+  const int64_t row_begin = (int64_t)chunk * g->rows_per_chunk;
+  const int64_t row_end = min(row_begin + (int64_t)g->rows_per_chunk, g->n_rows);
+  const double *__restrict__ src = row_terms + g->row_offset * MIST_ROW_TERMS;
+
+  const double lf = (double)l, lm1 = (double)max(l - 1, 0), cf = (double)c;
+  const double l_minus_c = (double)(l - c), l_minus_c_1 = (double)(l - c - 1);
+  const bool c_eq_l = c == l, c_ge_lm1 = c >= l - 1, c_eq_0 = c == 0;
+
+  for (int64_t base = row_begin; base < row_end; base += kStageRows) {
+    const int n_stage = (int)min((int64_t)kStageRows, row_end - base);
+    __syncthreads();
+    for (int i = threadIdx.x; i < n_stage * MIST_ROW_TERMS; i += MIST_LC_TILE)
+      lds_terms[i] = src[base * MIST_ROW_TERMS + i];
+    __syncthreads();
+    if (!active) continue;
+
+    for (int rr = 0; rr < n_stage; ++rr) {
+      const double *__restrict__ t = lds_terms + rr * MIST_ROW_TERMS;
+      const int32_t row = (int32_t)(base + rr);
+
+      // ---- objective values (mist/utils/pareto.py:138: r * x + y in float64) ----
+      CellLatency lat;
+      if (first_p_tile) lat = cell_latency<true>(t, l, c, k);
+      else lat = cell_latency<false>(t, l, c, k);
+      const float y32 = lat.d / G32;  // float32 array / python int (:2815)
+      const double cost_base = ratio * (double)lat.x + (double)y32;
+      const double cost_pre = ratio * lat.sp + lat.dpre / G64;
+
+      // ---- memory that does not depend on p (:2150-2162, 2358-2385, 2760-2769) ----
+      const double S_ck = t[MIST_T_S_CK], S_nock = t[MIST_T_S_NOCK];
+      const double fwd_states = t[MIST_T_FWD_STATES0] + lf * t[MIST_T_PWG] + lm1 * t[MIST_T_PO];
+      const double bwd_states = t[MIST_T_BWD_STATES0] + lf * t[MIST_T_PWGO];
+      const double cur_saved = c_eq_l ? (lf - 1.0) * S_ck : cf * S_ck + l_minus_c_1 * S_nock;
+      const double mod_saved = S_ck * cf + S_nock * l_minus_c;
+      const double ck_delta = c_ge_lm1 ? t[MIST_T_D_CK] : t[MIST_T_D_NOCK];
+      const double fwd_pk = t[MIST_T_FWD_PEAK], bwd_pk = t[MIST_T_BWD_PEAK];
+      const double out = t[MIST_T_OUT], gcb = t[MIST_T_GCB];
+      const double out2 = out * 2.0;
+      const double mf_base = t[MIST_T_MF_BASE], mf_pp = t[MIST_T_MF_PP];
+
+#pragma unroll
+      for (int j = 0; j < MIST_P_TILE; ++j) {
+        const int p = p0 + j;
+        const double pf64 = (double)p;
+        const double pipe_saved = pf64 * mod_saved + cur_saved;
+        const double outp2 = out * pf64 * 2.0;
+        const double peak_f = fwd_states + pipe_saved + ck_delta + fwd_pk + outp2 + gcb;
+        const double peak_b = bwd_states + pipe_saved + ck_delta + bwd_pk + outp2 + out2 + gcb;
+        const bool in_range = p < num_p;
+        const bool ok_base = in_range && fmax(peak_f, peak_b) * mf_base <= cap;
+        take_min(best[j], best_row[j], ok_base, cost_base, row);
+        const double pre_p = pf64 * pre_saved;
+        const double peak_f_pre = pre_p + peak_f + pre_sas;
+        const double peak_b_pre = pre_p + peak_b + pre_sas;
+        const bool ok_pre = in_range && fmax(peak_f_pre, peak_b_pre) * mf_pp <= cap;
+        take_min(best[MIST_P_TILE + j], best_row[MIST_P_TILE + j], ok_pre, cost_pre, row);
+
+        if (j == 0 && first_p_tile) {
+          // ---- last stage / single stage, p == 0 only (:2946-3106) ----
+          const double f_in = fwd_states + post_states + mod_saved + post_fwd_peak + gcb;
+          const double b_in = bwd_states + post_states + mod_saved + post_bwd_peak +
+                              (c_eq_0 ? t[MIST_T_RD] : 0.0) + gcb;
+          const double pf_post = fmax(f_in, peak_f + post_states);
+          const double pb_post = fmax(b_in, peak_b - out + post_states) + post_output;
+          const bool ok_post = fmax(pf_post, pb_post) * mf_pp <= cap;
+          const double cost_post = ratio * lat.spost + lat.dpost / G64;
+          take_min(best[2 * MIST_P_TILE], best_row[2 * MIST_P_TILE], ok_post, cost_post, row);
+          if (do_nopp) {
+            const double pf_pp = pf_post + pre_states + pre_saved;
+            const double pb_pp = pb_post + pre_states + pre_saved;
+            const bool ok_pp = fmax(pf_pp, pb_pp) * t[MIST_T_MF] <= cap;
+            const double cost_pp = ratio * lat.spp + lat.dpp / G64;
+            take_min(best[2 * MIST_P_TILE + 1], best_row[2 * MIST_P_TILE + 1], ok_pp, cost_pp,
+                     row);
+          }
+        }
+      }
+    }
+  }
+
+  const int64_t out_base = (int64_t)blockIdx.x * kSlots * MIST_LC_TILE + threadIdx.x;
+#pragma unroll
+  for (int s = 0; s < kSlots; ++s) {
+    partial_cost[out_base + (int64_t)s * MIST_LC_TILE] = best[s];
+    partial_index[out_base + (int64_t)s * MIST_LC_TILE] = best_row[s];
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// Kernel 3: combine chunks in order, recompute the winner's stable / delta, scatter.
+// One thread per (group, (l, c) pair, slot); slots as in the reduce kernel but over all p.
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void finalize_kernel(
+    const MistProblem prob, const MistGroupDesc *__restrict__ groups, int n_groups,
+    const int32_t *__restrict__ block_prefix, const double *__restrict__ row_terms,
+    const double *__restrict__ partial_cost, const int32_t *__restrict__ partial_index,
+    int sample_index, MistOutTables tables) {
+  const int L = prob.num_layers;
+  const int n_pairs = L * (L + 1) / 2 + L;
+  const int gi = blockIdx.z;
+  const MistGroupDesc *g = groups + gi;
+  const int pair_idx = blockIdx.x * blockDim.x + threadIdx.x;
+  // blockIdx.y: 0..p_dim-1 base, p_dim..2*p_dim-1 with_pre, 2*p_dim with_post, 2*p_dim+1 no_pp
+  const int P1 = prob.p_dim;
+  const int slot = blockIdx.y;
+  if (pair_idx >= n_pairs) return;
+  int variant, p;
+  if (slot < P1) { variant = 0; p = slot; }
+  else if (slot < 2 * P1) { variant = 1; p = slot - P1; }
+  else { variant = 2 + (slot - 2 * P1); p = 0; }
+  if (p >= g->num_p) return;
+  const PairIndex pc = decode_pair(pair_idx);
+  const int l = pc.l, c = pc.c;
+  // Cells the reference never writes (batched_module_analyzer.py:3021-3023 rebinds the layer
+  // mask inside the p == 0 branch, so it also governs base / with_pre for p >= 1; :3103).
+  if (variant <= 1 && p >= 1 && c == l - 1) return;
+  if (variant == 2 && c == l - 1) return;
+  if (variant == 3 && (l != L || c == L - 1)) return;
+
+  const int lc_tile = pair_idx / MIST_LC_TILE, lane = pair_idx % MIST_LC_TILE;
+  const int p_tile = p / MIST_P_TILE;
+  int kslot;
+  if (variant == 0) kslot = p % MIST_P_TILE;
+  else if (variant == 1) kslot = MIST_P_TILE + p % MIST_P_TILE;
+  else kslot = 2 * MIST_P_TILE + (variant - 2);
+  const int64_t first_block =
+      (int64_t)block_prefix[gi] + (int64_t)(lc_tile * g->n_p_tiles + p_tile) * g->n_chunks;
+  double best = INFINITY;
+  int32_t best_row = -1;
+  for (int ch = 0; ch < g->n_chunks; ++ch) {
+    const int64_t at = ((first_block + ch) * kSlots + kslot) * MIST_LC_TILE + lane;
+    const double cost = partial_cost[at];
+    const int32_t row = partial_index[at];
+    take_min(best, best_row, row >= 0, cost, row);
+  }
+
+  double stable = INFINITY, delta = INFINITY;
+  if (best_row >= 0) {
+    const double *t = row_terms + (g->row_offset + best_row) * MIST_ROW_TERMS;
+    const CellLatency lat = cell_latency<true>(t, l, c, group_consts(g));
+    if (variant == 0) { stable = (double)lat.x; delta = (double)lat.d; }
+    else if (variant == 1) { stable = lat.sp; delta = lat.dpre; }
+    else if (variant == 2) { stable = lat.spost; delta = lat.dpost; }
+    else { stable = lat.spp; delta = lat.dpp; }
+  }
+
+  const int S = prob.sample_size;
+  const int64_t gq = (int64_t)g->g_index * prob.num_mesh + g->q_index;
+  int64_t at;
+  if (variant <= 1) at = (((gq * P1 + p) * L + (l - 1)) * (L + 1) + c) * S + sample_index;
+  else if (variant == 2) at = ((gq * L + (l - 1)) * (L + 1) + c) * S + sample_index;
+  else at = (gq * (L + 1) + c) * S + sample_index;
+  tables.stable[variant][at] = stable;
+  tables.delta[variant][at] = delta;
+  tables.index[variant][at] = best_row;
+}
+
+int check_common(const void *d_problem, const void *d_groups, int n_groups) {
+  if (!d_problem || !d_groups) return fail(MIST_E_INVALID, "null problem / group pointer");
+  if (n_groups <= 0) return fail(MIST_E_INVALID, "n_groups must be positive, got %d", n_groups);
+  return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *mist_version(void) { return "mist_search 0.1 (gfx950)"; }
+const char *mist_last_error(void) { return g_last_error; }
+int mist_sizeof_problem(void) { return (int)sizeof(MistProblem); }
+int mist_sizeof_group(void) { return (int)sizeof(MistGroupDesc); }
+
+int mist_row_terms(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,
+                   const int32_t *d_block_prefix, int n_blocks, double *d_row_terms,
+                   void *stream) {
+  if (int rc = check_common(problem, d_groups, n_groups)) return rc;
+  if (!d_block_prefix || !d_row_terms) return fail(MIST_E_INVALID, "null workspace pointer");
+  if (n_blocks <= 0) return fail(MIST_E_INVALID, "n_blocks must be positive, got %d", n_blocks);
+  hipLaunchKernelGGL(row_terms_kernel, dim3(n_blocks), dim3(kTermsBlock), 0, (hipStream_t)stream,
+                     *problem, d_groups, n_groups, d_block_prefix, d_row_terms);
+  MIST_HIP_CHECK(hipGetLastError());
+  return 0;
+}
+
+int mist_eval_reduce(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,
+                     const int32_t *d_block_prefix, int n_blocks, const double *d_row_terms,
+                     double ratio, double *d_partial_cost, int32_t *d_partial_index,
+                     void *stream) {
+  if (int rc = check_common(problem, d_groups, n_groups)) return rc;
+  if (!d_block_prefix || !d_row_terms || !d_partial_cost || !d_partial_index)
+    return fail(MIST_E_INVALID, "null workspace pointer");
+  if (n_blocks <= 0) return fail(MIST_E_INVALID, "n_blocks must be positive, got %d", n_blocks);
+  if (!(ratio >= 0.0)) return fail(MIST_E_INVALID, "ratio must be non-negative");
+  hipLaunchKernelGGL(eval_reduce_kernel, dim3(n_blocks), dim3(MIST_LC_TILE), 0,
+                     (hipStream_t)stream, *problem, d_groups, n_groups, d_block_prefix,
+                     d_row_terms, ratio, d_partial_cost, d_partial_index);
+  MIST_HIP_CHECK(hipGetLastError());
+  return 0;
+}
+
+int mist_finalize(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,
+                  const int32_t *d_block_prefix, const double *d_row_terms,
+                  const double *d_partial_cost, const int32_t *d_partial_index,
+                  int sample_index, const MistOutTables *tables, void *stream) {
+  if (int rc = check_common(problem, d_groups, n_groups)) return rc;
+  if (!d_block_prefix || !d_row_terms || !d_partial_cost || !d_partial_index || !tables)
+    return fail(MIST_E_INVALID, "null pointer argument");
+  for (int v = 0; v < 4; ++v)
+    if (!tables->stable[v] || !tables->delta[v] || !tables->index[v])
+      return fail(MIST_E_INVALID, "output table %d is null", v);
+  const MistProblem &prob = *problem;
+  const int L = prob.num_layers, P1 = prob.p_dim;
+  if (L <= 0 || P1 <= 0 || prob.sample_size <= 0)
+    return fail(MIST_E_INVALID, "bad problem extents L=%d P+1=%d S=%d", L, P1, prob.sample_size);
+  if (sample_index < 0 || sample_index >= prob.sample_size)
+    return fail(MIST_E_INVALID, "sample_index %d outside [0, %d)", sample_index, prob.sample_size);
+  if (n_groups > 65535) return fail(MIST_E_INVALID, "too many groups for one launch: %d", n_groups);
+  const int n_pairs = L * (L + 1) / 2 + L;
+  dim3 grid((n_pairs + 255) / 256, 2 * P1 + 2, n_groups);
+  hipLaunchKernelGGL(finalize_kernel, grid, dim3(256), 0, (hipStream_t)stream, prob, d_groups,
+                     n_groups, d_block_prefix, d_row_terms, d_partial_cost, d_partial_index,
+                     sample_index, *tables);
+  MIST_HIP_CHECK(hipGetLastError());
+  return 0;
+}
+
+int mist_intra_stage_eval(const MistProblem *problem, const MistGroupDesc *d_groups,
+                          int n_groups, const int32_t *d_terms_block_prefix, int n_terms_blocks,
+                          const int32_t *d_reduce_block_prefix, int n_reduce_blocks,
+                          double *d_row_terms, double *d_partial_cost, int32_t *d_partial_index,
+                          double ratio, int sample_index, int compute_terms,
+                          const MistOutTables *tables, void *stream) {
+  if (compute_terms) {
+    if (int rc = mist_row_terms(problem, d_groups, n_groups, d_terms_block_prefix,
+                                n_terms_blocks, d_row_terms, stream))
+      return rc;
+  }
+  if (int rc = mist_eval_reduce(problem, d_groups, n_groups, d_reduce_block_prefix,
+                                n_reduce_blocks, d_row_terms, ratio, d_partial_cost,
+                                d_partial_index, stream))
+    return rc;
+  return mist_finalize(problem, d_groups, n_groups, d_reduce_block_prefix, d_row_terms,
+                       d_partial_cost, d_partial_index, sample_index, tables, stream);
+}
+
+}  // extern "C"

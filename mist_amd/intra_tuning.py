@@ -1,0 +1,293 @@
+"""Intra-stage tuner: the drop-in for the reference's ``mist/analyzer/intra_tuning.py``.
+
+``IntraStageTuner.tune()`` (reference :169-282) loops the gradient-accumulation candidates and
+device meshes and calls the numpy evaluation once per (G, mesh).  Here the host only prepares
+one small descriptor per (G, mesh) group; all groups of a tuner call are then evaluated by three
+kernel launches on the GPU (row terms, evaluate+mask+argmin, finalize) and the result tables
+stay resident in HBM for the inter-stage search.  ``IntraStageTunerOutput`` exposes the same
+fields and layouts as the reference (:59-82); numpy copies are made lazily on first access.
+"""
+from __future__ import annotations
+
+import ctypes
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from . import _lib
+from .config import MistConfig
+from .layer_tables import LayerTables
+from .search_space import SearchSpace, create_search_space_for_a_block_layer
+from .stage_inputs import GroupInputBuilder, make_problem
+
+SAMPLE_SIZE = 30  # reference default (batched_module_analyzer.py:67)
+VARIANTS = ("", "_with_pre", "_with_post", "_no_pp")
+TARGET_REDUCE_BLOCKS = 6144
+
+
+def alpha_ratios(sample_size: int) -> np.ndarray:
+    """``alpha_k / (1 - alpha_k)`` for ``alpha = linspace(0, 1, S + 2)[1:-1]``
+    (mist/utils/pareto.py:53-55,138)."""
+    alpha = np.linspace(0, 1, sample_size + 2)[1:-1]
+    return alpha / (1 - alpha)
+
+
+def _ptr(t: Optional[torch.Tensor]) -> int:
+    return 0 if t is None else t.data_ptr()
+
+
+@dataclass
+class DeviceTables:
+    """float64 cost tables and int32 row-index tables in HBM, reference layout."""
+
+    stable: List[torch.Tensor]
+    delta: List[torch.Tensor]
+    index: List[torch.Tensor]
+
+    def as_struct(self) -> _lib.OutTables:
+        s = _lib.OutTables()
+        for v in range(4):
+            s.stable[v] = self.stable[v].data_ptr()
+            s.delta[v] = self.delta[v].data_ptr()
+            s.index[v] = self.index[v].data_ptr()
+        return s
+
+
+class IntraStageTunerOutput:
+    """Same attributes as the reference's ``IntraStageTunerOutput`` (intra_tuning.py:59-82):
+    ``costs_stable*`` / ``costs_delta*`` float32, ``solutions*`` float64 with ``inf`` fill.
+    Additionally ``indices*`` (row index per cell, -1 = none) and ``device`` (the HBM tables)."""
+
+    def __init__(
+        self,
+        gradient_accumulation_steps_candidates: List[int],
+        device_mesh_candidates: List[Tuple[int, int]],
+        device: DeviceTables,
+        spaces: Dict[Tuple[int, int], SearchSpace],
+        sample_slots: Sequence[int],
+    ):
+        self.gradient_accumulation_steps_candidates = list(gradient_accumulation_steps_candidates)
+        self.device_mesh_candidates = list(device_mesh_candidates)
+        self.device = device
+        self.spaces = spaces
+        self.sample_slots = tuple(sample_slots)
+        self._host: Dict[str, np.ndarray] = {}
+
+    def _fetch(self, kind: str, v: int) -> np.ndarray:
+        key = f"{kind}{v}"
+        if key not in self._host:
+            self._host[key] = getattr(self.device, kind)[v].cpu().numpy()
+        return self._host[key]
+
+    def costs_f64(self, kind: str, variant: int) -> np.ndarray:
+        """float64 ``stable`` / ``delta`` table of variant 0..3 as computed on the GPU."""
+        return self._fetch(kind, variant)
+
+    def _solutions(self, v: int) -> np.ndarray:
+        key = f"solutions{v}"
+        if key not in self._host:
+            idx = self._fetch("index", v)
+            out = np.full(idx.shape + (10,), np.inf, dtype=np.float64)
+            for (g, q), space in self.spaces.items():
+                out[g, q] = space.decode(idx[g, q])
+            self._host[key] = out
+        return self._host[key]
+
+    def __getattr__(self, name: str):
+        for v, suffix in enumerate(VARIANTS):
+            if name == "costs_stable" + suffix:
+                return self._fetch("stable", v).astype(np.float32)
+            if name == "costs_delta" + suffix:
+                return self._fetch("delta", v).astype(np.float32)
+            if name == "solutions" + suffix:
+                return self._solutions(v)
+            if name == "indices" + suffix:
+                return self._fetch("index", v).astype(np.int64)
+        raise AttributeError(name)
+
+    def __repr__(self) -> str:
+        return (
+            f"IntraStageTunerOutput("
+            f"gradient_accumulation_steps_candidates={self.gradient_accumulation_steps_candidates}, "
+            f"device_mesh_candidates={self.device_mesh_candidates}."
+        )
+
+
+class IntraStageTuner:
+    """Reference: ``IntraStageTuner`` (mist/analyzer/intra_tuning.py:84-282).  ``layer_tables``
+    replaces the three ``LayerInfo`` arguments."""
+
+    def __init__(
+        self,
+        layer_tables: LayerTables,
+        num_layers: int,
+        device_mesh_candidates: List[Tuple[int, int]],
+        gradient_accumulation_steps_candidates: List[int],
+        tp_size: Optional[int],
+        config: MistConfig,
+        disable_tqdm: bool = True,
+        sample_size: int = SAMPLE_SIZE,
+        sample_slots: Optional[Sequence[int]] = None,
+        device: str = "cuda:0",
+    ):
+        self.layer_tables = layer_tables
+        self.num_layers = int(num_layers)
+        self.device_mesh_candidates = list(device_mesh_candidates)
+        self.gradient_accumulation_steps_candidates = list(gradient_accumulation_steps_candidates)
+        self.tp_size = tp_size
+        self.config = config
+        self.sample_size = int(sample_size)
+        # Which of the S alpha samples to evaluate (default: all); unevaluated slots stay inf / -1.
+        self.sample_slots = tuple(range(self.sample_size)) if sample_slots is None else tuple(sample_slots)
+        self.device = torch.device(device)
+        # intra_tuning.py:117-126
+        self.max_possible_num_stages = min(
+            max(n * m for n, m in self.device_mesh_candidates), self.num_layers
+        )
+        self.max_possible_pre_saved_micro_batches = (
+            min(self.max_possible_num_stages, max(self.gradient_accumulation_steps_candidates)) - 1
+        )
+        self.results: Optional[IntraStageTunerOutput] = None
+        self.stats: Dict[str, float] = {}
+
+    # ------------------------------------------------------------------ host side
+    def prepare(self):
+        """Builds the group descriptors and the launch decomposition (host only, no GPU)."""
+        cfg, L = self.config, self.num_layers
+        Gs, Q = self.gradient_accumulation_steps_candidates, self.device_mesh_candidates
+        P = self.max_possible_pre_saved_micro_batches
+        builder = GroupInputBuilder(cfg, self.layer_tables)
+        spaces: Dict[Tuple[int, int], SearchSpace] = {}
+        pending = []
+        for g, G in enumerate(Gs):
+            for q, (n, m) in enumerate(Q):
+                space = create_search_space_for_a_block_layer(
+                    n, m, cfg.training.global_batch_size, G, cfg,
+                    constraint_fn=self.layer_tables.constraint, tp_size=self.tp_size,
+                )
+                spaces[(g, q)] = space
+                if space.n_rows == 0:
+                    continue  # the reference returns all-inf tables for an empty space (:648-666)
+                if space.n_rows >= 2**31:
+                    raise ValueError(f"group (G={G}, mesh={(n, m)}) has {space.n_rows} rows (>= 2**31)")
+                num_p = min(G, L, P + 1)  # intra_tuning.py:185-193
+                pending.append((g, q, n, m, G, num_p, space))
+        groups = np.zeros(len(pending), dtype=_lib.GROUP_DTYPE)
+        for i, (g, q, n, m, G, num_p, space) in enumerate(pending):
+            builder.fill(groups[i], space, g, q, n, m, G, num_p)
+
+        n_pairs = L * (L + 1) // 2 + L
+        n_lc_tiles = -(-n_pairs // _lib.LC_TILE)
+        if len(pending):
+            n_p_tiles = -(-groups["num_p"] // _lib.P_TILE)
+            tile_rows = int(np.sum(groups["n_rows"] * n_lc_tiles * n_p_tiles))
+            rows_per_chunk = -(-tile_rows // TARGET_REDUCE_BLOCKS)
+            rows_per_chunk = max(256, min(16384, -(-rows_per_chunk // _lib.STAGE_ROWS) * _lib.STAGE_ROWS))
+            groups["rows_per_chunk"] = rows_per_chunk
+            groups["n_chunks"] = -(-groups["n_rows"] // rows_per_chunk)
+            groups["n_lc_tiles"] = n_lc_tiles
+            groups["n_p_tiles"] = n_p_tiles
+            groups["row_offset"] = np.concatenate(([0], np.cumsum(groups["n_rows"])[:-1]))
+            terms_blocks = -(-groups["n_rows"] // _lib.TERMS_BLOCK)
+            reduce_blocks = groups["n_chunks"].astype(np.int64) * n_lc_tiles * n_p_tiles
+        else:
+            terms_blocks = reduce_blocks = np.zeros(0, dtype=np.int64)
+        terms_prefix = np.concatenate(([0], np.cumsum(terms_blocks))).astype(np.int64)
+        reduce_prefix = np.concatenate(([0], np.cumsum(reduce_blocks))).astype(np.int64)
+        if terms_prefix[-1] >= 2**31 or reduce_prefix[-1] >= 2**31:
+            raise ValueError("launch decomposition exceeds 2**31 workgroups")
+        problem = make_problem(cfg, L, P + 1, self.sample_size, len(Gs), len(Q))
+        return dict(
+            problem=problem, groups=groups, spaces=spaces,
+            terms_prefix=terms_prefix.astype(np.int32), reduce_prefix=reduce_prefix.astype(np.int32),
+            total_rows=int(groups["n_rows"].sum()) if len(pending) else 0,
+        )
+
+    def allocate_tables(self) -> DeviceTables:
+        Gn, Qn = len(self.gradient_accumulation_steps_candidates), len(self.device_mesh_candidates)
+        P1, L, S = self.max_possible_pre_saved_micro_batches + 1, self.num_layers, self.sample_size
+        shapes = [(Gn, Qn, P1, L, L + 1, S), (Gn, Qn, P1, L, L + 1, S), (Gn, Qn, L, L + 1, S), (Gn, Qn, L + 1, S)]
+        dev = self.device
+        return DeviceTables(
+            stable=[torch.full(s, float("inf"), dtype=torch.float64, device=dev) for s in shapes],
+            delta=[torch.full(s, float("inf"), dtype=torch.float64, device=dev) for s in shapes],
+            index=[torch.full(s, -1, dtype=torch.int32, device=dev) for s in shapes],
+        )
+
+    # ------------------------------------------------------------------ device side
+    def upload(self, plan) -> dict:
+        dev = self.device
+        def to_dev(a: np.ndarray) -> torch.Tensor:
+            return torch.from_numpy(np.ascontiguousarray(a).view(np.uint8).reshape(-1)).to(dev)
+        n_groups = len(plan["groups"])
+        n_reduce_blocks = int(plan["reduce_prefix"][-1])
+        return dict(
+            n_groups=n_groups,
+            groups=to_dev(plan["groups"]) if n_groups else None,
+            terms_prefix=to_dev(plan["terms_prefix"]),
+            reduce_prefix=to_dev(plan["reduce_prefix"]),
+            n_terms_blocks=int(plan["terms_prefix"][-1]),
+            n_reduce_blocks=n_reduce_blocks,
+            row_terms=torch.empty(max(plan["total_rows"], 1) * _lib.ROW_TERMS, dtype=torch.float64, device=dev),
+            partial_cost=torch.empty(max(n_reduce_blocks, 1) * _lib.SLOTS * _lib.LC_TILE, dtype=torch.float64, device=dev),
+            partial_index=torch.empty(max(n_reduce_blocks, 1) * _lib.SLOTS * _lib.LC_TILE, dtype=torch.int32, device=dev),
+        )
+
+    def launch(self, plan, dev_plan, tables: DeviceTables) -> None:
+        """Enqueues the kernels for every requested sample on the current stream."""
+        if dev_plan["n_groups"] == 0:
+            return
+        lib = _lib.load()
+        stream = ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+        ratios = alpha_ratios(self.sample_size)
+        out = tables.as_struct()
+        prob_ptr = ctypes.c_void_p(plan["problem"].ctypes.data)
+        for i, slot in enumerate(self.sample_slots):
+            rc = lib.mist_intra_stage_eval(
+                prob_ptr, _ptr(dev_plan["groups"]), dev_plan["n_groups"],
+                _ptr(dev_plan["terms_prefix"]), dev_plan["n_terms_blocks"],
+                _ptr(dev_plan["reduce_prefix"]), dev_plan["n_reduce_blocks"],
+                _ptr(dev_plan["row_terms"]), _ptr(dev_plan["partial_cost"]),
+                _ptr(dev_plan["partial_index"]), float(ratios[slot]), int(slot),
+                1 if i == 0 else 0, ctypes.byref(out), stream,
+            )
+            _lib.check(rc, "mist_intra_stage_eval")
+
+    def tune(self) -> IntraStageTunerOutput:
+        if self.device.type != "cuda" or not torch.cuda.is_available():
+            raise _lib.MistLibraryError("IntraStageTuner needs a GPU: the search kernels have no CPU path")
+        _lib.load()
+        plan = self.prepare()
+        with torch.cuda.device(self.device):
+            dev_plan = self.upload(plan)
+            tables = self.allocate_tables()
+            self.launch(plan, dev_plan, tables)
+        self._plan, self._dev_plan = plan, dev_plan
+        self.results = IntraStageTunerOutput(
+            self.gradient_accumulation_steps_candidates, self.device_mesh_candidates, tables,
+            plan["spaces"], self.sample_slots,
+        )
+        return self.results
+
+
+def intra_stage_tune(
+    layer_tables: LayerTables,
+    num_layers: int,
+    device_mesh_candidates: List[Tuple[int, int]],
+    gradient_accumulation_steps_candidates: List[int],
+    tp_size: Optional[int],
+    mist_config: MistConfig,
+    disable_tqdm: bool = True,
+    sample_size: int = SAMPLE_SIZE,
+    sample_slots: Optional[Sequence[int]] = None,
+    device: str = "cuda:0",
+) -> IntraStageTunerOutput:
+    """Reference: ``intra_stage_tune`` (mist/analyzer/intra_tuning.py:285-370) without the
+    pickle cache (results are recomputed; a tuner call takes milliseconds here)."""
+    return IntraStageTuner(
+        layer_tables, num_layers, device_mesh_candidates, gradient_accumulation_steps_candidates,
+        tp_size, mist_config, disable_tqdm=disable_tqdm, sample_size=sample_size,
+        sample_slots=sample_slots, device=device,
+    ).tune()

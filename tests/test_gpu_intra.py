@@ -1,0 +1,138 @@
+"""GPU parity of the intra-stage search against the numpy oracle (bit-exact).
+
+Bar: float64 row terms and cost tables equal bit for bit (stricter than the 1e-12 relative
+tolerance the task states), chosen row indices identical including ties.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+
+from tests.util import assert_same_f64, load_plan, oracle_terms, tiny_plan
+
+pytestmark = pytest.mark.gpu
+
+
+def _gpu_tuner(cfg, tables, tp, S=1, meshes=None, Gs=None, slots=None):
+    from mist_amd.intra_tuning import IntraStageTuner
+    from mist_amd.search_space import _get_device_mesh_candidates, _get_grad_accumu_steps_candidates
+
+    hw = cfg.hardware
+    meshes = meshes or _get_device_mesh_candidates(hw.num_nodes, hw.num_gpus_per_node, False)
+    Gs = Gs or _get_grad_accumu_steps_candidates(cfg.training.global_batch_size)
+    return IntraStageTuner(
+        tables, cfg.model.num_hidden_layers, meshes, Gs, tp, cfg, sample_size=S, sample_slots=slots
+    )
+
+
+def _oracle(cfg, tables, tp, S, meshes, Gs):
+    from oracle.intra import intra_stage_tune
+
+    return intra_stage_tune(tables, cfg, cfg.model.num_hidden_layers, meshes, Gs, tp, S)
+
+
+def _compare(cfg, tables, tp, S=1, slots=None):
+    tuner = _gpu_tuner(cfg, tables, tp, S=S, slots=slots)
+    got = tuner.tune()
+    want = _oracle(cfg, tables, tp, S, tuner.device_mesh_candidates,
+                   tuner.gradient_accumulation_steps_candidates)
+    slots = list(range(S)) if slots is None else list(slots)
+    names = ["", "_with_pre", "_with_post", "_no_pp"]
+    n_finite = 0
+    for v, suffix in enumerate(names):
+        gi = getattr(got, "indices" + suffix)[..., slots]
+        wi = getattr(want, "indices" + suffix)[..., slots]
+        assert np.array_equal(gi, wi), (
+            f"indices{suffix}: {np.sum(gi != wi)} of {gi.size} differ, first at "
+            f"{tuple(np.argwhere(gi != wi)[0])}"
+        )
+        for kind in ("stable", "delta"):
+            g32 = getattr(got, f"costs_{kind}{suffix}")[..., slots]
+            w32 = getattr(want, f"costs_{kind}{suffix}")[..., slots]
+            assert g32.dtype == np.float32 and w32.dtype == np.float32
+            assert_same_f64(g32, w32, f"costs_{kind}{suffix}")
+        gs = getattr(got, "solutions" + suffix)[..., slots, :]
+        ws = getattr(want, "solutions" + suffix)[..., slots, :]
+        assert_same_f64(gs, ws, f"solutions{suffix}")
+        n_finite += int(np.isfinite(getattr(got, "costs_stable" + suffix)).sum())
+    assert n_finite > 0, "degenerate case: nothing feasible anywhere"
+    return got, want
+
+
+def test_row_terms_bit_exact():
+    """Kernel 1 against the oracle's row-invariant arrays, every (G, mesh) group of plan 1."""
+    import torch
+
+    from mist_amd import _lib
+    from oracle.stage import batched_tune_best_latency_for_stage
+
+    for tp in (1, 2):
+        cfg, tables = load_plan(1)
+        tuner = _gpu_tuner(cfg, tables, tp)
+        plan = tuner.prepare()
+        dev = tuner.upload(plan)
+        lib = _lib.load()
+        rc = lib.mist_row_terms(
+            ctypes.c_void_p(plan["problem"].ctypes.data), dev["groups"].data_ptr(), dev["n_groups"],
+            dev["terms_prefix"].data_ptr(), dev["n_terms_blocks"], dev["row_terms"].data_ptr(),
+            ctypes.c_void_p(torch.cuda.current_stream().cuda_stream),
+        )
+        _lib.check(rc, "mist_row_terms")
+        torch.cuda.synchronize()
+        terms = dev["row_terms"].cpu().numpy().reshape(-1, _lib.ROW_TERMS)
+        L = cfg.model.num_hidden_layers
+        assert len(plan["groups"]) > 0
+        for rec in plan["groups"]:
+            dbg = {}
+            batched_tune_best_latency_for_stage(
+                tables, cfg, [0], list(range(1, L + 1)), [0, 1], int(rec["num_nodes"]),
+                int(rec["num_gpus_per_node"]), int(rec["grad_accum"]), tp_size=tp, sample_size=1,
+                debug=dbg,
+            )
+            n = int(rec["n_rows"])
+            assert dbg["rows"].shape[0] == n
+            want = oracle_terms(dbg, n)
+            got = terms[int(rec["row_offset"]): int(rec["row_offset"]) + n]
+            for j, name in enumerate(_lib.TERM_NAMES):
+                assert_same_f64(got[:, j], want[:, j], f"tp={tp} G={rec['grad_accum']} term {name}")
+
+
+@pytest.mark.parametrize("tp", [1, 2])
+def test_plan1_tables_match_oracle(tp):
+    """Plan 1 (GPT-1.3B, 1x2, B=8) complete, S = 1."""
+    cfg, tables = load_plan(1)
+    _compare(cfg, tables, tp)
+
+
+@pytest.mark.parametrize(
+    "overrides",
+    [
+        dict(),
+        dict(model__use_flash_attn=True),
+        dict(tuning__pre_post_strategy="intra-node-tp-with-ore"),
+        dict(tuning__pre_post_strategy="intra-node-tp-without-ore"),
+        dict(enable_advanced_opt_in_first_block=False),
+        dict(hardware__memory_capacity=6.0),
+        dict(hardware__memory_capacity=3.0, training__global_batch_size=16),
+        dict(hardware__num_nodes=2, hardware__num_gpus_per_node=4, training__global_batch_size=32,
+             hardware__memory_capacity=8.0),
+    ],
+)
+def test_tiny_variants_match_oracle(overrides):
+    cfg, tables = tiny_plan(1, layers=6, **overrides)
+    from mist_amd.config import tp_candidates
+
+    for tp in tp_candidates(cfg):
+        _compare(cfg, tables, tp)
+
+
+def test_multi_sample_matches_oracle():
+    """S = 4 alpha samples (unfused r*x + y on both sides)."""
+    cfg, tables = tiny_plan(1, layers=5, hardware__memory_capacity=6.0)
+    _compare(cfg, tables, 1, S=4)
+
+
+def test_sample_subset():
+    """Only slot 0 of S = 30 (what the uniform inter-stage search consumes)."""
+    cfg, tables = tiny_plan(1, layers=5)
+    _compare(cfg, tables, 1, S=30, slots=[0])

@@ -1,0 +1,72 @@
+/*
+ * C ABI of the inter-stage pipeline-partition DP (part of libmist_search.so).
+ * Conventions as in mist_search.h: `d_*` pointers are caller-owned DEVICE memory, small structs
+ * are HOST memory copied into kernel arguments, `stream` is a hipStream_t passed as void*,
+ * return 0 / negative MIST_E_* with mist_last_error().
+ */
+#ifndef MIST_DP_H
+#define MIST_DP_H
+
+#include <stdint.h>
+
+#include "mist_search.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Shape of one DP instance family (reference: inter_stage_tune_dp_impl,
+ * mist/analyzer/inter_tuning.py:220-355). */
+typedef struct MistDpShape {
+  int32_t num_layers;   /* L */
+  int32_t num_devices;  /* D */
+  int32_t num_mesh;     /* Q <= MIST_MAX_MESH, in candidate-list order */
+  int32_t p_dim;        /* P+1: extent of the pre-saved-micro-batch axis of the cost tables */
+  int32_t max_stages;   /* S_max = min(max(n*m), L) // 2 */
+  int32_t reserved[3];
+  int32_t mesh_n[MIST_MAX_MESH], mesh_m[MIST_MAX_MESH];
+} MistDpShape;
+
+/* float32 stage-cost tables for one gradient-accumulation candidate, C-contiguous:
+ *   costs, costs_pre : [Q][p_dim][L][L+1]    costs_post : [Q][L][L+1]    costs_nopp : [Q][L+1] */
+typedef struct MistDpCosts {
+  const float *costs, *costs_pre, *costs_post, *costs_nopp;
+} MistDpCosts;
+
+int mist_sizeof_dp_shape(void);
+
+/* Builds the float32 DP cost tables of every gradient-accumulation candidate from the float64
+ * stable / delta tables of the intra-stage search at sample position `slot`:
+ *   cost = (float)stable + (float)delta / (float)G          (float32 arithmetic)
+ * This is the combination the reference's uniform search applies (mist/analyzer/
+ * inter_tuning_uniform.py:300-316); the reference's DP expects it precomputed in fields its
+ * intra tuner no longer emits (mist/analyzer/inter_tuning.py:75-92).
+ * d_grad_accum[num_grad_accum]: G per g index.  d_out[v]: variant v table for all g, i.e. the
+ * layouts of MistOutTables without the trailing sample axis. */
+int mist_dp_cost_tables(const MistProblem *problem, const MistOutTables *tables,
+                        const int32_t *d_grad_accum, int slot, float *const d_out[4],
+                        void *stream);
+
+/* Host helper: applies the reference's gap rule (inter_tuning.py:198: skip t when
+ * t - last_run < 1e-6, float32 difference compared in float64) to an ascending list of
+ * candidate t_max values; writes the kept values to out and returns their count. */
+int mist_dp_filter_tmax(const float *sorted_unique, int n, double gap, float *out);
+
+/* Runs the DP for n_tmax thresholds in one launch (one workgroup per threshold):
+ *   F(s,k,d) = min over mesh q (n*m <= d), end layer i >= k, ckpt j in 0..L-i of
+ *              cost(s,k,i,q,j) + F(s-1,i+1,d-n*m)   subject to cost <= t_max,
+ * float32 adds, strict "<" in the reference's (q, i, j) order.  Outputs per threshold:
+ * d_best_s (-1 = infeasible), d_best_sum = F(best_s,0,D), d_stage_max = running max of the
+ * chosen stage costs.  d_argmin (may be NULL; needs n_tmax == 1):
+ * [max_stages+1][L+1][D+1][4] int32 = (end layer, n, m, ckpt), -1 where unset.
+ * d_scratch: 4 * n_tmax * (L+1) * (D+1) floats, used only when the state does not fit in LDS
+ * (may be NULL when mist_dp_scratch_floats() returns 0). */
+int64_t mist_dp_scratch_floats(const MistDpShape *shape, int n_tmax);
+int mist_dp_run(const MistDpShape *shape, const MistDpCosts *costs, const float *d_tmax,
+                int n_tmax, int32_t *d_best_s, float *d_best_sum, float *d_stage_max,
+                int32_t *d_argmin, float *d_scratch, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MIST_DP_H */

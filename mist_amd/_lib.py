@@ -124,7 +124,38 @@ def exported_symbols():
     return tuple(_SIGNATURES) + tuple(_DP_SIGNATURES)
 
 
-_DP_SIGNATURES = {}
+DP_SHAPE_DTYPE = np.dtype(
+    [
+        ("num_layers", "<i4"), ("num_devices", "<i4"), ("num_mesh", "<i4"), ("p_dim", "<i4"),
+        ("max_stages", "<i4"), ("reserved", "<i4", (3,)),
+        ("mesh_n", "<i4", (MAX_MESH,)), ("mesh_m", "<i4", (MAX_MESH,)),
+    ],
+    align=True,
+)
+
+
+class DpCosts(ctypes.Structure):
+    _fields_ = [
+        ("costs", ctypes.c_void_p),
+        ("costs_pre", ctypes.c_void_p),
+        ("costs_post", ctypes.c_void_p),
+        ("costs_nopp", ctypes.c_void_p),
+    ]
+
+
+_DP_SIGNATURES = {
+    "mist_sizeof_dp_shape": (ctypes.c_int, []),
+    "mist_dp_cost_tables": (
+        ctypes.c_int,
+        [_VP, ctypes.POINTER(OutTables), _VP, ctypes.c_int, ctypes.c_void_p * 4, _VP],
+    ),
+    "mist_dp_filter_tmax": (ctypes.c_int, [_VP, ctypes.c_int, ctypes.c_double, _VP]),
+    "mist_dp_scratch_floats": (ctypes.c_int64, [_VP, ctypes.c_int]),
+    "mist_dp_run": (
+        ctypes.c_int,
+        [_VP, ctypes.POINTER(DpCosts), _VP, ctypes.c_int, _VP, _VP, _VP, _VP, _VP, _VP],
+    ),
+}
 
 
 def load():
@@ -145,6 +176,10 @@ def load():
     if lib.mist_sizeof_problem() != PROBLEM_DTYPE.itemsize:
         raise MistLibraryError(
             f"MistProblem layout mismatch: C {lib.mist_sizeof_problem()} vs numpy {PROBLEM_DTYPE.itemsize}"
+        )
+    if lib.mist_sizeof_dp_shape() != DP_SHAPE_DTYPE.itemsize:
+        raise MistLibraryError(
+            f"MistDpShape layout mismatch: C {lib.mist_sizeof_dp_shape()} vs numpy {DP_SHAPE_DTYPE.itemsize}"
         )
     if lib.mist_sizeof_group() != GROUP_DTYPE.itemsize:
         raise MistLibraryError(

@@ -12,12 +12,14 @@
 #include <cstdio>
 #include <cstring>
 
+#include "mist_common.h"
 #include "mist_search.h"
 
 namespace {
-
 thread_local char g_last_error[512] = "";
+}  // namespace
 
+namespace mist {
 int fail(int code, const char *fmt, ...) {
   va_list ap;
   va_start(ap, fmt);
@@ -25,13 +27,11 @@ int fail(int code, const char *fmt, ...) {
   va_end(ap);
   return code;
 }
+}  // namespace mist
 
-#define MIST_HIP_CHECK(expr)                                                              \
-  do {                                                                                    \
-    hipError_t err__ = (expr);                                                            \
-    if (err__ != hipSuccess)                                                              \
-      return fail(MIST_E_HIP, "%s failed: %s", #expr, hipGetErrorString(err__));          \
-  } while (0)
+namespace {
+
+using mist::fail;
 
 constexpr int kTermsBlock = 256;  // rows per workgroup of the row-term kernel
 constexpr int kStageRows = 32;    // rows staged through LDS per step of the reduce kernel

@@ -1,0 +1,211 @@
+"""``tune_one_case``: resolved tuning YAML in, best strategy out.
+
+Drop-in for the reference's ``benchmark/mist/tune/tune_one_case.py`` (``tune`` :104-415,
+``best_solution_yaml`` :62-101, ``main`` :418-451) for the configuration-search path, with the
+evaluation running on the GPU.  Differences, all forced by what the path needs here:
+
+* the three traced ``LayerInfo`` objects are replaced by ``LayerTables`` (closed-form tables);
+* hydra / omegaconf are not used: ``main`` takes ``--config <yaml>`` plus ``key=value``
+  overrides, and the YAML written is produced with PyYAML;
+* ``tuning_granularity``: ``inter-stage`` (the DP), ``uniform-pp``,
+  ``uniform-pp-simple-heuristic-mem-opt`` and ``no-pp`` are implemented.  The reference's
+  ``inter-stage`` and ``no-pp`` branches call ``intra_stage_tune`` without the required
+  ``tp_size`` and read cost fields that no longer exist; here they loop the tensor-parallel
+  candidates like the working branches (:199-203) and use the stable/delta adapter.
+  ``uniform-device-pp`` and ``uniform-device-pp-mip`` (external MILP solver) raise
+  ``NotImplementedError``.
+"""
+from __future__ import annotations
+
+import argparse
+import copy
+import json
+import os
+import time
+from pprint import pformat
+from typing import Any, Dict, List, Optional
+
+import numpy as np
+import yaml
+
+from .config import OFFLOADING_RATIO_CANDIDATES, MistConfig, tp_candidates
+from .inter_tuning import inter_stage_tune
+from .inter_tuning_uniform import inter_stage_tune as inter_stage_tune_uniform
+from .intra_tuning import SAMPLE_SIZE, intra_stage_tune
+from .layer_tables import LayerTables
+from .search_space import _get_device_mesh_candidates, _get_grad_accumu_steps_candidates
+
+
+def best_solution_yaml(cfg: Dict[str, Any], best_solution: List[Any]) -> str:
+    """tune_one_case.py:62-101 on a plain dict: fills the ``strategy`` block."""
+    assert len(best_solution) == 2, f"len(best_solution)={len(best_solution)}. best_solution={best_solution}."
+    gradient_accumulation_steps, stage_solutions = best_solution
+    layer_partitions, device_assignment, gradient_checkpointing, stage_strategies = [], [], [], []
+    for stage_solution in stage_solutions:
+        (layer_partition, device_mesh, num_ckpt, _policy_index), stage_strategy = stage_solution
+        layer_start, layer_end = layer_partition
+        layer_partitions.append(int(layer_end - layer_start + 1))
+        device_assignment.append([int(x) for x in device_mesh])
+        gradient_checkpointing.append(int(num_ckpt))
+        stage_strategies.append([int(x) for x in stage_strategy[:6]] + [float(x) for x in stage_strategy[6:]])
+    pre_post_strategy_array = [None, None, None, 0, 0, 1, 0, 0, 0, 0]
+    pre_post_strategy_array[:3] = stage_strategies[-1][:3]
+    cfg = copy.deepcopy(cfg)
+    strategy = cfg.setdefault("strategy", {})
+    strategy["enabled"] = True
+    strategy["gradient_accumulation_steps"] = int(gradient_accumulation_steps)
+    strategy["layer_partitions"] = layer_partitions
+    strategy["device_assignment"] = device_assignment
+    strategy["gradient_checkpointing"] = gradient_checkpointing
+    strategy["stage_strategies"] = stage_strategies
+    strategy["pre_post_strategy"] = "preset"
+    strategy["pre_post_strategy_array"] = pre_post_strategy_array
+    return yaml.safe_dump(cfg, sort_keys=False)
+
+
+def _no_pp(mist_config, tables, device, stats):
+    """tune_one_case.py:123-184 with the tensor-parallel loop and the stable/delta adapter:
+    cost per (G, ckpt) = (float32(stable) + float32(delta) / G) * G, first minimum wins."""
+    hw, model, tuning = mist_config.hardware, mist_config.model, mist_config.tuning
+    meshes = [(hw.num_nodes, hw.num_gpus_per_node)]
+    Gs = _get_grad_accumu_steps_candidates(mist_config.training.global_batch_size)
+    L = model.num_hidden_layers
+    best_cost, best_solution = float("inf"), None
+    for tp_size in tp_candidates(mist_config):
+        r = intra_stage_tune(tables, L, meshes, Gs, tp_size, mist_config, sample_size=1, device=device)
+        with np.errstate(invalid="ignore"):
+            costs = r.costs_stable_no_pp[..., 0] + r.costs_delta_no_pp[..., 0] / np.array(
+                Gs, dtype=np.float32
+            ).reshape(-1, 1, 1)
+        solutions = r.solutions_no_pp[..., 0, :]
+        if not tuning.activation_checkpointing_tuning_enabled:
+            costs, solutions = costs[..., -1:], solutions[..., -1:, :]
+        costs = costs * np.array(Gs, dtype=np.float32).reshape(-1, 1, 1)
+        if not np.isfinite(costs).any():
+            continue
+        idx = np.unravel_index(np.argmin(costs), costs.shape)
+        if float(costs[idx]) < best_cost:
+            row = solutions[idx].tolist()
+            row[:6] = [int(x) for x in row[:6]]
+            ckpt = int(idx[2]) if tuning.activation_checkpointing_tuning_enabled else L
+            best_cost = float(costs[idx])
+            best_solution = [Gs[idx[0]], [(((0, L - 1), meshes[idx[1]], ckpt, 0), tuple(row))]]
+    return best_cost, best_solution
+
+
+def tune(mist_config: MistConfig, device: str = "cuda:0", stats: Optional[dict] = None):
+    """tune_one_case.py:104-415.  Returns ``(best_cost, best_solution)`` with
+    ``best_solution = [G, [(((l0, l1), (n, m), ckpt, policy), (b, dp, tp, wre, gre, ore, wo, go,
+    oo, ao)), ...per stage]]``."""
+    model, hw, tuning = mist_config.model, mist_config.hardware, mist_config.tuning
+    if tuning is None:
+        raise ValueError("the tuning block is missing or disabled")
+    tables = LayerTables(mist_config)
+    granularity = tuning.tuning_granularity
+    stats = {} if stats is None else stats
+    t_start = time.perf_counter()
+
+    if granularity == "no-pp":
+        best_cost, best_solution = _no_pp(mist_config, tables, device, stats)
+    elif granularity in ("uniform-pp", "uniform-pp-simple-heuristic-mem-opt", "inter-stage"):
+        meshes = _get_device_mesh_candidates(hw.num_nodes, hw.num_gpus_per_node, contiguous_inter_node=False)
+        Gs = _get_grad_accumu_steps_candidates(mist_config.training.global_batch_size)
+        L = model.num_hidden_layers
+        best_cost, best_solution = float("inf"), None
+        if granularity == "uniform-pp-simple-heuristic-mem-opt":
+            sweeps = list(OFFLOADING_RATIO_CANDIDATES)  # tune_one_case.py:258-262
+        else:
+            sweeps = [None]
+        for oo_ratio in sweeps:
+            if oo_ratio is not None:
+                mist_config._original_config["fixed_oo_ratio"] = oo_ratio
+                mist_config.tuning.activation_offloading_enabled = False
+            for tp_size in tp_candidates(mist_config):
+                t0 = time.perf_counter()
+                if granularity == "inter-stage":
+                    r = intra_stage_tune(tables, L, meshes, Gs, tp_size, mist_config,
+                                         sample_size=tuning.sample_size, sample_slots=[0], device=device)
+                    t1 = time.perf_counter()
+                    cost, solution = inter_stage_tune(
+                        L, hw.num_nodes * hw.num_gpus_per_node, meshes, Gs, r, slot=0, stats=stats
+                    )
+                else:
+                    # The reference does not forward tuning.sample_size here (:206-217): the
+                    # default of 30 applies and the uniform search reads sample 0 only.
+                    r = intra_stage_tune(tables, L, meshes, Gs, tp_size, mist_config,
+                                         sample_size=SAMPLE_SIZE, sample_slots=[0], device=device)
+                    t1 = time.perf_counter()
+                    cost, solution = inter_stage_tune_uniform(
+                        L, hw.num_nodes, hw.num_gpus_per_node, Gs, r, mist_config
+                    )
+                t2 = time.perf_counter()
+                stats["intra_s"] = stats.get("intra_s", 0.0) + (t1 - t0)
+                stats["inter_s"] = stats.get("inter_s", 0.0) + (t2 - t1)
+                if cost < best_cost:
+                    best_cost, best_solution = cost, solution
+    elif granularity in ("uniform-device-pp", "uniform-device-pp-mip"):
+        raise NotImplementedError(
+            f"tuning_granularity '{granularity}' is not part of the GPU search path "
+            "(uniform-device DP / external MILP solver)"
+        )
+    else:
+        raise ValueError(f"Unknown tuning granularity: {granularity}")
+    stats["tune_s"] = time.perf_counter() - t_start
+    return best_cost, best_solution
+
+
+def _apply_override(raw: Dict[str, Any], item: str) -> None:
+    key, _, value = item.partition("=")
+    node = raw
+    parts = key.split(".")
+    for p in parts[:-1]:
+        node = node.setdefault(p, {})
+    node[parts[-1]] = yaml.safe_load(value)
+
+
+def main(argv: Optional[List[str]] = None) -> None:
+    """tune_one_case.py:418-451: tunes, writes ``<output_path>.yaml`` and ``summary.json``."""
+    parser = argparse.ArgumentParser(description=__doc__.splitlines()[0])
+    parser.add_argument("--config", required=True, help="resolved tuning YAML")
+    parser.add_argument("--device", default="cuda:0")
+    parser.add_argument("overrides", nargs="*", help="key.path=value overrides, e.g. output_path=out/x")
+    args = parser.parse_args(argv)
+    with open(args.config) as f:
+        raw = yaml.safe_load(f)
+    for item in args.overrides:
+        _apply_override(raw, item)
+    raw.setdefault("strategy", {})["enabled"] = False
+    raw.setdefault("tuning", {})["enabled"] = True
+    mist_config = MistConfig(raw)
+    stats: Dict[str, Any] = {}
+    best_cost, best_solution = tune(mist_config, device=args.device, stats=stats)
+    print(f"Best cost: {best_cost}")
+    print(f"Best solution: {pformat(best_solution)}")
+    print(f"Tuning time: {stats.get('tune_s', 0.0):.3f} s")
+    if best_solution is None:
+        raise SystemExit("no feasible strategy found")
+    text = best_solution_yaml(raw, best_solution)
+    output_path = raw.get("output_path")
+    if output_path is not None:
+        folder = os.path.dirname(output_path) or "."
+        os.makedirs(folder, exist_ok=True)
+        if not output_path.endswith(".yaml"):
+            output_path += ".yaml"
+        name = os.path.basename(output_path).split(".")[0]
+        with open(output_path, "w") as f:
+            f.write(text)
+        summary_path = os.path.join(folder, "summary.json")
+        data = {}
+        if os.path.exists(summary_path):
+            with open(summary_path) as f:
+                data = json.load(f)
+        data.setdefault(name, {}).update(
+            {"tuning_best_cost": f"{best_cost:.4f}", "tuning_best_solution": pformat(best_solution)}
+        )
+        with open(summary_path, "w") as f:
+            json.dump(data, f, indent=2)
+        print(f"Saved the best solution to {output_path}")
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,125 @@
+"""GPU parity of the inter-stage DP and of the end-to-end tuner against the oracle."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from tests.util import tiny_plan, load_plan
+
+pytestmark = pytest.mark.gpu
+
+
+def _random_tables(rng, Q, P1, L, inf_frac=0.2, quantum=None):
+    def rand(shape):
+        a = rng.uniform(0.1, 1.0, size=shape).astype(np.float32)
+        if quantum:
+            a = (np.round(a / quantum) * quantum).astype(np.float32)  # many exact ties
+        a[rng.random(shape) < inf_frac] = np.inf
+        return a
+    return rand((Q, P1, L, L + 1)), rand((Q, P1, L, L + 1)), rand((Q, L, L + 1)), rand((Q, L + 1))
+
+
+def _gpu_dp(meshes, L, D, P1, tabs, tmax, want_argmin=False):
+    import torch
+    from mist_amd import _lib
+
+    lib = _lib.load()
+    Q = len(meshes)
+    shape = np.zeros(1, dtype=_lib.DP_SHAPE_DTYPE)
+    shape["num_layers"], shape["num_devices"], shape["num_mesh"], shape["p_dim"] = L, D, Q, P1
+    S = min(max(n * m for n, m in meshes), L) // 2
+    shape["max_stages"] = S
+    shape["mesh_n"][0, :Q] = [n for n, _ in meshes]
+    shape["mesh_m"][0, :Q] = [m for _, m in meshes]
+    dev = [torch.from_numpy(t).cuda() for t in tabs]
+    costs = _lib.DpCosts(*[t.data_ptr() for t in dev])
+    n = len(tmax)
+    d_t = torch.tensor(tmax, dtype=torch.float32).cuda()
+    d_s = torch.empty(n, dtype=torch.int32).cuda()
+    d_sum = torch.empty(n, dtype=torch.float32).cuda()
+    d_max = torch.empty(n, dtype=torch.float32).cuda()
+    n_scr = lib.mist_dp_scratch_floats(ctypes.c_void_p(shape.ctypes.data), n)
+    scr = torch.empty(max(n_scr, 1), dtype=torch.float32).cuda()
+    arg = torch.full((S + 1, L + 1, D + 1, 4), -1, dtype=torch.int32).cuda() if want_argmin else None
+    rc = lib.mist_dp_run(
+        ctypes.c_void_p(shape.ctypes.data), ctypes.byref(costs), d_t.data_ptr(), n, d_s.data_ptr(),
+        d_sum.data_ptr(), d_max.data_ptr(), arg.data_ptr() if want_argmin else None,
+        scr.data_ptr() if n_scr else None, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream),
+    )
+    _lib.check(rc, "mist_dp_run")
+    torch.cuda.synchronize()
+    out = (d_s.cpu().numpy(), d_sum.cpu().numpy(), d_max.cpu().numpy())
+    return out + ((arg.cpu().numpy(),) if want_argmin else ())
+
+
+@pytest.mark.parametrize(
+    "L,D,meshes,P1,quantum",
+    [
+        (6, 4, [(1, 1), (1, 2), (1, 4)], 3, None),
+        (9, 8, [(1, 1), (1, 2), (1, 4), (2, 4)], 5, 0.125),
+        (12, 16, [(1, 1), (1, 2), (1, 4), (1, 8), (2, 8)], 7, 0.0625),
+        (40, 80, [(1, 1), (1, 2), (1, 4), (1, 8), (2, 8), (4, 8), (8, 8)], 21, 0.03125),  # global-scratch path
+    ],
+)
+def test_dp_kernel_matches_c_oracle(L, D, meshes, P1, quantum):
+    from oracle.dp_c import _load
+
+    rng = np.random.default_rng(L * 100 + D)
+    tabs = _random_tables(rng, len(meshes), P1, L, quantum=quantum)
+    tmax = np.sort(rng.uniform(0.1, 1.1, size=24)).astype(np.float32)
+    got_s, got_sum, got_max = _gpu_dp(meshes, L, D, P1, tabs, tmax)
+    lib = _load()
+    S = min(max(n * m for n, m in meshes), L) // 2
+    mesh_n = np.array([n for n, _ in meshes], dtype=np.int32)
+    mesh_m = np.array([m for _, m in meshes], dtype=np.int32)
+    ptr = lambda a: a.ctypes.data_as(ctypes.c_void_p)
+    n_feasible = 0
+    for i, t in enumerate(tmax):
+        bs, bsum, smax = ctypes.c_int(), ctypes.c_float(), ctypes.c_float()
+        arg = np.empty((S + 1, L + 1, D + 1, 4), dtype=np.int32)
+        assert lib.mist_oracle_dp(
+            ctypes.c_float(float(t)), L, D, len(meshes), ptr(mesh_n), ptr(mesh_m), P1, ptr(tabs[0]),
+            ptr(tabs[1]), ptr(tabs[2]), ptr(tabs[3]), ctypes.byref(bs), ctypes.byref(bsum),
+            ctypes.byref(smax), ptr(arg)) == 0
+        assert got_s[i] == bs.value, (i, t)
+        if bs.value >= 0:
+            n_feasible += 1
+            assert got_sum[i] == np.float32(bsum.value) and got_max[i] == np.float32(smax.value), (i, t)
+            g = _gpu_dp(meshes, L, D, P1, tabs, [t], want_argmin=True)
+            assert np.array_equal(g[3], arg), f"back-pointers differ at t={t}"
+    assert n_feasible > 0
+
+
+@pytest.mark.parametrize(
+    "overrides",
+    [
+        dict(hardware__num_nodes=2, hardware__num_gpus_per_node=4, training__global_batch_size=32,
+             hardware__memory_capacity=8.0),
+        dict(hardware__num_nodes=1, hardware__num_gpus_per_node=8, training__global_batch_size=16,
+             hardware__memory_capacity=5.0, model__use_flash_attn=True),
+        dict(hardware__num_nodes=2, hardware__num_gpus_per_node=4, training__global_batch_size=32,
+             hardware__memory_capacity=8.0, tuning__tuning_granularity="uniform-pp"),
+    ],
+)
+def test_tune_end_to_end_matches_oracle(overrides):
+    """YAML in, best strategy out: identical cost (bit for bit) and identical solution."""
+    from mist_amd.tune_one_case import tune
+    from oracle.tune import tune as oracle_tune
+
+    cfg, tables = tiny_plan(1, layers=8, **overrides)
+    got_cost, got_sol = tune(cfg)
+    want_cost, want_sol = oracle_tune(cfg, tables)
+    assert want_sol is not None, "degenerate case"
+    assert got_cost == want_cost
+    assert got_sol == want_sol
+
+
+def test_plan1_end_to_end():
+    from mist_amd.tune_one_case import tune
+    from oracle.tune import tune as oracle_tune
+
+    cfg, tables = load_plan(1)
+    got = tune(cfg)
+    want = oracle_tune(cfg, tables)
+    assert want[1] is not None
+    assert got == want

@@ -235,8 +235,10 @@ class IntraStageTuner:
             partial_index=torch.empty(max(n_reduce_blocks, 1) * _lib.SLOTS * _lib.LC_TILE, dtype=torch.int32, device=dev),
         )
 
-    def launch(self, plan, dev_plan, tables: DeviceTables) -> None:
-        """Enqueues the kernels for every requested sample on the current stream."""
+    def launch(self, plan, dev_plan, tables: DeviceTables, events: Optional[list] = None) -> None:
+        """Enqueues the kernels for every requested sample on the current stream.  With
+        ``events`` (a list) the three kernels are launched through their own entry points and
+        ``(name, start_event, end_event)`` triples recorded on that stream are appended."""
         if dev_plan["n_groups"] == 0:
             return
         lib = _lib.load()
@@ -244,16 +246,51 @@ class IntraStageTuner:
         ratios = alpha_ratios(self.sample_size)
         out = tables.as_struct()
         prob_ptr = ctypes.c_void_p(plan["problem"].ctypes.data)
+        d = dev_plan
         for i, slot in enumerate(self.sample_slots):
-            rc = lib.mist_intra_stage_eval(
-                prob_ptr, _ptr(dev_plan["groups"]), dev_plan["n_groups"],
-                _ptr(dev_plan["terms_prefix"]), dev_plan["n_terms_blocks"],
-                _ptr(dev_plan["reduce_prefix"]), dev_plan["n_reduce_blocks"],
-                _ptr(dev_plan["row_terms"]), _ptr(dev_plan["partial_cost"]),
-                _ptr(dev_plan["partial_index"]), float(ratios[slot]), int(slot),
-                1 if i == 0 else 0, ctypes.byref(out), stream,
-            )
-            _lib.check(rc, "mist_intra_stage_eval")
+            if events is None:
+                rc = lib.mist_intra_stage_eval(
+                    prob_ptr, _ptr(d["groups"]), d["n_groups"],
+                    _ptr(d["terms_prefix"]), d["n_terms_blocks"],
+                    _ptr(d["reduce_prefix"]), d["n_reduce_blocks"],
+                    _ptr(d["row_terms"]), _ptr(d["partial_cost"]),
+                    _ptr(d["partial_index"]), float(ratios[slot]), int(slot),
+                    1 if i == 0 else 0, ctypes.byref(out), stream,
+                )
+                _lib.check(rc, "mist_intra_stage_eval")
+                continue
+
+            def timed(name, call):
+                start = torch.cuda.Event(enable_timing=True)
+                end = torch.cuda.Event(enable_timing=True)
+                start.record()
+                _lib.check(call(), name)
+                end.record()
+                events.append((name, start, end))
+
+            if i == 0:
+                timed("row_terms", lambda: lib.mist_row_terms(
+                    prob_ptr, _ptr(d["groups"]), d["n_groups"], _ptr(d["terms_prefix"]),
+                    d["n_terms_blocks"], _ptr(d["row_terms"]), stream))
+            timed("eval_reduce", lambda: lib.mist_eval_reduce(
+                prob_ptr, _ptr(d["groups"]), d["n_groups"], _ptr(d["reduce_prefix"]),
+                d["n_reduce_blocks"], _ptr(d["row_terms"]), float(ratios[slot]),
+                _ptr(d["partial_cost"]), _ptr(d["partial_index"]), stream))
+            timed("finalize", lambda: lib.mist_finalize(
+                prob_ptr, _ptr(d["groups"]), d["n_groups"], _ptr(d["reduce_prefix"]),
+                _ptr(d["row_terms"]), _ptr(d["partial_cost"]), _ptr(d["partial_index"]), int(slot),
+                ctypes.byref(out), stream))
+
+    def run_prepared(self, plan, dev_plan) -> IntraStageTunerOutput:
+        """Device part only: fresh output tables + kernel launches for an uploaded plan."""
+        with torch.cuda.device(self.device):
+            tables = self.allocate_tables()
+            self.launch(plan, dev_plan, tables)
+        self.results = IntraStageTunerOutput(
+            self.gradient_accumulation_steps_candidates, self.device_mesh_candidates, tables,
+            plan["spaces"], self.sample_slots,
+        )
+        return self.results
 
     def tune(self) -> IntraStageTunerOutput:
         if self.device.type != "cuda" or not torch.cuda.is_available():

@@ -26,12 +26,13 @@ from pprint import pformat
 from typing import Any, Dict, List, Optional
 
 import numpy as np
+import torch
 import yaml
 
 from .config import OFFLOADING_RATIO_CANDIDATES, MistConfig, tp_candidates
 from .inter_tuning import inter_stage_tune
 from .inter_tuning_uniform import inter_stage_tune as inter_stage_tune_uniform
-from .intra_tuning import SAMPLE_SIZE, intra_stage_tune
+from .intra_tuning import SAMPLE_SIZE, IntraStageTuner, intra_stage_tune
 from .layer_tables import LayerTables
 from .search_space import _get_device_mesh_candidates, _get_grad_accumu_steps_candidates
 
@@ -93,56 +94,95 @@ def _no_pp(mist_config, tables, device, stats):
     return best_cost, best_solution
 
 
+class PreparedSearch:
+    """The host-side preparation of one ``tune`` call, separated from its execution: group
+    descriptors are built and uploaded once (``__init__``), ``run`` then only launches kernels
+    and the inter-stage search.  ``tune`` is ``PreparedSearch(config).run()``."""
+
+    def __init__(self, mist_config: MistConfig, device: str = "cuda:0"):
+        model, hw, tuning = mist_config.model, mist_config.hardware, mist_config.tuning
+        self.config = mist_config
+        self.granularity = tuning.tuning_granularity
+        if self.granularity not in ("uniform-pp", "uniform-pp-simple-heuristic-mem-opt", "inter-stage"):
+            raise ValueError(f"PreparedSearch does not cover '{self.granularity}'")
+        self.tables = LayerTables(mist_config)
+        self.meshes = _get_device_mesh_candidates(hw.num_nodes, hw.num_gpus_per_node, contiguous_inter_node=False)
+        self.Gs = _get_grad_accumu_steps_candidates(mist_config.training.global_batch_size)
+        self.L = model.num_hidden_layers
+        # The reference forwards tuning.sample_size only on its MIP branch; the uniform
+        # branch runs with the default of 30 and reads sample 0 (:206-217).
+        sample_size = tuning.sample_size if self.granularity == "inter-stage" else SAMPLE_SIZE
+        self.tuners = []
+        for tp_size in tp_candidates(mist_config):
+            tuner = IntraStageTuner(self.tables, self.L, self.meshes, self.Gs, tp_size, mist_config,
+                                    sample_size=sample_size, sample_slots=[0], device=device)
+            plan = tuner.prepare()
+            with torch.cuda.device(tuner.device):
+                dev_plan = tuner.upload(plan)
+            self.tuners.append((tuner, plan, dev_plan))
+
+    def counts(self) -> Dict[str, int]:
+        """Search-space sizes: strategy rows, candidates = rows * (L + 1), base-variant cells
+        = rows * sum_l (l + 1) * (#pre-saved micro-batch values), groups."""
+        L = self.L
+        pairs = L * (L + 1) // 2 + L
+        rows = cells = groups = 0
+        for _, plan, _ in self.tuners:
+            g = plan["groups"]
+            rows += int(g["n_rows"].sum())
+            cells += int((g["n_rows"] * g["num_p"]).sum()) * pairs
+            groups += len(g)
+        return dict(rows=rows, candidates=rows * (L + 1), cells=cells, groups=groups)
+
+    def run(self, stats: Optional[dict] = None):
+        stats = {} if stats is None else stats
+        hw = self.config.hardware
+        best_cost, best_solution = float("inf"), None
+        for tuner, plan, dev_plan in self.tuners:
+            t0 = time.perf_counter()
+            r = tuner.run_prepared(plan, dev_plan)
+            t1 = time.perf_counter()
+            if self.granularity == "inter-stage":
+                cost, solution = inter_stage_tune(
+                    self.L, hw.num_nodes * hw.num_gpus_per_node, self.meshes, self.Gs, r, slot=0, stats=stats
+                )
+            else:
+                cost, solution = inter_stage_tune_uniform(
+                    self.L, hw.num_nodes, hw.num_gpus_per_node, self.Gs, r, self.config
+                )
+            t2 = time.perf_counter()
+            stats["intra_launch_s"] = stats.get("intra_launch_s", 0.0) + (t1 - t0)
+            stats["inter_s"] = stats.get("inter_s", 0.0) + (t2 - t1)
+            if cost < best_cost:
+                best_cost, best_solution = cost, solution
+        return best_cost, best_solution
+
+
 def tune(mist_config: MistConfig, device: str = "cuda:0", stats: Optional[dict] = None):
     """tune_one_case.py:104-415.  Returns ``(best_cost, best_solution)`` with
     ``best_solution = [G, [(((l0, l1), (n, m), ckpt, policy), (b, dp, tp, wre, gre, ore, wo, go,
     oo, ao)), ...per stage]]``."""
-    model, hw, tuning = mist_config.model, mist_config.hardware, mist_config.tuning
+    tuning = mist_config.tuning
     if tuning is None:
         raise ValueError("the tuning block is missing or disabled")
-    tables = LayerTables(mist_config)
     granularity = tuning.tuning_granularity
     stats = {} if stats is None else stats
     t_start = time.perf_counter()
 
     if granularity == "no-pp":
-        best_cost, best_solution = _no_pp(mist_config, tables, device, stats)
-    elif granularity in ("uniform-pp", "uniform-pp-simple-heuristic-mem-opt", "inter-stage"):
-        meshes = _get_device_mesh_candidates(hw.num_nodes, hw.num_gpus_per_node, contiguous_inter_node=False)
-        Gs = _get_grad_accumu_steps_candidates(mist_config.training.global_batch_size)
-        L = model.num_hidden_layers
+        best_cost, best_solution = _no_pp(mist_config, LayerTables(mist_config), device, stats)
+    elif granularity in ("uniform-pp", "inter-stage"):
+        best_cost, best_solution = PreparedSearch(mist_config, device).run(stats)
+    elif granularity == "uniform-pp-simple-heuristic-mem-opt":
+        # tune_one_case.py:258-262: sweep a fixed optimizer-offload ratio, activation offload off.
         best_cost, best_solution = float("inf"), None
-        if granularity == "uniform-pp-simple-heuristic-mem-opt":
-            sweeps = list(OFFLOADING_RATIO_CANDIDATES)  # tune_one_case.py:258-262
-        else:
-            sweeps = [None]
-        for oo_ratio in sweeps:
-            if oo_ratio is not None:
-                mist_config._original_config["fixed_oo_ratio"] = oo_ratio
-                mist_config.tuning.activation_offloading_enabled = False
-            for tp_size in tp_candidates(mist_config):
-                t0 = time.perf_counter()
-                if granularity == "inter-stage":
-                    r = intra_stage_tune(tables, L, meshes, Gs, tp_size, mist_config,
-                                         sample_size=tuning.sample_size, sample_slots=[0], device=device)
-                    t1 = time.perf_counter()
-                    cost, solution = inter_stage_tune(
-                        L, hw.num_nodes * hw.num_gpus_per_node, meshes, Gs, r, slot=0, stats=stats
-                    )
-                else:
-                    # The reference does not forward tuning.sample_size here (:206-217): the
-                    # default of 30 applies and the uniform search reads sample 0 only.
-                    r = intra_stage_tune(tables, L, meshes, Gs, tp_size, mist_config,
-                                         sample_size=SAMPLE_SIZE, sample_slots=[0], device=device)
-                    t1 = time.perf_counter()
-                    cost, solution = inter_stage_tune_uniform(
-                        L, hw.num_nodes, hw.num_gpus_per_node, Gs, r, mist_config
-                    )
-                t2 = time.perf_counter()
-                stats["intra_s"] = stats.get("intra_s", 0.0) + (t1 - t0)
-                stats["inter_s"] = stats.get("inter_s", 0.0) + (t2 - t1)
-                if cost < best_cost:
-                    best_cost, best_solution = cost, solution
+        for oo_ratio in OFFLOADING_RATIO_CANDIDATES:
+            raw = mist_config.raw()
+            raw["fixed_oo_ratio"] = oo_ratio
+            raw["tuning"]["activation_offloading_enabled"] = False
+            cost, solution = PreparedSearch(MistConfig(raw), device).run(stats)
+            if cost < best_cost:
+                best_cost, best_solution = cost, solution
     elif granularity in ("uniform-device-pp", "uniform-device-pp-mip"):
         raise NotImplementedError(
             f"tuning_granularity '{granularity}' is not part of the GPU search path "

@@ -1,0 +1,230 @@
+"""CPU tests of the package's host side: configuration, kernel-input preparation (bit-exact
+against the oracle's own derivation), launch decomposition, output formatting, and the C ABI
+(library loads and exports every symbol the headers declare; no compute calls)."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import yaml
+
+from mist_amd import _lib
+from mist_amd.config import MistConfig, tp_candidates
+from mist_amd.intra_tuning import IntraStageTuner, alpha_ratios
+from mist_amd.search_space import _get_device_mesh_candidates, _get_grad_accumu_steps_candidates
+from mist_amd.stage_inputs import interference_factor_table, make_problem
+from oracle.interference import mask_factor_table
+from oracle.pareto import alpha_ratios as oracle_alpha_ratios
+from oracle.stage import batched_tune_best_latency_for_stage
+from tests.util import REPO, assert_same_f64, load_plan, load_raw, tiny_plan
+
+
+def test_config_surface():
+    cfg, _ = load_plan(2)
+    assert cfg.hardware.memory_capacity == 80.0 * 0.88
+    assert cfg.tuning.tuning_granularity == "inter-stage" and cfg.strategy is None
+    assert cfg.enable_advanced_opt_in_first_block is True
+    assert getattr(cfg, "fixed_wo_ratio", None) is None
+    with pytest.raises(AttributeError):
+        cfg.not_a_key
+    assert tp_candidates(cfg) == [1, 2, 4, 8]
+    cfg1, _ = load_plan(1, disable_tp_tuning=True)
+    assert tp_candidates(cfg1) == [1]
+    raw = load_raw(1)
+    raw["tuning"]["tuning_granularity"] = "bogus"
+    with pytest.raises(AssertionError):
+        MistConfig(raw)
+    raw = load_raw(1)
+    raw["hardware"]["interference_model_params"] = [1.0] * 27
+    with pytest.raises(AssertionError):
+        MistConfig(raw)
+    # defaults of the optional search-space block are the reference's module constants
+    raw = load_raw(1)
+    del raw["tuning"]["search_space"]
+    t = MistConfig(raw).tuning
+    assert t.batch_size_candidates == (1, 2, 4)
+    assert t.offloading_ratio_candidates == (0.0, 0.25, 0.375, 0.5, 0.625, 0.75, 0.875, 1.0)
+    assert t.sparse_offloading_ratio_candidates == (0.0, 0.25, 0.375, 0.5, 0.75, 1.0)
+    assert t.zero_flag_choices == ((0, 0, 1), (0, 1, 1), (1, 1, 1))
+
+
+def test_interference_table_and_ratios_match_oracle():
+    p = np.random.default_rng(0).uniform(1, 3, 28)
+    table = interference_factor_table(p)
+    bits = [0xF, 0x7, 0xB, 0xD, 0xE, 0x3, 0x5, 0x9, 0x6, 0xA, 0xC]  # kMaskBits of the kernel
+    for row, ((mask, factors), b) in enumerate(zip(mask_factor_table(p), bits)):
+        assert np.array_equal(table[row], factors)
+        assert sum(1 << j for j in range(4) if mask[j]) == b
+    for S in (1, 4, 30):
+        assert np.array_equal(alpha_ratios(S), oracle_alpha_ratios(S))
+    with pytest.raises(ValueError):
+        interference_factor_table(p[:20])
+
+
+@pytest.mark.parametrize("overrides,tp", [
+    (dict(), 1), (dict(), 2),
+    (dict(tuning__pre_post_strategy="intra-node-tp-with-ore", model__use_flash_attn=True), 2),
+    (dict(hardware__num_nodes=2, hardware__num_gpus_per_node=4, training__global_batch_size=64,
+          tuning__pre_post_strategy="intra-node-tp-without-ore"), 4),
+])
+def test_group_descriptors_bit_exact_against_oracle(overrides, tp):
+    """Every per-group scalar and per-(b, tp) table value that is handed to the kernels equals
+    what the oracle derives for the same group, bit for bit."""
+    cfg, tables = tiny_plan(1, layers=4, **overrides)
+    hw = cfg.hardware
+    meshes = _get_device_mesh_candidates(hw.num_nodes, hw.num_gpus_per_node, False)
+    Gs = _get_grad_accumu_steps_candidates(cfg.training.global_batch_size)
+    tuner = IntraStageTuner(tables, 4, meshes, Gs, tp, cfg, sample_size=1, device="cpu")
+    plan = tuner.prepare()
+    assert len(plan["groups"]) > 0
+    P = _lib.PAR
+    for rec in plan["groups"]:
+        n, m, G = int(rec["num_nodes"]), int(rec["num_gpus_per_node"]), int(rec["grad_accum"])
+        dbg = {}
+        batched_tune_best_latency_for_stage(tables, cfg, [0], [1, 2, 3, 4], [0, 1, 2, 3, 4], n, m, G,
+                                            tp_size=tp, sample_size=1, debug=dbg)
+        rows = dbg["rows"]
+        assert rows.shape[0] == rec["n_rows"]
+        space = plan["spaces"][(int(rec["g_index"]), int(rec["q_index"]))]
+        assert np.array_equal(space.materialize(), rows)
+        first = np.arange(0, rows.shape[0], int(rec["n_off"]))  # first row of every parallelism block
+        par = rec["par"][: int(rec["n_par"])]
+        assert np.array_equal(par[:, :6], rows[first, :6])
+        bc = lambda a: np.broadcast_to(np.asarray(a, dtype=np.float64), (rows.shape[0],))[first]
+        for name, key in [("exec_fwd", "exec_fwd"), ("exec_bwd", "exec_bwd_nock"), ("extra_fwd", "extra_fwd"),
+                          ("extra_bwd", "extra_bwd"), ("fwd_peak", "fwd_peak_nock"), ("bwd_peak", "bwd_peak"),
+                          ("out", "out"), ("gcb", "gcb")]:
+            assert_same_f64(par[:, P[name]], bc(dbg[key]), name)
+        # raw saved activations: S = raw * (1 - ao) with ao == 0 in the first row of each block
+        assert_same_f64(par[:, P["raw_ck"]], bc(dbg["S_ck"]), "raw_ck")
+        assert_same_f64(par[:, P["raw_nock"]], bc(dbg["S_nock"]), "raw_nock")
+        pre, post = dbg["pre"], dbg["post"]
+        for name, want in [
+            ("pre_full_w", pre["W"]), ("pre_full_g", pre["G"]), ("post_full_w", post["W"]),
+            ("post_full_g", post["G"]), ("pre_states", pre["states"]), ("pre_saved", pre["saved"]),
+            ("pre_states_and_saved", pre["states"] + pre["saved"]), ("post_states", post["states"]),
+            ("post_fwd_peak", post["fwd_peak"]), ("post_bwd_peak", post["bwd_peak"]),
+            ("post_output", post["output"]), ("pre_fwd", pre["fwd"]), ("pre_bwd", pre["bwd"]),
+            ("post_fwd", post["fwd"]), ("post_bwd", post["bwd"]), ("pre_ag", pre["AG"]),
+            ("pre_rs", pre["RS"]), ("post_ag", post["AG"]), ("post_rs", post["RS"]),
+        ]:
+            assert_same_f64(np.array([rec[name]]), np.asarray(want, dtype=np.float64).reshape(1), name)
+    prob = plan["problem"][0]
+    assert prob["mem_cap_mb"] == cfg.hardware.memory_capacity * (1 << 30) / (1 << 20)
+    assert prob["num_layers"] == 4 and prob["sample_size"] == 1
+
+
+def test_launch_decomposition_covers_every_row_once():
+    cfg, tables = load_plan(2)
+    hw = cfg.hardware
+    meshes = _get_device_mesh_candidates(hw.num_nodes, hw.num_gpus_per_node, False)
+    Gs = _get_grad_accumu_steps_candidates(cfg.training.global_batch_size)
+    tuner = IntraStageTuner(tables, 32, meshes, Gs, 2, cfg, sample_size=1, device="cpu")
+    plan = tuner.prepare()
+    g = plan["groups"]
+    assert np.all(g["n_chunks"] * g["rows_per_chunk"] >= g["n_rows"])
+    assert np.all((g["n_chunks"] - 1) * g["rows_per_chunk"] < g["n_rows"])
+    assert np.all(g["rows_per_chunk"] % _lib.STAGE_ROWS == 0)
+    assert np.array_equal(g["row_offset"], np.concatenate(([0], np.cumsum(g["n_rows"])[:-1])))
+    assert np.all(g["n_p_tiles"] * _lib.P_TILE >= g["num_p"])
+    pairs = 32 * 33 // 2 + 32
+    assert np.all(g["n_lc_tiles"] * _lib.LC_TILE >= pairs)
+    blocks = np.diff(plan["reduce_prefix"])
+    assert np.array_equal(blocks, g["n_chunks"] * g["n_lc_tiles"] * g["n_p_tiles"])
+    assert np.array_equal(np.diff(plan["terms_prefix"]), -(-g["n_rows"] // _lib.TERMS_BLOCK))
+    assert tuner.max_possible_pre_saved_micro_batches == 31
+    assert plan["total_rows"] == int(g["n_rows"].sum()) == 913308
+
+
+def test_best_solution_yaml_format():
+    from mist_amd.tune_one_case import best_solution_yaml
+
+    raw = load_raw(1)
+    sol = [16, [(((0, 11), (1, 1), 5, 0), (2, 1, 1, 0, 0, 1, 0.0, 0.0, 0.0, 0.0)),
+                (((12, 23), (1, 1), 0, 0), (2, 1, 1, 0, 0, 1, 0.0, 0.0, 0.0, 0.0))]]
+    out = yaml.safe_load(best_solution_yaml(raw, sol))
+    s = out["strategy"]
+    assert s["enabled"] is True and s["gradient_accumulation_steps"] == 16
+    assert s["layer_partitions"] == [12, 12] and s["device_assignment"] == [[1, 1], [1, 1]]
+    assert s["gradient_checkpointing"] == [5, 0]
+    assert s["stage_strategies"] == [[2, 1, 1, 0, 0, 1, 0.0, 0.0, 0.0, 0.0]] * 2
+    assert s["pre_post_strategy"] == "preset"
+    assert s["pre_post_strategy_array"] == [2, 1, 1, 0, 0, 1, 0, 0, 0, 0]
+    assert out["model"] == raw["model"]
+
+
+def test_unsupported_granularities_raise():
+    from mist_amd.tune_one_case import tune
+
+    for gran in ("uniform-device-pp", "uniform-device-pp-mip"):
+        cfg, _ = load_plan(1, tuning__tuning_granularity=gran)
+        with pytest.raises(NotImplementedError):
+            tune(cfg)
+
+
+def _declared_functions():
+    names = []
+    for header in ("mist_search.h", "mist_dp.h"):
+        text = open(os.path.join(REPO, "include", header)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names += re.findall(r"\b(mist_[a-z0-9_]+)\s*\(", text)
+    return sorted(set(names))
+
+
+def test_library_loads_and_exports_every_declared_symbol():
+    lib = _lib.load()
+    declared = _declared_functions()
+    assert len(declared) >= 12
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared in include/ but not exported"
+    assert set(_lib.exported_symbols()) == set(declared)
+    assert lib.mist_sizeof_problem() == _lib.PROBLEM_DTYPE.itemsize
+    assert lib.mist_sizeof_group() == _lib.GROUP_DTYPE.itemsize
+    assert lib.mist_sizeof_dp_shape() == _lib.DP_SHAPE_DTYPE.itemsize
+    assert b"gfx950" in lib.mist_version()
+
+
+def test_argument_checks_reject_before_any_launch():
+    """Host-side validation paths of the C ABI (no GPU needed: they return before launching)."""
+    lib = _lib.load()
+    assert lib.mist_row_terms(None, None, 1, None, 1, None, None) == -1
+    assert b"null" in lib.mist_last_error()
+    prob = make_problem(load_plan(1)[0], 4, 2, 1, 4, 2)
+    pp = ctypes.c_void_p(prob.ctypes.data)
+    fake = ctypes.c_void_p(4096)
+    assert lib.mist_row_terms(pp, fake, 0, fake, 1, fake, None) == -1
+    assert lib.mist_eval_reduce(pp, fake, 1, fake, 0, fake, 1.0, fake, fake, None) == -1
+    assert lib.mist_eval_reduce(pp, fake, 1, fake, 1, fake, -1.0, fake, fake, None) == -1
+    tabs = _lib.OutTables()
+    assert lib.mist_finalize(pp, fake, 1, fake, fake, fake, fake, 0, ctypes.byref(tabs), None) == -1
+    shape = np.zeros(1, dtype=_lib.DP_SHAPE_DTYPE)
+    assert lib.mist_dp_scratch_floats(ctypes.c_void_p(shape.ctypes.data), 4) == -1
+    shape["num_layers"], shape["num_devices"], shape["num_mesh"], shape["p_dim"] = 8, 8, 2, 4
+    shape["max_stages"] = 4
+    shape["mesh_n"][0, :2], shape["mesh_m"][0, :2] = [1, 1], [1, 2]
+    assert lib.mist_dp_scratch_floats(ctypes.c_void_p(shape.ctypes.data), 4) == 0
+    shape["num_layers"], shape["num_devices"] = 80, 256
+    assert lib.mist_dp_scratch_floats(ctypes.c_void_p(shape.ctypes.data), 4) == 4 * 4 * 81 * 257
+    costs = _lib.DpCosts(4096, 4096, 4096, 4096)
+    sp = ctypes.c_void_p(shape.ctypes.data)
+    assert lib.mist_dp_run(sp, ctypes.byref(costs), fake, 2, fake, fake, fake, fake, None, None) == -1
+    assert b"argmin" in lib.mist_last_error()
+    assert lib.mist_dp_run(sp, ctypes.byref(costs), fake, 1, fake, fake, fake, None, None, None) == -1
+    assert b"scratch" in lib.mist_last_error()
+
+
+def test_gap_filter_matches_oracle_rule():
+    lib = _lib.load()
+    rng = np.random.default_rng(0)
+    t = np.unique(np.concatenate([rng.uniform(0.01, 2, 500), 0.5 + np.arange(40) * 3e-7]).astype(np.float32))
+    out = np.empty_like(t)
+    n = lib.mist_dp_filter_tmax(ctypes.c_void_p(t.ctypes.data), len(t), 1e-6, ctypes.c_void_p(out.ctypes.data))
+    want, last = [], np.float32(0)
+    for v in t:
+        if float(np.float32(v - last)) < 1e-6:
+            continue
+        want.append(v)
+        last = v
+    assert n == len(want) and np.array_equal(out[:n], np.array(want, dtype=np.float32))
+    assert 0 < n < len(t)

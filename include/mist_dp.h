@@ -27,11 +27,16 @@ typedef struct MistDpShape {
   int32_t mesh_n[MIST_MAX_MESH], mesh_m[MIST_MAX_MESH];
 } MistDpShape;
 
-/* float32 stage-cost tables for one gradient-accumulation candidate, C-contiguous:
- *   costs, costs_pre : [Q][p_dim][L][L+1]    costs_post : [Q][L][L+1]    costs_nopp : [Q][L+1] */
+/* float32 stage-cost tables of all gradient-accumulation candidates, C-contiguous per g:
+ *   costs, costs_pre : [g][Q][p_dim][L][L+1]   costs_post : [g][Q][L][L+1]   costs_nopp : [g][Q][L+1]
+ * g_stride[v] = elements between consecutive g of table v (costs, pre, post, nopp). */
 typedef struct MistDpCosts {
   const float *costs, *costs_pre, *costs_post, *costs_nopp;
+  int64_t g_stride[4];
 } MistDpCosts;
+
+#define MIST_DP_THRESHOLD 0  /* sum of stage costs subject to cost <= t_max */
+#define MIST_DP_BOTTLENECK 1 /* smallest achievable maximum stage cost; t_max is ignored */
 
 int mist_sizeof_dp_shape(void);
 
@@ -52,19 +57,26 @@ int mist_dp_cost_tables(const MistProblem *problem, const MistOutTables *tables,
  * candidate t_max values; writes the kept values to out and returns their count. */
 int mist_dp_filter_tmax(const float *sorted_unique, int n, double gap, float *out);
 
-/* Runs the DP for n_tmax thresholds in one launch (one workgroup per threshold):
+/* Runs n_tmax DP instances at once (max_stages launches, one thread per (instance, start
+ * layer, devices) state).  Instance t uses the cost tables of g = d_g_index[t].
+ * MIST_DP_THRESHOLD (reference: inter_stage_tune_dp_impl, inter_tuning.py:220-355):
  *   F(s,k,d) = min over mesh q (n*m <= d), end layer i >= k, ckpt j in 0..L-i of
- *              cost(s,k,i,q,j) + F(s-1,i+1,d-n*m)   subject to cost <= t_max,
- * float32 adds, strict "<" in the reference's (q, i, j) order.  Outputs per threshold:
- * d_best_s (-1 = infeasible), d_best_sum = F(best_s,0,D), d_stage_max = running max of the
- * chosen stage costs.  d_argmin (may be NULL; needs n_tmax == 1):
- * [max_stages+1][L+1][D+1][4] int32 = (end layer, n, m, ckpt), -1 where unset.
- * d_scratch: 4 * n_tmax * (L+1) * (D+1) floats, used only when the state does not fit in LDS
- * (may be NULL when mist_dp_scratch_floats() returns 0). */
+ *              cost(s,k,i,q,j) + F(s-1,i+1,d-n*m)   subject to cost <= d_tmax[t],
+ *   float32 adds, strict "<" in the reference's (q, i, j) order.  Outputs per instance:
+ *   d_best_s (-1 = infeasible), d_best_sum = F(best_s,0,D), d_stage_max = running max of the
+ *   chosen stage costs.
+ * MIST_DP_BOTTLENECK: same recurrence with max() in place of "+" and no threshold; d_best_sum
+ *   is the smallest threshold for which the instance is feasible (+inf if none).  The reference
+ *   finds that point by running the threshold DP for every smaller candidate, all of which
+ *   return "infeasible" and change nothing.
+ * d_argmin (may be NULL; needs n_tmax == 1): [max_stages+1][L+1][D+1][4] int32 =
+ *   (end layer, n, m, ckpt), pre-filled with -1 by the caller.
+ * d_scratch: mist_dp_scratch_floats() = 4 * n_tmax * (L+1) * (D+1) floats of state. */
 int64_t mist_dp_scratch_floats(const MistDpShape *shape, int n_tmax);
 int mist_dp_run(const MistDpShape *shape, const MistDpCosts *costs, const float *d_tmax,
-                int n_tmax, int32_t *d_best_s, float *d_best_sum, float *d_stage_max,
-                int32_t *d_argmin, float *d_scratch, void *stream);
+                const int32_t *d_g_index, int n_tmax, int mode, int32_t *d_best_s,
+                float *d_best_sum, float *d_stage_max, int32_t *d_argmin, float *d_scratch,
+                void *stream);
 
 #ifdef __cplusplus
 }

@@ -22,6 +22,7 @@ SLOTS = 2 * P_TILE + 2
 STAGE_ROWS = 32
 TERMS_BLOCK = 256
 MAX_MESH = 16
+DP_THRESHOLD, DP_BOTTLENECK = 0, 1
 
 PAR_NAMES = (
     "b", "dp", "tp", "wre", "gre", "ore", "W", "G", "O", "raw_ck", "raw_nock", "fwd_peak",
@@ -140,6 +141,7 @@ class DpCosts(ctypes.Structure):
         ("costs_pre", ctypes.c_void_p),
         ("costs_post", ctypes.c_void_p),
         ("costs_nopp", ctypes.c_void_p),
+        ("g_stride", ctypes.c_int64 * 4),
     ]
 
 
@@ -153,7 +155,7 @@ _DP_SIGNATURES = {
     "mist_dp_scratch_floats": (ctypes.c_int64, [_VP, ctypes.c_int]),
     "mist_dp_run": (
         ctypes.c_int,
-        [_VP, ctypes.POINTER(DpCosts), _VP, ctypes.c_int, _VP, _VP, _VP, _VP, _VP, _VP],
+        [_VP, ctypes.POINTER(DpCosts), _VP, _VP, ctypes.c_int, ctypes.c_int, _VP, _VP, _VP, _VP, _VP, _VP],
     ),
 }
 

@@ -1,12 +1,10 @@
 // Inter-stage pipeline-partition DP on MI355X (gfx950).
 //
-// One workgroup per t_max threshold.  The stage index s is the sequential (wavefront) axis;
-// the (start layer k, devices d) states of one s are independent and are spread over the
-// threads.  F(s-1, ., .) / F(s, ., .) and the running stage maxima live in LDS when they fit
-// (4 * (L+1) * (D+1) floats), otherwise in a caller-provided global scratch slab that stays in
-// L2.  Each thread walks its state's (mesh, end layer, ckpt) candidates in the reference's
-// order with float32 adds and strict "<", so ties resolve exactly as in the reference loop
-// nest (mist/analyzer/inter_tuning.py:298-333).
+// The stage index s is the sequential (wavefront) axis: one launch per s.  The (threshold,
+// start layer k, devices d) states of one s are independent and are spread over the whole GPU,
+// one thread each.  Each thread walks its state's (mesh, end layer, ckpt) candidates in the
+// reference's order with float32 adds and strict "<", so ties resolve exactly as in the
+// reference loop nest (mist/analyzer/inter_tuning.py:298-333).
 #include <hip/hip_runtime.h>
 
 #include <cmath>
@@ -19,8 +17,7 @@ namespace {
 
 using mist::fail;
 
-constexpr int kDpThreads = 512;
-constexpr int kLdsStateFloats = 12 * 1024;  // 48 KB of float32 state per workgroup
+constexpr int kDpThreads = 64;  // one wavefront per workgroup
 
 // ------------------------------------------------------------------------------------------
 // Adapter: float64 (stable, delta) tables -> float32 DP cost tables for every g.
@@ -40,105 +37,115 @@ __global__ __launch_bounds__(256) void cost_table_kernel(const double *__restric
 }
 
 // ------------------------------------------------------------------------------------------
-// DP kernel.
+// DP kernels.  The stage index s is the sequential axis: one launch per s.  Within a launch
+// every (threshold, start layer k, devices d) state is one thread; workgroups are single
+// wavefronts so that even a handful of thresholds spreads over many CUs.  F(s-1) / F(s) and
+// the running stage maxima ping-pong between two planes per threshold in a global scratch slab
+// (L2 resident: 4 * (L+1) * (D+1) floats per threshold).
 // ------------------------------------------------------------------------------------------
-template <bool kUseLds>
-__global__ __launch_bounds__(kDpThreads) void dp_kernel(
+__global__ __launch_bounds__(256) void dp_init_kernel(const MistDpShape shape, int n_tmax,
+                                                      float *__restrict__ scratch,
+                                                      int32_t *__restrict__ best_s,
+                                                      float *__restrict__ best_sum,
+                                                      float *__restrict__ stage_max) {
+  const int W = shape.num_devices + 1;
+  const int plane = (shape.num_layers + 1) * W;
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (int64_t)n_tmax * plane) return;
+  const int t = (int)(i / plane), e = (int)(i % plane);
+  float *state = scratch + (int64_t)t * 4 * plane;
+  // plane 0 holds F(0, ., .): 0 at (k = L, d = 0), +inf elsewhere; maxima start at 0.
+  state[e] = e == shape.num_layers * W ? 0.0f : INFINITY;
+  state[2 * plane + e] = 0.0f;
+  if (e == 0) {
+    best_s[t] = -1;
+    best_sum[t] = INFINITY;
+    stage_max[t] = 0.0f;
+  }
+}
+
+template <bool kBottleneck>
+__global__ __launch_bounds__(kDpThreads) void dp_step_kernel(
     const MistDpShape shape, const MistDpCosts tabs, const float *__restrict__ tmax_list,
-    int32_t *__restrict__ best_s_out, float *__restrict__ best_sum_out,
-    float *__restrict__ stage_max_out, int32_t *__restrict__ argmin, float *__restrict__ scratch) {
-  extern __shared__ float lds_state[];
+    const int32_t *__restrict__ g_list, int s, float *__restrict__ scratch,
+    int32_t *__restrict__ best_s_out,
+    float *__restrict__ best_sum_out, float *__restrict__ stage_max_out,
+    int32_t *__restrict__ argmin) {
   const int L = shape.num_layers, D = shape.num_devices, Q = shape.num_mesh;
-  const int P1 = shape.p_dim, S = shape.max_stages;
+  const int P1 = shape.p_dim;
   const int W = D + 1;            // row pitch of a state plane
   const int plane = (L + 1) * W;  // states per s
   const int C = L + 1;            // ckpt extent of the cost tables
-  float *state = kUseLds ? lds_state : scratch + (int64_t)blockIdx.x * 4 * plane;
-  float *f_prev = state, *f_cur = state + plane;
-  float *m_prev = state + 2 * plane, *m_cur = state + 3 * plane;
-  const float t_max = tmax_list[blockIdx.x];
+  const int e = blockIdx.x * kDpThreads + threadIdx.x;
+  if (e >= plane) return;
+  const int t = blockIdx.y;
+  float *state = scratch + (int64_t)t * 4 * plane;
+  const int cur = s & 1, prv = cur ^ 1;
+  const float *__restrict__ f_prev = state + prv * plane;
+  const float *__restrict__ m_prev = state + (2 + prv) * plane;
+  float *__restrict__ f_cur = state + cur * plane;
+  float *__restrict__ m_cur = state + (2 + cur) * plane;
+  const float t_max = kBottleneck ? INFINITY : tmax_list[t];
+  const int64_t g = g_list[t];
+  const float *__restrict__ tab_costs = tabs.costs + g * tabs.g_stride[0];
+  const float *__restrict__ tab_pre = tabs.costs_pre + g * tabs.g_stride[1];
+  const float *__restrict__ tab_post = tabs.costs_post + g * tabs.g_stride[2];
+  const float *__restrict__ tab_nopp = tabs.costs_nopp + g * tabs.g_stride[3];
+  const int k = e / W, d = e % W;
+  const int p = s - 1;
 
-  for (int i = threadIdx.x; i < plane; i += kDpThreads) {
-    f_prev[i] = INFINITY;
-    m_prev[i] = 0.0f;
-  }
-  __syncthreads();
-  if (threadIdx.x == 0) f_prev[L * W + 0] = 0.0f;  // F(0, L, 0) = 0
-  int best_s = -1;
-  float best_sum = INFINITY, best_max = 0.0f;
-  __syncthreads();
-
-  for (int s = 1; s <= S; ++s) {
-    const int p = s - 1;
-    // States of this step: k = 0..L-s, d = 1..D; everything else stays (inf, 0).
-    for (int i = threadIdx.x; i < plane; i += kDpThreads) {
-      f_cur[i] = INFINITY;
-      m_cur[i] = 0.0f;
-    }
-    __syncthreads();
-    const int n_states = (L - s + 1) * D;
-    for (int st = threadIdx.x; st < n_states; st += kDpThreads) {
-      // Largest loops (small k) first so that long states start early.
-      const int k = st / D, d = st % D + 1;
-      float best = INFINITY, best_m = 0.0f;
-      int arg_i = -1, arg_q = -1, arg_j = -1;
-      for (int q = 0; q < Q; ++q) {
-        const int nm = shape.mesh_n[q] * shape.mesh_m[q];
-        if (nm > d) continue;
-        for (int i = k; i < L; ++i) {
-          const int from = (i + 1) * W + (d - nm);
-          const float prev = f_prev[from];
-          const int l = i - k + 1;
-          const float *__restrict__ row;
-          if (k == 0 && i == L - 1) row = tabs.costs_nopp + (int64_t)q * C;
-          else if (k == 0) row = tabs.costs_pre + (((int64_t)q * P1 + p) * L + (l - 1)) * C;
-          else if (i == L - 1) row = tabs.costs_post + ((int64_t)q * L + (l - 1)) * C;
-          else row = tabs.costs + (((int64_t)q * P1 + p) * L + (l - 1)) * C;
-          // A state reachable only through an unreachable successor cannot improve: inf + c is
-          // never < best.  Skipping it changes nothing and saves the inner loop.
-          if (prev == INFINITY) continue;
-          const float prev_m = m_prev[from];
-          const int j_end = L - i;
-          for (int j = 0; j <= j_end; ++j) {
-            const float stage_cost = row[j];
-            const float new_cost = stage_cost + prev;
-            if (stage_cost <= t_max && new_cost < best) {
-              best = new_cost;
-              best_m = fmaxf(prev_m, stage_cost);
-              arg_i = i;
-              arg_q = q;
-              arg_j = j;
-            }
+  float best = INFINITY, best_m = 0.0f;
+  int arg_i = -1, arg_q = -1, arg_j = -1;
+  if (k <= L - s && d >= 1) {
+    for (int q = 0; q < Q; ++q) {
+      const int nm = shape.mesh_n[q] * shape.mesh_m[q];
+      if (nm > d) continue;
+      for (int i = k; i < L; ++i) {
+        const int from = (i + 1) * W + (d - nm);
+        const float prev = f_prev[from];
+        // A state reachable only through an unreachable successor cannot improve: inf + c is
+        // never < best.  Skipping it changes nothing and saves the inner loop.
+        if (prev == INFINITY) continue;
+        const int l = i - k + 1;
+        const float *__restrict__ row;
+        if (k == 0 && i == L - 1) row = tab_nopp + (int64_t)q * C;
+        else if (k == 0) row = tab_pre + (((int64_t)q * P1 + p) * L + (l - 1)) * C;
+        else if (i == L - 1) row = tab_post + ((int64_t)q * L + (l - 1)) * C;
+        else row = tab_costs + (((int64_t)q * P1 + p) * L + (l - 1)) * C;
+        const float prev_m = m_prev[from];
+        const int j_end = L - i;
+#pragma unroll 4
+        for (int j = 0; j <= j_end; ++j) {
+          const float stage_cost = row[j];
+          // Threshold mode: sum of stage costs under cost <= t_max.  Bottleneck mode: the
+          // smallest achievable maximum stage cost (comparisons only, no rounding).
+          const float new_cost = kBottleneck ? fmaxf(stage_cost, prev) : stage_cost + prev;
+          if (stage_cost <= t_max && new_cost < best) {
+            best = new_cost;
+            best_m = fmaxf(prev_m, stage_cost);
+            arg_i = i;
+            arg_q = q;
+            arg_j = j;
           }
         }
       }
-      f_cur[k * W + d] = best;
-      m_cur[k * W + d] = best_m;
-      if (argmin != nullptr && arg_i >= 0) {
-        int32_t *a = argmin + ((int64_t)s * plane + k * W + d) * 4;
-        a[0] = arg_i;
-        a[1] = shape.mesh_n[arg_q];
-        a[2] = shape.mesh_m[arg_q];
-        a[3] = arg_j;
-      }
     }
-    __syncthreads();
-    if (threadIdx.x == 0) {
-      const float v = f_cur[0 * W + D];
-      if (v < best_sum) {  // first s wins ties (inter_tuning.py:335-340)
-        best_sum = v;
-        best_s = s;
-        best_max = m_cur[0 * W + D];
-      }
-    }
-    float *t0 = f_prev; f_prev = f_cur; f_cur = t0;
-    float *t1 = m_prev; m_prev = m_cur; m_cur = t1;
-    __syncthreads();
   }
-  if (threadIdx.x == 0) {
-    best_s_out[blockIdx.x] = best_s;
-    best_sum_out[blockIdx.x] = best_sum;
-    stage_max_out[blockIdx.x] = best_max;
+  f_cur[e] = best;
+  m_cur[e] = best_m;
+  if (argmin != nullptr && arg_i >= 0) {
+    int32_t *a = argmin + ((int64_t)s * plane + e) * 4;
+    a[0] = arg_i;
+    a[1] = shape.mesh_n[arg_q];
+    a[2] = shape.mesh_m[arg_q];
+    a[3] = arg_j;
+  }
+  // The state (k = 0, d = D) is the answer of this stage count; first s wins ties
+  // (inter_tuning.py:335-340).  The same thread handles it in every launch.
+  if (k == 0 && d == D && best < best_sum_out[t]) {
+    best_sum_out[t] = best;
+    best_s_out[t] = s;
+    stage_max_out[t] = best_m;
   }
 }
 
@@ -159,11 +166,6 @@ int check_shape(const MistDpShape *shape) {
     if (shape->mesh_n[q] <= 0 || shape->mesh_m[q] <= 0)
       return fail(MIST_E_INVALID, "mesh %d is (%d, %d)", q, shape->mesh_n[q], shape->mesh_m[q]);
   return 0;
-}
-
-bool fits_lds(const MistDpShape *shape) {
-  const int64_t plane = (int64_t)(shape->num_layers + 1) * (shape->num_devices + 1);
-  return 4 * plane <= kLdsStateFloats;
 }
 
 }  // namespace
@@ -211,33 +213,43 @@ int mist_dp_filter_tmax(const float *sorted_unique, int n, double gap, float *ou
 
 int64_t mist_dp_scratch_floats(const MistDpShape *shape, int n_tmax) {
   if (check_shape(shape) != 0 || n_tmax <= 0) return -1;
-  if (fits_lds(shape)) return 0;
   return (int64_t)4 * n_tmax * (shape->num_layers + 1) * (shape->num_devices + 1);
 }
 
 int mist_dp_run(const MistDpShape *shape, const MistDpCosts *costs, const float *d_tmax,
-                int n_tmax, int32_t *d_best_s, float *d_best_sum, float *d_stage_max,
-                int32_t *d_argmin, float *d_scratch, void *stream) {
+                const int32_t *d_g_index, int n_tmax, int mode, int32_t *d_best_s,
+                float *d_best_sum, float *d_stage_max, int32_t *d_argmin, float *d_scratch,
+                void *stream) {
   if (int rc = check_shape(shape)) return rc;
   if (!costs || !costs->costs || !costs->costs_pre || !costs->costs_post || !costs->costs_nopp)
     return fail(MIST_E_INVALID, "null cost table");
-  if (!d_tmax || !d_best_s || !d_best_sum || !d_stage_max)
+  if (!d_tmax || !d_g_index || !d_best_s || !d_best_sum || !d_stage_max)
     return fail(MIST_E_INVALID, "null threshold / output pointer");
-  if (n_tmax <= 0) return fail(MIST_E_INVALID, "n_tmax must be positive, got %d", n_tmax);
+  if (!d_scratch) return fail(MIST_E_INVALID, "null scratch pointer");
+  if (n_tmax <= 0 || n_tmax > 65535)
+    return fail(MIST_E_INVALID, "n_tmax must be in [1, 65535], got %d", n_tmax);
+  if (mode != MIST_DP_THRESHOLD && mode != MIST_DP_BOTTLENECK)
+    return fail(MIST_E_INVALID, "unknown DP mode %d", mode);
   if (d_argmin && n_tmax != 1)
     return fail(MIST_E_INVALID, "argmin output needs n_tmax == 1, got %d", n_tmax);
   const int plane = (shape->num_layers + 1) * (shape->num_devices + 1);
-  if (fits_lds(shape)) {
-    hipLaunchKernelGGL(dp_kernel<true>, dim3(n_tmax), dim3(kDpThreads),
-                       4 * plane * sizeof(float), (hipStream_t)stream, *shape, *costs, d_tmax,
-                       d_best_s, d_best_sum, d_stage_max, d_argmin, (float *)nullptr);
-  } else {
-    if (!d_scratch) return fail(MIST_E_INVALID, "state does not fit in LDS: scratch is required");
-    hipLaunchKernelGGL(dp_kernel<false>, dim3(n_tmax), dim3(kDpThreads), 0, (hipStream_t)stream,
-                       *shape, *costs, d_tmax, d_best_s, d_best_sum, d_stage_max, d_argmin,
-                       d_scratch);
-  }
+  const int64_t n_init = (int64_t)n_tmax * plane;
+  hipLaunchKernelGGL(dp_init_kernel, dim3((unsigned)((n_init + 255) / 256)), dim3(256), 0,
+                     (hipStream_t)stream, *shape, n_tmax, d_scratch, d_best_s, d_best_sum,
+                     d_stage_max);
   MIST_HIP_CHECK(hipGetLastError());
+  const dim3 grid((plane + kDpThreads - 1) / kDpThreads, n_tmax);
+  for (int s = 1; s <= shape->max_stages; ++s) {
+    if (mode == MIST_DP_BOTTLENECK)
+      hipLaunchKernelGGL(dp_step_kernel<true>, grid, dim3(kDpThreads), 0, (hipStream_t)stream,
+                         *shape, *costs, d_tmax, d_g_index, s, d_scratch, d_best_s, d_best_sum,
+                         d_stage_max, d_argmin);
+    else
+      hipLaunchKernelGGL(dp_step_kernel<false>, grid, dim3(kDpThreads), 0, (hipStream_t)stream,
+                         *shape, *costs, d_tmax, d_g_index, s, d_scratch, d_best_s, d_best_sum,
+                         d_stage_max, d_argmin);
+    MIST_HIP_CHECK(hipGetLastError());
+  }
   return 0;
 }
 

@@ -3,12 +3,14 @@
 ``inter_stage_tune_with_fixed_grad_accumu`` :163-217, ``inter_stage_tune_dp_impl`` :220-355).
 
 The reference runs one numba DP per candidate ``t_max`` in an ascending host loop that stops
-once ``t_max * G >= best``.  Here the DP for many thresholds runs in one launch (one workgroup
-per threshold) and the host replays the reference's sequential rules on the returned
-``(best_s, sum, stage_max)`` triples, so the accepted thresholds, the winner and all ties are
-the reference's.  Two exact shortcuts: thresholds below the first feasible one are located by a
-multi-way search instead of being run one by one (feasibility is monotone in ``t_max`` and an
-infeasible run changes nothing), and thresholds past the stop condition are never used.
+once ``t_max * G >= best``, G after G.  Here many DP instances (any mix of G and thresholds)
+run in one batch of launches and the host replays the reference's sequential rules on the
+returned ``(best_s, sum, stage_max)`` triples, so the accepted thresholds, the winner and all
+ties are the reference's.  Exact shortcuts: (1) thresholds below the smallest feasible one are
+not run one by one; that point comes from one bottleneck (min-max) DP per G (an infeasible
+run changes nothing in the reference's scan); (2) thresholds are computed ahead speculatively
+under a bound on the running best that the sequential scan is certain to have reached, and the
+replay asks for more wherever it runs out, so a wrong guess costs time, never correctness.
 
 The reference's DP reads ``costs / costs_with_pre / ...`` fields that its intra tuner no longer
 emits; the cost tables are built from the stable / delta tables as
@@ -19,6 +21,7 @@ accepts them.
 from __future__ import annotations
 
 import ctypes
+import time
 from typing import List, Optional, Tuple
 
 import numpy as np
@@ -27,8 +30,8 @@ import torch
 from . import _lib
 from .intra_tuning import IntraStageTunerOutput
 
-PROBES = 256      # thresholds per launch while searching for the first feasible one
-CHUNK = 1024      # thresholds per launch while scanning
+FIRST_CHUNK = 48  # thresholds per G in the first speculative scan launch
+MAX_CHUNK = 4096  # most thresholds per G in one launch
 GAP = 1e-6        # inter_tuning.py:177
 
 
@@ -37,7 +40,7 @@ def _stream(device) -> ctypes.c_void_p:
 
 
 class _DpRunner:
-    """Owns the float32 cost tables of all g and runs batches of thresholds for one g."""
+    """Owns the float32 cost tables of all g and runs batches of DP instances."""
 
     def __init__(self, results: IntraStageTunerOutput, num_layers: int, num_devices: int,
                  meshes: List[Tuple[int, int]], slot: int):
@@ -49,7 +52,7 @@ class _DpRunner:
         assert L == num_layers and C == L + 1
         if list(meshes) != list(results.device_mesh_candidates):
             raise ValueError("the DP needs the mesh list the intra-stage tables were built for")
-        self.L, self.D, self.Q, self.P1 = L, num_devices, Q, P1
+        self.L, self.D, self.Q, self.P1, self.Gn = L, num_devices, Q, P1, Gn
         shape = np.zeros(1, dtype=_lib.DP_SHAPE_DTYPE)
         shape["num_layers"], shape["num_devices"], shape["num_mesh"], shape["p_dim"] = L, num_devices, Q, P1
         self.S_max = min(max(n * m for n, m in meshes), L) // 2  # inter_tuning.py:278-280
@@ -57,6 +60,7 @@ class _DpRunner:
         shape["mesh_n"][0, :Q] = [n for n, _ in meshes]
         shape["mesh_m"][0, :Q] = [m for _, m in meshes]
         self.shape = shape
+        self.plane = (L + 1) * (num_devices + 1)
         problem = np.zeros(1, dtype=_lib.PROBLEM_DTYPE)
         problem["num_layers"], problem["p_dim"], problem["sample_size"] = L, P1, S
         problem["num_grad_accum"], problem["num_mesh"] = Gn, Q
@@ -73,104 +77,127 @@ class _DpRunner:
                 out_ptrs, _stream(self.device),
             )
             _lib.check(rc, "mist_dp_cost_tables")
+        self.costs_struct = _lib.DpCosts(*[t.data_ptr() for t in self.cost])
+        for v in range(4):
+            self.costs_struct.g_stride[v] = self.cost[v][0].numel()
         self.launches = 0
         self.thresholds_run = 0
 
-    def thresholds(self, g: int) -> np.ndarray:
-        """Ascending unique finite stage costs of g (inter_tuning.py:180-186) after the gap
-        rule (:198), float32."""
-        allv = torch.cat([self.cost[v][g].reshape(-1) for v in range(3)])
-        allv = torch.unique(allv[torch.isfinite(allv)])  # sorted ascending
-        host = allv.cpu().numpy()
-        kept = np.empty_like(host)
-        n = self.lib.mist_dp_filter_tmax(
-            ctypes.c_void_p(host.ctypes.data), len(host), GAP, ctypes.c_void_p(kept.ctypes.data)
-        )
-        return kept[:n]
+    def thresholds(self) -> List[np.ndarray]:
+        """Per g: ascending unique finite stage costs (inter_tuning.py:180-186) after the gap
+        rule (:198), float32.  One device sort for all g, the sequential rule on the host."""
+        allv = torch.cat([self.cost[v].reshape(self.Gn, -1) for v in range(3)], dim=1)
+        host = torch.sort(allv, dim=1).values.cpu().numpy()  # +inf sorts last
+        out = []
+        kept = np.empty(host.shape[1], dtype=np.float32)
+        for g in range(self.Gn):
+            row = np.ascontiguousarray(host[g])
+            n_finite = int(np.searchsorted(row, np.inf, side="left"))
+            # duplicates have a zero difference to the last kept value and fall to the gap rule
+            n = self.lib.mist_dp_filter_tmax(
+                ctypes.c_void_p(row.ctypes.data), n_finite, GAP, ctypes.c_void_p(kept.ctypes.data)
+            )
+            out.append(kept[:n].copy())
+        return out
 
-    def run(self, g: int, tmax: np.ndarray, want_argmin: bool = False):
-        """DP for every threshold in ``tmax`` -> (best_s int32, best_sum f32, stage_max f32
+    def run(self, g_index: np.ndarray, tmax: np.ndarray, mode: int = _lib.DP_THRESHOLD,
+            want_argmin: bool = False):
+        """DP instances (g_index[i], tmax[i]) -> (best_s int32, best_sum f32, stage_max f32
         [, argmin])."""
         n = len(tmax)
         dev = self.device
         with torch.cuda.device(dev):
-            d_t = torch.from_numpy(np.ascontiguousarray(tmax, dtype=np.float32)).to(dev)
-            d_s = torch.empty(n, dtype=torch.int32, device=dev)
-            d_sum = torch.empty(n, dtype=torch.float32, device=dev)
-            d_max = torch.empty(n, dtype=torch.float32, device=dev)
-            n_scratch = self.lib.mist_dp_scratch_floats(ctypes.c_void_p(self.shape.ctypes.data), n)
-            if n_scratch < 0:
-                _lib.check(-1, "mist_dp_scratch_floats")
-            scratch = torch.empty(n_scratch, dtype=torch.float32, device=dev) if n_scratch else None
+            packed = np.empty((2, n), dtype=np.float32)
+            packed[0] = tmax
+            packed[1].view(np.int32)[:] = g_index
+            d_in = torch.from_numpy(packed).to(dev)
+            d_out = torch.empty((3, n), dtype=torch.float32, device=dev)
+            scratch = torch.empty(4 * n * self.plane, dtype=torch.float32, device=dev)
             argmin = None
             if want_argmin:
                 argmin = torch.full((self.S_max + 1, self.L + 1, self.D + 1, 4), -1,
                                     dtype=torch.int32, device=dev)
-            costs = _lib.DpCosts(*[self.cost[v][g].data_ptr() for v in range(4)])
             rc = self.lib.mist_dp_run(
-                ctypes.c_void_p(self.shape.ctypes.data), ctypes.byref(costs), d_t.data_ptr(), n,
-                d_s.data_ptr(), d_sum.data_ptr(), d_max.data_ptr(),
-                argmin.data_ptr() if want_argmin else None,
-                scratch.data_ptr() if scratch is not None else None, _stream(dev),
+                ctypes.c_void_p(self.shape.ctypes.data), ctypes.byref(self.costs_struct),
+                d_in[0].data_ptr(), d_in[1].data_ptr(), n, mode,
+                d_out[0].data_ptr(), d_out[1].data_ptr(), d_out[2].data_ptr(),
+                argmin.data_ptr() if want_argmin else None, scratch.data_ptr(), _stream(dev),
             )
             _lib.check(rc, "mist_dp_run")
             self.launches += 1
             self.thresholds_run += n
-            out = (d_s.cpu().numpy(), d_sum.cpu().numpy(), d_max.cpu().numpy())
+            host = d_out.cpu().numpy()
+            out = (host[0].view(np.int32), host[1], host[2])
             if want_argmin:
                 out = out + (argmin.cpu().numpy(),)
         return out
 
-    def first_feasible(self, g: int, tmax: np.ndarray) -> int:
-        """Index of the smallest feasible threshold (len(tmax) if none): multi-way search."""
-        lo, hi = 0, len(tmax)  # invariant: everything below lo is infeasible
-        if hi == 0:
-            return 0
-        best_s, _, _ = self.run(g, tmax[-1:])
-        if best_s[0] < 0:
-            return hi
-        hi -= 1  # tmax[hi] is feasible
-        while hi - lo > 0:
-            probes = np.unique(np.linspace(lo, hi, min(PROBES, hi - lo + 1)).astype(np.int64))
-            best_s, _, _ = self.run(g, tmax[probes])
-            feas = np.nonzero(best_s >= 0)[0]
-            first = int(feas[0])  # probes[-1] == hi is feasible, so this exists
-            hi = int(probes[first])
-            lo = int(probes[first - 1]) + 1 if first > 0 else lo
-            if first == 0:
-                break
-        return hi
 
+class _Scan:
+    """Replay state of ``inter_stage_tune_with_fixed_grad_accumu`` (inter_tuning.py:163-217) for
+    one G: ``pos`` = next threshold the sequential scan would look at, ``results`` = DP outcomes
+    already computed for tmax[lo : lo + len]."""
 
-def inter_stage_tune_with_fixed_grad_accumu(
-    runner: _DpRunner, g: int, gradient_accumulation_steps: int, best_cost: float = float("inf"),
-):
-    """inter_tuning.py:163-217 -> (best_cost, best_t_max or None)."""
-    G = gradient_accumulation_steps
-    tmax = runner.thresholds(g)
-    best_t = None
-    if len(tmax) == 0:
-        return best_cost, best_t
-    # float32 scalar * python int is float64 under the reference's numpy 1.24.
-    scaled = tmax.astype(np.float64) * G
-    start = runner.first_feasible(g, tmax[: int(np.searchsorted(scaled, best_cost, side="left"))])
-    pos = start
-    while pos < len(tmax):
-        if scaled[pos] >= best_cost:
-            break
-        stop = int(np.searchsorted(scaled, best_cost, side="left"))
-        chunk = tmax[pos: min(pos + CHUNK, stop)]
-        best_s, best_sum, stage_max = runner.run(g, chunk)
-        for i in range(len(chunk)):
-            if scaled[pos + i] >= best_cost:
-                return best_cost, best_t
-            if best_s[i] < 0:
-                continue
-            cost = float(np.float64(best_sum[i]) + np.float64(G - 1) * np.float64(stage_max[i]))
-            if cost < best_cost:
-                best_cost, best_t = cost, chunk[i]
-        pos += len(chunk)
-    return best_cost, best_t
+    def __init__(self, G: int, tmax: np.ndarray, first: int):
+        self.G, self.tmax = G, tmax
+        # float32 scalar * python int is float64 under the reference's numpy 1.24.
+        self.scaled = tmax.astype(np.float64) * G
+        self.pos = first          # everything below is infeasible: the scan passes it unchanged
+        self.have_lo = first
+        self.best_s = np.empty(0, dtype=np.int32)
+        self.best_sum = np.empty(0, dtype=np.float32)
+        self.stage_max = np.empty(0, dtype=np.float32)
+        self.limit = FIRST_CHUNK
+
+    def wanted(self, best_cost: float) -> Tuple[int, int]:
+        """Index range [a, b) of thresholds to compute next under the bound ``best_cost``; the
+        range grows fourfold every time the same G asks again."""
+        a = self.have_lo + len(self.best_s)
+        stop = int(np.searchsorted(self.scaled, best_cost, side="left"))
+        b = max(a, min(stop, a + self.limit))
+        if b > a:
+            self.limit = min(MAX_CHUNK, self.limit * 4)
+        return a, b
+
+    def runs_out(self, best_cost: float) -> bool:
+        """Dry run of ``replay`` under the bound ``best_cost`` (the true running best when this G
+        is reached is no larger, so the true scan stops no later): True if the computed results
+        would not suffice."""
+        pos, hi, G = self.pos, self.have_lo + len(self.best_s), self.G
+        while pos < len(self.tmax):
+            if self.scaled[pos] >= best_cost:
+                return False
+            if pos >= hi:
+                return True
+            i = pos - self.have_lo
+            if self.best_s[i] >= 0:
+                cost = float(np.float64(self.best_sum[i]) + np.float64(G - 1) * np.float64(self.stage_max[i]))
+                best_cost = min(best_cost, cost)
+            pos += 1
+        return False
+
+    def add(self, best_s, best_sum, stage_max):
+        self.best_s = np.concatenate([self.best_s, best_s])
+        self.best_sum = np.concatenate([self.best_sum, best_sum])
+        self.stage_max = np.concatenate([self.stage_max, stage_max])
+
+    def replay(self, best_cost: float, best_t):
+        """Advances the sequential scan as far as the computed results allow.  Returns
+        (best_cost, best_t, finished)."""
+        G = self.G
+        hi = self.have_lo + len(self.best_s)
+        while self.pos < len(self.tmax):
+            if self.scaled[self.pos] >= best_cost:  # inter_tuning.py:196-197
+                return best_cost, best_t, True
+            if self.pos >= hi:
+                return best_cost, best_t, False     # needs more DP results
+            i = self.pos - self.have_lo
+            if self.best_s[i] >= 0:
+                cost = float(np.float64(self.best_sum[i]) + np.float64(G - 1) * np.float64(self.stage_max[i]))
+                if cost < best_cost:
+                    best_cost, best_t = cost, self.tmax[self.pos]
+            self.pos += 1
+        return best_cost, best_t, True
 
 
 def get_solution_from_intra_stage_tuner_output(
@@ -182,12 +209,12 @@ def get_solution_from_intra_stage_tuner_output(
     l = layer_end - layer_start + 1
     r = intra_stage_results
     if layer_start == 0 and layer_end == num_layers - 1:
-        return r.solutions_no_pp[g, q, c, slot]
+        return r.solution_at(3, (g, q, c, slot))
     if layer_start == 0:
-        return r.solutions_with_pre[g, q, p, l - 1, c, slot]
+        return r.solution_at(1, (g, q, p, l - 1, c, slot))
     if layer_end == num_layers - 1:
-        return r.solutions_with_post[g, q, l - 1, c, slot]
-    return r.solutions[g, q, p, l - 1, c, slot]
+        return r.solution_at(2, (g, q, l - 1, c, slot))
+    return r.solution_at(0, (g, q, p, l - 1, c, slot))
 
 
 def inter_stage_tune(
@@ -205,15 +232,62 @@ def inter_stage_tune(
         raise TypeError(
             f"intra_stage_results must be an instance of IntraStageTunerOutput, got {type(intra_stage_results)}"
         )
+    t_start = time.perf_counter()
     runner = _DpRunner(intra_stage_results, num_layers, num_devices, device_mesh_candidates, slot)
     g_index = {G: i for i, G in enumerate(intra_stage_results.gradient_accumulation_steps_candidates)}
     q_index = {q: i for i, q in enumerate(intra_stage_results.device_mesh_candidates)}
+    Gs = list(gradient_accumulation_steps_candidates)
+    gs = np.array([g_index[G] for G in Gs], dtype=np.int32)
+    t_0 = time.perf_counter()
+    tmax_all = runner.thresholds()
+    t_1 = time.perf_counter()
+
+    # Smallest feasible threshold of every G in one launch (bottleneck DP).
+    _, bottleneck, _ = runner.run(gs, np.zeros(len(Gs), dtype=np.float32), _lib.DP_BOTTLENECK)
+    scans = []
+    for i, G in enumerate(Gs):
+        tmax = tmax_all[gs[i]]
+        first = int(np.searchsorted(tmax, bottleneck[i], side="left")) if np.isfinite(bottleneck[i]) else len(tmax)
+        scans.append(_Scan(G, tmax, first))
+
+    # Speculative batches + sequential replay.  A bound on the running best that the sequential
+    # scan is certain to have reached decides how much of each G is worth computing ahead; the
+    # replay then applies the reference's rules in order and asks for more where it runs out.
     best_cost, best_G, best_t = float("inf"), None, None
-    for G in gradient_accumulation_steps_candidates:
-        cost, t = inter_stage_tune_with_fixed_grad_accumu(runner, g_index[G], G, best_cost)
-        if cost < best_cost and t is not None:
-            best_cost, best_G, best_t = cost, G, t
+    current = 0  # scans[:current] are finished
+    while True:
+        while current < len(scans):  # commit the sequential scan as far as results allow
+            sc = scans[current]
+            cost, t, finished = sc.replay(best_cost, None)
+            if t is not None:
+                best_cost, best_G, best_t = cost, sc.G, t
+            if not finished:
+                break
+            current += 1
+        if current == len(scans):
+            break
+        req_g, req_t, req_span = [], [], []
+        for i in range(current, len(scans)):
+            sc = scans[i]
+            if i > current and not sc.runs_out(best_cost):
+                continue
+            a, b = sc.wanted(best_cost)
+            if b > a:
+                req_g.append(np.full(b - a, gs[i], dtype=np.int32))
+                req_t.append(sc.tmax[a:b])
+                req_span.append((i, b - a))
+        if not req_span:
+            raise RuntimeError("inter-stage scan made no progress")  # cannot happen: guards a hang
+        bs, bsum, smax = runner.run(np.concatenate(req_g), np.concatenate(req_t))
+        off = 0
+        for i, n in req_span:
+            scans[i].add(bs[off:off + n], bsum[off:off + n], smax[off:off + n])
+            off += n
+    t_2 = time.perf_counter()
     if stats is not None:
+        stats["dp_setup_s"] = stats.get("dp_setup_s", 0.0) + (t_0 - t_start)
+        stats["dp_thresholds_s"] = stats.get("dp_thresholds_s", 0.0) + (t_1 - t_0)
+        stats["dp_scan_s"] = stats.get("dp_scan_s", 0.0) + (t_2 - t_1)
         stats["dp_launches"] = stats.get("dp_launches", 0) + runner.launches
         stats["dp_thresholds"] = stats.get("dp_thresholds", 0) + runner.thresholds_run
     if best_G is None:
@@ -221,7 +295,8 @@ def inter_stage_tune(
 
     # Back-pointers of the winning (G, t_max) run (inter_tuning.py:341-355).
     g = g_index[best_G]
-    best_s, best_sum, stage_max, argmin = runner.run(g, np.array([best_t], dtype=np.float32), True)
+    best_s, best_sum, stage_max, argmin = runner.run(
+        np.array([g], dtype=np.int32), np.array([best_t], dtype=np.float32), want_argmin=True)
     cs, cl, cd = int(best_s[0]), 0, num_devices
     inter = []
     while cs > 0 and cl < num_layers and cd > 0:

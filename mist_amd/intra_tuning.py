@@ -95,6 +95,16 @@ class IntraStageTunerOutput:
             self._host[key] = out
         return self._host[key]
 
+    def solution_at(self, variant: int, cell: Tuple[int, ...]) -> np.ndarray:
+        """One strategy row ``solutions<variant>[cell]`` (cell = full index incl. g, q and the
+        sample slot) without building the whole solutions table: a single index is read back."""
+        key = f"solutions{variant}"
+        if key in self._host:
+            return self._host[key][cell]
+        idx = self._host.get(f"index{variant}")
+        row = int(idx[cell]) if idx is not None else int(self.device.index[variant][cell].item())
+        return self.spaces[(cell[0], cell[1])].decode(np.array(row))
+
     def __getattr__(self, name: str):
         for v, suffix in enumerate(VARIANTS):
             if name == "costs_stable" + suffix:

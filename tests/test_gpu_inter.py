@@ -19,7 +19,7 @@ def _random_tables(rng, Q, P1, L, inf_frac=0.2, quantum=None):
     return rand((Q, P1, L, L + 1)), rand((Q, P1, L, L + 1)), rand((Q, L, L + 1)), rand((Q, L + 1))
 
 
-def _gpu_dp(meshes, L, D, P1, tabs, tmax, want_argmin=False):
+def _gpu_dp(meshes, L, D, P1, tabs, tmax, want_argmin=False, mode=0):
     import torch
     from mist_amd import _lib
 
@@ -35,6 +35,7 @@ def _gpu_dp(meshes, L, D, P1, tabs, tmax, want_argmin=False):
     costs = _lib.DpCosts(*[t.data_ptr() for t in dev])
     n = len(tmax)
     d_t = torch.tensor(tmax, dtype=torch.float32).cuda()
+    d_g = torch.zeros(n, dtype=torch.int32).cuda()
     d_s = torch.empty(n, dtype=torch.int32).cuda()
     d_sum = torch.empty(n, dtype=torch.float32).cuda()
     d_max = torch.empty(n, dtype=torch.float32).cuda()
@@ -42,9 +43,9 @@ def _gpu_dp(meshes, L, D, P1, tabs, tmax, want_argmin=False):
     scr = torch.empty(max(n_scr, 1), dtype=torch.float32).cuda()
     arg = torch.full((S + 1, L + 1, D + 1, 4), -1, dtype=torch.int32).cuda() if want_argmin else None
     rc = lib.mist_dp_run(
-        ctypes.c_void_p(shape.ctypes.data), ctypes.byref(costs), d_t.data_ptr(), n, d_s.data_ptr(),
-        d_sum.data_ptr(), d_max.data_ptr(), arg.data_ptr() if want_argmin else None,
-        scr.data_ptr() if n_scr else None, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream),
+        ctypes.c_void_p(shape.ctypes.data), ctypes.byref(costs), d_t.data_ptr(), d_g.data_ptr(), n,
+        mode, d_s.data_ptr(), d_sum.data_ptr(), d_max.data_ptr(), arg.data_ptr() if want_argmin else None,
+        scr.data_ptr(), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream),
     )
     _lib.check(rc, "mist_dp_run")
     torch.cuda.synchronize()
@@ -58,7 +59,7 @@ def _gpu_dp(meshes, L, D, P1, tabs, tmax, want_argmin=False):
         (6, 4, [(1, 1), (1, 2), (1, 4)], 3, None),
         (9, 8, [(1, 1), (1, 2), (1, 4), (2, 4)], 5, 0.125),
         (12, 16, [(1, 1), (1, 2), (1, 4), (1, 8), (2, 8)], 7, 0.0625),
-        (40, 80, [(1, 1), (1, 2), (1, 4), (1, 8), (2, 8), (4, 8), (8, 8)], 21, 0.03125),  # global-scratch path
+        (40, 80, [(1, 1), (1, 2), (1, 4), (1, 8), (2, 8), (4, 8), (8, 8)], 21, 0.03125),  # large state planes
     ],
 )
 def test_dp_kernel_matches_c_oracle(L, D, meshes, P1, quantum):
@@ -88,6 +89,14 @@ def test_dp_kernel_matches_c_oracle(L, D, meshes, P1, quantum):
             g = _gpu_dp(meshes, L, D, P1, tabs, [t], want_argmin=True)
             assert np.array_equal(g[3], arg), f"back-pointers differ at t={t}"
     assert n_feasible > 0
+    # bottleneck mode = the smallest threshold for which the threshold DP is feasible
+    _, bott, _ = _gpu_dp(meshes, L, D, P1, tabs, [0.0], mode=1)
+    cand = np.unique(np.concatenate([t.ravel() for t in tabs[:3]]))
+    cand = cand[np.isfinite(cand)]
+    feas = _gpu_dp(meshes, L, D, P1, tabs, cand)[0] >= 0
+    # (single-stage costs are not threshold candidates, so the bottleneck itself may be absent)
+    assert feas.any() and cand[np.argmax(feas)] == cand[cand >= bott[0]].min()
+    assert np.all(feas[np.argmax(feas):]) and not feas[: np.argmax(feas)].any()
 
 
 @pytest.mark.parametrize(

@@ -203,15 +203,17 @@ def test_argument_checks_reject_before_any_launch():
     shape["num_layers"], shape["num_devices"], shape["num_mesh"], shape["p_dim"] = 8, 8, 2, 4
     shape["max_stages"] = 4
     shape["mesh_n"][0, :2], shape["mesh_m"][0, :2] = [1, 1], [1, 2]
-    assert lib.mist_dp_scratch_floats(ctypes.c_void_p(shape.ctypes.data), 4) == 0
+    assert lib.mist_dp_scratch_floats(ctypes.c_void_p(shape.ctypes.data), 4) == 4 * 4 * 9 * 9
     shape["num_layers"], shape["num_devices"] = 80, 256
     assert lib.mist_dp_scratch_floats(ctypes.c_void_p(shape.ctypes.data), 4) == 4 * 4 * 81 * 257
     costs = _lib.DpCosts(4096, 4096, 4096, 4096)
     sp = ctypes.c_void_p(shape.ctypes.data)
-    assert lib.mist_dp_run(sp, ctypes.byref(costs), fake, 2, fake, fake, fake, fake, None, None) == -1
+    assert lib.mist_dp_run(sp, ctypes.byref(costs), fake, fake, 2, 0, fake, fake, fake, fake, fake, None) == -1
     assert b"argmin" in lib.mist_last_error()
-    assert lib.mist_dp_run(sp, ctypes.byref(costs), fake, 1, fake, fake, fake, None, None, None) == -1
+    assert lib.mist_dp_run(sp, ctypes.byref(costs), fake, fake, 1, 0, fake, fake, fake, None, None, None) == -1
     assert b"scratch" in lib.mist_last_error()
+    assert lib.mist_dp_run(sp, ctypes.byref(costs), fake, fake, 70000, 0, fake, fake, fake, None, fake, None) == -1
+    assert lib.mist_dp_run(sp, ctypes.byref(costs), fake, fake, 1, 7, fake, fake, fake, None, fake, None) == -1
 
 
 def test_gap_filter_matches_oracle_rule():

@@ -27,7 +27,9 @@ extern "C" {
 #define MIST_PAR_FIELDS 20
 #define MIST_ROW_TERMS 34   /* doubles per candidate row produced by mist_row_terms */
 #define MIST_LC_TILE 256    /* (layers, ckpt) pairs per workgroup of the reduce kernel */
-#define MIST_P_TILE 8       /* pre-saved micro-batch values per thread of the reduce kernel */
+#ifndef MIST_P_TILE
+#define MIST_P_TILE 16      /* pre-saved micro-batch values per thread of the reduce kernel */
+#endif
 #define MIST_MAX_MESH 16    /* device-mesh candidates of the inter-stage DP */
 
 #define MIST_E_INVALID (-1) /* argument / shape check failed, nothing was launched */
@@ -133,6 +135,7 @@ const char *mist_version(void);
 const char *mist_last_error(void);
 int mist_sizeof_problem(void);
 int mist_sizeof_group(void);
+int mist_reduce_p_tile(void); /* MIST_P_TILE the library was built with */
 
 /* Row-invariant terms of every candidate row: decodes the row index, evaluates the alpha-beta
  * communication terms, the 36 interference evaluations and the memory pieces that do not

@@ -17,7 +17,7 @@ MAX_PAIRS = MAX_RATIOS * MAX_RATIOS
 PAR_FIELDS = 20
 ROW_TERMS = 34
 LC_TILE = 256
-P_TILE = 8
+P_TILE = 32  # replaced by the library's own value in load()
 SLOTS = 2 * P_TILE + 2
 STAGE_ROWS = 32
 TERMS_BLOCK = 256
@@ -103,6 +103,7 @@ _SIGNATURES = {
     "mist_last_error": (ctypes.c_char_p, []),
     "mist_sizeof_problem": (ctypes.c_int, []),
     "mist_sizeof_group": (ctypes.c_int, []),
+    "mist_reduce_p_tile": (ctypes.c_int, []),
     "mist_row_terms": (ctypes.c_int, [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, _VP]),
     "mist_eval_reduce": (
         ctypes.c_int,
@@ -187,6 +188,9 @@ def load():
         raise MistLibraryError(
             f"MistGroupDesc layout mismatch: C {lib.mist_sizeof_group()} vs numpy {GROUP_DTYPE.itemsize}"
         )
+    global P_TILE, SLOTS
+    P_TILE = lib.mist_reduce_p_tile()
+    SLOTS = 2 * P_TILE + 2
     _LIB = lib
     return lib
 

@@ -26,7 +26,8 @@ HIPCC_FLAGS = [
 def build_library(verbose: bool = False) -> str:
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     sources = [s for s in SOURCES if os.path.exists(s)]
-    cmd = [hipcc, *HIPCC_FLAGS, "-I" + os.path.join(REPO_DIR, "include"), *sources, "-o", LIB_PATH]
+    extra = os.environ.get("MIST_HIPCC_EXTRA", "").split()
+    cmd = [hipcc, *HIPCC_FLAGS, *extra, "-I" + os.path.join(REPO_DIR, "include"), *sources, "-o", LIB_PATH]
     if verbose:
         print(" ".join(cmd))
     proc = subprocess.run(cmd, capture_output=True, text=True)

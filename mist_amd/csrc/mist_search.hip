@@ -418,6 +418,13 @@ __device__ __forceinline__ void take_min(double &best, int32_t &best_row, bool f
 // through LDS (every lane reads the same row: broadcast reads, no bank conflicts) and each
 // thread keeps the minima of MIST_P_TILE pre-saved micro-batch values for its own (l, c).
 // No cross-lane reduction is needed: the reduction axis (rows) is the loop, not the lanes.
+//
+// Memory feasibility is monotone in p: the peaks are built from p * (non-negative) terms by
+// additions only, every floating-point add / multiply is monotone in each operand, and the
+// host rejects negative table values.  So per (row, l, c) the feasible p form a prefix
+// [0, count) and `count` is found by bisection with the exact peak formula at the probed p
+// (no closed-form shortcut: the comparison that decides is the reference's own expression).
+// A row then updates exactly the slots p < count where its cost is strictly smaller.
 // ------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(MIST_LC_TILE) void eval_reduce_kernel(
     const MistProblem prob, const MistGroupDesc *__restrict__ groups, int n_groups,
@@ -440,7 +447,9 @@ __global__ __launch_bounds__(MIST_LC_TILE) void eval_reduce_kernel(
   const int l = pc.l, c = pc.c;
 
   const int p0 = p_tile * MIST_P_TILE;
-  const int num_p = g->num_p;
+  const int n_tile = min(MIST_P_TILE, g->num_p - p0);  // p values of this tile: p0 .. p0+n_tile-1
+  int steps = 0;  // bisection steps that separate the n_tile + 1 possible counts
+  while ((1 << steps) < n_tile + 1) ++steps;
   const bool first_p_tile = p_tile == 0;
   const bool do_nopp = first_p_tile && l == L;
   const GroupConsts k = group_consts(g);
@@ -452,13 +461,18 @@ __global__ __launch_bounds__(MIST_LC_TILE) void eval_reduce_kernel(
   const double post_states = g->post_states, post_fwd_peak = g->post_fwd_peak;
   const double post_bwd_peak = g->post_bwd_peak, post_output = g->post_output;
 
-  double best[kSlots];
-  int32_t best_row[kSlots];
+  double best_b[MIST_P_TILE], best_p[MIST_P_TILE];
+  int32_t row_b[MIST_P_TILE], row_p[MIST_P_TILE];
 #pragma unroll
-  for (int s = 0; s < kSlots; ++s) {
-    best[s] = INFINITY;
-    best_row[s] = -1;
+  for (int j = 0; j < MIST_P_TILE; ++j) {
+    best_b[j] = best_p[j] = INFINITY;
+    row_b[j] = row_p[j] = -1;
   }
+  double best_post = INFINITY, best_pp = INFINITY;
+  int32_t row_post = -1, row_pp = -1;
+  // Largest minimum of the tile (slot n_tile - 1): a row that does not beat it cannot change
+  // any slot, because the minima are non-decreasing in p.
+  double top_b = INFINITY, top_p = INFINITY;
 
   const int64_t row_begin = (int64_t)chunk * g->rows_per_chunk;
   const int64_t row_end = min(row_begin + (int64_t)g->rows_per_chunk, g->n_rows);
@@ -487,6 +501,8 @@ __global__ __launch_bounds__(MIST_LC_TILE) void eval_reduce_kernel(
       const float y32 = lat.d / G32;  // float32 array / python int (:2815)
       const double cost_base = ratio * (double)lat.x + (double)y32;
       const double cost_pre = ratio * lat.sp + lat.dpre / G64;
+      const bool try_b = cost_base < top_b, try_p = cost_pre < top_p;
+      if (!(try_b || try_p || first_p_tile)) continue;
 
       // ---- memory that does not depend on p (:2150-2162, 2358-2385, 2760-2769) ----
       const double S_ck = t[MIST_T_S_CK], S_nock = t[MIST_T_S_NOCK];
@@ -498,43 +514,79 @@ __global__ __launch_bounds__(MIST_LC_TILE) void eval_reduce_kernel(
       const double fwd_pk = t[MIST_T_FWD_PEAK], bwd_pk = t[MIST_T_BWD_PEAK];
       const double out = t[MIST_T_OUT], gcb = t[MIST_T_GCB];
       const double out2 = out * 2.0;
-      const double mf_base = t[MIST_T_MF_BASE], mf_pp = t[MIST_T_MF_PP];
 
-#pragma unroll
-      for (int j = 0; j < MIST_P_TILE; ++j) {
-        const int p = p0 + j;
+      // Peaks of the middle-stage variant for p pre-saved micro-batches (:2755-2786).
+      auto peaks = [&](int p, double &peak_f, double &peak_b) {
         const double pf64 = (double)p;
         const double pipe_saved = pf64 * mod_saved + cur_saved;
         const double outp2 = out * pf64 * 2.0;
-        const double peak_f = fwd_states + pipe_saved + ck_delta + fwd_pk + outp2 + gcb;
-        const double peak_b = bwd_states + pipe_saved + ck_delta + bwd_pk + outp2 + out2 + gcb;
-        const bool in_range = p < num_p;
-        const bool ok_base = in_range && fmax(peak_f, peak_b) * mf_base <= cap;
-        take_min(best[j], best_row[j], ok_base, cost_base, row);
-        const double pre_p = pf64 * pre_saved;
-        const double peak_f_pre = pre_p + peak_f + pre_sas;
-        const double peak_b_pre = pre_p + peak_b + pre_sas;
-        const bool ok_pre = in_range && fmax(peak_f_pre, peak_b_pre) * mf_pp <= cap;
-        take_min(best[MIST_P_TILE + j], best_row[MIST_P_TILE + j], ok_pre, cost_pre, row);
+        peak_f = fwd_states + pipe_saved + ck_delta + fwd_pk + outp2 + gcb;
+        peak_b = bwd_states + pipe_saved + ck_delta + bwd_pk + outp2 + out2 + gcb;
+      };
 
-        if (j == 0 && first_p_tile) {
-          // ---- last stage / single stage, p == 0 only (:2946-3106) ----
-          const double f_in = fwd_states + post_states + mod_saved + post_fwd_peak + gcb;
-          const double b_in = bwd_states + post_states + mod_saved + post_bwd_peak +
-                              (c_eq_0 ? t[MIST_T_RD] : 0.0) + gcb;
-          const double pf_post = fmax(f_in, peak_f + post_states);
-          const double pb_post = fmax(b_in, peak_b - out + post_states) + post_output;
-          const bool ok_post = fmax(pf_post, pb_post) * mf_pp <= cap;
-          const double cost_post = ratio * lat.spost + lat.dpost / G64;
-          take_min(best[2 * MIST_P_TILE], best_row[2 * MIST_P_TILE], ok_post, cost_post, row);
-          if (do_nopp) {
-            const double pf_pp = pf_post + pre_states + pre_saved;
-            const double pb_pp = pb_post + pre_states + pre_saved;
-            const bool ok_pp = fmax(pf_pp, pb_pp) * t[MIST_T_MF] <= cap;
-            const double cost_pp = ratio * lat.spp + lat.dpp / G64;
-            take_min(best[2 * MIST_P_TILE + 1], best_row[2 * MIST_P_TILE + 1], ok_pp, cost_pp,
-                     row);
-          }
+      if (try_b) {
+        const double mf_base = t[MIST_T_MF_BASE];
+        int lo = 0, hi = n_tile;  // number of feasible p of this tile lies in [lo, hi]
+        for (int it = 0; it < steps; ++it) {
+          const int mid = (lo + hi) >> 1;
+          double pf, pb;
+          peaks(p0 + mid, pf, pb);
+          const bool ok = fmax(pf, pb) * mf_base <= cap;  // (:2805-2812)
+          const bool open = lo < hi;
+          lo = (open && ok) ? mid + 1 : lo;
+          hi = (open && !ok) ? mid : hi;
+        }
+#pragma unroll
+        for (int j = 0; j < MIST_P_TILE; ++j) {
+          const bool better = j < lo && cost_base < best_b[j];
+          best_b[j] = better ? cost_base : best_b[j];
+          row_b[j] = better ? row : row_b[j];
+        }
+        top_b = (n_tile <= lo) ? cost_base : top_b;  // slot n_tile - 1 was among the updated
+      }
+      if (try_p) {
+        const double mf_pp = t[MIST_T_MF_PP];
+        int lo = 0, hi = n_tile;
+        for (int it = 0; it < steps; ++it) {
+          const int mid = (lo + hi) >> 1;
+          double pf, pb;
+          peaks(p0 + mid, pf, pb);
+          const double pre_p = (double)(p0 + mid) * pre_saved;  // (:2866-2875)
+          const double pf_pre = pre_p + pf + pre_sas;
+          const double pb_pre = pre_p + pb + pre_sas;
+          const bool ok = fmax(pf_pre, pb_pre) * mf_pp <= cap;  // (:2893-2897)
+          const bool open = lo < hi;
+          lo = (open && ok) ? mid + 1 : lo;
+          hi = (open && !ok) ? mid : hi;
+        }
+#pragma unroll
+        for (int j = 0; j < MIST_P_TILE; ++j) {
+          const bool better = j < lo && cost_pre < best_p[j];
+          best_p[j] = better ? cost_pre : best_p[j];
+          row_p[j] = better ? row : row_p[j];
+        }
+        top_p = (n_tile <= lo) ? cost_pre : top_p;
+      }
+
+      if (first_p_tile) {
+        // ---- last stage / single stage, p == 0 only (:2946-3106) ----
+        double peak_f, peak_b;
+        peaks(0, peak_f, peak_b);
+        const double mf_pp = t[MIST_T_MF_PP];
+        const double f_in = fwd_states + post_states + mod_saved + post_fwd_peak + gcb;
+        const double b_in = bwd_states + post_states + mod_saved + post_bwd_peak +
+                            (c_eq_0 ? t[MIST_T_RD] : 0.0) + gcb;
+        const double pf_post = fmax(f_in, peak_f + post_states);
+        const double pb_post = fmax(b_in, peak_b - out + post_states) + post_output;
+        const bool ok_post = fmax(pf_post, pb_post) * mf_pp <= cap;
+        const double cost_post = ratio * lat.spost + lat.dpost / G64;
+        take_min(best_post, row_post, ok_post, cost_post, row);
+        if (do_nopp) {
+          const double pf_pp = pf_post + pre_states + pre_saved;
+          const double pb_pp = pb_post + pre_states + pre_saved;
+          const bool ok_pp = fmax(pf_pp, pb_pp) * t[MIST_T_MF] <= cap;
+          const double cost_pp = ratio * lat.spp + lat.dpp / G64;
+          take_min(best_pp, row_pp, ok_pp, cost_pp, row);
         }
       }
     }
@@ -542,10 +594,16 @@ __global__ __launch_bounds__(MIST_LC_TILE) void eval_reduce_kernel(
 
   const int64_t out_base = (int64_t)blockIdx.x * kSlots * MIST_LC_TILE + threadIdx.x;
 #pragma unroll
-  for (int s = 0; s < kSlots; ++s) {
-    partial_cost[out_base + (int64_t)s * MIST_LC_TILE] = best[s];
-    partial_index[out_base + (int64_t)s * MIST_LC_TILE] = best_row[s];
+  for (int j = 0; j < MIST_P_TILE; ++j) {
+    partial_cost[out_base + (int64_t)j * MIST_LC_TILE] = best_b[j];
+    partial_index[out_base + (int64_t)j * MIST_LC_TILE] = row_b[j];
+    partial_cost[out_base + (int64_t)(MIST_P_TILE + j) * MIST_LC_TILE] = best_p[j];
+    partial_index[out_base + (int64_t)(MIST_P_TILE + j) * MIST_LC_TILE] = row_p[j];
   }
+  partial_cost[out_base + (int64_t)(2 * MIST_P_TILE) * MIST_LC_TILE] = best_post;
+  partial_index[out_base + (int64_t)(2 * MIST_P_TILE) * MIST_LC_TILE] = row_post;
+  partial_cost[out_base + (int64_t)(2 * MIST_P_TILE + 1) * MIST_LC_TILE] = best_pp;
+  partial_index[out_base + (int64_t)(2 * MIST_P_TILE + 1) * MIST_LC_TILE] = row_pp;
 }
 
 // ------------------------------------------------------------------------------------------
@@ -631,6 +689,7 @@ const char *mist_version(void) { return "mist_search 0.1 (gfx950)"; }
 const char *mist_last_error(void) { return g_last_error; }
 int mist_sizeof_problem(void) { return (int)sizeof(MistProblem); }
 int mist_sizeof_group(void) { return (int)sizeof(MistGroupDesc); }
+int mist_reduce_p_tile(void) { return MIST_P_TILE; }
 
 int mist_row_terms(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,
                    const int32_t *d_block_prefix, int n_blocks, double *d_row_terms,

@@ -165,6 +165,7 @@ class IntraStageTuner:
     # ------------------------------------------------------------------ host side
     def prepare(self):
         """Builds the group descriptors and the launch decomposition (host only, no GPU)."""
+        _lib.load()  # the tile sizes of the decomposition are the library's
         cfg, L = self.config, self.num_layers
         Gs, Q = self.gradient_accumulation_steps_candidates, self.device_mesh_candidates
         P = self.max_possible_pre_saved_micro_batches

@@ -132,24 +132,22 @@ def main():
     kernel_ms = {}
     for rep in range(3):
         events = []
-        for tuner, plan, dev_plan in search.tuners:
-            tables = tuner.allocate_tables()
-            tuner.launch(plan, dev_plan, tables, events=events)
+        tables = search.tuner.allocate_tables()
+        search.tuner.launch(search.plan, search.dev_plan, tables, events=events)
         torch.cuda.synchronize()
         if rep == 0:
             continue  # warm-up of the separately launched entry points
         for name, start, end in events:
             kernel_ms[name] = kernel_ms.get(name, 0.0) + start.elapsed_time(end)
-        for (tuner, plan, dev_plan) in search.tuners:
-            flops += reduce_kernel_flops(plan, search.L)
-            n_launches += 1
+        flops += reduce_kernel_flops(search.plan, search.L)
+        n_launches += 1
     dur_ms = kernel_ms["eval_reduce"]
     achieved = flops / (dur_ms * 1e-3) / 1e12
     roofline = dict(
         bound="fp64-valu", kernel="eval_reduce_kernel", achieved=achieved,
         peak=FP64_VECTOR_PEAK / 1e12, unit="TFLOP/s", frac=achieved / (FP64_VECTOR_PEAK / 1e12),
         traffic=None, avg_launch_ms=dur_ms / n_launches, flop_per_launch=flops / n_launches,
-        launches_per_step=len(search.tuners),
+        launches_per_step=1,
     )
     intra_ms_per_step = sum(kernel_ms.values()) / 2
 

@@ -69,7 +69,7 @@ int mist_dp_filter_tmax(const float *sorted_unique, int n, double gap, float *ou
  *   is the smallest threshold for which the instance is feasible (+inf if none).  The reference
  *   finds that point by running the threshold DP for every smaller candidate, all of which
  *   return "infeasible" and change nothing.
- * d_argmin (may be NULL; needs n_tmax == 1): [max_stages+1][L+1][D+1][4] int32 =
+ * d_argmin (may be NULL): [n_tmax][max_stages+1][L+1][D+1][4] int32 =
  *   (end layer, n, m, ckpt), pre-filled with -1 by the caller.
  * d_scratch: mist_dp_scratch_floats() = 4 * n_tmax * (L+1) * (D+1) floats of state. */
 int64_t mist_dp_scratch_floats(const MistDpShape *shape, int n_tmax);

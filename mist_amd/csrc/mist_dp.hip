@@ -134,7 +134,7 @@ __global__ __launch_bounds__(kDpThreads) void dp_step_kernel(
   f_cur[e] = best;
   m_cur[e] = best_m;
   if (argmin != nullptr && arg_i >= 0) {
-    int32_t *a = argmin + ((int64_t)s * plane + e) * 4;
+    int32_t *a = argmin + (((int64_t)t * (shape.max_stages + 1) + s) * plane + e) * 4;
     a[0] = arg_i;
     a[1] = shape.mesh_n[arg_q];
     a[2] = shape.mesh_m[arg_q];
@@ -230,8 +230,6 @@ int mist_dp_run(const MistDpShape *shape, const MistDpCosts *costs, const float 
     return fail(MIST_E_INVALID, "n_tmax must be in [1, 65535], got %d", n_tmax);
   if (mode != MIST_DP_THRESHOLD && mode != MIST_DP_BOTTLENECK)
     return fail(MIST_E_INVALID, "unknown DP mode %d", mode);
-  if (d_argmin && n_tmax != 1)
-    return fail(MIST_E_INVALID, "argmin output needs n_tmax == 1, got %d", n_tmax);
   const int plane = (shape->num_layers + 1) * (shape->num_devices + 1);
   const int64_t n_init = (int64_t)n_tmax * plane;
   hipLaunchKernelGGL(dp_init_kernel, dim3((unsigned)((n_init + 255) / 256)), dim3(256), 0,

@@ -426,19 +426,16 @@ __device__ __forceinline__ void take_min(double &best, int32_t &best_row, bool f
 // (no closed-form shortcut: the comparison that decides is the reference's own expression).
 // A row then updates exactly the slots p < count where its cost is strictly smaller.
 // ------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(MIST_LC_TILE) void eval_reduce_kernel(
-    const MistProblem prob, const MistGroupDesc *__restrict__ groups, int n_groups,
-    const int32_t *__restrict__ block_prefix, const double *__restrict__ row_terms, double ratio,
+// kPow2G: the group's G is a power of two, so x / G == x * (1 / G) bit for bit (float32 and
+// float64) and the division leaves the inner loop; other G divide.  kFirstTile: this workgroup
+// owns p = 0 and therefore also the last-stage and single-stage variants.
+constexpr int kRowUnroll = 4;  // rows whose objective values are computed together (ILP)
+
+template <bool kPow2G, bool kFirstTile>
+__device__ __forceinline__ void reduce_block(
+    const MistProblem &prob, const MistGroupDesc *__restrict__ g, int chunk, int p_tile,
+    int lc_tile, const double *__restrict__ row_terms, double ratio, double *lds_terms,
     double *__restrict__ partial_cost, int32_t *__restrict__ partial_index) {
-  __shared__ double lds_terms[kStageRows * MIST_ROW_TERMS];
-
-  int local_block;
-  const MistGroupDesc *g = find_group(groups, block_prefix, n_groups, blockIdx.x, &local_block);
-  const int chunk = local_block % g->n_chunks;
-  const int tile = local_block / g->n_chunks;
-  const int p_tile = tile % g->n_p_tiles;
-  const int lc_tile = tile / g->n_p_tiles;
-
   const int L = prob.num_layers;
   const int n_pairs = L * (L + 1) / 2 + L;  // sum over l = 1..L of (l + 1)
   const int pair_idx = lc_tile * MIST_LC_TILE + threadIdx.x;
@@ -450,12 +447,13 @@ __global__ __launch_bounds__(MIST_LC_TILE) void eval_reduce_kernel(
   const int n_tile = min(MIST_P_TILE, g->num_p - p0);  // p values of this tile: p0 .. p0+n_tile-1
   int steps = 0;  // bisection steps that separate the n_tile + 1 possible counts
   while ((1 << steps) < n_tile + 1) ++steps;
-  const bool first_p_tile = p_tile == 0;
-  const bool do_nopp = first_p_tile && l == L;
+  const bool do_nopp = kFirstTile && l == L;
   const GroupConsts k = group_consts(g);
   const double cap = prob.mem_cap_mb;
   const double G64 = (double)g->grad_accum;
   const float G32 = (float)g->grad_accum;
+  const double inv_G64 = 1.0 / G64;
+  const float inv_G32 = 1.0f / G32;
   const double pre_saved = g->pre_saved, pre_sas = g->pre_states_and_saved;
   const double pre_states = g->pre_states;
   const double post_states = g->post_states, post_fwd_peak = g->post_fwd_peak;
@@ -470,9 +468,10 @@ __global__ __launch_bounds__(MIST_LC_TILE) void eval_reduce_kernel(
   }
   double best_post = INFINITY, best_pp = INFINITY;
   int32_t row_post = -1, row_pp = -1;
-  // Largest minimum of the tile (slot n_tile - 1): a row that does not beat it cannot change
-  // any slot, because the minima are non-decreasing in p.
-  double top_b = INFINITY, top_p = INFINITY;
+  // The minima of a tile are non-decreasing in p and finite on a prefix [0, fin); `top` is the
+  // largest finite one.  A row that does not beat `top` can only fill the first empty slot.
+  int fin_b = 0, fin_p = 0;
+  double top_b = -INFINITY, top_p = -INFINITY;
 
   const int64_t row_begin = (int64_t)chunk * g->rows_per_chunk;
   const int64_t row_end = min(row_begin + (int64_t)g->rows_per_chunk, g->n_rows);
@@ -482,6 +481,15 @@ __global__ __launch_bounds__(MIST_LC_TILE) void eval_reduce_kernel(
   const double l_minus_c = (double)(l - c), l_minus_c_1 = (double)(l - c - 1);
   const bool c_eq_l = c == l, c_ge_lm1 = c >= l - 1, c_eq_0 = c == 0;
 
+  // get_latencies (:2165-2216): which family member a lane needs is fixed by its (l, c), so the
+  // choice is made once as a column index instead of a per-row select.
+  const int lm2 = max(l - 2, 0);
+  const double n_ck = (double)min(max(c - 1, 0), lm2);
+  const double n_nock = (double)(lm2 - min(max(c - 1, 0), lm2));
+  const int first_col = c_eq_l ? 0 : 1, last_col = c_eq_0 ? 1 : 0;  // *_CK precedes *_NOCK
+  const int post_col = c > 0 ? 0 : 1;
+  auto div_G = [&](double v) { return kPow2G ? v * inv_G64 : v / G64; };
+
   for (int64_t base = row_begin; base < row_end; base += kStageRows) {
     const int n_stage = (int)min((int64_t)kStageRows, row_end - base);
     __syncthreads();
@@ -490,103 +498,154 @@ __global__ __launch_bounds__(MIST_LC_TILE) void eval_reduce_kernel(
     __syncthreads();
     if (!active) continue;
 
-    for (int rr = 0; rr < n_stage; ++rr) {
-      const double *__restrict__ t = lds_terms + rr * MIST_ROW_TERMS;
-      const int32_t row = (int32_t)(base + rr);
-
-      // ---- objective values (mist/utils/pareto.py:138: r * x + y in float64) ----
-      CellLatency lat;
-      if (first_p_tile) lat = cell_latency<true>(t, l, c, k);
-      else lat = cell_latency<false>(t, l, c, k);
-      const float y32 = lat.d / G32;  // float32 array / python int (:2815)
-      const double cost_base = ratio * (double)lat.x + (double)y32;
-      const double cost_pre = ratio * lat.sp + lat.dpre / G64;
-      const bool try_b = cost_base < top_b, try_p = cost_pre < top_p;
-      if (!(try_b || try_p || first_p_tile)) continue;
-
-      // ---- memory that does not depend on p (:2150-2162, 2358-2385, 2760-2769) ----
-      const double S_ck = t[MIST_T_S_CK], S_nock = t[MIST_T_S_NOCK];
-      const double fwd_states = t[MIST_T_FWD_STATES0] + lf * t[MIST_T_PWG] + lm1 * t[MIST_T_PO];
-      const double bwd_states = t[MIST_T_BWD_STATES0] + lf * t[MIST_T_PWGO];
-      const double cur_saved = c_eq_l ? (lf - 1.0) * S_ck : cf * S_ck + l_minus_c_1 * S_nock;
-      const double mod_saved = S_ck * cf + S_nock * l_minus_c;
-      const double ck_delta = c_ge_lm1 ? t[MIST_T_D_CK] : t[MIST_T_D_NOCK];
-      const double fwd_pk = t[MIST_T_FWD_PEAK], bwd_pk = t[MIST_T_BWD_PEAK];
-      const double out = t[MIST_T_OUT], gcb = t[MIST_T_GCB];
-      const double out2 = out * 2.0;
-
-      // Peaks of the middle-stage variant for p pre-saved micro-batches (:2755-2786).
-      auto peaks = [&](int p, double &peak_f, double &peak_b) {
-        const double pf64 = (double)p;
-        const double pipe_saved = pf64 * mod_saved + cur_saved;
-        const double outp2 = out * pf64 * 2.0;
-        peak_f = fwd_states + pipe_saved + ck_delta + fwd_pk + outp2 + gcb;
-        peak_b = bwd_states + pipe_saved + ck_delta + bwd_pk + outp2 + out2 + gcb;
-      };
-
-      if (try_b) {
-        const double mf_base = t[MIST_T_MF_BASE];
-        int lo = 0, hi = n_tile;  // number of feasible p of this tile lies in [lo, hi]
-        for (int it = 0; it < steps; ++it) {
-          const int mid = (lo + hi) >> 1;
-          double pf, pb;
-          peaks(p0 + mid, pf, pb);
-          const bool ok = fmax(pf, pb) * mf_base <= cap;  // (:2805-2812)
-          const bool open = lo < hi;
-          lo = (open && ok) ? mid + 1 : lo;
-          hi = (open && !ok) ? mid : hi;
-        }
+    for (int r0 = 0; r0 < n_stage; r0 += kRowUnroll) {
+      // ---- latencies and objective values of kRowUnroll rows (:2165-2351; pareto.py:138:
+      // r * x + y in float64).  Independent of the running minima, hence computed together;
+      // rows past the end of the stage read stale LDS and are ignored below. ----
+      double cost_base[kRowUnroll], cost_pre[kRowUnroll], cost_post[kRowUnroll],
+          cost_pp[kRowUnroll];
 #pragma unroll
-        for (int j = 0; j < MIST_P_TILE; ++j) {
-          const bool better = j < lo && cost_base < best_b[j];
-          best_b[j] = better ? cost_base : best_b[j];
-          row_b[j] = better ? row : row_b[j];
+      for (int u = 0; u < kRowUnroll; ++u) {
+        const double *__restrict__ t = lds_terms + min(r0 + u, kStageRows - 1) * MIST_ROW_TERMS;
+        const double stable = n_ck * t[MIST_T_S_LAYER_CK] + n_nock * t[MIST_T_S_LAYER_NOCK] +
+                              t[MIST_T_S_FIRST_CK + first_col] + t[MIST_T_S_LAST_CK + last_col];
+        const double delta = n_ck * t[MIST_T_D_LAYER_CK] + n_nock * t[MIST_T_D_LAYER_NOCK] +
+                             t[MIST_T_D_FIRST_CK + first_col] + t[MIST_T_D_LAST_CK + last_col];
+        const float x32 = (float)stable, d32 = (float)delta;  // (:2212-2213)
+        const double x = (double)x32, d = (double)d32;
+        const float y32 = kPow2G ? d32 * inv_G32 : d32 / G32;  // float32 array / python int (:2815)
+        cost_base[u] = ratio * x + (double)y32;
+        cost_pre[u] = ratio * (x + k.pre_fwd + k.pre_bwd + k.w1 + k.w2) + div_G(d + k.w1d + k.w2d);
+        if (kFirstTile) {
+          const double nag = t[MIST_T_NAG_CK + post_col], nrs = t[MIST_T_NRS_CK + post_col];
+          const double ps1 = k.pp_wre ? nag : 0.0, ps2 = k.pp_gre ? nrs : 0.0;
+          const double pd1 = k.pp_wre ? 0.0 : nag, pd2 = k.pp_gre ? 0.0 : nrs;
+          const double opb = t[MIST_T_OPB];
+          cost_post[u] = ratio * (x + k.post_fwd + opb + ps1 + ps2) + div_G(d + pd1 + pd2);
+          cost_pp[u] =
+              ratio * (x + k.pre_fwd + k.pre_bwd + k.post_fwd + opb + k.w1 + k.w2 + ps1 + ps2) +
+              div_G(d + k.w1d + k.w2d + pd1 + pd2);
+        } else {
+          cost_post[u] = cost_pp[u] = 0.0;
         }
-        top_b = (n_tile <= lo) ? cost_base : top_b;  // slot n_tile - 1 was among the updated
-      }
-      if (try_p) {
-        const double mf_pp = t[MIST_T_MF_PP];
-        int lo = 0, hi = n_tile;
-        for (int it = 0; it < steps; ++it) {
-          const int mid = (lo + hi) >> 1;
-          double pf, pb;
-          peaks(p0 + mid, pf, pb);
-          const double pre_p = (double)(p0 + mid) * pre_saved;  // (:2866-2875)
-          const double pf_pre = pre_p + pf + pre_sas;
-          const double pb_pre = pre_p + pb + pre_sas;
-          const bool ok = fmax(pf_pre, pb_pre) * mf_pp <= cap;  // (:2893-2897)
-          const bool open = lo < hi;
-          lo = (open && ok) ? mid + 1 : lo;
-          hi = (open && !ok) ? mid : hi;
-        }
-#pragma unroll
-        for (int j = 0; j < MIST_P_TILE; ++j) {
-          const bool better = j < lo && cost_pre < best_p[j];
-          best_p[j] = better ? cost_pre : best_p[j];
-          row_p[j] = better ? row : row_p[j];
-        }
-        top_p = (n_tile <= lo) ? cost_pre : top_p;
       }
 
-      if (first_p_tile) {
-        // ---- last stage / single stage, p == 0 only (:2946-3106) ----
-        double peak_f, peak_b;
-        peaks(0, peak_f, peak_b);
-        const double mf_pp = t[MIST_T_MF_PP];
-        const double f_in = fwd_states + post_states + mod_saved + post_fwd_peak + gcb;
-        const double b_in = bwd_states + post_states + mod_saved + post_bwd_peak +
-                            (c_eq_0 ? t[MIST_T_RD] : 0.0) + gcb;
-        const double pf_post = fmax(f_in, peak_f + post_states);
-        const double pb_post = fmax(b_in, peak_b - out + post_states) + post_output;
-        const bool ok_post = fmax(pf_post, pb_post) * mf_pp <= cap;
-        const double cost_post = ratio * lat.spost + lat.dpost / G64;
-        take_min(best_post, row_post, ok_post, cost_post, row);
-        if (do_nopp) {
-          const double pf_pp = pf_post + pre_states + pre_saved;
-          const double pb_pp = pb_post + pre_states + pre_saved;
-          const bool ok_pp = fmax(pf_pp, pb_pp) * t[MIST_T_MF] <= cap;
-          const double cost_pp = ratio * lat.spp + lat.dpp / G64;
-          take_min(best_pp, row_pp, ok_pp, cost_pp, row);
+#pragma unroll
+      for (int u = 0; u < kRowUnroll; ++u) {
+        if (r0 + u >= n_stage) break;
+        const double *__restrict__ t = lds_terms + (r0 + u) * MIST_ROW_TERMS;
+        const int32_t row = (int32_t)(base + r0 + u);
+        // Lowest slot the row could improve: the minima are non-decreasing in p, so it is the
+        // number of slots whose minimum the row does not beat (empty slots hold +inf).  The row
+        // changes something iff it is feasible at that slot (feasibility is monotone in p).
+        int lo_b = fin_b, lo_p = fin_p;
+        if (cost_base[u] < top_b) {
+          lo_b = 0;
+#pragma unroll
+          for (int j = 0; j < MIST_P_TILE; ++j) lo_b += cost_base[u] >= best_b[j] ? 1 : 0;
+        }
+        if (cost_pre[u] < top_p) {
+          lo_p = 0;
+#pragma unroll
+          for (int j = 0; j < MIST_P_TILE; ++j) lo_p += cost_pre[u] >= best_p[j] ? 1 : 0;
+        }
+        bool need_b = lo_b < n_tile, need_p = lo_p < n_tile;
+        const bool need_post = kFirstTile && cost_post[u] < best_post;
+        const bool need_pp = do_nopp && cost_pp[u] < best_pp;
+        if (!(need_b || need_p || need_post || need_pp)) continue;
+
+        // ---- memory that does not depend on p (:2150-2162, 2358-2385, 2760-2769) ----
+        const double S_ck = t[MIST_T_S_CK], S_nock = t[MIST_T_S_NOCK];
+        const double fwd_states = t[MIST_T_FWD_STATES0] + lf * t[MIST_T_PWG] + lm1 * t[MIST_T_PO];
+        const double bwd_states = t[MIST_T_BWD_STATES0] + lf * t[MIST_T_PWGO];
+        const double cur_saved = c_eq_l ? (lf - 1.0) * S_ck : cf * S_ck + l_minus_c_1 * S_nock;
+        const double mod_saved = S_ck * cf + S_nock * l_minus_c;
+        const double ck_delta = c_ge_lm1 ? t[MIST_T_D_CK] : t[MIST_T_D_NOCK];
+        const double fwd_pk = t[MIST_T_FWD_PEAK], bwd_pk = t[MIST_T_BWD_PEAK];
+        const double out = t[MIST_T_OUT], gcb = t[MIST_T_GCB];
+        const double out2 = out * 2.0;
+        const double mf_base = t[MIST_T_MF_BASE], mf_pp = t[MIST_T_MF_PP];
+
+        // Peaks of the middle-stage variant for p pre-saved micro-batches (:2755-2786).
+        auto peaks = [&](int p, double &peak_f, double &peak_b) {
+          const double pf64 = (double)p;
+          const double pipe_saved = pf64 * mod_saved + cur_saved;
+          const double outp2 = out * pf64 * 2.0;
+          peak_f = fwd_states + pipe_saved + ck_delta + fwd_pk + outp2 + gcb;
+          peak_b = bwd_states + pipe_saved + ck_delta + bwd_pk + outp2 + out2 + gcb;
+        };
+        auto feasible_base = [&](int p) {  // (:2805-2812)
+          double pf, pb;
+          peaks(p, pf, pb);
+          return fmax(pf, pb) * mf_base <= cap;
+        };
+        auto feasible_pre = [&](int p) {  // (:2866-2875, 2893-2897)
+          double pf, pb;
+          peaks(p, pf, pb);
+          const double pre_p = (double)p * pre_saved;
+          return fmax(pre_p + pf + pre_sas, pre_p + pb + pre_sas) * mf_pp <= cap;
+        };
+
+        need_b = need_b && feasible_base(p0 + lo_b);
+        need_p = need_p && feasible_pre(p0 + lo_p);
+
+        if (need_b) {
+          const double cost = cost_base[u];
+          int lo = lo_b + 1, hi = n_tile;  // number of feasible p of this tile lies in [lo, hi]
+          for (int it = 0; it < steps; ++it) {
+            const int mid = (lo + hi) >> 1;
+            const bool ok = feasible_base(p0 + mid);
+            const bool open = lo < hi;
+            lo = (open && ok) ? mid + 1 : lo;
+            hi = (open && !ok) ? mid : hi;
+          }
+#pragma unroll
+          for (int j = 0; j < MIST_P_TILE; ++j) {
+            const bool better = j >= lo_b && j < lo;  // exactly the slots with cost < minimum
+            best_b[j] = better ? cost : best_b[j];
+            row_b[j] = better ? row : row_b[j];
+          }
+          // Bookkeeping of (fin, top) without indexing the register array dynamically.
+          if (lo > fin_b) { fin_b = lo; top_b = cost; }
+          else if (lo == fin_b && cost < top_b) top_b = cost;
+        }
+        if (need_p) {
+          const double cost = cost_pre[u];
+          int lo = lo_p + 1, hi = n_tile;
+          for (int it = 0; it < steps; ++it) {
+            const int mid = (lo + hi) >> 1;
+            const bool ok = feasible_pre(p0 + mid);
+            const bool open = lo < hi;
+            lo = (open && ok) ? mid + 1 : lo;
+            hi = (open && !ok) ? mid : hi;
+          }
+#pragma unroll
+          for (int j = 0; j < MIST_P_TILE; ++j) {
+            const bool better = j >= lo_p && j < lo;
+            best_p[j] = better ? cost : best_p[j];
+            row_p[j] = better ? row : row_p[j];
+          }
+          if (lo > fin_p) { fin_p = lo; top_p = cost; }
+          else if (lo == fin_p && cost < top_p) top_p = cost;
+        }
+
+        if (need_post || need_pp) {
+          // ---- last stage / single stage, p == 0 only (:2946-3106) ----
+          double peak_f, peak_b;
+          peaks(0, peak_f, peak_b);
+          const double f_in = fwd_states + post_states + mod_saved + post_fwd_peak + gcb;
+          const double b_in = bwd_states + post_states + mod_saved + post_bwd_peak +
+                              (c_eq_0 ? t[MIST_T_RD] : 0.0) + gcb;
+          const double pf_post = fmax(f_in, peak_f + post_states);
+          const double pb_post = fmax(b_in, peak_b - out + post_states) + post_output;
+          const bool ok_post = fmax(pf_post, pb_post) * mf_pp <= cap;
+          take_min(best_post, row_post, need_post && ok_post, cost_post[u], row);
+          if (need_pp) {
+            const double pf_pp = pf_post + pre_states + pre_saved;
+            const double pb_pp = pb_post + pre_states + pre_saved;
+            const bool ok_pp = fmax(pf_pp, pb_pp) * t[MIST_T_MF] <= cap;
+            take_min(best_pp, row_pp, ok_pp, cost_pp[u], row);
+          }
         }
       }
     }
@@ -604,6 +663,29 @@ __global__ __launch_bounds__(MIST_LC_TILE) void eval_reduce_kernel(
   partial_index[out_base + (int64_t)(2 * MIST_P_TILE) * MIST_LC_TILE] = row_post;
   partial_cost[out_base + (int64_t)(2 * MIST_P_TILE + 1) * MIST_LC_TILE] = best_pp;
   partial_index[out_base + (int64_t)(2 * MIST_P_TILE + 1) * MIST_LC_TILE] = row_pp;
+}
+
+__global__ __launch_bounds__(MIST_LC_TILE, 2) void eval_reduce_kernel(
+    const MistProblem prob, const MistGroupDesc *__restrict__ groups, int n_groups,
+    const int32_t *__restrict__ block_prefix, const double *__restrict__ row_terms, double ratio,
+    double *__restrict__ partial_cost, int32_t *__restrict__ partial_index) {
+  __shared__ double lds_terms[kStageRows * MIST_ROW_TERMS];
+  int local_block;
+  const MistGroupDesc *g = find_group(groups, block_prefix, n_groups, blockIdx.x, &local_block);
+  const int chunk = local_block % g->n_chunks;
+  const int tile = local_block / g->n_chunks;
+  const int p_tile = tile % g->n_p_tiles;
+  const int lc_tile = tile / g->n_p_tiles;
+  const bool pow2 = (g->grad_accum & (g->grad_accum - 1)) == 0;
+#define MIST_REDUCE(P2, FT)                                                                   \
+  reduce_block<P2, FT>(prob, g, chunk, p_tile, lc_tile, row_terms, ratio, lds_terms,          \
+                       partial_cost, partial_index)
+  if (pow2) {
+    if (p_tile == 0) MIST_REDUCE(true, true); else MIST_REDUCE(true, false);
+  } else {
+    if (p_tile == 0) MIST_REDUCE(false, true); else MIST_REDUCE(false, false);
+  }
+#undef MIST_REDUCE
 }
 
 // ------------------------------------------------------------------------------------------

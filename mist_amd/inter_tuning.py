@@ -45,10 +45,12 @@ class _DpRunner:
     def __init__(self, results: IntraStageTunerOutput, num_layers: int, num_devices: int,
                  meshes: List[Tuple[int, int]], slot: int):
         self.lib = _lib.load()
-        dev_tabs = results.device
+        dev_tabs = results.batch  # tables of every tp candidate of the same launch
         self.device = dev_tabs.stable[0].device
-        Gs = results.gradient_accumulation_steps_candidates
         Gn, Q, P1, L, C, S = dev_tabs.stable[0].shape
+        n_g = len(results.gradient_accumulation_steps_candidates)
+        assert Gn % n_g == 0
+        Gs = list(results.gradient_accumulation_steps_candidates) * (Gn // n_g)
         assert L == num_layers and C == L + 1
         if list(meshes) != list(results.device_mesh_candidates):
             raise ValueError("the DP needs the mesh list the intra-stage tables were built for")
@@ -87,7 +89,9 @@ class _DpRunner:
         """Per g: ascending unique finite stage costs (inter_tuning.py:180-186) after the gap
         rule (:198), float32.  One device sort for all g, the sequential rule on the host."""
         allv = torch.cat([self.cost[v].reshape(self.Gn, -1) for v in range(3)], dim=1)
-        host = torch.sort(allv, dim=1).values.cpu().numpy()  # +inf sorts last
+        n_fin = int(torch.isfinite(allv).sum(dim=1).max().item())
+        # +inf sorts last: only the finite prefix is copied to the host
+        host = torch.sort(allv, dim=1).values[:, :max(n_fin, 1)].contiguous().cpu().numpy()
         out = []
         kept = np.empty(host.shape[1], dtype=np.float32)
         for g in range(self.Gn):
@@ -115,7 +119,7 @@ class _DpRunner:
             scratch = torch.empty(4 * n * self.plane, dtype=torch.float32, device=dev)
             argmin = None
             if want_argmin:
-                argmin = torch.full((self.S_max + 1, self.L + 1, self.D + 1, 4), -1,
+                argmin = torch.full((n, self.S_max + 1, self.L + 1, self.D + 1, 4), -1,
                                     dtype=torch.int32, device=dev)
             rc = self.lib.mist_dp_run(
                 ctypes.c_void_p(self.shape.ctypes.data), ctypes.byref(self.costs_struct),
@@ -217,6 +221,146 @@ def get_solution_from_intra_stage_tuner_output(
     return r.solution_at(0, (g, q, p, l - 1, c, slot))
 
 
+def _same_batch(results_list) -> bool:
+    first = results_list[0]
+    return all(
+        r.batch is first.batch and r.batch_index == i for i, r in enumerate(results_list)
+    ) and first.batch.stable[0].shape[0] == len(results_list) * len(first.gradient_accumulation_steps_candidates)
+
+
+def inter_stage_tune_batch(
+    num_layers: int,
+    num_devices: int,
+    device_mesh_candidates: List[Tuple[int, int]],
+    gradient_accumulation_steps_candidates: List[int],
+    results_list: List[IntraStageTunerOutput],
+    slot: int = 0,
+    stats: Optional[dict] = None,
+):
+    """``inter_stage_tune`` for several intra-stage results at once (the tensor-parallel
+    candidates of one ``tune`` call).  Each entry is searched exactly as if it were alone (its
+    own running best, its own stop rule); only the launches are shared.  Returns a list of
+    ``(best_cost, best_solution)``."""
+    for r in results_list:
+        if not isinstance(r, IntraStageTunerOutput):
+            raise TypeError(
+                f"intra_stage_results must be an instance of IntraStageTunerOutput, got {type(r)}"
+            )
+    if not _same_batch(results_list):
+        out = []
+        for r in results_list:
+            one = r if r.batch is r.device else IntraStageTunerOutput(
+                r.gradient_accumulation_steps_candidates, r.device_mesh_candidates, r.device,
+                r.spaces, r.sample_slots)
+            out += inter_stage_tune_batch(num_layers, num_devices, device_mesh_candidates,
+                                          gradient_accumulation_steps_candidates, [one], slot, stats)
+        return out
+    t_start = time.perf_counter()
+    first = results_list[0]
+    runner = _DpRunner(first, num_layers, num_devices, device_mesh_candidates, slot)
+    n_g = len(first.gradient_accumulation_steps_candidates)
+    g_index = {G: i for i, G in enumerate(first.gradient_accumulation_steps_candidates)}
+    q_index = {q: i for i, q in enumerate(first.device_mesh_candidates)}
+    Gs = list(gradient_accumulation_steps_candidates)
+    n_inst = len(results_list)
+    # table row of (instance, G)
+    rows = np.array([[t * n_g + g_index[G] for G in Gs] for t in range(n_inst)], dtype=np.int32)
+    t_0 = time.perf_counter()
+    tmax_all = runner.thresholds()
+    t_1 = time.perf_counter()
+
+    # Smallest feasible threshold of every (instance, G) in one launch (bottleneck DP).
+    flat = rows.reshape(-1)
+    _, bottleneck, _ = runner.run(flat, np.zeros(len(flat), dtype=np.float32), _lib.DP_BOTTLENECK)
+    bottleneck = bottleneck.reshape(rows.shape)
+    chains = []
+    for t in range(n_inst):
+        scans = []
+        for i, G in enumerate(Gs):
+            tmax = tmax_all[rows[t, i]]
+            b = bottleneck[t, i]
+            start = int(np.searchsorted(tmax, b, side="left")) if np.isfinite(b) else len(tmax)
+            scans.append(_Scan(G, tmax, start))
+        chains.append(dict(scans=scans, current=0, best=(float("inf"), None, None)))
+
+    # Speculative batches + sequential replay (see the module docstring).
+    while True:
+        req_g, req_t, req_span = [], [], []
+        for t, ch in enumerate(chains):
+            scans = ch["scans"]
+            best_cost, best_G, best_t = ch["best"]
+            while ch["current"] < len(scans):  # commit the sequential scan as far as results allow
+                sc = scans[ch["current"]]
+                cost, tt, finished = sc.replay(best_cost, None)
+                if tt is not None:
+                    best_cost, best_G, best_t = cost, sc.G, tt
+                if not finished:
+                    break
+                ch["current"] += 1
+            ch["best"] = (best_cost, best_G, best_t)
+            for i in range(ch["current"], len(scans)):
+                sc = scans[i]
+                if i > ch["current"] and not sc.runs_out(best_cost):
+                    continue
+                a, b = sc.wanted(best_cost)
+                if b > a:
+                    req_g.append(np.full(b - a, rows[t, i], dtype=np.int32))
+                    req_t.append(sc.tmax[a:b])
+                    req_span.append((t, i, b - a))
+        if all(ch["current"] == len(ch["scans"]) for ch in chains):
+            break
+        if not req_span:
+            raise RuntimeError("inter-stage scan made no progress")  # cannot happen: guards a hang
+        bs, bsum, smax = runner.run(np.concatenate(req_g), np.concatenate(req_t))
+        off = 0
+        for t, i, n in req_span:
+            chains[t]["scans"][i].add(bs[off:off + n], bsum[off:off + n], smax[off:off + n])
+            off += n
+    t_2 = time.perf_counter()
+
+    # Back-pointers of each winning (G, t_max) run (inter_tuning.py:341-355), one launch.
+    winners = [t for t, ch in enumerate(chains) if ch["best"][1] is not None]
+    back = {}
+    if winners:
+        w_rows = np.array([t * n_g + g_index[chains[t]["best"][1]] for t in winners], dtype=np.int32)
+        w_tmax = np.array([chains[t]["best"][2] for t in winners], dtype=np.float32)
+        best_s, _, _, argmin = runner.run(w_rows, w_tmax, want_argmin=True)
+        back = {t: (int(best_s[i]), argmin[i]) for i, t in enumerate(winners)}
+    out = []
+    for t, ch in enumerate(chains):
+        best_cost, best_G, best_t = ch["best"]
+        if best_G is None:
+            out.append((float("inf"), None))
+            continue
+        r = results_list[t]
+        g = g_index[best_G]
+        cs, argmin = back[t]
+        cl, cd = 0, num_devices
+        inter = []
+        while cs > 0 and cl < num_layers and cd > 0:
+            end, n, m, ckpt = (int(v) for v in argmin[cs, cl, cd])
+            assert end != -1
+            inter.append(((cl, end), (n, m), ckpt))
+            cs, cl, cd = cs - 1, end + 1, cd - n * m
+        assert cs == 0 and cl == num_layers and cd == 0
+        solution = [best_G, []]
+        for i, ((l0, l1), (n, m), ckpt) in enumerate(inter):
+            row = get_solution_from_intra_stage_tuner_output(
+                r, num_layers, g, len(inter) - i - 1, l0, l1, q_index[(n, m)], ckpt, slot
+            ).tolist()
+            row[:6] = [int(x) for x in row[:6]]
+            solution[1].append((((l0, l1), (n, m), ckpt, 0), tuple(row)))
+        out.append((best_cost, solution))
+    if stats is not None:
+        stats["dp_setup_s"] = stats.get("dp_setup_s", 0.0) + (t_0 - t_start)
+        stats["dp_thresholds_s"] = stats.get("dp_thresholds_s", 0.0) + (t_1 - t_0)
+        stats["dp_scan_s"] = stats.get("dp_scan_s", 0.0) + (t_2 - t_1)
+        stats["dp_backtrack_s"] = stats.get("dp_backtrack_s", 0.0) + (time.perf_counter() - t_2)
+        stats["dp_launches"] = stats.get("dp_launches", 0) + runner.launches
+        stats["dp_thresholds"] = stats.get("dp_thresholds", 0) + runner.thresholds_run
+    return out
+
+
 def inter_stage_tune(
     num_layers: int,
     num_devices: int,
@@ -228,88 +372,7 @@ def inter_stage_tune(
 ):
     """Reference signature (inter_tuning.py:63-69).  Returns ``(best_cost, [G, [(((l0, l1),
     (n, m), ckpt, 0), strategy_row), ...]])`` or ``(inf, None)`` when nothing is feasible."""
-    if not isinstance(intra_stage_results, IntraStageTunerOutput):
-        raise TypeError(
-            f"intra_stage_results must be an instance of IntraStageTunerOutput, got {type(intra_stage_results)}"
-        )
-    t_start = time.perf_counter()
-    runner = _DpRunner(intra_stage_results, num_layers, num_devices, device_mesh_candidates, slot)
-    g_index = {G: i for i, G in enumerate(intra_stage_results.gradient_accumulation_steps_candidates)}
-    q_index = {q: i for i, q in enumerate(intra_stage_results.device_mesh_candidates)}
-    Gs = list(gradient_accumulation_steps_candidates)
-    gs = np.array([g_index[G] for G in Gs], dtype=np.int32)
-    t_0 = time.perf_counter()
-    tmax_all = runner.thresholds()
-    t_1 = time.perf_counter()
-
-    # Smallest feasible threshold of every G in one launch (bottleneck DP).
-    _, bottleneck, _ = runner.run(gs, np.zeros(len(Gs), dtype=np.float32), _lib.DP_BOTTLENECK)
-    scans = []
-    for i, G in enumerate(Gs):
-        tmax = tmax_all[gs[i]]
-        first = int(np.searchsorted(tmax, bottleneck[i], side="left")) if np.isfinite(bottleneck[i]) else len(tmax)
-        scans.append(_Scan(G, tmax, first))
-
-    # Speculative batches + sequential replay.  A bound on the running best that the sequential
-    # scan is certain to have reached decides how much of each G is worth computing ahead; the
-    # replay then applies the reference's rules in order and asks for more where it runs out.
-    best_cost, best_G, best_t = float("inf"), None, None
-    current = 0  # scans[:current] are finished
-    while True:
-        while current < len(scans):  # commit the sequential scan as far as results allow
-            sc = scans[current]
-            cost, t, finished = sc.replay(best_cost, None)
-            if t is not None:
-                best_cost, best_G, best_t = cost, sc.G, t
-            if not finished:
-                break
-            current += 1
-        if current == len(scans):
-            break
-        req_g, req_t, req_span = [], [], []
-        for i in range(current, len(scans)):
-            sc = scans[i]
-            if i > current and not sc.runs_out(best_cost):
-                continue
-            a, b = sc.wanted(best_cost)
-            if b > a:
-                req_g.append(np.full(b - a, gs[i], dtype=np.int32))
-                req_t.append(sc.tmax[a:b])
-                req_span.append((i, b - a))
-        if not req_span:
-            raise RuntimeError("inter-stage scan made no progress")  # cannot happen: guards a hang
-        bs, bsum, smax = runner.run(np.concatenate(req_g), np.concatenate(req_t))
-        off = 0
-        for i, n in req_span:
-            scans[i].add(bs[off:off + n], bsum[off:off + n], smax[off:off + n])
-            off += n
-    t_2 = time.perf_counter()
-    if stats is not None:
-        stats["dp_setup_s"] = stats.get("dp_setup_s", 0.0) + (t_0 - t_start)
-        stats["dp_thresholds_s"] = stats.get("dp_thresholds_s", 0.0) + (t_1 - t_0)
-        stats["dp_scan_s"] = stats.get("dp_scan_s", 0.0) + (t_2 - t_1)
-        stats["dp_launches"] = stats.get("dp_launches", 0) + runner.launches
-        stats["dp_thresholds"] = stats.get("dp_thresholds", 0) + runner.thresholds_run
-    if best_G is None:
-        return float("inf"), None
-
-    # Back-pointers of the winning (G, t_max) run (inter_tuning.py:341-355).
-    g = g_index[best_G]
-    best_s, best_sum, stage_max, argmin = runner.run(
-        np.array([g], dtype=np.int32), np.array([best_t], dtype=np.float32), want_argmin=True)
-    cs, cl, cd = int(best_s[0]), 0, num_devices
-    inter = []
-    while cs > 0 and cl < num_layers and cd > 0:
-        end, n, m, ckpt = (int(v) for v in argmin[cs, cl, cd])
-        assert end != -1
-        inter.append(((cl, end), (n, m), ckpt))
-        cs, cl, cd = cs - 1, end + 1, cd - n * m
-    assert cs == 0 and cl == num_layers and cd == 0
-    solution = [best_G, []]
-    for i, ((l0, l1), (n, m), ckpt) in enumerate(inter):
-        row = get_solution_from_intra_stage_tuner_output(
-            intra_stage_results, num_layers, g, len(inter) - i - 1, l0, l1, q_index[(n, m)], ckpt, slot
-        ).tolist()
-        row[:6] = [int(x) for x in row[:6]]
-        solution[1].append((((l0, l1), (n, m), ckpt, 0), tuple(row)))
-    return best_cost, solution
+    return inter_stage_tune_batch(
+        num_layers, num_devices, device_mesh_candidates, gradient_accumulation_steps_candidates,
+        [intra_stage_results], slot, stats,
+    )[0]

@@ -67,12 +67,18 @@ class IntraStageTunerOutput:
         device: DeviceTables,
         spaces: Dict[Tuple[int, int], SearchSpace],
         sample_slots: Sequence[int],
+        batch: Optional[DeviceTables] = None,
+        batch_index: int = 0,
     ):
         self.gradient_accumulation_steps_candidates = list(gradient_accumulation_steps_candidates)
         self.device_mesh_candidates = list(device_mesh_candidates)
         self.device = device
         self.spaces = spaces
         self.sample_slots = tuple(sample_slots)
+        # Tables of every tensor-parallel candidate evaluated in the same launch (leading axis
+        # = batch_index * len(G candidates) + g); ``device`` is this candidate's slice of them.
+        self.batch = device if batch is None else batch
+        self.batch_index = batch_index
         self._host: Dict[str, np.ndarray] = {}
 
     def _fetch(self, kind: str, v: int) -> np.ndarray:
@@ -147,6 +153,8 @@ class IntraStageTuner:
         self.device_mesh_candidates = list(device_mesh_candidates)
         self.gradient_accumulation_steps_candidates = list(gradient_accumulation_steps_candidates)
         self.tp_size = tp_size
+        # A list of tp sizes evaluates all of them in one batch of launches (``tune_all``).
+        self.tp_sizes = list(tp_size) if isinstance(tp_size, (list, tuple)) else [tp_size]
         self.config = config
         self.sample_size = int(sample_size)
         # Which of the S alpha samples to evaluate (default: all); unevaluated slots stay inf / -1.
@@ -170,21 +178,22 @@ class IntraStageTuner:
         Gs, Q = self.gradient_accumulation_steps_candidates, self.device_mesh_candidates
         P = self.max_possible_pre_saved_micro_batches
         builder = GroupInputBuilder(cfg, self.layer_tables)
-        spaces: Dict[Tuple[int, int], SearchSpace] = {}
+        spaces: Dict[Tuple[int, int, int], SearchSpace] = {}
         pending = []
-        for g, G in enumerate(Gs):
-            for q, (n, m) in enumerate(Q):
-                space = create_search_space_for_a_block_layer(
-                    n, m, cfg.training.global_batch_size, G, cfg,
-                    constraint_fn=self.layer_tables.constraint, tp_size=self.tp_size,
-                )
-                spaces[(g, q)] = space
-                if space.n_rows == 0:
-                    continue  # the reference returns all-inf tables for an empty space (:648-666)
-                if space.n_rows >= 2**31:
-                    raise ValueError(f"group (G={G}, mesh={(n, m)}) has {space.n_rows} rows (>= 2**31)")
-                num_p = min(G, L, P + 1)  # intra_tuning.py:185-193
-                pending.append((g, q, n, m, G, num_p, space))
+        for t, tp_size in enumerate(self.tp_sizes):
+            for g, G in enumerate(Gs):
+                for q, (n, m) in enumerate(Q):
+                    space = create_search_space_for_a_block_layer(
+                        n, m, cfg.training.global_batch_size, G, cfg,
+                        constraint_fn=self.layer_tables.constraint, tp_size=tp_size,
+                    )
+                    spaces[(t, g, q)] = space
+                    if space.n_rows == 0:
+                        continue  # the reference returns all-inf tables for an empty space (:648-666)
+                    if space.n_rows >= 2**31:
+                        raise ValueError(f"group (G={G}, mesh={(n, m)}) has {space.n_rows} rows (>= 2**31)")
+                    num_p = min(G, L, P + 1)  # intra_tuning.py:185-193
+                    pending.append((t * len(Gs) + g, q, n, m, G, num_p, space))
         groups = np.zeros(len(pending), dtype=_lib.GROUP_DTYPE)
         for i, (g, q, n, m, G, num_p, space) in enumerate(pending):
             builder.fill(groups[i], space, g, q, n, m, G, num_p)
@@ -209,7 +218,7 @@ class IntraStageTuner:
         reduce_prefix = np.concatenate(([0], np.cumsum(reduce_blocks))).astype(np.int64)
         if terms_prefix[-1] >= 2**31 or reduce_prefix[-1] >= 2**31:
             raise ValueError("launch decomposition exceeds 2**31 workgroups")
-        problem = make_problem(cfg, L, P + 1, self.sample_size, len(Gs), len(Q))
+        problem = make_problem(cfg, L, P + 1, self.sample_size, len(self.tp_sizes) * len(Gs), len(Q))
         return dict(
             problem=problem, groups=groups, spaces=spaces,
             terms_prefix=terms_prefix.astype(np.int32), reduce_prefix=reduce_prefix.astype(np.int32),
@@ -217,7 +226,8 @@ class IntraStageTuner:
         )
 
     def allocate_tables(self) -> DeviceTables:
-        Gn, Qn = len(self.gradient_accumulation_steps_candidates), len(self.device_mesh_candidates)
+        Gn = len(self.tp_sizes) * len(self.gradient_accumulation_steps_candidates)
+        Qn = len(self.device_mesh_candidates)
         P1, L, S = self.max_possible_pre_saved_micro_batches + 1, self.num_layers, self.sample_size
         shapes = [(Gn, Qn, P1, L, L + 1, S), (Gn, Qn, P1, L, L + 1, S), (Gn, Qn, L, L + 1, S), (Gn, Qn, L + 1, S)]
         dev = self.device
@@ -292,31 +302,44 @@ class IntraStageTuner:
                 _ptr(d["row_terms"]), _ptr(d["partial_cost"]), _ptr(d["partial_index"]), int(slot),
                 ctypes.byref(out), stream))
 
-    def run_prepared(self, plan, dev_plan) -> IntraStageTunerOutput:
-        """Device part only: fresh output tables + kernel launches for an uploaded plan."""
+    def _outputs(self, plan, tables: DeviceTables) -> List[IntraStageTunerOutput]:
+        Gn = len(self.gradient_accumulation_steps_candidates)
+        outs = []
+        for t in range(len(self.tp_sizes)):
+            view = DeviceTables(
+                stable=[x[t * Gn:(t + 1) * Gn] for x in tables.stable],
+                delta=[x[t * Gn:(t + 1) * Gn] for x in tables.delta],
+                index=[x[t * Gn:(t + 1) * Gn] for x in tables.index],
+            )
+            spaces = {(g, q): sp for (tt, g, q), sp in plan["spaces"].items() if tt == t}
+            outs.append(IntraStageTunerOutput(
+                self.gradient_accumulation_steps_candidates, self.device_mesh_candidates, view,
+                spaces, self.sample_slots, batch=tables, batch_index=t,
+            ))
+        return outs
+
+    def run_prepared(self, plan, dev_plan) -> List[IntraStageTunerOutput]:
+        """Device part only: fresh output tables + kernel launches for an uploaded plan; one
+        output per tp size, all resident in the same tables."""
         with torch.cuda.device(self.device):
             tables = self.allocate_tables()
             self.launch(plan, dev_plan, tables)
-        self.results = IntraStageTunerOutput(
-            self.gradient_accumulation_steps_candidates, self.device_mesh_candidates, tables,
-            plan["spaces"], self.sample_slots,
-        )
-        return self.results
+        return self._outputs(plan, tables)
 
-    def tune(self) -> IntraStageTunerOutput:
+    def tune_all(self) -> List[IntraStageTunerOutput]:
         if self.device.type != "cuda" or not torch.cuda.is_available():
             raise _lib.MistLibraryError("IntraStageTuner needs a GPU: the search kernels have no CPU path")
         _lib.load()
         plan = self.prepare()
         with torch.cuda.device(self.device):
             dev_plan = self.upload(plan)
-            tables = self.allocate_tables()
-            self.launch(plan, dev_plan, tables)
         self._plan, self._dev_plan = plan, dev_plan
-        self.results = IntraStageTunerOutput(
-            self.gradient_accumulation_steps_candidates, self.device_mesh_candidates, tables,
-            plan["spaces"], self.sample_slots,
-        )
+        return self.run_prepared(plan, dev_plan)
+
+    def tune(self) -> IntraStageTunerOutput:
+        if len(self.tp_sizes) != 1:
+            raise ValueError("tune() returns one table set; use tune_all() for several tp sizes")
+        self.results = self.tune_all()[0]
         return self.results
 
 

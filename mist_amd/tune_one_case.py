@@ -30,7 +30,7 @@ import torch
 import yaml
 
 from .config import OFFLOADING_RATIO_CANDIDATES, MistConfig, tp_candidates
-from .inter_tuning import inter_stage_tune
+from .inter_tuning import inter_stage_tune, inter_stage_tune_batch
 from .inter_tuning_uniform import inter_stage_tune as inter_stage_tune_uniform
 from .intra_tuning import SAMPLE_SIZE, IntraStageTuner, intra_stage_tune
 from .layer_tables import LayerTables
@@ -112,47 +112,44 @@ class PreparedSearch:
         # The reference forwards tuning.sample_size only on its MIP branch; the uniform
         # branch runs with the default of 30 and reads sample 0 (:206-217).
         sample_size = tuning.sample_size if self.granularity == "inter-stage" else SAMPLE_SIZE
-        self.tuners = []
-        for tp_size in tp_candidates(mist_config):
-            tuner = IntraStageTuner(self.tables, self.L, self.meshes, self.Gs, tp_size, mist_config,
-                                    sample_size=sample_size, sample_slots=[0], device=device)
-            plan = tuner.prepare()
-            with torch.cuda.device(tuner.device):
-                dev_plan = tuner.upload(plan)
-            self.tuners.append((tuner, plan, dev_plan))
+        # All tensor-parallel candidates go through one batch of launches.
+        self.tuner = IntraStageTuner(self.tables, self.L, self.meshes, self.Gs,
+                                     tp_candidates(mist_config), mist_config,
+                                     sample_size=sample_size, sample_slots=[0], device=device)
+        self.plan = self.tuner.prepare()
+        with torch.cuda.device(self.tuner.device):
+            self.dev_plan = self.tuner.upload(self.plan)
 
     def counts(self) -> Dict[str, int]:
         """Search-space sizes: strategy rows, candidates = rows * (L + 1), base-variant cells
         = rows * sum_l (l + 1) * (#pre-saved micro-batch values), groups."""
         L = self.L
         pairs = L * (L + 1) // 2 + L
-        rows = cells = groups = 0
-        for _, plan, _ in self.tuners:
-            g = plan["groups"]
-            rows += int(g["n_rows"].sum())
-            cells += int((g["n_rows"] * g["num_p"]).sum()) * pairs
-            groups += len(g)
+        g = self.plan["groups"]
+        rows = int(g["n_rows"].sum())
+        cells = int((g["n_rows"] * g["num_p"]).sum()) * pairs
+        groups = len(g)
         return dict(rows=rows, candidates=rows * (L + 1), cells=cells, groups=groups)
 
     def run(self, stats: Optional[dict] = None):
         stats = {} if stats is None else stats
         hw = self.config.hardware
+        t0 = time.perf_counter()
+        results = self.tuner.run_prepared(self.plan, self.dev_plan)
+        t1 = time.perf_counter()
+        if self.granularity == "inter-stage":
+            outcomes = inter_stage_tune_batch(
+                self.L, hw.num_nodes * hw.num_gpus_per_node, self.meshes, self.Gs, results, slot=0, stats=stats
+            )
+        else:
+            outcomes = [
+                inter_stage_tune_uniform(self.L, hw.num_nodes, hw.num_gpus_per_node, self.Gs, r, self.config)
+                for r in results
+            ]
+        stats["intra_launch_s"] = stats.get("intra_launch_s", 0.0) + (t1 - t0)
+        stats["inter_s"] = stats.get("inter_s", 0.0) + (time.perf_counter() - t1)
         best_cost, best_solution = float("inf"), None
-        for tuner, plan, dev_plan in self.tuners:
-            t0 = time.perf_counter()
-            r = tuner.run_prepared(plan, dev_plan)
-            t1 = time.perf_counter()
-            if self.granularity == "inter-stage":
-                cost, solution = inter_stage_tune(
-                    self.L, hw.num_nodes * hw.num_gpus_per_node, self.meshes, self.Gs, r, slot=0, stats=stats
-                )
-            else:
-                cost, solution = inter_stage_tune_uniform(
-                    self.L, hw.num_nodes, hw.num_gpus_per_node, self.Gs, r, self.config
-                )
-            t2 = time.perf_counter()
-            stats["intra_launch_s"] = stats.get("intra_launch_s", 0.0) + (t1 - t0)
-            stats["inter_s"] = stats.get("inter_s", 0.0) + (t2 - t1)
+        for cost, solution in outcomes:  # tune_one_case.py:228-231: the first best tp wins
             if cost < best_cost:
                 best_cost, best_solution = cost, solution
         return best_cost, best_solution

@@ -41,7 +41,7 @@ def _gpu_dp(meshes, L, D, P1, tabs, tmax, want_argmin=False, mode=0):
     d_max = torch.empty(n, dtype=torch.float32).cuda()
     n_scr = lib.mist_dp_scratch_floats(ctypes.c_void_p(shape.ctypes.data), n)
     scr = torch.empty(max(n_scr, 1), dtype=torch.float32).cuda()
-    arg = torch.full((S + 1, L + 1, D + 1, 4), -1, dtype=torch.int32).cuda() if want_argmin else None
+    arg = torch.full((n, S + 1, L + 1, D + 1, 4), -1, dtype=torch.int32).cuda() if want_argmin else None
     rc = lib.mist_dp_run(
         ctypes.c_void_p(shape.ctypes.data), ctypes.byref(costs), d_t.data_ptr(), d_g.data_ptr(), n,
         mode, d_s.data_ptr(), d_sum.data_ptr(), d_max.data_ptr(), arg.data_ptr() if want_argmin else None,
@@ -87,7 +87,7 @@ def test_dp_kernel_matches_c_oracle(L, D, meshes, P1, quantum):
             n_feasible += 1
             assert got_sum[i] == np.float32(bsum.value) and got_max[i] == np.float32(smax.value), (i, t)
             g = _gpu_dp(meshes, L, D, P1, tabs, [t], want_argmin=True)
-            assert np.array_equal(g[3], arg), f"back-pointers differ at t={t}"
+            assert np.array_equal(g[3][0], arg), f"back-pointers differ at t={t}"
     assert n_feasible > 0
     # bottleneck mode = the smallest threshold for which the threshold DP is feasible
     _, bott, _ = _gpu_dp(meshes, L, D, P1, tabs, [0.0], mode=1)

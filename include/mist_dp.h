@@ -32,6 +32,8 @@ typedef struct MistDpShape {
  * g_stride[v] = elements between consecutive g of table v (costs, pre, post, nopp). */
 typedef struct MistDpCosts {
   const float *costs, *costs_pre, *costs_post, *costs_nopp;
+  /* running minima along the ckpt axis, same layouts: pmin[..][j] = min(costs[..][0..j]) */
+  const float *pmin, *pmin_pre, *pmin_post, *pmin_nopp;
   int64_t g_stride[4];
 } MistDpCosts;
 
@@ -47,10 +49,11 @@ int mist_sizeof_dp_shape(void);
  * inter_tuning_uniform.py:300-316); the reference's DP expects it precomputed in fields its
  * intra tuner no longer emits (mist/analyzer/inter_tuning.py:75-92).
  * d_grad_accum[num_grad_accum]: G per g index.  d_out[v]: variant v table for all g, i.e. the
- * layouts of MistOutTables without the trailing sample axis. */
+ * layouts of MistOutTables without the trailing sample axis; d_out_pmin[v]: its running minimum
+ * along the ckpt axis (what MistDpCosts.pmin* expects). */
 int mist_dp_cost_tables(const MistProblem *problem, const MistOutTables *tables,
                         const int32_t *d_grad_accum, int slot, float *const d_out[4],
-                        void *stream);
+                        float *const d_out_pmin[4], void *stream);
 
 /* Host helper: applies the reference's gap rule (inter_tuning.py:198: skip t when
  * t - last_run < 1e-6, float32 difference compared in float64) to an ascending list of

@@ -142,6 +142,10 @@ class DpCosts(ctypes.Structure):
         ("costs_pre", ctypes.c_void_p),
         ("costs_post", ctypes.c_void_p),
         ("costs_nopp", ctypes.c_void_p),
+        ("pmin", ctypes.c_void_p),
+        ("pmin_pre", ctypes.c_void_p),
+        ("pmin_post", ctypes.c_void_p),
+        ("pmin_nopp", ctypes.c_void_p),
         ("g_stride", ctypes.c_int64 * 4),
     ]
 
@@ -150,7 +154,7 @@ _DP_SIGNATURES = {
     "mist_sizeof_dp_shape": (ctypes.c_int, []),
     "mist_dp_cost_tables": (
         ctypes.c_int,
-        [_VP, ctypes.POINTER(OutTables), _VP, ctypes.c_int, ctypes.c_void_p * 4, _VP],
+        [_VP, ctypes.POINTER(OutTables), _VP, ctypes.c_int, ctypes.c_void_p * 4, ctypes.c_void_p * 4, _VP],
     ),
     "mist_dp_filter_tmax": (ctypes.c_int, [_VP, ctypes.c_int, ctypes.c_double, _VP]),
     "mist_dp_scratch_floats": (ctypes.c_int64, [_VP, ctypes.c_int]),

@@ -22,18 +22,28 @@ constexpr int kDpThreads = 64;  // one wavefront per workgroup
 // ------------------------------------------------------------------------------------------
 // Adapter: float64 (stable, delta) tables -> float32 DP cost tables for every g.
 // ------------------------------------------------------------------------------------------
+// One thread per table row (fixed g, mesh, p, layers): the L+1 ckpt entries are converted in
+// order and their running minimum is stored alongside (pmin[j] = min(cost[0..j])).
 __global__ __launch_bounds__(256) void cost_table_kernel(const double *__restrict__ stable,
                                                          const double *__restrict__ delta,
                                                          const int32_t *__restrict__ grad_accum,
-                                                         int64_t n_cells, int64_t cells_per_g,
-                                                         int sample_size, int slot,
-                                                         float *__restrict__ out) {
-  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n_cells) return;
-  const float G = (float)grad_accum[i / cells_per_g];
-  const float s = (float)stable[i * sample_size + slot];
-  const float d = (float)delta[i * sample_size + slot];
-  out[i] = s + d / G;
+                                                         int64_t n_rows, int64_t rows_per_g,
+                                                         int row_len, int sample_size, int slot,
+                                                         float *__restrict__ out,
+                                                         float *__restrict__ pmin) {
+  const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= n_rows) return;
+  const float G = (float)grad_accum[r / rows_per_g];
+  float run = INFINITY;
+  for (int j = 0; j < row_len; ++j) {
+    const int64_t i = r * row_len + j;
+    const float s = (float)stable[i * sample_size + slot];
+    const float d = (float)delta[i * sample_size + slot];
+    const float c = s + d / G;
+    run = fminf(run, c);
+    out[i] = c;
+    pmin[i] = run;
+  }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -87,10 +97,8 @@ __global__ __launch_bounds__(kDpThreads) void dp_step_kernel(
   float *__restrict__ m_cur = state + (2 + cur) * plane;
   const float t_max = kBottleneck ? INFINITY : tmax_list[t];
   const int64_t g = g_list[t];
-  const float *__restrict__ tab_costs = tabs.costs + g * tabs.g_stride[0];
-  const float *__restrict__ tab_pre = tabs.costs_pre + g * tabs.g_stride[1];
-  const float *__restrict__ tab_post = tabs.costs_post + g * tabs.g_stride[2];
-  const float *__restrict__ tab_nopp = tabs.costs_nopp + g * tabs.g_stride[3];
+  const int64_t off[4] = {g * tabs.g_stride[0], g * tabs.g_stride[1], g * tabs.g_stride[2],
+                          g * tabs.g_stride[3]};
   const int k = e / W, d = e % W;
   const int p = s - 1;
 
@@ -104,28 +112,41 @@ __global__ __launch_bounds__(kDpThreads) void dp_step_kernel(
         const int from = (i + 1) * W + (d - nm);
         const float prev = f_prev[from];
         // A state reachable only through an unreachable successor cannot improve: inf + c is
-        // never < best.  Skipping it changes nothing and saves the inner loop.
+        // never < best.  Skipping it changes nothing.
         if (prev == INFINITY) continue;
         const int l = i - k + 1;
-        const float *__restrict__ row;
-        if (k == 0 && i == L - 1) row = tab_nopp + (int64_t)q * C;
-        else if (k == 0) row = tab_pre + (((int64_t)q * P1 + p) * L + (l - 1)) * C;
-        else if (i == L - 1) row = tab_post + ((int64_t)q * L + (l - 1)) * C;
-        else row = tab_costs + (((int64_t)q * P1 + p) * L + (l - 1)) * C;
-        const float prev_m = m_prev[from];
-        const int j_end = L - i;
-#pragma unroll 4
-        for (int j = 0; j <= j_end; ++j) {
-          const float stage_cost = row[j];
-          // Threshold mode: sum of stage costs under cost <= t_max.  Bottleneck mode: the
-          // smallest achievable maximum stage cost (comparisons only, no rounding).
-          const float new_cost = kBottleneck ? fmaxf(stage_cost, prev) : stage_cost + prev;
-          if (stage_cost <= t_max && new_cost < best) {
-            best = new_cost;
-            best_m = fmaxf(prev_m, stage_cost);
-            arg_i = i;
-            arg_q = q;
-            arg_j = j;
+        int64_t at;  // start of the ckpt row of this (variant, mesh, p, layers)
+        int v;
+        if (k == 0 && i == L - 1) { v = 3; at = (int64_t)q * C; }
+        else if (k == 0) { v = 1; at = (((int64_t)q * P1 + p) * L + (l - 1)) * C; }
+        else if (i == L - 1) { v = 2; at = ((int64_t)q * L + (l - 1)) * C; }
+        else { v = 0; at = (((int64_t)q * P1 + p) * L + (l - 1)) * C; }
+        const float *__restrict__ cost_tab = v == 0 ? tabs.costs : v == 1 ? tabs.costs_pre
+                                             : v == 2 ? tabs.costs_post : tabs.costs_nopp;
+        const float *__restrict__ pmin_tab = v == 0 ? tabs.pmin : v == 1 ? tabs.pmin_pre
+                                             : v == 2 ? tabs.pmin_post : tabs.pmin_nopp;
+        const int j_end = L - i;  // ckpt candidates 0..L-i (inter_tuning.py:315)
+        // The reference walks j = 0..j_end with "cost <= t_max and cost + prev < best".  "+ prev"
+        // is monotone, so the smallest reachable sum is (smallest admissible cost) + prev, and
+        // the smallest admissible cost is the row's running minimum if that is <= t_max (else
+        // nothing is admissible).  Only when this sum beats `best` is the row walked, to find
+        // the first j that attains it: that is the entry the reference's strict "<" keeps.
+        const float rmin = pmin_tab[off[v] + at + j_end];
+        if (!(rmin <= t_max)) continue;
+        const float target = kBottleneck ? fmaxf(rmin, prev) : rmin + prev;
+        if (!(target < best)) continue;
+        best = target;
+        arg_i = i;
+        arg_q = q;
+        if (!kBottleneck) {
+          const float *__restrict__ row = cost_tab + off[v] + at;
+          for (int j = 0; j <= j_end; ++j) {
+            const float stage_cost = row[j];
+            if (stage_cost <= t_max && stage_cost + prev == target) {
+              arg_j = j;
+              best_m = fmaxf(m_prev[from], stage_cost);
+              break;
+            }
           }
         }
       }
@@ -176,22 +197,22 @@ int mist_sizeof_dp_shape(void) { return (int)sizeof(MistDpShape); }
 
 int mist_dp_cost_tables(const MistProblem *problem, const MistOutTables *tables,
                         const int32_t *d_grad_accum, int slot, float *const d_out[4],
-                        void *stream) {
-  if (!problem || !tables || !d_grad_accum || !d_out)
+                        float *const d_out_pmin[4], void *stream) {
+  if (!problem || !tables || !d_grad_accum || !d_out || !d_out_pmin)
     return fail(MIST_E_INVALID, "null pointer argument");
   const int64_t L = problem->num_layers, P1 = problem->p_dim, S = problem->sample_size;
   const int64_t Gn = problem->num_grad_accum, Q = problem->num_mesh;
   if (L <= 0 || P1 <= 0 || S <= 0 || Gn <= 0 || Q <= 0)
     return fail(MIST_E_INVALID, "bad problem extents");
   if (slot < 0 || slot >= S) return fail(MIST_E_INVALID, "slot %d outside [0, %d)", slot, (int)S);
-  const int64_t per_g[4] = {Q * P1 * L * (L + 1), Q * P1 * L * (L + 1), Q * L * (L + 1), Q * (L + 1)};
+  const int64_t rows_per_g[4] = {Q * P1 * L, Q * P1 * L, Q * L, Q};
   for (int v = 0; v < 4; ++v) {
-    if (!tables->stable[v] || !tables->delta[v] || !d_out[v])
+    if (!tables->stable[v] || !tables->delta[v] || !d_out[v] || !d_out_pmin[v])
       return fail(MIST_E_INVALID, "table %d is null", v);
-    const int64_t n = Gn * per_g[v];
+    const int64_t n = Gn * rows_per_g[v];
     hipLaunchKernelGGL(cost_table_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
                        (hipStream_t)stream, tables->stable[v], tables->delta[v], d_grad_accum, n,
-                       per_g[v], (int)S, slot, d_out[v]);
+                       rows_per_g[v], (int)(L + 1), (int)S, slot, d_out[v], d_out_pmin[v]);
     MIST_HIP_CHECK(hipGetLastError());
   }
   return 0;
@@ -221,7 +242,8 @@ int mist_dp_run(const MistDpShape *shape, const MistDpCosts *costs, const float 
                 float *d_best_sum, float *d_stage_max, int32_t *d_argmin, float *d_scratch,
                 void *stream) {
   if (int rc = check_shape(shape)) return rc;
-  if (!costs || !costs->costs || !costs->costs_pre || !costs->costs_post || !costs->costs_nopp)
+  if (!costs || !costs->costs || !costs->costs_pre || !costs->costs_post || !costs->costs_nopp ||
+      !costs->pmin || !costs->pmin_pre || !costs->pmin_post || !costs->pmin_nopp)
     return fail(MIST_E_INVALID, "null cost table");
   if (!d_tmax || !d_g_index || !d_best_s || !d_best_sum || !d_stage_max)
     return fail(MIST_E_INVALID, "null threshold / output pointer");

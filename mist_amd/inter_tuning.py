@@ -71,15 +71,17 @@ class _DpRunner:
                 torch.empty(tuple(t.shape[:-1]), dtype=torch.float32, device=self.device)
                 for t in dev_tabs.stable
             ]
+            self.pmin = [torch.empty_like(t) for t in self.cost]
             d_G = torch.tensor(Gs, dtype=torch.int32, device=self.device)
             out_ptrs = (ctypes.c_void_p * 4)(*[t.data_ptr() for t in self.cost])
+            pmin_ptrs = (ctypes.c_void_p * 4)(*[t.data_ptr() for t in self.pmin])
             tabs = dev_tabs.as_struct()
             rc = self.lib.mist_dp_cost_tables(
                 ctypes.c_void_p(problem.ctypes.data), ctypes.byref(tabs), d_G.data_ptr(), slot,
-                out_ptrs, _stream(self.device),
+                out_ptrs, pmin_ptrs, _stream(self.device),
             )
             _lib.check(rc, "mist_dp_cost_tables")
-        self.costs_struct = _lib.DpCosts(*[t.data_ptr() for t in self.cost])
+        self.costs_struct = _lib.DpCosts(*[t.data_ptr() for t in self.cost + self.pmin])
         for v in range(4):
             self.costs_struct.g_stride[v] = self.cost[v][0].numel()
         self.launches = 0

@@ -32,6 +32,7 @@ def _gpu_dp(meshes, L, D, P1, tabs, tmax, want_argmin=False, mode=0):
     shape["mesh_n"][0, :Q] = [n for n, _ in meshes]
     shape["mesh_m"][0, :Q] = [m for _, m in meshes]
     dev = [torch.from_numpy(t).cuda() for t in tabs]
+    dev += [torch.cummin(t, dim=-1).values.contiguous() for t in dev]  # running minima over ckpt
     costs = _lib.DpCosts(*[t.data_ptr() for t in dev])
     n = len(tmax)
     d_t = torch.tensor(tmax, dtype=torch.float32).cuda()

@@ -206,7 +206,7 @@ def test_argument_checks_reject_before_any_launch():
     assert lib.mist_dp_scratch_floats(ctypes.c_void_p(shape.ctypes.data), 4) == 4 * 4 * 9 * 9
     shape["num_layers"], shape["num_devices"] = 80, 256
     assert lib.mist_dp_scratch_floats(ctypes.c_void_p(shape.ctypes.data), 4) == 4 * 4 * 81 * 257
-    costs = _lib.DpCosts(4096, 4096, 4096, 4096)
+    costs = _lib.DpCosts(4096, 4096, 4096, 4096, 4096, 4096, 4096, 4096)
     sp = ctypes.c_void_p(shape.ctypes.data)
     assert lib.mist_dp_run(sp, ctypes.byref(costs), fake, fake, 1, 0, fake, fake, fake, None, None, None) == -1
     assert b"scratch" in lib.mist_last_error()

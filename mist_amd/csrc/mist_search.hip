@@ -429,7 +429,13 @@ __device__ __forceinline__ void take_min(double &best, int32_t &best_row, bool f
 // kPow2G: the group's G is a power of two, so x / G == x * (1 / G) bit for bit (float32 and
 // float64) and the division leaves the inner loop; other G divide.  kFirstTile: this workgroup
 // owns p = 0 and therefore also the last-stage and single-stage variants.
-constexpr int kRowUnroll = 4;  // rows whose objective values are computed together (ILP)
+#ifndef MIST_ROW_UNROLL
+#define MIST_ROW_UNROLL 4
+#endif
+#ifndef MIST_REDUCE_MIN_WAVES
+#define MIST_REDUCE_MIN_WAVES 2
+#endif
+constexpr int kRowUnroll = MIST_ROW_UNROLL;  // rows whose objective values are computed together (ILP)
 
 template <bool kPow2G, bool kFirstTile>
 __device__ __forceinline__ void reduce_block(
@@ -502,8 +508,7 @@ __device__ __forceinline__ void reduce_block(
       // ---- latencies and objective values of kRowUnroll rows (:2165-2351; pareto.py:138:
       // r * x + y in float64).  Independent of the running minima, hence computed together;
       // rows past the end of the stage read stale LDS and are ignored below. ----
-      double cost_base[kRowUnroll], cost_pre[kRowUnroll], cost_post[kRowUnroll],
-          cost_pp[kRowUnroll];
+      double xs[kRowUnroll], ds[kRowUnroll], cost_base[kRowUnroll], bound[kRowUnroll];
 #pragma unroll
       for (int u = 0; u < kRowUnroll; ++u) {
         const double *__restrict__ t = lds_terms + min(r0 + u, kStageRows - 1) * MIST_ROW_TERMS;
@@ -512,22 +517,13 @@ __device__ __forceinline__ void reduce_block(
         const double delta = n_ck * t[MIST_T_D_LAYER_CK] + n_nock * t[MIST_T_D_LAYER_NOCK] +
                              t[MIST_T_D_FIRST_CK + first_col] + t[MIST_T_D_LAST_CK + last_col];
         const float x32 = (float)stable, d32 = (float)delta;  // (:2212-2213)
-        const double x = (double)x32, d = (double)d32;
+        xs[u] = (double)x32;
+        ds[u] = (double)d32;
         const float y32 = kPow2G ? d32 * inv_G32 : d32 / G32;  // float32 array / python int (:2815)
-        cost_base[u] = ratio * x + (double)y32;
-        cost_pre[u] = ratio * (x + k.pre_fwd + k.pre_bwd + k.w1 + k.w2) + div_G(d + k.w1d + k.w2d);
-        if (kFirstTile) {
-          const double nag = t[MIST_T_NAG_CK + post_col], nrs = t[MIST_T_NRS_CK + post_col];
-          const double ps1 = k.pp_wre ? nag : 0.0, ps2 = k.pp_gre ? nrs : 0.0;
-          const double pd1 = k.pp_wre ? 0.0 : nag, pd2 = k.pp_gre ? 0.0 : nrs;
-          const double opb = t[MIST_T_OPB];
-          cost_post[u] = ratio * (x + k.post_fwd + opb + ps1 + ps2) + div_G(d + pd1 + pd2);
-          cost_pp[u] =
-              ratio * (x + k.pre_fwd + k.pre_bwd + k.post_fwd + opb + k.w1 + k.w2 + ps1 + ps2) +
-              div_G(d + k.w1d + k.w2d + pd1 + pd2);
-        } else {
-          cost_post[u] = cost_pp[u] = 0.0;
-        }
+        cost_base[u] = ratio * xs[u] + (double)y32;
+        // Lower bound of the three composite objectives: they add non-negative terms to x and
+        // d before the same monotone operations, so none of them can be below this value.
+        bound[u] = ratio * xs[u] + div_G(ds[u]);
       }
 
 #pragma unroll
@@ -535,6 +531,27 @@ __device__ __forceinline__ void reduce_block(
         if (r0 + u >= n_stage) break;
         const double *__restrict__ t = lds_terms + (r0 + u) * MIST_ROW_TERMS;
         const int32_t row = (int32_t)(base + r0 + u);
+        const double x = xs[u], d = ds[u];
+        // Which composite objectives can still matter for this row.
+        const bool want_pre = bound[u] < top_p || fin_p < n_tile;
+        const bool want_post = kFirstTile && bound[u] < best_post;
+        const bool want_pp = do_nopp && bound[u] < best_pp;
+        if (!(cost_base[u] < top_b || fin_b < n_tile || want_pre || want_post || want_pp)) continue;
+
+        double cost_pre = INFINITY, cost_post = INFINITY, cost_pp = INFINITY;
+        if (want_pre)
+          cost_pre = ratio * (x + k.pre_fwd + k.pre_bwd + k.w1 + k.w2) + div_G(d + k.w1d + k.w2d);
+        if (want_post || want_pp) {
+          const double nag = t[MIST_T_NAG_CK + post_col], nrs = t[MIST_T_NRS_CK + post_col];
+          const double ps1 = k.pp_wre ? nag : 0.0, ps2 = k.pp_gre ? nrs : 0.0;
+          const double pd1 = k.pp_wre ? 0.0 : nag, pd2 = k.pp_gre ? 0.0 : nrs;
+          const double opb = t[MIST_T_OPB];
+          cost_post = ratio * (x + k.post_fwd + opb + ps1 + ps2) + div_G(d + pd1 + pd2);
+          cost_pp =
+              ratio * (x + k.pre_fwd + k.pre_bwd + k.post_fwd + opb + k.w1 + k.w2 + ps1 + ps2) +
+              div_G(d + k.w1d + k.w2d + pd1 + pd2);
+        }
+
         // Lowest slot the row could improve: the minima are non-decreasing in p, so it is the
         // number of slots whose minimum the row does not beat (empty slots hold +inf).  The row
         // changes something iff it is feasible at that slot (feasibility is monotone in p).
@@ -544,14 +561,14 @@ __device__ __forceinline__ void reduce_block(
 #pragma unroll
           for (int j = 0; j < MIST_P_TILE; ++j) lo_b += cost_base[u] >= best_b[j] ? 1 : 0;
         }
-        if (cost_pre[u] < top_p) {
+        if (cost_pre < top_p) {
           lo_p = 0;
 #pragma unroll
-          for (int j = 0; j < MIST_P_TILE; ++j) lo_p += cost_pre[u] >= best_p[j] ? 1 : 0;
+          for (int j = 0; j < MIST_P_TILE; ++j) lo_p += cost_pre >= best_p[j] ? 1 : 0;
         }
-        bool need_b = lo_b < n_tile, need_p = lo_p < n_tile;
-        const bool need_post = kFirstTile && cost_post[u] < best_post;
-        const bool need_pp = do_nopp && cost_pp[u] < best_pp;
+        bool need_b = lo_b < n_tile, need_p = want_pre && lo_p < n_tile;
+        const bool need_post = want_post && cost_post < best_post;
+        const bool need_pp = want_pp && cost_pp < best_pp;
         if (!(need_b || need_p || need_post || need_pp)) continue;
 
         // ---- memory that does not depend on p (:2150-2162, 2358-2385, 2760-2769) ----
@@ -610,7 +627,7 @@ __device__ __forceinline__ void reduce_block(
           else if (lo == fin_b && cost < top_b) top_b = cost;
         }
         if (need_p) {
-          const double cost = cost_pre[u];
+          const double cost = cost_pre;
           int lo = lo_p + 1, hi = n_tile;
           for (int it = 0; it < steps; ++it) {
             const int mid = (lo + hi) >> 1;
@@ -639,12 +656,12 @@ __device__ __forceinline__ void reduce_block(
           const double pf_post = fmax(f_in, peak_f + post_states);
           const double pb_post = fmax(b_in, peak_b - out + post_states) + post_output;
           const bool ok_post = fmax(pf_post, pb_post) * mf_pp <= cap;
-          take_min(best_post, row_post, need_post && ok_post, cost_post[u], row);
+          take_min(best_post, row_post, need_post && ok_post, cost_post, row);
           if (need_pp) {
             const double pf_pp = pf_post + pre_states + pre_saved;
             const double pb_pp = pb_post + pre_states + pre_saved;
             const bool ok_pp = fmax(pf_pp, pb_pp) * t[MIST_T_MF] <= cap;
-            take_min(best_pp, row_pp, ok_pp, cost_pp[u], row);
+            take_min(best_pp, row_pp, ok_pp, cost_pp, row);
           }
         }
       }
@@ -665,7 +682,7 @@ __device__ __forceinline__ void reduce_block(
   partial_index[out_base + (int64_t)(2 * MIST_P_TILE + 1) * MIST_LC_TILE] = row_pp;
 }
 
-__global__ __launch_bounds__(MIST_LC_TILE, 2) void eval_reduce_kernel(
+__global__ __launch_bounds__(MIST_LC_TILE, MIST_REDUCE_MIN_WAVES) void eval_reduce_kernel(
     const MistProblem prob, const MistGroupDesc *__restrict__ groups, int n_groups,
     const int32_t *__restrict__ block_prefix, const double *__restrict__ row_terms, double ratio,
     double *__restrict__ partial_cost, int32_t *__restrict__ partial_index) {

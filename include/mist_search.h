@@ -26,7 +26,9 @@ extern "C" {
 #define MIST_MAX_PAIRS (MIST_MAX_RATIOS * MIST_MAX_RATIOS)
 #define MIST_PAR_FIELDS 20
 #define MIST_ROW_TERMS 34   /* doubles per candidate row produced by mist_row_terms */
-#define MIST_LC_TILE 256    /* (layers, ckpt) pairs per workgroup of the reduce kernel */
+#ifndef MIST_LC_TILE
+#define MIST_LC_TILE 64     /* (layers, ckpt) pairs per workgroup (one wavefront) of the reduce kernel */
+#endif
 #ifndef MIST_P_TILE
 #define MIST_P_TILE 16      /* pre-saved micro-batch values per thread of the reduce kernel */
 #endif
@@ -104,7 +106,8 @@ typedef struct MistGroupDesc {
   int32_t n_par, n_pair, n_oo, n_ao, n_off;
   int32_t pp_wre, pp_gre;       /* ZeRO flags of the pre/post layer strategy */
   int32_t rows_per_chunk, n_chunks, n_lc_tiles, n_p_tiles; /* decomposition of the reduce kernel */
-  int32_t reserved0;
+  int32_t scout_stride;         /* reduce kernel: the scout pass visits every scout_stride-th
+                                 * stage of mist_reduce_stage_rows() rows; 0 = no scout pass */
   int64_t n_rows;               /* n_par * n_off */
   int64_t row_offset;           /* first row of this group in the row-term workspace */
   double par[MIST_MAX_PAR][MIST_PAR_FIELDS];
@@ -136,6 +139,8 @@ const char *mist_last_error(void);
 int mist_sizeof_problem(void);
 int mist_sizeof_group(void);
 int mist_reduce_p_tile(void); /* MIST_P_TILE the library was built with */
+int mist_reduce_lc_tile(void); /* MIST_LC_TILE the library was built with */
+int mist_reduce_stage_rows(void); /* rows per LDS stage; rows_per_chunk must be a multiple */
 
 /* Row-invariant terms of every candidate row: decodes the row index, evaluates the alpha-beta
  * communication terms, the 36 interference evaluations and the memory pieces that do not
@@ -155,13 +160,19 @@ int mist_row_terms(const MistProblem *problem, const MistGroupDesc *d_groups, in
  * and compute_indices (mist/utils/pareto.py:124-144) for one ratio r = alpha/(1-alpha).
  * d_block_prefix[n_groups+1]: first workgroup of each group; a group owns
  * n_lc_tiles*n_p_tiles*n_chunks workgroups ordered (lc_tile, p_tile, chunk), chunk fastest.
- * d_partial_cost / d_partial_index: [n_blocks][2*MIST_P_TILE+2][MIST_LC_TILE]. */
+ * Optional scout pass (n_scout_blocks > 0): d_scout_prefix[n_groups+1] gives each group
+ * n_lc_tiles*n_p_tiles workgroups that first reduce every scout_stride-th stage of the whole
+ * group; every chunk then starts from those minima (they belong to real rows of the group, so
+ * the result is unchanged) and lets far fewer rows through to the memory model.
+ * d_partial_cost / d_partial_index: [n_blocks + n_scout_blocks][2*MIST_P_TILE+2][MIST_LC_TILE];
+ * the first n_blocks slabs are the per-chunk results mist_finalize reads. */
 int mist_eval_reduce(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,
-                     const int32_t *d_block_prefix, int n_blocks, const double *d_row_terms,
-                     double ratio, double *d_partial_cost, int32_t *d_partial_index,
-                     void *stream);
+                     const int32_t *d_block_prefix, int n_blocks,
+                     const int32_t *d_scout_prefix, int n_scout_blocks,
+                     const double *d_row_terms, double ratio, double *d_partial_cost,
+                     int32_t *d_partial_index, void *stream);
 
-/* Combines the per-chunk partial minima in chunk order (strict <, so the first row wins ties),
+/* Combines the per-chunk partial minima (smallest cost, lowest row among equals),
  * recomputes stable / delta of the winning row and scatters into the output tables at sample
  * position `sample_index`, reproducing which cells the reference leaves unwritten
  * (batched_module_analyzer.py:2819-2834, 2915-2923, 3021-3033, 3103-3106). */
@@ -176,7 +187,7 @@ int mist_finalize(const MistProblem *problem, const MistGroupDesc *d_groups, int
 int mist_intra_stage_eval(const MistProblem *problem, const MistGroupDesc *d_groups,
                           int n_groups, const int32_t *d_terms_block_prefix, int n_terms_blocks,
                           const int32_t *d_reduce_block_prefix, int n_reduce_blocks,
-                          double *d_row_terms, double *d_partial_cost, int32_t *d_partial_index,
+                          const int32_t *d_scout_prefix, int n_scout_blocks, double *d_row_terms, double *d_partial_cost, int32_t *d_partial_index,
                           double ratio, int sample_index, int compute_terms,
                           const MistOutTables *tables, void *stream);
 

@@ -16,10 +16,10 @@ MAX_RATIOS = 32
 MAX_PAIRS = MAX_RATIOS * MAX_RATIOS
 PAR_FIELDS = 20
 ROW_TERMS = 34
-LC_TILE = 256
+LC_TILE = 64  # replaced by the library's own value in load()
 P_TILE = 32  # replaced by the library's own value in load()
 SLOTS = 2 * P_TILE + 2
-STAGE_ROWS = 32
+STAGE_ROWS = 64  # replaced by the library's own value in load()
 TERMS_BLOCK = 256
 MAX_MESH = 16
 DP_THRESHOLD, DP_BOTTLENECK = 0, 1
@@ -66,7 +66,7 @@ GROUP_DTYPE = np.dtype(
         ("n_par", "<i4"), ("n_pair", "<i4"), ("n_oo", "<i4"), ("n_ao", "<i4"), ("n_off", "<i4"),
         ("pp_wre", "<i4"), ("pp_gre", "<i4"),
         ("rows_per_chunk", "<i4"), ("n_chunks", "<i4"), ("n_lc_tiles", "<i4"),
-        ("n_p_tiles", "<i4"), ("reserved0", "<i4"),
+        ("n_p_tiles", "<i4"), ("scout_stride", "<i4"),
         ("n_rows", "<i8"), ("row_offset", "<i8"),
         ("par", "<f8", (MAX_PAR, PAR_FIELDS)),
         ("wo", "<f8", (MAX_RATIOS,)), ("go", "<f8", (MAX_RATIOS,)),
@@ -104,10 +104,13 @@ _SIGNATURES = {
     "mist_sizeof_problem": (ctypes.c_int, []),
     "mist_sizeof_group": (ctypes.c_int, []),
     "mist_reduce_p_tile": (ctypes.c_int, []),
+    "mist_reduce_stage_rows": (ctypes.c_int, []),
+    "mist_reduce_lc_tile": (ctypes.c_int, []),
     "mist_row_terms": (ctypes.c_int, [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, _VP]),
     "mist_eval_reduce": (
         ctypes.c_int,
-        [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, ctypes.c_double, _VP, _VP, _VP],
+        [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, ctypes.c_double,
+         _VP, _VP, _VP],
     ),
     "mist_finalize": (
         ctypes.c_int,
@@ -115,8 +118,8 @@ _SIGNATURES = {
     ),
     "mist_intra_stage_eval": (
         ctypes.c_int,
-        [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, _VP, _VP,
-         ctypes.c_double, ctypes.c_int, ctypes.c_int, ctypes.POINTER(OutTables), _VP],
+        [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, ctypes.c_int,
+         _VP, _VP, _VP, ctypes.c_double, ctypes.c_int, ctypes.c_int, ctypes.POINTER(OutTables), _VP],
     ),
 }
 
@@ -192,7 +195,9 @@ def load():
         raise MistLibraryError(
             f"MistGroupDesc layout mismatch: C {lib.mist_sizeof_group()} vs numpy {GROUP_DTYPE.itemsize}"
         )
-    global P_TILE, SLOTS
+    global P_TILE, SLOTS, STAGE_ROWS, LC_TILE
+    LC_TILE = lib.mist_reduce_lc_tile()
+    STAGE_ROWS = lib.mist_reduce_stage_rows()
     P_TILE = lib.mist_reduce_p_tile()
     SLOTS = 2 * P_TILE + 2
     _LIB = lib

@@ -11,6 +11,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <type_traits>
 
 #include "mist_common.h"
 #include "mist_search.h"
@@ -34,7 +35,7 @@ namespace {
 using mist::fail;
 
 constexpr int kTermsBlock = 256;  // rows per workgroup of the row-term kernel
-constexpr int kStageRows = 32;    // rows staged through LDS per step of the reduce kernel
+constexpr int kStageRows = 64;    // rows staged through LDS per step of the reduce kernel
 constexpr int kSlots = 2 * MIST_P_TILE + 2;  // per-thread running minima: base, with_pre, post, no_pp
 
 // ------------------------------------------------------------------------------------------
@@ -403,28 +404,44 @@ __device__ __forceinline__ CellLatency cell_latency(const double *__restrict__ t
   return r;
 }
 
-// Lexicographic running minimum: strictly smaller cost wins; rows arrive in ascending order so
-// the first row keeps ties, exactly like the strict "<" scan of mist/utils/pareto.py:134-142.
+// Lexicographic (cost, row) minimum.  The reference scans rows in ascending order with a strict
+// "<" (mist/utils/pareto.py:134-142), i.e. it keeps the lowest row among those with the
+// smallest cost; comparing (cost, row) pairs gives the same winner in any processing order.
+__device__ __forceinline__ bool lex_less(double cost, int32_t row, double best, int32_t best_row) {
+  return cost < best || (cost == best && row < best_row);
+}
+
 __device__ __forceinline__ void take_min(double &best, int32_t &best_row, bool feasible,
                                          double cost, int32_t row) {
-  const bool better = feasible && cost < best;
+  const bool better = feasible && lex_less(cost, row, best, best_row);
   best = better ? cost : best;
   best_row = better ? row : best_row;
 }
 
 // ------------------------------------------------------------------------------------------
 // Kernel 2: evaluate + mask + running argmin.
-// Workgroup = 256 threads = one tile of (l, c) pairs; it streams one chunk of candidate rows
-// through LDS (every lane reads the same row: broadcast reads, no bank conflicts) and each
-// thread keeps the minima of MIST_P_TILE pre-saved micro-batch values for its own (l, c).
-// No cross-lane reduction is needed: the reduction axis (rows) is the loop, not the lanes.
+// Workgroup = 256 threads = one tile of (l, c) pairs; it streams candidate rows through LDS
+// and each thread keeps the minima of MIST_P_TILE pre-saved micro-batch values for its own
+// (l, c).  No cross-lane reduction is needed: the reduction axis (rows) is the loop.
 //
 // Memory feasibility is monotone in p: the peaks are built from p * (non-negative) terms by
 // additions only, every floating-point add / multiply is monotone in each operand, and the
 // host rejects negative table values.  So per (row, l, c) the feasible p form a prefix
 // [0, count) and `count` is found by bisection with the exact peak formula at the probed p
 // (no closed-form shortcut: the comparison that decides is the reference's own expression).
-// A row then updates exactly the slots p < count where its cost is strictly smaller.
+// The minima of a thread are therefore non-decreasing in p, and a row changes a slot iff it is
+// feasible at the lowest slot whose minimum it beats.
+//
+// Almost no row changes anything, so a stage of kStageRows rows goes through three sieves, each
+// keeping a per-lane bit mask of surviving rows so that a lane only pays for its own survivors
+// (a wave executes a sieve as often as its busiest lane, not once per row):
+//   A  objective value against the largest minimum (all rows, straight-line code);
+//   B  lowest improvable slot and the exact memory test at that slot (minima as of stage start:
+//      they only decrease afterwards, so nothing that could matter later is dropped);
+//   C  survivors in row order against the live minima: bisection for `count`, update.
+// A scout pass runs the same code over every scout_stride-th stage of a whole group first; the
+// main pass starts every chunk from the scout's minima (real rows of the same group, hence valid
+// upper bounds), which removes the warm-up in which a fresh chunk lets most rows through.
 // ------------------------------------------------------------------------------------------
 // kPow2G: the group's G is a power of two, so x / G == x * (1 / G) bit for bit (float32 and
 // float64) and the division leaves the inner loop; other G divide.  kFirstTile: this workgroup
@@ -436,12 +453,23 @@ __device__ __forceinline__ void take_min(double &best, int32_t &best_row, bool f
 #define MIST_REDUCE_MIN_WAVES 2
 #endif
 constexpr int kRowUnroll = MIST_ROW_UNROLL;  // rows whose objective values are computed together (ILP)
+constexpr int kLdsRowStride = MIST_ROW_TERMS + 1;  // odd number of doubles: lanes reading the
+                                                   // same term of different rows hit different banks
+static_assert(kStageRows == 64, "the sieve masks are 64-bit");
+
+struct ReduceRange {
+  int64_t row_begin, row_end;  // rows of the group this workgroup covers (multiples of kStageRows)
+  int stage_step;              // visit every stage_step-th stage of the range
+  int skip_stride;             // > 0: skip stages whose index is a multiple (the scout did them)
+};
 
 template <bool kPow2G, bool kFirstTile>
 __device__ __forceinline__ void reduce_block(
-    const MistProblem &prob, const MistGroupDesc *__restrict__ g, int chunk, int p_tile,
-    int lc_tile, const double *__restrict__ row_terms, double ratio, double *lds_terms,
-    double *__restrict__ partial_cost, int32_t *__restrict__ partial_index) {
+    const MistProblem &prob, const MistGroupDesc *__restrict__ g, const ReduceRange range,
+    int p_tile, int lc_tile, const double *__restrict__ row_terms, double ratio,
+    double *lds_terms, const double *__restrict__ seed_cost,
+    const int32_t *__restrict__ seed_index, double *__restrict__ out_cost,
+    int32_t *__restrict__ out_index) {
   const int L = prob.num_layers;
   const int n_pairs = L * (L + 1) / 2 + L;  // sum over l = 1..L of (l + 1)
   const int pair_idx = lc_tile * MIST_LC_TILE + threadIdx.x;
@@ -450,10 +478,14 @@ __device__ __forceinline__ void reduce_block(
   const int l = pc.l, c = pc.c;
 
   const int p0 = p_tile * MIST_P_TILE;
-  const int n_tile = min(MIST_P_TILE, g->num_p - p0);  // p values of this tile: p0 .. p0+n_tile-1
+  const int n_tile_full = min(MIST_P_TILE, g->num_p - p0);  // p values of this tile
+  // Cells with c == l - 1 are only kept for p == 0 of the base / with_pre variants
+  // (batched_module_analyzer.py:3021-3023, 3103), so such a lane has at most one slot.
+  const int n_tile = c == l - 1 ? (kFirstTile ? min(n_tile_full, 1) : 0) : n_tile_full;
   int steps = 0;  // bisection steps that separate the n_tile + 1 possible counts
   while ((1 << steps) < n_tile + 1) ++steps;
-  const bool do_nopp = kFirstTile && l == L;
+  const bool do_post = kFirstTile && c != l - 1;
+  const bool do_nopp = kFirstTile && l == L && c != l - 1;
   const GroupConsts k = group_consts(g);
   const double cap = prob.mem_cap_mb;
   const double G64 = (double)g->grad_accum;
@@ -467,20 +499,33 @@ __device__ __forceinline__ void reduce_block(
 
   double best_b[MIST_P_TILE], best_p[MIST_P_TILE];
   int32_t row_b[MIST_P_TILE], row_p[MIST_P_TILE];
+  double best_post = INFINITY, best_pp = INFINITY;
+  int32_t row_post = -1, row_pp = -1;
+  // The minima of a tile are non-decreasing in p and finite on a prefix [0, fin); `top` is the
+  // largest finite one.  A row that does not reach `top` can only fill the first empty slot.
+  int fin_b = 0, fin_p = 0;
+  double top_b = -INFINITY, top_p = -INFINITY;
 #pragma unroll
   for (int j = 0; j < MIST_P_TILE; ++j) {
     best_b[j] = best_p[j] = INFINITY;
     row_b[j] = row_p[j] = -1;
   }
-  double best_post = INFINITY, best_pp = INFINITY;
-  int32_t row_post = -1, row_pp = -1;
-  // The minima of a tile are non-decreasing in p and finite on a prefix [0, fin); `top` is the
-  // largest finite one.  A row that does not beat `top` can only fill the first empty slot.
-  int fin_b = 0, fin_p = 0;
-  double top_b = -INFINITY, top_p = -INFINITY;
+  if (seed_cost != nullptr && active) {
+#pragma unroll
+    for (int j = 0; j < MIST_P_TILE; ++j) {
+      best_b[j] = seed_cost[j * MIST_LC_TILE + threadIdx.x];
+      row_b[j] = seed_index[j * MIST_LC_TILE + threadIdx.x];
+      best_p[j] = seed_cost[(MIST_P_TILE + j) * MIST_LC_TILE + threadIdx.x];
+      row_p[j] = seed_index[(MIST_P_TILE + j) * MIST_LC_TILE + threadIdx.x];
+      if (row_b[j] >= 0) { fin_b = j + 1; top_b = best_b[j]; }
+      if (row_p[j] >= 0) { fin_p = j + 1; top_p = best_p[j]; }
+    }
+    best_post = seed_cost[(2 * MIST_P_TILE) * MIST_LC_TILE + threadIdx.x];
+    row_post = seed_index[(2 * MIST_P_TILE) * MIST_LC_TILE + threadIdx.x];
+    best_pp = seed_cost[(2 * MIST_P_TILE + 1) * MIST_LC_TILE + threadIdx.x];
+    row_pp = seed_index[(2 * MIST_P_TILE + 1) * MIST_LC_TILE + threadIdx.x];
+  }
 
-  const int64_t row_begin = (int64_t)chunk * g->rows_per_chunk;
-  const int64_t row_end = min(row_begin + (int64_t)g->rows_per_chunk, g->n_rows);
   const double *__restrict__ src = row_terms + g->row_offset * MIST_ROW_TERMS;
 
   const double lf = (double)l, lm1 = (double)max(l - 1, 0), cf = (double)c;
@@ -496,207 +541,279 @@ __device__ __forceinline__ void reduce_block(
   const int post_col = c > 0 ? 0 : 1;
   auto div_G = [&](double v) { return kPow2G ? v * inv_G64 : v / G64; };
 
-  for (int64_t base = row_begin; base < row_end; base += kStageRows) {
-    const int n_stage = (int)min((int64_t)kStageRows, row_end - base);
+  // Stable / delta latency rounded to float32 (:2212-2213), the base objective r * x + y in
+  // float64 (pareto.py:138; y = float32 array / python int, :2815) and a lower bound of the three
+  // composite objectives: they add non-negative terms to x and d before the same monotone
+  // operations, so none of them can be below it.
+  auto objective = [&](const double *__restrict__ t, double &x, double &d, double &cost_base,
+                       double &bound) {
+    const double stable = n_ck * t[MIST_T_S_LAYER_CK] + n_nock * t[MIST_T_S_LAYER_NOCK] +
+                          t[MIST_T_S_FIRST_CK + first_col] + t[MIST_T_S_LAST_CK + last_col];
+    const double delta = n_ck * t[MIST_T_D_LAYER_CK] + n_nock * t[MIST_T_D_LAYER_NOCK] +
+                         t[MIST_T_D_FIRST_CK + first_col] + t[MIST_T_D_LAST_CK + last_col];
+    const float x32 = (float)stable, d32 = (float)delta;
+    x = (double)x32;
+    d = (double)d32;
+    const float y32 = kPow2G ? d32 * inv_G32 : d32 / G32;
+    const double rx = ratio * x;
+    cost_base = rx + (double)y32;
+    bound = rx + div_G(d);
+  };
+
+  // Sieves B (kCommit == false: would the row change anything, judged against the current
+  // minima) and C (kCommit == true: apply it).  Returns whether the row survives / changed a slot.
+  auto examine = [&](const double *__restrict__ t, int32_t row, auto commit_tag) -> bool {
+    constexpr bool kCommit = decltype(commit_tag)::value;
+    double x, d, cost_base, bound;
+    objective(t, x, d, cost_base, bound);
+    const bool cand_b = cost_base <= top_b || fin_b < n_tile;
+    const bool want_pre = bound <= top_p || fin_p < n_tile;
+    const bool want_post = do_post && bound <= best_post;
+    const bool want_pp = do_nopp && bound <= best_pp;
+    if (!(cand_b || want_pre || want_post || want_pp)) return false;
+
+    double cost_pre = INFINITY, cost_post = INFINITY, cost_pp = INFINITY;
+    if (want_pre)
+      cost_pre = ratio * (x + k.pre_fwd + k.pre_bwd + k.w1 + k.w2) + div_G(d + k.w1d + k.w2d);
+    if (want_post || want_pp) {
+      const double nag = t[MIST_T_NAG_CK + post_col], nrs = t[MIST_T_NRS_CK + post_col];
+      const double ps1 = k.pp_wre ? nag : 0.0, ps2 = k.pp_gre ? nrs : 0.0;
+      const double pd1 = k.pp_wre ? 0.0 : nag, pd2 = k.pp_gre ? 0.0 : nrs;
+      const double opb = t[MIST_T_OPB];
+      cost_post = ratio * (x + k.post_fwd + opb + ps1 + ps2) + div_G(d + pd1 + pd2);
+      cost_pp = ratio * (x + k.pre_fwd + k.pre_bwd + k.post_fwd + opb + k.w1 + k.w2 + ps1 + ps2) +
+                div_G(d + k.w1d + k.w2d + pd1 + pd2);
+    }
+
+    // Lowest slot the row could change: the minima are non-decreasing in p, so it is the number
+    // of slots whose minimum is strictly below the row's value (empty slots hold +inf; a tie is
+    // decided by the row index when the slot is updated).
+    int lo_b = fin_b, lo_p = fin_p;
+    if (cost_base <= top_b) {
+      lo_b = 0;
+#pragma unroll
+      for (int j = 0; j < MIST_P_TILE; ++j) lo_b += best_b[j] < cost_base ? 1 : 0;
+    }
+    if (cost_pre <= top_p) {
+      lo_p = 0;
+#pragma unroll
+      for (int j = 0; j < MIST_P_TILE; ++j) lo_p += best_p[j] < cost_pre ? 1 : 0;
+    }
+    bool need_b = cand_b && lo_b < n_tile, need_p = want_pre && lo_p < n_tile;
+    bool need_post = want_post && cost_post <= best_post;
+    bool need_pp = want_pp && cost_pp <= best_pp;
+    if (!(need_b || need_p || need_post || need_pp)) return false;
+
+    // ---- memory that does not depend on p (:2150-2162, 2358-2385, 2760-2769) ----
+    const double S_ck = t[MIST_T_S_CK], S_nock = t[MIST_T_S_NOCK];
+    const double fwd_states = t[MIST_T_FWD_STATES0] + lf * t[MIST_T_PWG] + lm1 * t[MIST_T_PO];
+    const double bwd_states = t[MIST_T_BWD_STATES0] + lf * t[MIST_T_PWGO];
+    const double cur_saved = c_eq_l ? (lf - 1.0) * S_ck : cf * S_ck + l_minus_c_1 * S_nock;
+    const double mod_saved = S_ck * cf + S_nock * l_minus_c;
+    const double ck_delta = c_ge_lm1 ? t[MIST_T_D_CK] : t[MIST_T_D_NOCK];
+    const double fwd_pk = t[MIST_T_FWD_PEAK], bwd_pk = t[MIST_T_BWD_PEAK];
+    const double out = t[MIST_T_OUT], gcb = t[MIST_T_GCB];
+    const double out2 = out * 2.0;
+    const double mf_base = t[MIST_T_MF_BASE], mf_pp = t[MIST_T_MF_PP];
+
+    // Peaks of the middle-stage variant for p pre-saved micro-batches (:2755-2786).
+    auto peaks = [&](int p, double &peak_f, double &peak_b) {
+      const double pf64 = (double)p;
+      const double pipe_saved = pf64 * mod_saved + cur_saved;
+      const double outp2 = out * pf64 * 2.0;
+      peak_f = fwd_states + pipe_saved + ck_delta + fwd_pk + outp2 + gcb;
+      peak_b = bwd_states + pipe_saved + ck_delta + bwd_pk + outp2 + out2 + gcb;
+    };
+    auto feasible_base = [&](int p) {  // (:2805-2812)
+      double pf, pb;
+      peaks(p, pf, pb);
+      return fmax(pf, pb) * mf_base <= cap;
+    };
+    auto feasible_pre = [&](int p) {  // (:2866-2875, 2893-2897)
+      double pf, pb;
+      peaks(p, pf, pb);
+      const double pre_p = (double)p * pre_saved;
+      return fmax(pre_p + pf + pre_sas, pre_p + pb + pre_sas) * mf_pp <= cap;
+    };
+
+    need_b = need_b && feasible_base(p0 + lo_b);
+    need_p = need_p && feasible_pre(p0 + lo_p);
+    bool ok_pp = false;
+    if (need_post || need_pp) {
+      // ---- last stage / single stage, p == 0 only (:2946-3106) ----
+      double peak_f, peak_b;
+      peaks(0, peak_f, peak_b);
+      const double f_in = fwd_states + post_states + mod_saved + post_fwd_peak + gcb;
+      const double b_in = bwd_states + post_states + mod_saved + post_bwd_peak +
+                          (c_eq_0 ? t[MIST_T_RD] : 0.0) + gcb;
+      const double pf_post = fmax(f_in, peak_f + post_states);
+      const double pb_post = fmax(b_in, peak_b - out + post_states) + post_output;
+      const bool ok_post = fmax(pf_post, pb_post) * mf_pp <= cap;
+      if (need_pp) {
+        const double pf_pp = pf_post + pre_states + pre_saved;
+        const double pb_pp = pb_post + pre_states + pre_saved;
+        ok_pp = fmax(pf_pp, pb_pp) * t[MIST_T_MF] <= cap;
+      }
+      need_post = need_post && ok_post;
+      need_pp = need_pp && ok_pp;
+    }
+    if (!kCommit) return need_b || need_p || need_post || need_pp;
+
+    bool changed = false;
+    if (need_b) {
+      const double cost = cost_base;
+      int lo = lo_b + 1, hi = n_tile;  // number of feasible p of this tile lies in [lo, hi]
+      for (int it = 0; it < steps; ++it) {
+        const int mid = (lo + hi) >> 1;
+        const bool ok = feasible_base(p0 + mid);
+        const bool open = lo < hi;
+        lo = (open && ok) ? mid + 1 : lo;
+        hi = (open && !ok) ? mid : hi;
+      }
+#pragma unroll
+      for (int j = 0; j < MIST_P_TILE; ++j) {
+        const bool better = j >= lo_b && j < lo && lex_less(cost, row, best_b[j], row_b[j]);
+        best_b[j] = better ? cost : best_b[j];
+        row_b[j] = better ? row : row_b[j];
+        changed |= better;
+      }
+      // Bookkeeping of (fin, top) without indexing the register array dynamically.
+      if (lo > fin_b) { fin_b = lo; top_b = cost; }
+      else if (lo == fin_b) top_b = fmin(top_b, cost);
+    }
+    if (need_p) {
+      const double cost = cost_pre;
+      int lo = lo_p + 1, hi = n_tile;
+      for (int it = 0; it < steps; ++it) {
+        const int mid = (lo + hi) >> 1;
+        const bool ok = feasible_pre(p0 + mid);
+        const bool open = lo < hi;
+        lo = (open && ok) ? mid + 1 : lo;
+        hi = (open && !ok) ? mid : hi;
+      }
+#pragma unroll
+      for (int j = 0; j < MIST_P_TILE; ++j) {
+        const bool better = j >= lo_p && j < lo && lex_less(cost, row, best_p[j], row_p[j]);
+        best_p[j] = better ? cost : best_p[j];
+        row_p[j] = better ? row : row_p[j];
+        changed |= better;
+      }
+      if (lo > fin_p) { fin_p = lo; top_p = cost; }
+      else if (lo == fin_p) top_p = fmin(top_p, cost);
+    }
+    if (need_post) {
+      changed |= lex_less(cost_post, row, best_post, row_post);
+      take_min(best_post, row_post, true, cost_post, row);
+    }
+    if (need_pp) {
+      changed |= lex_less(cost_pp, row, best_pp, row_pp);
+      take_min(best_pp, row_pp, true, cost_pp, row);
+    }
+    return changed;
+  };
+
+  const int64_t first_stage = range.row_begin / kStageRows;
+  const int64_t end_stage = (range.row_end + kStageRows - 1) / kStageRows;
+  for (int64_t stage = first_stage; stage < end_stage; stage += range.stage_step) {
+    if (range.skip_stride > 0 && stage % range.skip_stride == 0) continue;
+    const int64_t base = stage * kStageRows;
+    const int n_stage = (int)min((int64_t)kStageRows, range.row_end - base);
     __syncthreads();
     for (int i = threadIdx.x; i < n_stage * MIST_ROW_TERMS; i += MIST_LC_TILE)
-      lds_terms[i] = src[base * MIST_ROW_TERMS + i];
+      lds_terms[(i / MIST_ROW_TERMS) * kLdsRowStride + i % MIST_ROW_TERMS] =
+          src[base * MIST_ROW_TERMS + i];
     __syncthreads();
     if (!active) continue;
 
-    for (int r0 = 0; r0 < n_stage; r0 += kRowUnroll) {
-      // ---- latencies and objective values of kRowUnroll rows (:2165-2351; pareto.py:138:
-      // r * x + y in float64).  Independent of the running minima, hence computed together;
-      // rows past the end of the stage read stale LDS and are ignored below. ----
-      double xs[kRowUnroll], ds[kRowUnroll], cost_base[kRowUnroll], bound[kRowUnroll];
+    // ---- sieve A: all rows of the stage against the largest minima ----
+    const double thr_b = fin_b < n_tile ? INFINITY : top_b;
+    double thr_o = fin_p < n_tile ? INFINITY : top_p;
+    if (do_post) thr_o = fmax(thr_o, best_post);
+    if (do_nopp) thr_o = fmax(thr_o, best_pp);
+    uint64_t sieve = 0;
+    for (int r0 = 0; r0 < kStageRows; r0 += kRowUnroll) {
 #pragma unroll
       for (int u = 0; u < kRowUnroll; ++u) {
-        const double *__restrict__ t = lds_terms + min(r0 + u, kStageRows - 1) * MIST_ROW_TERMS;
-        const double stable = n_ck * t[MIST_T_S_LAYER_CK] + n_nock * t[MIST_T_S_LAYER_NOCK] +
-                              t[MIST_T_S_FIRST_CK + first_col] + t[MIST_T_S_LAST_CK + last_col];
-        const double delta = n_ck * t[MIST_T_D_LAYER_CK] + n_nock * t[MIST_T_D_LAYER_NOCK] +
-                             t[MIST_T_D_FIRST_CK + first_col] + t[MIST_T_D_LAST_CK + last_col];
-        const float x32 = (float)stable, d32 = (float)delta;  // (:2212-2213)
-        xs[u] = (double)x32;
-        ds[u] = (double)d32;
-        const float y32 = kPow2G ? d32 * inv_G32 : d32 / G32;  // float32 array / python int (:2815)
-        cost_base[u] = ratio * xs[u] + (double)y32;
-        // Lower bound of the three composite objectives: they add non-negative terms to x and
-        // d before the same monotone operations, so none of them can be below this value.
-        bound[u] = ratio * xs[u] + div_G(ds[u]);
+        double x, d, cost_base, bound;
+        objective(lds_terms + (r0 + u) * kLdsRowStride, x, d, cost_base, bound);
+        const bool pass = cost_base <= thr_b || bound <= thr_o;
+        sieve |= (uint64_t)(pass ? 1 : 0) << (r0 + u);
       }
+    }
+    // Rows past the end of the stage hold stale LDS contents.
+    if (n_stage < kStageRows) sieve &= (1ull << n_stage) - 1ull;
 
-#pragma unroll
-      for (int u = 0; u < kRowUnroll; ++u) {
-        if (r0 + u >= n_stage) break;
-        const double *__restrict__ t = lds_terms + (r0 + u) * MIST_ROW_TERMS;
-        const int32_t row = (int32_t)(base + r0 + u);
-        const double x = xs[u], d = ds[u];
-        // Which composite objectives can still matter for this row.
-        const bool want_pre = bound[u] < top_p || fin_p < n_tile;
-        const bool want_post = kFirstTile && bound[u] < best_post;
-        const bool want_pp = do_nopp && bound[u] < best_pp;
-        if (!(cost_base[u] < top_b || fin_b < n_tile || want_pre || want_post || want_pp)) continue;
+    // ---- sieve B: lowest improvable slot and the memory test there, per-lane survivors ----
+    uint64_t keep = 0;
+    while (sieve != 0) {
+      const int r = __ffsll((unsigned long long)sieve) - 1;
+      sieve &= sieve - 1;
+      const bool hit = examine(lds_terms + r * kLdsRowStride, (int32_t)(base + r),
+                               std::false_type{});
+      keep |= (uint64_t)(hit ? 1 : 0) << r;
+    }
 
-        double cost_pre = INFINITY, cost_post = INFINITY, cost_pp = INFINITY;
-        if (want_pre)
-          cost_pre = ratio * (x + k.pre_fwd + k.pre_bwd + k.w1 + k.w2) + div_G(d + k.w1d + k.w2d);
-        if (want_post || want_pp) {
-          const double nag = t[MIST_T_NAG_CK + post_col], nrs = t[MIST_T_NRS_CK + post_col];
-          const double ps1 = k.pp_wre ? nag : 0.0, ps2 = k.pp_gre ? nrs : 0.0;
-          const double pd1 = k.pp_wre ? 0.0 : nag, pd2 = k.pp_gre ? 0.0 : nrs;
-          const double opb = t[MIST_T_OPB];
-          cost_post = ratio * (x + k.post_fwd + opb + ps1 + ps2) + div_G(d + pd1 + pd2);
-          cost_pp =
-              ratio * (x + k.pre_fwd + k.pre_bwd + k.post_fwd + opb + k.w1 + k.w2 + ps1 + ps2) +
-              div_G(d + k.w1d + k.w2d + pd1 + pd2);
-        }
-
-        // Lowest slot the row could improve: the minima are non-decreasing in p, so it is the
-        // number of slots whose minimum the row does not beat (empty slots hold +inf).  The row
-        // changes something iff it is feasible at that slot (feasibility is monotone in p).
-        int lo_b = fin_b, lo_p = fin_p;
-        if (cost_base[u] < top_b) {
-          lo_b = 0;
-#pragma unroll
-          for (int j = 0; j < MIST_P_TILE; ++j) lo_b += cost_base[u] >= best_b[j] ? 1 : 0;
-        }
-        if (cost_pre < top_p) {
-          lo_p = 0;
-#pragma unroll
-          for (int j = 0; j < MIST_P_TILE; ++j) lo_p += cost_pre >= best_p[j] ? 1 : 0;
-        }
-        bool need_b = lo_b < n_tile, need_p = want_pre && lo_p < n_tile;
-        const bool need_post = want_post && cost_post < best_post;
-        const bool need_pp = want_pp && cost_pp < best_pp;
-        if (!(need_b || need_p || need_post || need_pp)) continue;
-
-        // ---- memory that does not depend on p (:2150-2162, 2358-2385, 2760-2769) ----
-        const double S_ck = t[MIST_T_S_CK], S_nock = t[MIST_T_S_NOCK];
-        const double fwd_states = t[MIST_T_FWD_STATES0] + lf * t[MIST_T_PWG] + lm1 * t[MIST_T_PO];
-        const double bwd_states = t[MIST_T_BWD_STATES0] + lf * t[MIST_T_PWGO];
-        const double cur_saved = c_eq_l ? (lf - 1.0) * S_ck : cf * S_ck + l_minus_c_1 * S_nock;
-        const double mod_saved = S_ck * cf + S_nock * l_minus_c;
-        const double ck_delta = c_ge_lm1 ? t[MIST_T_D_CK] : t[MIST_T_D_NOCK];
-        const double fwd_pk = t[MIST_T_FWD_PEAK], bwd_pk = t[MIST_T_BWD_PEAK];
-        const double out = t[MIST_T_OUT], gcb = t[MIST_T_GCB];
-        const double out2 = out * 2.0;
-        const double mf_base = t[MIST_T_MF_BASE], mf_pp = t[MIST_T_MF_PP];
-
-        // Peaks of the middle-stage variant for p pre-saved micro-batches (:2755-2786).
-        auto peaks = [&](int p, double &peak_f, double &peak_b) {
-          const double pf64 = (double)p;
-          const double pipe_saved = pf64 * mod_saved + cur_saved;
-          const double outp2 = out * pf64 * 2.0;
-          peak_f = fwd_states + pipe_saved + ck_delta + fwd_pk + outp2 + gcb;
-          peak_b = bwd_states + pipe_saved + ck_delta + bwd_pk + outp2 + out2 + gcb;
-        };
-        auto feasible_base = [&](int p) {  // (:2805-2812)
-          double pf, pb;
-          peaks(p, pf, pb);
-          return fmax(pf, pb) * mf_base <= cap;
-        };
-        auto feasible_pre = [&](int p) {  // (:2866-2875, 2893-2897)
-          double pf, pb;
-          peaks(p, pf, pb);
-          const double pre_p = (double)p * pre_saved;
-          return fmax(pre_p + pf + pre_sas, pre_p + pb + pre_sas) * mf_pp <= cap;
-        };
-
-        need_b = need_b && feasible_base(p0 + lo_b);
-        need_p = need_p && feasible_pre(p0 + lo_p);
-
-        if (need_b) {
-          const double cost = cost_base[u];
-          int lo = lo_b + 1, hi = n_tile;  // number of feasible p of this tile lies in [lo, hi]
-          for (int it = 0; it < steps; ++it) {
-            const int mid = (lo + hi) >> 1;
-            const bool ok = feasible_base(p0 + mid);
-            const bool open = lo < hi;
-            lo = (open && ok) ? mid + 1 : lo;
-            hi = (open && !ok) ? mid : hi;
-          }
-#pragma unroll
-          for (int j = 0; j < MIST_P_TILE; ++j) {
-            const bool better = j >= lo_b && j < lo;  // exactly the slots with cost < minimum
-            best_b[j] = better ? cost : best_b[j];
-            row_b[j] = better ? row : row_b[j];
-          }
-          // Bookkeeping of (fin, top) without indexing the register array dynamically.
-          if (lo > fin_b) { fin_b = lo; top_b = cost; }
-          else if (lo == fin_b && cost < top_b) top_b = cost;
-        }
-        if (need_p) {
-          const double cost = cost_pre;
-          int lo = lo_p + 1, hi = n_tile;
-          for (int it = 0; it < steps; ++it) {
-            const int mid = (lo + hi) >> 1;
-            const bool ok = feasible_pre(p0 + mid);
-            const bool open = lo < hi;
-            lo = (open && ok) ? mid + 1 : lo;
-            hi = (open && !ok) ? mid : hi;
-          }
-#pragma unroll
-          for (int j = 0; j < MIST_P_TILE; ++j) {
-            const bool better = j >= lo_p && j < lo;
-            best_p[j] = better ? cost : best_p[j];
-            row_p[j] = better ? row : row_p[j];
-          }
-          if (lo > fin_p) { fin_p = lo; top_p = cost; }
-          else if (lo == fin_p && cost < top_p) top_p = cost;
-        }
-
-        if (need_post || need_pp) {
-          // ---- last stage / single stage, p == 0 only (:2946-3106) ----
-          double peak_f, peak_b;
-          peaks(0, peak_f, peak_b);
-          const double f_in = fwd_states + post_states + mod_saved + post_fwd_peak + gcb;
-          const double b_in = bwd_states + post_states + mod_saved + post_bwd_peak +
-                              (c_eq_0 ? t[MIST_T_RD] : 0.0) + gcb;
-          const double pf_post = fmax(f_in, peak_f + post_states);
-          const double pb_post = fmax(b_in, peak_b - out + post_states) + post_output;
-          const bool ok_post = fmax(pf_post, pb_post) * mf_pp <= cap;
-          take_min(best_post, row_post, need_post && ok_post, cost_post, row);
-          if (need_pp) {
-            const double pf_pp = pf_post + pre_states + pre_saved;
-            const double pb_pp = pb_post + pre_states + pre_saved;
-            const bool ok_pp = fmax(pf_pp, pb_pp) * t[MIST_T_MF] <= cap;
-            take_min(best_pp, row_pp, ok_pp, cost_pp, row);
-          }
-        }
-      }
+    // ---- sieve C: survivors in row order against the live minima ----
+    while (keep != 0) {
+      const int r = __ffsll((unsigned long long)keep) - 1;
+      keep &= keep - 1;
+      examine(lds_terms + r * kLdsRowStride, (int32_t)(base + r), std::true_type{});
     }
   }
 
-  const int64_t out_base = (int64_t)blockIdx.x * kSlots * MIST_LC_TILE + threadIdx.x;
 #pragma unroll
   for (int j = 0; j < MIST_P_TILE; ++j) {
-    partial_cost[out_base + (int64_t)j * MIST_LC_TILE] = best_b[j];
-    partial_index[out_base + (int64_t)j * MIST_LC_TILE] = row_b[j];
-    partial_cost[out_base + (int64_t)(MIST_P_TILE + j) * MIST_LC_TILE] = best_p[j];
-    partial_index[out_base + (int64_t)(MIST_P_TILE + j) * MIST_LC_TILE] = row_p[j];
+    out_cost[j * MIST_LC_TILE + threadIdx.x] = best_b[j];
+    out_index[j * MIST_LC_TILE + threadIdx.x] = row_b[j];
+    out_cost[(MIST_P_TILE + j) * MIST_LC_TILE + threadIdx.x] = best_p[j];
+    out_index[(MIST_P_TILE + j) * MIST_LC_TILE + threadIdx.x] = row_p[j];
   }
-  partial_cost[out_base + (int64_t)(2 * MIST_P_TILE) * MIST_LC_TILE] = best_post;
-  partial_index[out_base + (int64_t)(2 * MIST_P_TILE) * MIST_LC_TILE] = row_post;
-  partial_cost[out_base + (int64_t)(2 * MIST_P_TILE + 1) * MIST_LC_TILE] = best_pp;
-  partial_index[out_base + (int64_t)(2 * MIST_P_TILE + 1) * MIST_LC_TILE] = row_pp;
+  out_cost[(2 * MIST_P_TILE) * MIST_LC_TILE + threadIdx.x] = best_post;
+  out_index[(2 * MIST_P_TILE) * MIST_LC_TILE + threadIdx.x] = row_post;
+  out_cost[(2 * MIST_P_TILE + 1) * MIST_LC_TILE + threadIdx.x] = best_pp;
+  out_index[(2 * MIST_P_TILE + 1) * MIST_LC_TILE + threadIdx.x] = row_pp;
 }
 
+// scout != 0: one workgroup per (group, (l, c) tile, p tile) over every scout_stride-th stage of
+// the whole group, results in slab n_blocks + blockIdx.x.  scout == 0: one workgroup per row
+// chunk of such a tile, seeded from the scout's slab when the group has one.
 __global__ __launch_bounds__(MIST_LC_TILE, MIST_REDUCE_MIN_WAVES) void eval_reduce_kernel(
     const MistProblem prob, const MistGroupDesc *__restrict__ groups, int n_groups,
-    const int32_t *__restrict__ block_prefix, const double *__restrict__ row_terms, double ratio,
-    double *__restrict__ partial_cost, int32_t *__restrict__ partial_index) {
-  __shared__ double lds_terms[kStageRows * MIST_ROW_TERMS];
+    const int32_t *__restrict__ block_prefix, int n_blocks,
+    const int32_t *__restrict__ scout_prefix, int scout, const double *__restrict__ row_terms,
+    double ratio, double *__restrict__ partial_cost, int32_t *__restrict__ partial_index) {
+  __shared__ double lds_terms[kStageRows * kLdsRowStride];
   int local_block;
-  const MistGroupDesc *g = find_group(groups, block_prefix, n_groups, blockIdx.x, &local_block);
-  const int chunk = local_block % g->n_chunks;
-  const int tile = local_block / g->n_chunks;
+  const MistGroupDesc *g = find_group(groups, scout ? scout_prefix : block_prefix, n_groups,
+                                      blockIdx.x, &local_block);
+  const int gi = (int)(g - groups);
+  const bool seeded = scout_prefix != nullptr && g->scout_stride > 0;
+  int tile;
+  ReduceRange range;
+  int64_t out_slab;
+  if (scout) {
+    if (g->scout_stride <= 0) return;
+    tile = local_block;
+    range = ReduceRange{0, g->n_rows, g->scout_stride, 0};
+    out_slab = (int64_t)n_blocks + blockIdx.x;
+  } else {
+    const int chunk = local_block % g->n_chunks;
+    tile = local_block / g->n_chunks;
+    const int64_t row_begin = (int64_t)chunk * g->rows_per_chunk;
+    range = ReduceRange{row_begin, min(row_begin + (int64_t)g->rows_per_chunk, g->n_rows), 1,
+                        seeded ? g->scout_stride : 0};
+    out_slab = blockIdx.x;
+  }
   const int p_tile = tile % g->n_p_tiles;
   const int lc_tile = tile / g->n_p_tiles;
+  const int64_t slab = (int64_t)kSlots * MIST_LC_TILE;
+  const int64_t seed_slab = (int64_t)n_blocks + (seeded ? scout_prefix[gi] + tile : 0);
+  const double *seed_cost = (!scout && seeded) ? partial_cost + seed_slab * slab : nullptr;
+  const int32_t *seed_index = (!scout && seeded) ? partial_index + seed_slab * slab : nullptr;
   const bool pow2 = (g->grad_accum & (g->grad_accum - 1)) == 0;
 #define MIST_REDUCE(P2, FT)                                                                   \
-  reduce_block<P2, FT>(prob, g, chunk, p_tile, lc_tile, row_terms, ratio, lds_terms,          \
-                       partial_cost, partial_index)
+  reduce_block<P2, FT>(prob, g, range, p_tile, lc_tile, row_terms, ratio, lds_terms, seed_cost, \
+                       seed_index, partial_cost + out_slab * slab, partial_index + out_slab * slab)
   if (pow2) {
     if (p_tile == 0) MIST_REDUCE(true, true); else MIST_REDUCE(true, false);
   } else {
@@ -706,7 +823,7 @@ __global__ __launch_bounds__(MIST_LC_TILE, MIST_REDUCE_MIN_WAVES) void eval_redu
 }
 
 // ------------------------------------------------------------------------------------------
-// Kernel 3: combine chunks in order, recompute the winner's stable / delta, scatter.
+// Kernel 3: combine the chunks' (cost, row) minima, recompute the winner's stable / delta, scatter.
 // One thread per (group, (l, c) pair, slot); slots as in the reduce kernel but over all p.
 // ------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void finalize_kernel(
@@ -802,18 +919,33 @@ int mist_row_terms(const MistProblem *problem, const MistGroupDesc *d_groups, in
   return 0;
 }
 
+int mist_reduce_stage_rows(void) { return kStageRows; }
+int mist_reduce_lc_tile(void) { return MIST_LC_TILE; }
+
 int mist_eval_reduce(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,
-                     const int32_t *d_block_prefix, int n_blocks, const double *d_row_terms,
-                     double ratio, double *d_partial_cost, int32_t *d_partial_index,
-                     void *stream) {
+                     const int32_t *d_block_prefix, int n_blocks,
+                     const int32_t *d_scout_prefix, int n_scout_blocks,
+                     const double *d_row_terms, double ratio, double *d_partial_cost,
+                     int32_t *d_partial_index, void *stream) {
   if (int rc = check_common(problem, d_groups, n_groups)) return rc;
   if (!d_block_prefix || !d_row_terms || !d_partial_cost || !d_partial_index)
     return fail(MIST_E_INVALID, "null workspace pointer");
   if (n_blocks <= 0) return fail(MIST_E_INVALID, "n_blocks must be positive, got %d", n_blocks);
   if (!(ratio >= 0.0)) return fail(MIST_E_INVALID, "ratio must be non-negative");
+  if (n_scout_blocks < 0 || (n_scout_blocks > 0 && !d_scout_prefix))
+    return fail(MIST_E_INVALID, "scout blocks need a scout prefix (n_scout_blocks=%d)",
+                n_scout_blocks);
+  const int32_t *scout_prefix = n_scout_blocks > 0 ? d_scout_prefix : nullptr;
+  if (scout_prefix) {
+    hipLaunchKernelGGL(eval_reduce_kernel, dim3(n_scout_blocks), dim3(MIST_LC_TILE), 0,
+                       (hipStream_t)stream, *problem, d_groups, n_groups, d_block_prefix,
+                       n_blocks, scout_prefix, 1, d_row_terms, ratio, d_partial_cost,
+                       d_partial_index);
+    MIST_HIP_CHECK(hipGetLastError());
+  }
   hipLaunchKernelGGL(eval_reduce_kernel, dim3(n_blocks), dim3(MIST_LC_TILE), 0,
-                     (hipStream_t)stream, *problem, d_groups, n_groups, d_block_prefix,
-                     d_row_terms, ratio, d_partial_cost, d_partial_index);
+                     (hipStream_t)stream, *problem, d_groups, n_groups, d_block_prefix, n_blocks,
+                     scout_prefix, 0, d_row_terms, ratio, d_partial_cost, d_partial_index);
   MIST_HIP_CHECK(hipGetLastError());
   return 0;
 }
@@ -847,7 +979,7 @@ int mist_finalize(const MistProblem *problem, const MistGroupDesc *d_groups, int
 int mist_intra_stage_eval(const MistProblem *problem, const MistGroupDesc *d_groups,
                           int n_groups, const int32_t *d_terms_block_prefix, int n_terms_blocks,
                           const int32_t *d_reduce_block_prefix, int n_reduce_blocks,
-                          double *d_row_terms, double *d_partial_cost, int32_t *d_partial_index,
+                          const int32_t *d_scout_prefix, int n_scout_blocks, double *d_row_terms, double *d_partial_cost, int32_t *d_partial_index,
                           double ratio, int sample_index, int compute_terms,
                           const MistOutTables *tables, void *stream) {
   if (compute_terms) {
@@ -856,8 +988,8 @@ int mist_intra_stage_eval(const MistProblem *problem, const MistGroupDesc *d_gro
       return rc;
   }
   if (int rc = mist_eval_reduce(problem, d_groups, n_groups, d_reduce_block_prefix,
-                                n_reduce_blocks, d_row_terms, ratio, d_partial_cost,
-                                d_partial_index, stream))
+                                n_reduce_blocks, d_scout_prefix, n_scout_blocks, d_row_terms,
+                                ratio, d_partial_cost, d_partial_index, stream))
     return rc;
   return mist_finalize(problem, d_groups, n_groups, d_reduce_block_prefix, d_row_terms,
                        d_partial_cost, d_partial_index, sample_index, tables, stream);

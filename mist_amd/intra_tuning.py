@@ -24,7 +24,9 @@ from .stage_inputs import GroupInputBuilder, make_problem
 
 SAMPLE_SIZE = 30  # reference default (batched_module_analyzer.py:67)
 VARIANTS = ("", "_with_pre", "_with_post", "_no_pp")
-TARGET_REDUCE_BLOCKS = 6144
+TARGET_REDUCE_WAVES = 24576  # wavefronts of the reduce kernel the row chunks are sized for
+SCOUT_STAGES = 32      # stages of a group the scout pass of the reduce kernel samples
+MIN_SCOUT_STRIDE = 4   # groups with fewer than SCOUT_STAGES * this many stages get no scout pass
 
 
 def alpha_ratios(sample_size: int) -> np.ndarray:
@@ -203,7 +205,7 @@ class IntraStageTuner:
         if len(pending):
             n_p_tiles = -(-groups["num_p"] // _lib.P_TILE)
             tile_rows = int(np.sum(groups["n_rows"] * n_lc_tiles * n_p_tiles))
-            rows_per_chunk = -(-tile_rows // TARGET_REDUCE_BLOCKS)
+            rows_per_chunk = -(-tile_rows // max(TARGET_REDUCE_WAVES * 64 // _lib.LC_TILE, 1))
             rows_per_chunk = max(256, min(16384, -(-rows_per_chunk // _lib.STAGE_ROWS) * _lib.STAGE_ROWS))
             groups["rows_per_chunk"] = rows_per_chunk
             groups["n_chunks"] = -(-groups["n_rows"] // rows_per_chunk)
@@ -212,16 +214,25 @@ class IntraStageTuner:
             groups["row_offset"] = np.concatenate(([0], np.cumsum(groups["n_rows"])[:-1]))
             terms_blocks = -(-groups["n_rows"] // _lib.TERMS_BLOCK)
             reduce_blocks = groups["n_chunks"].astype(np.int64) * n_lc_tiles * n_p_tiles
+            # Scout pass: about SCOUT_STAGES evenly spaced stages of each group seed its chunks.
+            n_stages = -(-groups["n_rows"] // _lib.STAGE_ROWS)
+            stride = n_stages // SCOUT_STAGES if SCOUT_STAGES > 0 else np.zeros_like(n_stages)
+            groups["scout_stride"] = np.where(stride >= MIN_SCOUT_STRIDE, stride, 0)
+            scout_blocks = np.full(len(pending), n_lc_tiles, dtype=np.int64) * n_p_tiles
+            if not np.any(groups["scout_stride"] > 0):
+                scout_blocks[:] = 0
         else:
-            terms_blocks = reduce_blocks = np.zeros(0, dtype=np.int64)
+            terms_blocks = reduce_blocks = scout_blocks = np.zeros(0, dtype=np.int64)
         terms_prefix = np.concatenate(([0], np.cumsum(terms_blocks))).astype(np.int64)
         reduce_prefix = np.concatenate(([0], np.cumsum(reduce_blocks))).astype(np.int64)
-        if terms_prefix[-1] >= 2**31 or reduce_prefix[-1] >= 2**31:
+        scout_prefix = np.concatenate(([0], np.cumsum(scout_blocks))).astype(np.int64)
+        if terms_prefix[-1] >= 2**31 or reduce_prefix[-1] + scout_prefix[-1] >= 2**31:
             raise ValueError("launch decomposition exceeds 2**31 workgroups")
         problem = make_problem(cfg, L, P + 1, self.sample_size, len(self.tp_sizes) * len(Gs), len(Q))
         return dict(
             problem=problem, groups=groups, spaces=spaces,
             terms_prefix=terms_prefix.astype(np.int32), reduce_prefix=reduce_prefix.astype(np.int32),
+            scout_prefix=scout_prefix.astype(np.int32),
             total_rows=int(groups["n_rows"].sum()) if len(pending) else 0,
         )
 
@@ -244,6 +255,8 @@ class IntraStageTuner:
             return torch.from_numpy(np.ascontiguousarray(a).view(np.uint8).reshape(-1)).to(dev)
         n_groups = len(plan["groups"])
         n_reduce_blocks = int(plan["reduce_prefix"][-1])
+        n_scout_blocks = int(plan["scout_prefix"][-1])
+        n_slabs = max(n_reduce_blocks + n_scout_blocks, 1)
         return dict(
             n_groups=n_groups,
             groups=to_dev(plan["groups"]) if n_groups else None,
@@ -251,9 +264,11 @@ class IntraStageTuner:
             reduce_prefix=to_dev(plan["reduce_prefix"]),
             n_terms_blocks=int(plan["terms_prefix"][-1]),
             n_reduce_blocks=n_reduce_blocks,
+            scout_prefix=to_dev(plan["scout_prefix"]),
+            n_scout_blocks=n_scout_blocks,
             row_terms=torch.empty(max(plan["total_rows"], 1) * _lib.ROW_TERMS, dtype=torch.float64, device=dev),
-            partial_cost=torch.empty(max(n_reduce_blocks, 1) * _lib.SLOTS * _lib.LC_TILE, dtype=torch.float64, device=dev),
-            partial_index=torch.empty(max(n_reduce_blocks, 1) * _lib.SLOTS * _lib.LC_TILE, dtype=torch.int32, device=dev),
+            partial_cost=torch.empty(n_slabs * _lib.SLOTS * _lib.LC_TILE, dtype=torch.float64, device=dev),
+            partial_index=torch.empty(n_slabs * _lib.SLOTS * _lib.LC_TILE, dtype=torch.int32, device=dev),
         )
 
     def launch(self, plan, dev_plan, tables: DeviceTables, events: Optional[list] = None) -> None:
@@ -274,6 +289,7 @@ class IntraStageTuner:
                     prob_ptr, _ptr(d["groups"]), d["n_groups"],
                     _ptr(d["terms_prefix"]), d["n_terms_blocks"],
                     _ptr(d["reduce_prefix"]), d["n_reduce_blocks"],
+                    _ptr(d["scout_prefix"]), d["n_scout_blocks"],
                     _ptr(d["row_terms"]), _ptr(d["partial_cost"]),
                     _ptr(d["partial_index"]), float(ratios[slot]), int(slot),
                     1 if i == 0 else 0, ctypes.byref(out), stream,
@@ -295,7 +311,8 @@ class IntraStageTuner:
                     d["n_terms_blocks"], _ptr(d["row_terms"]), stream))
             timed("eval_reduce", lambda: lib.mist_eval_reduce(
                 prob_ptr, _ptr(d["groups"]), d["n_groups"], _ptr(d["reduce_prefix"]),
-                d["n_reduce_blocks"], _ptr(d["row_terms"]), float(ratios[slot]),
+                d["n_reduce_blocks"], _ptr(d["scout_prefix"]), d["n_scout_blocks"],
+                _ptr(d["row_terms"]), float(ratios[slot]),
                 _ptr(d["partial_cost"]), _ptr(d["partial_index"]), stream))
             timed("finalize", lambda: lib.mist_finalize(
                 prob_ptr, _ptr(d["groups"]), d["n_groups"], _ptr(d["reduce_prefix"]),

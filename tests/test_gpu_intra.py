@@ -136,3 +136,20 @@ def test_sample_subset():
     """Only slot 0 of S = 30 (what the uniform inter-stage search consumes)."""
     cfg, tables = tiny_plan(1, layers=5)
     _compare(cfg, tables, 1, S=30, slots=[0])
+
+
+@pytest.mark.parametrize("scout_stages, min_stride", [(1, 1), (3, 1), (7, 2), (0, 1)])
+def test_scout_pass_leaves_results_unchanged(monkeypatch, scout_stages, min_stride):
+    """The scout pass only seeds the chunks with minima of real rows: forcing it on (with
+    different sampling densities) or off must give the oracle's tables, ties included."""
+    from mist_amd import intra_tuning
+
+    monkeypatch.setattr(intra_tuning, "SCOUT_STAGES", scout_stages)
+    monkeypatch.setattr(intra_tuning, "MIN_SCOUT_STRIDE", min_stride)
+    cfg, tables = tiny_plan(1, layers=6, hardware__memory_capacity=6.0)
+    tuner = _gpu_tuner(cfg, tables, 1)
+    strides = tuner.prepare()["groups"]["scout_stride"]
+    assert (strides > 0).any() == (scout_stages > 0)
+    _compare(cfg, tables, 1)
+    cfg, tables = load_plan(1)
+    _compare(cfg, tables, 2)

@@ -194,8 +194,10 @@ def test_argument_checks_reject_before_any_launch():
     pp = ctypes.c_void_p(prob.ctypes.data)
     fake = ctypes.c_void_p(4096)
     assert lib.mist_row_terms(pp, fake, 0, fake, 1, fake, None) == -1
-    assert lib.mist_eval_reduce(pp, fake, 1, fake, 0, fake, 1.0, fake, fake, None) == -1
-    assert lib.mist_eval_reduce(pp, fake, 1, fake, 1, fake, -1.0, fake, fake, None) == -1
+    assert lib.mist_eval_reduce(pp, fake, 1, fake, 0, None, 0, fake, 1.0, fake, fake, None) == -1
+    assert lib.mist_eval_reduce(pp, fake, 1, fake, 1, None, 0, fake, -1.0, fake, fake, None) == -1
+    assert lib.mist_eval_reduce(pp, fake, 1, fake, 1, None, 3, fake, 1.0, fake, fake, None) == -1
+    assert b"scout" in lib.mist_last_error()
     tabs = _lib.OutTables()
     assert lib.mist_finalize(pp, fake, 1, fake, fake, fake, fake, 0, ctypes.byref(tabs), None) == -1
     shape = np.zeros(1, dtype=_lib.DP_SHAPE_DTYPE)

@@ -26,9 +26,7 @@ extern "C" {
 #define MIST_MAX_PAIRS (MIST_MAX_RATIOS * MIST_MAX_RATIOS)
 #define MIST_PAR_FIELDS 20
 #define MIST_ROW_TERMS 34   /* doubles per candidate row produced by mist_row_terms */
-#ifndef MIST_LC_TILE
 #define MIST_LC_TILE 64     /* (layers, ckpt) pairs per workgroup (one wavefront) of the reduce kernel */
-#endif
 #ifndef MIST_P_TILE
 #define MIST_P_TILE 16      /* pre-saved micro-batch values per thread of the reduce kernel */
 #endif
@@ -140,6 +138,7 @@ int mist_sizeof_problem(void);
 int mist_sizeof_group(void);
 int mist_reduce_p_tile(void); /* MIST_P_TILE the library was built with */
 int mist_reduce_lc_tile(void); /* MIST_LC_TILE the library was built with */
+int mist_reduce_scout_split(void); /* scout workgroups per (group, (l, c) tile, p tile) */
 int mist_reduce_stage_rows(void); /* rows per LDS stage; rows_per_chunk must be a multiple */
 
 /* Row-invariant terms of every candidate row: decodes the row index, evaluates the alpha-beta
@@ -149,7 +148,10 @@ int mist_reduce_stage_rows(void); /* rows per LDS stage; rows_per_chunk must be 
  * (with predict_gpu_gpu_comm_latency / predict_cpu_gpu_comm_latency /
  * interference_estimate_for_one_group of mist/tools/optimize.py:201-303,459-470,1012-1122).
  * d_block_prefix[n_groups+1]: first workgroup of each group, 256 rows per workgroup.
- * d_row_terms: [total_rows][MIST_ROW_TERMS] float64. */
+ * d_row_terms: [total_rows][MIST_ROW_TERMS] float64.  Within a group the workspace is ordered
+ *   position = ((par * n_ao + ao) * n_oo + oo) * n_pair + pair
+ * (rows of similar memory footprint next to each other, which the reduce kernel's per-stage
+ * bound relies on for speed, not for correctness); all results carry reference row numbers. */
 int mist_row_terms(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,
                    const int32_t *d_block_prefix, int n_blocks, double *d_row_terms,
                    void *stream);
@@ -159,10 +161,10 @@ int mist_row_terms(const MistProblem *problem, const MistGroupDesc *d_groups, in
  * Replaces the two hot loops of batched_stage_analyze (batched_module_analyzer.py:2218-3106)
  * and compute_indices (mist/utils/pareto.py:124-144) for one ratio r = alpha/(1-alpha).
  * d_block_prefix[n_groups+1]: first workgroup of each group; a group owns
- * n_lc_tiles*n_p_tiles*n_chunks workgroups ordered (lc_tile, p_tile, chunk), chunk fastest.
+ * n_lc_tiles*n_p_tiles*n_chunks workgroups ordered (chunk, lc_tile, p_tile), p_tile fastest.
  * Optional scout pass (n_scout_blocks > 0): d_scout_prefix[n_groups+1] gives each group
- * n_lc_tiles*n_p_tiles workgroups that first reduce every scout_stride-th stage of the whole
- * group; every chunk then starts from those minima (they belong to real rows of the group, so
+ * n_lc_tiles*n_p_tiles*mist_reduce_scout_split() workgroups that first reduce every
+ * scout_stride-th stage of the whole group; every chunk then starts from those minima (they belong to real rows of the group, so
  * the result is unchanged) and lets far fewer rows through to the memory model.
  * d_partial_cost / d_partial_index: [n_blocks + n_scout_blocks][2*MIST_P_TILE+2][MIST_LC_TILE];
  * the first n_blocks slabs are the per-chunk results mist_finalize reads. */

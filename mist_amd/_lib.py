@@ -19,6 +19,7 @@ ROW_TERMS = 34
 LC_TILE = 64  # replaced by the library's own value in load()
 P_TILE = 32  # replaced by the library's own value in load()
 SLOTS = 2 * P_TILE + 2
+SCOUT_SPLIT = 4  # replaced by the library's own value in load()
 STAGE_ROWS = 64  # replaced by the library's own value in load()
 TERMS_BLOCK = 256
 MAX_MESH = 16
@@ -106,6 +107,7 @@ _SIGNATURES = {
     "mist_reduce_p_tile": (ctypes.c_int, []),
     "mist_reduce_stage_rows": (ctypes.c_int, []),
     "mist_reduce_lc_tile": (ctypes.c_int, []),
+    "mist_reduce_scout_split": (ctypes.c_int, []),
     "mist_row_terms": (ctypes.c_int, [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, _VP]),
     "mist_eval_reduce": (
         ctypes.c_int,
@@ -122,6 +124,17 @@ _SIGNATURES = {
          _VP, _VP, _VP, ctypes.c_double, ctypes.c_int, ctypes.c_int, ctypes.POINTER(OutTables), _VP],
     ),
 }
+
+
+def workspace_positions(n_par: int, n_pair: int, n_oo: int, n_ao: int) -> np.ndarray:
+    """Position in the row-term workspace of every reference row of a group (see
+    include/mist_search.h: the workspace is ordered (par, ao, oo, pair), the reference numbers
+    rows (par, pair, oo, ao))."""
+    n_off = n_pair * n_oo * n_ao
+    row = np.arange(n_par * n_off, dtype=np.int64)
+    par, off = row // n_off, row % n_off
+    pair, oo, ao = off // (n_oo * n_ao), (off // n_ao) % n_oo, off % n_ao
+    return par * n_off + (ao * n_oo + oo) * n_pair + pair
 
 
 def exported_symbols():
@@ -195,7 +208,8 @@ def load():
         raise MistLibraryError(
             f"MistGroupDesc layout mismatch: C {lib.mist_sizeof_group()} vs numpy {GROUP_DTYPE.itemsize}"
         )
-    global P_TILE, SLOTS, STAGE_ROWS, LC_TILE
+    global P_TILE, SLOTS, STAGE_ROWS, LC_TILE, SCOUT_SPLIT
+    SCOUT_SPLIT = lib.mist_reduce_scout_split()
     LC_TILE = lib.mist_reduce_lc_tile()
     STAGE_ROWS = lib.mist_reduce_stage_rows()
     P_TILE = lib.mist_reduce_p_tile()

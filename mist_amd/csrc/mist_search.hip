@@ -139,24 +139,57 @@ __device__ __forceinline__ const MistGroupDesc *find_group(const MistGroupDesc *
   return groups + lo;
 }
 
+// Workspace order.  The reference numbers a group's rows parallelism-major with the activation
+// offload ratio fastest (batched_module_analyzer.py:490-534); the workspace holds them as
+//   position = ((par * n_ao + ao) * n_oo + oo) * n_pair + pair,
+// i.e. rows that are consecutive in memory share the two ratios that move the memory footprint
+// most (activations, optimizer states).  A stage of the reduce kernel then covers rows of
+// similar footprint and one bound per stage prunes most of them.  Results carry row numbers.
+struct RowParts {
+  int par, pair, oo, ao;
+};
+
+__device__ __forceinline__ RowParts parts_of_position(const MistGroupDesc *g, int64_t pos) {
+  RowParts r;
+  r.par = (int)(pos / g->n_off);
+  int rem = (int)(pos % g->n_off);
+  const int per_ao = g->n_oo * g->n_pair;
+  r.ao = rem / per_ao;
+  rem -= r.ao * per_ao;
+  r.oo = rem / g->n_pair;
+  r.pair = rem - r.oo * g->n_pair;
+  return r;
+}
+
+__device__ __forceinline__ int32_t row_of_position(const MistGroupDesc *g, int64_t pos) {
+  const RowParts r = parts_of_position(g, pos);
+  return (int32_t)((int64_t)r.par * g->n_off + (r.pair * g->n_oo + r.oo) * g->n_ao + r.ao);
+}
+
+__device__ __forceinline__ int64_t position_of_row(const MistGroupDesc *g, int64_t row) {
+  const int par = (int)(row / g->n_off);
+  const int off = (int)(row % g->n_off);
+  const int n_tail = g->n_oo * g->n_ao;
+  const int pair = off / n_tail;
+  const int oo = (off / g->n_ao) % g->n_oo;
+  const int ao = off % g->n_ao;
+  return (int64_t)par * g->n_off + ((int64_t)(ao * g->n_oo + oo)) * g->n_pair + pair;
+}
+
 // ------------------------------------------------------------------------------------------
-// Kernel 1: row-invariant terms.  One thread per candidate row.
+// Kernel 1: row-invariant terms.  One thread per candidate row (workspace position).
 // ------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(kTermsBlock) void row_terms_kernel(
     const MistProblem prob, const MistGroupDesc *__restrict__ groups, int n_groups,
     const int32_t *__restrict__ block_prefix, double *__restrict__ row_terms) {
   int local_block;
   const MistGroupDesc *g = find_group(groups, block_prefix, n_groups, blockIdx.x, &local_block);
-  const int64_t row = (int64_t)local_block * kTermsBlock + threadIdx.x;
+  const int64_t row = (int64_t)local_block * kTermsBlock + threadIdx.x;  // workspace position
   if (row >= g->n_rows) return;
 
   // ---- index decomposition (batched_module_analyzer.py:490-534) ----
-  const int par_i = (int)(row / g->n_off);
-  const int off = (int)(row % g->n_off);
-  const int n_tail = g->n_oo * g->n_ao;
-  const int pair = off / n_tail;
-  const int oo_i = (off / g->n_ao) % g->n_oo;
-  const int ao_i = off % g->n_ao;
+  const RowParts parts = parts_of_position(g, row);
+  const int par_i = parts.par, pair = parts.pair, oo_i = parts.oo, ao_i = parts.ao;
   const double wo = g->wo[g->pair_wo[pair]];
   const double go = g->go[g->pair_go[pair]];
   const double oo = g->oo[oo_i];
@@ -453,9 +486,63 @@ __device__ __forceinline__ void take_min(double &best, int32_t &best_row, bool f
 #define MIST_REDUCE_MIN_WAVES 2
 #endif
 constexpr int kRowUnroll = MIST_ROW_UNROLL;  // rows whose objective values are computed together (ILP)
+constexpr int kScoutSplit = 4;  // scout workgroups per (group, (l, c) tile, p tile)
+constexpr int kPairFields = 4;  // per-pair table of sieve A: thr_b, thr_o, n_ck, n_nock
 constexpr int kLdsRowStride = MIST_ROW_TERMS + 1;  // odd number of doubles: lanes reading the
                                                    // same term of different rows hit different banks
 static_assert(kStageRows == 64, "the sieve masks are 64-bit");
+static_assert(MIST_ROW_TERMS % 2 == 0, "rows are staged as 16-byte pairs");
+static_assert(MIST_LC_TILE == 64, "one wavefront per workgroup: the stage minima use wave shuffles");
+static_assert(MIST_T_GCB - MIST_T_FWD_STATES0 == 15, "memory terms must be 16 consecutive columns");
+
+struct LaneMemory {
+  double fwd_states, bwd_states, cur_saved, mod_saved, ck_delta, fwd_pk, bwd_pk, out, gcb;
+  double mf_base, mf_pp;
+
+  // Peaks of the middle-stage variant for p pre-saved micro-batches (:2755-2786).
+  __device__ __forceinline__ void peaks(int p, double &peak_f, double &peak_b) const {
+    const double pf64 = (double)p;
+    const double pipe_saved = pf64 * mod_saved + cur_saved;
+    const double outp2 = out * pf64 * 2.0;
+    const double out2 = out * 2.0;
+    peak_f = fwd_states + pipe_saved + ck_delta + fwd_pk + outp2 + gcb;
+    peak_b = bwd_states + pipe_saved + ck_delta + bwd_pk + outp2 + out2 + gcb;
+  }
+  // Left-hand sides of the reference's memory tests; a candidate is feasible iff <= capacity.
+  __device__ __forceinline__ double scaled_base(int p) const {  // (:2805-2812)
+    double pf, pb;
+    peaks(p, pf, pb);
+    return fmax(pf, pb) * mf_base;
+  }
+  __device__ __forceinline__ double scaled_pre(int p, double pre_saved,
+                                               double pre_sas) const {  // (:2866-2875, 2893-2897)
+    double pf, pb;
+    peaks(p, pf, pb);
+    const double pre_p = (double)p * pre_saved;
+    return fmax(pre_p + pf + pre_sas, pre_p + pb + pre_sas) * mf_pp;
+  }
+  __device__ __forceinline__ bool feasible_base(int p, double cap) const {
+    return scaled_base(p) <= cap;
+  }
+  __device__ __forceinline__ bool feasible_pre(int p, double cap, double pre_saved,
+                                               double pre_sas) const {
+    return scaled_pre(p, pre_saved, pre_sas) <= cap;
+  }
+};
+
+// Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  Logical workgroups
+// that stream the same rows are consecutive, so runs of kXcdRun logical workgroups are given to
+// one XCD (and the runs round-robin, which keeps the XCDs evenly loaded).  The grid is padded to
+// a multiple of kNumXcd * kXcdRun; logical indices past the end do nothing.
+constexpr int kNumXcd = 8;
+constexpr int kXcdRun = 16;
+__device__ __forceinline__ int xcd_run_block(int physical) {
+  const int xcd = physical % kNumXcd, slot = physical / kNumXcd;
+  return ((slot / kXcdRun) * kNumXcd + xcd) * kXcdRun + slot % kXcdRun;
+}
+__host__ __device__ constexpr int xcd_padded_grid(int n_blocks) {
+  return (n_blocks + kNumXcd * kXcdRun - 1) / (kNumXcd * kXcdRun) * (kNumXcd * kXcdRun);
+}
 
 struct ReduceRange {
   int64_t row_begin, row_end;  // rows of the group this workgroup covers (multiples of kStageRows)
@@ -467,7 +554,8 @@ template <bool kPow2G, bool kFirstTile>
 __device__ __forceinline__ void reduce_block(
     const MistProblem &prob, const MistGroupDesc *__restrict__ g, const ReduceRange range,
     int p_tile, int lc_tile, const double *__restrict__ row_terms, double ratio,
-    double *lds_terms, const double *__restrict__ seed_cost,
+    double *lds_terms, double *lds_min, double *lds_pair, int *lds_pair_lane,
+    const double *__restrict__ seed_cost,
     const int32_t *__restrict__ seed_index, double *__restrict__ out_cost,
     int32_t *__restrict__ out_index) {
   const int L = prob.num_layers;
@@ -481,11 +569,13 @@ __device__ __forceinline__ void reduce_block(
   const int n_tile_full = min(MIST_P_TILE, g->num_p - p0);  // p values of this tile
   // Cells with c == l - 1 are only kept for p == 0 of the base / with_pre variants
   // (batched_module_analyzer.py:3021-3023, 3103), so such a lane has at most one slot.
-  const int n_tile = c == l - 1 ? (kFirstTile ? min(n_tile_full, 1) : 0) : n_tile_full;
+  // Lanes past the last pair of the tile keep no slots; they still hold rows in sieve A.
+  const int n_tile =
+      !active ? 0 : (c == l - 1 ? (kFirstTile ? min(n_tile_full, 1) : 0) : n_tile_full);
   int steps = 0;  // bisection steps that separate the n_tile + 1 possible counts
   while ((1 << steps) < n_tile + 1) ++steps;
-  const bool do_post = kFirstTile && c != l - 1;
-  const bool do_nopp = kFirstTile && l == L && c != l - 1;
+  const bool do_post = kFirstTile && active && c != l - 1;
+  const bool do_nopp = kFirstTile && active && l == L && c != l - 1;
   const GroupConsts k = group_consts(g);
   const double cap = prob.mem_cap_mb;
   const double G64 = (double)g->grad_accum;
@@ -511,22 +601,43 @@ __device__ __forceinline__ void reduce_block(
     row_b[j] = row_p[j] = -1;
   }
   if (seed_cost != nullptr && active) {
+    const int64_t slab = (int64_t)kSlots * MIST_LC_TILE;
+    for (int k = 0; k < kScoutSplit; ++k) {
+      const double *sc = seed_cost + k * slab + threadIdx.x;
+      const int32_t *si = seed_index + k * slab + threadIdx.x;
+#pragma unroll
+      for (int j = 0; j < MIST_P_TILE; ++j) {
+        const int32_t rb = si[j * MIST_LC_TILE], rp = si[(MIST_P_TILE + j) * MIST_LC_TILE];
+        take_min(best_b[j], row_b[j], rb >= 0, sc[j * MIST_LC_TILE], rb);
+        take_min(best_p[j], row_p[j], rp >= 0, sc[(MIST_P_TILE + j) * MIST_LC_TILE], rp);
+      }
+      const int32_t r2 = si[(2 * MIST_P_TILE) * MIST_LC_TILE];
+      const int32_t r3 = si[(2 * MIST_P_TILE + 1) * MIST_LC_TILE];
+      take_min(best_post, row_post, r2 >= 0, sc[(2 * MIST_P_TILE) * MIST_LC_TILE], r2);
+      take_min(best_pp, row_pp, r3 >= 0, sc[(2 * MIST_P_TILE + 1) * MIST_LC_TILE], r3);
+    }
 #pragma unroll
     for (int j = 0; j < MIST_P_TILE; ++j) {
-      best_b[j] = seed_cost[j * MIST_LC_TILE + threadIdx.x];
-      row_b[j] = seed_index[j * MIST_LC_TILE + threadIdx.x];
-      best_p[j] = seed_cost[(MIST_P_TILE + j) * MIST_LC_TILE + threadIdx.x];
-      row_p[j] = seed_index[(MIST_P_TILE + j) * MIST_LC_TILE + threadIdx.x];
       if (row_b[j] >= 0) { fin_b = j + 1; top_b = best_b[j]; }
       if (row_p[j] >= 0) { fin_p = j + 1; top_p = best_p[j]; }
     }
-    best_post = seed_cost[(2 * MIST_P_TILE) * MIST_LC_TILE + threadIdx.x];
-    row_post = seed_index[(2 * MIST_P_TILE) * MIST_LC_TILE + threadIdx.x];
-    best_pp = seed_cost[(2 * MIST_P_TILE + 1) * MIST_LC_TILE + threadIdx.x];
-    row_pp = seed_index[(2 * MIST_P_TILE + 1) * MIST_LC_TILE + threadIdx.x];
   }
 
   const double *__restrict__ src = row_terms + g->row_offset * MIST_ROW_TERMS;
+
+  // Sieve A visits the tile's pairs class by class (which first / last family member the
+  // latency uses is fixed per class): 0 = 0 < c < l, 1 = c == 0, 2 = c == l.  Each lane gets a
+  // slot of the per-pair table in that order.
+  const int pair_class = !active ? 3 : (c == 0 ? 1 : (c == l ? 2 : 0));
+  const uint64_t lanes_below = (1ull << threadIdx.x) - 1ull;
+  const uint64_t in_class0 = __ballot(pair_class == 0), in_class1 = __ballot(pair_class == 1);
+  const uint64_t in_class2 = __ballot(pair_class == 2);
+  const int n_class0 = __popcll(in_class0), n_class1 = __popcll(in_class1);
+  const int n_class2 = __popcll(in_class2);
+  const int pair_slot =
+      pair_class == 0 ? __popcll(in_class0 & lanes_below)
+      : pair_class == 1 ? n_class0 + __popcll(in_class1 & lanes_below)
+                        : n_class0 + n_class1 + __popcll(in_class2 & lanes_below);
 
   const double lf = (double)l, lm1 = (double)max(l - 1, 0), cf = (double)c;
   const double l_minus_c = (double)(l - c), l_minus_c_1 = (double)(l - c - 1);
@@ -539,7 +650,63 @@ __device__ __forceinline__ void reduce_block(
   const double n_nock = (double)(lm2 - min(max(c - 1, 0), lm2));
   const int first_col = c_eq_l ? 0 : 1, last_col = c_eq_0 ? 1 : 0;  // *_CK precedes *_NOCK
   const int post_col = c > 0 ? 0 : 1;
+  if (active) {
+    lds_pair[pair_slot * kPairFields + 2] = n_ck;
+    lds_pair[pair_slot * kPairFields + 3] = n_nock;
+    lds_pair_lane[pair_slot] = (int)threadIdx.x;
+  }
   auto div_G = [&](double v) { return kPow2G ? v * inv_G64 : v / G64; };
+
+  // Memory model of one candidate row for this lane's (l, c) (:2150-2162, 2358-2385, 2755-2786).
+  // `t` may also be the term-wise minimum of a stage: every operation below is monotone in
+  // every term, so the peaks of that pseudo row bound the peaks of each row of the stage from
+  // below.
+  auto lane_memory = [&](const double *__restrict__ t) {
+    LaneMemory mem;
+    const double S_ck = t[MIST_T_S_CK], S_nock = t[MIST_T_S_NOCK];
+    mem.fwd_states = t[MIST_T_FWD_STATES0] + lf * t[MIST_T_PWG] + lm1 * t[MIST_T_PO];
+    mem.bwd_states = t[MIST_T_BWD_STATES0] + lf * t[MIST_T_PWGO];
+    mem.cur_saved = c_eq_l ? (lf - 1.0) * S_ck : cf * S_ck + l_minus_c_1 * S_nock;
+    mem.mod_saved = S_ck * cf + S_nock * l_minus_c;
+    mem.ck_delta = c_ge_lm1 ? t[MIST_T_D_CK] : t[MIST_T_D_NOCK];
+    mem.fwd_pk = t[MIST_T_FWD_PEAK];
+    mem.bwd_pk = t[MIST_T_BWD_PEAK];
+    mem.out = t[MIST_T_OUT];
+    mem.gcb = t[MIST_T_GCB];
+    mem.mf_base = t[MIST_T_MF_BASE];
+    mem.mf_pp = t[MIST_T_MF_PP];
+    return mem;
+  };
+  // Number of feasible p of this tile, in [lo, n_tile], by bisection with the exact test.
+  auto feasible_count = [&](auto feasible, int lo) {
+    int hi = n_tile;
+    for (int it = 0; it < steps; ++it) {
+      const int mid = (lo + hi) >> 1;
+      const bool ok = feasible(p0 + mid);
+      const bool open = lo < hi;
+      lo = (open && ok) ? mid + 1 : lo;
+      hi = (open && !ok) ? mid : hi;
+    }
+    return lo;
+  };
+
+  // Upper bound of that number for the pseudo row of a stage.  The peaks are linear in p up to
+  // rounding, so the first infeasible slot is estimated from the values at the first two slots
+  // and confirmed with the exact test: any slot at which the pseudo row is infeasible bounds the
+  // count (monotonicity); an unconfirmed estimate falls back to the whole tile.
+  auto count_bound = [&](auto scaled) {
+    const double m0 = scaled(p0);
+    if (!(m0 <= cap)) return 0;
+    if (n_tile <= 1) return n_tile;
+    const float slope = (float)(scaled(p0 + 1) - m0);
+    if (!(slope > 0.0f)) return n_tile;
+    const float est = fminf((float)(cap - m0) * __frcp_rn(slope), (float)n_tile);
+    const int guess = (int)est + 1;  // slots 0 .. floor(est) are expected to be feasible
+    if (guess >= n_tile) return n_tile;
+    if (!(scaled(p0 + guess) <= cap)) return guess;
+    if (guess + 1 < n_tile && !(scaled(p0 + guess + 1) <= cap)) return guess + 1;
+    return n_tile;
+  };
 
   // Stable / delta latency rounded to float32 (:2212-2213), the base objective r * x + y in
   // float64 (pareto.py:138; y = float32 array / python int, :2815) and a lower bound of the three
@@ -562,7 +729,7 @@ __device__ __forceinline__ void reduce_block(
 
   // Sieves B (kCommit == false: would the row change anything, judged against the current
   // minima) and C (kCommit == true: apply it).  Returns whether the row survives / changed a slot.
-  auto examine = [&](const double *__restrict__ t, int32_t row, auto commit_tag) -> bool {
+  auto examine = [&](const double *__restrict__ t, int64_t pos, auto commit_tag) -> bool {
     constexpr bool kCommit = decltype(commit_tag)::value;
     double x, d, cost_base, bound;
     objective(t, x, d, cost_base, bound);
@@ -604,37 +771,9 @@ __device__ __forceinline__ void reduce_block(
     bool need_pp = want_pp && cost_pp <= best_pp;
     if (!(need_b || need_p || need_post || need_pp)) return false;
 
-    // ---- memory that does not depend on p (:2150-2162, 2358-2385, 2760-2769) ----
-    const double S_ck = t[MIST_T_S_CK], S_nock = t[MIST_T_S_NOCK];
-    const double fwd_states = t[MIST_T_FWD_STATES0] + lf * t[MIST_T_PWG] + lm1 * t[MIST_T_PO];
-    const double bwd_states = t[MIST_T_BWD_STATES0] + lf * t[MIST_T_PWGO];
-    const double cur_saved = c_eq_l ? (lf - 1.0) * S_ck : cf * S_ck + l_minus_c_1 * S_nock;
-    const double mod_saved = S_ck * cf + S_nock * l_minus_c;
-    const double ck_delta = c_ge_lm1 ? t[MIST_T_D_CK] : t[MIST_T_D_NOCK];
-    const double fwd_pk = t[MIST_T_FWD_PEAK], bwd_pk = t[MIST_T_BWD_PEAK];
-    const double out = t[MIST_T_OUT], gcb = t[MIST_T_GCB];
-    const double out2 = out * 2.0;
-    const double mf_base = t[MIST_T_MF_BASE], mf_pp = t[MIST_T_MF_PP];
-
-    // Peaks of the middle-stage variant for p pre-saved micro-batches (:2755-2786).
-    auto peaks = [&](int p, double &peak_f, double &peak_b) {
-      const double pf64 = (double)p;
-      const double pipe_saved = pf64 * mod_saved + cur_saved;
-      const double outp2 = out * pf64 * 2.0;
-      peak_f = fwd_states + pipe_saved + ck_delta + fwd_pk + outp2 + gcb;
-      peak_b = bwd_states + pipe_saved + ck_delta + bwd_pk + outp2 + out2 + gcb;
-    };
-    auto feasible_base = [&](int p) {  // (:2805-2812)
-      double pf, pb;
-      peaks(p, pf, pb);
-      return fmax(pf, pb) * mf_base <= cap;
-    };
-    auto feasible_pre = [&](int p) {  // (:2866-2875, 2893-2897)
-      double pf, pb;
-      peaks(p, pf, pb);
-      const double pre_p = (double)p * pre_saved;
-      return fmax(pre_p + pf + pre_sas, pre_p + pb + pre_sas) * mf_pp <= cap;
-    };
+    const LaneMemory mem = lane_memory(t);
+    auto feasible_base = [&](int p) { return mem.feasible_base(p, cap); };
+    auto feasible_pre = [&](int p) { return mem.feasible_pre(p, cap, pre_saved, pre_sas); };
 
     need_b = need_b && feasible_base(p0 + lo_b);
     need_p = need_p && feasible_pre(p0 + lo_p);
@@ -642,13 +781,13 @@ __device__ __forceinline__ void reduce_block(
     if (need_post || need_pp) {
       // ---- last stage / single stage, p == 0 only (:2946-3106) ----
       double peak_f, peak_b;
-      peaks(0, peak_f, peak_b);
-      const double f_in = fwd_states + post_states + mod_saved + post_fwd_peak + gcb;
-      const double b_in = bwd_states + post_states + mod_saved + post_bwd_peak +
-                          (c_eq_0 ? t[MIST_T_RD] : 0.0) + gcb;
+      mem.peaks(0, peak_f, peak_b);
+      const double f_in = mem.fwd_states + post_states + mem.mod_saved + post_fwd_peak + mem.gcb;
+      const double b_in = mem.bwd_states + post_states + mem.mod_saved + post_bwd_peak +
+                          (c_eq_0 ? t[MIST_T_RD] : 0.0) + mem.gcb;
       const double pf_post = fmax(f_in, peak_f + post_states);
-      const double pb_post = fmax(b_in, peak_b - out + post_states) + post_output;
-      const bool ok_post = fmax(pf_post, pb_post) * mf_pp <= cap;
+      const double pb_post = fmax(b_in, peak_b - mem.out + post_states) + post_output;
+      const bool ok_post = fmax(pf_post, pb_post) * mem.mf_pp <= cap;
       if (need_pp) {
         const double pf_pp = pf_post + pre_states + pre_saved;
         const double pb_pp = pb_post + pre_states + pre_saved;
@@ -659,17 +798,11 @@ __device__ __forceinline__ void reduce_block(
     }
     if (!kCommit) return need_b || need_p || need_post || need_pp;
 
+    const int32_t row = row_of_position(g, pos);
     bool changed = false;
     if (need_b) {
       const double cost = cost_base;
-      int lo = lo_b + 1, hi = n_tile;  // number of feasible p of this tile lies in [lo, hi]
-      for (int it = 0; it < steps; ++it) {
-        const int mid = (lo + hi) >> 1;
-        const bool ok = feasible_base(p0 + mid);
-        const bool open = lo < hi;
-        lo = (open && ok) ? mid + 1 : lo;
-        hi = (open && !ok) ? mid : hi;
-      }
+      const int lo = feasible_count(feasible_base, lo_b + 1);  // slot lo_b is known feasible
 #pragma unroll
       for (int j = 0; j < MIST_P_TILE; ++j) {
         const bool better = j >= lo_b && j < lo && lex_less(cost, row, best_b[j], row_b[j]);
@@ -683,14 +816,7 @@ __device__ __forceinline__ void reduce_block(
     }
     if (need_p) {
       const double cost = cost_pre;
-      int lo = lo_p + 1, hi = n_tile;
-      for (int it = 0; it < steps; ++it) {
-        const int mid = (lo + hi) >> 1;
-        const bool ok = feasible_pre(p0 + mid);
-        const bool open = lo < hi;
-        lo = (open && ok) ? mid + 1 : lo;
-        hi = (open && !ok) ? mid : hi;
-      }
+      const int lo = feasible_count(feasible_pre, lo_p + 1);
 #pragma unroll
       for (int j = 0; j < MIST_P_TILE; ++j) {
         const bool better = j >= lo_p && j < lo && lex_less(cost, row, best_p[j], row_p[j]);
@@ -719,37 +845,125 @@ __device__ __forceinline__ void reduce_block(
     const int64_t base = stage * kStageRows;
     const int n_stage = (int)min((int64_t)kStageRows, range.row_end - base);
     __syncthreads();
-    for (int i = threadIdx.x; i < n_stage * MIST_ROW_TERMS; i += MIST_LC_TILE)
-      lds_terms[(i / MIST_ROW_TERMS) * kLdsRowStride + i % MIST_ROW_TERMS] =
-          src[base * MIST_ROW_TERMS + i];
-    __syncthreads();
-    if (!active) continue;
-
-    // ---- sieve A: all rows of the stage against the largest minima ----
-    const double thr_b = fin_b < n_tile ? INFINITY : top_b;
-    double thr_o = fin_p < n_tile ? INFINITY : top_p;
-    if (do_post) thr_o = fmax(thr_o, best_post);
-    if (do_nopp) thr_o = fmax(thr_o, best_pp);
-    uint64_t sieve = 0;
-    for (int r0 = 0; r0 < kStageRows; r0 += kRowUnroll) {
-#pragma unroll
-      for (int u = 0; u < kRowUnroll; ++u) {
-        double x, d, cost_base, bound;
-        objective(lds_terms + (r0 + u) * kLdsRowStride, x, d, cost_base, bound);
-        const bool pass = cost_base <= thr_b || bound <= thr_o;
-        sieve |= (uint64_t)(pass ? 1 : 0) << (r0 + u);
+    {  // 16-byte loads: a row is 17 such pairs and starts 16-byte aligned
+      const double2 *__restrict__ src2 =
+          reinterpret_cast<const double2 *>(src + base * MIST_ROW_TERMS);
+      for (int i = threadIdx.x; i < n_stage * (MIST_ROW_TERMS / 2); i += MIST_LC_TILE) {
+        const double2 v = src2[i];
+        const int at = (i / (MIST_ROW_TERMS / 2)) * kLdsRowStride + 2 * (i % (MIST_ROW_TERMS / 2));
+        lds_terms[at] = v.x;
+        lds_terms[at + 1] = v.y;
       }
     }
-    // Rows past the end of the stage hold stale LDS contents.
-    if (n_stage < kStageRows) sieve &= (1ull << n_stage) - 1ull;
+    __syncthreads();
+    // Term-wise minimum of the stage's memory terms (MIST_T_FWD_STATES0 .. MIST_T_GCB), plus the
+    // maximum of the one term the last-stage peak subtracts: lane = (term, quarter of the rows).
+    {
+      const int term = threadIdx.x & 15, quarter = threadIdx.x >> 4;
+      double lo_v = INFINITY, hi_v = 0.0;
+      for (int r = quarter * (kStageRows / 4); r < (quarter + 1) * (kStageRows / 4); ++r) {
+        if (r < n_stage) {
+          const double v = lds_terms[r * kLdsRowStride + MIST_T_FWD_STATES0 + term];
+          lo_v = fmin(lo_v, v);
+          hi_v = fmax(hi_v, v);
+        }
+      }
+      lo_v = fmin(lo_v, __shfl_xor(lo_v, 16));
+      lo_v = fmin(lo_v, __shfl_xor(lo_v, 32));
+      hi_v = fmax(hi_v, __shfl_xor(hi_v, 16));
+      hi_v = fmax(hi_v, __shfl_xor(hi_v, 32));
+      if (threadIdx.x < 16) lds_min[threadIdx.x] = lo_v;
+      if (threadIdx.x == MIST_T_OUT - MIST_T_FWD_STATES0) lds_min[16] = hi_v;
+    }
+    __syncthreads();
+
+    // ---- per-stage thresholds: no row of the stage is feasible beyond the pseudo row's count,
+    // so only the minima of the slots below it can be beaten ----
+    const LaneMemory floor_mem = lane_memory(lds_min - MIST_T_FWD_STATES0);
+    const int cnt_b = count_bound([&](int p) { return floor_mem.scaled_base(p); });
+    const int cnt_p =
+        count_bound([&](int p) { return floor_mem.scaled_pre(p, pre_saved, pre_sas); });
+    double thr_b = -INFINITY, thr_o = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < MIST_P_TILE; ++j) {  // minima are non-decreasing; empty slots hold +inf
+      thr_b = j < cnt_b ? best_b[j] : thr_b;
+      thr_o = j < cnt_p ? best_p[j] : thr_o;
+    }
+    if (do_post) {
+      // Lower bounds of the last-stage / single-stage peaks (:2946-3106) from the pseudo row.
+      double peak_f, peak_b;
+      floor_mem.peaks(0, peak_f, peak_b);
+      const double f_in =
+          floor_mem.fwd_states + post_states + floor_mem.mod_saved + post_fwd_peak + floor_mem.gcb;
+      const double b_in =
+          floor_mem.bwd_states + post_states + floor_mem.mod_saved + post_bwd_peak + floor_mem.gcb;
+      const double pf_post = fmax(f_in, peak_f + post_states);
+      const double pb_post = fmax(b_in, peak_b - lds_min[16] + post_states) + post_output;
+      if (fmax(pf_post, pb_post) * floor_mem.mf_pp <= cap) thr_o = fmax(thr_o, best_post);
+      if (do_nopp) {
+        const double pf_pp = pf_post + pre_states + pre_saved;
+        const double pb_pp = pb_post + pre_states + pre_saved;
+        if (fmax(pf_pp, pb_pp) * lds_min[MIST_T_MF - MIST_T_FWD_STATES0] <= cap)
+          thr_o = fmax(thr_o, best_pp);
+      }
+    }
+
+    // ---- sieve A: all rows of the stage against those thresholds.  Transposed: a lane holds
+    // the latency terms of ONE ROW in registers and the loop runs over the tile's pairs, whose
+    // constants and thresholds are wave-uniform reads of the per-pair table.  The wave-wide
+    // comparison result is exactly the 64-row survivor mask of that pair; it is handed to the
+    // pair's lane. ----
+    if (active) {
+      lds_pair[pair_slot * kPairFields + 0] = thr_b;
+      lds_pair[pair_slot * kPairFields + 1] = thr_o;
+    }
+    double rt[MIST_T_D_LAST_NOCK + 1];
+#pragma unroll
+    for (int i = 0; i <= MIST_T_D_LAST_NOCK; ++i)
+      rt[i] = lds_terms[threadIdx.x * kLdsRowStride + i];  // stale beyond n_stage, masked below
+    __syncthreads();
+    const uint64_t valid_rows = n_stage < kStageRows ? (1ull << n_stage) - 1ull : ~0ull;
+    uint64_t sieve = 0;
+    auto sieve_class = [&](int k_begin, int k_end, auto first_col_tag, auto last_col_tag) {
+      constexpr int kFirstCol = decltype(first_col_tag)::value;
+      constexpr int kLastCol = decltype(last_col_tag)::value;
+      const double s_first = rt[MIST_T_S_FIRST_CK + kFirstCol];
+      const double s_last = rt[MIST_T_S_LAST_CK + kLastCol];
+      const double d_first = rt[MIST_T_D_FIRST_CK + kFirstCol];
+      const double d_last = rt[MIST_T_D_LAST_CK + kLastCol];
+#pragma unroll 2
+      for (int k = k_begin; k < k_end; ++k) {
+        const double pair_thr_b = lds_pair[k * kPairFields + 0];
+        const double pair_thr_o = lds_pair[k * kPairFields + 1];
+        const double pair_n_ck = lds_pair[k * kPairFields + 2];
+        const double pair_n_nock = lds_pair[k * kPairFields + 3];
+        const int pair_lane = lds_pair_lane[k];
+        const double stable = pair_n_ck * rt[MIST_T_S_LAYER_CK] +
+                              pair_n_nock * rt[MIST_T_S_LAYER_NOCK] + s_first + s_last;
+        const double delta = pair_n_ck * rt[MIST_T_D_LAYER_CK] +
+                             pair_n_nock * rt[MIST_T_D_LAYER_NOCK] + d_first + d_last;
+        const float x32 = (float)stable, d32 = (float)delta;
+        const float y32 = kPow2G ? d32 * inv_G32 : d32 / G32;
+        const double rx = ratio * (double)x32;
+        const double cost_base = rx + (double)y32;
+        const double bound = rx + div_G((double)d32);
+        const uint64_t survivors =
+            __ballot(cost_base <= pair_thr_b || bound <= pair_thr_o) & valid_rows;
+        sieve = (int)threadIdx.x == pair_lane ? survivors : sieve;
+      }
+    };
+    sieve_class(0, n_class0, std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{});
+    sieve_class(n_class0, n_class0 + n_class1, std::integral_constant<int, 1>{},
+                std::integral_constant<int, 1>{});
+    sieve_class(n_class0 + n_class1, n_class0 + n_class1 + n_class2,
+                std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{});
 
     // ---- sieve B: lowest improvable slot and the memory test there, per-lane survivors ----
     uint64_t keep = 0;
     while (sieve != 0) {
       const int r = __ffsll((unsigned long long)sieve) - 1;
       sieve &= sieve - 1;
-      const bool hit = examine(lds_terms + r * kLdsRowStride, (int32_t)(base + r),
-                               std::false_type{});
+      const bool hit = examine(lds_terms + r * kLdsRowStride, base + r, std::false_type{});
       keep |= (uint64_t)(hit ? 1 : 0) << r;
     }
 
@@ -757,7 +971,7 @@ __device__ __forceinline__ void reduce_block(
     while (keep != 0) {
       const int r = __ffsll((unsigned long long)keep) - 1;
       keep &= keep - 1;
-      examine(lds_terms + r * kLdsRowStride, (int32_t)(base + r), std::true_type{});
+      examine(lds_terms + r * kLdsRowStride, base + r, std::true_type{});
     }
   }
 
@@ -774,8 +988,8 @@ __device__ __forceinline__ void reduce_block(
   out_index[(2 * MIST_P_TILE + 1) * MIST_LC_TILE + threadIdx.x] = row_pp;
 }
 
-// scout != 0: one workgroup per (group, (l, c) tile, p tile) over every scout_stride-th stage of
-// the whole group, results in slab n_blocks + blockIdx.x.  scout == 0: one workgroup per row
+// scout != 0: kScoutSplit workgroups per (group, (l, c) tile, p tile) share every
+// scout_stride-th stage of the whole group, results in slab n_blocks + blockIdx.x.  scout == 0: one workgroup per row
 // chunk of such a tile, seeded from the scout's slab when the group has one.
 __global__ __launch_bounds__(MIST_LC_TILE, MIST_REDUCE_MIN_WAVES) void eval_reduce_kernel(
     const MistProblem prob, const MistGroupDesc *__restrict__ groups, int n_groups,
@@ -783,9 +997,14 @@ __global__ __launch_bounds__(MIST_LC_TILE, MIST_REDUCE_MIN_WAVES) void eval_redu
     const int32_t *__restrict__ scout_prefix, int scout, const double *__restrict__ row_terms,
     double ratio, double *__restrict__ partial_cost, int32_t *__restrict__ partial_index) {
   __shared__ double lds_terms[kStageRows * kLdsRowStride];
+  __shared__ double lds_min[17];
+  __shared__ double lds_pair[MIST_LC_TILE * kPairFields];
+  __shared__ int lds_pair_lane[MIST_LC_TILE];
+  const int block = xcd_run_block(blockIdx.x);
+  if (block >= (scout ? scout_prefix[n_groups] : n_blocks)) return;
   int local_block;
   const MistGroupDesc *g = find_group(groups, scout ? scout_prefix : block_prefix, n_groups,
-                                      blockIdx.x, &local_block);
+                                      block, &local_block);
   const int gi = (int)(g - groups);
   const bool seeded = scout_prefix != nullptr && g->scout_stride > 0;
   int tile;
@@ -793,27 +1012,32 @@ __global__ __launch_bounds__(MIST_LC_TILE, MIST_REDUCE_MIN_WAVES) void eval_redu
   int64_t out_slab;
   if (scout) {
     if (g->scout_stride <= 0) return;
-    tile = local_block;
-    range = ReduceRange{0, g->n_rows, g->scout_stride, 0};
-    out_slab = (int64_t)n_blocks + blockIdx.x;
+    tile = local_block / kScoutSplit;
+    const int part = local_block % kScoutSplit;  // sampled stages part, part + split, ...
+    range = ReduceRange{(int64_t)part * g->scout_stride * kStageRows, g->n_rows,
+                        g->scout_stride * kScoutSplit, 0};
+    out_slab = (int64_t)n_blocks + block;
   } else {
-    const int chunk = local_block % g->n_chunks;
-    tile = local_block / g->n_chunks;
+    const int n_tiles = g->n_lc_tiles * g->n_p_tiles;
+    const int chunk = local_block / n_tiles;  // the tiles of one chunk are neighbours
+    tile = local_block % n_tiles;
     const int64_t row_begin = (int64_t)chunk * g->rows_per_chunk;
     range = ReduceRange{row_begin, min(row_begin + (int64_t)g->rows_per_chunk, g->n_rows), 1,
                         seeded ? g->scout_stride : 0};
-    out_slab = blockIdx.x;
+    out_slab = block;
   }
   const int p_tile = tile % g->n_p_tiles;
   const int lc_tile = tile / g->n_p_tiles;
   const int64_t slab = (int64_t)kSlots * MIST_LC_TILE;
-  const int64_t seed_slab = (int64_t)n_blocks + (seeded ? scout_prefix[gi] + tile : 0);
+  const int64_t seed_slab =
+      (int64_t)n_blocks + (seeded ? scout_prefix[gi] + tile * kScoutSplit : 0);
   const double *seed_cost = (!scout && seeded) ? partial_cost + seed_slab * slab : nullptr;
   const int32_t *seed_index = (!scout && seeded) ? partial_index + seed_slab * slab : nullptr;
   const bool pow2 = (g->grad_accum & (g->grad_accum - 1)) == 0;
 #define MIST_REDUCE(P2, FT)                                                                   \
-  reduce_block<P2, FT>(prob, g, range, p_tile, lc_tile, row_terms, ratio, lds_terms, seed_cost, \
-                       seed_index, partial_cost + out_slab * slab, partial_index + out_slab * slab)
+  reduce_block<P2, FT>(prob, g, range, p_tile, lc_tile, row_terms, ratio, lds_terms, lds_min,  \
+                       lds_pair, lds_pair_lane, seed_cost, seed_index,                        \
+                       partial_cost + out_slab * slab, partial_index + out_slab * slab)
   if (pow2) {
     if (p_tile == 0) MIST_REDUCE(true, true); else MIST_REDUCE(true, false);
   } else {
@@ -859,12 +1083,13 @@ __global__ __launch_bounds__(256) void finalize_kernel(
   if (variant == 0) kslot = p % MIST_P_TILE;
   else if (variant == 1) kslot = MIST_P_TILE + p % MIST_P_TILE;
   else kslot = 2 * MIST_P_TILE + (variant - 2);
-  const int64_t first_block =
-      (int64_t)block_prefix[gi] + (int64_t)(lc_tile * g->n_p_tiles + p_tile) * g->n_chunks;
+  const int n_tiles = g->n_lc_tiles * g->n_p_tiles;
+  const int64_t first_block = (int64_t)block_prefix[gi] + (lc_tile * g->n_p_tiles + p_tile);
   double best = INFINITY;
   int32_t best_row = -1;
   for (int ch = 0; ch < g->n_chunks; ++ch) {
-    const int64_t at = ((first_block + ch) * kSlots + kslot) * MIST_LC_TILE + lane;
+    const int64_t at =
+        ((first_block + (int64_t)ch * n_tiles) * kSlots + kslot) * MIST_LC_TILE + lane;
     const double cost = partial_cost[at];
     const int32_t row = partial_index[at];
     take_min(best, best_row, row >= 0, cost, row);
@@ -872,7 +1097,7 @@ __global__ __launch_bounds__(256) void finalize_kernel(
 
   double stable = INFINITY, delta = INFINITY;
   if (best_row >= 0) {
-    const double *t = row_terms + (g->row_offset + best_row) * MIST_ROW_TERMS;
+    const double *t = row_terms + (g->row_offset + position_of_row(g, best_row)) * MIST_ROW_TERMS;
     const CellLatency lat = cell_latency<true>(t, l, c, group_consts(g));
     if (variant == 0) { stable = (double)lat.x; delta = (double)lat.d; }
     else if (variant == 1) { stable = lat.sp; delta = lat.dpre; }
@@ -921,6 +1146,7 @@ int mist_row_terms(const MistProblem *problem, const MistGroupDesc *d_groups, in
 
 int mist_reduce_stage_rows(void) { return kStageRows; }
 int mist_reduce_lc_tile(void) { return MIST_LC_TILE; }
+int mist_reduce_scout_split(void) { return kScoutSplit; }
 
 int mist_eval_reduce(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,
                      const int32_t *d_block_prefix, int n_blocks,
@@ -937,13 +1163,13 @@ int mist_eval_reduce(const MistProblem *problem, const MistGroupDesc *d_groups, 
                 n_scout_blocks);
   const int32_t *scout_prefix = n_scout_blocks > 0 ? d_scout_prefix : nullptr;
   if (scout_prefix) {
-    hipLaunchKernelGGL(eval_reduce_kernel, dim3(n_scout_blocks), dim3(MIST_LC_TILE), 0,
+    hipLaunchKernelGGL(eval_reduce_kernel, dim3(xcd_padded_grid(n_scout_blocks)), dim3(MIST_LC_TILE), 0,
                        (hipStream_t)stream, *problem, d_groups, n_groups, d_block_prefix,
                        n_blocks, scout_prefix, 1, d_row_terms, ratio, d_partial_cost,
                        d_partial_index);
     MIST_HIP_CHECK(hipGetLastError());
   }
-  hipLaunchKernelGGL(eval_reduce_kernel, dim3(n_blocks), dim3(MIST_LC_TILE), 0,
+  hipLaunchKernelGGL(eval_reduce_kernel, dim3(xcd_padded_grid(n_blocks)), dim3(MIST_LC_TILE), 0,
                      (hipStream_t)stream, *problem, d_groups, n_groups, d_block_prefix, n_blocks,
                      scout_prefix, 0, d_row_terms, ratio, d_partial_cost, d_partial_index);
   MIST_HIP_CHECK(hipGetLastError());

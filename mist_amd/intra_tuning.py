@@ -218,7 +218,7 @@ class IntraStageTuner:
             n_stages = -(-groups["n_rows"] // _lib.STAGE_ROWS)
             stride = n_stages // SCOUT_STAGES if SCOUT_STAGES > 0 else np.zeros_like(n_stages)
             groups["scout_stride"] = np.where(stride >= MIN_SCOUT_STRIDE, stride, 0)
-            scout_blocks = np.full(len(pending), n_lc_tiles, dtype=np.int64) * n_p_tiles
+            scout_blocks = np.full(len(pending), n_lc_tiles * _lib.SCOUT_SPLIT, dtype=np.int64) * n_p_tiles
             if not np.any(groups["scout_stride"] > 0):
                 scout_blocks[:] = 0
         else:

@@ -92,7 +92,8 @@ def test_row_terms_bit_exact():
             n = int(rec["n_rows"])
             assert dbg["rows"].shape[0] == n
             want = oracle_terms(dbg, n)
-            got = terms[int(rec["row_offset"]): int(rec["row_offset"]) + n]
+            pos = _lib.workspace_positions(*(int(rec[k]) for k in ("n_par", "n_pair", "n_oo", "n_ao")))
+            got = terms[int(rec["row_offset"]) + pos]
             for j, name in enumerate(_lib.TERM_NAMES):
                 assert_same_f64(got[:, j], want[:, j], f"tp={tp} G={rec['grad_accum']} term {name}")
 

@@ -86,25 +86,48 @@ class _DpRunner:
             self.costs_struct.g_stride[v] = self.cost[v][0].numel()
         self.launches = 0
         self.thresholds_run = 0
+        self._cand = None
+        self.fetches = 0
 
-    def thresholds(self) -> List[np.ndarray]:
-        """Per g: ascending unique finite stage costs (inter_tuning.py:180-186) after the gap
-        rule (:198), float32.  One device sort for all g, the sequential rule on the host."""
-        allv = torch.cat([self.cost[v].reshape(self.Gn, -1) for v in range(3)], dim=1)
-        n_fin = int(torch.isfinite(allv).sum(dim=1).max().item())
-        # +inf sorts last: only the finite prefix is copied to the host
-        host = torch.sort(allv, dim=1).values[:, :max(n_fin, 1)].contiguous().cpu().numpy()
-        out = []
-        kept = np.empty(host.shape[1], dtype=np.float32)
-        for g in range(self.Gn):
-            row = np.ascontiguousarray(host[g])
-            n_finite = int(np.searchsorted(row, np.inf, side="left"))
-            # duplicates have a zero difference to the last kept value and fall to the gap rule
-            n = self.lib.mist_dp_filter_tmax(
-                ctypes.c_void_p(row.ctypes.data), n_finite, GAP, ctypes.c_void_p(kept.ctypes.data)
-            )
-            out.append(kept[:n].copy())
+    def _all_candidates(self) -> torch.Tensor:
+        """[Gn, N] float32: every stage cost the reference collects as a t_max candidate
+        (costs, costs_with_pre, costs_with_post; inter_tuning.py:180-186)."""
+        if self._cand is None:
+            self._cand = torch.cat([self.cost[v].reshape(self.Gn, -1) for v in range(3)], dim=1)
+        return self._cand
+
+    def candidates_between(self, rows: np.ndarray, lo: np.ndarray, hi: np.ndarray):
+        """Per requested table row g: the ascending candidates v with lo < v <= hi (lo = -inf
+        includes everything below), and how many finite candidates lie above hi.  One pass on
+        the device over all requested rows, only the selected values come back."""
+        dev = self.device
+        self.fetches += 1
+        allv = self._all_candidates()
+        with torch.cuda.device(dev):
+            bounds = torch.from_numpy(np.stack([lo, hi]).astype(np.float32)).to(dev)
+            sel = allv if len(rows) == self.Gn and np.array_equal(rows, np.arange(self.Gn)) \
+                else allv[torch.from_numpy(rows.astype(np.int64)).to(dev)]
+            finite = torch.isfinite(sel)
+            inside = finite & (sel > bounds[0][:, None]) & (sel <= bounds[1][:, None])
+            above = (finite & (sel > bounds[1][:, None])).sum(dim=1)
+            counts = torch.stack([inside.sum(dim=1), above]).cpu().numpy()
+            values = sel[inside].cpu().numpy()
+        out, off = [], 0
+        for i in range(len(rows)):
+            n = int(counts[0, i])
+            out.append((np.sort(values[off:off + n]), int(counts[1, i])))
+            off += n
         return out
+
+    def filter_gap(self, ascending: np.ndarray) -> np.ndarray:
+        """The reference's gap rule (inter_tuning.py:198) applied from the first element on
+        (which is kept); duplicates have a zero difference to the last kept value."""
+        ascending = np.ascontiguousarray(ascending, dtype=np.float32)
+        kept = np.empty(len(ascending), dtype=np.float32)
+        n = self.lib.mist_dp_filter_tmax(
+            ctypes.c_void_p(ascending.ctypes.data), len(ascending), GAP,
+            ctypes.c_void_p(kept.ctypes.data))
+        return kept[:n]
 
     def run(self, g_index: np.ndarray, tmax: np.ndarray, mode: int = _lib.DP_THRESHOLD,
             want_argmin: bool = False):
@@ -139,15 +162,106 @@ class _DpRunner:
         return out
 
 
+def _gap_reached(a: np.ndarray, b: np.ndarray) -> np.ndarray:
+    """not (a - b < 1e-6) with the reference's arithmetic: float32 difference, float64 compare."""
+    return ~((a.astype(np.float32) - b.astype(np.float32)).astype(np.float64) < GAP)
+
+
+class _Window:
+    """Kept t_max candidates of one table row, materialised lazily.
+
+    The reference sorts every finite stage cost and walks the list with the gap rule from the
+    bottom (inter_tuning.py:180-198).  Whether a candidate is kept only depends on the last kept
+    one, and a candidate whose predecessor is at least the gap below is always kept, so the
+    walk can start at such a candidate just below the smallest feasible threshold instead of
+    at the bottom; everything below is infeasible and leaves the scan unchanged."""
+
+    def __init__(self, runner: "_DpRunner", row: int, G: int, start_value: float, start_sum: float):
+        self.runner, self.row, self.G, self.start_value = runner, row, G, np.float32(start_value)
+        # Sum of stage costs of the DP at the smallest feasible threshold.  At the first kept
+        # candidate t_s >= start_value that solution is still admissible, so the scan's running
+        # best is at most start_sum + (G - 1) * t_s once it has looked at t_s; candidates with
+        # t * G beyond that are never reached.
+        self.start_sum = float(start_sum)
+        self.bound = float("inf")
+        self.kept = np.empty(0, dtype=np.float32)
+        self.scaled = np.empty(0, dtype=np.float64)
+        self.hi = None          # every candidate <= hi has been walked
+        self.complete = False   # no finite candidate above hi
+
+    def lower_margin(self, widen: int) -> np.float32:
+        return np.float32(self.start_value - (1e-4 + 1e-5 * abs(float(self.start_value))) * 4.0 ** widen)
+
+    def begin(self, values: np.ndarray, n_above: int, lo: np.float32, hi: np.float32) -> bool:
+        """First fetch: ``values`` = ascending candidates in (lo, hi].  Returns False if no
+        certain start of the walk lies in the fetched part (the caller widens ``lo``)."""
+        self.hi, self.complete = hi, n_above == 0
+        if len(values) == 0:
+            return True
+        below = np.isneginf(lo)
+        prev = np.concatenate(([lo if not below else np.float32(0)], values[:-1]))
+        certain = _gap_reached(values, prev)   # kept whatever happened before
+        certain[0] = certain[0] or below        # the walk's true start
+        at_or_below = np.nonzero(certain & (values <= self.start_value))[0]
+        if len(at_or_below):
+            first = int(at_or_below[-1])
+        elif values[0] > self.start_value and certain[0]:
+            first = 0
+        else:
+            return False
+        self._append(self.runner.filter_gap(values[first:]))
+        return True
+
+    def _append(self, kept: np.ndarray) -> None:
+        self.kept = np.concatenate([self.kept, kept])
+        # float32 scalar * python int is float64 under the reference's numpy 1.24.
+        self.scaled = self.kept.astype(np.float64) * self.G
+        if not np.isfinite(self.bound):
+            i = int(np.searchsorted(self.kept, self.start_value, side="left"))
+            if i < len(self.kept):
+                self.bound = self.start_sum + (self.G - 1) * float(self.kept[i])
+
+    def covers(self, best_cost: float) -> bool:
+        """True if every kept candidate the scan can reach under the running best ``best_cost``
+        is materialised."""
+        need = min(best_cost, self.bound)
+        return self.complete or float(np.float64(self.hi) * self.G) >= need
+
+    def extension_target(self, best_cost: float) -> np.float32:
+        # at least a geometric step, so that repeated calls end (an unbounded best_cost, i.e. no
+        # solution yet, asks for "more" rather than for everything)
+        want = np.float32(self.hi + max(16 * (abs(self.hi) * 1e-4 + 1e-4),
+                                        2.0 * abs(float(self.hi) - float(self.start_value))))
+        need = min(best_cost, self.bound)
+        if np.isfinite(need):
+            want = max(want, np.nextafter(np.float32(need / self.G), np.float32(np.inf)))
+        return want
+
+    def apply_extension(self, values: np.ndarray, n_above: int, want: np.float32) -> None:
+        """``values`` = ascending candidates in (hi, want]."""
+        if len(self.kept):
+            # continue the walk from the last kept candidate: put it in front and drop it again
+            values = self.runner.filter_gap(np.concatenate((self.kept[-1:], values)))[1:]
+        else:
+            values = self.runner.filter_gap(values)
+        self.hi, self.complete = want, n_above == 0
+        self._append(values)
+
+    def extend(self, best_cost: float) -> None:
+        want = self.extension_target(best_cost)
+        (values, n_above), = self.runner.candidates_between(
+            np.array([self.row]), np.array([self.hi], dtype=np.float32),
+            np.array([want], dtype=np.float32))
+        self.apply_extension(values, n_above, want)
+
+
 class _Scan:
     """Replay state of ``inter_stage_tune_with_fixed_grad_accumu`` (inter_tuning.py:163-217) for
     one G: ``pos`` = next threshold the sequential scan would look at, ``results`` = DP outcomes
     already computed for tmax[lo : lo + len]."""
 
-    def __init__(self, G: int, tmax: np.ndarray, first: int):
-        self.G, self.tmax = G, tmax
-        # float32 scalar * python int is float64 under the reference's numpy 1.24.
-        self.scaled = tmax.astype(np.float64) * G
+    def __init__(self, G: int, window: Optional[_Window], first: int):
+        self.G, self.window = G, window
         self.pos = first          # everything below is infeasible: the scan passes it unchanged
         self.have_lo = first
         self.best_s = np.empty(0, dtype=np.int32)
@@ -155,10 +269,27 @@ class _Scan:
         self.stage_max = np.empty(0, dtype=np.float32)
         self.limit = FIRST_CHUNK
 
+    @property
+    def tmax(self) -> np.ndarray:
+        return self.window.kept if self.window is not None else np.empty(0, dtype=np.float32)
+
+    @property
+    def scaled(self) -> np.ndarray:
+        return self.window.scaled if self.window is not None else np.empty(0, dtype=np.float64)
+
+    def _reach(self, pos: int, best_cost: float) -> bool:
+        """Makes sure threshold ``pos`` is materialised if the scan can get there; False if the
+        scan ends before it."""
+        w = self.window
+        while w is not None and pos >= len(w.kept) and not w.covers(best_cost):
+            w.extend(best_cost)
+        return pos < len(self.tmax)
+
     def wanted(self, best_cost: float) -> Tuple[int, int]:
         """Index range [a, b) of thresholds to compute next under the bound ``best_cost``; the
         range grows fourfold every time the same G asks again."""
         a = self.have_lo + len(self.best_s)
+        self._reach(a + self.limit, best_cost)
         stop = int(np.searchsorted(self.scaled, best_cost, side="left"))
         b = max(a, min(stop, a + self.limit))
         if b > a:
@@ -170,7 +301,7 @@ class _Scan:
         is reached is no larger, so the true scan stops no later): True if the computed results
         would not suffice."""
         pos, hi, G = self.pos, self.have_lo + len(self.best_s), self.G
-        while pos < len(self.tmax):
+        while self._reach(pos, best_cost):
             if self.scaled[pos] >= best_cost:
                 return False
             if pos >= hi:
@@ -192,7 +323,7 @@ class _Scan:
         (best_cost, best_t, finished)."""
         G = self.G
         hi = self.have_lo + len(self.best_s)
-        while self.pos < len(self.tmax):
+        while self._reach(self.pos, best_cost):
             if self.scaled[self.pos] >= best_cost:  # inter_tuning.py:196-197
                 return best_cost, best_t, True
             if self.pos >= hi:
@@ -268,21 +399,49 @@ def inter_stage_tune_batch(
     # table row of (instance, G)
     rows = np.array([[t * n_g + g_index[G] for G in Gs] for t in range(n_inst)], dtype=np.int32)
     t_0 = time.perf_counter()
-    tmax_all = runner.thresholds()
-    t_1 = time.perf_counter()
 
-    # Smallest feasible threshold of every (instance, G) in one launch (bottleneck DP).
+    # Smallest feasible threshold of every (instance, G) in one launch (bottleneck DP), then one
+    # threshold DP there: its cost bounds how far up the scan of that G can get.
     flat = rows.reshape(-1)
+    flat_G = np.tile(np.array(Gs, dtype=np.int64), n_inst)
     _, bottleneck, _ = runner.run(flat, np.zeros(len(flat), dtype=np.float32), _lib.DP_BOTTLENECK)
-    bottleneck = bottleneck.reshape(rows.shape)
+    feasible = np.isfinite(bottleneck)
+    windows: List[Optional[_Window]] = [None] * len(flat)
+    if feasible.any():
+        idx = np.nonzero(feasible)[0]
+        bs0, sum0, max0 = runner.run(flat[idx], bottleneck[idx])
+        assert (bs0 >= 0).all()
+        bound = sum0.astype(np.float64) + (flat_G[idx] - 1).astype(np.float64) * max0.astype(np.float64)
+        hi = np.nextafter((bound * (1.0 + 1e-5) / flat_G[idx]).astype(np.float32), np.float32(np.inf))
+        hi = np.maximum(hi, np.nextafter(bottleneck[idx], np.float32(np.inf)))
+        for k, i in enumerate(idx):
+            windows[i] = _Window(runner, int(flat[i]), int(flat_G[i]), bottleneck[i], float(sum0[k]))
+        pending, widen = list(range(len(idx))), 0
+        while pending:
+            lo = np.array([windows[idx[k]].lower_margin(widen) for k in pending], dtype=np.float32)
+            if widen >= 8:
+                lo[:] = -np.inf
+            got = runner.candidates_between(flat[idx[pending]], lo, hi[pending])
+            pending = [k for j, k in enumerate(pending)
+                       if not windows[idx[k]].begin(got[j][0], got[j][1], lo[j], hi[k])]
+            widen += 1
+        # one more pass for the windows whose first kept candidate turned out to lie higher
+        # than assumed (the remaining cases extend one by one while the scan runs)
+        short = [windows[i] for i in idx if not windows[i].covers(float("inf"))]
+        if short:
+            want = np.array([w.extension_target(float("inf")) for w in short], dtype=np.float32)
+            got = runner.candidates_between(
+                np.array([w.row for w in short]), np.array([w.hi for w in short], dtype=np.float32), want)
+            for w, (values, n_above), hi_w in zip(short, got, want):
+                w.apply_extension(values, n_above, hi_w)
+    t_1 = time.perf_counter()
     chains = []
     for t in range(n_inst):
         scans = []
         for i, G in enumerate(Gs):
-            tmax = tmax_all[rows[t, i]]
-            b = bottleneck[t, i]
-            start = int(np.searchsorted(tmax, b, side="left")) if np.isfinite(b) else len(tmax)
-            scans.append(_Scan(G, tmax, start))
+            w = windows[t * len(Gs) + i]
+            start = int(np.searchsorted(w.kept, w.start_value, side="left")) if w is not None else 0
+            scans.append(_Scan(G, w, start))
         chains.append(dict(scans=scans, current=0, best=(float("inf"), None, None)))
 
     # Speculative batches + sequential replay (see the module docstring).
@@ -359,6 +518,7 @@ def inter_stage_tune_batch(
         stats["dp_scan_s"] = stats.get("dp_scan_s", 0.0) + (t_2 - t_1)
         stats["dp_backtrack_s"] = stats.get("dp_backtrack_s", 0.0) + (time.perf_counter() - t_2)
         stats["dp_launches"] = stats.get("dp_launches", 0) + runner.launches
+        stats["dp_window_fetches"] = stats.get("dp_window_fetches", 0) + runner.fetches
         stats["dp_thresholds"] = stats.get("dp_thresholds", 0) + runner.thresholds_run
     return out
 

@@ -230,3 +230,68 @@ def test_gap_filter_matches_oracle_rule():
         last = v
     assert n == len(want) and np.array_equal(out[:n], np.array(want, dtype=np.float32))
     assert 0 < n < len(t)
+
+
+class _FakeRunner:
+    """Host stand-in of the DP runner's candidate store for one table row."""
+
+    def __init__(self, values):
+        from mist_amd import _lib
+
+        self.values = np.sort(np.asarray(values, dtype=np.float32))
+        self.lib = _lib.load()
+        self.fetches = 0
+
+    def candidates_between(self, rows, lo, hi):
+        self.fetches += 1
+        out = []
+        for l, h in zip(lo, hi):
+            v = self.values
+            out.append((v[(v > l) & (v <= h)], int((v > h).sum())))
+        return out
+
+    def filter_gap(self, ascending):
+        from mist_amd.inter_tuning import _DpRunner
+
+        return _DpRunner.filter_gap(self, ascending)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_threshold_window_equals_full_walk(seed):
+    """The lazily materialised window of kept t_max candidates must equal the reference's walk
+    over the complete sorted list (inter_tuning.py:180-198) from the smallest feasible
+    threshold on, whatever the spacing of the candidates below it."""
+    from mist_amd.inter_tuning import GAP, _Window
+
+    rng = np.random.default_rng(seed)
+    centres = rng.uniform(0.05, 40.0, size=300)
+    dense = (centres[:, None] + rng.uniform(0, 3e-6, size=(300, 6)) * rng.integers(0, 2, size=(300, 1))).ravel()
+    values = np.unique(np.concatenate([dense, rng.uniform(0.05, 40.0, size=500)]).astype(np.float32))
+    runner = _FakeRunner(values)
+    full = runner.filter_gap(values)
+    # reference walk written out: keep t unless t - last < gap (float32 difference)
+    last, want_full = None, []
+    for t in values:
+        if last is not None and np.float64(np.float32(t) - np.float32(last)) < GAP:
+            continue
+        want_full.append(t)
+        last = t
+    assert np.array_equal(full, np.array(want_full, dtype=np.float32))
+
+    for trial in range(20):
+        start = values[rng.integers(len(values))] if trial % 2 else np.float32(rng.uniform(0.0, 41.0))
+        G = int(rng.choice([1, 2, 8, 64]))
+        w = _Window(runner, 0, G, start, start_sum=float(start) * 2)
+        widen = 0
+        while True:
+            lo = w.lower_margin(widen) if widen < 8 else np.float32(-np.inf)
+            hi = np.float32(start + rng.uniform(0, 0.5))
+            (vals, above), = runner.candidates_between([0], [lo], [hi])
+            if w.begin(vals, above, lo, hi):
+                break
+            widen += 1
+        while not w.complete:
+            w.extend(float("inf"))
+        want = full[full >= start]
+        got = w.kept[np.searchsorted(w.kept, start, side="left"):]
+        assert np.array_equal(got, want), (seed, trial)

@@ -133,3 +133,73 @@ def test_plan1_end_to_end():
     want = oracle_tune(cfg, tables)
     assert want[1] is not None
     assert got == want
+
+
+def test_full_size_dp_matches_c_oracle_on_gpt7b_tables():
+    """GPT-7B plan at full size (L = 32, 32 devices, 6 meshes, 32 pre-saved micro-batch values):
+    the intra-stage tables come from the GPU search (checked elsewhere); the DP kernel is compared
+    with the C oracle on those tables at the thresholds that matter - just below the smallest
+    feasible one, at it, a run of kept candidates above it and the winning one, back-pointers
+    included.  (The reference's full ascending scan needs ~10^5 DP runs per G on the CPU.)"""
+    from mist_amd import _lib
+    from mist_amd.inter_tuning import _DpRunner, _Window, inter_stage_tune
+    from mist_amd.intra_tuning import IntraStageTuner
+    from mist_amd.search_space import _get_device_mesh_candidates, _get_grad_accumu_steps_candidates
+    from oracle.dp_c import dp_impl_c
+    from oracle.inter_dp import dp_cost_tables
+
+    cfg, tables = load_plan(2)
+    hw, L = cfg.hardware, cfg.model.num_hidden_layers
+    D = hw.num_nodes * hw.num_gpus_per_node
+    meshes = _get_device_mesh_candidates(hw.num_nodes, hw.num_gpus_per_node, False)
+    Gs = _get_grad_accumu_steps_candidates(cfg.training.global_batch_size)
+    res = IntraStageTuner(tables, L, meshes, Gs, 8, cfg, sample_size=1).tune()
+    best_cost, best_solution = inter_stage_tune(L, D, meshes, Gs, res)
+    assert best_solution is not None
+    runner = _DpRunner(res, L, D, meshes, 0)
+    n_checked = 0
+    for g in (Gs.index(best_solution[0]), Gs.index(32), len(Gs) - 1):
+        G = Gs[g]
+        tabs = dp_cost_tables(res, g)
+        _, bott, _ = runner.run(np.array([g], dtype=np.int32), np.zeros(1, dtype=np.float32),
+                                _lib.DP_BOTTLENECK)
+        assert np.isfinite(bott[0])
+        lo = np.float32(bott[0] * 0.98)
+        (vals, _), = runner.candidates_between(np.array([g]), np.array([lo]), np.array([bott[0] * 1.02], dtype=np.float32))
+        vals = np.unique(vals)
+        at = int(np.searchsorted(vals, bott[0]))
+        tmax = np.concatenate([vals[max(at - 3, 0):at], vals[at:at + 9]])
+        bs, bsum, smax, arg = runner.run(np.full(len(tmax), g, dtype=np.int32), tmax, want_argmin=True)
+        for i, t in enumerate(tmax):
+            want_cost, want_sol = dp_impl_c(t, L, D, meshes, G, *tabs)
+            assert (bs[i] >= 0) == (want_sol is not None), (G, t)
+            assert (t >= bott[0]) == (bs[i] >= 0), "bottleneck DP disagrees with the threshold DP"
+            if want_sol is None:
+                continue
+            got_cost = float(np.float64(bsum[i]) + np.float64(G - 1) * np.float64(smax[i]))
+            assert got_cost == want_cost, (G, t)
+            sol, cs, cl, cd = [], int(bs[i]), 0, D
+            while cs > 0:
+                end, n, m, ckpt = (int(v) for v in arg[i][cs, cl, cd])
+                sol.append(((cl, end), (n, m), ckpt))
+                cs, cl, cd = cs - 1, end + 1, cd - n * m
+            assert sol == want_sol, (G, t)
+            n_checked += 1
+    assert n_checked >= 12
+    # the search's answer is one of the DP solutions: recompute it at its own bottleneck
+    g = Gs.index(best_solution[0])
+    tabs = dp_cost_tables(res, g)
+    inter = [s[0][:3] for s in best_solution[1]]
+    costs = []
+    for i, ((l0, l1), mesh, ckpt) in enumerate(inter):
+        q, l, p = meshes.index(mesh), l1 - l0 + 1, len(inter) - i - 1
+        if len(inter) == 1:
+            costs.append(tabs[3][q, ckpt])
+        elif i == 0:
+            costs.append(tabs[1][q, p, l - 1, ckpt])
+        elif i == len(inter) - 1:
+            costs.append(tabs[2][q, l - 1, ckpt])
+        else:
+            costs.append(tabs[0][q, p, l - 1, ckpt])
+    want_cost, want_sol = dp_impl_c(np.float32(max(costs)), L, D, meshes, Gs[g], *tabs)
+    assert want_cost == best_cost and want_sol == inter

@@ -31,8 +31,8 @@ def _oracle(cfg, tables, tp, S, meshes, Gs):
     return intra_stage_tune(tables, cfg, cfg.model.num_hidden_layers, meshes, Gs, tp, S)
 
 
-def _compare(cfg, tables, tp, S=1, slots=None):
-    tuner = _gpu_tuner(cfg, tables, tp, S=S, slots=slots)
+def _compare(cfg, tables, tp, S=1, slots=None, meshes=None, Gs=None):
+    tuner = _gpu_tuner(cfg, tables, tp, S=S, slots=slots, meshes=meshes, Gs=Gs)
     got = tuner.tune()
     want = _oracle(cfg, tables, tp, S, tuner.device_mesh_candidates,
                    tuner.gradient_accumulation_steps_candidates)
@@ -154,3 +154,34 @@ def test_scout_pass_leaves_results_unchanged(monkeypatch, scout_stages, min_stri
     _compare(cfg, tables, 1)
     cfg, tables = load_plan(1)
     _compare(cfg, tables, 2)
+
+
+@pytest.mark.parametrize(
+    "plan, G, mesh, tp", [(2, 64, (1, 1), 1), (2, 128, (1, 8), 8), (3, 64, (1, 8), 8)]
+)
+def test_full_size_groups_match_oracle(plan, G, mesh, tp):
+    """Whole (G, mesh, tp) groups of the large plans at their real shape (10^4 rows, all layer /
+    ckpt counts, 32..40 pre-saved micro-batch values = 2..3 p tiles, scout pass and many row
+    chunks in play).  The GPU searches the complete plan; the numpy oracle needs ~10 s per
+    group, so only these groups are compared."""
+    from oracle.intra import intra_stage_tune
+
+    cfg, tables = load_plan(plan)
+    tuner = _gpu_tuner(cfg, tables, tp)
+    meshes, Gs = tuner.device_mesh_candidates, tuner.gradient_accumulation_steps_candidates
+    g, q = Gs.index(G), meshes.index(mesh)
+    rec = [r for r in tuner.prepare()["groups"] if r["g_index"] == g and r["q_index"] == q]
+    assert len(rec) == 1 and rec[0]["scout_stride"] > 0 and rec[0]["n_chunks"] > 1
+    assert rec[0]["n_p_tiles"] >= 2
+    got = tuner.tune()
+    want = intra_stage_tune(tables, cfg, cfg.model.num_hidden_layers, meshes, Gs, tp, 1,
+                            groups=[(g, q)])
+    n_finite = 0
+    for suffix in ("", "_with_pre", "_with_post", "_no_pp"):
+        gi, wi = getattr(got, "indices" + suffix)[g, q], getattr(want, "indices" + suffix)[g, q]
+        assert np.array_equal(gi, wi), f"indices{suffix}: {np.sum(gi != wi)} of {gi.size} differ"
+        for kind in ("stable", "delta"):
+            assert_same_f64(getattr(got, f"costs_{kind}{suffix}")[g, q],
+                            getattr(want, f"costs_{kind}{suffix}")[g, q], f"costs_{kind}{suffix}")
+        n_finite += int((gi >= 0).sum())
+    assert n_finite > 1000

@@ -83,6 +83,9 @@ def main():
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one plain 1 GiB device copy (known HBM traffic to scale the "
+                         "FETCH_SIZE / WRITE_SIZE counters of a profiler run against)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU only (got --gpus {args.gpus}): the search runs on a "
@@ -150,6 +153,12 @@ def main():
         launches_per_step=1,
     )
     intra_ms_per_step = sum(kernel_ms.values()) / 2
+    if args.copy_calibration:
+        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda:0").normal_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)  # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
 
     result = {
         "metric": "candidate configs evaluated/sec (fp64), GPT-7B space",

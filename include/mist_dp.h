@@ -22,8 +22,15 @@ typedef struct MistDpShape {
   int32_t num_devices;  /* D */
   int32_t num_mesh;     /* Q <= MIST_MAX_MESH, in candidate-list order */
   int32_t p_dim;        /* P+1: extent of the pre-saved-micro-batch axis of the cost tables */
-  int32_t max_stages;   /* S_max = min(max(n*m), L) // 2 */
-  int32_t reserved[3];
+  int32_t max_stages;   /* stage counts 1..max_stages are searched (<= p_dim, <= L) */
+  int32_t ckpt_rule;    /* ckpt candidates j of a stage of l layers ending at layer i:
+                         * MIST_DP_CKPT_TAIL 0..L-i (inter_tuning.py:315),
+                         * MIST_DP_CKPT_STAGE 0..l, MIST_DP_CKPT_ALL only l
+                         * (inter_tuning_uniform_device.py:400-404) */
+  int32_t free_devices; /* != 0: stages do not consume devices (every stage runs on mesh 0 and the
+                         * stage count alone decides feasibility; inter_tuning_uniform_device.py);
+                         * num_devices must then be 0 and num_mesh 1 */
+  int32_t reserved;
   int32_t mesh_n[MIST_MAX_MESH], mesh_m[MIST_MAX_MESH];
 } MistDpShape;
 
@@ -36,6 +43,10 @@ typedef struct MistDpCosts {
   const float *pmin, *pmin_pre, *pmin_post, *pmin_nopp;
   int64_t g_stride[4];
 } MistDpCosts;
+
+#define MIST_DP_CKPT_TAIL 0
+#define MIST_DP_CKPT_STAGE 1
+#define MIST_DP_CKPT_ALL 2
 
 #define MIST_DP_THRESHOLD 0  /* sum of stage costs subject to cost <= t_max */
 #define MIST_DP_BOTTLENECK 1 /* smallest achievable maximum stage cost; t_max is ignored */
@@ -63,7 +74,7 @@ int mist_dp_filter_tmax(const float *sorted_unique, int n, double gap, float *ou
 /* Runs n_tmax DP instances at once (max_stages launches, one thread per (instance, start
  * layer, devices) state).  Instance t uses the cost tables of g = d_g_index[t].
  * MIST_DP_THRESHOLD (reference: inter_stage_tune_dp_impl, inter_tuning.py:220-355):
- *   F(s,k,d) = min over mesh q (n*m <= d), end layer i >= k, ckpt j in 0..L-i of
+ *   F(s,k,d) = min over mesh q (n*m <= d), end layer i >= k, ckpt j (shape->ckpt_rule) of
  *              cost(s,k,i,q,j) + F(s-1,i+1,d-n*m)   subject to cost <= d_tmax[t],
  *   float32 adds, strict "<" in the reference's (q, i, j) order.  Outputs per instance:
  *   d_best_s (-1 = infeasible), d_best_sum = F(best_s,0,D), d_stage_max = running max of the

@@ -23,6 +23,7 @@ SCOUT_SPLIT = 4  # replaced by the library's own value in load()
 STAGE_ROWS = 64  # replaced by the library's own value in load()
 TERMS_BLOCK = 256
 MAX_MESH = 16
+DP_CKPT_TAIL, DP_CKPT_STAGE, DP_CKPT_ALL = 0, 1, 2
 DP_THRESHOLD, DP_BOTTLENECK = 0, 1
 
 PAR_NAMES = (
@@ -145,7 +146,7 @@ def exported_symbols():
 DP_SHAPE_DTYPE = np.dtype(
     [
         ("num_layers", "<i4"), ("num_devices", "<i4"), ("num_mesh", "<i4"), ("p_dim", "<i4"),
-        ("max_stages", "<i4"), ("reserved", "<i4", (3,)),
+        ("max_stages", "<i4"), ("ckpt_rule", "<i4"), ("free_devices", "<i4"), ("reserved", "<i4"),
         ("mesh_n", "<i4", (MAX_MESH,)), ("mesh_m", "<i4", (MAX_MESH,)),
     ],
     align=True,

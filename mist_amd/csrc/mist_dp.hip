@@ -102,11 +102,14 @@ __global__ __launch_bounds__(kDpThreads) void dp_step_kernel(
   const int k = e / W, d = e % W;
   const int p = s - 1;
 
+  const bool free_devices = shape.free_devices != 0;
+  const int rule = shape.ckpt_rule;
+
   float best = INFINITY, best_m = 0.0f;
   int arg_i = -1, arg_q = -1, arg_j = -1;
-  if (k <= L - s && d >= 1) {
+  if (k <= L - s && (d >= 1 || free_devices)) {
     for (int q = 0; q < Q; ++q) {
-      const int nm = shape.mesh_n[q] * shape.mesh_m[q];
+      const int nm = free_devices ? 0 : shape.mesh_n[q] * shape.mesh_m[q];
       if (nm > d) continue;
       for (int i = k; i < L; ++i) {
         const int from = (i + 1) * W + (d - nm);
@@ -125,13 +128,17 @@ __global__ __launch_bounds__(kDpThreads) void dp_step_kernel(
                                              : v == 2 ? tabs.costs_post : tabs.costs_nopp;
         const float *__restrict__ pmin_tab = v == 0 ? tabs.pmin : v == 1 ? tabs.pmin_pre
                                              : v == 2 ? tabs.pmin_post : tabs.pmin_nopp;
-        const int j_end = L - i;  // ckpt candidates 0..L-i (inter_tuning.py:315)
+        // ckpt candidates j_begin..j_end: 0..L-i (inter_tuning.py:315), or 0..l / only l
+        // (inter_tuning_uniform_device.py:400-404)
+        const int j_end = rule == MIST_DP_CKPT_TAIL ? L - i : l;
+        const int j_begin = rule == MIST_DP_CKPT_ALL ? l : 0;
         // The reference walks j = 0..j_end with "cost <= t_max and cost + prev < best".  "+ prev"
         // is monotone, so the smallest reachable sum is (smallest admissible cost) + prev, and
         // the smallest admissible cost is the row's running minimum if that is <= t_max (else
         // nothing is admissible).  Only when this sum beats `best` is the row walked, to find
         // the first j that attains it: that is the entry the reference's strict "<" keeps.
-        const float rmin = pmin_tab[off[v] + at + j_end];
+        const float rmin = rule == MIST_DP_CKPT_ALL ? cost_tab[off[v] + at + l]
+                                                    : pmin_tab[off[v] + at + j_end];
         if (!(rmin <= t_max)) continue;
         const float target = kBottleneck ? fmaxf(rmin, prev) : rmin + prev;
         if (!(target < best)) continue;
@@ -140,7 +147,7 @@ __global__ __launch_bounds__(kDpThreads) void dp_step_kernel(
         arg_q = q;
         if (!kBottleneck) {
           const float *__restrict__ row = cost_tab + off[v] + at;
-          for (int j = 0; j <= j_end; ++j) {
+          for (int j = j_begin; j <= j_end; ++j) {
             const float stage_cost = row[j];
             if (stage_cost <= t_max && stage_cost + prev == target) {
               arg_j = j;
@@ -172,7 +179,13 @@ __global__ __launch_bounds__(kDpThreads) void dp_step_kernel(
 
 int check_shape(const MistDpShape *shape) {
   if (!shape) return fail(MIST_E_INVALID, "null DP shape");
-  if (shape->num_layers <= 0 || shape->num_devices <= 0 || shape->p_dim <= 0)
+  if (shape->free_devices != 0 && (shape->num_devices != 0 || shape->num_mesh != 1))
+    return fail(MIST_E_INVALID, "free_devices needs num_devices = 0 and one mesh (got D=%d Q=%d)",
+                shape->num_devices, shape->num_mesh);
+  if (shape->ckpt_rule < MIST_DP_CKPT_TAIL || shape->ckpt_rule > MIST_DP_CKPT_ALL)
+    return fail(MIST_E_INVALID, "unknown ckpt_rule %d", shape->ckpt_rule);
+  if (shape->num_layers <= 0 || shape->p_dim <= 0 ||
+      (shape->free_devices ? shape->num_devices != 0 : shape->num_devices <= 0))
     return fail(MIST_E_INVALID, "bad DP extents L=%d D=%d P+1=%d", shape->num_layers,
                 shape->num_devices, shape->p_dim);
   if (shape->num_mesh <= 0 || shape->num_mesh > MIST_MAX_MESH)

@@ -39,11 +39,24 @@ def _stream(device) -> ctypes.c_void_p:
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 
+class _DpFamily:
+    """One recurrence the DP kernel can run: a MistDpShape plus the cost tables it reads."""
+
+    def __init__(self, shape: np.ndarray, costs_struct, consumes_devices: bool):
+        self.shape, self.costs_struct, self.consumes_devices = shape, costs_struct, consumes_devices
+        self.L, self.D = int(shape["num_layers"][0]), int(shape["num_devices"][0])
+        self.S_max = int(shape["max_stages"][0])
+        self.plane = (self.L + 1) * (self.D + 1)
+
+
 class _DpRunner:
-    """Owns the float32 cost tables of all g and runs batches of DP instances."""
+    """Owns the float32 cost tables of all g and runs batches of DP instances.  A search is made
+    of one or more *families* (recurrences): the per-mesh DP has one, the uniform-device DP one
+    per admissible stage count; an instance's cost is the smallest family cost, the first
+    family winning ties."""
 
     def __init__(self, results: IntraStageTunerOutput, num_layers: int, num_devices: int,
-                 meshes: List[Tuple[int, int]], slot: int):
+                 meshes: List[Tuple[int, int]], slot: int, uniform_device: Optional[dict] = None):
         self.lib = _lib.load()
         dev_tabs = results.batch  # tables of every tp candidate of the same launch
         self.device = dev_tabs.stable[0].device
@@ -55,14 +68,6 @@ class _DpRunner:
         if list(meshes) != list(results.device_mesh_candidates):
             raise ValueError("the DP needs the mesh list the intra-stage tables were built for")
         self.L, self.D, self.Q, self.P1, self.Gn = L, num_devices, Q, P1, Gn
-        shape = np.zeros(1, dtype=_lib.DP_SHAPE_DTYPE)
-        shape["num_layers"], shape["num_devices"], shape["num_mesh"], shape["p_dim"] = L, num_devices, Q, P1
-        self.S_max = min(max(n * m for n, m in meshes), L) // 2  # inter_tuning.py:278-280
-        shape["max_stages"] = self.S_max
-        shape["mesh_n"][0, :Q] = [n for n, _ in meshes]
-        shape["mesh_m"][0, :Q] = [m for _, m in meshes]
-        self.shape = shape
-        self.plane = (L + 1) * (num_devices + 1)
         problem = np.zeros(1, dtype=_lib.PROBLEM_DTYPE)
         problem["num_layers"], problem["p_dim"], problem["sample_size"] = L, P1, S
         problem["num_grad_accum"], problem["num_mesh"] = Gn, Q
@@ -81,13 +86,59 @@ class _DpRunner:
                 out_ptrs, pmin_ptrs, _stream(self.device),
             )
             _lib.check(rc, "mist_dp_cost_tables")
-        self.costs_struct = _lib.DpCosts(*[t.data_ptr() for t in self.cost + self.pmin])
-        for v in range(4):
-            self.costs_struct.g_stride[v] = self.cost[v][0].numel()
+        if uniform_device is None:
+            self.families = [self._per_mesh_family(meshes)]
+        else:
+            self.families = self._uniform_device_families(meshes, **uniform_device)
         self.launches = 0
         self.thresholds_run = 0
         self._cand = None
         self.fetches = 0
+
+    def _costs_struct(self, q: int = 0):
+        """Table pointers starting at mesh ``q`` (strides between g unchanged)."""
+        per_q = [self.cost[v][0, 0].numel() for v in range(4)]
+        ptrs = [t.data_ptr() + 4 * q * per_q[v] for v, t in enumerate(self.cost)]
+        ptrs += [t.data_ptr() + 4 * q * per_q[v] for v, t in enumerate(self.pmin)]
+        cs = _lib.DpCosts(*ptrs)
+        for v in range(4):
+            cs.g_stride[v] = self.cost[v][0].numel()
+        return cs
+
+    def _per_mesh_family(self, meshes) -> _DpFamily:
+        shape = np.zeros(1, dtype=_lib.DP_SHAPE_DTYPE)
+        shape["num_layers"], shape["num_devices"] = self.L, self.D
+        shape["num_mesh"], shape["p_dim"] = self.Q, self.P1
+        shape["max_stages"] = min(max(n * m for n, m in meshes), self.L) // 2  # inter_tuning.py:278-280
+        shape["ckpt_rule"] = _lib.DP_CKPT_TAIL
+        shape["mesh_n"][0, :self.Q] = [n for n, _ in meshes]
+        shape["mesh_m"][0, :self.Q] = [m for _, m in meshes]
+        return _DpFamily(shape, self._costs_struct(), True)
+
+    def _uniform_device_families(self, meshes, num_nodes, num_gpus_per_node, ckpt_tuning):
+        """One family per stage count S whose even split of the cluster is a mesh candidate
+        (inter_tuning_uniform_device.py:312-334, 360-367): s <= S stages, all on that mesh."""
+        from .inter_tuning_uniform import _uniform_device_mesh_partition
+
+        fams = []
+        for S in range(1, self.L + 1):
+            mesh = _uniform_device_mesh_partition(S, num_nodes, num_gpus_per_node)
+            if mesh is None:
+                continue
+            if mesh not in meshes:
+                raise ValueError(f"uniform mesh {mesh} of {S} stages is not a mesh candidate")
+            q = max(i for i, nm in enumerate(meshes) if nm == mesh)
+            shape = np.zeros(1, dtype=_lib.DP_SHAPE_DTYPE)
+            shape["num_layers"], shape["num_devices"], shape["num_mesh"] = self.L, 0, 1
+            shape["p_dim"] = self.P1
+            # stage counts beyond the p axis of the tables cost +inf (the reference indexes out
+            # of bounds there), so they need not be run
+            shape["max_stages"] = min(S, self.P1, self.L)
+            shape["ckpt_rule"] = _lib.DP_CKPT_STAGE if ckpt_tuning else _lib.DP_CKPT_ALL
+            shape["free_devices"] = 1
+            shape["mesh_n"][0, 0], shape["mesh_m"][0, 0] = mesh
+            fams.append(_DpFamily(shape, self._costs_struct(q), False))
+        return fams
 
     def _all_candidates(self) -> torch.Tensor:
         """[Gn, N] float32: every stage cost the reference collects as a t_max candidate
@@ -130,9 +181,10 @@ class _DpRunner:
         return kept[:n]
 
     def run(self, g_index: np.ndarray, tmax: np.ndarray, mode: int = _lib.DP_THRESHOLD,
-            want_argmin: bool = False):
-        """DP instances (g_index[i], tmax[i]) -> (best_s int32, best_sum f32, stage_max f32
-        [, argmin])."""
+            want_argmin: bool = False, family: Optional[_DpFamily] = None):
+        """DP instances (g_index[i], tmax[i]) of one family -> (best_s int32, best_sum f32,
+        stage_max f32 [, argmin])."""
+        fam = self.families[0] if family is None else family
         n = len(tmax)
         dev = self.device
         with torch.cuda.device(dev):
@@ -141,13 +193,13 @@ class _DpRunner:
             packed[1].view(np.int32)[:] = g_index
             d_in = torch.from_numpy(packed).to(dev)
             d_out = torch.empty((3, n), dtype=torch.float32, device=dev)
-            scratch = torch.empty(4 * n * self.plane, dtype=torch.float32, device=dev)
+            scratch = torch.empty(4 * n * fam.plane, dtype=torch.float32, device=dev)
             argmin = None
             if want_argmin:
-                argmin = torch.full((n, self.S_max + 1, self.L + 1, self.D + 1, 4), -1,
+                argmin = torch.full((n, fam.S_max + 1, fam.L + 1, fam.D + 1, 4), -1,
                                     dtype=torch.int32, device=dev)
             rc = self.lib.mist_dp_run(
-                ctypes.c_void_p(self.shape.ctypes.data), ctypes.byref(self.costs_struct),
+                ctypes.c_void_p(fam.shape.ctypes.data), ctypes.byref(fam.costs_struct),
                 d_in[0].data_ptr(), d_in[1].data_ptr(), n, mode,
                 d_out[0].data_ptr(), d_out[1].data_ptr(), d_out[2].data_ptr(),
                 argmin.data_ptr() if want_argmin else None, scratch.data_ptr(), _stream(dev),
@@ -160,6 +212,60 @@ class _DpRunner:
             if want_argmin:
                 out = out + (argmin.cpu().numpy(),)
         return out
+
+    @staticmethod
+    def _total(best_s, best_sum, stage_max, G) -> np.ndarray:
+        """``best + (g - 1) * f_stage_max`` in float64 (inter_tuning.py:342), inf if infeasible."""
+        total = best_sum.astype(np.float64) + (np.asarray(G, dtype=np.float64) - 1.0) * stage_max.astype(np.float64)
+        return np.where(best_s >= 0, total, np.inf)
+
+    def evaluate(self, g_index: np.ndarray, tmax: np.ndarray, G: np.ndarray):
+        """Cost of every instance = smallest family total (first family on ties), the family
+        that attains it (-1 if none) and the smallest feasible family sum."""
+        cost = np.full(len(tmax), np.inf)
+        winner = np.full(len(tmax), -1, dtype=np.int32)
+        min_sum = np.full(len(tmax), np.inf)
+        for f, fam in enumerate(self.families):
+            bs, bsum, smax = self.run(g_index, tmax, family=fam)
+            total = self._total(bs, bsum, smax, G)
+            better = total < cost
+            cost = np.where(better, total, cost)
+            winner = np.where(better, f, winner)
+            min_sum = np.minimum(min_sum, np.where(bs >= 0, bsum.astype(np.float64), np.inf))
+        return cost, winner, min_sum
+
+    def bottleneck(self, g_index: np.ndarray) -> np.ndarray:
+        """Smallest threshold for which any family is feasible (float32, +inf if none)."""
+        b = np.full(len(g_index), np.inf, dtype=np.float32)
+        zeros = np.zeros(len(g_index), dtype=np.float32)
+        for fam in self.families:
+            _, bott, _ = self.run(g_index, zeros, _lib.DP_BOTTLENECK, family=fam)
+            b = np.minimum(b, bott)
+        return b
+
+    def partition(self, g: int, tmax: np.float32, G: int):
+        """``(stage count, [((l0, l1), (n, m), ckpt), ...])`` of the winning family of one
+        instance, from its back-pointers (inter_tuning.py:341-355)."""
+        best = (np.inf, None)
+        for fam in self.families:
+            bs, bsum, smax, argmin = self.run(np.array([g], dtype=np.int32),
+                                              np.array([tmax], dtype=np.float32),
+                                              want_argmin=True, family=fam)
+            total = float(self._total(bs, bsum, smax, G)[0])
+            if total < best[0]:
+                best = (total, (fam, int(bs[0]), argmin[0]))
+        assert best[1] is not None
+        fam, cs, argmin = best[1]
+        cl, cd, inter = 0, fam.D, []
+        while cs > 0 and cl < fam.L and (cd > 0 or not fam.consumes_devices):
+            end, n, m, ckpt = (int(v) for v in argmin[cs, cl, cd])
+            assert end != -1
+            inter.append(((cl, end), (n, m), ckpt))
+            cs, cl = cs - 1, end + 1
+            if fam.consumes_devices:
+                cd -= n * m
+        assert cs == 0 and cl == fam.L and cd == 0
+        return best[0], inter
 
 
 def _gap_reached(a: np.ndarray, b: np.ndarray) -> np.ndarray:
@@ -264,9 +370,7 @@ class _Scan:
         self.G, self.window = G, window
         self.pos = first          # everything below is infeasible: the scan passes it unchanged
         self.have_lo = first
-        self.best_s = np.empty(0, dtype=np.int32)
-        self.best_sum = np.empty(0, dtype=np.float32)
-        self.stage_max = np.empty(0, dtype=np.float32)
+        self.cost = np.empty(0, dtype=np.float64)  # DP outcome per computed threshold, inf = infeasible
         self.limit = FIRST_CHUNK
 
     @property
@@ -288,7 +392,7 @@ class _Scan:
     def wanted(self, best_cost: float) -> Tuple[int, int]:
         """Index range [a, b) of thresholds to compute next under the bound ``best_cost``; the
         range grows fourfold every time the same G asks again."""
-        a = self.have_lo + len(self.best_s)
+        a = self.have_lo + len(self.cost)
         self._reach(a + self.limit, best_cost)
         stop = int(np.searchsorted(self.scaled, best_cost, side="left"))
         b = max(a, min(stop, a + self.limit))
@@ -300,39 +404,32 @@ class _Scan:
         """Dry run of ``replay`` under the bound ``best_cost`` (the true running best when this G
         is reached is no larger, so the true scan stops no later): True if the computed results
         would not suffice."""
-        pos, hi, G = self.pos, self.have_lo + len(self.best_s), self.G
+        pos, hi, G = self.pos, self.have_lo + len(self.cost), self.G
         while self._reach(pos, best_cost):
             if self.scaled[pos] >= best_cost:
                 return False
             if pos >= hi:
                 return True
-            i = pos - self.have_lo
-            if self.best_s[i] >= 0:
-                cost = float(np.float64(self.best_sum[i]) + np.float64(G - 1) * np.float64(self.stage_max[i]))
-                best_cost = min(best_cost, cost)
+            best_cost = min(best_cost, float(self.cost[pos - self.have_lo]))
             pos += 1
         return False
 
-    def add(self, best_s, best_sum, stage_max):
-        self.best_s = np.concatenate([self.best_s, best_s])
-        self.best_sum = np.concatenate([self.best_sum, best_sum])
-        self.stage_max = np.concatenate([self.stage_max, stage_max])
+    def add(self, cost: np.ndarray):
+        self.cost = np.concatenate([self.cost, cost])
 
     def replay(self, best_cost: float, best_t):
         """Advances the sequential scan as far as the computed results allow.  Returns
         (best_cost, best_t, finished)."""
         G = self.G
-        hi = self.have_lo + len(self.best_s)
+        hi = self.have_lo + len(self.cost)
         while self._reach(self.pos, best_cost):
             if self.scaled[self.pos] >= best_cost:  # inter_tuning.py:196-197
                 return best_cost, best_t, True
             if self.pos >= hi:
                 return best_cost, best_t, False     # needs more DP results
-            i = self.pos - self.have_lo
-            if self.best_s[i] >= 0:
-                cost = float(np.float64(self.best_sum[i]) + np.float64(G - 1) * np.float64(self.stage_max[i]))
-                if cost < best_cost:
-                    best_cost, best_t = cost, self.tmax[self.pos]
+            cost = float(self.cost[self.pos - self.have_lo])
+            if cost < best_cost:
+                best_cost, best_t = cost, self.tmax[self.pos]
             self.pos += 1
         return best_cost, best_t, True
 
@@ -361,58 +458,26 @@ def _same_batch(results_list) -> bool:
     ) and first.batch.stable[0].shape[0] == len(results_list) * len(first.gradient_accumulation_steps_candidates)
 
 
-def inter_stage_tune_batch(
-    num_layers: int,
-    num_devices: int,
-    device_mesh_candidates: List[Tuple[int, int]],
-    gradient_accumulation_steps_candidates: List[int],
-    results_list: List[IntraStageTunerOutput],
-    slot: int = 0,
-    stats: Optional[dict] = None,
-):
-    """``inter_stage_tune`` for several intra-stage results at once (the tensor-parallel
-    candidates of one ``tune`` call).  Each entry is searched exactly as if it were alone (its
-    own running best, its own stop rule); only the launches are shared.  Returns a list of
-    ``(best_cost, best_solution)``."""
-    for r in results_list:
-        if not isinstance(r, IntraStageTunerOutput):
-            raise TypeError(
-                f"intra_stage_results must be an instance of IntraStageTunerOutput, got {type(r)}"
-            )
-    if not _same_batch(results_list):
-        out = []
-        for r in results_list:
-            one = r if r.batch is r.device else IntraStageTunerOutput(
-                r.gradient_accumulation_steps_candidates, r.device_mesh_candidates, r.device,
-                r.spaces, r.sample_slots)
-            out += inter_stage_tune_batch(num_layers, num_devices, device_mesh_candidates,
-                                          gradient_accumulation_steps_candidates, [one], slot, stats)
-        return out
-    t_start = time.perf_counter()
-    first = results_list[0]
-    runner = _DpRunner(first, num_layers, num_devices, device_mesh_candidates, slot)
-    n_g = len(first.gradient_accumulation_steps_candidates)
-    g_index = {G: i for i, G in enumerate(first.gradient_accumulation_steps_candidates)}
-    q_index = {q: i for i, q in enumerate(first.device_mesh_candidates)}
-    Gs = list(gradient_accumulation_steps_candidates)
-    n_inst = len(results_list)
-    # table row of (instance, G)
-    rows = np.array([[t * n_g + g_index[G] for G in Gs] for t in range(n_inst)], dtype=np.int32)
+def _search(runner: _DpRunner, rows: np.ndarray, Gs: List[int], stats: Optional[dict]):
+    """The reference's scan (G after G, ascending kept thresholds, stop rule, strict "<";
+    inter_tuning.py:163-217 and :119-143) for ``rows.shape[0]`` independent instances whose
+    table row for G index i is ``rows[t, i]``.  Returns per instance ``(best_cost, G, t_max)``
+    (``G`` None if nothing is feasible)."""
+    n_inst = rows.shape[0]
     t_0 = time.perf_counter()
 
-    # Smallest feasible threshold of every (instance, G) in one launch (bottleneck DP), then one
+    # Smallest feasible threshold of every (instance, G) in one batch (bottleneck DP), then one
     # threshold DP there: its cost bounds how far up the scan of that G can get.
     flat = rows.reshape(-1)
     flat_G = np.tile(np.array(Gs, dtype=np.int64), n_inst)
-    _, bottleneck, _ = runner.run(flat, np.zeros(len(flat), dtype=np.float32), _lib.DP_BOTTLENECK)
+    bottleneck = runner.bottleneck(flat)
     feasible = np.isfinite(bottleneck)
     windows: List[Optional[_Window]] = [None] * len(flat)
     if feasible.any():
         idx = np.nonzero(feasible)[0]
-        bs0, sum0, max0 = runner.run(flat[idx], bottleneck[idx])
-        assert (bs0 >= 0).all()
-        bound = sum0.astype(np.float64) + (flat_G[idx] - 1).astype(np.float64) * max0.astype(np.float64)
-        hi = np.nextafter((bound * (1.0 + 1e-5) / flat_G[idx]).astype(np.float32), np.float32(np.inf))
+        cost0, _, sum0 = runner.evaluate(flat[idx], bottleneck[idx], flat_G[idx])
+        assert np.isfinite(cost0).all()
+        hi = np.nextafter((cost0 * (1.0 + 1e-5) / flat_G[idx]).astype(np.float32), np.float32(np.inf))
         hi = np.maximum(hi, np.nextafter(bottleneck[idx], np.float32(np.inf)))
         for k, i in enumerate(idx):
             windows[i] = _Window(runner, int(flat[i]), int(flat_G[i]), bottleneck[i], float(sum0[k]))
@@ -446,7 +511,7 @@ def inter_stage_tune_batch(
 
     # Speculative batches + sequential replay (see the module docstring).
     while True:
-        req_g, req_t, req_span = [], [], []
+        req_g, req_t, req_G, req_span = [], [], [], []
         for t, ch in enumerate(chains):
             scans = ch["scans"]
             best_cost, best_G, best_t = ch["best"]
@@ -467,43 +532,36 @@ def inter_stage_tune_batch(
                 if b > a:
                     req_g.append(np.full(b - a, rows[t, i], dtype=np.int32))
                     req_t.append(sc.tmax[a:b])
+                    req_G.append(np.full(b - a, sc.G, dtype=np.int64))
                     req_span.append((t, i, b - a))
         if all(ch["current"] == len(ch["scans"]) for ch in chains):
             break
         if not req_span:
             raise RuntimeError("inter-stage scan made no progress")  # cannot happen: guards a hang
-        bs, bsum, smax = runner.run(np.concatenate(req_g), np.concatenate(req_t))
+        cost, _, _ = runner.evaluate(np.concatenate(req_g), np.concatenate(req_t), np.concatenate(req_G))
         off = 0
         for t, i, n in req_span:
-            chains[t]["scans"][i].add(bs[off:off + n], bsum[off:off + n], smax[off:off + n])
+            chains[t]["scans"][i].add(cost[off:off + n])
             off += n
     t_2 = time.perf_counter()
+    if stats is not None:
+        stats["dp_thresholds_s"] = stats.get("dp_thresholds_s", 0.0) + (t_1 - t_0)
+        stats["dp_scan_s"] = stats.get("dp_scan_s", 0.0) + (t_2 - t_1)
+    return [ch["best"] for ch in chains]
 
-    # Back-pointers of each winning (G, t_max) run (inter_tuning.py:341-355), one launch.
-    winners = [t for t, ch in enumerate(chains) if ch["best"][1] is not None]
-    back = {}
-    if winners:
-        w_rows = np.array([t * n_g + g_index[chains[t]["best"][1]] for t in winners], dtype=np.int32)
-        w_tmax = np.array([chains[t]["best"][2] for t in winners], dtype=np.float32)
-        best_s, _, _, argmin = runner.run(w_rows, w_tmax, want_argmin=True)
-        back = {t: (int(best_s[i]), argmin[i]) for i, t in enumerate(winners)}
+
+def _solutions(runner: _DpRunner, results_list, bests, n_g, g_index, q_index, num_layers, slot):
+    """Back-pointers of each winning (G, t_max) run (inter_tuning.py:341-355) and the stage
+    strategies that go with them."""
     out = []
-    for t, ch in enumerate(chains):
-        best_cost, best_G, best_t = ch["best"]
+    for t, (best_cost, best_G, best_t) in enumerate(bests):
         if best_G is None:
             out.append((float("inf"), None))
             continue
         r = results_list[t]
         g = g_index[best_G]
-        cs, argmin = back[t]
-        cl, cd = 0, num_devices
-        inter = []
-        while cs > 0 and cl < num_layers and cd > 0:
-            end, n, m, ckpt = (int(v) for v in argmin[cs, cl, cd])
-            assert end != -1
-            inter.append(((cl, end), (n, m), ckpt))
-            cs, cl, cd = cs - 1, end + 1, cd - n * m
-        assert cs == 0 and cl == num_layers and cd == 0
+        total, inter = runner.partition(t * n_g + g, best_t, best_G)
+        assert total == best_cost
         solution = [best_G, []]
         for i, ((l0, l1), (n, m), ckpt) in enumerate(inter):
             row = get_solution_from_intra_stage_tuner_output(
@@ -512,10 +570,54 @@ def inter_stage_tune_batch(
             row[:6] = [int(x) for x in row[:6]]
             solution[1].append((((l0, l1), (n, m), ckpt, 0), tuple(row)))
         out.append((best_cost, solution))
+    return out
+
+
+def inter_stage_tune_batch(
+    num_layers: int,
+    num_devices: int,
+    device_mesh_candidates: List[Tuple[int, int]],
+    gradient_accumulation_steps_candidates: List[int],
+    results_list: List[IntraStageTunerOutput],
+    slot: int = 0,
+    stats: Optional[dict] = None,
+    uniform_device: Optional[dict] = None,
+):
+    """``inter_stage_tune`` for several intra-stage results at once (the tensor-parallel
+    candidates of one ``tune`` call).  Each entry is searched exactly as if it were alone (its
+    own running best, its own stop rule); only the launches are shared.  Returns a list of
+    ``(best_cost, best_solution)``.  ``uniform_device`` (``num_nodes``, ``num_gpus_per_node``,
+    ``ckpt_tuning``) selects the recurrence of inter_tuning_uniform_device.py instead."""
+    for r in results_list:
+        if not isinstance(r, IntraStageTunerOutput):
+            raise TypeError(
+                f"intra_stage_results must be an instance of IntraStageTunerOutput, got {type(r)}"
+            )
+    if not _same_batch(results_list):
+        out = []
+        for r in results_list:
+            one = r if r.batch is r.device else IntraStageTunerOutput(
+                r.gradient_accumulation_steps_candidates, r.device_mesh_candidates, r.device,
+                r.spaces, r.sample_slots)
+            out += inter_stage_tune_batch(num_layers, num_devices, device_mesh_candidates,
+                                          gradient_accumulation_steps_candidates, [one], slot, stats,
+                                          uniform_device)
+        return out
+    t_start = time.perf_counter()
+    first = results_list[0]
+    runner = _DpRunner(first, num_layers, num_devices, device_mesh_candidates, slot, uniform_device)
+    n_g = len(first.gradient_accumulation_steps_candidates)
+    g_index = {G: i for i, G in enumerate(first.gradient_accumulation_steps_candidates)}
+    q_index = {q: i for i, q in enumerate(first.device_mesh_candidates)}
+    Gs = list(gradient_accumulation_steps_candidates)
+    # table row of (instance, G)
+    rows = np.array([[t * n_g + g_index[G] for G in Gs] for t in range(len(results_list))], dtype=np.int32)
+    t_0 = time.perf_counter()
+    bests = _search(runner, rows, Gs, stats)
+    t_2 = time.perf_counter()
+    out = _solutions(runner, results_list, bests, n_g, g_index, q_index, num_layers, slot)
     if stats is not None:
         stats["dp_setup_s"] = stats.get("dp_setup_s", 0.0) + (t_0 - t_start)
-        stats["dp_thresholds_s"] = stats.get("dp_thresholds_s", 0.0) + (t_1 - t_0)
-        stats["dp_scan_s"] = stats.get("dp_scan_s", 0.0) + (t_2 - t_1)
         stats["dp_backtrack_s"] = stats.get("dp_backtrack_s", 0.0) + (time.perf_counter() - t_2)
         stats["dp_launches"] = stats.get("dp_launches", 0) + runner.launches
         stats["dp_window_fetches"] = stats.get("dp_window_fetches", 0) + runner.fetches

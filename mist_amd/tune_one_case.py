@@ -7,13 +7,13 @@ evaluation running on the GPU.  Differences, all forced by what the path needs h
 * the three traced ``LayerInfo`` objects are replaced by ``LayerTables`` (closed-form tables);
 * hydra / omegaconf are not used: ``main`` takes ``--config <yaml>`` plus ``key=value``
   overrides, and the YAML written is produced with PyYAML;
-* ``tuning_granularity``: ``inter-stage`` (the DP), ``uniform-pp``,
-  ``uniform-pp-simple-heuristic-mem-opt`` and ``no-pp`` are implemented.  The reference's
-  ``inter-stage`` and ``no-pp`` branches call ``intra_stage_tune`` without the required
-  ``tp_size`` and read cost fields that no longer exist; here they loop the tensor-parallel
-  candidates like the working branches (:199-203) and use the stable/delta adapter.
-  ``uniform-device-pp`` and ``uniform-device-pp-mip`` (external MILP solver) raise
-  ``NotImplementedError``.
+* ``tuning_granularity``: ``inter-stage`` (the per-mesh DP), ``uniform-device-pp`` (the DP with
+  one uniform mesh per stage count), ``uniform-pp``, ``uniform-pp-simple-heuristic-mem-opt`` and
+  ``no-pp`` are implemented.  The reference's ``inter-stage``, ``uniform-device-pp`` and ``no-pp``
+  branches call ``intra_stage_tune`` without the required ``tp_size`` and read cost fields that
+  no longer exist; here they cover the tensor-parallel candidates like the working branches
+  (:199-203), use the stable/delta adapter and take ``tuning.sample_size`` samples (slot 0).
+  ``uniform-device-pp-mip`` (external MILP solver) raises ``NotImplementedError``.
 """
 from __future__ import annotations
 
@@ -32,6 +32,7 @@ import yaml
 from .config import OFFLOADING_RATIO_CANDIDATES, MistConfig, tp_candidates
 from .inter_tuning import inter_stage_tune, inter_stage_tune_batch
 from .inter_tuning_uniform import inter_stage_tune as inter_stage_tune_uniform
+from .inter_tuning_uniform_device import inter_stage_tune_batch_uniform_device
 from .intra_tuning import SAMPLE_SIZE, IntraStageTuner, intra_stage_tune
 from .layer_tables import LayerTables
 from .search_space import _get_device_mesh_candidates, _get_grad_accumu_steps_candidates
@@ -103,7 +104,8 @@ class PreparedSearch:
         model, hw, tuning = mist_config.model, mist_config.hardware, mist_config.tuning
         self.config = mist_config
         self.granularity = tuning.tuning_granularity
-        if self.granularity not in ("uniform-pp", "uniform-pp-simple-heuristic-mem-opt", "inter-stage"):
+        if self.granularity not in ("uniform-pp", "uniform-pp-simple-heuristic-mem-opt", "inter-stage",
+                                    "uniform-device-pp"):
             raise ValueError(f"PreparedSearch does not cover '{self.granularity}'")
         self.tables = LayerTables(mist_config)
         self.meshes = _get_device_mesh_candidates(hw.num_nodes, hw.num_gpus_per_node, contiguous_inter_node=False)
@@ -111,7 +113,8 @@ class PreparedSearch:
         self.L = model.num_hidden_layers
         # The reference forwards tuning.sample_size only on its MIP branch; the uniform
         # branch runs with the default of 30 and reads sample 0 (:206-217).
-        sample_size = tuning.sample_size if self.granularity == "inter-stage" else SAMPLE_SIZE
+        sample_size = (tuning.sample_size if self.granularity in ("inter-stage", "uniform-device-pp")
+                       else SAMPLE_SIZE)
         # All tensor-parallel candidates go through one batch of launches.
         self.tuner = IntraStageTuner(self.tables, self.L, self.meshes, self.Gs,
                                      tp_candidates(mist_config), mist_config,
@@ -141,6 +144,11 @@ class PreparedSearch:
             outcomes = inter_stage_tune_batch(
                 self.L, hw.num_nodes * hw.num_gpus_per_node, self.meshes, self.Gs, results, slot=0, stats=stats
             )
+        elif self.granularity == "uniform-device-pp":
+            outcomes = inter_stage_tune_batch_uniform_device(
+                self.L, hw.num_nodes, hw.num_gpus_per_node, self.meshes, self.Gs, results,
+                self.config, slot=0, stats=stats,
+            )
         else:
             outcomes = [
                 inter_stage_tune_uniform(self.L, hw.num_nodes, hw.num_gpus_per_node, self.Gs, r, self.config)
@@ -168,7 +176,7 @@ def tune(mist_config: MistConfig, device: str = "cuda:0", stats: Optional[dict] 
 
     if granularity == "no-pp":
         best_cost, best_solution = _no_pp(mist_config, LayerTables(mist_config), device, stats)
-    elif granularity in ("uniform-pp", "inter-stage"):
+    elif granularity in ("uniform-pp", "inter-stage", "uniform-device-pp"):
         best_cost, best_solution = PreparedSearch(mist_config, device).run(stats)
     elif granularity == "uniform-pp-simple-heuristic-mem-opt":
         # tune_one_case.py:258-262: sweep a fixed optimizer-offload ratio, activation offload off.
@@ -180,10 +188,10 @@ def tune(mist_config: MistConfig, device: str = "cuda:0", stats: Optional[dict] 
             cost, solution = PreparedSearch(MistConfig(raw), device).run(stats)
             if cost < best_cost:
                 best_cost, best_solution = cost, solution
-    elif granularity in ("uniform-device-pp", "uniform-device-pp-mip"):
+    elif granularity == "uniform-device-pp-mip":
         raise NotImplementedError(
             f"tuning_granularity '{granularity}' is not part of the GPU search path "
-            "(uniform-device DP / external MILP solver)"
+            "(it hands the stage tables to an external MILP solver)"
         )
     else:
         raise ValueError(f"Unknown tuning granularity: {granularity}")

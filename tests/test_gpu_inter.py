@@ -203,3 +203,91 @@ def test_full_size_dp_matches_c_oracle_on_gpt7b_tables():
             costs.append(tabs[0][q, p, l - 1, ckpt])
     want_cost, want_sol = dp_impl_c(np.float32(max(costs)), L, D, meshes, Gs[g], *tabs)
     assert want_cost == best_cost and want_sol == inter
+
+
+@pytest.mark.parametrize("ckpt_tuning", [True, False])
+@pytest.mark.parametrize("L,num_nodes,gpn,P1,quantum", [(6, 1, 4, 7, None), (7, 2, 4, 4, 0.125), (9, 2, 2, 10, 0.25)])
+def test_uniform_device_dp_kernel_matches_oracle(L, num_nodes, gpn, P1, quantum, ckpt_tuning):
+    """The free-device / per-stage ckpt-rule mode of the DP kernel, one launch family per
+    admissible stage count, against the literal restatement of
+    inter_tuning_uniform_device.py:276-441 (total over all S, partition, ties)."""
+    import torch
+    from mist_amd import _lib
+    from oracle.inter_uniform_device import dp_impl as ud_dp, uniform_device_mesh_partition as udmp
+
+    rng = np.random.default_rng(L * 10 + gpn)
+    meshes = [(1, 2 ** i) for i in range(4) if 2 ** i <= gpn]
+    meshes += [(2 ** j, gpn) for j in range(1, 4) if 2 ** j <= num_nodes]
+    tabs = _random_tables(rng, len(meshes), P1, L, quantum=quantum)
+    lib = _lib.load()
+    dev = [torch.from_numpy(t).cuda() for t in tabs]
+    dev += [torch.cummin(t, dim=-1).values.contiguous() for t in dev]
+    G = 5
+    tmax = np.sort(rng.uniform(0.1, 1.1, size=16)).astype(np.float32)
+    n = len(tmax)
+    best = [(np.inf, None)] * n
+    for S in range(1, L + 1):
+        mesh = udmp(S, num_nodes, gpn)
+        if mesh is None:
+            continue
+        q = meshes.index(mesh)
+        shape = np.zeros(1, dtype=_lib.DP_SHAPE_DTYPE)
+        shape["num_layers"], shape["num_devices"], shape["num_mesh"], shape["p_dim"] = L, 0, 1, P1
+        shape["max_stages"] = min(S, P1, L)
+        shape["ckpt_rule"] = _lib.DP_CKPT_STAGE if ckpt_tuning else _lib.DP_CKPT_ALL
+        shape["free_devices"] = 1
+        shape["mesh_n"][0, 0], shape["mesh_m"][0, 0] = mesh
+        per_q = [t[0].numel() for t in dev[:4]]
+        costs = _lib.DpCosts(*[t.data_ptr() + 4 * q * per_q[v % 4] for v, t in enumerate(dev)])
+        d_t = torch.from_numpy(tmax).cuda()
+        d_g = torch.zeros(n, dtype=torch.int32).cuda()
+        d_s = torch.empty(n, dtype=torch.int32).cuda()
+        d_sum = torch.empty(n, dtype=torch.float32).cuda()
+        d_max = torch.empty(n, dtype=torch.float32).cuda()
+        Sm = int(shape["max_stages"][0])
+        scr = torch.empty(lib.mist_dp_scratch_floats(ctypes.c_void_p(shape.ctypes.data), n), dtype=torch.float32).cuda()
+        arg = torch.full((n, Sm + 1, L + 1, 1, 4), -1, dtype=torch.int32).cuda()
+        _lib.check(lib.mist_dp_run(
+            ctypes.c_void_p(shape.ctypes.data), ctypes.byref(costs), d_t.data_ptr(), d_g.data_ptr(), n, 0,
+            d_s.data_ptr(), d_sum.data_ptr(), d_max.data_ptr(), arg.data_ptr(), scr.data_ptr(),
+            ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)), "mist_dp_run")
+        torch.cuda.synchronize()
+        bs, bsum, smax, argmin = d_s.cpu().numpy(), d_sum.cpu().numpy(), d_max.cpu().numpy(), arg.cpu().numpy()
+        for i in range(n):
+            if bs[i] < 0:
+                continue
+            total = float(np.float64(bsum[i]) + np.float64(G - 1) * np.float64(smax[i]))
+            if total < best[i][0]:
+                sol, cs, cl = [], int(bs[i]), 0
+                while cs > 0:
+                    end, nn, mm, ck = (int(v) for v in argmin[i][cs, cl, 0])
+                    sol.append(((cl, end), (nn, mm), ck))
+                    cs, cl = cs - 1, end + 1
+                best[i] = (total, sol)
+    n_feasible = 0
+    for i, t in enumerate(tmax):
+        want = ud_dp(t, L, num_nodes, gpn, meshes, G, *tabs, ckpt_tuning=ckpt_tuning)
+        assert best[i] == want, (i, t)
+        n_feasible += want[1] is not None
+    assert n_feasible > 0
+
+
+@pytest.mark.parametrize(
+    "overrides",
+    [
+        dict(hardware__num_nodes=2, hardware__num_gpus_per_node=4, training__global_batch_size=32,
+             hardware__memory_capacity=8.0),
+        dict(hardware__memory_capacity=5.0),
+        dict(hardware__num_nodes=1, hardware__num_gpus_per_node=4, training__global_batch_size=16,
+             hardware__memory_capacity=6.0, tuning__activation_checkpointing_tuning_enabled=False),
+    ],
+)
+def test_uniform_device_tune_end_to_end_matches_oracle(overrides):
+    from mist_amd.tune_one_case import tune
+    from oracle.tune import tune as oracle_tune
+
+    cfg, tables = tiny_plan(1, layers=6, tuning__tuning_granularity="uniform-device-pp", **overrides)
+    got = tune(cfg)
+    want = oracle_tune(cfg, tables)
+    assert got == want
+    assert want[1] is not None

@@ -157,7 +157,7 @@ def test_best_solution_yaml_format():
 def test_unsupported_granularities_raise():
     from mist_amd.tune_one_case import tune
 
-    for gran in ("uniform-device-pp", "uniform-device-pp-mip"):
+    for gran in ("uniform-device-pp-mip",):
         cfg, _ = load_plan(1, tuning__tuning_granularity=gran)
         with pytest.raises(NotImplementedError):
             tune(cfg)

@@ -190,3 +190,87 @@ def test_uniform_search_equals_brute_force():
     assert sum(l1 - l0 + 1 for ((l0, l1), _, _, _), _ in sol[1]) == L
     for (_, mesh, _, policy), row in sol[1]:
         assert policy == 0 and row[0] * row[1] * G == 16 and row[1] * row[2] == mesh[0] * mesh[1]
+
+
+def _brute_force_uniform_device(t_max, L, num_nodes, gpn, meshes, tabs, ckpt_tuning, S):
+    """min float32 suffix-accumulated sum over every split into s <= S stages and every ckpt
+    choice, all stages on the uniform mesh of S stages; also the best s (first on ties)."""
+    from oracle.inter_uniform_device import uniform_device_mesh_partition as udmp
+
+    q = meshes.index(udmp(S, num_nodes, gpn))
+    best_per_s = []
+    for n_stages in range(1, S + 1):
+        best = np.float32(np.inf)
+        for cuts in itertools.combinations(range(1, L), n_stages - 1):
+            bounds = [0, *cuts, L]
+            spans = [(bounds[a], bounds[a + 1] - 1) for a in range(n_stages)]
+            options = []
+            for a, (k, i) in enumerate(spans):
+                l = i - k + 1
+                js = range(l + 1) if ckpt_tuning else [l]
+                cs = [_stage_cost(tabs, L, n_stages - a, k, i, q, j) for j in js]
+                options.append([c for c in cs if c <= t_max])
+            if any(len(o) == 0 for o in options):
+                continue
+            for combo in itertools.product(*options):
+                acc = np.float32(0)
+                for cst in reversed(combo):
+                    acc = np.float32(cst + acc)
+                best = min(best, acc)
+        best_per_s.append(best)
+    return best_per_s
+
+
+@pytest.mark.parametrize("ckpt_tuning", [True, False])
+@pytest.mark.parametrize("L,num_nodes,gpn,seed", [(4, 1, 4, 0), (5, 2, 2, 1), (4, 2, 4, 2)])
+def test_uniform_device_dp_equals_brute_force(L, num_nodes, gpn, seed, ckpt_tuning):
+    from oracle.inter_uniform_device import dp_impl as ud_dp, uniform_device_mesh_partition as udmp
+
+    rng = np.random.default_rng(100 + seed)
+    meshes = [(1, 2 ** i) for i in range(gpn.bit_length()) if 2 ** i <= gpn]
+    meshes += [(2 ** j, gpn) for j in range(1, num_nodes.bit_length()) if 2 ** j <= num_nodes]
+    tabs = _tables(rng, len(meshes), L + 1, L, quantum=0.125 if seed % 2 else None)
+    G, hits = 4, 0
+    for t in (0.3, 0.55, 0.8, 1.1):
+        t32 = np.float32(t)
+        cost, sol = ud_dp(t, L, num_nodes, gpn, meshes, G, *tabs, ckpt_tuning=ckpt_tuning)
+        # candidates per S: the minimum sum over s <= S (first s on ties); the stage maximum that
+        # goes with it is the DP's own, so the total is checked on the returned partition
+        sums = {}
+        for S in range(1, L + 1):
+            if udmp(S, num_nodes, gpn) is None:
+                continue
+            per_s = _brute_force_uniform_device(t32, L, num_nodes, gpn, meshes, tabs, ckpt_tuning, S)
+            if np.isfinite(min(per_s)):
+                sums[S] = min(per_s)
+        if sol is None:
+            assert not sums
+            continue
+        hits += 1
+        mesh = sol[0][1]
+        assert all(m == mesh for _, m, _ in sol) and sol[0][0][0] == 0 and sol[-1][0][1] == L - 1
+        q = meshes.index(mesh)
+        stage = [_stage_cost(tabs, L, len(sol) - a, l0, l1, q, ck) for a, ((l0, l1), _, ck) in enumerate(sol)]
+        assert all(c <= t32 for c in stage)
+        if not ckpt_tuning:
+            assert all(ck == l1 - l0 + 1 for (l0, l1), _, ck in sol)
+        acc = np.float32(0)
+        for c in reversed(stage):
+            acc = np.float32(c + acc)
+        assert cost == float(np.float64(acc) + (G - 1) * np.float64(max(stage)))
+        # the partition's sum is the optimum (over s <= S) of a stage count S with that mesh
+        S_of_mesh = [S for S in sums if udmp(S, num_nodes, gpn) == mesh]
+        assert any(acc == sums[S] for S in S_of_mesh)
+    assert hits > 0
+
+
+def test_uniform_device_mesh_closed_form():
+    from oracle.inter_uniform_device import uniform_device_mesh_partition as udmp
+
+    assert udmp(1, 4, 8) == (4, 8) and udmp(2, 4, 8) == (2, 8) and udmp(4, 4, 8) == (1, 8)
+    assert udmp(8, 4, 8) == (1, 4) and udmp(32, 4, 8) == (1, 1)
+    assert udmp(3, 4, 8) is None and udmp(64, 4, 8) is None and udmp(6, 2, 4) is None
+    for S in range(1, 40):
+        got = udmp(S, 4, 8)
+        if got is not None:
+            assert got[0] * got[1] * S == 32  # the stages share all devices evenly

@@ -139,6 +139,7 @@ int mist_sizeof_group(void);
 int mist_reduce_p_tile(void); /* MIST_P_TILE the library was built with */
 int mist_reduce_lc_tile(void); /* MIST_LC_TILE the library was built with */
 int mist_reduce_scout_split(void); /* scout workgroups per (group, (l, c) tile, p tile) */
+int mist_terms_block_rows(void); /* candidate rows per workgroup of mist_row_terms */
 int mist_reduce_stage_rows(void); /* rows per LDS stage; rows_per_chunk must be a multiple */
 
 /* Row-invariant terms of every candidate row: decodes the row index, evaluates the alpha-beta
@@ -147,7 +148,8 @@ int mist_reduce_stage_rows(void); /* rows per LDS stage; rows_per_chunk must be 
  * Replaces batched_stage_analyze lines 1144-2162 of mist/analyzer/batched_module_analyzer.py
  * (with predict_gpu_gpu_comm_latency / predict_cpu_gpu_comm_latency /
  * interference_estimate_for_one_group of mist/tools/optimize.py:201-303,459-470,1012-1122).
- * d_block_prefix[n_groups+1]: first workgroup of each group, 256 rows per workgroup.
+ * d_block_prefix[n_groups+1]: first workgroup of each group, mist_terms_block_rows() rows per
+ * workgroup.
  * d_row_terms: [total_rows][MIST_ROW_TERMS] float64.  Within a group the workspace is ordered
  *   position = ((par * n_ao + ao) * n_oo + oo) * n_pair + pair
  * (rows of similar memory footprint next to each other, which the reduce kernel's per-stage

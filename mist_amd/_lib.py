@@ -21,7 +21,7 @@ P_TILE = 32  # replaced by the library's own value in load()
 SLOTS = 2 * P_TILE + 2
 SCOUT_SPLIT = 4  # replaced by the library's own value in load()
 STAGE_ROWS = 64  # replaced by the library's own value in load()
-TERMS_BLOCK = 256
+TERMS_BLOCK = 128  # replaced by the library's own value in load()
 MAX_MESH = 16
 DP_CKPT_TAIL, DP_CKPT_STAGE, DP_CKPT_ALL = 0, 1, 2
 DP_THRESHOLD, DP_BOTTLENECK = 0, 1
@@ -108,6 +108,7 @@ _SIGNATURES = {
     "mist_reduce_p_tile": (ctypes.c_int, []),
     "mist_reduce_stage_rows": (ctypes.c_int, []),
     "mist_reduce_lc_tile": (ctypes.c_int, []),
+    "mist_terms_block_rows": (ctypes.c_int, []),
     "mist_reduce_scout_split": (ctypes.c_int, []),
     "mist_row_terms": (ctypes.c_int, [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, _VP]),
     "mist_eval_reduce": (
@@ -209,7 +210,8 @@ def load():
         raise MistLibraryError(
             f"MistGroupDesc layout mismatch: C {lib.mist_sizeof_group()} vs numpy {GROUP_DTYPE.itemsize}"
         )
-    global P_TILE, SLOTS, STAGE_ROWS, LC_TILE, SCOUT_SPLIT
+    global P_TILE, SLOTS, STAGE_ROWS, LC_TILE, SCOUT_SPLIT, TERMS_BLOCK
+    TERMS_BLOCK = lib.mist_terms_block_rows()
     SCOUT_SPLIT = lib.mist_reduce_scout_split()
     LC_TILE = lib.mist_reduce_lc_tile()
     STAGE_ROWS = lib.mist_reduce_stage_rows()

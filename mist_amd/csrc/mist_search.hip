@@ -34,7 +34,7 @@ namespace {
 
 using mist::fail;
 
-constexpr int kTermsBlock = 256;  // rows per workgroup of the row-term kernel
+constexpr int kTermsBlock = 128;  // rows per workgroup of the row-term kernel
 constexpr int kStageRows = 64;    // rows staged through LDS per step of the reduce kernel
 constexpr int kSlots = 2 * MIST_P_TILE + 2;  // per-thread running minima: base, with_pre, post, no_pp
 
@@ -91,6 +91,12 @@ __constant__ unsigned char kMaskBits[11] = {
     0x3, 0x5, 0x9, 0x6, 0xA, 0xC,
 };
 
+// Index into kMaskBits of the mask equal to a non-zero pattern, -1 for patterns with fewer than
+// two bits.
+__constant__ signed char kMaskOfPattern[16] = {
+    -1, -1, -1, 5, -1, 6, 8, 1, -1, 7, 9, 2, 10, 3, 4, 0,
+};
+
 struct Interference {
   const double (*factor)[4];
 
@@ -99,13 +105,18 @@ struct Interference {
   __device__ __noinline__ double operator()(double exec, double g2g, double g2c, double c2g) const {
     double x0 = exec, x1 = g2g, x2 = c2g, x3 = g2c;
     double out = 0.0;
+    // The reference tries the 11 masks in order and applies the one equal to the non-zero
+    // pattern of X.  A pattern equals at most one mask, and after a peel the pattern has fewer
+    // bits, i.e. it can only equal a mask further down the list (4-way, then 3-way, then
+    // 2-way).  So the mask to apply is looked up from the pattern: at most three rounds.
 #pragma unroll 1
-    for (int m = 0; m < 11; ++m) {
+    for (int round = 0; round < 3; ++round) {
       // "not isclose(x, 0)" with numpy's default tolerances: |x| > 1e-8 (NaN counts as non-zero).
       const unsigned nz = (!(fabs(x0) <= 1e-8) ? 1u : 0u) | (!(fabs(x1) <= 1e-8) ? 2u : 0u) |
                           (!(fabs(x2) <= 1e-8) ? 4u : 0u) | (!(fabs(x3) <= 1e-8) ? 8u : 0u);
-      const unsigned mask = kMaskBits[m];
-      if (nz != mask) continue;
+      const int m = kMaskOfPattern[nz];
+      if (m < 0) break;  // fewer than two busy resources: nothing overlaps
+      const unsigned mask = nz;
       const double f0 = factor[m][0], f1 = factor[m][1], f2 = factor[m][2], f3 = factor[m][3];
       const double s0 = x0 * f0, s1 = x1 * f1, s2 = x2 * f2, s3 = x3 * f3;
       double ov = INFINITY;
@@ -126,6 +137,16 @@ struct Interference {
 struct Family {
   double layer, first, last, extra_pre, extra_post;
 };
+
+__device__ __forceinline__ Family pick_family(bool second, const Family &a, const Family &b) {
+  Family r;
+  r.layer = second ? b.layer : a.layer;
+  r.first = second ? b.first : a.first;
+  r.last = second ? b.last : a.last;
+  r.extra_pre = second ? b.extra_pre : a.extra_pre;
+  r.extra_post = second ? b.extra_post : a.extra_post;
+  return r;
+}
 
 __device__ __forceinline__ const MistGroupDesc *find_group(const MistGroupDesc *groups,
                                                            const int32_t *prefix, int n_groups,
@@ -184,8 +205,21 @@ __global__ __launch_bounds__(kTermsBlock) void row_terms_kernel(
     const int32_t *__restrict__ block_prefix, double *__restrict__ row_terms) {
   int local_block;
   const MistGroupDesc *g = find_group(groups, block_prefix, n_groups, blockIdx.x, &local_block);
-  const int64_t row = (int64_t)local_block * kTermsBlock + threadIdx.x;  // workspace position
-  if (row >= g->n_rows) return;
+  // The block's terms are assembled in LDS (row pitch 35 doubles: conflict-free) and written out
+  // as one contiguous, fully coalesced range; a lane writing its own 272-byte row would touch
+  // 34 partial cache lines.
+  __shared__ double lds_out[kTermsBlock * (MIST_ROW_TERMS + 1)];
+  // Tables indexed at run time are read from LDS: indexing the by-value kernel argument would
+  // make every lane keep a private copy of the whole struct in scratch memory.
+  __shared__ double lds_factor[11][4];
+  __shared__ double lds_gpu_gpu[32];
+  if (threadIdx.x < 44) lds_factor[threadIdx.x / 4][threadIdx.x % 4] = prob.interf_factor[threadIdx.x / 4][threadIdx.x % 4];
+  if (threadIdx.x >= 64 && threadIdx.x < 96) lds_gpu_gpu[threadIdx.x - 64] = prob.gpu_gpu[threadIdx.x - 64];
+  __syncthreads();
+  const int64_t block_first = (int64_t)local_block * kTermsBlock;
+  const int rows_here = (int)min((int64_t)kTermsBlock, g->n_rows - block_first);
+  // Lanes past the end recompute the last row (no divergent barrier); their result is dropped.
+  const int64_t row = block_first + min((int)threadIdx.x, rows_here - 1);  // workspace position
 
   // ---- index decomposition (batched_module_analyzer.py:490-534) ----
   const RowParts parts = parts_of_position(g, row);
@@ -245,11 +279,11 @@ __global__ __launch_bounds__(kTermsBlock) void row_terms_kernel(
   const double n_nodes = (double)g->num_nodes;
   const double dp_inter = dp > n_nodes ? n_nodes : dp;
   const double dp_intra = dp > n_nodes ? floor(dp / n_nodes) : 1.0;
-  const double AG_w = gpu_gpu_latency(prob.gpu_gpu, W, dp_inter, dp_intra, 1.0);
-  const double RS_g = gpu_gpu_latency(prob.gpu_gpu, Gr, dp_inter, dp_intra, 1.1);
-  const double AR_g = gpu_gpu_latency(prob.gpu_gpu, Gr, dp_inter, dp_intra, 2.1);
+  const double AG_w = gpu_gpu_latency(lds_gpu_gpu, W, dp_inter, dp_intra, 1.0);
+  const double RS_g = gpu_gpu_latency(lds_gpu_gpu, Gr, dp_inter, dp_intra, 1.1);
+  const double AR_g = gpu_gpu_latency(lds_gpu_gpu, Gr, dp_inter, dp_intra, 2.1);
 
-  const Interference I{prob.interf_factor};
+  const Interference I{lds_factor};
   const bool adv = prob.adv_first_block != 0;
 
   // ---- forward phases (:1432-1621): index 0 = first micro-batch, 1 = not first ----
@@ -305,11 +339,14 @@ __global__ __launch_bounds__(kTermsBlock) void row_terms_kernel(
   }
 
   // ---- stable / delta families (:1910-2028) ----
-  double *t = row_terms + (g->row_offset + row) * MIST_ROW_TERMS;
+  double *t = lds_out + threadIdx.x * (MIST_ROW_TERMS + 1);
   const int st = g->grad_accum == 1 ? 0 : 1;  // phase index that forms the stable part
 #pragma unroll
   for (int k = 0; k < 2; ++k) {
-    const Family &f = fwd[st][k], &w = bwd[st][k];
+    // selected field by field: indexing the arrays with a run-time phase would put them in
+    // scratch memory
+    const Family f = pick_family(st == 1, fwd[0][k], fwd[1][k]);
+    const Family w = pick_family(st == 1, bwd[0][k], bwd[1][k]);
     const double s_layer = f.layer + w.layer;
     const double s_first = f.extra_pre + w.extra_post + f.first + w.first;
     const double s_last = f.extra_post + w.extra_pre + f.last + w.last;
@@ -357,6 +394,14 @@ __global__ __launch_bounds__(kTermsBlock) void row_terms_kernel(
   t[MIST_T_NRS_NOCK] = fmax(g->post_rs - ovg_nock, 0.0);
   t[MIST_T_OPB] = fmax(g->post_bwd - bwd[1][1].extra_pre, 0.0);
   t[MIST_T_RD] = raw_nock - S_nock;
+
+  __syncthreads();
+  double2 *__restrict__ dst =
+      reinterpret_cast<double2 *>(row_terms + (g->row_offset + block_first) * MIST_ROW_TERMS);
+  for (int i = threadIdx.x; i < rows_here * (MIST_ROW_TERMS / 2); i += kTermsBlock) {
+    const int at = (i / (MIST_ROW_TERMS / 2)) * (MIST_ROW_TERMS + 1) + 2 * (i % (MIST_ROW_TERMS / 2));
+    dst[i] = make_double2(lds_out[at], lds_out[at + 1]);
+  }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -1146,6 +1191,7 @@ int mist_row_terms(const MistProblem *problem, const MistGroupDesc *d_groups, in
 
 int mist_reduce_stage_rows(void) { return kStageRows; }
 int mist_reduce_lc_tile(void) { return MIST_LC_TILE; }
+int mist_terms_block_rows(void) { return kTermsBlock; }
 int mist_reduce_scout_split(void) { return kScoutSplit; }
 
 int mist_eval_reduce(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,

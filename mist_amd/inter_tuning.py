@@ -243,29 +243,32 @@ class _DpRunner:
             b = np.minimum(b, bott)
         return b
 
-    def partition(self, g: int, tmax: np.float32, G: int):
-        """``(stage count, [((l0, l1), (n, m), ckpt), ...])`` of the winning family of one
-        instance, from its back-pointers (inter_tuning.py:341-355)."""
-        best = (np.inf, None)
+    def partitions(self, g_index: np.ndarray, tmax: np.ndarray, G: np.ndarray):
+        """Per instance ``(total, [((l0, l1), (n, m), ckpt), ...])`` of its winning family, from
+        the back-pointers (inter_tuning.py:341-355); one launch batch per family."""
+        n = len(tmax)
+        best = [(np.inf, None)] * n
         for fam in self.families:
-            bs, bsum, smax, argmin = self.run(np.array([g], dtype=np.int32),
-                                              np.array([tmax], dtype=np.float32),
-                                              want_argmin=True, family=fam)
-            total = float(self._total(bs, bsum, smax, G)[0])
-            if total < best[0]:
-                best = (total, (fam, int(bs[0]), argmin[0]))
-        assert best[1] is not None
-        fam, cs, argmin = best[1]
-        cl, cd, inter = 0, fam.D, []
-        while cs > 0 and cl < fam.L and (cd > 0 or not fam.consumes_devices):
-            end, n, m, ckpt = (int(v) for v in argmin[cs, cl, cd])
-            assert end != -1
-            inter.append(((cl, end), (n, m), ckpt))
-            cs, cl = cs - 1, end + 1
-            if fam.consumes_devices:
-                cd -= n * m
-        assert cs == 0 and cl == fam.L and cd == 0
-        return best[0], inter
+            bs, bsum, smax, argmin = self.run(g_index, tmax, want_argmin=True, family=fam)
+            total = self._total(bs, bsum, smax, G)
+            for i in range(n):
+                if total[i] < best[i][0]:
+                    best[i] = (float(total[i]), (fam, int(bs[i]), argmin[i]))
+        out = []
+        for total, found in best:
+            assert found is not None
+            fam, cs, argmin = found
+            cl, cd, inter = 0, fam.D, []
+            while cs > 0 and cl < fam.L and (cd > 0 or not fam.consumes_devices):
+                end, n_, m_, ckpt = (int(v) for v in argmin[cs, cl, cd])
+                assert end != -1
+                inter.append(((cl, end), (n_, m_), ckpt))
+                cs, cl = cs - 1, end + 1
+                if fam.consumes_devices:
+                    cd -= n_ * m_
+            assert cs == 0 and cl == fam.L and cd == 0
+            out.append((total, inter))
+        return out
 
 
 def _gap_reached(a: np.ndarray, b: np.ndarray) -> np.ndarray:
@@ -553,6 +556,14 @@ def _search(runner: _DpRunner, rows: np.ndarray, Gs: List[int], stats: Optional[
 def _solutions(runner: _DpRunner, results_list, bests, n_g, g_index, q_index, num_layers, slot):
     """Back-pointers of each winning (G, t_max) run (inter_tuning.py:341-355) and the stage
     strategies that go with them."""
+    winners = [t for t, (_, best_G, _) in enumerate(bests) if best_G is not None]
+    found = {}
+    if winners:
+        parts = runner.partitions(
+            np.array([t * n_g + g_index[bests[t][1]] for t in winners], dtype=np.int32),
+            np.array([bests[t][2] for t in winners], dtype=np.float32),
+            np.array([bests[t][1] for t in winners], dtype=np.int64))
+        found = dict(zip(winners, parts))
     out = []
     for t, (best_cost, best_G, best_t) in enumerate(bests):
         if best_G is None:
@@ -560,7 +571,7 @@ def _solutions(runner: _DpRunner, results_list, bests, n_g, g_index, q_index, nu
             continue
         r = results_list[t]
         g = g_index[best_G]
-        total, inter = runner.partition(t * n_g + g, best_t, best_G)
+        total, inter = found[t]
         assert total == best_cost
         solution = [best_G, []]
         for i, ((l0, l1), (n, m), ckpt) in enumerate(inter):

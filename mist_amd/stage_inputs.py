@@ -128,6 +128,17 @@ def make_problem(
     prob["num_grad_accum"] = num_grad_accum
     prob["num_mesh"] = num_mesh
     prob["adv_first_block"] = 1 if config.enable_advanced_opt_in_first_block else 0
+    bandwidths = np.concatenate([prob["gpu_gpu"][0][0::2], prob["cpu_gpu"][0][:1], prob["gpu_cpu"][0][:1]])
+    offsets = np.concatenate([prob["gpu_gpu"][0][1::2], prob["cpu_gpu"][0][1:], prob["gpu_cpu"][0][1:]])
+    if not (np.all(np.isfinite(bandwidths)) and np.all(bandwidths > 0)):
+        raise ValueError("communication bandwidths (k of every (k, b) pair) must be positive and finite")
+    if not (np.all(np.isfinite(offsets)) and np.all(offsets >= 0)):
+        raise ValueError("communication latencies (b of every (k, b) pair) must be non-negative and finite")
+    factors = prob["interf_factor"][0]
+    if not (np.all(np.isfinite(factors)) and np.all(factors > 0)):
+        raise ValueError("interference factors must be positive and finite")
+    if not (np.isfinite(prob["mem_cap_mb"][0]) and prob["mem_cap_mb"][0] > 0):
+        raise ValueError("memory capacity must be positive and finite")
     return prob
 
 
@@ -260,3 +271,22 @@ class GroupInputBuilder:
             rec["post_ag"] = self._gpu_gpu("all_gather", post_W, pp_dp, n)
             rec["pre_rs"] = self._gpu_gpu("reduce_scatter", pre_G, pp_dp, n)
             rec["post_rs"] = self._gpu_gpu("reduce_scatter", post_G, pp_dp, n)
+        self._validate(rec, space)
+
+    @staticmethod
+    def _validate(rec: np.void, space: SearchSpace) -> None:
+        """The reduce kernel prunes with bounds that rely on every memory and latency input being
+        finite and non-negative and on ratios in [0, 1] (then peaks are monotone in the number of
+        pre-saved micro-batches and in every row term).  Real tables always are; a violation is
+        rejected here instead of silently changing which rows get evaluated."""
+        par = rec["par"][: space.n_par]
+        if not np.all(np.isfinite(par)) or np.any(par < 0):
+            raise ValueError("layer table values must be finite and non-negative")
+        for name in ("wo", "go", "oo", "ao"):
+            v = np.asarray(getattr(space, name), dtype=np.float64)
+            if np.any(~np.isfinite(v)) or np.any(v < 0) or np.any(v > 1):
+                raise ValueError(f"offload ratios '{name}' must lie in [0, 1], got {v}")
+        for name in rec.dtype.names[rec.dtype.names.index("pre_full_w"):]:
+            v = float(rec[name])
+            if not np.isfinite(v) or v < 0:
+                raise ValueError(f"pre/post layer input '{name}' must be finite and non-negative, got {v}")

@@ -295,3 +295,27 @@ def test_threshold_window_equals_full_walk(seed):
         want = full[full >= start]
         got = w.kept[np.searchsorted(w.kept, start, side="left"):]
         assert np.array_equal(got, want), (seed, trial)
+
+
+def test_inputs_outside_the_kernels_preconditions_are_rejected():
+    """Negative or non-finite table values / hardware parameters would break the monotonicity
+    the reduce kernel's exact pruning relies on: the host refuses them before any launch."""
+    from mist_amd.intra_tuning import IntraStageTuner
+    from mist_amd.stage_inputs import make_problem
+
+    cfg, tables = tiny_plan(1, layers=4)
+    with pytest.raises(ValueError, match="interference factors"):
+        make_problem(load_plan(1, hardware__interference_model_params=[0.0] * 28)[0], 4, 2, 1, 1, 1)
+    bad = list(cfg.hardware.gpu_gpu_comm_params)
+    bad[0] = -1.0
+    with pytest.raises(ValueError, match="bandwidths"):
+        make_problem(load_plan(1, hardware__gpu_gpu_comm_params=bad)[0], 4, 2, 1, 1, 1)
+
+    class NegativeTables(type(tables)):
+        def mem_output(self, kind, b, tp):
+            return -super().mem_output(kind, b, tp)
+
+    broken = NegativeTables(cfg)
+    tuner = IntraStageTuner(broken, 4, [(1, 1), (1, 2)], [1, 2, 4, 8], 1, cfg, sample_size=1)
+    with pytest.raises(ValueError, match="non-negative"):
+        tuner.prepare()

@@ -524,13 +524,9 @@ __device__ __forceinline__ void take_min(double &best, int32_t &best_row, bool f
 // kPow2G: the group's G is a power of two, so x / G == x * (1 / G) bit for bit (float32 and
 // float64) and the division leaves the inner loop; other G divide.  kFirstTile: this workgroup
 // owns p = 0 and therefore also the last-stage and single-stage variants.
-#ifndef MIST_ROW_UNROLL
-#define MIST_ROW_UNROLL 4
-#endif
 #ifndef MIST_REDUCE_MIN_WAVES
 #define MIST_REDUCE_MIN_WAVES 2
 #endif
-constexpr int kRowUnroll = MIST_ROW_UNROLL;  // rows whose objective values are computed together (ILP)
 constexpr int kScoutSplit = 4;  // scout workgroups per (group, (l, c) tile, p tile)
 constexpr int kPairFields = 4;  // per-pair table of sieve A: thr_b, thr_o, n_ck, n_nock
 constexpr int kLdsRowStride = MIST_ROW_TERMS + 1;  // odd number of doubles: lanes reading the

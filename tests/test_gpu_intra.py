@@ -185,3 +185,12 @@ def test_full_size_groups_match_oracle(plan, G, mesh, tp):
                             getattr(want, f"costs_{kind}{suffix}")[g, q], f"costs_{kind}{suffix}")
         n_finite += int((gi >= 0).sum())
     assert n_finite > 1000
+
+
+def test_gradient_accumulation_steps_that_are_not_powers_of_two():
+    """The tuner's own G candidates are powers of two (the kernel then multiplies by an exact
+    reciprocal); a caller-supplied list may hold any divisor of the batch size, which takes the
+    true-division path."""
+    cfg, tables = tiny_plan(1, layers=5, training__global_batch_size=24, hardware__memory_capacity=6.0)
+    got, _ = _compare(cfg, tables, 1, Gs=[3, 6, 12, 24], meshes=[(1, 1), (1, 2)])
+    assert np.isfinite(got.costs_stable).any()

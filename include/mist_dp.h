@@ -80,7 +80,9 @@ int mist_dp_filter_tmax(const float *sorted_unique, int n, double gap, float *ou
  *   d_best_s (-1 = infeasible), d_best_sum = F(best_s,0,D), d_stage_max = running max of the
  *   chosen stage costs.
  * MIST_DP_BOTTLENECK: same recurrence with max() in place of "+" and no threshold; d_best_sum
- *   is the smallest threshold for which the instance is feasible (+inf if none).  The reference
+ *   is the smallest threshold for which the instance is feasible (+inf if none) and d_stage_max
+ *   the float32 sum of the stage costs of the partition that attains it (so the threshold DP at
+ *   that threshold returns a sum no larger).  The reference
  *   finds that point by running the threshold DP for every smaller candidate, all of which
  *   return "infeasible" and change nothing.
  * d_argmin (may be NULL): [n_tmax][max_stages+1][L+1][D+1][4] int32 =

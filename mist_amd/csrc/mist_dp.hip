@@ -145,7 +145,12 @@ __global__ __launch_bounds__(kDpThreads) void dp_step_kernel(
         best = target;
         arg_i = i;
         arg_q = q;
-        if (!kBottleneck) {
+        if (kBottleneck) {
+          // the maxima plane carries the SUM of the stage costs along the min-max path: a
+          // partition that is admissible at the returned threshold, with its float32 sum
+          // accumulated in the threshold DP's order
+          best_m = rmin + m_prev[from];
+        } else {
           const float *__restrict__ row = cost_tab + off[v] + at;
           for (int j = j_begin; j <= j_end; ++j) {
             const float stage_cost = row[j];

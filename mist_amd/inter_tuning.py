@@ -234,14 +234,18 @@ class _DpRunner:
             min_sum = np.minimum(min_sum, np.where(bs >= 0, bsum.astype(np.float64), np.inf))
         return cost, winner, min_sum
 
-    def bottleneck(self, g_index: np.ndarray) -> np.ndarray:
-        """Smallest threshold for which any family is feasible (float32, +inf if none)."""
+    def bottleneck(self, g_index: np.ndarray):
+        """Smallest threshold for which any family is feasible (float32, +inf if none) and the
+        stage-cost sum of a partition that is admissible there."""
         b = np.full(len(g_index), np.inf, dtype=np.float32)
+        path_sum = np.full(len(g_index), np.inf)
         zeros = np.zeros(len(g_index), dtype=np.float32)
         for fam in self.families:
-            _, bott, _ = self.run(g_index, zeros, _lib.DP_BOTTLENECK, family=fam)
-            b = np.minimum(b, bott)
-        return b
+            _, bott, psum = self.run(g_index, zeros, _lib.DP_BOTTLENECK, family=fam)
+            better = bott < b
+            b = np.where(better, bott, b)
+            path_sum = np.where(better, psum.astype(np.float64), path_sum)
+        return b, path_sum
 
     def partitions(self, g_index: np.ndarray, tmax: np.ndarray, G: np.ndarray):
         """Per instance ``(total, [((l0, l1), (n, m), ckpt), ...])`` of its winning family, from
@@ -287,10 +291,10 @@ class _Window:
 
     def __init__(self, runner: "_DpRunner", row: int, G: int, start_value: float, start_sum: float):
         self.runner, self.row, self.G, self.start_value = runner, row, G, np.float32(start_value)
-        # Sum of stage costs of the DP at the smallest feasible threshold.  At the first kept
-        # candidate t_s >= start_value that solution is still admissible, so the scan's running
-        # best is at most start_sum + (G - 1) * t_s once it has looked at t_s; candidates with
-        # t * G beyond that are never reached.
+        # Stage-cost sum of a partition that is admissible at the smallest feasible threshold.
+        # At the first kept candidate t_s >= start_value it still is, so the scan's running best
+        # is at most start_sum + (G - 1) * t_s once it has looked at t_s; candidates with t * G
+        # beyond that are never reached.
         self.start_sum = float(start_sum)
         self.bound = float("inf")
         self.kept = np.empty(0, dtype=np.float32)
@@ -473,13 +477,14 @@ def _search(runner: _DpRunner, rows: np.ndarray, Gs: List[int], stats: Optional[
     # threshold DP there: its cost bounds how far up the scan of that G can get.
     flat = rows.reshape(-1)
     flat_G = np.tile(np.array(Gs, dtype=np.int64), n_inst)
-    bottleneck = runner.bottleneck(flat)
+    bottleneck, path_sum = runner.bottleneck(flat)
     feasible = np.isfinite(bottleneck)
     windows: List[Optional[_Window]] = [None] * len(flat)
     if feasible.any():
         idx = np.nonzero(feasible)[0]
-        cost0, _, sum0 = runner.evaluate(flat[idx], bottleneck[idx], flat_G[idx])
-        assert np.isfinite(cost0).all()
+        # the min-max partition is admissible at the bottleneck: its total bounds the scan's best
+        sum0 = path_sum[idx]
+        cost0 = sum0 + (flat_G[idx] - 1).astype(np.float64) * bottleneck[idx].astype(np.float64)
         hi = np.nextafter((cost0 * (1.0 + 1e-5) / flat_G[idx]).astype(np.float32), np.float32(np.inf))
         hi = np.maximum(hi, np.nextafter(bottleneck[idx], np.float32(np.inf)))
         for k, i in enumerate(idx):

@@ -12,6 +12,8 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import Callable, List, Optional, Sequence, Tuple
 
+from functools import lru_cache
+
 import numpy as np
 
 from ._lib import MAX_PAIRS, MAX_PAR, MAX_RATIOS
@@ -93,6 +95,19 @@ class SearchSpace:
         return self.decode(np.arange(self.n_rows))
 
 
+@lru_cache(maxsize=None)
+def _valid_pairs(wo: Tuple[float, ...], go: Tuple[float, ...]):
+    """(wo index, go index) of ``itertools.product(wo, go)`` minus ``wo > 0 and go == 0``
+    (batched_module_analyzer.py:522-530); the same lists recur for every (G, mesh, tp) group."""
+    pair_wo, pair_go = [], []
+    for i, w in enumerate(wo):
+        for j, g in enumerate(go):
+            if not (w > 0 and g == 0):
+                pair_wo.append(i)
+                pair_go.append(j)
+    return tuple(pair_wo), tuple(pair_go)
+
+
 def create_search_space_for_a_block_layer(
     num_nodes: int,
     num_gpus_per_node: int,
@@ -159,12 +174,7 @@ def create_search_space_for_a_block_layer(
     else:
         ao = (0.0,)
 
-    pair_wo, pair_go = [], []
-    for i, w in enumerate(wo):
-        for j, g in enumerate(go):
-            if not (w > 0 and g == 0):
-                pair_wo.append(i)
-                pair_go.append(j)
+    pair_wo, pair_go = _valid_pairs(tuple(wo), tuple(go))
 
     for name, values in (("wo", wo), ("go", go), ("oo", oo), ("ao", ao)):
         if len(values) > MAX_RATIOS:

@@ -91,7 +91,10 @@ def test_dp_kernel_matches_c_oracle(L, D, meshes, P1, quantum):
             assert np.array_equal(g[3][0], arg), f"back-pointers differ at t={t}"
     assert n_feasible > 0
     # bottleneck mode = the smallest threshold for which the threshold DP is feasible
-    _, bott, _ = _gpu_dp(meshes, L, D, P1, tabs, [0.0], mode=1)
+    _, bott, path_sum = _gpu_dp(meshes, L, D, P1, tabs, [0.0], mode=1)
+    # ... and the sum reported with it belongs to a partition admissible at that threshold
+    at_bott = _gpu_dp(meshes, L, D, P1, tabs, [bott[0]])
+    assert at_bott[0][0] >= 0 and at_bott[1][0] <= path_sum[0] and at_bott[2][0] == bott[0]
     cand = np.unique(np.concatenate([t.ravel() for t in tabs[:3]]))
     cand = cand[np.isfinite(cand)]
     feas = _gpu_dp(meshes, L, D, P1, tabs, cand)[0] >= 0

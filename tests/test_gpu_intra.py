@@ -31,7 +31,7 @@ def _oracle(cfg, tables, tp, S, meshes, Gs):
     return intra_stage_tune(tables, cfg, cfg.model.num_hidden_layers, meshes, Gs, tp, S)
 
 
-def _compare(cfg, tables, tp, S=1, slots=None, meshes=None, Gs=None):
+def _compare(cfg, tables, tp, S=1, slots=None, meshes=None, Gs=None, require_finite=True):
     tuner = _gpu_tuner(cfg, tables, tp, S=S, slots=slots, meshes=meshes, Gs=Gs)
     got = tuner.tune()
     want = _oracle(cfg, tables, tp, S, tuner.device_mesh_candidates,
@@ -55,7 +55,7 @@ def _compare(cfg, tables, tp, S=1, slots=None, meshes=None, Gs=None):
         ws = getattr(want, "solutions" + suffix)[..., slots, :]
         assert_same_f64(gs, ws, f"solutions{suffix}")
         n_finite += int(np.isfinite(getattr(got, "costs_stable" + suffix)).sum())
-    assert n_finite > 0, "degenerate case: nothing feasible anywhere"
+    assert n_finite > 0 or not require_finite, "degenerate case: nothing feasible anywhere"
     return got, want
 
 
@@ -194,3 +194,40 @@ def test_gradient_accumulation_steps_that_are_not_powers_of_two():
     cfg, tables = tiny_plan(1, layers=5, training__global_batch_size=24, hardware__memory_capacity=6.0)
     got, _ = _compare(cfg, tables, 1, Gs=[3, 6, 12, 24], meshes=[(1, 1), (1, 2)])
     assert np.isfinite(got.costs_stable).any()
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_randomized_plans_match_oracle(seed, monkeypatch):
+    """Seeded random tiny plans: hardware coefficients, interference factors, memory capacity
+    (from "nothing fits" to "everything fits"), model shape, batch size, mesh shape, flash
+    attention, advanced first-block option and pre/post strategy are all drawn at random.  The
+    reduce kernel's pruning must leave every table bit-identical to the unpruned numpy
+    evaluation whatever the balance between latency and memory looks like."""
+    from mist_amd import intra_tuning
+    from mist_amd.config import tp_candidates
+
+    if seed % 2:  # groups this small get no scout pass by default: force one on every other seed
+        monkeypatch.setattr(intra_tuning, "SCOUT_STAGES", 3)
+        monkeypatch.setattr(intra_tuning, "MIN_SCOUT_STRIDE", 1)
+    rng = np.random.default_rng(9000 + seed)
+    gg = []
+    for _ in range(16):
+        gg += [float(rng.uniform(8, 500)), float(rng.uniform(2e-6, 8e-5))]
+    overrides = dict(
+        hardware__gpu_gpu_comm_params=gg,
+        hardware__cpu_gpu_comm_params=[float(rng.uniform(5, 60)), float(rng.uniform(2e-6, 3e-5))],
+        hardware__gpu_cpu_comm_params=[float(rng.uniform(5, 60)), float(rng.uniform(2e-6, 3e-5))],
+        hardware__interference_model_params=[float(x) for x in rng.uniform(1.0, 4.0, size=28)],
+        hardware__memory_capacity=float(rng.choice([1.0, 2.5, 4.0, 6.0, 9.0, 16.0, 80.0])),
+        hardware__num_nodes=int(rng.choice([1, 2])),
+        hardware__num_gpus_per_node=int(rng.choice([2, 4])),
+        training__global_batch_size=int(rng.choice([8, 16, 32, 48])),
+        model__hidden_size=int(rng.choice([1024, 2048, 3072])),
+        model__use_flash_attn=bool(rng.integers(2)),
+        enable_advanced_opt_in_first_block=bool(rng.integers(2)),
+        tuning__pre_post_strategy=str(rng.choice(["dp", "intra-node-tp-with-ore", "intra-node-tp-without-ore"])),
+        synthetic__seed=int(rng.integers(1 << 20)),
+    )
+    cfg, tables = tiny_plan(1, layers=int(rng.integers(3, 8)), **overrides)
+    for tp in tp_candidates(cfg):
+        _compare(cfg, tables, tp, S=int(rng.choice([1, 1, 3])), require_finite=False)

@@ -105,60 +105,79 @@ __global__ __launch_bounds__(kDpThreads) void dp_step_kernel(
   const bool free_devices = shape.free_devices != 0;
   const int rule = shape.ckpt_rule;
 
-  float best = INFINITY, best_m = 0.0f;
+  float best = INFINITY, best_m = 0.0f, best_rmin = 0.0f;
   int arg_i = -1, arg_q = -1, arg_j = -1;
+
+  // Where the ckpt row of (variant, mesh q, p, layers k..i) starts and which table holds it.
+  struct RowRef {
+    int v;
+    int64_t at;
+  };
+  auto row_ref = [&](int q, int i) {
+    const int l = i - k + 1;
+    RowRef r;
+    if (k == 0 && i == L - 1) { r.v = 3; r.at = (int64_t)q * C; }
+    else if (k == 0) { r.v = 1; r.at = (((int64_t)q * P1 + p) * L + (l - 1)) * C; }
+    else if (i == L - 1) { r.v = 2; r.at = ((int64_t)q * L + (l - 1)) * C; }
+    else { r.v = 0; r.at = (((int64_t)q * P1 + p) * L + (l - 1)) * C; }
+    r.at += off[r.v];
+    return r;
+  };
+  auto table = [&](int v, bool running_min) -> const float *__restrict__ {
+    if (running_min)
+      return v == 0 ? tabs.pmin : v == 1 ? tabs.pmin_pre : v == 2 ? tabs.pmin_post : tabs.pmin_nopp;
+    return v == 0 ? tabs.costs : v == 1 ? tabs.costs_pre : v == 2 ? tabs.costs_post : tabs.costs_nopp;
+  };
+  // ckpt candidates j_begin..j_end of a stage k..i: 0..L-i (inter_tuning.py:315), or 0..l / only l
+  // (inter_tuning_uniform_device.py:400-404)
+  auto j_last = [&](int i) { return rule == MIST_DP_CKPT_TAIL ? L - i : i - k + 1; };
+
   if (k <= L - s && (d >= 1 || free_devices)) {
     for (int q = 0; q < Q; ++q) {
       const int nm = free_devices ? 0 : shape.mesh_n[q] * shape.mesh_m[q];
       if (nm > d) continue;
       for (int i = k; i < L; ++i) {
-        const int from = (i + 1) * W + (d - nm);
-        const float prev = f_prev[from];
+        const float prev = f_prev[(i + 1) * W + (d - nm)];
         // A state reachable only through an unreachable successor cannot improve: inf + c is
-        // never < best.  Skipping it changes nothing.
+        // never < best.  Skipping it changes nothing (and most successors are unreachable).
         if (prev == INFINITY) continue;
-        const int l = i - k + 1;
-        int64_t at;  // start of the ckpt row of this (variant, mesh, p, layers)
-        int v;
-        if (k == 0 && i == L - 1) { v = 3; at = (int64_t)q * C; }
-        else if (k == 0) { v = 1; at = (((int64_t)q * P1 + p) * L + (l - 1)) * C; }
-        else if (i == L - 1) { v = 2; at = ((int64_t)q * L + (l - 1)) * C; }
-        else { v = 0; at = (((int64_t)q * P1 + p) * L + (l - 1)) * C; }
-        const float *__restrict__ cost_tab = v == 0 ? tabs.costs : v == 1 ? tabs.costs_pre
-                                             : v == 2 ? tabs.costs_post : tabs.costs_nopp;
-        const float *__restrict__ pmin_tab = v == 0 ? tabs.pmin : v == 1 ? tabs.pmin_pre
-                                             : v == 2 ? tabs.pmin_post : tabs.pmin_nopp;
-        // ckpt candidates j_begin..j_end: 0..L-i (inter_tuning.py:315), or 0..l / only l
-        // (inter_tuning_uniform_device.py:400-404)
-        const int j_end = rule == MIST_DP_CKPT_TAIL ? L - i : l;
-        const int j_begin = rule == MIST_DP_CKPT_ALL ? l : 0;
-        // The reference walks j = 0..j_end with "cost <= t_max and cost + prev < best".  "+ prev"
-        // is monotone, so the smallest reachable sum is (smallest admissible cost) + prev, and
-        // the smallest admissible cost is the row's running minimum if that is <= t_max (else
-        // nothing is admissible).  Only when this sum beats `best` is the row walked, to find
-        // the first j that attains it: that is the entry the reference's strict "<" keeps.
-        const float rmin = rule == MIST_DP_CKPT_ALL ? cost_tab[off[v] + at + l]
-                                                    : pmin_tab[off[v] + at + j_end];
+        const RowRef r = row_ref(q, i);
+        // The reference walks j = j_begin..j_end with "cost <= t_max and cost + prev < best".
+        // "+ prev" is monotone, so the smallest reachable sum is (smallest admissible cost) +
+        // prev, and the smallest admissible cost is the row's running minimum if that is
+        // <= t_max (else nothing is admissible).
+        const float rmin = rule == MIST_DP_CKPT_ALL ? table(r.v, false)[r.at + (i - k + 1)]
+                                                    : table(r.v, true)[r.at + j_last(i)];
         if (!(rmin <= t_max)) continue;
         const float target = kBottleneck ? fmaxf(rmin, prev) : rmin + prev;
         if (!(target < best)) continue;
         best = target;
+        best_rmin = rmin;
         arg_i = i;
         arg_q = q;
-        if (kBottleneck) {
-          // the maxima plane carries the SUM of the stage costs along the min-max path: a
-          // partition that is admissible at the returned threshold, with its float32 sum
-          // accumulated in the threshold DP's order
-          best_m = rmin + m_prev[from];
-        } else {
-          const float *__restrict__ row = cost_tab + off[v] + at;
-          for (int j = j_begin; j <= j_end; ++j) {
-            const float stage_cost = row[j];
-            if (stage_cost <= t_max && stage_cost + prev == target) {
-              arg_j = j;
-              best_m = fmaxf(m_prev[from], stage_cost);
-              break;
-            }
+      }
+    }
+    // The winner's ckpt count and stage maximum: the first j attaining the sum is the entry the
+    // reference's strict "<" keeps.  Only the final winner matters, so the row is walked once.
+    if (arg_i >= 0) {
+      const int nm = free_devices ? 0 : shape.mesh_n[arg_q] * shape.mesh_m[arg_q];
+      const int from = (arg_i + 1) * W + (d - nm);
+      if (kBottleneck) {
+        // the maxima plane carries the SUM of the stage costs along the min-max path: a
+        // partition that is admissible at the returned threshold, with its float32 sum
+        // accumulated in the threshold DP's order
+        best_m = best_rmin + m_prev[from];
+      } else {
+        const RowRef r = row_ref(arg_q, arg_i);
+        const float *__restrict__ row = table(r.v, false) + r.at;
+        const float prev = f_prev[from];
+        const int j_begin = rule == MIST_DP_CKPT_ALL ? arg_i - k + 1 : 0;
+        for (int j = j_begin; j <= j_last(arg_i); ++j) {
+          const float stage_cost = row[j];
+          if (stage_cost <= t_max && stage_cost + prev == best) {
+            arg_j = j;
+            best_m = fmaxf(m_prev[from], stage_cost);
+            break;
           }
         }
       }

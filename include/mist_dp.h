@@ -71,6 +71,19 @@ int mist_dp_cost_tables(const MistProblem *problem, const MistOutTables *tables,
  * candidate t_max values; writes the kept values to out and returns their count. */
 int mist_dp_filter_tmax(const float *sorted_unique, int n, double gap, float *out);
 
+/* t_max candidates of value windows (reference: the sort + scan over every finite stage cost,
+ * inter_tuning.py:180-199, restricted to where the scan can get).  Request r selects the finite
+ * values v of the costs / with_pre / with_post tables of table row d_rows[r] with
+ * d_lo[r] < v <= d_hi[r] (-inf / +inf for open ends).  Selected values are appended unordered to
+ * d_out_values with their request number in d_out_request (capacity entries each).
+ * d_counts[1 + n_requests], zeroed by the caller: [0] = values selected in total (if larger than
+ * capacity the lists are incomplete: call again with larger lists), [1 + r] = finite values of
+ * request r above d_hi[r]. */
+int mist_dp_select_candidates(const MistDpCosts *costs, int n_requests, const int32_t *d_rows,
+                              const float *d_lo, const float *d_hi, float *d_out_values,
+                              int32_t *d_out_request, int capacity, int32_t *d_counts,
+                              void *stream);
+
 /* Runs n_tmax DP instances at once (max_stages launches, one thread per (instance, start
  * layer, devices) state).  Instance t uses the cost tables of g = d_g_index[t].
  * MIST_DP_THRESHOLD (reference: inter_stage_tune_dp_impl, inter_tuning.py:220-355):

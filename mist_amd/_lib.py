@@ -175,6 +175,10 @@ _DP_SIGNATURES = {
         [_VP, ctypes.POINTER(OutTables), _VP, ctypes.c_int, ctypes.c_void_p * 4, ctypes.c_void_p * 4, _VP],
     ),
     "mist_dp_filter_tmax": (ctypes.c_int, [_VP, ctypes.c_int, ctypes.c_double, _VP]),
+    "mist_dp_select_candidates": (
+        ctypes.c_int,
+        [ctypes.POINTER(DpCosts), ctypes.c_int, _VP, _VP, _VP, _VP, _VP, ctypes.c_int, _VP, _VP],
+    ),
     "mist_dp_scratch_floats": (ctypes.c_int64, [_VP, ctypes.c_int]),
     "mist_dp_run": (
         ctypes.c_int,

@@ -7,6 +7,8 @@
 // reference loop nest (mist/analyzer/inter_tuning.py:298-333).
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
+
 #include <cmath>
 #include <cstdint>
 
@@ -44,6 +46,43 @@ __global__ __launch_bounds__(256) void cost_table_kernel(const double *__restric
     out[i] = c;
     pmin[i] = run;
   }
+}
+
+// ------------------------------------------------------------------------------------------
+// t_max candidates of a value window: one pass over the three cost tables of a table row g
+// (costs, with_pre, with_post; inter_tuning.py:180-186).  Request r selects the finite values v
+// of row rows[r] with lo[r] < v <= hi[r]; they are appended, unordered, to one output list as
+// (value, request) pairs; counts[0] = pairs wanted in total (may exceed the capacity, then the
+// caller retries with a larger list), counts[1 + r] = finite values of request r above hi[r].
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void select_candidates_kernel(
+    const MistDpCosts tabs, const int32_t *__restrict__ rows, const float *__restrict__ lo,
+    const float *__restrict__ hi, float *__restrict__ out_values, int32_t *__restrict__ out_request,
+    int capacity, int32_t *__restrict__ counts) {
+  const int r = blockIdx.y;
+  const int64_t g = rows[r];
+  const int64_t n0 = tabs.g_stride[0], n1 = tabs.g_stride[1], n2 = tabs.g_stride[2];
+  const float lo_r = lo[r], hi_r = hi[r];
+  int above = 0;
+  for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < n0 + n1 + n2;
+       e += (int64_t)gridDim.x * blockDim.x) {
+    const float v = e < n0 ? tabs.costs[g * n0 + e]
+                    : e < n0 + n1 ? tabs.costs_pre[g * n1 + (e - n0)]
+                                  : tabs.costs_post[g * n2 + (e - n0 - n1)];
+    if (!(v < INFINITY)) continue;  // +inf (nothing feasible) and NaN are not candidates
+    if (v > hi_r) {
+      ++above;
+    } else if (v > lo_r) {
+      const int at = atomicAdd(&counts[0], 1);
+      if (at < capacity) {
+        out_values[at] = v;
+        out_request[at] = r;
+      }
+    }
+  }
+  // one atomic per wavefront for the "above" count
+  for (int step = 32; step >= 1; step >>= 1) above += __shfl_xor(above, step);
+  if ((threadIdx.x & 63) == 0 && above > 0) atomicAdd(&counts[1 + r], above);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -267,6 +306,25 @@ int mist_dp_filter_tmax(const float *sorted_unique, int n, double gap, float *ou
     last = t;
   }
   return kept;
+}
+
+int mist_dp_select_candidates(const MistDpCosts *costs, int n_requests, const int32_t *d_rows,
+                              const float *d_lo, const float *d_hi, float *d_out_values,
+                              int32_t *d_out_request, int capacity, int32_t *d_counts,
+                              void *stream) {
+  if (!costs || !costs->costs || !costs->costs_pre || !costs->costs_post)
+    return fail(MIST_E_INVALID, "null cost tables");
+  if (n_requests <= 0 || n_requests > 65535)
+    return fail(MIST_E_INVALID, "n_requests %d outside [1, 65535]", n_requests);
+  if (!d_rows || !d_lo || !d_hi || !d_out_values || !d_out_request || !d_counts || capacity <= 0)
+    return fail(MIST_E_INVALID, "null pointer / empty output list");
+  const int64_t per_row = costs->g_stride[0] + costs->g_stride[1] + costs->g_stride[2];
+  const unsigned blocks = (unsigned)std::min<int64_t>((per_row + 255) / 256, 512);
+  hipLaunchKernelGGL(select_candidates_kernel, dim3(blocks, n_requests), dim3(256), 0,
+                     (hipStream_t)stream, *costs, d_rows, d_lo, d_hi, d_out_values, d_out_request,
+                     capacity, d_counts);
+  MIST_HIP_CHECK(hipGetLastError());
+  return 0;
 }
 
 int64_t mist_dp_scratch_floats(const MistDpShape *shape, int n_tmax) {

@@ -92,8 +92,10 @@ class _DpRunner:
             self.families = self._uniform_device_families(meshes, **uniform_device)
         self.launches = 0
         self.thresholds_run = 0
-        self._cand = None
+        self._all_costs = self._costs_struct()
+        self._select_capacity = 1 << 18
         self.fetches = 0
+        self.selected = 0
 
     def _costs_struct(self, q: int = 0):
         """Table pointers starting at mesh ``q`` (strides between g unchanged)."""
@@ -140,35 +142,41 @@ class _DpRunner:
             fams.append(_DpFamily(shape, self._costs_struct(q), False))
         return fams
 
-    def _all_candidates(self) -> torch.Tensor:
-        """[Gn, N] float32: every stage cost the reference collects as a t_max candidate
-        (costs, costs_with_pre, costs_with_post; inter_tuning.py:180-186)."""
-        if self._cand is None:
-            self._cand = torch.cat([self.cost[v].reshape(self.Gn, -1) for v in range(3)], dim=1)
-        return self._cand
-
     def candidates_between(self, rows: np.ndarray, lo: np.ndarray, hi: np.ndarray):
-        """Per requested table row g: the ascending candidates v with lo < v <= hi (lo = -inf
-        includes everything below), and how many finite candidates lie above hi.  One pass on
-        the device over all requested rows, only the selected values come back."""
+        """Per requested table row g: the ascending t_max candidates v (finite stage costs of the
+        costs / with_pre / with_post tables, inter_tuning.py:180-186) with lo < v <= hi (lo = -inf
+        includes everything below), and how many finite candidates lie above hi.  One kernel
+        pass over the requested rows; only the selected values come back."""
         dev = self.device
         self.fetches += 1
-        allv = self._all_candidates()
+        n = len(rows)
         with torch.cuda.device(dev):
-            bounds = torch.from_numpy(np.stack([lo, hi]).astype(np.float32)).to(dev)
-            sel = allv if len(rows) == self.Gn and np.array_equal(rows, np.arange(self.Gn)) \
-                else allv[torch.from_numpy(rows.astype(np.int64)).to(dev)]
-            finite = torch.isfinite(sel)
-            inside = finite & (sel > bounds[0][:, None]) & (sel <= bounds[1][:, None])
-            above = (finite & (sel > bounds[1][:, None])).sum(dim=1)
-            counts = torch.stack([inside.sum(dim=1), above]).cpu().numpy()
-            values = sel[inside].cpu().numpy()
-        out, off = [], 0
-        for i in range(len(rows)):
-            n = int(counts[0, i])
-            out.append((np.sort(values[off:off + n]), int(counts[1, i])))
-            off += n
-        return out
+            req = np.empty((3, n), dtype=np.float32)
+            req[0].view(np.int32)[:] = rows
+            req[1], req[2] = lo, hi
+            d_req = torch.from_numpy(req).to(dev)
+            capacity = self._select_capacity
+            while True:
+                counts = torch.zeros(1 + n, dtype=torch.int32, device=dev)
+                values = torch.empty(capacity, dtype=torch.float32, device=dev)
+                request = torch.empty(capacity, dtype=torch.int32, device=dev)
+                rc = self.lib.mist_dp_select_candidates(
+                    ctypes.byref(self._all_costs), n, d_req[0].data_ptr(), d_req[1].data_ptr(),
+                    d_req[2].data_ptr(), values.data_ptr(), request.data_ptr(), capacity,
+                    counts.data_ptr(), _stream(dev))
+                _lib.check(rc, "mist_dp_select_candidates")
+                h_counts = counts.cpu().numpy()
+                total = int(h_counts[0])
+                if total <= capacity:
+                    break
+                capacity = self._select_capacity = 2 * total
+            h_values = values[:total].cpu().numpy()
+            h_request = request[:total].cpu().numpy()
+        self.selected += total
+        order = np.argsort(h_request, kind="stable")  # group by request (small integer keys)
+        h_values, h_request = h_values[order], h_request[order]
+        bounds = np.searchsorted(h_request, np.arange(n + 1))
+        return [(np.sort(h_values[bounds[i]:bounds[i + 1]]), int(h_counts[1 + i])) for i in range(n)]
 
     def filter_gap(self, ascending: np.ndarray) -> np.ndarray:
         """The reference's gap rule (inter_tuning.py:198) applied from the first element on
@@ -637,6 +645,7 @@ def inter_stage_tune_batch(
         stats["dp_backtrack_s"] = stats.get("dp_backtrack_s", 0.0) + (time.perf_counter() - t_2)
         stats["dp_launches"] = stats.get("dp_launches", 0) + runner.launches
         stats["dp_window_fetches"] = stats.get("dp_window_fetches", 0) + runner.fetches
+        stats["dp_window_values"] = stats.get("dp_window_values", 0) + runner.selected
         stats["dp_thresholds"] = stats.get("dp_thresholds", 0) + runner.thresholds_run
     return out
 

@@ -294,3 +294,33 @@ def test_uniform_device_tune_end_to_end_matches_oracle(overrides):
     want = oracle_tune(cfg, tables)
     assert got == want
     assert want[1] is not None
+
+
+def test_candidate_window_selection_matches_numpy():
+    """mist_dp_select_candidates against a numpy filter of the same tables, including open
+    ends, empty windows and the retry when the output list is too small."""
+    from mist_amd.inter_tuning import _DpRunner
+    from mist_amd.intra_tuning import IntraStageTuner
+    from mist_amd.search_space import _get_device_mesh_candidates, _get_grad_accumu_steps_candidates
+
+    cfg, tables = load_plan(1)
+    hw, L = cfg.hardware, cfg.model.num_hidden_layers
+    meshes = _get_device_mesh_candidates(hw.num_nodes, hw.num_gpus_per_node, False)
+    Gs = _get_grad_accumu_steps_candidates(cfg.training.global_batch_size)
+    res = IntraStageTuner(tables, L, meshes, Gs, 1, cfg, sample_size=1).tune()
+    runner = _DpRunner(res, L, hw.num_nodes * hw.num_gpus_per_node, meshes, 0)
+    runner._select_capacity = 16  # force the retry path
+    host = [np.concatenate([runner.cost[v][g].cpu().numpy().ravel() for v in range(3)]) for g in range(len(Gs))]
+    finite = np.concatenate([h[np.isfinite(h)] for h in host])
+    assert len(finite) > 100
+    q = np.quantile(finite, [0.1, 0.4, 0.6, 0.9]).astype(np.float32)
+    rows = np.array([0, 1, len(Gs) - 1, 1, 2, 0], dtype=np.int32)
+    lo = np.array([-np.inf, q[0], q[1], q[3], q[2], 1e30], dtype=np.float32)
+    hi = np.array([q[1], q[2], np.inf, q[3], q[3], np.inf], dtype=np.float32)
+    got = runner.candidates_between(rows, lo, hi)
+    for (values, above), g, a, b in zip(got, rows, lo, hi):
+        h = host[g][np.isfinite(host[g])]
+        want = np.sort(h[(h > a) & (h <= b)])
+        assert np.array_equal(values, want)
+        assert above == int((h > b).sum())
+    assert len(got[3][0]) == 0 and len(got[5][0]) == 0 and len(got[0][0]) > 0

@@ -20,6 +20,7 @@ namespace {
 using mist::fail;
 
 constexpr int kDpThreads = 64;  // one wavefront per workgroup
+constexpr int kDpWideTeam = 8;  // lanes that share one DP state in small batches
 
 // ------------------------------------------------------------------------------------------
 // Adapter: float64 (stable, delta) tables -> float32 DP cost tables for every g.
@@ -113,7 +114,7 @@ __global__ __launch_bounds__(256) void dp_init_kernel(const MistDpShape shape, i
   }
 }
 
-template <bool kBottleneck>
+template <bool kBottleneck, int kDpTeam>
 __global__ __launch_bounds__(kDpThreads) void dp_step_kernel(
     const MistDpShape shape, const MistDpCosts tabs, const float *__restrict__ tmax_list,
     const int32_t *__restrict__ g_list, int s, float *__restrict__ scratch,
@@ -125,8 +126,17 @@ __global__ __launch_bounds__(kDpThreads) void dp_step_kernel(
   const int W = D + 1;            // row pitch of a state plane
   const int plane = (L + 1) * W;  // states per s
   const int C = L + 1;            // ckpt extent of the cost tables
-  const int e = blockIdx.x * kDpThreads + threadIdx.x;
-  if (e >= plane) return;
+  // kDpTeam consecutive lanes share one state and split its end layers between them.  The scan
+  // of a state is a chain of dependent L2 reads: in a small batch its latency, not the
+  // arithmetic, sets the time of a launch (team of 8); a batch that fills the GPU anyway runs
+  // one lane per state, which prunes better.
+  const int member = threadIdx.x % kDpTeam;
+  const int e_raw = (blockIdx.x * kDpThreads + threadIdx.x) / kDpTeam;
+  const bool real = e_raw < plane;  // the last team of a plane may be a dummy (kept for shuffles)
+  if constexpr (kDpTeam == 1) {
+    if (!real) return;
+  }
+  const int e = real ? e_raw : plane - 1;
   const int t = blockIdx.y;
   float *state = scratch + (int64_t)t * 4 * plane;
   const int cur = s & 1, prv = cur ^ 1;
@@ -171,33 +181,9 @@ __global__ __launch_bounds__(kDpThreads) void dp_step_kernel(
   // (inter_tuning_uniform_device.py:400-404)
   auto j_last = [&](int i) { return rule == MIST_DP_CKPT_TAIL ? L - i : i - k + 1; };
 
-  if (k <= L - s && (d >= 1 || free_devices)) {
-    for (int q = 0; q < Q; ++q) {
-      const int nm = free_devices ? 0 : shape.mesh_n[q] * shape.mesh_m[q];
-      if (nm > d) continue;
-      for (int i = k; i < L; ++i) {
-        const float prev = f_prev[(i + 1) * W + (d - nm)];
-        // A state reachable only through an unreachable successor cannot improve: inf + c is
-        // never < best.  Skipping it changes nothing (and most successors are unreachable).
-        if (prev == INFINITY) continue;
-        const RowRef r = row_ref(q, i);
-        // The reference walks j = j_begin..j_end with "cost <= t_max and cost + prev < best".
-        // "+ prev" is monotone, so the smallest reachable sum is (smallest admissible cost) +
-        // prev, and the smallest admissible cost is the row's running minimum if that is
-        // <= t_max (else nothing is admissible).
-        const float rmin = rule == MIST_DP_CKPT_ALL ? table(r.v, false)[r.at + (i - k + 1)]
-                                                    : table(r.v, true)[r.at + j_last(i)];
-        if (!(rmin <= t_max)) continue;
-        const float target = kBottleneck ? fmaxf(rmin, prev) : rmin + prev;
-        if (!(target < best)) continue;
-        best = target;
-        best_rmin = rmin;
-        arg_i = i;
-        arg_q = q;
-      }
-    }
-    // The winner's ckpt count and stage maximum: the first j attaining the sum is the entry the
-    // reference's strict "<" keeps.  Only the final winner matters, so the row is walked once.
+  // The winner's ckpt count and stage maximum: the first j attaining the sum is the entry the
+  // reference's strict "<" keeps.  Only the final winner matters, so the row is walked once.
+  auto finish_winner = [&]() {
     if (arg_i >= 0) {
       const int nm = free_devices ? 0 : shape.mesh_n[arg_q] * shape.mesh_m[arg_q];
       const int from = (arg_i + 1) * W + (d - nm);
@@ -221,6 +207,57 @@ __global__ __launch_bounds__(kDpThreads) void dp_step_kernel(
         }
       }
     }
+  };
+
+  const bool live = k <= L - s && (d >= 1 || free_devices);
+  if (live) {
+    for (int q = 0; q < Q; ++q) {
+      const int nm = free_devices ? 0 : shape.mesh_n[q] * shape.mesh_m[q];
+      if (nm > d) continue;
+      for (int i = k + member; i < L; i += kDpTeam) {
+        const float prev = f_prev[(i + 1) * W + (d - nm)];
+        // A state reachable only through an unreachable successor cannot improve: inf + c is
+        // never < best.  Skipping it changes nothing (and most successors are unreachable).
+        if (prev == INFINITY) continue;
+        const RowRef r = row_ref(q, i);
+        // The reference walks j = j_begin..j_end with "cost <= t_max and cost + prev < best".
+        // "+ prev" is monotone, so the smallest reachable sum is (smallest admissible cost) +
+        // prev, and the smallest admissible cost is the row's running minimum if that is
+        // <= t_max (else nothing is admissible).
+        const float rmin = rule == MIST_DP_CKPT_ALL ? table(r.v, false)[r.at + (i - k + 1)]
+                                                    : table(r.v, true)[r.at + j_last(i)];
+        if (!(rmin <= t_max)) continue;
+        const float target = kBottleneck ? fmaxf(rmin, prev) : rmin + prev;
+        if (!(target < best)) continue;
+        best = target;
+        best_rmin = rmin;
+        arg_i = i;
+        arg_q = q;
+      }
+    }
+    if constexpr (kDpTeam == 1) finish_winner();
+  }
+  // Team reduction.  The reference visits (q, i) in ascending order and replaces on a strict "<":
+  // the winner is the first candidate that attains the minimum, i.e. the lexicographic minimum
+  // of (target, q, i).  Each lane holds that minimum over its own candidates.
+  if constexpr (kDpTeam > 1) {
+    int order = arg_i >= 0 ? arg_q * L + arg_i : 0x7fffffff;
+#pragma unroll
+    for (int step = 1; step < kDpTeam; step <<= 1) {
+      const float o_best = __shfl_xor(best, step);
+      const float o_rmin = __shfl_xor(best_rmin, step);
+      const int o_order = __shfl_xor(order, step);
+      const bool take = o_best < best || (o_best == best && o_order < order);
+      best = take ? o_best : best;
+      best_rmin = take ? o_rmin : best_rmin;
+      order = take ? o_order : order;
+    }
+    arg_q = order == 0x7fffffff ? -1 : order / L;
+    arg_i = order == 0x7fffffff ? -1 : order % L;
+  }
+  if constexpr (kDpTeam > 1) {
+    if (!real || member != 0) return;
+    if (live) finish_winner();
   }
   f_cur[e] = best;
   m_cur[e] = best_m;
@@ -353,16 +390,21 @@ int mist_dp_run(const MistDpShape *shape, const MistDpCosts *costs, const float 
                      (hipStream_t)stream, *shape, n_tmax, d_scratch, d_best_s, d_best_sum,
                      d_stage_max);
   MIST_HIP_CHECK(hipGetLastError());
-  const dim3 grid((plane + kDpThreads - 1) / kDpThreads, n_tmax);
+  // Small batches are latency-bound: spread every state over a team of lanes.
+  const bool wide = (int64_t)n_tmax * plane <= (1 << 19);
+  const int states_per_block = kDpThreads / (wide ? kDpWideTeam : 1);
+  const dim3 grid((plane + states_per_block - 1) / states_per_block, n_tmax);
   for (int s = 1; s <= shape->max_stages; ++s) {
-    if (mode == MIST_DP_BOTTLENECK)
-      hipLaunchKernelGGL(dp_step_kernel<true>, grid, dim3(kDpThreads), 0, (hipStream_t)stream,
-                         *shape, *costs, d_tmax, d_g_index, s, d_scratch, d_best_s, d_best_sum,
-                         d_stage_max, d_argmin);
-    else
-      hipLaunchKernelGGL(dp_step_kernel<false>, grid, dim3(kDpThreads), 0, (hipStream_t)stream,
-                         *shape, *costs, d_tmax, d_g_index, s, d_scratch, d_best_s, d_best_sum,
-                         d_stage_max, d_argmin);
+#define MIST_DP_STEP(BOTTLENECK, TEAM)                                                         \
+  hipLaunchKernelGGL((dp_step_kernel<BOTTLENECK, TEAM>), grid, dim3(kDpThreads), 0,            \
+                     (hipStream_t)stream, *shape, *costs, d_tmax, d_g_index, s, d_scratch,     \
+                     d_best_s, d_best_sum, d_stage_max, d_argmin)
+    if (mode == MIST_DP_BOTTLENECK) {
+      if (wide) MIST_DP_STEP(true, kDpWideTeam); else MIST_DP_STEP(true, 1);
+    } else {
+      if (wide) MIST_DP_STEP(false, kDpWideTeam); else MIST_DP_STEP(false, 1);
+    }
+#undef MIST_DP_STEP
     MIST_HIP_CHECK(hipGetLastError());
   }
   return 0;

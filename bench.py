@@ -192,7 +192,10 @@ def main():
         "tune_end_to_end_s": tune_end_to_end_s,
         "intra_kernels_ms_per_step": intra_ms_per_step,
         "intra_kernel_ms": {k: v / 2 for k, v in kernel_ms.items()},
-        "inter_stage_ms_per_step": 1e3 * stats.get("inter_s", 0.0) / args.steps,
+        # host time of the inter-stage search after the intra-stage tables are complete
+        # (bottleneck DP + threshold windows, scan batches, back-pointers)
+        "inter_stage_ms_per_step": 1e3 * sum(
+            stats.get(k, 0.0) for k in ("dp_thresholds_s", "dp_scan_s", "dp_backtrack_s")) / args.steps,
         "dp_thresholds_per_step": stats.get("dp_thresholds", 0) / args.steps,
         "best_cost": cost,
         "best_solution": repr(solution),

@@ -324,3 +324,39 @@ def test_candidate_window_selection_matches_numpy():
         assert np.array_equal(values, want)
         assert above == int((h > b).sum())
     assert len(got[3][0]) == 0 and len(got[5][0]) == 0 and len(got[0][0]) > 0
+
+
+@pytest.mark.parametrize("granularity", ["inter-stage", "uniform-device-pp", "uniform-pp", "no-pp"])
+def test_infeasible_plan_returns_inf_none(granularity):
+    """Nothing fits into 0.2 GB: every table stays +inf / -1, the searches find no partition and
+    the reference's contract is (inf, None) (inter_tuning.py:146-147), also through the oracle."""
+    from mist_amd.tune_one_case import tune
+    from oracle.tune import tune as oracle_tune
+
+    cfg, tables = tiny_plan(1, layers=4, hardware__memory_capacity=0.2,
+                            tuning__tuning_granularity=granularity)
+    cost, solution = tune(cfg)
+    assert cost == float("inf") and solution is None
+    if granularity != "no-pp":
+        assert oracle_tune(cfg, tables) == (float("inf"), None)
+
+
+def test_groups_without_candidates_stay_empty():
+    """A (G, mesh) pair without a valid (batch size, dp, tp) factorisation has no rows; the
+    reference returns all-inf tables for it (batched_module_analyzer.py:648-666) and so must the
+    batched launch, which simply has no group descriptor for it."""
+    from mist_amd.intra_tuning import IntraStageTuner
+
+    cfg, tables = tiny_plan(1, layers=4)
+    meshes, Gs = [(1, 1), (1, 2)], [1, 8]
+    tuner = IntraStageTuner(tables, 4, meshes, Gs, 2, cfg, sample_size=1)
+    plan = tuner.prepare()
+    present = {(int(r["g_index"]), int(r["q_index"])) for r in plan["groups"]}
+    missing = {(g, q) for g in range(2) for q in range(2)} - present
+    assert missing, "the case is meant to contain an empty group"
+    got = tuner.tune()
+    for g, q in missing:
+        assert np.all(np.isinf(got.costs_stable[g, q])) and np.all(got.indices[g, q] == -1)
+    from oracle.intra import intra_stage_tune
+    want = intra_stage_tune(tables, cfg, 4, meshes, Gs, 2, 1)
+    assert np.array_equal(got.indices, want.indices)

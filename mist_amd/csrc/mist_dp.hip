@@ -114,11 +114,33 @@ __global__ __launch_bounds__(256) void dp_init_kernel(const MistDpShape shape, i
   }
 }
 
+// Rows of plane `which` (F of the stage count just finished) that are reachable, per instance
+// and device column: most states are not, and the next step only scans [first, last].
+__global__ __launch_bounds__(256) void dp_ranges_kernel(const MistDpShape shape, int n_tmax,
+                                                        int which, const float *__restrict__ scratch,
+                                                        int32_t *__restrict__ ranges) {
+  const int W = shape.num_devices + 1, L = shape.num_layers;
+  const int plane = (L + 1) * W;
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (int64_t)n_tmax * W) return;
+  const int t = (int)(i / W), col = (int)(i % W);
+  const float *f = scratch + (int64_t)t * 4 * plane + (int64_t)which * plane + col;
+  int first = L + 1, last = -1;
+  for (int k = 0; k <= L; ++k) {
+    if (f[(int64_t)k * W] < INFINITY) {
+      first = min(first, k);
+      last = k;
+    }
+  }
+  ranges[2 * i] = first;
+  ranges[2 * i + 1] = last;
+}
+
 template <bool kBottleneck, int kDpTeam>
 __global__ __launch_bounds__(kDpThreads) void dp_step_kernel(
     const MistDpShape shape, const MistDpCosts tabs, const float *__restrict__ tmax_list,
     const int32_t *__restrict__ g_list, int s, float *__restrict__ scratch,
-    int32_t *__restrict__ best_s_out,
+    const int32_t *__restrict__ ranges, int32_t *__restrict__ best_s_out,
     float *__restrict__ best_sum_out, float *__restrict__ stage_max_out,
     int32_t *__restrict__ argmin) {
   const int L = shape.num_layers, D = shape.num_devices, Q = shape.num_mesh;
@@ -214,7 +236,10 @@ __global__ __launch_bounds__(kDpThreads) void dp_step_kernel(
     for (int q = 0; q < Q; ++q) {
       const int nm = free_devices ? 0 : shape.mesh_n[q] * shape.mesh_m[q];
       if (nm > d) continue;
-      for (int i = k + member; i < L; i += kDpTeam) {
+      // reachable start layers i + 1 of the remaining stages on d - nm devices
+      const int32_t *reach = ranges + 2 * ((int64_t)t * W + (d - nm));
+      const int i_first = max(k, reach[0] - 1), i_last = min(L - 1, reach[1] - 1);
+      for (int i = i_first + member; i <= i_last; i += kDpTeam) {
         const float prev = f_prev[(i + 1) * W + (d - nm)];
         // A state reachable only through an unreachable successor cannot improve: inf + c is
         // never < best.  Skipping it changes nothing (and most successors are unreachable).
@@ -366,7 +391,9 @@ int mist_dp_select_candidates(const MistDpCosts *costs, int n_requests, const in
 
 int64_t mist_dp_scratch_floats(const MistDpShape *shape, int n_tmax) {
   if (check_shape(shape) != 0 || n_tmax <= 0) return -1;
-  return (int64_t)4 * n_tmax * (shape->num_layers + 1) * (shape->num_devices + 1);
+  // four state planes per instance, then (first, last) reachable row per instance and column
+  return (int64_t)4 * n_tmax * (shape->num_layers + 1) * (shape->num_devices + 1) +
+         (int64_t)2 * n_tmax * (shape->num_devices + 1);
 }
 
 int mist_dp_run(const MistDpShape *shape, const MistDpCosts *costs, const float *d_tmax,
@@ -390,6 +417,12 @@ int mist_dp_run(const MistDpShape *shape, const MistDpCosts *costs, const float 
                      (hipStream_t)stream, *shape, n_tmax, d_scratch, d_best_s, d_best_sum,
                      d_stage_max);
   MIST_HIP_CHECK(hipGetLastError());
+  int32_t *d_ranges = reinterpret_cast<int32_t *>(d_scratch + (int64_t)4 * n_tmax * plane);
+  const int64_t n_cols = (int64_t)n_tmax * (shape->num_devices + 1);
+  const dim3 ranges_grid((unsigned)((n_cols + 255) / 256));
+  hipLaunchKernelGGL(dp_ranges_kernel, ranges_grid, dim3(256), 0, (hipStream_t)stream, *shape,
+                     n_tmax, 0, d_scratch, d_ranges);
+  MIST_HIP_CHECK(hipGetLastError());
   // Small batches are latency-bound: spread every state over a team of lanes.
   const bool wide = (int64_t)n_tmax * plane <= (1 << 19);
   const int states_per_block = kDpThreads / (wide ? kDpWideTeam : 1);
@@ -398,7 +431,7 @@ int mist_dp_run(const MistDpShape *shape, const MistDpCosts *costs, const float 
 #define MIST_DP_STEP(BOTTLENECK, TEAM)                                                         \
   hipLaunchKernelGGL((dp_step_kernel<BOTTLENECK, TEAM>), grid, dim3(kDpThreads), 0,            \
                      (hipStream_t)stream, *shape, *costs, d_tmax, d_g_index, s, d_scratch,     \
-                     d_best_s, d_best_sum, d_stage_max, d_argmin)
+                     d_ranges, d_best_s, d_best_sum, d_stage_max, d_argmin)
     if (mode == MIST_DP_BOTTLENECK) {
       if (wide) MIST_DP_STEP(true, kDpWideTeam); else MIST_DP_STEP(true, 1);
     } else {
@@ -406,6 +439,11 @@ int mist_dp_run(const MistDpShape *shape, const MistDpCosts *costs, const float 
     }
 #undef MIST_DP_STEP
     MIST_HIP_CHECK(hipGetLastError());
+    if (s < shape->max_stages) {
+      hipLaunchKernelGGL(dp_ranges_kernel, ranges_grid, dim3(256), 0, (hipStream_t)stream, *shape,
+                         n_tmax, s & 1, d_scratch, d_ranges);
+      MIST_HIP_CHECK(hipGetLastError());
+    }
   }
   return 0;
 }

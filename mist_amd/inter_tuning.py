@@ -201,7 +201,8 @@ class _DpRunner:
             packed[1].view(np.int32)[:] = g_index
             d_in = torch.from_numpy(packed).to(dev)
             d_out = torch.empty((3, n), dtype=torch.float32, device=dev)
-            scratch = torch.empty(4 * n * fam.plane, dtype=torch.float32, device=dev)
+            n_scratch = self.lib.mist_dp_scratch_floats(ctypes.c_void_p(fam.shape.ctypes.data), n)
+            scratch = torch.empty(n_scratch, dtype=torch.float32, device=dev)
             argmin = None
             if want_argmin:
                 argmin = torch.full((n, fam.S_max + 1, fam.L + 1, fam.D + 1, 4), -1,

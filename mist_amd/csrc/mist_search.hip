@@ -498,8 +498,8 @@ __device__ __forceinline__ void take_min(double &best, int32_t &best_row, bool f
 
 // ------------------------------------------------------------------------------------------
 // Kernel 2: evaluate + mask + running argmin.
-// Workgroup = 256 threads = one tile of (l, c) pairs; it streams candidate rows through LDS
-// and each thread keeps the minima of MIST_P_TILE pre-saved micro-batch values for its own
+// Workgroup = one wavefront = one tile of 64 (l, c) pairs; it streams candidate rows through LDS
+// and each lane keeps the minima of MIST_P_TILE pre-saved micro-batch values for its own
 // (l, c).  No cross-lane reduction is needed: the reduction axis (rows) is the loop.
 //
 // Memory feasibility is monotone in p: the peaks are built from p * (non-negative) terms by
@@ -513,7 +513,9 @@ __device__ __forceinline__ void take_min(double &best, int32_t &best_row, bool f
 // Almost no row changes anything, so a stage of kStageRows rows goes through three sieves, each
 // keeping a per-lane bit mask of surviving rows so that a lane only pays for its own survivors
 // (a wave executes a sieve as often as its busiest lane, not once per row):
-//   A  objective value against the largest minimum (all rows, straight-line code);
+//   A  objective value against the minimum of the highest slot the stage can reach (a bound
+//      from the term-wise minimum of the stage's memory terms); evaluated transposed, a lane
+//      holding one ROW and the loop running over the tile's pairs;
 //   B  lowest improvable slot and the exact memory test at that slot (minima as of stage start:
 //      they only decrease afterwards, so nothing that could matter later is dropped);
 //   C  survivors in row order against the live minima: bisection for `count`, update.
@@ -1030,8 +1032,9 @@ __device__ __forceinline__ void reduce_block(
 }
 
 // scout != 0: kScoutSplit workgroups per (group, (l, c) tile, p tile) share every
-// scout_stride-th stage of the whole group, results in slab n_blocks + blockIdx.x.  scout == 0: one workgroup per row
-// chunk of such a tile, seeded from the scout's slab when the group has one.
+// scout_stride-th stage of the whole group, results in slab n_blocks + logical workgroup.
+// scout == 0: one workgroup per row chunk of such a tile, seeded from the scout's slabs when the
+// group has them.
 __global__ __launch_bounds__(MIST_LC_TILE, MIST_REDUCE_MIN_WAVES) void eval_reduce_kernel(
     const MistProblem prob, const MistGroupDesc *__restrict__ groups, int n_groups,
     const int32_t *__restrict__ block_prefix, int n_blocks,

@@ -140,8 +140,8 @@ def workspace_positions(n_par: int, n_pair: int, n_oo: int, n_ao: int) -> np.nda
 
 
 def exported_symbols():
-    """Names every entry point declared in include/mist_search.h and include/mist_dp.h."""
-    return tuple(_SIGNATURES) + tuple(_DP_SIGNATURES)
+    """Names every entry point declared in include/mist_search.h, mist_dp.h and mist_mip.h."""
+    return tuple(_SIGNATURES) + tuple(_DP_SIGNATURES) + tuple(_MIP_SIGNATURES)
 
 
 DP_SHAPE_DTYPE = np.dtype(
@@ -187,6 +187,46 @@ _DP_SIGNATURES = {
 }
 
 
+MIP_CKPT_TUNED, MIP_CKPT_FIXED, MIP_CKPT_FULL = 0, 1, 2
+MIP_MAX_SAMPLES = 64
+MIP_MAX_VALUE = 1000000.0
+
+
+class MipShape(ctypes.Structure):
+    """``MistMipShape`` of include/mist_mip.h."""
+
+    _fields_ = [
+        ("num_layers", ctypes.c_int32),
+        ("p_dim", ctypes.c_int32),
+        ("sample_size", ctypes.c_int32),
+        ("num_stages", ctypes.c_int32),
+        ("layers_min", ctypes.c_int32),
+        ("layers_max", ctypes.c_int32),
+        ("ckpt_mode", ctypes.c_int32),
+        ("fixed_ckpt", ctypes.c_int32),
+    ]
+
+
+class MipTables(ctypes.Structure):
+    """``MistMipTables``: device pointers of one (gradient accumulation, mesh) slice."""
+
+    _fields_ = [("stable", ctypes.c_void_p * 4), ("delta", ctypes.c_void_p * 4)]
+
+
+_MIP_SIGNATURES = {
+    "mist_sizeof_mip_shape": (ctypes.c_int, []),
+    "mist_mip_stage_samples": (
+        ctypes.c_int,
+        [ctypes.POINTER(MipShape), ctypes.POINTER(MipTables), _VP, _VP, _VP, _VP, _VP, _VP],
+    ),
+    "mist_mip_solve": (
+        ctypes.c_int,
+        [ctypes.POINTER(MipShape), ctypes.c_int, ctypes.c_double, _VP, _VP, _VP,
+         ctypes.POINTER(ctypes.c_double), _VP, _VP],
+    ),
+}
+
+
 def load():
     """Loads the shared library once; raises if it has not been built."""
     global _LIB
@@ -198,7 +238,7 @@ def load():
             "(there is no CPU fallback for the search kernels)"
         )
     lib = ctypes.CDLL(LIB_PATH)
-    for name, (restype, argtypes) in {**_SIGNATURES, **_DP_SIGNATURES}.items():
+    for name, (restype, argtypes) in {**_SIGNATURES, **_DP_SIGNATURES, **_MIP_SIGNATURES}.items():
         fn = getattr(lib, name)
         fn.restype = restype
         fn.argtypes = argtypes
@@ -209,6 +249,10 @@ def load():
     if lib.mist_sizeof_dp_shape() != DP_SHAPE_DTYPE.itemsize:
         raise MistLibraryError(
             f"MistDpShape layout mismatch: C {lib.mist_sizeof_dp_shape()} vs numpy {DP_SHAPE_DTYPE.itemsize}"
+        )
+    if lib.mist_sizeof_mip_shape() != ctypes.sizeof(MipShape):
+        raise MistLibraryError(
+            f"MistMipShape layout mismatch: C {lib.mist_sizeof_mip_shape()} vs ctypes {ctypes.sizeof(MipShape)}"
         )
     if lib.mist_sizeof_group() != GROUP_DTYPE.itemsize:
         raise MistLibraryError(

@@ -1,0 +1,250 @@
+// Stage-assignment search of the `uniform-device-pp-mip` granularity
+// (reference: mist/analyzer/inter_tuning_mip.py).
+//
+//   stage_samples_kernel  one workgroup (one wavefront) per (stage, layer count): stages the
+//                         candidate row in LDS as float32 pairs, lane a scans it for sample a,
+//                         then the lanes compare their picks to drop repeated pairs.
+//   mist_mip_solve        host: exact optimum of the assignment the reference gives to CBC.
+//
+// Why the host solver is exact.  For fixed stage choices let Z_0 = 0, Z_{i+1} = T_i + max(Z_i,
+// D_i).  By induction Z_i = sum_{i'<i} T_i' + max(0, max_{i'<i} (D_i' - sum_{i''<i'} T_i'')), so
+// Z_S is the objective without its (G - 1) * max T term.  Z_{i+1} grows with Z_i, hence the
+// smallest Z per (stages done, layers used) is all a recurrence over the stages has to keep.
+// The optimum's max T equals one of the entry values: for every such value tau (ascending) the
+// recurrence runs over the entries with T <= tau and (G - 1) * tau + Z_S is a candidate total.
+#include <algorithm>
+#include <cmath>
+#include <cstdint>
+#include <limits>
+#include <vector>
+
+#include "mist_common.h"
+#include "mist_mip.h"
+
+using mist::fail;
+
+namespace {
+
+constexpr int kSampleLanes = 64;
+
+struct StageRow {
+  const double *stable, *delta;  // first candidate of the row, nullptr = every candidate +inf
+};
+
+// Table row of stage `stage` holding `layers` layers (inter_tuning_mip.py:453-468; later
+// assignments there overwrite earlier ones, which fixes the order of the tests below).
+__device__ StageRow stage_row(const MistMipShape &s, const MistMipTables &t, int stage,
+                              int layers) {
+  const int64_t L = s.num_layers, P = s.sample_size;
+  const int64_t row = (L + 1) * P;  // one (ckpt, policy) plane
+  if (stage == 0 && layers == L) return {t.stable[3], t.delta[3]};
+  if (stage == s.num_stages - 1) {
+    const int64_t off = (int64_t)(layers - 1) * row;
+    return {t.stable[2] + off, t.delta[2] + off};
+  }
+  const int p = s.num_stages - stage - 1;  // pre-saved micro-batches of this stage
+  if (p >= s.p_dim) return {nullptr, nullptr};
+  const int64_t off = ((int64_t)p * L + (layers - 1)) * row;
+  const int v = stage == 0 ? 1 : 0;
+  return {t.stable[v] + off, t.delta[v] + off};
+}
+
+__global__ __launch_bounds__(kSampleLanes) void stage_samples_kernel(
+    MistMipShape shape, MistMipTables tables, const double *__restrict__ ratios,
+    float *__restrict__ out_stable, float *__restrict__ out_delta, int32_t *__restrict__ out_index,
+    uint8_t *__restrict__ out_keep) {
+  extern __shared__ float lds[];
+  const int P = shape.sample_size, L = shape.num_layers;
+  const int nl = shape.layers_max - shape.layers_min + 1;
+  const int stage = blockIdx.x / nl, layers = shape.layers_min + blockIdx.x % nl;
+  const int lane = threadIdx.x;
+
+  int n_cand = P, first = 0;  // candidates of the row: all planes, or one ckpt plane
+  if (shape.ckpt_mode == MIST_MIP_CKPT_TUNED) n_cand = (L + 1) * P;
+  else if (shape.ckpt_mode == MIST_MIP_CKPT_FIXED) first = shape.fixed_ckpt * P;
+  else first = layers * P;
+
+  float *x = lds, *y = lds + n_cand;
+  float *pick_x = y + n_cand, *pick_y = pick_x + kSampleLanes;
+  const StageRow row = stage_row(shape, tables, stage, layers);
+  for (int n = lane; n < n_cand; n += kSampleLanes) {
+    x[n] = row.stable ? (float)row.stable[first + n] : INFINITY;
+    y[n] = row.delta ? (float)row.delta[first + n] : INFINITY;
+  }
+  __syncthreads();
+
+  int best = -1;
+  float sx = 0.0f, sy = 0.0f;
+  if (lane < P) {
+    const double r = ratios[lane];
+    double best_cost = INFINITY;
+    for (int n = 0; n < n_cand; ++n) {
+      const double cost = r * (double)x[n] + (double)y[n];
+      if (cost < best_cost) {
+        best_cost = cost;
+        best = n;
+      }
+    }
+    // numpy reads index -1 as the last candidate (pareto.py:76-77)
+    sx = x[best >= 0 ? best : n_cand - 1];
+    sy = y[best >= 0 ? best : n_cand - 1];
+    pick_x[lane] = sx;
+    pick_y[lane] = sy;
+  }
+  __syncthreads();
+  if (lane >= P) return;
+  bool keep = true;
+  for (int a = 0; a < lane; ++a) keep = keep && !(pick_x[a] == sx && pick_y[a] == sy);
+  if (!keep) sx = sy = INFINITY;
+  if (sx < 0.0f) sx = 0.0f;
+  if (sy < 0.0f) sy = 0.0f;
+  if (sx == INFINITY) sx = MIST_MIP_MAX_VALUE;
+  if (sy == INFINITY) sy = MIST_MIP_MAX_VALUE;
+  const int64_t o = (int64_t)blockIdx.x * P + lane;
+  out_stable[o] = sx;
+  out_delta[o] = sy;
+  out_index[o] = best;
+  out_keep[o] = keep ? 1 : 0;
+}
+
+int check_mip_shape(const MistMipShape *s) {
+  if (!s) return fail(MIST_E_INVALID, "null MistMipShape");
+  if (s->num_layers < 1 || s->num_stages < 1 || s->num_stages > s->num_layers)
+    return fail(MIST_E_INVALID, "num_stages %d outside [1, num_layers %d]", s->num_stages,
+                s->num_layers);
+  if (s->sample_size < 1 || s->sample_size > MIST_MIP_MAX_SAMPLES)
+    return fail(MIST_E_INVALID, "sample_size %d outside [1, %d]", s->sample_size,
+                MIST_MIP_MAX_SAMPLES);
+  if (s->layers_min < 1 || s->layers_max > s->num_layers)
+    return fail(MIST_E_INVALID, "layer counts %d..%d outside [1, %d]", s->layers_min,
+                s->layers_max, s->num_layers);
+  if (s->p_dim < 1) return fail(MIST_E_INVALID, "p_dim %d < 1", s->p_dim);
+  if (s->ckpt_mode < MIST_MIP_CKPT_TUNED || s->ckpt_mode > MIST_MIP_CKPT_FULL)
+    return fail(MIST_E_INVALID, "unknown ckpt_mode %d", s->ckpt_mode);
+  if (s->ckpt_mode == MIST_MIP_CKPT_FIXED && (s->fixed_ckpt < 0 || s->fixed_ckpt > s->num_layers))
+    return fail(MIST_E_INVALID, "fixed_ckpt %d outside [0, %d]", s->fixed_ckpt, s->num_layers);
+  return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mist_sizeof_mip_shape(void) { return (int)sizeof(MistMipShape); }
+
+int mist_mip_stage_samples(const MistMipShape *shape, const MistMipTables *tables,
+                           const double *d_ratios, float *d_t_stable, float *d_t_delta,
+                           int32_t *d_index, uint8_t *d_keep, void *stream) {
+  if (int rc = check_mip_shape(shape)) return rc;
+  if (shape->layers_min > shape->layers_max) return 0;  // no layer count to sample
+  if (!tables || !d_ratios || !d_t_stable || !d_t_delta || !d_index || !d_keep)
+    return fail(MIST_E_INVALID, "null pointer");
+  for (int v = 0; v < 4; ++v)
+    if (!tables->stable[v] || !tables->delta[v])
+      return fail(MIST_E_INVALID, "null table of variant %d", v);
+  const int64_t n_cand = shape->ckpt_mode == MIST_MIP_CKPT_TUNED
+                             ? (int64_t)(shape->num_layers + 1) * shape->sample_size
+                             : shape->sample_size;
+  const int64_t lds_bytes = (2 * n_cand + 2 * kSampleLanes) * (int64_t)sizeof(float);
+  if (lds_bytes > 64 * 1024)
+    return fail(MIST_E_INVALID, "%lld candidates per table row exceed the LDS staging buffer",
+                (long long)n_cand);
+  const int nl = shape->layers_max - shape->layers_min + 1;
+  hipLaunchKernelGGL(stage_samples_kernel, dim3((unsigned)(shape->num_stages * nl)),
+                     dim3(kSampleLanes), (size_t)lds_bytes, (hipStream_t)stream, *shape, *tables,
+                     d_ratios, d_t_stable, d_t_delta, d_index, d_keep);
+  MIST_HIP_CHECK(hipGetLastError());
+  return 0;
+}
+
+int mist_mip_solve(const MistMipShape *shape, int grad_accum, double best_cost,
+                   const float *t_stable, const float *t_delta, const uint8_t *keep,
+                   double *out_cost, int32_t *out_layers, int32_t *out_slot) {
+  if (int rc = check_mip_shape(shape)) return rc;
+  if (grad_accum < 1) return fail(MIST_E_INVALID, "grad_accum %d < 1", grad_accum);
+  if (!out_cost || !out_layers || !out_slot) return fail(MIST_E_INVALID, "null output");
+  const double inf = std::numeric_limits<double>::infinity();
+  *out_cost = inf;
+  if (shape->layers_min > shape->layers_max) return 0;
+  if (!t_stable || !t_delta || !keep) return fail(MIST_E_INVALID, "null pointer");
+  const int S = shape->num_stages, L = shape->num_layers, P = shape->sample_size;
+  const int lo = shape->layers_min, nl = shape->layers_max - lo + 1;
+  const int per_stage = nl * P;
+
+  std::vector<double> z((size_t)(S + 1) * (L + 1));
+  std::vector<int32_t> back((size_t)S * (L + 1));
+  std::vector<int32_t> picks((size_t)S);
+  // Smallest Z_S[L] over kept entries with T <= tau; fills `picks` (entry index per stage).
+  auto chain = [&](double tau) -> double {
+    std::fill(z.begin(), z.end(), inf);
+    z[0] = 0.0;
+    for (int i = 0; i < S; ++i) {
+      const double *prev = &z[(size_t)i * (L + 1)];
+      double *cur = &z[(size_t)(i + 1) * (L + 1)];
+      const int64_t base = (int64_t)i * per_stage;
+      for (int m = 0; m <= L; ++m) {
+        double best = inf;
+        int32_t arg = -1;
+        for (int a = 0; a < nl; ++a) {
+          const int from = m - (lo + a);
+          if (from < 0) break;
+          const double zp = prev[from];
+          if (!(zp < inf)) continue;
+          for (int k = 0; k < P; ++k) {
+            const int64_t e = base + (int64_t)a * P + k;
+            const double t = (double)t_stable[e];
+            if (!keep[e] || !(t <= tau)) continue;
+            const double cand = t + std::max(zp, (double)t_delta[e]);
+            if (cand < best) {
+              best = cand;
+              arg = (int32_t)(a * P + k);
+            }
+          }
+        }
+        cur[m] = best;
+        back[(size_t)i * (L + 1) + m] = arg;
+      }
+    }
+    const double total = z[(size_t)S * (L + 1) + L];
+    if (!(total < inf)) return inf;
+    int m = L;
+    for (int i = S - 1; i >= 0; --i) {
+      const int32_t arg = back[(size_t)i * (L + 1) + m];
+      picks[i] = arg;
+      m -= lo + arg / P;
+    }
+    return total;
+  };
+  auto emit = [&](double cost) {
+    *out_cost = cost;
+    for (int i = 0; i < S; ++i) {
+      out_layers[i] = lo + picks[i] / P;
+      out_slot[i] = picks[i] % P;
+    }
+  };
+
+  const double z_free = chain(inf);
+  if (!(z_free < inf)) return 0;
+  if (grad_accum == 1) {
+    emit(z_free);
+    return 1;
+  }
+  std::vector<double> taus;
+  for (int64_t e = 0; e < (int64_t)S * per_stage; ++e)
+    if (keep[e] && std::isfinite(t_stable[e])) taus.push_back((double)t_stable[e]);
+  std::sort(taus.begin(), taus.end());
+  taus.erase(std::unique(taus.begin(), taus.end()), taus.end());
+  double best = inf;
+  for (double tau : taus) {
+    const double weight = (double)(grad_accum - 1) * tau;
+    if (weight > best_cost || weight + z_free >= best) break;
+    const double zs = chain(tau);
+    if (zs < inf && weight + zs < best) {
+      best = weight + zs;
+      emit(best);
+    }
+  }
+  return best < inf ? 1 : 0;
+}
+
+}  // extern "C"

@@ -7,13 +7,15 @@ evaluation running on the GPU.  Differences, all forced by what the path needs h
 * the three traced ``LayerInfo`` objects are replaced by ``LayerTables`` (closed-form tables);
 * hydra / omegaconf are not used: ``main`` takes ``--config <yaml>`` plus ``key=value``
   overrides, and the YAML written is produced with PyYAML;
-* ``tuning_granularity``: ``inter-stage`` (the per-mesh DP), ``uniform-device-pp`` (the DP with
-  one uniform mesh per stage count), ``uniform-pp``, ``uniform-pp-simple-heuristic-mem-opt`` and
-  ``no-pp`` are implemented.  The reference's ``inter-stage``, ``uniform-device-pp`` and ``no-pp``
-  branches call ``intra_stage_tune`` without the required ``tp_size`` and read cost fields that
-  no longer exist; here they cover the tensor-parallel candidates like the working branches
-  (:199-203), use the stable/delta adapter and take ``tuning.sample_size`` samples (slot 0).
-  ``uniform-device-pp-mip`` (external MILP solver) raises ``NotImplementedError``.
+* ``tuning_granularity``: every value of the reference is implemented: ``inter-stage`` (the
+  per-mesh DP), ``uniform-device-pp`` (the DP with one uniform mesh per stage count),
+  ``uniform-device-pp-mip`` (the stage assignment over sampled policies; an exact solver in the
+  library stands in for the external MILP solver), ``uniform-pp``,
+  ``uniform-pp-simple-heuristic-mem-opt`` and ``no-pp``.  The reference's ``inter-stage``,
+  ``uniform-device-pp`` and ``no-pp`` branches call ``intra_stage_tune`` without the required
+  ``tp_size`` and read cost fields that no longer exist; here they cover the tensor-parallel
+  candidates like the working branches (:199-203), use the stable/delta adapter and take
+  ``tuning.sample_size`` samples (slot 0).
 """
 from __future__ import annotations
 
@@ -33,6 +35,7 @@ from .config import OFFLOADING_RATIO_CANDIDATES, MistConfig, tp_candidates
 from .inter_tuning import inter_stage_tune, inter_stage_tune_batch
 from .inter_tuning_uniform import inter_stage_tune as inter_stage_tune_uniform
 from .inter_tuning_uniform_device import inter_stage_tune_batch_uniform_device
+from .inter_tuning_mip import inter_stage_tune as inter_stage_tune_mip
 from .intra_tuning import SAMPLE_SIZE, IntraStageTuner, intra_stage_tune
 from .layer_tables import LayerTables
 from .search_space import _get_device_mesh_candidates, _get_grad_accumu_steps_candidates
@@ -92,6 +95,31 @@ def _no_pp(mist_config, tables, device, stats):
             ckpt = int(idx[2]) if tuning.activation_checkpointing_tuning_enabled else L
             best_cost = float(costs[idx])
             best_solution = [Gs[idx[0]], [(((0, L - 1), meshes[idx[1]], ckpt, 0), tuple(row))]]
+    return best_cost, best_solution
+
+
+def _uniform_device_pp_mip(mist_config, device, stats):
+    """tune_one_case.py:360-402: per tensor-parallel candidate the intra-stage tables with every
+    one of ``tuning.sample_size`` samples, then the stage assignment; the first best tp wins.
+    One tp at a time keeps a single set of sampled tables in HBM."""
+    hw, tuning = mist_config.hardware, mist_config.tuning
+    tables = LayerTables(mist_config)
+    meshes = _get_device_mesh_candidates(hw.num_nodes, hw.num_gpus_per_node, contiguous_inter_node=False)
+    Gs = _get_grad_accumu_steps_candidates(mist_config.training.global_batch_size)
+    L = mist_config.model.num_hidden_layers
+    best_cost, best_solution = float("inf"), None
+    for tp_size in tp_candidates(mist_config):
+        t0 = time.perf_counter()
+        r = intra_stage_tune(tables, L, meshes, Gs, tp_size, mist_config,
+                             sample_size=tuning.sample_size, device=device)
+        t1 = time.perf_counter()
+        cost, solution = inter_stage_tune_mip(
+            L, hw.num_nodes, hw.num_gpus_per_node, meshes, Gs, r, mist_config, stats=stats)
+        stats["intra_s"] = stats.get("intra_s", 0.0) + (t1 - t0)
+        stats["inter_s"] = stats.get("inter_s", 0.0) + (time.perf_counter() - t1)
+        if cost < best_cost:
+            best_cost, best_solution = cost, solution
+        del r
     return best_cost, best_solution
 
 
@@ -189,10 +217,7 @@ def tune(mist_config: MistConfig, device: str = "cuda:0", stats: Optional[dict] 
             if cost < best_cost:
                 best_cost, best_solution = cost, solution
     elif granularity == "uniform-device-pp-mip":
-        raise NotImplementedError(
-            f"tuning_granularity '{granularity}' is not part of the GPU search path "
-            "(it hands the stage tables to an external MILP solver)"
-        )
+        best_cost, best_solution = _uniform_device_pp_mip(mist_config, device, stats)
     else:
         raise ValueError(f"Unknown tuning granularity: {granularity}")
     stats["tune_s"] = time.perf_counter() - t_start

@@ -8,6 +8,7 @@ tensor-parallel candidates, strict ``<`` keeps the first best) with the inter-st
 from .dp_c import dp_impl_c
 from .inter_dp import dp_impl, inter_stage_tune
 from .inter_uniform import inter_stage_tune_uniform
+from .inter_mip import inter_stage_tune as inter_stage_tune_mip
 from .inter_uniform_device import inter_stage_tune as inter_stage_tune_uniform_device
 from .intra import intra_stage_tune
 from .search_space import device_mesh_candidates, grad_accumu_steps_candidates
@@ -37,6 +38,9 @@ def tune(config, tables, use_c_dp=True):
             r = intra_stage_tune(tables, config, L, meshes, Gs, tp, config.tuning.sample_size)
             cost, sol = inter_stage_tune_uniform_device(
                 L, hw.num_nodes, hw.num_gpus_per_node, meshes, Gs, r, config, slot=0)
+        elif gran == "uniform-device-pp-mip":
+            r = intra_stage_tune(tables, config, L, meshes, Gs, tp, config.tuning.sample_size)
+            cost, sol = inter_stage_tune_mip(L, hw.num_nodes, hw.num_gpus_per_node, meshes, Gs, r, config)
         elif gran in ("uniform-pp", "uniform-pp-simple-heuristic-mem-opt"):
             r = intra_stage_tune(tables, config, L, meshes, Gs, tp, 30)
             cost, sol = inter_stage_tune_uniform(

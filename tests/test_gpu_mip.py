@@ -1,0 +1,222 @@
+"""GPU parity of the ``uniform-device-pp-mip`` path: the sampling kernel against the oracle's
+preprocessing (bit for bit), the end-to-end tuner against the oracle, and at full size the
+invariants the assignment must satisfy."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from tests.util import load_plan, tiny_plan
+
+pytestmark = pytest.mark.gpu
+
+
+def _random_tables(rng, P1, L, P, inf_frac=0.2, quantum=None, neg_frac=0.0):
+    shapes = [(P1, L, L + 1, P), (P1, L, L + 1, P), (L, L + 1, P), (L + 1, P)]
+    stable, delta = [], []
+    for shape in shapes:
+        s = rng.uniform(0.05, 1.0, size=shape)
+        d = rng.uniform(0.05, 1.0, size=shape)
+        if quantum:
+            s, d = np.round(s / quantum) * quantum, np.round(d / quantum) * quantum
+        bad = rng.random(shape[:-1]) < inf_frac
+        tail = rng.random(shape) < inf_frac / 2
+        s[bad], d[bad] = np.inf, np.inf
+        s[tail], d[tail] = np.inf, np.inf
+        if neg_frac:
+            d[(rng.random(shape) < neg_frac) & np.isfinite(d)] *= -1
+        stable.append(s)
+        delta.append(d)
+    return stable, delta
+
+
+def _gpu_samples(stable, delta, S, lo, hi, mode, fixed):
+    import torch
+    from mist_amd import _lib
+    from mist_amd.intra_tuning import alpha_ratios
+
+    lib = _lib.load()
+    P1, L, _, P = stable[0].shape
+    dev_s = [torch.from_numpy(np.ascontiguousarray(t)).cuda() for t in stable]
+    dev_d = [torch.from_numpy(np.ascontiguousarray(t)).cuda() for t in delta]
+    tabs = _lib.MipTables()
+    for v in range(4):
+        tabs.stable[v], tabs.delta[v] = dev_s[v].data_ptr(), dev_d[v].data_ptr()
+    shape = _lib.MipShape(num_layers=L, p_dim=P1, sample_size=P, num_stages=S, layers_min=lo,
+                          layers_max=hi, ckpt_mode=mode, fixed_ckpt=fixed)
+    n = S * (hi - lo + 1) * P
+    ratios = torch.from_numpy(alpha_ratios(P)).cuda()
+    ts = torch.empty(n, dtype=torch.float32).cuda()
+    td = torch.empty(n, dtype=torch.float32).cuda()
+    ix = torch.empty(n, dtype=torch.int32).cuda()
+    kp = torch.empty(n, dtype=torch.uint8).cuda()
+    rc = lib.mist_mip_stage_samples(
+        ctypes.byref(shape), ctypes.byref(tabs), ratios.data_ptr(), ts.data_ptr(), td.data_ptr(),
+        ix.data_ptr(), kp.data_ptr(), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    _lib.check(rc, "mist_mip_stage_samples")
+    torch.cuda.synchronize()
+    dims = (S, hi - lo + 1, P)
+    return (ts.cpu().numpy().reshape(dims), td.cpu().numpy().reshape(dims),
+            ix.cpu().numpy().reshape(dims), kp.cpu().numpy().reshape(dims))
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2])
+@pytest.mark.parametrize("L,P1,P,quantum", [(5, 3, 4, 0.125), (12, 6, 9, None), (32, 8, 30, 0.03125)])
+def test_sampling_kernel_matches_oracle_preprocessing(mode, L, P1, P, quantum):
+    from oracle import inter_mip
+
+    rng = np.random.default_rng(L * 10 + mode)
+    fixed = L // 2
+    for S in sorted({1, 2, 3, min(P1 + 1, L), L}):
+        stable, delta = _random_tables(rng, P1, L, P, quantum=quantum, neg_frac=0.03)
+        f32 = lambda a: a.astype(np.float32)
+        choices, want_s, want_d, (ck, pol) = inter_mip.preprocess_stable_and_delta_costs(
+            S, mode == 0, fixed if mode == 1 else None,
+            f32(stable[0]), f32(delta[0]), f32(stable[1]), f32(delta[1]),
+            f32(stable[2]), f32(delta[2]), f32(stable[3]), f32(delta[3]))
+        lo, hi = 1, L   # every layer count, more than the search itself asks for
+        got_s, got_d, got_i, got_k = _gpu_samples(stable, delta, S, lo, hi, mode, fixed)
+        assert np.array_equal(got_s, want_s[:, lo:hi + 1]), (S, "stable")
+        assert np.array_equal(got_d, want_d[:, lo:hi + 1]), (S, "delta")
+        want_k = np.zeros_like(got_k)
+        for i in range(S):
+            for j in range(lo, hi + 1):
+                want_k[i, j - lo, choices[i][j]] = 1
+        assert np.array_equal(got_k, want_k), (S, "keep")
+        if mode == 0:
+            assert np.array_equal(got_i // P, ck[:, lo:hi + 1]) and np.array_equal(got_i % P, pol[:, lo:hi + 1])
+        else:
+            assert np.array_equal(got_i, pol[:, lo:hi + 1])
+
+
+def test_sampling_kernel_rejects_bad_arguments():
+    import torch
+    from mist_amd import _lib
+
+    lib = _lib.load()
+    buf = torch.zeros(4096, dtype=torch.float64).cuda()
+    tabs = _lib.MipTables()
+    for v in range(4):
+        tabs.stable[v], tabs.delta[v] = buf.data_ptr(), buf.data_ptr()
+    args = (buf.data_ptr(),) * 5 + (None,)
+    big = _lib.MipShape(num_layers=400, p_dim=2, sample_size=64, num_stages=2, layers_min=1,
+                        layers_max=3, ckpt_mode=0, fixed_ckpt=0)
+    assert lib.mist_mip_stage_samples(ctypes.byref(big), ctypes.byref(tabs), *args) == -1
+    assert b"LDS" in lib.mist_last_error()
+    bad = _lib.MipShape(num_layers=8, p_dim=2, sample_size=4, num_stages=9, layers_min=1,
+                        layers_max=3, ckpt_mode=0, fixed_ckpt=0)
+    assert lib.mist_mip_stage_samples(ctypes.byref(bad), ctypes.byref(tabs), *args) == -1
+    tabs.delta[2] = None
+    ok = _lib.MipShape(num_layers=8, p_dim=2, sample_size=4, num_stages=2, layers_min=1,
+                       layers_max=3, ckpt_mode=0, fixed_ckpt=0)
+    assert lib.mist_mip_stage_samples(ctypes.byref(ok), ctypes.byref(tabs), *args) == -1
+
+
+@pytest.mark.parametrize(
+    "overrides",
+    [
+        dict(hardware__num_nodes=2, hardware__num_gpus_per_node=4, training__global_batch_size=32,
+             hardware__memory_capacity=8.0, tuning__sample_size=4),
+        dict(hardware__memory_capacity=5.0, tuning__sample_size=6),
+        dict(hardware__num_nodes=1, hardware__num_gpus_per_node=4, training__global_batch_size=16,
+             hardware__memory_capacity=6.0, tuning__sample_size=3,
+             tuning__activation_checkpointing_tuning_enabled=False),
+        dict(hardware__num_nodes=1, hardware__num_gpus_per_node=4, training__global_batch_size=16,
+             hardware__memory_capacity=6.0, tuning__sample_size=3, fixed_ckpt_value=2,
+             tuning__activation_checkpointing_tuning_enabled=False),
+    ],
+)
+def test_mip_tune_end_to_end_matches_oracle(overrides):
+    """YAML in, best strategy out.  The oracle solves the assignment with the same exact method
+    and tie rule, on tables the kernels reproduce bit for bit: cost and solution are identical."""
+    from mist_amd.tune_one_case import tune
+    from oracle.tune import tune as oracle_tune
+
+    cfg, tables = tiny_plan(1, layers=6, tuning__tuning_granularity="uniform-device-pp-mip", **overrides)
+    got = tune(cfg)
+    want = oracle_tune(cfg, tables)
+    assert want[1] is not None, "degenerate case"
+    assert got == want
+
+
+def test_mip_infeasible_plan_returns_inf_none():
+    from mist_amd.tune_one_case import tune
+    from oracle.tune import tune as oracle_tune
+
+    cfg, tables = tiny_plan(1, layers=4, hardware__memory_capacity=0.2, tuning__sample_size=3,
+                            tuning__tuning_granularity="uniform-device-pp-mip")
+    assert tune(cfg) == (float("inf"), None)
+    assert oracle_tune(cfg, tables) == (float("inf"), None)
+
+
+def test_mip_needs_every_sample():
+    from mist_amd.inter_tuning_mip import inter_stage_tune
+    from mist_amd.intra_tuning import IntraStageTuner
+    from mist_amd.search_space import _get_device_mesh_candidates, _get_grad_accumu_steps_candidates
+
+    cfg, tables = tiny_plan(1, layers=4)
+    hw = cfg.hardware
+    meshes = _get_device_mesh_candidates(hw.num_nodes, hw.num_gpus_per_node, False)
+    Gs = _get_grad_accumu_steps_candidates(cfg.training.global_batch_size)
+    res = IntraStageTuner(tables, 4, meshes, Gs, 1, cfg, sample_size=3, sample_slots=[0]).tune()
+    with pytest.raises(ValueError, match="every sample"):
+        inter_stage_tune(4, hw.num_nodes, hw.num_gpus_per_node, meshes, Gs, res, cfg)
+    with pytest.raises(TypeError):
+        inter_stage_tune(4, hw.num_nodes, hw.num_gpus_per_node, meshes, Gs, object(), cfg)
+
+
+def _check_solution_invariants(cfg, cost, solution):
+    """Size-independent checks of a returned strategy: stages tile the layers, all stages use
+    the uniform mesh of their count, and the cost equals the objective recomputed from the
+    float32 stage times of the chosen table cells."""
+    from mist_amd.inter_tuning_uniform import _uniform_device_mesh_partition
+
+    L, hw = cfg.model.num_hidden_layers, cfg.hardware
+    G, stages = solution
+    S = len(stages)
+    mesh = _uniform_device_mesh_partition(S, hw.num_nodes, hw.num_gpus_per_node)
+    covered = 0
+    for (span, stage_mesh, ckpt, policy), row in stages:
+        assert span[0] == covered and span[1] >= span[0]
+        covered = span[1] + 1
+        assert tuple(stage_mesh) == tuple(mesh)
+        assert 0 <= ckpt <= L and 0 <= policy < cfg.tuning.sample_size
+        assert np.all(np.isfinite(row)) and len(row) == 10
+    assert covered == L
+    return G, S, mesh
+
+
+@pytest.mark.parametrize("plan", [1, 2])
+def test_mip_full_size_invariants(plan):
+    """Plan 1 and the GPT-7B plan at their real sizes with 30 samples per cell."""
+    from mist_amd.inter_tuning_mip import inter_stage_tune
+    from mist_amd.intra_tuning import IntraStageTuner
+    from mist_amd.search_space import _get_device_mesh_candidates, _get_grad_accumu_steps_candidates
+    from oracle.inter_mip import MAX_VALUE, objective
+
+    cfg, tables = load_plan(plan, tuning__tuning_granularity="uniform-device-pp-mip",
+                            tuning__sample_size=30)
+    hw, L = cfg.hardware, cfg.model.num_hidden_layers
+    meshes = _get_device_mesh_candidates(hw.num_nodes, hw.num_gpus_per_node, False)
+    Gs = _get_grad_accumu_steps_candidates(cfg.training.global_batch_size)
+    tp = 1 if plan == 1 else 2
+    res = IntraStageTuner(tables, L, meshes, Gs, tp, cfg, sample_size=30).tune()
+    cost, solution = inter_stage_tune(L, hw.num_nodes, hw.num_gpus_per_node, meshes, Gs, res, cfg)
+    assert solution is not None and cost < MAX_VALUE
+    G, S, mesh = _check_solution_invariants(cfg, cost, solution)
+    g, q = Gs.index(G), meshes.index(mesh)
+    T, D = [], []
+    for i, ((span, _, ckpt, policy), row) in enumerate(solution[1]):
+        l, p = span[1] - span[0] + 1, S - i - 1
+        if S == 1:
+            cell, v = (g, q, ckpt, policy), 3
+        elif i == 0:
+            cell, v = (g, q, p, l - 1, ckpt, policy), 1
+        elif i == S - 1:
+            cell, v = (g, q, l - 1, ckpt, policy), 2
+        else:
+            cell, v = (g, q, p, l - 1, ckpt, policy), 0
+        T.append(np.float32(res.device.stable[v][cell].item()))
+        D.append(max(np.float32(res.device.delta[v][cell].item()), np.float32(0)))
+        assert np.array_equal(res.solution_at(v, cell), np.asarray(row, dtype=np.float64))
+    assert objective(T, D, G) == pytest.approx(cost, rel=1e-12, abs=0)

@@ -154,18 +154,35 @@ def test_best_solution_yaml_format():
     assert out["model"] == raw["model"]
 
 
-def test_unsupported_granularities_raise():
+def test_mip_search_needs_the_gpu_library_path():
+    """The MIP granularity has no CPU path either: without a GPU the intra-stage tuner refuses."""
+    import torch
+
+    from mist_amd._lib import MistLibraryError
     from mist_amd.tune_one_case import tune
 
-    for gran in ("uniform-device-pp-mip",):
-        cfg, _ = load_plan(1, tuning__tuning_granularity=gran)
-        with pytest.raises(NotImplementedError):
-            tune(cfg)
+    if torch.cuda.is_available():
+        pytest.skip("covers the host without a GPU")
+    cfg, _ = load_plan(1, tuning__tuning_granularity="uniform-device-pp-mip")
+    with pytest.raises(MistLibraryError):
+        tune(cfg)
+
+
+def test_mip_layer_candidates_match_oracle():
+    from mist_amd.inter_tuning_mip import layer_candidates
+    from oracle.inter_mip import layer_candidates as want
+
+    for L in (1, 2, 7, 10, 14, 32, 80):
+        for S in range(1, L + 1):
+            for G in (1, 2, 64):
+                for off in (0, 1, 2, 3):
+                    lo, hi = layer_candidates(L, S, G, off)
+                    assert list(range(lo, hi + 1)) == want(L, S, G, off), (L, S, G, off)
 
 
 def _declared_functions():
     names = []
-    for header in ("mist_search.h", "mist_dp.h"):
+    for header in ("mist_search.h", "mist_dp.h", "mist_mip.h"):
         text = open(os.path.join(REPO, "include", header)).read()
         text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
         names += re.findall(r"\b(mist_[a-z0-9_]+)\s*\(", text)
@@ -205,9 +222,9 @@ def test_argument_checks_reject_before_any_launch():
     shape["num_layers"], shape["num_devices"], shape["num_mesh"], shape["p_dim"] = 8, 8, 2, 4
     shape["max_stages"] = 4
     shape["mesh_n"][0, :2], shape["mesh_m"][0, :2] = [1, 1], [1, 2]
-    assert lib.mist_dp_scratch_floats(ctypes.c_void_p(shape.ctypes.data), 4) == 4 * 4 * 9 * 9
+    assert lib.mist_dp_scratch_floats(ctypes.c_void_p(shape.ctypes.data), 4) == 4 * 4 * 9 * 9 + 2 * 4 * 9
     shape["num_layers"], shape["num_devices"] = 80, 256
-    assert lib.mist_dp_scratch_floats(ctypes.c_void_p(shape.ctypes.data), 4) == 4 * 4 * 81 * 257
+    assert lib.mist_dp_scratch_floats(ctypes.c_void_p(shape.ctypes.data), 4) == 4 * 4 * 81 * 257 + 2 * 4 * 257
     costs = _lib.DpCosts(4096, 4096, 4096, 4096, 4096, 4096, 4096, 4096)
     sp = ctypes.c_void_p(shape.ctypes.data)
     assert lib.mist_dp_run(sp, ctypes.byref(costs), fake, fake, 1, 0, fake, fake, fake, None, None, None) == -1

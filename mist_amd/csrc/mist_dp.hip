@@ -25,8 +25,11 @@ constexpr int kDpWideTeam = 8;  // lanes that share one DP state in small batche
 // ------------------------------------------------------------------------------------------
 // Adapter: float64 (stable, delta) tables -> float32 DP cost tables for every g.
 // ------------------------------------------------------------------------------------------
-// One thread per table row (fixed g, mesh, p, layers): the L+1 ckpt entries are converted in
-// order and their running minimum is stored alongside (pmin[j] = min(cost[0..j])).
+// Table rows (fixed g, mesh, p, layers) hold the L+1 ckpt entries: cost = (float)stable +
+// (float)delta / G, and alongside its running minimum pmin[j] = min(cost[0..j]).  A workgroup
+// takes as many whole rows as fit its 256 lanes, one lane per entry, so that loads and stores
+// are contiguous; the running minimum is read back from LDS.  Rows longer than the workgroup
+// are walked in passes of 256 entries with the minimum of the earlier passes carried along.
 __global__ __launch_bounds__(256) void cost_table_kernel(const double *__restrict__ stable,
                                                          const double *__restrict__ delta,
                                                          const int32_t *__restrict__ grad_accum,
@@ -34,18 +37,35 @@ __global__ __launch_bounds__(256) void cost_table_kernel(const double *__restric
                                                          int row_len, int sample_size, int slot,
                                                          float *__restrict__ out,
                                                          float *__restrict__ pmin) {
-  const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (r >= n_rows) return;
-  const float G = (float)grad_accum[r / rows_per_g];
-  float run = INFINITY;
-  for (int j = 0; j < row_len; ++j) {
+  __shared__ float lds[256];
+  const int seg = min(row_len, 256);  // entries of a row per pass
+  const int rows_here = 256 / seg;
+  const int local_row = threadIdx.x / seg, j0 = threadIdx.x % seg;
+  const int64_t r = (int64_t)blockIdx.x * rows_here + local_row;
+  const bool live_row = local_row < rows_here && r < n_rows;
+  const float G = live_row ? (float)grad_accum[r / rows_per_g] : 1.0f;
+  float carry = INFINITY;
+  for (int base = 0; base < row_len; base += seg) {
+    const int j = base + j0;
+    const bool live = live_row && j < row_len;
     const int64_t i = r * row_len + j;
-    const float s = (float)stable[i * sample_size + slot];
-    const float d = (float)delta[i * sample_size + slot];
-    const float c = s + d / G;
-    run = fminf(run, c);
-    out[i] = c;
-    pmin[i] = run;
+    float c = INFINITY;
+    if (live) {
+      const float s = (float)stable[i * sample_size + slot];
+      const float d = (float)delta[i * sample_size + slot];
+      c = s + d / G;
+      out[i] = c;
+    }
+    lds[threadIdx.x] = c;
+    __syncthreads();
+    if (live) {
+      float run = carry;
+      for (int a = threadIdx.x - j0; a <= (int)threadIdx.x; ++a) run = fminf(run, lds[a]);
+      pmin[i] = run;
+    }
+    if (base + seg < row_len)  // only rows longer than one pass
+      for (int a = 0; a < seg; ++a) carry = fminf(carry, lds[threadIdx.x - j0 + a]);
+    __syncthreads();
   }
 }
 
@@ -95,12 +115,25 @@ __global__ __launch_bounds__(256) void select_candidates_kernel(
 // ------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void dp_init_kernel(const MistDpShape shape, int n_tmax,
                                                       float *__restrict__ scratch,
+                                                      int32_t *__restrict__ ranges,
                                                       int32_t *__restrict__ best_s,
                                                       float *__restrict__ best_sum,
                                                       float *__restrict__ stage_max) {
   const int W = shape.num_devices + 1;
   const int plane = (shape.num_layers + 1) * W;
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < (int64_t)n_tmax * W) {
+    // Reachable start layers [first, last] per instance and device column, three buffers used
+    // in rotation by the steps.  F(0) is reachable at (k = L, d = 0) only.
+    const int64_t stride = (int64_t)n_tmax * W * 2;
+    const bool origin = i % W == 0;
+    ranges[2 * i] = origin ? shape.num_layers : shape.num_layers + 1;
+    ranges[2 * i + 1] = origin ? shape.num_layers : -1;
+    for (int b = 1; b < 3; ++b) {
+      ranges[b * stride + 2 * i] = shape.num_layers + 1;
+      ranges[b * stride + 2 * i + 1] = -1;
+    }
+  }
   if (i >= (int64_t)n_tmax * plane) return;
   const int t = (int)(i / plane), e = (int)(i % plane);
   float *state = scratch + (int64_t)t * 4 * plane;
@@ -114,33 +147,11 @@ __global__ __launch_bounds__(256) void dp_init_kernel(const MistDpShape shape, i
   }
 }
 
-// Rows of plane `which` (F of the stage count just finished) that are reachable, per instance
-// and device column: most states are not, and the next step only scans [first, last].
-__global__ __launch_bounds__(256) void dp_ranges_kernel(const MistDpShape shape, int n_tmax,
-                                                        int which, const float *__restrict__ scratch,
-                                                        int32_t *__restrict__ ranges) {
-  const int W = shape.num_devices + 1, L = shape.num_layers;
-  const int plane = (L + 1) * W;
-  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= (int64_t)n_tmax * W) return;
-  const int t = (int)(i / W), col = (int)(i % W);
-  const float *f = scratch + (int64_t)t * 4 * plane + (int64_t)which * plane + col;
-  int first = L + 1, last = -1;
-  for (int k = 0; k <= L; ++k) {
-    if (f[(int64_t)k * W] < INFINITY) {
-      first = min(first, k);
-      last = k;
-    }
-  }
-  ranges[2 * i] = first;
-  ranges[2 * i + 1] = last;
-}
-
 template <bool kBottleneck, int kDpTeam>
 __global__ __launch_bounds__(kDpThreads) void dp_step_kernel(
     const MistDpShape shape, const MistDpCosts tabs, const float *__restrict__ tmax_list,
     const int32_t *__restrict__ g_list, int s, float *__restrict__ scratch,
-    const int32_t *__restrict__ ranges, int32_t *__restrict__ best_s_out,
+    int32_t *__restrict__ ranges, int32_t *__restrict__ best_s_out,
     float *__restrict__ best_sum_out, float *__restrict__ stage_max_out,
     int32_t *__restrict__ argmin) {
   const int L = shape.num_layers, D = shape.num_devices, Q = shape.num_mesh;
@@ -172,6 +183,13 @@ __global__ __launch_bounds__(kDpThreads) void dp_step_kernel(
                           g * tabs.g_stride[3]};
   const int k = e / W, d = e % W;
   const int p = s - 1;
+  // Most states are unreachable.  Every step records, per instance and device column, the first
+  // and last start layer it reached (buffer s % 3); the next step scans only that range.  The
+  // buffer after that one is reset here: its last readers ran in the step before this one.
+  const int64_t range_stride = (int64_t)gridDim.y * W * 2;
+  const int32_t *range_prev = ranges + ((s + 2) % 3) * range_stride + (int64_t)t * W * 2;
+  int32_t *range_cur = ranges + (s % 3) * range_stride + (int64_t)t * W * 2;
+  int32_t *range_next = ranges + ((s + 1) % 3) * range_stride + (int64_t)t * W * 2;
 
   const bool free_devices = shape.free_devices != 0;
   const int rule = shape.ckpt_rule;
@@ -237,7 +255,7 @@ __global__ __launch_bounds__(kDpThreads) void dp_step_kernel(
       const int nm = free_devices ? 0 : shape.mesh_n[q] * shape.mesh_m[q];
       if (nm > d) continue;
       // reachable start layers i + 1 of the remaining stages on d - nm devices
-      const int32_t *reach = ranges + 2 * ((int64_t)t * W + (d - nm));
+      const int32_t *reach = range_prev + 2 * (d - nm);
       const int i_first = max(k, reach[0] - 1), i_last = min(L - 1, reach[1] - 1);
       for (int i = i_first + member; i <= i_last; i += kDpTeam) {
         const float prev = f_prev[(i + 1) * W + (d - nm)];
@@ -286,6 +304,14 @@ __global__ __launch_bounds__(kDpThreads) void dp_step_kernel(
   }
   f_cur[e] = best;
   m_cur[e] = best_m;
+  if (best < INFINITY) {
+    atomicMin(&range_cur[2 * d], k);
+    atomicMax(&range_cur[2 * d + 1], k);
+  }
+  if (k == 0) {
+    range_next[2 * d] = L + 1;
+    range_next[2 * d + 1] = -1;
+  }
   if (argmin != nullptr && arg_i >= 0) {
     int32_t *a = argmin + (((int64_t)t * (shape.max_stages + 1) + s) * plane + e) * 4;
     a[0] = arg_i;
@@ -348,7 +374,9 @@ int mist_dp_cost_tables(const MistProblem *problem, const MistOutTables *tables,
     if (!tables->stable[v] || !tables->delta[v] || !d_out[v] || !d_out_pmin[v])
       return fail(MIST_E_INVALID, "table %d is null", v);
     const int64_t n = Gn * rows_per_g[v];
-    hipLaunchKernelGGL(cost_table_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+    const int64_t rows_per_block = 256 / std::min<int64_t>(L + 1, 256);
+    hipLaunchKernelGGL(cost_table_kernel,
+                       dim3((unsigned)((n + rows_per_block - 1) / rows_per_block)), dim3(256), 0,
                        (hipStream_t)stream, tables->stable[v], tables->delta[v], d_grad_accum, n,
                        rows_per_g[v], (int)(L + 1), (int)S, slot, d_out[v], d_out_pmin[v]);
     MIST_HIP_CHECK(hipGetLastError());
@@ -391,9 +419,10 @@ int mist_dp_select_candidates(const MistDpCosts *costs, int n_requests, const in
 
 int64_t mist_dp_scratch_floats(const MistDpShape *shape, int n_tmax) {
   if (check_shape(shape) != 0 || n_tmax <= 0) return -1;
-  // four state planes per instance, then (first, last) reachable row per instance and column
+  // four state planes per instance, then three buffers of (first, last) reachable row per
+  // instance and device column
   return (int64_t)4 * n_tmax * (shape->num_layers + 1) * (shape->num_devices + 1) +
-         (int64_t)2 * n_tmax * (shape->num_devices + 1);
+         (int64_t)6 * n_tmax * (shape->num_devices + 1);
 }
 
 int mist_dp_run(const MistDpShape *shape, const MistDpCosts *costs, const float *d_tmax,
@@ -413,15 +442,10 @@ int mist_dp_run(const MistDpShape *shape, const MistDpCosts *costs, const float 
     return fail(MIST_E_INVALID, "unknown DP mode %d", mode);
   const int plane = (shape->num_layers + 1) * (shape->num_devices + 1);
   const int64_t n_init = (int64_t)n_tmax * plane;
-  hipLaunchKernelGGL(dp_init_kernel, dim3((unsigned)((n_init + 255) / 256)), dim3(256), 0,
-                     (hipStream_t)stream, *shape, n_tmax, d_scratch, d_best_s, d_best_sum,
-                     d_stage_max);
-  MIST_HIP_CHECK(hipGetLastError());
   int32_t *d_ranges = reinterpret_cast<int32_t *>(d_scratch + (int64_t)4 * n_tmax * plane);
-  const int64_t n_cols = (int64_t)n_tmax * (shape->num_devices + 1);
-  const dim3 ranges_grid((unsigned)((n_cols + 255) / 256));
-  hipLaunchKernelGGL(dp_ranges_kernel, ranges_grid, dim3(256), 0, (hipStream_t)stream, *shape,
-                     n_tmax, 0, d_scratch, d_ranges);
+  hipLaunchKernelGGL(dp_init_kernel, dim3((unsigned)((n_init + 255) / 256)), dim3(256), 0,
+                     (hipStream_t)stream, *shape, n_tmax, d_scratch, d_ranges, d_best_s,
+                     d_best_sum, d_stage_max);
   MIST_HIP_CHECK(hipGetLastError());
   // Small batches are latency-bound: spread every state over a team of lanes.
   const bool wide = (int64_t)n_tmax * plane <= (1 << 19);
@@ -439,11 +463,6 @@ int mist_dp_run(const MistDpShape *shape, const MistDpCosts *costs, const float 
     }
 #undef MIST_DP_STEP
     MIST_HIP_CHECK(hipGetLastError());
-    if (s < shape->max_stages) {
-      hipLaunchKernelGGL(dp_ranges_kernel, ranges_grid, dim3(256), 0, (hipStream_t)stream, *shape,
-                         n_tmax, s & 1, d_scratch, d_ranges);
-      MIST_HIP_CHECK(hipGetLastError());
-    }
   }
   return 0;
 }

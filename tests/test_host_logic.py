@@ -222,9 +222,9 @@ def test_argument_checks_reject_before_any_launch():
     shape["num_layers"], shape["num_devices"], shape["num_mesh"], shape["p_dim"] = 8, 8, 2, 4
     shape["max_stages"] = 4
     shape["mesh_n"][0, :2], shape["mesh_m"][0, :2] = [1, 1], [1, 2]
-    assert lib.mist_dp_scratch_floats(ctypes.c_void_p(shape.ctypes.data), 4) == 4 * 4 * 9 * 9 + 2 * 4 * 9
+    assert lib.mist_dp_scratch_floats(ctypes.c_void_p(shape.ctypes.data), 4) == 4 * 4 * 9 * 9 + 6 * 4 * 9
     shape["num_layers"], shape["num_devices"] = 80, 256
-    assert lib.mist_dp_scratch_floats(ctypes.c_void_p(shape.ctypes.data), 4) == 4 * 4 * 81 * 257 + 2 * 4 * 257
+    assert lib.mist_dp_scratch_floats(ctypes.c_void_p(shape.ctypes.data), 4) == 4 * 4 * 81 * 257 + 6 * 4 * 257
     costs = _lib.DpCosts(4096, 4096, 4096, 4096, 4096, 4096, 4096, 4096)
     sp = ctypes.c_void_p(shape.ctypes.data)
     assert lib.mist_dp_run(sp, ctypes.byref(costs), fake, fake, 1, 0, fake, fake, fake, None, None, None) == -1

@@ -80,30 +80,48 @@ __global__ __launch_bounds__(256) void select_candidates_kernel(
     const MistDpCosts tabs, const int32_t *__restrict__ rows, const float *__restrict__ lo,
     const float *__restrict__ hi, float *__restrict__ out_values, int32_t *__restrict__ out_request,
     int capacity, int32_t *__restrict__ counts) {
+  __shared__ int above_of_wave[4];
   const int r = blockIdx.y;
   const int64_t g = rows[r];
   const int64_t n0 = tabs.g_stride[0], n1 = tabs.g_stride[1], n2 = tabs.g_stride[2];
+  const int64_t n = n0 + n1 + n2;
   const float lo_r = lo[r], hi_r = hi[r];
+  const int lane = threadIdx.x & 63;
   int above = 0;
-  for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < n0 + n1 + n2;
-       e += (int64_t)gridDim.x * blockDim.x) {
-    const float v = e < n0 ? tabs.costs[g * n0 + e]
-                    : e < n0 + n1 ? tabs.costs_pre[g * n1 + (e - n0)]
-                                  : tabs.costs_post[g * n2 + (e - n0 - n1)];
-    if (!(v < INFINITY)) continue;  // +inf (nothing feasible) and NaN are not candidates
-    if (v > hi_r) {
-      ++above;
-    } else if (v > lo_r) {
-      const int at = atomicAdd(&counts[0], 1);
-      if (at < capacity) {
+  // every lane of a wavefront runs the same number of rounds (the ballot needs all of them)
+  for (int64_t base = (int64_t)blockIdx.x * blockDim.x; base < n;
+       base += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t e = base + threadIdx.x;
+    float v = INFINITY;
+    if (e < n)
+      v = e < n0 ? tabs.costs[g * n0 + e]
+          : e < n0 + n1 ? tabs.costs_pre[g * n1 + (e - n0)]
+                        : tabs.costs_post[g * n2 + (e - n0 - n1)];
+    const bool finite = v < INFINITY;  // +inf (nothing feasible) and NaN are not candidates
+    above += finite && v > hi_r;
+    const bool take = finite && v > lo_r && v <= hi_r;
+    // one atomic per wavefront reserves the slots of all its selected values
+    const unsigned long long takers = __ballot(take);
+    if (takers != 0) {
+      const int leader = __ffsll(takers) - 1;
+      int first = 0;
+      if (lane == leader) first = atomicAdd(&counts[0], __popcll(takers));
+      first = __shfl(first, leader);
+      const int at = first + __popcll(takers & ((1ull << lane) - 1));
+      if (take && at < capacity) {
         out_values[at] = v;
         out_request[at] = r;
       }
     }
   }
-  // one atomic per wavefront for the "above" count
+  // one atomic per workgroup for the "above" count
   for (int step = 32; step >= 1; step >>= 1) above += __shfl_xor(above, step);
-  if ((threadIdx.x & 63) == 0 && above > 0) atomicAdd(&counts[1 + r], above);
+  if (lane == 0) above_of_wave[threadIdx.x >> 6] = above;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const int total = above_of_wave[0] + above_of_wave[1] + above_of_wave[2] + above_of_wave[3];
+    if (total > 0) atomicAdd(&counts[1 + r], total);
+  }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -409,7 +427,7 @@ int mist_dp_select_candidates(const MistDpCosts *costs, int n_requests, const in
   if (!d_rows || !d_lo || !d_hi || !d_out_values || !d_out_request || !d_counts || capacity <= 0)
     return fail(MIST_E_INVALID, "null pointer / empty output list");
   const int64_t per_row = costs->g_stride[0] + costs->g_stride[1] + costs->g_stride[2];
-  const unsigned blocks = (unsigned)std::min<int64_t>((per_row + 255) / 256, 512);
+  const unsigned blocks = (unsigned)std::min<int64_t>((per_row + 2047) / 2048, 256);
   hipLaunchKernelGGL(select_candidates_kernel, dim3(blocks, n_requests), dim3(256), 0,
                      (hipStream_t)stream, *costs, d_rows, d_lo, d_hi, d_out_values, d_out_request,
                      capacity, d_counts);

@@ -531,12 +531,14 @@ __device__ __forceinline__ void take_min(double &best, int32_t &best_row, bool f
 #endif
 constexpr int kScoutSplit = 4;  // scout workgroups per (group, (l, c) tile, p tile)
 constexpr int kPairFields = 4;  // per-pair table of sieve A: thr_b, thr_o, n_ck, n_nock
+constexpr int kStageMaxOut = MIST_T_GCB + 1;  // slot of max(MIST_T_OUT) behind the stage minima
 constexpr int kLdsRowStride = MIST_ROW_TERMS + 1;  // odd number of doubles: lanes reading the
                                                    // same term of different rows hit different banks
 static_assert(kStageRows == 64, "the sieve masks are 64-bit");
 static_assert(MIST_ROW_TERMS % 2 == 0, "rows are staged as 16-byte pairs");
 static_assert(MIST_LC_TILE == 64, "one wavefront per workgroup: the stage minima use wave shuffles");
-static_assert(MIST_T_GCB - MIST_T_FWD_STATES0 == 15, "memory terms must be 16 consecutive columns");
+static_assert(MIST_T_S_LAYER_CK == 0 && MIST_T_GCB < 32,
+              "latency and memory terms must be the first columns: one lane per term in the stage minima");
 
 struct LaneMemory {
   double fwd_states, bwd_states, cur_saved, mod_saved, ck_delta, fwd_pk, bwd_pk, out, gcb;
@@ -597,7 +599,7 @@ template <bool kPow2G, bool kFirstTile>
 __device__ __forceinline__ void reduce_block(
     const MistProblem &prob, const MistGroupDesc *__restrict__ g, const ReduceRange range,
     int p_tile, int lc_tile, const double *__restrict__ row_terms, double ratio,
-    double *lds_terms, double *lds_min, double *lds_pair, int *lds_pair_lane,
+    double *lds_terms, double *lds_min, double *lds_pair,
     const double *__restrict__ seed_cost,
     const int32_t *__restrict__ seed_index, double *__restrict__ out_cost,
     int32_t *__restrict__ out_index) {
@@ -668,19 +670,11 @@ __device__ __forceinline__ void reduce_block(
 
   const double *__restrict__ src = row_terms + g->row_offset * MIST_ROW_TERMS;
 
-  // Sieve A visits the tile's pairs class by class (which first / last family member the
-  // latency uses is fixed per class): 0 = 0 < c < l, 1 = c == 0, 2 = c == l.  Each lane gets a
-  // slot of the per-pair table in that order.
+  // Sieve A visits pairs class by class (which first / last family member the latency uses is
+  // fixed per class): 0 = 0 < c < l, 1 = c == 0, 2 = c == l.
   const int pair_class = !active ? 3 : (c == 0 ? 1 : (c == l ? 2 : 0));
-  const uint64_t lanes_below = (1ull << threadIdx.x) - 1ull;
   const uint64_t in_class0 = __ballot(pair_class == 0), in_class1 = __ballot(pair_class == 1);
   const uint64_t in_class2 = __ballot(pair_class == 2);
-  const int n_class0 = __popcll(in_class0), n_class1 = __popcll(in_class1);
-  const int n_class2 = __popcll(in_class2);
-  const int pair_slot =
-      pair_class == 0 ? __popcll(in_class0 & lanes_below)
-      : pair_class == 1 ? n_class0 + __popcll(in_class1 & lanes_below)
-                        : n_class0 + n_class1 + __popcll(in_class2 & lanes_below);
 
   const double lf = (double)l, lm1 = (double)max(l - 1, 0), cf = (double)c;
   const double l_minus_c = (double)(l - c), l_minus_c_1 = (double)(l - c - 1);
@@ -693,11 +687,8 @@ __device__ __forceinline__ void reduce_block(
   const double n_nock = (double)(lm2 - min(max(c - 1, 0), lm2));
   const int first_col = c_eq_l ? 0 : 1, last_col = c_eq_0 ? 1 : 0;  // *_CK precedes *_NOCK
   const int post_col = c > 0 ? 0 : 1;
-  if (active) {
-    lds_pair[pair_slot * kPairFields + 2] = n_ck;
-    lds_pair[pair_slot * kPairFields + 3] = n_nock;
-    lds_pair_lane[pair_slot] = (int)threadIdx.x;
-  }
+  lds_pair[threadIdx.x * kPairFields + 2] = n_ck;
+  lds_pair[threadIdx.x * kPairFields + 3] = n_nock;
   auto div_G = [&](double v) { return kPow2G ? v * inv_G64 : v / G64; };
 
   // Memory model of one candidate row for this lane's (l, c) (:2150-2162, 2358-2385, 2755-2786).
@@ -899,30 +890,29 @@ __device__ __forceinline__ void reduce_block(
       }
     }
     __syncthreads();
-    // Term-wise minimum of the stage's memory terms (MIST_T_FWD_STATES0 .. MIST_T_GCB), plus the
-    // maximum of the one term the last-stage peak subtracts: lane = (term, quarter of the rows).
+    // Term-wise minimum of the stage's latency and memory terms (columns 0 .. MIST_T_GCB), plus
+    // the maximum of the one term the last-stage peak subtracts: lane = (term, half of the rows).
     {
-      const int term = threadIdx.x & 15, quarter = threadIdx.x >> 4;
+      const int term = threadIdx.x & 31, half = threadIdx.x >> 5;
       double lo_v = INFINITY, hi_v = 0.0;
-      for (int r = quarter * (kStageRows / 4); r < (quarter + 1) * (kStageRows / 4); ++r) {
-        if (r < n_stage) {
-          const double v = lds_terms[r * kLdsRowStride + MIST_T_FWD_STATES0 + term];
+      if (term <= MIST_T_GCB) {
+        const int r_end = min((half + 1) * (kStageRows / 2), n_stage);
+        for (int r = half * (kStageRows / 2); r < r_end; ++r) {
+          const double v = lds_terms[r * kLdsRowStride + term];
           lo_v = fmin(lo_v, v);
           hi_v = fmax(hi_v, v);
         }
       }
-      lo_v = fmin(lo_v, __shfl_xor(lo_v, 16));
       lo_v = fmin(lo_v, __shfl_xor(lo_v, 32));
-      hi_v = fmax(hi_v, __shfl_xor(hi_v, 16));
       hi_v = fmax(hi_v, __shfl_xor(hi_v, 32));
-      if (threadIdx.x < 16) lds_min[threadIdx.x] = lo_v;
-      if (threadIdx.x == MIST_T_OUT - MIST_T_FWD_STATES0) lds_min[16] = hi_v;
+      if (threadIdx.x <= MIST_T_GCB) lds_min[threadIdx.x] = lo_v;
+      if (threadIdx.x == MIST_T_OUT) lds_min[kStageMaxOut] = hi_v;
     }
     __syncthreads();
 
     // ---- per-stage thresholds: no row of the stage is feasible beyond the pseudo row's count,
     // so only the minima of the slots below it can be beaten ----
-    const LaneMemory floor_mem = lane_memory(lds_min - MIST_T_FWD_STATES0);
+    const LaneMemory floor_mem = lane_memory(lds_min);
     const int cnt_b = count_bound([&](int p) { return floor_mem.scaled_base(p); });
     const int cnt_p =
         count_bound([&](int p) { return floor_mem.scaled_pre(p, pre_saved, pre_sas); });
@@ -941,65 +931,74 @@ __device__ __forceinline__ void reduce_block(
       const double b_in =
           floor_mem.bwd_states + post_states + floor_mem.mod_saved + post_bwd_peak + floor_mem.gcb;
       const double pf_post = fmax(f_in, peak_f + post_states);
-      const double pb_post = fmax(b_in, peak_b - lds_min[16] + post_states) + post_output;
+      const double pb_post = fmax(b_in, peak_b - lds_min[kStageMaxOut] + post_states) + post_output;
       if (fmax(pf_post, pb_post) * floor_mem.mf_pp <= cap) thr_o = fmax(thr_o, best_post);
       if (do_nopp) {
         const double pf_pp = pf_post + pre_states + pre_saved;
         const double pb_pp = pb_post + pre_states + pre_saved;
-        if (fmax(pf_pp, pb_pp) * lds_min[MIST_T_MF - MIST_T_FWD_STATES0] <= cap)
+        if (fmax(pf_pp, pb_pp) * lds_min[MIST_T_MF] <= cap)
           thr_o = fmax(thr_o, best_pp);
       }
     }
 
-    // ---- sieve A: all rows of the stage against those thresholds.  Transposed: a lane holds
-    // the latency terms of ONE ROW in registers and the loop runs over the tile's pairs, whose
-    // constants and thresholds are wave-uniform reads of the per-pair table.  The wave-wide
-    // comparison result is exactly the 64-row survivor mask of that pair; it is handed to the
-    // pair's lane. ----
-    if (active) {
-      lds_pair[pair_slot * kPairFields + 0] = thr_b;
-      lds_pair[pair_slot * kPairFields + 1] = thr_o;
-    }
-    double rt[MIST_T_D_LAST_NOCK + 1];
-#pragma unroll
-    for (int i = 0; i <= MIST_T_D_LAST_NOCK; ++i)
-      rt[i] = lds_terms[threadIdx.x * kLdsRowStride + i];  // stale beyond n_stage, masked below
-    __syncthreads();
-    const uint64_t valid_rows = n_stage < kStageRows ? (1ull << n_stage) - 1ull : ~0ull;
+    // ---- sieve A: the rows of the stage against those thresholds.  First the pseudo row of
+    // term-wise minima: the objective is monotone in every term, so a pair the pseudo row does
+    // not pass is passed by no row of the stage (two thirds of all stages end here).  For the
+    // other pairs the test runs transposed: a lane holds the latency terms of ONE ROW in
+    // registers and the loop runs over those pairs, whose constants and thresholds are
+    // wave-uniform reads of the per-pair table.  The wave-wide comparison result is exactly the
+    // 64-row survivor mask of that pair; it is handed to the pair's lane. ----
     uint64_t sieve = 0;
-    auto sieve_class = [&](int k_begin, int k_end, auto first_col_tag, auto last_col_tag) {
-      constexpr int kFirstCol = decltype(first_col_tag)::value;
-      constexpr int kLastCol = decltype(last_col_tag)::value;
-      const double s_first = rt[MIST_T_S_FIRST_CK + kFirstCol];
-      const double s_last = rt[MIST_T_S_LAST_CK + kLastCol];
-      const double d_first = rt[MIST_T_D_FIRST_CK + kFirstCol];
-      const double d_last = rt[MIST_T_D_LAST_CK + kLastCol];
-#pragma unroll 2
-      for (int k = k_begin; k < k_end; ++k) {
-        const double pair_thr_b = lds_pair[k * kPairFields + 0];
-        const double pair_thr_o = lds_pair[k * kPairFields + 1];
-        const double pair_n_ck = lds_pair[k * kPairFields + 2];
-        const double pair_n_nock = lds_pair[k * kPairFields + 3];
-        const int pair_lane = lds_pair_lane[k];
-        const double stable = pair_n_ck * rt[MIST_T_S_LAYER_CK] +
-                              pair_n_nock * rt[MIST_T_S_LAYER_NOCK] + s_first + s_last;
-        const double delta = pair_n_ck * rt[MIST_T_D_LAYER_CK] +
-                             pair_n_nock * rt[MIST_T_D_LAYER_NOCK] + d_first + d_last;
-        const float x32 = (float)stable, d32 = (float)delta;
-        const float y32 = kPow2G ? d32 * inv_G32 : d32 / G32;
-        const double rx = ratio * (double)x32;
-        const double cost_base = rx + (double)y32;
-        const double bound = rx + div_G((double)d32);
-        const uint64_t survivors =
-            __ballot(cost_base <= pair_thr_b || bound <= pair_thr_o) & valid_rows;
-        sieve = (int)threadIdx.x == pair_lane ? survivors : sieve;
-      }
-    };
-    sieve_class(0, n_class0, std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{});
-    sieve_class(n_class0, n_class0 + n_class1, std::integral_constant<int, 1>{},
-                std::integral_constant<int, 1>{});
-    sieve_class(n_class0 + n_class1, n_class0 + n_class1 + n_class2,
-                std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{});
+    uint64_t pairs_open;
+    {
+      double x, d, cost_base, bound;
+      objective(lds_min, x, d, cost_base, bound);
+      pairs_open = __ballot(active && (cost_base <= thr_b || bound <= thr_o));
+    }
+    if (pairs_open != 0) {
+      lds_pair[threadIdx.x * kPairFields + 0] = thr_b;
+      lds_pair[threadIdx.x * kPairFields + 1] = thr_o;
+      double rt[MIST_T_D_LAST_NOCK + 1];
+#pragma unroll
+      for (int i = 0; i <= MIST_T_D_LAST_NOCK; ++i)
+        rt[i] = lds_terms[threadIdx.x * kLdsRowStride + i];  // stale beyond n_stage, masked below
+      __syncthreads();
+      const uint64_t valid_rows = n_stage < kStageRows ? (1ull << n_stage) - 1ull : ~0ull;
+      auto sieve_class = [&](uint64_t todo, auto first_col_tag, auto last_col_tag) {
+        constexpr int kFirstCol = decltype(first_col_tag)::value;
+        constexpr int kLastCol = decltype(last_col_tag)::value;
+        const double s_first = rt[MIST_T_S_FIRST_CK + kFirstCol];
+        const double s_last = rt[MIST_T_S_LAST_CK + kLastCol];
+        const double d_first = rt[MIST_T_D_FIRST_CK + kFirstCol];
+        const double d_last = rt[MIST_T_D_LAST_CK + kLastCol];
+        while (todo != 0) {
+          const int pair_lane = __ffsll((unsigned long long)todo) - 1;
+          todo &= todo - 1;
+          const double pair_thr_b = lds_pair[pair_lane * kPairFields + 0];
+          const double pair_thr_o = lds_pair[pair_lane * kPairFields + 1];
+          const double pair_n_ck = lds_pair[pair_lane * kPairFields + 2];
+          const double pair_n_nock = lds_pair[pair_lane * kPairFields + 3];
+          const double stable = pair_n_ck * rt[MIST_T_S_LAYER_CK] +
+                                pair_n_nock * rt[MIST_T_S_LAYER_NOCK] + s_first + s_last;
+          const double delta = pair_n_ck * rt[MIST_T_D_LAYER_CK] +
+                               pair_n_nock * rt[MIST_T_D_LAYER_NOCK] + d_first + d_last;
+          const float x32 = (float)stable, d32 = (float)delta;
+          const float y32 = kPow2G ? d32 * inv_G32 : d32 / G32;
+          const double rx = ratio * (double)x32;
+          const double cost_base = rx + (double)y32;
+          const double bound = rx + div_G((double)d32);
+          const uint64_t survivors =
+              __ballot(cost_base <= pair_thr_b || bound <= pair_thr_o) & valid_rows;
+          sieve = (int)threadIdx.x == pair_lane ? survivors : sieve;
+        }
+      };
+      sieve_class(pairs_open & in_class0, std::integral_constant<int, 1>{},
+                  std::integral_constant<int, 0>{});
+      sieve_class(pairs_open & in_class1, std::integral_constant<int, 1>{},
+                  std::integral_constant<int, 1>{});
+      sieve_class(pairs_open & in_class2, std::integral_constant<int, 0>{},
+                  std::integral_constant<int, 0>{});
+    }
 
     // ---- sieve B: lowest improvable slot and the memory test there, per-lane survivors ----
     uint64_t keep = 0;
@@ -1041,9 +1040,8 @@ __global__ __launch_bounds__(MIST_LC_TILE, MIST_REDUCE_MIN_WAVES) void eval_redu
     const int32_t *__restrict__ scout_prefix, int scout, const double *__restrict__ row_terms,
     double ratio, double *__restrict__ partial_cost, int32_t *__restrict__ partial_index) {
   __shared__ double lds_terms[kStageRows * kLdsRowStride];
-  __shared__ double lds_min[17];
+  __shared__ double lds_min[kStageMaxOut + 1];
   __shared__ double lds_pair[MIST_LC_TILE * kPairFields];
-  __shared__ int lds_pair_lane[MIST_LC_TILE];
   const int block = xcd_run_block(blockIdx.x);
   if (block >= (scout ? scout_prefix[n_groups] : n_blocks)) return;
   int local_block;
@@ -1080,7 +1078,7 @@ __global__ __launch_bounds__(MIST_LC_TILE, MIST_REDUCE_MIN_WAVES) void eval_redu
   const bool pow2 = (g->grad_accum & (g->grad_accum - 1)) == 0;
 #define MIST_REDUCE(P2, FT)                                                                   \
   reduce_block<P2, FT>(prob, g, range, p_tile, lc_tile, row_terms, ratio, lds_terms, lds_min,  \
-                       lds_pair, lds_pair_lane, seed_cost, seed_index,                        \
+                       lds_pair, seed_cost, seed_index,                                       \
                        partial_cost + out_slab * slab, partial_index + out_slab * slab)
   if (pow2) {
     if (p_tile == 0) MIST_REDUCE(true, true); else MIST_REDUCE(true, false);

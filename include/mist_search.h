@@ -141,6 +141,8 @@ int mist_reduce_lc_tile(void); /* MIST_LC_TILE the library was built with */
 int mist_reduce_scout_split(void); /* scout workgroups per (group, (l, c) tile, p tile) */
 int mist_terms_block_rows(void); /* candidate rows per workgroup of mist_row_terms */
 int mist_reduce_stage_rows(void); /* rows per LDS stage; rows_per_chunk must be a multiple */
+/* doubles of the stage-summary workspace for `total_rows` workspace rows in `n_groups` groups */
+int64_t mist_stage_floor_doubles(int64_t total_rows, int n_groups);
 
 /* Row-invariant terms of every candidate row: decodes the row index, evaluates the alpha-beta
  * communication terms, the 36 interference evaluations and the memory pieces that do not
@@ -153,10 +155,13 @@ int mist_reduce_stage_rows(void); /* rows per LDS stage; rows_per_chunk must be 
  * d_row_terms: [total_rows][MIST_ROW_TERMS] float64.  Within a group the workspace is ordered
  *   position = ((par * n_ao + ao) * n_oo + oo) * n_pair + pair
  * (rows of similar memory footprint next to each other, which the reduce kernel's per-stage
- * bound relies on for speed, not for correctness); all results carry reference row numbers. */
+ * bound relies on for speed, not for correctness); all results carry reference row numbers.
+ * d_stage_floor: mist_stage_floor_doubles() float64, written here and read by mist_eval_reduce:
+ * per stage of mist_reduce_stage_rows() workspace rows the term-wise minimum of the latency and
+ * memory terms (the pseudo row that bounds every row of the stage from below). */
 int mist_row_terms(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,
                    const int32_t *d_block_prefix, int n_blocks, double *d_row_terms,
-                   void *stream);
+                   double *d_stage_floor, void *stream);
 
 /* Per (group, row chunk, (l, c) tile, p tile): evaluates latency and memory per cell, applies
  * the memory mask and keeps the running lexicographic (cost, row) minimum per bucket.
@@ -173,8 +178,8 @@ int mist_row_terms(const MistProblem *problem, const MistGroupDesc *d_groups, in
 int mist_eval_reduce(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,
                      const int32_t *d_block_prefix, int n_blocks,
                      const int32_t *d_scout_prefix, int n_scout_blocks,
-                     const double *d_row_terms, double ratio, double *d_partial_cost,
-                     int32_t *d_partial_index, void *stream);
+                     const double *d_row_terms, const double *d_stage_floor, double ratio,
+                     double *d_partial_cost, int32_t *d_partial_index, void *stream);
 
 /* Combines the per-chunk partial minima (smallest cost, lowest row among equals),
  * recomputes stable / delta of the winning row and scatters into the output tables at sample
@@ -191,7 +196,8 @@ int mist_finalize(const MistProblem *problem, const MistGroupDesc *d_groups, int
 int mist_intra_stage_eval(const MistProblem *problem, const MistGroupDesc *d_groups,
                           int n_groups, const int32_t *d_terms_block_prefix, int n_terms_blocks,
                           const int32_t *d_reduce_block_prefix, int n_reduce_blocks,
-                          const int32_t *d_scout_prefix, int n_scout_blocks, double *d_row_terms, double *d_partial_cost, int32_t *d_partial_index,
+                          const int32_t *d_scout_prefix, int n_scout_blocks, double *d_row_terms,
+                          double *d_stage_floor, double *d_partial_cost, int32_t *d_partial_index,
                           double ratio, int sample_index, int compute_terms,
                           const MistOutTables *tables, void *stream);
 

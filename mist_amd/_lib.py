@@ -110,10 +110,11 @@ _SIGNATURES = {
     "mist_reduce_lc_tile": (ctypes.c_int, []),
     "mist_terms_block_rows": (ctypes.c_int, []),
     "mist_reduce_scout_split": (ctypes.c_int, []),
-    "mist_row_terms": (ctypes.c_int, [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, _VP]),
+    "mist_stage_floor_doubles": (ctypes.c_int64, [ctypes.c_int64, ctypes.c_int]),
+    "mist_row_terms": (ctypes.c_int, [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, _VP, _VP]),
     "mist_eval_reduce": (
         ctypes.c_int,
-        [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, ctypes.c_double,
+        [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, _VP, ctypes.c_double,
          _VP, _VP, _VP],
     ),
     "mist_finalize": (
@@ -123,7 +124,7 @@ _SIGNATURES = {
     "mist_intra_stage_eval": (
         ctypes.c_int,
         [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, ctypes.c_int,
-         _VP, _VP, _VP, ctypes.c_double, ctypes.c_int, ctypes.c_int, ctypes.POINTER(OutTables), _VP],
+         _VP, _VP, _VP, _VP, ctypes.c_double, ctypes.c_int, ctypes.c_int, ctypes.POINTER(OutTables), _VP],
     ),
 }
 

@@ -37,6 +37,13 @@ using mist::fail;
 constexpr int kTermsBlock = 128;  // rows per workgroup of the row-term kernel
 constexpr int kStageRows = 64;    // rows staged through LDS per step of the reduce kernel
 constexpr int kSlots = 2 * MIST_P_TILE + 2;  // per-thread running minima: base, with_pre, post, no_pp
+// Stage summaries (written with the row terms, read by the reduce kernel): per stage of
+// kStageRows workspace rows the term-wise minimum of the latency and memory columns and the
+// maximum of MIST_T_OUT, kStageFloorPitch doubles per stage.
+constexpr int kStageFloorPitch = 32;
+constexpr int kStageMaxOut = MIST_T_GCB + 1;  // slot of max(MIST_T_OUT) behind the stage minima
+static_assert(kStageMaxOut < kStageFloorPitch, "a stage summary is one 32-lane load");
+static_assert(kStageRows == 2 * kStageFloorPitch, "lane = (column, half of the rows)");
 
 // ------------------------------------------------------------------------------------------
 // Communication models (mist/tools/optimize.py:257-303, 459-470).
@@ -148,6 +155,14 @@ __device__ __forceinline__ Family pick_family(bool second, const Family &a, cons
   return r;
 }
 
+// Slot of stage `stage` of group `group_index` in the stage-summary workspace.  Groups lie back
+// to back in the row workspace and need not start at a multiple of kStageRows; adding the group
+// index keeps the slots of consecutive groups apart (at most rows / kStageRows + groups + 1 slots).
+__device__ __forceinline__ int64_t stage_floor_slot(const MistGroupDesc *g, int group_index,
+                                                    int64_t stage) {
+  return g->row_offset / kStageRows + group_index + stage;
+}
+
 __device__ __forceinline__ const MistGroupDesc *find_group(const MistGroupDesc *groups,
                                                            const int32_t *prefix, int n_groups,
                                                            int block, int *local) {
@@ -202,7 +217,8 @@ __device__ __forceinline__ int64_t position_of_row(const MistGroupDesc *g, int64
 // ------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(kTermsBlock) void row_terms_kernel(
     const MistProblem prob, const MistGroupDesc *__restrict__ groups, int n_groups,
-    const int32_t *__restrict__ block_prefix, double *__restrict__ row_terms) {
+    const int32_t *__restrict__ block_prefix, double *__restrict__ row_terms,
+    double *__restrict__ stage_floor) {
   int local_block;
   const MistGroupDesc *g = find_group(groups, block_prefix, n_groups, blockIdx.x, &local_block);
   // The block's terms are assembled in LDS (row pitch 35 doubles: conflict-free) and written out
@@ -402,6 +418,30 @@ __global__ __launch_bounds__(kTermsBlock) void row_terms_kernel(
     const int at = (i / (MIST_ROW_TERMS / 2)) * (MIST_ROW_TERMS + 1) + 2 * (i % (MIST_ROW_TERMS / 2));
     dst[i] = make_double2(lds_out[at], lds_out[at + 1]);
   }
+  // Summary of each stage of kStageRows rows for the reduce kernel: lane = (column, half of the
+  // stage's rows); columns 0 .. MIST_T_GCB hold the minimum, column kStageMaxOut the maximum of
+  // MIST_T_OUT.
+  {
+    const int stage_here = threadIdx.x / kStageRows, lane = threadIdx.x % kStageRows;
+    const int col = lane & (kStageFloorPitch - 1), half = lane / kStageFloorPitch;
+    const int src_col = col == kStageMaxOut ? MIST_T_OUT : col;
+    const int r_begin = stage_here * kStageRows + half * (kStageRows / 2);
+    const int r_end = min(r_begin + kStageRows / 2, rows_here);
+    double lo_v = INFINITY, hi_v = 0.0;
+    if (col <= kStageMaxOut) {
+      for (int r = r_begin; r < r_end; ++r) {
+        const double v = lds_out[r * (MIST_ROW_TERMS + 1) + src_col];
+        lo_v = fmin(lo_v, v);
+        hi_v = fmax(hi_v, v);
+      }
+    }
+    lo_v = fmin(lo_v, __shfl_xor(lo_v, kStageFloorPitch));
+    hi_v = fmax(hi_v, __shfl_xor(hi_v, kStageFloorPitch));
+    if (half == 0 && stage_here * kStageRows < rows_here) {
+      const int64_t slot = stage_floor_slot(g, (int)(g - groups), block_first / kStageRows + stage_here);
+      stage_floor[slot * kStageFloorPitch + col] = col < kStageMaxOut ? lo_v : (col == kStageMaxOut ? hi_v : 0.0);
+    }
+  }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -531,7 +571,6 @@ __device__ __forceinline__ void take_min(double &best, int32_t &best_row, bool f
 #endif
 constexpr int kScoutSplit = 4;  // scout workgroups per (group, (l, c) tile, p tile)
 constexpr int kPairFields = 4;  // per-pair table of sieve A: thr_b, thr_o, n_ck, n_nock
-constexpr int kStageMaxOut = MIST_T_GCB + 1;  // slot of max(MIST_T_OUT) behind the stage minima
 constexpr int kLdsRowStride = MIST_ROW_TERMS + 1;  // odd number of doubles: lanes reading the
                                                    // same term of different rows hit different banks
 static_assert(kStageRows == 64, "the sieve masks are 64-bit");
@@ -598,7 +637,8 @@ struct ReduceRange {
 template <bool kPow2G, bool kFirstTile>
 __device__ __forceinline__ void reduce_block(
     const MistProblem &prob, const MistGroupDesc *__restrict__ g, const ReduceRange range,
-    int p_tile, int lc_tile, const double *__restrict__ row_terms, double ratio,
+    int p_tile, int lc_tile, const double *__restrict__ row_terms,
+    const double *__restrict__ stage_floor /* of this group's stage 0 */, double ratio,
     double *lds_terms, double *lds_min, double *lds_pair,
     const double *__restrict__ seed_cost,
     const int32_t *__restrict__ seed_index, double *__restrict__ out_cost,
@@ -872,42 +912,28 @@ __device__ __forceinline__ void reduce_block(
     return changed;
   };
 
-  const int64_t first_stage = range.row_begin / kStageRows;
+  // Stages this workgroup visits: every stage_step-th one of its range, without those the scout
+  // pass has done.  (skip_stride > 1 goes with stage_step == 1: two skips are never adjacent.)
   const int64_t end_stage = (range.row_end + kStageRows - 1) / kStageRows;
-  for (int64_t stage = first_stage; stage < end_stage; stage += range.stage_step) {
-    if (range.skip_stride > 0 && stage % range.skip_stride == 0) continue;
+  auto skipped = [&](int64_t st) { return range.skip_stride > 0 && st % range.skip_stride == 0; };
+  auto after = [&](int64_t st) {
+    st += range.stage_step;
+    return skipped(st) ? st + range.stage_step : st;
+  };
+  // The summary of a stage (term-wise minima of its rows, written with the row terms) is one
+  // 32-lane load; the next stage's is in flight while the current stage is processed.
+  auto load_floor = [&](int64_t st) {
+    return threadIdx.x < kStageFloorPitch ? stage_floor[st * kStageFloorPitch + threadIdx.x] : 0.0;
+  };
+  int64_t stage = range.row_begin / kStageRows;
+  if (skipped(stage)) stage += range.stage_step;
+  double floor_v = stage < end_stage ? load_floor(stage) : 0.0;
+  for (; stage < end_stage; stage = after(stage)) {
     const int64_t base = stage * kStageRows;
     const int n_stage = (int)min((int64_t)kStageRows, range.row_end - base);
     __syncthreads();
-    {  // 16-byte loads: a row is 17 such pairs and starts 16-byte aligned
-      const double2 *__restrict__ src2 =
-          reinterpret_cast<const double2 *>(src + base * MIST_ROW_TERMS);
-      for (int i = threadIdx.x; i < n_stage * (MIST_ROW_TERMS / 2); i += MIST_LC_TILE) {
-        const double2 v = src2[i];
-        const int at = (i / (MIST_ROW_TERMS / 2)) * kLdsRowStride + 2 * (i % (MIST_ROW_TERMS / 2));
-        lds_terms[at] = v.x;
-        lds_terms[at + 1] = v.y;
-      }
-    }
-    __syncthreads();
-    // Term-wise minimum of the stage's latency and memory terms (columns 0 .. MIST_T_GCB), plus
-    // the maximum of the one term the last-stage peak subtracts: lane = (term, half of the rows).
-    {
-      const int term = threadIdx.x & 31, half = threadIdx.x >> 5;
-      double lo_v = INFINITY, hi_v = 0.0;
-      if (term <= MIST_T_GCB) {
-        const int r_end = min((half + 1) * (kStageRows / 2), n_stage);
-        for (int r = half * (kStageRows / 2); r < r_end; ++r) {
-          const double v = lds_terms[r * kLdsRowStride + term];
-          lo_v = fmin(lo_v, v);
-          hi_v = fmax(hi_v, v);
-        }
-      }
-      lo_v = fmin(lo_v, __shfl_xor(lo_v, 32));
-      hi_v = fmax(hi_v, __shfl_xor(hi_v, 32));
-      if (threadIdx.x <= MIST_T_GCB) lds_min[threadIdx.x] = lo_v;
-      if (threadIdx.x == MIST_T_OUT) lds_min[kStageMaxOut] = hi_v;
-    }
+    if (threadIdx.x < kStageFloorPitch) lds_min[threadIdx.x] = floor_v;
+    if (after(stage) < end_stage) floor_v = load_floor(after(stage));
     __syncthreads();
 
     // ---- per-stage thresholds: no row of the stage is feasible beyond the pseudo row's count,
@@ -958,6 +984,18 @@ __device__ __forceinline__ void reduce_block(
     if (pairs_open != 0) {
       lds_pair[threadIdx.x * kPairFields + 0] = thr_b;
       lds_pair[threadIdx.x * kPairFields + 1] = thr_o;
+      {  // 16-byte loads: a row is 17 such pairs and starts 16-byte aligned
+        const double2 *__restrict__ src2 =
+            reinterpret_cast<const double2 *>(src + base * MIST_ROW_TERMS);
+        for (int i = threadIdx.x; i < n_stage * (MIST_ROW_TERMS / 2); i += MIST_LC_TILE) {
+          const double2 v = src2[i];
+          const int at =
+              (i / (MIST_ROW_TERMS / 2)) * kLdsRowStride + 2 * (i % (MIST_ROW_TERMS / 2));
+          lds_terms[at] = v.x;
+          lds_terms[at + 1] = v.y;
+        }
+      }
+      __syncthreads();
       double rt[MIST_T_D_LAST_NOCK + 1];
 #pragma unroll
       for (int i = 0; i <= MIST_T_D_LAST_NOCK; ++i)
@@ -1038,9 +1076,10 @@ __global__ __launch_bounds__(MIST_LC_TILE, MIST_REDUCE_MIN_WAVES) void eval_redu
     const MistProblem prob, const MistGroupDesc *__restrict__ groups, int n_groups,
     const int32_t *__restrict__ block_prefix, int n_blocks,
     const int32_t *__restrict__ scout_prefix, int scout, const double *__restrict__ row_terms,
-    double ratio, double *__restrict__ partial_cost, int32_t *__restrict__ partial_index) {
+    const double *__restrict__ stage_floor, double ratio, double *__restrict__ partial_cost,
+    int32_t *__restrict__ partial_index) {
   __shared__ double lds_terms[kStageRows * kLdsRowStride];
-  __shared__ double lds_min[kStageMaxOut + 1];
+  __shared__ double lds_min[kStageFloorPitch];
   __shared__ double lds_pair[MIST_LC_TILE * kPairFields];
   const int block = xcd_run_block(blockIdx.x);
   if (block >= (scout ? scout_prefix[n_groups] : n_blocks)) return;
@@ -1077,8 +1116,9 @@ __global__ __launch_bounds__(MIST_LC_TILE, MIST_REDUCE_MIN_WAVES) void eval_redu
   const int32_t *seed_index = (!scout && seeded) ? partial_index + seed_slab * slab : nullptr;
   const bool pow2 = (g->grad_accum & (g->grad_accum - 1)) == 0;
 #define MIST_REDUCE(P2, FT)                                                                   \
-  reduce_block<P2, FT>(prob, g, range, p_tile, lc_tile, row_terms, ratio, lds_terms, lds_min,  \
-                       lds_pair, seed_cost, seed_index,                                       \
+  reduce_block<P2, FT>(prob, g, range, p_tile, lc_tile, row_terms,                            \
+                       stage_floor + stage_floor_slot(g, gi, 0) * kStageFloorPitch, ratio,    \
+                       lds_terms, lds_min, lds_pair, seed_cost, seed_index,                   \
                        partial_cost + out_slab * slab, partial_index + out_slab * slab)
   if (pow2) {
     if (p_tile == 0) MIST_REDUCE(true, true); else MIST_REDUCE(true, false);
@@ -1176,12 +1216,13 @@ int mist_reduce_p_tile(void) { return MIST_P_TILE; }
 
 int mist_row_terms(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,
                    const int32_t *d_block_prefix, int n_blocks, double *d_row_terms,
-                   void *stream) {
+                   double *d_stage_floor, void *stream) {
   if (int rc = check_common(problem, d_groups, n_groups)) return rc;
-  if (!d_block_prefix || !d_row_terms) return fail(MIST_E_INVALID, "null workspace pointer");
+  if (!d_block_prefix || !d_row_terms || !d_stage_floor)
+    return fail(MIST_E_INVALID, "null workspace pointer");
   if (n_blocks <= 0) return fail(MIST_E_INVALID, "n_blocks must be positive, got %d", n_blocks);
   hipLaunchKernelGGL(row_terms_kernel, dim3(n_blocks), dim3(kTermsBlock), 0, (hipStream_t)stream,
-                     *problem, d_groups, n_groups, d_block_prefix, d_row_terms);
+                     *problem, d_groups, n_groups, d_block_prefix, d_row_terms, d_stage_floor);
   MIST_HIP_CHECK(hipGetLastError());
   return 0;
 }
@@ -1190,14 +1231,18 @@ int mist_reduce_stage_rows(void) { return kStageRows; }
 int mist_reduce_lc_tile(void) { return MIST_LC_TILE; }
 int mist_terms_block_rows(void) { return kTermsBlock; }
 int mist_reduce_scout_split(void) { return kScoutSplit; }
+int64_t mist_stage_floor_doubles(int64_t total_rows, int n_groups) {
+  if (total_rows < 0 || n_groups < 0) return -1;
+  return (total_rows / kStageRows + n_groups + 1) * kStageFloorPitch;
+}
 
 int mist_eval_reduce(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,
                      const int32_t *d_block_prefix, int n_blocks,
                      const int32_t *d_scout_prefix, int n_scout_blocks,
-                     const double *d_row_terms, double ratio, double *d_partial_cost,
-                     int32_t *d_partial_index, void *stream) {
+                     const double *d_row_terms, const double *d_stage_floor, double ratio,
+                     double *d_partial_cost, int32_t *d_partial_index, void *stream) {
   if (int rc = check_common(problem, d_groups, n_groups)) return rc;
-  if (!d_block_prefix || !d_row_terms || !d_partial_cost || !d_partial_index)
+  if (!d_block_prefix || !d_row_terms || !d_stage_floor || !d_partial_cost || !d_partial_index)
     return fail(MIST_E_INVALID, "null workspace pointer");
   if (n_blocks <= 0) return fail(MIST_E_INVALID, "n_blocks must be positive, got %d", n_blocks);
   if (!(ratio >= 0.0)) return fail(MIST_E_INVALID, "ratio must be non-negative");
@@ -1208,13 +1253,14 @@ int mist_eval_reduce(const MistProblem *problem, const MistGroupDesc *d_groups, 
   if (scout_prefix) {
     hipLaunchKernelGGL(eval_reduce_kernel, dim3(xcd_padded_grid(n_scout_blocks)), dim3(MIST_LC_TILE), 0,
                        (hipStream_t)stream, *problem, d_groups, n_groups, d_block_prefix,
-                       n_blocks, scout_prefix, 1, d_row_terms, ratio, d_partial_cost,
-                       d_partial_index);
+                       n_blocks, scout_prefix, 1, d_row_terms, d_stage_floor, ratio,
+                       d_partial_cost, d_partial_index);
     MIST_HIP_CHECK(hipGetLastError());
   }
   hipLaunchKernelGGL(eval_reduce_kernel, dim3(xcd_padded_grid(n_blocks)), dim3(MIST_LC_TILE), 0,
                      (hipStream_t)stream, *problem, d_groups, n_groups, d_block_prefix, n_blocks,
-                     scout_prefix, 0, d_row_terms, ratio, d_partial_cost, d_partial_index);
+                     scout_prefix, 0, d_row_terms, d_stage_floor, ratio, d_partial_cost,
+                     d_partial_index);
   MIST_HIP_CHECK(hipGetLastError());
   return 0;
 }
@@ -1248,17 +1294,18 @@ int mist_finalize(const MistProblem *problem, const MistGroupDesc *d_groups, int
 int mist_intra_stage_eval(const MistProblem *problem, const MistGroupDesc *d_groups,
                           int n_groups, const int32_t *d_terms_block_prefix, int n_terms_blocks,
                           const int32_t *d_reduce_block_prefix, int n_reduce_blocks,
-                          const int32_t *d_scout_prefix, int n_scout_blocks, double *d_row_terms, double *d_partial_cost, int32_t *d_partial_index,
+                          const int32_t *d_scout_prefix, int n_scout_blocks, double *d_row_terms,
+                          double *d_stage_floor, double *d_partial_cost, int32_t *d_partial_index,
                           double ratio, int sample_index, int compute_terms,
                           const MistOutTables *tables, void *stream) {
   if (compute_terms) {
     if (int rc = mist_row_terms(problem, d_groups, n_groups, d_terms_block_prefix,
-                                n_terms_blocks, d_row_terms, stream))
+                                n_terms_blocks, d_row_terms, d_stage_floor, stream))
       return rc;
   }
   if (int rc = mist_eval_reduce(problem, d_groups, n_groups, d_reduce_block_prefix,
                                 n_reduce_blocks, d_scout_prefix, n_scout_blocks, d_row_terms,
-                                ratio, d_partial_cost, d_partial_index, stream))
+                                d_stage_floor, ratio, d_partial_cost, d_partial_index, stream))
     return rc;
   return mist_finalize(problem, d_groups, n_groups, d_reduce_block_prefix, d_row_terms,
                        d_partial_cost, d_partial_index, sample_index, tables, stream);

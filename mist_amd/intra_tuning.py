@@ -267,6 +267,9 @@ class IntraStageTuner:
             scout_prefix=to_dev(plan["scout_prefix"]),
             n_scout_blocks=n_scout_blocks,
             row_terms=torch.empty(max(plan["total_rows"], 1) * _lib.ROW_TERMS, dtype=torch.float64, device=dev),
+            stage_floor=torch.empty(
+                _lib.load().mist_stage_floor_doubles(plan["total_rows"], n_groups),
+                dtype=torch.float64, device=dev),
             partial_cost=torch.empty(n_slabs * _lib.SLOTS * _lib.LC_TILE, dtype=torch.float64, device=dev),
             partial_index=torch.empty(n_slabs * _lib.SLOTS * _lib.LC_TILE, dtype=torch.int32, device=dev),
         )
@@ -290,7 +293,7 @@ class IntraStageTuner:
                     _ptr(d["terms_prefix"]), d["n_terms_blocks"],
                     _ptr(d["reduce_prefix"]), d["n_reduce_blocks"],
                     _ptr(d["scout_prefix"]), d["n_scout_blocks"],
-                    _ptr(d["row_terms"]), _ptr(d["partial_cost"]),
+                    _ptr(d["row_terms"]), _ptr(d["stage_floor"]), _ptr(d["partial_cost"]),
                     _ptr(d["partial_index"]), float(ratios[slot]), int(slot),
                     1 if i == 0 else 0, ctypes.byref(out), stream,
                 )
@@ -308,11 +311,11 @@ class IntraStageTuner:
             if i == 0:
                 timed("row_terms", lambda: lib.mist_row_terms(
                     prob_ptr, _ptr(d["groups"]), d["n_groups"], _ptr(d["terms_prefix"]),
-                    d["n_terms_blocks"], _ptr(d["row_terms"]), stream))
+                    d["n_terms_blocks"], _ptr(d["row_terms"]), _ptr(d["stage_floor"]), stream))
             timed("eval_reduce", lambda: lib.mist_eval_reduce(
                 prob_ptr, _ptr(d["groups"]), d["n_groups"], _ptr(d["reduce_prefix"]),
                 d["n_reduce_blocks"], _ptr(d["scout_prefix"]), d["n_scout_blocks"],
-                _ptr(d["row_terms"]), float(ratios[slot]),
+                _ptr(d["row_terms"]), _ptr(d["stage_floor"]), float(ratios[slot]),
                 _ptr(d["partial_cost"]), _ptr(d["partial_index"]), stream))
             timed("finalize", lambda: lib.mist_finalize(
                 prob_ptr, _ptr(d["groups"]), d["n_groups"], _ptr(d["reduce_prefix"]),

@@ -75,11 +75,22 @@ def test_row_terms_bit_exact():
         rc = lib.mist_row_terms(
             ctypes.c_void_p(plan["problem"].ctypes.data), dev["groups"].data_ptr(), dev["n_groups"],
             dev["terms_prefix"].data_ptr(), dev["n_terms_blocks"], dev["row_terms"].data_ptr(),
+            dev["stage_floor"].data_ptr(),
             ctypes.c_void_p(torch.cuda.current_stream().cuda_stream),
         )
         _lib.check(rc, "mist_row_terms")
         torch.cuda.synchronize()
         terms = dev["row_terms"].cpu().numpy().reshape(-1, _lib.ROW_TERMS)
+        # stage summaries: term-wise minima (and the maximum of "out") of each 64-row stage
+        floor = dev["stage_floor"].cpu().numpy().reshape(-1, 32)
+        n_floor_terms = _lib.TERM_NAMES.index("gcb") + 1
+        for gi, rec in enumerate(plan["groups"]):
+            off, n = int(rec["row_offset"]), int(rec["n_rows"])
+            for st in range((n + _lib.STAGE_ROWS - 1) // _lib.STAGE_ROWS):
+                rows = terms[off + st * _lib.STAGE_ROWS: off + min((st + 1) * _lib.STAGE_ROWS, n)]
+                got_floor = floor[off // _lib.STAGE_ROWS + gi + st]
+                assert np.array_equal(got_floor[:n_floor_terms], rows[:, :n_floor_terms].min(axis=0))
+                assert got_floor[n_floor_terms] == rows[:, _lib.TERM_NAMES.index("out")].max()
         L = cfg.model.num_hidden_layers
         assert len(plan["groups"]) > 0
         for rec in plan["groups"]:

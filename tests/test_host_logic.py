@@ -205,15 +205,17 @@ def test_library_loads_and_exports_every_declared_symbol():
 def test_argument_checks_reject_before_any_launch():
     """Host-side validation paths of the C ABI (no GPU needed: they return before launching)."""
     lib = _lib.load()
-    assert lib.mist_row_terms(None, None, 1, None, 1, None, None) == -1
+    assert lib.mist_row_terms(None, None, 1, None, 1, None, None, None) == -1
     assert b"null" in lib.mist_last_error()
     prob = make_problem(load_plan(1)[0], 4, 2, 1, 4, 2)
     pp = ctypes.c_void_p(prob.ctypes.data)
     fake = ctypes.c_void_p(4096)
-    assert lib.mist_row_terms(pp, fake, 0, fake, 1, fake, None) == -1
-    assert lib.mist_eval_reduce(pp, fake, 1, fake, 0, None, 0, fake, 1.0, fake, fake, None) == -1
-    assert lib.mist_eval_reduce(pp, fake, 1, fake, 1, None, 0, fake, -1.0, fake, fake, None) == -1
-    assert lib.mist_eval_reduce(pp, fake, 1, fake, 1, None, 3, fake, 1.0, fake, fake, None) == -1
+    assert lib.mist_row_terms(pp, fake, 0, fake, 1, fake, fake, None) == -1
+    assert lib.mist_row_terms(pp, fake, 1, fake, 1, fake, None, None) == -1
+    assert lib.mist_stage_floor_doubles(640, 3) == (10 + 3 + 1) * 32 and lib.mist_stage_floor_doubles(-1, 3) == -1
+    assert lib.mist_eval_reduce(pp, fake, 1, fake, 0, None, 0, fake, fake, 1.0, fake, fake, None) == -1
+    assert lib.mist_eval_reduce(pp, fake, 1, fake, 1, None, 0, fake, fake, -1.0, fake, fake, None) == -1
+    assert lib.mist_eval_reduce(pp, fake, 1, fake, 1, None, 3, fake, fake, 1.0, fake, fake, None) == -1
     assert b"scout" in lib.mist_last_error()
     tabs = _lib.OutTables()
     assert lib.mist_finalize(pp, fake, 1, fake, fake, fake, fake, 0, ctypes.byref(tabs), None) == -1

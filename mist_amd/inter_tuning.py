@@ -173,7 +173,9 @@ class _DpRunner:
             h_values = values[:total].cpu().numpy()
             h_request = request[:total].cpu().numpy()
         self.selected += total
-        order = np.argsort(h_request, kind="stable")  # group by request (small integer keys)
+        # group by request: 16-bit keys (the entry point takes at most 65535 requests) make the
+        # stable sort a radix sort
+        order = np.argsort(h_request.astype(np.uint16), kind="stable")
         h_values, h_request = h_values[order], h_request[order]
         bounds = np.searchsorted(h_request, np.arange(n + 1))
         return [(np.sort(h_values[bounds[i]:bounds[i + 1]]), int(h_counts[1 + i])) for i in range(n)]
@@ -420,7 +422,17 @@ class _Scan:
         """Dry run of ``replay`` under the bound ``best_cost`` (the true running best when this G
         is reached is no larger, so the true scan stops no later): True if the computed results
         would not suffice."""
-        pos, hi, G = self.pos, self.have_lo + len(self.cost), self.G
+        pos, hi = self.pos, self.have_lo + len(self.cost)
+        end = min(hi, len(self.scaled))
+        if pos < end:  # the part that is materialised and computed, as plain python floats
+            scaled = self.scaled[pos:end].tolist()
+            cost = self.cost[pos - self.have_lo:end - self.have_lo].tolist()
+            for s, c in zip(scaled, cost):
+                if s >= best_cost:
+                    return False
+                if c < best_cost:
+                    best_cost = c
+            pos = end
         while self._reach(pos, best_cost):
             if self.scaled[pos] >= best_cost:
                 return False
@@ -436,10 +448,21 @@ class _Scan:
     def replay(self, best_cost: float, best_t):
         """Advances the sequential scan as far as the computed results allow.  Returns
         (best_cost, best_t, finished)."""
-        G = self.G
         hi = self.have_lo + len(self.cost)
+        end = min(hi, len(self.scaled))
+        if self.pos < end:  # the part that is materialised and computed, as plain python floats
+            first = self.pos
+            scaled = self.scaled[first:end].tolist()
+            cost = self.cost[first - self.have_lo:end - self.have_lo].tolist()
+            for j, (s, c) in enumerate(zip(scaled, cost)):
+                if s >= best_cost:  # inter_tuning.py:196-197
+                    self.pos = first + j
+                    return best_cost, best_t, True
+                if c < best_cost:
+                    best_cost, best_t = c, self.tmax[first + j]
+            self.pos = end
         while self._reach(self.pos, best_cost):
-            if self.scaled[self.pos] >= best_cost:  # inter_tuning.py:196-197
+            if self.scaled[self.pos] >= best_cost:
                 return best_cost, best_t, True
             if self.pos >= hi:
                 return best_cost, best_t, False     # needs more DP results
@@ -450,21 +473,28 @@ class _Scan:
         return best_cost, best_t, True
 
 
+def _solution_cell(num_layers, g, p, layer_start, layer_end, q, c, slot=0):
+    """Table variant and cell of a stage's strategy (inter_tuning.py:38-60 with the sample slot
+    made explicit)."""
+    l = layer_end - layer_start + 1
+    if layer_start == 0 and layer_end == num_layers - 1:
+        return 3, (g, q, c, slot)
+    if layer_start == 0:
+        return 1, (g, q, p, l - 1, c, slot)
+    if layer_end == num_layers - 1:
+        return 2, (g, q, l - 1, c, slot)
+    return 0, (g, q, p, l - 1, c, slot)
+
+
 def get_solution_from_intra_stage_tuner_output(
     intra_stage_results, num_layers, gradient_accumulation_steps_index, pre_saved_micro_batches,
     layer_start, layer_end, device_mesh_idx, num_ckpt_layers, slot=0,
 ):
-    """inter_tuning.py:38-60 with the sample slot made explicit."""
-    g, q, p, c = gradient_accumulation_steps_index, device_mesh_idx, pre_saved_micro_batches, num_ckpt_layers
-    l = layer_end - layer_start + 1
-    r = intra_stage_results
-    if layer_start == 0 and layer_end == num_layers - 1:
-        return r.solution_at(3, (g, q, c, slot))
-    if layer_start == 0:
-        return r.solution_at(1, (g, q, p, l - 1, c, slot))
-    if layer_end == num_layers - 1:
-        return r.solution_at(2, (g, q, l - 1, c, slot))
-    return r.solution_at(0, (g, q, p, l - 1, c, slot))
+    """inter_tuning.py:38-60."""
+    variant, cell = _solution_cell(
+        num_layers, gradient_accumulation_steps_index, pre_saved_micro_batches, layer_start,
+        layer_end, device_mesh_idx, num_ckpt_layers, slot)
+    return intra_stage_results.solution_at(variant, cell)
 
 
 def _same_batch(results_list) -> bool:
@@ -578,20 +608,25 @@ def _solutions(runner: _DpRunner, results_list, bests, n_g, g_index, q_index, nu
             np.array([bests[t][2] for t in winners], dtype=np.float32),
             np.array([bests[t][1] for t in winners], dtype=np.int64))
         found = dict(zip(winners, parts))
+    # strategy rows of all stages of all winners: one read-back
+    requests = []
+    for t in winners:
+        g = g_index[bests[t][1]]
+        inter = found[t][1]
+        for i, ((l0, l1), (n, m), ckpt) in enumerate(inter):
+            variant, cell = _solution_cell(num_layers, g, len(inter) - i - 1, l0, l1, q_index[(n, m)], ckpt, slot)
+            requests.append((results_list[t], variant, cell))
+    rows = iter(IntraStageTunerOutput.solutions_at(requests)) if requests else iter(())
     out = []
     for t, (best_cost, best_G, best_t) in enumerate(bests):
         if best_G is None:
             out.append((float("inf"), None))
             continue
-        r = results_list[t]
-        g = g_index[best_G]
         total, inter = found[t]
         assert total == best_cost
         solution = [best_G, []]
-        for i, ((l0, l1), (n, m), ckpt) in enumerate(inter):
-            row = get_solution_from_intra_stage_tuner_output(
-                r, num_layers, g, len(inter) - i - 1, l0, l1, q_index[(n, m)], ckpt, slot
-            ).tolist()
+        for (l0, l1), (n, m), ckpt in inter:
+            row = next(rows).tolist()
             row[:6] = [int(x) for x in row[:6]]
             solution[1].append((((l0, l1), (n, m), ckpt, 0), tuple(row)))
         out.append((best_cost, solution))

@@ -201,6 +201,7 @@ def inter_stage_tune(
     prob, layers, slots = best
     nl = prob.shape.layers_max - prob.shape.layers_min + 1
     solution: List[Any] = [prob.G, []]
+    requests = []
     covered = 0
     for i in range(prob.S):
         j, a = int(layers[i]), int(slots[i])
@@ -212,7 +213,10 @@ def inter_stage_tune(
         l0, l1 = covered, covered + j - 1
         covered += j
         variant, cell = _variant_cell(num_layers, prob.g, prob.q, prob.S - i - 1, l0, l1, ckpt, policy)
-        row = res.solution_at(variant, cell).tolist()
+        requests.append((res, variant, cell))
+        solution[1].append(((l0, l1), prob.mesh, ckpt, policy))
+    for i, row in enumerate(IntraStageTunerOutput.solutions_at(requests)):  # one read-back
+        row = row.tolist()
         row[:6] = [int(v) for v in row[:6]]
-        solution[1].append((((l0, l1), prob.mesh, ckpt, policy), tuple(row)))
+        solution[1][i] = (solution[1][i], tuple(row))
     return best_cost, solution

@@ -113,6 +113,26 @@ class IntraStageTunerOutput:
         row = int(idx[cell]) if idx is not None else int(self.device.index[variant][cell].item())
         return self.spaces[(cell[0], cell[1])].decode(np.array(row))
 
+    @staticmethod
+    def solutions_at(requests) -> List[np.ndarray]:
+        """``solution_at`` for many ``(results, variant, cell)`` requests (results objects on one
+        device) with a single read-back of the row indices that are not on the host yet."""
+        rows: List[Optional[int]] = []
+        pending = []
+        for i, (res, variant, cell) in enumerate(requests):
+            idx = res._host.get(f"index{variant}")
+            rows.append(int(idx[cell]) if idx is not None else None)
+            if idx is None:
+                pending.append(i)
+        if pending:
+            fetched = torch.stack(
+                [requests[i][0].device.index[requests[i][1]][requests[i][2]] for i in pending]
+            ).cpu().numpy()
+            for i, row in zip(pending, fetched):
+                rows[i] = int(row)
+        return [res.spaces[(cell[0], cell[1])].decode(np.array(row))
+                for (res, _, cell), row in zip(requests, rows)]
+
     def __getattr__(self, name: str):
         for v, suffix in enumerate(VARIANTS):
             if name == "costs_stable" + suffix:

@@ -730,6 +730,24 @@ __device__ __forceinline__ void reduce_block(
   lds_pair[threadIdx.x * kPairFields + 2] = n_ck;
   lds_pair[threadIdx.x * kPairFields + 3] = n_nock;
   auto div_G = [&](double v) { return kPow2G ? v * inv_G64 : v / G64; };
+  // Group-wide terms the composite objectives add to the base latency (see `examine`): with x, d
+  // the float32-rounded stable / delta latency,
+  //   with_pre  = r (x + pre_fwd + pre_bwd + w1 + w2) + (d + w1d + w2d) / G
+  //   with_post = r (x + post_fwd + [row terms >= 0]) + (d + [row terms >= 0]) / G
+  //   no_pp     = r (x + pre_fwd + pre_bwd + post_fwd + [..] + w1 + w2 + [..]) + (d + w1d + w2d + [..]) / G
+  // so each is at least r x + d / G plus the offset below, up to a few roundings of relative
+  // size 1e-16 (all terms are non-negative).  A row can beat a minimum `t` of such an objective
+  // only if r x + d / G <= t - offset; the offsets are taken 1e-9 short and `t` 1e-9 long, far
+  // more than the roundings and far less than anything that matters for pruning.
+  constexpr double kSlack = 1e-9;
+  const double off_pre =
+      (ratio * (k.pre_fwd + k.pre_bwd + k.w1 + k.w2) + div_G(k.w1d + k.w2d)) * (1.0 - kSlack);
+  const double off_post = ratio * k.post_fwd * (1.0 - kSlack);
+  const double off_pp = (ratio * (k.pre_fwd + k.pre_bwd + k.post_fwd + k.w1 + k.w2) +
+                         div_G(k.w1d + k.w2d)) * (1.0 - kSlack);
+  auto below = [&](double t, double offset) {
+    return fabs(t) == INFINITY ? t : (t - offset) + kSlack * fabs(t);
+  };
 
   // Memory model of one candidate row for this lane's (l, c) (:2150-2162, 2358-2385, 2755-2786).
   // `t` may also be the term-wise minimum of a stage: every operation below is monotone in
@@ -942,12 +960,15 @@ __device__ __forceinline__ void reduce_block(
     const int cnt_b = count_bound([&](int p) { return floor_mem.scaled_base(p); });
     const int cnt_p =
         count_bound([&](int p) { return floor_mem.scaled_pre(p, pre_saved, pre_sas); });
-    double thr_b = -INFINITY, thr_o = -INFINITY;
+    double thr_b = -INFINITY, thr_p = -INFINITY;
 #pragma unroll
     for (int j = 0; j < MIST_P_TILE; ++j) {  // minima are non-decreasing; empty slots hold +inf
       thr_b = j < cnt_b ? best_b[j] : thr_b;
-      thr_o = j < cnt_p ? best_p[j] : thr_o;
+      thr_p = j < cnt_p ? best_p[j] : thr_p;
     }
+    // One threshold for the three composite objectives, expressed for `bound` (objective()):
+    // each of them exceeds `bound` by at least its group-wide offset.
+    double thr_o = below(thr_p, off_pre);
     if (do_post) {
       // Lower bounds of the last-stage / single-stage peaks (:2946-3106) from the pseudo row.
       double peak_f, peak_b;
@@ -958,12 +979,13 @@ __device__ __forceinline__ void reduce_block(
           floor_mem.bwd_states + post_states + floor_mem.mod_saved + post_bwd_peak + floor_mem.gcb;
       const double pf_post = fmax(f_in, peak_f + post_states);
       const double pb_post = fmax(b_in, peak_b - lds_min[kStageMaxOut] + post_states) + post_output;
-      if (fmax(pf_post, pb_post) * floor_mem.mf_pp <= cap) thr_o = fmax(thr_o, best_post);
+      if (fmax(pf_post, pb_post) * floor_mem.mf_pp <= cap)
+        thr_o = fmax(thr_o, below(best_post, off_post));
       if (do_nopp) {
         const double pf_pp = pf_post + pre_states + pre_saved;
         const double pb_pp = pb_post + pre_states + pre_saved;
         if (fmax(pf_pp, pb_pp) * lds_min[MIST_T_MF] <= cap)
-          thr_o = fmax(thr_o, best_pp);
+          thr_o = fmax(thr_o, below(best_pp, off_pp));
       }
     }
 

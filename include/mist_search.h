@@ -201,6 +201,21 @@ int mist_intra_stage_eval(const MistProblem *problem, const MistGroupDesc *d_gro
                           double ratio, int sample_index, int compute_terms,
                           const MistOutTables *tables, void *stream);
 
+/* Analysis path: what batched_stage_analyze(get_best_solution=False) reports
+ * (mist/analyzer/batched_module_analyzer.py:2788-2803, 2876-2892, 2980-2996, 3063-3079) for given
+ * strategy rows, without the memory mask.  d_requests: [n_requests][5] int32 = (group, workspace
+ * position of the row within the group, layers l, ckpt layers c <= l, pre-saved micro-batches p);
+ * d_row_terms as written by mist_row_terms.  d_out: [n_requests][MIST_ANALYZE_FIELDS] float64 =
+ * for the variants middle stage, first stage (with_pre), last stage (with_post) and single stage
+ * (pre_and_post), five values each: stable latency, delta latency, stable + delta / G, forward
+ * peak MB, backward peak MB.  The last two variants are evaluated with the peaks at the request's
+ * p; the reference reports them for p == 0 only.  An invalid request yields NaN. */
+#define MIST_ANALYZE_REQUEST_FIELDS 5
+#define MIST_ANALYZE_FIELDS 20
+int mist_stage_analyze(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,
+                       const double *d_row_terms, const int32_t *d_requests, int n_requests,
+                       double *d_out, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

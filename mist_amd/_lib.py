@@ -121,6 +121,8 @@ _SIGNATURES = {
         ctypes.c_int,
         [_VP, _VP, ctypes.c_int, _VP, _VP, _VP, _VP, ctypes.c_int, ctypes.POINTER(OutTables), _VP],
     ),
+    "mist_stage_analyze": (
+        ctypes.c_int, [_VP, _VP, ctypes.c_int, _VP, _VP, ctypes.c_int, _VP, _VP]),
     "mist_intra_stage_eval": (
         ctypes.c_int,
         [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, ctypes.c_int,
@@ -188,6 +190,7 @@ _DP_SIGNATURES = {
 }
 
 
+ANALYZE_REQUEST_FIELDS, ANALYZE_FIELDS = 5, 20
 MIP_CKPT_TUNED, MIP_CKPT_FIXED, MIP_CKPT_FULL = 0, 1, 2
 MIP_MAX_SAMPLES = 64
 MIP_MAX_VALUE = 1000000.0

@@ -1,0 +1,233 @@
+"""Analysis path: predicted iteration latency and peak memory of ONE given strategy.
+
+Drop-in for the reference's ``benchmark/mist/analysis/run.py`` (``analyze`` :37-185) and for the
+``get_best_solution=False`` mode of ``batched_stage_analyze``
+(mist/analyzer/batched_module_analyzer.py:687-3144, result entries :2788-2803, 2876-2892,
+2980-2996, 3063-3079).  The strategy comes from the ``strategy`` block of the configuration, in
+the form ``tune_one_case`` writes it.
+
+A stage is one group descriptor whose search space is the single given row; the row-terms kernel
+and ``mist_stage_analyze`` evaluate it on the GPU with the code the search uses (there is no CPU
+path).  Of the ~100 entries of the reference's per-cell dictionaries the ones its driver reads
+are returned: ``latency``, ``mem_fwd_peak``, ``mem_bwd_peak`` and the stable / delta latency of
+each variant (``****latency_stable`` ..., :2550-2567); the other entries only serve its log
+output.  As in the reference the pre/post layer strategy is ``strategy.pre_post_strategy``
+(``preset``, ``dp``, ``intra-node-tp-*`` or ``tuned``), nothing is masked by the memory capacity,
+and a pre/post batch size outside 1..4 yields empty dictionaries (:868-880).
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+from typing import Any, Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from . import _lib
+from .comm_model import gpu_gpu_comm_latency
+from .config import BATCH_SIZE_CANDIDATES, MistConfig
+from .layer_tables import LayerTables
+from .search_space import SearchSpace
+from .stage_inputs import GroupInputBuilder, make_problem, pre_post_strategy_fields
+
+_VARIANT_KEYS = ("", "_with_pre", "_with_post", "_with_pre_and_post")
+
+
+def _single_row_space(row: Sequence[float]) -> SearchSpace:
+    return SearchSpace(
+        par=np.array([list(row[:6])], dtype=np.float64),
+        wo=(float(row[6]),), go=(float(row[7]),), oo=(float(row[8]),), ao=(float(row[9]),),
+        pair_wo=np.zeros(1, dtype=np.uint8), pair_go=np.zeros(1, dtype=np.uint8),
+    )
+
+
+def _pre_post_batch_ok(config: MistConfig, n: int, m: int, G: int, row) -> bool:
+    """batched_module_analyzer.py:862-880."""
+    pp_dp = pre_post_strategy_fields(config, n, m, row)[0]
+    b = config.training.global_batch_size // G // pp_dp
+    return 1 <= b <= max(BATCH_SIZE_CANDIDATES)
+
+
+def analyze_cells(config: MistConfig, tables: LayerTables, stages, device: str = "cuda:0"):
+    """``stages``: list of ``(num_nodes, num_gpus_per_node, G, strategy_row, [(p, l, c), ...])``.
+    Returns per stage a dict ``(p, l, c) -> float64[4][5]`` (variant x (stable, delta, stable +
+    delta / G, forward peak, backward peak)), or None for a stage whose pre/post batch size is
+    out of range.  One launch of each kernel for all stages."""
+    dev = torch.device(device)
+    if dev.type != "cuda" or not torch.cuda.is_available():
+        raise _lib.MistLibraryError("the analysis path needs a GPU: the kernels have no CPU path")
+    lib = _lib.load()
+    L = int(config.model.num_hidden_layers)
+    live = [i for i, (n, m, G, row, _) in enumerate(stages) if _pre_post_batch_ok(config, n, m, G, row)]
+    out: List[Optional[Dict[Tuple[int, int, int], np.ndarray]]] = [None] * len(stages)
+    if not live:
+        return out
+    builder = GroupInputBuilder(config, tables)
+    groups = np.zeros(len(live), dtype=_lib.GROUP_DTYPE)
+    requests = []
+    for gi, i in enumerate(live):
+        n, m, G, row, cells = stages[i]
+        builder.fill(groups[gi], _single_row_space(row), 0, gi, n, m, G, 1, analysis_row=row)
+        groups[gi]["row_offset"] = gi
+        for p, l, c in cells:
+            if not (1 <= l <= L and 0 <= c <= l and p >= 0):
+                raise ValueError(f"cell (p={p}, l={l}, c={c}) outside 1 <= l <= {L}, 0 <= c <= l, p >= 0")
+            requests.append((gi, 0, l, c, p))
+    if not requests:
+        return [({} if i in live else None) for i in range(len(stages))]
+    problem = make_problem(config, L, 1, 1, 1, len(live))
+    n_groups = len(live)
+    terms_prefix = np.arange(n_groups + 1, dtype=np.int32)  # one workgroup per single-row group
+    req = np.asarray(requests, dtype=np.int32)
+    with torch.cuda.device(dev):
+        to_dev = lambda a: torch.from_numpy(np.ascontiguousarray(a).view(np.uint8).reshape(-1)).to(dev)
+        d_groups, d_prefix, d_req = to_dev(groups), to_dev(terms_prefix), to_dev(req)
+        row_terms = torch.empty(n_groups * _lib.ROW_TERMS, dtype=torch.float64, device=dev)
+        stage_floor = torch.empty(lib.mist_stage_floor_doubles(n_groups, n_groups), dtype=torch.float64, device=dev)
+        result = torch.empty((len(requests), _lib.ANALYZE_FIELDS), dtype=torch.float64, device=dev)
+        stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+        prob_ptr = ctypes.c_void_p(problem.ctypes.data)
+        _lib.check(lib.mist_row_terms(prob_ptr, d_groups.data_ptr(), n_groups, d_prefix.data_ptr(),
+                                      n_groups, row_terms.data_ptr(), stage_floor.data_ptr(), stream),
+                   "mist_row_terms")
+        _lib.check(lib.mist_stage_analyze(prob_ptr, d_groups.data_ptr(), n_groups, row_terms.data_ptr(),
+                                          d_req.data_ptr(), len(requests), result.data_ptr(), stream),
+                   "mist_stage_analyze")
+        host = result.cpu().numpy().reshape(len(requests), 4, 5)
+    for i in live:
+        out[i] = {}
+    for (gi, _, l, c, p), values in zip(requests, host):
+        out[live[gi]][(p, l, c)] = values
+    return out
+
+
+def _p2p_output_latency(config: MistConfig, tables: LayerTables, m: int, row) -> float:
+    """Twice the p2p latency of the layer output (batched_module_analyzer.py:1298-1308)."""
+    out_mb = float(tables.mem_output("block", np.float64(row[0]), np.float64(row[2])))
+    across_nodes = m == config.hardware.num_gpus_per_node
+    return float(gpu_gpu_comm_latency(
+        "p2p", np.float64(out_mb) / 1024, inter_size=1 if across_nodes else None,
+        intra_size=None if across_nodes else 1,
+        gpu_gpu_comm_params=config.hardware.gpu_gpu_comm_params)) * 2
+
+
+def _entries(values: np.ndarray, p: int, p2p: float):
+    """The four per-variant dictionaries of one cell; the last two only exist for p == 0."""
+    dicts = []
+    for v, suffix in enumerate(_VARIANT_KEYS):
+        if v >= 2 and p != 0:
+            dicts.append(None)
+            continue
+        stable, delta, latency, fwd, bwd = (float(x) for x in values[v])
+        entry = {
+            # the pre-and-post variant carries no p2p term (:3071)
+            "latency": latency if v == 3 else latency + p2p,
+            "mem_fwd_peak": fwd,
+            "mem_bwd_peak": bwd,
+        }
+        for w, key in enumerate(_VARIANT_KEYS):
+            if w >= 2 and p != 0:
+                continue
+            entry["****latency_stable" + key] = float(values[w][0])
+            entry["****latency_delta" + key] = float(values[w][1])
+        dicts.append(entry)
+    return dicts
+
+
+def batched_stage_analyze(
+    layer_tables: LayerTables,
+    pre_saved_micro_batches_candidates: List[int],
+    num_layers_candidates: List[int],
+    num_ckpt_layers_candidates: List[int],
+    num_nodes: int,
+    num_gpus_per_node: int,
+    gradient_accumulation_steps: int,
+    stage_strategies,
+    config: MistConfig,
+    device: str = "cuda:0",
+):
+    """``batched_stage_analyze(..., get_best_solution=False)`` of the reference for one strategy
+    row (the three ``LayerInfo`` arguments are replaced by ``layer_tables``).  Returns the four
+    dictionaries ``results, results_with_pre, results_with_post, results_with_pre_and_post`` keyed
+    ``(pre_saved_micro_batches, num_layers, num_ckpt_layers)``."""
+    row = np.asarray(stage_strategies, dtype=np.float64).reshape(-1)
+    if row.shape[0] != 10:
+        raise ValueError("the analysis path takes exactly one strategy row of 10 values")
+    cells = [(p, l, c) for c in num_ckpt_layers_candidates for p in pre_saved_micro_batches_candidates
+             for l in num_layers_candidates if c <= l]
+    (found,) = analyze_cells(
+        config, layer_tables, [(num_nodes, num_gpus_per_node, gradient_accumulation_steps, row, cells)],
+        device)
+    results: Tuple[Dict, Dict, Dict, Dict] = ({}, {}, {}, {})
+    if found is None:
+        return results
+    p2p = _p2p_output_latency(config, layer_tables, num_gpus_per_node, row)
+    for (p, l, c), values in found.items():
+        for v, entry in enumerate(_entries(values, p, p2p)):
+            if entry is not None:
+                results[v][(p, l, c)] = entry
+    return results
+
+
+def analyze(mist_config: MistConfig, layer_tables: Optional[LayerTables] = None, device: str = "cuda:0"):
+    """run.py:37-185.  Returns ``(total_latency, stage_stable_latencies, stage_delta_latencies,
+    stage_peak_memories)``."""
+    st = mist_config.strategy
+    if st is None or "layer_partitions" not in st:
+        raise ValueError("the strategy block is missing or disabled")
+    tables = LayerTables(mist_config) if layer_tables is None else layer_tables
+    S, G = st.num_stages, st.gradient_accumulation_steps
+    stages, keys = [], []
+    for i in range(S):
+        p = min(S - i - 1, G - 1)                                            # run.py:57-59
+        l, c = st.layer_partitions[i], st.gradient_checkpointing[i]
+        n, m = st.device_assignment[i]
+        stages.append((n, m, G, st.stage_strategies[i], [(p, l, c)]))
+        keys.append((p, l, c))
+    found = analyze_cells(mist_config, tables, stages, device)
+    results = []
+    for i, (cells, key) in enumerate(zip(found, keys)):
+        variant = 3 if S == 1 else (1 if i == 0 else (2 if i == S - 1 else 0))
+        entry = None
+        if cells is not None:
+            p2p = _p2p_output_latency(mist_config, tables, stages[i][1], stages[i][3])
+            entry = _entries(cells[key], key[0], p2p)[variant]
+        if entry is None:
+            raise KeyError(key)  # the reference indexes its empty result dictionary (run.py:84-93)
+        results.append((entry, _VARIANT_KEYS[variant]))
+    if S == 1:
+        entry, _ = results[0]
+        total = entry["latency"] * G
+        # run.py:113-114 overwrites the stable list with [0] and leaves the delta list empty
+        return total, [0], [], [max(entry["mem_fwd_peak"], entry["mem_bwd_peak"])]
+    uniform = bool(getattr(mist_config, "disable_non_uniform_pp_micro_batch_analysis", False))
+    stable, delta, peaks = [], [], []
+    for entry, suffix in results:
+        if uniform:
+            stable.append(entry["latency"])
+            delta.append(0)
+        else:
+            stable.append(entry["****latency_stable" + suffix])
+            delta.append(entry["****latency_delta" + suffix])
+        peaks.append(max(entry["mem_fwd_peak"], entry["mem_bwd_peak"]))
+    total = sum(stable) + max(stable) * (G - 1)
+    if not uniform:
+        total = total + max(d - sum(stable[i] for i in range(s)) for s, d in enumerate(delta))
+    return total, stable, delta, peaks
+
+
+def main(argv: Optional[List[str]] = None) -> None:
+    parser = argparse.ArgumentParser(description="Predicted latency and peak memory of the strategy block of a plan")
+    parser.add_argument("--config", required=True, help="resolved YAML with an enabled strategy block")
+    parser.add_argument("--device", default="cuda:0")
+    args = parser.parse_args(argv)
+    total, stable, delta, peaks = analyze(MistConfig.from_yaml(args.config), device=args.device)
+    print(f"Stage Stable Latencies: {stable}")
+    print(f"Stage Delta Latencies: {delta}")
+    print(f"Total latency: {total}")
+    print(f"Peak memory (MB): {peaks}")
+
+
+if __name__ == "__main__":
+    main()

@@ -130,6 +130,36 @@ class TuningConfig(_Section):
             d[key] = bool(d.get(key, False))
 
 
+class StrategyConfig(_Section):
+    """mist/config.py:425-492: one strategy (the tuner's output, the analysis path's input)."""
+
+    def __init__(self, data: Dict[str, Any]):
+        super().__init__(data)
+        d = object.__getattribute__(self, "_data")
+        n = len(d["layer_partitions"])
+        assert n == len(d["device_assignment"]) == len(d["stage_strategies"]) == len(d["gradient_checkpointing"]), (
+            "The length of layer_partitions, device_assignment, stage_strategies, and "
+            "gradient_checkpointing should be the same."
+        )
+        d["num_stages"] = n
+        d["layer_partitions"] = [int(x) for x in d["layer_partitions"]]
+        d["gradient_checkpointing"] = [int(x) for x in d["gradient_checkpointing"]]
+        d["gradient_accumulation_steps"] = int(d["gradient_accumulation_steps"])
+        for a in d["device_assignment"]:
+            assert len(a) == 2, f"Device assignment should be [num_nodes, num_gpus_per_node], got {a}"
+        d["device_assignment"] = [tuple(int(x) for x in a) for a in d["device_assignment"]]
+
+        def row(r):
+            assert len(r) == 10, f"a strategy row has 10 entries, got {r}"
+            return tuple([int(x) for x in r[:3]] + [bool(x) for x in r[3:6]] + [float(x) for x in r[6:]])
+
+        d["stage_strategies"] = [row(r) for r in d["stage_strategies"]]
+        d.setdefault("pre_post_strategy", "heuristic")
+        if d["pre_post_strategy"] == "preset":
+            assert d.get("pre_post_strategy_array") is not None, "preset needs pre_post_strategy_array"
+            d["pre_post_strategy_array"] = list(row(d["pre_post_strategy_array"]))
+
+
 class MistConfig:
     """Attribute-compatible stand-in for the reference's ``MistConfig``."""
 
@@ -143,7 +173,11 @@ class MistConfig:
         tuning = raw.get("tuning")
         self.tuning = TuningConfig(tuning) if tuning and tuning.get("enabled", True) else None
         strategy = raw.get("strategy")
-        self.strategy = _Section(strategy) if strategy and strategy.get("enabled", False) else None
+        if strategy and strategy.get("enabled", False):
+            # a block without partitions only carries the preset pre/post strategy of a tuning run
+            self.strategy = StrategyConfig(strategy) if "layer_partitions" in strategy else _Section(strategy)
+        else:
+            self.strategy = None
 
     def __getattr__(self, name: str):
         # Only reached when normal lookup fails: fall through to the raw YAML top level

@@ -1220,6 +1220,89 @@ __global__ __launch_bounds__(256) void finalize_kernel(
   tables.index[variant][at] = best_row;
 }
 
+// ------------------------------------------------------------------------------------------
+// Analysis path: the quantities batched_stage_analyze(get_best_solution=False) reports for ONE
+// given strategy row and one (layers, ckpt, pre-saved micro-batches) cell
+// (batched_module_analyzer.py:2788-2803, 2876-2892, 2980-2996, 3063-3079), unmasked.
+// One thread per request; per variant (middle, first, last, single stage): stable latency, delta
+// latency, stable + delta / G, forward peak, backward peak.
+// ------------------------------------------------------------------------------------------
+__device__ __forceinline__ LaneMemory cell_memory(const double *__restrict__ t, int l, int c) {
+  const double lf = (double)l, lm1 = (double)max(l - 1, 0), cf = (double)c;
+  const double S_ck = t[MIST_T_S_CK], S_nock = t[MIST_T_S_NOCK];
+  LaneMemory mem;
+  mem.fwd_states = t[MIST_T_FWD_STATES0] + lf * t[MIST_T_PWG] + lm1 * t[MIST_T_PO];  // :2150-2162
+  mem.bwd_states = t[MIST_T_BWD_STATES0] + lf * t[MIST_T_PWGO];
+  mem.cur_saved = c == l ? (lf - 1.0) * S_ck : cf * S_ck + (double)(l - c - 1) * S_nock;  // :2358-2385
+  mem.mod_saved = S_ck * cf + S_nock * (double)(l - c);
+  mem.ck_delta = c >= l - 1 ? t[MIST_T_D_CK] : t[MIST_T_D_NOCK];  // :2760-2769
+  mem.fwd_pk = t[MIST_T_FWD_PEAK];
+  mem.bwd_pk = t[MIST_T_BWD_PEAK];
+  mem.out = t[MIST_T_OUT];
+  mem.gcb = t[MIST_T_GCB];
+  mem.mf_base = t[MIST_T_MF_BASE];
+  mem.mf_pp = t[MIST_T_MF_PP];
+  return mem;
+}
+
+__global__ __launch_bounds__(64) void analyze_kernel(
+    const MistProblem prob, const MistGroupDesc *__restrict__ groups, int n_groups,
+    const double *__restrict__ row_terms, const int32_t *__restrict__ requests, int n_requests,
+    double *__restrict__ out) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n_requests) return;
+  const int32_t *req = requests + (int64_t)i * MIST_ANALYZE_REQUEST_FIELDS;
+  double *o = out + (int64_t)i * MIST_ANALYZE_FIELDS;
+  const int gi = req[0], l = req[2], c = req[3], p = req[4];
+  const int64_t pos = req[1];
+  const bool ok = gi >= 0 && gi < n_groups && l >= 1 && l <= prob.num_layers && c >= 0 && c <= l &&
+                  p >= 0 && pos >= 0 && pos < groups[min(max(gi, 0), n_groups - 1)].n_rows;
+  if (!ok) {
+    for (int f = 0; f < MIST_ANALYZE_FIELDS; ++f) o[f] = NAN;
+    return;
+  }
+  const MistGroupDesc *g = groups + gi;
+  const double *t = row_terms + (g->row_offset + pos) * MIST_ROW_TERMS;
+  const GroupConsts k = group_consts(g);
+  const CellLatency lat = cell_latency<true>(t, l, c, k);
+  const LaneMemory mem = cell_memory(t, l, c);
+  const double G64 = (double)g->grad_accum;
+  const float G32 = (float)g->grad_accum;
+  double peak_f, peak_b;
+  mem.peaks(p, peak_f, peak_b);
+  // middle stage: float32 stable + float32 delta / G stays float32 (:2212-2216)
+  o[0] = (double)lat.x;
+  o[1] = (double)lat.d;
+  o[2] = (double)(lat.x + lat.d / G32);
+  o[3] = peak_f;
+  o[4] = peak_b;
+  // first stage (:2866-2875)
+  const double pre_p = (double)p * g->pre_saved;
+  o[5] = lat.sp;
+  o[6] = lat.dpre;
+  o[7] = lat.sp + lat.dpre / G64;
+  o[8] = pre_p + peak_f + g->pre_states_and_saved;
+  o[9] = pre_p + peak_b + g->pre_states_and_saved;
+  // last stage (:2946-2979); the reference evaluates it for p == 0 only
+  const double f_in =
+      mem.fwd_states + g->post_states + mem.mod_saved + g->post_fwd_peak + mem.gcb;
+  const double b_in = mem.bwd_states + g->post_states + mem.mod_saved + g->post_bwd_peak +
+                      (c == 0 ? t[MIST_T_RD] : 0.0) + mem.gcb;
+  const double pf_post = fmax(f_in, peak_f + g->post_states);
+  const double pb_post = fmax(b_in, peak_b - mem.out + g->post_states) + g->post_output;
+  o[10] = lat.spost;
+  o[11] = lat.dpost;
+  o[12] = lat.spost + lat.dpost / G64;
+  o[13] = pf_post;
+  o[14] = pb_post;
+  // single stage (:3057-3062)
+  o[15] = lat.spp;
+  o[16] = lat.dpp;
+  o[17] = lat.spp + lat.dpp / G64;
+  o[18] = pf_post + g->pre_states + g->pre_saved;
+  o[19] = pb_post + g->pre_states + g->pre_saved;
+}
+
 int check_common(const void *d_problem, const void *d_groups, int n_groups) {
   if (!d_problem || !d_groups) return fail(MIST_E_INVALID, "null problem / group pointer");
   if (n_groups <= 0) return fail(MIST_E_INVALID, "n_groups must be positive, got %d", n_groups);
@@ -1331,6 +1414,18 @@ int mist_intra_stage_eval(const MistProblem *problem, const MistGroupDesc *d_gro
     return rc;
   return mist_finalize(problem, d_groups, n_groups, d_reduce_block_prefix, d_row_terms,
                        d_partial_cost, d_partial_index, sample_index, tables, stream);
+}
+
+int mist_stage_analyze(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,
+                       const double *d_row_terms, const int32_t *d_requests, int n_requests,
+                       double *d_out, void *stream) {
+  if (int rc = check_common(problem, d_groups, n_groups)) return rc;
+  if (!d_row_terms || !d_requests || !d_out) return fail(MIST_E_INVALID, "null pointer");
+  if (n_requests <= 0) return fail(MIST_E_INVALID, "n_requests must be positive, got %d", n_requests);
+  hipLaunchKernelGGL(analyze_kernel, dim3((n_requests + 63) / 64), dim3(64), 0, (hipStream_t)stream,
+                     *problem, d_groups, n_groups, d_row_terms, d_requests, n_requests, d_out);
+  MIST_HIP_CHECK(hipGetLastError());
+  return 0;
 }
 
 }  // extern "C"

@@ -89,10 +89,21 @@ def latency_exec(
     )
 
 
-def pre_post_strategy_fields(config: MistConfig, num_nodes: int, num_gpus_per_node: int):
+def pre_post_strategy_fields(config: MistConfig, num_nodes: int, num_gpus_per_node: int,
+                             analysis_row=None):
     """(dp, tp, wre, gre, ore, wo, go, oo, ac) of the pre / post layers
-    (batched_module_analyzer.py:788-845, tuning path)."""
-    strategy = config.tuning.pre_post_strategy
+    (batched_module_analyzer.py:777-845).  The tuning path reads ``tuning.pre_post_strategy``; the
+    analysis path (``analysis_row`` = the strategy row) reads ``strategy.pre_post_strategy`` and
+    also knows ``tuned`` (the row's own parallelism, :789-799)."""
+    if analysis_row is None:
+        strategy = config.tuning.pre_post_strategy
+    else:
+        if config.strategy is None:
+            raise ValueError("the analysis path needs an enabled strategy block")
+        strategy = config.strategy.pre_post_strategy
+        if strategy == "tuned":
+            r = analysis_row
+            return int(r[1]), int(r[2]), bool(r[3]), bool(r[4]), bool(r[5]), 0.0, 0.0, 0.0, 0.0
     if strategy == "preset":
         if config.strategy is None:
             raise ValueError(
@@ -198,7 +209,7 @@ class GroupInputBuilder:
 
     def fill(
         self, rec: np.void, space: SearchSpace, g_index: int, q_index: int, num_nodes: int,
-        num_gpus_per_node: int, grad_accum: int, num_p: int,
+        num_gpus_per_node: int, grad_accum: int, num_p: int, analysis_row=None,
     ) -> None:
         """Fills one record of a ``GROUP_DTYPE`` array (decomposition fields are set later)."""
         cfg, t = self.config, self.tables
@@ -233,7 +244,7 @@ class GroupInputBuilder:
 
         # ---- pre / post layers ----
         pp_dp, pp_tp, pp_wre, pp_gre, pp_ore, pp_wo, pp_go, pp_oo, _pp_ac = pre_post_strategy_fields(
-            cfg, n, m
+            cfg, n, m, analysis_row
         )
         pp_b = cfg.training.global_batch_size // G // pp_dp
         fb, ftp = np.float64(pp_b), np.float64(pp_tp)

@@ -21,6 +21,8 @@ from .interference import interference_one_group
 from .pareto import sample_pareto_frontier
 from .search_space import create_search_space
 
+BATCH_SIZE_CANDIDATES = (1, 2, 4)  # batched_module_analyzer.py:53 (the module constant, :870)
+
 MEM_INF = 1e12
 GB = 1 << 30
 MB = 1 << 20
@@ -71,9 +73,17 @@ def _arr(x):
     return np.array([x])
 
 
-def pre_post_strategy_fields(config, num_nodes, num_gpus_per_node):
-    """:788-845 (tuning path): (dp, tp, wre, gre, ore, wo, go, oo, ac) of the pre/post layers."""
-    strategy = config.tuning.pre_post_strategy
+def pre_post_strategy_fields(config, num_nodes, num_gpus_per_node, analysis_rows=None):
+    """:777-845: (dp, tp, wre, gre, ore, wo, go, oo, ac) of the pre/post layers.  The tuning path
+    reads ``config.tuning.pre_post_strategy``; the analysis path (``analysis_rows`` = the
+    strategy rows) reads ``config.strategy.pre_post_strategy`` and also knows ``tuned``."""
+    if analysis_rows is None:
+        strategy = config.tuning.pre_post_strategy
+    else:
+        strategy = config.strategy.pre_post_strategy
+        if strategy == "tuned":  # :789-799
+            r = analysis_rows
+            return r[:, 1], r[:, 2], r[:, 3], r[:, 4], r[:, 5], 0.0, 0.0, 0.0, 0.0
     if strategy == "preset":
         # The reference reads ``config.strategy.pre_post_strategy_array`` here (:801-809).
         a = config.strategy.pre_post_strategy_array
@@ -98,8 +108,15 @@ def batched_stage_analyze(
     stage_strategies,
     sample_size,
     debug=None,
+    analysis=None,
 ):
     """:687-3144 with ``get_best_solution=True``.
+
+    ``analysis`` (a list of four dicts) additionally receives what the ``get_best_solution=False``
+    path returns (:2788-2803, 2876-2892, 2980-2996, 3063-3079): per variant and ``(p, l, c)`` the
+    per-row arrays ``latency`` (incl. twice the p2p latency of the layer output, :1298-1308,
+    except for the pre-and-post variant), ``mem_fwd_peak``, ``mem_bwd_peak`` and the stable /
+    delta latency of that variant (the ``****latency_*`` entries, :2550-2567), unmasked.
 
     Returns four tuples ``(costs_stable, costs_delta, solutions, indices)`` for the variants
     base / with_pre / with_post / no_pp; ``indices`` (row index into ``stage_strategies``, -1
@@ -149,9 +166,12 @@ def batched_stage_analyze(
 
     # ------------------------------------------------------------------ pre / post layers (:777-1138)
     (pp_dp, pp_tp, pp_wre, pp_gre, pp_ore, pp_wo, pp_go, pp_oo, pp_ac) = [
-        _arr(v) for v in pre_post_strategy_fields(config, num_nodes, num_gpus_per_node)
+        _arr(v) for v in pre_post_strategy_fields(
+            config, num_nodes, num_gpus_per_node, rows if analysis is not None else None)
     ]
     pp_b = config.training.global_batch_size // G // pp_dp
+    if analysis is not None and pp_b.size == 1 and not 1 <= int(pp_b[0]) <= max(BATCH_SIZE_CANDIDATES):
+        return None  # :868-880: the analysis path returns its (empty) dicts here
 
     def full_states(kind, item, tp):
         return np.atleast_1d(tables.mem_full_states(kind, item, np.asarray(tp, dtype=np.float64)))
@@ -450,6 +470,20 @@ def batched_stage_analyze(
 
     cap = hw.memory_capacity * GB / MB
     ar_n = np.arange(n)[:, None]
+    if analysis is not None:
+        across_nodes = num_gpus_per_node == hw.num_gpus_per_node  # :1299
+        p2p = gpu_gpu("p2p", out, inter_size=1 if across_nodes else None,
+                      intra_size=None if across_nodes else 1) * 2
+
+    def record(variant, p, c, stable_v, delta_v, latency_v, fwd, bwd):
+        for i, l in enumerate(num_layers_candidates):
+            analysis[variant][(p, l, c)] = {
+                "latency": np.broadcast_to(latency_v, stable_v.shape)[i],
+                "mem_fwd_peak": np.broadcast_to(fwd, stable_v.shape)[i],
+                "mem_bwd_peak": np.broadcast_to(bwd, stable_v.shape)[i],
+                "latency_stable": stable_v[i],
+                "latency_delta": np.broadcast_to(delta_v, stable_v.shape)[i],
+            }
 
     def reduce_and_gather(x, y_num, mask):
         """:2813-2824: indices, gathered stable / delta / rows with -1 -> inf."""
@@ -503,6 +537,10 @@ def batched_stage_analyze(
             peak_b = (
                 bwd_states + pipe_saved + ck_delta + bwd_peak + out * p * 2 + out * 2 + gcb
             )
+            if analysis is not None:
+                # :2212-2216: float32 stable + float32 delta / python int stays float32
+                lat32 = stable + delta / G
+                record(0, p, c, stable, delta, lat32 + p2p, peak_f, peak_b)
             mask = np.maximum(peak_f, peak_b) * (mf_pp + 0.01) <= cap
             ind, s_, d_, sol_ = reduce_and_gather(stable, delta, mask)
             costs_stable[p, valid_l, c] = s_[valid_l]
@@ -512,6 +550,8 @@ def batched_stage_analyze(
 
             pf = p * pre_saved + peak_f + pre_states_and_saved
             pb = p * pre_saved + peak_b + pre_states_and_saved
+            if analysis is not None:
+                record(1, p, c, stable_pre, delta_pre, stable_pre + delta_pre / G + p2p, pf, pb)
             mask = np.maximum(pf, pb) * mf_pp <= cap
             ind, s_, d_, sol_ = reduce_and_gather(stable_pre, delta_pre, mask)
             costs_stable_pre[p, valid_l, c] = s_[valid_l]
@@ -531,6 +571,8 @@ def batched_stage_analyze(
                 )
                 pf = np.maximum(f_in, peak_f + post_states)
                 pb = np.maximum(b_in, peak_b - out + post_states) + post_output
+                if analysis is not None:
+                    record(2, p, c, stable_post, delta_post, stable_post + delta_post / G + p2p, pf, pb)
                 mask = np.maximum(pf, pb) * mf_pp <= cap
                 ind, s_, d_, sol_ = reduce_and_gather(stable_post, delta_post, mask)
                 # The reference rebinds the layer mask here (:3021-3023); the narrowed mask
@@ -543,6 +585,8 @@ def batched_stage_analyze(
 
                 pf = pf + pre_states + pre_saved
                 pb = pb + pre_states + pre_saved
+                if analysis is not None:  # no p2p term here (:3071)
+                    record(3, p, c, stable_pp, delta_pp, stable_pp + delta_pp / G, pf, pb)
                 mask = np.maximum(pf, pb) * mf <= cap
                 ind, s_, d_, sol_ = reduce_and_gather(stable_pp, delta_pp, mask)
                 if c != Cmax - 1:  # :3103

@@ -1060,8 +1060,15 @@ __device__ __forceinline__ void reduce_block(
                   std::integral_constant<int, 0>{});
     }
 
-    // ---- sieve B: lowest improvable slot and the memory test there, per-lane survivors ----
+    // ---- sieve B: lowest improvable slot and the memory test there, per-lane survivors.  It
+    // pays when it rejects most rows (the main pass: 96 %); the scout pass starts from empty
+    // minima and most of what reaches it also changes a slot, so there C takes the rows as they
+    // come (C repeats every test of B). ----
     uint64_t keep = 0;
+    if (range.stage_step > 1) {
+      keep = sieve;
+      sieve = 0;
+    }
     while (sieve != 0) {
       const int r = __ffsll((unsigned long long)sieve) - 1;
       sieve &= sieve - 1;

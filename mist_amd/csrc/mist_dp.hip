@@ -21,6 +21,7 @@ using mist::fail;
 
 constexpr int kDpThreads = 64;  // one wavefront per workgroup
 constexpr int kDpWideTeam = 8;  // lanes that share one DP state in small batches
+constexpr int kDpBatch = 4;  // end layers whose reads a lane of the one-lane-per-state kernel overlaps
 
 // ------------------------------------------------------------------------------------------
 // Adapter: float64 (stable, delta) tables -> float32 DP cost tables for every g.
@@ -275,25 +276,46 @@ __global__ __launch_bounds__(kDpThreads) void dp_step_kernel(
       // reachable start layers i + 1 of the remaining stages on d - nm devices
       const int32_t *reach = range_prev + 2 * (d - nm);
       const int i_first = max(k, reach[0] - 1), i_last = min(L - 1, reach[1] - 1);
-      for (int i = i_first + member; i <= i_last; i += kDpTeam) {
-        const float prev = f_prev[(i + 1) * W + (d - nm)];
-        // A state reachable only through an unreachable successor cannot improve: inf + c is
-        // never < best.  Skipping it changes nothing (and most successors are unreachable).
-        if (prev == INFINITY) continue;
+      // The reference walks j = j_begin..j_end with "cost <= t_max and cost + prev < best".
+      // "+ prev" is monotone, so the smallest reachable sum is (smallest admissible cost) + prev,
+      // and the smallest admissible cost is the row's running minimum if that is <= t_max (else
+      // nothing is admissible).  A state reachable only through an unreachable successor cannot
+      // improve: inf + c is never < best; skipping it changes nothing.
+      auto row_min = [&](int i) {
         const RowRef r = row_ref(q, i);
-        // The reference walks j = j_begin..j_end with "cost <= t_max and cost + prev < best".
-        // "+ prev" is monotone, so the smallest reachable sum is (smallest admissible cost) +
-        // prev, and the smallest admissible cost is the row's running minimum if that is
-        // <= t_max (else nothing is admissible).
-        const float rmin = rule == MIST_DP_CKPT_ALL ? table(r.v, false)[r.at + (i - k + 1)]
-                                                    : table(r.v, true)[r.at + j_last(i)];
-        if (!(rmin <= t_max)) continue;
+        return rule == MIST_DP_CKPT_ALL ? table(r.v, false)[r.at + (i - k + 1)]
+                                        : table(r.v, true)[r.at + j_last(i)];
+      };
+      auto consider = [&](int i, float prev, float rmin) {
+        if (prev == INFINITY || !(rmin <= t_max)) return;
         const float target = kBottleneck ? fmaxf(rmin, prev) : rmin + prev;
-        if (!(target < best)) continue;
+        if (!(target < best)) return;
         best = target;
         best_rmin = rmin;
         arg_i = i;
         arg_q = q;
+      };
+      if constexpr (kDpTeam == 1) {
+        // One lane per state: the scan is a chain of L2 reads.  kDpBatch end layers at a time,
+        // first all their successor values, then the row minima of the reachable ones, so that
+        // the reads of a batch are in flight together; the comparisons keep the order.
+        for (int i0 = i_first; i0 <= i_last; i0 += kDpBatch) {
+          float prev[kDpBatch], rmin[kDpBatch];
+#pragma unroll
+          for (int u = 0; u < kDpBatch; ++u)
+            prev[u] = i0 + u <= i_last ? f_prev[(i0 + u + 1) * W + (d - nm)] : INFINITY;
+#pragma unroll
+          for (int u = 0; u < kDpBatch; ++u)
+            rmin[u] = prev[u] == INFINITY ? INFINITY : row_min(i0 + u);
+#pragma unroll
+          for (int u = 0; u < kDpBatch; ++u) consider(i0 + u, prev[u], rmin[u]);
+        }
+      } else {
+        for (int i = i_first + member; i <= i_last; i += kDpTeam) {
+          const float prev = f_prev[(i + 1) * W + (d - nm)];
+          if (prev == INFINITY) continue;
+          consider(i, prev, row_min(i));
+        }
       }
     }
     if constexpr (kDpTeam == 1) finish_winner();

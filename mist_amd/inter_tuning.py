@@ -524,8 +524,13 @@ def _search(runner: _DpRunner, rows: np.ndarray, Gs: List[int], stats: Optional[
         # the min-max partition is admissible at the bottleneck: its total bounds the scan's best
         sum0 = path_sum[idx]
         cost0 = sum0 + (flat_G[idx] - 1).astype(np.float64) * bottleneck[idx].astype(np.float64)
-        hi = np.nextafter((cost0 * (1.0 + 1e-5) / flat_G[idx]).astype(np.float32), np.float32(np.inf))
-        hi = np.maximum(hi, np.nextafter(bottleneck[idx], np.float32(np.inf)))
+        # The scan's bound uses the first KEPT candidate at or above the bottleneck, which the gap
+        # rule can push up by a few gaps: leave room for that, or the window needs a second fetch.
+        room = (flat_G[idx] - 1).astype(np.float64) * (4 * GAP)
+        hi = np.nextafter(((cost0 + room) * (1.0 + 1e-5) / flat_G[idx]).astype(np.float32), np.float32(np.inf))
+        # ... and when the smallest feasible threshold is no candidate itself (a single-stage
+        # cost is none), the first candidate above it lies a little further up
+        hi = np.maximum(hi, (bottleneck[idx].astype(np.float64) * (1.0 + 2e-3) + 2e-4).astype(np.float32))
         for k, i in enumerate(idx):
             windows[i] = _Window(runner, int(flat[i]), int(flat_G[i]), bottleneck[i], float(sum0[k]))
         pending, widen = list(range(len(idx))), 0

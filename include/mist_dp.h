@@ -71,6 +71,19 @@ int mist_dp_cost_tables(const MistProblem *problem, const MistOutTables *tables,
  * candidate t_max values; writes the kept values to out and returns their count. */
 int mist_dp_filter_tmax(const float *sorted_unique, int n, double gap, float *out);
 
+/* Host helper for a walk that does not start at the bottom of the candidate list.  `ascending`
+ * holds the candidates in (lo, hi] of one table row (all candidates up to hi when `open_below`).
+ * Whether the reference's walk keeps a candidate only depends on the last kept one, and a
+ * candidate whose predecessor is at least the gap below it is kept in any case: the walk is
+ * restarted at the last such candidate that is <= start_value (the smallest feasible threshold;
+ * everything below is infeasible and leaves the scan of inter_tuning.py:189-217 unchanged), or at
+ * the first fetched candidate when that lies above start_value and is certain itself.  Writes
+ * the kept values from there on and returns their count, or MIST_DP_NO_START when the fetched
+ * part holds no certain start (the caller fetches from further below). */
+#define MIST_DP_NO_START (-3)
+int mist_dp_window_begin(const float *ascending, int n, float lo, int open_below,
+                         float start_value, double gap, float *out);
+
 /* t_max candidates of value windows (reference: the sort + scan over every finite stage cost,
  * inter_tuning.py:180-199, restricted to where the scan can get).  Request r selects the finite
  * values v of the costs / with_pre / with_post tables of table row d_rows[r] with

@@ -23,6 +23,7 @@ SCOUT_SPLIT = 4  # replaced by the library's own value in load()
 STAGE_ROWS = 64  # replaced by the library's own value in load()
 TERMS_BLOCK = 128  # replaced by the library's own value in load()
 MAX_MESH = 16
+DP_NO_START = -3
 DP_CKPT_TAIL, DP_CKPT_STAGE, DP_CKPT_ALL = 0, 1, 2
 DP_THRESHOLD, DP_BOTTLENECK = 0, 1
 
@@ -178,6 +179,9 @@ _DP_SIGNATURES = {
         [_VP, ctypes.POINTER(OutTables), _VP, ctypes.c_int, ctypes.c_void_p * 4, ctypes.c_void_p * 4, _VP],
     ),
     "mist_dp_filter_tmax": (ctypes.c_int, [_VP, ctypes.c_int, ctypes.c_double, _VP]),
+    "mist_dp_window_begin": (
+        ctypes.c_int,
+        [_VP, ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_float, ctypes.c_double, _VP]),
     "mist_dp_select_candidates": (
         ctypes.c_int,
         [ctypes.POINTER(DpCosts), ctypes.c_int, _VP, _VP, _VP, _VP, _VP, ctypes.c_int, _VP, _VP],

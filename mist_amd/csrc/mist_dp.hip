@@ -438,6 +438,30 @@ int mist_dp_filter_tmax(const float *sorted_unique, int n, double gap, float *ou
   return kept;
 }
 
+int mist_dp_window_begin(const float *ascending, int n, float lo, int open_below,
+                         float start_value, double gap, float *out) {
+  if (n < 0 || (n > 0 && (!ascending || !out))) return fail(MIST_E_INVALID, "bad candidate list");
+  if (n == 0) return 0;
+  // A candidate whose predecessor is at least the gap below it is kept whatever the walk did
+  // before (float32 difference, float64 comparison, as in mist_dp_filter_tmax); the predecessor
+  // of the first fetched candidate is unknown unless the fetch was open below.
+  int first = -1;
+  for (int i = 0; i < n && ascending[i] <= start_value; ++i) {
+    const float prev = i == 0 ? (open_below ? 0.0f : lo) : ascending[i - 1];
+    const float diff = ascending[i] - prev;
+    const bool certain = !((double)diff < gap) || (i == 0 && open_below);
+    if (certain) first = i;
+  }
+  if (first < 0) {
+    const float prev = open_below ? 0.0f : lo;
+    const float diff = ascending[0] - prev;
+    const bool certain0 = !((double)diff < gap) || open_below;
+    if (!(ascending[0] > start_value && certain0)) return MIST_DP_NO_START;
+    first = 0;
+  }
+  return mist_dp_filter_tmax(ascending + first, n - first, gap, out);  // the walk from there
+}
+
 int mist_dp_select_candidates(const MistDpCosts *costs, int n_requests, const int32_t *d_rows,
                               const float *d_lo, const float *d_hi, float *d_out_values,
                               int32_t *d_out_request, int capacity, int32_t *d_counts,

@@ -318,22 +318,22 @@ class _Window:
 
     def begin(self, values: np.ndarray, n_above: int, lo: np.float32, hi: np.float32) -> bool:
         """First fetch: ``values`` = ascending candidates in (lo, hi].  Returns False if no
-        certain start of the walk lies in the fetched part (the caller widens ``lo``)."""
+        certain start of the walk lies in the fetched part (the caller widens ``lo``).  The
+        start is found and the walk done by ``mist_dp_window_begin``."""
         self.hi, self.complete = hi, n_above == 0
         if len(values) == 0:
             return True
-        below = np.isneginf(lo)
-        prev = np.concatenate(([lo if not below else np.float32(0)], values[:-1]))
-        certain = _gap_reached(values, prev)   # kept whatever happened before
-        certain[0] = certain[0] or below        # the walk's true start
-        at_or_below = np.nonzero(certain & (values <= self.start_value))[0]
-        if len(at_or_below):
-            first = int(at_or_below[-1])
-        elif values[0] > self.start_value and certain[0]:
-            first = 0
-        else:
+        below = bool(np.isneginf(lo))
+        values = np.ascontiguousarray(values, dtype=np.float32)
+        kept = np.empty(len(values), dtype=np.float32)
+        n = self.runner.lib.mist_dp_window_begin(
+            ctypes.c_void_p(values.ctypes.data), len(values), 0.0 if below else float(lo),
+            1 if below else 0, float(self.start_value), GAP, ctypes.c_void_p(kept.ctypes.data))
+        if n == _lib.DP_NO_START:
             return False
-        self._append(self.runner.filter_gap(values[first:]))
+        if n < 0:
+            _lib.check(n, "mist_dp_window_begin")
+        self._append(kept[:n])
         return True
 
     def _append(self, kept: np.ndarray) -> None:

@@ -235,6 +235,53 @@ def test_argument_checks_reject_before_any_launch():
     assert lib.mist_dp_run(sp, ctypes.byref(costs), fake, fake, 1, 7, fake, fake, fake, None, fake, None) == -1
 
 
+def test_window_begin_matches_numpy_formulation():
+    """mist_dp_window_begin against the rule written with numpy: a candidate is certain to be
+    kept if its predecessor is at least the gap below; start at the last certain candidate that
+    is <= start_value, else at the first one if it is certain and above start_value."""
+    lib = _lib.load()
+    rng = np.random.default_rng(7)
+    gap = 1e-6
+    outcomes = set()
+    for trial in range(400):
+        n = int(rng.integers(0, 40))
+        base = np.sort(rng.uniform(0.5, 0.5002, n)).astype(np.float32)
+        if n and rng.random() < 0.5:   # clusters closer than the gap
+            base = np.sort(np.concatenate([base, base[: n // 2] + np.float32(3e-7)])).astype(np.float32)
+        values = np.unique(base)
+        below = bool(rng.random() < 0.3)
+        lo = np.float32(-np.inf) if below else np.float32(0.5 - rng.uniform(0, 2e-6))
+        values = values[values > lo] if not below else values
+        if len(values) and not below and rng.random() < 0.4:   # the fetch starts inside a cluster
+            lo = np.float32(values[0] - np.float32(2e-7))
+            values = values[: 1 + int(np.searchsorted(values, values[0] + np.float32(8e-7)))]
+        start = np.float32(rng.uniform(0.4999, 0.5003))
+        kept = np.empty(max(len(values), 1), dtype=np.float32)
+        got = lib.mist_dp_window_begin(
+            values.ctypes.data, len(values), 0.0 if below else float(lo), int(below), float(start), gap,
+            kept.ctypes.data)
+        if len(values) == 0:
+            assert got == 0
+            continue
+        prev = np.concatenate(([np.float32(0) if below else lo], values[:-1])).astype(np.float32)
+        certain = ~((values - prev).astype(np.float64) < gap)
+        certain[0] = certain[0] or below
+        cand = np.nonzero(certain & (values <= start))[0]
+        if len(cand):
+            first = int(cand[-1])
+        elif values[0] > start and certain[0]:
+            first = 0
+        else:
+            assert got == _lib.DP_NO_START
+            outcomes.add("none")
+            continue
+        want = np.empty_like(values)
+        n_want = lib.mist_dp_filter_tmax(values[first:].copy().ctypes.data, len(values) - first, gap, want.ctypes.data)
+        assert got == n_want and np.array_equal(kept[:got], want[:n_want]), trial
+        outcomes.add("mid" if first else "first")
+    assert outcomes == {"none", "mid", "first"}
+
+
 def test_gap_filter_matches_oracle_rule():
     lib = _lib.load()
     rng = np.random.default_rng(0)

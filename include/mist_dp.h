@@ -42,6 +42,13 @@ typedef struct MistDpCosts {
   /* running minima along the ckpt axis, same layouts: pmin[..][j] = min(costs[..][0..j]) */
   const float *pmin, *pmin_pre, *pmin_post, *pmin_nopp;
   int64_t g_stride[4];
+  /* Optional (NULL = absent): the running minima the recurrence reads, re-laid by
+   * mist_dp_stage_minima() as [g][p = stage count - 1][Q][triangle over (k, i >= k)], with
+   * stage_min_g_stride elements between consecutive g.  With it mist_dp_run() may keep a whole
+   * instance in one workgroup's LDS (one launch instead of one per stage count); the results
+   * are the same either way. */
+  const float *stage_min;
+  int64_t stage_min_g_stride;
 } MistDpCosts;
 
 #define MIST_DP_CKPT_TAIL 0
@@ -65,6 +72,15 @@ int mist_sizeof_dp_shape(void);
 int mist_dp_cost_tables(const MistProblem *problem, const MistOutTables *tables,
                         const int32_t *d_grad_accum, int slot, float *const d_out[4],
                         float *const d_out_pmin[4], void *stream);
+
+/* Fills MistDpCosts.stage_min for a DP family: d_out[num_grad_accum][mist_dp_stage_minima_floats()]
+ * (max_stages * Q * L(L+1)/2 floats per g).  Entry (g, p, q, k, i) is the smallest cost over the
+ * ckpt candidates shape->ckpt_rule admits of the stage k..i on mesh q followed by p stages, i.e.
+ * what inter_tuning.py:312-322 compares with t_max first; entries no stage count reaches are
+ * +inf.  `costs` needs its eight table pointers and g_stride only. */
+int64_t mist_dp_stage_minima_floats(const MistDpShape *shape);
+int mist_dp_stage_minima(const MistDpShape *shape, const MistDpCosts *costs, int num_grad_accum,
+                         float *d_out, void *stream);
 
 /* Host helper: applies the reference's gap rule (inter_tuning.py:198: skip t when
  * t - last_run < 1e-6, float32 difference compared in float64) to an ascending list of
@@ -97,8 +113,10 @@ int mist_dp_select_candidates(const MistDpCosts *costs, int n_requests, const in
                               int32_t *d_out_request, int capacity, int32_t *d_counts,
                               void *stream);
 
-/* Runs n_tmax DP instances at once (max_stages launches, one thread per (instance, start
- * layer, devices) state).  Instance t uses the cost tables of g = d_g_index[t].
+/* Runs n_tmax DP instances at once: one launch per stage count with a thread (or a team of
+ * lanes) per (instance, start layer, devices) state, or, for large batches whose state planes fit
+ * the LDS of a compute unit and whose costs->stage_min is set, one workgroup per instance.
+ * Instance t uses the cost tables of g = d_g_index[t].
  * MIST_DP_THRESHOLD (reference: inter_stage_tune_dp_impl, inter_tuning.py:220-355):
  *   F(s,k,d) = min over mesh q (n*m <= d), end layer i >= k, ckpt j (shape->ckpt_rule) of
  *              cost(s,k,i,q,j) + F(s-1,i+1,d-n*m)   subject to cost <= d_tmax[t],

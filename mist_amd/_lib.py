@@ -169,6 +169,8 @@ class DpCosts(ctypes.Structure):
         ("pmin_post", ctypes.c_void_p),
         ("pmin_nopp", ctypes.c_void_p),
         ("g_stride", ctypes.c_int64 * 4),
+        ("stage_min", ctypes.c_void_p),
+        ("stage_min_g_stride", ctypes.c_int64),
     ]
 
 
@@ -187,6 +189,8 @@ _DP_SIGNATURES = {
         [ctypes.POINTER(DpCosts), ctypes.c_int, _VP, _VP, _VP, _VP, _VP, ctypes.c_int, _VP, _VP],
     ),
     "mist_dp_scratch_floats": (ctypes.c_int64, [_VP, ctypes.c_int]),
+    "mist_dp_stage_minima_floats": (ctypes.c_int64, [_VP]),
+    "mist_dp_stage_minima": (ctypes.c_int, [_VP, ctypes.POINTER(DpCosts), ctypes.c_int, _VP, _VP]),
     "mist_dp_run": (
         ctypes.c_int,
         [_VP, ctypes.POINTER(DpCosts), _VP, _VP, ctypes.c_int, ctypes.c_int, _VP, _VP, _VP, _VP, _VP, _VP],

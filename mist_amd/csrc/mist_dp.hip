@@ -1,16 +1,20 @@
 // Inter-stage pipeline-partition DP on MI355X (gfx950).
 //
-// The stage index s is the sequential (wavefront) axis: one launch per s.  The (threshold,
-// start layer k, devices d) states of one s are independent and are spread over the whole GPU,
-// one thread each.  Each thread walks its state's (mesh, end layer, ckpt) candidates in the
-// reference's order with float32 adds and strict "<", so ties resolve exactly as in the
-// reference loop nest (mist/analyzer/inter_tuning.py:298-333).
+// The stage index s is the sequential axis.  The (threshold, start layer k, devices d) states
+// of one s are independent; each is scanned by one thread (or a team of lanes) that walks its
+// (mesh, end layer, ckpt) candidates in the reference's order with float32 adds and strict "<",
+// so ties resolve exactly as in the reference loop nest (mist/analyzer/inter_tuning.py:298-333).
+// Two schedules: one launch per s with the states of all instances spread over the GPU
+// (dp_step_kernel), or one workgroup per instance that keeps its state planes in LDS and loops
+// over s itself (dp_fused_kernel).
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
-
 #include <cmath>
 #include <cstdint>
+#include <map>
+#include <mutex>
+#include <utility>
 
 #include "mist_common.h"
 #include "mist_dp.h"
@@ -21,6 +25,9 @@ using mist::fail;
 
 constexpr int kDpThreads = 64;  // one wavefront per workgroup
 constexpr int kDpWideTeam = 8;  // lanes that share one DP state in small batches
+constexpr size_t kDpLdsPerCu = 160 * 1024;  // LDS of a gfx950 compute unit
+constexpr int kDpFusedThreads = 1024;  // largest workgroup of the one-launch kernel
+constexpr int kDpStageBatch = 8;   // row minima a lane copies together in the one-launch kernel
 constexpr int kDpBatch = 4;  // end layers whose reads a lane of the one-lane-per-state kernel overlaps
 
 // ------------------------------------------------------------------------------------------
@@ -166,6 +173,150 @@ __global__ __launch_bounds__(256) void dp_init_kernel(const MistDpShape shape, i
   }
 }
 
+// Where the ckpt row of (variant, mesh q, pre-saved micro-batches p, layers k..i) starts and which
+// table holds it.
+struct DpRowRef {
+  int v;
+  int64_t at;
+};
+__device__ __forceinline__ DpRowRef dp_row_ref(const MistDpShape &shape, const int64_t (&off)[4],
+                                               int p, int k, int q, int i) {
+  const int L = shape.num_layers, P1 = shape.p_dim, C = L + 1;
+  const int l = i - k + 1;
+  DpRowRef r;
+  if (k == 0 && i == L - 1) { r.v = 3; r.at = (int64_t)q * C; }
+  else if (k == 0) { r.v = 1; r.at = (((int64_t)q * P1 + p) * L + (l - 1)) * C; }
+  else if (i == L - 1) { r.v = 2; r.at = ((int64_t)q * L + (l - 1)) * C; }
+  else { r.v = 0; r.at = (((int64_t)q * P1 + p) * L + (l - 1)) * C; }
+  r.at += off[r.v];
+  return r;
+}
+__device__ __forceinline__ const float *dp_table(const MistDpCosts &tabs, int v, bool running_min) {
+  if (running_min)
+    return v == 0 ? tabs.pmin : v == 1 ? tabs.pmin_pre : v == 2 ? tabs.pmin_post : tabs.pmin_nopp;
+  return v == 0 ? tabs.costs : v == 1 ? tabs.costs_pre : v == 2 ? tabs.costs_post : tabs.costs_nopp;
+}
+// ckpt candidates j_begin..j_end of a stage k..i: 0..L-i (inter_tuning.py:315), or 0..l / only l
+// (inter_tuning_uniform_device.py:400-404)
+__device__ __forceinline__ int dp_j_last(const MistDpShape &shape, int k, int i) {
+  return shape.ckpt_rule == MIST_DP_CKPT_TAIL ? shape.num_layers - i : i - k + 1;
+}
+// The reference walks j = j_begin..j_end with "cost <= t_max and cost + prev < best".  "+ prev" is
+// monotone, so the smallest reachable sum is (smallest admissible cost) + prev, and the smallest
+// admissible cost is the row's running minimum if that is <= t_max (else nothing is admissible).
+__device__ __forceinline__ float dp_row_min(const MistDpShape &shape, const MistDpCosts &tabs,
+                                            const int64_t (&off)[4], int p, int k, int q, int i) {
+  const DpRowRef r = dp_row_ref(shape, off, p, k, q, i);
+  return shape.ckpt_rule == MIST_DP_CKPT_ALL ? dp_table(tabs, r.v, false)[r.at + (i - k + 1)]
+                                             : dp_table(tabs, r.v, true)[r.at + dp_j_last(shape, k, i)];
+}
+
+// Re-laid row minima (mist_dp_stage_minima): per (g, p, mesh) a triangle over (k, i >= k), row k
+// at dp_triangle_row(L, k), entry i - k.
+__device__ __host__ __forceinline__ int dp_triangle(int L) { return L * (L + 1) / 2; }
+__device__ __host__ __forceinline__ int dp_triangle_row(int L, int k) {
+  return k * L - k * (k - 1) / 2;
+}
+
+// Running winner of one state's scan.  The reference visits (q, i) in ascending order and
+// replaces on a strict "<".  A state reachable only through an unreachable successor cannot
+// improve (inf + c is never < best); skipping it changes nothing.
+struct DpBest {
+  float best = INFINITY, best_m = 0.0f, best_rmin = 0.0f;
+  int arg_i = -1, arg_q = -1, arg_j = -1;
+};
+template <bool kBottleneck>
+__device__ __forceinline__ void dp_consider(DpBest &w, float t_max, int q, int i, float prev,
+                                            float rmin) {
+  if (prev == INFINITY || !(rmin <= t_max)) return;
+  const float target = kBottleneck ? fmaxf(rmin, prev) : rmin + prev;
+  if (!(target < w.best)) return;
+  w.best = target;
+  w.best_rmin = rmin;
+  w.arg_i = i;
+  w.arg_q = q;
+}
+
+// The winner's ckpt count and stage maximum: the first j attaining the sum is the entry the
+// reference's strict "<" keeps.  Only the final winner matters, so the row is walked once.
+template <bool kBottleneck>
+__device__ __forceinline__ void dp_finish_winner(DpBest &w, const MistDpShape &shape,
+                                                 const MistDpCosts &tabs, const int64_t (&off)[4],
+                                                 float t_max, int p, int k, int d,
+                                                 const float *f_prev, const float *m_prev) {
+  if (w.arg_i < 0) return;
+  const int W = shape.num_devices + 1;
+  const int nm = shape.free_devices != 0 ? 0 : shape.mesh_n[w.arg_q] * shape.mesh_m[w.arg_q];
+  const int from = (w.arg_i + 1) * W + (d - nm);
+  if (kBottleneck) {
+    // the maxima plane carries the SUM of the stage costs along the min-max path: a partition
+    // that is admissible at the returned threshold, with its float32 sum accumulated in the
+    // threshold DP's order
+    w.best_m = w.best_rmin + m_prev[from];
+    return;
+  }
+  const DpRowRef r = dp_row_ref(shape, off, p, k, w.arg_q, w.arg_i);
+  const float *__restrict__ row = dp_table(tabs, r.v, false) + r.at;
+  const float prev = f_prev[from];
+  const int j_begin = shape.ckpt_rule == MIST_DP_CKPT_ALL ? w.arg_i - k + 1 : 0;
+  const int j_end = dp_j_last(shape, k, w.arg_i);
+  // kDpBatch entries are read together and tested in order
+  for (int j0 = j_begin; j0 <= j_end; j0 += kDpBatch) {
+    float stage_cost[kDpBatch];
+#pragma unroll
+    for (int u = 0; u < kDpBatch; ++u) stage_cost[u] = j0 + u <= j_end ? row[j0 + u] : INFINITY;
+#pragma unroll
+    for (int u = 0; u < kDpBatch; ++u) {
+      if (j0 + u <= j_end && stage_cost[u] <= t_max && stage_cost[u] + prev == w.best) {
+        w.arg_j = j0 + u;
+        w.best_m = fmaxf(m_prev[from], stage_cost[u]);
+        return;
+      }
+    }
+  }
+}
+
+// Scan of one state (start layer k, devices d) by one lane (member 0 of 1) or by its share of a
+// team: meshes q and end layers i in the reachable range of the successor column.
+// `row_min(q, i)` returns dp_row_min of the stage k..i on mesh q.
+template <bool kBottleneck, int kDpTeam, typename RowMin>
+__device__ __forceinline__ void dp_scan_state(DpBest &w, const MistDpShape &shape, float t_max,
+                                              int k, int d, int member, const float *f_prev,
+                                              const int32_t *range_prev, RowMin row_min) {
+  const int L = shape.num_layers, W = shape.num_devices + 1;
+  const bool free_devices = shape.free_devices != 0;
+  for (int q = 0; q < shape.num_mesh; ++q) {
+    const int nm = free_devices ? 0 : shape.mesh_n[q] * shape.mesh_m[q];
+    if (nm > d) continue;
+    // reachable start layers i + 1 of the remaining stages on d - nm devices
+    const int32_t *reach = range_prev + 2 * (d - nm);
+    const int i_first = max(k, reach[0] - 1), i_last = min(L - 1, reach[1] - 1);
+    if constexpr (kDpTeam == 1) {
+      // One lane per state: the scan is a chain of reads.  kDpBatch end layers at a time, first
+      // all their successor values, then the row minima of the reachable ones, so that the reads
+      // of a batch are in flight together; the comparisons keep the order.
+      for (int i0 = i_first; i0 <= i_last; i0 += kDpBatch) {
+        float prev[kDpBatch], rmin[kDpBatch];
+#pragma unroll
+        for (int u = 0; u < kDpBatch; ++u)
+          prev[u] = i0 + u <= i_last ? f_prev[(i0 + u + 1) * W + (d - nm)] : INFINITY;
+#pragma unroll
+        for (int u = 0; u < kDpBatch; ++u)
+          rmin[u] = prev[u] == INFINITY ? INFINITY : row_min(q, i0 + u);
+#pragma unroll
+        for (int u = 0; u < kDpBatch; ++u)
+          dp_consider<kBottleneck>(w, t_max, q, i0 + u, prev[u], rmin[u]);
+      }
+    } else {
+      for (int i = i_first + member; i <= i_last; i += kDpTeam) {
+        const float prev = f_prev[(i + 1) * W + (d - nm)];
+        if (prev == INFINITY) continue;
+        dp_consider<kBottleneck>(w, t_max, q, i, prev, row_min(q, i));
+      }
+    }
+  }
+}
+
 template <bool kBottleneck, int kDpTeam>
 __global__ __launch_bounds__(kDpThreads) void dp_step_kernel(
     const MistDpShape shape, const MistDpCosts tabs, const float *__restrict__ tmax_list,
@@ -173,11 +324,9 @@ __global__ __launch_bounds__(kDpThreads) void dp_step_kernel(
     int32_t *__restrict__ ranges, int32_t *__restrict__ best_s_out,
     float *__restrict__ best_sum_out, float *__restrict__ stage_max_out,
     int32_t *__restrict__ argmin) {
-  const int L = shape.num_layers, D = shape.num_devices, Q = shape.num_mesh;
-  const int P1 = shape.p_dim;
+  const int L = shape.num_layers, D = shape.num_devices;
   const int W = D + 1;            // row pitch of a state plane
   const int plane = (L + 1) * W;  // states per s
-  const int C = L + 1;            // ckpt extent of the cost tables
   // kDpTeam consecutive lanes share one state and split its end layers between them.  The scan
   // of a state is a chain of dependent L2 reads: in a small batch its latency, not the
   // arithmetic, sets the time of a launch (team of 8); a batch that fills the GPU anyway runs
@@ -210,141 +359,47 @@ __global__ __launch_bounds__(kDpThreads) void dp_step_kernel(
   int32_t *range_cur = ranges + (s % 3) * range_stride + (int64_t)t * W * 2;
   int32_t *range_next = ranges + ((s + 1) % 3) * range_stride + (int64_t)t * W * 2;
 
-  const bool free_devices = shape.free_devices != 0;
-  const int rule = shape.ckpt_rule;
-
-  float best = INFINITY, best_m = 0.0f, best_rmin = 0.0f;
-  int arg_i = -1, arg_q = -1, arg_j = -1;
-
-  // Where the ckpt row of (variant, mesh q, p, layers k..i) starts and which table holds it.
-  struct RowRef {
-    int v;
-    int64_t at;
-  };
-  auto row_ref = [&](int q, int i) {
-    const int l = i - k + 1;
-    RowRef r;
-    if (k == 0 && i == L - 1) { r.v = 3; r.at = (int64_t)q * C; }
-    else if (k == 0) { r.v = 1; r.at = (((int64_t)q * P1 + p) * L + (l - 1)) * C; }
-    else if (i == L - 1) { r.v = 2; r.at = ((int64_t)q * L + (l - 1)) * C; }
-    else { r.v = 0; r.at = (((int64_t)q * P1 + p) * L + (l - 1)) * C; }
-    r.at += off[r.v];
-    return r;
-  };
-  auto table = [&](int v, bool running_min) -> const float *__restrict__ {
-    if (running_min)
-      return v == 0 ? tabs.pmin : v == 1 ? tabs.pmin_pre : v == 2 ? tabs.pmin_post : tabs.pmin_nopp;
-    return v == 0 ? tabs.costs : v == 1 ? tabs.costs_pre : v == 2 ? tabs.costs_post : tabs.costs_nopp;
-  };
-  // ckpt candidates j_begin..j_end of a stage k..i: 0..L-i (inter_tuning.py:315), or 0..l / only l
-  // (inter_tuning_uniform_device.py:400-404)
-  auto j_last = [&](int i) { return rule == MIST_DP_CKPT_TAIL ? L - i : i - k + 1; };
-
-  // The winner's ckpt count and stage maximum: the first j attaining the sum is the entry the
-  // reference's strict "<" keeps.  Only the final winner matters, so the row is walked once.
-  auto finish_winner = [&]() {
-    if (arg_i >= 0) {
-      const int nm = free_devices ? 0 : shape.mesh_n[arg_q] * shape.mesh_m[arg_q];
-      const int from = (arg_i + 1) * W + (d - nm);
-      if (kBottleneck) {
-        // the maxima plane carries the SUM of the stage costs along the min-max path: a
-        // partition that is admissible at the returned threshold, with its float32 sum
-        // accumulated in the threshold DP's order
-        best_m = best_rmin + m_prev[from];
-      } else {
-        const RowRef r = row_ref(arg_q, arg_i);
-        const float *__restrict__ row = table(r.v, false) + r.at;
-        const float prev = f_prev[from];
-        const int j_begin = rule == MIST_DP_CKPT_ALL ? arg_i - k + 1 : 0;
-        for (int j = j_begin; j <= j_last(arg_i); ++j) {
-          const float stage_cost = row[j];
-          if (stage_cost <= t_max && stage_cost + prev == best) {
-            arg_j = j;
-            best_m = fmaxf(m_prev[from], stage_cost);
-            break;
-          }
-        }
-      }
-    }
-  };
-
-  const bool live = k <= L - s && (d >= 1 || free_devices);
+  // the row minima of this stage count in (mesh, k, i) order, if the caller prepared them
+  const int tri = dp_triangle(L);
+  const float *__restrict__ relaid =
+      tabs.stage_min == nullptr
+          ? nullptr
+          : tabs.stage_min + g * tabs.stage_min_g_stride + (int64_t)p * shape.num_mesh * tri +
+                dp_triangle_row(L, k) - k;
+  DpBest w;
+  const bool live = k <= L - s && (d >= 1 || shape.free_devices != 0);
   if (live) {
-    for (int q = 0; q < Q; ++q) {
-      const int nm = free_devices ? 0 : shape.mesh_n[q] * shape.mesh_m[q];
-      if (nm > d) continue;
-      // reachable start layers i + 1 of the remaining stages on d - nm devices
-      const int32_t *reach = range_prev + 2 * (d - nm);
-      const int i_first = max(k, reach[0] - 1), i_last = min(L - 1, reach[1] - 1);
-      // The reference walks j = j_begin..j_end with "cost <= t_max and cost + prev < best".
-      // "+ prev" is monotone, so the smallest reachable sum is (smallest admissible cost) + prev,
-      // and the smallest admissible cost is the row's running minimum if that is <= t_max (else
-      // nothing is admissible).  A state reachable only through an unreachable successor cannot
-      // improve: inf + c is never < best; skipping it changes nothing.
-      auto row_min = [&](int i) {
-        const RowRef r = row_ref(q, i);
-        return rule == MIST_DP_CKPT_ALL ? table(r.v, false)[r.at + (i - k + 1)]
-                                        : table(r.v, true)[r.at + j_last(i)];
-      };
-      auto consider = [&](int i, float prev, float rmin) {
-        if (prev == INFINITY || !(rmin <= t_max)) return;
-        const float target = kBottleneck ? fmaxf(rmin, prev) : rmin + prev;
-        if (!(target < best)) return;
-        best = target;
-        best_rmin = rmin;
-        arg_i = i;
-        arg_q = q;
-      };
-      if constexpr (kDpTeam == 1) {
-        // One lane per state: the scan is a chain of L2 reads.  kDpBatch end layers at a time,
-        // first all their successor values, then the row minima of the reachable ones, so that
-        // the reads of a batch are in flight together; the comparisons keep the order.
-        for (int i0 = i_first; i0 <= i_last; i0 += kDpBatch) {
-          float prev[kDpBatch], rmin[kDpBatch];
-#pragma unroll
-          for (int u = 0; u < kDpBatch; ++u)
-            prev[u] = i0 + u <= i_last ? f_prev[(i0 + u + 1) * W + (d - nm)] : INFINITY;
-#pragma unroll
-          for (int u = 0; u < kDpBatch; ++u)
-            rmin[u] = prev[u] == INFINITY ? INFINITY : row_min(i0 + u);
-#pragma unroll
-          for (int u = 0; u < kDpBatch; ++u) consider(i0 + u, prev[u], rmin[u]);
-        }
-      } else {
-        for (int i = i_first + member; i <= i_last; i += kDpTeam) {
-          const float prev = f_prev[(i + 1) * W + (d - nm)];
-          if (prev == INFINITY) continue;
-          consider(i, prev, row_min(i));
-        }
-      }
-    }
-    if constexpr (kDpTeam == 1) finish_winner();
+    dp_scan_state<kBottleneck, kDpTeam>(
+        w, shape, t_max, k, d, member, f_prev, range_prev,
+        [&](int q, int i) {
+          return relaid != nullptr ? relaid[q * tri + i] : dp_row_min(shape, tabs, off, p, k, q, i);
+        });
+    if constexpr (kDpTeam == 1)
+      dp_finish_winner<kBottleneck>(w, shape, tabs, off, t_max, p, k, d, f_prev, m_prev);
   }
-  // Team reduction.  The reference visits (q, i) in ascending order and replaces on a strict "<":
-  // the winner is the first candidate that attains the minimum, i.e. the lexicographic minimum
-  // of (target, q, i).  Each lane holds that minimum over its own candidates.
+  // Team reduction: the winner is the first candidate that attains the minimum, i.e. the
+  // lexicographic minimum of (target, q, i).  Each lane holds that minimum over its own
+  // candidates.
   if constexpr (kDpTeam > 1) {
-    int order = arg_i >= 0 ? arg_q * L + arg_i : 0x7fffffff;
+    int order = w.arg_i >= 0 ? w.arg_q * L + w.arg_i : 0x7fffffff;
 #pragma unroll
     for (int step = 1; step < kDpTeam; step <<= 1) {
-      const float o_best = __shfl_xor(best, step);
-      const float o_rmin = __shfl_xor(best_rmin, step);
+      const float o_best = __shfl_xor(w.best, step);
+      const float o_rmin = __shfl_xor(w.best_rmin, step);
       const int o_order = __shfl_xor(order, step);
-      const bool take = o_best < best || (o_best == best && o_order < order);
-      best = take ? o_best : best;
-      best_rmin = take ? o_rmin : best_rmin;
+      const bool take = o_best < w.best || (o_best == w.best && o_order < order);
+      w.best = take ? o_best : w.best;
+      w.best_rmin = take ? o_rmin : w.best_rmin;
       order = take ? o_order : order;
     }
-    arg_q = order == 0x7fffffff ? -1 : order / L;
-    arg_i = order == 0x7fffffff ? -1 : order % L;
-  }
-  if constexpr (kDpTeam > 1) {
+    w.arg_q = order == 0x7fffffff ? -1 : order / L;
+    w.arg_i = order == 0x7fffffff ? -1 : order % L;
     if (!real || member != 0) return;
-    if (live) finish_winner();
+    if (live) dp_finish_winner<kBottleneck>(w, shape, tabs, off, t_max, p, k, d, f_prev, m_prev);
   }
-  f_cur[e] = best;
-  m_cur[e] = best_m;
-  if (best < INFINITY) {
+  f_cur[e] = w.best;
+  m_cur[e] = w.best_m;
+  if (w.best < INFINITY) {
     atomicMin(&range_cur[2 * d], k);
     atomicMax(&range_cur[2 * d + 1], k);
   }
@@ -352,20 +407,192 @@ __global__ __launch_bounds__(kDpThreads) void dp_step_kernel(
     range_next[2 * d] = L + 1;
     range_next[2 * d + 1] = -1;
   }
-  if (argmin != nullptr && arg_i >= 0) {
+  if (argmin != nullptr && w.arg_i >= 0) {
     int32_t *a = argmin + (((int64_t)t * (shape.max_stages + 1) + s) * plane + e) * 4;
-    a[0] = arg_i;
-    a[1] = shape.mesh_n[arg_q];
-    a[2] = shape.mesh_m[arg_q];
-    a[3] = arg_j;
+    a[0] = w.arg_i;
+    a[1] = shape.mesh_n[w.arg_q];
+    a[2] = shape.mesh_m[w.arg_q];
+    a[3] = w.arg_j;
   }
   // The state (k = 0, d = D) is the answer of this stage count; first s wins ties
   // (inter_tuning.py:335-340).  The same thread handles it in every launch.
-  if (k == 0 && d == D && best < best_sum_out[t]) {
-    best_sum_out[t] = best;
+  if (k == 0 && d == D && w.best < best_sum_out[t]) {
+    best_sum_out[t] = w.best;
     best_s_out[t] = s;
-    stage_max_out[t] = best_m;
+    stage_max_out[t] = w.best_m;
   }
+}
+
+// ------------------------------------------------------------------------------------------
+// The same recurrence with the whole instance in one workgroup: the four state planes and the
+// reachable ranges live in LDS, the stage counts are a loop with a barrier between them, and one
+// launch replaces init + max_stages step launches.  Used whenever the planes fit (16 bytes per
+// state); the arithmetic per state is the code above.
+// ------------------------------------------------------------------------------------------
+template <bool kBottleneck>
+__global__ __launch_bounds__(kDpFusedThreads) void dp_fused_kernel(
+    const MistDpShape shape, const MistDpCosts tabs, const float *__restrict__ tmax_list,
+    const int32_t *__restrict__ g_list, int32_t *__restrict__ best_s_out,
+    float *__restrict__ best_sum_out, float *__restrict__ stage_max_out,
+    int32_t *__restrict__ argmin) {
+  extern __shared__ float dp_lds[];
+  const int L = shape.num_layers, D = shape.num_devices;
+  const int W = D + 1, plane = (L + 1) * W;
+  float *f_plane = dp_lds;              // [2][plane]
+  float *m_plane = dp_lds + 2 * plane;  // [2][plane]
+  int32_t *range = reinterpret_cast<int32_t *>(dp_lds + 4 * plane);  // [3][W][2]
+  // row minima of the current stage count: per mesh a triangle (k, i >= k)
+  float *stage_min = dp_lds + 4 * plane + 6 * W;
+  const int tri = dp_triangle(L), n_stage = shape.num_mesh * tri;
+  const int t = blockIdx.x;
+  const float t_max = kBottleneck ? INFINITY : tmax_list[t];
+  const int64_t g = g_list[t];
+  const int64_t off[4] = {g * tabs.g_stride[0], g * tabs.g_stride[1], g * tabs.g_stride[2],
+                          g * tabs.g_stride[3]};
+  const float *__restrict__ relaid = tabs.stage_min + g * tabs.stage_min_g_stride;
+  // F(0, ., .): 0 at (k = L, d = 0), +inf elsewhere; maxima start at 0; only that state is
+  // reachable.
+  for (int e = threadIdx.x; e < plane; e += blockDim.x) {
+    f_plane[e] = e == L * W ? 0.0f : INFINITY;
+    m_plane[e] = 0.0f;
+  }
+  for (int col = threadIdx.x; col < W; col += blockDim.x) {
+    range[2 * col] = col == 0 ? L : L + 1;
+    range[2 * col + 1] = col == 0 ? L : -1;
+    for (int b = 1; b < 3; ++b) {
+      range[(b * W + col) * 2] = L + 1;
+      range[(b * W + col) * 2 + 1] = -1;
+    }
+  }
+  // a thread's states are blockDim.x apart: (k, d) advance by fixed steps
+  const int k_first = threadIdx.x / W, d_first = threadIdx.x % W;
+  const int k_step = blockDim.x / W, d_step = blockDim.x % W;
+  // the answer state (k = 0, d = D) belongs to the same thread in every step
+  float answer_sum = INFINITY, answer_max = 0.0f;
+  int answer_s = -1;
+  __syncthreads();
+  for (int s = 1; s <= shape.max_stages; ++s) {
+    const int cur = s & 1, prv = cur ^ 1, p = s - 1;
+    const float *f_prev = f_plane + prv * plane, *m_prev = m_plane + prv * plane;
+    float *f_cur = f_plane + cur * plane, *m_cur = m_plane + cur * plane;
+    const int32_t *range_prev = range + ((s + 2) % 3) * W * 2;
+    int32_t *range_cur = range + (s % 3) * W * 2;
+    int32_t *range_next = range + ((s + 1) % 3) * W * 2;
+    // Every state with start layer k reads the same row minima: copy the block of this stage
+    // count (contiguous in the re-laid table) once per workgroup, kDpStageBatch loads per lane
+    // in flight, so that the scans below touch LDS only.  (The previous step's scans ended at
+    // the barrier that closed it.)
+    const float *__restrict__ block = relaid + (int64_t)p * n_stage;
+    for (int x0 = threadIdx.x; x0 < n_stage; x0 += kDpStageBatch * blockDim.x) {
+      float value[kDpStageBatch];
+#pragma unroll
+      for (int u = 0; u < kDpStageBatch; ++u) {
+        const int x = x0 + u * blockDim.x;
+        if (x < n_stage) value[u] = block[x];
+      }
+#pragma unroll
+      for (int u = 0; u < kDpStageBatch; ++u) {
+        const int x = x0 + u * blockDim.x;
+        if (x < n_stage) stage_min[x] = value[u];
+      }
+    }
+    __syncthreads();
+    int k = k_first, d = d_first;
+    for (int e = threadIdx.x; e < plane; e += blockDim.x) {
+      DpBest w;
+      if (k <= L - s && (d >= 1 || shape.free_devices != 0)) {
+        const float *mine = stage_min + dp_triangle_row(L, k) - k;
+        dp_scan_state<kBottleneck, 1>(w, shape, t_max, k, d, 0, f_prev, range_prev,
+                                      [&](int q, int i) { return mine[q * tri + i]; });
+        dp_finish_winner<kBottleneck>(w, shape, tabs, off, t_max, p, k, d, f_prev, m_prev);
+      }
+      f_cur[e] = w.best;
+      m_cur[e] = w.best_m;
+      if (w.best < INFINITY) {
+        atomicMin(&range_cur[2 * d], k);
+        atomicMax(&range_cur[2 * d + 1], k);
+      }
+      if (k == 0) {
+        range_next[2 * d] = L + 1;
+        range_next[2 * d + 1] = -1;
+      }
+      if (argmin != nullptr && w.arg_i >= 0) {
+        int32_t *a = argmin + (((int64_t)t * (shape.max_stages + 1) + s) * plane + e) * 4;
+        a[0] = w.arg_i;
+        a[1] = shape.mesh_n[w.arg_q];
+        a[2] = shape.mesh_m[w.arg_q];
+        a[3] = w.arg_j;
+      }
+      if (e == D && w.best < answer_sum) {  // first s wins ties (inter_tuning.py:335-340)
+        answer_sum = w.best;
+        answer_s = s;
+        answer_max = w.best_m;
+      }
+      k += k_step;  // state e + blockDim.x
+      d += d_step;
+      if (d >= W) {
+        d -= W;
+        ++k;
+      }
+    }
+    __syncthreads();
+  }
+  if ((int)threadIdx.x == D % (int)blockDim.x) {
+    best_s_out[t] = answer_s;
+    best_sum_out[t] = answer_sum;
+    stage_max_out[t] = answer_max;
+  }
+}
+
+// Row minima in the order the recurrence reads them: out[g][p][q][triangle(k, i)] =
+// dp_row_min(p, k, q, i).  A workgroup scanning stage count p + 1 of g finds all it needs in one
+// contiguous block, and the end layers i of one (q, k) lie next to each other.
+__global__ __launch_bounds__(256) void stage_minima_kernel(const MistDpShape shape,
+                                                           const MistDpCosts tabs,
+                                                           float *__restrict__ out) {
+  const int L = shape.num_layers, tri = dp_triangle(L);
+  const int x = blockIdx.x * 256 + threadIdx.x;
+  if (x >= L * L) return;
+  const int k = x / L, di = x % L;
+  if (k + di >= L) return;
+  const int p = blockIdx.y / shape.num_mesh, q = blockIdx.y % shape.num_mesh;
+  const int64_t g = blockIdx.z;
+  const int64_t off[4] = {g * tabs.g_stride[0], g * tabs.g_stride[1], g * tabs.g_stride[2],
+                          g * tabs.g_stride[3]};
+  // a stage count of p + 1 leaves start layers k <= L - 1 - p
+  const float value = k <= L - 1 - p ? dp_row_min(shape, tabs, off, p, k, q, k + di) : INFINITY;
+  out[((g * shape.max_stages + p) * shape.num_mesh + q) * tri + dp_triangle_row(L, k) + di] = value;
+}
+
+// Dynamic LDS the one-launch kernel may use on the current device: what the device reports per
+// workgroup, once the kernel has been allowed more than the default 64 KB (0 if that failed).
+template <bool kBottleneck>
+size_t fused_lds_limit_of() {
+  int device = 0, most = 0;
+  if (hipGetDevice(&device) != hipSuccess ||
+      hipDeviceGetAttribute(&most, hipDeviceAttributeMaxSharedMemoryPerBlock, device) != hipSuccess)
+    return 0;
+  if (most > 64 * 1024 &&
+      hipFuncSetAttribute(reinterpret_cast<const void *>(&dp_fused_kernel<kBottleneck>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, most) != hipSuccess) {
+    (void)hipGetLastError();
+    most = 64 * 1024;
+  }
+  return (size_t)most;
+}
+size_t fused_lds_limit(int mode) {
+  // per device: the attribute belongs to the device's copy of the kernel
+  static std::mutex lock;
+  static std::map<std::pair<int, int>, size_t> known;
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) return 0;
+  std::lock_guard<std::mutex> guard(lock);
+  const auto key = std::make_pair(device, mode);
+  auto it = known.find(key);
+  if (it == known.end())
+    it = known.emplace(key, mode == MIST_DP_BOTTLENECK ? fused_lds_limit_of<true>()
+                                                       : fused_lds_limit_of<false>()).first;
+  return it->second;
 }
 
 int check_shape(const MistDpShape *shape) {
@@ -421,6 +648,30 @@ int mist_dp_cost_tables(const MistProblem *problem, const MistOutTables *tables,
                        rows_per_g[v], (int)(L + 1), (int)S, slot, d_out[v], d_out_pmin[v]);
     MIST_HIP_CHECK(hipGetLastError());
   }
+  return 0;
+}
+
+int64_t mist_dp_stage_minima_floats(const MistDpShape *shape) {
+  if (check_shape(shape) != 0) return -1;
+  return (int64_t)shape->max_stages * shape->num_mesh * dp_triangle(shape->num_layers);
+}
+
+int mist_dp_stage_minima(const MistDpShape *shape, const MistDpCosts *costs, int num_grad_accum,
+                         float *d_out, void *stream) {
+  if (int rc = check_shape(shape)) return rc;
+  if (!costs || !costs->costs || !costs->costs_pre || !costs->costs_post || !costs->costs_nopp ||
+      !costs->pmin || !costs->pmin_pre || !costs->pmin_post || !costs->pmin_nopp)
+    return fail(MIST_E_INVALID, "null cost table");
+  if (!d_out) return fail(MIST_E_INVALID, "null output pointer");
+  if (num_grad_accum < 1 || num_grad_accum > 65535)
+    return fail(MIST_E_INVALID, "num_grad_accum must be in [1, 65535], got %d", num_grad_accum);
+  const int L = shape->num_layers;
+  hipLaunchKernelGGL(stage_minima_kernel,
+                     dim3((unsigned)((L * L + 255) / 256),
+                          (unsigned)(shape->max_stages * shape->num_mesh),
+                          (unsigned)num_grad_accum),
+                     dim3(256), 0, (hipStream_t)stream, *shape, *costs, d_out);
+  MIST_HIP_CHECK(hipGetLastError());
   return 0;
 }
 
@@ -505,14 +756,35 @@ int mist_dp_run(const MistDpShape *shape, const MistDpCosts *costs, const float 
   if (mode != MIST_DP_THRESHOLD && mode != MIST_DP_BOTTLENECK)
     return fail(MIST_E_INVALID, "unknown DP mode %d", mode);
   const int plane = (shape->num_layers + 1) * (shape->num_devices + 1);
+  // Small batches are latency-bound: spread every state over a team of lanes.
+  const bool wide = (int64_t)n_tmax * plane <= (1 << 19);
+  // Larger ones: one workgroup per instance with its planes in LDS when they fit and the caller
+  // prepared the re-laid row minima.
+  const size_t fused_lds =
+      ((size_t)4 * plane + (size_t)6 * (shape->num_devices + 1) +
+       (size_t)shape->num_mesh * dp_triangle(shape->num_layers)) *
+      sizeof(float);
+  if (!wide && costs->stage_min != nullptr && fused_lds <= fused_lds_limit(mode)) {
+    // one workgroup per CU when the planes take more than half of the LDS: then a larger one
+    const int most = 2 * fused_lds > kDpLdsPerCu ? kDpFusedThreads : kDpFusedThreads / 2;
+    const int threads = std::min(most, (plane + 63) / 64 * 64);
+    if (mode == MIST_DP_BOTTLENECK)
+      hipLaunchKernelGGL(dp_fused_kernel<true>, dim3(n_tmax), dim3(threads), fused_lds,
+                         (hipStream_t)stream, *shape, *costs, d_tmax, d_g_index, d_best_s,
+                         d_best_sum, d_stage_max, d_argmin);
+    else
+      hipLaunchKernelGGL(dp_fused_kernel<false>, dim3(n_tmax), dim3(threads), fused_lds,
+                         (hipStream_t)stream, *shape, *costs, d_tmax, d_g_index, d_best_s,
+                         d_best_sum, d_stage_max, d_argmin);
+    MIST_HIP_CHECK(hipGetLastError());
+    return 0;
+  }
   const int64_t n_init = (int64_t)n_tmax * plane;
   int32_t *d_ranges = reinterpret_cast<int32_t *>(d_scratch + (int64_t)4 * n_tmax * plane);
   hipLaunchKernelGGL(dp_init_kernel, dim3((unsigned)((n_init + 255) / 256)), dim3(256), 0,
                      (hipStream_t)stream, *shape, n_tmax, d_scratch, d_ranges, d_best_s,
                      d_best_sum, d_stage_max);
   MIST_HIP_CHECK(hipGetLastError());
-  // Small batches are latency-bound: spread every state over a team of lanes.
-  const bool wide = (int64_t)n_tmax * plane <= (1 << 19);
   const int states_per_block = kDpThreads / (wide ? kDpWideTeam : 1);
   const dim3 grid((plane + states_per_block - 1) / states_per_block, n_tmax);
   for (int s = 1; s <= shape->max_stages; ++s) {

@@ -88,6 +88,9 @@ class _DpRunner:
             _lib.check(rc, "mist_dp_cost_tables")
         if uniform_device is None:
             self.families = [self._per_mesh_family(meshes)]
+            # large batches of this family run one workgroup per instance, which reads the row
+            # minima in stage-count order (the uniform-device batches are far too small for that)
+            self._prepare_stage_minima(self.families[0])
         else:
             self.families = self._uniform_device_families(meshes, **uniform_device)
         self.launches = 0
@@ -106,6 +109,20 @@ class _DpRunner:
         for v in range(4):
             cs.g_stride[v] = self.cost[v][0].numel()
         return cs
+
+    def _prepare_stage_minima(self, fam: _DpFamily) -> None:
+        """Fills ``MistDpCosts.stage_min`` of a family (``mist_dp_stage_minima``)."""
+        shape_ptr = ctypes.c_void_p(fam.shape.ctypes.data)
+        per_g = self.lib.mist_dp_stage_minima_floats(shape_ptr)
+        if per_g < 0:
+            _lib.check(-1, "mist_dp_stage_minima_floats")
+        with torch.cuda.device(self.device):
+            fam.stage_min = torch.empty((self.Gn, per_g), dtype=torch.float32, device=self.device)
+            rc = self.lib.mist_dp_stage_minima(shape_ptr, ctypes.byref(fam.costs_struct), self.Gn,
+                                               fam.stage_min.data_ptr(), _stream(self.device))
+            _lib.check(rc, "mist_dp_stage_minima")
+        fam.costs_struct.stage_min = fam.stage_min.data_ptr()
+        fam.costs_struct.stage_min_g_stride = per_g
 
     def _per_mesh_family(self, meshes) -> _DpFamily:
         shape = np.zeros(1, dtype=_lib.DP_SHAPE_DTYPE)

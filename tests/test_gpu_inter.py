@@ -19,7 +19,7 @@ def _random_tables(rng, Q, P1, L, inf_frac=0.2, quantum=None):
     return rand((Q, P1, L, L + 1)), rand((Q, P1, L, L + 1)), rand((Q, L, L + 1)), rand((Q, L + 1))
 
 
-def _gpu_dp(meshes, L, D, P1, tabs, tmax, want_argmin=False, mode=0):
+def _gpu_dp(meshes, L, D, P1, tabs, tmax, want_argmin=False, mode=0, relaid=True):
     import torch
     from mist_amd import _lib
 
@@ -34,6 +34,14 @@ def _gpu_dp(meshes, L, D, P1, tabs, tmax, want_argmin=False, mode=0):
     dev = [torch.from_numpy(t).cuda() for t in tabs]
     dev += [torch.cummin(t, dim=-1).values.contiguous() for t in dev]  # running minima over ckpt
     costs = _lib.DpCosts(*[t.data_ptr() for t in dev])
+    if relaid:
+        # the row minima in stage-count order: large batches then run a workgroup per instance
+        per_g = lib.mist_dp_stage_minima_floats(ctypes.c_void_p(shape.ctypes.data))
+        stage_min = torch.empty(per_g, dtype=torch.float32).cuda()
+        _lib.check(lib.mist_dp_stage_minima(
+            ctypes.c_void_p(shape.ctypes.data), ctypes.byref(costs), 1, stage_min.data_ptr(),
+            ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)), "mist_dp_stage_minima")
+        costs.stage_min, costs.stage_min_g_stride = stage_min.data_ptr(), per_g
     n = len(tmax)
     d_t = torch.tensor(tmax, dtype=torch.float32).cuda()
     d_g = torch.zeros(n, dtype=torch.int32).cuda()
@@ -76,6 +84,7 @@ def test_dp_kernel_matches_c_oracle(L, D, meshes, P1, quantum):
     mesh_m = np.array([m for _, m in meshes], dtype=np.int32)
     ptr = lambda a: a.ctypes.data_as(ctypes.c_void_p)
     n_feasible = 0
+    want = []
     for i, t in enumerate(tmax):
         bs, bsum, smax = ctypes.c_int(), ctypes.c_float(), ctypes.c_float()
         arg = np.empty((S + 1, L + 1, D + 1, 4), dtype=np.int32)
@@ -83,6 +92,7 @@ def test_dp_kernel_matches_c_oracle(L, D, meshes, P1, quantum):
             ctypes.c_float(float(t)), L, D, len(meshes), ptr(mesh_n), ptr(mesh_m), P1, ptr(tabs[0]),
             ptr(tabs[1]), ptr(tabs[2]), ptr(tabs[3]), ctypes.byref(bs), ctypes.byref(bsum),
             ctypes.byref(smax), ptr(arg)) == 0
+        want.append((bs.value, np.float32(bsum.value), np.float32(smax.value), arg))
         assert got_s[i] == bs.value, (i, t)
         if bs.value >= 0:
             n_feasible += 1
@@ -90,11 +100,55 @@ def test_dp_kernel_matches_c_oracle(L, D, meshes, P1, quantum):
             g = _gpu_dp(meshes, L, D, P1, tabs, [t], want_argmin=True)
             assert np.array_equal(g[3][0], arg), f"back-pointers differ at t={t}"
     assert n_feasible > 0
+    # The library picks its kernels by batch size (teams of lanes per state for small batches; for
+    # large ones a workgroup per instance with the planes in LDS, or a lane per state when they
+    # do not fit): the same thresholds repeated until the batch passes 2^19 states.
+    reps = (1 << 19) // ((L + 1) * (D + 1) * len(tmax)) + 1
+    for relaid in (True, False):  # without the re-laid minima: always a launch per stage count
+        big_s, big_sum, big_max, big_arg = _gpu_dp(meshes, L, D, P1, tabs, np.tile(tmax, reps),
+                                                   want_argmin=True, relaid=relaid)
+        for r in range(reps):
+            for i, (bs, bsum, smax, arg) in enumerate(want):
+                at = r * len(tmax) + i
+                assert big_s[at] == bs, (relaid, r, i)
+                if bs >= 0:
+                    assert big_sum[at] == bsum and big_max[at] == smax, (relaid, r, i)
+                    assert np.array_equal(big_arg[at], arg), (relaid, r, i)
+    # the re-laid table itself: entry (p, q, k, i) is the smallest admissible-ckpt cost
+    import torch
+    from mist_amd import _lib as lib_mod
+    shape = np.zeros(1, dtype=lib_mod.DP_SHAPE_DTYPE)
+    shape["num_layers"], shape["num_devices"], shape["num_mesh"], shape["p_dim"] = L, D, len(meshes), P1
+    shape["max_stages"] = S
+    shape["mesh_n"][0, :len(meshes)], shape["mesh_m"][0, :len(meshes)] = mesh_n, mesh_m
+    glib = lib_mod.load()
+    per_g = glib.mist_dp_stage_minima_floats(ctypes.c_void_p(shape.ctypes.data))
+    tri = L * (L + 1) // 2
+    assert per_g == S * len(meshes) * tri
+    dev = [torch.from_numpy(t).cuda() for t in tabs]
+    dev += [torch.cummin(t, dim=-1).values.contiguous() for t in dev]
+    costs = lib_mod.DpCosts(*[t.data_ptr() for t in dev])
+    out = torch.empty(per_g, dtype=torch.float32).cuda()
+    lib_mod.check(glib.mist_dp_stage_minima(
+        ctypes.c_void_p(shape.ctypes.data), ctypes.byref(costs), 1, out.data_ptr(),
+        ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)), "mist_dp_stage_minima")
+    got = out.cpu().numpy().reshape(S, len(meshes), tri)
+    for p_ in range(S):
+        for q in range(len(meshes)):
+            for k in range(L):
+                for i in range(k, L):
+                    l = i - k + 1
+                    row = (tabs[3][q] if k == 0 and i == L - 1 else tabs[1][q, p_, l - 1] if k == 0
+                           else tabs[2][q, l - 1] if i == L - 1 else tabs[0][q, p_, l - 1])
+                    expect = row[: L - i + 1].min() if k <= L - 1 - p_ else np.inf
+                    assert got[p_, q, k * L - k * (k - 1) // 2 + i - k] == expect, (p_, q, k, i)
     # bottleneck mode = the smallest threshold for which the threshold DP is feasible
     _, bott, path_sum = _gpu_dp(meshes, L, D, P1, tabs, [0.0], mode=1)
     # ... and the sum reported with it belongs to a partition admissible at that threshold
     at_bott = _gpu_dp(meshes, L, D, P1, tabs, [bott[0]])
     assert at_bott[0][0] >= 0 and at_bott[1][0] <= path_sum[0] and at_bott[2][0] == bott[0]
+    big = _gpu_dp(meshes, L, D, P1, tabs, np.zeros(reps * len(tmax), dtype=np.float32), mode=1)
+    assert np.all(big[1] == bott[0]) and np.all(big[2] == path_sum[0]) and np.all(big[0] == _[0])
     cand = np.unique(np.concatenate([t.ravel() for t in tabs[:3]]))
     cand = cand[np.isfinite(cand)]
     feas = _gpu_dp(meshes, L, D, P1, tabs, cand)[0] >= 0
@@ -256,6 +310,33 @@ def test_uniform_device_dp_kernel_matches_oracle(L, num_nodes, gpn, P1, quantum,
             ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)), "mist_dp_run")
         torch.cuda.synchronize()
         bs, bsum, smax, argmin = d_s.cpu().numpy(), d_sum.cpu().numpy(), d_max.cpu().numpy(), arg.cpu().numpy()
+        # the same thresholds as a batch of more than 2^19 states (another kernel of the library)
+        reps = (1 << 19) // ((L + 1) * n) + 1
+        if reps * n <= 65535:
+            N = reps * n
+            b_t = d_t.repeat(reps)
+            b_g = torch.zeros(N, dtype=torch.int32).cuda()
+            b_s = torch.empty(N, dtype=torch.int32).cuda()
+            b_sum = torch.empty(N, dtype=torch.float32).cuda()
+            b_max = torch.empty(N, dtype=torch.float32).cuda()
+            b_scr = torch.empty(lib.mist_dp_scratch_floats(ctypes.c_void_p(shape.ctypes.data), N), dtype=torch.float32).cuda()
+            b_arg = torch.full((N, Sm + 1, L + 1, 1, 4), -1, dtype=torch.int32).cuda()
+            per_g = lib.mist_dp_stage_minima_floats(ctypes.c_void_p(shape.ctypes.data))
+            stage_min = torch.empty(per_g, dtype=torch.float32).cuda()
+            _lib.check(lib.mist_dp_stage_minima(
+                ctypes.c_void_p(shape.ctypes.data), ctypes.byref(costs), 1, stage_min.data_ptr(),
+                ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)), "mist_dp_stage_minima")
+            costs.stage_min, costs.stage_min_g_stride = stage_min.data_ptr(), per_g
+            _lib.check(lib.mist_dp_run(
+                ctypes.c_void_p(shape.ctypes.data), ctypes.byref(costs), b_t.data_ptr(), b_g.data_ptr(), N, 0,
+                b_s.data_ptr(), b_sum.data_ptr(), b_max.data_ptr(), b_arg.data_ptr(), b_scr.data_ptr(),
+                ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)), "mist_dp_run")
+            torch.cuda.synchronize()
+            assert np.array_equal(b_s.cpu().numpy(), np.tile(bs, reps))
+            ok = np.tile(bs, reps) >= 0
+            assert np.array_equal(b_sum.cpu().numpy()[ok], np.tile(bsum, reps)[ok])
+            assert np.array_equal(b_max.cpu().numpy()[ok], np.tile(smax, reps)[ok])
+            assert np.array_equal(b_arg.cpu().numpy()[ok], np.tile(argmin, (reps, 1, 1, 1, 1))[ok])
         for i in range(n):
             if bs[i] < 0:
                 continue

@@ -100,6 +100,14 @@ int mist_dp_filter_tmax(const float *sorted_unique, int n, double gap, float *ou
 int mist_dp_window_begin(const float *ascending, int n, float lo, int open_below,
                          float start_value, double gap, float *out);
 
+/* mist_dp_window_begin for n_windows walks in one call: window w owns
+ * ascending[offsets[w] .. offsets[w + 1]) and writes its kept values to the same range of out;
+ * out_count[w] = number kept, or MIST_DP_NO_START. */
+int mist_dp_window_begin_many(const float *ascending, const int64_t *offsets, int n_windows,
+                              const float *lo, const uint8_t *open_below,
+                              const float *start_value, double gap, float *out,
+                              int32_t *out_count);
+
 /* t_max candidates of value windows (reference: the sort + scan over every finite stage cost,
  * inter_tuning.py:180-199, restricted to where the scan can get).  Request r selects the finite
  * values v of the costs / with_pre / with_post tables of table row d_rows[r] with

@@ -184,6 +184,8 @@ _DP_SIGNATURES = {
     "mist_dp_window_begin": (
         ctypes.c_int,
         [_VP, ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_float, ctypes.c_double, _VP]),
+    "mist_dp_window_begin_many": (
+        ctypes.c_int, [_VP, _VP, ctypes.c_int, _VP, _VP, _VP, ctypes.c_double, _VP, _VP]),
     "mist_dp_select_candidates": (
         ctypes.c_int,
         [ctypes.POINTER(DpCosts), ctypes.c_int, _VP, _VP, _VP, _VP, _VP, ctypes.c_int, _VP, _VP],

@@ -713,6 +713,27 @@ int mist_dp_window_begin(const float *ascending, int n, float lo, int open_below
   return mist_dp_filter_tmax(ascending + first, n - first, gap, out);  // the walk from there
 }
 
+int mist_dp_window_begin_many(const float *ascending, const int64_t *offsets, int n_windows,
+                              const float *lo, const uint8_t *open_below,
+                              const float *start_value, double gap, float *out,
+                              int32_t *out_count) {
+  if (n_windows < 0) return fail(MIST_E_INVALID, "n_windows %d < 0", n_windows);
+  if (n_windows == 0) return 0;
+  if (!offsets || !lo || !open_below || !start_value || !out_count)
+    return fail(MIST_E_INVALID, "null pointer argument");
+  for (int w = 0; w < n_windows; ++w) {
+    const int64_t first = offsets[w], count = offsets[w + 1] - first;
+    if (first < 0 || count < 0 || count > INT32_MAX)
+      return fail(MIST_E_INVALID, "offsets of window %d are not ascending", w);
+    const int kept =
+        mist_dp_window_begin(count ? ascending + first : nullptr, (int)count, lo[w], open_below[w],
+                             start_value[w], gap, count ? out + first : nullptr);
+    if (kept < 0 && kept != MIST_DP_NO_START) return kept;
+    out_count[w] = kept;
+  }
+  return 0;
+}
+
 int mist_dp_select_candidates(const MistDpCosts *costs, int n_requests, const int32_t *d_rows,
                               const float *d_lo, const float *d_hi, float *d_out_values,
                               int32_t *d_out_request, int capacity, int32_t *d_counts,

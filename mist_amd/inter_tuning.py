@@ -159,11 +159,12 @@ class _DpRunner:
             fams.append(_DpFamily(shape, self._costs_struct(q), False))
         return fams
 
-    def candidates_between(self, rows: np.ndarray, lo: np.ndarray, hi: np.ndarray):
+    def candidates_between_flat(self, rows: np.ndarray, lo: np.ndarray, hi: np.ndarray):
         """Per requested table row g: the ascending t_max candidates v (finite stage costs of the
         costs / with_pre / with_post tables, inter_tuning.py:180-186) with lo < v <= hi (lo = -inf
         includes everything below), and how many finite candidates lie above hi.  One kernel
-        pass over the requested rows; only the selected values come back."""
+        pass over the requested rows; only the selected values come back: ``(values, bounds,
+        above)`` with request i owning ``values[bounds[i]:bounds[i + 1]]``."""
         dev = self.device
         self.fetches += 1
         n = len(rows)
@@ -194,8 +195,16 @@ class _DpRunner:
         # stable sort a radix sort
         order = np.argsort(h_request.astype(np.uint16), kind="stable")
         h_values, h_request = h_values[order], h_request[order]
-        bounds = np.searchsorted(h_request, np.arange(n + 1))
-        return [(np.sort(h_values[bounds[i]:bounds[i + 1]]), int(h_counts[1 + i])) for i in range(n)]
+        bounds = np.searchsorted(h_request, np.arange(n + 1)).astype(np.int64)
+        for i in range(n):
+            h_values[bounds[i]:bounds[i + 1]].sort()
+        return h_values, bounds, h_counts[1:]
+
+    def candidates_between(self, rows: np.ndarray, lo: np.ndarray, hi: np.ndarray):
+        """``candidates_between_flat`` as one ``(ascending values, candidates above hi)`` pair
+        per requested row."""
+        values, bounds, above = self.candidates_between_flat(rows, lo, hi)
+        return [(values[bounds[i]:bounds[i + 1]], int(above[i])) for i in range(len(above))]
 
     def filter_gap(self, ascending: np.ndarray) -> np.ndarray:
         """The reference's gap rule (inter_tuning.py:198) applied from the first element on
@@ -352,6 +361,39 @@ class _Window:
             _lib.check(n, "mist_dp_window_begin")
         self._append(kept[:n])
         return True
+
+    @staticmethod
+    def begin_many(windows, values: np.ndarray, bounds: np.ndarray, above: np.ndarray,
+                   lo: np.ndarray, hi: np.ndarray) -> List[bool]:
+        """``begin`` of several windows on the flat result of one fetch (one library call)."""
+        if not windows:
+            return []
+        n = len(windows)
+        lib = windows[0].runner.lib
+        values = np.ascontiguousarray(values, dtype=np.float32)
+        bounds = np.ascontiguousarray(bounds, dtype=np.int64)
+        below = np.isneginf(lo)
+        lo_arg = np.where(below, np.float32(0.0), lo).astype(np.float32)
+        open_below = below.astype(np.uint8)
+        start = np.array([w.start_value for w in windows], dtype=np.float32)
+        kept = np.empty(len(values), dtype=np.float32)
+        count = np.empty(n, dtype=np.int32)
+        rc = lib.mist_dp_window_begin_many(
+            ctypes.c_void_p(values.ctypes.data), ctypes.c_void_p(bounds.ctypes.data), n,
+            ctypes.c_void_p(lo_arg.ctypes.data), ctypes.c_void_p(open_below.ctypes.data),
+            ctypes.c_void_p(start.ctypes.data), GAP, ctypes.c_void_p(kept.ctypes.data),
+            ctypes.c_void_p(count.ctypes.data))
+        _lib.check(rc, "mist_dp_window_begin_many")
+        done = []
+        for j, w in enumerate(windows):
+            w.hi, w.complete = hi[j], above[j] == 0
+            if count[j] == _lib.DP_NO_START:
+                done.append(False)
+                continue
+            if count[j] > 0:
+                w._append(kept[bounds[j]:bounds[j] + count[j]])
+            done.append(True)
+        return done
 
     def _append(self, kept: np.ndarray) -> None:
         self.kept = np.concatenate([self.kept, kept])
@@ -555,9 +597,10 @@ def _search(runner: _DpRunner, rows: np.ndarray, Gs: List[int], stats: Optional[
             lo = np.array([windows[idx[k]].lower_margin(widen) for k in pending], dtype=np.float32)
             if widen >= 8:
                 lo[:] = -np.inf
-            got = runner.candidates_between(flat[idx[pending]], lo, hi[pending])
-            pending = [k for j, k in enumerate(pending)
-                       if not windows[idx[k]].begin(got[j][0], got[j][1], lo[j], hi[k])]
+            values, bounds, above = runner.candidates_between_flat(flat[idx[pending]], lo, hi[pending])
+            done = _Window.begin_many([windows[idx[k]] for k in pending], values, bounds, above,
+                                      lo, hi[pending])
+            pending = [k for k, ok in zip(pending, done) if not ok]
             widen += 1
         # one more pass for the windows whose first kept candidate turned out to lie higher
         # than assumed (the remaining cases extend one by one while the scan runs)

@@ -369,6 +369,45 @@ def test_threshold_window_equals_full_walk(seed):
         assert np.array_equal(got, want), (seed, trial)
 
 
+def test_window_begin_many_equals_single_begins():
+    """One library call for the first fetch of many windows gives what the per-window call gives
+    (kept values, fetched range, completeness, and which windows must fetch from further below)."""
+    from mist_amd.inter_tuning import _Window
+
+    rng = np.random.default_rng(11)
+    centres = rng.uniform(0.05, 40.0, size=200)
+    dense = (centres[:, None] + rng.uniform(0, 3e-6, size=(200, 6)) * rng.integers(0, 2, size=(200, 1))).ravel()
+    values = np.unique(np.concatenate([dense, rng.uniform(0.05, 40.0, size=300)]).astype(np.float32))
+    runner = _FakeRunner(values)
+    outcomes = set()
+    for widen in (0, 3, 8):
+        starts = [values[rng.integers(len(values))] if k % 2 else np.float32(rng.uniform(0.0, 41.0)) for k in range(24)]
+        single = [_Window(runner, 0, 4, s, start_sum=float(s)) for s in starts]
+        many = [_Window(runner, 0, 4, s, start_sum=float(s)) for s in starts]
+        lo = np.array([w.lower_margin(widen) if widen < 8 else -np.inf for w in single], dtype=np.float32)
+        hi = np.array([s + rng.uniform(0, 0.3) for s in starts], dtype=np.float32)
+        hi[::5] = np.float32(41.0)   # nothing above
+        lo[1::7] = hi[1::7]          # empty fetch
+        for k in range(2, len(starts), 3):  # fetch that begins inside a run of near-equal values
+            inside = np.float32(dense[rng.integers(len(dense))])
+            single[k].start_value = many[k].start_value = inside
+            lo[k], hi[k] = inside - np.float32(4e-7), inside + np.float32(0.1)
+        got = runner.candidates_between(np.zeros(len(starts)), lo, hi)
+        want_ok = [w.begin(v, a, l, h) for w, (v, a), l, h in zip(single, got, lo, hi)]
+        flat = np.concatenate([v for v, _ in got]) if got else np.empty(0, dtype=np.float32)
+        bounds = np.concatenate([[0], np.cumsum([len(v) for v, _ in got])]).astype(np.int64)
+        above = np.array([a for _, a in got], dtype=np.int32)
+        ok = _Window.begin_many(many, flat, bounds, above, lo, hi)
+        assert ok == want_ok
+        outcomes.update(ok)
+        for a, b in zip(single, many):
+            assert np.array_equal(a.kept, b.kept) and a.hi == b.hi and a.complete == b.complete
+            assert a.bound == b.bound or (np.isinf(a.bound) and np.isinf(b.bound))
+    assert outcomes == {True, False}
+    assert _Window.begin_many([], np.empty(0, dtype=np.float32), np.zeros(1, dtype=np.int64),
+                              np.empty(0, dtype=np.int32), np.empty(0), np.empty(0)) == []
+
+
 def test_inputs_outside_the_kernels_preconditions_are_rejected():
     """Negative or non-finite table values / hardware parameters would break the monotonicity
     the reduce kernel's exact pruning relies on: the host refuses them before any launch."""

@@ -147,6 +147,16 @@ int mist_dp_run(const MistDpShape *shape, const MistDpCosts *costs, const float 
                 float *d_best_sum, float *d_stage_max, int32_t *d_argmin, float *d_scratch,
                 void *stream);
 
+/* Partition of every instance of a mist_dp_run() call that recorded back-pointers
+ * (reference: the walk of inter_tuning.py:341-355, here on the GPU so that only the partitions
+ * travel to the host).  d_path[n_tmax][max_stages][4] int32: stage i of instance t in pipeline
+ * order as (end layer, n, m, ckpt), -1 in the unused tail (all -1 if d_best_s[t] < 0).  The
+ * stages start at layer 0 and each starts after the previous one's end; a walk that meets an
+ * entry the DP did not write stops early, which the caller can tell from the last end layer.
+ * d_argmin needs no pre-fill for this. */
+int mist_dp_backtrack(const MistDpShape *shape, const int32_t *d_argmin, const int32_t *d_best_s,
+                      int n_tmax, int32_t *d_path, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

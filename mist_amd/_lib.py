@@ -191,6 +191,7 @@ _DP_SIGNATURES = {
         [ctypes.POINTER(DpCosts), ctypes.c_int, _VP, _VP, _VP, _VP, _VP, ctypes.c_int, _VP, _VP],
     ),
     "mist_dp_scratch_floats": (ctypes.c_int64, [_VP, ctypes.c_int]),
+    "mist_dp_backtrack": (ctypes.c_int, [_VP, _VP, _VP, ctypes.c_int, _VP, _VP]),
     "mist_dp_stage_minima_floats": (ctypes.c_int64, [_VP]),
     "mist_dp_stage_minima": (ctypes.c_int, [_VP, ctypes.POINTER(DpCosts), ctypes.c_int, _VP, _VP]),
     "mist_dp_run": (

@@ -544,6 +544,39 @@ __global__ __launch_bounds__(kDpFusedThreads) void dp_fused_kernel(
   }
 }
 
+// Follows the back-pointers of each instance from (best_s, layer 0, all devices) and writes its
+// stages in pipeline order (inter_tuning.py:341-355); one thread per instance.  Only entries the
+// DP wrote are read: a state with a finite value has a winner, and so has every successor on
+// its path.
+__global__ __launch_bounds__(64) void backtrack_kernel(const MistDpShape shape,
+                                                       const int32_t *__restrict__ argmin,
+                                                       const int32_t *__restrict__ best_s, int n,
+                                                       int32_t *__restrict__ path) {
+  const int t = blockIdx.x * 64 + threadIdx.x;
+  if (t >= n) return;
+  const int L = shape.num_layers, W = shape.num_devices + 1;
+  const int64_t plane = (int64_t)(L + 1) * W;
+  int32_t *out = path + (int64_t)t * shape.max_stages * 4;
+  for (int i = 0; i < shape.max_stages * 4; ++i) out[i] = -1;
+  int s = best_s[t], k = 0, d = shape.num_devices, stage = 0;
+  while (s > 0 && k < L && stage < shape.max_stages) {
+    const int32_t *a = argmin + (((int64_t)t * (shape.max_stages + 1) + s) * plane + k * W + d) * 4;
+    const int end = a[0], mesh_n = a[1], mesh_m = a[2];
+    // an entry the DP did not write (caller's fill or stale memory) ends the walk: the host sees
+    // a path that does not cover the layers
+    if (end < k || end >= L || mesh_n < 1 || mesh_m < 1) break;
+    if (shape.free_devices == 0 && mesh_n * mesh_m > d) break;
+    out[stage * 4 + 0] = end;
+    out[stage * 4 + 1] = mesh_n;
+    out[stage * 4 + 2] = mesh_m;
+    out[stage * 4 + 3] = a[3];
+    ++stage;
+    --s;
+    k = end + 1;
+    if (shape.free_devices == 0) d -= mesh_n * mesh_m;
+  }
+}
+
 // Row minima in the order the recurrence reads them: out[g][p][q][triangle(k, i)] =
 // dp_row_min(p, k, q, i).  A workgroup scanning stage count p + 1 of g finds all it needs in one
 // contiguous block, and the end layers i of one (q, k) lie next to each other.
@@ -648,6 +681,18 @@ int mist_dp_cost_tables(const MistProblem *problem, const MistOutTables *tables,
                        rows_per_g[v], (int)(L + 1), (int)S, slot, d_out[v], d_out_pmin[v]);
     MIST_HIP_CHECK(hipGetLastError());
   }
+  return 0;
+}
+
+int mist_dp_backtrack(const MistDpShape *shape, const int32_t *d_argmin, const int32_t *d_best_s,
+                      int n_tmax, int32_t *d_path, void *stream) {
+  if (int rc = check_shape(shape)) return rc;
+  if (!d_argmin || !d_best_s || !d_path) return fail(MIST_E_INVALID, "null pointer argument");
+  if (n_tmax <= 0 || n_tmax > 65535)
+    return fail(MIST_E_INVALID, "n_tmax must be in [1, 65535], got %d", n_tmax);
+  hipLaunchKernelGGL(backtrack_kernel, dim3((unsigned)((n_tmax + 63) / 64)), dim3(64), 0,
+                     (hipStream_t)stream, *shape, d_argmin, d_best_s, n_tmax, d_path);
+  MIST_HIP_CHECK(hipGetLastError());
   return 0;
 }
 

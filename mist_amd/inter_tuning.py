@@ -217,9 +217,11 @@ class _DpRunner:
         return kept[:n]
 
     def run(self, g_index: np.ndarray, tmax: np.ndarray, mode: int = _lib.DP_THRESHOLD,
-            want_argmin: bool = False, family: Optional[_DpFamily] = None):
+            want_argmin: bool = False, family: Optional[_DpFamily] = None,
+            want_path: bool = False):
         """DP instances (g_index[i], tmax[i]) of one family -> (best_s int32, best_sum f32,
-        stage_max f32 [, argmin])."""
+        stage_max f32 [, argmin] [, path]).  ``path`` [n, max_stages, 4]: the stages of each
+        instance's partition as (end layer, n, m, ckpt), walked on the GPU."""
         fam = self.families[0] if family is None else family
         n = len(tmax)
         dev = self.device
@@ -232,22 +234,33 @@ class _DpRunner:
             n_scratch = self.lib.mist_dp_scratch_floats(ctypes.c_void_p(fam.shape.ctypes.data), n)
             scratch = torch.empty(n_scratch, dtype=torch.float32, device=dev)
             argmin = None
+            arg_shape = (n, fam.S_max + 1, fam.L + 1, fam.D + 1, 4)
             if want_argmin:
-                argmin = torch.full((n, fam.S_max + 1, fam.L + 1, fam.D + 1, 4), -1,
-                                    dtype=torch.int32, device=dev)
+                argmin = torch.full(arg_shape, -1, dtype=torch.int32, device=dev)
+            elif want_path:  # the walk only reads entries the DP wrote: no fill
+                argmin = torch.empty(arg_shape, dtype=torch.int32, device=dev)
             rc = self.lib.mist_dp_run(
                 ctypes.c_void_p(fam.shape.ctypes.data), ctypes.byref(fam.costs_struct),
                 d_in[0].data_ptr(), d_in[1].data_ptr(), n, mode,
                 d_out[0].data_ptr(), d_out[1].data_ptr(), d_out[2].data_ptr(),
-                argmin.data_ptr() if want_argmin else None, scratch.data_ptr(), _stream(dev),
+                argmin.data_ptr() if argmin is not None else None, scratch.data_ptr(), _stream(dev),
             )
             _lib.check(rc, "mist_dp_run")
             self.launches += 1
             self.thresholds_run += n
+            path = None
+            if want_path:
+                path = torch.empty((n, fam.S_max, 4), dtype=torch.int32, device=dev)
+                rc = self.lib.mist_dp_backtrack(
+                    ctypes.c_void_p(fam.shape.ctypes.data), argmin.data_ptr(), d_out[0].data_ptr(),
+                    n, path.data_ptr(), _stream(dev))
+                _lib.check(rc, "mist_dp_backtrack")
             host = d_out.cpu().numpy()
             out = (host[0].view(np.int32), host[1], host[2])
             if want_argmin:
                 out = out + (argmin.cpu().numpy(),)
+            if want_path:
+                out = out + (path.cpu().numpy(),)
         return out
 
     @staticmethod
@@ -290,24 +303,24 @@ class _DpRunner:
         n = len(tmax)
         best = [(np.inf, None)] * n
         for fam in self.families:
-            bs, bsum, smax, argmin = self.run(g_index, tmax, want_argmin=True, family=fam)
+            bs, bsum, smax, path = self.run(g_index, tmax, family=fam, want_path=True)
             total = self._total(bs, bsum, smax, G)
             for i in range(n):
                 if total[i] < best[i][0]:
-                    best[i] = (float(total[i]), (fam, int(bs[i]), argmin[i]))
+                    best[i] = (float(total[i]), (fam, int(bs[i]), path[i]))
         out = []
         for total, found in best:
             assert found is not None
-            fam, cs, argmin = found
+            fam, n_stages, path = found
+            stages = path[:n_stages].tolist()
             cl, cd, inter = 0, fam.D, []
-            while cs > 0 and cl < fam.L and (cd > 0 or not fam.consumes_devices):
-                end, n_, m_, ckpt = (int(v) for v in argmin[cs, cl, cd])
-                assert end != -1
+            for end, n_, m_, ckpt in stages:
+                assert end >= cl, "back-pointer walk left the DP's states"
                 inter.append(((cl, end), (n_, m_), ckpt))
-                cs, cl = cs - 1, end + 1
+                cl = end + 1
                 if fam.consumes_devices:
                     cd -= n_ * m_
-            assert cs == 0 and cl == fam.L and cd == 0
+            assert len(inter) == n_stages and cl == fam.L and (cd == 0 or not fam.consumes_devices)
             out.append((total, inter))
         return out
 

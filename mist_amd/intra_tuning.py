@@ -262,11 +262,15 @@ class IntraStageTuner:
         P1, L, S = self.max_possible_pre_saved_micro_batches + 1, self.num_layers, self.sample_size
         shapes = [(Gn, Qn, P1, L, L + 1, S), (Gn, Qn, P1, L, L + 1, S), (Gn, Qn, L, L + 1, S), (Gn, Qn, L + 1, S)]
         dev = self.device
-        return DeviceTables(
-            stable=[torch.full(s, float("inf"), dtype=torch.float64, device=dev) for s in shapes],
-            delta=[torch.full(s, float("inf"), dtype=torch.float64, device=dev) for s in shapes],
-            index=[torch.full(s, -1, dtype=torch.int32, device=dev) for s in shapes],
-        )
+        # one allocation and one fill per element type; the tables are views of it
+        sizes = [int(np.prod(s)) for s in shapes]
+        starts = np.concatenate([[0], np.cumsum(sizes)])
+        costs = torch.full((2 * int(starts[-1]),), float("inf"), dtype=torch.float64, device=dev)
+        index = torch.full((int(starts[-1]),), -1, dtype=torch.int32, device=dev)
+        def views(flat, base):
+            return [flat[base + int(starts[v]):base + int(starts[v + 1])].view(shapes[v]) for v in range(4)]
+        return DeviceTables(stable=views(costs, 0), delta=views(costs, int(starts[-1])),
+                            index=views(index, 0))
 
     # ------------------------------------------------------------------ device side
     def upload(self, plan) -> dict:

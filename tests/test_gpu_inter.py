@@ -57,9 +57,26 @@ def _gpu_dp(meshes, L, D, P1, tabs, tmax, want_argmin=False, mode=0, relaid=True
         scr.data_ptr(), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream),
     )
     _lib.check(rc, "mist_dp_run")
+    path = None
+    if want_argmin:  # the partitions, walked on the GPU from the same back-pointers
+        path = torch.full((n, S, 4), -7, dtype=torch.int32).cuda()
+        _lib.check(lib.mist_dp_backtrack(
+            ctypes.c_void_p(shape.ctypes.data), arg.data_ptr(), d_s.data_ptr(), n, path.data_ptr(),
+            ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)), "mist_dp_backtrack")
     torch.cuda.synchronize()
     out = (d_s.cpu().numpy(), d_sum.cpu().numpy(), d_max.cpu().numpy())
-    return out + ((arg.cpu().numpy(),) if want_argmin else ())
+    return out + ((arg.cpu().numpy(), path.cpu().numpy()) if want_argmin else ())
+
+
+def _walk(arg, best_s, D):
+    """Partition from one instance's back-pointers, as the reference walks them
+    (inter_tuning.py:341-355): [(end layer, n, m, ckpt), ...] in pipeline order."""
+    out, cs, cl, cd = [], int(best_s), 0, D
+    while cs > 0:
+        end, n, m, ckpt = (int(v) for v in arg[cs, cl, cd])
+        out.append([end, n, m, ckpt])
+        cs, cl, cd = cs - 1, end + 1, cd - n * m
+    return out
 
 
 @pytest.mark.parametrize(
@@ -99,14 +116,16 @@ def test_dp_kernel_matches_c_oracle(L, D, meshes, P1, quantum):
             assert got_sum[i] == np.float32(bsum.value) and got_max[i] == np.float32(smax.value), (i, t)
             g = _gpu_dp(meshes, L, D, P1, tabs, [t], want_argmin=True)
             assert np.array_equal(g[3][0], arg), f"back-pointers differ at t={t}"
+            stages = _walk(arg, bs.value, D)
+            assert g[4][0][:len(stages)].tolist() == stages and np.all(g[4][0][len(stages):] == -1)
     assert n_feasible > 0
     # The library picks its kernels by batch size (teams of lanes per state for small batches; for
     # large ones a workgroup per instance with the planes in LDS, or a lane per state when they
     # do not fit): the same thresholds repeated until the batch passes 2^19 states.
     reps = (1 << 19) // ((L + 1) * (D + 1) * len(tmax)) + 1
     for relaid in (True, False):  # without the re-laid minima: always a launch per stage count
-        big_s, big_sum, big_max, big_arg = _gpu_dp(meshes, L, D, P1, tabs, np.tile(tmax, reps),
-                                                   want_argmin=True, relaid=relaid)
+        big_s, big_sum, big_max, big_arg, big_path = _gpu_dp(
+            meshes, L, D, P1, tabs, np.tile(tmax, reps), want_argmin=True, relaid=relaid)
         for r in range(reps):
             for i, (bs, bsum, smax, arg) in enumerate(want):
                 at = r * len(tmax) + i
@@ -114,6 +133,11 @@ def test_dp_kernel_matches_c_oracle(L, D, meshes, P1, quantum):
                 if bs >= 0:
                     assert big_sum[at] == bsum and big_max[at] == smax, (relaid, r, i)
                     assert np.array_equal(big_arg[at], arg), (relaid, r, i)
+                    stages = _walk(arg, bs, D)
+                    assert big_path[at][:len(stages)].tolist() == stages
+                    assert np.all(big_path[at][len(stages):] == -1)
+                else:
+                    assert np.all(big_path[at] == -1)
     # the re-laid table itself: entry (p, q, k, i) is the smallest admissible-ckpt cost
     import torch
     from mist_amd import _lib as lib_mod

@@ -233,6 +233,8 @@ def test_argument_checks_reject_before_any_launch():
     assert b"scratch" in lib.mist_last_error()
     assert lib.mist_dp_run(sp, ctypes.byref(costs), fake, fake, 70000, 0, fake, fake, fake, None, fake, None) == -1
     assert lib.mist_dp_run(sp, ctypes.byref(costs), fake, fake, 1, 7, fake, fake, fake, None, fake, None) == -1
+    assert lib.mist_dp_backtrack(sp, None, fake, 1, fake, None) == -1
+    assert lib.mist_dp_backtrack(sp, fake, fake, 0, fake, None) == -1
     # re-laid row minima: max_stages * Q * L (L + 1) / 2 floats per g
     assert lib.mist_dp_stage_minima_floats(sp) == 4 * 2 * (80 * 81 // 2)
     assert lib.mist_dp_stage_minima_floats(ctypes.c_void_p(np.zeros(1, dtype=_lib.DP_SHAPE_DTYPE).ctypes.data)) == -1

@@ -28,6 +28,7 @@ from . import _lib
 from .comm_model import gpu_gpu_comm_latency
 from .config import BATCH_SIZE_CANDIDATES, MistConfig
 from .layer_tables import LayerTables
+from .node_database import layer_tables_for
 from .search_space import SearchSpace
 from .stage_inputs import GroupInputBuilder, make_problem, pre_post_strategy_fields
 
@@ -176,7 +177,7 @@ def analyze(mist_config: MistConfig, layer_tables: Optional[LayerTables] = None,
     st = mist_config.strategy
     if st is None or "layer_partitions" not in st:
         raise ValueError("the strategy block is missing or disabled")
-    tables = LayerTables(mist_config) if layer_tables is None else layer_tables
+    tables = layer_tables_for(mist_config) if layer_tables is None else layer_tables
     S, G = st.num_stages, st.gradient_accumulation_steps
     stages, keys = [], []
     for i in range(S):

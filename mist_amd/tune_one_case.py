@@ -38,6 +38,7 @@ from .inter_tuning_uniform_device import inter_stage_tune_batch_uniform_device
 from .inter_tuning_mip import inter_stage_tune as inter_stage_tune_mip
 from .intra_tuning import SAMPLE_SIZE, IntraStageTuner, intra_stage_tune
 from .layer_tables import LayerTables
+from .node_database import layer_tables_for
 from .search_space import _get_device_mesh_candidates, _get_grad_accumu_steps_candidates
 
 
@@ -103,7 +104,7 @@ def _uniform_device_pp_mip(mist_config, device, stats):
     one of ``tuning.sample_size`` samples, then the stage assignment; the first best tp wins.
     One tp at a time keeps a single set of sampled tables in HBM."""
     hw, tuning = mist_config.hardware, mist_config.tuning
-    tables = LayerTables(mist_config)
+    tables = layer_tables_for(mist_config)
     meshes = _get_device_mesh_candidates(hw.num_nodes, hw.num_gpus_per_node, contiguous_inter_node=False)
     Gs = _get_grad_accumu_steps_candidates(mist_config.training.global_batch_size)
     L = mist_config.model.num_hidden_layers
@@ -135,7 +136,7 @@ class PreparedSearch:
         if self.granularity not in ("uniform-pp", "uniform-pp-simple-heuristic-mem-opt", "inter-stage",
                                     "uniform-device-pp"):
             raise ValueError(f"PreparedSearch does not cover '{self.granularity}'")
-        self.tables = LayerTables(mist_config)
+        self.tables = layer_tables_for(mist_config)
         self.meshes = _get_device_mesh_candidates(hw.num_nodes, hw.num_gpus_per_node, contiguous_inter_node=False)
         self.Gs = _get_grad_accumu_steps_candidates(mist_config.training.global_batch_size)
         self.L = model.num_hidden_layers
@@ -203,7 +204,7 @@ def tune(mist_config: MistConfig, device: str = "cuda:0", stats: Optional[dict] 
     t_start = time.perf_counter()
 
     if granularity == "no-pp":
-        best_cost, best_solution = _no_pp(mist_config, LayerTables(mist_config), device, stats)
+        best_cost, best_solution = _no_pp(mist_config, layer_tables_for(mist_config), device, stats)
     elif granularity in ("uniform-pp", "inter-stage", "uniform-device-pp"):
         best_cost, best_solution = PreparedSearch(mist_config, device).run(stats)
     elif granularity == "uniform-pp-simple-heuristic-mem-opt":

@@ -1,0 +1,123 @@
+"""Single-GPU hardware calibration (mist_amd/calibrate.py): the fitting half on synthetic
+measurements generated from known parameters (CPU), the measurement half on the GPU."""
+import numpy as np
+import pytest
+
+from mist_amd import calibrate
+from mist_amd.stage_inputs import THREE_CASE_MASKS, TWO_CASE_MASKS
+
+
+def _random_params(rng):
+    return rng.uniform(1.0, 3.0, size=28)
+
+
+def test_interference_estimate_equals_the_oracle_model():
+    """Product-side numpy model against the oracle's restatement of optimize.py:1012-1079
+    (itself pinned by brute force and closed-form cases) on random inputs with every non-zero
+    pattern."""
+    from oracle.interference import interference_one_group
+
+    rng = np.random.default_rng(3)
+    for _ in range(20):
+        params = _random_params(rng)
+        X = rng.uniform(0.0, 5e-3, size=(400, 4)) * rng.integers(0, 2, size=(400, 4))
+        got = calibrate.interference_estimate(X[:, 0], X[:, 1], X[:, 2], X[:, 3], params)
+        want = interference_one_group(X[:, 0], X[:, 1], X[:, 2], X[:, 3], params)
+        assert np.array_equal(got, want)
+    # one resource alone is not slowed down; all factors 1 -> the longest resource
+    assert calibrate.interference_estimate(2e-3, 0, 0, 0, params)[0] == 2e-3
+    assert calibrate.interference_estimate(1e-3, 2e-3, 5e-4, 0, np.ones(28))[0] == 2e-3
+
+
+def test_mask_slices_tile_the_parameter_vector():
+    seen = []
+    for mask in [(True,) * 4] + list(THREE_CASE_MASKS) + list(TWO_CASE_MASKS):
+        sl = calibrate.mask_slice(mask)
+        assert sl.stop - sl.start == sum(mask)
+        seen += list(range(sl.start, sl.stop))
+    assert seen == list(range(28))
+    assert len(calibrate.SINGLE_GPU_MASKS) == 4
+    assert sum(sum(m) for m in calibrate.SINGLE_GPU_MASKS) == 9
+    with pytest.raises(ValueError):
+        calibrate.mask_slice((True, False, False, False))
+
+
+def _synthetic_cases(rng, params, c2g, g2c, tflops=900.0, noise=0.0):
+    """Result-file cases of the single-GPU sweep whose latencies follow the models exactly."""
+    cases = {}
+    for n, c2g_mb, g2c_mb in calibrate.sweep(tflops, c2g[0]):
+        comp = n * calibrate.COMPUTE_M * calibrate.COMPUTE_K / (tflops * 1e12)
+        lat = calibrate.interference_estimate(
+            comp, 0.0, calibrate.cpu_gpu_latency(c2g_mb / 1024, c2g),
+            calibrate.cpu_gpu_latency(g2c_mb / 1024, g2c), params)[0]
+        lat *= 1.0 + noise * rng.standard_normal()
+        cases[calibrate.case_name(n, 0, c2g_mb, g2c_mb)] = {
+            "compute_n": str(n), "gpu_to_gpu_mbytes": "0", "cpu_to_gpu_mbytes": str(c2g_mb),
+            "gpu_to_cpu_mbytes": str(g2c_mb), "latency": f"{lat * 1e3:.6f} ms", "std": "0.0001 ms",
+            "std/mean": "0.0100", "world_size": "1", "intra_group_size": "1", "inter_group_size": "1"}
+    return cases
+
+
+def test_fit_recovers_the_parameters_that_generated_the_data():
+    rng = np.random.default_rng(5)
+    params = np.ones(28)
+    for mask in calibrate.SINGLE_GPU_MASKS:
+        params[calibrate.mask_slice(mask)] = rng.uniform(1.1, 1.9, size=sum(mask))
+    c2g, g2c = (48.0, 12e-6), (52.0, 9e-6)
+    cases = _synthetic_cases(rng, params, c2g, g2c)
+    assert 124 <= len(cases) <= 2 * 15 + 5 ** 3 - 1  # copy-only cases + grid without the empty case
+    out = calibrate.fit(cases)
+    assert np.allclose(out["cpu_gpu_comm_params"], c2g, rtol=1e-3, atol=1e-7)
+    assert np.allclose(out["gpu_cpu_comm_params"], g2c, rtol=1e-3, atol=1e-7)
+    fitted = out["fitted_interference_indices"]
+    assert len(fitted) == 9
+    got = np.array(out["interference_model_params"])
+    assert out["mean_error"] < 2e-3
+    # the prediction is what matters; the factors themselves are recovered where the data
+    # determines them (each resource of a mask is the shortest one in some case)
+    assert np.allclose(got[fitted], params[fitted], rtol=0.05)
+    others = [i for i in range(28) if i not in fitted]
+    assert np.all(got[others] == 1.0)
+    assert len(out["not_measured"]) == 2 and out["overlapped_cases"] > 50
+
+
+def test_fit_tolerates_measurement_noise_and_skips_noisy_cases():
+    rng = np.random.default_rng(6)
+    params = np.ones(28)
+    for mask in calibrate.SINGLE_GPU_MASKS:
+        params[calibrate.mask_slice(mask)] = rng.uniform(1.2, 2.0, size=sum(mask))
+    cases = _synthetic_cases(rng, params, (40.0, 1e-5), (45.0, 1e-5), noise=0.01)
+    first = next(iter(cases))
+    cases[first]["std/mean"] = "0.5000"     # optimize.py:60-65: skipped
+    cases[first]["latency"] = "999 ms"
+    out = calibrate.fit(cases)
+    assert out["mean_error"] < 0.03 and out["cases"] == len(cases) - 1
+    assert abs(out["cpu_gpu_comm_params"][0] - 40.0) < 2.0
+
+
+def test_result_schema_and_errors():
+    assert calibrate.case_name(8, 0, 64, 0) == "N_8-M_4096-K_4096-G2G_0-C2G_64-G2C_0-W_1-Intra_1-Inter_1"
+    assert calibrate._seconds("3.25 ms") == 3.25e-3 and calibrate._seconds("2 s") == 2.0
+    with pytest.raises(ValueError, match="not found"):
+        calibrate.preprocess_data({"x": {
+            "compute_n": "16", "gpu_to_gpu_mbytes": "0", "cpu_to_gpu_mbytes": "64", "gpu_to_cpu_mbytes": "0",
+            "latency": "1 ms", "std": "0 ms", "std/mean": "0.0", "world_size": "1",
+            "intra_group_size": "1", "inter_group_size": "1"}})
+    with pytest.raises(ValueError, match="copy-only"):
+        calibrate.fit_cpu_gpu_params(tuple(np.zeros(0) for _ in range(8)))
+
+
+@pytest.mark.gpu
+def test_measure_and_fit_on_the_gpu():
+    """A reduced sweep on the MI355X: the copy models come out at PCIe-class rates, the fitted
+    model reproduces the overlapped measurements, and the factors stay within their bounds."""
+    cases = calibrate.measure("cuda:0", warmup=3, number=5)
+    assert len(cases) >= 100
+    out = calibrate.fit(cases)
+    print(out)
+    for name in ("cpu_gpu_comm_params", "gpu_cpu_comm_params"):
+        k, b = out[name]
+        assert 5.0 < k < 200.0 and 0.0 <= b < 1e-3, (name, k, b)
+    params = np.array(out["interference_model_params"])
+    assert np.all(params >= 1.0) and np.all(params <= calibrate.UP_BOUND)
+    assert out["overlapped_cases"] > 30 and out["mean_error"] < 0.25

@@ -28,6 +28,8 @@ constexpr int kDpWideTeam = 8;  // lanes that share one DP state in small batche
 constexpr size_t kDpLdsPerCu = 160 * 1024;  // LDS of a gfx950 compute unit
 constexpr int kDpFusedThreads = 1024;  // largest workgroup of the one-launch kernel
 constexpr int kDpStageBatch = 8;   // row minima a lane copies together in the one-launch kernel
+constexpr int kSelectBatch = 8;  // table values a lane of the candidate selection reads together
+constexpr int kSelectBuffer = 4096;  // selected values a workgroup holds before it appends them
 constexpr int kDpBatch = 4;  // end layers whose reads a lane of the one-lane-per-state kernel overlaps
 
 // ------------------------------------------------------------------------------------------
@@ -88,6 +90,11 @@ __global__ __launch_bounds__(256) void select_candidates_kernel(
     const MistDpCosts tabs, const int32_t *__restrict__ rows, const float *__restrict__ lo,
     const float *__restrict__ hi, float *__restrict__ out_values, int32_t *__restrict__ out_request,
     int capacity, int32_t *__restrict__ counts) {
+  // Selected values collect in LDS and leave in one piece: appends to the one output list go
+  // through a single counter, and an atomic per wavefront round (thousands per launch) made
+  // that counter the bottleneck of the kernel.
+  __shared__ float kept[kSelectBuffer];
+  __shared__ int n_kept, flush_at;
   __shared__ int above_of_wave[4];
   const int r = blockIdx.y;
   const int64_t g = rows[r];
@@ -96,32 +103,57 @@ __global__ __launch_bounds__(256) void select_candidates_kernel(
   const float lo_r = lo[r], hi_r = hi[r];
   const int lane = threadIdx.x & 63;
   int above = 0;
-  // every lane of a wavefront runs the same number of rounds (the ballot needs all of them)
-  for (int64_t base = (int64_t)blockIdx.x * blockDim.x; base < n;
-       base += (int64_t)gridDim.x * blockDim.x) {
-    const int64_t e = base + threadIdx.x;
-    float v = INFINITY;
-    if (e < n)
-      v = e < n0 ? tabs.costs[g * n0 + e]
-          : e < n0 + n1 ? tabs.costs_pre[g * n1 + (e - n0)]
-                        : tabs.costs_post[g * n2 + (e - n0 - n1)];
-    const bool finite = v < INFINITY;  // +inf (nothing feasible) and NaN are not candidates
-    above += finite && v > hi_r;
-    const bool take = finite && v > lo_r && v <= hi_r;
-    // one atomic per wavefront reserves the slots of all its selected values
-    const unsigned long long takers = __ballot(take);
-    if (takers != 0) {
-      const int leader = __ffsll(takers) - 1;
-      int first = 0;
-      if (lane == leader) first = atomicAdd(&counts[0], __popcll(takers));
-      first = __shfl(first, leader);
-      const int at = first + __popcll(takers & ((1ull << lane) - 1));
-      if (take && at < capacity) {
-        out_values[at] = v;
+  if (threadIdx.x == 0) n_kept = 0;
+  __syncthreads();
+  auto flush = [&]() {  // called by the whole workgroup
+    if (threadIdx.x == 0) flush_at = n_kept > 0 ? atomicAdd(&counts[0], n_kept) : 0;
+    __syncthreads();
+    for (int i = threadIdx.x; i < n_kept; i += blockDim.x) {
+      const int at = flush_at + i;
+      if (at < capacity) {
+        out_values[at] = kept[i];
         out_request[at] = r;
       }
     }
+    __syncthreads();
+    if (threadIdx.x == 0) n_kept = 0;
+    __syncthreads();
+  };
+  // every workgroup of a request runs the same number of rounds; kSelectBatch values per lane
+  // are read together
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t base = (int64_t)blockIdx.x * blockDim.x; base < n; base += kSelectBatch * stride) {
+    float value[kSelectBatch];
+#pragma unroll
+    for (int u = 0; u < kSelectBatch; ++u) {
+      const int64_t e = base + u * stride + threadIdx.x;
+      value[u] = INFINITY;
+      if (e < n)
+        value[u] = e < n0 ? tabs.costs[g * n0 + e]
+                   : e < n0 + n1 ? tabs.costs_pre[g * n1 + (e - n0)]
+                                 : tabs.costs_post[g * n2 + (e - n0 - n1)];
+    }
+#pragma unroll
+    for (int u = 0; u < kSelectBatch; ++u) {
+      const float v = value[u];
+      const bool finite = v < INFINITY;  // +inf (nothing feasible) and NaN are not candidates
+      above += finite && v > hi_r;
+      const bool take = finite && v > lo_r && v <= hi_r;
+      // one LDS atomic per wavefront reserves the slots of all its selected values
+      const unsigned long long takers = __ballot(take);
+      if (takers != 0) {
+        const int leader = __ffsll(takers) - 1;
+        int first = 0;
+        if (lane == leader) first = atomicAdd(&n_kept, __popcll(takers));
+        first = __shfl(first, leader);
+        if (take) kept[first + __popcll(takers & ((1ull << lane) - 1))] = v;
+      }
+    }
+    __syncthreads();
+    // room for another round of kSelectBatch values per thread?
+    if (n_kept > kSelectBuffer - kSelectBatch * 256) flush();
   }
+  flush();
   // one atomic per workgroup for the "above" count
   for (int step = 32; step >= 1; step >>= 1) above += __shfl_xor(above, step);
   if (lane == 0) above_of_wave[threadIdx.x >> 6] = above;
@@ -790,7 +822,9 @@ int mist_dp_select_candidates(const MistDpCosts *costs, int n_requests, const in
   if (!d_rows || !d_lo || !d_hi || !d_out_values || !d_out_request || !d_counts || capacity <= 0)
     return fail(MIST_E_INVALID, "null pointer / empty output list");
   const int64_t per_row = costs->g_stride[0] + costs->g_stride[1] + costs->g_stride[2];
-  const unsigned blocks = (unsigned)std::min<int64_t>((per_row + 2047) / 2048, 256);
+  // few, long-running workgroups per request: each appends to the output list once per
+  // kSelectBuffer values at most
+  const unsigned blocks = (unsigned)std::min<int64_t>((per_row + 16383) / 16384, 64);
   hipLaunchKernelGGL(select_candidates_kernel, dim3(blocks, n_requests), dim3(256), 0,
                      (hipStream_t)stream, *costs, d_rows, d_lo, d_hi, d_out_values, d_out_request,
                      capacity, d_counts);

@@ -33,6 +33,7 @@ from .intra_tuning import IntraStageTunerOutput
 FIRST_CHUNK = 48  # thresholds per G in the first speculative scan launch
 MAX_CHUNK = 4096  # most thresholds per G in one launch
 GAP = 1e-6        # inter_tuning.py:177
+_SELECT_HEAD = 1 << 16  # selected candidates read back together with their counts
 
 
 def _stream(device) -> ctypes.c_void_p:
@@ -178,18 +179,27 @@ class _DpRunner:
                 counts = torch.zeros(1 + n, dtype=torch.int32, device=dev)
                 values = torch.empty(capacity, dtype=torch.float32, device=dev)
                 request = torch.empty(capacity, dtype=torch.int32, device=dev)
+                # the first values and requests travel with the counts (one read-back when
+                # they are all there is, which is the usual case)
+                head = min(capacity, _SELECT_HEAD)
                 rc = self.lib.mist_dp_select_candidates(
                     ctypes.byref(self._all_costs), n, d_req[0].data_ptr(), d_req[1].data_ptr(),
                     d_req[2].data_ptr(), values.data_ptr(), request.data_ptr(), capacity,
                     counts.data_ptr(), _stream(dev))
                 _lib.check(rc, "mist_dp_select_candidates")
-                h_counts = counts.cpu().numpy()
+                packed = torch.cat([counts.view(torch.float32), values[:head],
+                                    request[:head].view(torch.float32)]).cpu().numpy()
+                h_counts = packed[:1 + n].view(np.int32)
                 total = int(h_counts[0])
                 if total <= capacity:
                     break
                 capacity = self._select_capacity = 2 * total
-            h_values = values[:total].cpu().numpy()
-            h_request = request[:total].cpu().numpy()
+            if total <= head:
+                h_values = packed[1 + n:1 + n + total]
+                h_request = packed[1 + n + head:1 + n + head + total].view(np.int32)
+            else:
+                h_values = values[:total].cpu().numpy()
+                h_request = request[:total].cpu().numpy()
         self.selected += total
         # group by request: 16-bit keys (the entry point takes at most 65535 requests) make the
         # stable sort a radix sort
@@ -230,7 +240,10 @@ class _DpRunner:
             packed[0] = tmax
             packed[1].view(np.int32)[:] = g_index
             d_in = torch.from_numpy(packed).to(dev)
-            d_out = torch.empty((3, n), dtype=torch.float32, device=dev)
+            # outputs and (if asked for) the walked partitions share a buffer: one read-back
+            n_path = n * fam.S_max * 4 if want_path else 0
+            d_all = torch.empty(3 * n + n_path, dtype=torch.float32, device=dev)
+            d_out = d_all[:3 * n].view(3, n)
             n_scratch = self.lib.mist_dp_scratch_floats(ctypes.c_void_p(fam.shape.ctypes.data), n)
             scratch = torch.empty(n_scratch, dtype=torch.float32, device=dev)
             argmin = None
@@ -248,19 +261,18 @@ class _DpRunner:
             _lib.check(rc, "mist_dp_run")
             self.launches += 1
             self.thresholds_run += n
-            path = None
             if want_path:
-                path = torch.empty((n, fam.S_max, 4), dtype=torch.int32, device=dev)
                 rc = self.lib.mist_dp_backtrack(
                     ctypes.c_void_p(fam.shape.ctypes.data), argmin.data_ptr(), d_out[0].data_ptr(),
-                    n, path.data_ptr(), _stream(dev))
+                    n, d_all[3 * n:].data_ptr(), _stream(dev))
                 _lib.check(rc, "mist_dp_backtrack")
-            host = d_out.cpu().numpy()
+            host_all = d_all.cpu().numpy()
+            host = host_all[:3 * n].reshape(3, n)
             out = (host[0].view(np.int32), host[1], host[2])
             if want_argmin:
                 out = out + (argmin.cpu().numpy(),)
             if want_path:
-                out = out + (path.cpu().numpy(),)
+                out = out + (host_all[3 * n:].view(np.int32).reshape(n, fam.S_max, 4),)
         return out
 
     @staticmethod

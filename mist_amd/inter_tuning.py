@@ -687,10 +687,14 @@ def _search(runner: _DpRunner, rows: np.ndarray, Gs: List[int], stats: Optional[
     return [ch["best"] for ch in chains]
 
 
-def _solutions(runner: _DpRunner, results_list, bests, n_g, g_index, q_index, num_layers, slot):
+def _solutions(runner: _DpRunner, results_list, bests, n_g, g_index, q_index, num_layers, slot,
+               only_best=False):
     """Back-pointers of each winning (G, t_max) run (inter_tuning.py:341-355) and the stage
-    strategies that go with them."""
+    strategies that go with them.  ``only_best``: only the instance with the smallest cost (the
+    first of them) gets its solution; the others report their cost with ``None``."""
     winners = [t for t, (_, best_G, _) in enumerate(bests) if best_G is not None]
+    if only_best and winners:
+        winners = [min(winners, key=lambda t: bests[t][0])]  # min() keeps the first of equals
     found = {}
     if winners:
         parts = runner.partitions(
@@ -712,6 +716,9 @@ def _solutions(runner: _DpRunner, results_list, bests, n_g, g_index, q_index, nu
         if best_G is None:
             out.append((float("inf"), None))
             continue
+        if t not in found:
+            out.append((best_cost, None))
+            continue
         total, inter = found[t]
         assert total == best_cost
         solution = [best_G, []]
@@ -732,12 +739,15 @@ def inter_stage_tune_batch(
     slot: int = 0,
     stats: Optional[dict] = None,
     uniform_device: Optional[dict] = None,
+    only_best_solution: bool = False,
 ):
     """``inter_stage_tune`` for several intra-stage results at once (the tensor-parallel
     candidates of one ``tune`` call).  Each entry is searched exactly as if it were alone (its
     own running best, its own stop rule); only the launches are shared.  Returns a list of
     ``(best_cost, best_solution)``.  ``uniform_device`` (``num_nodes``, ``num_gpus_per_node``,
-    ``ckpt_tuning``) selects the recurrence of inter_tuning_uniform_device.py instead."""
+    ``ckpt_tuning``) selects the recurrence of inter_tuning_uniform_device.py instead.
+    ``only_best_solution``: a caller that keeps the best entry only (``tune``) gets the partition
+    and strategies of that entry; the other entries come back as ``(cost, None)``."""
     for r in results_list:
         if not isinstance(r, IntraStageTunerOutput):
             raise TypeError(
@@ -752,6 +762,10 @@ def inter_stage_tune_batch(
             out += inter_stage_tune_batch(num_layers, num_devices, device_mesh_candidates,
                                           gradient_accumulation_steps_candidates, [one], slot, stats,
                                           uniform_device)
+        if only_best_solution:
+            finite = [i for i, (cost, sol) in enumerate(out) if sol is not None]
+            keep = min(finite, key=lambda i: out[i][0]) if finite else None
+            out = [(cost, sol if i == keep else None) for i, (cost, sol) in enumerate(out)]
         return out
     t_start = time.perf_counter()
     first = results_list[0]
@@ -765,7 +779,8 @@ def inter_stage_tune_batch(
     t_0 = time.perf_counter()
     bests = _search(runner, rows, Gs, stats)
     t_2 = time.perf_counter()
-    out = _solutions(runner, results_list, bests, n_g, g_index, q_index, num_layers, slot)
+    out = _solutions(runner, results_list, bests, n_g, g_index, q_index, num_layers, slot,
+                     only_best_solution)
     if stats is not None:
         stats["dp_setup_s"] = stats.get("dp_setup_s", 0.0) + (t_0 - t_start)
         stats["dp_backtrack_s"] = stats.get("dp_backtrack_s", 0.0) + (time.perf_counter() - t_2)

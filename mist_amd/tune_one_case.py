@@ -171,12 +171,13 @@ class PreparedSearch:
         t1 = time.perf_counter()
         if self.granularity == "inter-stage":
             outcomes = inter_stage_tune_batch(
-                self.L, hw.num_nodes * hw.num_gpus_per_node, self.meshes, self.Gs, results, slot=0, stats=stats
+                self.L, hw.num_nodes * hw.num_gpus_per_node, self.meshes, self.Gs, results, slot=0, stats=stats,
+                only_best_solution=True,  # the loop below keeps the first best entry only
             )
         elif self.granularity == "uniform-device-pp":
             outcomes = inter_stage_tune_batch_uniform_device(
                 self.L, hw.num_nodes, hw.num_gpus_per_node, self.meshes, self.Gs, results,
-                self.config, slot=0, stats=stats,
+                self.config, slot=0, stats=stats, only_best_solution=True,
             )
         else:
             outcomes = [

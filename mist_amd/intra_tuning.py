@@ -25,8 +25,8 @@ from .stage_inputs import GroupInputBuilder, make_problem
 SAMPLE_SIZE = 30  # reference default (batched_module_analyzer.py:67)
 VARIANTS = ("", "_with_pre", "_with_post", "_no_pp")
 TARGET_REDUCE_WAVES = 24576  # wavefronts of the reduce kernel the row chunks are sized for
-SCOUT_STAGES = 32      # stages of a group the scout pass of the reduce kernel samples
-MIN_SCOUT_STRIDE = 4   # groups with fewer than SCOUT_STAGES * this many stages get no scout pass
+SCOUT_MIN_STAGES = 128  # groups with fewer stages get no scout pass (0 = never scout)
+SCOUT_MIN_PAIRS = 4     # ... and so do groups with fewer (weight, gradient) offload pairs
 
 
 def alpha_ratios(sample_size: int) -> np.ndarray:
@@ -234,10 +234,11 @@ class IntraStageTuner:
             groups["row_offset"] = np.concatenate(([0], np.cumsum(groups["n_rows"])[:-1]))
             terms_blocks = -(-groups["n_rows"] // _lib.TERMS_BLOCK)
             reduce_blocks = groups["n_chunks"].astype(np.int64) * n_lc_tiles * n_p_tiles
-            # Scout pass: about SCOUT_STAGES evenly spaced stages of each group seed its chunks.
+            # Scout pass: the rows of a group without weight / gradient offloading (one in n_pair)
+            # seed its chunks; groups that are small or have few offload pairs go without.
             n_stages = -(-groups["n_rows"] // _lib.STAGE_ROWS)
-            stride = n_stages // SCOUT_STAGES if SCOUT_STAGES > 0 else np.zeros_like(n_stages)
-            groups["scout_stride"] = np.where(stride >= MIN_SCOUT_STRIDE, stride, 0)
+            scout = (n_stages >= SCOUT_MIN_STAGES) & (groups["n_pair"] >= SCOUT_MIN_PAIRS) & (SCOUT_MIN_STAGES > 0)
+            groups["scout_stride"] = np.where(scout, 1, 0)
             scout_blocks = np.full(len(pending), n_lc_tiles * _lib.SCOUT_SPLIT, dtype=np.int64) * n_p_tiles
             if not np.any(groups["scout_stride"] > 0):
                 scout_blocks[:] = 0

@@ -150,18 +150,19 @@ def test_sample_subset():
     _compare(cfg, tables, 1, S=30, slots=[0])
 
 
-@pytest.mark.parametrize("scout_stages, min_stride", [(1, 1), (3, 1), (7, 2), (0, 1)])
-def test_scout_pass_leaves_results_unchanged(monkeypatch, scout_stages, min_stride):
-    """The scout pass only seeds the chunks with minima of real rows: forcing it on (with
-    different sampling densities) or off must give the oracle's tables, ties included."""
+@pytest.mark.parametrize("min_stages, min_pairs", [(1, 1), (1, 4), (2, 2), (0, 1)])
+def test_scout_pass_leaves_results_unchanged(monkeypatch, min_stages, min_pairs):
+    """The scout pass only seeds the chunks with minima of real rows (those without weight /
+    gradient offloading): forcing it on for small groups or off must give the oracle's tables,
+    ties included."""
     from mist_amd import intra_tuning
 
-    monkeypatch.setattr(intra_tuning, "SCOUT_STAGES", scout_stages)
-    monkeypatch.setattr(intra_tuning, "MIN_SCOUT_STRIDE", min_stride)
+    monkeypatch.setattr(intra_tuning, "SCOUT_MIN_STAGES", min_stages)
+    monkeypatch.setattr(intra_tuning, "SCOUT_MIN_PAIRS", min_pairs)
     cfg, tables = tiny_plan(1, layers=6, hardware__memory_capacity=6.0)
     tuner = _gpu_tuner(cfg, tables, 1)
     strides = tuner.prepare()["groups"]["scout_stride"]
-    assert (strides > 0).any() == (scout_stages > 0)
+    assert (strides > 0).any() == (min_stages > 0)
     _compare(cfg, tables, 1)
     cfg, tables = load_plan(1)
     _compare(cfg, tables, 2)
@@ -218,8 +219,8 @@ def test_randomized_plans_match_oracle(seed, monkeypatch):
     from mist_amd.config import tp_candidates
 
     if seed % 2:  # groups this small get no scout pass by default: force one on every other seed
-        monkeypatch.setattr(intra_tuning, "SCOUT_STAGES", 3)
-        monkeypatch.setattr(intra_tuning, "MIN_SCOUT_STRIDE", 1)
+        monkeypatch.setattr(intra_tuning, "SCOUT_MIN_STAGES", 1)
+        monkeypatch.setattr(intra_tuning, "SCOUT_MIN_PAIRS", 1)
     rng = np.random.default_rng(9000 + seed)
     gg = []
     for _ in range(16):

@@ -569,7 +569,7 @@ __device__ __forceinline__ void take_min(double &best, int32_t &best_row, bool f
 #ifndef MIST_REDUCE_MIN_WAVES
 #define MIST_REDUCE_MIN_WAVES 2
 #endif
-constexpr int kScoutSplit = 4;  // scout workgroups per (group, (l, c) tile, p tile)
+constexpr int kScoutSplit = 2;  // scout workgroups per (group, (l, c) tile, p tile)
 constexpr int kPairFields = 4;  // per-pair table of sieve A: thr_b, thr_o, n_ck, n_nock
 constexpr int kLdsRowStride = MIST_ROW_TERMS + 1;  // odd number of doubles: lanes reading the
                                                    // same term of different rows hit different banks
@@ -642,10 +642,14 @@ struct ReduceRange {
 // workspace order those rows are n_pair positions apart (one per (parallelism row, activation
 // ratio, optimizer ratio)); the scout pass gathers them, n_par * n_oo * n_ao rows per group,
 // and so seeds every chunk with minima that are final for most cells.
+// With scout_stride = m > 1 the rows of m - 1 more pairs, evenly spread up to the last one, follow.
 __device__ __forceinline__ int64_t gathered_position(const MistGroupDesc *g, int64_t q) {
   const int n_tail = g->n_oo * g->n_ao;
-  const int64_t par = q / n_tail, tail = q - par * n_tail;
-  return par * g->n_off + tail * g->n_pair;
+  const int64_t per_pair = (int64_t)g->n_par * n_tail;
+  const int64_t k = q / per_pair, rest = q - k * per_pair;
+  const int64_t par = rest / n_tail, tail = rest - par * n_tail;
+  const int64_t pair = g->scout_stride > 1 ? k * (g->n_pair - 1) / (g->scout_stride - 1) : 0;
+  return par * g->n_off + tail * g->n_pair + pair;
 }
 
 template <bool kPow2G, bool kFirstTile>
@@ -947,7 +951,7 @@ __device__ __forceinline__ void reduce_block(
   // Stages this workgroup visits: every stage_step-th one of its range, without those the scout
   // pass has done.  (skip_stride > 1 goes with stage_step == 1: two skips are never adjacent.)
   const bool gathered = range.gathered != 0;
-  const int64_t n_gather = (int64_t)g->n_par * g->n_oo * g->n_ao;
+  const int64_t n_gather = (int64_t)g->n_par * g->n_oo * g->n_ao * max(g->scout_stride, 1);
   const int64_t end_stage =
       ((gathered ? n_gather : range.row_end) + kStageRows - 1) / kStageRows;
   auto skipped = [&](int64_t st) { return range.skip_stride > 0 && st % range.skip_stride == 0; };

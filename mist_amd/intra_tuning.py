@@ -27,6 +27,8 @@ VARIANTS = ("", "_with_pre", "_with_post", "_no_pp")
 TARGET_REDUCE_WAVES = 24576  # wavefronts of the reduce kernel the row chunks are sized for
 SCOUT_MIN_STAGES = 128  # groups with fewer stages get no scout pass (0 = never scout)
 SCOUT_MIN_PAIRS = 4     # ... and so do groups with fewer (weight, gradient) offload pairs
+SCOUT_PAIRS = 1         # offload pairs whose rows the scout pass gathers: the first, (0, 0), then evenly spread ones
+SCOUT_PAIR_SPAN = 200   # ... one more for every so many pairs of the group (GPT-22B: 421 pairs, 3 gathered)
 
 
 def alpha_ratios(sample_size: int) -> np.ndarray:
@@ -238,7 +240,8 @@ class IntraStageTuner:
             # seed its chunks; groups that are small or have few offload pairs go without.
             n_stages = -(-groups["n_rows"] // _lib.STAGE_ROWS)
             scout = (n_stages >= SCOUT_MIN_STAGES) & (groups["n_pair"] >= SCOUT_MIN_PAIRS) & (SCOUT_MIN_STAGES > 0)
-            groups["scout_stride"] = np.where(scout, 1, 0)
+            pairs = np.minimum(SCOUT_PAIRS + groups["n_pair"] // SCOUT_PAIR_SPAN, groups["n_pair"])
+            groups["scout_stride"] = np.where(scout, pairs, 0)
             scout_blocks = np.full(len(pending), n_lc_tiles * _lib.SCOUT_SPLIT, dtype=np.int64) * n_p_tiles
             if not np.any(groups["scout_stride"] > 0):
                 scout_blocks[:] = 0

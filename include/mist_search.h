@@ -104,8 +104,10 @@ typedef struct MistGroupDesc {
   int32_t n_par, n_pair, n_oo, n_ao, n_off;
   int32_t pp_wre, pp_gre;       /* ZeRO flags of the pre/post layer strategy */
   int32_t rows_per_chunk, n_chunks, n_lc_tiles, n_p_tiles; /* decomposition of the reduce kernel */
-  int32_t scout_stride;         /* reduce kernel: the scout pass visits every scout_stride-th
-                                 * stage of mist_reduce_stage_rows() rows; 0 = no scout pass */
+  int32_t scout_stride;         /* reduce kernel: 0 = no scout pass for this group; m >= 1 = the
+                                 * scout pass reduces the rows of m (weight, gradient) offload
+                                 * pairs: the first one, (0, 0), and m - 1 evenly spread up to
+                                 * the last (n_par * n_oo * n_ao rows each) */
   int64_t n_rows;               /* n_par * n_off */
   int64_t row_offset;           /* first row of this group in the row-term workspace */
   double par[MIST_MAX_PAR][MIST_PAR_FIELDS];
@@ -170,9 +172,11 @@ int mist_row_terms(const MistProblem *problem, const MistGroupDesc *d_groups, in
  * d_block_prefix[n_groups+1]: first workgroup of each group; a group owns
  * n_lc_tiles*n_p_tiles*n_chunks workgroups ordered (chunk, lc_tile, p_tile), p_tile fastest.
  * Optional scout pass (n_scout_blocks > 0): d_scout_prefix[n_groups+1] gives each group
- * n_lc_tiles*n_p_tiles*mist_reduce_scout_split() workgroups that first reduce every
- * scout_stride-th stage of the whole group; every chunk then starts from those minima (they belong to real rows of the group, so
- * the result is unchanged) and lets far fewer rows through to the memory model.
+ * n_lc_tiles*n_p_tiles*mist_reduce_scout_split() workgroups that first reduce the rows of the
+ * group's scout pairs (MistGroupDesc.scout_stride; the search's winners sit almost exclusively
+ * on rows without weight / gradient offloading); every chunk then starts from those minima (they
+ * belong to real rows of the group, so the result is unchanged) and lets far fewer rows through
+ * to the memory model.
  * d_partial_cost / d_partial_index: [n_blocks + n_scout_blocks][2*MIST_P_TILE+2][MIST_LC_TILE];
  * the first n_blocks slabs are the per-chunk results mist_finalize reads. */
 int mist_eval_reduce(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,

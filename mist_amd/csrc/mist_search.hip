@@ -559,7 +559,8 @@ __device__ __forceinline__ void take_min(double &best, int32_t &best_row, bool f
 //   B  lowest improvable slot and the exact memory test at that slot (minima as of stage start:
 //      they only decrease afterwards, so nothing that could matter later is dropped);
 //   C  survivors in row order against the live minima: bisection for `count`, update.
-// A scout pass runs the same code over every scout_stride-th stage of a whole group first; the
+// A scout pass runs the same code over a few gathered rows of a whole group first (those of the
+// group's scout offload pairs, see gathered_position); the
 // main pass starts every chunk from the scout's minima (real rows of the same group, hence valid
 // upper bounds), which removes the warm-up in which a fresh chunk lets most rows through.
 // ------------------------------------------------------------------------------------------
@@ -1134,8 +1135,8 @@ __device__ __forceinline__ void reduce_block(
   out_index[(2 * MIST_P_TILE + 1) * MIST_LC_TILE + threadIdx.x] = row_pp;
 }
 
-// scout != 0: kScoutSplit workgroups per (group, (l, c) tile, p tile) share every
-// scout_stride-th stage of the whole group, results in slab n_blocks + logical workgroup.
+// scout != 0: kScoutSplit workgroups per (group, (l, c) tile, p tile) share the gathered rows
+// of the whole group, results in slab n_blocks + logical workgroup.
 // scout == 0: one workgroup per row chunk of such a tile, seeded from the scout's slabs when the
 // group has them.
 __global__ __launch_bounds__(MIST_LC_TILE, MIST_REDUCE_MIN_WAVES) void eval_reduce_kernel(

@@ -141,6 +141,7 @@ int mist_sizeof_group(void);
 int mist_reduce_p_tile(void); /* MIST_P_TILE the library was built with */
 int mist_reduce_lc_tile(void); /* MIST_LC_TILE the library was built with */
 int mist_reduce_scout_split(void); /* scout workgroups per (group, (l, c) tile, p tile) */
+int mist_workspace_oo_tile(void);  /* optimizer-ratio tile T of the workspace order (mist_row_terms) */
 int mist_terms_block_rows(void); /* candidate rows per workgroup of mist_row_terms */
 int mist_reduce_stage_rows(void); /* rows per LDS stage; rows_per_chunk must be a multiple */
 /* doubles of the stage-summary workspace for `total_rows` workspace rows in `n_groups` groups */
@@ -155,9 +156,11 @@ int64_t mist_stage_floor_doubles(int64_t total_rows, int n_groups);
  * d_block_prefix[n_groups+1]: first workgroup of each group, mist_terms_block_rows() rows per
  * workgroup.
  * d_row_terms: [total_rows][MIST_ROW_TERMS] float64.  Within a group the workspace is ordered
- *   position = ((par * n_ao + ao) * n_oo + oo) * n_pair + pair
- * (rows of similar memory footprint next to each other, which the reduce kernel's per-stage
- * bound relies on for speed, not for correctness); all results carry reference row numbers.
+ *   position = (par * n_ao + ao) * n_oo * n_pair + t * T * n_pair + pair * w + oo % T
+ * with T = mist_workspace_oo_tile(), t = oo / T and w = min(T, n_oo - t * T): per (par, ao) the
+ * optimizer ratios in tiles of T, pair by pair inside a tile (rows of similar latency and memory
+ * footprint next to each other, which the reduce kernel's per-stage bound relies on for speed,
+ * not for correctness); all results carry reference row numbers.
  * d_stage_floor: mist_stage_floor_doubles() float64, written here and read by mist_eval_reduce:
  * per stage of mist_reduce_stage_rows() workspace rows the term-wise minimum of the latency and
  * memory terms (the pseudo row that bounds every row of the stage from below). */

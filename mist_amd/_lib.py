@@ -108,6 +108,7 @@ _SIGNATURES = {
     "mist_sizeof_group": (ctypes.c_int, []),
     "mist_reduce_p_tile": (ctypes.c_int, []),
     "mist_reduce_stage_rows": (ctypes.c_int, []),
+    "mist_workspace_oo_tile": (ctypes.c_int, []),
     "mist_reduce_lc_tile": (ctypes.c_int, []),
     "mist_terms_block_rows": (ctypes.c_int, []),
     "mist_reduce_scout_split": (ctypes.c_int, []),
@@ -134,13 +135,17 @@ _SIGNATURES = {
 
 def workspace_positions(n_par: int, n_pair: int, n_oo: int, n_ao: int) -> np.ndarray:
     """Position in the row-term workspace of every reference row of a group (see
-    include/mist_search.h: the workspace is ordered (par, ao, oo, pair), the reference numbers
-    rows (par, pair, oo, ao))."""
+    include/mist_search.h: per (par, ao) the workspace holds the optimizer ratios in tiles of
+    ``mist_workspace_oo_tile()`` and the pairs inside a tile one after the other; the reference
+    numbers rows (par, pair, oo, ao))."""
+    T = load().mist_workspace_oo_tile()
     n_off = n_pair * n_oo * n_ao
     row = np.arange(n_par * n_off, dtype=np.int64)
     par, off = row // n_off, row % n_off
     pair, oo, ao = off // (n_oo * n_ao), (off // n_ao) % n_oo, off % n_ao
-    return par * n_off + (ao * n_oo + oo) * n_pair + pair
+    tile = oo // T
+    width = np.minimum(T, n_oo - tile * T)
+    return par * n_off + ao * (n_oo * n_pair) + tile * T * n_pair + pair * width + oo % T
 
 
 def exported_symbols():

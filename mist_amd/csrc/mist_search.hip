@@ -176,14 +176,28 @@ __device__ __forceinline__ const MistGroupDesc *find_group(const MistGroupDesc *
 }
 
 // Workspace order.  The reference numbers a group's rows parallelism-major with the activation
-// offload ratio fastest (batched_module_analyzer.py:490-534); the workspace holds them as
-//   position = ((par * n_ao + ao) * n_oo + oo) * n_pair + pair,
-// i.e. rows that are consecutive in memory share the two ratios that move the memory footprint
-// most (activations, optimizer states).  A stage of the reduce kernel then covers rows of
-// similar footprint and one bound per stage prunes most of them.  Results carry row numbers.
+// offload ratio fastest (batched_module_analyzer.py:490-534); the workspace holds them per
+// (parallelism row, activation ratio) in tiles of kOoTile optimizer ratios, and inside a tile
+// pair by pair:
+//   position = (par * n_ao + ao) * n_oo * n_pair + tile * kOoTile * n_pair + pair * width + oo % kOoTile
+// with tile = oo / kOoTile and width = ratios in that tile (kOoTile, fewer in the last one).  A
+// stage of the reduce kernel (64 consecutive positions) then covers 16 neighbouring (weight,
+// gradient) pairs at 4 neighbouring optimizer ratios: rows of similar latency AND footprint, so
+// the stage's term-wise minimum is close to a real row and its bounds prune.  (With all pairs of
+// one optimizer ratio in a run, a stage spanned half of the pair list: its minimum was as fast as
+// the rows without offloading and as small as those with all of it.)  Results carry row numbers.
+constexpr int kOoTile = 4;
+
 struct RowParts {
   int par, pair, oo, ao;
 };
+
+// Position inside the (par, ao) block of n_oo * n_pair rows.
+__device__ __forceinline__ int tile_position(const MistGroupDesc *g, int oo, int pair) {
+  const int tile = oo / kOoTile;
+  const int width = min(kOoTile, g->n_oo - tile * kOoTile);
+  return tile * kOoTile * g->n_pair + pair * width + (oo - tile * kOoTile);
+}
 
 __device__ __forceinline__ RowParts parts_of_position(const MistGroupDesc *g, int64_t pos) {
   RowParts r;
@@ -192,8 +206,11 @@ __device__ __forceinline__ RowParts parts_of_position(const MistGroupDesc *g, in
   const int per_ao = g->n_oo * g->n_pair;
   r.ao = rem / per_ao;
   rem -= r.ao * per_ao;
-  r.oo = rem / g->n_pair;
-  r.pair = rem - r.oo * g->n_pair;
+  const int tile = rem / (kOoTile * g->n_pair);
+  rem -= tile * kOoTile * g->n_pair;
+  const int width = min(kOoTile, g->n_oo - tile * kOoTile);
+  r.pair = rem / width;
+  r.oo = tile * kOoTile + (rem - r.pair * width);
   return r;
 }
 
@@ -209,7 +226,7 @@ __device__ __forceinline__ int64_t position_of_row(const MistGroupDesc *g, int64
   const int pair = off / n_tail;
   const int oo = (off / g->n_ao) % g->n_oo;
   const int ao = off % g->n_ao;
-  return (int64_t)par * g->n_off + ((int64_t)(ao * g->n_oo + oo)) * g->n_pair + pair;
+  return (int64_t)par * g->n_off + (int64_t)ao * g->n_oo * g->n_pair + tile_position(g, oo, pair);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -640,8 +657,8 @@ struct ReduceRange {
 
 // The search's winners sit almost exclusively on rows whose (weight, gradient) offload pair is
 // the first one, (0, 0): 99.8 % of all cells of the GPT-7B plan, 95 % for LLaMA-13B.  In the
-// workspace order those rows are n_pair positions apart (one per (parallelism row, activation
-// ratio, optimizer ratio)); the scout pass gathers them, n_par * n_oo * n_ao rows per group,
+// workspace order those rows are scattered (one per (parallelism row, activation ratio, optimizer
+// ratio)); the scout pass gathers them, n_par * n_oo * n_ao rows per group,
 // and so seeds every chunk with minima that are final for most cells.
 // With scout_stride = m > 1 the rows of m - 1 more pairs, evenly spread up to the last one, follow.
 __device__ __forceinline__ int64_t gathered_position(const MistGroupDesc *g, int64_t q) {
@@ -650,7 +667,8 @@ __device__ __forceinline__ int64_t gathered_position(const MistGroupDesc *g, int
   const int64_t k = q / per_pair, rest = q - k * per_pair;
   const int64_t par = rest / n_tail, tail = rest - par * n_tail;
   const int64_t pair = g->scout_stride > 1 ? k * (g->n_pair - 1) / (g->scout_stride - 1) : 0;
-  return par * g->n_off + tail * g->n_pair + pair;
+  const int ao = (int)(tail / g->n_oo), oo = (int)(tail - (int64_t)ao * g->n_oo);
+  return par * g->n_off + (int64_t)ao * g->n_oo * g->n_pair + tile_position(g, oo, (int)pair);
 }
 
 template <bool kPow2G, bool kFirstTile>
@@ -1380,6 +1398,7 @@ int mist_reduce_stage_rows(void) { return kStageRows; }
 int mist_reduce_lc_tile(void) { return MIST_LC_TILE; }
 int mist_terms_block_rows(void) { return kTermsBlock; }
 int mist_reduce_scout_split(void) { return kScoutSplit; }
+int mist_workspace_oo_tile(void) { return kOoTile; }
 int64_t mist_stage_floor_doubles(int64_t total_rows, int n_groups) {
   if (total_rows < 0 || n_groups < 0) return -1;
   return (total_rows / kStageRows + n_groups + 1) * kStageFloorPitch;

@@ -149,8 +149,9 @@ def workspace_positions(n_par: int, n_pair: int, n_oo: int, n_ao: int) -> np.nda
 
 
 def exported_symbols():
-    """Names every entry point declared in include/mist_search.h, mist_dp.h and mist_mip.h."""
-    return tuple(_SIGNATURES) + tuple(_DP_SIGNATURES) + tuple(_MIP_SIGNATURES)
+    """Names every entry point declared in include/mist_search.h, mist_dp.h, mist_mip.h and
+    mist_inter.h."""
+    return tuple(_SIGNATURES) + tuple(_DP_SIGNATURES) + tuple(_MIP_SIGNATURES) + tuple(_INTER_SIGNATURES)
 
 
 DP_SHAPE_DTYPE = np.dtype(
@@ -233,6 +234,13 @@ class MipTables(ctypes.Structure):
     _fields_ = [("stable", ctypes.c_void_p * 4), ("delta", ctypes.c_void_p * 4)]
 
 
+_INTER_SIGNATURES = {
+    "mist_inter_stage_search": (
+        ctypes.c_int,
+        [_VP, ctypes.POINTER(DpCosts), ctypes.c_int, ctypes.c_int, _VP, _VP, ctypes.c_int,
+         _VP, _VP, _VP, _VP, _VP, _VP, _VP]),
+}
+
 _MIP_SIGNATURES = {
     "mist_sizeof_mip_shape": (ctypes.c_int, []),
     "mist_mip_stage_samples": (
@@ -258,7 +266,8 @@ def load():
             "(there is no CPU fallback for the search kernels)"
         )
     lib = ctypes.CDLL(LIB_PATH)
-    for name, (restype, argtypes) in {**_SIGNATURES, **_DP_SIGNATURES, **_MIP_SIGNATURES}.items():
+    for name, (restype, argtypes) in {**_SIGNATURES, **_DP_SIGNATURES, **_MIP_SIGNATURES,
+                                      **_INTER_SIGNATURES}.items():
         fn = getattr(lib, name)
         fn.restype = restype
         fn.argtypes = argtypes

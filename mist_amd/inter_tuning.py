@@ -34,6 +34,7 @@ FIRST_CHUNK = 48  # thresholds per G in the first speculative scan launch
 MAX_CHUNK = 4096  # most thresholds per G in one launch
 GAP = 1e-6        # inter_tuning.py:177
 _SELECT_HEAD = 1 << 16  # selected candidates read back together with their counts
+NATIVE_SEARCH = True     # per-mesh search through mist_inter_stage_search (False: the Python driver below)
 
 
 def _stream(device) -> ctypes.c_void_p:
@@ -324,17 +325,22 @@ class _DpRunner:
         for total, found in best:
             assert found is not None
             fam, n_stages, path = found
-            stages = path[:n_stages].tolist()
-            cl, cd, inter = 0, fam.D, []
-            for end, n_, m_, ckpt in stages:
-                assert end >= cl, "back-pointer walk left the DP's states"
-                inter.append(((cl, end), (n_, m_), ckpt))
-                cl = end + 1
-                if fam.consumes_devices:
-                    cd -= n_ * m_
-            assert len(inter) == n_stages and cl == fam.L and (cd == 0 or not fam.consumes_devices)
-            out.append((total, inter))
+            out.append(self._partition_of(total, fam, n_stages, path))
         return out
+
+    @staticmethod
+    def _partition_of(total, fam, n_stages, path):
+        """``(total, [((l0, l1), (n, m), ckpt), ...])`` from a walked path (mist_dp_backtrack)."""
+        stages = path[:n_stages].tolist()
+        cl, cd, inter = 0, fam.D, []
+        for end, n_, m_, ckpt in stages:
+            assert end >= cl, "back-pointer walk left the DP's states"
+            inter.append(((cl, end), (n_, m_), ckpt))
+            cl = end + 1
+            if fam.consumes_devices:
+                cd -= n_ * m_
+        assert len(inter) == n_stages and cl == fam.L and (cd == 0 or not fam.consumes_devices)
+        return total, inter
 
 
 def _gap_reached(a: np.ndarray, b: np.ndarray) -> np.ndarray:
@@ -730,6 +736,67 @@ def _solutions(runner: _DpRunner, results_list, bests, n_g, g_index, q_index, nu
     return out
 
 
+def _native_search(runner: _DpRunner, results_list, rows, Gs, n_g, g_index, q_index, num_layers,
+                   slot, only_best, stats):
+    """The search of ``_search`` + the partitions of ``_solutions`` in one library call
+    (``mist_inter_stage_search``: the same steps without the interpreter between the dependent
+    GPU batches); the strategy rows of the stages are read back here."""
+    fam = runner.families[0]
+    n_inst = len(results_list)
+    rows = np.ascontiguousarray(rows, dtype=np.int32)
+    G_arr = np.array(Gs, dtype=np.int32)
+    cost = np.empty(n_inst, dtype=np.float64)
+    best_g = np.empty(n_inst, dtype=np.int32)
+    best_t = np.empty(n_inst, dtype=np.float32)
+    n_stages = np.empty(n_inst, dtype=np.int32)
+    path = np.empty((n_inst, fam.S_max, 4), dtype=np.int32)
+    counters = np.zeros(4, dtype=np.int64)
+    t_0 = time.perf_counter()
+    with torch.cuda.device(runner.device):
+        rc = runner.lib.mist_inter_stage_search(
+            ctypes.c_void_p(fam.shape.ctypes.data), ctypes.byref(fam.costs_struct), n_inst, len(Gs),
+            ctypes.c_void_p(rows.ctypes.data), ctypes.c_void_p(G_arr.ctypes.data),
+            1 if only_best else 0, ctypes.c_void_p(cost.ctypes.data),
+            ctypes.c_void_p(best_g.ctypes.data), ctypes.c_void_p(best_t.ctypes.data),
+            ctypes.c_void_p(n_stages.ctypes.data), ctypes.c_void_p(path.ctypes.data),
+            ctypes.c_void_p(counters.ctypes.data), _stream(runner.device))
+    _lib.check(rc, "mist_inter_stage_search")
+    t_1 = time.perf_counter()
+    partitions = {}
+    requests = []
+    for t in range(n_inst):
+        if best_g[t] < 0 or n_stages[t] <= 0:
+            continue
+        total, inter = _DpRunner._partition_of(float(cost[t]), fam, int(n_stages[t]), path[t])
+        partitions[t] = inter
+        g = g_index[Gs[int(best_g[t])]]
+        for i, ((l0, l1), (n, m), ckpt) in enumerate(inter):
+            variant, cell = _solution_cell(num_layers, g, len(inter) - i - 1, l0, l1, q_index[(n, m)], ckpt, slot)
+            requests.append((results_list[t], variant, cell))
+    strategy_rows = iter(IntraStageTunerOutput.solutions_at(requests)) if requests else iter(())
+    out = []
+    for t in range(n_inst):
+        if best_g[t] < 0:
+            out.append((float("inf"), None))
+        elif t not in partitions:
+            out.append((float(cost[t]), None))
+        else:
+            solution = [Gs[int(best_g[t])], []]
+            for (l0, l1), (n, m), ckpt in partitions[t]:
+                row = next(strategy_rows).tolist()
+                row[:6] = [int(x) for x in row[:6]]
+                solution[1].append((((l0, l1), (n, m), ckpt, 0), tuple(row)))
+            out.append((float(cost[t]), solution))
+    if stats is not None:
+        stats["dp_search_s"] = stats.get("dp_search_s", 0.0) + (t_1 - t_0)
+        stats["dp_backtrack_s"] = stats.get("dp_backtrack_s", 0.0) + (time.perf_counter() - t_1)
+        stats["dp_launches"] = stats.get("dp_launches", 0) + int(counters[0])
+        stats["dp_window_fetches"] = stats.get("dp_window_fetches", 0) + int(counters[1])
+        stats["dp_window_values"] = stats.get("dp_window_values", 0) + int(counters[2])
+        stats["dp_thresholds"] = stats.get("dp_thresholds", 0) + int(counters[3])
+    return out
+
+
 def inter_stage_tune_batch(
     num_layers: int,
     num_devices: int,
@@ -777,6 +844,12 @@ def inter_stage_tune_batch(
     # table row of (instance, G)
     rows = np.array([[t * n_g + g_index[G] for G in Gs] for t in range(len(results_list))], dtype=np.int32)
     t_0 = time.perf_counter()
+    if uniform_device is None and NATIVE_SEARCH:
+        out = _native_search(runner, results_list, rows, Gs, n_g, g_index, q_index, num_layers, slot,
+                             only_best_solution, stats)
+        if stats is not None:
+            stats["dp_setup_s"] = stats.get("dp_setup_s", 0.0) + (t_0 - t_start)
+        return out
     bests = _search(runner, rows, Gs, stats)
     t_2 = time.perf_counter()
     out = _solutions(runner, results_list, bests, n_g, g_index, q_index, num_layers, slot,

@@ -465,3 +465,40 @@ def test_groups_without_candidates_stay_empty():
     from oracle.intra import intra_stage_tune
     want = intra_stage_tune(tables, cfg, 4, meshes, Gs, 2, 1)
     assert np.array_equal(got.indices, want.indices)
+
+
+@pytest.mark.parametrize("plan, overrides", [
+    (1, {}), (2, {}), (3, {}),
+    (1, dict(model__num_hidden_layers=6, hardware__memory_capacity=6.0)),
+    (1, dict(model__num_hidden_layers=7, hardware__num_gpus_per_node=4, training__global_batch_size=16)),
+    (1, dict(model__num_hidden_layers=5, hardware__memory_capacity=1.0)),  # nothing fits
+])
+def test_native_search_equals_python_driver(monkeypatch, plan, overrides):
+    """``mist_inter_stage_search`` (the search without the interpreter between the GPU batches)
+    against the Python driver it mirrors: cost of every tensor-parallel entry, partitions and
+    strategies, and the same number of DP instances and batches (the two make the same
+    speculation decisions)."""
+    from mist_amd import inter_tuning
+    from mist_amd.config import tp_candidates
+    from mist_amd.intra_tuning import IntraStageTuner
+    from mist_amd.search_space import _get_device_mesh_candidates, _get_grad_accumu_steps_candidates
+
+    cfg, tables = load_plan(plan, **overrides)
+    hw, L = cfg.hardware, cfg.model.num_hidden_layers
+    D = hw.num_nodes * hw.num_gpus_per_node
+    meshes = _get_device_mesh_candidates(hw.num_nodes, hw.num_gpus_per_node, False)
+    Gs = _get_grad_accumu_steps_candidates(cfg.training.global_batch_size)
+    results = IntraStageTuner(tables, L, meshes, Gs, tp_candidates(cfg), cfg, sample_size=1).tune_all()
+    out = {}
+    for native in (True, False):
+        monkeypatch.setattr(inter_tuning, "NATIVE_SEARCH", native)
+        for only_best in (False, True):
+            stats = {}
+            got = inter_tuning.inter_stage_tune_batch(L, D, meshes, Gs, results, stats=stats,
+                                                      only_best_solution=only_best)
+            out[native, only_best] = (got, stats["dp_thresholds"], stats["dp_launches"],
+                                      stats["dp_window_values"])
+    for only_best in (False, True):
+        assert out[True, only_best] == out[False, only_best]
+    assert any(sol is not None for _, sol in out[True, False][0]) == (plan != 1 or overrides.get("hardware__memory_capacity") != 1.0)
+

@@ -182,7 +182,7 @@ def test_mip_layer_candidates_match_oracle():
 
 def _declared_functions():
     names = []
-    for header in ("mist_search.h", "mist_dp.h", "mist_mip.h"):
+    for header in ("mist_search.h", "mist_dp.h", "mist_mip.h", "mist_inter.h"):
         text = open(os.path.join(REPO, "include", header)).read()
         text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
         names += re.findall(r"\b(mist_[a-z0-9_]+)\s*\(", text)
@@ -235,6 +235,24 @@ def test_argument_checks_reject_before_any_launch():
     assert lib.mist_dp_run(sp, ctypes.byref(costs), fake, fake, 1, 7, fake, fake, fake, None, fake, None) == -1
     assert lib.mist_dp_backtrack(sp, None, fake, 1, fake, None) == -1
     assert lib.mist_dp_backtrack(sp, fake, fake, 0, fake, None) == -1
+    # the search driver checks its arguments before it touches the GPU
+    shape_ok = np.zeros(1, dtype=_lib.DP_SHAPE_DTYPE)
+    shape_ok["num_layers"], shape_ok["num_devices"], shape_ok["num_mesh"], shape_ok["p_dim"] = 8, 8, 2, 4
+    shape_ok["max_stages"] = 4
+    shape_ok["mesh_n"][0, :2], shape_ok["mesh_m"][0, :2] = [1, 1], [1, 2]
+    so = ctypes.c_void_p(shape_ok.ctypes.data)
+    one = np.ones(1, dtype=np.int32)
+    op = ctypes.c_void_p(one.ctypes.data)
+    search = lambda shape_ptr, n_inst, n_g, G: lib.mist_inter_stage_search(
+        shape_ptr, ctypes.byref(costs), n_inst, n_g, op, G, 0, fake, fake, fake, fake, fake, None, None)
+    assert search(so, 0, 1, op) == -1
+    assert search(so, 1, 1, ctypes.c_void_p(np.zeros(1, dtype=np.int32).ctypes.data)) == -1
+    assert b"grad_accum" in lib.mist_last_error()
+    assert search(None, 1, 1, op) == -1
+    free = shape_ok.copy()
+    free["free_devices"], free["num_devices"], free["num_mesh"] = 1, 0, 1
+    assert search(ctypes.c_void_p(free.ctypes.data), 1, 1, op) == -1
+    assert b"per-mesh" in lib.mist_last_error()
     # re-laid row minima: max_stages * Q * L (L + 1) / 2 floats per g
     assert lib.mist_dp_stage_minima_floats(sp) == 4 * 2 * (80 * 81 // 2)
     assert lib.mist_dp_stage_minima_floats(ctypes.c_void_p(np.zeros(1, dtype=_lib.DP_SHAPE_DTYPE).ctypes.data)) == -1

@@ -27,6 +27,7 @@ constexpr int kDpThreads = 64;  // one wavefront per workgroup
 constexpr int kDpWideTeam = 8;  // lanes that share one DP state in small batches
 constexpr size_t kDpLdsPerCu = 160 * 1024;  // LDS of a gfx950 compute unit
 constexpr int kDpFusedThreads = 1024;  // largest workgroup of the one-launch kernel
+constexpr int kDpFusedMinInstances = 64;  // threshold batches of at least this size use it
 constexpr int kDpStageBatch = 8;   // row minima a lane copies together in the one-launch kernel
 constexpr int kSelectBatch = 8;  // table values a lane of the candidate selection reads together
 constexpr int kSelectBuffer = 4096;  // selected values a workgroup holds before it appends them
@@ -864,7 +865,10 @@ int mist_dp_run(const MistDpShape *shape, const MistDpCosts *costs, const float 
       ((size_t)4 * plane + (size_t)6 * (shape->num_devices + 1) +
        (size_t)shape->num_mesh * dp_triangle(shape->num_layers)) *
       sizeof(float);
-  if (!wide && costs->stage_min != nullptr && fused_lds <= fused_lds_limit(mode)) {
+  // (threshold batches from about 64 instances on: a workgroup's run through all stage counts
+  // takes as long as the 1 + max_stages launches of a few dozen instances)
+  const bool fused_pays = mode == MIST_DP_THRESHOLD ? n_tmax >= kDpFusedMinInstances : !wide;
+  if (fused_pays && costs->stage_min != nullptr && fused_lds <= fused_lds_limit(mode)) {
     // one workgroup per CU when the planes take more than half of the LDS: then a larger one
     const int most = 2 * fused_lds > kDpLdsPerCu ? kDpFusedThreads : kDpFusedThreads / 2;
     const int threads = std::min(most, (plane + 63) / 64 * 64);

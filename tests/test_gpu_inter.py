@@ -205,6 +205,33 @@ def test_tune_end_to_end_matches_oracle(overrides):
     assert got_sol == want_sol
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_randomized_tune_end_to_end_matches_oracle(seed):
+    """Seeded random tiny plans through the whole tuner (intra-stage kernels, the search driver
+    in the library, back-pointers, strategy read-back) against the oracle's tune: hardware
+    coefficients, interference factors, memory capacity, cluster shape, batch size and layer count
+    are drawn at random, so the scan meets different bottlenecks, window widths and stop points."""
+    from mist_amd.tune_one_case import tune
+    from oracle.tune import tune as oracle_tune
+
+    rng = np.random.default_rng(4200 + seed)
+    gg = []
+    for _ in range(16):
+        gg += [float(rng.uniform(8, 500)), float(rng.uniform(2e-6, 8e-5))]
+    nodes, gpn = [(1, 2), (1, 4), (2, 2), (2, 4), (1, 8), (2, 4)][seed]
+    overrides = dict(
+        hardware__gpu_gpu_comm_params=gg,
+        hardware__interference_model_params=[float(x) for x in rng.uniform(1.0, 3.0, size=28)],
+        hardware__memory_capacity=float(rng.choice([3.0, 5.0, 8.0, 16.0])),
+        hardware__num_nodes=nodes, hardware__num_gpus_per_node=gpn,
+        training__global_batch_size=int(rng.choice([16, 32, 64])),
+    )
+    cfg, tables = tiny_plan(1, layers=int(rng.integers(5, 10)), **overrides)
+    got = tune(cfg)
+    want = oracle_tune(cfg, tables)
+    assert got == want
+
+
 def test_plan1_end_to_end():
     from mist_amd.tune_one_case import tune
     from oracle.tune import tune as oracle_tune

@@ -46,9 +46,10 @@ def reduce_kernel_flops(plan, L):
     return 15 * rows * L + 22 * rows * pairs + (30 + 12) * cells + (25 + 10) * rows * pairs
 
 
-def cpu_baseline(cfg, tables, budget_s=20.0):
+def cpu_baseline(cfg, tables, budget_s=15.0):
     """Times the numpy oracle (a port of the reference's formulation, single thread) on whole
-    (G, mesh, tp) groups of the same plan, smallest first, until ``budget_s`` is used."""
+    (G, mesh, tp) groups of the same plan (single-device mesh, about 9 s each) until ``budget_s``
+    is used."""
     from mist_amd.search_space import _get_device_mesh_candidates, _get_grad_accumu_steps_candidates
     from oracle.intra import max_pre_saved_micro_batches
     from oracle.stage import batched_tune_best_latency_for_stage
@@ -58,7 +59,7 @@ def cpu_baseline(cfg, tables, budget_s=20.0):
     meshes = _get_device_mesh_candidates(hw.num_nodes, hw.num_gpus_per_node, False)
     Gs = _get_grad_accumu_steps_candidates(cfg.training.global_batch_size)
     P = max_pre_saved_micro_batches(meshes, Gs, L)
-    sample = [(512, (1, 1), 1), (256, (1, 2), 1), (128, (1, 4), 1)]
+    sample = [(512, (1, 1), 1), (256, (1, 1), 1), (128, (1, 1), 1), (64, (1, 1), 1)]
     done, cand, cells, elapsed = [], 0, 0, 0.0
     for G, (n, m), tp in sample:
         dbg = {}

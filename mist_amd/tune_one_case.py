@@ -163,11 +163,17 @@ class PreparedSearch:
         groups = len(g)
         return dict(rows=rows, candidates=rows * (L + 1), cells=cells, groups=groups)
 
-    def run(self, stats: Optional[dict] = None):
+    def run(self, stats: Optional[dict] = None, split_timing: bool = False):
+        """``split_timing`` waits for the intra-stage kernels before the inter-stage search
+        starts, so that ``stats['intra_launch_s']`` and ``stats['inter_s']`` are the wall times
+        of the two halves (otherwise the first is launch time only and the second includes the
+        wait for the kernels)."""
         stats = {} if stats is None else stats
         hw = self.config.hardware
         t0 = time.perf_counter()
         results = self.tuner.run_prepared(self.plan, self.dev_plan)
+        if split_timing:
+            torch.cuda.synchronize(self.tuner.device)
         t1 = time.perf_counter()
         if self.granularity == "inter-stage":
             outcomes = inter_stage_tune_batch(

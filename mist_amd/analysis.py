@@ -75,6 +75,7 @@ def analyze_cells(config: MistConfig, tables: LayerTables, stages, device: str =
             if not (1 <= l <= L and 0 <= c <= l and p >= 0):
                 raise ValueError(f"cell (p={p}, l={l}, c={c}) outside 1 <= l <= {L}, 0 <= c <= l, p >= 0")
             requests.append((gi, 0, l, c, p))
+    builder.validate(groups)
     if not requests:
         return [({} if i in live else None) for i in range(len(stages))]
     problem = make_problem(config, L, 1, 1, 1, len(live))

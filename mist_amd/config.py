@@ -189,8 +189,10 @@ class MistConfig:
 
     @classmethod
     def from_yaml(cls, path: str) -> "MistConfig":
+        # the C parser of PyYAML when the installation has it (same documents, ~10x faster)
+        loader = getattr(yaml, "CSafeLoader", yaml.SafeLoader)
         with open(path) as f:
-            return cls(yaml.safe_load(f))
+            return cls(yaml.load(f, Loader=loader))
 
     def raw(self) -> Dict[str, Any]:
         return copy.deepcopy(self._original_config)

@@ -221,6 +221,7 @@ class IntraStageTuner:
         groups = np.zeros(len(pending), dtype=_lib.GROUP_DTYPE)
         for i, (g, q, n, m, G, num_p, space) in enumerate(pending):
             builder.fill(groups[i], space, g, q, n, m, G, num_p)
+        builder.validate(groups)
 
         n_pairs = L * (L + 1) // 2 + L
         n_lc_tiles = -(-n_pairs // _lib.LC_TILE)

@@ -148,29 +148,44 @@ def create_search_space_for_a_block_layer(
             par.append((batch_size, dp_size, tp_size, wre, gre, ore))
     par_np = np.array(par, dtype=np.float64).reshape(-1, 6)
 
-    dense = tuple(tuning.offloading_ratio_candidates)
-    sparse = tuple(tuning.sparse_offloading_ratio_candidates)
-    if tuning.state_offloading_enabled:
+    wo, go, oo, ao, pair_wo, pair_go = _offload_lists(
+        bool(tuning.state_offloading_enabled), bool(tuning.activation_offloading_enabled),
+        tuple(tuning.offloading_ratio_candidates), tuple(tuning.sparse_offloading_ratio_candidates),
+        bool(getattr(config, "disable_wo_tuning", False)), bool(getattr(config, "disable_go_tuning", False)),
+        bool(getattr(config, "disable_oo_tuning", False)),
+        *(getattr(config, f"fixed_{k}_ratio", None) for k in ("wo", "go", "oo", "ao")),
+    )
+    if par_np.shape[0] > MAX_PAR:
+        raise ValueError(f"{par_np.shape[0]} parallelism rows; at most {MAX_PAR} are supported")
+    return SearchSpace(par=par_np, wo=wo, go=go, oo=oo, ao=ao, pair_wo=pair_wo, pair_go=pair_go)
+
+
+@lru_cache(maxsize=64)
+def _offload_lists(state_offloading, activation_offloading, dense, sparse, disable_wo, disable_go,
+                   disable_oo, fixed_wo, fixed_go, fixed_oo, fixed_ao):
+    """Ratio lists and valid (wo, go) pairs of a configuration (batched_module_analyzer.py:
+    487-531); they do not depend on the group, so the 100+ groups of a plan share one result
+    (the index arrays are read-only)."""
+    if state_offloading:
         wo, go, oo = sparse, sparse, dense
-        if getattr(config, "disable_wo_tuning", False):
+        if disable_wo:
             wo = (0.0,)
-        if getattr(config, "disable_go_tuning", False):
+        if disable_go:
             go = (0.0,)
-        if getattr(config, "disable_oo_tuning", False):
+        if disable_oo:
             oo = (0.0,)
     else:
         wo, go, oo = (0.0,), (0.0,), (0.0,)
-    fixed = {k: getattr(config, f"fixed_{k}_ratio", None) for k in ("wo", "go", "oo", "ao")}
-    if fixed["wo"] is not None:
-        wo = (float(fixed["wo"]),)
-    if fixed["go"] is not None:
-        go = (float(fixed["go"]),)
-    if fixed["oo"] is not None:
-        oo = (float(fixed["oo"]),)
-    if tuning.activation_offloading_enabled:
+    if fixed_wo is not None:
+        wo = (float(fixed_wo),)
+    if fixed_go is not None:
+        go = (float(fixed_go),)
+    if fixed_oo is not None:
+        oo = (float(fixed_oo),)
+    if activation_offloading:
         ao = dense
-    elif fixed["ao"] is not None:
-        ao = (float(fixed["ao"]),)
+    elif fixed_ao is not None:
+        ao = (float(fixed_ao),)
     else:
         ao = (0.0,)
 
@@ -179,15 +194,9 @@ def create_search_space_for_a_block_layer(
     for name, values in (("wo", wo), ("go", go), ("oo", oo), ("ao", ao)):
         if len(values) > MAX_RATIOS:
             raise ValueError(f"{name} ratio list has {len(values)} values; at most {MAX_RATIOS}")
-    if par_np.shape[0] > MAX_PAR:
-        raise ValueError(f"{par_np.shape[0]} parallelism rows; at most {MAX_PAR} are supported")
     assert len(pair_wo) <= MAX_PAIRS
-    return SearchSpace(
-        par=par_np,
-        wo=tuple(float(x) for x in wo),
-        go=tuple(float(x) for x in go),
-        oo=tuple(float(x) for x in oo),
-        ao=tuple(float(x) for x in ao),
-        pair_wo=np.array(pair_wo, dtype=np.uint8),
-        pair_go=np.array(pair_go, dtype=np.uint8),
-    )
+    pair_wo_np, pair_go_np = np.array(pair_wo, dtype=np.uint8), np.array(pair_go, dtype=np.uint8)
+    pair_wo_np.setflags(write=False)
+    pair_go_np.setflags(write=False)
+    return (tuple(float(x) for x in wo), tuple(float(x) for x in go), tuple(float(x) for x in oo),
+            tuple(float(x) for x in ao), pair_wo_np, pair_go_np)

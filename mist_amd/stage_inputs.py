@@ -167,6 +167,8 @@ class GroupInputBuilder:
         self.hw = config.hardware
         self._exec = lru_cache(maxsize=None)(self._exec_uncached)
         self._block = lru_cache(maxsize=None)(self._block_uncached)
+        self._par_fields = lru_cache(maxsize=None)(self._par_fields_uncached)
+        self._pre_post = lru_cache(maxsize=None)(self._pre_post_uncached)
 
     def _exec_uncached(self, kind, b, tp, inter, intra, G):
         return latency_exec(self.tables, kind, b, tp, inter, intra, G)
@@ -197,6 +199,20 @@ class GroupInputBuilder:
             gcb=gcb,
         )
 
+    def _par_fields_uncached(self, b: int, tp: int, gpus_per_node: int, grad_accum: int) -> np.ndarray:
+        """The table look-ups of a parallelism row (``MIST_PAR_*`` fields from W on; the six
+        strategy fields in front stay zero) - the same (b, tp) recurs in most groups of a plan."""
+        P, m = _lib.PAR, gpus_per_node
+        v = np.zeros(_lib.PAR_FIELDS, dtype=np.float64)
+        for name, value in self._block(b, tp).items():
+            v[P[name]] = value
+        inter = tp // m if tp > m else 1
+        intra = m if tp > m else tp
+        fwd, bwd, efwd, ebwd = self._exec("block", b, tp, inter, intra, grad_accum)
+        v[P["exec_fwd"]], v[P["exec_bwd"]] = fwd, bwd
+        v[P["extra_fwd"]], v[P["extra_bwd"]] = efwd, ebwd
+        return v
+
     def _gpu_gpu(self, op_name: str, mbytes: float, dp: int, num_nodes: int) -> float:
         inter = num_nodes if dp > num_nodes else dp
         intra = dp // num_nodes if dp > num_nodes else 1
@@ -211,7 +227,8 @@ class GroupInputBuilder:
         self, rec: np.void, space: SearchSpace, g_index: int, q_index: int, num_nodes: int,
         num_gpus_per_node: int, grad_accum: int, num_p: int, analysis_row=None,
     ) -> None:
-        """Fills one record of a ``GROUP_DTYPE`` array (decomposition fields are set later)."""
+        """Fills one record of a ``GROUP_DTYPE`` array (decomposition fields are set later; the
+        caller runs ``validate`` over the filled records)."""
         cfg, t = self.config, self.tables
         n, m, G = num_nodes, num_gpus_per_node, grad_accum
         rec["g_index"], rec["q_index"] = g_index, q_index
@@ -228,21 +245,23 @@ class GroupInputBuilder:
         rec["pair_go"][: space.n_pair] = space.pair_go
 
         # ---- parallelism rows: table look-ups at (b, tp) ----
-        P = _lib.PAR
-        for i in range(space.n_par):
-            b, dp, tp = (int(v) for v in space.par[i, :3])
-            row = rec["par"][i]
-            row[:6] = space.par[i]
-            blk = self._block(b, tp)
-            for name in ("W", "G", "O", "raw_ck", "raw_nock", "fwd_peak", "bwd_peak", "out", "gcb"):
-                row[P[name]] = blk[name]
-            inter = tp // m if tp > m else 1
-            intra = m if tp > m else tp
-            fwd, bwd, efwd, ebwd = self._exec("block", b, tp, inter, intra, G)
-            row[P["exec_fwd"]], row[P["exec_bwd"]] = fwd, bwd
-            row[P["extra_fwd"]], row[P["extra_bwd"]] = efwd, ebwd
+        if space.n_par:
+            rows = np.stack([self._par_fields(int(r[0]), int(r[2]), m, G) for r in space.par])
+            rows[:, :6] = space.par
+            rec["par"][: space.n_par] = rows
 
-        # ---- pre / post layers ----
+        # ---- pre / post layers: the same for every tp candidate of a (mesh, G) ----
+        if analysis_row is None:
+            fields = self._pre_post(n, m, G)
+        else:
+            fields = self._pre_post_uncached(n, m, G, analysis_row)
+        for name, value in fields.items():
+            rec[name] = value
+
+    def _pre_post_uncached(self, n: int, m: int, G: int, analysis_row=None) -> dict:
+        """``MistGroupDesc`` fields of the pre and post layers of a (mesh, G) group."""
+        cfg, t = self.config, self.tables
+        rec = {}
         pp_dp, pp_tp, pp_wre, pp_gre, pp_ore, pp_wo, pp_go, pp_oo, _pp_ac = pre_post_strategy_fields(
             cfg, n, m, analysis_row
         )
@@ -282,22 +301,24 @@ class GroupInputBuilder:
             rec["post_ag"] = self._gpu_gpu("all_gather", post_W, pp_dp, n)
             rec["pre_rs"] = self._gpu_gpu("reduce_scatter", pre_G, pp_dp, n)
             rec["post_rs"] = self._gpu_gpu("reduce_scatter", post_G, pp_dp, n)
-        self._validate(rec, space)
+        return rec
 
     @staticmethod
-    def _validate(rec: np.void, space: SearchSpace) -> None:
+    def validate(recs: np.ndarray) -> None:
         """The reduce kernel prunes with bounds that rely on every memory and latency input being
         finite and non-negative and on ratios in [0, 1] (then peaks are monotone in the number of
         pre-saved micro-batches and in every row term).  Real tables always are; a violation is
-        rejected here instead of silently changing which rows get evaluated."""
-        par = rec["par"][: space.n_par]
+        rejected here instead of silently changing which rows get evaluated.  ``recs``: filled
+        ``GROUP_DTYPE`` records (unused array slots hold zero)."""
+        par = recs["par"]
         if not np.all(np.isfinite(par)) or np.any(par < 0):
             raise ValueError("layer table values must be finite and non-negative")
         for name in ("wo", "go", "oo", "ao"):
-            v = np.asarray(getattr(space, name), dtype=np.float64)
-            if np.any(~np.isfinite(v)) or np.any(v < 0) or np.any(v > 1):
-                raise ValueError(f"offload ratios '{name}' must lie in [0, 1], got {v}")
-        for name in rec.dtype.names[rec.dtype.names.index("pre_full_w"):]:
-            v = float(rec[name])
-            if not np.isfinite(v) or v < 0:
+            v = recs[name]
+            if not np.all((v >= 0) & (v <= 1)):
+                raise ValueError(f"offload ratios '{name}' must lie in [0, 1], got {v[~((v >= 0) & (v <= 1))]}")
+        names = recs.dtype.names
+        for name in names[names.index("pre_full_w"):]:
+            v = recs[name]
+            if not np.all(np.isfinite(v) & (v >= 0)):
                 raise ValueError(f"pre/post layer input '{name}' must be finite and non-negative, got {v}")

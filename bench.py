@@ -163,6 +163,9 @@ def main():
         peak=FP64_VECTOR_PEAK / 1e12, unit="TFLOP/s", frac=achieved / (FP64_VECTOR_PEAK / 1e12),
         traffic=EVAL_REDUCE_HBM_BYTES, avg_launch_ms=dur_ms / n_launches,
         flop_per_launch=flops / n_launches, launches_per_step=1,
+        # the HBM side alongside: measured traffic of the launch pair over its duration
+        hbm=dict(achieved=EVAL_REDUCE_HBM_BYTES / (dur_ms / n_launches * 1e-3) / 1e9, peak=8000.0,
+                 unit="GB/s", frac=EVAL_REDUCE_HBM_BYTES / (dur_ms / n_launches * 1e-3) / 8e12),
         note="achieved = ALGORITHMIC flops (the reference's formulas for every cell) / time; the "
              "kernel prunes exactly and executes a fraction of them, so frac can exceed 1 "
              "(executed: 8.3e8 VALU wave-instructions per call, 32 % of the issue slots, in the "

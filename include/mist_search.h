@@ -181,7 +181,10 @@ int mist_row_terms(const MistProblem *problem, const MistGroupDesc *d_groups, in
  * belong to real rows of the group, so the result is unchanged) and lets far fewer rows through
  * to the memory model.
  * d_partial_cost / d_partial_index: [n_blocks + n_scout_blocks][2*MIST_P_TILE+2][MIST_LC_TILE];
- * the first n_blocks slabs are the per-chunk results mist_finalize reads. */
+ * the first n_blocks slabs are the per-chunk results mist_finalize reads.  A chunk other than
+ * the first of its tile whose minima are still its seeds does not write its slab: it stores -2
+ * as the slab's first row index (rows are >= -1) and mist_finalize skips the slab; the first
+ * chunk always writes and carries the seeds. */
 int mist_eval_reduce(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,
                      const int32_t *d_block_prefix, int n_blocks,
                      const int32_t *d_scout_prefix, int n_scout_blocks,

@@ -588,6 +588,7 @@ __device__ __forceinline__ void take_min(double &best, int32_t &best_row, bool f
 #define MIST_REDUCE_MIN_WAVES 2
 #endif
 constexpr int kScoutSplit = 2;  // scout workgroups per (group, (l, c) tile, p tile)
+constexpr int32_t kSlabUnchanged = -2;  // first row index of a slab that was not written (rows are >= -1)
 constexpr int kPairFields = 4;  // per-pair table of sieve A: thr_b, thr_o, n_ck, n_nock
 constexpr int kLdsRowStride = MIST_ROW_TERMS + 1;  // odd number of doubles: lanes reading the
                                                    // same term of different rows hit different banks
@@ -679,7 +680,7 @@ __device__ __forceinline__ void reduce_block(
     double *lds_terms, double *lds_min, double *lds_pair, int32_t *lds_rowpos,
     const double *__restrict__ seed_cost,
     const int32_t *__restrict__ seed_index, double *__restrict__ out_cost,
-    int32_t *__restrict__ out_index) {
+    int32_t *__restrict__ out_index, bool skip_unchanged) {
   const int L = prob.num_layers;
   const int n_pairs = L * (L + 1) / 2 + L;  // sum over l = 1..L of (l + 1)
   const int pair_idx = lc_tile * MIST_LC_TILE + threadIdx.x;
@@ -717,6 +718,7 @@ __device__ __forceinline__ void reduce_block(
   // largest finite one.  A row that does not reach `top` can only fill the first empty slot.
   int fin_b = 0, fin_p = 0;
   double top_b = -INFINITY, top_p = -INFINITY;
+  bool dirty = false;  // some slot of this lane differs from its seed
 #pragma unroll
   for (int j = 0; j < MIST_P_TILE; ++j) {
     best_b[j] = best_p[j] = INFINITY;
@@ -1136,8 +1138,16 @@ __device__ __forceinline__ void reduce_block(
     while (keep != 0) {
       const int r = __ffsll((unsigned long long)keep) - 1;
       keep &= keep - 1;
-      examine(lds_terms + r * kLdsRowStride, lds_rowpos[r], std::true_type{});
+      dirty |= examine(lds_terms + r * kLdsRowStride, lds_rowpos[r], std::true_type{});
     }
+  }
+
+  // A chunk that changed no slot holds exactly its seeds, which the first chunk of the tile
+  // writes out anyway: it leaves a mark instead of its 26 KB slab, and the combining kernel
+  // skips it.
+  if (skip_unchanged && !__any(dirty)) {
+    if (threadIdx.x == 0) out_index[0] = kSlabUnchanged;
+    return;
   }
 
 #pragma unroll
@@ -1177,6 +1187,7 @@ __global__ __launch_bounds__(MIST_LC_TILE, MIST_REDUCE_MIN_WAVES) void eval_redu
   int tile;
   ReduceRange range;
   int64_t out_slab;
+  bool skip_unchanged = false;  // only the chunks after the first of a tile may leave a mark
   if (scout) {
     if (g->scout_stride <= 0) return;
     tile = local_block / kScoutSplit;
@@ -1190,6 +1201,7 @@ __global__ __launch_bounds__(MIST_LC_TILE, MIST_REDUCE_MIN_WAVES) void eval_redu
     const int64_t row_begin = (int64_t)chunk * g->rows_per_chunk;
     range = ReduceRange{row_begin, min(row_begin + (int64_t)g->rows_per_chunk, g->n_rows), 1, 0, 0};
     out_slab = block;
+    skip_unchanged = chunk > 0;
   }
   const int p_tile = tile % g->n_p_tiles;
   const int lc_tile = tile / g->n_p_tiles;
@@ -1203,7 +1215,8 @@ __global__ __launch_bounds__(MIST_LC_TILE, MIST_REDUCE_MIN_WAVES) void eval_redu
   reduce_block<P2, FT>(prob, g, range, p_tile, lc_tile, row_terms,                            \
                        stage_floor + stage_floor_slot(g, gi, 0) * kStageFloorPitch, ratio,    \
                        lds_terms, lds_min, lds_pair, lds_rowpos, seed_cost, seed_index,                   \
-                       partial_cost + out_slab * slab, partial_index + out_slab * slab)
+                       partial_cost + out_slab * slab, partial_index + out_slab * slab,       \
+                       skip_unchanged)
   if (pow2) {
     if (p_tile == 0) MIST_REDUCE(true, true); else MIST_REDUCE(true, false);
   } else {
@@ -1254,8 +1267,9 @@ __global__ __launch_bounds__(256) void finalize_kernel(
   double best = INFINITY;
   int32_t best_row = -1;
   for (int ch = 0; ch < g->n_chunks; ++ch) {
-    const int64_t at =
-        ((first_block + (int64_t)ch * n_tiles) * kSlots + kslot) * MIST_LC_TILE + lane;
+    const int64_t slab_at = (first_block + (int64_t)ch * n_tiles) * kSlots * MIST_LC_TILE;
+    if (ch > 0 && partial_index[slab_at] == kSlabUnchanged) continue;  // holds the seeds only
+    const int64_t at = slab_at + (int64_t)kslot * MIST_LC_TILE + lane;
     const double cost = partial_cost[at];
     const int32_t row = partial_index[at];
     take_min(best, best_row, row >= 0, cost, row);

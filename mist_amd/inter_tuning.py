@@ -79,7 +79,9 @@ class _DpRunner:
                 for t in dev_tabs.stable
             ]
             self.pmin = [torch.empty_like(t) for t in self.cost]
-            d_G = torch.tensor(Gs, dtype=torch.int32, device=self.device)
+            d_G = getattr(dev_tabs, "grad_accum", None)
+            if d_G is None or d_G.numel() != Gn:
+                d_G = torch.tensor(Gs, dtype=torch.int32, device=self.device)
             out_ptrs = (ctypes.c_void_p * 4)(*[t.data_ptr() for t in self.cost])
             pmin_ptrs = (ctypes.c_void_p * 4)(*[t.data_ptr() for t in self.pmin])
             tabs = dev_tabs.as_struct()

@@ -49,6 +49,9 @@ class DeviceTables:
     stable: List[torch.Tensor]
     delta: List[torch.Tensor]
     index: List[torch.Tensor]
+    # gradient-accumulation count of every table row g (int32, on the device), uploaded with the
+    # plan so that the inter-stage search need not wait for the kernels to copy it
+    grad_accum: Optional[torch.Tensor] = None
 
     def as_struct(self) -> _lib.OutTables:
         s = _lib.OutTables()
@@ -301,6 +304,9 @@ class IntraStageTuner:
                 dtype=torch.float64, device=dev),
             partial_cost=torch.empty(n_slabs * _lib.SLOTS * _lib.LC_TILE, dtype=torch.float64, device=dev),
             partial_index=torch.empty(n_slabs * _lib.SLOTS * _lib.LC_TILE, dtype=torch.int32, device=dev),
+            grad_accum=torch.tensor(
+                list(self.gradient_accumulation_steps_candidates) * len(self.tp_sizes),
+                dtype=torch.int32, device=dev),
         )
 
     def launch(self, plan, dev_plan, tables: DeviceTables, events: Optional[list] = None) -> None:
@@ -372,6 +378,7 @@ class IntraStageTuner:
         output per tp size, all resident in the same tables."""
         with torch.cuda.device(self.device):
             tables = self.allocate_tables()
+            tables.grad_accum = dev_plan.get("grad_accum")
             self.launch(plan, dev_plan, tables)
         return self._outputs(plan, tables)
 

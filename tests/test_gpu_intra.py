@@ -168,6 +168,25 @@ def test_scout_pass_leaves_results_unchanged(monkeypatch, min_stages, min_pairs)
     _compare(cfg, tables, 2)
 
 
+@pytest.mark.parametrize("waves, scout", [(1 << 22, 1), (1 << 22, 0), (1, 1)])
+def test_row_chunking_leaves_results_unchanged(monkeypatch, waves, scout):
+    """Groups cut into the smallest row chunks (256 rows: many chunks per tile, most of which
+    change no slot once the first ones or the scout pass have found the minima, and then leave
+    only a mark for the combining kernel) or into one chunk each give the oracle's tables."""
+    from mist_amd import intra_tuning
+
+    monkeypatch.setattr(intra_tuning, "TARGET_REDUCE_WAVES", waves)
+    monkeypatch.setattr(intra_tuning, "SCOUT_MIN_STAGES", scout)
+    monkeypatch.setattr(intra_tuning, "SCOUT_MIN_PAIRS", 1)
+    cfg, tables = tiny_plan(1, layers=6, hardware__memory_capacity=6.0)
+    groups = _gpu_tuner(cfg, tables, 1).prepare()["groups"]
+    assert (groups["n_chunks"].max() > 3) == (waves > 1)
+    assert (groups["scout_stride"] > 0).any() == (scout > 0)
+    _compare(cfg, tables, 1)
+    cfg, tables = load_plan(1)
+    _compare(cfg, tables, 2)
+
+
 @pytest.mark.parametrize(
     "plan, G, mesh, tp", [(2, 64, (1, 1), 1), (2, 128, (1, 8), 8), (3, 64, (1, 8), 8)]
 )

@@ -109,35 +109,68 @@ struct Interference {
 
   // Arguments in the order of the reference's get_layer_critical_latency
   // (batched_module_analyzer.py:1413-1422): exec, gpu<->gpu, gpu->cpu, cpu->gpu.
-  __device__ __noinline__ double operator()(double exec, double g2g, double g2c, double c2g) const {
-    double x0 = exec, x1 = g2g, x2 = c2g, x3 = g2c;
+  // kLive: bit i set when X[i] (exec, gpu<->gpu, cpu->gpu, gpu->cpu) can be non-zero at this call
+  // site; the others are literal zeros there, never part of a mask, and their share of a round
+  // (a multiplication and a division each) is left out at compile time.  The sums keep all four
+  // operands, so the value is the one of the general form.
+  template <unsigned kLive>
+  __device__ __noinline__ double eval(double exec, double g2g, double g2c, double c2g) const {
+    double x0 = (kLive & 1u) ? exec : 0.0, x1 = (kLive & 2u) ? g2g : 0.0;
+    double x2 = (kLive & 4u) ? c2g : 0.0, x3 = (kLive & 8u) ? g2c : 0.0;
     double out = 0.0;
     // The reference tries the 11 masks in order and applies the one equal to the non-zero
     // pattern of X.  A pattern equals at most one mask, and after a peel the pattern has fewer
     // bits, i.e. it can only equal a mask further down the list (4-way, then 3-way, then
-    // 2-way).  So the mask to apply is looked up from the pattern: at most three rounds.
+    // 2-way).  So the mask to apply is looked up from the pattern: at most three rounds (one
+    // fewer than there are live operands).
+    constexpr int kRounds = __builtin_popcount(kLive) - 1;
 #pragma unroll 1
-    for (int round = 0; round < 3; ++round) {
+    for (int round = 0; round < kRounds; ++round) {
       // "not isclose(x, 0)" with numpy's default tolerances: |x| > 1e-8 (NaN counts as non-zero).
-      const unsigned nz = (!(fabs(x0) <= 1e-8) ? 1u : 0u) | (!(fabs(x1) <= 1e-8) ? 2u : 0u) |
-                          (!(fabs(x2) <= 1e-8) ? 4u : 0u) | (!(fabs(x3) <= 1e-8) ? 8u : 0u);
+      const unsigned nz = (((kLive & 1u) && !(fabs(x0) <= 1e-8)) ? 1u : 0u) |
+                          (((kLive & 2u) && !(fabs(x1) <= 1e-8)) ? 2u : 0u) |
+                          (((kLive & 4u) && !(fabs(x2) <= 1e-8)) ? 4u : 0u) |
+                          (((kLive & 8u) && !(fabs(x3) <= 1e-8)) ? 8u : 0u);
       const int m = kMaskOfPattern[nz];
       if (m < 0) break;  // fewer than two busy resources: nothing overlaps
       const unsigned mask = nz;
       const double f0 = factor[m][0], f1 = factor[m][1], f2 = factor[m][2], f3 = factor[m][3];
       const double s0 = x0 * f0, s1 = x1 * f1, s2 = x2 * f2, s3 = x3 * f3;
       double ov = INFINITY;
-      if (mask & 1u) ov = fmin(ov, s0);
-      if (mask & 2u) ov = fmin(ov, s1);
-      if (mask & 4u) ov = fmin(ov, s2);
-      if (mask & 8u) ov = fmin(ov, s3);
-      if (mask & 1u) x0 = (s0 - ov) / f0 * 1.0;
-      if (mask & 2u) x1 = (s1 - ov) / f1 * 1.0;
-      if (mask & 4u) x2 = (s2 - ov) / f2 * 1.0;
-      if (mask & 8u) x3 = (s3 - ov) / f3 * 1.0;
+      if ((kLive & 1u) && (mask & 1u)) ov = fmin(ov, s0);
+      if ((kLive & 2u) && (mask & 2u)) ov = fmin(ov, s1);
+      if ((kLive & 4u) && (mask & 4u)) ov = fmin(ov, s2);
+      if ((kLive & 8u) && (mask & 8u)) ov = fmin(ov, s3);
+      if ((kLive & 1u) && (mask & 1u)) x0 = (s0 - ov) / f0 * 1.0;
+      if ((kLive & 2u) && (mask & 2u)) x1 = (s1 - ov) / f1 * 1.0;
+      if ((kLive & 4u) && (mask & 4u)) x2 = (s2 - ov) / f2 * 1.0;
+      if ((kLive & 8u) && (mask & 8u)) x3 = (s3 - ov) / f3 * 1.0;
       out = out + ov;
     }
     return out + (((x0 + x1) + x2) + x3);
+  }
+
+  __device__ __forceinline__ double operator()(double exec, double g2g, double g2c, double c2g) const {
+    return eval<15u>(exec, g2g, g2c, c2g);
+  }
+  // Call sites whose literal zeros are known: operands named by what is live.
+  __device__ __forceinline__ double exec_g2g_c2g(double exec, double g2g, double c2g) const {
+    return eval<1u | 2u | 4u>(exec, g2g, 0.0, c2g);
+  }
+  __device__ __forceinline__ double exec_g2g_g2c(double exec, double g2g, double g2c) const {
+    return eval<1u | 2u | 8u>(exec, g2g, g2c, 0.0);
+  }
+  __device__ __forceinline__ double g2g_c2g(double g2g, double c2g) const {
+    return eval<2u | 4u>(0.0, g2g, 0.0, c2g);
+  }
+  __device__ __forceinline__ double g2g_g2c(double g2g, double g2c) const {
+    return eval<2u | 8u>(0.0, g2g, g2c, 0.0);
+  }
+  __device__ __forceinline__ double exec_g2c(double exec, double g2c) const {
+    return eval<1u | 8u>(exec, 0.0, g2c, 0.0);
+  }
+  __device__ __forceinline__ double g2c_only(double g2c) const {
+    return eval<8u>(0.0, 0.0, g2c, 0.0);
   }
 };
 
@@ -329,16 +362,16 @@ __global__ __launch_bounds__(kTermsBlock) void row_terms_kernel(
   for (int ph = 0; ph < 2; ++ph) {
     const double pre_g2g = (ph == 0 || adv) ? g2g_F[ph] : 0.0;
     const double pre_c2g = adv ? c2g_F[ph] : 0.0;
-    const double first = I(E_f, g2g_F[ph], 0.0, c2g_F[ph]) + extra_fwd;
-    const double extra_pre = I(0.0, pre_g2g, 0.0, pre_c2g);
+    const double first = I.exec_g2g_c2g(E_f, g2g_F[ph], c2g_F[ph]) + extra_fwd;
+    const double extra_pre = I.g2g_c2g(pre_g2g, pre_c2g);
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
       const double g2c = g2c_F[ph] + (k ? so_A_ck : so_A_nock);
       fwd[ph][k].layer = I(E_f, g2g_F[ph], g2c, c2g_F[ph]) + extra_fwd;
       fwd[ph][k].first = first;
-      fwd[ph][k].last = I(E_f, 0.0, g2c, 0.0) + extra_fwd;
+      fwd[ph][k].last = I.exec_g2c(E_f, g2c) + extra_fwd;
       fwd[ph][k].extra_pre = extra_pre;
-      fwd[ph][k].extra_post = I(0.0, 0.0, g2c, 0.0);
+      fwd[ph][k].extra_post = I.g2c_only(g2c);
     }
   }
 
@@ -364,10 +397,10 @@ __global__ __launch_bounds__(kTermsBlock) void row_terms_kernel(
       // With checkpointing the reference adds the (always zero) all-gather of saved tensors.
       const double g2g_layer = k ? g2g_B[ph] + 0.0 : g2g_B[ph];
       bwd[ph][k].layer = I(E, g2g_layer, g2c_B, c2g) + extra;
-      bwd[ph][k].last = I(E, ag_wre, 0.0, c2g) + extra;
-      bwd[ph][k].first = I(E, red, first_g2c, 0.0) + extra;
-      bwd[ph][k].extra_pre = I(0.0, ag_wre, 0.0, c2g);
-      bwd[ph][k].extra_post = I(0.0, red, first_g2c, 0.0);
+      bwd[ph][k].last = I.exec_g2g_c2g(E, ag_wre, c2g) + extra;
+      bwd[ph][k].first = I.exec_g2g_g2c(E, red, first_g2c) + extra;
+      bwd[ph][k].extra_pre = I.g2g_c2g(ag_wre, c2g);
+      bwd[ph][k].extra_post = I.g2g_g2c(red, first_g2c);
     }
   }
 

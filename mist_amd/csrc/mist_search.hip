@@ -121,19 +121,19 @@ struct Interference {
     // The reference tries the 11 masks in order and applies the one equal to the non-zero
     // pattern of X.  A pattern equals at most one mask, and after a peel the pattern has fewer
     // bits, i.e. it can only equal a mask further down the list (4-way, then 3-way, then
-    // 2-way).  So the mask to apply is looked up from the pattern: at most three rounds (one
-    // fewer than there are live operands).
-    constexpr int kRounds = __builtin_popcount(kLive) - 1;
-#pragma unroll 1
-    for (int round = 0; round < kRounds; ++round) {
-      // "not isclose(x, 0)" with numpy's default tolerances: |x| > 1e-8 (NaN counts as non-zero).
-      const unsigned nz = (((kLive & 1u) && !(fabs(x0) <= 1e-8)) ? 1u : 0u) |
-                          (((kLive & 2u) && !(fabs(x1) <= 1e-8)) ? 2u : 0u) |
-                          (((kLive & 4u) && !(fabs(x2) <= 1e-8)) ? 4u : 0u) |
-                          (((kLive & 8u) && !(fabs(x3) <= 1e-8)) ? 8u : 0u);
-      const int m = kMaskOfPattern[nz];
-      if (m < 0) break;  // fewer than two busy resources: nothing overlaps
-      const unsigned mask = nz;
+    // 2-way).  So the rounds are taken by the size of the pattern: a lane joins at the size of
+    // its own pattern, and the wave runs each size once.
+    // "not isclose(x, 0)" with numpy's default tolerances: |x| > 1e-8.
+    auto pattern = [&]() {
+      return (((kLive & 1u) && !(fabs(x0) <= 1e-8)) ? 1u : 0u) |
+             (((kLive & 2u) && !(fabs(x1) <= 1e-8)) ? 2u : 0u) |
+             (((kLive & 4u) && !(fabs(x2) <= 1e-8)) ? 4u : 0u) |
+             (((kLive & 8u) && !(fabs(x3) <= 1e-8)) ? 8u : 0u);
+    };
+    // One peel as the reference writes it: every busy resource gives up the smallest scaled
+    // time.
+    auto peel = [&](unsigned mask) {
+      const int m = kMaskOfPattern[mask];
       const double f0 = factor[m][0], f1 = factor[m][1], f2 = factor[m][2], f3 = factor[m][3];
       const double s0 = x0 * f0, s1 = x1 * f1, s2 = x2 * f2, s3 = x3 * f3;
       double ov = INFINITY;
@@ -146,6 +146,45 @@ struct Interference {
       if ((kLive & 4u) && (mask & 4u)) x2 = (s2 - ov) / f2 * 1.0;
       if ((kLive & 8u) && (mask & 8u)) x3 = (s3 - ov) / f3 * 1.0;
       out = out + ov;
+    };
+    // The same peel for two busy resources with one division: the one with the smaller scaled
+    // time is left with (s - s) / f = +0 (factors are positive and finite), the other with
+    // (larger - smaller) / its factor; with equal times both quotients are +0.
+    auto peel_pair = [&](unsigned mask) {
+      const int m = kMaskOfPattern[mask];
+      const double f0 = factor[m][0], f1 = factor[m][1], f2 = factor[m][2], f3 = factor[m][3];
+      const double s0 = x0 * f0, s1 = x1 * f1, s2 = x2 * f2, s3 = x3 * f3;
+      const bool b0 = (kLive & 1u) && (mask & 1u), b1 = (kLive & 2u) && (mask & 2u);
+      const bool b2 = (kLive & 4u) && (mask & 4u), b3 = (kLive & 8u) && (mask & 8u);
+      double lo = INFINITY, hi = -INFINITY;
+      if (b0) { lo = fmin(lo, s0); hi = fmax(hi, s0); }
+      if (b1) { lo = fmin(lo, s1); hi = fmax(hi, s1); }
+      if (b2) { lo = fmin(lo, s2); hi = fmax(hi, s2); }
+      if (b3) { lo = fmin(lo, s3); hi = fmax(hi, s3); }
+      double den = 1.0;
+      if (b0 && s0 == hi) den = f0;
+      if (b1 && s1 == hi) den = f1;
+      if (b2 && s2 == hi) den = f2;
+      if (b3 && s3 == hi) den = f3;
+      const double rest = (hi - lo) / den * 1.0;
+      if (b0) x0 = s0 == hi ? rest : 0.0;
+      if (b1) x1 = s1 == hi ? rest : 0.0;
+      if (b2) x2 = s2 == hi ? rest : 0.0;
+      if (b3) x3 = s3 == hi ? rest : 0.0;
+      out = out + lo;
+    };
+    constexpr int kLiveCount = __builtin_popcount(kLive);
+    if constexpr (kLiveCount == 4) {
+      const unsigned nz = pattern();
+      if (nz == 15u) peel(nz);
+    }
+    if constexpr (kLiveCount >= 3) {
+      const unsigned nz = pattern();
+      if (__popc(nz) == 3) peel(nz);
+    }
+    if constexpr (kLiveCount >= 2) {
+      const unsigned nz = pattern();
+      if (__popc(nz) == 2) peel_pair(nz);
     }
     return out + (((x0 + x1) + x2) + x3);
   }
@@ -1435,6 +1474,13 @@ int mist_row_terms(const MistProblem *problem, const MistGroupDesc *d_groups, in
   if (!d_block_prefix || !d_row_terms || !d_stage_floor)
     return fail(MIST_E_INVALID, "null workspace pointer");
   if (n_blocks <= 0) return fail(MIST_E_INVALID, "n_blocks must be positive, got %d", n_blocks);
+  for (int m = 0; m < 11; ++m)
+    for (int i = 0; i < 4; ++i) {
+      const double f = problem->interf_factor[m][i];
+      // the kernel takes 0 / f == +0 for granted
+      if (!(f > 0.0) || std::isinf(f))
+        return fail(MIST_E_INVALID, "interference factor [%d][%d] must be positive and finite", m, i);
+    }
   hipLaunchKernelGGL(row_terms_kernel, dim3(n_blocks), dim3(kTermsBlock), 0, (hipStream_t)stream,
                      *problem, d_groups, n_groups, d_block_prefix, d_row_terms, d_stage_floor);
   MIST_HIP_CHECK(hipGetLastError());

@@ -163,7 +163,10 @@ int64_t mist_stage_floor_doubles(int64_t total_rows, int n_groups);
  * not for correctness); all results carry reference row numbers.
  * d_stage_floor: mist_stage_floor_doubles() float64, written here and read by mist_eval_reduce:
  * per stage of mist_reduce_stage_rows() workspace rows the term-wise minimum of the latency and
- * memory terms (the pseudo row that bounds every row of the stage from below). */
+ * memory terms (the pseudo row that bounds every row of the stage from below).
+ * Fails with MIST_E_INVALID when an interference factor of `problem` is not positive and finite
+ * (the kernel peels two overlapping resources with one division and takes 0 / f == +0 for the
+ * other one). */
 int mist_row_terms(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,
                    const int32_t *d_block_prefix, int n_blocks, double *d_row_terms,
                    double *d_stage_floor, void *stream);

@@ -180,7 +180,8 @@ int mist_row_terms(const MistProblem *problem, const MistGroupDesc *d_groups, in
  * Optional scout pass (n_scout_blocks > 0): d_scout_prefix[n_groups+1] gives each group
  * n_lc_tiles*n_p_tiles*mist_reduce_scout_split() workgroups that first reduce the rows of the
  * group's scout pairs (MistGroupDesc.scout_stride; the search's winners sit almost exclusively
- * on rows without weight / gradient offloading); every chunk then starts from those minima (they
+ * on rows without weight / gradient offloading; a small kernel then combines the slabs of a
+ * tile's scout workgroups into the first of them); every chunk then starts from those minima (they
  * belong to real rows of the group, so the result is unchanged) and lets far fewer rows through
  * to the memory model.
  * d_partial_cost / d_partial_index: [n_blocks + n_scout_blocks][2*MIST_P_TILE+2][MIST_LC_TILE];

@@ -797,10 +797,9 @@ __device__ __forceinline__ void reduce_block(
     row_b[j] = row_p[j] = -1;
   }
   if (seed_cost != nullptr && active) {
-    const int64_t slab = (int64_t)kSlots * MIST_LC_TILE;
-    for (int k = 0; k < kScoutSplit; ++k) {
-      const double *sc = seed_cost + k * slab + threadIdx.x;
-      const int32_t *si = seed_index + k * slab + threadIdx.x;
+    {  // the first slab of the tile's scout workgroups holds their combined minima
+      const double *sc = seed_cost + threadIdx.x;
+      const int32_t *si = seed_index + threadIdx.x;
 #pragma unroll
       for (int j = 0; j < MIST_P_TILE; ++j) {
         const int32_t rb = si[j * MIST_LC_TILE], rp = si[(MIST_P_TILE + j) * MIST_LC_TILE];
@@ -1297,6 +1296,26 @@ __global__ __launch_bounds__(MIST_LC_TILE, MIST_REDUCE_MIN_WAVES) void eval_redu
 #undef MIST_REDUCE
 }
 
+// Combines the slabs of the kScoutSplit scout workgroups of every tile into the first of them,
+// so that each chunk of the main launch reads one slab of seeds instead of kScoutSplit.
+// Workgroup = tile; the scout slabs of tile t are n_blocks + t * kScoutSplit + k.
+__global__ __launch_bounds__(256) void merge_scout_kernel(int n_blocks,
+                                                          double *__restrict__ partial_cost,
+                                                          int32_t *__restrict__ partial_index) {
+  const int64_t slab = (int64_t)kSlots * MIST_LC_TILE;
+  const int64_t first = ((int64_t)n_blocks + (int64_t)blockIdx.x * kScoutSplit) * slab;
+  for (int e = threadIdx.x; e < (int)slab; e += blockDim.x) {
+    double best = INFINITY;
+    int32_t best_row = -1;
+    for (int k = 0; k < kScoutSplit; ++k) {
+      const int32_t row = partial_index[first + k * slab + e];
+      take_min(best, best_row, row >= 0, partial_cost[first + k * slab + e], row);
+    }
+    partial_cost[first + e] = best;
+    partial_index[first + e] = best_row;
+  }
+}
+
 // ------------------------------------------------------------------------------------------
 // Kernel 3: combine the chunks' (cost, row) minima, recompute the winner's stable / delta, scatter.
 // One thread per (group, (l, c) pair, slot); slots as in the reduce kernel but over all p.
@@ -1517,6 +1536,14 @@ int mist_eval_reduce(const MistProblem *problem, const MistGroupDesc *d_groups, 
                        n_blocks, scout_prefix, 1, d_row_terms, d_stage_floor, ratio,
                        d_partial_cost, d_partial_index);
     MIST_HIP_CHECK(hipGetLastError());
+    if (kScoutSplit > 1) {
+      if (n_scout_blocks % kScoutSplit != 0)
+        return fail(MIST_E_INVALID, "n_scout_blocks %d is not a multiple of the scout split %d",
+                    n_scout_blocks, kScoutSplit);
+      hipLaunchKernelGGL(merge_scout_kernel, dim3(n_scout_blocks / kScoutSplit), dim3(256), 0,
+                         (hipStream_t)stream, n_blocks, d_partial_cost, d_partial_index);
+      MIST_HIP_CHECK(hipGetLastError());
+    }
   }
   hipLaunchKernelGGL(eval_reduce_kernel, dim3(xcd_padded_grid(n_blocks)), dim3(MIST_LC_TILE), 0,
                      (hipStream_t)stream, *problem, d_groups, n_groups, d_block_prefix, n_blocks,

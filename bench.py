@@ -28,9 +28,9 @@ if REPO not in sys.path:
 PLAN = os.path.join(REPO, "mist_amd", "configs", "gpt-7b-b512-4x8.yaml")
 FP64_VECTOR_PEAK = 78.6e12  # MI355X published fp64 vector peak, FLOP/s
 # HBM bytes of one mist_eval_reduce call (scout, seed merge and main launch) on this workload, from two
-# rocprofv3 --pmc runs (FETCH_SIZE 4.671e5 KiB scaled x2.0, WRITE_SIZE 1.485e5 KiB scaled x1.0
+# rocprofv3 --pmc runs (FETCH_SIZE 4.572e5 KiB scaled x2.0, WRITE_SIZE 1.526e5 KiB scaled x1.0
 # by what a 1 GiB device copy reads on the same counters; profiles/bench_gpt7b_kernel_stats.md).
-EVAL_REDUCE_HBM_BYTES = int((4.671e5 * 2.0 + 1.485e5) * 1024)
+EVAL_REDUCE_HBM_BYTES = int((4.572e5 * 2.0 + 1.526e5) * 1024)
 
 
 def reduce_kernel_flops(plan, L):
@@ -168,7 +168,7 @@ def main():
                  unit="GB/s", frac=EVAL_REDUCE_HBM_BYTES / (dur_ms / n_launches * 1e-3) / 8e12),
         note="achieved = ALGORITHMIC flops (the reference's formulas for every cell) / time; the "
              "kernel prunes exactly and executes a fraction of them, so frac can exceed 1 "
-             "(executed: 8.6e8 VALU wave-instructions per call, 37 % of the issue slots, in the "
+             "(executed: 8.7e8 VALU wave-instructions per call, 39 % of the issue slots, in the "
              "rocprofv3 --pmc run under profiles/)",
     )
     intra_ms_per_step = sum(kernel_ms.values()) / 2

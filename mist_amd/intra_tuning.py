@@ -24,9 +24,9 @@ from .stage_inputs import GroupInputBuilder, make_problem
 
 SAMPLE_SIZE = 30  # reference default (batched_module_analyzer.py:67)
 VARIANTS = ("", "_with_pre", "_with_post", "_no_pp")
-# wavefronts of the reduce kernel the row chunks are sized for: ~48 per SIMD, so that the tail of
+# wavefronts of the reduce kernel the row chunks are sized for: 64 per SIMD, so that the tail of
 # the launch is short; a chunk that changes no slot writes no slab, which keeps small chunks cheap
-TARGET_REDUCE_WAVES = 49152
+TARGET_REDUCE_WAVES = 65536
 SCOUT_MIN_STAGES = 128  # groups with fewer stages get no scout pass (0 = never scout)
 SCOUT_MIN_PAIRS = 4     # ... and so do groups with fewer (weight, gradient) offload pairs
 SCOUT_PAIRS = 1         # offload pairs whose rows the scout pass gathers: the first, (0, 0), then evenly spread ones

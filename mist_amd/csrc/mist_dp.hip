@@ -151,8 +151,12 @@ __global__ __launch_bounds__(256) void select_candidates_kernel(
       }
     }
     __syncthreads();
-    // room for another round of kSelectBatch values per thread?
-    if (n_kept > kSelectBuffer - kSelectBatch * 256) flush();
+    // Room for another round of kSelectBatch values per thread?  Every wave reads the count
+    // before any wave adds to it again (second barrier), so the whole workgroup takes the
+    // same branch and flush()'s barriers are reached by all of its waves.
+    const int kept_now = n_kept;
+    __syncthreads();
+    if (kept_now > kSelectBuffer - kSelectBatch * 256) flush();
   }
   flush();
   // one atomic per workgroup for the "above" count

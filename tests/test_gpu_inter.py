@@ -458,6 +458,39 @@ def test_candidate_window_selection_matches_numpy():
     assert len(got[3][0]) == 0 and len(got[5][0]) == 0 and len(got[0][0]) > 0
 
 
+def test_candidate_selection_of_wide_windows_matches_numpy():
+    """Windows that select (nearly) every finite stage cost of a table row of the GPT-7B plan:
+    each workgroup of the selection kernel then buffers several times its 4096-value LDS list
+    and appends it in pieces, a path the small tables never reach.  The selected multiset must
+    equal numpy's filter of the same row."""
+    from mist_amd.config import tp_candidates
+    from mist_amd.inter_tuning import _DpRunner
+    from mist_amd.intra_tuning import IntraStageTuner
+    from mist_amd.search_space import _get_device_mesh_candidates, _get_grad_accumu_steps_candidates
+
+    cfg, tables = load_plan(2)
+    hw, L = cfg.hardware, cfg.model.num_hidden_layers
+    meshes = _get_device_mesh_candidates(hw.num_nodes, hw.num_gpus_per_node, False)
+    Gs = _get_grad_accumu_steps_candidates(cfg.training.global_batch_size)
+    res = IntraStageTuner(tables, L, meshes, Gs, 1, cfg, sample_size=1).tune()
+    runner = _DpRunner(res, L, hw.num_nodes * hw.num_gpus_per_node, meshes, 0)
+    host = [np.concatenate([runner.cost[v][g].cpu().numpy().ravel() for v in range(3)]) for g in range(len(Gs))]
+    dense = int(np.argmax([np.isfinite(h).sum() for h in host]))
+    h = host[dense][np.isfinite(host[dense])]
+    assert len(h) > 20 * 4096, "the row must overflow the LDS list of its workgroups many times"
+    med = np.float32(np.median(h))
+    rows = np.array([dense, dense, dense, (dense + 1) % len(Gs)], dtype=np.int32)
+    lo = np.array([-np.inf, med, -np.inf, -np.inf], dtype=np.float32)
+    hi = np.array([np.inf, np.inf, med, np.inf], dtype=np.float32)
+    for _ in range(3):  # the interleaving of the workgroups' waves differs from launch to launch
+        got = runner.candidates_between(rows, lo, hi)
+        for (values, above), g, a, b in zip(got, rows, lo, hi):
+            hg = host[g][np.isfinite(host[g])]
+            want = np.sort(hg[(hg > a) & (hg <= b)])
+            assert np.array_equal(values, want)
+            assert above == int((hg > b).sum())
+
+
 @pytest.mark.parametrize("granularity", ["inter-stage", "uniform-device-pp", "uniform-pp", "no-pp"])
 def test_infeasible_plan_returns_inf_none(granularity):
     """Nothing fits into 0.2 GB: every table stays +inf / -1, the searches find no partition and

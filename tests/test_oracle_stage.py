@@ -127,7 +127,7 @@ def test_unwritten_cells_and_shapes():
             for p in range(P):
                 unwritten = c > l or (p >= 1 and c == l - 1)
                 for t in (base, pre):
-                    assert (t[3][p, l - 1, c, 0] == -1) == unwritten or c <= l
+                    assert (t[3][p, l - 1, c, 0] == -1) == unwritten
                     if unwritten:
                         assert t[3][p, l - 1, c, 0] == -1 and np.isinf(t[0][p, l - 1, c, 0])
                     else:

@@ -1,5 +1,6 @@
 """Shared helpers of the test-suite: plan loading, tiny plan variants, oracle <-> kernel maps."""
 import copy
+import hashlib
 import os
 
 import numpy as np
@@ -85,3 +86,20 @@ def assert_same_f64(got, want, what=""):
             f"{what}: {len(bad)} of {got.size} differ; first at {first}: got {got[first]!r} "
             f"want {want[first]!r} (rel {abs(got[first]-want[first])/max(abs(want[first]),1e-300):.3e})"
         )
+
+
+def group_key(tp, G, mesh):
+    """Name of a (tensor-parallel size, gradient-accumulation steps, stage mesh) group in the
+    fixtures of tests/golden/search_tables_plan*.json."""
+    return f"tp{tp}/G{G}/{mesh[0]}x{mesh[1]}"
+
+
+def table_digest(index, stable, delta):
+    """Digest of one result table of a group: row indices as little-endian int32, then the
+    stable and delta costs as little-endian float32 (-0 folded into +0), all in C order."""
+    h = hashlib.sha256()
+    h.update(np.ascontiguousarray(index).astype("<i4").tobytes())
+    for a in (stable, delta):
+        a = np.ascontiguousarray(a).astype(np.float32) + np.float32(0)
+        h.update(a.astype("<f4").tobytes())
+    return h.hexdigest()[:32]

@@ -147,6 +147,20 @@ int mist_dp_run(const MistDpShape *shape, const MistDpCosts *costs, const float 
                 float *d_best_sum, float *d_stage_max, int32_t *d_argmin, float *d_scratch,
                 void *stream);
 
+/* mist_dp_run() for callers that cannot allocate device memory (code under HIP graph capture,
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same
+ * arguments, results and argument checks as mist_dp_run() without d_scratch: the state planes
+ * live in an array built into the library, mist_dp_static_scratch_floats() floats (16 MiB) per
+ * GPU, held until the process ends.  Always runs the one-launch-per-stage-count schedule (the
+ * one that uses the scratch).  Calls no hipMalloc / hipFree or any other allocating routine.
+ * Fails with MIST_E_INVALID when mist_dp_scratch_floats(shape, n_tmax) exceeds the built-in
+ * array.  All calls on one GPU share that array: calls that overlap in time on one GPU (two
+ * streams, two threads) race and must be serialised by the caller. */
+int64_t mist_dp_static_scratch_floats(void);
+int mist_dp_run_static(const MistDpShape *shape, const MistDpCosts *costs, const float *d_tmax,
+                       const int32_t *d_g_index, int n_tmax, int mode, int32_t *d_best_s,
+                       float *d_best_sum, float *d_stage_max, int32_t *d_argmin, void *stream);
+
 /* Partition of every instance of a mist_dp_run() call that recorded back-pointers
  * (reference: the walk of inter_tuning.py:341-355, here on the GPU so that only the partitions
  * travel to the host).  d_path[n_tmax][max_stages][4] int32: stage i of instance t in pipeline

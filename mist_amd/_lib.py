@@ -204,6 +204,11 @@ _DP_SIGNATURES = {
         ctypes.c_int,
         [_VP, ctypes.POINTER(DpCosts), _VP, _VP, ctypes.c_int, ctypes.c_int, _VP, _VP, _VP, _VP, _VP, _VP],
     ),
+    "mist_dp_static_scratch_floats": (ctypes.c_int64, []),
+    "mist_dp_run_static": (
+        ctypes.c_int,
+        [_VP, ctypes.POINTER(DpCosts), _VP, _VP, ctypes.c_int, ctypes.c_int, _VP, _VP, _VP, _VP, _VP],
+    ),
 }
 
 

@@ -665,6 +665,34 @@ size_t fused_lds_limit(int mode) {
   return it->second;
 }
 
+// Scratch of mist_dp_run_static: callers that must not allocate (HIP graph capture, serving
+// loops) get the state planes from this array instead of a workspace argument.  Every GPU the
+// library runs on holds its own copy at its own address until the process ends.
+constexpr int64_t kStaticScratchFloats = (int64_t)4 << 20;  // 16 MiB
+static __device__ __align__(256) float scratch[kStaticScratchFloats];
+constexpr int kMaxKnownDevices = 64;
+
+// Device address of `scratch` on the current device.  In host code the array's name is only a
+// handle for hipGetSymbolAddress, never a pointer a kernel can use; the address is looked up
+// once per device (with that device current) and kept.
+int static_scratch_of_current_device(float **out) {
+  static std::mutex lock;
+  static float *known[kMaxKnownDevices] = {};
+  int device = 0;
+  MIST_HIP_CHECK(hipGetDevice(&device));
+  if (device < 0 || device >= kMaxKnownDevices)
+    return fail(MIST_E_INVALID, "device ordinal %d outside [0, %d)", device, kMaxKnownDevices);
+  std::lock_guard<std::mutex> guard(lock);
+  if (known[device] == nullptr) {
+    void *ptr = nullptr;
+    MIST_HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    if (ptr == nullptr) return fail(MIST_E_HIP, "hipGetSymbolAddress returned a null address");
+    known[device] = static_cast<float *>(ptr);
+  }
+  *out = known[device];
+  return 0;
+}
+
 int check_shape(const MistDpShape *shape) {
   if (!shape) return fail(MIST_E_INVALID, "null DP shape");
   if (shape->free_devices != 0 && (shape->num_devices != 0 || shape->num_mesh != 1))
@@ -687,6 +715,58 @@ int check_shape(const MistDpShape *shape) {
   for (int q = 0; q < shape->num_mesh; ++q)
     if (shape->mesh_n[q] <= 0 || shape->mesh_m[q] <= 0)
       return fail(MIST_E_INVALID, "mesh %d is (%d, %d)", q, shape->mesh_n[q], shape->mesh_m[q]);
+  return 0;
+}
+
+int check_run_arguments(const MistDpShape *shape, const MistDpCosts *costs, const float *d_tmax,
+                        const int32_t *d_g_index, int n_tmax, int mode, const int32_t *d_best_s,
+                        const float *d_best_sum, const float *d_stage_max) {
+  if (int rc = check_shape(shape)) return rc;
+  if (!costs || !costs->costs || !costs->costs_pre || !costs->costs_post || !costs->costs_nopp ||
+      !costs->pmin || !costs->pmin_pre || !costs->pmin_post || !costs->pmin_nopp)
+    return fail(MIST_E_INVALID, "null cost table");
+  if (!d_tmax || !d_g_index || !d_best_s || !d_best_sum || !d_stage_max)
+    return fail(MIST_E_INVALID, "null threshold / output pointer");
+  if (n_tmax <= 0 || n_tmax > 65535)
+    return fail(MIST_E_INVALID, "n_tmax must be in [1, 65535], got %d", n_tmax);
+  if (mode != MIST_DP_THRESHOLD && mode != MIST_DP_BOTTLENECK)
+    return fail(MIST_E_INVALID, "unknown DP mode %d", mode);
+  return 0;
+}
+
+// Small batches are latency-bound: spread every state over a team of lanes.
+bool dp_wide_teams(int n_tmax, int plane) { return (int64_t)n_tmax * plane <= (1 << 19); }
+
+// One launch per stage count; the state planes and reachable ranges of all instances live in
+// d_scratch (mist_dp_scratch_floats() floats, no particular contents expected on entry: the
+// first kernel writes everything a later one reads).
+int run_step_schedule(const MistDpShape *shape, const MistDpCosts *costs, const float *d_tmax,
+                      const int32_t *d_g_index, int n_tmax, int mode, int32_t *d_best_s,
+                      float *d_best_sum, float *d_stage_max, int32_t *d_argmin, float *d_scratch,
+                      void *stream) {
+  const int plane = (shape->num_layers + 1) * (shape->num_devices + 1);
+  const bool wide = dp_wide_teams(n_tmax, plane);
+  const int64_t n_init = (int64_t)n_tmax * plane;
+  int32_t *d_ranges = reinterpret_cast<int32_t *>(d_scratch + (int64_t)4 * n_tmax * plane);
+  hipLaunchKernelGGL(dp_init_kernel, dim3((unsigned)((n_init + 255) / 256)), dim3(256), 0,
+                     (hipStream_t)stream, *shape, n_tmax, d_scratch, d_ranges, d_best_s,
+                     d_best_sum, d_stage_max);
+  MIST_HIP_CHECK(hipGetLastError());
+  const int states_per_block = kDpThreads / (wide ? kDpWideTeam : 1);
+  const dim3 grid((plane + states_per_block - 1) / states_per_block, n_tmax);
+  for (int s = 1; s <= shape->max_stages; ++s) {
+#define MIST_DP_STEP(BOTTLENECK, TEAM)                                                         \
+  hipLaunchKernelGGL((dp_step_kernel<BOTTLENECK, TEAM>), grid, dim3(kDpThreads), 0,            \
+                     (hipStream_t)stream, *shape, *costs, d_tmax, d_g_index, s, d_scratch,     \
+                     d_ranges, d_best_s, d_best_sum, d_stage_max, d_argmin)
+    if (mode == MIST_DP_BOTTLENECK) {
+      if (wide) MIST_DP_STEP(true, kDpWideTeam); else MIST_DP_STEP(true, 1);
+    } else {
+      if (wide) MIST_DP_STEP(false, kDpWideTeam); else MIST_DP_STEP(false, 1);
+    }
+#undef MIST_DP_STEP
+    MIST_HIP_CHECK(hipGetLastError());
+  }
   return 0;
 }
 
@@ -849,20 +929,12 @@ int mist_dp_run(const MistDpShape *shape, const MistDpCosts *costs, const float 
                 const int32_t *d_g_index, int n_tmax, int mode, int32_t *d_best_s,
                 float *d_best_sum, float *d_stage_max, int32_t *d_argmin, float *d_scratch,
                 void *stream) {
-  if (int rc = check_shape(shape)) return rc;
-  if (!costs || !costs->costs || !costs->costs_pre || !costs->costs_post || !costs->costs_nopp ||
-      !costs->pmin || !costs->pmin_pre || !costs->pmin_post || !costs->pmin_nopp)
-    return fail(MIST_E_INVALID, "null cost table");
-  if (!d_tmax || !d_g_index || !d_best_s || !d_best_sum || !d_stage_max)
-    return fail(MIST_E_INVALID, "null threshold / output pointer");
+  if (int rc = check_run_arguments(shape, costs, d_tmax, d_g_index, n_tmax, mode, d_best_s,
+                                   d_best_sum, d_stage_max))
+    return rc;
   if (!d_scratch) return fail(MIST_E_INVALID, "null scratch pointer");
-  if (n_tmax <= 0 || n_tmax > 65535)
-    return fail(MIST_E_INVALID, "n_tmax must be in [1, 65535], got %d", n_tmax);
-  if (mode != MIST_DP_THRESHOLD && mode != MIST_DP_BOTTLENECK)
-    return fail(MIST_E_INVALID, "unknown DP mode %d", mode);
   const int plane = (shape->num_layers + 1) * (shape->num_devices + 1);
-  // Small batches are latency-bound: spread every state over a team of lanes.
-  const bool wide = (int64_t)n_tmax * plane <= (1 << 19);
+  const bool wide = dp_wide_teams(n_tmax, plane);
   // Larger ones: one workgroup per instance with its planes in LDS when they fit and the caller
   // prepared the re-laid row minima.
   const size_t fused_lds =
@@ -887,28 +959,29 @@ int mist_dp_run(const MistDpShape *shape, const MistDpCosts *costs, const float 
     MIST_HIP_CHECK(hipGetLastError());
     return 0;
   }
-  const int64_t n_init = (int64_t)n_tmax * plane;
-  int32_t *d_ranges = reinterpret_cast<int32_t *>(d_scratch + (int64_t)4 * n_tmax * plane);
-  hipLaunchKernelGGL(dp_init_kernel, dim3((unsigned)((n_init + 255) / 256)), dim3(256), 0,
-                     (hipStream_t)stream, *shape, n_tmax, d_scratch, d_ranges, d_best_s,
-                     d_best_sum, d_stage_max);
-  MIST_HIP_CHECK(hipGetLastError());
-  const int states_per_block = kDpThreads / (wide ? kDpWideTeam : 1);
-  const dim3 grid((plane + states_per_block - 1) / states_per_block, n_tmax);
-  for (int s = 1; s <= shape->max_stages; ++s) {
-#define MIST_DP_STEP(BOTTLENECK, TEAM)                                                         \
-  hipLaunchKernelGGL((dp_step_kernel<BOTTLENECK, TEAM>), grid, dim3(kDpThreads), 0,            \
-                     (hipStream_t)stream, *shape, *costs, d_tmax, d_g_index, s, d_scratch,     \
-                     d_ranges, d_best_s, d_best_sum, d_stage_max, d_argmin)
-    if (mode == MIST_DP_BOTTLENECK) {
-      if (wide) MIST_DP_STEP(true, kDpWideTeam); else MIST_DP_STEP(true, 1);
-    } else {
-      if (wide) MIST_DP_STEP(false, kDpWideTeam); else MIST_DP_STEP(false, 1);
-    }
-#undef MIST_DP_STEP
-    MIST_HIP_CHECK(hipGetLastError());
-  }
-  return 0;
+  return run_step_schedule(shape, costs, d_tmax, d_g_index, n_tmax, mode, d_best_s, d_best_sum,
+                           d_stage_max, d_argmin, d_scratch, stream);
+}
+
+int64_t mist_dp_static_scratch_floats(void) { return kStaticScratchFloats; }
+
+int mist_dp_run_static(const MistDpShape *shape, const MistDpCosts *costs, const float *d_tmax,
+                       const int32_t *d_g_index, int n_tmax, int mode, int32_t *d_best_s,
+                       float *d_best_sum, float *d_stage_max, int32_t *d_argmin, void *stream) {
+  if (int rc = check_run_arguments(shape, costs, d_tmax, d_g_index, n_tmax, mode, d_best_s,
+                                   d_best_sum, d_stage_max))
+    return rc;
+  const int64_t need = mist_dp_scratch_floats(shape, n_tmax);
+  if (need < 0 || need > kStaticScratchFloats)
+    return fail(MIST_E_INVALID,
+                "mist_dp_run_static: %d instances of (L=%d, D=%d) need %lld scratch floats, the "
+                "built-in scratch holds %lld; use mist_dp_run with a caller-owned scratch",
+                n_tmax, shape->num_layers, shape->num_devices, (long long)need,
+                (long long)kStaticScratchFloats);
+  float *d_scratch = nullptr;
+  if (int rc = static_scratch_of_current_device(&d_scratch)) return rc;
+  return run_step_schedule(shape, costs, d_tmax, d_g_index, n_tmax, mode, d_best_s, d_best_sum,
+                           d_stage_max, d_argmin, d_scratch, stream);
 }
 
 }  // extern "C"

@@ -238,6 +238,15 @@ def test_argument_checks_reject_before_any_launch():
     assert b"scratch" in lib.mist_last_error()
     assert lib.mist_dp_run(sp, ctypes.byref(costs), fake, fake, 70000, 0, fake, fake, fake, None, fake, None) == -1
     assert lib.mist_dp_run(sp, ctypes.byref(costs), fake, fake, 1, 7, fake, fake, fake, None, fake, None) == -1
+    # the variant with the built-in scratch refuses batches beyond that scratch (80 x 256 planes:
+    # 84 810 floats per instance) and the same bad arguments, all before any GPU call
+    limit = lib.mist_dp_static_scratch_floats()
+    assert limit == 4 << 20
+    assert lib.mist_dp_scratch_floats(sp, 50) > limit >= lib.mist_dp_scratch_floats(sp, 49)
+    assert lib.mist_dp_run_static(sp, ctypes.byref(costs), fake, fake, 50, 0, fake, fake, fake, None, None) == -1
+    assert b"built-in scratch" in lib.mist_last_error()
+    assert lib.mist_dp_run_static(sp, ctypes.byref(costs), fake, fake, 1, 7, fake, fake, fake, None, None) == -1
+    assert lib.mist_dp_run_static(sp, ctypes.byref(costs), None, fake, 1, 0, fake, fake, fake, None, None) == -1
     assert lib.mist_dp_backtrack(sp, None, fake, 1, fake, None) == -1
     assert lib.mist_dp_backtrack(sp, fake, fake, 0, fake, None) == -1
     # the search driver checks its arguments before it touches the GPU

@@ -5,6 +5,8 @@ oracle's end-to-end ``(best_cost, best_solution)`` where every group of the plan
 
     python tests/golden/make_search_fixtures.py --plan 2 --workers 7            # all groups
     python tests/golden/make_search_fixtures.py --plan 4 --select subset        # listed groups
+    python tests/golden/make_search_fixtures.py --plan 5 --shard 0/4 --out parts  # a quarter of the
+        groups; --merge parts then joins the part files into the fixture
 
 Runs on the CPU only (the oracle never touches the GPU library).  A group is one call of the
 oracle's ``batched_tune_best_latency_for_stage`` with ``sample_size = 1`` (the slot the
@@ -262,7 +264,30 @@ def main():
     ap.add_argument("--workers", type=int, default=4)
     ap.add_argument("--cache", default="/tmp/mist_oracle_cache")
     ap.add_argument("--no-tune", action="store_true", help="skip the end-to-end search")
+    ap.add_argument("--shard", default="0/1", help="i/n: only every n-th group, starting at the i-th")
+    ap.add_argument("--out", default=HERE, help="directory the fixture is written to")
+    ap.add_argument("--merge", default=None, help="join the part files of this directory and exit")
     a = ap.parse_args()
+    if a.merge:
+        import glob
+
+        parts = sorted(glob.glob(os.path.join(a.merge, f"search_tables_plan{a.plan}.part*.json")))
+        out = None
+        for p in parts:
+            with open(p) as f:
+                d = json.load(f)
+            if out is None:
+                out = d
+            else:
+                out["groups"].update(d["groups"])
+        n = int(parts[0].rsplit("of", 1)[1].split(".")[0])
+        assert len(parts) == n, f"{len(parts)} of {n} parts present"
+        path = os.path.join(HERE, f"search_tables_plan{a.plan}.json")
+        with open(path, "w") as f:
+            json.dump(out, f, indent=1, sort_keys=True)
+            f.write("\n")
+        print("wrote", path, len(out["groups"]), "groups")
+        return
     cfg, tables = load_plan(a.plan)
     meshes, Gs, tps = plan_axes(cfg)
     if a.select == "all":
@@ -275,6 +300,8 @@ def main():
         if n > 0:
             jobs.append((n * min(G, cfg.model.num_hidden_layers), (a.plan, tp, G, tuple(mesh), a.cache)))
     jobs.sort(key=lambda j: -j[0])  # long groups first
+    shard, n_shards = (int(x) for x in a.shard.split("/"))
+    jobs = jobs[shard::n_shards]
     groups = {}
     t0 = time.time()
     with get_context("fork").Pool(a.workers, maxtasksperchild=1) as pool:
@@ -288,10 +315,12 @@ def main():
         groups={k: dict(rows=groups[k]["rows"], finite=groups[k]["finite"], digest=groups[k]["digest"])
                 for k in sorted(groups)},
     )
-    if a.select == "all" and not a.no_tune:
+    if a.select == "all" and not a.no_tune and n_shards == 1:
         out["tune"] = end_to_end(a.plan, a.cache, a.workers)
         print("tune:", out["tune"]["cost"], out["tune"]["solution"], flush=True)
-    path = os.path.join(HERE, f"search_tables_plan{a.plan}.json")
+    part = "" if n_shards == 1 else f".part{shard}of{n_shards}"
+    os.makedirs(a.out, exist_ok=True)
+    path = os.path.join(a.out, f"search_tables_plan{a.plan}{part}.json")
     with open(path, "w") as f:
         json.dump(out, f, indent=1, sort_keys=True)
         f.write("\n")

@@ -1,0 +1,89 @@
+"""The pruned GPU search against the CPU oracle at full size, through committed fixtures.
+
+tests/golden/search_tables_plan<N>.json (written by tests/golden/make_search_fixtures.py on the
+CPU) holds, per (tp, G, mesh) group of a benchmark plan, a digest of each of the oracle's four
+result tables (row indices + float32 stable / delta costs) and, where every group of the plan is
+covered, the oracle's end-to-end search result.  Here the HIP kernels search the whole plan in
+one batch (scout pass, row chunks, p tiles, sieves: everything the timed workload uses), the
+same digests are taken from their tables and compared, and ``tune`` must return the oracle's
+cost (bit-equal float64) and strategy.
+"""
+import glob
+import json
+import os
+import re
+
+import numpy as np
+import pytest
+
+from util import group_key, load_plan, table_digest
+
+pytestmark = pytest.mark.gpu
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+FIXTURES = sorted(glob.glob(os.path.join(HERE, "golden", "search_tables_plan*.json")))
+
+
+def _plan_of(path):
+    return int(re.search(r"plan(\d+)\.json$", path).group(1))
+
+
+def _listify(x):
+    """Tuples -> lists, numpy scalars -> python numbers (what a JSON round trip leaves)."""
+    return json.loads(json.dumps(x, default=lambda o: o.item()))
+
+
+def test_fixtures_cover_every_benchmark_plan():
+    assert {_plan_of(p) for p in FIXTURES} == {1, 2, 3, 4, 5}
+
+
+@pytest.mark.parametrize("path", FIXTURES, ids=lambda p: f"plan{_plan_of(p)}")
+def test_tables_and_tune_equal_the_oracle_fixture(path):
+    from mist_amd.inter_tuning import inter_stage_tune_batch
+    from mist_amd.tune_one_case import PreparedSearch
+
+    with open(path) as f:
+        fixture = json.load(f)
+    plan = _plan_of(path)
+    cfg, _ = load_plan(plan)
+    assert cfg.tuning.tuning_granularity == "inter-stage" and cfg.tuning.sample_size == 1
+    search = PreparedSearch(cfg)
+    tuner = search.tuner
+    results = tuner.run_prepared(search.plan, search.dev_plan)
+    Gs, meshes = search.Gs, search.meshes
+    present = {(int(r["g_index"]), int(r["q_index"])) for r in search.plan["groups"]}
+    suffix = ("base", "with_pre", "with_post", "no_pp")
+    bad, n_groups = [], 0
+    for t, tp in enumerate(tuner.tp_sizes):
+        res = results[t]
+        host = [(res._fetch("index", v), res._fetch("stable", v), res._fetch("delta", v)) for v in range(4)]
+        for g, G in enumerate(Gs):
+            for q, mesh in enumerate(meshes):
+                want = fixture["groups"].get(group_key(tp, G, mesh))
+                if want is None:
+                    # a plan covered in full lists every group that has candidate rows
+                    assert fixture["select"] != "all" or (t * len(Gs) + g, q) not in present
+                    continue
+                n_groups += 1
+                for v in range(4):
+                    index, stable, delta = (a[g, q] for a in host[v])
+                    if int((index >= 0).sum()) != want["finite"][v] or \
+                            table_digest(index, stable, delta) != want["digest"][v]:
+                        bad.append((group_key(tp, G, mesh), suffix[v], int((index >= 0).sum()), want["finite"][v]))
+        del host
+    assert n_groups == len(fixture["groups"])
+    assert not bad, f"{len(bad)} of {4 * n_groups} tables differ from the oracle: {bad[:8]}"
+
+    if "tune" not in fixture:
+        return
+    hw = cfg.hardware
+    outcomes = inter_stage_tune_batch(
+        search.L, hw.num_nodes * hw.num_gpus_per_node, meshes, Gs, results, slot=0, only_best_solution=False)
+    for tp, (cost, solution) in zip(tuner.tp_sizes, outcomes):
+        want = fixture["tune"]["per_tp"][str(tp)]
+        assert cost == float(want["cost"]), (tp, cost, want["cost"])
+        assert _listify(solution) == want["solution"], tp
+    cost, solution = search.run()
+    assert cost == float(fixture["tune"]["cost"])
+    assert _listify(solution) == fixture["tune"]["solution"]
+    assert solution is not None

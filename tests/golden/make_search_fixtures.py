@@ -36,14 +36,15 @@ for p in (REPO, os.path.join(REPO, "tests")):
 
 from util import PLAN_FILES, group_key, load_plan, table_digest  # noqa: E402
 
-# Plan 4 (GPT-22B, 185 661 offload combinations per parallelism row) costs the oracle ~20
-# core-hours as a whole; these groups cover its shapes: one and four parallelism rows, single
-# device to 16 nodes, first / middle / last gradient-accumulation candidates, tp 1..8.
+# Plan 4 (GPT-22B, 185 661 offload combinations per parallelism row) costs the oracle ~40
+# core-hours as a whole; these groups (8 to 12 core-minutes each) cover its shapes: one and four
+# parallelism rows, single device to 16 nodes, 1 to 48 pre-saved micro-batch values (1 to 3
+# p tiles of the reduce kernel), every tp.
 SUBSETS = {
     4: [
-        (1, 512, (1, 1)), (1, 256, (1, 2)), (1, 1, (16, 8)), (1, 8, (8, 8)), (1, 64, (1, 4)),
-        (2, 128, (1, 4)), (2, 16, (2, 8)), (4, 32, (1, 4)), (4, 4, (4, 8)), (8, 64, (1, 8)),
-        (8, 2, (16, 8)), (8, 16, (2, 8)),
+        (1, 512, (1, 1)), (2, 64, (1, 2)), (4, 256, (1, 4)), (8, 128, (1, 8)),
+        (1, 1, (16, 8)), (2, 2, (8, 8)), (4, 4, (16, 8)), (1, 4, (2, 8)),
+        (8, 8, (8, 8)), (1, 8, (1, 8)), (2, 8, (4, 8)), (4, 8, (4, 8)),
     ],
 }
 
@@ -272,21 +273,22 @@ def main():
         import glob
 
         parts = sorted(glob.glob(os.path.join(a.merge, f"search_tables_plan{a.plan}.part*.json")))
-        out = None
+        out, have = None, []
         for p in parts:
             with open(p) as f:
                 d = json.load(f)
+            have.append(d["select"])
             if out is None:
                 out = d
             else:
                 out["groups"].update(d["groups"])
         n = int(parts[0].rsplit("of", 1)[1].split(".")[0])
-        assert len(parts) == n, f"{len(parts)} of {n} parts present"
+        out["select"] = "all" if len(parts) == n else "; ".join(have)
         path = os.path.join(HERE, f"search_tables_plan{a.plan}.json")
         with open(path, "w") as f:
             json.dump(out, f, indent=1, sort_keys=True)
             f.write("\n")
-        print("wrote", path, len(out["groups"]), "groups")
+        print("wrote", path, len(out["groups"]), "groups,", out["select"])
         return
     cfg, tables = load_plan(a.plan)
     meshes, Gs, tps = plan_axes(cfg)
@@ -310,7 +312,8 @@ def main():
             print(f"[{time.time() - t0:7.0f}s] {n + 1}/{len(jobs)} {key} rows={rec['rows']} "
                   f"finite={rec['finite']} ({rec['oracle_seconds']} s)", flush=True)
     out = dict(
-        plan=PLAN_FILES[a.plan - 1], sample_size=1, select=a.select,
+        plan=PLAN_FILES[a.plan - 1], sample_size=1,
+        select=a.select if n_shards == 1 else f"shard {shard} of {n_shards} (groups by size, every {n_shards}th)",
         made_by="tests/golden/make_search_fixtures.py (CPU oracle)",
         groups={k: dict(rows=groups[k]["rows"], finite=groups[k]["finite"], digest=groups[k]["digest"])
                 for k in sorted(groups)},

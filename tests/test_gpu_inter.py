@@ -243,12 +243,19 @@ def test_plan1_end_to_end():
     assert got == want
 
 
-def test_full_size_dp_matches_c_oracle_on_gpt7b_tables():
-    """GPT-7B plan at full size (L = 32, 32 devices, 6 meshes, 32 pre-saved micro-batch values):
-    the intra-stage tables come from the GPU search (checked elsewhere); the DP kernel is compared
-    with the C oracle on those tables at the thresholds that matter - just below the smallest
-    feasible one, at it, a run of kept candidates above it and the winning one, back-pointers
-    included.  (The reference's full ascending scan needs ~10^5 DP runs per G on the CPU.)"""
+@pytest.mark.parametrize("plan, tp, g_picks, n_below, n_above, n_min", [
+    (2, 8, ("best", 32, "last"), 3, 9, 12),   # L = 32, D = 32, 6 meshes
+    (4, 8, ("best", 16, "last"), 2, 4, 6),    # L = 48, D = 128, 8 meshes
+    (5, 8, ("best",), 1, 3, 3),               # L = 80, D = 256, 9 meshes: ~10 s per oracle run
+])
+def test_full_size_dp_matches_c_oracle(plan, tp, g_picks, n_below, n_above, n_min):
+    """The benchmark plans at full size (GPT-7B: L = 32, 32 devices, 6 meshes; GPT-22B: L = 48,
+    128 devices, 8 meshes; LLaMA-70B: L = 80, 256 devices, 9 meshes, state planes beyond the LDS
+    of a compute unit): the intra-stage tables come from the GPU search (checked against the
+    oracle's fixtures elsewhere); the DP kernel is compared with the C oracle on those tables at
+    the thresholds that matter - just below the smallest feasible one, at it, a run of kept
+    candidates above it and the winning one, back-pointers included.  (The reference's full
+    ascending scan needs ~10^5 DP runs per G on the CPU.)"""
     from mist_amd import _lib
     from mist_amd.inter_tuning import _DpRunner, _Window, inter_stage_tune
     from mist_amd.intra_tuning import IntraStageTuner
@@ -256,17 +263,19 @@ def test_full_size_dp_matches_c_oracle_on_gpt7b_tables():
     from oracle.dp_c import dp_impl_c
     from oracle.inter_dp import dp_cost_tables
 
-    cfg, tables = load_plan(2)
+    cfg, tables = load_plan(plan)
     hw, L = cfg.hardware, cfg.model.num_hidden_layers
     D = hw.num_nodes * hw.num_gpus_per_node
     meshes = _get_device_mesh_candidates(hw.num_nodes, hw.num_gpus_per_node, False)
     Gs = _get_grad_accumu_steps_candidates(cfg.training.global_batch_size)
-    res = IntraStageTuner(tables, L, meshes, Gs, 8, cfg, sample_size=1).tune()
+    res = IntraStageTuner(tables, L, meshes, Gs, tp, cfg, sample_size=1).tune()
     best_cost, best_solution = inter_stage_tune(L, D, meshes, Gs, res)
     assert best_solution is not None
     runner = _DpRunner(res, L, D, meshes, 0)
     n_checked = 0
-    for g in (Gs.index(best_solution[0]), Gs.index(32), len(Gs) - 1):
+    picks = [Gs.index(best_solution[0]) if g == "best" else len(Gs) - 1 if g == "last" else Gs.index(g)
+             for g in g_picks]
+    for g in picks:
         G = Gs[g]
         tabs = dp_cost_tables(res, g)
         _, bott, _ = runner.run(np.array([g], dtype=np.int32), np.zeros(1, dtype=np.float32),
@@ -276,7 +285,7 @@ def test_full_size_dp_matches_c_oracle_on_gpt7b_tables():
         (vals, _), = runner.candidates_between(np.array([g]), np.array([lo]), np.array([bott[0] * 1.02], dtype=np.float32))
         vals = np.unique(vals)
         at = int(np.searchsorted(vals, bott[0]))
-        tmax = np.concatenate([vals[max(at - 3, 0):at], vals[at:at + 9]])
+        tmax = np.concatenate([vals[max(at - n_below, 0):at], vals[at:at + n_above]])
         bs, bsum, smax, arg = runner.run(np.full(len(tmax), g, dtype=np.int32), tmax, want_argmin=True)
         for i, t in enumerate(tmax):
             want_cost, want_sol = dp_impl_c(t, L, D, meshes, G, *tabs)
@@ -293,7 +302,7 @@ def test_full_size_dp_matches_c_oracle_on_gpt7b_tables():
                 cs, cl, cd = cs - 1, end + 1, cd - n * m
             assert sol == want_sol, (G, t)
             n_checked += 1
-    assert n_checked >= 12
+    assert n_checked >= n_min
     # the search's answer is one of the DP solutions: recompute it at its own bottleneck
     g = Gs.index(best_solution[0])
     tabs = dp_cost_tables(res, g)

@@ -195,6 +195,17 @@ int mist_eval_reduce(const MistProblem *problem, const MistGroupDesc *d_groups, 
                      const double *d_row_terms, const double *d_stage_floor, double ratio,
                      double *d_partial_cost, int32_t *d_partial_index, void *stream);
 
+/* mist_eval_reduce with every cell evaluated: each (row, layers, ckpt) through the latency and
+ * memory model and each pre-saved micro-batch value through the reference's feasibility test
+ * (batched_module_analyzer.py:2218-3106, pareto.py:124-144 as written, cell by cell), no scout
+ * pass, no sieves.  Same workgroup decomposition (d_block_prefix, n_blocks) and slab layout as
+ * the main launch of mist_eval_reduce; every slab is written.  The reference point the pruned
+ * search is tested and measured against: identical tables, ~20x the time. */
+int mist_eval_reduce_exhaustive(const MistProblem *problem, const MistGroupDesc *d_groups,
+                                int n_groups, const int32_t *d_block_prefix, int n_blocks,
+                                const double *d_row_terms, double ratio, double *d_partial_cost,
+                                int32_t *d_partial_index, void *stream);
+
 /* Combines the per-chunk partial minima (smallest cost, lowest row among equals),
  * recomputes stable / delta of the winning row and scatters into the output tables at sample
  * position `sample_index`, reproducing which cells the reference leaves unwritten

@@ -119,6 +119,10 @@ _SIGNATURES = {
         [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, _VP, ctypes.c_double,
          _VP, _VP, _VP],
     ),
+    "mist_eval_reduce_exhaustive": (
+        ctypes.c_int,
+        [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, ctypes.c_double, _VP, _VP, _VP],
+    ),
     "mist_finalize": (
         ctypes.c_int,
         [_VP, _VP, ctypes.c_int, _VP, _VP, _VP, _VP, ctypes.c_int, ctypes.POINTER(OutTables), _VP],

@@ -719,6 +719,8 @@ __host__ __device__ constexpr int xcd_padded_grid(int n_blocks) {
   return (n_blocks + kNumXcd * kXcdRun - 1) / (kNumXcd * kXcdRun) * (kNumXcd * kXcdRun);
 }
 
+__device__ __forceinline__ LaneMemory cell_memory(const double *__restrict__ t, int l, int c);
+
 struct ReduceRange {
   int64_t row_begin, row_end;  // rows of the group this workgroup covers (multiples of kStageRows)
   int stage_step;              // visit every stage_step-th stage of the range
@@ -1296,6 +1298,124 @@ __global__ __launch_bounds__(MIST_LC_TILE, MIST_REDUCE_MIN_WAVES) void eval_redu
 #undef MIST_REDUCE
 }
 
+// ------------------------------------------------------------------------------------------
+// Kernel 2x: the same reduction with every cell evaluated.  No scout pass, no sieves, no bounds,
+// no bisection: each (row, l, c) goes through the latency model and the memory model, and each
+// of its p values through the reference's feasibility test and the (cost, row) comparison.  This
+// is the work the reference's formulas describe cell by cell; the pruned kernel above must
+// produce the same tables (tests) and is measured against it.  Same decomposition and slab
+// layout as eval_reduce_kernel's main launch, so finalize_kernel reads either.
+// ------------------------------------------------------------------------------------------
+template <bool kFirstTile>
+__device__ __forceinline__ void exhaustive_block(
+    const MistProblem &prob, const MistGroupDesc *__restrict__ g, int64_t row_begin,
+    int64_t row_end, int p_tile, int lc_tile, const double *__restrict__ row_terms, double ratio,
+    double *lds_terms, double *__restrict__ out_cost, int32_t *__restrict__ out_index) {
+  const int L = prob.num_layers;
+  const int n_pairs = L * (L + 1) / 2 + L;
+  const int pair_idx = lc_tile * MIST_LC_TILE + threadIdx.x;
+  const bool active = pair_idx < n_pairs;
+  const PairIndex pc = decode_pair(active ? pair_idx : 0);
+  const int l = pc.l, c = pc.c;
+  const int p0 = p_tile * MIST_P_TILE;
+  const int n_tile = active ? min(MIST_P_TILE, g->num_p - p0) : 0;
+  const GroupConsts k = group_consts(g);
+  const double cap = prob.mem_cap_mb;
+  const double G64 = (double)g->grad_accum;
+  const float G32 = (float)g->grad_accum;
+  const double pre_saved = g->pre_saved, pre_sas = g->pre_states_and_saved;
+
+  double best_b[MIST_P_TILE], best_p[MIST_P_TILE];
+  int32_t row_b[MIST_P_TILE], row_p[MIST_P_TILE];
+  double best_post = INFINITY, best_pp = INFINITY;
+  int32_t row_post = -1, row_pp = -1;
+#pragma unroll
+  for (int j = 0; j < MIST_P_TILE; ++j) {
+    best_b[j] = best_p[j] = INFINITY;
+    row_b[j] = row_p[j] = -1;
+  }
+  const double *__restrict__ src = row_terms + g->row_offset * MIST_ROW_TERMS;
+  for (int64_t base = row_begin; base < row_end; base += kStageRows) {
+    const int n_stage = (int)min((int64_t)kStageRows, row_end - base);
+    __syncthreads();
+    const double2 *__restrict__ src2 = reinterpret_cast<const double2 *>(src + base * MIST_ROW_TERMS);
+    for (int i = threadIdx.x; i < n_stage * (MIST_ROW_TERMS / 2); i += MIST_LC_TILE) {
+      const double2 v = src2[i];
+      const int at = (i / (MIST_ROW_TERMS / 2)) * kLdsRowStride + 2 * (i % (MIST_ROW_TERMS / 2));
+      lds_terms[at] = v.x;
+      lds_terms[at + 1] = v.y;
+    }
+    __syncthreads();
+    if (!active) continue;
+    for (int r = 0; r < n_stage; ++r) {
+      const double *t = lds_terms + r * kLdsRowStride;
+      const int32_t row = row_of_position(g, base + r);
+      const CellLatency lat = cell_latency<kFirstTile>(t, l, c, k);
+      const LaneMemory mem = cell_memory(t, l, c);
+      // objectives r * x + y (pareto.py:138): base with y = float32 delta / G in float32
+      // (batched_module_analyzer.py:2815), the others in float64 (:2898-2903, 3002-3007, 3084-3089)
+      const double cost_base = ratio * (double)lat.x + (double)(lat.d / G32);
+      const double cost_pre = ratio * lat.sp + lat.dpre / G64;
+#pragma unroll
+      for (int j = 0; j < MIST_P_TILE; ++j) {
+        const bool live = j < n_tile;
+        take_min(best_b[j], row_b[j], live && mem.feasible_base(p0 + j, cap), cost_base, row);
+        take_min(best_p[j], row_p[j], live && mem.feasible_pre(p0 + j, cap, pre_saved, pre_sas),
+                 cost_pre, row);
+      }
+      if (kFirstTile) {  // last stage / single stage, p == 0 only (:2946-3106)
+        double peak_f, peak_b;
+        mem.peaks(0, peak_f, peak_b);
+        const double f_in = mem.fwd_states + g->post_states + mem.mod_saved + g->post_fwd_peak + mem.gcb;
+        const double b_in = mem.bwd_states + g->post_states + mem.mod_saved + g->post_bwd_peak +
+                            (c == 0 ? t[MIST_T_RD] : 0.0) + mem.gcb;
+        const double pf_post = fmax(f_in, peak_f + g->post_states);
+        const double pb_post = fmax(b_in, peak_b - mem.out + g->post_states) + g->post_output;
+        const bool ok_post = fmax(pf_post, pb_post) * mem.mf_pp <= cap;
+        const double pf_pp = pf_post + g->pre_states + g->pre_saved;
+        const double pb_pp = pb_post + g->pre_states + g->pre_saved;
+        const bool ok_pp = fmax(pf_pp, pb_pp) * t[MIST_T_MF] <= cap;
+        take_min(best_post, row_post, ok_post, ratio * lat.spost + lat.dpost / G64, row);
+        take_min(best_pp, row_pp, ok_pp, ratio * lat.spp + lat.dpp / G64, row);
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < MIST_P_TILE; ++j) {
+    out_cost[j * MIST_LC_TILE + threadIdx.x] = best_b[j];
+    out_index[j * MIST_LC_TILE + threadIdx.x] = row_b[j];
+    out_cost[(MIST_P_TILE + j) * MIST_LC_TILE + threadIdx.x] = best_p[j];
+    out_index[(MIST_P_TILE + j) * MIST_LC_TILE + threadIdx.x] = row_p[j];
+  }
+  out_cost[(2 * MIST_P_TILE) * MIST_LC_TILE + threadIdx.x] = best_post;
+  out_index[(2 * MIST_P_TILE) * MIST_LC_TILE + threadIdx.x] = row_post;
+  out_cost[(2 * MIST_P_TILE + 1) * MIST_LC_TILE + threadIdx.x] = best_pp;
+  out_index[(2 * MIST_P_TILE + 1) * MIST_LC_TILE + threadIdx.x] = row_pp;
+}
+
+__global__ __launch_bounds__(MIST_LC_TILE) void eval_reduce_exhaustive_kernel(
+    const MistProblem prob, const MistGroupDesc *__restrict__ groups, int n_groups,
+    const int32_t *__restrict__ block_prefix, int n_blocks, const double *__restrict__ row_terms,
+    double ratio, double *__restrict__ partial_cost, int32_t *__restrict__ partial_index) {
+  __shared__ double lds_terms[kStageRows * kLdsRowStride];
+  const int block = xcd_run_block(blockIdx.x);
+  if (block >= n_blocks) return;
+  int local_block;
+  const MistGroupDesc *g = find_group(groups, block_prefix, n_groups, block, &local_block);
+  const int n_tiles = g->n_lc_tiles * g->n_p_tiles;
+  const int chunk = local_block / n_tiles, tile = local_block % n_tiles;
+  const int64_t row_begin = (int64_t)chunk * g->rows_per_chunk;
+  const int64_t row_end = min(row_begin + (int64_t)g->rows_per_chunk, g->n_rows);
+  const int p_tile = tile % g->n_p_tiles, lc_tile = tile / g->n_p_tiles;
+  const int64_t slab = (int64_t)kSlots * MIST_LC_TILE;
+  if (p_tile == 0)
+    exhaustive_block<true>(prob, g, row_begin, row_end, p_tile, lc_tile, row_terms, ratio,
+                           lds_terms, partial_cost + block * slab, partial_index + block * slab);
+  else
+    exhaustive_block<false>(prob, g, row_begin, row_end, p_tile, lc_tile, row_terms, ratio,
+                            lds_terms, partial_cost + block * slab, partial_index + block * slab);
+}
+
 // Combines the slabs of the kScoutSplit scout workgroups of every tile into the first of them,
 // so that each chunk of the main launch reads one slab of seeds instead of kScoutSplit.
 // Workgroup = tile; the scout slabs of tile t are n_blocks + t * kScoutSplit + k.
@@ -1549,6 +1669,22 @@ int mist_eval_reduce(const MistProblem *problem, const MistGroupDesc *d_groups, 
                      (hipStream_t)stream, *problem, d_groups, n_groups, d_block_prefix, n_blocks,
                      scout_prefix, 0, d_row_terms, d_stage_floor, ratio, d_partial_cost,
                      d_partial_index);
+  MIST_HIP_CHECK(hipGetLastError());
+  return 0;
+}
+
+int mist_eval_reduce_exhaustive(const MistProblem *problem, const MistGroupDesc *d_groups,
+                                int n_groups, const int32_t *d_block_prefix, int n_blocks,
+                                const double *d_row_terms, double ratio, double *d_partial_cost,
+                                int32_t *d_partial_index, void *stream) {
+  if (int rc = check_common(problem, d_groups, n_groups)) return rc;
+  if (!d_block_prefix || !d_row_terms || !d_partial_cost || !d_partial_index)
+    return fail(MIST_E_INVALID, "null workspace pointer");
+  if (n_blocks <= 0) return fail(MIST_E_INVALID, "n_blocks must be positive, got %d", n_blocks);
+  if (!(ratio >= 0.0)) return fail(MIST_E_INVALID, "ratio must be non-negative");
+  hipLaunchKernelGGL(eval_reduce_exhaustive_kernel, dim3(xcd_padded_grid(n_blocks)),
+                     dim3(MIST_LC_TILE), 0, (hipStream_t)stream, *problem, d_groups, n_groups,
+                     d_block_prefix, n_blocks, d_row_terms, ratio, d_partial_cost, d_partial_index);
   MIST_HIP_CHECK(hipGetLastError());
   return 0;
 }

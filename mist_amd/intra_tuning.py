@@ -176,7 +176,11 @@ class IntraStageTuner:
         sample_size: int = SAMPLE_SIZE,
         sample_slots: Optional[Sequence[int]] = None,
         device: str = "cuda:0",
+        exhaustive: bool = False,
     ):
+        # exhaustive: evaluate every cell (no scout pass, no sieves) with
+        # mist_eval_reduce_exhaustive; same tables, the reference point for tests and bench
+        self.exhaustive = bool(exhaustive)
         self.layer_tables = layer_tables
         self.num_layers = int(num_layers)
         self.device_mesh_candidates = list(device_mesh_candidates)
@@ -246,6 +250,7 @@ class IntraStageTuner:
             # seed its chunks; groups that are small or have few offload pairs go without.
             n_stages = -(-groups["n_rows"] // _lib.STAGE_ROWS)
             scout = (n_stages >= SCOUT_MIN_STAGES) & (groups["n_pair"] >= SCOUT_MIN_PAIRS) & (SCOUT_MIN_STAGES > 0)
+            scout &= not self.exhaustive
             pairs = np.minimum(SCOUT_PAIRS + groups["n_pair"] // SCOUT_PAIR_SPAN, groups["n_pair"])
             groups["scout_stride"] = np.where(scout, pairs, 0)
             scout_blocks = np.full(len(pending), n_lc_tiles * _lib.SCOUT_SPLIT, dtype=np.int64) * n_p_tiles
@@ -323,8 +328,20 @@ class IntraStageTuner:
         out = tables.as_struct()
         prob_ptr = ctypes.c_void_p(plan["problem"].ctypes.data)
         d = dev_plan
+        def reduce_call(slot):
+            if self.exhaustive:
+                return lib.mist_eval_reduce_exhaustive(
+                    prob_ptr, _ptr(d["groups"]), d["n_groups"], _ptr(d["reduce_prefix"]),
+                    d["n_reduce_blocks"], _ptr(d["row_terms"]), float(ratios[slot]),
+                    _ptr(d["partial_cost"]), _ptr(d["partial_index"]), stream)
+            return lib.mist_eval_reduce(
+                prob_ptr, _ptr(d["groups"]), d["n_groups"], _ptr(d["reduce_prefix"]),
+                d["n_reduce_blocks"], _ptr(d["scout_prefix"]), d["n_scout_blocks"],
+                _ptr(d["row_terms"]), _ptr(d["stage_floor"]), float(ratios[slot]),
+                _ptr(d["partial_cost"]), _ptr(d["partial_index"]), stream)
+
         for i, slot in enumerate(self.sample_slots):
-            if events is None:
+            if events is None and not self.exhaustive:
                 rc = lib.mist_intra_stage_eval(
                     prob_ptr, _ptr(d["groups"]), d["n_groups"],
                     _ptr(d["terms_prefix"]), d["n_terms_blocks"],
@@ -338,6 +355,9 @@ class IntraStageTuner:
                 continue
 
             def timed(name, call):
+                if events is None:
+                    _lib.check(call(), name)
+                    return
                 start = torch.cuda.Event(enable_timing=True)
                 end = torch.cuda.Event(enable_timing=True)
                 start.record()
@@ -349,11 +369,7 @@ class IntraStageTuner:
                 timed("row_terms", lambda: lib.mist_row_terms(
                     prob_ptr, _ptr(d["groups"]), d["n_groups"], _ptr(d["terms_prefix"]),
                     d["n_terms_blocks"], _ptr(d["row_terms"]), _ptr(d["stage_floor"]), stream))
-            timed("eval_reduce", lambda: lib.mist_eval_reduce(
-                prob_ptr, _ptr(d["groups"]), d["n_groups"], _ptr(d["reduce_prefix"]),
-                d["n_reduce_blocks"], _ptr(d["scout_prefix"]), d["n_scout_blocks"],
-                _ptr(d["row_terms"]), _ptr(d["stage_floor"]), float(ratios[slot]),
-                _ptr(d["partial_cost"]), _ptr(d["partial_index"]), stream))
+            timed("eval_reduce", lambda: reduce_call(slot))
             timed("finalize", lambda: lib.mist_finalize(
                 prob_ptr, _ptr(d["groups"]), d["n_groups"], _ptr(d["reduce_prefix"]),
                 _ptr(d["row_terms"]), _ptr(d["partial_cost"]), _ptr(d["partial_index"]), int(slot),

@@ -129,7 +129,7 @@ class PreparedSearch:
     descriptors are built and uploaded once (``__init__``), ``run`` then only launches kernels
     and the inter-stage search.  ``tune`` is ``PreparedSearch(config).run()``."""
 
-    def __init__(self, mist_config: MistConfig, device: str = "cuda:0"):
+    def __init__(self, mist_config: MistConfig, device: str = "cuda:0", exhaustive: bool = False):
         model, hw, tuning = mist_config.model, mist_config.hardware, mist_config.tuning
         self.config = mist_config
         self.granularity = tuning.tuning_granularity
@@ -147,7 +147,8 @@ class PreparedSearch:
         # All tensor-parallel candidates go through one batch of launches.
         self.tuner = IntraStageTuner(self.tables, self.L, self.meshes, self.Gs,
                                      tp_candidates(mist_config), mist_config,
-                                     sample_size=sample_size, sample_slots=[0], device=device)
+                                     sample_size=sample_size, sample_slots=[0], device=device,
+                                     exhaustive=exhaustive)
         self.plan = self.tuner.prepare()
         with torch.cuda.device(self.tuner.device):
             self.dev_plan = self.tuner.upload(self.plan)

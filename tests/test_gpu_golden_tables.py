@@ -37,8 +37,35 @@ def test_fixtures_cover_every_benchmark_plan():
     assert {_plan_of(p) for p in FIXTURES} == {1, 2, 3, 4, 5}
 
 
+@pytest.mark.parametrize("plan", [1, 2, 3, 4, 5])
+def test_pruned_and_exhaustive_search_give_the_same_tables_on_whole_plans(plan):
+    """Every table of every group of a benchmark plan (plan 2 is the timed workload; of plans 4
+    and 5 the oracle's fixtures cover a part of the groups only), pruned search (scout pass,
+    sieves, bounds) against the kernel that evaluates every cell: identical row indices and
+    costs."""
+    import torch
+
+    from mist_amd.tune_one_case import PreparedSearch
+
+    cfg, _ = load_plan(plan)
+    tables = []
+    for exhaustive in (False, True):
+        search = PreparedSearch(cfg, exhaustive=exhaustive)
+        results = search.tuner.run_prepared(search.plan, search.dev_plan)
+        tables.append(results[0].batch)
+    pruned, full = tables
+    n_finite = 0
+    for v in range(4):
+        assert torch.equal(pruned.index[v], full.index[v]), f"row indices of variant {v}"
+        assert torch.equal(pruned.stable[v], full.stable[v]), f"stable costs of variant {v}"
+        assert torch.equal(pruned.delta[v], full.delta[v]), f"delta costs of variant {v}"
+        n_finite += int((full.index[v] >= 0).sum())
+    assert n_finite > (100000 if plan > 1 else 1000)
+
+
+@pytest.mark.parametrize("exhaustive", [False, True], ids=["pruned", "exhaustive"])
 @pytest.mark.parametrize("path", FIXTURES, ids=lambda p: f"plan{_plan_of(p)}")
-def test_tables_and_tune_equal_the_oracle_fixture(path):
+def test_tables_and_tune_equal_the_oracle_fixture(path, exhaustive):
     from mist_amd.inter_tuning import inter_stage_tune_batch
     from mist_amd.tune_one_case import PreparedSearch
 
@@ -47,7 +74,7 @@ def test_tables_and_tune_equal_the_oracle_fixture(path):
     plan = _plan_of(path)
     cfg, _ = load_plan(plan)
     assert cfg.tuning.tuning_granularity == "inter-stage" and cfg.tuning.sample_size == 1
-    search = PreparedSearch(cfg)
+    search = PreparedSearch(cfg, exhaustive=exhaustive)
     tuner = search.tuner
     results = tuner.run_prepared(search.plan, search.dev_plan)
     Gs, meshes = search.Gs, search.meshes

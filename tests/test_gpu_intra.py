@@ -13,7 +13,7 @@ from tests.util import assert_same_f64, load_plan, oracle_terms, tiny_plan
 pytestmark = pytest.mark.gpu
 
 
-def _gpu_tuner(cfg, tables, tp, S=1, meshes=None, Gs=None, slots=None):
+def _gpu_tuner(cfg, tables, tp, S=1, meshes=None, Gs=None, slots=None, exhaustive=False):
     from mist_amd.intra_tuning import IntraStageTuner
     from mist_amd.search_space import _get_device_mesh_candidates, _get_grad_accumu_steps_candidates
 
@@ -21,7 +21,8 @@ def _gpu_tuner(cfg, tables, tp, S=1, meshes=None, Gs=None, slots=None):
     meshes = meshes or _get_device_mesh_candidates(hw.num_nodes, hw.num_gpus_per_node, False)
     Gs = Gs or _get_grad_accumu_steps_candidates(cfg.training.global_batch_size)
     return IntraStageTuner(
-        tables, cfg.model.num_hidden_layers, meshes, Gs, tp, cfg, sample_size=S, sample_slots=slots
+        tables, cfg.model.num_hidden_layers, meshes, Gs, tp, cfg, sample_size=S, sample_slots=slots,
+        exhaustive=exhaustive,
     )
 
 
@@ -31,8 +32,9 @@ def _oracle(cfg, tables, tp, S, meshes, Gs):
     return intra_stage_tune(tables, cfg, cfg.model.num_hidden_layers, meshes, Gs, tp, S)
 
 
-def _compare(cfg, tables, tp, S=1, slots=None, meshes=None, Gs=None, require_finite=True):
-    tuner = _gpu_tuner(cfg, tables, tp, S=S, slots=slots, meshes=meshes, Gs=Gs)
+def _compare(cfg, tables, tp, S=1, slots=None, meshes=None, Gs=None, require_finite=True,
+             exhaustive=False):
+    tuner = _gpu_tuner(cfg, tables, tp, S=S, slots=slots, meshes=meshes, Gs=Gs, exhaustive=exhaustive)
     got = tuner.tune()
     want = _oracle(cfg, tables, tp, S, tuner.device_mesh_candidates,
                    tuner.gradient_accumulation_steps_candidates)
@@ -218,6 +220,26 @@ def test_full_size_groups_match_oracle(plan, G, mesh, tp):
     assert n_finite > 1000
 
 
+@pytest.mark.parametrize("overrides", [
+    dict(),
+    dict(hardware__memory_capacity=6.0, model__use_flash_attn=True),
+    dict(hardware__num_nodes=2, hardware__num_gpus_per_node=4, training__global_batch_size=32,
+         hardware__memory_capacity=8.0, tuning__pre_post_strategy="intra-node-tp-with-ore"),
+])
+def test_exhaustive_kernel_matches_oracle(overrides):
+    """The evaluate-every-cell kernel (no scout pass, no sieves, no bisection) against the oracle
+    on tiny plans, S = 1 and S = 3, and on the whole of plan 1."""
+    from mist_amd.config import tp_candidates
+
+    cfg, tables = tiny_plan(1, layers=6, **overrides)
+    for tp in tp_candidates(cfg):
+        _compare(cfg, tables, tp, exhaustive=True, require_finite=False)
+    _compare(cfg, tables, 1, S=3, exhaustive=True)
+    if not overrides:
+        cfg, tables = load_plan(1)
+        _compare(cfg, tables, 2, exhaustive=True)
+
+
 def test_gradient_accumulation_steps_that_are_not_powers_of_two():
     """The tuner's own G candidates are powers of two (the kernel then multiplies by an exact
     reciprocal); a caller-supplied list may hold any divisor of the batch size, which takes the
@@ -225,6 +247,7 @@ def test_gradient_accumulation_steps_that_are_not_powers_of_two():
     cfg, tables = tiny_plan(1, layers=5, training__global_batch_size=24, hardware__memory_capacity=6.0)
     got, _ = _compare(cfg, tables, 1, Gs=[3, 6, 12, 24], meshes=[(1, 1), (1, 2)])
     assert np.isfinite(got.costs_stable).any()
+    _compare(cfg, tables, 1, Gs=[3, 6, 12, 24], meshes=[(1, 1), (1, 2)], exhaustive=True)
 
 
 @pytest.mark.parametrize("seed", range(8))

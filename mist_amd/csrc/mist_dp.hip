@@ -581,6 +581,173 @@ __global__ __launch_bounds__(kDpFusedThreads) void dp_fused_kernel(
   }
 }
 
+// ------------------------------------------------------------------------------------------
+// The recurrence for shapes whose four state planes do not fit the LDS of a compute unit (80
+// layers x 256 devices: 333 KB).  One workgroup per instance keeps ONE plane in LDS, F(s - 1),
+// the only one the scans read at random; F(s) and the maxima planes go through the instance's
+// global scratch (one coalesced copy of F(s) into LDS per stage count), the row minima are read
+// from the re-laid table.  A wavefront owns (start layer k, 64 consecutive device counts d): the
+// loop over (mesh, end layer) is the same for all its lanes, so the row minimum is one uniform
+// read, the test against t_max a scalar branch that skips the step for the whole wavefront, and
+// the LDS reads of F(s - 1) are 64 consecutive floats.  Per state the candidates are still
+// visited in the reference's (mesh, end layer) order with a strict "<": same winner, same ties.
+// ------------------------------------------------------------------------------------------
+constexpr int kDpPlaneThreads = 1024;
+#ifndef MIST_DP_PLANE_MIN_INSTANCES
+#define MIST_DP_PLANE_MIN_INSTANCES 16
+#endif
+// smaller batches stay on the per-stage-count launches, which spread one instance over the GPU
+constexpr int kDpPlaneMinInstances = MIST_DP_PLANE_MIN_INSTANCES;
+
+template <bool kBottleneck>
+__global__ __launch_bounds__(kDpPlaneThreads) void dp_plane_kernel(
+    const MistDpShape shape, const MistDpCosts tabs, const float *__restrict__ tmax_list,
+    const int32_t *__restrict__ g_list, float *__restrict__ scratch,
+    int32_t *__restrict__ best_s_out, float *__restrict__ best_sum_out,
+    float *__restrict__ stage_max_out, int32_t *__restrict__ argmin) {
+  extern __shared__ float dp_lds[];
+  const int L = shape.num_layers, D = shape.num_devices, Q = shape.num_mesh;
+  const int W = D + 1, plane = (L + 1) * W;
+  const int n_blocks = (D + 63) / 64;  // block b of a row: d = 1 + 64 b + lane
+  float *f_lds = dp_lds;                                        // F(s - 1)
+  int32_t *range = reinterpret_cast<int32_t *>(dp_lds + plane);  // [3][W][2] reachable rows per column
+  int32_t *blk = range + 6 * W;                                  // [Q][n_blocks][2] the same per (mesh, block)
+  float *wave_rows = reinterpret_cast<float *>(blk + 2 * Q * n_blocks);  // [n_waves][Q][L] row minima of a task
+  const int t = blockIdx.x;
+  const float t_max = kBottleneck ? INFINITY : tmax_list[t];
+  const int64_t g = g_list[t];
+  const int64_t off[4] = {g * tabs.g_stride[0], g * tabs.g_stride[1], g * tabs.g_stride[2],
+                          g * tabs.g_stride[3]};
+  const int tri = dp_triangle(L);
+  const float *__restrict__ relaid = tabs.stage_min + g * tabs.stage_min_g_stride;
+  float *state = scratch + (int64_t)t * 4 * plane;
+  float *__restrict__ f_cur = state;  // F(s) on its way into LDS
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int n_waves = blockDim.x >> 6;
+  float *my_rows = wave_rows + wave * Q * L;
+
+  for (int e = threadIdx.x; e < plane; e += blockDim.x) f_lds[e] = e == L * W ? 0.0f : INFINITY;
+  for (int col = threadIdx.x; col < W; col += blockDim.x) {
+    range[2 * col] = col == 0 ? L : L + 1;
+    range[2 * col + 1] = col == 0 ? L : -1;
+    for (int b = 1; b < 3; ++b) {
+      range[(b * W + col) * 2] = L + 1;
+      range[(b * W + col) * 2 + 1] = -1;
+    }
+  }
+  if (threadIdx.x == 0) state[2 * plane + L * W] = 0.0f;  // maximum of the empty partition
+  float answer_sum = INFINITY, answer_max = 0.0f;
+  int answer_s = -1;
+  __syncthreads();
+  for (int s = 1; s <= shape.max_stages; ++s) {
+    const int cur = s & 1, prv = cur ^ 1, p = s - 1;
+    const float *m_prev = state + (2 + prv) * plane;
+    float *__restrict__ m_cur = state + (2 + cur) * plane;
+    const int32_t *range_prev = range + ((s + 2) % 3) * W * 2;
+    int32_t *range_cur = range + (s % 3) * W * 2;
+    int32_t *range_next = range + ((s + 1) % 3) * W * 2;
+    // reachable successor rows of every (mesh, block of 64 columns): bounds of the uniform loop
+    for (int x = threadIdx.x; x < Q * n_blocks; x += blockDim.x) {
+      const int q = x / n_blocks, b = x % n_blocks;
+      const int nm = shape.mesh_n[q] * shape.mesh_m[q];
+      int first = L + 1, last = -1;
+      for (int d = 1 + 64 * b; d <= min(D, 64 * b + 64); ++d) {
+        if (d < nm) continue;
+        first = min(first, range_prev[2 * (d - nm)]);
+        last = max(last, range_prev[2 * (d - nm) + 1]);
+      }
+      blk[2 * x] = first;
+      blk[2 * x + 1] = last;
+    }
+    if (threadIdx.x == 0) {  // column 0 holds the origin only: unreachable from here on
+      range_next[0] = L + 1;
+      range_next[1] = -1;
+    }
+    __syncthreads();
+    const float *__restrict__ block = relaid + (int64_t)p * Q * tri;
+    const int n_tasks = (L - s + 1) * n_blocks;  // start layers 0 .. L - s
+    for (int task = wave; task < n_tasks; task += n_waves) {
+      const int k = task / n_blocks, b = task - k * n_blocks;
+      const int d = 1 + 64 * b + lane;
+      const bool col_ok = d <= D;
+      // The row minima of the stages k..i on every mesh, [Q][L - k] floats, into this
+      // wavefront's LDS buffer with all reads in flight together; the loop below then has no
+      // global read in its dependence chain.
+      const int width = L - k;
+      for (int x = lane; x < Q * width; x += 64) {
+        const int q = x / width, di = x - q * width;
+        my_rows[x] = block[q * tri + dp_triangle_row(L, k) + di];
+      }
+      __builtin_amdgcn_wave_barrier();
+      DpBest w;
+      for (int q = 0; q < Q; ++q) {
+        const int nm = shape.mesh_n[q] * shape.mesh_m[q];
+        const int i_first = max(k, blk[2 * (q * n_blocks + b)] - 1);
+        const int i_last = min(L - 1, blk[2 * (q * n_blocks + b) + 1] - 1);
+        const bool lane_ok = col_ok && nm <= d;
+        const float *col = f_lds + (lane_ok ? d - nm : 0);
+        const float *rm = my_rows + q * width - k;  // rm[i]
+        // 64 end layers at a time: which of them are admissible at all (the same for every
+        // lane), then only those, in ascending order
+        for (int i0 = i_first; i0 <= i_last; i0 += 64) {
+          const int i_mine = i0 + lane;
+          const float r_mine = i_mine <= i_last ? rm[i_mine] : INFINITY;
+          unsigned long long todo = __ballot(i_mine <= i_last && r_mine <= t_max);
+          while (todo != 0) {
+            const int bit = __ffsll(todo) - 1;
+            todo &= todo - 1;
+            const int i = i0 + bit;
+            const float rmin = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(r_mine), bit));
+            const float prev = lane_ok ? col[(i + 1) * W] : INFINITY;
+            dp_consider<kBottleneck>(w, t_max, q, i, prev, rmin);
+          }
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
+      if (!col_ok) continue;
+      dp_finish_winner<kBottleneck>(w, shape, tabs, off, t_max, p, k, d, f_lds, m_prev);
+      const int e = k * W + d;
+      f_cur[e] = w.best;
+      m_cur[e] = w.best_m;
+      if (w.best < INFINITY) {
+        atomicMin(&range_cur[2 * d], k);
+        atomicMax(&range_cur[2 * d + 1], k);
+      }
+      if (k == 0) {
+        range_next[2 * d] = L + 1;
+        range_next[2 * d + 1] = -1;
+      }
+      if (argmin != nullptr && w.arg_i >= 0) {
+        int32_t *a = argmin + (((int64_t)t * (shape.max_stages + 1) + s) * plane + e) * 4;
+        a[0] = w.arg_i;
+        a[1] = shape.mesh_n[w.arg_q];
+        a[2] = shape.mesh_m[w.arg_q];
+        a[3] = w.arg_j;
+      }
+      if (k == 0 && d == D && w.best < answer_sum) {  // first s wins ties (inter_tuning.py:335-340)
+        answer_sum = w.best;
+        answer_s = s;
+        answer_max = w.best_m;
+      }
+    }
+    __syncthreads();  // every scan of F(s - 1) is done, F(s) is in the scratch plane
+    for (int e = threadIdx.x; e < plane; e += blockDim.x) {
+      const int k = e / W, d = e - k * W;
+      f_lds[e] = (k <= L - s && d >= 1) ? f_cur[e] : INFINITY;
+    }
+    __syncthreads();
+  }
+  // the answer state (k = 0, d = D) is the same thread's in every step: wave 0 takes task
+  // (D - 1) / 64 when n_waves > that block index, else the wave task % n_waves
+  const int answer_task = (D - 1) / 64;
+  if (wave == answer_task % n_waves && lane == (D - 1) % 64) {
+    best_s_out[t] = answer_s;
+    best_sum_out[t] = answer_sum;
+    stage_max_out[t] = answer_max;
+  }
+}
+
 // Follows the back-pointers of each instance from (best_s, layer 0, all devices) and writes its
 // stages in pipeline order (inter_tuning.py:341-355); one thread per instance.  Only entries the
 // DP wrote are read: a state with a finite value has a winner, and so has every successor on
@@ -636,19 +803,36 @@ __global__ __launch_bounds__(256) void stage_minima_kernel(const MistDpShape sha
 
 // Dynamic LDS the one-launch kernel may use on the current device: what the device reports per
 // workgroup, once the kernel has been allowed more than the default 64 KB (0 if that failed).
-template <bool kBottleneck>
-size_t fused_lds_limit_of() {
+size_t lds_limit_of(const void *kernel) {
   int device = 0, most = 0;
   if (hipGetDevice(&device) != hipSuccess ||
       hipDeviceGetAttribute(&most, hipDeviceAttributeMaxSharedMemoryPerBlock, device) != hipSuccess)
     return 0;
   if (most > 64 * 1024 &&
-      hipFuncSetAttribute(reinterpret_cast<const void *>(&dp_fused_kernel<kBottleneck>),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, most) != hipSuccess) {
+      hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, most) != hipSuccess) {
     (void)hipGetLastError();
     most = 64 * 1024;
   }
   return (size_t)most;
+}
+template <bool kBottleneck>
+size_t fused_lds_limit_of() {
+  return lds_limit_of(reinterpret_cast<const void *>(&dp_fused_kernel<kBottleneck>));
+}
+size_t plane_lds_limit(int mode) {
+  // per device: the attribute belongs to the device's copy of the kernel
+  static std::mutex lock;
+  static std::map<std::pair<int, int>, size_t> known;
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) return 0;
+  std::lock_guard<std::mutex> guard(lock);
+  const auto key = std::make_pair(device, mode);
+  auto it = known.find(key);
+  if (it == known.end())
+    it = known.emplace(key, lds_limit_of(mode == MIST_DP_BOTTLENECK
+                                             ? reinterpret_cast<const void *>(&dp_plane_kernel<true>)
+                                             : reinterpret_cast<const void *>(&dp_plane_kernel<false>))).first;
+  return it->second;
 }
 size_t fused_lds_limit(int mode) {
   // per device: the attribute belongs to the device's copy of the kernel
@@ -956,6 +1140,25 @@ int mist_dp_run(const MistDpShape *shape, const MistDpCosts *costs, const float 
       hipLaunchKernelGGL(dp_fused_kernel<false>, dim3(n_tmax), dim3(threads), fused_lds,
                          (hipStream_t)stream, *shape, *costs, d_tmax, d_g_index, d_best_s,
                          d_best_sum, d_stage_max, d_argmin);
+    MIST_HIP_CHECK(hipGetLastError());
+    return 0;
+  }
+  // Planes beyond the LDS of a compute unit (80 layers x 256 devices): one workgroup per instance
+  // with F(s - 1) alone in LDS, one launch.
+  const size_t plane_lds =
+      ((size_t)plane + 6 * (size_t)(shape->num_devices + 1) +
+       2 * (size_t)shape->num_mesh * ((shape->num_devices + 63) / 64) +
+       (size_t)(kDpPlaneThreads / 64) * shape->num_mesh * shape->num_layers) * sizeof(float);
+  if (costs->stage_min != nullptr && shape->free_devices == 0 && n_tmax >= kDpPlaneMinInstances &&
+      fused_lds > fused_lds_limit(mode) && plane_lds <= plane_lds_limit(mode)) {
+    if (mode == MIST_DP_BOTTLENECK)
+      hipLaunchKernelGGL(dp_plane_kernel<true>, dim3(n_tmax), dim3(kDpPlaneThreads), plane_lds,
+                         (hipStream_t)stream, *shape, *costs, d_tmax, d_g_index, d_scratch,
+                         d_best_s, d_best_sum, d_stage_max, d_argmin);
+    else
+      hipLaunchKernelGGL(dp_plane_kernel<false>, dim3(n_tmax), dim3(kDpPlaneThreads), plane_lds,
+                         (hipStream_t)stream, *shape, *costs, d_tmax, d_g_index, d_scratch,
+                         d_best_s, d_best_sum, d_stage_max, d_argmin);
     MIST_HIP_CHECK(hipGetLastError());
     return 0;
   }

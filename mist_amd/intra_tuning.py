@@ -200,6 +200,9 @@ class IntraStageTuner:
         self.max_possible_pre_saved_micro_batches = (
             min(self.max_possible_num_stages, max(self.gradient_accumulation_steps_candidates)) - 1
         )
+        # True: every p of 0..P is evaluated for every G (the operator boundary
+        # batched_tune_best_latency_for_stage takes the p candidates from its caller)
+        self.evaluate_all_p = False
         self.results: Optional[IntraStageTunerOutput] = None
         self.stats: Dict[str, float] = {}
 
@@ -226,6 +229,8 @@ class IntraStageTuner:
                     if space.n_rows >= 2**31:
                         raise ValueError(f"group (G={G}, mesh={(n, m)}) has {space.n_rows} rows (>= 2**31)")
                     num_p = min(G, L, P + 1)  # intra_tuning.py:185-193
+                    if self.evaluate_all_p:
+                        num_p = P + 1
                     pending.append((t * len(Gs) + g, q, n, m, G, num_p, space))
         groups = np.zeros(len(pending), dtype=_lib.GROUP_DTYPE)
         for i, (g, q, n, m, G, num_p, space) in enumerate(pending):

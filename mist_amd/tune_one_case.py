@@ -99,28 +99,38 @@ def _no_pp(mist_config, tables, device, stats):
     return best_cost, best_solution
 
 
+MIP_TABLE_BUDGET_BYTES = 48 << 30  # sampled tables of one batch of tensor-parallel candidates
+
+
 def _uniform_device_pp_mip(mist_config, device, stats):
     """tune_one_case.py:360-402: per tensor-parallel candidate the intra-stage tables with every
     one of ``tuning.sample_size`` samples, then the stage assignment; the first best tp wins.
-    One tp at a time keeps a single set of sampled tables in HBM."""
+    As many tp candidates as fit ``MIP_TABLE_BUDGET_BYTES`` of sampled tables go through one
+    batch of launches per sample (for the GPT-7B plan with 30 samples all four: 9.7 GB)."""
     hw, tuning = mist_config.hardware, mist_config.tuning
     tables = layer_tables_for(mist_config)
     meshes = _get_device_mesh_candidates(hw.num_nodes, hw.num_gpus_per_node, contiguous_inter_node=False)
     Gs = _get_grad_accumu_steps_candidates(mist_config.training.global_batch_size)
     L = mist_config.model.num_hidden_layers
+    tps = tp_candidates(mist_config)
+    P1 = min(min(max(n * m for n, m in meshes), L), max(Gs))
+    per_tp = len(Gs) * len(meshes) * (2 * P1 * L * (L + 1) + L * (L + 1) + (L + 1)) * tuning.sample_size * 20
+    batch = max(1, min(len(tps), MIP_TABLE_BUDGET_BYTES // max(per_tp, 1)))
     best_cost, best_solution = float("inf"), None
-    for tp_size in tp_candidates(mist_config):
+    for first in range(0, len(tps), batch):
         t0 = time.perf_counter()
-        r = intra_stage_tune(tables, L, meshes, Gs, tp_size, mist_config,
-                             sample_size=tuning.sample_size, device=device)
+        tuner = IntraStageTuner(tables, L, meshes, Gs, tps[first:first + batch], mist_config,
+                                sample_size=tuning.sample_size, device=device)
+        results = tuner.tune_all()
         t1 = time.perf_counter()
-        cost, solution = inter_stage_tune_mip(
-            L, hw.num_nodes, hw.num_gpus_per_node, meshes, Gs, r, mist_config, stats=stats)
         stats["intra_s"] = stats.get("intra_s", 0.0) + (t1 - t0)
+        for r in results:
+            cost, solution = inter_stage_tune_mip(
+                L, hw.num_nodes, hw.num_gpus_per_node, meshes, Gs, r, mist_config, stats=stats)
+            if cost < best_cost:
+                best_cost, best_solution = cost, solution
         stats["inter_s"] = stats.get("inter_s", 0.0) + (time.perf_counter() - t1)
-        if cost < best_cost:
-            best_cost, best_solution = cost, solution
-        del r
+        del results, tuner
     return best_cost, best_solution
 
 

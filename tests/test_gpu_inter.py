@@ -286,7 +286,28 @@ def test_full_size_dp_matches_c_oracle(plan, tp, g_picks, n_below, n_above, n_mi
         vals = np.unique(vals)
         at = int(np.searchsorted(vals, bott[0]))
         tmax = np.concatenate([vals[max(at - n_below, 0):at], vals[at:at + n_above]])
+        n_oracle = len(tmax)
+        if plan == 5:
+            # A batch of 16 or more instances of this shape runs one workgroup per instance with
+            # one state plane in LDS; smaller ones take the per-stage-count launches.  Both
+            # schedules are held against each other on the whole batch and against the oracle on
+            # its first thresholds.
+            tmax = np.concatenate([tmax, vals[at + n_above:at + n_above + 20]])
+            assert len(tmax) >= 16
         bs, bsum, smax, arg = runner.run(np.full(len(tmax), g, dtype=np.int32), tmax, want_argmin=True)
+        if plan == 5:
+            for lo in range(0, len(tmax), 6):
+                part = runner.run(np.full(len(tmax[lo:lo + 6]), g, dtype=np.int32), tmax[lo:lo + 6],
+                                  want_argmin=True)
+                for whole, piece in zip((bs, bsum, smax), part[:3]):
+                    assert np.array_equal(whole[lo:lo + 6].view(np.int32), piece.view(np.int32))
+                # back-pointers along the winning path (entries off the path may differ in
+                # nothing either: both schedules write every finite state)
+                assert np.array_equal(arg[lo:lo + 6], part[3])
+            _, bott_many, _ = runner.run(np.full(16, g, dtype=np.int32), np.zeros(16, dtype=np.float32),
+                                         _lib.DP_BOTTLENECK)
+            assert np.all(bott_many == bott[0])
+        tmax = tmax[:n_oracle]
         for i, t in enumerate(tmax):
             want_cost, want_sol = dp_impl_c(t, L, D, meshes, G, *tabs)
             assert (bs[i] >= 0) == (want_sol is not None), (G, t)

@@ -285,3 +285,35 @@ def test_randomized_plans_match_oracle(seed, monkeypatch):
     cfg, tables = tiny_plan(1, layers=int(rng.integers(3, 8)), **overrides)
     for tp in tp_candidates(cfg):
         _compare(cfg, tables, tp, S=int(rng.choice([1, 1, 3])), require_finite=False)
+
+
+@pytest.mark.parametrize("G, mesh, tp, p_cands, S", [
+    (4, (1, 2), None, range(3), 1),    # tp latches to the first feasible batch size
+    (2, (2, 4), 2, range(5), 2),       # more pre-saved micro-batch values than G
+    (8, (1, 1), 1, range(1), 3),
+    (16, (2, 4), 8, range(2), 1),      # no factorisation with tp = 8 > gpus per node: empty space
+])
+def test_operator_boundary_matches_oracle(G, mesh, tp, p_cands, S):
+    """``mist_amd.batched_module_analyzer.batched_tune_best_latency_for_stage`` (the reference's
+    operator signature, batched_module_analyzer.py:581-684) against the oracle's restatement of
+    the same function: every table of the four result tuples, float64, bit for bit."""
+    from mist_amd.batched_module_analyzer import batched_tune_best_latency_for_stage as gpu_op
+    from oracle.stage import batched_tune_best_latency_for_stage as oracle_op
+
+    cfg, tables = tiny_plan(1, layers=6, hardware__num_nodes=2, hardware__num_gpus_per_node=4,
+                            training__global_batch_size=32, hardware__memory_capacity=8.0)
+    L = cfg.model.num_hidden_layers
+    args = (list(p_cands), list(range(1, L + 1)), list(range(L + 1)), mesh[0], mesh[1], G)
+    got = gpu_op(tables, tables, None, *args, cfg, tp_size=tp, sample_size=S)
+    want = oracle_op(tables, cfg, *args, tp_size=tp, sample_size=S)
+    assert len(got) == 4
+    finite = 0
+    for v in range(4):
+        assert len(got[v]) == 3
+        for k, name in enumerate(("costs_stable", "costs_delta", "solutions")):
+            assert got[v][k].dtype == np.float64
+            assert_same_f64(got[v][k], want[v][k], f"variant {v} {name}")
+        finite += int(np.isfinite(got[v][0]).sum())
+    assert (finite > 0) == (tp != 8)
+    with pytest.raises(AssertionError):
+        gpu_op(tables, None, None, [0, 2], *args[1:], cfg, tp_size=tp, sample_size=S)

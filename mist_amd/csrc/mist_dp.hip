@@ -593,6 +593,8 @@ __global__ __launch_bounds__(kDpFusedThreads) void dp_fused_kernel(
 // visited in the reference's (mesh, end layer) order with a strict "<": same winner, same ties.
 // ------------------------------------------------------------------------------------------
 constexpr int kDpPlaneThreads = 1024;
+constexpr int kDpPlaneCols = 4;    // device counts per lane: d = 1 + lane + 64 j, so D <= 256
+constexpr int kDpPlaneLoads = 20;  // row minima a lane fetches per start layer: Q * L <= 1280
 #ifndef MIST_DP_PLANE_MIN_INSTANCES
 #define MIST_DP_PLANE_MIN_INSTANCES 16
 #endif
@@ -608,11 +610,10 @@ __global__ __launch_bounds__(kDpPlaneThreads) void dp_plane_kernel(
   extern __shared__ float dp_lds[];
   const int L = shape.num_layers, D = shape.num_devices, Q = shape.num_mesh;
   const int W = D + 1, plane = (L + 1) * W;
-  const int n_blocks = (D + 63) / 64;  // block b of a row: d = 1 + 64 b + lane
   float *f_lds = dp_lds;                                        // F(s - 1)
   int32_t *range = reinterpret_cast<int32_t *>(dp_lds + plane);  // [3][W][2] reachable rows per column
-  int32_t *blk = range + 6 * W;                                  // [Q][n_blocks][2] the same per (mesh, block)
-  float *wave_rows = reinterpret_cast<float *>(blk + 2 * Q * n_blocks);  // [n_waves][Q][L] row minima of a task
+  int32_t *reach_q = range + 6 * W;                              // [Q][2] the same per mesh, all columns
+  float *wave_rows = reinterpret_cast<float *>(reach_q + 2 * Q);  // [n_waves][Q][L] row minima of a task
   const int t = blockIdx.x;
   const float t_max = kBottleneck ? INFINITY : tmax_list[t];
   const int64_t g = g_list[t];
@@ -626,6 +627,13 @@ __global__ __launch_bounds__(kDpPlaneThreads) void dp_plane_kernel(
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int n_waves = blockDim.x >> 6;
   float *my_rows = wave_rows + wave * Q * L;
+  int d_of[kDpPlaneCols];
+  bool col_ok[kDpPlaneCols];
+#pragma unroll
+  for (int j = 0; j < kDpPlaneCols; ++j) {
+    d_of[j] = 1 + lane + 64 * j;
+    col_ok[j] = d_of[j] <= D;
+  }
 
   for (int e = threadIdx.x; e < plane; e += blockDim.x) f_lds[e] = e == L * W ? 0.0f : INFINITY;
   for (int col = threadIdx.x; col < W; col += blockDim.x) {
@@ -647,18 +655,30 @@ __global__ __launch_bounds__(kDpPlaneThreads) void dp_plane_kernel(
     const int32_t *range_prev = range + ((s + 2) % 3) * W * 2;
     int32_t *range_cur = range + (s % 3) * W * 2;
     int32_t *range_next = range + ((s + 1) % 3) * W * 2;
-    // reachable successor rows of every (mesh, block of 64 columns): bounds of the uniform loop
-    for (int x = threadIdx.x; x < Q * n_blocks; x += blockDim.x) {
-      const int q = x / n_blocks, b = x % n_blocks;
+    // reachable successor rows per mesh (over all columns): bounds of the uniform loop
+    if (wave < Q) {
+      const int q = wave;
       const int nm = shape.mesh_n[q] * shape.mesh_m[q];
       int first = L + 1, last = -1;
-      for (int d = 1 + 64 * b; d <= min(D, 64 * b + 64); ++d) {
-        if (d < nm) continue;
-        first = min(first, range_prev[2 * (d - nm)]);
-        last = max(last, range_prev[2 * (d - nm) + 1]);
+      for (int c = lane; c + nm <= D; c += 64) {  // successor column c = d - nm of some d <= D
+        first = min(first, range_prev[2 * c]);
+        last = max(last, range_prev[2 * c + 1]);
       }
-      blk[2 * x] = first;
-      blk[2 * x + 1] = last;
+#pragma unroll
+      for (int step = 32; step >= 1; step >>= 1) {
+        first = min(first, __shfl_xor(first, step));
+        last = max(last, __shfl_xor(last, step));
+      }
+      if (lane == 0) {
+        reach_q[2 * q] = first;
+        reach_q[2 * q + 1] = last;
+      }
+    }
+    for (int q = n_waves + wave; q < Q; q += n_waves) {  // (more meshes than wavefronts)
+      if (lane == 0) {
+        reach_q[2 * q] = 0;
+        reach_q[2 * q + 1] = L;
+      }
     }
     if (threadIdx.x == 0) {  // column 0 holds the origin only: unreachable from here on
       range_next[0] = L + 1;
@@ -666,27 +686,50 @@ __global__ __launch_bounds__(kDpPlaneThreads) void dp_plane_kernel(
     }
     __syncthreads();
     const float *__restrict__ block = relaid + (int64_t)p * Q * tri;
-    const int n_tasks = (L - s + 1) * n_blocks;  // start layers 0 .. L - s
-    for (int task = wave; task < n_tasks; task += n_waves) {
-      const int k = task / n_blocks, b = task - k * n_blocks;
-      const int d = 1 + 64 * b + lane;
-      const bool col_ok = d <= D;
-      // The row minima of the stages k..i on every mesh, [Q][L - k] floats, into this
-      // wavefront's LDS buffer with all reads in flight together; the loop below then has no
-      // global read in its dependence chain.
+    // One task = one start layer k with all its device counts.  Tasks go to the wavefronts in
+    // snake order (their cost falls with k).  A task's row minima, [Q][L - k] floats, are fetched
+    // one task ahead into registers and laid into this wavefront's LDS buffer, so the loops
+    // below have no global read in their dependence chain.
+    const int n_tasks = L - s + 1;  // start layers 0 .. L - s
+    auto task_k = [&](int round) {
+      const int at = round * n_waves + ((round & 1) ? n_waves - 1 - wave : wave);
+      return at < n_tasks ? at : -1;
+    };
+    float fetched[kDpPlaneLoads];
+    auto fetch = [&](int k) {
       const int width = L - k;
-      for (int x = lane; x < Q * width; x += 64) {
-        const int q = x / width, di = x - q * width;
-        my_rows[x] = block[q * tri + dp_triangle_row(L, k) + di];
+#pragma unroll
+      for (int u = 0; u < kDpPlaneLoads; ++u) {
+        const int x = lane + 64 * u;
+        if (k >= 0 && x < Q * width) {
+          const int q = x / width, di = x - q * width;
+          fetched[u] = block[q * tri + dp_triangle_row(L, k) + di];
+        }
       }
+    };
+    fetch(task_k(0));
+    for (int round = 0; task_k(round) >= 0; ++round) {
+      const int k = task_k(round);
+      const int width = L - k;
+#pragma unroll
+      for (int u = 0; u < kDpPlaneLoads; ++u) {
+        const int x = lane + 64 * u;
+        if (x < Q * width) my_rows[x] = fetched[u];
+      }
+      fetch(task_k(round + 1));
       __builtin_amdgcn_wave_barrier();
-      DpBest w;
+      DpBest w[kDpPlaneCols];
       for (int q = 0; q < Q; ++q) {
         const int nm = shape.mesh_n[q] * shape.mesh_m[q];
-        const int i_first = max(k, blk[2 * (q * n_blocks + b)] - 1);
-        const int i_last = min(L - 1, blk[2 * (q * n_blocks + b) + 1] - 1);
-        const bool lane_ok = col_ok && nm <= d;
-        const float *col = f_lds + (lane_ok ? d - nm : 0);
+        const int i_first = max(k, reach_q[2 * q] - 1);
+        const int i_last = min(L - 1, reach_q[2 * q + 1] - 1);
+        bool lane_ok[kDpPlaneCols];
+        const float *col[kDpPlaneCols];
+#pragma unroll
+        for (int j = 0; j < kDpPlaneCols; ++j) {
+          lane_ok[j] = col_ok[j] && nm <= d_of[j];
+          col[j] = f_lds + (lane_ok[j] ? d_of[j] - nm : 0);
+        }
         const float *rm = my_rows + q * width - k;  // rm[i]
         // 64 end layers at a time: which of them are admissible at all (the same for every
         // lane), then only those, in ascending order
@@ -699,36 +742,47 @@ __global__ __launch_bounds__(kDpPlaneThreads) void dp_plane_kernel(
             todo &= todo - 1;
             const int i = i0 + bit;
             const float rmin = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(r_mine), bit));
-            const float prev = lane_ok ? col[(i + 1) * W] : INFINITY;
-            dp_consider<kBottleneck>(w, t_max, q, i, prev, rmin);
+            float prev[kDpPlaneCols];
+#pragma unroll
+            for (int j = 0; j < kDpPlaneCols; ++j)
+              prev[j] = lane_ok[j] ? col[j][(i + 1) * W] : INFINITY;
+#pragma unroll
+            for (int j = 0; j < kDpPlaneCols; ++j)
+              dp_consider<kBottleneck>(w[j], t_max, q, i, prev[j], rmin);
           }
         }
       }
       __builtin_amdgcn_wave_barrier();
-      if (!col_ok) continue;
-      dp_finish_winner<kBottleneck>(w, shape, tabs, off, t_max, p, k, d, f_lds, m_prev);
-      const int e = k * W + d;
-      f_cur[e] = w.best;
-      m_cur[e] = w.best_m;
-      if (w.best < INFINITY) {
-        atomicMin(&range_cur[2 * d], k);
-        atomicMax(&range_cur[2 * d + 1], k);
-      }
-      if (k == 0) {
-        range_next[2 * d] = L + 1;
-        range_next[2 * d + 1] = -1;
-      }
-      if (argmin != nullptr && w.arg_i >= 0) {
-        int32_t *a = argmin + (((int64_t)t * (shape.max_stages + 1) + s) * plane + e) * 4;
-        a[0] = w.arg_i;
-        a[1] = shape.mesh_n[w.arg_q];
-        a[2] = shape.mesh_m[w.arg_q];
-        a[3] = w.arg_j;
-      }
-      if (k == 0 && d == D && w.best < answer_sum) {  // first s wins ties (inter_tuning.py:335-340)
-        answer_sum = w.best;
-        answer_s = s;
-        answer_max = w.best_m;
+#pragma unroll
+      for (int j = 0; j < kDpPlaneCols; ++j) {
+        if (!col_ok[j]) continue;
+        const int d = d_of[j];
+        dp_finish_winner<kBottleneck>(w[j], shape, tabs, off, t_max, p, k, d, f_lds, m_prev);
+        const int e = k * W + d;
+        f_cur[e] = w[j].best;
+        m_cur[e] = w[j].best_m;
+        if (w[j].best < INFINITY) {
+          atomicMin(&range_cur[2 * d], k);
+          atomicMax(&range_cur[2 * d + 1], k);
+        }
+        if (k == 0) {
+          range_next[2 * d] = L + 1;
+          range_next[2 * d + 1] = -1;
+        }
+        if (argmin != nullptr && w[j].arg_i >= 0) {
+          int32_t *a = argmin + (((int64_t)t * (shape.max_stages + 1) + s) * plane + e) * 4;
+          a[0] = w[j].arg_i;
+          a[1] = shape.mesh_n[w[j].arg_q];
+          a[2] = shape.mesh_m[w[j].arg_q];
+          a[3] = w[j].arg_j;
+        }
+        // first s wins ties (inter_tuning.py:335-340); (k = 0, d = D) is wavefront 0's first
+        // task in every step, the same lane's
+        if (k == 0 && d == D && w[j].best < answer_sum) {
+          answer_sum = w[j].best;
+          answer_s = s;
+          answer_max = w[j].best_m;
+        }
       }
     }
     __syncthreads();  // every scan of F(s - 1) is done, F(s) is in the scratch plane
@@ -738,10 +792,7 @@ __global__ __launch_bounds__(kDpPlaneThreads) void dp_plane_kernel(
     }
     __syncthreads();
   }
-  // the answer state (k = 0, d = D) is the same thread's in every step: wave 0 takes task
-  // (D - 1) / 64 when n_waves > that block index, else the wave task % n_waves
-  const int answer_task = (D - 1) / 64;
-  if (wave == answer_task % n_waves && lane == (D - 1) % 64) {
+  if (wave == 0 && lane == (D - 1) % 64) {
     best_s_out[t] = answer_s;
     best_sum_out[t] = answer_sum;
     stage_max_out[t] = answer_max;
@@ -1146,11 +1197,12 @@ int mist_dp_run(const MistDpShape *shape, const MistDpCosts *costs, const float 
   // Planes beyond the LDS of a compute unit (80 layers x 256 devices): one workgroup per instance
   // with F(s - 1) alone in LDS, one launch.
   const size_t plane_lds =
-      ((size_t)plane + 6 * (size_t)(shape->num_devices + 1) +
-       2 * (size_t)shape->num_mesh * ((shape->num_devices + 63) / 64) +
+      ((size_t)plane + 6 * (size_t)(shape->num_devices + 1) + 2 * (size_t)shape->num_mesh +
        (size_t)(kDpPlaneThreads / 64) * shape->num_mesh * shape->num_layers) * sizeof(float);
+  const bool plane_shape_ok = shape->num_devices <= 64 * kDpPlaneCols &&
+                              shape->num_mesh * shape->num_layers <= 64 * kDpPlaneLoads;
   if (costs->stage_min != nullptr && shape->free_devices == 0 && n_tmax >= kDpPlaneMinInstances &&
-      fused_lds > fused_lds_limit(mode) && plane_lds <= plane_lds_limit(mode)) {
+      plane_shape_ok && fused_lds > fused_lds_limit(mode) && plane_lds <= plane_lds_limit(mode)) {
     if (mode == MIST_DP_BOTTLENECK)
       hipLaunchKernelGGL(dp_plane_kernel<true>, dim3(n_tmax), dim3(kDpPlaneThreads), plane_lds,
                          (hipStream_t)stream, *shape, *costs, d_tmax, d_g_index, d_scratch,

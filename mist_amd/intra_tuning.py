@@ -31,6 +31,11 @@ SCOUT_MIN_STAGES = 128  # groups with fewer stages get no scout pass (0 = never 
 SCOUT_MIN_PAIRS = 4     # ... and so do groups with fewer (weight, gradient) offload pairs
 SCOUT_PAIRS = 1         # offload pairs whose rows the scout pass gathers: the first, (0, 0), then evenly spread ones
 SCOUT_PAIR_SPAN = 200   # ... one more for every so many pairs of the group (GPT-22B: 421 pairs, 3 gathered)
+# Upper bound of the row-term workspace (272 bytes per candidate row): the groups of a tuner call
+# go through the kernels in batches of consecutive groups whose rows fit it (a group larger than
+# the bound is a batch of its own).  GPT-7B (0.88 GB) and LLaMA-13B (1.4 GB) are one batch,
+# GPT-22B (18.4 GB of row terms) ten; with more than one batch two such workspaces alternate.
+ROW_TERMS_BUDGET_BYTES = 2 << 30
 
 
 def alpha_ratios(sample_size: int) -> np.ndarray:
@@ -203,6 +208,7 @@ class IntraStageTuner:
         # True: every p of 0..P is evaluated for every G (the operator boundary
         # batched_tune_best_latency_for_stage takes the p candidates from its caller)
         self.evaluate_all_p = False
+        self._side_stream = None
         self.results: Optional[IntraStageTunerOutput] = None
         self.stats: Dict[str, float] = {}
 
@@ -241,11 +247,14 @@ class IntraStageTuner:
         n_lc_tiles = -(-n_pairs // _lib.LC_TILE)
         if len(pending):
             n_p_tiles = -(-groups["num_p"] // _lib.P_TILE)
-            tile_rows = int(np.sum(groups["n_rows"] * n_lc_tiles * n_p_tiles))
-            rows_per_chunk = -(-tile_rows // max(TARGET_REDUCE_WAVES * 64 // _lib.LC_TILE, 1))
-            rows_per_chunk = max(256, min(16384, -(-rows_per_chunk // _lib.STAGE_ROWS) * _lib.STAGE_ROWS))
-            groups["rows_per_chunk"] = rows_per_chunk
-            groups["n_chunks"] = -(-groups["n_rows"] // rows_per_chunk)
+            # the row chunks are sized per batch of groups (one reduce launch each, see below)
+            for first, last in self._batch_bounds(groups["n_rows"]):
+                sel = slice(first, last)
+                tile_rows = int(np.sum(groups["n_rows"][sel] * n_lc_tiles * n_p_tiles[sel]))
+                rows_per_chunk = -(-tile_rows // max(TARGET_REDUCE_WAVES * 64 // _lib.LC_TILE, 1))
+                rows_per_chunk = max(256, min(16384, -(-rows_per_chunk // _lib.STAGE_ROWS) * _lib.STAGE_ROWS))
+                groups["rows_per_chunk"][sel] = rows_per_chunk
+            groups["n_chunks"] = -(-groups["n_rows"] // groups["rows_per_chunk"])
             groups["n_lc_tiles"] = n_lc_tiles
             groups["n_p_tiles"] = n_p_tiles
             groups["row_offset"] = np.concatenate(([0], np.cumsum(groups["n_rows"])[:-1]))
@@ -269,12 +278,40 @@ class IntraStageTuner:
         if terms_prefix[-1] >= 2**31 or reduce_prefix[-1] + scout_prefix[-1] >= 2**31:
             raise ValueError("launch decomposition exceeds 2**31 workgroups")
         problem = make_problem(cfg, L, P + 1, self.sample_size, len(self.tp_sizes) * len(Gs), len(Q))
+        # Batches of consecutive groups under the workspace bound: each holds its own copy of the
+        # descriptors with row offsets that start at 0 and its own workgroup prefixes.
+        batches = []
+        for first, last in self._batch_bounds(groups["n_rows"]) if len(pending) else []:
+            rows = int(groups["n_rows"][first:last].sum())
+            sub = groups[first:last].copy()
+            sub["row_offset"] -= groups["row_offset"][first]
+            rebase = lambda prefix: (prefix[first:last + 1] - prefix[first]).astype(np.int32)
+            batches.append(dict(
+                first=first, last=last, groups=sub, total_rows=rows,
+                terms_prefix=rebase(terms_prefix), reduce_prefix=rebase(reduce_prefix),
+                scout_prefix=rebase(scout_prefix),
+            ))
         return dict(
-            problem=problem, groups=groups, spaces=spaces,
+            problem=problem, groups=groups, spaces=spaces, batches=batches,
             terms_prefix=terms_prefix.astype(np.int32), reduce_prefix=reduce_prefix.astype(np.int32),
             scout_prefix=scout_prefix.astype(np.int32),
             total_rows=int(groups["n_rows"].sum()) if len(pending) else 0,
         )
+
+    @staticmethod
+    def _batch_bounds(n_rows) -> List[Tuple[int, int]]:
+        """Runs of consecutive groups whose rows fit the row-term workspace bound (a larger
+        group is a run of its own)."""
+        budget_rows = max(ROW_TERMS_BUDGET_BYTES // (8 * _lib.ROW_TERMS), 1)
+        bounds, first = [], 0
+        while first < len(n_rows):
+            last, rows = first, 0
+            while last < len(n_rows) and (last == first or rows + int(n_rows[last]) <= budget_rows):
+                rows += int(n_rows[last])
+                last += 1
+            bounds.append((first, last))
+            first = last
+        return bounds
 
     def allocate_tables(self) -> DeviceTables:
         Gn = len(self.tp_sizes) * len(self.gradient_accumulation_steps_candidates)
@@ -294,91 +331,121 @@ class IntraStageTuner:
 
     # ------------------------------------------------------------------ device side
     def upload(self, plan) -> dict:
+        """Descriptors and workgroup prefixes of every batch to the device; one workspace (row
+        terms, stage summaries, partial minima) sized for the largest batch and shared by all.
+        The top-level entries are those of the first batch (all there is for most plans)."""
         dev = self.device
         def to_dev(a: np.ndarray) -> torch.Tensor:
             return torch.from_numpy(np.ascontiguousarray(a).view(np.uint8).reshape(-1)).to(dev)
-        n_groups = len(plan["groups"])
-        n_reduce_blocks = int(plan["reduce_prefix"][-1])
-        n_scout_blocks = int(plan["scout_prefix"][-1])
-        n_slabs = max(n_reduce_blocks + n_scout_blocks, 1)
-        return dict(
-            n_groups=n_groups,
-            groups=to_dev(plan["groups"]) if n_groups else None,
-            terms_prefix=to_dev(plan["terms_prefix"]),
-            reduce_prefix=to_dev(plan["reduce_prefix"]),
-            n_terms_blocks=int(plan["terms_prefix"][-1]),
-            n_reduce_blocks=n_reduce_blocks,
-            scout_prefix=to_dev(plan["scout_prefix"]),
-            n_scout_blocks=n_scout_blocks,
-            row_terms=torch.empty(max(plan["total_rows"], 1) * _lib.ROW_TERMS, dtype=torch.float64, device=dev),
-            stage_floor=torch.empty(
-                _lib.load().mist_stage_floor_doubles(plan["total_rows"], n_groups),
-                dtype=torch.float64, device=dev),
-            partial_cost=torch.empty(n_slabs * _lib.SLOTS * _lib.LC_TILE, dtype=torch.float64, device=dev),
-            partial_index=torch.empty(n_slabs * _lib.SLOTS * _lib.LC_TILE, dtype=torch.int32, device=dev),
+        lib = _lib.load()
+        batches = []
+        for b in plan["batches"]:
+            batches.append(dict(
+                n_groups=len(b["groups"]), groups=to_dev(b["groups"]),
+                terms_prefix=to_dev(b["terms_prefix"]), reduce_prefix=to_dev(b["reduce_prefix"]),
+                scout_prefix=to_dev(b["scout_prefix"]),
+                n_terms_blocks=int(b["terms_prefix"][-1]), n_reduce_blocks=int(b["reduce_prefix"][-1]),
+                n_scout_blocks=int(b["scout_prefix"][-1]), total_rows=b["total_rows"],
+            ))
+        max_rows = max([b["total_rows"] for b in batches], default=0)
+        max_groups = max([b["n_groups"] for b in batches], default=0)
+        n_slabs = max([b["n_reduce_blocks"] + b["n_scout_blocks"] for b in batches] + [1])
+        def workspace():
+            return dict(
+                row_terms=torch.empty(max(max_rows, 1) * _lib.ROW_TERMS, dtype=torch.float64, device=dev),
+                stage_floor=torch.empty(lib.mist_stage_floor_doubles(max_rows, max_groups),
+                                        dtype=torch.float64, device=dev),
+                partial_cost=torch.empty(n_slabs * _lib.SLOTS * _lib.LC_TILE, dtype=torch.float64, device=dev),
+                partial_index=torch.empty(n_slabs * _lib.SLOTS * _lib.LC_TILE, dtype=torch.int32, device=dev),
+            )
+        # several batches alternate between two workspaces on two streams, so that the tail of
+        # one batch's launches overlaps the start of the next
+        workspaces = [workspace() for _ in range(2 if len(batches) > 1 else 1)]
+        out = dict(
+            batches=batches, workspaces=workspaces, **workspaces[0],
+            n_groups=0, groups=None, terms_prefix=None, reduce_prefix=None, scout_prefix=None,
+            n_terms_blocks=0, n_reduce_blocks=0, n_scout_blocks=0,
             grad_accum=torch.tensor(
                 list(self.gradient_accumulation_steps_candidates) * len(self.tp_sizes),
                 dtype=torch.int32, device=dev),
         )
+        if batches:
+            out.update({k: batches[0][k] for k in (
+                "n_groups", "groups", "terms_prefix", "reduce_prefix", "scout_prefix",
+                "n_terms_blocks", "n_reduce_blocks", "n_scout_blocks")})
+        return out
 
     def launch(self, plan, dev_plan, tables: DeviceTables, events: Optional[list] = None) -> None:
         """Enqueues the kernels for every requested sample on the current stream.  With
         ``events`` (a list) the three kernels are launched through their own entry points and
         ``(name, start_event, end_event)`` triples recorded on that stream are appended."""
-        if dev_plan["n_groups"] == 0:
+        if not dev_plan["batches"]:
             return
         lib = _lib.load()
-        stream = ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+        current = torch.cuda.current_stream(self.device)
+        streams = [current]
+        if len(dev_plan["workspaces"]) > 1 and events is None:
+            if self._side_stream is None:
+                self._side_stream = torch.cuda.Stream(device=self.device)
+            streams.append(self._side_stream)
+            self._side_stream.wait_stream(current)  # the tables are filled on the current stream
         ratios = alpha_ratios(self.sample_size)
         out = tables.as_struct()
         prob_ptr = ctypes.c_void_p(plan["problem"].ctypes.data)
-        d = dev_plan
-        def reduce_call(slot):
-            if self.exhaustive:
-                return lib.mist_eval_reduce_exhaustive(
-                    prob_ptr, _ptr(d["groups"]), d["n_groups"], _ptr(d["reduce_prefix"]),
-                    d["n_reduce_blocks"], _ptr(d["row_terms"]), float(ratios[slot]),
-                    _ptr(d["partial_cost"]), _ptr(d["partial_index"]), stream)
-            return lib.mist_eval_reduce(
-                prob_ptr, _ptr(d["groups"]), d["n_groups"], _ptr(d["reduce_prefix"]),
-                d["n_reduce_blocks"], _ptr(d["scout_prefix"]), d["n_scout_blocks"],
-                _ptr(d["row_terms"]), _ptr(d["stage_floor"]), float(ratios[slot]),
-                _ptr(d["partial_cost"]), _ptr(d["partial_index"]), stream)
 
-        for i, slot in enumerate(self.sample_slots):
-            if events is None and not self.exhaustive:
-                rc = lib.mist_intra_stage_eval(
-                    prob_ptr, _ptr(d["groups"]), d["n_groups"],
-                    _ptr(d["terms_prefix"]), d["n_terms_blocks"],
-                    _ptr(d["reduce_prefix"]), d["n_reduce_blocks"],
-                    _ptr(d["scout_prefix"]), d["n_scout_blocks"],
-                    _ptr(d["row_terms"]), _ptr(d["stage_floor"]), _ptr(d["partial_cost"]),
-                    _ptr(d["partial_index"]), float(ratios[slot]), int(slot),
-                    1 if i == 0 else 0, ctypes.byref(out), stream,
-                )
-                _lib.check(rc, "mist_intra_stage_eval")
-                continue
-
-            def timed(name, call):
-                if events is None:
-                    _lib.check(call(), name)
-                    return
-                start = torch.cuda.Event(enable_timing=True)
-                end = torch.cuda.Event(enable_timing=True)
-                start.record()
+        def timed(name, call):
+            if events is None:
                 _lib.check(call(), name)
-                end.record()
-                events.append((name, start, end))
+                return
+            start = torch.cuda.Event(enable_timing=True)
+            end = torch.cuda.Event(enable_timing=True)
+            start.record()
+            _lib.check(call(), name)
+            end.record()
+            events.append((name, start, end))
 
-            if i == 0:
-                timed("row_terms", lambda: lib.mist_row_terms(
-                    prob_ptr, _ptr(d["groups"]), d["n_groups"], _ptr(d["terms_prefix"]),
-                    d["n_terms_blocks"], _ptr(d["row_terms"]), _ptr(d["stage_floor"]), stream))
-            timed("eval_reduce", lambda: reduce_call(slot))
-            timed("finalize", lambda: lib.mist_finalize(
-                prob_ptr, _ptr(d["groups"]), d["n_groups"], _ptr(d["reduce_prefix"]),
-                _ptr(d["row_terms"]), _ptr(d["partial_cost"]), _ptr(d["partial_index"]), int(slot),
-                ctypes.byref(out), stream))
+        for bi, d in enumerate(dev_plan["batches"]):
+            # batch bi: stream bi % 2 and workspace bi % 2 (the same pairing every time, so a
+            # workspace is reused in stream order)
+            stream = ctypes.c_void_p(streams[bi % len(streams)].cuda_stream)
+            w = dev_plan["workspaces"][bi % len(dev_plan["workspaces"])]
+
+            def reduce_call(slot):
+                if self.exhaustive:
+                    return lib.mist_eval_reduce_exhaustive(
+                        prob_ptr, _ptr(d["groups"]), d["n_groups"], _ptr(d["reduce_prefix"]),
+                        d["n_reduce_blocks"], _ptr(w["row_terms"]), float(ratios[slot]),
+                        _ptr(w["partial_cost"]), _ptr(w["partial_index"]), stream)
+                return lib.mist_eval_reduce(
+                    prob_ptr, _ptr(d["groups"]), d["n_groups"], _ptr(d["reduce_prefix"]),
+                    d["n_reduce_blocks"], _ptr(d["scout_prefix"]), d["n_scout_blocks"],
+                    _ptr(w["row_terms"]), _ptr(w["stage_floor"]), float(ratios[slot]),
+                    _ptr(w["partial_cost"]), _ptr(w["partial_index"]), stream)
+
+            for i, slot in enumerate(self.sample_slots):
+                if events is None and not self.exhaustive:
+                    rc = lib.mist_intra_stage_eval(
+                        prob_ptr, _ptr(d["groups"]), d["n_groups"],
+                        _ptr(d["terms_prefix"]), d["n_terms_blocks"],
+                        _ptr(d["reduce_prefix"]), d["n_reduce_blocks"],
+                        _ptr(d["scout_prefix"]), d["n_scout_blocks"],
+                        _ptr(w["row_terms"]), _ptr(w["stage_floor"]), _ptr(w["partial_cost"]),
+                        _ptr(w["partial_index"]), float(ratios[slot]), int(slot),
+                        1 if i == 0 else 0, ctypes.byref(out), stream,
+                    )
+                    _lib.check(rc, "mist_intra_stage_eval")
+                    continue
+                if i == 0:
+                    timed("row_terms", lambda: lib.mist_row_terms(
+                        prob_ptr, _ptr(d["groups"]), d["n_groups"], _ptr(d["terms_prefix"]),
+                        d["n_terms_blocks"], _ptr(w["row_terms"]), _ptr(w["stage_floor"]), stream))
+                timed("eval_reduce", lambda: reduce_call(slot))
+                timed("finalize", lambda: lib.mist_finalize(
+                    prob_ptr, _ptr(d["groups"]), d["n_groups"], _ptr(d["reduce_prefix"]),
+                    _ptr(w["row_terms"]), _ptr(w["partial_cost"]), _ptr(w["partial_index"]), int(slot),
+                    ctypes.byref(out), stream))
+        if len(streams) > 1:
+            current.wait_stream(streams[1])
 
     def _outputs(self, plan, tables: DeviceTables) -> List[IntraStageTunerOutput]:
         Gn = len(self.gradient_accumulation_steps_candidates)

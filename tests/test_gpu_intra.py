@@ -240,6 +240,24 @@ def test_exhaustive_kernel_matches_oracle(overrides):
         _compare(cfg, tables, 2, exhaustive=True)
 
 
+@pytest.mark.parametrize("budget_rows", [1, 2700, 6000])
+def test_workspace_batches_leave_results_unchanged(monkeypatch, budget_rows):
+    """The groups of a tuner call go through the kernels in batches that share one bounded
+    row-term workspace: one group per batch, a few, or all in one must give the oracle's tables
+    (S = 3 as well: the row terms of a batch are computed once and reduced per sample)."""
+    from mist_amd import _lib, intra_tuning
+
+    monkeypatch.setattr(intra_tuning, "ROW_TERMS_BUDGET_BYTES", budget_rows * 8 * _lib.ROW_TERMS)
+    cfg, tables = load_plan(1)
+    plan = _gpu_tuner(cfg, tables, 1).prepare()
+    n_groups = len(plan["groups"])
+    assert (len(plan["batches"]) == n_groups) if budget_rows == 1 else (1 < len(plan["batches"]) < n_groups)
+    _compare(cfg, tables, 1)
+    cfg, tables = tiny_plan(1, layers=6, hardware__memory_capacity=6.0)
+    _compare(cfg, tables, 1, S=3)
+    _compare(cfg, tables, 2, exhaustive=True)
+
+
 def test_gradient_accumulation_steps_that_are_not_powers_of_two():
     """The tuner's own G candidates are powers of two (the kernel then multiplies by an exact
     reciprocal); a caller-supplied list may hold any divisor of the batch size, which takes the

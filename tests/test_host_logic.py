@@ -137,6 +137,38 @@ def test_launch_decomposition_covers_every_row_once():
     assert plan["total_rows"] == int(g["n_rows"].sum()) == 913308
 
 
+def test_workspace_batches_partition_the_groups(monkeypatch):
+    """Batches are runs of consecutive groups under the row-term workspace bound, each with row
+    offsets and workgroup prefixes that start at zero."""
+    from mist_amd import _lib, intra_tuning
+    from mist_amd.intra_tuning import IntraStageTuner
+    from mist_amd.search_space import _get_device_mesh_candidates, _get_grad_accumu_steps_candidates
+
+    cfg, tables = load_plan(1)
+    hw = cfg.hardware
+    meshes = _get_device_mesh_candidates(hw.num_nodes, hw.num_gpus_per_node, False)
+    Gs = _get_grad_accumu_steps_candidates(cfg.training.global_batch_size)
+    for budget_rows in (1, 700, 3000, 10**9):
+        monkeypatch.setattr(intra_tuning, "ROW_TERMS_BUDGET_BYTES", budget_rows * 8 * _lib.ROW_TERMS)
+        plan = IntraStageTuner(tables, cfg.model.num_hidden_layers, meshes, Gs, [1, 2], cfg, sample_size=1).prepare()
+        groups, batches = plan["groups"], plan["batches"]
+        assert [b["first"] for b in batches] == [0] + [b["last"] for b in batches[:-1]]
+        assert batches[-1]["last"] == len(groups)
+        for b in batches:
+            sub, whole = b["groups"], groups[b["first"]:b["last"]]
+            assert b["total_rows"] == int(whole["n_rows"].sum())
+            assert len(sub) == 1 or b["total_rows"] <= budget_rows
+            assert sub["row_offset"][0] == 0
+            assert np.array_equal(np.diff(sub["row_offset"]), whole["n_rows"][:-1])
+            for name in ("terms_prefix", "reduce_prefix", "scout_prefix"):
+                assert b[name][0] == 0 and len(b[name]) == len(sub) + 1
+                assert np.array_equal(np.diff(b[name]), np.diff(plan[name][b["first"]:b["last"] + 1]))
+            for field in ("g_index", "q_index", "n_rows", "n_chunks", "scout_stride"):
+                assert np.array_equal(sub[field], whole[field])
+        if budget_rows == 10**9:
+            assert len(batches) == 1
+
+
 def test_best_solution_yaml_format():
     from mist_amd.tune_one_case import best_solution_yaml
 

@@ -659,7 +659,10 @@ __device__ __forceinline__ void take_min(double &best, int32_t &best_row, bool f
 #ifndef MIST_REDUCE_MIN_WAVES
 #define MIST_REDUCE_MIN_WAVES 2
 #endif
-constexpr int kScoutSplit = 2;  // scout workgroups per (group, (l, c) tile, p tile)
+#ifndef MIST_SCOUT_SPLIT
+#define MIST_SCOUT_SPLIT 2
+#endif
+constexpr int kScoutSplit = MIST_SCOUT_SPLIT;  // scout workgroups per (group, (l, c) tile, p tile)
 constexpr int32_t kSlabUnchanged = -2;  // first row index of a slab that was not written (rows are >= -1)
 constexpr int kPairFields = 4;  // per-pair table of sieve A: thr_b, thr_o, n_ck, n_nock
 constexpr int kLdsRowStride = MIST_ROW_TERMS + 1;  // odd number of doubles: lanes reading the
@@ -1077,6 +1080,20 @@ __device__ __forceinline__ void reduce_block(
     if (after(stage) < end_stage) floor_v = load_floor(after(stage));
     __syncthreads();
 
+    // ---- the pseudo row (term-wise minimum of the stage) against the loosest thresholds, the
+    // largest minimum of each objective: the thresholds below are no larger, so a stage that
+    // no lane passes here is closed, and its memory bounds need not be formed ----
+    double floor_x, floor_d, floor_cost, floor_bound;
+    objective(lds_min, floor_x, floor_d, floor_cost, floor_bound);
+    {
+      const double loose_b = fin_b < n_tile ? (double)INFINITY : top_b;
+      const double loose_p = fin_p < n_tile ? (double)INFINITY : top_p;
+      double loose_o = below(loose_p, off_pre);
+      if (do_post) loose_o = fmax(loose_o, below(best_post, off_post));
+      if (do_nopp) loose_o = fmax(loose_o, below(best_pp, off_pp));
+      if (!__any(active && (floor_cost <= loose_b || floor_bound <= loose_o))) continue;
+    }
+
     // ---- per-stage thresholds: no row of the stage is feasible beyond the pseudo row's count,
     // so only the minima of the slots below it can be beaten ----
     const LaneMemory floor_mem = lane_memory(lds_min);
@@ -1121,11 +1138,7 @@ __device__ __forceinline__ void reduce_block(
     // 64-row survivor mask of that pair; it is handed to the pair's lane. ----
     uint64_t sieve = 0;
     uint64_t pairs_open;
-    {
-      double x, d, cost_base, bound;
-      objective(lds_min, x, d, cost_base, bound);
-      pairs_open = __ballot(active && (cost_base <= thr_b || bound <= thr_o));
-    }
+    pairs_open = __ballot(active && (floor_cost <= thr_b || floor_bound <= thr_o));
     if (pairs_open != 0) {
       lds_pair[threadIdx.x * kPairFields + 0] = thr_b;
       lds_pair[threadIdx.x * kPairFields + 1] = thr_o;
@@ -1310,7 +1323,8 @@ template <bool kFirstTile>
 __device__ __forceinline__ void exhaustive_block(
     const MistProblem &prob, const MistGroupDesc *__restrict__ g, int64_t row_begin,
     int64_t row_end, int p_tile, int lc_tile, const double *__restrict__ row_terms, double ratio,
-    double *lds_terms, double *__restrict__ out_cost, int32_t *__restrict__ out_index) {
+    double *lds_terms, int32_t *lds_row, double *__restrict__ out_cost,
+    int32_t *__restrict__ out_index) {
   const int L = prob.num_layers;
   const int n_pairs = L * (L + 1) / 2 + L;
   const int pair_idx = lc_tile * MIST_LC_TILE + threadIdx.x;
@@ -1345,11 +1359,13 @@ __device__ __forceinline__ void exhaustive_block(
       lds_terms[at] = v.x;
       lds_terms[at + 1] = v.y;
     }
+    // the reference's number of each staged row (lane = row: the index arithmetic once per row)
+    lds_row[threadIdx.x] = row_of_position(g, min(base + threadIdx.x, row_end - 1));
     __syncthreads();
     if (!active) continue;
     for (int r = 0; r < n_stage; ++r) {
       const double *t = lds_terms + r * kLdsRowStride;
-      const int32_t row = row_of_position(g, base + r);
+      const int32_t row = lds_row[r];
       const CellLatency lat = cell_latency<kFirstTile>(t, l, c, k);
       const LaneMemory mem = cell_memory(t, l, c);
       // objectives r * x + y (pareto.py:138): base with y = float32 delta / G in float32
@@ -1398,6 +1414,7 @@ __global__ __launch_bounds__(MIST_LC_TILE) void eval_reduce_exhaustive_kernel(
     const int32_t *__restrict__ block_prefix, int n_blocks, const double *__restrict__ row_terms,
     double ratio, double *__restrict__ partial_cost, int32_t *__restrict__ partial_index) {
   __shared__ double lds_terms[kStageRows * kLdsRowStride];
+  __shared__ int32_t lds_row[kStageRows];
   const int block = xcd_run_block(blockIdx.x);
   if (block >= n_blocks) return;
   int local_block;
@@ -1410,10 +1427,10 @@ __global__ __launch_bounds__(MIST_LC_TILE) void eval_reduce_exhaustive_kernel(
   const int64_t slab = (int64_t)kSlots * MIST_LC_TILE;
   if (p_tile == 0)
     exhaustive_block<true>(prob, g, row_begin, row_end, p_tile, lc_tile, row_terms, ratio,
-                           lds_terms, partial_cost + block * slab, partial_index + block * slab);
+                           lds_terms, lds_row, partial_cost + block * slab, partial_index + block * slab);
   else
     exhaustive_block<false>(prob, g, row_begin, row_end, p_tile, lc_tile, row_terms, ratio,
-                            lds_terms, partial_cost + block * slab, partial_index + block * slab);
+                            lds_terms, lds_row, partial_cost + block * slab, partial_index + block * slab);
 }
 
 // Combines the slabs of the kScoutSplit scout workgroups of every tile into the first of them,

@@ -65,6 +65,24 @@ int mist_mip_stage_samples(const MistMipShape *shape, const MistMipTables *table
                            const double *d_ratios, float *d_t_stable, float *d_t_delta,
                            int32_t *d_index, uint8_t *d_keep, void *stream);
 
+/* mist_mip_stage_samples for every problem of a search (all G, all stage counts) in ONE launch.
+ * items[n_items] (HOST) and d_items (the same array in DEVICE memory, uploaded by the caller):
+ * problem i owns workgroups first_block .. first_block + S_i * nl_i - 1 and writes its
+ * [S_i][nl_i][P] outputs from element out_offset on; both must continue the list (first_block
+ * and out_offset of problem 0 are 0, of problem i + 1 those of i plus its counts); problems
+ * without a layer count to sample are left out by the caller. */
+typedef struct MistMipBatchItem {
+  MistMipShape shape;
+  MistMipTables tables;
+  int64_t out_offset;
+  int32_t first_block, reserved;
+} MistMipBatchItem;
+int mist_sizeof_mip_batch_item(void);
+int mist_mip_stage_samples_batch(const MistMipBatchItem *items, const MistMipBatchItem *d_items,
+                                 int n_items, const double *d_ratios, float *d_t_stable,
+                                 float *d_t_delta, int32_t *d_index, uint8_t *d_keep,
+                                 void *stream);
+
 /* Exact solver for the assignment problem, on the host (replaces the PuLP / CBC call,
  * inter_tuning_mip.py:317-400).  `t_stable`, `t_delta`, `keep` are HOST copies of the arrays
  * above.  Writes the optimal objective and, per stage, the layer count and the sample slot.

@@ -31,6 +31,7 @@ extern "C" {
 #define MIST_P_TILE 16      /* pre-saved micro-batch values per thread of the reduce kernel */
 #endif
 #define MIST_MAX_MESH 16    /* device-mesh candidates of the inter-stage DP */
+#define MIST_MAX_SAMPLE_BATCH 16 /* alpha samples per mist_eval_reduce_samples call */
 
 #define MIST_E_INVALID (-1) /* argument / shape check failed, nothing was launched */
 #define MIST_E_HIP (-2)     /* a HIP runtime call failed */
@@ -194,6 +195,20 @@ int mist_eval_reduce(const MistProblem *problem, const MistGroupDesc *d_groups, 
                      const int32_t *d_scout_prefix, int n_scout_blocks,
                      const double *d_row_terms, const double *d_stage_floor, double ratio,
                      double *d_partial_cost, int32_t *d_partial_index, void *stream);
+
+/* mist_eval_reduce + mist_finalize for n_samples <= MIST_MAX_SAMPLE_BATCH ratios of the same
+ * row terms (reference: the S samples of one compute_indices call, mist/utils/pareto.py:124-144):
+ * the scout passes of all samples run as ONE launch (a single one fills a tenth of the GPU), then
+ * per sample the main launch seeded from its own scout slabs and the finalize into sample
+ * position sample_index[i].  `ratios` and `sample_index` are HOST arrays.
+ * d_partial_cost / d_partial_index: [n_blocks + n_samples * n_scout_blocks] slabs. */
+int mist_eval_reduce_samples(const MistProblem *problem, const MistGroupDesc *d_groups,
+                             int n_groups, const int32_t *d_block_prefix, int n_blocks,
+                             const int32_t *d_scout_prefix, int n_scout_blocks,
+                             const double *d_row_terms, const double *d_stage_floor,
+                             const double *ratios, const int32_t *sample_index, int n_samples,
+                             double *d_partial_cost, int32_t *d_partial_index,
+                             const MistOutTables *tables, void *stream);
 
 /* mist_eval_reduce with every cell evaluated: each (row, layers, ckpt) through the latency and
  * memory model and each pre-saved micro-batch value through the reference's feasibility test

@@ -23,6 +23,7 @@ SCOUT_SPLIT = 4  # replaced by the library's own value in load()
 STAGE_ROWS = 64  # replaced by the library's own value in load()
 TERMS_BLOCK = 128  # replaced by the library's own value in load()
 MAX_MESH = 16
+MAX_SAMPLE_BATCH = 16  # MIST_MAX_SAMPLE_BATCH
 DP_NO_START = -3
 DP_CKPT_TAIL, DP_CKPT_STAGE, DP_CKPT_ALL = 0, 1, 2
 DP_THRESHOLD, DP_BOTTLENECK = 0, 1
@@ -118,6 +119,11 @@ _SIGNATURES = {
         ctypes.c_int,
         [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, _VP, ctypes.c_double,
          _VP, _VP, _VP],
+    ),
+    "mist_eval_reduce_samples": (
+        ctypes.c_int,
+        [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, _VP, _VP, _VP,
+         ctypes.c_int, _VP, _VP, ctypes.POINTER(OutTables), _VP],
     ),
     "mist_eval_reduce_exhaustive": (
         ctypes.c_int,
@@ -243,6 +249,13 @@ class MipTables(ctypes.Structure):
     _fields_ = [("stable", ctypes.c_void_p * 4), ("delta", ctypes.c_void_p * 4)]
 
 
+class MipBatchItem(ctypes.Structure):
+    """``MistMipBatchItem``: one problem of a batched ``mist_mip_stage_samples_batch`` call."""
+
+    _fields_ = [("shape", MipShape), ("tables", MipTables), ("out_offset", ctypes.c_int64),
+                ("first_block", ctypes.c_int32), ("reserved", ctypes.c_int32)]
+
+
 _INTER_SIGNATURES = {
     "mist_inter_stage_search": (
         ctypes.c_int,
@@ -256,6 +269,9 @@ _MIP_SIGNATURES = {
         ctypes.c_int,
         [ctypes.POINTER(MipShape), ctypes.POINTER(MipTables), _VP, _VP, _VP, _VP, _VP, _VP],
     ),
+    "mist_sizeof_mip_batch_item": (ctypes.c_int, []),
+    "mist_mip_stage_samples_batch": (
+        ctypes.c_int, [_VP, _VP, ctypes.c_int, _VP, _VP, _VP, _VP, _VP, _VP]),
     "mist_mip_solve": (
         ctypes.c_int,
         [ctypes.POINTER(MipShape), ctypes.c_int, ctypes.c_double, _VP, _VP, _VP,
@@ -292,6 +308,10 @@ def load():
         raise MistLibraryError(
             f"MistMipShape layout mismatch: C {lib.mist_sizeof_mip_shape()} vs ctypes {ctypes.sizeof(MipShape)}"
         )
+    if lib.mist_sizeof_mip_batch_item() != ctypes.sizeof(MipBatchItem):
+        raise MistLibraryError(
+            f"MistMipBatchItem layout mismatch: C {lib.mist_sizeof_mip_batch_item()} vs ctypes "
+            f"{ctypes.sizeof(MipBatchItem)}")
     if lib.mist_sizeof_group() != GROUP_DTYPE.itemsize:
         raise MistLibraryError(
             f"MistGroupDesc layout mismatch: C {lib.mist_sizeof_group()} vs numpy {GROUP_DTYPE.itemsize}"

@@ -49,14 +49,15 @@ __device__ StageRow stage_row(const MistMipShape &s, const MistMipTables &t, int
   return {t.stable[v] + off, t.delta[v] + off};
 }
 
-__global__ __launch_bounds__(kSampleLanes) void stage_samples_kernel(
-    MistMipShape shape, MistMipTables tables, const double *__restrict__ ratios,
-    float *__restrict__ out_stable, float *__restrict__ out_delta, int32_t *__restrict__ out_index,
+// One (stage, layer count) row of one problem: `block` = stage * nl + (layers - layers_min).
+__device__ __forceinline__ void stage_samples_row(
+    const MistMipShape &shape, const MistMipTables &tables, int block, float *lds,
+    const double *__restrict__ ratios, float *__restrict__ out_stable,
+    float *__restrict__ out_delta, int32_t *__restrict__ out_index,
     uint8_t *__restrict__ out_keep) {
-  extern __shared__ float lds[];
   const int P = shape.sample_size, L = shape.num_layers;
   const int nl = shape.layers_max - shape.layers_min + 1;
-  const int stage = blockIdx.x / nl, layers = shape.layers_min + blockIdx.x % nl;
+  const int stage = block / nl, layers = shape.layers_min + block % nl;
   const int lane = threadIdx.x;
 
   int n_cand = P, first = 0;  // candidates of the row: all planes, or one ckpt plane
@@ -100,11 +101,38 @@ __global__ __launch_bounds__(kSampleLanes) void stage_samples_kernel(
   if (sy < 0.0f) sy = 0.0f;
   if (sx == INFINITY) sx = MIST_MIP_MAX_VALUE;
   if (sy == INFINITY) sy = MIST_MIP_MAX_VALUE;
-  const int64_t o = (int64_t)blockIdx.x * P + lane;
+  const int64_t o = (int64_t)block * P + lane;
   out_stable[o] = sx;
   out_delta[o] = sy;
   out_index[o] = best;
   out_keep[o] = keep ? 1 : 0;
+}
+
+__global__ __launch_bounds__(kSampleLanes) void stage_samples_kernel(
+    MistMipShape shape, MistMipTables tables, const double *__restrict__ ratios,
+    float *__restrict__ out_stable, float *__restrict__ out_delta, int32_t *__restrict__ out_index,
+    uint8_t *__restrict__ out_keep) {
+  extern __shared__ float lds[];
+  stage_samples_row(shape, tables, blockIdx.x, lds, ratios, out_stable, out_delta, out_index,
+                    out_keep);
+}
+
+// Every problem of a search in one launch: workgroup -> (problem, row) through the problems'
+// first workgroups (ascending); outputs of problem i start at its out_offset.
+__global__ __launch_bounds__(kSampleLanes) void stage_samples_batch_kernel(
+    const MistMipBatchItem *__restrict__ items, int n_items, const double *__restrict__ ratios,
+    float *__restrict__ out_stable, float *__restrict__ out_delta, int32_t *__restrict__ out_index,
+    uint8_t *__restrict__ out_keep) {
+  extern __shared__ float lds[];
+  int lo = 0, hi = n_items;  // items[lo].first_block <= blockIdx.x < items[hi].first_block
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (items[mid].first_block <= (int)blockIdx.x) lo = mid; else hi = mid;
+  }
+  const MistMipBatchItem &it = items[lo];
+  const int64_t o = it.out_offset;
+  stage_samples_row(it.shape, it.tables, (int)blockIdx.x - it.first_block, lds, ratios,
+                    out_stable + o, out_delta + o, out_index + o, out_keep + o);
 }
 
 int check_mip_shape(const MistMipShape *s) {
@@ -153,6 +181,43 @@ int mist_mip_stage_samples(const MistMipShape *shape, const MistMipTables *table
   hipLaunchKernelGGL(stage_samples_kernel, dim3((unsigned)(shape->num_stages * nl)),
                      dim3(kSampleLanes), (size_t)lds_bytes, (hipStream_t)stream, *shape, *tables,
                      d_ratios, d_t_stable, d_t_delta, d_index, d_keep);
+  MIST_HIP_CHECK(hipGetLastError());
+  return 0;
+}
+
+int mist_sizeof_mip_batch_item(void) { return (int)sizeof(MistMipBatchItem); }
+
+int mist_mip_stage_samples_batch(const MistMipBatchItem *items, const MistMipBatchItem *d_items,
+                                 int n_items, const double *d_ratios, float *d_t_stable,
+                                 float *d_t_delta, int32_t *d_index, uint8_t *d_keep,
+                                 void *stream) {
+  if (!items || !d_items || n_items <= 0)
+    return fail(MIST_E_INVALID, "null / empty problem list (n_items=%d)", n_items);
+  if (!d_ratios || !d_t_stable || !d_t_delta || !d_index || !d_keep)
+    return fail(MIST_E_INVALID, "null pointer");
+  int64_t blocks = 0, lds_bytes = 0, out = 0;
+  for (int i = 0; i < n_items; ++i) {
+    const MistMipShape *s = &items[i].shape;
+    if (int rc = check_mip_shape(s)) return rc;
+    const int nl = s->layers_max - s->layers_min + 1;
+    if (nl <= 0) return fail(MIST_E_INVALID, "problem %d has no layer count to sample", i);
+    for (int v = 0; v < 4; ++v)
+      if (!items[i].tables.stable[v] || !items[i].tables.delta[v])
+        return fail(MIST_E_INVALID, "problem %d: null table of variant %d", i, v);
+    if (items[i].first_block != blocks || items[i].out_offset != out)
+      return fail(MIST_E_INVALID, "problem %d: first_block / out_offset do not continue the list", i);
+    blocks += (int64_t)s->num_stages * nl;
+    out += (int64_t)s->num_stages * nl * s->sample_size;
+    const int64_t n_cand = s->ckpt_mode == MIST_MIP_CKPT_TUNED
+                               ? (int64_t)(s->num_layers + 1) * s->sample_size : s->sample_size;
+    lds_bytes = std::max<int64_t>(lds_bytes, (2 * n_cand + 2 * kSampleLanes) * (int64_t)sizeof(float));
+  }
+  if (lds_bytes > 64 * 1024)
+    return fail(MIST_E_INVALID, "candidates per table row exceed the LDS staging buffer");
+  if (blocks >= (int64_t)1 << 31) return fail(MIST_E_INVALID, "too many rows for one launch");
+  hipLaunchKernelGGL(stage_samples_batch_kernel, dim3((unsigned)blocks), dim3(kSampleLanes),
+                     (size_t)lds_bytes, (hipStream_t)stream, d_items, n_items, d_ratios,
+                     d_t_stable, d_t_delta, d_index, d_keep);
   MIST_HIP_CHECK(hipGetLastError());
   return 0;
 }

@@ -749,6 +749,11 @@ __device__ __forceinline__ int64_t gathered_position(const MistGroupDesc *g, int
   return par * g->n_off + (int64_t)ao * g->n_oo * g->n_pair + tile_position(g, oo, (int)pair);
 }
 
+// alpha / (1 - alpha) of the samples of one launch (by value in the kernel arguments)
+struct RatioList {
+  double r[MIST_MAX_SAMPLE_BATCH];
+};
+
 template <bool kPow2G, bool kFirstTile>
 __device__ __forceinline__ void reduce_block(
     const MistProblem &prob, const MistGroupDesc *__restrict__ g, const ReduceRange range,
@@ -1257,14 +1262,19 @@ __global__ __launch_bounds__(MIST_LC_TILE, MIST_REDUCE_MIN_WAVES) void eval_redu
     const MistProblem prob, const MistGroupDesc *__restrict__ groups, int n_groups,
     const int32_t *__restrict__ block_prefix, int n_blocks,
     const int32_t *__restrict__ scout_prefix, int scout, const double *__restrict__ row_terms,
-    const double *__restrict__ stage_floor, double ratio, double *__restrict__ partial_cost,
-    int32_t *__restrict__ partial_index) {
+    const double *__restrict__ stage_floor, const RatioList ratios, int seed_sample,
+    double *__restrict__ partial_cost, int32_t *__restrict__ partial_index) {
   __shared__ double lds_terms[kStageRows * kLdsRowStride];
   __shared__ double lds_min[kStageFloorPitch];
   __shared__ double lds_pair[MIST_LC_TILE * kPairFields];
   __shared__ int32_t lds_rowpos[kStageRows];
+  // Scout launch: blockIdx.y = sample, its slabs follow those of the samples before it.  Main
+  // launch: one sample, seeded from the scout slabs of sample `seed_sample`.
+  const int sample = scout ? (int)blockIdx.y : 0;
+  const double ratio = ratios.r[sample];
+  const int n_scout_total = scout_prefix != nullptr ? scout_prefix[n_groups] : 0;
   const int block = xcd_run_block(blockIdx.x);
-  if (block >= (scout ? scout_prefix[n_groups] : n_blocks)) return;
+  if (block >= (scout ? n_scout_total : n_blocks)) return;
   int local_block;
   const MistGroupDesc *g = find_group(groups, scout ? scout_prefix : block_prefix, n_groups,
                                       block, &local_block);
@@ -1279,7 +1289,7 @@ __global__ __launch_bounds__(MIST_LC_TILE, MIST_REDUCE_MIN_WAVES) void eval_redu
     tile = local_block / kScoutSplit;
     const int part = local_block % kScoutSplit;  // gathered stages part, part + split, ...
     range = ReduceRange{(int64_t)part * kStageRows, g->n_rows, kScoutSplit, 0, 1};
-    out_slab = (int64_t)n_blocks + block;
+    out_slab = (int64_t)n_blocks + (int64_t)sample * n_scout_total + block;
   } else {
     const int n_tiles = g->n_lc_tiles * g->n_p_tiles;
     const int chunk = local_block / n_tiles;  // the tiles of one chunk are neighbours
@@ -1292,8 +1302,8 @@ __global__ __launch_bounds__(MIST_LC_TILE, MIST_REDUCE_MIN_WAVES) void eval_redu
   const int p_tile = tile % g->n_p_tiles;
   const int lc_tile = tile / g->n_p_tiles;
   const int64_t slab = (int64_t)kSlots * MIST_LC_TILE;
-  const int64_t seed_slab =
-      (int64_t)n_blocks + (seeded ? scout_prefix[gi] + tile * kScoutSplit : 0);
+  const int64_t seed_slab = (int64_t)n_blocks + (int64_t)seed_sample * n_scout_total +
+                            (seeded ? scout_prefix[gi] + tile * kScoutSplit : 0);
   const double *seed_cost = (!scout && seeded) ? partial_cost + seed_slab * slab : nullptr;
   const int32_t *seed_index = (!scout && seeded) ? partial_index + seed_slab * slab : nullptr;
   const bool pow2 = (g->grad_accum & (g->grad_accum - 1)) == 0;
@@ -1436,11 +1446,12 @@ __global__ __launch_bounds__(MIST_LC_TILE) void eval_reduce_exhaustive_kernel(
 // Combines the slabs of the kScoutSplit scout workgroups of every tile into the first of them,
 // so that each chunk of the main launch reads one slab of seeds instead of kScoutSplit.
 // Workgroup = tile; the scout slabs of tile t are n_blocks + t * kScoutSplit + k.
-__global__ __launch_bounds__(256) void merge_scout_kernel(int n_blocks,
+__global__ __launch_bounds__(256) void merge_scout_kernel(int n_blocks, int n_scout_total,
                                                           double *__restrict__ partial_cost,
                                                           int32_t *__restrict__ partial_index) {
   const int64_t slab = (int64_t)kSlots * MIST_LC_TILE;
-  const int64_t first = ((int64_t)n_blocks + (int64_t)blockIdx.x * kScoutSplit) * slab;
+  const int64_t first = ((int64_t)n_blocks + (int64_t)blockIdx.y * n_scout_total +
+                         (int64_t)blockIdx.x * kScoutSplit) * slab;
   for (int e = threadIdx.x; e < (int)slab; e += blockDim.x) {
     double best = INFINITY;
     int32_t best_row = -1;
@@ -1653,40 +1664,108 @@ int64_t mist_stage_floor_doubles(int64_t total_rows, int n_groups) {
   return (total_rows / kStageRows + n_groups + 1) * kStageFloorPitch;
 }
 
+// Scout launch + slab merge for n_samples ratios at once (grid.y = sample).
+static int launch_scout(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,
+                        const int32_t *d_block_prefix, int n_blocks, const int32_t *scout_prefix,
+                        int n_scout_blocks, const double *d_row_terms, const double *d_stage_floor,
+                        const RatioList &ratios, int n_samples, double *d_partial_cost,
+                        int32_t *d_partial_index, void *stream) {
+  if (n_scout_blocks % kScoutSplit != 0)
+    return fail(MIST_E_INVALID, "n_scout_blocks %d is not a multiple of the scout split %d",
+                n_scout_blocks, kScoutSplit);
+  hipLaunchKernelGGL(eval_reduce_kernel, dim3(xcd_padded_grid(n_scout_blocks), n_samples),
+                     dim3(MIST_LC_TILE), 0, (hipStream_t)stream, *problem, d_groups, n_groups,
+                     d_block_prefix, n_blocks, scout_prefix, 1, d_row_terms, d_stage_floor, ratios,
+                     0, d_partial_cost, d_partial_index);
+  MIST_HIP_CHECK(hipGetLastError());
+  if (kScoutSplit > 1) {
+    hipLaunchKernelGGL(merge_scout_kernel, dim3(n_scout_blocks / kScoutSplit, n_samples), dim3(256),
+                       0, (hipStream_t)stream, n_blocks, n_scout_blocks, d_partial_cost,
+                       d_partial_index);
+    MIST_HIP_CHECK(hipGetLastError());
+  }
+  return 0;
+}
+
+static int check_reduce_arguments(const MistProblem *problem, const MistGroupDesc *d_groups,
+                                  int n_groups, const int32_t *d_block_prefix, int n_blocks,
+                                  const int32_t *d_scout_prefix, int n_scout_blocks,
+                                  const double *d_row_terms, const double *d_stage_floor,
+                                  const double *d_partial_cost, const int32_t *d_partial_index) {
+  if (int rc = check_common(problem, d_groups, n_groups)) return rc;
+  if (!d_block_prefix || !d_row_terms || !d_stage_floor || !d_partial_cost || !d_partial_index)
+    return fail(MIST_E_INVALID, "null workspace pointer");
+  if (n_blocks <= 0) return fail(MIST_E_INVALID, "n_blocks must be positive, got %d", n_blocks);
+  if (n_scout_blocks < 0 || (n_scout_blocks > 0 && !d_scout_prefix))
+    return fail(MIST_E_INVALID, "scout blocks need a scout prefix (n_scout_blocks=%d)",
+                n_scout_blocks);
+  return 0;
+}
+
 int mist_eval_reduce(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,
                      const int32_t *d_block_prefix, int n_blocks,
                      const int32_t *d_scout_prefix, int n_scout_blocks,
                      const double *d_row_terms, const double *d_stage_floor, double ratio,
                      double *d_partial_cost, int32_t *d_partial_index, void *stream) {
-  if (int rc = check_common(problem, d_groups, n_groups)) return rc;
-  if (!d_block_prefix || !d_row_terms || !d_stage_floor || !d_partial_cost || !d_partial_index)
-    return fail(MIST_E_INVALID, "null workspace pointer");
-  if (n_blocks <= 0) return fail(MIST_E_INVALID, "n_blocks must be positive, got %d", n_blocks);
+  if (int rc = check_reduce_arguments(problem, d_groups, n_groups, d_block_prefix, n_blocks,
+                                      d_scout_prefix, n_scout_blocks, d_row_terms, d_stage_floor,
+                                      d_partial_cost, d_partial_index))
+    return rc;
   if (!(ratio >= 0.0)) return fail(MIST_E_INVALID, "ratio must be non-negative");
-  if (n_scout_blocks < 0 || (n_scout_blocks > 0 && !d_scout_prefix))
-    return fail(MIST_E_INVALID, "scout blocks need a scout prefix (n_scout_blocks=%d)",
-                n_scout_blocks);
   const int32_t *scout_prefix = n_scout_blocks > 0 ? d_scout_prefix : nullptr;
-  if (scout_prefix) {
-    hipLaunchKernelGGL(eval_reduce_kernel, dim3(xcd_padded_grid(n_scout_blocks)), dim3(MIST_LC_TILE), 0,
-                       (hipStream_t)stream, *problem, d_groups, n_groups, d_block_prefix,
-                       n_blocks, scout_prefix, 1, d_row_terms, d_stage_floor, ratio,
-                       d_partial_cost, d_partial_index);
-    MIST_HIP_CHECK(hipGetLastError());
-    if (kScoutSplit > 1) {
-      if (n_scout_blocks % kScoutSplit != 0)
-        return fail(MIST_E_INVALID, "n_scout_blocks %d is not a multiple of the scout split %d",
-                    n_scout_blocks, kScoutSplit);
-      hipLaunchKernelGGL(merge_scout_kernel, dim3(n_scout_blocks / kScoutSplit), dim3(256), 0,
-                         (hipStream_t)stream, n_blocks, d_partial_cost, d_partial_index);
-      MIST_HIP_CHECK(hipGetLastError());
-    }
-  }
+  RatioList ratios = {};
+  ratios.r[0] = ratio;
+  if (scout_prefix)
+    if (int rc = launch_scout(problem, d_groups, n_groups, d_block_prefix, n_blocks, scout_prefix,
+                              n_scout_blocks, d_row_terms, d_stage_floor, ratios, 1,
+                              d_partial_cost, d_partial_index, stream))
+      return rc;
   hipLaunchKernelGGL(eval_reduce_kernel, dim3(xcd_padded_grid(n_blocks)), dim3(MIST_LC_TILE), 0,
                      (hipStream_t)stream, *problem, d_groups, n_groups, d_block_prefix, n_blocks,
-                     scout_prefix, 0, d_row_terms, d_stage_floor, ratio, d_partial_cost,
+                     scout_prefix, 0, d_row_terms, d_stage_floor, ratios, 0, d_partial_cost,
                      d_partial_index);
   MIST_HIP_CHECK(hipGetLastError());
+  return 0;
+}
+
+int mist_eval_reduce_samples(const MistProblem *problem, const MistGroupDesc *d_groups,
+                             int n_groups, const int32_t *d_block_prefix, int n_blocks,
+                             const int32_t *d_scout_prefix, int n_scout_blocks,
+                             const double *d_row_terms, const double *d_stage_floor,
+                             const double *ratios, const int32_t *sample_index, int n_samples,
+                             double *d_partial_cost, int32_t *d_partial_index,
+                             const MistOutTables *tables, void *stream) {
+  if (int rc = check_reduce_arguments(problem, d_groups, n_groups, d_block_prefix, n_blocks,
+                                      d_scout_prefix, n_scout_blocks, d_row_terms, d_stage_floor,
+                                      d_partial_cost, d_partial_index))
+    return rc;
+  if (!ratios || !sample_index || n_samples < 1 || n_samples > MIST_MAX_SAMPLE_BATCH)
+    return fail(MIST_E_INVALID, "n_samples %d outside [1, %d] or null sample lists", n_samples,
+                MIST_MAX_SAMPLE_BATCH);
+  RatioList all = {};
+  for (int i = 0; i < n_samples; ++i) {
+    if (!(ratios[i] >= 0.0)) return fail(MIST_E_INVALID, "ratio %d must be non-negative", i);
+    all.r[i] = ratios[i];
+  }
+  const int32_t *scout_prefix = n_scout_blocks > 0 ? d_scout_prefix : nullptr;
+  // the scout passes of all samples in one launch: a single one occupies a tenth of the GPU
+  if (scout_prefix)
+    if (int rc = launch_scout(problem, d_groups, n_groups, d_block_prefix, n_blocks, scout_prefix,
+                              n_scout_blocks, d_row_terms, d_stage_floor, all, n_samples,
+                              d_partial_cost, d_partial_index, stream))
+      return rc;
+  for (int i = 0; i < n_samples; ++i) {
+    RatioList one = {};
+    one.r[0] = ratios[i];
+    hipLaunchKernelGGL(eval_reduce_kernel, dim3(xcd_padded_grid(n_blocks)), dim3(MIST_LC_TILE), 0,
+                       (hipStream_t)stream, *problem, d_groups, n_groups, d_block_prefix, n_blocks,
+                       scout_prefix, 0, d_row_terms, d_stage_floor, one, i, d_partial_cost,
+                       d_partial_index);
+    MIST_HIP_CHECK(hipGetLastError());
+    if (int rc = mist_finalize(problem, d_groups, n_groups, d_block_prefix, d_row_terms,
+                               d_partial_cost, d_partial_index, sample_index[i], tables, stream))
+      return rc;
+  }
   return 0;
 }
 

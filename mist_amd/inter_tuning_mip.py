@@ -83,18 +83,24 @@ def stage_samples(results: IntraStageTunerOutput, problems: List[_Problem]):
         index = torch.empty(max(total, 1), dtype=torch.int32, device=dev)
         keep = torch.empty(max(total, 1), dtype=torch.uint8, device=dev)
         stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
-        for p in problems:
-            if p.count == 0:
-                continue
-            slices = _lib.MipTables()
-            for v in range(4):
-                slices.stable[v] = tables.stable[v][p.g, p.q].data_ptr()
-                slices.delta[v] = tables.delta[v][p.g, p.q].data_ptr()
-            rc = lib.mist_mip_stage_samples(
-                ctypes.byref(p.shape), ctypes.byref(slices), ratios.data_ptr(),
-                t_stable.data_ptr() + 4 * p.offset, t_delta.data_ptr() + 4 * p.offset,
-                index.data_ptr() + 4 * p.offset, keep.data_ptr() + p.offset, stream)
-            _lib.check(rc, "mist_mip_stage_samples")
+        live = [p for p in problems if p.count > 0]
+        if live:
+            # every problem in one launch: the rows are a few hundred candidates each, and one
+            # launch per problem (~220 for a 32-layer plan) left the GPU to one wavefront per row
+            items = (_lib.MipBatchItem * len(live))()
+            first_block = 0
+            for item, p in zip(items, live):
+                item.shape = p.shape
+                for v in range(4):
+                    item.tables.stable[v] = tables.stable[v][p.g, p.q].data_ptr()
+                    item.tables.delta[v] = tables.delta[v][p.g, p.q].data_ptr()
+                item.out_offset, item.first_block = p.offset, first_block
+                first_block += p.count // P
+            d_items = torch.frombuffer(bytearray(bytes(items)), dtype=torch.uint8).to(dev)
+            rc = lib.mist_mip_stage_samples_batch(
+                ctypes.byref(items), d_items.data_ptr(), len(live), ratios.data_ptr(),
+                t_stable.data_ptr(), t_delta.data_ptr(), index.data_ptr(), keep.data_ptr(), stream)
+            _lib.check(rc, "mist_mip_stage_samples_batch")
         return (t_stable.cpu().numpy(), t_delta.cpu().numpy(), index.cpu().numpy(),
                 keep.cpu().numpy())
 

@@ -349,7 +349,9 @@ class IntraStageTuner:
             ))
         max_rows = max([b["total_rows"] for b in batches], default=0)
         max_groups = max([b["n_groups"] for b in batches], default=0)
-        n_slabs = max([b["n_reduce_blocks"] + b["n_scout_blocks"] for b in batches] + [1])
+        # several samples share one scout launch: their scout slabs lie behind one another
+        self._sample_batch = min(len(self.sample_slots), _lib.MAX_SAMPLE_BATCH)
+        n_slabs = max([b["n_reduce_blocks"] + self._sample_batch * b["n_scout_blocks"] for b in batches] + [1])
         def workspace():
             return dict(
                 row_terms=torch.empty(max(max_rows, 1) * _lib.ROW_TERMS, dtype=torch.float64, device=dev),
@@ -422,6 +424,23 @@ class IntraStageTuner:
                     _ptr(w["row_terms"]), _ptr(w["stage_floor"]), float(ratios[slot]),
                     _ptr(w["partial_cost"]), _ptr(w["partial_index"]), stream)
 
+            if events is None and not self.exhaustive and len(self.sample_slots) > 1:
+                _lib.check(lib.mist_row_terms(
+                    prob_ptr, _ptr(d["groups"]), d["n_groups"], _ptr(d["terms_prefix"]),
+                    d["n_terms_blocks"], _ptr(w["row_terms"]), _ptr(w["stage_floor"]), stream),
+                    "mist_row_terms")
+                for first in range(0, len(self.sample_slots), self._sample_batch):
+                    slots = np.array(self.sample_slots[first:first + self._sample_batch], dtype=np.int32)
+                    batch_ratios = np.ascontiguousarray(ratios[slots], dtype=np.float64)
+                    rc = lib.mist_eval_reduce_samples(
+                        prob_ptr, _ptr(d["groups"]), d["n_groups"], _ptr(d["reduce_prefix"]),
+                        d["n_reduce_blocks"], _ptr(d["scout_prefix"]), d["n_scout_blocks"],
+                        _ptr(w["row_terms"]), _ptr(w["stage_floor"]),
+                        ctypes.c_void_p(batch_ratios.ctypes.data), ctypes.c_void_p(slots.ctypes.data),
+                        len(slots), _ptr(w["partial_cost"]), _ptr(w["partial_index"]),
+                        ctypes.byref(out), stream)
+                    _lib.check(rc, "mist_eval_reduce_samples")
+                continue
             for i, slot in enumerate(self.sample_slots):
                 if events is None and not self.exhaustive:
                     rc = lib.mist_intra_stage_eval(

@@ -87,7 +87,10 @@ typedef struct MistProblem {
   int32_t num_grad_accum;  /* extent of the g axis */
   int32_t num_mesh;        /* extent of the q axis */
   int32_t adv_first_block; /* enable_advanced_opt_in_first_block */
-  int32_t reserved[2];
+  int32_t max_scout_rows;  /* largest n_par * n_oo * n_ao * scout_stride of the call's groups with a
+                            * scout pass; 0 = unknown (mist_intra_stage_eval then runs the row
+                            * terms and the scout pass one after the other) */
+  int32_t reserved;
 } MistProblem;
 
 /* One (gradient-accumulation steps, device mesh) group = one call of the reference's

@@ -57,7 +57,8 @@ PROBLEM_DTYPE = np.dtype(
         ("num_grad_accum", "<i4"),
         ("num_mesh", "<i4"),
         ("adv_first_block", "<i4"),
-        ("reserved", "<i4", (2,)),
+        ("max_scout_rows", "<i4"),
+        ("reserved", "<i4"),
     ],
     align=True,
 )

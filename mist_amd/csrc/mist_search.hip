@@ -11,6 +11,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <type_traits>
 
 #include "mist_common.h"
@@ -304,12 +305,36 @@ __device__ __forceinline__ int64_t position_of_row(const MistGroupDesc *g, int64
 // ------------------------------------------------------------------------------------------
 // Kernel 1: row-invariant terms.  One thread per candidate row (workspace position).
 // ------------------------------------------------------------------------------------------
+// kMode 0: every row of every group.  kMode 1: only the rows the scout pass gathers (workgroup
+// = (128 gathered rows, group); no stage summaries), so that the scout pass can start while
+// kMode 2 computes everything: that one leaves the stores of the gathered rows out (the scout
+// pass may be reading them) and is otherwise kMode 0.
+__device__ __forceinline__ int64_t gathered_position(const MistGroupDesc *g, int64_t q);
+__device__ __forceinline__ bool is_scout_pair(const MistGroupDesc *g, int pair) {
+  if (g->scout_stride <= 0) return false;
+  if (g->scout_stride == 1) return pair == 0;
+  for (int k = 0; k < g->scout_stride; ++k)
+    if (pair == (int)((int64_t)k * (g->n_pair - 1) / (g->scout_stride - 1))) return true;
+  return false;
+}
+
+template <int kMode>
 __global__ __launch_bounds__(kTermsBlock) void row_terms_kernel(
     const MistProblem prob, const MistGroupDesc *__restrict__ groups, int n_groups,
     const int32_t *__restrict__ block_prefix, double *__restrict__ row_terms,
     double *__restrict__ stage_floor) {
   int local_block;
-  const MistGroupDesc *g = find_group(groups, block_prefix, n_groups, blockIdx.x, &local_block);
+  const MistGroupDesc *g;
+  int64_t n_here_total;  // rows this launch computes for the group
+  if (kMode == 1) {
+    g = groups + blockIdx.y;
+    local_block = blockIdx.x;
+    n_here_total = g->scout_stride > 0 ? (int64_t)g->n_par * g->n_oo * g->n_ao * g->scout_stride : 0;
+    if ((int64_t)local_block * kTermsBlock >= n_here_total) return;
+  } else {
+    g = find_group(groups, block_prefix, n_groups, blockIdx.x, &local_block);
+    n_here_total = g->n_rows;
+  }
   // The block's terms are assembled in LDS (row pitch 35 doubles: conflict-free) and written out
   // as one contiguous, fully coalesced range; a lane writing its own 272-byte row would touch
   // 34 partial cache lines.
@@ -318,13 +343,15 @@ __global__ __launch_bounds__(kTermsBlock) void row_terms_kernel(
   // make every lane keep a private copy of the whole struct in scratch memory.
   __shared__ double lds_factor[11][4];
   __shared__ double lds_gpu_gpu[32];
+  __shared__ unsigned char lds_skip[kTermsBlock];
   if (threadIdx.x < 44) lds_factor[threadIdx.x / 4][threadIdx.x % 4] = prob.interf_factor[threadIdx.x / 4][threadIdx.x % 4];
   if (threadIdx.x >= 64 && threadIdx.x < 96) lds_gpu_gpu[threadIdx.x - 64] = prob.gpu_gpu[threadIdx.x - 64];
   __syncthreads();
   const int64_t block_first = (int64_t)local_block * kTermsBlock;
-  const int rows_here = (int)min((int64_t)kTermsBlock, g->n_rows - block_first);
+  const int rows_here = (int)min((int64_t)kTermsBlock, n_here_total - block_first);
   // Lanes past the end recompute the last row (no divergent barrier); their result is dropped.
-  const int64_t row = block_first + min((int)threadIdx.x, rows_here - 1);  // workspace position
+  const int64_t nth = block_first + min((int)threadIdx.x, rows_here - 1);
+  const int64_t row = kMode == 1 ? gathered_position(g, nth) : nth;  // workspace position
 
   // ---- index decomposition (batched_module_analyzer.py:490-534) ----
   const RowParts parts = parts_of_position(g, row);
@@ -501,10 +528,22 @@ __global__ __launch_bounds__(kTermsBlock) void row_terms_kernel(
   t[MIST_T_RD] = raw_nock - S_nock;
 
   __syncthreads();
+  if (kMode == 1) {  // scattered rows: every lane writes its own
+    if ((int)threadIdx.x < rows_here) {
+      double2 *__restrict__ mine =
+          reinterpret_cast<double2 *>(row_terms + (g->row_offset + row) * MIST_ROW_TERMS);
+      for (int i = 0; i < MIST_ROW_TERMS / 2; ++i) mine[i] = make_double2(t[2 * i], t[2 * i + 1]);
+    }
+    return;
+  }
   double2 *__restrict__ dst =
       reinterpret_cast<double2 *>(row_terms + (g->row_offset + block_first) * MIST_ROW_TERMS);
+  if (kMode == 2) lds_skip[threadIdx.x] = is_scout_pair(g, pair) ? 1 : 0;
+  if (kMode == 2) __syncthreads();
   for (int i = threadIdx.x; i < rows_here * (MIST_ROW_TERMS / 2); i += kTermsBlock) {
-    const int at = (i / (MIST_ROW_TERMS / 2)) * (MIST_ROW_TERMS + 1) + 2 * (i % (MIST_ROW_TERMS / 2));
+    const int r = i / (MIST_ROW_TERMS / 2);
+    if (kMode == 2 && lds_skip[r]) continue;  // written by the kMode 1 launch
+    const int at = r * (MIST_ROW_TERMS + 1) + 2 * (i % (MIST_ROW_TERMS / 2));
     dst[i] = make_double2(lds_out[at], lds_out[at + 1]);
   }
   // Summary of each stage of kStageRows rows for the reduce kernel: lane = (column, half of the
@@ -1618,6 +1657,17 @@ __global__ __launch_bounds__(64) void analyze_kernel(
   o[19] = pb_post + g->pre_states + g->pre_saved;
 }
 
+int check_factors(const MistProblem *problem) {
+  for (int m = 0; m < 11; ++m)
+    for (int i = 0; i < 4; ++i) {
+      const double f = problem->interf_factor[m][i];
+      // the kernel takes 0 / f == +0 for granted
+      if (!(f > 0.0) || std::isinf(f))
+        return fail(MIST_E_INVALID, "interference factor [%d][%d] must be positive and finite", m, i);
+    }
+  return 0;
+}
+
 int check_common(const void *d_problem, const void *d_groups, int n_groups) {
   if (!d_problem || !d_groups) return fail(MIST_E_INVALID, "null problem / group pointer");
   if (n_groups <= 0) return fail(MIST_E_INVALID, "n_groups must be positive, got %d", n_groups);
@@ -1641,14 +1691,8 @@ int mist_row_terms(const MistProblem *problem, const MistGroupDesc *d_groups, in
   if (!d_block_prefix || !d_row_terms || !d_stage_floor)
     return fail(MIST_E_INVALID, "null workspace pointer");
   if (n_blocks <= 0) return fail(MIST_E_INVALID, "n_blocks must be positive, got %d", n_blocks);
-  for (int m = 0; m < 11; ++m)
-    for (int i = 0; i < 4; ++i) {
-      const double f = problem->interf_factor[m][i];
-      // the kernel takes 0 / f == +0 for granted
-      if (!(f > 0.0) || std::isinf(f))
-        return fail(MIST_E_INVALID, "interference factor [%d][%d] must be positive and finite", m, i);
-    }
-  hipLaunchKernelGGL(row_terms_kernel, dim3(n_blocks), dim3(kTermsBlock), 0, (hipStream_t)stream,
+  if (int rc = check_factors(problem)) return rc;
+  hipLaunchKernelGGL(row_terms_kernel<0>, dim3(n_blocks), dim3(kTermsBlock), 0, (hipStream_t)stream,
                      *problem, d_groups, n_groups, d_block_prefix, d_row_terms, d_stage_floor);
   MIST_HIP_CHECK(hipGetLastError());
   return 0;
@@ -1811,6 +1855,31 @@ int mist_finalize(const MistProblem *problem, const MistGroupDesc *d_groups, int
   return 0;
 }
 
+// Second stream and events of mist_intra_stage_eval, one set per device, kept for the life of
+// the process.
+namespace {
+struct OverlapStreams {
+  hipStream_t side = nullptr;
+  hipEvent_t rows_ready = nullptr, scout_done = nullptr;
+};
+int overlap_streams(OverlapStreams **out) {
+  static std::mutex lock;
+  static OverlapStreams known[64];
+  int device = 0;
+  MIST_HIP_CHECK(hipGetDevice(&device));
+  if (device < 0 || device >= 64) return fail(MIST_E_INVALID, "device ordinal %d outside [0, 64)", device);
+  std::lock_guard<std::mutex> guard(lock);
+  OverlapStreams &s = known[device];
+  if (s.side == nullptr) {
+    MIST_HIP_CHECK(hipStreamCreateWithFlags(&s.side, hipStreamNonBlocking));  // default priority
+    MIST_HIP_CHECK(hipEventCreateWithFlags(&s.rows_ready, hipEventDisableTiming));
+    MIST_HIP_CHECK(hipEventCreateWithFlags(&s.scout_done, hipEventDisableTiming));
+  }
+  *out = &s;
+  return 0;
+}
+}  // namespace
+
 int mist_intra_stage_eval(const MistProblem *problem, const MistGroupDesc *d_groups,
                           int n_groups, const int32_t *d_terms_block_prefix, int n_terms_blocks,
                           const int32_t *d_reduce_block_prefix, int n_reduce_blocks,
@@ -1818,6 +1887,49 @@ int mist_intra_stage_eval(const MistProblem *problem, const MistGroupDesc *d_gro
                           double *d_stage_floor, double *d_partial_cost, int32_t *d_partial_index,
                           double ratio, int sample_index, int compute_terms,
                           const MistOutTables *tables, void *stream) {
+  if (compute_terms && n_scout_blocks > 0 && problem != nullptr && problem->max_scout_rows > 0 &&
+      n_groups > 0 && n_groups <= 65535) {
+    // The scout pass reads a few hundred rows per group and leaves most of the GPU idle; the row
+    // terms of everything else are computed beside it.  Stream order: [terms of the gathered
+    // rows] -> side stream: scout pass + merge || this stream: all other row terms -> main
+    // launch -> finalize.
+    if (int rc = check_reduce_arguments(problem, d_groups, n_groups, d_reduce_block_prefix,
+                                        n_reduce_blocks, d_scout_prefix, n_scout_blocks,
+                                        d_row_terms, d_stage_floor, d_partial_cost, d_partial_index))
+      return rc;
+    if (!d_terms_block_prefix || n_terms_blocks <= 0)
+      return fail(MIST_E_INVALID, "null / empty row-term decomposition");
+    if (int rc = check_factors(problem)) return rc;
+    if (!(ratio >= 0.0)) return fail(MIST_E_INVALID, "ratio must be non-negative");
+    OverlapStreams *os = nullptr;
+    if (int rc = overlap_streams(&os)) return rc;
+    hipStream_t main_stream = (hipStream_t)stream;
+    const unsigned scout_term_blocks = (unsigned)((problem->max_scout_rows + kTermsBlock - 1) / kTermsBlock);
+    hipLaunchKernelGGL(row_terms_kernel<1>, dim3(scout_term_blocks, n_groups), dim3(kTermsBlock), 0,
+                       main_stream, *problem, d_groups, n_groups, d_terms_block_prefix, d_row_terms,
+                       d_stage_floor);
+    MIST_HIP_CHECK(hipGetLastError());
+    MIST_HIP_CHECK(hipEventRecord(os->rows_ready, main_stream));
+    MIST_HIP_CHECK(hipStreamWaitEvent(os->side, os->rows_ready, 0));
+    RatioList ratios = {};
+    ratios.r[0] = ratio;
+    if (int rc = launch_scout(problem, d_groups, n_groups, d_reduce_block_prefix, n_reduce_blocks,
+                              d_scout_prefix, n_scout_blocks, d_row_terms, d_stage_floor, ratios, 1,
+                              d_partial_cost, d_partial_index, os->side))
+      return rc;
+    MIST_HIP_CHECK(hipEventRecord(os->scout_done, os->side));
+    hipLaunchKernelGGL(row_terms_kernel<2>, dim3(n_terms_blocks), dim3(kTermsBlock), 0, main_stream,
+                       *problem, d_groups, n_groups, d_terms_block_prefix, d_row_terms, d_stage_floor);
+    MIST_HIP_CHECK(hipGetLastError());
+    MIST_HIP_CHECK(hipStreamWaitEvent(main_stream, os->scout_done, 0));
+    hipLaunchKernelGGL(eval_reduce_kernel, dim3(xcd_padded_grid(n_reduce_blocks)), dim3(MIST_LC_TILE),
+                       0, main_stream, *problem, d_groups, n_groups, d_reduce_block_prefix,
+                       n_reduce_blocks, d_scout_prefix, 0, d_row_terms, d_stage_floor, ratios, 0,
+                       d_partial_cost, d_partial_index);
+    MIST_HIP_CHECK(hipGetLastError());
+    return mist_finalize(problem, d_groups, n_groups, d_reduce_block_prefix, d_row_terms,
+                         d_partial_cost, d_partial_index, sample_index, tables, stream);
+  }
   if (compute_terms) {
     if (int rc = mist_row_terms(problem, d_groups, n_groups, d_terms_block_prefix,
                                 n_terms_blocks, d_row_terms, d_stage_floor, stream))

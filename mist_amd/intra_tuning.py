@@ -278,6 +278,10 @@ class IntraStageTuner:
         if terms_prefix[-1] >= 2**31 or reduce_prefix[-1] + scout_prefix[-1] >= 2**31:
             raise ValueError("launch decomposition exceeds 2**31 workgroups")
         problem = make_problem(cfg, L, P + 1, self.sample_size, len(self.tp_sizes) * len(Gs), len(Q))
+        if len(pending):
+            scouted = groups["scout_stride"] > 0
+            gathered = groups["n_par"] * groups["n_oo"] * groups["n_ao"] * groups["scout_stride"]
+            problem["max_scout_rows"] = int(gathered[scouted].max()) if scouted.any() else 0
         # Batches of consecutive groups under the workspace bound: each holds its own copy of the
         # descriptors with row offsets that start at 0 and its own workgroup prefixes.
         batches = []

@@ -31,6 +31,7 @@ extern "C" {
 #define MIST_P_TILE 16      /* pre-saved micro-batch values per thread of the reduce kernel */
 #endif
 #define MIST_MAX_MESH 16    /* device-mesh candidates of the inter-stage DP */
+#define MIST_MAX_SCOUT_PAIRS 8 /* offload pairs whose rows the scout pass of a group gathers */
 #define MIST_MAX_SAMPLE_BATCH 16 /* alpha samples per mist_eval_reduce_samples call */
 
 #define MIST_E_INVALID (-1) /* argument / shape check failed, nothing was launched */
@@ -109,9 +110,9 @@ typedef struct MistGroupDesc {
   int32_t pp_wre, pp_gre;       /* ZeRO flags of the pre/post layer strategy */
   int32_t rows_per_chunk, n_chunks, n_lc_tiles, n_p_tiles; /* decomposition of the reduce kernel */
   int32_t scout_stride;         /* reduce kernel: 0 = no scout pass for this group; m >= 1 = the
-                                 * scout pass reduces the rows of m (weight, gradient) offload
-                                 * pairs: the first one, (0, 0), and m - 1 evenly spread up to
-                                 * the last (n_par * n_oo * n_ao rows each) */
+                                 * scout pass reduces the rows of the m (weight, gradient) offload
+                                 * pairs scout_pair[0 .. m-1] (n_par * n_oo * n_ao rows each) */
+  int16_t scout_pair[MIST_MAX_SCOUT_PAIRS]; /* indices into the pair list, distinct */
   int64_t n_rows;               /* n_par * n_off */
   int64_t row_offset;           /* first row of this group in the row-term workspace */
   double par[MIST_MAX_PAR][MIST_PAR_FIELDS];

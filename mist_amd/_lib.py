@@ -24,6 +24,7 @@ STAGE_ROWS = 64  # replaced by the library's own value in load()
 TERMS_BLOCK = 128  # replaced by the library's own value in load()
 MAX_MESH = 16
 MAX_SAMPLE_BATCH = 16  # MIST_MAX_SAMPLE_BATCH
+MAX_SCOUT_PAIRS = 8  # MIST_MAX_SCOUT_PAIRS
 DP_NO_START = -3
 DP_CKPT_TAIL, DP_CKPT_STAGE, DP_CKPT_ALL = 0, 1, 2
 DP_THRESHOLD, DP_BOTTLENECK = 0, 1
@@ -72,6 +73,7 @@ GROUP_DTYPE = np.dtype(
         ("pp_wre", "<i4"), ("pp_gre", "<i4"),
         ("rows_per_chunk", "<i4"), ("n_chunks", "<i4"), ("n_lc_tiles", "<i4"),
         ("n_p_tiles", "<i4"), ("scout_stride", "<i4"),
+        ("scout_pair", "<i2", (MAX_SCOUT_PAIRS,)),
         ("n_rows", "<i8"), ("row_offset", "<i8"),
         ("par", "<f8", (MAX_PAR, PAR_FIELDS)),
         ("wo", "<f8", (MAX_RATIOS,)), ("go", "<f8", (MAX_RATIOS,)),

@@ -311,10 +311,8 @@ __device__ __forceinline__ int64_t position_of_row(const MistGroupDesc *g, int64
 // pass may be reading them) and is otherwise kMode 0.
 __device__ __forceinline__ int64_t gathered_position(const MistGroupDesc *g, int64_t q);
 __device__ __forceinline__ bool is_scout_pair(const MistGroupDesc *g, int pair) {
-  if (g->scout_stride <= 0) return false;
-  if (g->scout_stride == 1) return pair == 0;
   for (int k = 0; k < g->scout_stride; ++k)
-    if (pair == (int)((int64_t)k * (g->n_pair - 1) / (g->scout_stride - 1))) return true;
+    if (pair == g->scout_pair[k]) return true;
   return false;
 }
 
@@ -777,13 +775,13 @@ struct ReduceRange {
 // workspace order those rows are scattered (one per (parallelism row, activation ratio, optimizer
 // ratio)); the scout pass gathers them, n_par * n_oo * n_ao rows per group,
 // and so seeds every chunk with minima that are final for most cells.
-// With scout_stride = m > 1 the rows of m - 1 more pairs, evenly spread up to the last one, follow.
+// With scout_stride = m > 1 the rows of the pairs scout_pair[1 .. m-1] follow.
 __device__ __forceinline__ int64_t gathered_position(const MistGroupDesc *g, int64_t q) {
   const int n_tail = g->n_oo * g->n_ao;
   const int64_t per_pair = (int64_t)g->n_par * n_tail;
   const int64_t k = q / per_pair, rest = q - k * per_pair;
   const int64_t par = rest / n_tail, tail = rest - par * n_tail;
-  const int64_t pair = g->scout_stride > 1 ? k * (g->n_pair - 1) / (g->scout_stride - 1) : 0;
+  const int64_t pair = g->scout_pair[k];
   const int ao = (int)(tail / g->n_oo), oo = (int)(tail - (int64_t)ao * g->n_oo);
   return par * g->n_off + (int64_t)ao * g->n_oo * g->n_pair + tile_position(g, oo, (int)pair);
 }

@@ -38,6 +38,16 @@ SCOUT_PAIR_SPAN = 200   # ... one more for every so many pairs of the group (GPT
 ROW_TERMS_BUDGET_BYTES = 2 << 30
 
 
+def _scout_pairs(group, count: int) -> List[int]:
+    """The (weight, gradient) offload pairs whose rows the scout pass of a group gathers: the
+    first one, (0, 0), then evenly spread ones up to the last.  Any set of distinct pairs gives
+    the same tables (scout rows only seed the search); the choice is about speed."""
+    n_pair = int(group["n_pair"])
+    if count <= 1:
+        return [0] * count
+    return sorted({k * (n_pair - 1) // (count - 1) for k in range(count)})
+
+
 def alpha_ratios(sample_size: int) -> np.ndarray:
     """``alpha_k / (1 - alpha_k)`` for ``alpha = linspace(0, 1, S + 2)[1:-1]``
     (mist/utils/pareto.py:53-55,138)."""
@@ -265,8 +275,13 @@ class IntraStageTuner:
             n_stages = -(-groups["n_rows"] // _lib.STAGE_ROWS)
             scout = (n_stages >= SCOUT_MIN_STAGES) & (groups["n_pair"] >= SCOUT_MIN_PAIRS) & (SCOUT_MIN_STAGES > 0)
             scout &= not self.exhaustive
-            pairs = np.minimum(SCOUT_PAIRS + groups["n_pair"] // SCOUT_PAIR_SPAN, groups["n_pair"])
+            pairs = np.minimum(np.minimum(SCOUT_PAIRS + groups["n_pair"] // SCOUT_PAIR_SPAN, groups["n_pair"]),
+                               _lib.MAX_SCOUT_PAIRS)
             groups["scout_stride"] = np.where(scout, pairs, 0)
+            for i in range(len(groups)):
+                picked = _scout_pairs(groups[i], int(groups["scout_stride"][i]))
+                groups["scout_stride"][i] = len(picked)
+                groups["scout_pair"][i, :len(picked)] = picked
             scout_blocks = np.full(len(pending), n_lc_tiles * _lib.SCOUT_SPLIT, dtype=np.int64) * n_p_tiles
             if not np.any(groups["scout_stride"] > 0):
                 scout_blocks[:] = 0

@@ -33,6 +33,7 @@ namespace {
 constexpr int kFirstChunk = 48;   // thresholds per G in the first speculative batch
 constexpr int kMaxChunk = 4096;   // most thresholds per G in one batch
 constexpr double kGap = 1e-6;     // inter_tuning.py:177
+constexpr int kSelectHead = 1 << 16;  // selected candidates that travel with the counts of a fetch
 const double kInf = std::numeric_limits<double>::infinity();
 
 // ---- buffers that live as long as the process: device and pinned host memory per device ----
@@ -200,7 +201,7 @@ struct Search {
     MIST_HIP_CHECK(hipMemcpyAsync(ws->d_req.ptr, h_req, sizeof(float) * 3 * n,
                                   hipMemcpyHostToDevice, stream));
     float *d_req = ws->d_req.as<float>();
-    int total = 0;
+    int total = 0, head = 0;
     for (;;) {
       const int capacity = ws->select_capacity;
       if (int rc = ws->d_values.reserve(sizeof(float) * capacity)) return rc;
@@ -213,6 +214,15 @@ struct Search {
         return rc;
       MIST_HIP_CHECK(hipMemcpyAsync(ws->h_counts.ptr, ws->d_counts.ptr, sizeof(int32_t) * (1 + n),
                                     hipMemcpyDeviceToHost, stream));
+      // the first kSelectHead values and requests travel with the counts: when they are all
+      // there is (the usual case) the fetch is one round trip
+      head = std::min(capacity, kSelectHead);
+      if (int rc = ws->h_values.reserve(sizeof(float) * head)) return rc;
+      if (int rc = ws->h_request.reserve(sizeof(int32_t) * head)) return rc;
+      MIST_HIP_CHECK(hipMemcpyAsync(ws->h_values.ptr, ws->d_values.ptr, sizeof(float) * head,
+                                    hipMemcpyDeviceToHost, stream));
+      MIST_HIP_CHECK(hipMemcpyAsync(ws->h_request.ptr, ws->d_request.ptr, sizeof(int32_t) * head,
+                                    hipMemcpyDeviceToHost, stream));
       MIST_HIP_CHECK(hipStreamSynchronize(stream));
       total = ws->h_counts.as<int32_t>()[0];
       if (total <= capacity) break;
@@ -222,13 +232,15 @@ struct Search {
     const int32_t *h_counts = ws->h_counts.as<int32_t>();
     for (int r = 0; r < n; ++r) (*out)[r].above = h_counts[1 + r];
     if (total == 0) return 0;
-    if (int rc = ws->h_values.reserve(sizeof(float) * total)) return rc;
-    if (int rc = ws->h_request.reserve(sizeof(int32_t) * total)) return rc;
-    MIST_HIP_CHECK(hipMemcpyAsync(ws->h_values.ptr, ws->d_values.ptr, sizeof(float) * total,
-                                  hipMemcpyDeviceToHost, stream));
-    MIST_HIP_CHECK(hipMemcpyAsync(ws->h_request.ptr, ws->d_request.ptr, sizeof(int32_t) * total,
-                                  hipMemcpyDeviceToHost, stream));
-    MIST_HIP_CHECK(hipStreamSynchronize(stream));
+    if (total > head) {
+      if (int rc = ws->h_values.reserve(sizeof(float) * total)) return rc;
+      if (int rc = ws->h_request.reserve(sizeof(int32_t) * total)) return rc;
+      MIST_HIP_CHECK(hipMemcpyAsync(ws->h_values.ptr, ws->d_values.ptr, sizeof(float) * total,
+                                    hipMemcpyDeviceToHost, stream));
+      MIST_HIP_CHECK(hipMemcpyAsync(ws->h_request.ptr, ws->d_request.ptr, sizeof(int32_t) * total,
+                                    hipMemcpyDeviceToHost, stream));
+      MIST_HIP_CHECK(hipStreamSynchronize(stream));
+    }
     const float *values = ws->h_values.as<float>();
     const int32_t *request = ws->h_request.as<int32_t>();
     std::vector<int> count(n, 0);

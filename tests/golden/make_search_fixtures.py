@@ -306,6 +306,14 @@ def main():
     jobs = jobs[shard::n_shards]
     groups = {}
     t0 = time.time()
+    import threading
+
+    def heartbeat():  # long groups finish minutes apart: show that the run is alive
+        while True:
+            time.sleep(60)
+            print(f"[{time.time() - t0:7.0f}s] ... {len(groups)}/{len(jobs)} groups done", flush=True)
+
+    threading.Thread(target=heartbeat, daemon=True).start()
     with get_context("fork").Pool(a.workers, maxtasksperchild=1) as pool:
         for n, (key, rec) in enumerate(pool.imap_unordered(run_group, [j[1] for j in jobs])):
             groups[key] = rec

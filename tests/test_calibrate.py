@@ -117,7 +117,17 @@ def test_measure_and_fit_on_the_gpu():
     print(out)
     for name in ("cpu_gpu_comm_params", "gpu_cpu_comm_params"):
         k, b = out[name]
-        assert 5.0 < k < 200.0 and 0.0 <= b < 1e-3, (name, k, b)
+        assert 15.0 < k < 130.0 and 0.0 <= b < 1e-3, (name, k, b)  # PCIe 4 / 5 x16 class links
     params = np.array(out["interference_model_params"])
     assert np.all(params >= 1.0) and np.all(params <= calibrate.UP_BOUND)
-    assert out["overlapped_cases"] > 30 and out["mean_error"] < 0.25
+    # the fitted model reproduces the overlapped measurements (0.2 % on the box this was
+    # written on; the bound leaves room for a noisier host)
+    assert out["overlapped_cases"] > 30 and out["mean_error"] < 0.08
+    # and the copy models the copy-only cases they were fitted on
+    data = calibrate.preprocess_data(cases)
+    latency, n, _, G2G, C2G, G2C = data[:6]  # GB columns
+    for col, other, name in ((C2G, G2C, "cpu_gpu_comm_params"), (G2C, C2G, "gpu_cpu_comm_params")):
+        only = (col > 0) & (other == 0) & (n == 0) & (G2G == 0)
+        assert only.sum() >= 3
+        model = calibrate.cpu_gpu_latency(col[only], out[name])
+        assert np.max(np.abs(model - latency[only]) / latency[only]) < 0.15, name

@@ -1358,6 +1358,14 @@ __global__ __launch_bounds__(MIST_LC_TILE, MIST_REDUCE_MIN_WAVES) void eval_redu
 #undef MIST_REDUCE
 }
 
+// Rows offered in ascending order: the first of equal costs stays (pareto.py:134-142 as written).
+__device__ __forceinline__ void take_first(double &best, int32_t &best_row, bool feasible,
+                                           double cost, int32_t row) {
+  const bool better = feasible && cost < best;
+  best = better ? cost : best;
+  best_row = better ? row : best_row;
+}
+
 // ------------------------------------------------------------------------------------------
 // Kernel 2x: the same reduction with every cell evaluated.  No scout pass, no sieves, no bounds,
 // no bisection: each (row, l, c) goes through the latency model and the memory model, and each
@@ -1399,20 +1407,23 @@ __device__ __forceinline__ void exhaustive_block(
   for (int64_t base = row_begin; base < row_end; base += kStageRows) {
     const int n_stage = (int)min((int64_t)kStageRows, row_end - base);
     __syncthreads();
-    const double2 *__restrict__ src2 = reinterpret_cast<const double2 *>(src + base * MIST_ROW_TERMS);
+    // Rows are visited in the REFERENCE's order (the chunk is a range of row numbers, gathered
+    // from wherever the workspace order put them; lane = row for the index arithmetic), so that
+    // within a chunk a strict "<" keeps the first of equal costs like the reference's scan does.
+    lds_row[threadIdx.x] = (int32_t)position_of_row(g, min(base + threadIdx.x, row_end - 1));
+    __syncthreads();
+    const double2 *__restrict__ src2 = reinterpret_cast<const double2 *>(src);
     for (int i = threadIdx.x; i < n_stage * (MIST_ROW_TERMS / 2); i += MIST_LC_TILE) {
-      const double2 v = src2[i];
-      const int at = (i / (MIST_ROW_TERMS / 2)) * kLdsRowStride + 2 * (i % (MIST_ROW_TERMS / 2));
-      lds_terms[at] = v.x;
-      lds_terms[at + 1] = v.y;
+      const int r = i / (MIST_ROW_TERMS / 2), c2 = i % (MIST_ROW_TERMS / 2);
+      const double2 v = src2[(int64_t)lds_row[r] * (MIST_ROW_TERMS / 2) + c2];
+      lds_terms[r * kLdsRowStride + 2 * c2] = v.x;
+      lds_terms[r * kLdsRowStride + 2 * c2 + 1] = v.y;
     }
-    // the reference's number of each staged row (lane = row: the index arithmetic once per row)
-    lds_row[threadIdx.x] = row_of_position(g, min(base + threadIdx.x, row_end - 1));
     __syncthreads();
     if (!active) continue;
     for (int r = 0; r < n_stage; ++r) {
       const double *t = lds_terms + r * kLdsRowStride;
-      const int32_t row = lds_row[r];
+      const int32_t row = (int32_t)(base + r);
       const CellLatency lat = cell_latency<kFirstTile>(t, l, c, k);
       const LaneMemory mem = cell_memory(t, l, c);
       // objectives r * x + y (pareto.py:138): base with y = float32 delta / G in float32
@@ -1422,8 +1433,8 @@ __device__ __forceinline__ void exhaustive_block(
 #pragma unroll
       for (int j = 0; j < MIST_P_TILE; ++j) {
         const bool live = j < n_tile;
-        take_min(best_b[j], row_b[j], live && mem.feasible_base(p0 + j, cap), cost_base, row);
-        take_min(best_p[j], row_p[j], live && mem.feasible_pre(p0 + j, cap, pre_saved, pre_sas),
+        take_first(best_b[j], row_b[j], live && mem.feasible_base(p0 + j, cap), cost_base, row);
+        take_first(best_p[j], row_p[j], live && mem.feasible_pre(p0 + j, cap, pre_saved, pre_sas),
                  cost_pre, row);
       }
       if (kFirstTile) {  // last stage / single stage, p == 0 only (:2946-3106)
@@ -1438,8 +1449,8 @@ __device__ __forceinline__ void exhaustive_block(
         const double pf_pp = pf_post + g->pre_states + g->pre_saved;
         const double pb_pp = pb_post + g->pre_states + g->pre_saved;
         const bool ok_pp = fmax(pf_pp, pb_pp) * t[MIST_T_MF] <= cap;
-        take_min(best_post, row_post, ok_post, ratio * lat.spost + lat.dpost / G64, row);
-        take_min(best_pp, row_pp, ok_pp, ratio * lat.spp + lat.dpp / G64, row);
+        take_first(best_post, row_post, ok_post, ratio * lat.spost + lat.dpost / G64, row);
+        take_first(best_pp, row_pp, ok_pp, ratio * lat.spp + lat.dpp / G64, row);
       }
     }
   }
@@ -1901,6 +1912,10 @@ int mist_intra_stage_eval(const MistProblem *problem, const MistGroupDesc *d_gro
     if (!(ratio >= 0.0)) return fail(MIST_E_INVALID, "ratio must be non-negative");
     OverlapStreams *os = nullptr;
     if (int rc = overlap_streams(&os)) return rc;
+    // the second stream and its events are shared by all callers: one call's records and waits
+    // are enqueued as a unit
+    static std::mutex enqueue_lock;
+    std::lock_guard<std::mutex> enqueue_guard(enqueue_lock);
     hipStream_t main_stream = (hipStream_t)stream;
     const unsigned scout_term_blocks = (unsigned)((problem->max_scout_rows + kTermsBlock - 1) / kTermsBlock);
     hipLaunchKernelGGL(row_terms_kernel<1>, dim3(scout_term_blocks, n_groups), dim3(kTermsBlock), 0,

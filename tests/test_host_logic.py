@@ -254,6 +254,18 @@ def test_argument_checks_reject_before_any_launch():
     assert lib.mist_eval_reduce(pp, fake, 1, fake, 1, None, 0, fake, fake, -1.0, fake, fake, None) == -1
     assert lib.mist_eval_reduce(pp, fake, 1, fake, 1, None, 3, fake, fake, 1.0, fake, fake, None) == -1
     assert b"scout" in lib.mist_last_error()
+    # the evaluate-every-cell launch and the multi-sample call check the same things
+    assert lib.mist_eval_reduce_exhaustive(pp, fake, 1, fake, 0, fake, 1.0, fake, fake, None) == -1
+    assert lib.mist_eval_reduce_exhaustive(pp, fake, 1, fake, 1, fake, -1.0, fake, fake, None) == -1
+    assert lib.mist_eval_reduce_exhaustive(pp, fake, 1, fake, 1, None, 1.0, fake, fake, None) == -1
+    ratios = np.array([0.5, 1.0, -2.0])
+    slots = np.arange(3, dtype=np.int32)
+    rp, sp_ = ctypes.c_void_p(ratios.ctypes.data), ctypes.c_void_p(slots.ctypes.data)
+    some_tables = _lib.OutTables()
+    samples = lambda n, r=rp: lib.mist_eval_reduce_samples(
+        pp, fake, 1, fake, 1, None, 0, fake, fake, r, sp_, n, fake, fake, ctypes.byref(some_tables), None)
+    assert samples(0) == -1 and samples(_lib.MAX_SAMPLE_BATCH + 1) == -1 and samples(2, None) == -1
+    assert samples(3) == -1 and b"ratio 2" in lib.mist_last_error()
     tabs = _lib.OutTables()
     assert lib.mist_finalize(pp, fake, 1, fake, fake, fake, fake, 0, ctypes.byref(tabs), None) == -1
     shape = np.zeros(1, dtype=_lib.DP_SHAPE_DTYPE)
@@ -305,6 +317,21 @@ def test_argument_checks_reject_before_any_launch():
     assert lib.mist_dp_stage_minima(sp, ctypes.byref(costs), 1, None, None) == -1
     assert lib.mist_dp_stage_minima(sp, ctypes.byref(costs), 0, fake, None) == -1
     assert lib.mist_dp_stage_minima(sp, ctypes.byref(_lib.DpCosts()), 1, fake, None) == -1
+    # batched stage sampling: the problem list must be consistent before anything is launched
+    items = (_lib.MipBatchItem * 2)()
+    for it in items:
+        it.shape = _lib.MipShape(num_layers=8, p_dim=4, sample_size=4, num_stages=2, layers_min=3,
+                                 layers_max=5, ckpt_mode=_lib.MIP_CKPT_TUNED, fixed_ckpt=0)
+        for v in range(4):
+            it.tables.stable[v] = it.tables.delta[v] = 4096
+    items[1].first_block, items[1].out_offset = 6, 24
+    batch = lambda n: lib.mist_mip_stage_samples_batch(ctypes.byref(items), fake, n, fake, fake, fake, fake, fake, None)
+    items[1].out_offset = 23
+    assert batch(2) == -1 and b"continue the list" in lib.mist_last_error()
+    items[1].out_offset = 24
+    items[1].tables.delta[2] = None
+    assert batch(2) == -1 and b"null table" in lib.mist_last_error()
+    assert batch(0) == -1
 
 
 def test_window_begin_matches_numpy_formulation():

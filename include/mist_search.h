@@ -26,6 +26,8 @@ extern "C" {
 #define MIST_MAX_PAIRS (MIST_MAX_RATIOS * MIST_MAX_RATIOS)
 #define MIST_PAR_FIELDS 20
 #define MIST_ROW_TERMS 34   /* doubles per candidate row produced by mist_row_terms */
+#define MIST_KEY_TERMS 28   /* doubles per (parallelism row, activation ratio, offload pair) of the
+                             * key-term workspace of mist_row_terms */
 #define MIST_LC_TILE 64     /* (layers, ckpt) pairs per workgroup (one wavefront) of the reduce kernel */
 #ifndef MIST_P_TILE
 #define MIST_P_TILE 16      /* pre-saved micro-batch values per thread of the reduce kernel */
@@ -91,7 +93,8 @@ typedef struct MistProblem {
   int32_t max_scout_rows;  /* largest n_par * n_oo * n_ao * scout_stride of the call's groups with a
                             * scout pass; 0 = unknown (mist_intra_stage_eval then runs the row
                             * terms and the scout pass one after the other) */
-  int32_t reserved;
+  int32_t max_group_keys;  /* largest n_par * n_ao * n_pair of the call's groups; 0 = unknown
+                            * (mist_row_terms then evaluates every row on its own) */
 } MistProblem;
 
 /* One (gradient-accumulation steps, device mesh) group = one call of the reference's
@@ -115,6 +118,8 @@ typedef struct MistGroupDesc {
   int16_t scout_pair[MIST_MAX_SCOUT_PAIRS]; /* indices into the pair list, distinct */
   int64_t n_rows;               /* n_par * n_off */
   int64_t row_offset;           /* first row of this group in the row-term workspace */
+  int64_t key_offset;           /* first key of this group in the key-term workspace: keys are
+                                 * (par * n_ao + ao) * n_pair + pair, n_par * n_ao * n_pair per group */
   double par[MIST_MAX_PAR][MIST_PAR_FIELDS];
   double wo[MIST_MAX_RATIOS], go[MIST_MAX_RATIOS], oo[MIST_MAX_RATIOS], ao[MIST_MAX_RATIOS];
   uint8_t pair_wo[MIST_MAX_PAIRS], pair_go[MIST_MAX_PAIRS];
@@ -151,6 +156,8 @@ int mist_terms_block_rows(void); /* candidate rows per workgroup of mist_row_ter
 int mist_reduce_stage_rows(void); /* rows per LDS stage; rows_per_chunk must be a multiple */
 /* doubles of the stage-summary workspace for `total_rows` workspace rows in `n_groups` groups */
 int64_t mist_stage_floor_doubles(int64_t total_rows, int n_groups);
+/* doubles of the key-term workspace for `total_keys` keys (sum of n_par * n_ao * n_pair) */
+int64_t mist_key_terms_doubles(int64_t total_keys);
 
 /* Row-invariant terms of every candidate row: decodes the row index, evaluates the alpha-beta
  * communication terms, the 36 interference evaluations and the memory pieces that do not
@@ -169,12 +176,17 @@ int64_t mist_stage_floor_doubles(int64_t total_rows, int n_groups);
  * d_stage_floor: mist_stage_floor_doubles() float64, written here and read by mist_eval_reduce:
  * per stage of mist_reduce_stage_rows() workspace rows the term-wise minimum of the latency and
  * memory terms (the pseudo row that bounds every row of the stage from below).
+ * d_key_terms: mist_key_terms_doubles() float64 or NULL.  28 of a row's 36 interference
+ * evaluations do not depend on its optimizer-offload ratio; with this workspace (and
+ * MistProblem.max_group_keys, MistGroupDesc.key_offset set) a first kernel evaluates them once
+ * per (parallelism row, activation ratio, offload pair) and the rows read them; without it every
+ * row evaluates all 36.  Same operations on the same operands either way: identical row terms.
  * Fails with MIST_E_INVALID when an interference factor of `problem` is not positive and finite
  * (the kernel peels two overlapping resources with one division and takes 0 / f == +0 for the
  * other one). */
 int mist_row_terms(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,
                    const int32_t *d_block_prefix, int n_blocks, double *d_row_terms,
-                   double *d_stage_floor, void *stream);
+                   double *d_stage_floor, double *d_key_terms, void *stream);
 
 /* Per (group, row chunk, (l, c) tile, p tile): evaluates latency and memory per cell, applies
  * the memory mask and keeps the running lexicographic (cost, row) minimum per bucket.
@@ -236,14 +248,14 @@ int mist_finalize(const MistProblem *problem, const MistGroupDesc *d_groups, int
 
 /* mist_row_terms (when `compute_terms` != 0) + mist_eval_reduce + mist_finalize for one ratio:
  * the device side of IntraStageTuner.tune (mist/analyzer/intra_tuning.py:169-282) for one tp
- * candidate and one sample. */
+ * candidate and one sample.  d_key_terms: as for mist_row_terms, may be NULL. */
 int mist_intra_stage_eval(const MistProblem *problem, const MistGroupDesc *d_groups,
                           int n_groups, const int32_t *d_terms_block_prefix, int n_terms_blocks,
                           const int32_t *d_reduce_block_prefix, int n_reduce_blocks,
                           const int32_t *d_scout_prefix, int n_scout_blocks, double *d_row_terms,
-                          double *d_stage_floor, double *d_partial_cost, int32_t *d_partial_index,
-                          double ratio, int sample_index, int compute_terms,
-                          const MistOutTables *tables, void *stream);
+                          double *d_stage_floor, double *d_key_terms, double *d_partial_cost,
+                          int32_t *d_partial_index, double ratio, int sample_index,
+                          int compute_terms, const MistOutTables *tables, void *stream);
 
 /* Analysis path: what batched_stage_analyze(get_best_solution=False) reports
  * (mist/analyzer/batched_module_analyzer.py:2788-2803, 2876-2892, 2980-2996, 3063-3079) for given

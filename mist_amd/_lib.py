@@ -25,6 +25,7 @@ TERMS_BLOCK = 128  # replaced by the library's own value in load()
 MAX_MESH = 16
 MAX_SAMPLE_BATCH = 16  # MIST_MAX_SAMPLE_BATCH
 MAX_SCOUT_PAIRS = 8  # MIST_MAX_SCOUT_PAIRS
+KEY_TERMS = 28  # MIST_KEY_TERMS
 DP_NO_START = -3
 DP_CKPT_TAIL, DP_CKPT_STAGE, DP_CKPT_ALL = 0, 1, 2
 DP_THRESHOLD, DP_BOTTLENECK = 0, 1
@@ -59,7 +60,7 @@ PROBLEM_DTYPE = np.dtype(
         ("num_mesh", "<i4"),
         ("adv_first_block", "<i4"),
         ("max_scout_rows", "<i4"),
-        ("reserved", "<i4"),
+        ("max_group_keys", "<i4"),
     ],
     align=True,
 )
@@ -74,7 +75,7 @@ GROUP_DTYPE = np.dtype(
         ("rows_per_chunk", "<i4"), ("n_chunks", "<i4"), ("n_lc_tiles", "<i4"),
         ("n_p_tiles", "<i4"), ("scout_stride", "<i4"),
         ("scout_pair", "<i2", (MAX_SCOUT_PAIRS,)),
-        ("n_rows", "<i8"), ("row_offset", "<i8"),
+        ("n_rows", "<i8"), ("row_offset", "<i8"), ("key_offset", "<i8"),
         ("par", "<f8", (MAX_PAR, PAR_FIELDS)),
         ("wo", "<f8", (MAX_RATIOS,)), ("go", "<f8", (MAX_RATIOS,)),
         ("oo", "<f8", (MAX_RATIOS,)), ("ao", "<f8", (MAX_RATIOS,)),
@@ -117,7 +118,8 @@ _SIGNATURES = {
     "mist_terms_block_rows": (ctypes.c_int, []),
     "mist_reduce_scout_split": (ctypes.c_int, []),
     "mist_stage_floor_doubles": (ctypes.c_int64, [ctypes.c_int64, ctypes.c_int]),
-    "mist_row_terms": (ctypes.c_int, [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, _VP, _VP]),
+    "mist_key_terms_doubles": (ctypes.c_int64, [ctypes.c_int64]),
+    "mist_row_terms": (ctypes.c_int, [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, _VP, _VP, _VP]),
     "mist_eval_reduce": (
         ctypes.c_int,
         [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, _VP, ctypes.c_double,
@@ -141,7 +143,7 @@ _SIGNATURES = {
     "mist_intra_stage_eval": (
         ctypes.c_int,
         [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, ctypes.c_int,
-         _VP, _VP, _VP, _VP, ctypes.c_double, ctypes.c_int, ctypes.c_int, ctypes.POINTER(OutTables), _VP],
+         _VP, _VP, _VP, _VP, _VP, ctypes.c_double, ctypes.c_int, ctypes.c_int, ctypes.POINTER(OutTables), _VP],
     ),
 }
 

@@ -91,7 +91,7 @@ def analyze_cells(config: MistConfig, tables: LayerTables, stages, device: str =
         stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
         prob_ptr = ctypes.c_void_p(problem.ctypes.data)
         _lib.check(lib.mist_row_terms(prob_ptr, d_groups.data_ptr(), n_groups, d_prefix.data_ptr(),
-                                      n_groups, row_terms.data_ptr(), stage_floor.data_ptr(), stream),
+                                      n_groups, row_terms.data_ptr(), stage_floor.data_ptr(), None, stream),
                    "mist_row_terms")
         _lib.check(lib.mist_stage_analyze(prob_ptr, d_groups.data_ptr(), n_groups, row_terms.data_ptr(),
                                           d_req.data_ptr(), len(requests), result.data_ptr(), stream),

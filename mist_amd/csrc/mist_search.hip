@@ -16,6 +16,8 @@
 
 #include "mist_common.h"
 #include "mist_search.h"
+#define MIST_ARITH_FN __device__ __forceinline__
+#include "exact_arith.h"
 
 namespace {
 thread_local char g_last_error[512] = "";
@@ -73,6 +75,8 @@ __device__ __forceinline__ double host_link_latency(const double *kb, double mby
 
 // numpy's float64 floor_divide (npy_divmod), for a >= 0 and b > 0 as well as the general case.
 __device__ __forceinline__ double np_floor_divide(double a, double b) {
+  if (__builtin_expect(mist_arith::floor_divide_is_tame(a, b), 1))
+    return mist_arith::floor_divide_tame(a, b);
   if (b == 0.0) return a / b;
   double mod = fmod(a, b);
   double div = (a - mod) / b;
@@ -93,20 +97,44 @@ __device__ __forceinline__ double np_floor_divide(double a, double b) {
 // Four-resource interference model (mist/tools/optimize.py:1012-1122).  X = [C, G2G, C2G, G2C].
 // Masks in evaluation order: 4-way, four 3-way, six 2-way; bit j set = resource j in the mask.
 // ------------------------------------------------------------------------------------------
-__constant__ unsigned char kMaskBits[11] = {
+constexpr unsigned char kMaskBits[11] = {
     0xF,
     0x7, 0xB, 0xD, 0xE,
     0x3, 0x5, 0x9, 0x6, 0xA, 0xC,
 };
 
-// Index into kMaskBits of the mask equal to a non-zero pattern, -1 for patterns with fewer than
-// two bits.
-__constant__ signed char kMaskOfPattern[16] = {
-    -1, -1, -1, 5, -1, 6, 8, 1, -1, 7, 9, 2, 10, 3, 4, 0,
-};
+// Index into kMaskBits of the mask equal to a pattern of two or more bits, as 16 nibbles of one
+// constant (a table in memory would cost every peel a dependent load).
+constexpr uint64_t pack_mask_of_pattern() {
+  uint64_t packed = 0;
+  for (int m = 0; m < 11; ++m) packed |= (uint64_t)m << (4 * kMaskBits[m]);
+  return packed;
+}
+constexpr uint64_t kMaskOfPatternPacked = pack_mask_of_pattern();
+__device__ __forceinline__ int mask_of_pattern(unsigned pattern) {
+  return (int)((kMaskOfPatternPacked >> (4 * pattern)) & 0xF);
+}
+static_assert(((kMaskOfPatternPacked >> (4 * 0xF)) & 0xF) == 0 && ((kMaskOfPatternPacked >> (4 * 0x3)) & 0xF) == 5 &&
+                  ((kMaskOfPatternPacked >> (4 * 0xC)) & 0xF) == 10 && ((kMaskOfPatternPacked >> (4 * 0xE)) & 0xF) == 4,
+              "pattern -> mask index");
 
-struct Interference {
-  const double (*factor)[4];
+// The factor table lives in LDS and is read through a pointer of that address space: the model
+// is out of line, and through a generic pointer every read would be a flat load.
+typedef const __attribute__((address_space(3))) double LdsDouble;
+constexpr int kFactorPitch = 8;  // per mask: the four factors, then their four reciprocals
+
+// kInline: the model is expanded at every call site (for a kernel with few of them: its loads
+// stay in flight across the evaluations, which a call would make it wait for) instead of called.
+template <bool kInline>
+struct InterferenceModel {
+  LdsDouble *table;   // [11][kFactorPitch]: factor[m][0..3], 1 / factor[m][0..3] correctly rounded
+  bool factors_tame;  // every factor lies in the divisor range of the reciprocal quotient
+
+  // Operands (seconds) below this bound keep every scaled time and every quotient of a peel
+  // inside the range where the reciprocal quotient is the IEEE quotient; a peel only divides
+  // differences of scaled times of resources busier than 1e-8 s, which are zero or no smaller
+  // than an ulp of 1e-8.
+  static constexpr double kOperandBound = 0x1p500;
 
   // Arguments in the order of the reference's get_layer_critical_latency
   // (batched_module_analyzer.py:1413-1422): exec, gpu<->gpu, gpu->cpu, cpu->gpu.
@@ -114,8 +142,22 @@ struct Interference {
   // site; the others are literal zeros there, never part of a mask, and their share of a round
   // (a multiplication and a division each) is left out at compile time.  The sums keep all four
   // operands, so the value is the one of the general form.
-  template <unsigned kLive>
-  __device__ __noinline__ double eval(double exec, double g2g, double g2c, double c2g) const {
+  // kByReciprocal: the quotients (s - overlap) / factor are taken with the stored reciprocals
+  // (five multiply-adds, no branch, so that the four quotients of a peel interleave) instead of
+  // the division sequence; eval() picks it when every operand of the wave is in range.
+  template <unsigned kLive, bool kByReciprocal>
+  __device__ __noinline__ double eval_called(double exec, double g2g, double g2c, double c2g) const {
+    return eval_body<kLive, kByReciprocal>(exec, g2g, g2c, c2g);
+  }
+  template <unsigned kLive, bool kByReciprocal>
+  __device__ __forceinline__ double eval_as(double exec, double g2g, double g2c, double c2g) const {
+    if constexpr (kInline || __builtin_popcount(kLive) < 2)
+      return eval_body<kLive, kByReciprocal>(exec, g2g, g2c, c2g);
+    else
+      return eval_called<kLive, kByReciprocal>(exec, g2g, g2c, c2g);
+  }
+  template <unsigned kLive, bool kByReciprocal>
+  __device__ __forceinline__ double eval_body(double exec, double g2g, double g2c, double c2g) const {
     double x0 = (kLive & 1u) ? exec : 0.0, x1 = (kLive & 2u) ? g2g : 0.0;
     double x2 = (kLive & 4u) ? c2g : 0.0, x3 = (kLive & 8u) ? g2c : 0.0;
     double out = 0.0;
@@ -131,29 +173,35 @@ struct Interference {
              (((kLive & 4u) && !(fabs(x2) <= 1e-8)) ? 4u : 0u) |
              (((kLive & 8u) && !(fabs(x3) <= 1e-8)) ? 8u : 0u);
     };
+    // a / f for a = s - overlap >= +0 (never -0: a difference of equal numbers is +0).
+    auto quotient = [&](double a, double f, double y) {
+      if (!kByReciprocal) return a / f;
+      return mist_arith::quotient_by_reciprocal<false>(a, f, y, a * y);
+    };
     // One peel as the reference writes it: every busy resource gives up the smallest scaled
-    // time.
+    // time.  (s - ov) / f * 1.0 there: the product with 1.0 changes nothing.
     auto peel = [&](unsigned mask) {
-      const int m = kMaskOfPattern[mask];
-      const double f0 = factor[m][0], f1 = factor[m][1], f2 = factor[m][2], f3 = factor[m][3];
+      LdsDouble *row = table + mask_of_pattern(mask) * kFactorPitch;
+      const double f0 = row[0], f1 = row[1], f2 = row[2], f3 = row[3];
+      const double y0 = row[4], y1 = row[5], y2 = row[6], y3 = row[7];
       const double s0 = x0 * f0, s1 = x1 * f1, s2 = x2 * f2, s3 = x3 * f3;
       double ov = INFINITY;
       if ((kLive & 1u) && (mask & 1u)) ov = fmin(ov, s0);
       if ((kLive & 2u) && (mask & 2u)) ov = fmin(ov, s1);
       if ((kLive & 4u) && (mask & 4u)) ov = fmin(ov, s2);
       if ((kLive & 8u) && (mask & 8u)) ov = fmin(ov, s3);
-      if ((kLive & 1u) && (mask & 1u)) x0 = (s0 - ov) / f0 * 1.0;
-      if ((kLive & 2u) && (mask & 2u)) x1 = (s1 - ov) / f1 * 1.0;
-      if ((kLive & 4u) && (mask & 4u)) x2 = (s2 - ov) / f2 * 1.0;
-      if ((kLive & 8u) && (mask & 8u)) x3 = (s3 - ov) / f3 * 1.0;
+      if ((kLive & 1u) && (mask & 1u)) x0 = quotient(s0 - ov, f0, y0);
+      if ((kLive & 2u) && (mask & 2u)) x1 = quotient(s1 - ov, f1, y1);
+      if ((kLive & 4u) && (mask & 4u)) x2 = quotient(s2 - ov, f2, y2);
+      if ((kLive & 8u) && (mask & 8u)) x3 = quotient(s3 - ov, f3, y3);
       out = out + ov;
     };
     // The same peel for two busy resources with one division: the one with the smaller scaled
     // time is left with (s - s) / f = +0 (factors are positive and finite), the other with
     // (larger - smaller) / its factor; with equal times both quotients are +0.
     auto peel_pair = [&](unsigned mask) {
-      const int m = kMaskOfPattern[mask];
-      const double f0 = factor[m][0], f1 = factor[m][1], f2 = factor[m][2], f3 = factor[m][3];
+      LdsDouble *row = table + mask_of_pattern(mask) * kFactorPitch;
+      const double f0 = row[0], f1 = row[1], f2 = row[2], f3 = row[3];
       const double s0 = x0 * f0, s1 = x1 * f1, s2 = x2 * f2, s3 = x3 * f3;
       const bool b0 = (kLive & 1u) && (mask & 1u), b1 = (kLive & 2u) && (mask & 2u);
       const bool b2 = (kLive & 4u) && (mask & 4u), b3 = (kLive & 8u) && (mask & 8u);
@@ -162,12 +210,12 @@ struct Interference {
       if (b1) { lo = fmin(lo, s1); hi = fmax(hi, s1); }
       if (b2) { lo = fmin(lo, s2); hi = fmax(hi, s2); }
       if (b3) { lo = fmin(lo, s3); hi = fmax(hi, s3); }
-      double den = 1.0;
-      if (b0 && s0 == hi) den = f0;
-      if (b1 && s1 == hi) den = f1;
-      if (b2 && s2 == hi) den = f2;
-      if (b3 && s3 == hi) den = f3;
-      const double rest = (hi - lo) / den * 1.0;
+      double den = 1.0, rden = 1.0;
+      if (b0 && s0 == hi) { den = f0; rden = row[4]; }
+      if (b1 && s1 == hi) { den = f1; rden = row[5]; }
+      if (b2 && s2 == hi) { den = f2; rden = row[6]; }
+      if (b3 && s3 == hi) { den = f3; rden = row[7]; }
+      const double rest = quotient(hi - lo, den, rden);
       if (b0) x0 = s0 == hi ? rest : 0.0;
       if (b1) x1 = s1 == hi ? rest : 0.0;
       if (b2) x2 = s2 == hi ? rest : 0.0;
@@ -188,6 +236,22 @@ struct Interference {
       if (__popc(nz) == 2) peel_pair(nz);
     }
     return out + (((x0 + x1) + x2) + x3);
+  }
+
+  template <unsigned kLive>
+  __device__ __forceinline__ double eval(double exec, double g2g, double g2c, double c2g) const {
+    if constexpr (__builtin_popcount(kLive) < 2) {
+      return eval_as<kLive, false>(exec, g2g, g2c, c2g);  // nothing to divide
+    } else {
+      // NaN and infinities fail the comparisons and take the division sequence, wave-wide.
+      const bool tame = factors_tame &&
+                        (!(kLive & 1u) || fabs(exec) < kOperandBound) &&
+                        (!(kLive & 2u) || fabs(g2g) < kOperandBound) &&
+                        (!(kLive & 4u) || fabs(c2g) < kOperandBound) &&
+                        (!(kLive & 8u) || fabs(g2c) < kOperandBound);
+      if (__builtin_expect(__all(tame), 1)) return eval_as<kLive, true>(exec, g2g, g2c, c2g);
+      return eval_called<kLive, false>(exec, g2g, g2c, c2g);  // never expanded in place: cold
+    }
   }
 
   __device__ __forceinline__ double operator()(double exec, double g2g, double g2c, double c2g) const {
@@ -305,10 +369,195 @@ __device__ __forceinline__ int64_t position_of_row(const MistGroupDesc *g, int64
 // ------------------------------------------------------------------------------------------
 // Kernel 1: row-invariant terms.  One thread per candidate row (workspace position).
 // ------------------------------------------------------------------------------------------
+// Of a row's 36 evaluations of the interference model only the eight of the forward phase of the
+// first micro-batch see the optimizer ratio (through the optimizer-state swaps); the other 28
+// are the same for the n_oo rows of one "key" = (parallelism, activation ratio, offload pair).
+// key_terms_kernel evaluates those once per key into MIST_KEY_TERMS doubles, row_terms_kernel
+// reads them: the same operations on the same operands as when every row evaluates everything
+// (which it does when the caller passes no key-term workspace, and for the rows of the scout
+// pass, which are computed ahead of all others).
+constexpr int kKeyBwd = 0;        // [last?0:1 micro-batch][nock, ck] x (layer, first, last, extra_pre, extra_post)
+constexpr int kKeyFwd = 20;       // forward, not the first micro-batch: [nock, ck] x (layer, last, extra_post)
+constexpr int kKeyFwdFirst = 26;  //   its `first` and `extra_pre`, which do not depend on ckpt
+constexpr int kKeyFwdExtraPre = 27;
+static_assert(MIST_KEY_TERMS == 28 && MIST_KEY_TERMS % 2 == 0, "key terms are read as 16-byte pairs");
+
+// Model tables of a workgroup in LDS (tables indexed at run time: indexing the by-value kernel
+// argument would make every lane keep a private copy of the whole struct in scratch memory).
+// Returns whether every interference factor is in the divisor range of the reciprocal quotient.
+__device__ __forceinline__ bool load_model_tables(const MistProblem &prob,
+                                                  double (*lds_factor)[kFactorPitch],
+                                                  double *lds_gpu_gpu) {
+  bool factors_tame = true;
+  if (threadIdx.x < 44) {
+    const double f = prob.interf_factor[threadIdx.x / 4][threadIdx.x % 4];
+    lds_factor[threadIdx.x / 4][threadIdx.x % 4] = f;
+    lds_factor[threadIdx.x / 4][4 + threadIdx.x % 4] = 1.0 / f;
+    factors_tame = f >= mist_arith::kDivisorMin && f <= mist_arith::kDivisorMax;
+  }
+  if (threadIdx.x >= 64 && threadIdx.x < 96) lds_gpu_gpu[threadIdx.x - 64] = prob.gpu_gpu[threadIdx.x - 64];
+  return __syncthreads_and(factors_tame) != 0;
+}
+
+// Operands of the interference evaluations that do not depend on the optimizer ratio: swap and
+// collective latencies (:1362-1408) of one (parallelism row, offload pair, activation ratio).
+struct KeyInputs {
+  double exec_fwd, exec_bwd_nock, exec_bwd_ck, extra_fwd, extra_bwd, extra_fb;
+  double wre, gre, ore;
+  double so_W, si_W, so_G, si_G, so_A_ck, si_A_ck, so_A_nock, si_A_nock;
+  double AG_w, RS_g, AR_g;
+  double E_f, ag_wre, g2c_B, c2g_B, first_g2c, g2g_B[2];
+};
+
+__device__ __forceinline__ KeyInputs key_inputs(const MistProblem &prob, const double *lds_gpu_gpu,
+                                                const MistGroupDesc *g, const double *par,
+                                                double wo, double go, double ao) {
+  KeyInputs in;
+  const double dp = par[MIST_PAR_DP];
+  in.wre = par[MIST_PAR_WRE];
+  in.gre = par[MIST_PAR_GRE];
+  in.ore = par[MIST_PAR_ORE];
+  const double W = par[MIST_PAR_W], Gr = par[MIST_PAR_G];
+  const double raw_ck = par[MIST_PAR_RAW_CK], raw_nock = par[MIST_PAR_RAW_NOCK];
+  in.exec_fwd = par[MIST_PAR_EXEC_FWD];
+  in.exec_bwd_nock = par[MIST_PAR_EXEC_BWD];
+  in.extra_fwd = par[MIST_PAR_EXTRA_FWD];
+  in.extra_bwd = par[MIST_PAR_EXTRA_BWD];
+  const double wre_size = in.wre == 1.0 ? dp : 1.0;
+  const double gre_size = in.gre == 1.0 ? dp : 1.0;
+  in.so_W = host_link_latency(prob.gpu_cpu, W / wre_size * wo);
+  in.si_W = host_link_latency(prob.cpu_gpu, W / wre_size * wo);
+  in.so_G = host_link_latency(prob.gpu_cpu, Gr / gre_size * go);
+  in.si_G = host_link_latency(prob.cpu_gpu, Gr / gre_size * go);
+  in.so_A_ck = host_link_latency(prob.gpu_cpu, raw_ck * ao);
+  in.si_A_ck = host_link_latency(prob.cpu_gpu, raw_ck * ao);
+  in.so_A_nock = host_link_latency(prob.gpu_cpu, raw_nock * ao);
+  in.si_A_nock = host_link_latency(prob.cpu_gpu, raw_nock * ao);
+  const double n_nodes = (double)g->num_nodes;
+  const double dp_inter = dp > n_nodes ? n_nodes : dp;
+  const double dp_intra = dp > n_nodes ? floor(dp / n_nodes) : 1.0;
+  in.AG_w = gpu_gpu_latency(lds_gpu_gpu, W, dp_inter, dp_intra, 1.0);
+  in.RS_g = gpu_gpu_latency(lds_gpu_gpu, Gr, dp_inter, dp_intra, 1.1);
+  in.AR_g = gpu_gpu_latency(lds_gpu_gpu, Gr, dp_inter, dp_intra, 2.1);
+  const bool adv = prob.adv_first_block != 0;
+  in.E_f = in.exec_fwd - in.extra_fwd;
+  in.ag_wre = in.AG_w * in.wre;
+  in.g2c_B = in.so_G;
+  in.c2g_B = in.si_W + in.si_G;
+  in.first_g2c = adv ? in.g2c_B : 0.0;
+  in.g2g_B[0] = in.ag_wre + in.RS_g * in.ore + in.AR_g * (1.0 - in.ore);
+  in.g2g_B[1] = in.ag_wre + in.RS_g * in.gre;
+  in.extra_fb = in.extra_fwd + in.extra_bwd;
+  in.exec_bwd_ck = in.exec_fwd + in.exec_bwd_nock;
+  return in;
+}
+
+// Forward phases (:1432-1621): phase 0 = first micro-batch (the optimizer-state swaps so_O /
+// si_O run beside it), phase 1 = the others.
+struct FwdOperands {
+  double g2c, c2g, g2g;
+};
+__device__ __forceinline__ FwdOperands fwd_operands(const KeyInputs &in, bool first_micro_batch,
+                                                    double so_O, double si_O) {
+  if (first_micro_batch) return FwdOperands{so_O + in.so_W, si_O + in.si_G, in.AG_w * in.ore};
+  return FwdOperands{0.0, in.si_W, in.AG_w * in.wre};
+}
+// the members of a forward family that do not depend on ckpt ...
+template <class Interference>
+__device__ __forceinline__ void fwd_common(const Interference &I, const KeyInputs &in,
+                                           const FwdOperands &op, bool first_micro_batch, bool adv,
+                                           double &first, double &extra_pre) {
+  const double pre_g2g = (first_micro_batch || adv) ? op.g2g : 0.0;
+  const double pre_c2g = adv ? op.c2g : 0.0;
+  first = I.exec_g2g_c2g(in.E_f, op.g2g, op.c2g) + in.extra_fwd;
+  extra_pre = I.g2g_c2g(pre_g2g, pre_c2g);
+}
+// ... and those that do (with_ckpt: the saved activations of a checkpointed layer are swapped)
+template <class Interference>
+__device__ __forceinline__ void fwd_of_ckpt(const Interference &I, const KeyInputs &in,
+                                            const FwdOperands &op, bool with_ckpt, double &layer,
+                                            double &last, double &extra_post) {
+  const double g2c = op.g2c + (with_ckpt ? in.so_A_ck : in.so_A_nock);
+  layer = I(in.E_f, op.g2g, g2c, op.c2g) + in.extra_fwd;
+  last = I.exec_g2c(in.E_f, g2c) + in.extra_fwd;
+  extra_post = I.g2c_only(g2c);
+}
+
+// Backward phases (:1646-1902): not_last = false for the last micro-batch.
+template <class Interference>
+__device__ __forceinline__ Family bwd_family(const Interference &I, const KeyInputs &in,
+                                             bool not_last, bool with_ckpt) {
+  const bool k = with_ckpt;
+  const double E = k ? in.exec_bwd_ck - in.extra_fb : in.exec_bwd_nock - in.extra_bwd;
+  const double extra = k ? in.extra_fb : in.extra_bwd;
+  const double c2g = in.c2g_B + (k ? in.si_A_ck : in.si_A_nock);
+  const double red_last =
+      k ? (in.ore == 1.0 ? in.RS_g : in.AR_g) : in.RS_g * in.ore + in.AR_g * (1.0 - in.ore);
+  const double red = not_last ? in.RS_g * in.gre : red_last;
+  // With checkpointing the reference adds the (always zero) all-gather of saved tensors.
+  const double g2g_phase = not_last ? in.g2g_B[1] : in.g2g_B[0];
+  const double g2g_layer = k ? g2g_phase + 0.0 : g2g_phase;
+  Family f;
+  f.layer = I(E, g2g_layer, in.g2c_B, c2g) + extra;
+  f.last = I.exec_g2g_c2g(E, in.ag_wre, c2g) + extra;
+  f.first = I.exec_g2g_g2c(E, red, in.first_g2c) + extra;
+  f.extra_pre = I.g2g_c2g(in.ag_wre, c2g);
+  f.extra_post = I.g2g_g2c(red, in.first_g2c);
+  return f;
+}
+
+// Workgroup = (32 keys of one group) x (4 lanes per key); grid.y = group, grid.x covers the
+// group with the most keys.  Lane j of a key evaluates backward family j (= 2 * not_last + ckpt)
+// and the forward family of the later micro-batches with ckpt = j & 1.
+__global__ __launch_bounds__(kTermsBlock) void key_terms_kernel(
+    const MistProblem prob, const MistGroupDesc *__restrict__ groups, double *__restrict__ key_terms) {
+  const MistGroupDesc *g = groups + blockIdx.y;
+  const int n_keys = g->n_par * g->n_ao * g->n_pair;
+  constexpr int kKeysPerBlock = kTermsBlock / 4;
+  if ((int)blockIdx.x * kKeysPerBlock >= n_keys) return;
+  __shared__ __align__(16) double lds_factor[11][kFactorPitch];
+  __shared__ double lds_gpu_gpu[32];
+  InterferenceModel<false> I;
+  I.factors_tame = load_model_tables(prob, lds_factor, lds_gpu_gpu);
+  I.table = (LdsDouble *)&lds_factor[0][0];
+  const int key_here = (int)blockIdx.x * kKeysPerBlock + (int)threadIdx.x / 4;
+  const int key = min(key_here, n_keys - 1);  // lanes past the end redo the last key, unwritten
+  const int j = threadIdx.x & 3;
+  const int pair = key % g->n_pair;
+  const int ao_i = (key / g->n_pair) % g->n_ao;
+  const int par_i = key / (g->n_pair * g->n_ao);
+  const KeyInputs in = key_inputs(prob, lds_gpu_gpu, g, g->par[par_i], g->wo[g->pair_wo[pair]],
+                                  g->go[g->pair_go[pair]], g->ao[ao_i]);
+  const Family back = bwd_family(I, in, (j & 2) != 0, (j & 1) != 0);
+  const FwdOperands op = fwd_operands(in, false, 0.0, 0.0);
+  double first, extra_pre, layer, last, extra_post;
+  fwd_common(I, in, op, false, prob.adv_first_block != 0, first, extra_pre);
+  fwd_of_ckpt(I, in, op, (j & 1) != 0, layer, last, extra_post);
+  if (key_here >= n_keys) return;
+  double *out = key_terms + (g->key_offset + key) * MIST_KEY_TERMS;
+  double *b = out + kKeyBwd + j * 5;
+  b[0] = back.layer;
+  b[1] = back.first;
+  b[2] = back.last;
+  b[3] = back.extra_pre;
+  b[4] = back.extra_post;
+  if (j < 2) {
+    double *f = out + kKeyFwd + j * 3;
+    f[0] = layer;
+    f[1] = last;
+    f[2] = extra_post;
+  }
+  if (j == 0) {
+    out[kKeyFwdFirst] = first;
+    out[kKeyFwdExtraPre] = extra_pre;
+  }
+}
+
 // kMode 0: every row of every group.  kMode 1: only the rows the scout pass gathers (workgroup
 // = (128 gathered rows, group); no stage summaries), so that the scout pass can start while
 // kMode 2 computes everything: that one leaves the stores of the gathered rows out (the scout
-// pass may be reading them) and is otherwise kMode 0.
+// pass may be reading them) and is otherwise kMode 0.  kFromKeys: the key terms are read from
+// `key_terms` (written by key_terms_kernel) instead of evaluated per row.
 __device__ __forceinline__ int64_t gathered_position(const MistGroupDesc *g, int64_t q);
 __device__ __forceinline__ bool is_scout_pair(const MistGroupDesc *g, int pair) {
   for (int k = 0; k < g->scout_stride; ++k)
@@ -316,11 +565,11 @@ __device__ __forceinline__ bool is_scout_pair(const MistGroupDesc *g, int pair) 
   return false;
 }
 
-template <int kMode>
+template <int kMode, bool kFromKeys>
 __global__ __launch_bounds__(kTermsBlock) void row_terms_kernel(
     const MistProblem prob, const MistGroupDesc *__restrict__ groups, int n_groups,
     const int32_t *__restrict__ block_prefix, double *__restrict__ row_terms,
-    double *__restrict__ stage_floor) {
+    double *__restrict__ stage_floor, const double *__restrict__ key_terms) {
   int local_block;
   const MistGroupDesc *g;
   int64_t n_here_total;  // rows this launch computes for the group
@@ -333,18 +582,19 @@ __global__ __launch_bounds__(kTermsBlock) void row_terms_kernel(
     g = find_group(groups, block_prefix, n_groups, blockIdx.x, &local_block);
     n_here_total = g->n_rows;
   }
-  // The block's terms are assembled in LDS (row pitch 35 doubles: conflict-free) and written out
-  // as one contiguous, fully coalesced range; a lane writing its own 272-byte row would touch
-  // 34 partial cache lines.
-  __shared__ double lds_out[kTermsBlock * (MIST_ROW_TERMS + 1)];
-  // Tables indexed at run time are read from LDS: indexing the by-value kernel argument would
-  // make every lane keep a private copy of the whole struct in scratch memory.
-  __shared__ double lds_factor[11][4];
+  // The block's terms are written out as one contiguous, fully coalesced range (a lane writing
+  // its own 272-byte row would touch 34 partial cache lines): wavefront by wavefront through one
+  // LDS buffer of kStageRows rows (row pitch 35 doubles: conflict-free).  One buffer for the
+  // block, not one per wavefront: LDS is what bounds the number of resident wavefronts here, and
+  // the kernel is a chain of dependent loads and evaluations that needs them.
+  __shared__ double lds_out[kStageRows * (MIST_ROW_TERMS + 1)];
+  __shared__ __align__(16) double lds_factor[11][kFactorPitch];
   __shared__ double lds_gpu_gpu[32];
   __shared__ unsigned char lds_skip[kTermsBlock];
-  if (threadIdx.x < 44) lds_factor[threadIdx.x / 4][threadIdx.x % 4] = prob.interf_factor[threadIdx.x / 4][threadIdx.x % 4];
-  if (threadIdx.x >= 64 && threadIdx.x < 96) lds_gpu_gpu[threadIdx.x - 64] = prob.gpu_gpu[threadIdx.x - 64];
-  __syncthreads();
+  __shared__ double lds_part[kTermsBlock / kStageRows - 1][2][kStageFloorPitch];  // stage summaries
+  InterferenceModel<kFromKeys> I;  // with key terms only the first forward phase is evaluated here
+  I.factors_tame = load_model_tables(prob, lds_factor, lds_gpu_gpu);
+  I.table = (LdsDouble *)&lds_factor[0][0];
   const int64_t block_first = (int64_t)local_block * kTermsBlock;
   const int rows_here = (int)min((int64_t)kTermsBlock, n_here_total - block_first);
   // Lanes past the end recompute the last row (no divergent barrier); their result is dropped.
@@ -359,13 +609,26 @@ __global__ __launch_bounds__(kTermsBlock) void row_terms_kernel(
   const double oo = g->oo[oo_i];
   const double ao = g->ao[ao_i];
 
+  // the key terms are fetched first and used last: the loads are in flight across everything
+  // computed here
+  double v[kFromKeys ? MIST_KEY_TERMS : 2];
+  if (kFromKeys) {
+    const int64_t key = (int64_t)(par_i * g->n_ao + ao_i) * g->n_pair + pair;
+    const double2 *__restrict__ kt =
+        reinterpret_cast<const double2 *>(key_terms + (g->key_offset + key) * MIST_KEY_TERMS);
+#pragma unroll
+    for (int i = 0; i < MIST_KEY_TERMS / 2; ++i) {
+      const double2 two = kt[i];
+      v[2 * i] = two.x;
+      v[2 * i + 1] = two.y;
+    }
+  }
+
   const double *par = g->par[par_i];
   const double b = par[MIST_PAR_B], dp = par[MIST_PAR_DP], tp = par[MIST_PAR_TP];
   const double wre = par[MIST_PAR_WRE], gre = par[MIST_PAR_GRE], ore = par[MIST_PAR_ORE];
   const double W = par[MIST_PAR_W], Gr = par[MIST_PAR_G], O = par[MIST_PAR_O];
   const double raw_ck = par[MIST_PAR_RAW_CK], raw_nock = par[MIST_PAR_RAW_NOCK];
-  const double exec_fwd = par[MIST_PAR_EXEC_FWD], exec_bwd_nock = par[MIST_PAR_EXEC_BWD];
-  const double extra_fwd = par[MIST_PAR_EXTRA_FWD], extra_bwd = par[MIST_PAR_EXTRA_BWD];
   const double wre_size = wre == 1.0 ? dp : 1.0;
   const double gre_size = gre == 1.0 ? dp : 1.0;
   const double ore_size = ore == 1.0 ? dp : 1.0;
@@ -396,80 +659,52 @@ __global__ __launch_bounds__(kTermsBlock) void row_terms_kernel(
   const double two_buf = 2.0 * (Wbuf + Gbuf);
 
   // ---- swap and collective latencies (:1362-1408) ----
-  const double so_W = host_link_latency(prob.gpu_cpu, W / wre_size * wo);
-  const double si_W = host_link_latency(prob.cpu_gpu, W / wre_size * wo);
-  const double so_G = host_link_latency(prob.gpu_cpu, Gr / gre_size * go);
-  const double si_G = host_link_latency(prob.cpu_gpu, Gr / gre_size * go);
+  const KeyInputs in = key_inputs(prob, lds_gpu_gpu, g, par, wo, go, ao);
   const double so_O = host_link_latency(prob.gpu_cpu, O / ore_size * oo);
   const double si_O = host_link_latency(prob.cpu_gpu, O / ore_size * oo);
-  const double so_A_ck = host_link_latency(prob.gpu_cpu, raw_ck * ao);
-  const double si_A_ck = host_link_latency(prob.cpu_gpu, raw_ck * ao);
-  const double so_A_nock = host_link_latency(prob.gpu_cpu, raw_nock * ao);
-  const double si_A_nock = host_link_latency(prob.cpu_gpu, raw_nock * ao);
-  const double n_nodes = (double)g->num_nodes;
-  const double dp_inter = dp > n_nodes ? n_nodes : dp;
-  const double dp_intra = dp > n_nodes ? floor(dp / n_nodes) : 1.0;
-  const double AG_w = gpu_gpu_latency(lds_gpu_gpu, W, dp_inter, dp_intra, 1.0);
-  const double RS_g = gpu_gpu_latency(lds_gpu_gpu, Gr, dp_inter, dp_intra, 1.1);
-  const double AR_g = gpu_gpu_latency(lds_gpu_gpu, Gr, dp_inter, dp_intra, 2.1);
-
-  const Interference I{lds_factor};
   const bool adv = prob.adv_first_block != 0;
 
-  // ---- forward phases (:1432-1621): index 0 = first micro-batch, 1 = not first ----
-  const double g2c_F[2] = {so_O + so_W, 0.0};
-  const double c2g_F[2] = {si_O + si_G, si_W};
-  const double g2g_F[2] = {AG_w * ore, AG_w * wre};
-  const double E_f = exec_fwd - extra_fwd;
-  Family fwd[2][2];  // [phase][0 = nock, 1 = ck]
-#pragma unroll
-  for (int ph = 0; ph < 2; ++ph) {
-    const double pre_g2g = (ph == 0 || adv) ? g2g_F[ph] : 0.0;
-    const double pre_c2g = adv ? c2g_F[ph] : 0.0;
-    const double first = I.exec_g2g_c2g(E_f, g2g_F[ph], c2g_F[ph]) + extra_fwd;
-    const double extra_pre = I.g2g_c2g(pre_g2g, pre_c2g);
+  // ---- forward (:1432-1621) and backward (:1646-1902) families ----
+  Family fwd[2][2];  // [0 = first micro-batch, 1 = not first][0 = nock, 1 = ck]
+  Family bwd[2][2];  // [0 = last micro-batch, 1 = not last][0 = nock, 1 = ck]
+  {
+    const FwdOperands op = fwd_operands(in, true, so_O, si_O);
+    double first, extra_pre;
+    fwd_common(I, in, op, true, adv, first, extra_pre);
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
-      const double g2c = g2c_F[ph] + (k ? so_A_ck : so_A_nock);
-      fwd[ph][k].layer = I(E_f, g2g_F[ph], g2c, c2g_F[ph]) + extra_fwd;
-      fwd[ph][k].first = first;
-      fwd[ph][k].last = I.exec_g2c(E_f, g2c) + extra_fwd;
-      fwd[ph][k].extra_pre = extra_pre;
-      fwd[ph][k].extra_post = I.g2c_only(g2c);
+      fwd[0][k].first = first;
+      fwd[0][k].extra_pre = extra_pre;
+      fwd_of_ckpt(I, in, op, k != 0, fwd[0][k].layer, fwd[0][k].last, fwd[0][k].extra_post);
     }
   }
-
-  // ---- backward phases (:1646-1902): index 0 = last micro-batch, 1 = not last ----
-  const double g2c_B = so_G;
-  const double c2g_B = si_W + si_G;
-  const double ag_wre = AG_w * wre;
-  const double g2g_B[2] = {ag_wre + RS_g * ore + AR_g * (1.0 - ore), ag_wre + RS_g * gre};
-  const double extra_fb = extra_fwd + extra_bwd;
-  const double exec_bwd_ck = exec_fwd + exec_bwd_nock;
-  const double first_g2c = adv ? g2c_B : 0.0;
-  Family bwd[2][2];
+  if (kFromKeys) {
 #pragma unroll
-  for (int ph = 0; ph < 2; ++ph) {
+    for (int j = 0; j < 4; ++j) {
+      const double *f = v + kKeyBwd + j * 5;
+      bwd[j >> 1][j & 1] = Family{f[0], f[1], f[2], f[3], f[4]};
+    }
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
-      const double E = k ? exec_bwd_ck - extra_fb : exec_bwd_nock - extra_bwd;
-      const double extra = k ? extra_fb : extra_bwd;
-      const double c2g = c2g_B + (k ? si_A_ck : si_A_nock);
-      double red;
-      if (ph == 0) red = k ? (ore == 1.0 ? RS_g : AR_g) : RS_g * ore + AR_g * (1.0 - ore);
-      else red = RS_g * gre;
-      // With checkpointing the reference adds the (always zero) all-gather of saved tensors.
-      const double g2g_layer = k ? g2g_B[ph] + 0.0 : g2g_B[ph];
-      bwd[ph][k].layer = I(E, g2g_layer, g2c_B, c2g) + extra;
-      bwd[ph][k].last = I.exec_g2g_c2g(E, ag_wre, c2g) + extra;
-      bwd[ph][k].first = I.exec_g2g_g2c(E, red, first_g2c) + extra;
-      bwd[ph][k].extra_pre = I.g2g_c2g(ag_wre, c2g);
-      bwd[ph][k].extra_post = I.g2g_g2c(red, first_g2c);
+      const double *f = v + kKeyFwd + k * 3;
+      fwd[1][k] = Family{f[0], v[kKeyFwdFirst], f[1], v[kKeyFwdExtraPre], f[2]};
     }
+  } else {
+    const FwdOperands op = fwd_operands(in, false, 0.0, 0.0);
+    double first, extra_pre;
+    fwd_common(I, in, op, false, adv, first, extra_pre);
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      fwd[1][k].first = first;
+      fwd[1][k].extra_pre = extra_pre;
+      fwd_of_ckpt(I, in, op, k != 0, fwd[1][k].layer, fwd[1][k].last, fwd[1][k].extra_post);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) bwd[j >> 1][j & 1] = bwd_family(I, in, (j & 2) != 0, (j & 1) != 0);
   }
 
   // ---- stable / delta families (:1910-2028) ----
-  double *t = lds_out + threadIdx.x * (MIST_ROW_TERMS + 1);
+  double t[MIST_ROW_TERMS];  // compile-time indices only: registers
   const int st = g->grad_accum == 1 ? 0 : 1;  // phase index that forms the stable part
 #pragma unroll
   for (int k = 0; k < 2; ++k) {
@@ -514,56 +749,74 @@ __global__ __launch_bounds__(kTermsBlock) void row_terms_kernel(
   t[MIST_T_GCB] = par[MIST_PAR_GCB];
 
   // ---- post-layer overlap pieces (:2251-2292) ----
-  const double ovw_ck = fmax(exec_fwd - 0.0 - so_A_ck, 0.0);
-  const double ovw_nock = fmax(exec_fwd - 0.0 - so_A_nock, 0.0);
+  const double ovw_ck = fmax(in.exec_fwd - 0.0 - in.so_A_ck, 0.0);
+  const double ovw_nock = fmax(in.exec_fwd - 0.0 - in.so_A_nock, 0.0);
   t[MIST_T_NAG_CK] = fmax(g->post_ag - ovw_ck, 0.0);
   t[MIST_T_NAG_NOCK] = fmax(g->post_ag - ovw_nock, 0.0);
-  const double ovg_ck = fmax(exec_bwd_ck - ag_wre - c2g_B - si_A_ck, 0.0);
-  const double ovg_nock = fmax(exec_bwd_nock - ag_wre - c2g_B - si_A_nock, 0.0);
+  const double ovg_ck = fmax(in.exec_bwd_ck - in.ag_wre - in.c2g_B - in.si_A_ck, 0.0);
+  const double ovg_nock = fmax(in.exec_bwd_nock - in.ag_wre - in.c2g_B - in.si_A_nock, 0.0);
   t[MIST_T_NRS_CK] = fmax(g->post_rs - ovg_ck, 0.0);
   t[MIST_T_NRS_NOCK] = fmax(g->post_rs - ovg_nock, 0.0);
   t[MIST_T_OPB] = fmax(g->post_bwd - bwd[1][1].extra_pre, 0.0);
   t[MIST_T_RD] = raw_nock - S_nock;
 
-  __syncthreads();
   if (kMode == 1) {  // scattered rows: every lane writes its own
     if ((int)threadIdx.x < rows_here) {
       double2 *__restrict__ mine =
           reinterpret_cast<double2 *>(row_terms + (g->row_offset + row) * MIST_ROW_TERMS);
+#pragma unroll
       for (int i = 0; i < MIST_ROW_TERMS / 2; ++i) mine[i] = make_double2(t[2 * i], t[2 * i + 1]);
     }
     return;
   }
-  double2 *__restrict__ dst =
-      reinterpret_cast<double2 *>(row_terms + (g->row_offset + block_first) * MIST_ROW_TERMS);
   if (kMode == 2) lds_skip[threadIdx.x] = is_scout_pair(g, pair) ? 1 : 0;
-  if (kMode == 2) __syncthreads();
-  for (int i = threadIdx.x; i < rows_here * (MIST_ROW_TERMS / 2); i += kTermsBlock) {
-    const int r = i / (MIST_ROW_TERMS / 2);
-    if (kMode == 2 && lds_skip[r]) continue;  // written by the kMode 1 launch
-    const int at = r * (MIST_ROW_TERMS + 1) + 2 * (i % (MIST_ROW_TERMS / 2));
-    dst[i] = make_double2(lds_out[at], lds_out[at + 1]);
-  }
-  // Summary of each stage of kStageRows rows for the reduce kernel: lane = (column, half of the
-  // stage's rows); columns 0 .. MIST_T_GCB hold the minimum, column kStageMaxOut the maximum of
-  // MIST_T_OUT.
-  {
-    const int stage_here = threadIdx.x / kStageRows, lane = threadIdx.x % kStageRows;
-    const int col = lane & (kStageFloorPitch - 1), half = lane / kStageFloorPitch;
+  static_assert(kTermsBlock % kStageRows == 0 && kStageRows == 64, "a wavefront's rows are one stage");
+  const int wave = threadIdx.x / kStageRows, lane = threadIdx.x % kStageRows;
+  for (int stage_here = 0; stage_here < kTermsBlock / kStageRows; ++stage_here) {
+    if (wave == stage_here) {
+#pragma unroll
+      for (int i = 0; i < MIST_ROW_TERMS; ++i) lds_out[lane * (MIST_ROW_TERMS + 1) + i] = t[i];
+    }
+    __syncthreads();
+    const int stage_first = stage_here * kStageRows;
+    const int stage_rows = min(kStageRows, rows_here - stage_first);  // <= 0: nothing left
+    double2 *__restrict__ dst = reinterpret_cast<double2 *>(
+        row_terms + (g->row_offset + block_first + stage_first) * MIST_ROW_TERMS);
+    for (int i = threadIdx.x; i < stage_rows * (MIST_ROW_TERMS / 2); i += kTermsBlock) {
+      const int r = i / (MIST_ROW_TERMS / 2);
+      if (kMode == 2 && lds_skip[stage_first + r]) continue;  // written by the kMode 1 launch
+      const int at = r * (MIST_ROW_TERMS + 1) + 2 * (i % (MIST_ROW_TERMS / 2));
+      dst[i] = make_double2(lds_out[at], lds_out[at + 1]);
+    }
+    // Summary of the stage for the reduce kernel: thread = (column, one of kTermsBlock / 32
+    // runs of the stage's rows); columns 0 .. MIST_T_GCB hold the minimum, column kStageMaxOut
+    // the maximum of MIST_T_OUT.  The runs of a wavefront meet by shuffle, the wavefronts in LDS.
+    constexpr int kRuns = kTermsBlock / kStageFloorPitch, kRunRows = kStageRows / kRuns;
+    const int col = threadIdx.x & (kStageFloorPitch - 1), run = threadIdx.x / kStageFloorPitch;
     const int src_col = col == kStageMaxOut ? MIST_T_OUT : col;
-    const int r_begin = stage_here * kStageRows + half * (kStageRows / 2);
-    const int r_end = min(r_begin + kStageRows / 2, rows_here);
     double lo_v = INFINITY, hi_v = 0.0;
     if (col <= kStageMaxOut) {
-      for (int r = r_begin; r < r_end; ++r) {
-        const double v = lds_out[r * (MIST_ROW_TERMS + 1) + src_col];
-        lo_v = fmin(lo_v, v);
-        hi_v = fmax(hi_v, v);
+#pragma unroll
+      for (int i = 0; i < kRunRows; ++i) {
+        const int r = run * kRunRows + i;
+        const double x = lds_out[min(r, kStageRows - 1) * (MIST_ROW_TERMS + 1) + src_col];
+        lo_v = fmin(lo_v, r < stage_rows ? x : INFINITY);
+        hi_v = fmax(hi_v, r < stage_rows ? x : 0.0);
       }
     }
     lo_v = fmin(lo_v, __shfl_xor(lo_v, kStageFloorPitch));
     hi_v = fmax(hi_v, __shfl_xor(hi_v, kStageFloorPitch));
-    if (half == 0 && stage_here * kStageRows < rows_here) {
+    if (wave > 0 && lane < kStageFloorPitch) {
+      lds_part[wave - 1][0][col] = lo_v;
+      lds_part[wave - 1][1][col] = hi_v;
+    }
+    __syncthreads();  // every read of this stage is done; the other wavefronts' parts are in LDS
+    if (wave == 0 && lane < kStageFloorPitch && stage_rows > 0) {
+#pragma unroll
+      for (int w = 0; w < kTermsBlock / kStageRows - 1; ++w) {
+        lo_v = fmin(lo_v, lds_part[w][0][col]);
+        hi_v = fmax(hi_v, lds_part[w][1][col]);
+      }
       const int64_t slot = stage_floor_slot(g, (int)(g - groups), block_first / kStageRows + stage_here);
       stage_floor[slot * kStageFloorPitch + col] = col < kStageMaxOut ? lo_v : (col == kStageMaxOut ? hi_v : 0.0);
     }
@@ -1693,18 +1946,45 @@ int mist_sizeof_problem(void) { return (int)sizeof(MistProblem); }
 int mist_sizeof_group(void) { return (int)sizeof(MistGroupDesc); }
 int mist_reduce_p_tile(void) { return MIST_P_TILE; }
 
+// key_terms_kernel over every group when the caller gave a key-term workspace and the bound the
+// grid needs; *launched tells whether the row-term kernel can read key terms.
+static int launch_key_terms(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,
+                            double *d_key_terms, hipStream_t stream, bool *launched) {
+  *launched = d_key_terms != nullptr && problem->max_group_keys > 0 && n_groups <= 65535;
+  if (!*launched) return 0;
+  constexpr int kKeysPerBlock = kTermsBlock / 4;
+  const unsigned blocks = (unsigned)((problem->max_group_keys + kKeysPerBlock - 1) / kKeysPerBlock);
+  hipLaunchKernelGGL(key_terms_kernel, dim3(blocks, n_groups), dim3(kTermsBlock), 0, stream, *problem,
+                     d_groups, d_key_terms);
+  MIST_HIP_CHECK(hipGetLastError());
+  return 0;
+}
+
 int mist_row_terms(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,
                    const int32_t *d_block_prefix, int n_blocks, double *d_row_terms,
-                   double *d_stage_floor, void *stream) {
+                   double *d_stage_floor, double *d_key_terms, void *stream) {
   if (int rc = check_common(problem, d_groups, n_groups)) return rc;
   if (!d_block_prefix || !d_row_terms || !d_stage_floor)
     return fail(MIST_E_INVALID, "null workspace pointer");
   if (n_blocks <= 0) return fail(MIST_E_INVALID, "n_blocks must be positive, got %d", n_blocks);
   if (int rc = check_factors(problem)) return rc;
-  hipLaunchKernelGGL(row_terms_kernel<0>, dim3(n_blocks), dim3(kTermsBlock), 0, (hipStream_t)stream,
-                     *problem, d_groups, n_groups, d_block_prefix, d_row_terms, d_stage_floor);
+  bool from_keys = false;
+  if (int rc = launch_key_terms(problem, d_groups, n_groups, d_key_terms, (hipStream_t)stream, &from_keys))
+    return rc;
+  if (from_keys)
+    hipLaunchKernelGGL((row_terms_kernel<0, true>), dim3(n_blocks), dim3(kTermsBlock), 0,
+                       (hipStream_t)stream, *problem, d_groups, n_groups, d_block_prefix, d_row_terms,
+                       d_stage_floor, d_key_terms);
+  else
+    hipLaunchKernelGGL((row_terms_kernel<0, false>), dim3(n_blocks), dim3(kTermsBlock), 0,
+                       (hipStream_t)stream, *problem, d_groups, n_groups, d_block_prefix, d_row_terms,
+                       d_stage_floor, nullptr);
   MIST_HIP_CHECK(hipGetLastError());
   return 0;
+}
+
+int64_t mist_key_terms_doubles(int64_t total_keys) {
+  return total_keys < 0 ? -1 : total_keys * MIST_KEY_TERMS;
 }
 
 int mist_reduce_stage_rows(void) { return kStageRows; }
@@ -1893,9 +2173,9 @@ int mist_intra_stage_eval(const MistProblem *problem, const MistGroupDesc *d_gro
                           int n_groups, const int32_t *d_terms_block_prefix, int n_terms_blocks,
                           const int32_t *d_reduce_block_prefix, int n_reduce_blocks,
                           const int32_t *d_scout_prefix, int n_scout_blocks, double *d_row_terms,
-                          double *d_stage_floor, double *d_partial_cost, int32_t *d_partial_index,
-                          double ratio, int sample_index, int compute_terms,
-                          const MistOutTables *tables, void *stream) {
+                          double *d_stage_floor, double *d_key_terms, double *d_partial_cost,
+                          int32_t *d_partial_index, double ratio, int sample_index,
+                          int compute_terms, const MistOutTables *tables, void *stream) {
   if (compute_terms && n_scout_blocks > 0 && problem != nullptr && problem->max_scout_rows > 0 &&
       n_groups > 0 && n_groups <= 65535) {
     // The scout pass reads a few hundred rows per group and leaves most of the GPU idle; the row
@@ -1918,9 +2198,9 @@ int mist_intra_stage_eval(const MistProblem *problem, const MistGroupDesc *d_gro
     std::lock_guard<std::mutex> enqueue_guard(enqueue_lock);
     hipStream_t main_stream = (hipStream_t)stream;
     const unsigned scout_term_blocks = (unsigned)((problem->max_scout_rows + kTermsBlock - 1) / kTermsBlock);
-    hipLaunchKernelGGL(row_terms_kernel<1>, dim3(scout_term_blocks, n_groups), dim3(kTermsBlock), 0,
-                       main_stream, *problem, d_groups, n_groups, d_terms_block_prefix, d_row_terms,
-                       d_stage_floor);
+    hipLaunchKernelGGL((row_terms_kernel<1, false>), dim3(scout_term_blocks, n_groups),
+                       dim3(kTermsBlock), 0, main_stream, *problem, d_groups, n_groups,
+                       d_terms_block_prefix, d_row_terms, d_stage_floor, nullptr);
     MIST_HIP_CHECK(hipGetLastError());
     MIST_HIP_CHECK(hipEventRecord(os->rows_ready, main_stream));
     MIST_HIP_CHECK(hipStreamWaitEvent(os->side, os->rows_ready, 0));
@@ -1931,8 +2211,17 @@ int mist_intra_stage_eval(const MistProblem *problem, const MistGroupDesc *d_gro
                               d_partial_cost, d_partial_index, os->side))
       return rc;
     MIST_HIP_CHECK(hipEventRecord(os->scout_done, os->side));
-    hipLaunchKernelGGL(row_terms_kernel<2>, dim3(n_terms_blocks), dim3(kTermsBlock), 0, main_stream,
-                       *problem, d_groups, n_groups, d_terms_block_prefix, d_row_terms, d_stage_floor);
+    bool from_keys = false;
+    if (int rc = launch_key_terms(problem, d_groups, n_groups, d_key_terms, main_stream, &from_keys))
+      return rc;
+    if (from_keys)
+      hipLaunchKernelGGL((row_terms_kernel<2, true>), dim3(n_terms_blocks), dim3(kTermsBlock), 0,
+                         main_stream, *problem, d_groups, n_groups, d_terms_block_prefix, d_row_terms,
+                         d_stage_floor, d_key_terms);
+    else
+      hipLaunchKernelGGL((row_terms_kernel<2, false>), dim3(n_terms_blocks), dim3(kTermsBlock), 0,
+                         main_stream, *problem, d_groups, n_groups, d_terms_block_prefix, d_row_terms,
+                         d_stage_floor, nullptr);
     MIST_HIP_CHECK(hipGetLastError());
     MIST_HIP_CHECK(hipStreamWaitEvent(main_stream, os->scout_done, 0));
     hipLaunchKernelGGL(eval_reduce_kernel, dim3(xcd_padded_grid(n_reduce_blocks)), dim3(MIST_LC_TILE),
@@ -1945,7 +2234,7 @@ int mist_intra_stage_eval(const MistProblem *problem, const MistGroupDesc *d_gro
   }
   if (compute_terms) {
     if (int rc = mist_row_terms(problem, d_groups, n_groups, d_terms_block_prefix,
-                                n_terms_blocks, d_row_terms, d_stage_floor, stream))
+                                n_terms_blocks, d_row_terms, d_stage_floor, d_key_terms, stream))
       return rc;
   }
   if (int rc = mist_eval_reduce(problem, d_groups, n_groups, d_reduce_block_prefix,

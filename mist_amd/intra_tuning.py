@@ -268,6 +268,10 @@ class IntraStageTuner:
             groups["n_lc_tiles"] = n_lc_tiles
             groups["n_p_tiles"] = n_p_tiles
             groups["row_offset"] = np.concatenate(([0], np.cumsum(groups["n_rows"])[:-1]))
+            # keys = (parallelism row, activation ratio, offload pair): what 28 of a row's 36
+            # interference evaluations depend on; evaluated once per key, not once per row
+            n_keys = groups["n_par"].astype(np.int64) * groups["n_ao"] * groups["n_pair"]
+            groups["key_offset"] = np.concatenate(([0], np.cumsum(n_keys)[:-1]))
             terms_blocks = -(-groups["n_rows"] // _lib.TERMS_BLOCK)
             reduce_blocks = groups["n_chunks"].astype(np.int64) * n_lc_tiles * n_p_tiles
             # Scout pass: the rows of a group without weight / gradient offloading (one in n_pair)
@@ -297,6 +301,7 @@ class IntraStageTuner:
             scouted = groups["scout_stride"] > 0
             gathered = groups["n_par"] * groups["n_oo"] * groups["n_ao"] * groups["scout_stride"]
             problem["max_scout_rows"] = int(gathered[scouted].max()) if scouted.any() else 0
+            problem["max_group_keys"] = int(n_keys.max())
         # Batches of consecutive groups under the workspace bound: each holds its own copy of the
         # descriptors with row offsets that start at 0 and its own workgroup prefixes.
         batches = []
@@ -304,9 +309,11 @@ class IntraStageTuner:
             rows = int(groups["n_rows"][first:last].sum())
             sub = groups[first:last].copy()
             sub["row_offset"] -= groups["row_offset"][first]
+            sub["key_offset"] -= groups["key_offset"][first]
             rebase = lambda prefix: (prefix[first:last + 1] - prefix[first]).astype(np.int32)
             batches.append(dict(
                 first=first, last=last, groups=sub, total_rows=rows,
+                total_keys=int(n_keys[first:last].sum()),
                 terms_prefix=rebase(terms_prefix), reduce_prefix=rebase(reduce_prefix),
                 scout_prefix=rebase(scout_prefix),
             ))
@@ -365,9 +372,11 @@ class IntraStageTuner:
                 scout_prefix=to_dev(b["scout_prefix"]),
                 n_terms_blocks=int(b["terms_prefix"][-1]), n_reduce_blocks=int(b["reduce_prefix"][-1]),
                 n_scout_blocks=int(b["scout_prefix"][-1]), total_rows=b["total_rows"],
+                total_keys=b["total_keys"],
             ))
         max_rows = max([b["total_rows"] for b in batches], default=0)
         max_groups = max([b["n_groups"] for b in batches], default=0)
+        max_keys = max([b["total_keys"] for b in batches], default=0)
         # several samples share one scout launch: their scout slabs lie behind one another
         self._sample_batch = min(len(self.sample_slots), _lib.MAX_SAMPLE_BATCH)
         n_slabs = max([b["n_reduce_blocks"] + self._sample_batch * b["n_scout_blocks"] for b in batches] + [1])
@@ -376,6 +385,8 @@ class IntraStageTuner:
                 row_terms=torch.empty(max(max_rows, 1) * _lib.ROW_TERMS, dtype=torch.float64, device=dev),
                 stage_floor=torch.empty(lib.mist_stage_floor_doubles(max_rows, max_groups),
                                         dtype=torch.float64, device=dev),
+                key_terms=torch.empty(max(lib.mist_key_terms_doubles(max_keys), 1),
+                                      dtype=torch.float64, device=dev),
                 partial_cost=torch.empty(n_slabs * _lib.SLOTS * _lib.LC_TILE, dtype=torch.float64, device=dev),
                 partial_index=torch.empty(n_slabs * _lib.SLOTS * _lib.LC_TILE, dtype=torch.int32, device=dev),
             )
@@ -446,8 +457,8 @@ class IntraStageTuner:
             if events is None and not self.exhaustive and len(self.sample_slots) > 1:
                 _lib.check(lib.mist_row_terms(
                     prob_ptr, _ptr(d["groups"]), d["n_groups"], _ptr(d["terms_prefix"]),
-                    d["n_terms_blocks"], _ptr(w["row_terms"]), _ptr(w["stage_floor"]), stream),
-                    "mist_row_terms")
+                    d["n_terms_blocks"], _ptr(w["row_terms"]), _ptr(w["stage_floor"]),
+                    _ptr(w["key_terms"]), stream), "mist_row_terms")
                 for first in range(0, len(self.sample_slots), self._sample_batch):
                     slots = np.array(self.sample_slots[first:first + self._sample_batch], dtype=np.int32)
                     batch_ratios = np.ascontiguousarray(ratios[slots], dtype=np.float64)
@@ -467,8 +478,8 @@ class IntraStageTuner:
                         _ptr(d["terms_prefix"]), d["n_terms_blocks"],
                         _ptr(d["reduce_prefix"]), d["n_reduce_blocks"],
                         _ptr(d["scout_prefix"]), d["n_scout_blocks"],
-                        _ptr(w["row_terms"]), _ptr(w["stage_floor"]), _ptr(w["partial_cost"]),
-                        _ptr(w["partial_index"]), float(ratios[slot]), int(slot),
+                        _ptr(w["row_terms"]), _ptr(w["stage_floor"]), _ptr(w["key_terms"]),
+                        _ptr(w["partial_cost"]), _ptr(w["partial_index"]), float(ratios[slot]), int(slot),
                         1 if i == 0 else 0, ctypes.byref(out), stream,
                     )
                     _lib.check(rc, "mist_intra_stage_eval")
@@ -476,7 +487,8 @@ class IntraStageTuner:
                 if i == 0:
                     timed("row_terms", lambda: lib.mist_row_terms(
                         prob_ptr, _ptr(d["groups"]), d["n_groups"], _ptr(d["terms_prefix"]),
-                        d["n_terms_blocks"], _ptr(w["row_terms"]), _ptr(w["stage_floor"]), stream))
+                        d["n_terms_blocks"], _ptr(w["row_terms"]), _ptr(w["stage_floor"]),
+                        _ptr(w["key_terms"]), stream))
                 timed("eval_reduce", lambda: reduce_call(slot))
                 timed("finalize", lambda: lib.mist_finalize(
                     prob_ptr, _ptr(d["groups"]), d["n_groups"], _ptr(d["reduce_prefix"]),

@@ -61,8 +61,11 @@ def _compare(cfg, tables, tp, S=1, slots=None, meshes=None, Gs=None, require_fin
     return got, want
 
 
-def test_row_terms_bit_exact():
-    """Kernel 1 against the oracle's row-invariant arrays, every (G, mesh) group of plan 1."""
+@pytest.mark.parametrize("key_terms", [True, False], ids=["terms-per-key", "every-row-on-its-own"])
+def test_row_terms_bit_exact(key_terms):
+    """Kernel 1 against the oracle's row-invariant arrays, every (G, mesh) group of plan 1; with
+    the interference evaluations shared per (parallelism, activation ratio, offload pair) and
+    with every row evaluating all of them."""
     import torch
 
     from mist_amd import _lib
@@ -77,7 +80,7 @@ def test_row_terms_bit_exact():
         rc = lib.mist_row_terms(
             ctypes.c_void_p(plan["problem"].ctypes.data), dev["groups"].data_ptr(), dev["n_groups"],
             dev["terms_prefix"].data_ptr(), dev["n_terms_blocks"], dev["row_terms"].data_ptr(),
-            dev["stage_floor"].data_ptr(),
+            dev["stage_floor"].data_ptr(), dev["key_terms"].data_ptr() if key_terms else None,
             ctypes.c_void_p(torch.cuda.current_stream().cuda_stream),
         )
         _lib.check(rc, "mist_row_terms")

@@ -237,17 +237,17 @@ def test_library_loads_and_exports_every_declared_symbol():
 def test_argument_checks_reject_before_any_launch():
     """Host-side validation paths of the C ABI (no GPU needed: they return before launching)."""
     lib = _lib.load()
-    assert lib.mist_row_terms(None, None, 1, None, 1, None, None, None) == -1
+    assert lib.mist_row_terms(None, None, 1, None, 1, None, None, None, None) == -1
     assert b"null" in lib.mist_last_error()
     prob = make_problem(load_plan(1)[0], 4, 2, 1, 4, 2)
     pp = ctypes.c_void_p(prob.ctypes.data)
     fake = ctypes.c_void_p(4096)
-    assert lib.mist_row_terms(pp, fake, 0, fake, 1, fake, fake, None) == -1
-    assert lib.mist_row_terms(pp, fake, 1, fake, 1, fake, None, None) == -1
+    assert lib.mist_row_terms(pp, fake, 0, fake, 1, fake, fake, None, None) == -1
+    assert lib.mist_row_terms(pp, fake, 1, fake, 1, fake, None, None, None) == -1
     for bad_factor in (0.0, -1.5, float("inf"), float("nan")):  # the kernel relies on 0 / f == +0
         bad = prob.copy()
         bad["interf_factor"][0][7, 2] = bad_factor
-        assert lib.mist_row_terms(ctypes.c_void_p(bad.ctypes.data), fake, 1, fake, 1, fake, fake, None) == -1
+        assert lib.mist_row_terms(ctypes.c_void_p(bad.ctypes.data), fake, 1, fake, 1, fake, fake, None, None) == -1
         assert b"interference factor [7][2]" in lib.mist_last_error()
     assert lib.mist_stage_floor_doubles(640, 3) == (10 + 3 + 1) * 32 and lib.mist_stage_floor_doubles(-1, 3) == -1
     assert lib.mist_eval_reduce(pp, fake, 1, fake, 0, None, 0, fake, fake, 1.0, fake, fake, None) == -1

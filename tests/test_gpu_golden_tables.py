@@ -39,8 +39,8 @@ def test_fixtures_cover_every_benchmark_plan():
 
 @pytest.mark.parametrize("plan", [1, 2, 3, 4, 5])
 def test_pruned_and_exhaustive_search_give_the_same_tables_on_whole_plans(plan):
-    """Every table of every group of a benchmark plan (plan 2 is the timed workload; of plans 4
-    and 5 the oracle's fixtures cover a part of the groups only), pruned search (scout pass,
+    """Every table of every group of a benchmark plan (plan 2 is the timed workload; of plan 4
+    the oracle's fixtures cover a part of the groups only), pruned search (scout pass,
     sieves, bounds) against the kernel that evaluates every cell: identical row indices and
     costs."""
     import torch

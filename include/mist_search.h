@@ -264,13 +264,40 @@ int mist_intra_stage_eval(const MistProblem *problem, const MistGroupDesc *d_gro
  * d_row_terms as written by mist_row_terms.  d_out: [n_requests][MIST_ANALYZE_FIELDS] float64 =
  * for the variants middle stage, first stage (with_pre), last stage (with_post) and single stage
  * (pre_and_post), five values each: stable latency, delta latency, stable + delta / G, forward
- * peak MB, backward peak MB.  The last two variants are evaluated with the peaks at the request's
- * p; the reference reports them for p == 0 only.  An invalid request yields NaN. */
+ * peak MB, backward peak MB; then the module-level memory of the cell that get_extra_info
+ * reports (:2401-2749): forward states, backward states, saved activations of one micro-batch.
+ * The last two variants are evaluated with the peaks at the request's p; the reference reports
+ * them for p == 0 only.  An invalid request yields NaN. */
 #define MIST_ANALYZE_REQUEST_FIELDS 5
-#define MIST_ANALYZE_FIELDS 20
+#define MIST_ANALYZE_FIELDS 23
 int mist_stage_analyze(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,
                        const double *d_row_terms, const int32_t *d_requests, int n_requests,
                        double *d_out, void *stream);
+
+/* What the row terms fold together, for the debugging entries of the reference's per-cell
+ * dictionaries (get_extra_info, mist/analyzer/batched_module_analyzer.py:2401-2749): swap and
+ * collective latencies (:1310-1408), the communication operands of the four phases without the
+ * activation swaps (:1432-1452, 1646-1670), the full weight / gradient buffers (:2120-2141),
+ * the partial weights / gradients, and the five members (layer, first layer, last layer, extra
+ * before, extra after) of the eight latency families (:1453-1902).
+ * d_requests: [n_requests][2] int32 = (group, workspace position of the row within the group);
+ * d_out: [n_requests][MIST_DIAG_FIELDS] float64, NaN for an invalid request. */
+enum MistDiagField {
+  MIST_DG_SO_W, MIST_DG_SI_W, MIST_DG_SO_G, MIST_DG_SI_G, MIST_DG_SO_O, MIST_DG_SI_O,
+  MIST_DG_SO_A_CK, MIST_DG_SI_A_CK, MIST_DG_SO_A_NOCK, MIST_DG_SI_A_NOCK, /* swap out / in, s */
+  MIST_DG_AG_W, MIST_DG_RS_G, MIST_DG_AR_G, /* all-gather weights, reduce-scatter / all-reduce grads */
+  MIST_DG_WBUF, MIST_DG_GBUF, MIST_DG_PW, MIST_DG_PG, /* MB */
+  /* gpu->cpu, cpu->gpu, gpu<->gpu operands: forward first / later micro-batch, backward (the
+   * first two are the same for the last and the other micro-batches) last / not last */
+  MIST_DG_G2C_F0, MIST_DG_C2G_F0, MIST_DG_G2G_F0, MIST_DG_G2C_F1, MIST_DG_C2G_F1, MIST_DG_G2G_F1,
+  MIST_DG_G2C_B, MIST_DG_C2G_B, MIST_DG_G2G_B0, MIST_DG_G2G_B1,
+  /* 8 families x (layer, first, last, extra_pre, extra_post): forward first micro-batch without /
+   * with ckpt, forward later, backward last micro-batch, backward not last */
+  MIST_DG_FAMILIES
+};
+#define MIST_DIAG_FIELDS (MIST_DG_FAMILIES + 40)
+int mist_row_diagnostics(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,
+                         const int32_t *d_requests, int n_requests, double *d_out, void *stream);
 
 #ifdef __cplusplus
 }

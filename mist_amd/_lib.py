@@ -140,6 +140,8 @@ _SIGNATURES = {
     ),
     "mist_stage_analyze": (
         ctypes.c_int, [_VP, _VP, ctypes.c_int, _VP, _VP, ctypes.c_int, _VP, _VP]),
+    "mist_row_diagnostics": (
+        ctypes.c_int, [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, _VP]),
     "mist_intra_stage_eval": (
         ctypes.c_int,
         [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, ctypes.c_int,
@@ -227,7 +229,19 @@ _DP_SIGNATURES = {
 }
 
 
-ANALYZE_REQUEST_FIELDS, ANALYZE_FIELDS = 5, 20
+ANALYZE_REQUEST_FIELDS, ANALYZE_FIELDS = 5, 23
+# MistDiagField: scalars, then 8 families x 5 members
+DIAG_NAMES = (
+    "so_W", "si_W", "so_G", "si_G", "so_O", "si_O", "so_A_ck", "si_A_ck", "so_A_nock", "si_A_nock",
+    "AG_w", "RS_g", "AR_g", "Wbuf", "Gbuf", "pW", "pG",
+    "g2c_F0", "c2g_F0", "g2g_F0", "g2c_F1", "c2g_F1", "g2g_F1", "g2c_B", "c2g_B", "g2g_B0", "g2g_B1",
+)
+DIAG = {name: i for i, name in enumerate(DIAG_NAMES)}
+DIAG_FAMILIES = len(DIAG_NAMES)
+DIAG_FAMILY_NAMES = ("fwd_first_nock", "fwd_first_ck", "fwd_later_nock", "fwd_later_ck",
+                     "bwd_last_nock", "bwd_last_ck", "bwd_not_last_nock", "bwd_not_last_ck")
+DIAG_MEMBERS = ("layer", "first", "last", "extra_pre", "extra_post")
+DIAG_FIELDS = DIAG_FAMILIES + len(DIAG_FAMILY_NAMES) * len(DIAG_MEMBERS)
 MIP_CKPT_TUNED, MIP_CKPT_FIXED, MIP_CKPT_FULL = 0, 1, 2
 MIP_MAX_SAMPLES = 64
 MIP_MAX_VALUE = 1000000.0

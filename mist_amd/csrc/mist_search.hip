@@ -1917,6 +1917,103 @@ __global__ __launch_bounds__(64) void analyze_kernel(
   o[17] = lat.spp + lat.dpp / G64;
   o[18] = pf_post + g->pre_states + g->pre_saved;
   o[19] = pb_post + g->pre_states + g->pre_saved;
+  // module-level memory of the cell (:2150-2162, 2378-2383), reported by get_extra_info
+  o[20] = mem.fwd_states;
+  o[21] = mem.bwd_states;
+  o[22] = mem.mod_saved;
+}
+
+// The intermediate quantities of one candidate row that the row terms fold together: what the
+// reference's get_extra_info (:2401-2749) reports besides them.  Thread = request = (group,
+// workspace position); the same device functions as row_terms_kernel, every row on its own.
+__global__ __launch_bounds__(kTermsBlock) void row_diagnostics_kernel(
+    const MistProblem prob, const MistGroupDesc *__restrict__ groups, int n_groups,
+    const int32_t *__restrict__ requests, int n_requests, double *__restrict__ out) {
+  __shared__ __align__(16) double lds_factor[11][kFactorPitch];
+  __shared__ double lds_gpu_gpu[32];
+  InterferenceModel<false> I;
+  I.factors_tame = load_model_tables(prob, lds_factor, lds_gpu_gpu);
+  I.table = (LdsDouble *)&lds_factor[0][0];
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  const int i_safe = min(i, n_requests - 1);  // no early exit: the model's wave-wide test wants every lane
+  const int32_t *req = requests + (int64_t)i_safe * 2;
+  const int gi = req[0];
+  const int64_t pos = req[1];
+  const bool ok = gi >= 0 && gi < n_groups && pos >= 0 && pos < groups[min(max(gi, 0), n_groups - 1)].n_rows;
+  const MistGroupDesc *g = groups + (ok ? gi : 0);
+  const RowParts parts = parts_of_position(g, ok ? pos : 0);
+  const double wo = g->wo[g->pair_wo[parts.pair]], go = g->go[g->pair_go[parts.pair]];
+  const double oo = g->oo[parts.oo], ao = g->ao[parts.ao];
+  const double *par = g->par[parts.par];
+  const double dp = par[MIST_PAR_DP], wre = par[MIST_PAR_WRE], gre = par[MIST_PAR_GRE];
+  const double ore = par[MIST_PAR_ORE], W = par[MIST_PAR_W], Gr = par[MIST_PAR_G], O = par[MIST_PAR_O];
+  const double wre_size = wre == 1.0 ? dp : 1.0, gre_size = gre == 1.0 ? dp : 1.0;
+  const double ore_size = ore == 1.0 ? dp : 1.0;
+  const KeyInputs in = key_inputs(prob, lds_gpu_gpu, g, par, wo, go, ao);
+  const double so_O = host_link_latency(prob.gpu_cpu, O / ore_size * oo);
+  const double si_O = host_link_latency(prob.cpu_gpu, O / ore_size * oo);
+  const bool adv = prob.adv_first_block != 0;
+  Family fam[8];  // forward first / later micro-batch, backward last / not last; nock, ck each
+#pragma unroll
+  for (int ph = 0; ph < 2; ++ph) {
+    const FwdOperands op = fwd_operands(in, ph == 0, so_O, si_O);
+    double first, extra_pre;
+    fwd_common(I, in, op, ph == 0, adv, first, extra_pre);
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      Family &f = fam[ph * 2 + k];
+      f.first = first;
+      f.extra_pre = extra_pre;
+      fwd_of_ckpt(I, in, op, k != 0, f.layer, f.last, f.extra_post);
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) fam[4 + j] = bwd_family(I, in, (j & 2) != 0, (j & 1) != 0);
+  if (i >= n_requests) return;
+  double *o = out + (int64_t)i * MIST_DIAG_FIELDS;
+  if (!ok) {
+    for (int f = 0; f < MIST_DIAG_FIELDS; ++f) o[f] = NAN;
+    return;
+  }
+  const bool wbuf_on = wre_size > 1.0 || g->pp_wre == 1 || wo > 0.0;
+  const bool gbuf_on = gre_size > 1.0 || g->pp_gre == 1 || go > 0.0;
+  const FwdOperands f0 = fwd_operands(in, true, so_O, si_O), f1 = fwd_operands(in, false, 0.0, 0.0);
+  o[MIST_DG_SO_W] = in.so_W;
+  o[MIST_DG_SI_W] = in.si_W;
+  o[MIST_DG_SO_G] = in.so_G;
+  o[MIST_DG_SI_G] = in.si_G;
+  o[MIST_DG_SO_O] = so_O;
+  o[MIST_DG_SI_O] = si_O;
+  o[MIST_DG_SO_A_CK] = in.so_A_ck;
+  o[MIST_DG_SI_A_CK] = in.si_A_ck;
+  o[MIST_DG_SO_A_NOCK] = in.so_A_nock;
+  o[MIST_DG_SI_A_NOCK] = in.si_A_nock;
+  o[MIST_DG_AG_W] = in.AG_w;
+  o[MIST_DG_RS_G] = in.RS_g;
+  o[MIST_DG_AR_G] = in.AR_g;
+  o[MIST_DG_WBUF] = wbuf_on ? fmax(fmax(g->pre_full_w, g->post_full_w), W) : 0.0;
+  o[MIST_DG_GBUF] = gbuf_on ? fmax(fmax(g->pre_full_g, g->post_full_g), Gr) : 0.0;
+  o[MIST_DG_PW] = W / wre_size * (1.0 - wo);
+  o[MIST_DG_PG] = Gr / gre_size * (1.0 - go);
+  o[MIST_DG_G2C_F0] = f0.g2c;
+  o[MIST_DG_C2G_F0] = f0.c2g;
+  o[MIST_DG_G2G_F0] = f0.g2g;
+  o[MIST_DG_G2C_F1] = f1.g2c;
+  o[MIST_DG_C2G_F1] = f1.c2g;
+  o[MIST_DG_G2G_F1] = f1.g2g;
+  o[MIST_DG_G2C_B] = in.g2c_B;
+  o[MIST_DG_C2G_B] = in.c2g_B;
+  o[MIST_DG_G2G_B0] = in.g2g_B[0];
+  o[MIST_DG_G2G_B1] = in.g2g_B[1];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    double *f = o + MIST_DG_FAMILIES + j * 5;
+    f[0] = fam[j].layer;
+    f[1] = fam[j].first;
+    f[2] = fam[j].last;
+    f[3] = fam[j].extra_pre;
+    f[4] = fam[j].extra_post;
+  }
 }
 
 int check_factors(const MistProblem *problem) {
@@ -2243,6 +2340,19 @@ int mist_intra_stage_eval(const MistProblem *problem, const MistGroupDesc *d_gro
     return rc;
   return mist_finalize(problem, d_groups, n_groups, d_reduce_block_prefix, d_row_terms,
                        d_partial_cost, d_partial_index, sample_index, tables, stream);
+}
+
+int mist_row_diagnostics(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,
+                         const int32_t *d_requests, int n_requests, double *d_out, void *stream) {
+  if (int rc = check_common(problem, d_groups, n_groups)) return rc;
+  if (!d_requests || !d_out) return fail(MIST_E_INVALID, "null pointer");
+  if (n_requests <= 0) return fail(MIST_E_INVALID, "n_requests must be positive, got %d", n_requests);
+  if (int rc = check_factors(problem)) return rc;
+  hipLaunchKernelGGL(row_diagnostics_kernel, dim3((n_requests + kTermsBlock - 1) / kTermsBlock),
+                     dim3(kTermsBlock), 0, (hipStream_t)stream, *problem, d_groups, n_groups,
+                     d_requests, n_requests, d_out);
+  MIST_HIP_CHECK(hipGetLastError());
+  return 0;
 }
 
 int mist_stage_analyze(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,

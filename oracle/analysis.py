@@ -46,7 +46,7 @@ def stage_results(tables, config, stage_idx):
 
 
 def _scalar(entry):
-    return {k: float(np.asarray(v).reshape(-1)[0]) for k, v in entry.items()}
+    return {k: float(np.asarray(v).reshape(-1)[0]) for k, v in entry.items() if k != "extra_info"}
 
 
 def analyze(config, tables):

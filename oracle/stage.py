@@ -475,6 +475,8 @@ def batched_stage_analyze(
         p2p = gpu_gpu("p2p", out, inter_size=1 if across_nodes else None,
                       intra_size=None if across_nodes else 1) * 2
 
+    extra_of_c = {}  # get_extra_info (:2401-2749) of the current c, per layer index
+
     def record(variant, p, c, stable_v, delta_v, latency_v, fwd, bwd):
         for i, l in enumerate(num_layers_candidates):
             analysis[variant][(p, l, c)] = {
@@ -483,7 +485,130 @@ def batched_stage_analyze(
                 "mem_bwd_peak": np.broadcast_to(bwd, stable_v.shape)[i],
                 "latency_stable": stable_v[i],
                 "latency_delta": np.broadcast_to(delta_v, stable_v.shape)[i],
+                "extra_info": extra_of_c.get(i),
             }
+
+    def row0(x):
+        """First (in the analysis path: only) row of a per-row quantity as a python float."""
+        return float(np.asarray(x, dtype=np.float64).reshape(-1)[0])
+
+    def extra_info(i, c, variants, mod_saved):
+        """The debugging entries of the reference's result dictionaries for layer index ``i``
+        (get_extra_info, :2401-2749; its per-row arrays are indexed there with the layer index,
+        which only works with one candidate: here they are the given row's values).
+        ``variants`` = ((stable, delta), ...) of base / with_pre / with_post / with_pre_and_post."""
+        k_last = "ck" if c > 0 else "nock"
+        e = {
+            "*****memory_factor": row0(mf),
+            "*****mem_per_full_weight_buffer": row0(Wbuf),
+            "*****mem_per_full_grad_buffer": row0(Gbuf),
+            "****non_overlapped_post_weights_all_gather_latency": row0(nAG[k_last]),
+            "****non_overlapped_post_grad_sync_latency": row0(nRS[k_last]),
+            "****overlapped_post_bwd_latency": row0(opb),
+        }
+        ck_name = {"nock": "without_ckpt", "ck": "with_ckpt"}
+        for k in ("nock", "ck"):
+            for ph, mb in (("F1", "first"), ("Fn", "not_first")):
+                f_ = fwd[ph, k]
+                e[f"****latency_first_layer_critical_fwd_{mb}_micro_batch_{ck_name[k]}"] = row0(f_["first"])
+                e[f"****latency_last_layer_critical_fwd_{mb}_micro_batch_{ck_name[k]}"] = row0(f_["last"])
+                e[f"****latency_extra_pre_fwd_{mb}_micro_batch_{ck_name[k]}"] = row0(f_["extra_pre"])
+                e[f"****latency_extra_post_fwd_{mb}_micro_batch_{ck_name[k]}"] = row0(f_["extra_post"])
+                stars = "**" if k == "nock" else "*"
+                e[f"{stars}_latency_layer_critical_fwd_{mb}_micro_batch_{ck_name[k]}"] = row0(f_["layer"])
+            for ph, mb in (("BL", "last"), ("Bn", "not_last")):
+                b_ = bwd[ph, k]
+                e[f"****latency_last_layer_critical_bwd_{mb}_micro_batch_{ck_name[k]}"] = row0(b_["last"])
+                e[f"****latency_first_layer_critical_bwd_{mb}_micro_batch_{ck_name[k]}"] = row0(b_["first"])
+                e[f"****latency_extra_pre_bwd_{mb}_micro_batch_{ck_name[k]}"] = row0(b_["extra_pre"])
+                e[f"****latency_extra_post_bwd_{mb}_micro_batch_{ck_name[k]}"] = row0(b_["extra_post"])
+                stars = "**" if k == "nock" else "*"
+                e[f"{stars}_latency_layer_critical_bwd_{mb}_micro_batch_{ck_name[k]}"] = row0(b_["layer"])
+            e[f"****latency_layer_critical_stable_{ck_name[k]}"] = row0(lat[k]["s_layer"])
+            e[f"****latency_layer_critical_delta_{ck_name[k]}"] = row0(lat[k]["d_layer"])
+            e[f"****latency_pre_fwd_and_post_bwd_and_first_layer_stable_{ck_name[k]}"] = row0(lat[k]["s_first"])
+            e[f"****latency_post_fwd_and_pre_bwd_and_last_layer_stable_{ck_name[k]}"] = row0(lat[k]["s_last"])
+            e[f"****latency_pre_fwd_and_post_bwd_and_first_layer_delta_{ck_name[k]}"] = row0(lat[k]["d_first"])
+            e[f"****latency_post_fwd_and_pre_bwd_and_last_layer_delta_{ck_name[k]}"] = row0(lat[k]["d_last"])
+        for (stable_v, delta_v), suffix in zip(variants, ("", "_with_pre", "_with_post", "_with_pre_and_post")):
+            e["****latency_stable" + suffix] = row0(np.asarray(stable_v)[i])
+            e["****latency_delta" + suffix] = row0(np.broadcast_to(delta_v, np.asarray(stable_v).shape)[i])
+        # pre / post layers (:1069-1138)
+        pre_AR = gpu_gpu("all_reduce", pre_G, **pp_dp_kwargs)
+        post_AR = gpu_gpu("all_reduce", post_G, **pp_dp_kwargs)
+        amortized = lambda flag, v: np.where(flag == 1, v, v / G)
+        e.update({
+            "_latency_pre_fwd_latency": row0(pre_fwd),
+            "_latency_pre_bwd_latency": row0(pre_bwd),
+            "_latency_pre_weights_all_gather_latency": row0(pre_AG),
+            "_latency_pre_weights_all_gather_latency_amortized": row0(amortized(pp_wre, pre_AG)),
+            "_latency_pre_grad_sync_latency": row0(pre_RS),
+            "_latency_pre_grad_sync_amortized": row0(np.where(pp_ore == 0, pre_AR / G, amortized(pp_gre, pre_RS))),
+            "_latency_post_fwd_latency": row0(post_fwd),
+            "_latency_post_bwd_latency": row0(post_bwd),
+            "_latentcy_post_weights_all_gather_latency_amortized": row0(amortized(pp_wre, post_AG)),
+            "_latency_post_grad_sync_amortized": row0(np.where(pp_ore == 0, post_AR / G, amortized(pp_gre, post_RS))),
+            "_latency_post_grad_sync_latency": row0(post_RS),
+            "_latency_post_weights_all_gather_latency": row0(post_AG),
+            "_latency_layer_exec_fwd": row0(exec_fwd),
+            "_latency_layer_exec_bwd_without_ckpt": row0(exec_bwd_nock),
+            "_latency_layer_exec_bwd_with_ckpt": row0(exec_bwd_ck),
+            "_latency_layer_gpu_to_cpu_fwd_first_micro_batch_exclude_act": row0(g2c_F1),
+            "_latency_layer_cpu_to_gpu_fwd_first_micro_batch_exclude_act": row0(c2g_F1),
+            "_latency_layer_gpu_gpu_fwd_first_micro_batch_exclude_act": row0(g2g_F1),
+            "_latency_layer_gpu_to_cpu_fwd_not_first_micro_batch_exclude_act": row0(g2c_Fn),
+            "_latency_layer_cpu_to_gpu_fwd_not_first_micro_batch_exclude_act": row0(c2g_Fn),
+            "_latency_layer_gpu_gpu_fwd_not_first_micro_batch_exclude_act": row0(g2g_Fn),
+            "_latency_layer_gpu_to_cpu_bwd_last_micro_batch_exclude_act": row0(g2c_B),
+            "_latency_layer_cpu_to_gpu_bwd_last_micro_batch_exclude_act": row0(c2g_B),
+            "_latency_layer_gpu_gpu_bwd_last_micro_batch_exclude_act": row0(g2g_BL),
+            "_latency_layer_gpu_to_cpu_bwd_not_last_micro_batch_exclude_act": row0(g2c_B),
+            "_latency_layer_cpu_to_gpu_bwd_not_last_micro_batch_exclude_act": row0(c2g_B),
+            "_latency_layer_gpu_gpu_bwd_not_last_micro_batch_exclude_act": row0(g2g_Bn),
+            "_latency_layer_swap_out_weights": row0(so_W),
+            "_latency_layer_swap_in_weights": row0(si_W),
+            "_latency_layer_all_gather_weights": row0(AG_w),
+            "_latency_layer_swap_in_grads": row0(si_G),
+            "_latency_layer_swap_in_activations_with_ckpt": row0(si_A_ck),
+            "_latency_layer_swap_in_activations_without_ckpt": row0(si_A_nock),
+            "_latency_layer_swap_out_grads": row0(so_G),
+            "_latency_layer_swap_out_activations_with_ckpt": row0(so_A_ck),
+            "_latency_layer_swap_out_activations_without_ckpt": row0(so_A_nock),
+            "_latency_layer_reduce_scatter_grads": row0(RS_g),
+            "_latency_layer_bwd_all_gather_saved_with_ckpt": row0(ag_saved_ck),
+            "_latency_p2p_output": row0(p2p),
+            "_mem_layer_full_weights": row0(W),
+            "_mem_layer_full_grads": row0(Gr),
+            "_mem_layer_full_opts": row0(O),
+            "_mem_layer_partial_weights": row0(pW),
+            "_mem_layer_partial_grads": row0(pG),
+            "_mem_layer_partial_opts": row0(pO),
+            "_mem_layer_saved_with_ckpt": row0(S_ck),
+            "_mem_layer_saved_without_ckpt": row0(S_nock),
+            "_mem_raw_layer_saved_with_ckpt": row0(raw_ck),
+            "_mem_raw_layer_saved_without_ckpt": row0(raw_nock),
+            "_mem_layer_fwd_peak_with_ckpt": row0(tables.mem_peak("block", "fwd", b, tp, True)),
+            "_mem_layer_fwd_peak_without_ckpt": row0(fwd_peak_nock),
+            "_mem_layer_bwd_peak": row0(bwd_peak),
+            "_mem_layer_output": row0(out),
+            "_mem_module_fwd_saved": row0(np.asarray(mod_saved)[i]),
+            "_mem_pre_layer_full_weights": row0(pre_W),
+            "_mem_pre_layer_full_grads": row0(pre_G),
+            "_mem_pre_layer_full_opts": row0(pre_O),
+            "_mem_pre_layer_saved_without_ckpt": row0(pre_saved),
+            "_mem_pre_layer_states": row0(pre_states),
+            "_mem_post_layer_full_weights": row0(post_W),
+            "_mem_post_layer_full_grads": row0(post_G),
+            "_mem_post_layer_full_opts": row0(post_O),
+            "_mem_post_layer_saved_without_ckpt": row0(tables.mem_saved("post", False, f64(pp_b), f64(pp_tp))),
+            "_mem_post_layer_states": row0(post_states),
+            "_mem_post_layer_fwd_peak": row0(post_fwd_peak),
+            "_mem_post_layer_bwd_peak": row0(post_bwd_peak),
+            "_mem_post_layer_output": row0(post_output),
+            "_mem_module_fwd_states": row0(np.asarray(fwd_states)[i]),
+            "_mem_module_bwd_states": row0(np.asarray(bwd_states)[i]),
+        })
+        return e
 
     def reduce_and_gather(x, y_num, mask):
         """:2813-2824: indices, gathered stable / delta / rows with -1 -> inf."""
@@ -526,6 +651,13 @@ def batched_stage_analyze(
         cur_saved = cur_if_eq * c_eq_l + cur_if_not * (1 - c_eq_l)
         mod_saved = S_ck * c + S_nock * (num_layers - c)
         mod_saved = np.where(num_layers >= c, mod_saved, MEM_INF)
+
+        if analysis is not None:
+            extra_of_c.clear()
+            for i in range(n):
+                extra_of_c[i] = extra_info(
+                    i, c, ((stable, delta), (stable_pre, delta_pre), (stable_post, delta_post),
+                           (stable_pp, delta_pp)), mod_saved)
 
         for p in pre_saved_micro_batches_candidates:
             pipe_saved = p * mod_saved + cur_saved

@@ -66,6 +66,11 @@ def test_stage_dictionaries_match_oracle(plan, layers, pre_post):
                 assert g[key] == float(np.asarray(w[key]).reshape(-1)[0]), (trial, v, key)
             assert g["****latency_stable" + _SUFFIX[v]] == float(np.asarray(w["latency_stable"]).reshape(-1)[0])
             assert g["****latency_delta" + _SUFFIX[v]] == float(np.asarray(w["latency_delta"]).reshape(-1)[0])
+            # the debugging entries (get_extra_info): the same keys, every value bit-equal
+            extra = w["extra_info"]
+            assert set(extra) | {"latency", "mem_fwd_peak", "mem_bwd_peak"} == set(g)
+            differing = [k for k in extra if not (g[k] == extra[k] or (g[k] != g[k] and extra[k] != extra[k]))]
+            assert not differing, (trial, v, differing[:5], [(g[k], extra[k]) for k in differing[:5]])
             checked += 1
     assert checked >= 4
 

@@ -98,3 +98,75 @@ def test_pre_post_batch_out_of_range_leaves_the_dictionaries_empty():
     raw["strategy"]["pre_post_strategy"] = "tuned"   # the row's own dp = 1: batch size 1
     total, _, _, peaks = analysis.analyze(MistConfig(raw), tables)
     assert np.isfinite(total) and total > 0 and peaks[0] > 0
+
+
+def test_extra_info_keys_and_structure():
+    """The debugging entries of the analysis path: the oracle reports exactly the keys of the
+    reference's get_extra_info (batched_module_analyzer.py:2401-2749; the names are held in
+    tests/golden/extra_info_keys.json), and the entries are tied to each other by the
+    reference's own combinations (:1910-2028 families -> stable / delta members, :2165-2216
+    members -> stage latency, :2150-2162 module states), which a mislabelled entry breaks."""
+    import json
+    import os
+
+    from oracle.stage import batched_stage_analyze
+
+    here = os.path.dirname(os.path.abspath(__file__))
+    with open(os.path.join(here, "golden", "extra_info_keys.json")) as f:
+        names = json.load(f)
+    assert len(names) == 135 and len(set(names)) == 135
+    cfg, tables = tiny_plan(1, layers=6)
+    raw = cfg.raw()
+    raw["strategy"] = dict(
+        enabled=True, gradient_accumulation_steps=4, layer_partitions=[6], device_assignment=[[1, 2]],
+        gradient_checkpointing=[0], stage_strategies=[[1, 1, 1, 0, 0, 1, 0.0, 0.0, 0.0, 0.0]],
+        pre_post_strategy="dp")
+    cfg = MistConfig(raw)
+    G, l = 4, 5
+    row = [2, 2, 1, 1, 1, 1, 0.5, 0.5, 0.3, 0.2]  # dp 2 with ZeRO-3 flags, every offload ratio in use
+    for c in (0, 2, 4, 5):
+        found = [{}, {}, {}, {}]
+        batched_stage_analyze(tables, cfg, [0], list(range(1, l + 1)), [c], 1, 2, G, [row], 1, analysis=found)
+        e = found[0][(0, l, c)]["extra_info"]
+        assert list(e) == names
+        for ck in ("without_ckpt", "with_ckpt"):
+            stars = "**" if ck == "without_ckpt" else "*"
+            layer = (e[f"{stars}_latency_layer_critical_fwd_not_first_micro_batch_{ck}"]
+                     + e[f"{stars}_latency_layer_critical_bwd_not_last_micro_batch_{ck}"])
+            assert layer == e[f"****latency_layer_critical_stable_{ck}"]
+            first = (e[f"****latency_extra_pre_fwd_not_first_micro_batch_{ck}"]
+                     + e[f"****latency_extra_post_bwd_not_last_micro_batch_{ck}"]
+                     + e[f"****latency_first_layer_critical_fwd_not_first_micro_batch_{ck}"]
+                     + e[f"****latency_first_layer_critical_bwd_not_last_micro_batch_{ck}"])
+            assert first == e[f"****latency_pre_fwd_and_post_bwd_and_first_layer_stable_{ck}"]
+            last_first_mb = (e[f"****latency_extra_post_fwd_first_micro_batch_{ck}"]
+                             + e[f"****latency_extra_pre_bwd_last_micro_batch_{ck}"]
+                             + e[f"****latency_last_layer_critical_fwd_first_micro_batch_{ck}"]
+                             + e[f"****latency_last_layer_critical_bwd_last_micro_batch_{ck}"])
+            assert (last_first_mb - e[f"****latency_post_fwd_and_pre_bwd_and_last_layer_stable_{ck}"]
+                    == e[f"****latency_post_fwd_and_pre_bwd_and_last_layer_delta_{ck}"])
+        n_ck = min(max(c - 1, 0), l - 2)
+        n_nock = l - 2 - n_ck
+        first_ck, last_ck = ("with_ckpt" if c == l else "without_ckpt"), ("without_ckpt" if c == 0 else "with_ckpt")
+        stable = (n_ck * e["****latency_layer_critical_stable_with_ckpt"]
+                  + n_nock * e["****latency_layer_critical_stable_without_ckpt"]
+                  + e[f"****latency_pre_fwd_and_post_bwd_and_first_layer_stable_{first_ck}"]
+                  + e[f"****latency_post_fwd_and_pre_bwd_and_last_layer_stable_{last_ck}"])
+        assert float(np.float32(stable)) == e["****latency_stable"]
+        assert e["****latency_stable_with_pre"] == (
+            e["****latency_stable"] + e["_latency_pre_fwd_latency"] + e["_latency_pre_bwd_latency"]
+            + 0 + 0)  # "dp": neither ZeRO flag of the pre/post layers is set
+        dp = row[1]
+        assert e["_mem_layer_partial_opts"] == e["_mem_layer_full_opts"] / dp * (1 - row[8])
+        assert e["_mem_layer_saved_with_ckpt"] == e["_mem_raw_layer_saved_with_ckpt"] * (1 - row[9])
+        buffers = 2 * (e["*****mem_per_full_weight_buffer"] + e["*****mem_per_full_grad_buffer"])
+        part = e["_mem_layer_partial_weights"] + e["_mem_layer_partial_grads"]
+        assert e["_mem_module_fwd_states"] == (
+            buffers + e["_mem_layer_full_opts"] // dp + l * part + (l - 1) * e["_mem_layer_partial_opts"])
+        assert e["_mem_module_bwd_states"] == buffers + l * (part + e["_mem_layer_partial_opts"])
+        assert e["_mem_module_fwd_saved"] == (
+            e["_mem_layer_saved_with_ckpt"] * c + e["_mem_layer_saved_without_ckpt"] * (l - c))
+        assert e["_latency_layer_exec_bwd_with_ckpt"] == (
+            e["_latency_layer_exec_fwd"] + e["_latency_layer_exec_bwd_without_ckpt"])
+        assert e["_latency_layer_gpu_to_cpu_bwd_last_micro_batch_exclude_act"] == e["_latency_layer_swap_out_grads"]
+        assert e["_latency_layer_cpu_to_gpu_fwd_not_first_micro_batch_exclude_act"] == e["_latency_layer_swap_in_weights"]

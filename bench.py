@@ -198,6 +198,9 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 1 GiB device copy (known HBM traffic to scale the "
                          "FETCH_SIZE / WRITE_SIZE counters of a profiler run against)")
+    ap.add_argument("--only-plan", default=None, metavar="YAML",
+                    help="profiling aid: run --steps search steps of this plan of mist_amd/configs "
+                         "with resident descriptors, print their time and exit (no bench line)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU only (got --gpus {args.gpus}): the search runs on a "
@@ -218,6 +221,19 @@ def main():
     if not torch.cuda.is_available():
         raise SystemExit("bench.py needs a GPU: the search kernels have no CPU path")
     torch.cuda.set_device(0)
+
+    if args.only_plan:
+        search = PreparedSearch(MistConfig.from_yaml(os.path.join(REPO, "mist_amd", "configs", args.only_plan)), "cuda:0")
+        for _ in range(max(args.warmup, 1)):
+            search.run()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            cost, solution = search.run()
+        torch.cuda.synchronize()
+        print(json.dumps(dict(plan=args.only_plan, steps=args.steps, cost=cost,
+                              ms_per_step=1e3 * (time.perf_counter() - t0) / args.steps, **search.counts())))
+        return
 
     cfg = MistConfig.from_yaml(PLAN)
     search = PreparedSearch(cfg, "cuda:0")

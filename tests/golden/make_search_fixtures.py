@@ -267,12 +267,22 @@ def main():
     ap.add_argument("--no-tune", action="store_true", help="skip the end-to-end search")
     ap.add_argument("--shard", default="0/1", help="i/n: only every n-th group, starting at the i-th")
     ap.add_argument("--out", default=HERE, help="directory the fixture is written to")
-    ap.add_argument("--merge", default=None, help="join the part files of this directory and exit")
+    ap.add_argument("--merge", default=None, help="join the part files of this directory (and the groups "
+                    "of the committed fixture of a partly covered plan) and exit")
+    ap.add_argument("--max-work", type=int, default=0,
+                    help="leave out groups with more than this many rows x pre-saved micro-batch values "
+                    "(one group runs on one core; 0 = no bound)")
+    ap.add_argument("--skip-covered", action="store_true", help="leave out the groups the committed fixture holds")
+    ap.add_argument("--deadline", type=float, default=0.0,
+                    help="seconds after which the run stops and keeps what it has (0 = none)")
     a = ap.parse_args()
     if a.merge:
         import glob
 
         parts = sorted(glob.glob(os.path.join(a.merge, f"search_tables_plan{a.plan}.part*.json")))
+        whole = os.path.join(a.merge, f"search_tables_plan{a.plan}.json")  # a run without --shard
+        if os.path.exists(whole) and os.path.abspath(a.merge) != os.path.abspath(HERE):
+            parts.append(whole)
         out, have = None, []
         for p in parts:
             with open(p) as f:
@@ -282,9 +292,17 @@ def main():
                 out = d
             else:
                 out["groups"].update(d["groups"])
-        n = int(parts[0].rsplit("of", 1)[1].split(".")[0])
-        out["select"] = "all" if len(parts) == n else "; ".join(have)
         path = os.path.join(HERE, f"search_tables_plan{a.plan}.json")
+        if os.path.exists(path):  # a partly covered plan grows: keep what the fixture already holds
+            with open(path) as f:
+                old = json.load(f)
+            if old["select"] != "all" and "tune" not in old:
+                have.insert(0, old["select"])
+                for k, v in old["groups"].items():
+                    out["groups"].setdefault(k, v)
+        n = int(parts[0].rsplit("of", 1)[1].split(".")[0]) if "of" in os.path.basename(parts[0]) else 1
+        bounded = any("at most" in h for h in have)
+        out["select"] = "all" if len(parts) == n and not bounded and len(have) == len(parts) else "; ".join(have)
         with open(path, "w") as f:
             json.dump(out, f, indent=1, sort_keys=True)
             f.write("\n")
@@ -297,11 +315,23 @@ def main():
     else:
         wanted = SUBSETS[a.plan]
     jobs = []
+    from mist_amd.search_space import create_search_space_for_a_block_layer
+
     for tp, G, mesh in wanted:
-        n = group_rows(cfg, tables, tp, G, mesh)
+        # sizing only: the factored search space counts the rows without listing them (the
+        # oracle's own count goes into the record, run_group)
+        n = create_search_space_for_a_block_layer(
+            mesh[0], mesh[1], cfg.training.global_batch_size, G, cfg, constraint_fn=tables.constraint,
+            tp_size=tp).n_rows
         if n > 0:
             jobs.append((n * min(G, cfg.model.num_hidden_layers), (a.plan, tp, G, tuple(mesh), a.cache)))
     jobs.sort(key=lambda j: -j[0])  # long groups first
+    if a.max_work > 0:
+        jobs = [j for j in jobs if j[0] <= a.max_work]
+    if a.skip_covered:
+        with open(os.path.join(HERE, f"search_tables_plan{a.plan}.json")) as f:
+            covered = set(json.load(f)["groups"])
+        jobs = [j for j in jobs if group_key(j[1][1], j[1][2], j[1][3]) not in covered]
     shard, n_shards = (int(x) for x in a.shard.split("/"))
     jobs = jobs[shard::n_shards]
     groups = {}
@@ -314,27 +344,52 @@ def main():
             print(f"[{time.time() - t0:7.0f}s] ... {len(groups)}/{len(jobs)} groups done", flush=True)
 
     threading.Thread(target=heartbeat, daemon=True).start()
-    with get_context("fork").Pool(a.workers, maxtasksperchild=1) as pool:
-        for n, (key, rec) in enumerate(pool.imap_unordered(run_group, [j[1] for j in jobs])):
-            groups[key] = rec
-            print(f"[{time.time() - t0:7.0f}s] {n + 1}/{len(jobs)} {key} rows={rec['rows']} "
-                  f"finite={rec['finite']} ({rec['oracle_seconds']} s)", flush=True)
-    out = dict(
-        plan=PLAN_FILES[a.plan - 1], sample_size=1,
-        select=a.select if n_shards == 1 else f"shard {shard} of {n_shards} (groups by size, every {n_shards}th)",
-        made_by="tests/golden/make_search_fixtures.py (CPU oracle)",
-        groups={k: dict(rows=groups[k]["rows"], finite=groups[k]["finite"], digest=groups[k]["digest"])
-                for k in sorted(groups)},
-    )
-    if a.select == "all" and not a.no_tune and n_shards == 1:
-        out["tune"] = end_to_end(a.plan, a.cache, a.workers)
-        print("tune:", out["tune"]["cost"], out["tune"]["solution"], flush=True)
+    select = a.select if n_shards == 1 else f"shard {shard} of {n_shards} (groups by size, every {n_shards}th)"
+    if a.max_work > 0:
+        select += f", groups of at most {a.max_work} rows x pre-saved micro-batch values"
+    if a.skip_covered:
+        select += ", without those already covered"
     part = "" if n_shards == 1 else f".part{shard}of{n_shards}"
     os.makedirs(a.out, exist_ok=True)
     path = os.path.join(a.out, f"search_tables_plan{a.plan}{part}.json")
-    with open(path, "w") as f:
-        json.dump(out, f, indent=1, sort_keys=True)
-        f.write("\n")
+
+    def write(out):
+        with open(path + ".tmp", "w") as f:
+            json.dump(out, f, indent=1, sort_keys=True)
+            f.write("\n")
+        os.replace(path + ".tmp", path)
+
+    def fixture():
+        return dict(
+            plan=PLAN_FILES[a.plan - 1], sample_size=1, select=select,
+            made_by="tests/golden/make_search_fixtures.py (CPU oracle)",
+            groups={k: dict(rows=groups[k]["rows"], finite=groups[k]["finite"], digest=groups[k]["digest"])
+                    for k in sorted(groups)},
+        )
+
+    with get_context("fork").Pool(a.workers, maxtasksperchild=1) as pool:
+        results = pool.imap_unordered(run_group, [j[1] for j in jobs])
+        for n in range(len(jobs)):
+            try:
+                key, rec = results.next(timeout=max(a.deadline - (time.time() - t0), 1.0) if a.deadline else None)
+            except Exception as e:  # multiprocessing.TimeoutError: the deadline has passed
+                if type(e).__name__ != "TimeoutError":
+                    raise
+                print(f"[{time.time() - t0:7.0f}s] deadline: {len(groups)} of {len(jobs)} groups kept", flush=True)
+                select += f" (stopped after {len(groups)} of {len(jobs)})"
+                write(fixture())
+                pool.terminate()  # the unfinished groups are given up
+                print("wrote", path, flush=True)
+                return
+            groups[key] = rec
+            print(f"[{time.time() - t0:7.0f}s] {n + 1}/{len(jobs)} {key} rows={rec['rows']} "
+                  f"finite={rec['finite']} ({rec['oracle_seconds']} s)", flush=True)
+            write(fixture())
+    out = fixture()
+    if a.select == "all" and not a.no_tune and n_shards == 1:
+        out["tune"] = end_to_end(a.plan, a.cache, a.workers)
+        print("tune:", out["tune"]["cost"], out["tune"]["solution"], flush=True)
+    write(out)
     print("wrote", path, flush=True)
 
 

@@ -45,7 +45,12 @@ constexpr int kSlots = 2 * MIST_P_TILE + 2;  // per-thread running minima: base,
 // maximum of MIST_T_OUT, kStageFloorPitch doubles per stage.
 constexpr int kStageFloorPitch = 32;
 constexpr int kStageMaxOut = MIST_T_GCB + 1;  // slot of max(MIST_T_OUT) behind the stage minima
-static_assert(kStageMaxOut < kStageFloorPitch, "a stage summary is one 32-lane load");
+// ... and behind it the minima of the post-layer terms that the last-stage / single-stage
+// objectives add to every row: MIST_T_OPB, the smaller of MIST_T_NAG_CK / _NOCK, the smaller of
+// MIST_T_NRS_CK / _NOCK.
+constexpr int kStageMinOpb = kStageMaxOut + 1, kStageMinNag = kStageMaxOut + 2, kStageMinNrs = kStageMaxOut + 3;
+static_assert(kStageMinNrs < kStageFloorPitch, "a stage summary is one 32-lane load");
+static_assert(MIST_T_NAG_NOCK == MIST_T_NAG_CK + 1 && MIST_T_NRS_NOCK == MIST_T_NRS_CK + 1, "ck / nock pairs");
 static_assert(kStageRows == 2 * kStageFloorPitch, "lane = (column, half of the rows)");
 
 // ------------------------------------------------------------------------------------------
@@ -790,16 +795,21 @@ __global__ __launch_bounds__(kTermsBlock) void row_terms_kernel(
     }
     // Summary of the stage for the reduce kernel: thread = (column, one of kTermsBlock / 32
     // runs of the stage's rows); columns 0 .. MIST_T_GCB hold the minimum, column kStageMaxOut
-    // the maximum of MIST_T_OUT.  The runs of a wavefront meet by shuffle, the wavefronts in LDS.
+    // the maximum of MIST_T_OUT, the three behind it minima of post-layer terms.  The runs of a wavefront meet by shuffle, the wavefronts in LDS.
     constexpr int kRuns = kTermsBlock / kStageFloorPitch, kRunRows = kStageRows / kRuns;
     const int col = threadIdx.x & (kStageFloorPitch - 1), run = threadIdx.x / kStageFloorPitch;
-    const int src_col = col == kStageMaxOut ? MIST_T_OUT : col;
+    const int src_col = col == kStageMaxOut ? MIST_T_OUT
+                        : col == kStageMinOpb ? MIST_T_OPB
+                        : col == kStageMinNag ? MIST_T_NAG_CK
+                        : col == kStageMinNrs ? MIST_T_NRS_CK : col;
+    const int second_col = (col == kStageMinNag || col == kStageMinNrs) ? src_col + 1 : src_col;
     double lo_v = INFINITY, hi_v = 0.0;
-    if (col <= kStageMaxOut) {
+    {
 #pragma unroll
       for (int i = 0; i < kRunRows; ++i) {
         const int r = run * kRunRows + i;
-        const double x = lds_out[min(r, kStageRows - 1) * (MIST_ROW_TERMS + 1) + src_col];
+        const double *row_at = lds_out + min(r, kStageRows - 1) * (MIST_ROW_TERMS + 1);
+        const double x = fmin(row_at[src_col], row_at[second_col]);
         lo_v = fmin(lo_v, r < stage_rows ? x : INFINITY);
         hi_v = fmax(hi_v, r < stage_rows ? x : 0.0);
       }
@@ -818,7 +828,7 @@ __global__ __launch_bounds__(kTermsBlock) void row_terms_kernel(
         hi_v = fmax(hi_v, lds_part[w][1][col]);
       }
       const int64_t slot = stage_floor_slot(g, (int)(g - groups), block_first / kStageRows + stage_here);
-      stage_floor[slot * kStageFloorPitch + col] = col < kStageMaxOut ? lo_v : (col == kStageMaxOut ? hi_v : 0.0);
+      stage_floor[slot * kStageFloorPitch + col] = col == kStageMaxOut ? hi_v : lo_v;
     }
   }
 }
@@ -1405,6 +1415,12 @@ __device__ __forceinline__ void reduce_block(
     // each of them exceeds `bound` by at least its group-wide offset.
     double thr_o = below(thr_p, off_pre);
     if (do_post) {
+      // What the last-stage / single-stage objectives add to every row of this stage on top of
+      // their group-wide offsets: at least the stage's smallest post-layer terms (same slack).
+      const double nag_min = lds_min[kStageMinNag], nrs_min = lds_min[kStageMinNrs];
+      const double stage_post =
+          (ratio * (lds_min[kStageMinOpb] + (k.pp_wre ? nag_min : 0.0) + (k.pp_gre ? nrs_min : 0.0)) +
+           div_G((k.pp_wre ? 0.0 : nag_min) + (k.pp_gre ? 0.0 : nrs_min))) * (1.0 - kSlack);
       // Lower bounds of the last-stage / single-stage peaks (:2946-3106) from the pseudo row.
       double peak_f, peak_b;
       floor_mem.peaks(0, peak_f, peak_b);
@@ -1415,12 +1431,12 @@ __device__ __forceinline__ void reduce_block(
       const double pf_post = fmax(f_in, peak_f + post_states);
       const double pb_post = fmax(b_in, peak_b - lds_min[kStageMaxOut] + post_states) + post_output;
       if (fmax(pf_post, pb_post) * floor_mem.mf_pp <= cap)
-        thr_o = fmax(thr_o, below(best_post, off_post));
+        thr_o = fmax(thr_o, below(best_post, off_post + stage_post));
       if (do_nopp) {
         const double pf_pp = pf_post + pre_states + pre_saved;
         const double pb_pp = pb_post + pre_states + pre_saved;
         if (fmax(pf_pp, pb_pp) * lds_min[MIST_T_MF] <= cap)
-          thr_o = fmax(thr_o, below(best_pp, off_pp));
+          thr_o = fmax(thr_o, below(best_pp, off_pp + stage_post));
       }
     }
 

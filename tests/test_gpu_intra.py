@@ -96,6 +96,11 @@ def test_row_terms_bit_exact(key_terms):
                 got_floor = floor[off // _lib.STAGE_ROWS + gi + st]
                 assert np.array_equal(got_floor[:n_floor_terms], rows[:, :n_floor_terms].min(axis=0))
                 assert got_floor[n_floor_terms] == rows[:, _lib.TERM_NAMES.index("out")].max()
+                # minima of the post-layer terms (ck / nock variants together)
+                T = _lib.TERM
+                assert got_floor[n_floor_terms + 1] == rows[:, T["opb"]].min()
+                assert got_floor[n_floor_terms + 2] == rows[:, [T["nAG_ck"], T["nAG_nock"]]].min()
+                assert got_floor[n_floor_terms + 3] == rows[:, [T["nRS_ck"], T["nRS_nock"]]].min()
         L = cfg.model.num_hidden_layers
         assert len(plan["groups"]) > 0
         for rec in plan["groups"]:

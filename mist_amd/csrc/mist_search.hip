@@ -1390,12 +1390,18 @@ __device__ __forceinline__ void reduce_block(
     // no lane passes here is closed, and its memory bounds need not be formed ----
     double floor_x, floor_d, floor_cost, floor_bound;
     objective(lds_min, floor_x, floor_d, floor_cost, floor_bound);
+    // What the last-stage / single-stage objectives add to every row of this stage on top of
+    // their group-wide offsets: at least the stage's smallest post-layer terms (same slack).
+    const double nag_min = lds_min[kStageMinNag], nrs_min = lds_min[kStageMinNrs];
+    const double stage_post =
+        (ratio * (lds_min[kStageMinOpb] + (k.pp_wre ? nag_min : 0.0) + (k.pp_gre ? nrs_min : 0.0)) +
+         div_G((k.pp_wre ? 0.0 : nag_min) + (k.pp_gre ? 0.0 : nrs_min))) * (1.0 - kSlack);
     {
       const double loose_b = fin_b < n_tile ? (double)INFINITY : top_b;
       const double loose_p = fin_p < n_tile ? (double)INFINITY : top_p;
       double loose_o = below(loose_p, off_pre);
-      if (do_post) loose_o = fmax(loose_o, below(best_post, off_post));
-      if (do_nopp) loose_o = fmax(loose_o, below(best_pp, off_pp));
+      if (do_post) loose_o = fmax(loose_o, below(best_post, off_post + stage_post));
+      if (do_nopp) loose_o = fmax(loose_o, below(best_pp, off_pp + stage_post));
       if (!__any(active && (floor_cost <= loose_b || floor_bound <= loose_o))) continue;
     }
 
@@ -1415,12 +1421,6 @@ __device__ __forceinline__ void reduce_block(
     // each of them exceeds `bound` by at least its group-wide offset.
     double thr_o = below(thr_p, off_pre);
     if (do_post) {
-      // What the last-stage / single-stage objectives add to every row of this stage on top of
-      // their group-wide offsets: at least the stage's smallest post-layer terms (same slack).
-      const double nag_min = lds_min[kStageMinNag], nrs_min = lds_min[kStageMinNrs];
-      const double stage_post =
-          (ratio * (lds_min[kStageMinOpb] + (k.pp_wre ? nag_min : 0.0) + (k.pp_gre ? nrs_min : 0.0)) +
-           div_G((k.pp_wre ? 0.0 : nag_min) + (k.pp_gre ? 0.0 : nrs_min))) * (1.0 - kSlack);
       // Lower bounds of the last-stage / single-stage peaks (:2946-3106) from the pseudo row.
       double peak_f, peak_b;
       floor_mem.peaks(0, peak_f, peak_b);

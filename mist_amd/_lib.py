@@ -309,6 +309,11 @@ def load():
             f"{LIB_PATH} is missing: build it with `python -m mist_amd.build` "
             "(there is no CPU fallback for the search kernels)"
         )
+    # PyTorch brings its own HIP runtime; loaded first, the library binds to that one, and the
+    # streams and device pointers torch hands over belong to the runtime the kernels run on
+    # (loaded the other way round, the library's runtime sees no device).
+    import torch  # noqa: F401
+
     lib = ctypes.CDLL(LIB_PATH)
     for name, (restype, argtypes) in {**_SIGNATURES, **_DP_SIGNATURES, **_MIP_SIGNATURES,
                                       **_INTER_SIGNATURES}.items():

@@ -1012,6 +1012,8 @@ struct LaneMemory {
 // that stream the same rows are consecutive, so runs of kXcdRun logical workgroups are given to
 // one XCD (and the runs round-robin, which keeps the XCDs evenly loaded).  The grid is padded to
 // a multiple of kNumXcd * kXcdRun; logical indices past the end do nothing.
+// Distinct layer counts of one (l, c) tile up to which sieve A also drops rows by memory.
+constexpr int kTileLayerCounts = 12;
 constexpr int kNumXcd = 8;
 constexpr int kXcdRun = 16;
 __device__ __forceinline__ int xcd_run_block(int physical) {
@@ -1129,6 +1131,16 @@ __device__ __forceinline__ void reduce_block(
   }
 
   const double *__restrict__ src = row_terms + g->row_offset * MIST_ROW_TERMS;
+
+  // The tile's pairs are in (l, c) order, so its lanes hold a few consecutive l.  Per stage and
+  // per such l, one wave-wide test tells which ROWS cannot fit any (c, p) of this tile with that
+  // l (row_fits below); it needs the group's pre / post terms to be non-negative.
+  const int l_lo = __shfl(l, 0);
+  const int n_active = __popcll((unsigned long long)__ballot(active));
+  const int n_tile_l = __shfl(l, max(n_active - 1, 0)) - l_lo + 1;
+  const bool rows_filtered = n_active > 0 && n_tile_l <= kTileLayerCounts && pre_saved >= 0.0 &&
+                             pre_sas >= 0.0 && pre_states >= 0.0 && post_states >= 0.0 &&
+                             post_output >= 0.0;
 
   // Sieve A visits pairs class by class (which first / last family member the latency uses is
   // fixed per class): 0 = 0 < c < l, 1 = c == 0, 2 = c == l.
@@ -1513,6 +1525,37 @@ __device__ __forceinline__ void reduce_block(
                   std::integral_constant<int, 1>{});
       sieve_class(pairs_open & in_class2, std::integral_constant<int, 0>{},
                   std::integral_constant<int, 0>{});
+      // Rows that exceed the capacity with tile_l layers whatever c, p and variant: every
+      // variant's tested quantity is at least
+      //   max(fwd, bwd) * (smallest of the row's three memory factors),
+      //   fwd = fwd_states + (l - 1) min(S_ck, S_nock) + min(D_ck, D_nock) + fwd_peak + gcb
+      //         + p0 (l min(S_ck, S_nock) + 2 out),   bwd likewise with out counted once
+      // (cur_saved and mod_saved are sums of l - 1 and l saved terms; the last-stage variants
+      // take one output off the backward peak; pre / post terms only add).  The bound is taken
+      // 1e-9 short, far more than the roundings of the two evaluation orders.
+      if (rows_filtered && __any(sieve != 0)) {
+        uint64_t fits = ~0ull;
+        const double *mine = lds_terms + threadIdx.x * kLdsRowStride;
+        const double s_min = fmin(mine[MIST_T_S_CK], mine[MIST_T_S_NOCK]);
+        const double d_min = fmin(mine[MIST_T_D_CK], mine[MIST_T_D_NOCK]);
+        const double out = mine[MIST_T_OUT], gcb = mine[MIST_T_GCB];
+        const double mf_min =
+            fmin(fmin(mine[MIST_T_MF_BASE], mine[MIST_T_MF_PP]), mine[MIST_T_MF]);
+        const double fwd0 = mine[MIST_T_FWD_STATES0] + d_min + mine[MIST_T_FWD_PEAK] + gcb;
+        const double bwd0 = mine[MIST_T_BWD_STATES0] + d_min + mine[MIST_T_BWD_PEAK] + out + gcb;
+        const double pwg = mine[MIST_T_PWG], po = mine[MIST_T_PO], pwgo = mine[MIST_T_PWGO];
+#pragma unroll 1
+        for (int i = 0; i < n_tile_l; ++i) {
+          const double tl = (double)(l_lo + i), tl1 = (double)max(l_lo + i - 1, 0);
+          const double per_p = tl * s_min + 2.0 * out;
+          const double shared = tl1 * s_min + (double)p0 * per_p;
+          const double low = fmax(fwd0 + tl * pwg + tl1 * po + shared, bwd0 + tl * pwgo + shared);
+          const bool too_big = s_min >= 0.0 && out >= 0.0 && low >= 0.0 && mf_min >= 0.0 &&
+                               low * mf_min * (1.0 - 1e-9) > cap;
+          fits = l - l_lo == i ? ~__ballot(too_big) : fits;
+        }
+        sieve &= fits;
+      }
     }
 
     // ---- sieve B: lowest improvable slot and the memory test there, per-lane survivors.  It

@@ -31,11 +31,35 @@ SCOUT_MIN_STAGES = 128  # groups with fewer stages get no scout pass (0 = never 
 SCOUT_MIN_PAIRS = 4     # ... and so do groups with fewer (weight, gradient) offload pairs
 SCOUT_PAIRS = 1         # offload pairs whose rows the scout pass gathers: the first, (0, 0), then evenly spread ones
 SCOUT_PAIR_SPAN = 200   # ... one more for every so many pairs of the group (GPT-22B: 421 pairs, 3 gathered)
+# ... and three for a group none of whose parallelism rows can hold this fraction of the model's
+# layers (weights, gradients and optimizer states of a layer at the group's tensor parallelism,
+# unsharded, nothing offloaded) within the memory capacity: such stages need sharding or
+# offloading, and the winners spread over the weight / gradient offload pairs.  (Speed only,
+# set from four plans: LLaMA-70B has 0.07 - 0.28 there for tp 1 - 4 and 0.55 for tp 8 and runs
+# 140 -> 98 ms with the two further pairs; GPT-7B has 0.73 - 5.9 and LLaMA-13B 0.37 - 3.0, and
+# they run 17 - 20 % slower with further pairs for every group, 2 % with them for tp 1.)
+SCOUT_TIGHT_FRACTION = 0.3
+SCOUT_TIGHT_PAIRS = 3
 # Upper bound of the row-term workspace (272 bytes per candidate row): the groups of a tuner call
 # go through the kernels in batches of consecutive groups whose rows fit it (a group larger than
 # the bound is a batch of its own).  GPT-7B (0.88 GB) and LLaMA-13B (1.4 GB) are one batch,
 # GPT-22B (18.4 GB of row terms) ten; with more than one batch two such workspaces alternate.
 ROW_TERMS_BUDGET_BYTES = 2 << 30
+
+
+_SIDE_STREAMS: Dict[str, "torch.cuda.Stream"] = {}
+
+
+def _side_stream(device) -> "torch.cuda.Stream":
+    """The second stream that plans of several batches alternate with, one per device for the
+    life of the process.  A stream per tuner would take another hardware queue each time (there
+    are four): sooner or later one shared with the caller's stream or with the library's own
+    scout stream, whose kernels then no longer overlap (GPT-22B: 150 ms became 164 to 187 ms,
+    depending on how many tuners the process had created before)."""
+    key = str(torch.device(device))
+    if key not in _SIDE_STREAMS:
+        _SIDE_STREAMS[key] = torch.cuda.Stream(device=device)
+    return _SIDE_STREAMS[key]
 
 
 def _scout_pairs(group, count: int) -> List[int]:
@@ -218,7 +242,6 @@ class IntraStageTuner:
         # True: every p of 0..P is evaluated for every G (the operator boundary
         # batched_tune_best_latency_for_stage takes the p candidates from its caller)
         self.evaluate_all_p = False
-        self._side_stream = None
         self.results: Optional[IntraStageTunerOutput] = None
         self.stats: Dict[str, float] = {}
 
@@ -279,8 +302,15 @@ class IntraStageTuner:
             n_stages = -(-groups["n_rows"] // _lib.STAGE_ROWS)
             scout = (n_stages >= SCOUT_MIN_STAGES) & (groups["n_pair"] >= SCOUT_MIN_PAIRS) & (SCOUT_MIN_STAGES > 0)
             scout &= not self.exhaustive
-            pairs = np.minimum(np.minimum(SCOUT_PAIRS + groups["n_pair"] // SCOUT_PAIR_SPAN, groups["n_pair"]),
-                               _lib.MAX_SCOUT_PAIRS)
+            pairs = SCOUT_PAIRS + groups["n_pair"] // SCOUT_PAIR_SPAN
+            par = groups["par"]
+            layer_states = par[..., _lib.PAR["W"]] + par[..., _lib.PAR["G"]] + par[..., _lib.PAR["O"]]
+            layer_states = np.where(np.arange(_lib.MAX_PAR)[None, :] < groups["n_par"][:, None],
+                                    layer_states, np.inf).min(axis=1)
+            capacity_mb = cfg.hardware.memory_capacity * 1024.0
+            tight = capacity_mb < SCOUT_TIGHT_FRACTION * L * layer_states
+            pairs = np.where(tight, np.maximum(pairs, SCOUT_TIGHT_PAIRS), pairs)
+            pairs = np.minimum(np.minimum(pairs, groups["n_pair"]), _lib.MAX_SCOUT_PAIRS)
             groups["scout_stride"] = np.where(scout, pairs, 0)
             for i in range(len(groups)):
                 picked = _scout_pairs(groups[i], int(groups["scout_stride"][i]))
@@ -417,10 +447,9 @@ class IntraStageTuner:
         current = torch.cuda.current_stream(self.device)
         streams = [current]
         if len(dev_plan["workspaces"]) > 1 and events is None:
-            if self._side_stream is None:
-                self._side_stream = torch.cuda.Stream(device=self.device)
-            streams.append(self._side_stream)
-            self._side_stream.wait_stream(current)  # the tables are filled on the current stream
+            side = _side_stream(self.device)
+            streams.append(side)
+            side.wait_stream(current)  # the tables are filled on the current stream
         ratios = alpha_ratios(self.sample_size)
         out = tables.as_struct()
         prob_ptr = ctypes.c_void_p(plan["problem"].ctypes.data)

@@ -175,6 +175,33 @@ def test_workspace_batches_partition_the_groups(monkeypatch):
             assert len(batches) == 1
 
 
+@pytest.mark.parametrize("plan, expected", [
+    (2, {1: 72}),           # GPT-7B: the first offload pair only
+    (3, {1: 110}),          # LLaMA-13B: likewise
+    (5, {1: 24, 3: 96}),    # LLaMA-70B: tp 8 alone holds 30 % of the layers of a stage unsharded
+])
+def test_scout_pairs_follow_the_memory_pressure_of_a_group(plan, expected):
+    """Which offload pairs the scout pass gathers (speed only, never results): the first one, and
+    the middle and last one as well for groups none of whose parallelism rows holds 30 % of the
+    model's layers within the capacity without sharding or offloading."""
+    cfg, tables = load_plan(plan)
+    hw = cfg.hardware
+    meshes = _get_device_mesh_candidates(hw.num_nodes, hw.num_gpus_per_node, False)
+    Gs = _get_grad_accumu_steps_candidates(cfg.training.global_batch_size)
+    L = cfg.model.num_hidden_layers
+    g = IntraStageTuner(tables, L, meshes, Gs, tp_candidates(cfg), cfg, sample_size=1,
+                        device="cpu").prepare()["groups"]
+    strides, counts = np.unique(g["scout_stride"], return_counts=True)
+    assert dict(zip(strides.tolist(), counts.tolist())) == expected
+    for d in g:
+        par = d["par"][:d["n_par"]]
+        states = (par[:, _lib.PAR["W"]] + par[:, _lib.PAR["G"]] + par[:, _lib.PAR["O"]]).min()
+        tight = hw.memory_capacity * 1024.0 < 0.3 * L * states
+        assert (d["scout_stride"] == 3) == tight
+        picked = d["scout_pair"][:d["scout_stride"]].tolist()
+        assert picked == ([0, (d["n_pair"] - 1) // 2, d["n_pair"] - 1] if tight else [0])
+
+
 def test_best_solution_yaml_format():
     from mist_amd.tune_one_case import best_solution_yaml
 

@@ -1008,12 +1008,13 @@ struct LaneMemory {
   }
 };
 
+// Distinct layer counts of one (l, c) tile up to which sieve A also drops rows by memory.
+constexpr int kTileLayerCounts = 12;
+
 // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  Logical workgroups
 // that stream the same rows are consecutive, so runs of kXcdRun logical workgroups are given to
 // one XCD (and the runs round-robin, which keeps the XCDs evenly loaded).  The grid is padded to
 // a multiple of kNumXcd * kXcdRun; logical indices past the end do nothing.
-// Distinct layer counts of one (l, c) tile up to which sieve A also drops rows by memory.
-constexpr int kTileLayerCounts = 12;
 constexpr int kNumXcd = 8;
 constexpr int kXcdRun = 16;
 __device__ __forceinline__ int xcd_run_block(int physical) {
@@ -1134,7 +1135,7 @@ __device__ __forceinline__ void reduce_block(
 
   // The tile's pairs are in (l, c) order, so its lanes hold a few consecutive l.  Per stage and
   // per such l, one wave-wide test tells which ROWS cannot fit any (c, p) of this tile with that
-  // l (row_fits below); it needs the group's pre / post terms to be non-negative.
+  // l (after sieve A's loops, below); it needs the group's pre / post terms to be non-negative.
   const int l_lo = __shfl(l, 0);
   const int n_active = __popcll((unsigned long long)__ballot(active));
   const int n_tile_l = __shfl(l, max(n_active - 1, 0)) - l_lo + 1;

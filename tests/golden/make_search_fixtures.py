@@ -7,6 +7,8 @@ oracle's end-to-end ``(best_cost, best_solution)`` where every group of the plan
     python tests/golden/make_search_fixtures.py --plan 4 --select subset        # listed groups
     python tests/golden/make_search_fixtures.py --plan 5 --shard 0/4 --out parts  # a quarter of the
         groups; --merge parts then joins the part files into the fixture
+    python tests/golden/make_search_fixtures.py --plan 4 --skip-covered --split-p 3 --deadline 1100
+        # the groups the fixture lacks, each as three jobs over a share of its p values
 
 Runs on the CPU only (the oracle never touches the GPU library).  A group is one call of the
 oracle's ``batched_tune_best_latency_for_stage`` with ``sample_size = 1`` (the slot the
@@ -70,24 +72,21 @@ def cache_path(cache, plan, tp, G, mesh):
     return os.path.join(cache, f"plan{plan}", f"tp{tp}_G{G}_{mesh[0]}x{mesh[1]}.npz")
 
 
-def run_group(args):
-    """One (tp, G, mesh) group through the oracle; returns its fixture record."""
-    plan, tp, G, mesh, cache = args
-    path = cache_path(cache, plan, tp, G, mesh)
-    if os.path.exists(path):
-        with np.load(path) as z:
-            return group_key(tp, G, mesh), json.loads(str(z["record"]))
+def p_values(cfg, G):
+    """The pre-saved micro-batch values of a group (intra_tuning.py:185-193) and the plan's P."""
     from oracle.intra import max_pre_saved_micro_batches
-    from oracle.stage import batched_tune_best_latency_for_stage
 
-    cfg, tables = load_plan(plan)
     meshes, Gs, _ = plan_axes(cfg)
     L = cfg.model.num_hidden_layers
     P = max_pre_saved_micro_batches(meshes, Gs, L)
-    t0 = time.time()
-    res = batched_tune_best_latency_for_stage(
-        tables, cfg, list(range(min(G, L, P + 1))), list(range(1, L + 1)), list(range(0, L + 1)),
-        mesh[0], mesh[1], G, tp_size=tp, sample_size=1)
+    return list(range(min(G, L, P + 1))), P
+
+
+def finish_group(res, cfg, tables, plan, tp, G, mesh, cache, seconds):
+    """Pads the oracle's four result tables to the tuner's shapes, digests them and stores them
+    in the cache; returns the fixture record."""
+    L = cfg.model.num_hidden_layers
+    _, P = p_values(cfg, G)
     shapes = [(P + 1, L, L + 1, 1), (P + 1, L, L + 1, 1), (L, L + 1, 1), (L + 1, 1)]
     record = dict(rows=int(group_rows(cfg, tables, tp, G, mesh)), digest=[], finite=[])
     keep = {}
@@ -102,12 +101,105 @@ def run_group(args):
         record["finite"].append(int((index >= 0).sum()))
         keep[f"stable{v}"], keep[f"delta{v}"] = stable, delta
         keep[f"index{v}"] = index.astype(np.int32)
-    record["oracle_seconds"] = round(time.time() - t0, 1)
+    record["oracle_seconds"] = round(seconds, 1)
+    path = cache_path(cache, plan, tp, G, mesh)
     os.makedirs(os.path.dirname(path), exist_ok=True)
     tmp = path + f".tmp{os.getpid()}.npz"
     np.savez_compressed(tmp, record=json.dumps(record), **keep)
     os.replace(tmp, path)
-    return group_key(tp, G, mesh), record
+    return record
+
+
+def run_group(args):
+    """One (tp, G, mesh) group through the oracle; returns its fixture record."""
+    plan, tp, G, mesh, cache = args
+    path = cache_path(cache, plan, tp, G, mesh)
+    if os.path.exists(path):
+        with np.load(path) as z:
+            return group_key(tp, G, mesh), json.loads(str(z["record"]))
+    from oracle.stage import batched_tune_best_latency_for_stage
+
+    cfg, tables = load_plan(plan)
+    L = cfg.model.num_hidden_layers
+    ps, _ = p_values(cfg, G)
+    t0 = time.time()
+    res = batched_tune_best_latency_for_stage(
+        tables, cfg, ps, list(range(1, L + 1)), list(range(0, L + 1)),
+        mesh[0], mesh[1], G, tp_size=tp, sample_size=1)
+    return group_key(tp, G, mesh), finish_group(res, cfg, tables, plan, tp, G, mesh, cache,
+                                                time.time() - t0)
+
+
+def part_values(ps, part, n_parts):
+    """The contiguous share ``part`` of the pre-saved micro-batch values ``ps``."""
+    lo, hi = round(part * len(ps) / n_parts), round((part + 1) * len(ps) / n_parts)
+    return ps[lo:hi]
+
+
+def part_path(cache, plan, tp, G, mesh, part, n_parts):
+    return cache_path(cache, plan, tp, G, mesh)[:-4] + f".part{part}of{n_parts}.npz"
+
+
+def run_part(args):
+    """A share of one group's pre-saved micro-batch values through the oracle (--split-p): a
+    group too long for one core within the time there is.  The oracle's loop over p carries one
+    thing from p = 0 to the later values of the same (l, c), the layer mask narrowed by the
+    last-stage variant (batched_module_analyzer.py:3021-3023), so every share starts with
+    p = 0; the other values are independent of each other."""
+    plan, tp, G, mesh, cache, part, n_parts = args
+    key = group_key(tp, G, mesh)
+    path = part_path(cache, plan, tp, G, mesh, part, n_parts)
+    if os.path.exists(cache_path(cache, plan, tp, G, mesh)) or os.path.exists(path):
+        return key, part
+    from oracle.search_space import create_search_space
+    from oracle.stage import batched_stage_analyze
+
+    cfg, tables = load_plan(plan)
+    L = cfg.model.num_hidden_layers
+    ps, _ = p_values(cfg, G)
+    mine = part_values(ps, part, n_parts)
+    t0 = time.time()
+    rows = create_search_space(mesh[0], mesh[1], cfg.training.global_batch_size, G, cfg,
+                               constraint_fn=tables.constraint, tp_size=tp)
+    res = batched_stage_analyze(
+        tables, cfg, mine if mine[0] == 0 else [0] + mine, list(range(1, L + 1)),
+        list(range(0, L + 1)), mesh[0], mesh[1], G, rows, 1)
+    keep = dict(seconds=time.time() - t0)
+    for v in range(4 if part == 0 else 2):  # the p == 0 variants come from the first share
+        keep[f"stable{v}"], keep[f"delta{v}"], keep[f"index{v}"] = res[v][0], res[v][1], res[v][3]
+    os.makedirs(os.path.dirname(path), exist_ok=True)
+    tmp = path + f".tmp{os.getpid()}.npz"
+    np.savez_compressed(tmp, **keep)
+    os.replace(tmp, path)
+    return key, part
+
+
+def merge_parts(plan, tp, G, mesh, cache, n_parts):
+    """Joins the shares of a group written by run_part into the result of one oracle call."""
+    cfg, tables = load_plan(plan)
+    ps, _ = p_values(cfg, G)
+    parts = [np.load(part_path(cache, plan, tp, G, mesh, i, n_parts)) for i in range(n_parts)]
+    res = []
+    for v in range(4):
+        if v >= 2:
+            res.append((parts[0][f"stable{v}"], parts[0][f"delta{v}"], None, parts[0][f"index{v}"]))
+            continue
+        whole = [np.array(parts[-1][f"{name}{v}"]) for name in ("stable", "delta", "index")]
+        assert whole[0].shape[0] == len(ps)
+        for i in range(n_parts - 1):
+            mine = part_values(ps, i, n_parts)
+            for k, name in enumerate(("stable", "delta", "index")):
+                whole[k][mine] = parts[i][f"{name}{v}"][mine]
+        res.append((whole[0], whole[1], None, whole[2]))
+    seconds = sum(float(z["seconds"]) for z in parts)
+    record = finish_group(res, cfg, tables, plan, tp, G, mesh, cache, seconds)
+    for i in range(n_parts):
+        os.remove(part_path(cache, plan, tp, G, mesh, i, n_parts))
+    return record
+
+
+def run_job(args):
+    return run_part(args) if len(args) == 7 else run_group(args)
 
 
 class CachedResults:
@@ -273,6 +365,9 @@ def main():
                     help="leave out groups with more than this many rows x pre-saved micro-batch values "
                     "(one group runs on one core; 0 = no bound)")
     ap.add_argument("--skip-covered", action="store_true", help="leave out the groups the committed fixture holds")
+    ap.add_argument("--split-p", type=int, default=1,
+                    help="run every group as this many jobs, each with a share of the pre-saved "
+                    "micro-batch values (for groups too long for one core within --deadline)")
     ap.add_argument("--deadline", type=float, default=0.0,
                     help="seconds after which the run stops and keeps what it has (0 = none)")
     a = ap.parse_args()
@@ -367,9 +462,19 @@ def main():
                     for k in sorted(groups)},
         )
 
+    tasks = [j[1] for j in jobs]
+    n_shares = {}
+    if a.split_p > 1:  # never more shares than a group has values of p
+        tasks = []
+        for j in jobs:
+            k = min(a.split_p, len(p_values(cfg, j[1][2])[0]))
+            n_shares[group_key(j[1][1], j[1][2], j[1][3])] = k
+            tasks += [j[1] + (part, k) for part in range(k)]
+        select += f", up to {a.split_p} jobs per group"
+    parts_done = {}
     with get_context("fork").Pool(a.workers, maxtasksperchild=1) as pool:
-        results = pool.imap_unordered(run_group, [j[1] for j in jobs])
-        for n in range(len(jobs)):
+        results = pool.imap_unordered(run_job, tasks)
+        for n in range(len(tasks)):
             try:
                 key, rec = results.next(timeout=max(a.deadline - (time.time() - t0), 1.0) if a.deadline else None)
             except Exception as e:  # multiprocessing.TimeoutError: the deadline has passed
@@ -381,8 +486,20 @@ def main():
                 pool.terminate()  # the unfinished groups are given up
                 print("wrote", path, flush=True)
                 return
+            if a.split_p > 1:  # rec = the share that is done; the last one completes the group
+                parts_done.setdefault(key, set()).add(rec)
+                print(f"[{time.time() - t0:7.0f}s] {key} share {rec + 1} of {n_shares[key]}", flush=True)
+                if len(parts_done[key]) < n_shares[key]:
+                    continue
+                job = next(j[1] for j in jobs if group_key(j[1][1], j[1][2], j[1][3]) == key)
+                final = cache_path(job[4], job[0], job[1], job[2], job[3])
+                if os.path.exists(final):
+                    with np.load(final) as z:
+                        rec = json.loads(str(z["record"]))
+                else:
+                    rec = merge_parts(job[0], job[1], job[2], job[3], job[4], n_shares[key])
             groups[key] = rec
-            print(f"[{time.time() - t0:7.0f}s] {n + 1}/{len(jobs)} {key} rows={rec['rows']} "
+            print(f"[{time.time() - t0:7.0f}s] {len(groups)}/{len(jobs)} {key} rows={rec['rows']} "
                   f"finite={rec['finite']} ({rec['oracle_seconds']} s)", flush=True)
             write(fixture())
     out = fixture()

@@ -140,7 +140,9 @@ int mist_dp_select_candidates(const MistDpCosts *costs, int n_requests, const in
  * d_argmin (may be NULL): [n_tmax][max_stages+1][L+1][D+1][4] int32 =
  *   (end layer, n, m, ckpt), pre-filled with -1 by the caller.
  * d_scratch: mist_dp_scratch_floats() floats (four (L+1)(D+1) state planes per instance plus the
- * reachable row range of every device column). */
+ * reachable row range of every device column).
+ * For tests the environment variable MIST_DP_FORCE_SCHEDULE (step | fused | plane) overrides the
+ * choice of schedule; a shape the forced schedule does not support fails with MIST_E_INVALID. */
 int64_t mist_dp_scratch_floats(const MistDpShape *shape, int n_tmax);
 int mist_dp_run(const MistDpShape *shape, const MistDpCosts *costs, const float *d_tmax,
                 const int32_t *d_g_index, int n_tmax, int mode, int32_t *d_best_s,

@@ -154,6 +154,9 @@ int mist_reduce_scout_split(void); /* scout workgroups per (group, (l, c) tile, 
 int mist_workspace_oo_tile(void);  /* optimizer-ratio tile T of the workspace order (mist_row_terms) */
 int mist_terms_block_rows(void); /* candidate rows per workgroup of mist_row_terms */
 int mist_reduce_stage_rows(void); /* rows per LDS stage; rows_per_chunk must be a multiple */
+int mist_max_sample_batch(void); /* MIST_MAX_SAMPLE_BATCH the library was built with */
+int mist_key_terms_per_key(void); /* MIST_KEY_TERMS the library was built with */
+int mist_max_scout_pairs(void);  /* MIST_MAX_SCOUT_PAIRS the library was built with */
 /* doubles of the stage-summary workspace for `total_rows` workspace rows in `n_groups` groups */
 int64_t mist_stage_floor_doubles(int64_t total_rows, int n_groups);
 /* doubles of the key-term workspace for `total_keys` keys (sum of n_par * n_ao * n_pair) */

@@ -23,9 +23,9 @@ SCOUT_SPLIT = 4  # replaced by the library's own value in load()
 STAGE_ROWS = 64  # replaced by the library's own value in load()
 TERMS_BLOCK = 128  # replaced by the library's own value in load()
 MAX_MESH = 16
-MAX_SAMPLE_BATCH = 16  # MIST_MAX_SAMPLE_BATCH
-MAX_SCOUT_PAIRS = 8  # MIST_MAX_SCOUT_PAIRS
-KEY_TERMS = 28  # MIST_KEY_TERMS
+MAX_SAMPLE_BATCH = 16  # MIST_MAX_SAMPLE_BATCH; replaced by the library's own value in load()
+MAX_SCOUT_PAIRS = 8  # MIST_MAX_SCOUT_PAIRS (sizes a field of GROUP_DTYPE; checked in load())
+KEY_TERMS = 28  # MIST_KEY_TERMS; replaced by the library's own value in load()
 DP_NO_START = -3
 DP_CKPT_TAIL, DP_CKPT_STAGE, DP_CKPT_ALL = 0, 1, 2
 DP_THRESHOLD, DP_BOTTLENECK = 0, 1
@@ -117,6 +117,9 @@ _SIGNATURES = {
     "mist_reduce_lc_tile": (ctypes.c_int, []),
     "mist_terms_block_rows": (ctypes.c_int, []),
     "mist_reduce_scout_split": (ctypes.c_int, []),
+    "mist_max_sample_batch": (ctypes.c_int, []),
+    "mist_key_terms_per_key": (ctypes.c_int, []),
+    "mist_max_scout_pairs": (ctypes.c_int, []),
     "mist_stage_floor_doubles": (ctypes.c_int64, [ctypes.c_int64, ctypes.c_int]),
     "mist_key_terms_doubles": (ctypes.c_int64, [ctypes.c_int64]),
     "mist_row_terms": (ctypes.c_int, [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, _VP, _VP, _VP]),
@@ -340,7 +343,12 @@ def load():
         raise MistLibraryError(
             f"MistGroupDesc layout mismatch: C {lib.mist_sizeof_group()} vs numpy {GROUP_DTYPE.itemsize}"
         )
-    global P_TILE, SLOTS, STAGE_ROWS, LC_TILE, SCOUT_SPLIT, TERMS_BLOCK
+    if lib.mist_max_scout_pairs() != MAX_SCOUT_PAIRS:
+        raise MistLibraryError(
+            f"MIST_MAX_SCOUT_PAIRS mismatch: C {lib.mist_max_scout_pairs()} vs python {MAX_SCOUT_PAIRS}")
+    global P_TILE, SLOTS, STAGE_ROWS, LC_TILE, SCOUT_SPLIT, TERMS_BLOCK, MAX_SAMPLE_BATCH, KEY_TERMS
+    MAX_SAMPLE_BATCH = lib.mist_max_sample_batch()
+    KEY_TERMS = lib.mist_key_terms_per_key()
     TERMS_BLOCK = lib.mist_terms_block_rows()
     SCOUT_SPLIT = lib.mist_reduce_scout_split()
     LC_TILE = lib.mist_reduce_lc_tile()

@@ -12,6 +12,8 @@
 #include <algorithm>
 #include <cmath>
 #include <cstdint>
+#include <cstring>
+#include <cstdlib>
 #include <map>
 #include <mutex>
 #include <utility>
@@ -1178,7 +1180,22 @@ int mist_dp_run(const MistDpShape *shape, const MistDpCosts *costs, const float 
       sizeof(float);
   // (threshold batches from about 64 instances on: a workgroup's run through all stage counts
   // takes as long as the 1 + max_stages launches of a few dozen instances)
-  const bool fused_pays = mode == MIST_DP_THRESHOLD ? n_tmax >= kDpFusedMinInstances : !wide;
+  bool fused_pays = mode == MIST_DP_THRESHOLD ? n_tmax >= kDpFusedMinInstances : !wide;
+  // For tests: MIST_DP_FORCE_SCHEDULE = step | fused | plane takes the choice of schedule away
+  // from the batch size and the LDS need, so that each schedule can be run on any shape it
+  // supports (a shape it does not support is an error, not a silent fallback).
+  const char *forced = getenv("MIST_DP_FORCE_SCHEDULE");
+  const bool force_step = forced && !strcmp(forced, "step");
+  const bool force_fused = forced && !strcmp(forced, "fused");
+  const bool force_plane = forced && !strcmp(forced, "plane");
+  if (forced && *forced && !force_step && !force_fused && !force_plane)
+    return fail(MIST_E_INVALID, "MIST_DP_FORCE_SCHEDULE=%s: expected step, fused or plane", forced);
+  if (force_fused) {
+    if (costs->stage_min == nullptr || fused_lds > fused_lds_limit(mode))
+      return fail(MIST_E_INVALID, "forced fused schedule: needs stage_min and %zu B of LDS", fused_lds);
+    fused_pays = true;
+  }
+  if (force_step || force_plane) fused_pays = false;
   if (fused_pays && costs->stage_min != nullptr && fused_lds <= fused_lds_limit(mode)) {
     // one workgroup per CU when the planes take more than half of the LDS: then a larger one
     const int most = 2 * fused_lds > kDpLdsPerCu ? kDpFusedThreads : kDpFusedThreads / 2;
@@ -1201,8 +1218,13 @@ int mist_dp_run(const MistDpShape *shape, const MistDpCosts *costs, const float 
        (size_t)(kDpPlaneThreads / 64) * shape->num_mesh * shape->num_layers) * sizeof(float);
   const bool plane_shape_ok = shape->num_devices <= 64 * kDpPlaneCols &&
                               shape->num_mesh * shape->num_layers <= 64 * kDpPlaneLoads;
-  if (costs->stage_min != nullptr && shape->free_devices == 0 && n_tmax >= kDpPlaneMinInstances &&
-      plane_shape_ok && fused_lds > fused_lds_limit(mode) && plane_lds <= plane_lds_limit(mode)) {
+  const bool plane_possible = costs->stage_min != nullptr && shape->free_devices == 0 &&
+                              plane_shape_ok && plane_lds <= plane_lds_limit(mode);
+  if (force_plane && !plane_possible)
+    return fail(MIST_E_INVALID, "forced plane schedule: needs stage_min, consumed devices, D <= %d, "
+                "Q * L <= %d and %zu B of LDS", 64 * kDpPlaneCols, 64 * kDpPlaneLoads, plane_lds);
+  if (plane_possible && !force_step &&
+      (force_plane || (n_tmax >= kDpPlaneMinInstances && fused_lds > fused_lds_limit(mode)))) {
     if (mode == MIST_DP_BOTTLENECK)
       hipLaunchKernelGGL(dp_plane_kernel<true>, dim3(n_tmax), dim3(kDpPlaneThreads), plane_lds,
                          (hipStream_t)stream, *shape, *costs, d_tmax, d_g_index, d_scratch,

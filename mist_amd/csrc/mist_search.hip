@@ -2149,6 +2149,9 @@ int mist_reduce_lc_tile(void) { return MIST_LC_TILE; }
 int mist_terms_block_rows(void) { return kTermsBlock; }
 int mist_reduce_scout_split(void) { return kScoutSplit; }
 int mist_workspace_oo_tile(void) { return kOoTile; }
+int mist_max_sample_batch(void) { return MIST_MAX_SAMPLE_BATCH; }
+int mist_key_terms_per_key(void) { return MIST_KEY_TERMS; }
+int mist_max_scout_pairs(void) { return MIST_MAX_SCOUT_PAIRS; }
 int64_t mist_stage_floor_doubles(int64_t total_rows, int n_groups) {
   if (total_rows < 0 || n_groups < 0) return -1;
   return (total_rows / kStageRows + n_groups + 1) * kStageFloorPitch;

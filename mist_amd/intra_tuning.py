@@ -231,6 +231,8 @@ class IntraStageTuner:
         self.sample_size = int(sample_size)
         # Which of the S alpha samples to evaluate (default: all); unevaluated slots stay inf / -1.
         self.sample_slots = tuple(range(self.sample_size)) if sample_slots is None else tuple(sample_slots)
+        if not self.sample_slots or not all(0 <= s < self.sample_size for s in self.sample_slots):
+            raise ValueError(f"sample_slots must be a non-empty subset of 0..{self.sample_size - 1}")
         self.device = torch.device(device)
         # intra_tuning.py:117-126
         self.max_possible_num_stages = min(

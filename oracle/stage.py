@@ -109,8 +109,15 @@ def batched_stage_analyze(
     sample_size,
     debug=None,
     analysis=None,
+    inner="numpy",
+    threads=0,
 ):
     """:687-3144 with ``get_best_solution=True``.
+
+    ``inner="c"`` runs the loops over (ckpt layers, pre-saved micro-batches) and the argmin scan
+    through oracle/stage_loop.c instead of the numpy statements below: the same expressions
+    cell by cell, bit-equal tables (tests/test_oracle_stage_c.py), two orders of magnitude
+    faster on the large plans.  Everything up to the loops is the numpy code either way.
 
     ``analysis`` (a list of four dicts) additionally receives what the ``get_best_solution=False``
     path returns (:2788-2803, 2876-2892, 2980-2996, 3063-3079): per variant and ``(p, l, c)`` the
@@ -621,6 +628,39 @@ def batched_stage_analyze(
         sel_sol[indices == -1] = np.inf
         return indices, sel_s, sel_d, sel_sol
 
+    if inner in ("c", "c-fused"):  # "c-fused": the argmin objective as one fused multiply-add
+        assert analysis is None, "the C loops cover the tuning path only"
+        assert list(pre_saved_micro_batches_candidates) == list(range(P + 1))
+        assert list(num_layers_candidates) == list(range(1, Lmax + 1))
+        assert list(num_ckpt_layers_candidates) == list(range(Cmax + 1))
+        from . import stage_c
+        from .pareto import alpha_ratios
+
+        res = stage_c.run(
+            rows.shape[0], Lmax, Cmax, P + 1, S, G, alpha_ratios(S),
+            lat=lat,
+            mem=dict(T0=2 * (Wbuf + Gbuf) + O // ore_size, T1=2 * (Wbuf + Gbuf), pWG=pW + pG,
+                     pO=pO, pWGO=pW + pG + pO, S_ck=S_ck, S_nock=S_nock, D_ck=D_ck, D_nock=D_nock,
+                     fwd_peak=fwd_peak_nock, bwd_peak=bwd_peak, out=out, gcb=gcb, mf=mf,
+                     RD=raw_nock - S_nock),
+            post=dict(nAG=nAG, nRS=nRS, opb=opb),
+            scalars=dict(
+                pre_fwd=pre_fwd, pre_bwd=pre_bwd, W1=np.where(pp_wre == 1, pre_AG, 0),
+                W2=np.where(pp_gre == 1, pre_RS, 0), W1d=np.where(pp_wre == 1, 0, pre_AG),
+                W2d=np.where(pp_gre == 1, 0, pre_RS), post_fwd=post_fwd, pre_saved=pre_saved,
+                pre_states=pre_states, pre_states_and_saved=pre_states_and_saved,
+                post_states=post_states, post_fwd_peak=post_fwd_peak,
+                post_bwd_peak=post_bwd_peak, post_output=post_output),
+            pp_wre=int(np.asarray(pp_wre).reshape(-1)[0] == 1),
+            pp_gre=int(np.asarray(pp_gre).reshape(-1)[0] == 1), cap=cap, threads=threads,
+            fused=inner == "c-fused")
+        out_tuples = []
+        for stable_t, delta_t, idx_t in res:
+            sol_t = rows[idx_t]  # :2819-2824: gather, then -1 -> inf
+            sol_t[idx_t == -1] = np.inf
+            out_tuples.append((stable_t, delta_t, sol_t, idx_t))
+        return tuple(out_tuples)
+
     for c in num_ckpt_layers_candidates:
         valid_l = c <= num_layers.flatten()
         c_eq_l = c == num_layers
@@ -747,6 +787,8 @@ def batched_tune_best_latency_for_stage(
     tp_size=None,
     sample_size=None,
     debug=None,
+    inner="numpy",
+    threads=0,
 ):
     """:581-684: enumerate the rows, return all-``inf`` tables when there are none."""
     for cands, lo in (
@@ -793,4 +835,6 @@ def batched_tune_best_latency_for_stage(
         rows,
         sample_size,
         debug=debug,
+        inner=inner,
+        threads=threads,
     )

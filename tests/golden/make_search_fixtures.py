@@ -1,22 +1,28 @@
-"""Writes tests/golden/search_tables_plan<N>.json: what the CPU oracle (``oracle/``, the numpy
-restatement of the reference's search) finds for whole (tp, G, mesh) groups of the five
-benchmark plans at their full size, as one digest per group and table variant, plus the
-oracle's end-to-end ``(best_cost, best_solution)`` where every group of the plan is covered.
+"""Writes tests/golden/search_tables_plan<N>[_s<S>].json: what the CPU oracle (``oracle/``, the
+restatement of the reference's search) finds for whole (tp, G, mesh) groups of the five benchmark
+plans at their full size, as one digest per group and table variant, plus the oracle's end-to-end
+``(best_cost, best_solution)``.
 
-    python tests/golden/make_search_fixtures.py --plan 2 --workers 7            # all groups
-    python tests/golden/make_search_fixtures.py --plan 4 --select subset        # listed groups
-    python tests/golden/make_search_fixtures.py --plan 5 --shard 0/4 --out parts  # a quarter of the
-        groups; --merge parts then joins the part files into the fixture
-    python tests/golden/make_search_fixtures.py --plan 4 --skip-covered --split-p 3 --deadline 1100
-        # the groups the fixture lacks, each as three jobs over a share of its p values
+    python tests/golden/make_search_fixtures.py --plan 2 --workers 4 --threads 2
+    python tests/golden/make_search_fixtures.py --plan 2 --sample-size 30      # ..._plan2_s30.json
+    python tests/golden/make_search_fixtures.py --plan 5 --tune-scope "8:64,128"
+        # end-to-end search for tensor-parallel size 8 over G in {64, 128} only (the inter-stage
+        # scan of the whole plan would take the C DP days)
 
 Runs on the CPU only (the oracle never touches the GPU library).  A group is one call of the
-oracle's ``batched_tune_best_latency_for_stage`` with ``sample_size = 1`` (the slot the
-inter-stage DP reads); its four result tables (middle / first / last / single stage), padded to
-the tuner's table shape like ``IntraStageTuner.tune`` pads them
-(mist/analyzer/intra_tuning.py:228-259), are reduced to ``tests.util.table_digest``.  Per-group
-results are kept in ``--cache`` so that an interrupted run resumes and the end-to-end search can
-read the cost tables back.
+oracle's ``batched_tune_best_latency_for_stage``; its four result tables (middle / first / last /
+single stage), padded to the tuner's table shape like ``IntraStageTuner.tune`` pads them
+(mist/analyzer/intra_tuning.py:228-259), are reduced to ``tests.util.table_digest``.  With
+``--inner c`` (default) the loops over (ckpt layers, pre-saved micro-batches) of a group run in
+oracle/stage_loop.c, with ``--inner numpy`` in the numpy statements of oracle/stage.py; both give
+the same tables bit for bit, and a run over a plan whose committed fixture was written the other
+way checks that (every digest the fixture holds must come out again, or the run stops).
+Per-group results are kept in ``--cache`` so that an interrupted run resumes and the end-to-end
+search can read the cost tables back.
+
+End-to-end block: for one sample (``inter-stage`` granularity) the reference's threshold scan
+with the C DP (inter_tuning.py:163-217); for several samples the ``uniform-device-pp-mip``
+granularity (inter_tuning_mip.py, oracle/inter_mip.py).
 
 The GPU tests (tests/test_gpu_golden_tables.py) compute the same digests from the tables the
 HIP kernels produce and compare.
@@ -38,11 +44,13 @@ for p in (REPO, os.path.join(REPO, "tests")):
 
 from util import PLAN_FILES, group_key, load_plan, table_digest  # noqa: E402
 
-# Plan 4 (GPT-22B, 185 661 offload combinations per parallelism row) costs the oracle ~40
-# core-hours as a whole; these groups (8 to 12 core-minutes each) cover its shapes: one and four
-# parallelism rows, single device to 16 nodes, 1 to 48 pre-saved micro-batch values (1 to 3
-# p tiles of the reduce kernel), every tp.
+# Groups for --select subset: a cross-section of a plan's shapes (one and four parallelism rows,
+# single device to all nodes, one to many pre-saved micro-batch values, every tp).
 SUBSETS = {
+    2: [
+        (1, 512, (1, 1)), (1, 16, (4, 8)), (2, 64, (1, 2)), (2, 32, (2, 8)), (4, 256, (1, 4)),
+        (4, 16, (4, 8)), (8, 128, (1, 8)), (8, 16, (4, 8)), (8, 32, (2, 8)), (1, 2, (4, 8)),
+    ],
     4: [
         (1, 512, (1, 1)), (2, 64, (1, 2)), (4, 256, (1, 4)), (8, 128, (1, 8)),
         (1, 1, (16, 8)), (2, 2, (8, 8)), (4, 4, (16, 8)), (1, 4, (2, 8)),
@@ -68,8 +76,22 @@ def group_rows(cfg, tables, tp, G, mesh):
                                constraint_fn=tables.constraint, tp_size=tp).shape[0]
 
 
+# How a group goes through the oracle (set from the command line before the workers fork):
+# the loops over (ckpt layers, pre-saved micro-batches) in C (oracle/stage_loop.c, bit-equal to
+# the numpy statements and ~100 times faster on the large plans) or in numpy, the OpenMP threads
+# of one C call, and the number of alpha samples per cell.
+INNER, THREADS, SAMPLES = "c", 0, 1
+
+
 def cache_path(cache, plan, tp, G, mesh):
-    return os.path.join(cache, f"plan{plan}", f"tp{tp}_G{G}_{mesh[0]}x{mesh[1]}.npz")
+    name = f"plan{plan}" if SAMPLES == 1 else f"plan{plan}_s{SAMPLES}"
+    if INNER == "c-fused":
+        name += "_fused"
+    return os.path.join(cache, name, f"tp{tp}_G{G}_{mesh[0]}x{mesh[1]}.npz")
+
+
+def fixture_name(plan):
+    return f"search_tables_plan{plan}.json" if SAMPLES == 1 else f"search_tables_plan{plan}_s{SAMPLES}.json"
 
 
 def p_values(cfg, G):
@@ -87,7 +109,8 @@ def finish_group(res, cfg, tables, plan, tp, G, mesh, cache, seconds):
     in the cache; returns the fixture record."""
     L = cfg.model.num_hidden_layers
     _, P = p_values(cfg, G)
-    shapes = [(P + 1, L, L + 1, 1), (P + 1, L, L + 1, 1), (L, L + 1, 1), (L + 1, 1)]
+    S = SAMPLES
+    shapes = [(P + 1, L, L + 1, S), (P + 1, L, L + 1, S), (L, L + 1, S), (L + 1, S)]
     record = dict(rows=int(group_rows(cfg, tables, tp, G, mesh)), digest=[], finite=[])
     keep = {}
     for v in range(4):
@@ -125,81 +148,9 @@ def run_group(args):
     t0 = time.time()
     res = batched_tune_best_latency_for_stage(
         tables, cfg, ps, list(range(1, L + 1)), list(range(0, L + 1)),
-        mesh[0], mesh[1], G, tp_size=tp, sample_size=1)
+        mesh[0], mesh[1], G, tp_size=tp, sample_size=SAMPLES, inner=INNER, threads=THREADS)
     return group_key(tp, G, mesh), finish_group(res, cfg, tables, plan, tp, G, mesh, cache,
                                                 time.time() - t0)
-
-
-def part_values(ps, part, n_parts):
-    """The contiguous share ``part`` of the pre-saved micro-batch values ``ps``."""
-    lo, hi = round(part * len(ps) / n_parts), round((part + 1) * len(ps) / n_parts)
-    return ps[lo:hi]
-
-
-def part_path(cache, plan, tp, G, mesh, part, n_parts):
-    return cache_path(cache, plan, tp, G, mesh)[:-4] + f".part{part}of{n_parts}.npz"
-
-
-def run_part(args):
-    """A share of one group's pre-saved micro-batch values through the oracle (--split-p): a
-    group too long for one core within the time there is.  The oracle's loop over p carries one
-    thing from p = 0 to the later values of the same (l, c), the layer mask narrowed by the
-    last-stage variant (batched_module_analyzer.py:3021-3023), so every share starts with
-    p = 0; the other values are independent of each other."""
-    plan, tp, G, mesh, cache, part, n_parts = args
-    key = group_key(tp, G, mesh)
-    path = part_path(cache, plan, tp, G, mesh, part, n_parts)
-    if os.path.exists(cache_path(cache, plan, tp, G, mesh)) or os.path.exists(path):
-        return key, part
-    from oracle.search_space import create_search_space
-    from oracle.stage import batched_stage_analyze
-
-    cfg, tables = load_plan(plan)
-    L = cfg.model.num_hidden_layers
-    ps, _ = p_values(cfg, G)
-    mine = part_values(ps, part, n_parts)
-    t0 = time.time()
-    rows = create_search_space(mesh[0], mesh[1], cfg.training.global_batch_size, G, cfg,
-                               constraint_fn=tables.constraint, tp_size=tp)
-    res = batched_stage_analyze(
-        tables, cfg, mine if mine[0] == 0 else [0] + mine, list(range(1, L + 1)),
-        list(range(0, L + 1)), mesh[0], mesh[1], G, rows, 1)
-    keep = dict(seconds=time.time() - t0)
-    for v in range(4 if part == 0 else 2):  # the p == 0 variants come from the first share
-        keep[f"stable{v}"], keep[f"delta{v}"], keep[f"index{v}"] = res[v][0], res[v][1], res[v][3]
-    os.makedirs(os.path.dirname(path), exist_ok=True)
-    tmp = path + f".tmp{os.getpid()}.npz"
-    np.savez_compressed(tmp, **keep)
-    os.replace(tmp, path)
-    return key, part
-
-
-def merge_parts(plan, tp, G, mesh, cache, n_parts):
-    """Joins the shares of a group written by run_part into the result of one oracle call."""
-    cfg, tables = load_plan(plan)
-    ps, _ = p_values(cfg, G)
-    parts = [np.load(part_path(cache, plan, tp, G, mesh, i, n_parts)) for i in range(n_parts)]
-    res = []
-    for v in range(4):
-        if v >= 2:
-            res.append((parts[0][f"stable{v}"], parts[0][f"delta{v}"], None, parts[0][f"index{v}"]))
-            continue
-        whole = [np.array(parts[-1][f"{name}{v}"]) for name in ("stable", "delta", "index")]
-        assert whole[0].shape[0] == len(ps)
-        for i in range(n_parts - 1):
-            mine = part_values(ps, i, n_parts)
-            for k, name in enumerate(("stable", "delta", "index")):
-                whole[k][mine] = parts[i][f"{name}{v}"][mine]
-        res.append((whole[0], whole[1], None, whole[2]))
-    seconds = sum(float(z["seconds"]) for z in parts)
-    record = finish_group(res, cfg, tables, plan, tp, G, mesh, cache, seconds)
-    for i in range(n_parts):
-        os.remove(part_path(cache, plan, tp, G, mesh, i, n_parts))
-    return record
-
-
-def run_job(args):
-    return run_part(args) if len(args) == 7 else run_group(args)
 
 
 class CachedResults:
@@ -215,7 +166,8 @@ class CachedResults:
 
         L = cfg.model.num_hidden_layers
         P = max_pre_saved_micro_batches(meshes, Gs, L)
-        shapes = [(P + 1, L, L + 1, 1), (P + 1, L, L + 1, 1), (L, L + 1, 1), (L + 1, 1)]
+        S = SAMPLES
+        shapes = [(P + 1, L, L + 1, S), (P + 1, L, L + 1, S), (L, L + 1, S), (L + 1, S)]
         lead = (len(Gs), len(meshes))
         self._stable = [np.full(lead + s, np.inf, dtype=np.float32) for s in shapes]
         self._delta = [np.full(lead + s, np.inf, dtype=np.float32) for s in shapes]
@@ -305,17 +257,21 @@ def scan_one(args):
     return tp, G, out
 
 
-def end_to_end(plan, cache, workers):
+def end_to_end(plan, cache, workers, scope=None):
     """``tune`` of the reference for the inter-stage granularity (tune_one_case.py:186-232,
     inter_tuning.py:63-217) on the cached oracle tables.  The scans of all (tp, G) run in
     parallel without a bound; replaying them in the reference's order (tp after tp with strict
     ``<``; within a tp G after G with the running best as the bound, ``t G >= best -> stop``)
     gives exactly the sequential result, because a bounded scan runs a prefix of the thresholds
-    of the unbounded one."""
+    of the unbounded one.  ``scope = (tp, [G, ...])`` restricts the search to one tensor-parallel
+    size and those gradient-accumulation counts (``inter_stage_tune`` called with that list)."""
     from oracle.inter_dp import get_intra_solution
 
     cfg, tables = load_plan(plan)
-    meshes, Gs, tps = plan_axes(cfg)
+    meshes, Gs_all, tps = plan_axes(cfg)
+    Gs = Gs_all
+    if scope is not None:
+        tps, Gs = [scope[0]], [G for G in Gs_all if G in scope[1]]
     L = cfg.model.num_hidden_layers
     jobs = [(plan, tp, G, cache) for tp in tps for G in Gs]
     with get_context("fork").Pool(workers, maxtasksperchild=1) as pool:
@@ -340,69 +296,59 @@ def end_to_end(plan, cache, workers):
             res = CachedResults(plan, cfg, tables, tp, cache)
             solution = [tp_G, []]
             for i, ((l0, l1), (n, m), ckpt) in enumerate(tp_inter):
-                row = get_intra_solution(res, L, Gs.index(tp_G), len(tp_inter) - i - 1, l0, l1,
+                row = get_intra_solution(res, L, Gs_all.index(tp_G), len(tp_inter) - i - 1, l0, l1,
                                          meshes.index((n, m)), ckpt, 0).tolist()
                 row[:6] = [int(x) for x in row[:6]]
                 solution[1].append([[[l0, l1], [n, m], ckpt, 0], row])
         per_tp[str(tp)] = dict(cost=repr(float(tp_best)), solution=solution, dp_runs_at_or_above_bottleneck=n_dp)
         if tp_best < best_cost:
             best_cost, best_solution = tp_best, solution
-    return dict(granularity="inter-stage", cost=repr(float(best_cost)), solution=best_solution, per_tp=per_tp)
+    out = dict(granularity="inter-stage", cost=repr(float(best_cost)), solution=best_solution, per_tp=per_tp)
+    if scope is not None:
+        out["scope"] = dict(tp=scope[0], Gs=Gs)
+    return out
+
+
+def end_to_end_mip(plan, cache):
+    """``tune`` of the reference for the ``uniform-device-pp-mip`` granularity
+    (tune_one_case.py:360-402) on the cached oracle tables with all their samples: per
+    tensor-parallel size the stage assignment of oracle/inter_mip.py, first best wins."""
+    from oracle.inter_mip import inter_stage_tune
+
+    cfg, tables = load_plan(plan, tuning__tuning_granularity="uniform-device-pp-mip",
+                            tuning__sample_size=SAMPLES)
+    meshes, Gs, tps = plan_axes(cfg)
+    hw, L = cfg.hardware, cfg.model.num_hidden_layers
+    best_cost, best_solution, per_tp = float("inf"), None, {}
+    for tp in tps:
+        res = CachedResults(plan, cfg, tables, tp, cache)
+        cost, sol = inter_stage_tune(L, hw.num_nodes, hw.num_gpus_per_node, meshes, Gs, res, cfg)
+        sol = json.loads(json.dumps(sol, default=lambda o: o.item()))
+        per_tp[str(tp)] = dict(cost=repr(float(cost)), solution=sol)
+        if cost < best_cost:
+            best_cost, best_solution = cost, sol
+    return dict(granularity="uniform-device-pp-mip", sample_size=SAMPLES, cost=repr(float(best_cost)),
+                solution=best_solution, per_tp=per_tp)
 
 
 def main():
+    global INNER, THREADS, SAMPLES
     ap = argparse.ArgumentParser()
     ap.add_argument("--plan", type=int, required=True)
     ap.add_argument("--select", default="all", choices=["all", "subset"])
-    ap.add_argument("--workers", type=int, default=4)
+    ap.add_argument("--sample-size", type=int, default=1, help="alpha samples per cell (1: the slot the DP reads)")
+    ap.add_argument("--inner", default="c", choices=["c", "numpy", "c-fused"],
+                    help="c-fused: the argmin objective r x + y as one fused multiply-add (what numba's "
+                    "fastmath permits); compares with the committed fixture and writes nothing")
+    ap.add_argument("--workers", type=int, default=4, help="groups in flight (processes)")
+    ap.add_argument("--threads", type=int, default=2, help="OpenMP threads of one group's C loops")
     ap.add_argument("--cache", default="/tmp/mist_oracle_cache")
     ap.add_argument("--no-tune", action="store_true", help="skip the end-to-end search")
-    ap.add_argument("--shard", default="0/1", help="i/n: only every n-th group, starting at the i-th")
-    ap.add_argument("--out", default=HERE, help="directory the fixture is written to")
-    ap.add_argument("--merge", default=None, help="join the part files of this directory (and the groups "
-                    "of the committed fixture of a partly covered plan) and exit")
-    ap.add_argument("--max-work", type=int, default=0,
-                    help="leave out groups with more than this many rows x pre-saved micro-batch values "
-                    "(one group runs on one core; 0 = no bound)")
-    ap.add_argument("--skip-covered", action="store_true", help="leave out the groups the committed fixture holds")
-    ap.add_argument("--split-p", type=int, default=1,
-                    help="run every group as this many jobs, each with a share of the pre-saved "
-                    "micro-batch values (for groups too long for one core within --deadline)")
-    ap.add_argument("--deadline", type=float, default=0.0,
-                    help="seconds after which the run stops and keeps what it has (0 = none)")
+    ap.add_argument("--tune-scope", default=None,
+                    help="'tp:G,G,...': end-to-end search over this tensor-parallel size and these "
+                    "gradient-accumulation counts only")
     a = ap.parse_args()
-    if a.merge:
-        import glob
-
-        parts = sorted(glob.glob(os.path.join(a.merge, f"search_tables_plan{a.plan}.part*.json")))
-        whole = os.path.join(a.merge, f"search_tables_plan{a.plan}.json")  # a run without --shard
-        if os.path.exists(whole) and os.path.abspath(a.merge) != os.path.abspath(HERE):
-            parts.append(whole)
-        out, have = None, []
-        for p in parts:
-            with open(p) as f:
-                d = json.load(f)
-            have.append(d["select"])
-            if out is None:
-                out = d
-            else:
-                out["groups"].update(d["groups"])
-        path = os.path.join(HERE, f"search_tables_plan{a.plan}.json")
-        if os.path.exists(path):  # a partly covered plan grows: keep what the fixture already holds
-            with open(path) as f:
-                old = json.load(f)
-            if old["select"] != "all" and "tune" not in old:
-                have.insert(0, old["select"])
-                for k, v in old["groups"].items():
-                    out["groups"].setdefault(k, v)
-        n = int(parts[0].rsplit("of", 1)[1].split(".")[0]) if "of" in os.path.basename(parts[0]) else 1
-        bounded = any("at most" in h for h in have)
-        out["select"] = "all" if len(parts) == n and not bounded and len(have) == len(parts) else "; ".join(have)
-        with open(path, "w") as f:
-            json.dump(out, f, indent=1, sort_keys=True)
-            f.write("\n")
-        print("wrote", path, len(out["groups"]), "groups,", out["select"])
-        return
+    INNER, THREADS, SAMPLES = a.inner, a.threads, a.sample_size
     cfg, tables = load_plan(a.plan)
     meshes, Gs, tps = plan_axes(cfg)
     if a.select == "all":
@@ -421,14 +367,11 @@ def main():
         if n > 0:
             jobs.append((n * min(G, cfg.model.num_hidden_layers), (a.plan, tp, G, tuple(mesh), a.cache)))
     jobs.sort(key=lambda j: -j[0])  # long groups first
-    if a.max_work > 0:
-        jobs = [j for j in jobs if j[0] <= a.max_work]
-    if a.skip_covered:
-        with open(os.path.join(HERE, f"search_tables_plan{a.plan}.json")) as f:
-            covered = set(json.load(f)["groups"])
-        jobs = [j for j in jobs if group_key(j[1][1], j[1][2], j[1][3]) not in covered]
-    shard, n_shards = (int(x) for x in a.shard.split("/"))
-    jobs = jobs[shard::n_shards]
+    path = os.path.join(HERE, fixture_name(a.plan))
+    old = {}
+    if os.path.exists(path):
+        with open(path) as f:
+            old = json.load(f)
     groups = {}
     t0 = time.time()
     import threading
@@ -439,74 +382,48 @@ def main():
             print(f"[{time.time() - t0:7.0f}s] ... {len(groups)}/{len(jobs)} groups done", flush=True)
 
     threading.Thread(target=heartbeat, daemon=True).start()
-    select = a.select if n_shards == 1 else f"shard {shard} of {n_shards} (groups by size, every {n_shards}th)"
-    if a.max_work > 0:
-        select += f", groups of at most {a.max_work} rows x pre-saved micro-batch values"
-    if a.skip_covered:
-        select += ", without those already covered"
-    part = "" if n_shards == 1 else f".part{shard}of{n_shards}"
-    os.makedirs(a.out, exist_ok=True)
-    path = os.path.join(a.out, f"search_tables_plan{a.plan}{part}.json")
-
-    def write(out):
-        with open(path + ".tmp", "w") as f:
-            json.dump(out, f, indent=1, sort_keys=True)
-            f.write("\n")
-        os.replace(path + ".tmp", path)
-
-    def fixture():
-        return dict(
-            plan=PLAN_FILES[a.plan - 1], sample_size=1, select=select,
-            made_by="tests/golden/make_search_fixtures.py (CPU oracle)",
-            groups={k: dict(rows=groups[k]["rows"], finite=groups[k]["finite"], digest=groups[k]["digest"])
-                    for k in sorted(groups)},
-        )
-
-    tasks = [j[1] for j in jobs]
-    n_shares = {}
-    if a.split_p > 1:  # never more shares than a group has values of p
-        tasks = []
-        for j in jobs:
-            k = min(a.split_p, len(p_values(cfg, j[1][2])[0]))
-            n_shares[group_key(j[1][1], j[1][2], j[1][3])] = k
-            tasks += [j[1] + (part, k) for part in range(k)]
-        select += f", up to {a.split_p} jobs per group"
-    parts_done = {}
+    reproduced, differing = 0, []
     with get_context("fork").Pool(a.workers, maxtasksperchild=1) as pool:
-        results = pool.imap_unordered(run_job, tasks)
-        for n in range(len(tasks)):
-            try:
-                key, rec = results.next(timeout=max(a.deadline - (time.time() - t0), 1.0) if a.deadline else None)
-            except Exception as e:  # multiprocessing.TimeoutError: the deadline has passed
-                if type(e).__name__ != "TimeoutError":
-                    raise
-                print(f"[{time.time() - t0:7.0f}s] deadline: {len(groups)} of {len(jobs)} groups kept", flush=True)
-                select += f" (stopped after {len(groups)} of {len(jobs)})"
-                write(fixture())
-                pool.terminate()  # the unfinished groups are given up
-                print("wrote", path, flush=True)
-                return
-            if a.split_p > 1:  # rec = the share that is done; the last one completes the group
-                parts_done.setdefault(key, set()).add(rec)
-                print(f"[{time.time() - t0:7.0f}s] {key} share {rec + 1} of {n_shares[key]}", flush=True)
-                if len(parts_done[key]) < n_shares[key]:
-                    continue
-                job = next(j[1] for j in jobs if group_key(j[1][1], j[1][2], j[1][3]) == key)
-                final = cache_path(job[4], job[0], job[1], job[2], job[3])
-                if os.path.exists(final):
-                    with np.load(final) as z:
-                        rec = json.loads(str(z["record"]))
-                else:
-                    rec = merge_parts(job[0], job[1], job[2], job[3], job[4], n_shares[key])
+        for key, rec in pool.imap_unordered(run_group, [j[1] for j in jobs]):
             groups[key] = rec
+            was = old.get("groups", {}).get(key)
+            if was is not None:  # written earlier, possibly by the other form of the loops
+                same = was["digest"] == rec["digest"] and was["finite"] == rec["finite"]
+                if INNER == "c-fused" and not same:
+                    differing.append(key)
+                else:
+                    assert same, f"{key}: the committed fixture holds other tables: {was} vs {rec}"
+                    reproduced += 1
             print(f"[{time.time() - t0:7.0f}s] {len(groups)}/{len(jobs)} {key} rows={rec['rows']} "
                   f"finite={rec['finite']} ({rec['oracle_seconds']} s)", flush=True)
-            write(fixture())
-    out = fixture()
-    if a.select == "all" and not a.no_tune and n_shards == 1:
-        out["tune"] = end_to_end(a.plan, a.cache, a.workers)
+    print(f"{reproduced} groups of the committed fixture reproduced", flush=True)
+    if INNER == "c-fused":
+        print(f"fused objective: {len(differing)} of {len(groups)} groups pick other winners: {differing}")
+        return
+    out = dict(
+        plan=PLAN_FILES[a.plan - 1], sample_size=SAMPLES, select=a.select,
+        made_by=f"tests/golden/make_search_fixtures.py (CPU oracle, --inner {INNER})",
+        groups={k: dict(rows=groups[k]["rows"], finite=groups[k]["finite"], digest=groups[k]["digest"])
+                for k in sorted(groups)},
+    )
+    for k in ("tune", "tune_scoped"):  # kept unless this run writes them again
+        if k in old and old.get("groups") == out["groups"]:
+            out[k] = old[k]
+    if a.tune_scope:
+        tp, gs = a.tune_scope.split(":")
+        out["tune_scoped"] = end_to_end(a.plan, a.cache, a.workers * max(a.threads, 1),
+                                        scope=(int(tp), [int(g) for g in gs.split(",")]))
+        print("tune (scoped):", out["tune_scoped"]["cost"], out["tune_scoped"]["solution"], flush=True)
+    elif a.select == "all" and not a.no_tune:
+        if SAMPLES == 1:
+            out["tune"] = end_to_end(a.plan, a.cache, a.workers * max(a.threads, 1))
+        else:
+            out["tune"] = end_to_end_mip(a.plan, a.cache)
         print("tune:", out["tune"]["cost"], out["tune"]["solution"], flush=True)
-    write(out)
+    with open(path + ".tmp", "w") as f:
+        json.dump(out, f, indent=1, sort_keys=True)
+        f.write("\n")
+    os.replace(path + ".tmp", path)
     print("wrote", path, flush=True)
 
 

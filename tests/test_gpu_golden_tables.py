@@ -21,11 +21,13 @@ from util import group_key, load_plan, table_digest
 pytestmark = pytest.mark.gpu
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-FIXTURES = sorted(glob.glob(os.path.join(HERE, "golden", "search_tables_plan*.json")))
+FIXTURES = sorted(glob.glob(os.path.join(HERE, "golden", "search_tables_plan?.json")))
+# the same for every alpha sample of a cell (the tables the uniform-device-pp-mip granularity reads)
+SAMPLED_FIXTURES = sorted(glob.glob(os.path.join(HERE, "golden", "search_tables_plan?_s*.json")))
 
 
 def _plan_of(path):
-    return int(re.search(r"plan(\d+)\.json$", path).group(1))
+    return int(re.search(r"plan(\d+)(_s\d+)?\.json$", path).group(1))
 
 
 def _listify(x):
@@ -35,6 +37,7 @@ def _listify(x):
 
 def test_fixtures_cover_every_benchmark_plan():
     assert {_plan_of(p) for p in FIXTURES} == {1, 2, 3, 4, 5}
+    assert {_plan_of(p) for p in SAMPLED_FIXTURES} >= {1, 2}
 
 
 @pytest.mark.parametrize("plan", [1, 2, 3, 4, 5])
@@ -111,6 +114,68 @@ def test_tables_and_tune_equal_the_oracle_fixture(path, exhaustive):
         assert cost == float(want["cost"]), (tp, cost, want["cost"])
         assert _listify(solution) == want["solution"], tp
     cost, solution = search.run()
+    assert cost == float(fixture["tune"]["cost"])
+    assert _listify(solution) == fixture["tune"]["solution"]
+    assert solution is not None
+
+
+@pytest.mark.parametrize("exhaustive", [False, True], ids=["pruned", "exhaustive"])
+@pytest.mark.parametrize("path", SAMPLED_FIXTURES, ids=lambda p: os.path.basename(p)[14:-5])
+def test_sampled_tables_and_mip_tune_equal_the_oracle_fixture(path, exhaustive):
+    """All alpha samples of every cell (mist/utils/pareto.py:124-144 with sample_size = 30, the
+    reference's default) for every group the fixture holds, from the batched multi-sample launches
+    (scout passes of 16 samples per launch, slabs behind one another) and from the kernel that
+    evaluates every cell; then the ``uniform-device-pp-mip`` search on those tables: the oracle's
+    cost and strategy per tensor-parallel size and overall."""
+    from mist_amd.inter_tuning_mip import inter_stage_tune as inter_stage_tune_mip
+    from mist_amd.intra_tuning import IntraStageTuner
+    from mist_amd.search_space import _get_device_mesh_candidates, _get_grad_accumu_steps_candidates
+    from mist_amd.tune_one_case import tp_candidates, tune
+
+    with open(path) as f:
+        fixture = json.load(f)
+    plan, S = _plan_of(path), fixture["sample_size"]
+    assert S > 1
+    cfg, tables = load_plan(plan, tuning__tuning_granularity="uniform-device-pp-mip", tuning__sample_size=S)
+    hw, L = cfg.hardware, cfg.model.num_hidden_layers
+    meshes = _get_device_mesh_candidates(hw.num_nodes, hw.num_gpus_per_node, contiguous_inter_node=False)
+    Gs = _get_grad_accumu_steps_candidates(cfg.training.global_batch_size)
+    tps = tp_candidates(cfg)
+    tuner = IntraStageTuner(tables, L, meshes, Gs, tps, cfg, sample_size=S, exhaustive=exhaustive)
+    results = tuner.tune_all()
+    suffix = ("base", "with_pre", "with_post", "no_pp")
+    bad, n_groups = [], 0
+    for t, tp in enumerate(tps):
+        res = results[t]
+        host = [(res._fetch("index", v), res._fetch("stable", v), res._fetch("delta", v)) for v in range(4)]
+        for g, G in enumerate(Gs):
+            for q, mesh in enumerate(meshes):
+                want = fixture["groups"].get(group_key(tp, G, mesh))
+                if want is None:
+                    continue
+                n_groups += 1
+                for v in range(4):
+                    index, stable, delta = (a[g, q] for a in host[v])
+                    assert index.shape[-1] == S
+                    if int((index >= 0).sum()) != want["finite"][v] or \
+                            table_digest(index, stable, delta) != want["digest"][v]:
+                        bad.append((group_key(tp, G, mesh), suffix[v], int((index >= 0).sum()), want["finite"][v]))
+        res._host.clear()
+        del host
+    assert n_groups == len(fixture["groups"])
+    assert not bad, f"{len(bad)} of {4 * n_groups} tables differ from the oracle: {bad[:8]}"
+    if "tune" not in fixture:
+        return
+    assert fixture["tune"]["granularity"] == "uniform-device-pp-mip"
+    for tp, res in zip(tps, results):
+        cost, solution = inter_stage_tune_mip(L, hw.num_nodes, hw.num_gpus_per_node, meshes, Gs, res, cfg)
+        want = fixture["tune"]["per_tp"][str(tp)]
+        assert cost == float(want["cost"]), (tp, cost, want["cost"])
+        assert _listify(solution) == want["solution"], tp
+    del results, tuner
+    if exhaustive:
+        return
+    cost, solution = tune(cfg)
     assert cost == float(fixture["tune"]["cost"])
     assert _listify(solution) == fixture["tune"]["solution"]
     assert solution is not None

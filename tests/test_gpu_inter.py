@@ -68,6 +68,108 @@ def _gpu_dp(meshes, L, D, P1, tabs, tmax, want_argmin=False, mode=0, relaid=True
     return out + ((arg.cpu().numpy(), path.cpu().numpy()) if want_argmin else ())
 
 
+def _gpu_dp_many(meshes, L, D, P1, tabs_per_g, g_index, tmax, mode, schedule):
+    """``mist_dp_run`` over instances of several gradient-accumulation rows (``tabs_per_g``: one
+    table set per row) with the schedule forced through MIST_DP_FORCE_SCHEDULE ('' = the
+    library's own choice); back-pointers included."""
+    import os
+
+    import torch
+    from mist_amd import _lib
+
+    lib = _lib.load()
+    Q, n_g, n = len(meshes), len(tabs_per_g), len(tmax)
+    shape = np.zeros(1, dtype=_lib.DP_SHAPE_DTYPE)
+    shape["num_layers"], shape["num_devices"], shape["num_mesh"], shape["p_dim"] = L, D, Q, P1
+    S = min(max(a * b for a, b in meshes), L) // 2
+    shape["max_stages"] = S
+    shape["mesh_n"][0, :Q] = [a for a, _ in meshes]
+    shape["mesh_m"][0, :Q] = [b for _, b in meshes]
+    sp = ctypes.c_void_p(shape.ctypes.data)
+    dev = [torch.from_numpy(np.stack([t[v] for t in tabs_per_g])).cuda() for v in range(4)]
+    dev += [torch.cummin(t, dim=-1).values.contiguous() for t in dev]
+    costs = _lib.DpCosts(*[t.data_ptr() for t in dev])
+    for v in range(4):
+        costs.g_stride[v] = dev[v][0].numel()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    per_g = lib.mist_dp_stage_minima_floats(sp)
+    stage_min = torch.empty(per_g * n_g, dtype=torch.float32).cuda()
+    _lib.check(lib.mist_dp_stage_minima(sp, ctypes.byref(costs), n_g, stage_min.data_ptr(), stream),
+               "mist_dp_stage_minima")
+    costs.stage_min, costs.stage_min_g_stride = stage_min.data_ptr(), per_g
+    d_t = torch.tensor(np.asarray(tmax, dtype=np.float32)).cuda()
+    d_g = torch.tensor(np.asarray(g_index, dtype=np.int32)).cuda()
+    d_s = torch.full((n,), -9, dtype=torch.int32).cuda()
+    d_sum = torch.full((n,), -9.0, dtype=torch.float32).cuda()
+    d_max = torch.full((n,), -9.0, dtype=torch.float32).cuda()
+    scr = torch.empty(max(lib.mist_dp_scratch_floats(sp, n), 1), dtype=torch.float32).cuda()
+    arg = torch.full((n, S + 1, L + 1, D + 1, 4), -1, dtype=torch.int32).cuda()
+    old = os.environ.get("MIST_DP_FORCE_SCHEDULE")
+    os.environ["MIST_DP_FORCE_SCHEDULE"] = schedule
+    try:
+        rc = lib.mist_dp_run(sp, ctypes.byref(costs), d_t.data_ptr(), d_g.data_ptr(), n, mode,
+                             d_s.data_ptr(), d_sum.data_ptr(), d_max.data_ptr(), arg.data_ptr(),
+                             scr.data_ptr(), stream)
+    finally:
+        if old is None:
+            del os.environ["MIST_DP_FORCE_SCHEDULE"]
+        else:
+            os.environ["MIST_DP_FORCE_SCHEDULE"] = old
+    _lib.check(rc, f"mist_dp_run ({schedule or 'auto'})")
+    torch.cuda.synchronize()
+    return d_s.cpu().numpy(), d_sum.cpu().numpy(), d_max.cpu().numpy(), arg.cpu().numpy()
+
+
+@pytest.mark.parametrize(
+    "L,D,meshes,P1,quantum",
+    [
+        (6, 4, [(1, 1), (1, 2), (1, 4)], 3, None),                      # D <= 64: three of a lane's four columns idle
+        (9, 8, [(1, 1), (1, 2), (1, 4), (2, 4)], 5, 0.125),
+        (12, 16, [(1, 1), (1, 2), (1, 4), (1, 8), (2, 8)], 7, 0.0625),
+        (23, 70, [(1, 1), (1, 2), (1, 5), (2, 5), (7, 5), (7, 10)], 12, 0.0625),  # D no multiple of 64
+        (40, 80, [(1, 1), (1, 2), (1, 4), (1, 8), (2, 8), (4, 8), (8, 8)], 21, 0.03125),
+        (79, 33, [(1, k) for k in range(1, 17)], 9, 0.03125),           # Q L = 1264 of at most 1280 row minima per start layer
+        (20, 256, [(1, 1), (1, 8), (4, 8), (32, 8)], 11, 0.125),         # the widest plane the schedule holds
+    ],
+)
+@pytest.mark.parametrize("mode", [0, 1], ids=["threshold", "bottleneck"])
+def test_every_dp_schedule_gives_the_same_states(L, D, meshes, P1, quantum, mode):
+    """The three schedules of ``mist_dp_run`` (one launch per stage count; one workgroup per
+    instance with all planes in LDS; one workgroup per instance with one plane in LDS, which the
+    library itself only picks for the 80-layer, 256-device shape) forced on the same batch of
+    DISTINCT instances - three gradient-accumulation rows with their own tables, a spread of
+    thresholds - must agree on every output incl. all back-pointers; the per-stage-count launches
+    are held against the C oracle in test_dp_kernel_matches_c_oracle."""
+    from mist_amd import _lib
+
+    rng = np.random.default_rng(L * 1000 + D + mode)
+    tabs = [_random_tables(rng, len(meshes), P1, L, quantum=quantum) for _ in range(3)]
+    n = 20
+    tmax = rng.uniform(0.1, 1.1, size=n).astype(np.float32)
+    g_index = rng.integers(0, 3, size=n).astype(np.int32)
+    g_index[:3] = (0, 1, 2)
+    want = _gpu_dp_many(meshes, L, D, P1, tabs, g_index, tmax, mode, "step")
+    assert not np.any(want[0] == -9)
+    if mode == 0:
+        assert (want[0] >= 0).any()
+    else:
+        assert len({float(v) for v in want[1][:3]}) == 3, "instances of different rows must differ"
+    lib = _lib.load()
+    for schedule in ("fused", "plane", ""):
+        try:
+            got = _gpu_dp_many(meshes, L, D, P1, tabs, g_index, tmax, mode, schedule)
+        except _lib.MistLibraryError as e:
+            # the all-planes-in-LDS schedule does not hold the largest shapes
+            assert schedule == "fused" and "forced fused schedule" in str(e), e
+            continue
+        for name, w, g in zip(("best_s", "best_sum", "stage_max", "argmin"), want, got):
+            if name == "stage_max" and mode == 0:
+                ok = np.array_equal(w[want[0] >= 0].view(np.int32), g[want[0] >= 0].view(np.int32))
+            else:
+                ok = np.array_equal(w.view(np.int32), g.view(np.int32))
+            assert ok, (schedule or "auto", name)
+
+
 def _walk(arg, best_s, D):
     """Partition from one instance's back-pointers, as the reference walks them
     (inter_tuning.py:341-355): [(end layer, n, m, ckpt), ...] in pipeline order."""

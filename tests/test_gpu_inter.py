@@ -150,10 +150,7 @@ def test_every_dp_schedule_gives_the_same_states(L, D, meshes, P1, quantum, mode
     g_index[:3] = (0, 1, 2)
     want = _gpu_dp_many(meshes, L, D, P1, tabs, g_index, tmax, mode, "step")
     assert not np.any(want[0] == -9)
-    if mode == 0:
-        assert (want[0] >= 0).any()
-    else:
-        assert len({float(v) for v in want[1][:3]}) == 3, "instances of different rows must differ"
+    assert (want[0] >= 0).any()
     lib = _lib.load()
     for schedule in ("fused", "plane", ""):
         try:

@@ -313,6 +313,72 @@ def test_randomized_plans_match_oracle(seed, monkeypatch):
         _compare(cfg, tables, tp, S=int(rng.choice([1, 1, 3])), require_finite=False)
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_randomized_full_size_plans_pruned_equals_exhaustive(seed):
+    """Seeded random plans at realistic sizes: 12 to 48 layers, 8 to 64 devices, the GPT-7B plan's
+    offload grid (13 431 offload combinations per parallelism row), random link, copy and
+    interference parameters, capacities from "nothing fits" to "everything fits".  Every table of
+    the pruned search (scout pass, stage summaries, sieves, bounds, row chunks) must equal the
+    kernel that evaluates every cell; three groups per plan are also held against the oracle (its
+    C loops).  The first mismatch stops the test and names the plan."""
+    import torch
+
+    from mist_amd.tune_one_case import PreparedSearch
+    from oracle.intra import max_pre_saved_micro_batches
+    from oracle.stage import batched_tune_best_latency_for_stage as oracle_op
+
+    rng = np.random.default_rng(777000 + seed)
+    gg = []
+    for _ in range(16):
+        gg += [float(rng.uniform(8, 500)), float(rng.uniform(2e-6, 8e-5))]
+    nodes, gpn = int(rng.choice([1, 2, 4, 8])), int(rng.choice([2, 4, 8]))
+    L = int(rng.integers(12, 49))
+    overrides = dict(
+        model__num_hidden_layers=L,
+        hardware__gpu_gpu_comm_params=gg,
+        hardware__cpu_gpu_comm_params=[float(rng.uniform(5, 60)), float(rng.uniform(2e-6, 3e-5))],
+        hardware__gpu_cpu_comm_params=[float(rng.uniform(5, 60)), float(rng.uniform(2e-6, 3e-5))],
+        hardware__interference_model_params=[float(x) for x in rng.uniform(1.0, 4.0, size=28)],
+        hardware__memory_capacity=float(np.exp(rng.uniform(np.log(3.0), np.log(300.0)))),
+        hardware__num_nodes=nodes, hardware__num_gpus_per_node=gpn,
+        training__global_batch_size=int(rng.choice([64, 128, 256, 512])),
+        model__use_flash_attn=bool(rng.integers(2)),
+        enable_advanced_opt_in_first_block=bool(rng.integers(2)),
+        tuning__pre_post_strategy=str(rng.choice(["dp", "intra-node-tp-with-ore", "intra-node-tp-without-ore"])),
+        synthetic__seed=int(rng.integers(1 << 20)),
+    )
+    cfg, layer_tables = load_plan(2, **overrides)
+    what = f"seed {seed}: L={L} {nodes}x{gpn} capacity {cfg.hardware.raw_memory_capacity:.1f} GB"
+    tables = []
+    for exhaustive in (False, True):
+        search = PreparedSearch(cfg, exhaustive=exhaustive)
+        results = search.tuner.run_prepared(search.plan, search.dev_plan)
+        tables.append(results)
+    pruned, full = tables[0][0].batch, tables[1][0].batch
+    for v in range(4):
+        assert torch.equal(pruned.index[v], full.index[v]), f"{what}: row indices of variant {v}"
+        assert torch.equal(pruned.stable[v], full.stable[v]), f"{what}: stable costs of variant {v}"
+        assert torch.equal(pruned.delta[v], full.delta[v]), f"{what}: delta costs of variant {v}"
+    # a few groups against the oracle
+    Gs, meshes, tps = search.Gs, search.meshes, search.tuner.tp_sizes
+    P = max_pre_saved_micro_batches(meshes, Gs, L)
+    present = sorted({(int(r["g_index"]), int(r["q_index"])) for r in search.plan["groups"]})
+    assert present, what
+    for k in rng.choice(len(present), size=min(3, len(present)), replace=False):
+        row_g, q = present[int(k)]
+        t, g = divmod(row_g, len(Gs))
+        G, (n, m) = Gs[g], meshes[q]
+        want = oracle_op(layer_tables, cfg, list(range(min(G, L, P + 1))), list(range(1, L + 1)),
+                         list(range(L + 1)), n, m, G, tp_size=tps[t], sample_size=1, inner="c", threads=4)
+        res = tables[0][t]
+        for v in range(4):
+            index = res._fetch("index", v)[g, q]
+            corner = tuple(slice(0, k_) for k_ in want[v][3].shape)
+            assert np.array_equal(index[corner][..., :1], want[v][3]), f"{what}: group {(tps[t], G, (n, m))} variant {v}"
+            assert_same_f64(res._fetch("stable", v)[g, q][corner][..., :1], want[v][0], f"{what} stable {v}")
+            assert_same_f64(res._fetch("delta", v)[g, q][corner][..., :1], want[v][1], f"{what} delta {v}")
+
+
 @pytest.mark.parametrize("G, mesh, tp, p_cands, S", [
     (4, (1, 2), None, range(3), 1),    # tp latches to the first feasible batch size
     (2, (2, 4), 2, range(5), 2),       # more pre-saved micro-batch values than G

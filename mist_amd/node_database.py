@@ -351,21 +351,37 @@ _COUNTERPART = {"reduce_scatter": "all_gather", "all_gather": "reduce_scatter",
 
 
 class GptNodeTemplate:
-    """Operator calls of the three layer kinds of the reference's flash-attention GPT
-    (mist/models/gpt.py with mist/modules/mha.py, mlp.py, fused_dense.py, embedding.py,
+    """Operator calls of the three layer kinds of the reference's decoder models
+    (mist/models/gpt.py, llama.py with mist/modules/mha.py, mlp.py, fused_dense.py, embedding.py,
     losses.py) for per-device batch ``b`` and tensor-parallel size ``tp``.
+
+    ``flash``: the attention core is one ``flash_attn_qkvpacked_func`` call, or - flash attention
+    off, as in the reference's kick-the-tires plan - the calls of ``SelfAttention.forward_fused_softmax``
+    (mist/modules/mha.py:316-391): unbind, the transposes of q / k / v and of the context,
+    ``torch.baddbmm`` into the score buffer, the fused causal softmax, the (identity) attention
+    dropout and ``torch.bmm``.  ``gated``: the MLP is ``ParallelGatedMlp`` with SiLU
+    (mist/modules/mlp.py:67-128: one projection to 2 x ffn, chunk, swiglu, projection back) instead
+    of ``ParallelMLP`` with GELU; ``norm`` "rmsnorm" swaps the norm function (mist/modules/rms_norm.py).
 
     The reference obtains these lists by tracing the model; this template is written from the
     module code and checked against the reference's shipped database, which holds an entry for
-    every call listed here at tp = 1 (the calls the tracer recorded): how often a call occurs
-    in a layer is this module's reading of the code, not something the database can confirm.
+    every call of the GELU / LayerNorm model listed here at tp = 1, with and without flash
+    attention (the calls the tracer recorded): how often a call occurs in a layer is this
+    module's reading of the code, not something the database can confirm.  The shipped database
+    has no gated or RMS-norm model: the operator names of that path (chunk, swiglu, rms_norm)
+    are read from the module code alone.
     """
 
     def __init__(self, hidden: int, heads: int, seq_len: int, vocab: int, ffn: Optional[int] = None,
-                 dtype: str = "torch.float16", layer_norm_epsilon: float = 1e-06):
+                 dtype: str = "torch.float16", layer_norm_epsilon: float = 1e-06, flash: bool = True,
+                 gated: bool = False, norm: str = "layernorm"):
         self.h, self.heads, self.s, self.v = int(hidden), int(heads), int(seq_len), int(vocab)
         self.ffn = int(ffn) if ffn else 4 * self.h
         self.dtype, self.eps = dtype, layer_norm_epsilon
+        self.flash, self.gated = bool(flash), bool(gated)
+        if norm not in ("layernorm", "rmsnorm"):
+            raise ValueError(f"norm: {norm}")
+        self.norm = norm
 
     def _t(self, *shape, grad=True, dtype=None) -> TensorSpec:
         return TensorSpec(shape, dtype or self.dtype, grad)
@@ -377,9 +393,52 @@ class GptNodeTemplate:
             return_residual=False, process_group=group, sequence_parallel=False)
 
     def _norm(self, b) -> NodeKey:
+        if self.norm == "rmsnorm":
+            return NodeKey.function(
+                "mist.modules.rms_norm.rms_norm", x=self._t(b, self.s, self.h),
+                weight=self._t(self.h), epsilon=self.eps)
         return NodeKey.function(
             "mist.modules.layer_norm.layer_norm", x=self._t(b, self.s, self.h),
             weight=self._t(self.h), bias=self._t(self.h), epsilon=self.eps)
+
+    def _attention_core(self, b, tp) -> List[NodeKey]:
+        """The calls between the qkv projection and the output projection."""
+        s, heads, d = self.s, self.heads // tp, self.h // self.heads
+        if self.flash:
+            return [NodeKey.function(
+                "mist.modules.flash_attn.flash_attn_qkvpacked_func",
+                qkv=self._t(b, s, 3, heads, d), dropout_p=0.0, softmax_scale=d ** -0.5, causal=True,
+                window_size=(-1, -1), return_attn_probs=False)]
+        transpose = lambda shape, d0, d1: NodeKey.method(
+            "torch._C._TensorBase.transpose", input=self._t(*shape), dim0=d0, dim1=d1)
+        bh = b * heads
+        return [
+            NodeKey.method("torch._C._TensorBase.unbind", input=self._t(b, s, 3, heads, d), dim=2),
+            transpose((b, s, heads, d), 1, 2),   # q -> (b, heads, t, d)
+            transpose((b, s, heads, d), 1, 2),   # k -> (b, heads, s, d)
+            transpose((b, heads, s, d), 2, 3),   # k -> (b, heads, d, s)
+            NodeKey.function(
+                "torch.baddbmm", input=self._t(bh, s, s, grad=False), batch1=self._t(bh, s, d),
+                batch2=self._t(bh, d, s), alpha=1, beta=0.0, out=None),
+            NodeKey.function(
+                "mist.modules.fused_softmax.scaled_upper_triang_masked_softmax_fn",
+                inputs=self._t(bh, s, s), scale=d ** -0.5),
+            NodeKey.module("torch.nn.modules.linear.Identity", {}, {}, {}, input=self._t(b, heads, s, s)),
+            transpose((b, s, heads, d), 1, 2),   # v -> (b, heads, s, d)
+            NodeKey.function("torch.bmm", input=self._t(bh, s, s), mat2=self._t(bh, s, d), out=None),
+            transpose((b, heads, s, d), 1, 2),   # context -> (b, t, heads, d)
+        ]
+
+    def _mlp(self, b, tp, group) -> List[NodeKey]:
+        s, f = self.s, self.ffn // tp
+        if not self.gated:
+            return [self._dense(b, self.h, f, group),
+                    NodeKey.function("torch._C._nn.gelu", input=self._t(b, s, f), approximate="tanh"),
+                    self._dense(b, f, self.h, None)]
+        return [self._dense(b, self.h, 2 * f, group),
+                NodeKey.method("torch._C._TensorBase.chunk", input=self._t(b, s, 2 * f), chunks=2, dim=-1),
+                NodeKey.function("mist.modules.activations.swiglu", x=self._t(b, s, f), y=self._t(b, s, f)),
+                self._dense(b, f, self.h, None)]
 
     def _dropout(self, b) -> NodeKey:
         return NodeKey.module("torch.nn.modules.dropout.Dropout", {"p": 0.0, "inplace": False}, {}, {},
@@ -409,20 +468,13 @@ class GptNodeTemplate:
                 input=self._t(b, s, grad=False, dtype="torch.int64"))]
         if kind == "block":
             out = [self._dropout(b), self._residual_add(b), self._norm(b),
-                   self._dense(b, h, 3 * h // tp, group),
-                   NodeKey.function(
-                       "mist.modules.flash_attn.flash_attn_qkvpacked_func",
-                       qkv=self._t(b, s, 3, self.heads // tp, head_dim), dropout_p=0.0,
-                       softmax_scale=head_dim ** -0.5, causal=True, window_size=(-1, -1),
-                       return_attn_probs=False),
-                   self._dense(b, h // tp, h, None)]
+                   self._dense(b, h, 3 * h // tp, group)]
+            out += self._attention_core(b, tp)
+            out.append(self._dense(b, h // tp, h, None))
             if tp > 1:
                 out.append(self._all_reduce(b, group))
-            out += [self._dropout(b), self._residual_add(b), self._norm(b),
-                    self._dense(b, h, self.ffn // tp, group),
-                    NodeKey.function("torch._C._nn.gelu", input=self._t(b, s, self.ffn // tp),
-                                     approximate="tanh"),
-                    self._dense(b, self.ffn // tp, h, None)]
+            out += [self._dropout(b), self._residual_add(b), self._norm(b)]
+            out += self._mlp(b, tp, group)
             if tp > 1:
                 out.append(self._all_reduce(b, group))
             return out
@@ -446,7 +498,9 @@ class GptNodeTemplate:
         if kind == "pre":
             return self.v // tp * h
         if kind == "block":
-            return (3 * h * h + h * h + 2 * h * self.ffn) // tp + 4 * h
+            n_fc1 = 2 if self.gated else 1
+            norm_params = 2 * h if self.norm == "rmsnorm" else 4 * h
+            return (3 * h * h + h * h + (n_fc1 + 1) * h * self.ffn) // tp + norm_params
         if kind == "post":
             # the shipped database holds the add of vocab * hidden elements only: the output
             # projection, without the final norm's 2 * hidden parameters
@@ -469,14 +523,19 @@ class DatabaseLayerTables(LayerTables):
         folder = folder or syn.get("node_database")
         if not folder:
             raise ValueError("DatabaseLayerTables needs a database folder (synthetic.node_database)")
-        if not self.flash or self.gated:
-            raise NotImplementedError("the operator template covers flash-attention GPT blocks with a plain MLP")
+        if self.kv_heads != self.heads:
+            raise NotImplementedError(
+                "the operator template covers blocks whose key / value heads equal the query heads "
+                "(the packed qkv projection of mist/modules/mha.py:863-891)")
         self.db = NodeLatencyDB(folder)
         dtype = {"float16": "torch.float16", "half": "torch.float16", "fp16": "torch.float16",
                  "bfloat16": "torch.bfloat16", "bf16": "torch.bfloat16"}.get(
                      str(config.training.params_dtype), "torch.float32")
+        model = config.model
+        norm = "rmsnorm" if str(getattr(model, "normalization", "layernorm")).lower().startswith("rms") else "layernorm"
         self.template = GptNodeTemplate(int(self.h), int(self.heads), int(self.s), int(self.vocab),
-                                        int(self.ffn), dtype)
+                                        int(self.ffn), dtype, flash=bool(self.flash), gated=bool(self.gated),
+                                        norm=norm)
 
     def op_profiles(self, kind: str, b, tp, inter_size, intra_size):
         out = []

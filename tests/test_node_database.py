@@ -112,25 +112,56 @@ def test_tensor_parallel_extras_follow_the_collective_model():
 
 def test_template_calls_are_the_ones_the_reference_recorded():
     """Every call the GPT template lists at tp = 1 has an entry in the shipped database for the
-    four batch sizes the reference profiled, and the block's operators are exactly the shipped
-    operator files minus those of the non-flash attention path and of the other layer kinds."""
+    four batch sizes the reference profiled - with flash attention and without - and the two
+    templates together use every shipped operator file except two that belong to another model
+    implementation (``torch.nn.functional.dropout`` and ``_make_viewless_tensor`` on (b, s, h)
+    tensors: the bias-dropout-add and the layer output of mist/model/transformer.py, which the
+    GPT plans do not instantiate)."""
     db = NodeLatencyDB(FOLDER)
-    t = GptNodeTemplate(2048, 16, 2048, 50304)
-    used = set()
-    for b in (1, 2, 4, 8):
-        for kind in ("pre", "block", "post"):
-            for key in t.nodes(kind, b, 1) + t.grad_accum_nodes(kind, 1):
-                db.profile(key)
-                used.add(key.identifier)
     non_flash = {"torch.baddbmm", "torch.bmm", "torch._C._TensorBase.transpose", "torch._C._TensorBase.unbind",
                  "mist.modules.fused_softmax.scaled_upper_triang_masked_softmax_fn",
-                 "torch.nn.modules.linear.Identity", "torch.nn.functional.dropout",
-                 "mist.utils.memory._make_viewless_tensor"}
-    assert used == set(db.identifiers()) - non_flash
+                 "torch.nn.modules.linear.Identity"}
+    other_model = {"torch.nn.functional.dropout", "mist.utils.memory._make_viewless_tensor"}
+    used = {}
+    for flash in (True, False):
+        t = GptNodeTemplate(2048, 16, 2048, 50304, flash=flash)
+        used[flash] = set()
+        for b in (1, 2, 4, 8):
+            for kind in ("pre", "block", "post"):
+                for key in t.nodes(kind, b, 1) + t.grad_accum_nodes(kind, 1):
+                    db.profile(key)  # raises for a call the reference did not record
+                    used[flash].add(key.identifier)
+    flash_only = {"mist.modules.flash_attn.flash_attn_qkvpacked_func"}
+    assert used[True] == set(db.identifiers()) - non_flash - other_model
+    assert used[False] == set(db.identifiers()) - flash_only - other_model
+    # without flash attention: every shipped entry of the attention-core files is one of the
+    # template's calls (three transposes per batch size, one call each of the others)
+    t = GptNodeTemplate(2048, 16, 2048, 50304, flash=False)
+    emitted = {key.format() for b in (1, 2, 4, 8) for key in t.nodes("block", b, 1)}
+    for identifier in non_flash:
+        assert set(db.entries(identifier)) <= emitted, identifier
     # the gradient-accumulation adds are the two flat-parameter sizes in the database
     assert t.params("pre", 1) == t.params("post", 1) == 103022592 and t.params("block", 1) == 50339840
     with pytest.raises(ValueError):
         t.nodes("block", 1, 3)
+
+
+def test_gated_block_template():
+    """SwiGLU block with RMS norm (LLaMA): one projection to 2 x ffn / tp, chunk, swiglu, the
+    projection back; keys print and parse; parameter count of the flat parameter.  The shipped
+    database holds no such model, so the operator names are this module's reading of
+    mist/modules/mlp.py:115-128 and rms_norm.py:14 (parity unpinned)."""
+    t = GptNodeTemplate(5120, 40, 4096, 32000, ffn=13824, dtype="torch.bfloat16", gated=True, norm="rmsnorm")
+    nodes = t.nodes("block", 2, 4)
+    names = [k.identifier.rsplit(".", 1)[-1] for k in nodes]
+    assert names == ["Dropout", "add", "rms_norm", "fused_dense_func", "flash_attn_qkvpacked_func",
+                     "fused_dense_func", "all_reduce", "Dropout", "add", "rms_norm", "fused_dense_func",
+                     "chunk", "swiglu", "fused_dense_func", "all_reduce"]
+    fc1, fc2 = nodes[10], nodes[13]
+    assert "shape=(6912, 5120)" in fc1.format() and "shape=(5120, 3456)" in fc2.format()
+    for key in nodes:
+        assert NodeKey.parse(key.format()).format() == key.format()
+    assert t.params("block", 1) == 4 * 5120 * 5120 + 3 * 5120 * 13824 + 2 * 5120
 
 
 def test_layer_latency_from_the_database_by_hand():
@@ -175,18 +206,23 @@ def test_plan_selects_the_provider():
     cfg_db, _ = load_plan(1, model__vocab_size=50304, model__use_flash_attn=True, synthetic__node_database=FOLDER)
     assert isinstance(layer_tables_for(cfg_db), DatabaseLayerTables)
     cfg_llama, _ = load_plan(3)
+    assert DatabaseLayerTables(cfg_llama, FOLDER).template.gated
+    cfg_gqa, _ = load_plan(5)  # 8 key / value heads for 64 query heads: not the packed projection
     with pytest.raises(NotImplementedError):
-        DatabaseLayerTables(cfg_llama, FOLDER)
+        DatabaseLayerTables(cfg_gqa, FOLDER)
 
 
 @pytest.mark.gpu
-def test_tune_on_database_latencies_matches_oracle():
+@pytest.mark.parametrize("flash", [True, False], ids=["flash", "no-flash"])
+def test_tune_on_database_latencies_matches_oracle(flash):
     """The search driven by the measured L4 latencies (GPT-1.3B, 2 GPUs, tp = 1 as profiled by
-    the reference) gives the oracle's answer on the same provider."""
+    the reference; without flash attention it is the reference's kick-the-tires plan,
+    benchmark/mist/configs/test-small-base.yaml, and the first benchmark configuration) gives
+    the oracle's answer on the same provider."""
     from mist_amd.tune_one_case import tune
     from oracle.tune import tune as oracle_tune
 
-    cfg, _ = load_plan(1, model__vocab_size=50304, model__use_flash_attn=True, disable_tp_tuning=True,
+    cfg, _ = load_plan(1, model__vocab_size=50304, model__use_flash_attn=flash, disable_tp_tuning=True,
                        synthetic__node_database=FOLDER)
     tables = layer_tables_for(cfg)
     got = tune(cfg)

@@ -218,15 +218,17 @@ int mist_eval_reduce(const MistProblem *problem, const MistGroupDesc *d_groups, 
 /* mist_eval_reduce + mist_finalize for n_samples <= MIST_MAX_SAMPLE_BATCH ratios of the same
  * row terms (reference: the S samples of one compute_indices call, mist/utils/pareto.py:124-144):
  * the scout passes of all samples run as ONE launch (a single one fills a tenth of the GPU), then
- * per sample the main launch seeded from its own scout slabs and the finalize into sample
- * position sample_index[i].  `ratios` and `sample_index` are HOST arrays.
- * d_partial_cost / d_partial_index: [n_blocks + n_samples * n_scout_blocks] slabs. */
+ * the main launches, each seeded from its sample's scout slabs, and the finalize launches into
+ * sample position sample_index[i], `main_batch` samples per launch (1 <= main_batch <= n_samples;
+ * the wavefronts of one sample's tail then run beside the next sample's).  `ratios` and
+ * `sample_index` are HOST arrays.
+ * d_partial_cost / d_partial_index: [main_batch * n_blocks + n_samples * n_scout_blocks] slabs. */
 int mist_eval_reduce_samples(const MistProblem *problem, const MistGroupDesc *d_groups,
                              int n_groups, const int32_t *d_block_prefix, int n_blocks,
                              const int32_t *d_scout_prefix, int n_scout_blocks,
                              const double *d_row_terms, const double *d_stage_floor,
                              const double *ratios, const int32_t *sample_index, int n_samples,
-                             double *d_partial_cost, int32_t *d_partial_index,
+                             int main_batch, double *d_partial_cost, int32_t *d_partial_index,
                              const MistOutTables *tables, void *stream);
 
 /* mist_eval_reduce with every cell evaluated: each (row, layers, ckpt) through the latency and

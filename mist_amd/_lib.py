@@ -131,7 +131,7 @@ _SIGNATURES = {
     "mist_eval_reduce_samples": (
         ctypes.c_int,
         [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, _VP, _VP, _VP,
-         ctypes.c_int, _VP, _VP, ctypes.POINTER(OutTables), _VP],
+         ctypes.c_int, ctypes.c_int, _VP, _VP, ctypes.POINTER(OutTables), _VP],
     ),
     "mist_eval_reduce_exhaustive": (
         ctypes.c_int,

@@ -7,6 +7,7 @@
 // written, use true divisions, and never reassociate.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -1056,6 +1057,10 @@ __device__ __forceinline__ int64_t gathered_position(const MistGroupDesc *g, int
 struct RatioList {
   double r[MIST_MAX_SAMPLE_BATCH];
 };
+// sample position in the output tables of each sample of one finalize launch
+struct SampleSlots {
+  int32_t at[MIST_MAX_SAMPLE_BATCH];
+};
 
 template <bool kPow2G, bool kFirstTile>
 __device__ __forceinline__ void reduce_block(
@@ -1612,15 +1617,16 @@ __global__ __launch_bounds__(MIST_LC_TILE, MIST_REDUCE_MIN_WAVES) void eval_redu
     const MistProblem prob, const MistGroupDesc *__restrict__ groups, int n_groups,
     const int32_t *__restrict__ block_prefix, int n_blocks,
     const int32_t *__restrict__ scout_prefix, int scout, const double *__restrict__ row_terms,
-    const double *__restrict__ stage_floor, const RatioList ratios, int seed_sample,
-    double *__restrict__ partial_cost, int32_t *__restrict__ partial_index) {
+    const double *__restrict__ stage_floor, const RatioList ratios, int first_sample,
+    int64_t scout_base, double *__restrict__ partial_cost, int32_t *__restrict__ partial_index) {
   __shared__ double lds_terms[kStageRows * kLdsRowStride];
   __shared__ double lds_min[kStageFloorPitch];
   __shared__ double lds_pair[MIST_LC_TILE * kPairFields];
   __shared__ int32_t lds_rowpos[kStageRows];
-  // Scout launch: blockIdx.y = sample, its slabs follow those of the samples before it.  Main
-  // launch: one sample, seeded from the scout slabs of sample `seed_sample`.
-  const int sample = scout ? (int)blockIdx.y : 0;
+  // blockIdx.y = sample first_sample + y of the ratio list.  Slabs: the main launch of its y-th
+  // sample writes slabs y * n_blocks + workgroup; the scout slabs of sample s (of the list) are
+  // scout_base + s * n_scout_total + workgroup, and seed the main launch of the same sample.
+  const int sample = first_sample + (int)blockIdx.y;
   const double ratio = ratios.r[sample];
   const int n_scout_total = scout_prefix != nullptr ? scout_prefix[n_groups] : 0;
   const int block = xcd_run_block(blockIdx.x);
@@ -1639,20 +1645,20 @@ __global__ __launch_bounds__(MIST_LC_TILE, MIST_REDUCE_MIN_WAVES) void eval_redu
     tile = local_block / kScoutSplit;
     const int part = local_block % kScoutSplit;  // gathered stages part, part + split, ...
     range = ReduceRange{(int64_t)part * kStageRows, g->n_rows, kScoutSplit, 0, 1};
-    out_slab = (int64_t)n_blocks + (int64_t)sample * n_scout_total + block;
+    out_slab = scout_base + (int64_t)sample * n_scout_total + block;
   } else {
     const int n_tiles = g->n_lc_tiles * g->n_p_tiles;
     const int chunk = local_block / n_tiles;  // the tiles of one chunk are neighbours
     tile = local_block % n_tiles;
     const int64_t row_begin = (int64_t)chunk * g->rows_per_chunk;
     range = ReduceRange{row_begin, min(row_begin + (int64_t)g->rows_per_chunk, g->n_rows), 1, 0, 0};
-    out_slab = block;
+    out_slab = (int64_t)blockIdx.y * n_blocks + block;
     skip_unchanged = chunk > 0;
   }
   const int p_tile = tile % g->n_p_tiles;
   const int lc_tile = tile / g->n_p_tiles;
   const int64_t slab = (int64_t)kSlots * MIST_LC_TILE;
-  const int64_t seed_slab = (int64_t)n_blocks + (int64_t)seed_sample * n_scout_total +
+  const int64_t seed_slab = scout_base + (int64_t)sample * n_scout_total +
                             (seeded ? scout_prefix[gi] + tile * kScoutSplit : 0);
   const double *seed_cost = (!scout && seeded) ? partial_cost + seed_slab * slab : nullptr;
   const int32_t *seed_index = (!scout && seeded) ? partial_index + seed_slab * slab : nullptr;
@@ -1806,12 +1812,12 @@ __global__ __launch_bounds__(MIST_LC_TILE) void eval_reduce_exhaustive_kernel(
 
 // Combines the slabs of the kScoutSplit scout workgroups of every tile into the first of them,
 // so that each chunk of the main launch reads one slab of seeds instead of kScoutSplit.
-// Workgroup = tile; the scout slabs of tile t are n_blocks + t * kScoutSplit + k.
-__global__ __launch_bounds__(256) void merge_scout_kernel(int n_blocks, int n_scout_total,
+// Workgroup = tile; the scout slabs of tile t are scout_base + t * kScoutSplit + k.
+__global__ __launch_bounds__(256) void merge_scout_kernel(int64_t scout_base, int n_scout_total,
                                                           double *__restrict__ partial_cost,
                                                           int32_t *__restrict__ partial_index) {
   const int64_t slab = (int64_t)kSlots * MIST_LC_TILE;
-  const int64_t first = ((int64_t)n_blocks + (int64_t)blockIdx.y * n_scout_total +
+  const int64_t first = (scout_base + (int64_t)blockIdx.y * n_scout_total +
                          (int64_t)blockIdx.x * kScoutSplit) * slab;
   for (int e = threadIdx.x; e < (int)slab; e += blockDim.x) {
     double best = INFINITY;
@@ -1833,12 +1839,17 @@ __global__ __launch_bounds__(256) void finalize_kernel(
     const MistProblem prob, const MistGroupDesc *__restrict__ groups, int n_groups,
     const int32_t *__restrict__ block_prefix, const double *__restrict__ row_terms,
     const double *__restrict__ partial_cost, const int32_t *__restrict__ partial_index,
-    int sample_index, MistOutTables tables) {
+    const SampleSlots samples, int n_blocks, MistOutTables tables) {
   const int L = prob.num_layers;
   const int n_pairs = L * (L + 1) / 2 + L;
   const int gi = blockIdx.z;
   const MistGroupDesc *g = groups + gi;
-  const int pair_idx = blockIdx.x * blockDim.x + threadIdx.x;
+  // blockIdx.x = (sample of the launch, block of 256 pairs); the slabs of the launch's m-th
+  // sample start at slab m * n_blocks
+  const int pair_blocks = (n_pairs + (int)blockDim.x - 1) / (int)blockDim.x;
+  const int m = blockIdx.x / pair_blocks;
+  const int sample_index = samples.at[m];
+  const int pair_idx = (blockIdx.x - m * pair_blocks) * blockDim.x + threadIdx.x;
   // blockIdx.y: 0..p_dim-1 base, p_dim..2*p_dim-1 with_pre, 2*p_dim with_post, 2*p_dim+1 no_pp
   const int P1 = prob.p_dim;
   const int slot = blockIdx.y;
@@ -1863,7 +1874,8 @@ __global__ __launch_bounds__(256) void finalize_kernel(
   else if (variant == 1) kslot = MIST_P_TILE + p % MIST_P_TILE;
   else kslot = 2 * MIST_P_TILE + (variant - 2);
   const int n_tiles = g->n_lc_tiles * g->n_p_tiles;
-  const int64_t first_block = (int64_t)block_prefix[gi] + (lc_tile * g->n_p_tiles + p_tile);
+  const int64_t first_block =
+      (int64_t)m * n_blocks + (int64_t)block_prefix[gi] + (lc_tile * g->n_p_tiles + p_tile);
   double best = INFINITY;
   int32_t best_row = -1;
   for (int ch = 0; ch < g->n_chunks; ++ch) {
@@ -2161,19 +2173,19 @@ int64_t mist_stage_floor_doubles(int64_t total_rows, int n_groups) {
 static int launch_scout(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,
                         const int32_t *d_block_prefix, int n_blocks, const int32_t *scout_prefix,
                         int n_scout_blocks, const double *d_row_terms, const double *d_stage_floor,
-                        const RatioList &ratios, int n_samples, double *d_partial_cost,
-                        int32_t *d_partial_index, void *stream) {
+                        const RatioList &ratios, int n_samples, int64_t scout_base,
+                        double *d_partial_cost, int32_t *d_partial_index, void *stream) {
   if (n_scout_blocks % kScoutSplit != 0)
     return fail(MIST_E_INVALID, "n_scout_blocks %d is not a multiple of the scout split %d",
                 n_scout_blocks, kScoutSplit);
   hipLaunchKernelGGL(eval_reduce_kernel, dim3(xcd_padded_grid(n_scout_blocks), n_samples),
                      dim3(MIST_LC_TILE), 0, (hipStream_t)stream, *problem, d_groups, n_groups,
                      d_block_prefix, n_blocks, scout_prefix, 1, d_row_terms, d_stage_floor, ratios,
-                     0, d_partial_cost, d_partial_index);
+                     0, scout_base, d_partial_cost, d_partial_index);
   MIST_HIP_CHECK(hipGetLastError());
   if (kScoutSplit > 1) {
     hipLaunchKernelGGL(merge_scout_kernel, dim3(n_scout_blocks / kScoutSplit, n_samples), dim3(256),
-                       0, (hipStream_t)stream, n_blocks, n_scout_blocks, d_partial_cost,
+                       0, (hipStream_t)stream, scout_base, n_scout_blocks, d_partial_cost,
                        d_partial_index);
     MIST_HIP_CHECK(hipGetLastError());
   }
@@ -2210,23 +2222,29 @@ int mist_eval_reduce(const MistProblem *problem, const MistGroupDesc *d_groups, 
   ratios.r[0] = ratio;
   if (scout_prefix)
     if (int rc = launch_scout(problem, d_groups, n_groups, d_block_prefix, n_blocks, scout_prefix,
-                              n_scout_blocks, d_row_terms, d_stage_floor, ratios, 1,
+                              n_scout_blocks, d_row_terms, d_stage_floor, ratios, 1, n_blocks,
                               d_partial_cost, d_partial_index, stream))
       return rc;
   hipLaunchKernelGGL(eval_reduce_kernel, dim3(xcd_padded_grid(n_blocks)), dim3(MIST_LC_TILE), 0,
                      (hipStream_t)stream, *problem, d_groups, n_groups, d_block_prefix, n_blocks,
-                     scout_prefix, 0, d_row_terms, d_stage_floor, ratios, 0, d_partial_cost,
-                     d_partial_index);
+                     scout_prefix, 0, d_row_terms, d_stage_floor, ratios, 0, (int64_t)n_blocks,
+                     d_partial_cost, d_partial_index);
   MIST_HIP_CHECK(hipGetLastError());
   return 0;
 }
+
+static int launch_finalize(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,
+                           const int32_t *d_block_prefix, const double *d_row_terms,
+                           const double *d_partial_cost, const int32_t *d_partial_index,
+                           const int32_t *sample_index, int n_samples, int n_blocks,
+                           const MistOutTables *tables, void *stream);
 
 int mist_eval_reduce_samples(const MistProblem *problem, const MistGroupDesc *d_groups,
                              int n_groups, const int32_t *d_block_prefix, int n_blocks,
                              const int32_t *d_scout_prefix, int n_scout_blocks,
                              const double *d_row_terms, const double *d_stage_floor,
                              const double *ratios, const int32_t *sample_index, int n_samples,
-                             double *d_partial_cost, int32_t *d_partial_index,
+                             int main_batch, double *d_partial_cost, int32_t *d_partial_index,
                              const MistOutTables *tables, void *stream) {
   if (int rc = check_reduce_arguments(problem, d_groups, n_groups, d_block_prefix, n_blocks,
                                       d_scout_prefix, n_scout_blocks, d_row_terms, d_stage_floor,
@@ -2235,28 +2253,33 @@ int mist_eval_reduce_samples(const MistProblem *problem, const MistGroupDesc *d_
   if (!ratios || !sample_index || n_samples < 1 || n_samples > MIST_MAX_SAMPLE_BATCH)
     return fail(MIST_E_INVALID, "n_samples %d outside [1, %d] or null sample lists", n_samples,
                 MIST_MAX_SAMPLE_BATCH);
+  if (main_batch < 1 || main_batch > n_samples)
+    return fail(MIST_E_INVALID, "main_batch %d outside [1, n_samples = %d]", main_batch, n_samples);
   RatioList all = {};
   for (int i = 0; i < n_samples; ++i) {
     if (!(ratios[i] >= 0.0)) return fail(MIST_E_INVALID, "ratio %d must be non-negative", i);
     all.r[i] = ratios[i];
   }
   const int32_t *scout_prefix = n_scout_blocks > 0 ? d_scout_prefix : nullptr;
+  const int64_t scout_base = (int64_t)main_batch * n_blocks;
   // the scout passes of all samples in one launch: a single one occupies a tenth of the GPU
   if (scout_prefix)
     if (int rc = launch_scout(problem, d_groups, n_groups, d_block_prefix, n_blocks, scout_prefix,
-                              n_scout_blocks, d_row_terms, d_stage_floor, all, n_samples,
+                              n_scout_blocks, d_row_terms, d_stage_floor, all, n_samples, scout_base,
                               d_partial_cost, d_partial_index, stream))
       return rc;
-  for (int i = 0; i < n_samples; ++i) {
-    RatioList one = {};
-    one.r[0] = ratios[i];
-    hipLaunchKernelGGL(eval_reduce_kernel, dim3(xcd_padded_grid(n_blocks)), dim3(MIST_LC_TILE), 0,
-                       (hipStream_t)stream, *problem, d_groups, n_groups, d_block_prefix, n_blocks,
-                       scout_prefix, 0, d_row_terms, d_stage_floor, one, i, d_partial_cost,
-                       d_partial_index);
+  // main launches and finalize launches of main_batch samples at a time (grid.y = sample): the
+  // tail of one sample's wavefronts runs beside the next sample's
+  for (int first = 0; first < n_samples; first += main_batch) {
+    const int count = std::min(main_batch, n_samples - first);
+    hipLaunchKernelGGL(eval_reduce_kernel, dim3(xcd_padded_grid(n_blocks), count), dim3(MIST_LC_TILE),
+                       0, (hipStream_t)stream, *problem, d_groups, n_groups, d_block_prefix, n_blocks,
+                       scout_prefix, 0, d_row_terms, d_stage_floor, all, first, scout_base,
+                       d_partial_cost, d_partial_index);
     MIST_HIP_CHECK(hipGetLastError());
-    if (int rc = mist_finalize(problem, d_groups, n_groups, d_block_prefix, d_row_terms,
-                               d_partial_cost, d_partial_index, sample_index[i], tables, stream))
+    if (int rc = launch_finalize(problem, d_groups, n_groups, d_block_prefix, d_row_terms,
+                                 d_partial_cost, d_partial_index, sample_index + first, count,
+                                 n_blocks, tables, stream))
       return rc;
   }
   return 0;
@@ -2278,10 +2301,11 @@ int mist_eval_reduce_exhaustive(const MistProblem *problem, const MistGroupDesc 
   return 0;
 }
 
-int mist_finalize(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,
-                  const int32_t *d_block_prefix, const double *d_row_terms,
-                  const double *d_partial_cost, const int32_t *d_partial_index,
-                  int sample_index, const MistOutTables *tables, void *stream) {
+static int launch_finalize(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,
+                           const int32_t *d_block_prefix, const double *d_row_terms,
+                           const double *d_partial_cost, const int32_t *d_partial_index,
+                           const int32_t *sample_index, int n_samples, int n_blocks,
+                           const MistOutTables *tables, void *stream) {
   if (int rc = check_common(problem, d_groups, n_groups)) return rc;
   if (!d_block_prefix || !d_row_terms || !d_partial_cost || !d_partial_index || !tables)
     return fail(MIST_E_INVALID, "null pointer argument");
@@ -2292,16 +2316,28 @@ int mist_finalize(const MistProblem *problem, const MistGroupDesc *d_groups, int
   const int L = prob.num_layers, P1 = prob.p_dim;
   if (L <= 0 || P1 <= 0 || prob.sample_size <= 0)
     return fail(MIST_E_INVALID, "bad problem extents L=%d P+1=%d S=%d", L, P1, prob.sample_size);
-  if (sample_index < 0 || sample_index >= prob.sample_size)
-    return fail(MIST_E_INVALID, "sample_index %d outside [0, %d)", sample_index, prob.sample_size);
+  SampleSlots slots = {};
+  for (int i = 0; i < n_samples; ++i) {
+    if (sample_index[i] < 0 || sample_index[i] >= prob.sample_size)
+      return fail(MIST_E_INVALID, "sample_index %d outside [0, %d)", sample_index[i], prob.sample_size);
+    slots.at[i] = sample_index[i];
+  }
   if (n_groups > 65535) return fail(MIST_E_INVALID, "too many groups for one launch: %d", n_groups);
   const int n_pairs = L * (L + 1) / 2 + L;
-  dim3 grid((n_pairs + 255) / 256, 2 * P1 + 2, n_groups);
+  dim3 grid((n_pairs + 255) / 256 * n_samples, 2 * P1 + 2, n_groups);
   hipLaunchKernelGGL(finalize_kernel, grid, dim3(256), 0, (hipStream_t)stream, prob, d_groups,
-                     n_groups, d_block_prefix, d_row_terms, d_partial_cost, d_partial_index,
-                     sample_index, *tables);
+                     n_groups, d_block_prefix, d_row_terms, d_partial_cost, d_partial_index, slots,
+                     n_blocks, *tables);
   MIST_HIP_CHECK(hipGetLastError());
   return 0;
+}
+
+int mist_finalize(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,
+                  const int32_t *d_block_prefix, const double *d_row_terms,
+                  const double *d_partial_cost, const int32_t *d_partial_index,
+                  int sample_index, const MistOutTables *tables, void *stream) {
+  return launch_finalize(problem, d_groups, n_groups, d_block_prefix, d_row_terms, d_partial_cost,
+                         d_partial_index, &sample_index, 1, 0, tables, stream);
 }
 
 // Second stream and events of mist_intra_stage_eval, one set per device, kept for the life of
@@ -2368,7 +2404,7 @@ int mist_intra_stage_eval(const MistProblem *problem, const MistGroupDesc *d_gro
     ratios.r[0] = ratio;
     if (int rc = launch_scout(problem, d_groups, n_groups, d_reduce_block_prefix, n_reduce_blocks,
                               d_scout_prefix, n_scout_blocks, d_row_terms, d_stage_floor, ratios, 1,
-                              d_partial_cost, d_partial_index, os->side))
+                              n_reduce_blocks, d_partial_cost, d_partial_index, os->side))
       return rc;
     MIST_HIP_CHECK(hipEventRecord(os->scout_done, os->side));
     bool from_keys = false;
@@ -2387,7 +2423,7 @@ int mist_intra_stage_eval(const MistProblem *problem, const MistGroupDesc *d_gro
     hipLaunchKernelGGL(eval_reduce_kernel, dim3(xcd_padded_grid(n_reduce_blocks)), dim3(MIST_LC_TILE),
                        0, main_stream, *problem, d_groups, n_groups, d_reduce_block_prefix,
                        n_reduce_blocks, d_scout_prefix, 0, d_row_terms, d_stage_floor, ratios, 0,
-                       d_partial_cost, d_partial_index);
+                       (int64_t)n_reduce_blocks, d_partial_cost, d_partial_index);
     MIST_HIP_CHECK(hipGetLastError());
     return mist_finalize(problem, d_groups, n_groups, d_reduce_block_prefix, d_row_terms,
                          d_partial_cost, d_partial_index, sample_index, tables, stream);

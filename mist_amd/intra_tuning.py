@@ -45,6 +45,9 @@ SCOUT_TIGHT_PAIRS = 3
 # the bound is a batch of its own).  GPT-7B (0.88 GB) and LLaMA-13B (1.4 GB) are one batch,
 # GPT-22B (18.4 GB of row terms) ten; with more than one batch two such workspaces alternate.
 ROW_TERMS_BUDGET_BYTES = 2 << 30
+# Partial-minima slabs the main launches of a multi-sample call may hold at once: samples in
+# flight = this / (workgroups of the launch x 26 KB); GPT-7B (63 232 workgroups): 4.
+MAIN_BATCH_SLAB_BYTES = 8 << 30
 
 
 _SIDE_STREAMS: Dict[str, "torch.cuda.Stream"] = {}
@@ -409,9 +412,15 @@ class IntraStageTuner:
         max_rows = max([b["total_rows"] for b in batches], default=0)
         max_groups = max([b["n_groups"] for b in batches], default=0)
         max_keys = max([b["total_keys"] for b in batches], default=0)
-        # several samples share one scout launch: their scout slabs lie behind one another
+        # several samples share one scout launch: their scout slabs lie behind one another; the
+        # main launches take as many samples at a time as their slabs (26 KB per workgroup and
+        # sample, written only where a chunk changes a minimum) fit MAIN_BATCH_SLAB_BYTES
         self._sample_batch = min(len(self.sample_slots), _lib.MAX_SAMPLE_BATCH)
-        n_slabs = max([b["n_reduce_blocks"] + self._sample_batch * b["n_scout_blocks"] for b in batches] + [1])
+        slab_bytes = _lib.SLOTS * _lib.LC_TILE * 12
+        most = max([b["n_reduce_blocks"] for b in batches] + [1])
+        self._main_batch = int(max(1, min(self._sample_batch, MAIN_BATCH_SLAB_BYTES // (most * slab_bytes))))
+        n_slabs = max([self._main_batch * b["n_reduce_blocks"] + self._sample_batch * b["n_scout_blocks"]
+                       for b in batches] + [1])
         def workspace():
             return dict(
                 row_terms=torch.empty(max(max_rows, 1) * _lib.ROW_TERMS, dtype=torch.float64, device=dev),
@@ -498,7 +507,8 @@ class IntraStageTuner:
                         d["n_reduce_blocks"], _ptr(d["scout_prefix"]), d["n_scout_blocks"],
                         _ptr(w["row_terms"]), _ptr(w["stage_floor"]),
                         ctypes.c_void_p(batch_ratios.ctypes.data), ctypes.c_void_p(slots.ctypes.data),
-                        len(slots), _ptr(w["partial_cost"]), _ptr(w["partial_index"]),
+                        len(slots), min(self._main_batch, len(slots)), _ptr(w["partial_cost"]),
+                        _ptr(w["partial_index"]),
                         ctypes.byref(out), stream)
                     _lib.check(rc, "mist_eval_reduce_samples")
                 continue

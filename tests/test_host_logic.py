@@ -295,10 +295,11 @@ def test_argument_checks_reject_before_any_launch():
     slots = np.arange(3, dtype=np.int32)
     rp, sp_ = ctypes.c_void_p(ratios.ctypes.data), ctypes.c_void_p(slots.ctypes.data)
     some_tables = _lib.OutTables()
-    samples = lambda n, r=rp: lib.mist_eval_reduce_samples(
-        pp, fake, 1, fake, 1, None, 0, fake, fake, r, sp_, n, fake, fake, ctypes.byref(some_tables), None)
+    samples = lambda n, r=rp, batch=1: lib.mist_eval_reduce_samples(
+        pp, fake, 1, fake, 1, None, 0, fake, fake, r, sp_, n, batch, fake, fake, ctypes.byref(some_tables), None)
     assert samples(0) == -1 and samples(_lib.MAX_SAMPLE_BATCH + 1) == -1 and samples(2, None) == -1
     assert samples(3) == -1 and b"ratio 2" in lib.mist_last_error()
+    assert samples(2, batch=0) == -1 and samples(2, batch=3) == -1 and b"main_batch" in lib.mist_last_error()
     tabs = _lib.OutTables()
     assert lib.mist_finalize(pp, fake, 1, fake, fake, fake, fake, 0, ctypes.byref(tabs), None) == -1
     shape = np.zeros(1, dtype=_lib.DP_SHAPE_DTYPE)

@@ -19,7 +19,7 @@ import torch
 from . import _lib
 from .config import MistConfig
 from .layer_tables import LayerTables
-from .search_space import SearchSpace, create_search_space_for_a_block_layer
+from .search_space import SearchSpace, SearchSpaceFactory, create_search_space_for_a_block_layer
 from .stage_inputs import GroupInputBuilder, make_problem
 
 SAMPLE_SIZE = 30  # reference default (batched_module_analyzer.py:67)
@@ -260,13 +260,12 @@ class IntraStageTuner:
         builder = GroupInputBuilder(cfg, self.layer_tables)
         spaces: Dict[Tuple[int, int, int], SearchSpace] = {}
         pending = []
+        factory = SearchSpaceFactory(cfg, self.layer_tables.constraint)
+        B = cfg.training.global_batch_size
         for t, tp_size in enumerate(self.tp_sizes):
             for g, G in enumerate(Gs):
                 for q, (n, m) in enumerate(Q):
-                    space = create_search_space_for_a_block_layer(
-                        n, m, cfg.training.global_batch_size, G, cfg,
-                        constraint_fn=self.layer_tables.constraint, tp_size=tp_size,
-                    )
+                    space = factory.make(n, m, B, G, tp_size)
                     spaces[(t, g, q)] = space
                     if space.n_rows == 0:
                         continue  # the reference returns all-inf tables for an empty space (:648-666)
@@ -277,8 +276,7 @@ class IntraStageTuner:
                         num_p = P + 1
                     pending.append((t * len(Gs) + g, q, n, m, G, num_p, space))
         groups = np.zeros(len(pending), dtype=_lib.GROUP_DTYPE)
-        for i, (g, q, n, m, G, num_p, space) in enumerate(pending):
-            builder.fill(groups[i], space, g, q, n, m, G, num_p)
+        builder.fill_many(groups, pending)
         builder.validate(groups)
 
         n_pairs = L * (L + 1) // 2 + L

@@ -108,6 +108,69 @@ def _valid_pairs(wo: Tuple[float, ...], go: Tuple[float, ...]):
     return tuple(pair_wo), tuple(pair_go)
 
 
+class SearchSpaceFactory:
+    """``create_search_space_for_a_block_layer`` for many groups of one configuration: what only
+    depends on the configuration (ratio lists, valid pairs, flags) is read once."""
+
+    def __init__(self, config: MistConfig, constraint_fn: Optional[Callable[[int, int], bool]] = None):
+        tuning = config.tuning
+        self.batch_sizes = tuple(tuning.batch_size_candidates)
+        self.zero_2_and_3 = bool(tuning.zero_2_and_3_enabled)
+        self.flag_choices = tuple(tuning.zero_flag_choices)
+        self.disable_tp = bool(getattr(config, "disable_tp_tuning", False))
+        self.constraint_fn = constraint_fn
+        self.lists = _offload_lists(
+            bool(tuning.state_offloading_enabled), bool(tuning.activation_offloading_enabled),
+            tuple(tuning.offloading_ratio_candidates), tuple(tuning.sparse_offloading_ratio_candidates),
+            bool(getattr(config, "disable_wo_tuning", False)), bool(getattr(config, "disable_go_tuning", False)),
+            bool(getattr(config, "disable_oo_tuning", False)),
+            *(getattr(config, f"fixed_{k}_ratio", None) for k in ("wo", "go", "oo", "ao")),
+        )
+        self._constraint = {}
+        self._empty = np.zeros((0, 6), dtype=np.float64)
+
+    def _allowed(self, batch_size: int, tp_size: int) -> bool:
+        key = (batch_size, tp_size)
+        if key not in self._constraint:
+            self._constraint[key] = bool(self.constraint_fn(batch_size, tp_size))
+        return self._constraint[key]
+
+    def make(self, num_nodes: int, num_gpus_per_node: int, global_batch_size: int,
+             gradient_accumulation_steps: int, tp_size: Optional[int] = None) -> SearchSpace:
+        """Reference: batched_module_analyzer.py:417-536 (same filters, same order)."""
+        num_gpus = num_nodes * num_gpus_per_node
+        per_micro_batch = global_batch_size // gradient_accumulation_steps
+        par = []
+        for batch_size in self.batch_sizes:
+            if batch_size > per_micro_batch or per_micro_batch % batch_size != 0:
+                continue
+            dp_size = per_micro_batch // batch_size
+            if dp_size > num_gpus or num_gpus % dp_size != 0:
+                continue
+            curr_tp_size = num_gpus // dp_size
+            if self.constraint_fn is not None and not self._allowed(batch_size, curr_tp_size):
+                continue
+            # The tp size latches to the first feasible batch size when the caller gave none.
+            tp_size = curr_tp_size if tp_size is None else tp_size
+            if tp_size != curr_tp_size:
+                continue
+            if tp_size > num_gpus_per_node:
+                continue
+            if self.disable_tp and tp_size > 1:
+                continue
+            if dp_size == 1 or not self.zero_2_and_3:
+                flag_choices: Sequence[Tuple[int, int, int]] = ((0, 0, 1),)
+            else:
+                flag_choices = self.flag_choices
+            for wre, gre, ore in flag_choices:
+                par.append((batch_size, dp_size, tp_size, wre, gre, ore))
+        par_np = np.array(par, dtype=np.float64).reshape(-1, 6) if par else self._empty
+        if par_np.shape[0] > MAX_PAR:
+            raise ValueError(f"{par_np.shape[0]} parallelism rows; at most {MAX_PAR} are supported")
+        wo, go, oo, ao, pair_wo, pair_go = self.lists
+        return SearchSpace(par=par_np, wo=wo, go=go, oo=oo, ao=ao, pair_wo=pair_wo, pair_go=pair_go)
+
+
 def create_search_space_for_a_block_layer(
     num_nodes: int,
     num_gpus_per_node: int,
@@ -118,46 +181,8 @@ def create_search_space_for_a_block_layer(
     tp_size: Optional[int] = None,
 ) -> SearchSpace:
     """Reference: batched_module_analyzer.py:417-536 (same filters, same order)."""
-    tuning = config.tuning
-    num_gpus = num_nodes * num_gpus_per_node
-    per_micro_batch = global_batch_size // gradient_accumulation_steps
-
-    par = []
-    for batch_size in tuning.batch_size_candidates:
-        if batch_size > per_micro_batch or per_micro_batch % batch_size != 0:
-            continue
-        dp_size = per_micro_batch // batch_size
-        if dp_size > num_gpus or num_gpus % dp_size != 0:
-            continue
-        curr_tp_size = num_gpus // dp_size
-        if constraint_fn is not None and not constraint_fn(batch_size, curr_tp_size):
-            continue
-        # The tp size latches to the first feasible batch size when the caller gave none.
-        tp_size = curr_tp_size if tp_size is None else tp_size
-        if tp_size != curr_tp_size:
-            continue
-        if tp_size > num_gpus_per_node:
-            continue
-        if getattr(config, "disable_tp_tuning", False) and tp_size > 1:
-            continue
-        if dp_size == 1 or not tuning.zero_2_and_3_enabled:
-            flag_choices: Sequence[Tuple[int, int, int]] = [(0, 0, 1)]
-        else:
-            flag_choices = tuning.zero_flag_choices
-        for wre, gre, ore in flag_choices:
-            par.append((batch_size, dp_size, tp_size, wre, gre, ore))
-    par_np = np.array(par, dtype=np.float64).reshape(-1, 6)
-
-    wo, go, oo, ao, pair_wo, pair_go = _offload_lists(
-        bool(tuning.state_offloading_enabled), bool(tuning.activation_offloading_enabled),
-        tuple(tuning.offloading_ratio_candidates), tuple(tuning.sparse_offloading_ratio_candidates),
-        bool(getattr(config, "disable_wo_tuning", False)), bool(getattr(config, "disable_go_tuning", False)),
-        bool(getattr(config, "disable_oo_tuning", False)),
-        *(getattr(config, f"fixed_{k}_ratio", None) for k in ("wo", "go", "oo", "ao")),
-    )
-    if par_np.shape[0] > MAX_PAR:
-        raise ValueError(f"{par_np.shape[0]} parallelism rows; at most {MAX_PAR} are supported")
-    return SearchSpace(par=par_np, wo=wo, go=go, oo=oo, ao=ao, pair_wo=pair_wo, pair_go=pair_go)
+    return SearchSpaceFactory(config, constraint_fn).make(
+        num_nodes, num_gpus_per_node, global_batch_size, gradient_accumulation_steps, tp_size)
 
 
 @lru_cache(maxsize=64)

@@ -115,6 +115,37 @@ def test_group_descriptors_bit_exact_against_oracle(overrides, tp):
     assert prob["num_layers"] == 4 and prob["sample_size"] == 1
 
 
+@pytest.mark.parametrize("plan", [2, 5])
+def test_column_wise_fill_equals_record_by_record_fill(plan):
+    """``GroupInputBuilder.fill_many`` (what a tuner call uses) writes the same bytes as ``fill``
+    record by record, for every group of a benchmark plan with all its tp candidates."""
+    from mist_amd.config import tp_candidates
+    from mist_amd.stage_inputs import GroupInputBuilder
+    from tests.util import load_plan
+
+    cfg, tables = load_plan(plan)
+    hw = cfg.hardware
+    meshes = _get_device_mesh_candidates(hw.num_nodes, hw.num_gpus_per_node, False)
+    Gs = _get_grad_accumu_steps_candidates(cfg.training.global_batch_size)
+    tuner = IntraStageTuner(tables, cfg.model.num_hidden_layers, meshes, Gs, tp_candidates(cfg), cfg,
+                            sample_size=1, device="cpu")
+    groups = tuner.prepare()["groups"]
+    assert len(groups) > 50
+    builder = GroupInputBuilder(cfg, tables)
+    one = np.zeros(len(groups), dtype=_lib.GROUP_DTYPE)
+    spaces = tuner.prepare()["spaces"]
+    for i, rec in enumerate(groups):
+        row_g, q = int(rec["g_index"]), int(rec["q_index"])
+        space = spaces[(row_g // len(Gs), row_g % len(Gs), q)]
+        builder.fill(one[i], space, row_g, q, int(rec["num_nodes"]), int(rec["num_gpus_per_node"]),
+                     int(rec["grad_accum"]), int(rec["num_p"]))
+    decomposition = ("rows_per_chunk", "n_chunks", "n_lc_tiles", "n_p_tiles", "scout_stride", "scout_pair",
+                     "row_offset", "key_offset")
+    for name in _lib.GROUP_DTYPE.names:
+        if name not in decomposition:
+            assert np.ascontiguousarray(one[name]).tobytes() == np.ascontiguousarray(groups[name]).tobytes(), name
+
+
 def test_launch_decomposition_covers_every_row_once():
     cfg, tables = load_plan(2)
     hw = cfg.hardware

@@ -980,7 +980,9 @@ struct LaneMemory {
 
   // Peaks of the middle-stage variant for p pre-saved micro-batches (:2755-2786).
   __device__ __forceinline__ void peaks(int p, double &peak_f, double &peak_b) const {
-    const double pf64 = (double)p;
+    peaks_at((double)p, peak_f, peak_b);
+  }
+  __device__ __forceinline__ void peaks_at(double pf64, double &peak_f, double &peak_b) const {
     const double pipe_saved = pf64 * mod_saved + cur_saved;
     const double outp2 = out * pf64 * 2.0;
     const double out2 = out * 2.0;
@@ -1749,12 +1751,19 @@ __device__ __forceinline__ void exhaustive_block(
       // (batched_module_analyzer.py:2815), the others in float64 (:2898-2903, 3002-3007, 3084-3089)
       const double cost_base = ratio * (double)lat.x + (double)(lat.d / G32);
       const double cost_pre = ratio * lat.sp + lat.dpre / G64;
+      // Every slot through both feasibility tests (:2805-2812, 2893-2897), straight-line: the two
+      // tests share the peaks of their p, and nothing is skipped by a branch (a lane whose tile
+      // ends early only masks the update).
 #pragma unroll
       for (int j = 0; j < MIST_P_TILE; ++j) {
+        double peak_f, peak_b;
+        mem.peaks(p0 + j, peak_f, peak_b);
+        const bool fits_base = fmax(peak_f, peak_b) * mem.mf_base <= cap;
+        const double pre_p = (double)(p0 + j) * pre_saved;
+        const bool fits_pre = fmax(pre_p + peak_f + pre_sas, pre_p + peak_b + pre_sas) * mem.mf_pp <= cap;
         const bool live = j < n_tile;
-        take_first(best_b[j], row_b[j], live && mem.feasible_base(p0 + j, cap), cost_base, row);
-        take_first(best_p[j], row_p[j], live && mem.feasible_pre(p0 + j, cap, pre_saved, pre_sas),
-                 cost_pre, row);
+        take_first(best_b[j], row_b[j], live & fits_base, cost_base, row);
+        take_first(best_p[j], row_p[j], live & fits_pre, cost_pre, row);
       }
       if (kFirstTile) {  // last stage / single stage, p == 0 only (:2946-3106)
         double peak_f, peak_b;
@@ -1786,7 +1795,10 @@ __device__ __forceinline__ void exhaustive_block(
   out_index[(2 * MIST_P_TILE + 1) * MIST_LC_TILE + threadIdx.x] = row_pp;
 }
 
-__global__ __launch_bounds__(MIST_LC_TILE) void eval_reduce_exhaustive_kernel(
+#ifndef MIST_EXHAUSTIVE_MIN_WAVES
+#define MIST_EXHAUSTIVE_MIN_WAVES 2
+#endif
+__global__ __launch_bounds__(MIST_LC_TILE, MIST_EXHAUSTIVE_MIN_WAVES) void eval_reduce_exhaustive_kernel(
     const MistProblem prob, const MistGroupDesc *__restrict__ groups, int n_groups,
     const int32_t *__restrict__ block_prefix, int n_blocks, const double *__restrict__ row_terms,
     double ratio, double *__restrict__ partial_cost, int32_t *__restrict__ partial_index) {

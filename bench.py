@@ -44,7 +44,23 @@ def profile_counters():
         m = re.match(r"^\|\s*([A-Z][A-Z0-9_]+)\s*\|\s*([0-9.eE+-]+)\s*\|\s*([0-9.eE+-]+)\s*\|", line)
         if m:
             out[m.group(1)] = dict(pruned=float(m.group(2)), exhaustive=float(m.group(3)))
+        m = re.match(r"^kernel source sha256: ([0-9a-f]+)", line)
+        if m:
+            out["_source_sha256"] = m.group(1)
     return out
+
+
+def kernel_source_sha256():
+    """Digest of the kernel sources the counters belong to (the profile records it)."""
+    import hashlib
+
+    h = hashlib.sha256()
+    for name in ("mist_search.hip", "exact_arith.h", "mist_common.h"):
+        with open(os.path.join(REPO, "mist_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    with open(os.path.join(REPO, "include", "mist_search.h"), "rb") as f:
+        h.update(f.read())
+    return h.hexdigest()[:16]
 
 
 def executed_fp64_flops(counters, which):
@@ -77,13 +93,14 @@ def reduce_kernel_flops(plan, L):
     return 15 * rows * L + 22 * rows * pairs + (30 + 12) * cells + (25 + 10) * rows * pairs
 
 
-def cpu_baseline(cfg, tables, results=None, budget_s=16.0, dp_budget_s=6.0):
-    """Times the numpy oracle (a port of the reference's formulation, single thread) on whole
-    (G, mesh, tp) groups of the same plan until ``budget_s`` is used: first a multi-node group
-    with four parallelism rows (53 724 candidate rows, two pre-saved micro-batch values), then
-    single-device groups (13 431 rows, 32 values, about 9 s each).  With ``results`` (the GPU
-    search's tables of tp = 1) the C restatement of the reference's DP kernel is timed on the
-    same cost tables for thresholds spread over the upper half of the candidates."""
+def cpu_baseline(cfg, tables, results=None, budget_s=14.0, dp_budget_s=6.0):
+    """Times the CPU oracle on whole (G, mesh, tp) groups of the same plan until ``budget_s`` is
+    used, twice: (1) its numpy form (a port of the reference's own formulation, one thread) and
+    (2) its C form (oracle/stage_loop.c: the same loops cell by cell, OpenMP over the (layers,
+    ckpt) pairs like the reference's numba ``prange``) on every core of the host.  The sample
+    starts with a multi-node group with four parallelism rows (53 724 candidate rows), then
+    single-device groups.  With ``results`` (the GPU search's tables of tp = 1) the C restatement
+    of the reference's DP kernel is timed on the same cost tables."""
     import numpy as np
 
     from mist_amd.search_space import _get_device_mesh_candidates, _get_grad_accumu_steps_candidates
@@ -96,24 +113,46 @@ def cpu_baseline(cfg, tables, results=None, budget_s=16.0, dp_budget_s=6.0):
     Gs = _get_grad_accumu_steps_candidates(cfg.training.global_batch_size)
     P = max_pre_saved_micro_batches(meshes, Gs, L)
     sample = [(2, (4, 8), 1), (512, (1, 1), 1), (256, (1, 1), 1), (128, (1, 1), 1)]
-    done, cand, cells, elapsed = [], 0, 0, 0.0
-    for G, (n, m), tp in sample:
-        dbg = {}
-        t0 = time.perf_counter()
-        batched_tune_best_latency_for_stage(
-            tables, cfg, list(range(min(G, L, P + 1))), list(range(1, L + 1)), list(range(L + 1)),
-            n, m, G, tp_size=tp, sample_size=1, debug=dbg,
-        )
-        elapsed += time.perf_counter() - t0
-        rows = dbg["rows"].shape[0]
-        cand += rows * (L + 1)
-        cells += rows * (L * (L + 1) // 2 + L) * min(G, L, P + 1)
-        done.append(f"G={G} mesh={n}x{m} tp={tp} rows={rows}")
-        if elapsed > budget_s:
-            break
+
+    def run(inner, groups, budget, threads=0):
+        done, cand, cells, elapsed = [], 0, 0, 0.0
+        for G, (n, m), tp in groups:
+            dbg = {}
+            t0 = time.perf_counter()
+            batched_tune_best_latency_for_stage(
+                tables, cfg, list(range(min(G, L, P + 1))), list(range(1, L + 1)), list(range(L + 1)),
+                n, m, G, tp_size=tp, sample_size=1, debug=dbg, inner=inner, threads=threads,
+            )
+            elapsed += time.perf_counter() - t0
+            rows = dbg["rows"].shape[0]
+            cand += rows * (L + 1)
+            cells += rows * (L * (L + 1) // 2 + L) * min(G, L, P + 1)
+            done.append(f"G={G} mesh={n}x{m} tp={tp} rows={rows}")
+            if elapsed > budget:
+                break
+        return done, cand, cells, elapsed
+
+    done, cand, cells, elapsed = run("numpy", sample, budget_s * 0.6)
     out = dict(
         value=cand / elapsed, unit="candidates/s", cores=1, kind="port",
         sample="; ".join(done) + f"; {elapsed:.1f} s of numpy, intra-stage evaluation only",
+        cells_per_s=cells / elapsed,
+    )
+    # the C loops on all cores: every group of tp = 1 in table order, as far as the budget goes
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    cores = max(1, min(cores, int(os.environ.get("OMP_NUM_THREADS", cores))))
+    many = sample + [(G, mesh, 1) for G in reversed(Gs) for mesh in meshes if (G, mesh, 1) not in sample]
+    from oracle.search_space import create_search_space
+
+    many = [(G, (n, m), tp) for G, (n, m), tp in many
+            if create_search_space(n, m, cfg.training.global_batch_size, G, cfg,
+                                   constraint_fn=tables.constraint, tp_size=tp).shape[0] > 0]
+    run("c", many[:1], 0.0, cores)  # loads the library, spins the thread pool up
+    done, cand, cells, elapsed = run("c", many, budget_s * 0.4, cores)
+    out["multicore"] = dict(
+        value=cand / elapsed, unit="candidates/s", cores=cores, kind="port",
+        sample=f"{len(done)} groups of tp=1 ({done[0]} ... {done[-1]}); {elapsed:.1f} s; row terms in numpy "
+               f"(one thread), the (ckpt, pre-saved micro-batch) loops and the argmin scan in C on {cores} threads",
         cells_per_s=cells / elapsed,
     )
     if results is not None:
@@ -185,12 +224,50 @@ def other_plans():
     return out
 
 
+def mip_searches(plans=("gpt-7b-b512-4x8.yaml", "llama-13b-b1024-8x8.yaml"), sample_size=30):
+    """``tune()`` with the reference's default granularity at HEAD, ``uniform-device-pp-mip``
+    with 30 alpha samples per cell (mist/utils/pareto.py:124-144, inter_tuning_mip.py): every
+    sample of every cell of every tensor-parallel candidate, then the stage assignment.  Whole
+    call from the configuration object (descriptor building included), median of 3."""
+    import hashlib
+
+    import torch
+    import yaml
+
+    from mist_amd.config import MistConfig
+    from mist_amd.tune_one_case import tune
+
+    out = {}
+    for name in plans:
+        with open(os.path.join(REPO, "mist_amd", "configs", name)) as f:
+            raw = yaml.safe_load(f)
+        raw["tuning"].update(tuning_granularity="uniform-device-pp-mip", sample_size=sample_size)
+        tune(MistConfig(raw))  # warm-up: buffers of this size
+        torch.cuda.synchronize()
+        times = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            cost, solution = tune(MistConfig(raw))
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+        out[name] = dict(tune_s=sorted(times)[1], sample_size=sample_size, cost=cost,
+                         grad_accum=solution[0] if solution else None,
+                         stages=len(solution[1]) if solution else 0,
+                         solution_sha256=hashlib.sha256(repr(solution).encode()).hexdigest()[:16])
+        torch.cuda.empty_cache()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--sustain-s", type=float, default=2.0,
+                    help="seconds the sustained leg repeats the step for (median step time)")
+    ap.add_argument("--no-mip", action="store_true",
+                    help="skip the 30-sample uniform-device-pp-mip searches")
     ap.add_argument("--no-other-plans", action="store_true",
                     help="skip the tune of the four other benchmark plans")
     ap.add_argument("--no-exhaustive", action="store_true",
@@ -250,6 +327,16 @@ def main():
     elapsed = time.perf_counter() - t0
     ms_per_step = 1e3 * elapsed / args.steps
 
+    # Sustained: the same step for at least two seconds, the median of the per-step wall times
+    # (each step ends with the strategy on the host, i.e. with a device synchronisation).
+    sustained = []
+    t_end = time.perf_counter() + args.sustain_s
+    while time.perf_counter() < t_end or len(sustained) < 3:
+        t1 = time.perf_counter()
+        search.run()
+        sustained.append(time.perf_counter() - t1)
+    sustained_ms = 1e3 * sorted(sustained)[len(sustained) // 2]
+
     # The two halves of a step timed apart (a device synchronisation between them, so their sum
     # is slightly above the step time).
     split = {}
@@ -284,6 +371,14 @@ def main():
 
     kernel_ms = time_kernels(search.tuner, search.plan, search.dev_plan, 2)
     counters = profile_counters()
+    # the counters belong to the kernel sources and the launch decomposition they were taken
+    # with: a profile of other sources or another grid gives no executed-work figures
+    main_waves = int(search.plan["reduce_prefix"][-1])
+    counters_stale = bool(counters) and (
+        counters.pop("_source_sha256", None) != kernel_source_sha256()
+        or int(counters.get("SQ_WAVES", {}).get("exhaustive", -1)) != main_waves)
+    if counters_stale:
+        counters = {}
     algorithmic = float(reduce_kernel_flops(search.plan, search.L))
     peak = FP64_VECTOR_PEAK / 1e12
 
@@ -323,6 +418,7 @@ def main():
     roofline["frac"] = roofline["achieved"] / peak if executed is not None else None
     roofline["pruning_gain"] = roofline["algorithmic_tflops"] / peak
     roofline["counters_from"] = os.path.relpath(PROFILE, REPO) if counters else None
+    roofline["counters_stale"] = counters_stale
     exhaustive = None
     if not args.no_exhaustive:
         full = PreparedSearch(cfg, "cuda:0", exhaustive=True)
@@ -376,12 +472,16 @@ def main():
         # back-pointers) until the strategy is on the host
         "intra_stage_ms_per_step": 1e3 * split["intra_launch_s"] / 5,
         "inter_stage_ms_per_step": 1e3 * split["inter_s"] / 5,
+        "sustained": {"seconds": args.sustain_s, "steps": len(sustained), "median_ms_per_step": sustained_ms,
+                      "candidates_per_s": counts["candidates"] / (sustained_ms * 1e-3)},
         "dp_thresholds_per_step": stats.get("dp_thresholds", 0) / args.steps,
         "best_cost": cost,
         "best_solution": repr(solution),
         "roofline": roofline,
         "exhaustive": exhaustive,
     }
+    if not args.no_mip:
+        result["mip_30_samples"] = mip_searches()
     if not args.no_other_plans:
         result["other_plans"] = other_plans()
     if not args.no_cpu_baseline:

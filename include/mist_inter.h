@@ -1,9 +1,9 @@
 /*
  * C ABI of the inter-stage search driver (part of libmist_search.so): the whole search of
- * inter_stage_tune (mist/analyzer/inter_tuning.py:95-217) for the per-mesh recurrence in one
- * call.  Conventions as in mist_search.h; this entry point allocates its own device and pinned
- * host buffers (kept per device for the life of the process) and synchronises `stream` between
- * its dependent batches.
+ * inter_stage_tune (mist/analyzer/inter_tuning.py:95-217; with several DP families the one of
+ * mist/analyzer/inter_tuning_uniform_device.py:312-367) in one call.  Conventions as in
+ * mist_search.h; these entry points allocate their own device and pinned host buffers (kept per
+ * device for the life of the process) and synchronise `stream` between their dependent batches.
  */
 #ifndef MIST_INTER_H
 #define MIST_INTER_H
@@ -15,6 +15,17 @@
 #ifdef __cplusplus
 extern "C" {
 #endif
+
+/* Row-index tables of the intra-stage search (MistOutTables.index of the launch that covers
+ * every table row the search uses) and how to address them: what
+ * get_solution_from_intra_stage_tuner_output (inter_tuning.py:38-60) reads for a stage. */
+typedef struct MistStrategyIndex {
+  const int32_t *index[4]; /* DEVICE: [g][Q][p_dim][L][L+1][S] x2, [g][Q][L][L+1][S], [g][Q][L+1][S] */
+  int32_t num_layers, p_dim, num_mesh, sample_size;
+  int32_t slot;            /* position on the sample axis */
+  int32_t mesh_n[MIST_MAX_MESH], mesh_m[MIST_MAX_MESH]; /* the q axis, in candidate-list order */
+} MistStrategyIndex;
+int mist_sizeof_strategy_index(void);
 
 /* Searches n_instances independent instances (the tensor-parallel candidates of one tune call)
  * over the same n_grad_accum gradient-accumulation candidates, each exactly as the reference does
@@ -39,6 +50,31 @@ int mist_inter_stage_search(const MistDpShape *shape, const MistDpCosts *costs, 
                             int only_best_path, double *out_cost, int32_t *out_g, float *out_tmax,
                             int32_t *out_stages, int32_t *out_path, int64_t *out_stats,
                             void *stream);
+
+/* The same search over n_families DP families (shapes[f], costs[f]; HOST arrays): the cost of a
+ * (G, threshold) pair is the smallest family total, the first family winning ties, as the
+ * reference's loop over stage counts with its strict "<" does
+ * (inter_tuning_uniform_device.py:360-367 around the DP of :370-470; one family with
+ * free_devices != 0 per admissible stage count).  One family with free_devices == 0 is the
+ * search of mist_inter_stage_search.
+ *   select_costs : the tables whose costs / with_pre / with_post entries of a table row are the
+ *                  threshold candidates of that row (inter_tuning.py:180-186); for the per-mesh
+ *                  recurrence the family's own tables
+ *   strategy     : may be NULL; with it the strategy rows of the winners' stages are read on the
+ *                  GPU in the same round trip as their partitions
+ * Additional outputs (HOST): out_family[n_instances] (family of the winning partition, -1 if not
+ * walked), out_path[n_instances][S][4] and out_rows[n_instances][S] with S = the largest
+ * max_stages of the families (out_rows: row index of stage i's strategy in its group's search
+ * space, -1 beyond the partition; may be NULL without `strategy`), out_stats[5] (may be NULL): as
+ * above, then the number of stream synchronisations the search waited for. */
+int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
+                                     const MistDpCosts *costs, const MistDpCosts *select_costs,
+                                     const MistStrategyIndex *strategy, int n_instances,
+                                     int n_grad_accum, const int32_t *rows,
+                                     const int32_t *grad_accum, int only_best_path, double *out_cost,
+                                     int32_t *out_g, float *out_tmax, int32_t *out_family,
+                                     int32_t *out_stages, int32_t *out_path, int32_t *out_rows,
+                                     int64_t *out_stats, void *stream);
 
 #ifdef __cplusplus
 }

@@ -278,11 +278,32 @@ class MipBatchItem(ctypes.Structure):
                 ("first_block", ctypes.c_int32), ("reserved", ctypes.c_int32)]
 
 
+class StrategyIndex(ctypes.Structure):
+    """``MistStrategyIndex`` of include/mist_inter.h."""
+
+    _fields_ = [
+        ("index", ctypes.c_void_p * 4),
+        ("num_layers", ctypes.c_int32),
+        ("p_dim", ctypes.c_int32),
+        ("num_mesh", ctypes.c_int32),
+        ("sample_size", ctypes.c_int32),
+        ("slot", ctypes.c_int32),
+        ("mesh_n", ctypes.c_int32 * MAX_MESH),
+        ("mesh_m", ctypes.c_int32 * MAX_MESH),
+    ]
+
+
 _INTER_SIGNATURES = {
+    "mist_sizeof_strategy_index": (ctypes.c_int, []),
     "mist_inter_stage_search": (
         ctypes.c_int,
         [_VP, ctypes.POINTER(DpCosts), ctypes.c_int, ctypes.c_int, _VP, _VP, ctypes.c_int,
          _VP, _VP, _VP, _VP, _VP, _VP, _VP]),
+    "mist_inter_stage_search_families": (
+        ctypes.c_int,
+        [ctypes.c_int, _VP, _VP, ctypes.POINTER(DpCosts), ctypes.POINTER(StrategyIndex),
+         ctypes.c_int, ctypes.c_int, _VP, _VP, ctypes.c_int,
+         _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP]),
 }
 
 _MIP_SIGNATURES = {
@@ -331,6 +352,10 @@ def load():
         raise MistLibraryError(
             f"MistDpShape layout mismatch: C {lib.mist_sizeof_dp_shape()} vs numpy {DP_SHAPE_DTYPE.itemsize}"
         )
+    if lib.mist_sizeof_strategy_index() != ctypes.sizeof(StrategyIndex):
+        raise MistLibraryError(
+            f"MistStrategyIndex layout mismatch: C {lib.mist_sizeof_strategy_index()} vs ctypes "
+            f"{ctypes.sizeof(StrategyIndex)}")
     if lib.mist_sizeof_mip_shape() != ctypes.sizeof(MipShape):
         raise MistLibraryError(
             f"MistMipShape layout mismatch: C {lib.mist_sizeof_mip_shape()} vs ctypes {ctypes.sizeof(MipShape)}"

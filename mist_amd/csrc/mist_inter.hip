@@ -1,10 +1,16 @@
-// Host orchestration of the inter-stage search for the per-mesh DP (reference:
-// inter_stage_tune / inter_stage_tune_with_fixed_grad_accumu, mist/analyzer/inter_tuning.py:
-// 95-217): bottleneck DP, threshold windows, speculative scan batches with the sequential replay
-// of the reference's rules, back-pointers of the winner.  Same steps as the Python driver
-// (mist_amd/inter_tuning.py), which stays the implementation for the uniform-device recurrence;
-// here they run without an interpreter between the batches: a search makes 5-6 dependent
-// round trips to the GPU, and the glue between them was half of its time.
+// Host orchestration of the inter-stage search (reference: inter_stage_tune /
+// inter_stage_tune_with_fixed_grad_accumu, mist/analyzer/inter_tuning.py:95-217, and the
+// uniform-device variant, mist/analyzer/inter_tuning_uniform_device.py:312-367): bottleneck DP,
+// threshold windows, speculative scan batches with the sequential replay of the reference's
+// rules, back-pointers of the winner, strategy rows of its stages.  Same steps as the Python
+// driver (mist_amd/inter_tuning.py); here they run without an interpreter between the batches: a
+// search makes 4-5 dependent round trips to the GPU, and the glue between them was half of its
+// time.
+//
+// A search runs over one or more DP families (shape + tables): the per-mesh recurrence is one
+// family, the uniform-device recurrence one family per admissible stage count.  The cost of a
+// (G, threshold) instance is the smallest family total, the first family winning ties; all
+// families of a batch run back to back on the stream and come back with one synchronisation.
 //
 // Everything that decides a result is shared with the Python driver through the C ABI:
 // mist_dp_run, mist_dp_select_candidates, mist_dp_window_begin, mist_dp_filter_tmax,
@@ -60,12 +66,13 @@ struct Buffer {
 };
 
 struct Workspace {
-  Buffer d_in, d_out, d_scratch, d_req, d_counts, d_values, d_request, d_argmin, d_path;
-  Buffer h_in, h_out, h_req, h_counts, h_values, h_request, h_path;
+  Buffer d_in, d_out, d_scratch, d_req, d_counts, d_values, d_request, d_argmin, d_path, d_rows,
+      d_grad;
+  Buffer h_in, h_out, h_req, h_counts, h_values, h_request, h_path, h_rows, h_grad;
   int select_capacity = 1 << 18;
   Workspace() {
     h_in.pinned = h_out.pinned = h_req.pinned = h_counts.pinned = h_values.pinned =
-        h_request.pinned = h_path.pinned = true;
+        h_request.pinned = h_path.pinned = h_rows.pinned = h_grad.pinned = true;
   }
 };
 
@@ -118,69 +125,199 @@ struct Fetched {  // one request of a candidate fetch: ascending values and how 
   int above = 0;
 };
 
+// ---- two small kernels that keep dependent steps on the GPU ----
+
+// Window request of every (instance, G) right after the bottleneck DP of all families
+// (out[f][3][n], rows 1 and 2 = smallest feasible threshold and the stage-cost sum there): the
+// family with the smallest threshold (the first of equals) gives the start of the window;
+// req[0][i] = table row, req[1][i] = lo, req[2][i] = hi of the candidates to fetch, an empty
+// window (lo = hi = +inf) when no family is feasible.  The bounds only size the fetch; what the
+// scan does with the candidates is decided on the host from the values that come back.
+__global__ void window_request_kernel(const float *__restrict__ out, int n_families, int n,
+                                      const int32_t *__restrict__ rows,
+                                      const int32_t *__restrict__ grad_accum, int n_grad_accum,
+                                      double gap, float *__restrict__ req) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  float bott = INFINITY, sum = INFINITY;
+  for (int f = 0; f < n_families; ++f) {
+    const float b = out[(size_t)f * 3 * n + n + i];
+    if (b < bott) {
+      bott = b;
+      sum = out[(size_t)f * 3 * n + 2 * n + i];
+    }
+  }
+  reinterpret_cast<int32_t *>(req)[i] = rows[i];
+  if (!(bott < INFINITY)) {
+    req[n + i] = INFINITY;
+    req[2 * n + i] = INFINITY;
+    return;
+  }
+  const double G = (double)grad_accum[i % n_grad_accum];
+  // the min-max partition is admissible at the bottleneck: its total bounds the scan's best;
+  // the first KEPT candidate may lie a few gaps above, and when the bottleneck is a single-stage
+  // cost (no candidate itself) a little further up
+  const double cost0 = (double)sum + (G - 1.0) * (double)bott;
+  const double room = (G - 1.0) * (4.0 * gap);
+  float hi = nextafterf((float)((cost0 + room) * (1.0 + 1e-5) / G), INFINITY);
+  hi = fmaxf(hi, (float)((double)bott * (1.0 + 2e-3) + 2e-4));
+  req[n + i] = bott - (float)(1e-4 + 1e-5 * fabs((double)bott));
+  req[2 * n + i] = hi;
+}
+
+// Strategy row of every stage of the walked partitions: stage i of partition k (path[k][i] =
+// (end layer, n, m, ckpt), stages[k] of them) reads the row-index table of its variant
+// (inter_tuning.py:38-60: whole model / first stage / last stage / inner stage) at table row
+// g_rows[k], mesh (n, m), pre-saved micro-batches = stages after it.
+__global__ void strategy_rows_kernel(const MistStrategyIndex tabs, const int32_t *__restrict__ path,
+                                     const int32_t *__restrict__ best_s,
+                                     const int32_t *__restrict__ g_rows, int n, int max_stages,
+                                     int32_t *__restrict__ out) {
+  const int e = blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= n * max_stages) return;
+  const int k = e / max_stages, i = e % max_stages;
+  const int n_stages = best_s[k];
+  int32_t row = -1;
+  if (i < n_stages) {
+    const int32_t *st = path + (size_t)e * 4;
+    const int start = i == 0 ? 0 : path[(size_t)(e - 1) * 4] + 1;
+    const int end = st[0], c = st[3];
+    int q = -1;
+    for (int m = 0; m < tabs.num_mesh; ++m)
+      if (tabs.mesh_n[m] == st[1] && tabs.mesh_m[m] == st[2]) q = m;
+    const int64_t L = tabs.num_layers, C = L + 1, S = tabs.sample_size, Q = tabs.num_mesh;
+    const int64_t g = g_rows[k], l = end - start + 1, p = n_stages - i - 1;
+    if (q >= 0 && end >= start && end < L && c >= 0 && c <= L && p < tabs.p_dim) {
+      if (start == 0 && end == L - 1)
+        row = tabs.index[3][((g * Q + q) * C + c) * S + tabs.slot];
+      else if (end == L - 1)
+        row = tabs.index[2][(((g * Q + q) * L + (l - 1)) * C + c) * S + tabs.slot];
+      else
+        row = tabs.index[start == 0 ? 1 : 0]
+                        [((((g * Q + q) * tabs.p_dim + p) * L + (l - 1)) * C + c) * S + tabs.slot];
+    }
+  }
+  out[e] = row;
+}
+
 struct Search {
-  const MistDpShape *shape;
-  const MistDpCosts *costs;
+  int n_families;
+  const MistDpShape *shapes;  // [n_families]
+  const MistDpCosts *costs;   // [n_families]
+  const MistDpCosts *select_costs;  // tables the threshold candidates are taken from
+  const MistStrategyIndex *strategy;  // may be null
   hipStream_t stream;
   Workspace *ws;
-  int64_t launches = 0, fetches = 0, selected = 0, thresholds_run = 0;
+  int64_t launches = 0, fetches = 0, selected = 0, thresholds_run = 0, round_trips = 0;
 
-  // DP instances (g_index[i], tmax[i]) -> outputs in ws->h_out as [3][n] (best_s bits, best_sum,
-  // stage_max); with `n_path` > 0 also the partitions of the first n (== n_path) instances.
+  size_t path_ints(int f) const { return (size_t)shapes[f].max_stages * 4; }
+  // ints in front of family f's partitions in the path buffers of a batch of n instances
+  size_t path_offset(int f, int n) const {
+    size_t at = 0;
+    for (int k = 0; k < f; ++k) at += path_ints(k) * n;
+    return at;
+  }
+
+  // DP instances (g_index[i], tmax[i]) of every family -> ws->h_out as [family][3][n] (best_s
+  // bits, best_sum, stage_max); with `want_path` also the partitions (ws->h_path, family after
+  // family) and, when strategy tables were given, the strategy rows of their stages
+  // (ws->h_rows, same order without the factor 4).  `sync` false leaves the copies of the
+  // outputs queued on the stream for the caller to wait for.
   int run(const std::vector<int32_t> &g_index, const std::vector<float> &tmax, int mode,
-          bool want_path) {
+          bool want_path, bool sync = true) {
     const int n = (int)tmax.size();
     if (n == 0) return 0;
+    const size_t n_out = (size_t)3 * n * n_families;
     if (int rc = ws->h_in.reserve(sizeof(float) * 2 * n)) return rc;
     if (int rc = ws->d_in.reserve(sizeof(float) * 2 * n)) return rc;
-    if (int rc = ws->d_out.reserve(sizeof(float) * 3 * n)) return rc;
-    if (int rc = ws->h_out.reserve(sizeof(float) * 3 * n)) return rc;
-    const int64_t n_scratch = mist_dp_scratch_floats(shape, n);
-    if (n_scratch < 0) return MIST_E_INVALID;
-    if (int rc = ws->d_scratch.reserve(sizeof(float) * (size_t)std::max<int64_t>(n_scratch, 1)))
-      return rc;
+    if (int rc = ws->d_out.reserve(sizeof(float) * n_out)) return rc;
+    if (int rc = ws->h_out.reserve(sizeof(float) * n_out)) return rc;
+    int64_t n_scratch = 1;
+    size_t slab = 0;
+    for (int f = 0; f < n_families; ++f) {
+      const int64_t want = mist_dp_scratch_floats(&shapes[f], n);
+      if (want < 0) return MIST_E_INVALID;
+      n_scratch = std::max(n_scratch, want);
+      slab = std::max(slab, (size_t)(shapes[f].max_stages + 1) * (shapes[f].num_layers + 1) *
+                                (shapes[f].num_devices + 1) * 4);
+    }
+    if (int rc = ws->d_scratch.reserve(sizeof(float) * (size_t)n_scratch)) return rc;
+    const size_t n_path = path_offset(n_families, n);
+    if (want_path) {
+      if (int rc = ws->d_argmin.reserve(sizeof(int32_t) * slab * n)) return rc;
+      if (int rc = ws->d_path.reserve(sizeof(int32_t) * n_path)) return rc;
+      if (int rc = ws->h_path.reserve(sizeof(int32_t) * n_path)) return rc;
+      if (int rc = ws->d_rows.reserve(sizeof(int32_t) * n_path / 4)) return rc;
+      if (int rc = ws->h_rows.reserve(sizeof(int32_t) * n_path / 4)) return rc;
+    }
     float *h_in = ws->h_in.as<float>();
     std::memcpy(h_in, tmax.data(), sizeof(float) * n);
     std::memcpy(h_in + n, g_index.data(), sizeof(int32_t) * n);
     MIST_HIP_CHECK(hipMemcpyAsync(ws->d_in.ptr, h_in, sizeof(float) * 2 * n, hipMemcpyHostToDevice,
                                   stream));
-    float *d_in = ws->d_in.as<float>(), *d_out = ws->d_out.as<float>();
-    int32_t *d_argmin = nullptr;
-    if (want_path) {
-      const size_t slab = (size_t)(shape->max_stages + 1) * (shape->num_layers + 1) *
-                          (shape->num_devices + 1) * 4;
-      if (int rc = ws->d_argmin.reserve(sizeof(int32_t) * slab * n)) return rc;
-      if (int rc = ws->d_path.reserve(sizeof(int32_t) * (size_t)n * shape->max_stages * 4)) return rc;
-      if (int rc = ws->h_path.reserve(sizeof(int32_t) * (size_t)n * shape->max_stages * 4)) return rc;
-      d_argmin = ws->d_argmin.as<int32_t>();  // no fill: the walk reads what the DP wrote
-    }
-    if (int rc = mist_dp_run(shape, costs, d_in, reinterpret_cast<int32_t *>(d_in + n), n, mode,
-                             reinterpret_cast<int32_t *>(d_out), d_out + n, d_out + 2 * n, d_argmin,
-                             ws->d_scratch.as<float>(), stream))
-      return rc;
-    if (want_path) {
-      if (int rc = mist_dp_backtrack(shape, d_argmin, reinterpret_cast<int32_t *>(d_out), n,
-                                     ws->d_path.as<int32_t>(), stream))
+    float *d_in = ws->d_in.as<float>();
+    const int32_t *d_g = reinterpret_cast<int32_t *>(d_in + n);
+    // the families share the state planes and the back-pointer slab: they run one after the
+    // other on the stream
+    for (int f = 0; f < n_families; ++f) {
+      float *d_out = ws->d_out.as<float>() + (size_t)f * 3 * n;
+      int32_t *d_argmin = want_path ? ws->d_argmin.as<int32_t>() : nullptr;  // no fill: the
+                                                     // walk reads what the DP wrote
+      if (int rc = mist_dp_run(&shapes[f], &costs[f], d_in, d_g, n, mode,
+                               reinterpret_cast<int32_t *>(d_out), d_out + n, d_out + 2 * n,
+                               d_argmin, ws->d_scratch.as<float>(), stream))
         return rc;
-      MIST_HIP_CHECK(hipMemcpyAsync(ws->h_path.ptr, ws->d_path.ptr,
-                                    sizeof(int32_t) * (size_t)n * shape->max_stages * 4,
-                                    hipMemcpyDeviceToHost, stream));
+      if (want_path) {
+        int32_t *d_path = ws->d_path.as<int32_t>() + path_offset(f, n);
+        if (int rc = mist_dp_backtrack(&shapes[f], d_argmin, reinterpret_cast<int32_t *>(d_out), n,
+                                       d_path, stream))
+          return rc;
+        if (strategy) {
+          const int cells = n * shapes[f].max_stages;
+          hipLaunchKernelGGL(strategy_rows_kernel, dim3((cells + 63) / 64), dim3(64), 0, stream,
+                             *strategy, d_path, reinterpret_cast<int32_t *>(d_out), d_g, n,
+                             shapes[f].max_stages, ws->d_rows.as<int32_t>() + path_offset(f, n) / 4);
+          MIST_HIP_CHECK(hipGetLastError());
+        }
+      }
     }
-    MIST_HIP_CHECK(hipMemcpyAsync(ws->h_out.ptr, d_out, sizeof(float) * 3 * n,
+    if (want_path) {
+      MIST_HIP_CHECK(hipMemcpyAsync(ws->h_path.ptr, ws->d_path.ptr, sizeof(int32_t) * n_path,
+                                    hipMemcpyDeviceToHost, stream));
+      if (strategy)
+        MIST_HIP_CHECK(hipMemcpyAsync(ws->h_rows.ptr, ws->d_rows.ptr, sizeof(int32_t) * n_path / 4,
+                                      hipMemcpyDeviceToHost, stream));
+    }
+    MIST_HIP_CHECK(hipMemcpyAsync(ws->h_out.ptr, ws->d_out.ptr, sizeof(float) * n_out,
                                   hipMemcpyDeviceToHost, stream));
-    MIST_HIP_CHECK(hipStreamSynchronize(stream));
-    ++launches;
-    thresholds_run += n;
+    launches += n_families;
+    thresholds_run += (int64_t)n * n_families;
+    if (sync) {
+      MIST_HIP_CHECK(hipStreamSynchronize(stream));
+      ++round_trips;
+    }
     return 0;
   }
 
-  // best + (g - 1) * f_stage_max in float64 (inter_tuning.py:342), inf if infeasible
-  double total(int i, int n, int G) const {
-    const float *h = ws->h_out.as<float>();
+  // best + (g - 1) * f_stage_max in float64 (inter_tuning.py:342) of family f, inf if infeasible
+  double total_of(int f, int i, int n, int G) const {
+    const float *h = ws->h_out.as<float>() + (size_t)f * 3 * n;
     int32_t best_s;
     std::memcpy(&best_s, h + i, sizeof(best_s));
     if (best_s < 0) return kInf;
     return (double)h[n + i] + ((double)G - 1.0) * (double)h[2 * n + i];
+  }
+  // smallest family total (the first family wins ties); *family = the one that attains it
+  double total(int i, int n, int G, int *family = nullptr) const {
+    double best = kInf;
+    for (int f = 0; f < n_families; ++f) {
+      const double c = total_of(f, i, n, G);
+      if (c < best) {
+        best = c;
+        if (family) *family = f;
+      }
+    }
+    return best;
   }
 
   // ascending candidates v of table row rows[r] with lo[r] < v <= hi[r], and how many lie above
@@ -189,17 +326,48 @@ struct Search {
     const int n = (int)rows.size();
     out->assign(n, Fetched());
     if (n == 0) return 0;
-    ++fetches;
     if (int rc = ws->h_req.reserve(sizeof(float) * 3 * n)) return rc;
     if (int rc = ws->d_req.reserve(sizeof(float) * 3 * n)) return rc;
-    if (int rc = ws->d_counts.reserve(sizeof(int32_t) * (1 + n))) return rc;
-    if (int rc = ws->h_counts.reserve(sizeof(int32_t) * (1 + n))) return rc;
     float *h_req = ws->h_req.as<float>();
     std::memcpy(h_req, rows.data(), sizeof(int32_t) * n);
     std::memcpy(h_req + n, lo.data(), sizeof(float) * n);
     std::memcpy(h_req + 2 * n, hi.data(), sizeof(float) * n);
     MIST_HIP_CHECK(hipMemcpyAsync(ws->d_req.ptr, h_req, sizeof(float) * 3 * n,
                                   hipMemcpyHostToDevice, stream));
+    return collect(n, out);
+  }
+
+  // The bottleneck DP of every (instance, G) and the first fetch of their windows in one round
+  // trip: the requests are made on the GPU from the DP's outputs.  ws->h_out holds the DP
+  // outputs afterwards, ws->h_req the requests as they were made ([3][n]: row, lo, hi).
+  int bottleneck_and_fetch(const std::vector<int32_t> &rows, const int32_t *grad_accum,
+                           int n_grad_accum, std::vector<Fetched> *out) {
+    const int n = (int)rows.size();
+    if (int rc = ws->h_grad.reserve(sizeof(int32_t) * n_grad_accum)) return rc;
+    if (int rc = ws->d_grad.reserve(sizeof(int32_t) * n_grad_accum)) return rc;
+    if (int rc = ws->h_req.reserve(sizeof(float) * 3 * n)) return rc;
+    if (int rc = ws->d_req.reserve(sizeof(float) * 3 * n)) return rc;
+    std::memcpy(ws->h_grad.ptr, grad_accum, sizeof(int32_t) * n_grad_accum);
+    MIST_HIP_CHECK(hipMemcpyAsync(ws->d_grad.ptr, ws->h_grad.ptr, sizeof(int32_t) * n_grad_accum,
+                                  hipMemcpyHostToDevice, stream));
+    const std::vector<float> zeros(n, 0.0f);
+    if (int rc = run(rows, zeros, MIST_DP_BOTTLENECK, false, /*sync=*/false)) return rc;
+    hipLaunchKernelGGL(window_request_kernel, dim3((n + 63) / 64), dim3(64), 0, stream,
+                       ws->d_out.as<float>(), n_families, n,
+                       reinterpret_cast<const int32_t *>(ws->d_in.as<float>() + n),
+                       ws->d_grad.as<int32_t>(), n_grad_accum, kGap, ws->d_req.as<float>());
+    MIST_HIP_CHECK(hipGetLastError());
+    MIST_HIP_CHECK(hipMemcpyAsync(ws->h_req.ptr, ws->d_req.ptr, sizeof(float) * 3 * n,
+                                  hipMemcpyDeviceToHost, stream));
+    out->assign(n, Fetched());
+    return collect(n, out);
+  }
+
+  // runs the n requests that lie in ws->d_req and sorts what comes back by request
+  int collect(int n, std::vector<Fetched> *out) {
+    ++fetches;
+    if (int rc = ws->d_counts.reserve(sizeof(int32_t) * (1 + n))) return rc;
+    if (int rc = ws->h_counts.reserve(sizeof(int32_t) * (1 + n))) return rc;
     float *d_req = ws->d_req.as<float>();
     int total = 0, head = 0;
     for (;;) {
@@ -208,7 +376,7 @@ struct Search {
       if (int rc = ws->d_request.reserve(sizeof(int32_t) * capacity)) return rc;
       MIST_HIP_CHECK(hipMemsetAsync(ws->d_counts.ptr, 0, sizeof(int32_t) * (1 + n), stream));
       if (int rc = mist_dp_select_candidates(
-              costs, n, reinterpret_cast<int32_t *>(d_req), d_req + n, d_req + 2 * n,
+              select_costs, n, reinterpret_cast<int32_t *>(d_req), d_req + n, d_req + 2 * n,
               ws->d_values.as<float>(), ws->d_request.as<int32_t>(), capacity,
               ws->d_counts.as<int32_t>(), stream))
         return rc;
@@ -224,6 +392,7 @@ struct Search {
       MIST_HIP_CHECK(hipMemcpyAsync(ws->h_request.ptr, ws->d_request.ptr, sizeof(int32_t) * head,
                                     hipMemcpyDeviceToHost, stream));
       MIST_HIP_CHECK(hipStreamSynchronize(stream));
+      ++round_trips;
       total = ws->h_counts.as<int32_t>()[0];
       if (total <= capacity) break;
       ws->select_capacity = 2 * total;
@@ -240,6 +409,7 @@ struct Search {
       MIST_HIP_CHECK(hipMemcpyAsync(ws->h_request.ptr, ws->d_request.ptr, sizeof(int32_t) * total,
                                     hipMemcpyDeviceToHost, stream));
       MIST_HIP_CHECK(hipStreamSynchronize(stream));
+      ++round_trips;
     }
     const float *values = ws->h_values.as<float>();
     const int32_t *request = ws->h_request.as<int32_t>();
@@ -324,75 +494,110 @@ struct Scan {
 
 extern "C" {
 
-int mist_inter_stage_search(const MistDpShape *shape, const MistDpCosts *costs, int n_instances,
-                            int n_grad_accum, const int32_t *rows, const int32_t *grad_accum,
-                            int only_best_path, double *out_cost, int32_t *out_g, float *out_tmax,
-                            int32_t *out_stages, int32_t *out_path, int64_t *out_stats,
-                            void *stream_) {
-  if (!shape || !costs || !rows || !grad_accum || !out_cost || !out_g || !out_tmax || !out_stages ||
-      !out_path)
+int mist_sizeof_strategy_index(void) { return (int)sizeof(MistStrategyIndex); }
+
+int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
+                                     const MistDpCosts *costs, const MistDpCosts *select_costs,
+                                     const MistStrategyIndex *strategy, int n_instances,
+                                     int n_grad_accum, const int32_t *rows,
+                                     const int32_t *grad_accum, int only_best_path, double *out_cost,
+                                     int32_t *out_g, float *out_tmax, int32_t *out_family,
+                                     int32_t *out_stages, int32_t *out_path, int32_t *out_rows,
+                                     int64_t *out_stats, void *stream_) {
+  if (!shapes || !costs || !select_costs || !rows || !grad_accum || !out_cost || !out_g ||
+      !out_tmax || !out_family || !out_stages || !out_path)
     return fail(MIST_E_INVALID, "null pointer argument");
+  if (n_families < 1) return fail(MIST_E_INVALID, "need at least one DP family, got %d", n_families);
   if (n_instances < 1 || n_grad_accum < 1)
     return fail(MIST_E_INVALID, "need at least one instance and one G, got %d x %d", n_instances,
                 n_grad_accum);
-  if (shape->free_devices != 0)
-    return fail(MIST_E_INVALID, "the search covers the per-mesh recurrence only");
-  const int64_t n_scr = mist_dp_scratch_floats(shape, 1);
-  if (n_scr < 0) return MIST_E_INVALID;  // bad shape: message set by the check
+  if ((int64_t)n_instances * n_grad_accum > 65535)
+    return fail(MIST_E_INVALID, "%d x %d (instance, G) pairs; at most 65535", n_instances,
+                n_grad_accum);
+  if (strategy && !out_rows) return fail(MIST_E_INVALID, "strategy tables without out_rows");
+  int S_max = 0;
+  for (int f = 0; f < n_families; ++f) {
+    if (mist_dp_scratch_floats(&shapes[f], 1) < 0) return MIST_E_INVALID;  // message set by the check
+    if (shapes[f].num_layers != shapes[0].num_layers)
+      return fail(MIST_E_INVALID, "family %d has %d layers, family 0 has %d", f,
+                  shapes[f].num_layers, shapes[0].num_layers);
+    S_max = std::max(S_max, shapes[f].max_stages);
+  }
+  if (strategy) {
+    if (strategy->num_layers != shapes[0].num_layers || strategy->num_mesh < 1 ||
+        strategy->num_mesh > MIST_MAX_MESH || strategy->p_dim < 1 || strategy->sample_size < 1 ||
+        strategy->slot < 0 || strategy->slot >= strategy->sample_size)
+      return fail(MIST_E_INVALID, "strategy tables do not fit the DP shape");
+    for (int v = 0; v < 4; ++v)
+      if (!strategy->index[v]) return fail(MIST_E_INVALID, "null strategy index table %d", v);
+  }
   for (int i = 0; i < n_grad_accum; ++i)
     if (grad_accum[i] < 1) return fail(MIST_E_INVALID, "grad_accum[%d] = %d < 1", i, grad_accum[i]);
 
   std::lock_guard<std::mutex> guard(g_lock);
   int device = 0;
   MIST_HIP_CHECK(hipGetDevice(&device));
-  Search S{shape, costs, (hipStream_t)stream_, &g_workspaces[device]};
+  Search S{n_families, shapes, costs, select_costs, strategy, (hipStream_t)stream_,
+           &g_workspaces[device]};
   const int n_flat = n_instances * n_grad_accum;
-  const int S_max = shape->max_stages;
 
-  // ---- smallest feasible threshold of every (instance, G) in one batch ----
+  // ---- smallest feasible threshold of every (instance, G) and the first fetch of its window:
+  // one round trip ----
   std::vector<int32_t> flat_rows(rows, rows + n_flat);
-  std::vector<float> zeros(n_flat, 0.0f);
-  if (int rc = S.run(flat_rows, zeros, MIST_DP_BOTTLENECK, false)) return rc;
+  std::vector<Fetched> first;
+  if (int rc = S.bottleneck_and_fetch(flat_rows, grad_accum, n_grad_accum, &first)) return rc;
   std::vector<Window> windows(n_flat);
   std::vector<int> feasible;
   std::vector<float> hi_first;
   {
     const float *h = S.ws->h_out.as<float>();
+    const float *req = S.ws->h_req.as<float>();
     for (int i = 0; i < n_flat; ++i) {
-      const float bott = h[n_flat + i];
+      float bott = std::numeric_limits<float>::infinity(), sum = bott;
+      for (int f = 0; f < n_families; ++f) {
+        const float b = h[(size_t)f * 3 * n_flat + n_flat + i];
+        if (b < bott) {
+          bott = b;
+          sum = h[(size_t)f * 3 * n_flat + 2 * n_flat + i];
+        }
+      }
       if (!std::isfinite(bott)) continue;
       Window &w = windows[i];
       w.exists = true;
       w.row = flat_rows[i];
       w.G = grad_accum[i % n_grad_accum];
       w.start_value = bott;
-      w.start_sum = (double)h[2 * n_flat + i];
-      // the min-max partition is admissible at the bottleneck: its total bounds the scan's
-      // best; the first KEPT candidate may lie a few gaps above, and when the bottleneck is a
-      // single-stage cost (no candidate itself) a little further up
-      const double cost0 = w.start_sum + (double)(w.G - 1) * (double)bott;
-      const double room = (double)(w.G - 1) * (4 * kGap);
-      float hi = std::nextafter((float)((cost0 + room) * (1.0 + 1e-5) / (double)w.G),
-                                std::numeric_limits<float>::infinity());
-      hi = std::max(hi, (float)((double)bott * (1.0 + 2e-3) + 2e-4));
+      w.start_sum = (double)sum;
       feasible.push_back(i);
-      hi_first.push_back(hi);
+      hi_first.push_back(req[2 * n_flat + i]);
     }
   }
   {
     std::vector<int> pending(feasible.size());
     for (size_t k = 0; k < pending.size(); ++k) pending[k] = (int)k;
+    // widen 0 is the fetch that came with the bottleneck DP; the requests of the later passes
+    // are made here
+    std::vector<Fetched> got;
+    std::vector<float> lo, hi;
+    for (int k : pending) {
+      got.push_back(std::move(first[feasible[k]]));
+      lo.push_back(S.ws->h_req.as<float>()[n_flat + feasible[k]]);
+      hi.push_back(hi_first[k]);
+    }
+    first.clear();
     for (int widen = 0; !pending.empty(); ++widen) {
-      std::vector<int32_t> r;
-      std::vector<float> lo, hi;
-      for (int k : pending) {
-        const Window &w = windows[feasible[k]];
-        r.push_back(w.row);
-        lo.push_back(widen >= 8 ? -std::numeric_limits<float>::infinity() : w.lower_margin(widen));
-        hi.push_back(hi_first[k]);
+      if (widen > 0) {
+        std::vector<int32_t> r;
+        lo.clear();
+        hi.clear();
+        for (int k : pending) {
+          const Window &w = windows[feasible[k]];
+          r.push_back(w.row);
+          lo.push_back(widen >= 8 ? -std::numeric_limits<float>::infinity() : w.lower_margin(widen));
+          hi.push_back(hi_first[k]);
+        }
+        if (int rc = S.fetch(r, lo, hi, &got)) return rc;
       }
-      std::vector<Fetched> got;
-      if (int rc = S.fetch(r, lo, hi, &got)) return rc;
       std::vector<int> again;
       std::vector<float> kept;
       for (size_t j = 0; j < pending.size(); ++j) {
@@ -420,16 +625,16 @@ int mist_inter_stage_search(const MistDpShape *shape, const MistDpCosts *costs, 
       if (!windows[i].covers(kInf)) brief.push_back(&windows[i]);
     if (!brief.empty()) {
       std::vector<int32_t> r;
-      std::vector<float> lo, want;
+      std::vector<float> from, want;
       for (Window *w : brief) {
         r.push_back(w->row);
-        lo.push_back(w->hi);
+        from.push_back(w->hi);
         want.push_back(w->extension_target(kInf));
       }
-      std::vector<Fetched> got;
-      if (int rc = S.fetch(r, lo, want, &got)) return rc;
+      std::vector<Fetched> more;
+      if (int rc = S.fetch(r, from, want, &more)) return rc;
       for (size_t j = 0; j < brief.size(); ++j)
-        if (int rc = S.apply_extension(brief[j], got[j], want[j])) return rc;
+        if (int rc = S.apply_extension(brief[j], more[j], want[j])) return rc;
     }
   }
 
@@ -565,8 +770,11 @@ int mist_inter_stage_search(const MistDpShape *shape, const MistDpCosts *costs, 
     out_cost[t] = ch.best_cost;
     out_g[t] = ch.best_g;
     out_tmax[t] = ch.best_g >= 0 ? ch.best_t : 0.0f;
+    out_family[t] = -1;
     out_stages[t] = 0;
     for (int k = 0; k < S_max * 4; ++k) out_path[(size_t)t * S_max * 4 + k] = -1;
+    if (out_rows)
+      for (int k = 0; k < S_max; ++k) out_rows[(size_t)t * S_max + k] = -1;
     if (ch.best_g >= 0) winners.push_back(t);
   }
   if (only_best_path && !winners.empty()) {
@@ -584,19 +792,23 @@ int mist_inter_stage_search(const MistDpShape *shape, const MistDpCosts *costs, 
     }
     if (int rc = S.run(g, tm, MIST_DP_THRESHOLD, true)) return rc;
     const int n = (int)winners.size();
-    const float *h = S.ws->h_out.as<float>();
-    const int32_t *path = S.ws->h_path.as<int32_t>();
     for (int k = 0; k < n; ++k) {
       const int t = winners[k];
-      int32_t best_s;
-      std::memcpy(&best_s, h + k, sizeof(best_s));
-      const double again = S.total(k, n, grad_accum[chains[t].best_g]);
-      if (best_s < 0 || again != chains[t].best_cost)
+      int family = -1;
+      const double again = S.total(k, n, grad_accum[chains[t].best_g], &family);
+      if (family < 0 || again != chains[t].best_cost)
         return fail(MIST_E_INVALID, "back-pointer run of instance %d gives %.17g, the scan %.17g", t,
                     again, chains[t].best_cost);
+      int32_t best_s;
+      std::memcpy(&best_s, S.ws->h_out.as<float>() + (size_t)family * 3 * n + k, sizeof(best_s));
+      const size_t per = S.path_ints(family), at = S.path_offset(family, n) + (size_t)k * per;
+      out_family[t] = family;
       out_stages[t] = best_s;
-      std::memcpy(out_path + (size_t)t * S_max * 4, path + (size_t)k * S_max * 4,
-                  sizeof(int32_t) * S_max * 4);
+      std::memcpy(out_path + (size_t)t * S_max * 4, S.ws->h_path.as<int32_t>() + at,
+                  sizeof(int32_t) * per);
+      if (strategy)
+        std::memcpy(out_rows + (size_t)t * S_max, S.ws->h_rows.as<int32_t>() + at / 4,
+                    sizeof(int32_t) * per / 4);
     }
   }
   if (out_stats) {
@@ -604,8 +816,27 @@ int mist_inter_stage_search(const MistDpShape *shape, const MistDpCosts *costs, 
     out_stats[1] = S.fetches;
     out_stats[2] = S.selected;
     out_stats[3] = S.thresholds_run;
+    out_stats[4] = S.round_trips;
   }
   return 0;
+}
+
+int mist_inter_stage_search(const MistDpShape *shape, const MistDpCosts *costs, int n_instances,
+                            int n_grad_accum, const int32_t *rows, const int32_t *grad_accum,
+                            int only_best_path, double *out_cost, int32_t *out_g, float *out_tmax,
+                            int32_t *out_stages, int32_t *out_path, int64_t *out_stats,
+                            void *stream) {
+  if (!shape) return fail(MIST_E_INVALID, "null pointer argument");
+  if (shape->free_devices != 0)
+    return fail(MIST_E_INVALID, "a single family must be the per-mesh recurrence");
+  if (n_instances < 1) return fail(MIST_E_INVALID, "need at least one instance, got %d", n_instances);
+  std::vector<int32_t> family(n_instances);
+  int64_t stats[5] = {0, 0, 0, 0, 0};
+  const int rc = mist_inter_stage_search_families(
+      1, shape, costs, costs, nullptr, n_instances, n_grad_accum, rows, grad_accum, only_best_path,
+      out_cost, out_g, out_tmax, family.data(), out_stages, out_path, nullptr, stats, stream);
+  if (out_stats) std::memcpy(out_stats, stats, sizeof(int64_t) * 4);
+  return rc;
 }
 
 }  // extern "C"

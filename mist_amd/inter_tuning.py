@@ -34,7 +34,7 @@ FIRST_CHUNK = 48  # thresholds per G in the first speculative scan launch
 MAX_CHUNK = 4096  # most thresholds per G in one launch
 GAP = 1e-6        # inter_tuning.py:177
 _SELECT_HEAD = 1 << 16  # selected candidates read back together with their counts
-NATIVE_SEARCH = True     # per-mesh search through mist_inter_stage_search (False: the Python driver below)
+NATIVE_SEARCH = True     # search through mist_inter_stage_search_families (False: the Python driver below)
 
 
 def _stream(device) -> ctypes.c_void_p:
@@ -97,6 +97,14 @@ class _DpRunner:
             self._prepare_stage_minima(self.families[0])
         else:
             self.families = self._uniform_device_families(meshes, **uniform_device)
+        self.strategy_index = _lib.StrategyIndex(
+            num_layers=L, p_dim=P1, num_mesh=Q, sample_size=S, slot=slot)
+        for v in range(4):
+            assert dev_tabs.index[v].dtype == torch.int32
+            self.strategy_index.index[v] = dev_tabs.index[v].data_ptr()
+        for i, (n, m) in enumerate(meshes):
+            self.strategy_index.mesh_n[i], self.strategy_index.mesh_m[i] = n, m
+        self._tables = dev_tabs  # the pointers above stay valid as long as the runner lives
         self.launches = 0
         self.thresholds_run = 0
         self._all_costs = self._costs_struct()
@@ -740,55 +748,59 @@ def _solutions(runner: _DpRunner, results_list, bests, n_g, g_index, q_index, nu
 
 def _native_search(runner: _DpRunner, results_list, rows, Gs, n_g, g_index, q_index, num_layers,
                    slot, only_best, stats):
-    """The search of ``_search`` + the partitions of ``_solutions`` in one library call
-    (``mist_inter_stage_search``: the same steps without the interpreter between the dependent
-    GPU batches); the strategy rows of the stages are read back here."""
-    fam = runner.families[0]
+    """The search of ``_search`` + the partitions and strategy rows of ``_solutions`` in one
+    library call (``mist_inter_stage_search_families``: the same steps without the interpreter
+    between the dependent GPU batches, for the per-mesh family or the uniform-device families
+    of ``runner``); only the decoding of the strategy rows happens here."""
+    fams = runner.families
     n_inst = len(results_list)
     rows = np.ascontiguousarray(rows, dtype=np.int32)
     G_arr = np.array(Gs, dtype=np.int32)
+    shapes = np.concatenate([f.shape for f in fams])
+    costs = (_lib.DpCosts * len(fams))()
+    for i, f in enumerate(fams):
+        ctypes.memmove(ctypes.byref(costs[i]), ctypes.byref(f.costs_struct), ctypes.sizeof(_lib.DpCosts))
+    select = fams[0].costs_struct if len(fams) == 1 and fams[0].consumes_devices else runner._all_costs
+    s_max = max(f.S_max for f in fams)
     cost = np.empty(n_inst, dtype=np.float64)
     best_g = np.empty(n_inst, dtype=np.int32)
     best_t = np.empty(n_inst, dtype=np.float32)
+    family = np.empty(n_inst, dtype=np.int32)
     n_stages = np.empty(n_inst, dtype=np.int32)
-    path = np.empty((n_inst, fam.S_max, 4), dtype=np.int32)
-    counters = np.zeros(4, dtype=np.int64)
+    path = np.empty((n_inst, s_max, 4), dtype=np.int32)
+    strategy_row = np.empty((n_inst, s_max), dtype=np.int32)
+    counters = np.zeros(5, dtype=np.int64)
     t_0 = time.perf_counter()
     with torch.cuda.device(runner.device):
-        rc = runner.lib.mist_inter_stage_search(
-            ctypes.c_void_p(fam.shape.ctypes.data), ctypes.byref(fam.costs_struct), n_inst, len(Gs),
+        rc = runner.lib.mist_inter_stage_search_families(
+            len(fams), ctypes.c_void_p(shapes.ctypes.data), ctypes.cast(costs, ctypes.c_void_p),
+            ctypes.byref(select), ctypes.byref(runner.strategy_index), n_inst, len(Gs),
             ctypes.c_void_p(rows.ctypes.data), ctypes.c_void_p(G_arr.ctypes.data),
             1 if only_best else 0, ctypes.c_void_p(cost.ctypes.data),
             ctypes.c_void_p(best_g.ctypes.data), ctypes.c_void_p(best_t.ctypes.data),
-            ctypes.c_void_p(n_stages.ctypes.data), ctypes.c_void_p(path.ctypes.data),
+            ctypes.c_void_p(family.ctypes.data), ctypes.c_void_p(n_stages.ctypes.data),
+            ctypes.c_void_p(path.ctypes.data), ctypes.c_void_p(strategy_row.ctypes.data),
             ctypes.c_void_p(counters.ctypes.data), _stream(runner.device))
-    _lib.check(rc, "mist_inter_stage_search")
+    _lib.check(rc, "mist_inter_stage_search_families")
     t_1 = time.perf_counter()
-    partitions = {}
-    requests = []
-    for t in range(n_inst):
-        if best_g[t] < 0 or n_stages[t] <= 0:
-            continue
-        total, inter = _DpRunner._partition_of(float(cost[t]), fam, int(n_stages[t]), path[t])
-        partitions[t] = inter
-        g = g_index[Gs[int(best_g[t])]]
-        for i, ((l0, l1), (n, m), ckpt) in enumerate(inter):
-            variant, cell = _solution_cell(num_layers, g, len(inter) - i - 1, l0, l1, q_index[(n, m)], ckpt, slot)
-            requests.append((results_list[t], variant, cell))
-    strategy_rows = iter(IntraStageTunerOutput.solutions_at(requests)) if requests else iter(())
     out = []
     for t in range(n_inst):
         if best_g[t] < 0:
             out.append((float("inf"), None))
-        elif t not in partitions:
+            continue
+        if n_stages[t] <= 0:
             out.append((float(cost[t]), None))
-        else:
-            solution = [Gs[int(best_g[t])], []]
-            for (l0, l1), (n, m), ckpt in partitions[t]:
-                row = next(strategy_rows).tolist()
-                row[:6] = [int(x) for x in row[:6]]
-                solution[1].append((((l0, l1), (n, m), ckpt, 0), tuple(row)))
-            out.append((float(cost[t]), solution))
+            continue
+        fam = fams[int(family[t])]
+        _, inter = _DpRunner._partition_of(float(cost[t]), fam, int(n_stages[t]), path[t, :fam.S_max])
+        G = Gs[int(best_g[t])]
+        spaces = results_list[t].spaces
+        solution = [G, []]
+        for i, ((l0, l1), (n, m), ckpt) in enumerate(inter):
+            row = spaces[(g_index[G], q_index[(n, m)])].decode(np.array(int(strategy_row[t, i]))).tolist()
+            row[:6] = [int(x) for x in row[:6]]
+            solution[1].append((((l0, l1), (n, m), ckpt, 0), tuple(row)))
+        out.append((float(cost[t]), solution))
     if stats is not None:
         stats["dp_search_s"] = stats.get("dp_search_s", 0.0) + (t_1 - t_0)
         stats["dp_backtrack_s"] = stats.get("dp_backtrack_s", 0.0) + (time.perf_counter() - t_1)
@@ -796,6 +808,7 @@ def _native_search(runner: _DpRunner, results_list, rows, Gs, n_g, g_index, q_in
         stats["dp_window_fetches"] = stats.get("dp_window_fetches", 0) + int(counters[1])
         stats["dp_window_values"] = stats.get("dp_window_values", 0) + int(counters[2])
         stats["dp_thresholds"] = stats.get("dp_thresholds", 0) + int(counters[3])
+        stats["dp_round_trips"] = stats.get("dp_round_trips", 0) + int(counters[4])
     return out
 
 
@@ -846,7 +859,7 @@ def inter_stage_tune_batch(
     # table row of (instance, G)
     rows = np.array([[t * n_g + g_index[G] for G in Gs] for t in range(len(results_list))], dtype=np.int32)
     t_0 = time.perf_counter()
-    if uniform_device is None and NATIVE_SEARCH:
+    if NATIVE_SEARCH:
         out = _native_search(runner, results_list, rows, Gs, n_g, g_index, q_index, num_layers, slot,
                              only_best_solution, stats)
         if stats is not None:

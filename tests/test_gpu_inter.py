@@ -691,3 +691,41 @@ def test_native_search_equals_python_driver(monkeypatch, plan, overrides):
         assert out[True, only_best] == out[False, only_best]
     assert any(sol is not None for _, sol in out[True, False][0]) == (plan != 1 or overrides.get("hardware__memory_capacity") != 1.0)
 
+
+@pytest.mark.parametrize("plan, overrides, ckpt_tuning", [
+    (1, {}, True), (2, {}, True), (2, {}, False),
+    (1, dict(model__num_hidden_layers=6, hardware__num_nodes=2, hardware__num_gpus_per_node=4,
+             training__global_batch_size=32, hardware__memory_capacity=8.0), True),
+    (1, dict(model__num_hidden_layers=5, hardware__memory_capacity=1.0), True),  # nothing fits
+])
+def test_native_search_of_uniform_device_families_equals_python_driver(monkeypatch, plan, overrides,
+                                                                        ckpt_tuning):
+    """``mist_inter_stage_search_families`` with one DP family per admissible stage count (the
+    uniform-device recurrence) against the Python driver: costs, partitions, strategies and the
+    number of DP instances run."""
+    from mist_amd import inter_tuning
+    from mist_amd.config import tp_candidates
+    from mist_amd.intra_tuning import IntraStageTuner
+    from mist_amd.search_space import _get_device_mesh_candidates, _get_grad_accumu_steps_candidates
+
+    cfg, tables = load_plan(plan, **overrides)
+    hw, L = cfg.hardware, cfg.model.num_hidden_layers
+    D = hw.num_nodes * hw.num_gpus_per_node
+    meshes = _get_device_mesh_candidates(hw.num_nodes, hw.num_gpus_per_node, False)
+    Gs = _get_grad_accumu_steps_candidates(cfg.training.global_batch_size)
+    results = IntraStageTuner(tables, L, meshes, Gs, tp_candidates(cfg), cfg, sample_size=1).tune_all()
+    uniform = dict(num_nodes=hw.num_nodes, num_gpus_per_node=hw.num_gpus_per_node, ckpt_tuning=ckpt_tuning)
+    out = {}
+    for native in (True, False):
+        monkeypatch.setattr(inter_tuning, "NATIVE_SEARCH", native)
+        for only_best in (False, True):
+            stats = {}
+            got = inter_tuning.inter_stage_tune_batch(L, D, meshes, Gs, results, stats=stats,
+                                                      uniform_device=uniform,
+                                                      only_best_solution=only_best)
+            out[native, only_best] = (got, stats["dp_thresholds"], stats["dp_window_values"])
+    for only_best in (False, True):
+        assert out[True, only_best] == out[False, only_best]
+    feasible = any(sol is not None for _, sol in out[True, False][0])
+    assert feasible == (overrides.get("hardware__memory_capacity") != 1.0)
+

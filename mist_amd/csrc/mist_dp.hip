@@ -317,11 +317,16 @@ __device__ __forceinline__ void dp_finish_winner(DpBest &w, const MistDpShape &s
 
 // Scan of one state (start layer k, devices d) by one lane (member 0 of 1) or by its share of a
 // team: meshes q and end layers i in the reachable range of the successor column.
-// `row_min(q, i)` returns dp_row_min of the stage k..i on mesh q.
-template <bool kBottleneck, int kDpTeam, typename RowMin>
+// `row_min(q, i)` returns dp_row_min of the stage k..i on mesh q; `narrow(q, i_first, i_last)`
+// may shrink the range of end layers to one that still holds every i with row_min <= t_max.
+struct DpKeepRange {
+  __device__ __forceinline__ void operator()(int, int &, int &) const {}
+};
+template <bool kBottleneck, int kDpTeam, typename RowMin, typename Narrow = DpKeepRange>
 __device__ __forceinline__ void dp_scan_state(DpBest &w, const MistDpShape &shape, float t_max,
                                               int k, int d, int member, const float *f_prev,
-                                              const int32_t *range_prev, RowMin row_min) {
+                                              const int32_t *range_prev, RowMin row_min,
+                                              Narrow narrow = Narrow()) {
   const int L = shape.num_layers, W = shape.num_devices + 1;
   const bool free_devices = shape.free_devices != 0;
   for (int q = 0; q < shape.num_mesh; ++q) {
@@ -329,7 +334,8 @@ __device__ __forceinline__ void dp_scan_state(DpBest &w, const MistDpShape &shap
     if (nm > d) continue;
     // reachable start layers i + 1 of the remaining stages on d - nm devices
     const int32_t *reach = range_prev + 2 * (d - nm);
-    const int i_first = max(k, reach[0] - 1), i_last = min(L - 1, reach[1] - 1);
+    int i_first = max(k, reach[0] - 1), i_last = min(L - 1, reach[1] - 1);
+    narrow(q, i_first, i_last);
     if constexpr (kDpTeam == 1) {
       // One lane per state: the scan is a chain of reads.  kDpBatch end layers at a time, first
       // all their successor values, then the row minima of the reachable ones, so that the reads
@@ -483,6 +489,8 @@ __global__ __launch_bounds__(kDpFusedThreads) void dp_fused_kernel(
   // row minima of the current stage count: per mesh a triangle (k, i >= k)
   float *stage_min = dp_lds + 4 * plane + 6 * W;
   const int tri = dp_triangle(L), n_stage = shape.num_mesh * tri;
+  // first and last end layer of a stage on mesh q from layer k whose row minimum is <= t_max
+  int32_t *admissible = reinterpret_cast<int32_t *>(stage_min + n_stage);  // [Q][L][2]
   const int t = blockIdx.x;
   const float t_max = kBottleneck ? INFINITY : tmax_list[t];
   const int64_t g = g_list[t];
@@ -536,13 +544,38 @@ __global__ __launch_bounds__(kDpFusedThreads) void dp_fused_kernel(
       }
     }
     __syncthreads();
+    // Near the smallest feasible threshold only short stages are admissible: the end layers
+    // outside [first, last] fail "cost <= t_max" for every device count, so the scans of all
+    // states with this start layer skip them (what lies inside is still tested one by one).
+    if (!kBottleneck) {
+      for (int x = threadIdx.x; x < shape.num_mesh * L; x += blockDim.x) {
+        const int q = x / L, k0 = x % L;
+        const float *row = stage_min + q * tri + dp_triangle_row(L, k0) - k0;
+        int first = L, last = -1;
+        for (int i = k0; i < L; ++i) {
+          if (row[i] <= t_max) {
+            first = min(first, i);
+            last = i;
+          }
+        }
+        admissible[2 * x] = first;
+        admissible[2 * x + 1] = last;
+      }
+      __syncthreads();
+    }
     int k = k_first, d = d_first;
     for (int e = threadIdx.x; e < plane; e += blockDim.x) {
       DpBest w;
       if (k <= L - s && (d >= 1 || shape.free_devices != 0)) {
         const float *mine = stage_min + dp_triangle_row(L, k) - k;
         dp_scan_state<kBottleneck, 1>(w, shape, t_max, k, d, 0, f_prev, range_prev,
-                                      [&](int q, int i) { return mine[q * tri + i]; });
+                                      [&](int q, int i) { return mine[q * tri + i]; },
+                                      [&](int q, int &i_first, int &i_last) {
+                                        if (kBottleneck) return;
+                                        const int32_t *a = admissible + 2 * (q * L + k);
+                                        i_first = max(i_first, a[0]);
+                                        i_last = min(i_last, a[1]);
+                                      });
         dp_finish_winner<kBottleneck>(w, shape, tabs, off, t_max, p, k, d, f_prev, m_prev);
       }
       f_cur[e] = w.best;
@@ -1176,7 +1209,8 @@ int mist_dp_run(const MistDpShape *shape, const MistDpCosts *costs, const float 
   // prepared the re-laid row minima.
   const size_t fused_lds =
       ((size_t)4 * plane + (size_t)6 * (shape->num_devices + 1) +
-       (size_t)shape->num_mesh * dp_triangle(shape->num_layers)) *
+       (size_t)shape->num_mesh * dp_triangle(shape->num_layers) +
+       (size_t)2 * shape->num_mesh * shape->num_layers) *
       sizeof(float);
   // (threshold batches from about 64 instances on: a workgroup's run through all stage counts
   // takes as long as the 1 + max_stages launches of a few dozen instances)

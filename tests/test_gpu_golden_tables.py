@@ -2,8 +2,9 @@
 
 tests/golden/search_tables_plan<N>.json (written by tests/golden/make_search_fixtures.py on the
 CPU) holds, per (tp, G, mesh) group of a benchmark plan, a digest of each of the oracle's four
-result tables (row indices + float32 stable / delta costs) and, where every group of the plan is
-covered, the oracle's end-to-end search result.  Here the HIP kernels search the whole plan in
+result tables (row indices + float32 stable / delta costs) and the oracle's end-to-end search
+result: over the whole plan (``tune``) or, for the two largest plans, over the winning
+tensor-parallel size and two gradient-accumulation candidates (``tune_scoped``).  Here the HIP kernels search the whole plan in
 one batch (scout pass, row chunks, p tiles, sieves: everything the timed workload uses), the
 same digests are taken from their tables and compared, and ``tune`` must return the oracle's
 cost (bit-equal float64) and strategy.
@@ -42,10 +43,9 @@ def test_fixtures_cover_every_benchmark_plan():
 
 @pytest.mark.parametrize("plan", [1, 2, 3, 4, 5])
 def test_pruned_and_exhaustive_search_give_the_same_tables_on_whole_plans(plan):
-    """Every table of every group of a benchmark plan (plan 2 is the timed workload; of plan 4
-    the oracle's fixtures cover a part of the groups only), pruned search (scout pass,
-    sieves, bounds) against the kernel that evaluates every cell: identical row indices and
-    costs."""
+    """Every table of every group of a benchmark plan (plan 2 is the timed workload), pruned
+    search (scout pass, sieves, bounds) against the kernel that evaluates every cell: identical
+    row indices and costs."""
     import torch
 
     from mist_amd.tune_one_case import PreparedSearch
@@ -104,9 +104,20 @@ def test_tables_and_tune_equal_the_oracle_fixture(path, exhaustive):
     assert n_groups == len(fixture["groups"])
     assert not bad, f"{len(bad)} of {4 * n_groups} tables differ from the oracle: {bad[:8]}"
 
+    hw = cfg.hardware
+    if "tune_scoped" in fixture:
+        # the oracle's sequential threshold scan restricted to one tensor-parallel size and a
+        # few G (the whole scan of a large plan takes the CPU hours): same restriction here
+        scoped = fixture["tune_scoped"]
+        tp, scope_Gs = scoped["scope"]["tp"], scoped["scope"]["Gs"]
+        cost, solution = inter_stage_tune_batch(
+            search.L, hw.num_nodes * hw.num_gpus_per_node, meshes, scope_Gs,
+            [results[tuner.tp_sizes.index(tp)]], slot=0)[0]
+        assert cost == float(scoped["cost"]), (cost, scoped["cost"])
+        assert _listify(solution) == scoped["solution"]
+        assert solution is not None
     if "tune" not in fixture:
         return
-    hw = cfg.hardware
     outcomes = inter_stage_tune_batch(
         search.L, hw.num_nodes * hw.num_gpus_per_node, meshes, Gs, results, slot=0, only_best_solution=False)
     for tp, (cost, solution) in zip(tuner.tp_sizes, outcomes):

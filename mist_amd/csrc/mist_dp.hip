@@ -33,6 +33,7 @@ constexpr int kDpFusedMinInstances = 64;  // threshold batches of at least this 
 constexpr int kDpStageBatch = 8;   // row minima a lane copies together in the one-launch kernel
 constexpr int kSelectBatch = 8;  // table values a lane of the candidate selection reads together
 constexpr int kSelectBuffer = 4096;  // selected values a workgroup holds before it appends them
+constexpr float kDpNoThreshold = 3.402823466e+38f;  // FLT_MAX: admits every finite stage cost
 constexpr int kDpBatch = 4;  // end layers whose reads a lane of the one-lane-per-state kernel overlaps
 
 // ------------------------------------------------------------------------------------------
@@ -315,6 +316,66 @@ __device__ __forceinline__ void dp_finish_winner(DpBest &w, const MistDpShape &s
   }
 }
 
+// Upper bound of the smallest feasible threshold, for the bottleneck DP of one instance: the
+// largest stage cost of any partition bounds the min-max optimum from above, and a stage that
+// costs more than such a bound is on no min-max partition, so the bottleneck DP may treat it as
+// inadmissible (same value, same first-wins path: every candidate it drops has a target above
+// the optimum).  The bound is the min-max optimum over the partitions that put every stage on
+// the same mesh q (n m s = D stages, or any s <= max_stages when stages do not consume devices)
+// with the layers split freely: a recurrence over (stage count, start layer) alone,
+//   B(s, k) = min over i >= k of max(cost(s, k, i, q), B(s - 1, i + 1)),
+// one wavefront per mesh, its two rows of B in `rows` (LDS, 2 (L + 1) of its `n_rows` floats per
+// wavefront).  Called by the whole workgroup; `slot` is one int of LDS.  +inf when no such
+// partition is feasible (or L > 128: a lane holds two start layers; or `rows` is too small).
+__device__ __forceinline__ float dp_uniform_mesh_bound(const MistDpShape &shape,
+                                                       const float *__restrict__ relaid,
+                                                       float *rows, int n_rows, int32_t *slot) {
+  const int L = shape.num_layers, D = shape.num_devices, Q = shape.num_mesh;
+  const int tri = dp_triangle(L);
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int n_waves = (blockDim.x + 63) >> 6;
+  if (threadIdx.x == 0) *slot = __float_as_int(INFINITY);
+  __syncthreads();
+  if (L <= 128 && n_waves * 2 * (L + 1) <= n_rows) {
+    float *prev = rows + wave * 2 * (L + 1), *cur = prev + (L + 1);
+    for (int q = wave; q < Q; q += n_waves) {
+      int s_last = shape.max_stages;
+      if (shape.free_devices == 0) {
+        const int nm = shape.mesh_n[q] * shape.mesh_m[q];
+        if (nm <= 0 || D % nm != 0 || D / nm > shape.max_stages) continue;
+        s_last = D / nm;
+      }
+      if (s_last > L) continue;
+      for (int k = lane; k <= L; k += 64) prev[k] = k == L ? 0.0f : INFINITY;
+      __builtin_amdgcn_wave_barrier();
+      float bound = INFINITY;
+      for (int s = 1; s <= s_last; ++s) {
+        const float *__restrict__ block = relaid + ((int64_t)(s - 1) * Q + q) * tri;
+        for (int k = lane; k <= L; k += 64) {
+          float best = INFINITY;
+          if (k <= L - s) {
+            const float *__restrict__ row = block + dp_triangle_row(L, k) - k;  // row[i]
+            // the s - 1 stages behind this one take a layer each at least
+            for (int i = k; i <= L - s; ++i) best = fminf(best, fmaxf(row[i], prev[i + 1]));
+          }
+          cur[k] = best;
+        }
+        __builtin_amdgcn_wave_barrier();
+        if (shape.free_devices != 0 || s == s_last) bound = fminf(bound, cur[0]);
+        float *swap = prev;
+        prev = cur;
+        cur = swap;
+        __builtin_amdgcn_wave_barrier();
+      }
+      // stage costs are not negative, and non-negative floats order like their bit patterns
+      if (lane == 0 && bound >= 0.0f && bound < INFINITY) atomicMin(slot, __float_as_int(bound));
+    }
+  }
+  __syncthreads();
+  return __int_as_float(*slot);
+}
+
 // Scan of one state (start layer k, devices d) by one lane (member 0 of 1) or by its share of a
 // team: meshes q and end layers i in the reachable range of the successor column.
 // `row_min(q, i)` returns dp_row_min of the stage k..i on mesh q; `narrow(q, i_first, i_last)`
@@ -390,7 +451,9 @@ __global__ __launch_bounds__(kDpThreads) void dp_step_kernel(
   const float *__restrict__ m_prev = state + (2 + prv) * plane;
   float *__restrict__ f_cur = state + cur * plane;
   float *__restrict__ m_cur = state + (2 + cur) * plane;
-  const float t_max = kBottleneck ? INFINITY : tmax_list[t];
+  // bottleneck mode has no threshold; the largest finite value skips the +inf entries, which
+  // improve no state (inf is never < best)
+  const float t_max = kBottleneck ? kDpNoThreshold : tmax_list[t];
   const int64_t g = g_list[t];
   const int64_t off[4] = {g * tabs.g_stride[0], g * tabs.g_stride[1], g * tabs.g_stride[2],
                           g * tabs.g_stride[3]};
@@ -492,11 +555,17 @@ __global__ __launch_bounds__(kDpFusedThreads) void dp_fused_kernel(
   // first and last end layer of a stage on mesh q from layer k whose row minimum is <= t_max
   int32_t *admissible = reinterpret_cast<int32_t *>(stage_min + n_stage);  // [Q][L][2]
   const int t = blockIdx.x;
-  const float t_max = kBottleneck ? INFINITY : tmax_list[t];
   const int64_t g = g_list[t];
   const int64_t off[4] = {g * tabs.g_stride[0], g * tabs.g_stride[1], g * tabs.g_stride[2],
                           g * tabs.g_stride[3]};
   const float *__restrict__ relaid = tabs.stage_min + g * tabs.stage_min_g_stride;
+  // the bottleneck DP has no threshold of its own: an upper bound of its answer serves as one
+  // (not with back-pointers: then every state gets the entry the unbounded recurrence gives it)
+  const float t_max = !kBottleneck       ? tmax_list[t]
+                      : argmin != nullptr
+                          ? kDpNoThreshold
+                          : fminf(kDpNoThreshold,
+                                  dp_uniform_mesh_bound(shape, relaid, stage_min, n_stage, admissible));
   // F(0, ., .): 0 at (k = L, d = 0), +inf elsewhere; maxima start at 0; only that state is
   // reachable.
   for (int e = threadIdx.x; e < plane; e += blockDim.x) {
@@ -547,7 +616,7 @@ __global__ __launch_bounds__(kDpFusedThreads) void dp_fused_kernel(
     // Near the smallest feasible threshold only short stages are admissible: the end layers
     // outside [first, last] fail "cost <= t_max" for every device count, so the scans of all
     // states with this start layer skip them (what lies inside is still tested one by one).
-    if (!kBottleneck) {
+    {
       for (int x = threadIdx.x; x < shape.num_mesh * L; x += blockDim.x) {
         const int q = x / L, k0 = x % L;
         const float *row = stage_min + q * tri + dp_triangle_row(L, k0) - k0;
@@ -571,7 +640,6 @@ __global__ __launch_bounds__(kDpFusedThreads) void dp_fused_kernel(
         dp_scan_state<kBottleneck, 1>(w, shape, t_max, k, d, 0, f_prev, range_prev,
                                       [&](int q, int i) { return mine[q * tri + i]; },
                                       [&](int q, int &i_first, int &i_last) {
-                                        if (kBottleneck) return;
                                         const int32_t *a = admissible + 2 * (q * L + k);
                                         i_first = max(i_first, a[0]);
                                         i_last = min(i_last, a[1]);
@@ -650,12 +718,20 @@ __global__ __launch_bounds__(kDpPlaneThreads) void dp_plane_kernel(
   int32_t *reach_q = range + 6 * W;                              // [Q][2] the same per mesh, all columns
   float *wave_rows = reinterpret_cast<float *>(reach_q + 2 * Q);  // [n_waves][Q][L] row minima of a task
   const int t = blockIdx.x;
-  const float t_max = kBottleneck ? INFINITY : tmax_list[t];
   const int64_t g = g_list[t];
   const int64_t off[4] = {g * tabs.g_stride[0], g * tabs.g_stride[1], g * tabs.g_stride[2],
                           g * tabs.g_stride[3]};
   const int tri = dp_triangle(L);
   const float *__restrict__ relaid = tabs.stage_min + g * tabs.stage_min_g_stride;
+  // the bottleneck DP has no threshold of its own: an upper bound of its answer serves as one
+  // (reach_q is free until the first stage count)
+  // (not with back-pointers: then every state gets the entry the unbounded recurrence gives it)
+  const float t_max = !kBottleneck       ? tmax_list[t]
+                      : argmin != nullptr
+                          ? kDpNoThreshold
+                          : fminf(kDpNoThreshold,
+                                  dp_uniform_mesh_bound(shape, relaid, wave_rows,
+                                                        (int)(blockDim.x >> 6) * Q * L, reach_q));
   float *state = scratch + (int64_t)t * 4 * plane;
   float *__restrict__ f_cur = state;  // F(s) on its way into LDS
   const int lane = threadIdx.x & 63;

@@ -373,7 +373,8 @@ def main():
     counters = profile_counters()
     # the counters belong to the kernel sources and the launch decomposition they were taken
     # with: a profile of other sources or another grid gives no executed-work figures
-    main_waves = int(search.plan["reduce_prefix"][-1])
+    # (the launch pads its grid to whole runs of 16 workgroups on each of the 8 XCDs)
+    main_waves = -(-int(search.plan["reduce_prefix"][-1]) // 128) * 128
     counters_stale = bool(counters) and (
         counters.pop("_source_sha256", None) != kernel_source_sha256()
         or int(counters.get("SQ_WAVES", {}).get("exhaustive", -1)) != main_waves)

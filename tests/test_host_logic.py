@@ -196,7 +196,7 @@ def test_workspace_batches_partition_the_groups(monkeypatch):
             assert np.array_equal(keys * whole["n_oo"], whole["n_rows"])
             assert sub["key_offset"][0] == 0 and np.array_equal(np.diff(sub["key_offset"]), keys[:-1])
             assert b["total_keys"] == int(keys.sum())
-            assert int(plan["problem"]["max_group_keys"]) >= int(keys.max())
+            assert int(plan["problem"]["max_group_keys"][0]) >= int(keys.max())
             for name in ("terms_prefix", "reduce_prefix", "scout_prefix"):
                 assert b[name][0] == 0 and len(b[name]) == len(sub) + 1
                 assert np.array_equal(np.diff(b[name]), np.diff(plan[name][b["first"]:b["last"] + 1]))

@@ -226,14 +226,19 @@ def other_plans():
 
 def mip_searches(plans=("gpt-7b-b512-4x8.yaml", "llama-13b-b1024-8x8.yaml"), sample_size=30):
     """``tune()`` with the reference's default granularity at HEAD, ``uniform-device-pp-mip``
-    with 30 alpha samples per cell (mist/utils/pareto.py:124-144, inter_tuning_mip.py): every
-    sample of every cell of every tensor-parallel candidate, then the stage assignment.  Whole
-    call from the configuration object (descriptor building included), median of 3."""
+    with 30 alpha samples per cell (mist/utils/pareto.py:124-144, inter_tuning_mip.py), then the
+    stage assignment.  Whole call from the configuration object (descriptor building included),
+    median of 3.  ``tune_s``: as ``tune`` runs it, with the intra-stage tables evaluated where
+    the assignment reads them (the layer counts within ``layers_offset`` of a stage count's
+    average, on that stage count's mesh); ``tune_all_cells_s``: with every sample of every cell
+    of every tensor-parallel candidate, as the reference's IntraStageTuner fills its tables.
+    Same cost and strategy either way (asserted)."""
     import hashlib
 
     import torch
     import yaml
 
+    from mist_amd import tune_one_case
     from mist_amd.config import MistConfig
     from mist_amd.tune_one_case import tune
 
@@ -242,19 +247,29 @@ def mip_searches(plans=("gpt-7b-b512-4x8.yaml", "llama-13b-b1024-8x8.yaml"), sam
         with open(os.path.join(REPO, "mist_amd", "configs", name)) as f:
             raw = yaml.safe_load(f)
         raw["tuning"].update(tuning_granularity="uniform-device-pp-mip", sample_size=sample_size)
-        tune(MistConfig(raw))  # warm-up: buffers of this size
-        torch.cuda.synchronize()
-        times = []
-        for _ in range(3):
-            t0 = time.perf_counter()
-            cost, solution = tune(MistConfig(raw))
-            torch.cuda.synchronize()
-            times.append(time.perf_counter() - t0)
-        out[name] = dict(tune_s=sorted(times)[1], sample_size=sample_size, cost=cost,
+        timing, answers = {}, []
+        for key, all_cells in (("tune_all_cells_s", True), ("tune_s", False)):
+            tune_one_case.MIP_EVALUATE_ALL_CELLS = all_cells
+            try:
+                tune(MistConfig(raw))  # warm-up: buffers of this size
+                torch.cuda.synchronize()
+                times = []
+                for _ in range(3):
+                    t0 = time.perf_counter()
+                    cost, solution = tune(MistConfig(raw))
+                    torch.cuda.synchronize()
+                    times.append(time.perf_counter() - t0)
+            finally:
+                tune_one_case.MIP_EVALUATE_ALL_CELLS = False
+            timing[key] = sorted(times)[1]
+            answers.append((cost, solution))
+            torch.cuda.empty_cache()
+        assert answers[0] == answers[1], "restricted and full tables give different strategies"
+        out[name] = dict(tune_s=timing["tune_s"], tune_all_cells_s=timing["tune_all_cells_s"],
+                         sample_size=sample_size, cost=cost,
                          grad_accum=solution[0] if solution else None,
                          stages=len(solution[1]) if solution else 0,
                          solution_sha256=hashlib.sha256(repr(solution).encode()).hexdigest()[:16])
-        torch.cuda.empty_cache()
     return out
 
 

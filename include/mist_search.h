@@ -112,6 +112,12 @@ typedef struct MistGroupDesc {
   int32_t n_par, n_pair, n_oo, n_ao, n_off;
   int32_t pp_wre, pp_gre;       /* ZeRO flags of the pre/post layer strategy */
   int32_t rows_per_chunk, n_chunks, n_lc_tiles, n_p_tiles; /* decomposition of the reduce kernel */
+  int32_t lc_tile_begin;        /* the group's n_lc_tiles tiles of 64 (layers, ckpt) pairs start at
+                                 * this tile of the pair list: 0 with all tiles for the whole
+                                 * tables; a caller that reads a range of layer counts only (the
+                                 * stage assignment of inter_tuning_mip.py:282-290) evaluates the
+                                 * tiles that hold it, the cells of the other tiles keep their
+                                 * pre-filled +inf / -1 */
   int32_t scout_stride;         /* reduce kernel: 0 = no scout pass for this group; m >= 1 = the
                                  * scout pass reduces the rows of the m (weight, gradient) offload
                                  * pairs scout_pair[0 .. m-1] (n_par * n_oo * n_ao rows each) */

@@ -73,7 +73,7 @@ GROUP_DTYPE = np.dtype(
         ("n_par", "<i4"), ("n_pair", "<i4"), ("n_oo", "<i4"), ("n_ao", "<i4"), ("n_off", "<i4"),
         ("pp_wre", "<i4"), ("pp_gre", "<i4"),
         ("rows_per_chunk", "<i4"), ("n_chunks", "<i4"), ("n_lc_tiles", "<i4"),
-        ("n_p_tiles", "<i4"), ("scout_stride", "<i4"),
+        ("n_p_tiles", "<i4"), ("lc_tile_begin", "<i4"), ("scout_stride", "<i4"),
         ("scout_pair", "<i2", (MAX_SCOUT_PAIRS,)),
         ("n_rows", "<i8"), ("row_offset", "<i8"), ("key_offset", "<i8"),
         ("par", "<f8", (MAX_PAR, PAR_FIELDS)),

@@ -1658,7 +1658,7 @@ __global__ __launch_bounds__(MIST_LC_TILE, MIST_REDUCE_MIN_WAVES) void eval_redu
     skip_unchanged = chunk > 0;
   }
   const int p_tile = tile % g->n_p_tiles;
-  const int lc_tile = tile / g->n_p_tiles;
+  const int lc_tile = g->lc_tile_begin + tile / g->n_p_tiles;  // position in the pair list
   const int64_t slab = (int64_t)kSlots * MIST_LC_TILE;
   const int64_t seed_slab = scout_base + (int64_t)sample * n_scout_total +
                             (seeded ? scout_prefix[gi] + tile * kScoutSplit : 0);
@@ -1812,7 +1812,7 @@ __global__ __launch_bounds__(MIST_LC_TILE, MIST_EXHAUSTIVE_MIN_WAVES) void eval_
   const int chunk = local_block / n_tiles, tile = local_block % n_tiles;
   const int64_t row_begin = (int64_t)chunk * g->rows_per_chunk;
   const int64_t row_end = min(row_begin + (int64_t)g->rows_per_chunk, g->n_rows);
-  const int p_tile = tile % g->n_p_tiles, lc_tile = tile / g->n_p_tiles;
+  const int p_tile = tile % g->n_p_tiles, lc_tile = g->lc_tile_begin + tile / g->n_p_tiles;
   const int64_t slab = (int64_t)kSlots * MIST_LC_TILE;
   if (p_tile == 0)
     exhaustive_block<true>(prob, g, row_begin, row_end, p_tile, lc_tile, row_terms, ratio,
@@ -1879,7 +1879,9 @@ __global__ __launch_bounds__(256) void finalize_kernel(
   if (variant == 2 && c == l - 1) return;
   if (variant == 3 && (l != L || c == L - 1)) return;
 
-  const int lc_tile = pair_idx / MIST_LC_TILE, lane = pair_idx % MIST_LC_TILE;
+  // the group's tiles are a window of the pair list; cells outside were not evaluated
+  const int lc_tile = pair_idx / MIST_LC_TILE - g->lc_tile_begin, lane = pair_idx % MIST_LC_TILE;
+  if (lc_tile < 0 || lc_tile >= g->n_lc_tiles) return;
   const int p_tile = p / MIST_P_TILE;
   int kslot;
   if (variant == 0) kslot = p % MIST_P_TILE;

@@ -48,6 +48,27 @@ def layer_candidates(num_layers: int, num_stages: int, grad_accum: int, layers_o
     return max(avg - layers_offset, 1), min(avg + layers_offset, num_layers - num_stages + 1)
 
 
+def cells_wanted(num_layers: int, num_nodes: int, num_gpus_per_node: int, layers_offset: int = 2):
+    """What the assignment reads of the intra-stage tables of a (G, mesh) group, for
+    ``IntraStageTuner.cells_wanted``: a mesh is read for the one stage count S whose even split
+    of the cluster it is (inter_tuning_mip.py:267-281), there for the layer counts of
+    ``layer_candidates`` and the pre-saved micro-batch values 0..S-1 (stage i of S keeps S - i - 1);
+    a mesh that is no such split is not read at all."""
+    num_devices = num_nodes * num_gpus_per_node
+
+    def wanted(G: int, mesh: Tuple[int, int]):
+        n, m = mesh
+        if n * m <= 0 or num_devices % (n * m) != 0:
+            return None
+        S = num_devices // (n * m)
+        if S > num_layers or _uniform_device_mesh_partition(S, num_nodes, num_gpus_per_node) != mesh:
+            return None
+        lo, hi = layer_candidates(num_layers, S, G, layers_offset)
+        return (lo, hi, S) if hi >= lo else None
+
+    return wanted
+
+
 class _Problem:
     """One (G, S) assignment problem: its shape and where its samples lie in the batch buffers."""
 

@@ -247,6 +247,12 @@ class IntraStageTuner:
         # True: every p of 0..P is evaluated for every G (the operator boundary
         # batched_tune_best_latency_for_stage takes the p candidates from its caller)
         self.evaluate_all_p = False
+        # Optional ``cells_wanted(G, (n, m)) -> None | (l_min, l_max, p_count)``: a caller that
+        # reads only a range of layer counts and the first ``p_count`` pre-saved micro-batch
+        # values of a (G, mesh) group - or nothing of it (None) - has only the tiles of (layers,
+        # ckpt) pairs that hold them evaluated; every other cell keeps its pre-filled inf / -1.
+        # The evaluated cells are the same as without it.
+        self.cells_wanted = None
         self.results: Optional[IntraStageTunerOutput] = None
         self.stats: Dict[str, float] = {}
 
@@ -262,6 +268,8 @@ class IntraStageTuner:
         pending = []
         factory = SearchSpaceFactory(cfg, self.layer_tables.constraint)
         B = cfg.training.global_batch_size
+        n_pairs = L * (L + 1) // 2 + L
+        tile_window = []  # per group: first tile of its (layers, ckpt) pairs and how many
         for t, tp_size in enumerate(self.tp_sizes):
             for g, G in enumerate(Gs):
                 for q, (n, m) in enumerate(Q):
@@ -274,19 +282,34 @@ class IntraStageTuner:
                     num_p = min(G, L, P + 1)  # intra_tuning.py:185-193
                     if self.evaluate_all_p:
                         num_p = P + 1
+                    window = (0, -(-n_pairs // _lib.LC_TILE))
+                    if self.cells_wanted is not None:
+                        wanted = self.cells_wanted(G, (n, m))
+                        if wanted is None:
+                            continue
+                        l_min, l_max, p_count = wanted
+                        l_min, l_max = max(int(l_min), 1), min(int(l_max), L)
+                        if l_min > l_max or p_count < 1:
+                            continue
+                        num_p = min(num_p, int(p_count))
+                        # pairs are numbered l-major: index(l, c) = l (l + 1) / 2 - 1 + c
+                        first = (l_min * (l_min + 1) // 2 - 1) // _lib.LC_TILE
+                        last = (l_max * (l_max + 1) // 2 - 1 + l_max) // _lib.LC_TILE
+                        window = (first, last - first + 1)
+                    tile_window.append(window)
                     pending.append((t * len(Gs) + g, q, n, m, G, num_p, space))
         groups = np.zeros(len(pending), dtype=_lib.GROUP_DTYPE)
         builder.fill_many(groups, pending)
         builder.validate(groups)
 
-        n_pairs = L * (L + 1) // 2 + L
-        n_lc_tiles = -(-n_pairs // _lib.LC_TILE)
         if len(pending):
+            groups["lc_tile_begin"] = [w[0] for w in tile_window]
+            n_lc_tiles = np.array([w[1] for w in tile_window], dtype=np.int64)
             n_p_tiles = -(-groups["num_p"] // _lib.P_TILE)
             # the row chunks are sized per batch of groups (one reduce launch each, see below)
             for first, last in self._batch_bounds(groups["n_rows"]):
                 sel = slice(first, last)
-                tile_rows = int(np.sum(groups["n_rows"][sel] * n_lc_tiles * n_p_tiles[sel]))
+                tile_rows = int(np.sum(groups["n_rows"][sel] * n_lc_tiles[sel] * n_p_tiles[sel]))
                 rows_per_chunk = -(-tile_rows // max(TARGET_REDUCE_WAVES * 64 // _lib.LC_TILE, 1))
                 rows_per_chunk = max(256, min(16384, -(-rows_per_chunk // _lib.STAGE_ROWS) * _lib.STAGE_ROWS))
                 groups["rows_per_chunk"][sel] = rows_per_chunk
@@ -319,7 +342,7 @@ class IntraStageTuner:
                 picked = _scout_pairs(groups[i], int(groups["scout_stride"][i]))
                 groups["scout_stride"][i] = len(picked)
                 groups["scout_pair"][i, :len(picked)] = picked
-            scout_blocks = np.full(len(pending), n_lc_tiles * _lib.SCOUT_SPLIT, dtype=np.int64) * n_p_tiles
+            scout_blocks = n_lc_tiles * _lib.SCOUT_SPLIT * n_p_tiles
             if not np.any(groups["scout_stride"] > 0):
                 scout_blocks[:] = 0
         else:

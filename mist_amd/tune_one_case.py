@@ -35,6 +35,7 @@ from .config import OFFLOADING_RATIO_CANDIDATES, MistConfig, tp_candidates
 from .inter_tuning import inter_stage_tune, inter_stage_tune_batch
 from .inter_tuning_uniform import inter_stage_tune as inter_stage_tune_uniform
 from .inter_tuning_uniform_device import inter_stage_tune_batch_uniform_device
+from .inter_tuning_mip import cells_wanted as mip_cells_wanted
 from .inter_tuning_mip import inter_stage_tune as inter_stage_tune_mip
 from .intra_tuning import SAMPLE_SIZE, IntraStageTuner, intra_stage_tune
 from .layer_tables import LayerTables
@@ -102,6 +103,13 @@ def _no_pp(mist_config, tables, device, stats):
 MIP_TABLE_BUDGET_BYTES = 48 << 30  # sampled tables of one batch of tensor-parallel candidates
 
 
+# The stage assignment reads a few layer counts per (G, mesh) group (the stage count's average
+# +- tuning.layers_offset): by default only the tiles of the intra-stage tables that hold them
+# are evaluated.  True: the whole tables, as the reference's IntraStageTuner fills them (same
+# result; what the fixtures of all 30 samples are compared with).
+MIP_EVALUATE_ALL_CELLS = False
+
+
 def _uniform_device_pp_mip(mist_config, device, stats):
     """tune_one_case.py:360-402: per tensor-parallel candidate the intra-stage tables with every
     one of ``tuning.sample_size`` samples, then the stage assignment; the first best tp wins.
@@ -121,6 +129,9 @@ def _uniform_device_pp_mip(mist_config, device, stats):
         t0 = time.perf_counter()
         tuner = IntraStageTuner(tables, L, meshes, Gs, tps[first:first + batch], mist_config,
                                 sample_size=tuning.sample_size, device=device)
+        if not MIP_EVALUATE_ALL_CELLS:
+            tuner.cells_wanted = mip_cells_wanted(
+                L, hw.num_nodes, hw.num_gpus_per_node, int(getattr(tuning, "layers_offset", 2)))
         results = tuner.tune_all()
         t1 = time.perf_counter()
         stats["intra_s"] = stats.get("intra_s", 0.0) + (t1 - t0)

@@ -220,3 +220,92 @@ def test_mip_full_size_invariants(plan):
         D.append(max(np.float32(res.device.delta[v][cell].item()), np.float32(0)))
         assert np.array_equal(res.solution_at(v, cell), np.asarray(row, dtype=np.float64))
     assert objective(T, D, G) == pytest.approx(cost, rel=1e-12, abs=0)
+
+
+@pytest.mark.parametrize("plan, samples, overrides", [
+    (1, 30, {}),
+    (2, 3, {}),
+    (1, 4, dict(model__num_hidden_layers=9, hardware__num_nodes=2, hardware__num_gpus_per_node=4,
+                training__global_batch_size=32, hardware__memory_capacity=10.0)),
+])
+def test_tables_restricted_to_the_cells_the_assignment_reads(monkeypatch, plan, samples, overrides):
+    """``IntraStageTuner.cells_wanted`` with the assignment's own description of what it reads
+    (inter_tuning_mip.py:267-290): every cell inside the evaluated tile windows equals the full
+    tables, every other cell keeps inf / -1, the windows hold every cell the assignment reads,
+    and ``tune`` returns the same cost and strategy either way."""
+    import torch
+
+    from mist_amd import _lib, tune_one_case
+    from mist_amd.inter_tuning_mip import cells_wanted, layer_candidates
+    from mist_amd.inter_tuning_uniform import _uniform_device_mesh_partition
+    from mist_amd.intra_tuning import IntraStageTuner
+    from mist_amd.search_space import _get_device_mesh_candidates, _get_grad_accumu_steps_candidates
+    from mist_amd.tune_one_case import tp_candidates
+
+    cfg, tables = load_plan(plan, tuning__tuning_granularity="uniform-device-pp-mip",
+                            tuning__sample_size=samples, **overrides)
+    hw, L = cfg.hardware, cfg.model.num_hidden_layers
+    D = hw.num_nodes * hw.num_gpus_per_node
+    meshes = _get_device_mesh_candidates(hw.num_nodes, hw.num_gpus_per_node, False)
+    Gs = _get_grad_accumu_steps_candidates(cfg.training.global_batch_size)
+    tps = tp_candidates(cfg)
+    full = IntraStageTuner(tables, L, meshes, Gs, tps, cfg, sample_size=samples).tune_all()[0].batch
+    tuner = IntraStageTuner(tables, L, meshes, Gs, tps, cfg, sample_size=samples)
+    wanted = tuner.cells_wanted = cells_wanted(L, hw.num_nodes, hw.num_gpus_per_node)
+    part = tuner.tune_all()[0].batch
+
+    # which (table row, mesh, layers) were evaluated, from the plan's tile windows
+    P1 = full.stable[0].shape[2]
+    evaluated = np.zeros((len(tps) * len(Gs), len(meshes), L + 1), dtype=bool)  # [g][q][l]
+    p_count = np.zeros((len(tps) * len(Gs), len(meshes)), dtype=np.int64)
+    window = {}  # (table row, mesh) -> first and last pair of the evaluated tiles
+    for rec in tuner._plan["groups"]:
+        first = int(rec["lc_tile_begin"]) * _lib.LC_TILE
+        last = first + int(rec["n_lc_tiles"]) * _lib.LC_TILE - 1
+        window[int(rec["g_index"]), int(rec["q_index"])] = (first, last)
+        for l in range(1, L + 1):
+            lo, hi = l * (l + 1) // 2 - 1, l * (l + 1) // 2 - 1 + l
+            # a layer count whose pairs straddle a window's edge is evaluated for some ckpt
+            # counts only: compared where it lies inside as a whole
+            evaluated[rec["g_index"], rec["q_index"], l] = first <= lo and hi <= last
+        p_count[rec["g_index"], rec["q_index"]] = rec["num_p"]
+    n_inside = n_outside = 0
+    for t in range(len(tps)):
+        for g, G in enumerate(Gs):
+            for q, mesh in enumerate(meshes):
+                row = t * len(Gs) + g
+                w = wanted(G, mesh)
+                if w is not None:  # everything the assignment reads lies inside
+                    assert evaluated[row, q, w[0]:w[1] + 1].all() or p_count[row, q] == 0
+                for l in range(1, L + 1):
+                    inside = evaluated[row, q, l]
+                    for v in range(4):
+                        if v == 3 and l != L:
+                            continue
+                        for name in ("stable", "delta", "index"):
+                            a, b = getattr(full, name)[v], getattr(part, name)[v]
+                            if v <= 1:
+                                a, b = a[row, q, :p_count[row, q], l - 1], b[row, q, :p_count[row, q], l - 1]
+                            elif v == 2:
+                                a, b = a[row, q, l - 1], b[row, q, l - 1]
+                            else:
+                                a, b = a[row, q], b[row, q]
+                            if inside:
+                                assert torch.equal(a, b), (tps[t], G, mesh, l, v, name)
+                            elif w is None or not (w[0] <= l <= w[1]):
+                                # straddling layer counts aside, nothing outside a window is written
+                                lo, hi = l * (l + 1) // 2 - 1, l * (l + 1) // 2 - 1 + l
+                                first, last = window.get((row, q), (0, -1))
+                                if hi < first or lo > last:
+                                    empty = torch.isinf(b).all() if name != "index" else (b == -1).all()
+                                    assert bool(empty), (tps[t], G, mesh, l, v, name)
+                    n_inside += inside
+                    n_outside += not inside
+    assert n_inside > 0 and n_outside > 0
+
+    results = {}
+    for all_cells in (False, True):
+        monkeypatch.setattr(tune_one_case, "MIP_EVALUATE_ALL_CELLS", all_cells)
+        results[all_cells] = tune_one_case.tune(cfg)
+    assert results[False] == results[True]
+    assert results[False][1] is not None

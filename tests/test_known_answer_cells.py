@@ -69,11 +69,11 @@ class ToyTables:
     @staticmethod
     def _like(value, b, tp):
         assert np.all(np.asarray(b) == 2) and np.all(np.asarray(tp) == 1), (b, tp)
-        return np.full(np.broadcast(np.atleast_1d(b), np.atleast_1d(tp)).shape, value)
+        return np.full(np.broadcast(b, tp).shape, value)[()]  # scalars in, scalar out
 
     def mem_full_states(self, kind, item, tp):
         assert np.all(np.asarray(tp) == 1)
-        return np.full(np.atleast_1d(tp).shape, self.FULL[kind][("weights", "grads", "opts").index(item)])
+        return np.full(np.shape(tp), self.FULL[kind][("weights", "grads", "opts").index(item)])[()]
 
     def mem_saved(self, kind, ckpt, b, tp):
         return self._like(self.SAVED[kind, bool(ckpt)], b, tp)

@@ -146,6 +146,46 @@ def test_column_wise_fill_equals_record_by_record_fill(plan):
             assert np.ascontiguousarray(one[name]).tobytes() == np.ascontiguousarray(groups[name]).tobytes(), name
 
 
+def test_tile_windows_hold_the_cells_the_stage_assignment_reads():
+    """``cells_wanted`` of the uniform-device-pp-mip granularity (inter_tuning_mip.py:267-290) turned
+    into tile windows by ``IntraStageTuner.prepare``: every (layers, ckpt) pair of the wanted layer
+    counts lies in its group's window, the window is not larger than the tiles those pairs touch,
+    groups whose mesh is no even split of the cluster are left out, and the pre-saved micro-batch
+    values stop at the stage count."""
+    from mist_amd.config import tp_candidates
+    from mist_amd.inter_tuning_mip import cells_wanted
+    from tests.util import load_plan
+
+    for plan_no in (2, 3):
+        cfg, tables = load_plan(plan_no)
+        hw, L = cfg.hardware, cfg.model.num_hidden_layers
+        D = hw.num_nodes * hw.num_gpus_per_node
+        meshes = _get_device_mesh_candidates(hw.num_nodes, hw.num_gpus_per_node, False)
+        Gs = _get_grad_accumu_steps_candidates(cfg.training.global_batch_size)
+        whole = IntraStageTuner(tables, L, meshes, Gs, tp_candidates(cfg), cfg, sample_size=1, device="cpu")
+        part = IntraStageTuner(tables, L, meshes, Gs, tp_candidates(cfg), cfg, sample_size=1, device="cpu")
+        wanted = part.cells_wanted = cells_wanted(L, hw.num_nodes, hw.num_gpus_per_node)
+        g_all, g_part = whole.prepare()["groups"], part.prepare()["groups"]
+        assert np.all(g_all["lc_tile_begin"] == 0)
+        assert 0 < len(g_part) <= len(g_all)
+        assert g_part["n_lc_tiles"].sum() * 2 < g_all["n_lc_tiles"][:len(g_part)].sum()
+        kept = set()
+        for rec in g_part:
+            G, mesh = int(rec["grad_accum"]), (int(rec["num_nodes"]), int(rec["num_gpus_per_node"]))
+            l_min, l_max, p_count = wanted(G, mesh)
+            assert D % (mesh[0] * mesh[1]) == 0 and p_count == D // (mesh[0] * mesh[1])
+            first_pair = l_min * (l_min + 1) // 2 - 1            # (l_min, ckpt 0)
+            last_pair = l_max * (l_max + 1) // 2 - 1 + l_max     # (l_max, ckpt l_max)
+            begin, count = int(rec["lc_tile_begin"]), int(rec["n_lc_tiles"])
+            assert begin == first_pair // _lib.LC_TILE
+            assert begin + count - 1 == last_pair // _lib.LC_TILE
+            assert rec["num_p"] <= p_count
+            kept.add((int(rec["g_index"]), int(rec["q_index"])))
+        for rec in g_all:  # what was left out is not read
+            if (int(rec["g_index"]), int(rec["q_index"])) not in kept:
+                assert wanted(int(rec["grad_accum"]), (int(rec["num_nodes"]), int(rec["num_gpus_per_node"]))) is None
+
+
 def test_launch_decomposition_covers_every_row_once():
     cfg, tables = load_plan(2)
     hw = cfg.hardware

@@ -121,10 +121,36 @@ int mist_dp_select_candidates(const MistDpCosts *costs, int n_requests, const in
                               int32_t *d_out_request, int capacity, int32_t *d_counts,
                               void *stream);
 
+/* The threshold windows of a search and its first scan batch, decided on the device (no
+ * counterpart in the reference: its sort + gap walk of inter_tuning.py:180-199 runs on the host
+ * over every finite stage cost).  Request r selects the candidates of table row d_rows[r] with
+ * d_lo[r] < v <= d_hi[r] as mist_dp_select_candidates does, into a list of its own; a workgroup
+ * per request sorts them, finds the start of the walk as mist_dp_window_begin does (the fetch is
+ * never open below) for the smallest feasible threshold d_start[r] (+inf: nothing feasible, the
+ * request is skipped), walks them with the gap rule and appends the kept thresholds, ascending,
+ * to d_kept; the first `first_chunk` kept thresholds at or above d_start[r] become the DP
+ * instances d_inst_tmax / d_inst_row[r * first_chunk + j] (row -1 in unused slots: mist_dp_run
+ * skips such instances and reports them infeasible).
+ *   window_capacity : candidates a request may select (a power of two in [64, 8192])
+ *   d_values[n_requests][window_capacity], d_counts[1 + 2 n_requests] : work space
+ *   d_meta[n_requests][8] : selected, candidates above d_hi[r], status, kept, offset of the
+ *                   kept thresholds in d_kept, kept thresholds below d_start[r], instances, 0
+ * status 0 = done; 1 = skipped (d_start[r] = +inf); 2 = more than window_capacity candidates;
+ * 3 = no certain start in the window (MIST_DP_NO_START); 4 = nothing kept at or above d_start[r];
+ * 5 = d_kept too small.  A caller that meets a status above 1 decides that window on the host
+ * (mist_dp_select_candidates + mist_dp_window_begin). */
+int mist_dp_windows_first_batch(const MistDpCosts *costs, int n_requests, const int32_t *d_rows,
+                                const float *d_lo, const float *d_hi, const float *d_start,
+                                double gap, int window_capacity, int first_chunk, float *d_values,
+                                int32_t *d_counts, float *d_kept, int kept_capacity,
+                                int32_t *d_meta, float *d_inst_tmax, int32_t *d_inst_row,
+                                void *stream);
+
 /* Runs n_tmax DP instances at once: one launch per stage count with a thread (or a team of
  * lanes) per (instance, start layer, devices) state, or, for large batches whose state planes fit
  * the LDS of a compute unit and whose costs->stage_min is set, one workgroup per instance.
- * Instance t uses the cost tables of g = d_g_index[t].
+ * Instance t uses the cost tables of g = d_g_index[t]; g < 0 marks an empty slot of the batch,
+ * reported as infeasible (d_best_s -1).
  * MIST_DP_THRESHOLD (reference: inter_stage_tune_dp_impl, inter_tuning.py:220-355):
  *   F(s,k,d) = min over mesh q (n*m <= d), end layer i >= k, ckpt j (shape->ckpt_rule) of
  *              cost(s,k,i,q,j) + F(s-1,i+1,d-n*m)   subject to cost <= d_tmax[t],

@@ -207,6 +207,10 @@ _DP_SIGNATURES = {
         [_VP, ctypes.POINTER(OutTables), _VP, ctypes.c_int, ctypes.c_void_p * 4, ctypes.c_void_p * 4, _VP],
     ),
     "mist_dp_filter_tmax": (ctypes.c_int, [_VP, ctypes.c_int, ctypes.c_double, _VP]),
+    "mist_dp_windows_first_batch": (
+        ctypes.c_int,
+        [ctypes.POINTER(DpCosts), ctypes.c_int, _VP, _VP, _VP, _VP, ctypes.c_double, ctypes.c_int,
+         ctypes.c_int, _VP, _VP, _VP, ctypes.c_int, _VP, _VP, _VP, _VP]),
     "mist_dp_window_begin": (
         ctypes.c_int,
         [_VP, ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_float, ctypes.c_double, _VP]),

@@ -90,10 +90,12 @@ __global__ __launch_bounds__(256) void cost_table_kernel(const double *__restric
 // (value, request) pairs; counts[0] = pairs wanted in total (may exceed the capacity, then the
 // caller retries with a larger list), counts[1 + r] = finite values of request r above hi[r].
 // ------------------------------------------------------------------------------------------
+// With `per_request` every request appends to a list of its own instead, out_values[r][capacity],
+// counted in counts[1 + n_requests + r] (then counts[0] and out_request are not touched).
 __global__ __launch_bounds__(256) void select_candidates_kernel(
     const MistDpCosts tabs, const int32_t *__restrict__ rows, const float *__restrict__ lo,
     const float *__restrict__ hi, float *__restrict__ out_values, int32_t *__restrict__ out_request,
-    int capacity, int32_t *__restrict__ counts) {
+    int capacity, int32_t *__restrict__ counts, bool per_request) {
   // Selected values collect in LDS and leave in one piece: appends to the one output list go
   // through a single counter, and an atomic per wavefront round (thousands per launch) made
   // that counter the bottleneck of the kernel.
@@ -109,14 +111,16 @@ __global__ __launch_bounds__(256) void select_candidates_kernel(
   int above = 0;
   if (threadIdx.x == 0) n_kept = 0;
   __syncthreads();
+  int32_t *list_count = per_request ? &counts[1 + gridDim.y + r] : &counts[0];
+  float *list = per_request ? out_values + (int64_t)r * capacity : out_values;
   auto flush = [&]() {  // called by the whole workgroup
-    if (threadIdx.x == 0) flush_at = n_kept > 0 ? atomicAdd(&counts[0], n_kept) : 0;
+    if (threadIdx.x == 0) flush_at = n_kept > 0 ? atomicAdd(list_count, n_kept) : 0;
     __syncthreads();
     for (int i = threadIdx.x; i < n_kept; i += blockDim.x) {
       const int at = flush_at + i;
       if (at < capacity) {
-        out_values[at] = kept[i];
-        out_request[at] = r;
+        list[at] = kept[i];
+        if (!per_request) out_request[at] = r;
       }
     }
     __syncthreads();
@@ -169,6 +173,164 @@ __global__ __launch_bounds__(256) void select_candidates_kernel(
   if (threadIdx.x == 0) {
     const int total = above_of_wave[0] + above_of_wave[1] + above_of_wave[2] + above_of_wave[3];
     if (total > 0) atomicAdd(&counts[1 + r], total);
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// The reference's gap rule (inter_tuning.py:198) and the start of a walk that does not begin at
+// the bottom of the candidate list (see mist_dp_window_begin in mist_dp.h): the same code for
+// the host entry points and for the kernel that walks the windows on the device.
+// ------------------------------------------------------------------------------------------
+// "t - last < 1e-6" as the reference evaluates it: float32 difference, float64 comparison
+__host__ __device__ inline bool gap_below(float t, float last, double gap) {
+  const float diff = t - last;
+  return (double)diff < gap;
+}
+// Index the walk over `ascending` starts at, or -1 when the fetched part holds no certain start.
+__host__ __device__ inline int window_walk_start(const float *ascending, int n, float lo,
+                                                 bool open_below, float start_value, double gap) {
+  // A candidate whose predecessor is at least the gap below it is kept whatever the walk did
+  // before; the predecessor of the first fetched candidate is unknown unless the fetch was open
+  // below.
+  int first = -1;
+  for (int i = 0; i < n && ascending[i] <= start_value; ++i) {
+    const float prev = i == 0 ? (open_below ? 0.0f : lo) : ascending[i - 1];
+    const bool certain = !gap_below(ascending[i], prev, gap) || (i == 0 && open_below);
+    if (certain) first = i;
+  }
+  if (first < 0) {
+    const bool certain0 = !gap_below(ascending[0], open_below ? 0.0f : lo, gap) || open_below;
+    if (ascending[0] > start_value && certain0) first = 0;
+  }
+  return first;
+}
+
+constexpr int kWindowThreads = 1024;
+// status of a window walked on the device (meta[r][2])
+constexpr int kWindowOk = 0, kWindowNone = 1, kWindowOverflow = 2, kWindowNoStart = 3,
+              kWindowNoBound = 4, kWindowKeptOverflow = 5;
+
+// One workgroup per request of a per-request candidate selection: sorts the request's values
+// (bitonic, in LDS), walks them with the gap rule from the certain start below `start[r]` (the
+// smallest feasible threshold; +inf = nothing feasible, the request is skipped), appends the kept
+// thresholds to one list (kept_out, cursor in counts[0]) and lays out the first scan batch: the
+// first `first_chunk` kept thresholds at or above start[r] as DP instances
+// inst_tmax / inst_row[r * first_chunk + j], unused slots with row -1.
+// meta[r][8] = (selected, above hi, status, kept, offset in kept_out, kept below start, instances, 0).
+__global__ __launch_bounds__(kWindowThreads) void window_walk_kernel(
+    const float *__restrict__ values, int capacity, int32_t *__restrict__ counts,
+    const int32_t *__restrict__ rows, const float *__restrict__ lo,
+    const float *__restrict__ start, double gap, int first_chunk, float *__restrict__ kept_out,
+    int kept_capacity, int32_t *__restrict__ meta, float *__restrict__ inst_tmax,
+    int32_t *__restrict__ inst_row) {
+  extern __shared__ float win_lds[];
+  float *v = win_lds;                                               // [capacity]
+  uint8_t *keep = reinterpret_cast<uint8_t *>(win_lds + capacity);  // [capacity]
+  __shared__ int32_t part_kept[kWindowThreads], part_below[kWindowThreads];
+  __shared__ int32_t walk_status, kept_base;
+  const int r = blockIdx.x, n_requests = gridDim.x, tid = threadIdx.x;
+  const int n_sel = counts[1 + n_requests + r];
+  const float start_r = start[r], lo_r = lo[r];
+  int status = kWindowOk;
+  if (!(start_r < INFINITY)) status = kWindowNone;
+  else if (n_sel > capacity) status = kWindowOverflow;
+  const int n = status == kWindowOk ? n_sel : 0;
+  for (int j = tid; j < first_chunk; j += blockDim.x) inst_row[r * first_chunk + j] = -1;
+  int m = 1;
+  while (m < n) m <<= 1;  // capacity is a power of two
+  for (int i = tid; i < m; i += blockDim.x) {
+    v[i] = i < n ? values[(int64_t)r * capacity + i] : INFINITY;
+    keep[i] = 0;
+  }
+  __syncthreads();
+  for (int k = 2; k <= m; k <<= 1) {
+    for (int j = k >> 1; j > 0; j >>= 1) {
+      for (int i = tid; i < m; i += blockDim.x) {
+        const int other = i ^ j;
+        if (other > i) {
+          const float a = v[i], b = v[other];
+          const bool ascending = (i & k) == 0;
+          if ((a > b) == ascending) {
+            v[i] = b;
+            v[other] = a;
+          }
+        }
+      }
+      __syncthreads();
+    }
+  }
+  if (tid == 0) {
+    int st = status;
+    if (st == kWindowOk && n > 0) {
+      const int first = window_walk_start(v, n, lo_r, false, start_r, gap);
+      if (first < 0) {
+        st = kWindowNoStart;
+      } else {
+        float last = 0.0f;  // the walk keeps its first element (mist_dp_filter_tmax)
+        for (int i = first; i < n; ++i) {
+          if (gap_below(v[i], last, gap)) continue;
+          keep[i] = 1;
+          last = v[i];
+        }
+      }
+    }
+    walk_status = st;
+  }
+  __syncthreads();
+  status = walk_status;
+  // kept values per thread (consecutive elements), those below the start among them
+  const int per = (m + blockDim.x - 1) / blockDim.x;
+  const int i0 = tid * per, i1 = min(i0 + per, n);
+  int mine = 0, below = 0;
+  if (status == kWindowOk)
+    for (int i = i0; i < i1; ++i) {
+      mine += keep[i];
+      below += keep[i] && v[i] < start_r;
+    }
+  part_kept[tid] = mine;
+  part_below[tid] = below;
+  __syncthreads();
+  for (int step = 1; step < (int)blockDim.x; step <<= 1) {  // inclusive scans
+    const int a = tid >= step ? part_kept[tid - step] : 0;
+    const int b = tid >= step ? part_below[tid - step] : 0;
+    __syncthreads();
+    part_kept[tid] += a;
+    part_below[tid] += b;
+    __syncthreads();
+  }
+  const int n_kept = part_kept[blockDim.x - 1], pos = part_below[blockDim.x - 1];
+  if (status == kWindowOk && pos >= n_kept) status = kWindowNoBound;  // nothing kept at or above the start
+  if (tid == 0) {
+    kept_base = 0;
+    if (status == kWindowOk) {
+      kept_base = atomicAdd(&counts[0], n_kept);
+      if (kept_base + n_kept > kept_capacity) walk_status = kWindowKeptOverflow;
+    }
+  }
+  __syncthreads();
+  if (status == kWindowOk && walk_status == kWindowKeptOverflow) status = kWindowKeptOverflow;
+  if (status == kWindowOk) {
+    int at = part_kept[tid] - mine;  // kept values in front of this thread's elements
+    for (int i = i0; i < i1; ++i) {
+      if (!keep[i]) continue;
+      kept_out[kept_base + at] = v[i];
+      if (at >= pos && at < pos + first_chunk) {
+        inst_tmax[r * first_chunk + at - pos] = v[i];
+        inst_row[r * first_chunk + at - pos] = rows[r];
+      }
+      ++at;
+    }
+  }
+  if (tid == 0) {
+    int32_t *out = meta + 8 * r;
+    out[0] = n_sel;
+    out[1] = counts[1 + r];
+    out[2] = status;
+    out[3] = status == kWindowOk ? n_kept : 0;
+    out[4] = kept_base;
+    out[5] = pos;
+    out[6] = status == kWindowOk ? min(first_chunk, n_kept - pos) : 0;
+    out[7] = 0;
   }
 }
 
@@ -455,6 +617,7 @@ __global__ __launch_bounds__(kDpThreads) void dp_step_kernel(
   // improve no state (inf is never < best)
   const float t_max = kBottleneck ? kDpNoThreshold : tmax_list[t];
   const int64_t g = g_list[t];
+  if (g < 0) return;  // an empty slot of the batch (the whole workgroup: blockIdx.y is the instance)
   const int64_t off[4] = {g * tabs.g_stride[0], g * tabs.g_stride[1], g * tabs.g_stride[2],
                           g * tabs.g_stride[3]};
   const int k = e / W, d = e % W;
@@ -556,6 +719,14 @@ __global__ __launch_bounds__(kDpFusedThreads) void dp_fused_kernel(
   int32_t *admissible = reinterpret_cast<int32_t *>(stage_min + n_stage);  // [Q][L][2]
   const int t = blockIdx.x;
   const int64_t g = g_list[t];
+  if (g < 0) {  // an empty slot of the batch
+    if (threadIdx.x == 0) {
+      best_s_out[t] = -1;
+      best_sum_out[t] = INFINITY;
+      stage_max_out[t] = 0.0f;
+    }
+    return;
+  }
   const int64_t off[4] = {g * tabs.g_stride[0], g * tabs.g_stride[1], g * tabs.g_stride[2],
                           g * tabs.g_stride[3]};
   const float *__restrict__ relaid = tabs.stage_min + g * tabs.stage_min_g_stride;
@@ -719,6 +890,14 @@ __global__ __launch_bounds__(kDpPlaneThreads) void dp_plane_kernel(
   float *wave_rows = reinterpret_cast<float *>(reach_q + 2 * Q);  // [n_waves][Q][L] row minima of a task
   const int t = blockIdx.x;
   const int64_t g = g_list[t];
+  if (g < 0) {  // an empty slot of the batch
+    if (threadIdx.x == 0) {
+      best_s_out[t] = -1;
+      best_sum_out[t] = INFINITY;
+      stage_max_out[t] = 0.0f;
+    }
+    return;
+  }
   const int64_t off[4] = {g * tabs.g_stride[0], g * tabs.g_stride[1], g * tabs.g_stride[2],
                           g * tabs.g_stride[3]};
   const int tri = dp_triangle(L);
@@ -1189,8 +1368,7 @@ int mist_dp_filter_tmax(const float *sorted_unique, int n, double gap, float *ou
   float last = 0.0f;
   for (int i = 0; i < n; ++i) {
     const float t = sorted_unique[i];
-    const float diff = t - last;  // float32 difference ...
-    if ((double)diff < gap) continue;  // ... compared in float64
+    if (gap_below(t, last, gap)) continue;
     out[kept++] = t;
     last = t;
   }
@@ -1201,23 +1379,8 @@ int mist_dp_window_begin(const float *ascending, int n, float lo, int open_below
                          float start_value, double gap, float *out) {
   if (n < 0 || (n > 0 && (!ascending || !out))) return fail(MIST_E_INVALID, "bad candidate list");
   if (n == 0) return 0;
-  // A candidate whose predecessor is at least the gap below it is kept whatever the walk did
-  // before (float32 difference, float64 comparison, as in mist_dp_filter_tmax); the predecessor
-  // of the first fetched candidate is unknown unless the fetch was open below.
-  int first = -1;
-  for (int i = 0; i < n && ascending[i] <= start_value; ++i) {
-    const float prev = i == 0 ? (open_below ? 0.0f : lo) : ascending[i - 1];
-    const float diff = ascending[i] - prev;
-    const bool certain = !((double)diff < gap) || (i == 0 && open_below);
-    if (certain) first = i;
-  }
-  if (first < 0) {
-    const float prev = open_below ? 0.0f : lo;
-    const float diff = ascending[0] - prev;
-    const bool certain0 = !((double)diff < gap) || open_below;
-    if (!(ascending[0] > start_value && certain0)) return MIST_DP_NO_START;
-    first = 0;
-  }
+  const int first = window_walk_start(ascending, n, lo, open_below != 0, start_value, gap);
+  if (first < 0) return MIST_DP_NO_START;
   return mist_dp_filter_tmax(ascending + first, n - first, gap, out);  // the walk from there
 }
 
@@ -1258,7 +1421,41 @@ int mist_dp_select_candidates(const MistDpCosts *costs, int n_requests, const in
   const unsigned blocks = (unsigned)std::min<int64_t>((per_row + 16383) / 16384, 64);
   hipLaunchKernelGGL(select_candidates_kernel, dim3(blocks, n_requests), dim3(256), 0,
                      (hipStream_t)stream, *costs, d_rows, d_lo, d_hi, d_out_values, d_out_request,
-                     capacity, d_counts);
+                     capacity, d_counts, false);
+  MIST_HIP_CHECK(hipGetLastError());
+  return 0;
+}
+
+int mist_dp_windows_first_batch(const MistDpCosts *costs, int n_requests, const int32_t *d_rows,
+                                const float *d_lo, const float *d_hi, const float *d_start,
+                                double gap, int window_capacity, int first_chunk, float *d_values,
+                                int32_t *d_counts, float *d_kept, int kept_capacity,
+                                int32_t *d_meta, float *d_inst_tmax, int32_t *d_inst_row,
+                                void *stream) {
+  if (!costs || !costs->costs || !costs->costs_pre || !costs->costs_post)
+    return fail(MIST_E_INVALID, "null cost tables");
+  if (n_requests <= 0 || n_requests > 65535)
+    return fail(MIST_E_INVALID, "n_requests %d outside [1, 65535]", n_requests);
+  if (!d_rows || !d_lo || !d_hi || !d_start || !d_values || !d_counts || !d_kept || !d_meta ||
+      !d_inst_tmax || !d_inst_row)
+    return fail(MIST_E_INVALID, "null pointer argument");
+  if (window_capacity < 64 || window_capacity > 8192 || (window_capacity & (window_capacity - 1)))
+    return fail(MIST_E_INVALID, "window_capacity %d is no power of two in [64, 8192]", window_capacity);
+  if (first_chunk < 1 || kept_capacity < 1 || (int64_t)n_requests * first_chunk > 65535)
+    return fail(MIST_E_INVALID, "first_chunk %d x %d requests outside [1, 65535] / empty kept list",
+                first_chunk, n_requests);
+  hipStream_t st = (hipStream_t)stream;
+  MIST_HIP_CHECK(hipMemsetAsync(d_counts, 0, sizeof(int32_t) * (1 + 2 * (size_t)n_requests), st));
+  const int64_t per_row = costs->g_stride[0] + costs->g_stride[1] + costs->g_stride[2];
+  const unsigned blocks = (unsigned)std::min<int64_t>((per_row + 16383) / 16384, 64);
+  hipLaunchKernelGGL(select_candidates_kernel, dim3(blocks, n_requests), dim3(256), 0, st, *costs,
+                     d_rows, d_lo, d_hi, d_values, (int32_t *)nullptr, window_capacity, d_counts,
+                     true);
+  MIST_HIP_CHECK(hipGetLastError());
+  const size_t lds = (size_t)window_capacity * (sizeof(float) + sizeof(uint8_t));
+  hipLaunchKernelGGL(window_walk_kernel, dim3(n_requests), dim3(kWindowThreads), lds, st, d_values,
+                     window_capacity, d_counts, d_rows, d_lo, d_start, gap, first_chunk, d_kept,
+                     kept_capacity, d_meta, d_inst_tmax, d_inst_row);
   MIST_HIP_CHECK(hipGetLastError());
   return 0;
 }

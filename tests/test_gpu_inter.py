@@ -620,6 +620,130 @@ def test_candidate_selection_of_wide_windows_matches_numpy():
             assert above == int((hg > b).sum())
 
 
+@pytest.mark.parametrize("capacity, first_chunk", [(8192, 48), (256, 7)])
+def test_windows_walked_on_the_device_equal_the_host_walk(capacity, first_chunk):
+    """``mist_dp_windows_first_batch`` (per-request selection, sort, start of the walk, gap walk
+    and first scan batch on the GPU) against the host route it replaces (numpy filter of the
+    same tables, ``mist_dp_window_begin``): kept thresholds, their number below the smallest
+    feasible threshold, the batch's instances and every status - windows of several widths
+    around the real smallest feasible thresholds of the GPT-7B plan, a window whose start cannot
+    be certain, an empty one, a skipped request, and (small capacity) windows that overflow."""
+    import ctypes
+
+    import torch
+
+    from mist_amd import _lib
+    from mist_amd.config import tp_candidates
+    from mist_amd.inter_tuning import GAP, _DpRunner
+    from mist_amd.intra_tuning import IntraStageTuner
+    from mist_amd.search_space import _get_device_mesh_candidates, _get_grad_accumu_steps_candidates
+
+    cfg, tables = load_plan(2)
+    hw, L = cfg.hardware, cfg.model.num_hidden_layers
+    meshes = _get_device_mesh_candidates(hw.num_nodes, hw.num_gpus_per_node, False)
+    Gs = _get_grad_accumu_steps_candidates(cfg.training.global_batch_size)
+    res = IntraStageTuner(tables, L, meshes, Gs, tp_candidates(cfg), cfg, sample_size=1).tune_all()
+    runner = _DpRunner(res[0], L, hw.num_nodes * hw.num_gpus_per_node, meshes, 0)
+    lib = runner.lib
+    all_rows = np.arange(len(Gs) * len(res), dtype=np.int32)
+    bott, _ = runner.bottleneck(all_rows)
+    feasible = all_rows[np.isfinite(bott)]
+    assert len(feasible) >= 8
+    rows, lo, hi, start = [], [], [], []
+    widths = [1.0005, 1.002, 1.01, 1.03, 1.1]
+    for k, g in enumerate(feasible):
+        b = np.float32(bott[g])
+        rows.append(g)
+        start.append(b)
+        lo.append(np.float32(b - np.float32(1e-4 + 1e-5 * abs(float(b)))))
+        hi.append(np.float32(b * widths[k % len(widths)]))
+    g0 = int(feasible[0])
+    b0 = np.float32(bott[g0])
+    # a skipped request, an empty window far above every cost, a window that begins one float
+    # below a candidate above the start value (that candidate's predecessor is unknown and may be
+    # within the gap: no certain start)
+    above_start, _ = runner.candidates_between(
+        np.array([g0], dtype=np.int32), np.array([b0 * 1.001], dtype=np.float32),
+        np.array([b0 * 1.01], dtype=np.float32))[0]
+    c = np.float32(above_start[0])
+    rows += [g0, g0, g0]
+    start += [np.float32(np.inf), b0, b0]
+    lo += [np.float32(0.0), np.float32(1e30), np.nextafter(c, np.float32(0.0))]
+    hi += [np.float32(1.0), np.float32(2e30), np.float32(b0 * 1.01)]
+    rows = np.array(rows, dtype=np.int32)
+    lo, hi, start = (np.array(x, dtype=np.float32) for x in (lo, hi, start))
+    n = len(rows)
+
+    dev = runner.device
+    kept_capacity = 1 << 18
+    d = lambda a: torch.from_numpy(a).to(dev)
+    d_rows, d_lo, d_hi, d_start = d(rows), d(lo), d(hi), d(start)
+    d_values = torch.empty(n * capacity, dtype=torch.float32, device=dev)
+    d_counts = torch.empty(1 + 2 * n, dtype=torch.int32, device=dev)
+    d_kept = torch.empty(kept_capacity, dtype=torch.float32, device=dev)
+    d_meta = torch.empty(n * 8, dtype=torch.int32, device=dev)
+    d_inst_t = torch.full((n * first_chunk,), -7.0, dtype=torch.float32, device=dev)
+    d_inst_row = torch.full((n * first_chunk,), -7, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        rc = lib.mist_dp_windows_first_batch(
+            ctypes.byref(runner._all_costs), n, d_rows.data_ptr(), d_lo.data_ptr(), d_hi.data_ptr(),
+            d_start.data_ptr(), GAP, capacity, first_chunk, d_values.data_ptr(), d_counts.data_ptr(),
+            d_kept.data_ptr(), kept_capacity, d_meta.data_ptr(), d_inst_t.data_ptr(),
+            d_inst_row.data_ptr(), None)
+        _lib.check(rc, "mist_dp_windows_first_batch")
+        torch.cuda.synchronize()
+    meta = d_meta.cpu().numpy().reshape(n, 8)
+    kept_all = d_kept.cpu().numpy()
+    inst_t = d_inst_t.cpu().numpy().reshape(n, first_chunk)
+    inst_row = d_inst_row.cpu().numpy().reshape(n, first_chunk)
+
+    host = runner.candidates_between(rows, lo, hi)
+    seen = set()
+    for r in range(n):
+        values, above = host[r]
+        n_sel, n_above, status, n_kept, base, pos, n_inst, _ = (int(x) for x in meta[r])
+        want_status = 0
+        kept = np.empty(0, dtype=np.float32)
+        if not np.isfinite(start[r]):
+            want_status = 1
+        elif len(values) > capacity:
+            want_status = 2
+        else:
+            out = np.empty(max(len(values), 1), dtype=np.float32)
+            k = lib.mist_dp_window_begin(
+                ctypes.c_void_p(np.ascontiguousarray(values).ctypes.data), len(values), float(lo[r]), 0,
+                float(start[r]), GAP, ctypes.c_void_p(out.ctypes.data))
+            if k == _lib.DP_NO_START:
+                want_status = 3
+            else:
+                assert k >= 0
+                kept = out[:k]
+                if not (kept >= start[r]).any():
+                    want_status = 4
+        seen.add(want_status)
+        assert status == want_status, (r, status, want_status)
+        assert n_sel == len(values) and n_above == above
+        if status != 0:
+            assert n_inst == 0 and np.all(inst_row[r] == -1)
+            continue
+        assert n_kept == len(kept) and np.array_equal(kept_all[base:base + n_kept], kept)
+        assert pos == int(np.searchsorted(kept, start[r], side="left"))
+        assert n_inst == min(first_chunk, n_kept - pos) > 0
+        assert np.array_equal(inst_t[r, :n_inst], kept[pos:pos + n_inst])
+        assert np.all(inst_row[r, :n_inst] == rows[r]) and np.all(inst_row[r, n_inst:] == -1)
+    assert {0, 1, 3, 4} <= seen and (capacity > 1024 or 2 in seen)
+
+    # the instances as a DP batch: empty slots come back infeasible, the others as on their own
+    fam = runner.families[0]
+    flat_row, flat_t = inst_row.reshape(-1), inst_t.reshape(-1)
+    live = flat_row >= 0
+    bs, bsum, smax = runner.run(np.where(live, flat_row, -1).astype(np.int32), np.where(live, flat_t, 0).astype(np.float32))
+    bs1, bsum1, smax1 = runner.run(flat_row[live], flat_t[live])
+    assert np.all(bs[~live] == -1)
+    assert np.array_equal(bs[live], bs1) and np.array_equal(bsum[live], bsum1)
+    assert np.array_equal(smax[live][bs1 >= 0], smax1[bs1 >= 0])
+
+
 @pytest.mark.parametrize("granularity", ["inter-stage", "uniform-device-pp", "uniform-pp", "no-pp"])
 def test_infeasible_plan_returns_inf_none(granularity):
     """Nothing fits into 0.2 GB: every table stays +inf / -1, the searches find no partition and

@@ -128,13 +128,14 @@ int mist_dp_select_candidates(const MistDpCosts *costs, int n_requests, const in
  * per request sorts them, finds the start of the walk as mist_dp_window_begin does (the fetch is
  * never open below) for the smallest feasible threshold d_start[r] (+inf: nothing feasible, the
  * request is skipped), walks them with the gap rule and appends the kept thresholds, ascending,
- * to d_kept; the first `first_chunk` kept thresholds at or above d_start[r] become the DP
- * instances d_inst_tmax / d_inst_row[r * first_chunk + j] (row -1 in unused slots: mist_dp_run
- * skips such instances and reports them infeasible).
- *   window_capacity : candidates a request may select (a power of two in [64, 8192])
- *   d_values[n_requests][window_capacity], d_counts[1 + 2 n_requests] : work space
+ * to d_kept; the first `first_chunk` kept thresholds at or above d_start[r] become DP instances,
+ * appended to d_inst_tmax / d_inst_row[n_requests * first_chunk] (row -1 in the unused tail:
+ * mist_dp_run skips such instances and reports them infeasible).
+ *   window_capacity : candidates a request may select (a power of two in [128, 8192])
+ *   d_values[n_requests][window_capacity], d_counts[2 + 2 n_requests] : work space
  *   d_meta[n_requests][8] : selected, candidates above d_hi[r], status, kept, offset of the
- *                   kept thresholds in d_kept, kept thresholds below d_start[r], instances, 0
+ *                   kept thresholds in d_kept, kept thresholds below d_start[r], instances,
+ *                   offset of the instances
  * status 0 = done; 1 = skipped (d_start[r] = +inf); 2 = more than window_capacity candidates;
  * 3 = no certain start in the window (MIST_DP_NO_START); 4 = nothing kept at or above d_start[r];
  * 5 = d_kept too small.  A caller that meets a status above 1 decides that window on the host

@@ -214,9 +214,19 @@ constexpr int kWindowOk = 0, kWindowNone = 1, kWindowOverflow = 2, kWindowNoStar
 // (bitonic, in LDS), walks them with the gap rule from the certain start below `start[r]` (the
 // smallest feasible threshold; +inf = nothing feasible, the request is skipped), appends the kept
 // thresholds to one list (kept_out, cursor in counts[0]) and lays out the first scan batch: the
-// first `first_chunk` kept thresholds at or above start[r] as DP instances
-// inst_tmax / inst_row[r * first_chunk + j], unused slots with row -1.
-// meta[r][8] = (selected, above hi, status, kept, offset in kept_out, kept below start, instances, 0).
+// first `first_chunk` kept thresholds at or above start[r] as DP instances, appended to
+// inst_tmax / inst_row (cursor in counts[1 + 2 n_requests]; the caller pre-fills inst_row with
+// -1, so that the live instances are the first workgroups of the DP launch and the empty slots
+// its tail).
+// meta[r][8] = (selected, above hi, status, kept, offset in kept_out, kept below start, instances,
+// offset of the instances).
+//
+// The walk is the host's (mist_dp_window_begin), taken apart along its own argument: a candidate
+// whose predecessor is at least the gap below it is kept whatever came before (the last kept
+// value is at most the predecessor, and the float32 difference is monotone), so the candidates
+// from such a one up to the next are a piece that is walked on its own, by the thread that owns
+// its first element; the piece that starts at the walk's first element begins with "nothing kept
+// yet" like the host's loop.
 __global__ __launch_bounds__(kWindowThreads) void window_walk_kernel(
     const float *__restrict__ values, int capacity, int32_t *__restrict__ counts,
     const int32_t *__restrict__ rows, const float *__restrict__ lo,
@@ -226,97 +236,131 @@ __global__ __launch_bounds__(kWindowThreads) void window_walk_kernel(
   extern __shared__ float win_lds[];
   float *v = win_lds;                                               // [capacity]
   uint8_t *keep = reinterpret_cast<uint8_t *>(win_lds + capacity);  // [capacity]
-  __shared__ int32_t part_kept[kWindowThreads], part_below[kWindowThreads];
-  __shared__ int32_t walk_status, kept_base;
+  __shared__ int32_t wave_kept[kWindowThreads / 64], wave_below[kWindowThreads / 64];
+  __shared__ int32_t walk_first, kept_base, kept_overflow, inst_base;
   const int r = blockIdx.x, n_requests = gridDim.x, tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6, n_waves = blockDim.x >> 6;
   const int n_sel = counts[1 + n_requests + r];
   const float start_r = start[r], lo_r = lo[r];
   int status = kWindowOk;
   if (!(start_r < INFINITY)) status = kWindowNone;
   else if (n_sel > capacity) status = kWindowOverflow;
   const int n = status == kWindowOk ? n_sel : 0;
-  for (int j = tid; j < first_chunk; j += blockDim.x) inst_row[r * first_chunk + j] = -1;
-  int m = 1;
-  while (m < n) m <<= 1;  // capacity is a power of two
+  int m = 128;  // a wavefront's share of a sorting step is 128 consecutive values
+  while (m < n) m <<= 1;  // capacity is a power of two >= 128
   for (int i = tid; i < m; i += blockDim.x) {
     v[i] = i < n ? values[(int64_t)r * capacity + i] : INFINITY;
     keep[i] = 0;
   }
+  if (tid == 0) {
+    walk_first = -1;
+    kept_overflow = 0;
+  }
   __syncthreads();
+  // Bitonic sort, one compare-exchange per thread and step: thread x holds the pair
+  // (i, i + j) with i = 2 j (x / j) + x % j.  For j <= 32 the 64 pairs of a wavefront lie in its
+  // own 128 consecutive values, and so do those of the following smaller j: those steps need no
+  // barrier between them (a wavefront's LDS accesses complete in order).
   for (int k = 2; k <= m; k <<= 1) {
     for (int j = k >> 1; j > 0; j >>= 1) {
-      for (int i = tid; i < m; i += blockDim.x) {
-        const int other = i ^ j;
-        if (other > i) {
-          const float a = v[i], b = v[other];
-          const bool ascending = (i & k) == 0;
-          if ((a > b) == ascending) {
-            v[i] = b;
-            v[other] = a;
-          }
+      for (int x = tid; x < m / 2; x += blockDim.x) {
+        const int i = 2 * j * (x / j) + x % j, other = i + j;
+        const float a = v[i], b = v[other];
+        const bool ascending = (i & k) == 0;
+        if ((a > b) == ascending) {
+          v[i] = b;
+          v[other] = a;
         }
       }
-      __syncthreads();
+      if (j > 32) __syncthreads();
+      else __builtin_amdgcn_wave_barrier();
     }
-  }
-  if (tid == 0) {
-    int st = status;
-    if (st == kWindowOk && n > 0) {
-      const int first = window_walk_start(v, n, lo_r, false, start_r, gap);
-      if (first < 0) {
-        st = kWindowNoStart;
-      } else {
-        float last = 0.0f;  // the walk keeps its first element (mist_dp_filter_tmax)
-        for (int i = first; i < n; ++i) {
-          if (gap_below(v[i], last, gap)) continue;
-          keep[i] = 1;
-          last = v[i];
-        }
-      }
-    }
-    walk_status = st;
+    if (k >= 64) __syncthreads();  // the next k starts with j = k: other wavefronts' values
   }
   __syncthreads();
-  status = walk_status;
-  // kept values per thread (consecutive elements), those below the start among them
+  // start of the walk (window_walk_start with a fetch that is not open below): the last
+  // candidate <= start_r whose predecessor is at least the gap below, else the first candidate
+  // if it lies above start_r and is certain itself
   const int per = (m + blockDim.x - 1) / blockDim.x;
   const int i0 = tid * per, i1 = min(i0 + per, n);
+  {
+    int mine = -1;
+    for (int i = i0; i < i1; ++i)
+      if (v[i] <= start_r && !gap_below(v[i], i == 0 ? lo_r : v[i - 1], gap)) mine = i;
+    if (mine >= 0) atomicMax(&walk_first, mine);
+  }
+  __syncthreads();
+  int first = walk_first;
+  if (status == kWindowOk && n > 0 && first < 0) {
+    if (v[0] > start_r && !gap_below(v[0], lo_r, gap)) first = 0;
+    else status = kWindowNoStart;
+  }
+  // the walk, piece by piece
+  if (status == kWindowOk && n > 0) {
+    for (int i = max(i0, first); i < i1; ++i) {
+      const bool head = i == first;
+      if (!head && gap_below(v[i], v[i - 1], gap)) continue;  // inside a piece: its owner walks it
+      float last = 0.0f;  // the walk's first piece starts with nothing kept (mist_dp_filter_tmax)
+      int j = i;
+      if (!head) {
+        keep[i] = 1;
+        last = v[i];
+        j = i + 1;
+      }
+      for (; j < n && (j == i || gap_below(v[j], v[j - 1], gap)); ++j) {
+        if (gap_below(v[j], last, gap)) continue;
+        keep[j] = 1;
+        last = v[j];
+      }
+    }
+  }
+  __syncthreads();
+  // kept values per thread (consecutive elements), those below the start among them
   int mine = 0, below = 0;
   if (status == kWindowOk)
     for (int i = i0; i < i1; ++i) {
       mine += keep[i];
       below += keep[i] && v[i] < start_r;
     }
-  part_kept[tid] = mine;
-  part_below[tid] = below;
-  __syncthreads();
-  for (int step = 1; step < (int)blockDim.x; step <<= 1) {  // inclusive scans
-    const int a = tid >= step ? part_kept[tid - step] : 0;
-    const int b = tid >= step ? part_below[tid - step] : 0;
-    __syncthreads();
-    part_kept[tid] += a;
-    part_below[tid] += b;
-    __syncthreads();
+  int scan_kept = mine, scan_below = below;  // inclusive scans over the wavefront
+  for (int step = 1; step < 64; step <<= 1) {
+    const int a = __shfl_up(scan_kept, step), b = __shfl_up(scan_below, step);
+    if (lane >= step) {
+      scan_kept += a;
+      scan_below += b;
+    }
   }
-  const int n_kept = part_kept[blockDim.x - 1], pos = part_below[blockDim.x - 1];
+  if (lane == 63) {
+    wave_kept[wave] = scan_kept;
+    wave_below[wave] = scan_below;
+  }
+  __syncthreads();
+  int before = 0, n_kept = 0, pos = 0;
+  for (int w = 0; w < n_waves; ++w) {
+    if (w < wave) before += wave_kept[w];
+    n_kept += wave_kept[w];
+    pos += wave_below[w];
+  }
   if (status == kWindowOk && pos >= n_kept) status = kWindowNoBound;  // nothing kept at or above the start
+  const int n_inst = status == kWindowOk ? min(first_chunk, n_kept - pos) : 0;
   if (tid == 0) {
-    kept_base = 0;
+    kept_base = inst_base = 0;
     if (status == kWindowOk) {
       kept_base = atomicAdd(&counts[0], n_kept);
-      if (kept_base + n_kept > kept_capacity) walk_status = kWindowKeptOverflow;
+      if (kept_base + n_kept > kept_capacity) kept_overflow = 1;
+      else inst_base = atomicAdd(&counts[1 + 2 * n_requests], n_inst);  // <= n_requests * first_chunk
     }
   }
   __syncthreads();
-  if (status == kWindowOk && walk_status == kWindowKeptOverflow) status = kWindowKeptOverflow;
+  if (status == kWindowOk && kept_overflow) status = kWindowKeptOverflow;
   if (status == kWindowOk) {
-    int at = part_kept[tid] - mine;  // kept values in front of this thread's elements
+    int at = before + scan_kept - mine;  // kept values in front of this thread's elements
     for (int i = i0; i < i1; ++i) {
       if (!keep[i]) continue;
       kept_out[kept_base + at] = v[i];
       if (at >= pos && at < pos + first_chunk) {
-        inst_tmax[r * first_chunk + at - pos] = v[i];
-        inst_row[r * first_chunk + at - pos] = rows[r];
+        inst_tmax[inst_base + at - pos] = v[i];
+        inst_row[inst_base + at - pos] = rows[r];
       }
       ++at;
     }
@@ -329,8 +373,8 @@ __global__ __launch_bounds__(kWindowThreads) void window_walk_kernel(
     out[3] = status == kWindowOk ? n_kept : 0;
     out[4] = kept_base;
     out[5] = pos;
-    out[6] = status == kWindowOk ? min(first_chunk, n_kept - pos) : 0;
-    out[7] = 0;
+    out[6] = status == kWindowOk ? n_inst : 0;
+    out[7] = inst_base;
   }
 }
 
@@ -1439,13 +1483,14 @@ int mist_dp_windows_first_batch(const MistDpCosts *costs, int n_requests, const 
   if (!d_rows || !d_lo || !d_hi || !d_start || !d_values || !d_counts || !d_kept || !d_meta ||
       !d_inst_tmax || !d_inst_row)
     return fail(MIST_E_INVALID, "null pointer argument");
-  if (window_capacity < 64 || window_capacity > 8192 || (window_capacity & (window_capacity - 1)))
-    return fail(MIST_E_INVALID, "window_capacity %d is no power of two in [64, 8192]", window_capacity);
+  if (window_capacity < 128 || window_capacity > 8192 || (window_capacity & (window_capacity - 1)))
+    return fail(MIST_E_INVALID, "window_capacity %d is no power of two in [128, 8192]", window_capacity);
   if (first_chunk < 1 || kept_capacity < 1 || (int64_t)n_requests * first_chunk > 65535)
     return fail(MIST_E_INVALID, "first_chunk %d x %d requests outside [1, 65535] / empty kept list",
                 first_chunk, n_requests);
   hipStream_t st = (hipStream_t)stream;
-  MIST_HIP_CHECK(hipMemsetAsync(d_counts, 0, sizeof(int32_t) * (1 + 2 * (size_t)n_requests), st));
+  MIST_HIP_CHECK(hipMemsetAsync(d_counts, 0, sizeof(int32_t) * (2 + 2 * (size_t)n_requests), st));
+  MIST_HIP_CHECK(hipMemsetAsync(d_inst_row, 0xFF, sizeof(int32_t) * (size_t)n_requests * first_chunk, st));
   const int64_t per_row = costs->g_stride[0] + costs->g_stride[1] + costs->g_stride[2];
   const unsigned blocks = (unsigned)std::min<int64_t>((per_row + 16383) / 16384, 64);
   hipLaunchKernelGGL(select_candidates_kernel, dim3(blocks, n_requests), dim3(256), 0, st, *costs,

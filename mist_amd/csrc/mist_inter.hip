@@ -22,6 +22,7 @@
 #include <algorithm>
 #include <cmath>
 #include <cstdint>
+#include <cstdlib>
 #include <cstring>
 #include <limits>
 #include <map>
@@ -40,6 +41,9 @@ constexpr int kFirstChunk = 48;   // thresholds per G in the first speculative b
 constexpr int kMaxChunk = 4096;   // most thresholds per G in one batch
 constexpr double kGap = 1e-6;     // inter_tuning.py:177
 constexpr int kSelectHead = 1 << 16;  // selected candidates that travel with the counts of a fetch
+constexpr int kWindowCapacity = 8192;  // candidates of a window that is walked on the device
+constexpr int kKeptCapacity = 1 << 18;  // kept thresholds of all windows of a search, on the device
+constexpr int kKeptHead = 1 << 15;      // of which this many travel with the first round trip
 const double kInf = std::numeric_limits<double>::infinity();
 
 // ---- buffers that live as long as the process: device and pinned host memory per device ----
@@ -69,10 +73,14 @@ struct Workspace {
   Buffer d_in, d_out, d_scratch, d_req, d_counts, d_values, d_request, d_argmin, d_path, d_rows,
       d_grad;
   Buffer h_in, h_out, h_req, h_counts, h_values, h_request, h_path, h_rows, h_grad;
+  // windows and first scan batch decided on the device
+  Buffer d_win_values, d_win_counts, d_kept, d_meta, d_inst_t, d_inst_row, d_out_first;
+  Buffer h_kept, h_meta, h_out_first;
   int select_capacity = 1 << 18;
   Workspace() {
     h_in.pinned = h_out.pinned = h_req.pinned = h_counts.pinned = h_values.pinned =
-        h_request.pinned = h_path.pinned = h_rows.pinned = h_grad.pinned = true;
+        h_request.pinned = h_path.pinned = h_rows.pinned = h_grad.pinned = h_kept.pinned =
+            h_meta.pinned = h_out_first.pinned = true;
   }
 };
 
@@ -130,9 +138,10 @@ struct Fetched {  // one request of a candidate fetch: ascending values and how 
 // Window request of every (instance, G) right after the bottleneck DP of all families
 // (out[f][3][n], rows 1 and 2 = smallest feasible threshold and the stage-cost sum there): the
 // family with the smallest threshold (the first of equals) gives the start of the window;
-// req[0][i] = table row, req[1][i] = lo, req[2][i] = hi of the candidates to fetch, an empty
-// window (lo = hi = +inf) when no family is feasible.  The bounds only size the fetch; what the
-// scan does with the candidates is decided on the host from the values that come back.
+// req[0][i] = table row, req[1][i] = lo, req[2][i] = hi of the candidates to fetch, req[3][i] =
+// the smallest feasible threshold itself; an empty window (lo = hi = +inf) when no family is
+// feasible.  The bounds only size the fetch; what the scan does with the candidates follows the
+// reference's rules on the values that lie inside.
 __global__ void window_request_kernel(const float *__restrict__ out, int n_families, int n,
                                       const int32_t *__restrict__ rows,
                                       const int32_t *__restrict__ grad_accum, int n_grad_accum,
@@ -148,6 +157,7 @@ __global__ void window_request_kernel(const float *__restrict__ out, int n_famil
     }
   }
   reinterpret_cast<int32_t *>(req)[i] = rows[i];
+  req[3 * n + i] = bott;
   if (!(bott < INFINITY)) {
     req[n + i] = INFINITY;
     req[2 * n + i] = INFINITY;
@@ -300,18 +310,18 @@ struct Search {
   }
 
   // best + (g - 1) * f_stage_max in float64 (inter_tuning.py:342) of family f, inf if infeasible
-  double total_of(int f, int i, int n, int G) const {
-    const float *h = ws->h_out.as<float>() + (size_t)f * 3 * n;
+  double total_of(int f, int i, int n, int G, const float *out = nullptr) const {
+    const float *h = (out ? out : ws->h_out.as<float>()) + (size_t)f * 3 * n;
     int32_t best_s;
     std::memcpy(&best_s, h + i, sizeof(best_s));
     if (best_s < 0) return kInf;
     return (double)h[n + i] + ((double)G - 1.0) * (double)h[2 * n + i];
   }
   // smallest family total (the first family wins ties); *family = the one that attains it
-  double total(int i, int n, int G, int *family = nullptr) const {
+  double total(int i, int n, int G, int *family = nullptr, const float *out = nullptr) const {
     double best = kInf;
     for (int f = 0; f < n_families; ++f) {
-      const double c = total_of(f, i, n, G);
+      const double c = total_of(f, i, n, G, out);
       if (c < best) {
         best = c;
         if (family) *family = f;
@@ -345,8 +355,8 @@ struct Search {
     const int n = (int)rows.size();
     if (int rc = ws->h_grad.reserve(sizeof(int32_t) * n_grad_accum)) return rc;
     if (int rc = ws->d_grad.reserve(sizeof(int32_t) * n_grad_accum)) return rc;
-    if (int rc = ws->h_req.reserve(sizeof(float) * 3 * n)) return rc;
-    if (int rc = ws->d_req.reserve(sizeof(float) * 3 * n)) return rc;
+    if (int rc = ws->h_req.reserve(sizeof(float) * 4 * n)) return rc;
+    if (int rc = ws->d_req.reserve(sizeof(float) * 4 * n)) return rc;
     std::memcpy(ws->h_grad.ptr, grad_accum, sizeof(int32_t) * n_grad_accum);
     MIST_HIP_CHECK(hipMemcpyAsync(ws->d_grad.ptr, ws->h_grad.ptr, sizeof(int32_t) * n_grad_accum,
                                   hipMemcpyHostToDevice, stream));
@@ -357,10 +367,93 @@ struct Search {
                        reinterpret_cast<const int32_t *>(ws->d_in.as<float>() + n),
                        ws->d_grad.as<int32_t>(), n_grad_accum, kGap, ws->d_req.as<float>());
     MIST_HIP_CHECK(hipGetLastError());
-    MIST_HIP_CHECK(hipMemcpyAsync(ws->h_req.ptr, ws->d_req.ptr, sizeof(float) * 3 * n,
+    MIST_HIP_CHECK(hipMemcpyAsync(ws->h_req.ptr, ws->d_req.ptr, sizeof(float) * 4 * n,
                                   hipMemcpyDeviceToHost, stream));
     out->assign(n, Fetched());
     return collect(n, out);
+  }
+
+  // The same, and the windows and the first scan batch with it (mist_dp_windows_first_batch +
+  // the threshold DP of its instances for every family): one round trip.  Afterwards
+  // ws->h_out holds the bottleneck DP's outputs, ws->h_req the requests ([4][n]: row, lo, hi,
+  // smallest feasible threshold), ws->h_meta the windows' descriptions ([n][8]), ws->h_kept
+  // their kept thresholds and ws->h_out_first the DP outputs of the batch
+  // ([family][3][n * first_chunk]; the instances of window r start at h_meta[r][7]).
+  int bottleneck_windows_first_batch(const std::vector<int32_t> &rows, const int32_t *grad_accum,
+                                     int n_grad_accum, int window_capacity, int first_chunk) {
+    const int n = (int)rows.size(), n_inst = n * first_chunk;
+    if (int rc = ws->h_grad.reserve(sizeof(int32_t) * n_grad_accum)) return rc;
+    if (int rc = ws->d_grad.reserve(sizeof(int32_t) * n_grad_accum)) return rc;
+    if (int rc = ws->h_req.reserve(sizeof(float) * 4 * n)) return rc;
+    if (int rc = ws->d_req.reserve(sizeof(float) * 4 * n)) return rc;
+    if (int rc = ws->d_win_values.reserve(sizeof(float) * (size_t)n * window_capacity)) return rc;
+    if (int rc = ws->d_win_counts.reserve(sizeof(int32_t) * (2 + 2 * (size_t)n))) return rc;
+    if (int rc = ws->d_kept.reserve(sizeof(float) * kKeptCapacity)) return rc;
+    if (int rc = ws->h_kept.reserve(sizeof(float) * kKeptCapacity)) return rc;
+    if (int rc = ws->d_meta.reserve(sizeof(int32_t) * 8 * n)) return rc;
+    if (int rc = ws->h_meta.reserve(sizeof(int32_t) * 8 * n)) return rc;
+    if (int rc = ws->d_inst_t.reserve(sizeof(float) * n_inst)) return rc;
+    if (int rc = ws->d_inst_row.reserve(sizeof(int32_t) * n_inst)) return rc;
+    const size_t n_out = (size_t)3 * n_inst * n_families;
+    if (int rc = ws->d_out_first.reserve(sizeof(float) * n_out)) return rc;
+    if (int rc = ws->h_out_first.reserve(sizeof(float) * n_out)) return rc;
+    // the state planes of the batch are the larger need: sized before anything is queued
+    int64_t n_scratch = 1;
+    for (int f = 0; f < n_families; ++f) {
+      const int64_t want = mist_dp_scratch_floats(&shapes[f], n_inst);
+      if (want < 0) return MIST_E_INVALID;
+      n_scratch = std::max(n_scratch, want);
+    }
+    if (int rc = ws->d_scratch.reserve(sizeof(float) * (size_t)n_scratch)) return rc;
+    std::memcpy(ws->h_grad.ptr, grad_accum, sizeof(int32_t) * n_grad_accum);
+    MIST_HIP_CHECK(hipMemcpyAsync(ws->d_grad.ptr, ws->h_grad.ptr, sizeof(int32_t) * n_grad_accum,
+                                  hipMemcpyHostToDevice, stream));
+    const std::vector<float> zeros(n, 0.0f);
+    if (int rc = run(rows, zeros, MIST_DP_BOTTLENECK, false, /*sync=*/false)) return rc;
+    float *d_req = ws->d_req.as<float>();
+    hipLaunchKernelGGL(window_request_kernel, dim3((n + 63) / 64), dim3(64), 0, stream,
+                       ws->d_out.as<float>(), n_families, n,
+                       reinterpret_cast<const int32_t *>(ws->d_in.as<float>() + n),
+                       ws->d_grad.as<int32_t>(), n_grad_accum, kGap, d_req);
+    MIST_HIP_CHECK(hipGetLastError());
+    if (int rc = mist_dp_windows_first_batch(
+            select_costs, n, reinterpret_cast<int32_t *>(d_req), d_req + n, d_req + 2 * n,
+            d_req + 3 * n, kGap, window_capacity, first_chunk, ws->d_win_values.as<float>(),
+            ws->d_win_counts.as<int32_t>(), ws->d_kept.as<float>(), kKeptCapacity,
+            ws->d_meta.as<int32_t>(), ws->d_inst_t.as<float>(), ws->d_inst_row.as<int32_t>(), stream))
+      return rc;
+    for (int f = 0; f < n_families; ++f) {
+      float *d_out = ws->d_out_first.as<float>() + (size_t)f * 3 * n_inst;
+      if (int rc = mist_dp_run(&shapes[f], &costs[f], ws->d_inst_t.as<float>(),
+                               ws->d_inst_row.as<int32_t>(), n_inst, MIST_DP_THRESHOLD,
+                               reinterpret_cast<int32_t *>(d_out), d_out + n_inst, d_out + 2 * n_inst,
+                               nullptr, ws->d_scratch.as<float>(), stream))
+        return rc;
+    }
+    MIST_HIP_CHECK(hipMemcpyAsync(ws->h_req.ptr, ws->d_req.ptr, sizeof(float) * 4 * n,
+                                  hipMemcpyDeviceToHost, stream));
+    MIST_HIP_CHECK(hipMemcpyAsync(ws->h_meta.ptr, ws->d_meta.ptr, sizeof(int32_t) * 8 * n,
+                                  hipMemcpyDeviceToHost, stream));
+    MIST_HIP_CHECK(hipMemcpyAsync(ws->h_kept.ptr, ws->d_kept.ptr, sizeof(float) * kKeptHead,
+                                  hipMemcpyDeviceToHost, stream));
+    MIST_HIP_CHECK(hipMemcpyAsync(ws->h_out_first.ptr, ws->d_out_first.ptr, sizeof(float) * n_out,
+                                  hipMemcpyDeviceToHost, stream));
+    MIST_HIP_CHECK(hipStreamSynchronize(stream));
+    ++round_trips;
+    // kept thresholds beyond the part that travelled with the rest
+    const int32_t *meta = ws->h_meta.as<int32_t>();
+    int64_t kept_end = 0;
+    for (int r = 0; r < n; ++r)
+      if (meta[8 * r + 2] == 0) kept_end = std::max<int64_t>(kept_end, (int64_t)meta[8 * r + 4] + meta[8 * r + 3]);
+    if (kept_end > kKeptHead) {
+      MIST_HIP_CHECK(hipMemcpyAsync(ws->h_kept.as<float>() + kKeptHead,
+                                    ws->d_kept.as<float>() + kKeptHead,
+                                    sizeof(float) * (size_t)(kept_end - kKeptHead),
+                                    hipMemcpyDeviceToHost, stream));
+      MIST_HIP_CHECK(hipStreamSynchronize(stream));
+      ++round_trips;
+    }
+    return 0;
   }
 
   // runs the n requests that lie in ws->d_req and sorts what comes back by request
@@ -541,26 +634,93 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
            &g_workspaces[device]};
   const int n_flat = n_instances * n_grad_accum;
 
-  // ---- smallest feasible threshold of every (instance, G) and the first fetch of its window:
-  // one round trip ----
   std::vector<int32_t> flat_rows(rows, rows + n_flat);
+  std::vector<Window> windows(n_flat);
+  // smallest feasible threshold (+inf if none) and the stage-cost sum there, from the outputs of
+  // the bottleneck DP of every family (the first family with the smallest threshold)
+  auto bottleneck_of = [&](int i, float *bott, float *sum) {
+    const float *h = S.ws->h_out.as<float>();
+    *bott = *sum = std::numeric_limits<float>::infinity();
+    for (int f = 0; f < n_families; ++f) {
+      const float b = h[(size_t)f * 3 * n_flat + n_flat + i];
+      if (b < *bott) {
+        *bott = b;
+        *sum = h[(size_t)f * 3 * n_flat + 2 * n_flat + i];
+      }
+    }
+  };
+
+  // ---- smallest feasible threshold of every (instance, G), its window of kept thresholds and
+  // the first scan batch, all decided on the device: one round trip.  A window the device
+  // cannot decide (more candidates than it holds, no certain start, nothing kept at or above the
+  // start inside the first fetch) sends the whole search down the host route below. ----
+  std::vector<int> first_batch(n_flat, 0);  // instances of a window the first batch has run
+  bool on_device = false;
+  const char *capacity_env = getenv("MIST_INTER_WINDOW_CAPACITY");  // for tests
+  const int window_capacity = capacity_env ? atoi(capacity_env) : kWindowCapacity;
+  if (!getenv("MIST_INTER_HOST_WINDOWS") && (int64_t)n_flat * kFirstChunk <= 65535) {
+    if (int rc = S.bottleneck_windows_first_batch(flat_rows, grad_accum, n_grad_accum,
+                                                  window_capacity, kFirstChunk))
+      return rc;
+    const float *req = S.ws->h_req.as<float>();
+    const int32_t *meta = S.ws->h_meta.as<int32_t>();
+    const float *kept = S.ws->h_kept.as<float>();
+    on_device = true;
+    int64_t selected = 0, instances = 0;
+    for (int i = 0; i < n_flat && on_device; ++i) {
+      float bott, sum;
+      bottleneck_of(i, &bott, &sum);
+      const int32_t *m = meta + 8 * i;
+      if (!std::isfinite(bott)) continue;
+      Window &w = windows[i];
+      w.exists = true;
+      w.row = flat_rows[i];
+      w.G = grad_accum[i % n_grad_accum];
+      w.start_value = bott;
+      w.start_sum = (double)sum;
+      w.hi = req[2 * n_flat + i];
+      w.complete = m[1] == 0;
+      if (m[2] != 0 || req[3 * n_flat + i] != bott) {
+        on_device = false;
+        break;
+      }
+      w.append(kept + m[4], (size_t)m[3]);
+      // the host route extends such a window before its first batch
+      const size_t pos = (size_t)(std::lower_bound(w.kept.begin(), w.kept.end(), w.start_value) -
+                                  w.kept.begin());
+      if (!w.covers(kInf) || pos != (size_t)m[5] ||
+          (pos + kFirstChunk >= w.kept.size() && !w.covers(kInf))) {
+        on_device = false;
+        break;
+      }
+      first_batch[i] = m[6];
+      selected += m[0];
+      instances += m[6];
+    }
+    if (on_device) {
+      ++S.fetches;
+      S.selected += selected;
+      if (instances > 0) S.launches += n_families;  // (an all-empty batch is no DP batch)
+      S.thresholds_run += instances * n_families;
+    } else {  // start over on the host route, counters included
+      windows.assign(n_flat, Window());
+      first_batch.assign(n_flat, 0);
+      S.launches = S.fetches = S.selected = S.thresholds_run = 0;
+    }
+  }
+
+  // ---- the host route: smallest feasible threshold of every (instance, G) and the first
+  // fetch of its window in one round trip, the windows decided here ----
+  if (!on_device) {
   std::vector<Fetched> first;
   if (int rc = S.bottleneck_and_fetch(flat_rows, grad_accum, n_grad_accum, &first)) return rc;
-  std::vector<Window> windows(n_flat);
   std::vector<int> feasible;
   std::vector<float> hi_first;
   {
-    const float *h = S.ws->h_out.as<float>();
     const float *req = S.ws->h_req.as<float>();
     for (int i = 0; i < n_flat; ++i) {
-      float bott = std::numeric_limits<float>::infinity(), sum = bott;
-      for (int f = 0; f < n_families; ++f) {
-        const float b = h[(size_t)f * 3 * n_flat + n_flat + i];
-        if (b < bott) {
-          bott = b;
-          sum = h[(size_t)f * 3 * n_flat + 2 * n_flat + i];
-        }
-      }
+      float bott, sum;
+      bottleneck_of(i, &bott, &sum);
       if (!std::isfinite(bott)) continue;
       Window &w = windows[i];
       w.exists = true;
@@ -637,6 +797,7 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
         if (int rc = S.apply_extension(brief[j], more[j], want[j])) return rc;
     }
   }
+  }  // host route
 
   // ---- speculative batches + sequential replay ----
   struct Chain {
@@ -658,6 +819,15 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
         sc.pos = (size_t)(std::lower_bound(w.kept.begin(), w.kept.end(), w.start_value) -
                           w.kept.begin());
       sc.have_lo = sc.pos;  // everything below is infeasible: the scan passes it unchanged
+      // the results of the first batch, when the device has run it: the thresholds the scan
+      // below would have asked for first (kFirstChunk from sc.pos on), the next request of this
+      // G grows as after any request
+      const int idx = t * n_grad_accum + i, n_first = first_batch[idx];
+      const int at = on_device ? S.ws->h_meta.as<int32_t>()[8 * idx + 7] : 0;
+      for (int k = 0; k < n_first; ++k)
+        sc.cost.push_back(S.total(at + k, n_flat * kFirstChunk, sc.G, nullptr,
+                                  S.ws->h_out_first.as<float>()));
+      if (n_first > 0) sc.limit = std::min(kMaxChunk, sc.limit * 4);
     }
   }
   int rc_inner = 0;

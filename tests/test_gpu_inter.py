@@ -679,7 +679,7 @@ def test_windows_walked_on_the_device_equal_the_host_walk(capacity, first_chunk)
     d = lambda a: torch.from_numpy(a).to(dev)
     d_rows, d_lo, d_hi, d_start = d(rows), d(lo), d(hi), d(start)
     d_values = torch.empty(n * capacity, dtype=torch.float32, device=dev)
-    d_counts = torch.empty(1 + 2 * n, dtype=torch.int32, device=dev)
+    d_counts = torch.empty(2 + 2 * n, dtype=torch.int32, device=dev)
     d_kept = torch.empty(kept_capacity, dtype=torch.float32, device=dev)
     d_meta = torch.empty(n * 8, dtype=torch.int32, device=dev)
     d_inst_t = torch.full((n * first_chunk,), -7.0, dtype=torch.float32, device=dev)
@@ -694,14 +694,14 @@ def test_windows_walked_on_the_device_equal_the_host_walk(capacity, first_chunk)
         torch.cuda.synchronize()
     meta = d_meta.cpu().numpy().reshape(n, 8)
     kept_all = d_kept.cpu().numpy()
-    inst_t = d_inst_t.cpu().numpy().reshape(n, first_chunk)
-    inst_row = d_inst_row.cpu().numpy().reshape(n, first_chunk)
+    inst_t = d_inst_t.cpu().numpy()
+    inst_row = d_inst_row.cpu().numpy()
 
     host = runner.candidates_between(rows, lo, hi)
-    seen = set()
+    seen, used = set(), []
     for r in range(n):
         values, above = host[r]
-        n_sel, n_above, status, n_kept, base, pos, n_inst, _ = (int(x) for x in meta[r])
+        n_sel, n_above, status, n_kept, base, pos, n_inst, inst_at = (int(x) for x in meta[r])
         want_status = 0
         kept = np.empty(0, dtype=np.float32)
         if not np.isfinite(start[r]):
@@ -724,18 +724,24 @@ def test_windows_walked_on_the_device_equal_the_host_walk(capacity, first_chunk)
         assert status == want_status, (r, status, want_status)
         assert n_sel == len(values) and n_above == above
         if status != 0:
-            assert n_inst == 0 and np.all(inst_row[r] == -1)
+            assert n_inst == 0
             continue
         assert n_kept == len(kept) and np.array_equal(kept_all[base:base + n_kept], kept)
         assert pos == int(np.searchsorted(kept, start[r], side="left"))
         assert n_inst == min(first_chunk, n_kept - pos) > 0
-        assert np.array_equal(inst_t[r, :n_inst], kept[pos:pos + n_inst])
-        assert np.all(inst_row[r, :n_inst] == rows[r]) and np.all(inst_row[r, n_inst:] == -1)
+        assert np.array_equal(inst_t[inst_at:inst_at + n_inst], kept[pos:pos + n_inst])
+        assert np.all(inst_row[inst_at:inst_at + n_inst] == rows[r])
+        used.append((inst_at, n_inst))
     assert {0, 1, 3, 4} <= seen and (capacity > 1024 or 2 in seen)
+    # the instances of all windows lie behind one another from slot 0 on, the rest is empty
+    used.sort()
+    assert used[0][0] == 0 and all(a + k == b for (a, k), (b, _) in zip(used, used[1:]))
+    n_live = used[-1][0] + used[-1][1]
+    assert np.all(inst_row[:n_live] >= 0) and np.all(inst_row[n_live:] == -1)
 
     # the instances as a DP batch: empty slots come back infeasible, the others as on their own
     fam = runner.families[0]
-    flat_row, flat_t = inst_row.reshape(-1), inst_t.reshape(-1)
+    flat_row, flat_t = inst_row, inst_t
     live = flat_row >= 0
     bs, bsum, smax = runner.run(np.where(live, flat_row, -1).astype(np.int32), np.where(live, flat_t, 0).astype(np.float32))
     bs1, bsum1, smax1 = runner.run(flat_row[live], flat_t[live])
@@ -814,6 +820,42 @@ def test_native_search_equals_python_driver(monkeypatch, plan, overrides):
     for only_best in (False, True):
         assert out[True, only_best] == out[False, only_best]
     assert any(sol is not None for _, sol in out[True, False][0]) == (plan != 1 or overrides.get("hardware__memory_capacity") != 1.0)
+
+
+@pytest.mark.parametrize("plan", [1, 2, 3])
+def test_search_decides_its_windows_on_the_device_or_on_the_host_alike(monkeypatch, plan):
+    """The library's search driver with the windows and the first scan batch decided on the
+    device (its default), on the host (``MIST_INTER_HOST_WINDOWS``), and on the host after the
+    device gave up on windows larger than it holds (``MIST_INTER_WINDOW_CAPACITY`` = 128): same
+    costs, partitions, strategies and counters; the device route saves a round trip."""
+    from mist_amd import inter_tuning
+    from mist_amd.config import tp_candidates
+    from mist_amd.intra_tuning import IntraStageTuner
+    from mist_amd.search_space import _get_device_mesh_candidates, _get_grad_accumu_steps_candidates
+
+    cfg, tables = load_plan(plan)
+    hw, L = cfg.hardware, cfg.model.num_hidden_layers
+    D = hw.num_nodes * hw.num_gpus_per_node
+    meshes = _get_device_mesh_candidates(hw.num_nodes, hw.num_gpus_per_node, False)
+    Gs = _get_grad_accumu_steps_candidates(cfg.training.global_batch_size)
+    results = IntraStageTuner(tables, L, meshes, Gs, tp_candidates(cfg), cfg, sample_size=1).tune_all()
+    out = {}
+    for route, env in (("device", {}), ("host", {"MIST_INTER_HOST_WINDOWS": "1"}),
+                       ("gave up", {"MIST_INTER_WINDOW_CAPACITY": "128"})):
+        for name in ("MIST_INTER_HOST_WINDOWS", "MIST_INTER_WINDOW_CAPACITY"):
+            monkeypatch.delenv(name, raising=False)
+        for name, value in env.items():
+            monkeypatch.setenv(name, value)
+        stats = {}
+        got = inter_tuning.inter_stage_tune_batch(L, D, meshes, Gs, results, stats=stats)
+        out[route] = (got, stats["dp_thresholds"], stats["dp_launches"], stats["dp_window_values"])
+        trips = stats["dp_round_trips"]
+        if route == "device":
+            device_trips = trips
+        elif route == "host":
+            assert trips == device_trips + 1 or plan == 1
+    assert out["device"] == out["host"] == out["gave up"]
+    assert any(sol is not None for _, sol in out["device"][0])
 
 
 @pytest.mark.parametrize("plan, overrides, ckpt_tuning", [

@@ -3,9 +3,9 @@
 // uniform-device variant, mist/analyzer/inter_tuning_uniform_device.py:312-367): bottleneck DP,
 // threshold windows, speculative scan batches with the sequential replay of the reference's
 // rules, back-pointers of the winner, strategy rows of its stages.  Same steps as the Python
-// driver (mist_amd/inter_tuning.py); here they run without an interpreter between the batches: a
-// search makes 4-5 dependent round trips to the GPU, and the glue between them was half of its
-// time.
+// driver (mist_amd/inter_tuning.py); here they run without an interpreter between the batches,
+// and the first three of them (bottleneck DP, windows, first scan batch) without the host: a
+// search waits for the GPU three times (that batch, the second scan batch, the back-pointers).
 //
 // A search runs over one or more DP families (shape + tables): the per-mesh recurrence is one
 // family, the uniform-device recurrence one family per admissible stage count.  The cost of a
@@ -14,7 +14,9 @@
 //
 // Everything that decides a result is shared with the Python driver through the C ABI:
 // mist_dp_run, mist_dp_select_candidates, mist_dp_window_begin, mist_dp_filter_tmax,
-// mist_dp_backtrack.  How far a window is fetched or how many thresholds a batch speculates on
+// mist_dp_backtrack (mist_dp_windows_first_batch walks the windows with the code of
+// mist_dp_window_begin, and a window it cannot decide sends the search down the host route).
+// How far a window is fetched or how many thresholds a batch speculates on
 // only changes the work done, never the outcome: the replay consumes DP results in the
 // reference's order with its stop rule and its strict "<".
 #include <hip/hip_runtime.h>

@@ -65,8 +65,10 @@ int mist_inter_stage_search(const MistDpShape *shape, const MistDpCosts *costs, 
  * Additional outputs (HOST): out_family[n_instances] (family of the winning partition, -1 if not
  * walked), out_path[n_instances][S][4] and out_rows[n_instances][S] with S = the largest
  * max_stages of the families (out_rows: row index of stage i's strategy in its group's search
- * space, -1 beyond the partition; may be NULL without `strategy`), out_stats[5] (may be NULL): as
- * above, then the number of stream synchronisations the search waited for. */
+ * space, -1 beyond the partition; may be NULL without `strategy`), out_stats[6] (may be NULL): as
+ * above, then the number of stream synchronisations the search waited for and the number of
+ * threshold windows the device left to the host (those join the scan one batch later, which
+ * changes the batches, not the results). */
 int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
                                      const MistDpCosts *costs, const MistDpCosts *select_costs,
                                      const MistStrategyIndex *strategy, int n_instances,

@@ -220,7 +220,8 @@ struct Search {
   const MistStrategyIndex *strategy;  // may be null
   hipStream_t stream;
   Workspace *ws;
-  int64_t launches = 0, fetches = 0, selected = 0, thresholds_run = 0, round_trips = 0;
+  int64_t launches = 0, fetches = 0, selected = 0, thresholds_run = 0, round_trips = 0,
+          left_to_host = 0;
 
   size_t path_ints(int f) const { return (size_t)shapes[f].max_stages * 4; }
   // ints in front of family f's partitions in the path buffers of a batch of n instances
@@ -652,108 +653,22 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
     }
   };
 
-  // ---- smallest feasible threshold of every (instance, G), its window of kept thresholds and
-  // the first scan batch, all decided on the device: one round trip.  A window the device
-  // cannot decide (more candidates than it holds, no certain start, nothing kept at or above the
-  // start inside the first fetch) sends the whole search down the host route below. ----
-  std::vector<int> first_batch(n_flat, 0);  // instances of a window the first batch has run
-  bool on_device = false;
-  const char *capacity_env = getenv("MIST_INTER_WINDOW_CAPACITY");  // for tests
-  const int window_capacity = capacity_env ? atoi(capacity_env) : kWindowCapacity;
-  if (!getenv("MIST_INTER_HOST_WINDOWS") && (int64_t)n_flat * kFirstChunk <= 65535) {
-    if (int rc = S.bottleneck_windows_first_batch(flat_rows, grad_accum, n_grad_accum,
-                                                  window_capacity, kFirstChunk))
-      return rc;
-    const float *req = S.ws->h_req.as<float>();
-    const int32_t *meta = S.ws->h_meta.as<int32_t>();
-    const float *kept = S.ws->h_kept.as<float>();
-    on_device = true;
-    int64_t selected = 0, instances = 0;
-    for (int i = 0; i < n_flat && on_device; ++i) {
-      float bott, sum;
-      bottleneck_of(i, &bott, &sum);
-      const int32_t *m = meta + 8 * i;
-      if (!std::isfinite(bott)) continue;
-      Window &w = windows[i];
-      w.exists = true;
-      w.row = flat_rows[i];
-      w.G = grad_accum[i % n_grad_accum];
-      w.start_value = bott;
-      w.start_sum = (double)sum;
-      w.hi = req[2 * n_flat + i];
-      w.complete = m[1] == 0;
-      if (m[2] != 0 || req[3 * n_flat + i] != bott) {
-        on_device = false;
-        break;
-      }
-      w.append(kept + m[4], (size_t)m[3]);
-      // the host route extends such a window before its first batch
-      const size_t pos = (size_t)(std::lower_bound(w.kept.begin(), w.kept.end(), w.start_value) -
-                                  w.kept.begin());
-      if (!w.covers(kInf) || pos != (size_t)m[5] ||
-          (pos + kFirstChunk >= w.kept.size() && !w.covers(kInf))) {
-        on_device = false;
-        break;
-      }
-      first_batch[i] = m[6];
-      selected += m[0];
-      instances += m[6];
-    }
-    if (on_device) {
-      ++S.fetches;
-      S.selected += selected;
-      if (instances > 0) S.launches += n_families;  // (an all-empty batch is no DP batch)
-      S.thresholds_run += instances * n_families;
-    } else {  // start over on the host route, counters included
-      windows.assign(n_flat, Window());
-      first_batch.assign(n_flat, 0);
-      S.launches = S.fetches = S.selected = S.thresholds_run = 0;
-    }
-  }
-
-  // ---- the host route: smallest feasible threshold of every (instance, G) and the first
-  // fetch of its window in one round trip, the windows decided here ----
-  if (!on_device) {
-  std::vector<Fetched> first;
-  if (int rc = S.bottleneck_and_fetch(flat_rows, grad_accum, n_grad_accum, &first)) return rc;
-  std::vector<int> feasible;
-  std::vector<float> hi_first;
-  {
-    const float *req = S.ws->h_req.as<float>();
-    for (int i = 0; i < n_flat; ++i) {
-      float bott, sum;
-      bottleneck_of(i, &bott, &sum);
-      if (!std::isfinite(bott)) continue;
-      Window &w = windows[i];
-      w.exists = true;
-      w.row = flat_rows[i];
-      w.G = grad_accum[i % n_grad_accum];
-      w.start_value = bott;
-      w.start_sum = (double)sum;
-      feasible.push_back(i);
-      hi_first.push_back(req[2 * n_flat + i]);
-    }
-  }
-  {
-    std::vector<int> pending(feasible.size());
+  // Decides windows on the host: `got[j]` = the ascending candidates of window todo[j] in
+  // (lo[j], hi[j]] and how many lie above.  A window whose fetched part holds no certain start
+  // of the walk is fetched again from further below; one whose first kept candidate lies higher
+  // than assumed is extended upwards.
+  auto decide_on_host = [&](const std::vector<int> &todo, std::vector<Fetched> got,
+                            std::vector<float> lo, std::vector<float> hi) -> int {
+    const std::vector<float> hi_first = hi;
+    std::vector<int> pending(todo.size());
     for (size_t k = 0; k < pending.size(); ++k) pending[k] = (int)k;
-    // widen 0 is the fetch that came with the bottleneck DP; the requests of the later passes
-    // are made here
-    std::vector<Fetched> got;
-    std::vector<float> lo, hi;
-    for (int k : pending) {
-      got.push_back(std::move(first[feasible[k]]));
-      lo.push_back(S.ws->h_req.as<float>()[n_flat + feasible[k]]);
-      hi.push_back(hi_first[k]);
-    }
-    first.clear();
     for (int widen = 0; !pending.empty(); ++widen) {
       if (widen > 0) {
         std::vector<int32_t> r;
         lo.clear();
         hi.clear();
         for (int k : pending) {
-          const Window &w = windows[feasible[k]];
+          const Window &w = windows[todo[k]];
           r.push_back(w.row);
           lo.push_back(widen >= 8 ? -std::numeric_limits<float>::infinity() : w.lower_margin(widen));
           hi.push_back(hi_first[k]);
@@ -763,7 +678,7 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
       std::vector<int> again;
       std::vector<float> kept;
       for (size_t j = 0; j < pending.size(); ++j) {
-        Window &w = windows[feasible[pending[j]]];
+        Window &w = windows[todo[pending[j]]];
         w.hi = hi[j];
         w.complete = got[j].above == 0;
         const std::vector<float> &v = got[j].values;
@@ -783,7 +698,7 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
     }
     // one more pass for the windows whose first kept candidate lies higher than assumed
     std::vector<Window *> brief;
-    for (int i : feasible)
+    for (int i : todo)
       if (!windows[i].covers(kInf)) brief.push_back(&windows[i]);
     if (!brief.empty()) {
       std::vector<int32_t> r;
@@ -798,8 +713,97 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
       for (size_t j = 0; j < brief.size(); ++j)
         if (int rc = S.apply_extension(brief[j], more[j], want[j])) return rc;
     }
+    return 0;
+  };
+  auto new_window = [&](int i, float bott, float sum) -> Window & {
+    Window &w = windows[i];
+    w = Window();
+    w.exists = true;
+    w.row = flat_rows[i];
+    w.G = grad_accum[i % n_grad_accum];
+    w.start_value = bott;
+    w.start_sum = (double)sum;
+    return w;
+  };
+
+  std::vector<int> first_batch(n_flat, 0);  // instances of a window the first batch has run
+  const char *capacity_env = getenv("MIST_INTER_WINDOW_CAPACITY");  // for tests
+  const int window_capacity = capacity_env ? atoi(capacity_env) : kWindowCapacity;
+  const bool on_device = !getenv("MIST_INTER_HOST_WINDOWS") && (int64_t)n_flat * kFirstChunk <= 65535;
+  if (on_device) {
+    // ---- smallest feasible threshold of every (instance, G), its window of kept thresholds
+    // and the first scan batch, all decided on the device: one round trip.  A window the
+    // device cannot decide (more candidates than it holds, no certain start, nothing kept at or
+    // above the start inside the first fetch) is decided on the host afterwards and joins the
+    // scan with the second batch. ----
+    if (int rc = S.bottleneck_windows_first_batch(flat_rows, grad_accum, n_grad_accum,
+                                                  window_capacity, kFirstChunk))
+      return rc;
+    const float *req = S.ws->h_req.as<float>();
+    const int32_t *meta = S.ws->h_meta.as<int32_t>();
+    const float *kept = S.ws->h_kept.as<float>();
+    std::vector<int> undecided;
+    std::vector<int32_t> u_rows;
+    std::vector<float> u_lo, u_hi;
+    int64_t instances = 0;
+    ++S.fetches;
+    for (int i = 0; i < n_flat; ++i) {
+      float bott, sum;
+      bottleneck_of(i, &bott, &sum);
+      if (!std::isfinite(bott)) continue;
+      const int32_t *m = meta + 8 * i;
+      Window &w = new_window(i, bott, sum);
+      bool decided = m[2] == 0 && req[3 * n_flat + i] == bott;
+      if (decided) {
+        w.hi = req[2 * n_flat + i];
+        w.complete = m[1] == 0;
+        w.append(kept + m[4], (size_t)m[3]);
+        const size_t pos = (size_t)(std::lower_bound(w.kept.begin(), w.kept.end(), w.start_value) -
+                                    w.kept.begin());
+        // (the host route extends a window that does not reach its bound before its first batch)
+        decided = w.covers(kInf) && pos == (size_t)m[5];
+      }
+      if (decided) {
+        first_batch[i] = m[6];
+        S.selected += m[0];
+        instances += m[6];
+      } else {
+        new_window(i, bott, sum);
+        undecided.push_back(i);
+        u_rows.push_back(flat_rows[i]);
+        u_lo.push_back(req[n_flat + i]);
+        u_hi.push_back(req[2 * n_flat + i]);
+      }
+    }
+    if (instances > 0) S.launches += n_families;  // (an all-empty batch is no DP batch)
+    S.thresholds_run += instances * n_families;
+    S.left_to_host = (int64_t)undecided.size();
+    if (!undecided.empty()) {
+      std::vector<Fetched> got;
+      if (int rc = S.fetch(u_rows, u_lo, u_hi, &got)) return rc;
+      if (int rc = decide_on_host(undecided, std::move(got), u_lo, u_hi)) return rc;
+    }
+  } else {
+    // ---- the host route: smallest feasible threshold of every (instance, G) and the first
+    // fetch of its window in one round trip, the windows decided here ----
+    std::vector<Fetched> first;
+    if (int rc = S.bottleneck_and_fetch(flat_rows, grad_accum, n_grad_accum, &first)) return rc;
+    const float *req = S.ws->h_req.as<float>();
+    std::vector<int> feasible;
+    std::vector<Fetched> got;
+    std::vector<float> lo, hi;
+    for (int i = 0; i < n_flat; ++i) {
+      float bott, sum;
+      bottleneck_of(i, &bott, &sum);
+      if (!std::isfinite(bott)) continue;
+      new_window(i, bott, sum);
+      feasible.push_back(i);
+      got.push_back(std::move(first[i]));
+      lo.push_back(req[n_flat + i]);
+      hi.push_back(req[2 * n_flat + i]);
+    }
+    if (int rc = decide_on_host(feasible, std::move(got), lo, hi)) return rc;
   }
-  }  // host route
 
   // ---- speculative batches + sequential replay ----
   struct Chain {
@@ -989,6 +993,7 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
     out_stats[2] = S.selected;
     out_stats[3] = S.thresholds_run;
     out_stats[4] = S.round_trips;
+    out_stats[5] = S.left_to_host;
   }
   return 0;
 }
@@ -1003,7 +1008,7 @@ int mist_inter_stage_search(const MistDpShape *shape, const MistDpCosts *costs, 
     return fail(MIST_E_INVALID, "a single family must be the per-mesh recurrence");
   if (n_instances < 1) return fail(MIST_E_INVALID, "need at least one instance, got %d", n_instances);
   std::vector<int32_t> family(n_instances);
-  int64_t stats[5] = {0, 0, 0, 0, 0};
+  int64_t stats[6] = {0, 0, 0, 0, 0, 0};
   const int rc = mist_inter_stage_search_families(
       1, shape, costs, costs, nullptr, n_instances, n_grad_accum, rows, grad_accum, only_best_path,
       out_cost, out_g, out_tmax, family.data(), out_stages, out_path, nullptr, stats, stream);

@@ -769,7 +769,7 @@ def _native_search(runner: _DpRunner, results_list, rows, Gs, n_g, g_index, q_in
     n_stages = np.empty(n_inst, dtype=np.int32)
     path = np.empty((n_inst, s_max, 4), dtype=np.int32)
     strategy_row = np.empty((n_inst, s_max), dtype=np.int32)
-    counters = np.zeros(5, dtype=np.int64)
+    counters = np.zeros(6, dtype=np.int64)
     t_0 = time.perf_counter()
     with torch.cuda.device(runner.device):
         rc = runner.lib.mist_inter_stage_search_families(
@@ -809,6 +809,7 @@ def _native_search(runner: _DpRunner, results_list, rows, Gs, n_g, g_index, q_in
         stats["dp_window_values"] = stats.get("dp_window_values", 0) + int(counters[2])
         stats["dp_thresholds"] = stats.get("dp_thresholds", 0) + int(counters[3])
         stats["dp_round_trips"] = stats.get("dp_round_trips", 0) + int(counters[4])
+        stats["dp_windows_left_to_host"] = stats.get("dp_windows_left_to_host", 0) + int(counters[5])
     return out
 
 

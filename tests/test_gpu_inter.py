@@ -817,8 +817,13 @@ def test_native_search_equals_python_driver(monkeypatch, plan, overrides):
                                                       only_best_solution=only_best)
             out[native, only_best] = (got, stats["dp_thresholds"], stats["dp_launches"],
                                       stats["dp_window_values"])
+            if stats.get("dp_windows_left_to_host", 0):
+                # a window the device left to the host joins the scan one batch later: other
+                # batches, the same results
+                out[native, only_best] = out[native, only_best][:1]
     for only_best in (False, True):
-        assert out[True, only_best] == out[False, only_best]
+        n = len(out[True, only_best])
+        assert out[True, only_best] == out[False, only_best][:n]
     assert any(sol is not None for _, sol in out[True, False][0]) == (plan != 1 or overrides.get("hardware__memory_capacity") != 1.0)
 
 
@@ -826,8 +831,9 @@ def test_native_search_equals_python_driver(monkeypatch, plan, overrides):
 def test_search_decides_its_windows_on_the_device_or_on_the_host_alike(monkeypatch, plan):
     """The library's search driver with the windows and the first scan batch decided on the
     device (its default), on the host (``MIST_INTER_HOST_WINDOWS``), and on the host after the
-    device gave up on windows larger than it holds (``MIST_INTER_WINDOW_CAPACITY`` = 128): same
-    costs, partitions, strategies and counters; the device route saves a round trip."""
+    device left the windows larger than it holds to it (``MIST_INTER_WINDOW_CAPACITY`` = 128): same
+    costs, partitions and strategies, the first two with the same counters; the device route saves
+    a round trip."""
     from mist_amd import inter_tuning
     from mist_amd.config import tp_candidates
     from mist_amd.intra_tuning import IntraStageTuner
@@ -854,7 +860,10 @@ def test_search_decides_its_windows_on_the_device_or_on_the_host_alike(monkeypat
             device_trips = trips
         elif route == "host":
             assert trips == device_trips + 1 or plan == 1
-    assert out["device"] == out["host"] == out["gave up"]
+    assert out["device"] == out["host"]
+    # windows the device left to the host join the scan one batch later: the same results from
+    # other batches
+    assert out["gave up"][0] == out["device"][0]
     assert any(sol is not None for _, sol in out["device"][0])
 
 
@@ -890,8 +899,11 @@ def test_native_search_of_uniform_device_families_equals_python_driver(monkeypat
                                                       uniform_device=uniform,
                                                       only_best_solution=only_best)
             out[native, only_best] = (got, stats["dp_thresholds"], stats["dp_window_values"])
+            if stats.get("dp_windows_left_to_host", 0):
+                out[native, only_best] = out[native, only_best][:1]
     for only_best in (False, True):
-        assert out[True, only_best] == out[False, only_best]
+        n = len(out[True, only_best])
+        assert out[True, only_best] == out[False, only_best][:n]
     feasible = any(sol is not None for _, sol in out[True, False][0])
     assert feasible == (overrides.get("hardware__memory_capacity") != 1.0)
 

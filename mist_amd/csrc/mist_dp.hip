@@ -30,6 +30,7 @@ constexpr int kDpWideTeam = 8;  // lanes that share one DP state in small batche
 constexpr size_t kDpLdsPerCu = 160 * 1024;  // LDS of a gfx950 compute unit
 constexpr int kDpFusedThreads = 1024;  // largest workgroup of the one-launch kernel
 constexpr int kDpFusedMinInstances = 64;  // threshold batches of at least this size use it
+constexpr int kDpFusedSmallPlane = 2048;  // (L + 1)(D + 1) up to which every batch uses it
 constexpr int kDpStageBatch = 8;   // row minima a lane copies together in the one-launch kernel
 constexpr int kSelectBatch = 8;  // table values a lane of the candidate selection reads together
 constexpr int kSelectBuffer = 4096;  // selected values a workgroup holds before it appends them
@@ -1533,6 +1534,10 @@ int mist_dp_run(const MistDpShape *shape, const MistDpCosts *costs, const float 
   // (threshold batches from about 64 instances on: a workgroup's run through all stage counts
   // takes as long as the 1 + max_stages launches of a few dozen instances)
   bool fused_pays = mode == MIST_DP_THRESHOLD ? n_tmax >= kDpFusedMinInstances : !wide;
+  // (small planes: a workgroup's run through all stage counts is shorter than the launches it
+  // replaces whatever the batch size - GPT-7B's 33 x 33 plane: bottleneck batch of 40 instances
+  // and the back-pointer run of one, 0.07 ms per search; 41 x 65 is already the other way round)
+  fused_pays = fused_pays || plane <= kDpFusedSmallPlane;
   // For tests: MIST_DP_FORCE_SCHEDULE = step | fused | plane takes the choice of schedule away
   // from the batch size and the LDS need, so that each schedule can be run on any shape it
   // supports (a shape it does not support is an error, not a silent fallback).

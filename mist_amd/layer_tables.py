@@ -114,10 +114,22 @@ class LayerTables:
         for name in OP_CLASSES:
             assert name in self.eff, f"synthetic.op_efficiency lacks '{name}'"
         self.gpu_gpu_comm_params = tuple(config.hardware.gpu_gpu_comm_params)
+        # scalar look-ups recur for every (G, mesh) group of a plan
+        self._params_cache: Dict[tuple, np.ndarray] = {}
+        self._act_cache: Dict[tuple, tuple] = {}
 
     # ------------------------------------------------------------------ parameters
     def _params(self, kind: str, tp):
         """Parameter count of one layer of ``kind`` on one tensor-parallel rank."""
+        if np.ndim(tp) == 0:
+            key = (kind, float(tp))
+            hit = self._params_cache.get(key)
+            if hit is None:
+                hit = self._params_cache[key] = self._params_uncached(kind, tp)
+            return hit
+        return self._params_uncached(kind, tp)
+
+    def _params_uncached(self, kind: str, tp):
         tp = _f64(tp)
         h = self.h
         if kind == "block":
@@ -147,6 +159,15 @@ class LayerTables:
 
     def _act_bytes(self, kind: str, b, tp):
         """(saved without checkpointing, extra transient fwd, extra transient bwd) in bytes."""
+        if np.ndim(b) == 0 and np.ndim(tp) == 0:
+            key = (kind, float(b), float(tp))
+            hit = self._act_cache.get(key)
+            if hit is None:
+                hit = self._act_cache[key] = self._act_bytes_uncached(kind, b, tp)
+            return hit
+        return self._act_bytes_uncached(kind, b, tp)
+
+    def _act_bytes_uncached(self, kind: str, b, tp):
         b, tp = _f64(b), _f64(tp)
         s, h = self.s, self.h
         bsh = b * s * h

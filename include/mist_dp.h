@@ -68,7 +68,9 @@ int mist_sizeof_dp_shape(void);
  * intra tuner no longer emits (mist/analyzer/inter_tuning.py:75-92).
  * d_grad_accum[num_grad_accum]: G per g index.  d_out[v]: variant v table for all g, i.e. the
  * layouts of MistOutTables without the trailing sample axis; d_out_pmin[v]: its running minimum
- * along the ckpt axis (what MistDpCosts.pmin* expects). */
+ * along the ckpt axis (what MistDpCosts.pmin* expects).  tables->index[v], when not NULL, must
+ * be the row-index table that belongs to the costs (-1 exactly where they are +inf, as the
+ * intra-stage search leaves them): the costs of such cells are then not read. */
 int mist_dp_cost_tables(const MistProblem *problem, const MistOutTables *tables,
                         const int32_t *d_grad_accum, int slot, float *const d_out[4],
                         float *const d_out_pmin[4], void *stream);

@@ -45,8 +45,12 @@ constexpr int kDpBatch = 4;  // end layers whose reads a lane of the one-lane-pe
 // takes as many whole rows as fit its 256 lanes, one lane per entry, so that loads and stores
 // are contiguous; the running minimum is read back from LDS.  Rows longer than the workgroup
 // are walked in passes of 256 entries with the minimum of the earlier passes carried along.
+// Most cells of a plan hold no strategy (no group for that (g, mesh), or nothing fits): their
+// row index is -1 and their costs +inf, so with the index table (may be null) the 16 bytes of
+// such a cell's costs are not read.
 __global__ __launch_bounds__(256) void cost_table_kernel(const double *__restrict__ stable,
                                                          const double *__restrict__ delta,
+                                                         const int32_t *__restrict__ index,
                                                          const int32_t *__restrict__ grad_accum,
                                                          int64_t n_rows, int64_t rows_per_g,
                                                          int row_len, int sample_size, int slot,
@@ -66,9 +70,11 @@ __global__ __launch_bounds__(256) void cost_table_kernel(const double *__restric
     const int64_t i = r * row_len + j;
     float c = INFINITY;
     if (live) {
-      const float s = (float)stable[i * sample_size + slot];
-      const float d = (float)delta[i * sample_size + slot];
-      c = s + d / G;
+      if (index == nullptr || index[i * sample_size + slot] >= 0) {
+        const float s = (float)stable[i * sample_size + slot];
+        const float d = (float)delta[i * sample_size + slot];
+        c = s + d / G;
+      }
       out[i] = c;
     }
     lds[threadIdx.x] = c;
@@ -1364,7 +1370,8 @@ int mist_dp_cost_tables(const MistProblem *problem, const MistOutTables *tables,
     const int64_t rows_per_block = 256 / std::min<int64_t>(L + 1, 256);
     hipLaunchKernelGGL(cost_table_kernel,
                        dim3((unsigned)((n + rows_per_block - 1) / rows_per_block)), dim3(256), 0,
-                       (hipStream_t)stream, tables->stable[v], tables->delta[v], d_grad_accum, n,
+                       (hipStream_t)stream, tables->stable[v], tables->delta[v], tables->index[v],
+                       d_grad_accum, n,
                        rows_per_g[v], (int)(L + 1), (int)S, slot, d_out[v], d_out_pmin[v]);
     MIST_HIP_CHECK(hipGetLastError());
   }

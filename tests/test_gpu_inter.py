@@ -907,3 +907,142 @@ def test_native_search_of_uniform_device_families_equals_python_driver(monkeypat
     feasible = any(sol is not None for _, sol in out[True, False][0])
     assert feasible == (overrides.get("hardware__memory_capacity") != 1.0)
 
+
+
+class _ToySpace:
+    """Stand-in for a group's strategy rows: row index -> ten numbers (the first six whole)."""
+
+    @staticmethod
+    def decode(idx):
+        idx = np.asarray(idx)
+        out = np.full(idx.shape + (10,), np.inf, dtype=np.float64)
+        ok = idx >= 0
+        base = idx[ok].astype(np.float64)
+        out[ok] = np.stack([base % 3 + 1, base % 5, base % 7, base % 2, base % 11, base % 13,
+                            base / 4, base / 8, base / 16, base / 32], axis=-1)
+        return out
+
+
+def _synthetic_results(rng, n_entries, Gs, meshes, L, P1, S, quantum, inf_frac, structured,
+                       structured_exponent=1.0, jitter=0.0):
+    """Random intra-stage tables for ``n_entries`` tensor-parallel entries: in HBM in the layout
+    the search kernels write (one leading axis over entry x G), and as the oracle's results
+    objects.  Values are multiples of ``quantum`` (exact in float32, many ties after the division
+    by G); ``structured`` makes a stage's cost grow with its layers and fall with its devices and
+    its micro-batch count, as real tables do; otherwise it is uniform noise times
+    ``(max G / G) ** structured_exponent``.  ``jitter`` adds 0..3 times itself to every stable
+    cost."""
+    import torch
+    from mist_amd.intra_tuning import DeviceTables, IntraStageTunerOutput
+    from oracle.intra import IntraStageTunerOutput as OracleOutput
+
+    Gn, Q = n_entries * len(Gs), len(meshes)
+    shapes = [(Gn, Q, P1, L, L + 1, S), (Gn, Q, P1, L, L + 1, S), (Gn, Q, L, L + 1, S), (Gn, Q, L + 1, S)]
+    layers = np.arange(1, L + 1, dtype=np.float64)
+    devices = np.array([n * m for n, m in meshes], dtype=np.float64)
+    stable, delta, index = [], [], []
+    for v, shape in enumerate(shapes):
+        # the whole model on one mesh costs about as much as its layers in stages
+        per_g = np.tile(max(Gs) / np.array(Gs, dtype=np.float64), n_entries).reshape((Gn,) + (1,) * (len(shape) - 1))
+        if structured:
+            per_q = (devices ** -0.7).reshape((Q,) + (1,) * (len(shape) - 2))
+            per_l = layers.reshape((L, 1, 1)) if v < 3 else L
+            scale = np.ones(shape) * per_l * per_q * per_g
+        else:
+            scale = np.ones(shape) * (1.0 if v < 3 else L / 2) * per_g ** structured_exponent
+        s = np.maximum(np.round(rng.uniform(0.3, 1.0, size=shape) * scale / quantum), 1) * quantum
+        d = np.round(rng.uniform(0.0, 0.5, size=shape) * scale / quantum) * quantum
+        if jitter:  # neighbours closer than the scan's gap of 1e-6
+            s = s + rng.integers(0, 4, size=shape) * jitter
+        none = rng.random(shape) < (inf_frac if v < 3 else max(inf_frac, 0.6))  # one mesh rarely holds it
+        s[none], d[none] = np.inf, np.inf
+        idx = rng.integers(0, 1000, size=shape).astype(np.int32)
+        idx[none] = -1
+        stable.append(s), delta.append(d), index.append(idx)
+    whole = DeviceTables(stable=[torch.from_numpy(a).cuda() for a in stable],
+                         delta=[torch.from_numpy(a).cuda() for a in delta],
+                         index=[torch.from_numpy(a).cuda() for a in index])
+    n_g = len(Gs)
+    spaces = {(g, q): _ToySpace for g in range(n_g) for q in range(Q)}
+    ours, theirs = [], []
+    for t in range(n_entries):
+        cut = slice(t * n_g, (t + 1) * n_g)
+        view = DeviceTables(stable=[x[cut] for x in whole.stable], delta=[x[cut] for x in whole.delta],
+                            index=[x[cut] for x in whole.index])
+        ours.append(IntraStageTunerOutput(Gs, meshes, view, spaces, range(S), batch=whole, batch_index=t))
+        f32 = [a[cut].astype(np.float32) for a in stable] + [a[cut].astype(np.float32) for a in delta]
+        theirs.append(OracleOutput(Gs, meshes, *f32, *[_ToySpace.decode(a[cut]) for a in index]))
+    return ours, theirs
+
+
+@pytest.mark.parametrize("seed, L, nodes, gpn, quantum, inf_frac", [
+    (0, 8, 1, 8, 1 / 16, 0.15),
+    (1, 10, 2, 4, 1 / 64, 0.3),
+    (2, 7, 2, 2, 1 / 8, 0.05),
+    (3, 11, 2, 4, 1 / 128, 0.2),
+    (4, 9, 1, 4, 1 / 32, 0.6),
+    (5, 6, 2, 4, 1 / 4, 0.0),
+    # larger shapes, up to 11 stages deep: per-mesh only (its oracle DP is compiled C)
+    (6, 16, 2, 8, 1 / 256, 0.25),
+    (7, 20, 4, 4, 1 / 512, 0.1),
+    (8, 24, 4, 8, 1 / 8, 0.4),
+])
+@pytest.mark.parametrize("recurrence", ["per-mesh", "uniform-device", "uniform-device, ckpt rule"])
+def test_search_on_random_tables_equals_the_reference_scan(monkeypatch, seed, L, nodes, gpn, quantum,
+                                                           inf_frac, recurrence):
+    """The search driver (windows, speculative scan batches, replay, back-pointer run) against
+    the reference's own procedure - every candidate threshold in ascending order through the DP,
+    with the gap and stop rules of inter_tuning.py:163-217 /
+    inter_tuning_uniform_device.py:212-273 - on random tables full of ties that no layer model
+    made: up to three tensor-parallel entries searched in one call, each with its own running best, a
+    sample slot other than the first, and the driver on each of its routes (windows decided on
+    the device, on the host, on the host after the device gave up, the Python driver)."""
+    from mist_amd import inter_tuning
+    from oracle import inter_dp, inter_uniform_device
+    from oracle.dp_c import dp_impl_c
+
+    if seed >= 6 and recurrence != "per-mesh":
+        pytest.skip("the uniform-device oracle is interpreted loops: small shapes only")
+    rng = np.random.default_rng(9100 + seed)
+    D = nodes * gpn
+    n_entries = {7: 2, 8: 1}.get(seed, 3)
+    meshes = [(1, 1 << k) for k in range(gpn.bit_length()) if (1 << k) <= gpn]
+    meshes += [(n, gpn) for n in range(2, nodes + 1) if nodes % n == 0]
+    Gs = [1, 2, 4, 8, 32][:3 + seed % 3]
+    P1 = min(D, L)
+    S, slot = 2, 1
+    ours, theirs = _synthetic_results(rng, n_entries, Gs, meshes, L, P1, S, quantum, inf_frac,
+                                      structured=seed % 2 == 0,
+                                      structured_exponent=(1.1, 1.0, 0.9)[seed // 2 % 3],
+                                      jitter=3e-7 if seed in (3, 4, 7) else 0.0)
+    if recurrence == "per-mesh":
+        uniform = None
+        want = [inter_dp.inter_stage_tune(L, D, meshes, Gs, r, slot, dp=dp_impl_c) for r in theirs]
+    else:
+        ckpt_tuning = recurrence == "uniform-device"
+        uniform = dict(num_nodes=nodes, num_gpus_per_node=gpn, ckpt_tuning=ckpt_tuning)
+
+        class Config:
+            class tuning:
+                activation_checkpointing_tuning_enabled = ckpt_tuning
+
+        want = [inter_uniform_device.inter_stage_tune(L, nodes, gpn, meshes, Gs, r, Config, slot)
+                for r in theirs]
+    if inf_frac < 0.5:
+        assert any(sol is not None for _, sol in want), "degenerate case"
+    routes = [(True, {}), (True, {"MIST_INTER_HOST_WINDOWS": "1"}),
+              (True, {"MIST_INTER_WINDOW_CAPACITY": "128"}), (False, {})]
+    for native, env in routes:
+        for name in ("MIST_INTER_HOST_WINDOWS", "MIST_INTER_WINDOW_CAPACITY"):
+            monkeypatch.delenv(name, raising=False)
+        for name, value in env.items():
+            monkeypatch.setenv(name, value)
+        monkeypatch.setattr(inter_tuning, "NATIVE_SEARCH", native)
+        got = inter_tuning.inter_stage_tune_batch(L, D, meshes, Gs, ours, slot=slot,
+                                                  uniform_device=uniform)
+        assert got == want, (native, env)
+    got = inter_tuning.inter_stage_tune_batch(L, D, meshes, Gs, ours, slot=slot, uniform_device=uniform,
+                                              only_best_solution=True)
+    finite = [i for i, (_, sol) in enumerate(want) if sol is not None]
+    keep = min(finite, key=lambda i: want[i][0]) if finite else None
+    assert got == [(cost, sol if i == keep else None) for i, (cost, sol) in enumerate(want)]

@@ -169,9 +169,10 @@ def workspace_positions(n_par: int, n_pair: int, n_oo: int, n_ao: int) -> np.nda
 
 
 def exported_symbols():
-    """Names every entry point declared in include/mist_search.h, mist_dp.h, mist_mip.h and
-    mist_inter.h."""
-    return tuple(_SIGNATURES) + tuple(_DP_SIGNATURES) + tuple(_MIP_SIGNATURES) + tuple(_INTER_SIGNATURES)
+    """Names every entry point declared in include/mist_search.h, mist_dp.h, mist_mip.h,
+    mist_inter.h and mist_plan.h."""
+    return (tuple(_SIGNATURES) + tuple(_DP_SIGNATURES) + tuple(_MIP_SIGNATURES) + tuple(_INTER_SIGNATURES)
+            + tuple(_PLAN_SIGNATURES))
 
 
 DP_SHAPE_DTYPE = np.dtype(
@@ -310,6 +311,81 @@ _INTER_SIGNATURES = {
          _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP]),
 }
 
+PLAN_MAX_LIST = 32
+PLAN_MAX_BATCH_SIZES = 64
+PLAN_UNSUPPORTED = -3  # MIST_E_PLAN_UNSUPPORTED
+# efficiency classes in the order of MistLayerShapes.efficiency (include/mist_plan.h)
+PLAN_OP_CLASSES = (
+    "qkv_gemm", "attn_core", "attn_softmax", "out_gemm", "fc1_gemm", "fc2_gemm", "activation",
+    "norm", "embedding", "lm_head_gemm", "xentropy", "grad_accum",
+)
+PLAN_PP_MODES = {"dp": 0, "intra-node-tp-with-ore": 1, "intra-node-tp-without-ore": 2, "preset": 3}
+
+
+class LayerShapes(ctypes.Structure):
+    """MistLayerShapes (include/mist_plan.h)."""
+    _fields_ = [
+        ("hidden", ctypes.c_double), ("heads", ctypes.c_double), ("kv_heads", ctypes.c_double),
+        ("ffn", ctypes.c_double), ("vocab", ctypes.c_double), ("seq_len", ctypes.c_double),
+        ("norm_params", ctypes.c_double), ("opt_mult", ctypes.c_double),
+        ("bytes_per_param", ctypes.c_double), ("peak_flops", ctypes.c_double),
+        ("hbm_bw", ctypes.c_double),
+        ("efficiency", (ctypes.c_double * 2) * len(PLAN_OP_CLASSES)),
+        ("flash", ctypes.c_int32), ("gated", ctypes.c_int32), ("abs_pos", ctypes.c_int32),
+        ("tied", ctypes.c_int32),
+    ]
+
+
+class PlanRequest(ctypes.Structure):
+    """MistPlanRequest (include/mist_plan.h)."""
+    _fields_ = [
+        ("layers", LayerShapes),
+        ("gpu_gpu", ctypes.c_double * 32),
+        ("memory_capacity_gb", ctypes.c_double),
+        ("wo", ctypes.c_double * MAX_RATIOS), ("go", ctypes.c_double * MAX_RATIOS),
+        ("oo", ctypes.c_double * MAX_RATIOS), ("ao", ctypes.c_double * MAX_RATIOS),
+        ("pp_preset", ctypes.c_double * 10),
+        ("scout_tight_fraction", ctypes.c_double),
+        ("global_batch_size", ctypes.c_int64),
+        ("workspace_rows", ctypes.c_int64),
+        ("model_heads", ctypes.c_int32), ("model_seq_len", ctypes.c_int32), ("model_flash", ctypes.c_int32),
+        ("num_layers", ctypes.c_int32), ("max_pre_saved", ctypes.c_int32),
+        ("evaluate_all_p", ctypes.c_int32), ("exhaustive", ctypes.c_int32),
+        ("n_tp", ctypes.c_int32), ("tp_size", ctypes.c_int32 * PLAN_MAX_LIST),
+        ("n_grad_accum", ctypes.c_int32), ("grad_accum", ctypes.c_int32 * PLAN_MAX_LIST),
+        ("n_mesh", ctypes.c_int32), ("mesh_n", ctypes.c_int32 * MAX_MESH), ("mesh_m", ctypes.c_int32 * MAX_MESH),
+        ("n_batch_sizes", ctypes.c_int32), ("batch_size", ctypes.c_int32 * PLAN_MAX_BATCH_SIZES),
+        ("zero_2_and_3", ctypes.c_int32), ("n_flag_choices", ctypes.c_int32),
+        ("flag_choice", (ctypes.c_int32 * 3) * PLAN_MAX_LIST),
+        ("disable_tp", ctypes.c_int32), ("check_shapes", ctypes.c_int32),
+        ("n_wo", ctypes.c_int32), ("n_go", ctypes.c_int32), ("n_oo", ctypes.c_int32),
+        ("n_ao", ctypes.c_int32), ("n_pair", ctypes.c_int32),
+        ("pair_wo", ctypes.c_uint8 * MAX_PAIRS), ("pair_go", ctypes.c_uint8 * MAX_PAIRS),
+        ("pp_mode", ctypes.c_int32),
+        ("target_reduce_waves", ctypes.c_int32), ("scout_min_stages", ctypes.c_int32),
+        ("scout_min_pairs", ctypes.c_int32), ("scout_pairs", ctypes.c_int32),
+        ("scout_pair_span", ctypes.c_int32), ("scout_tight_pairs", ctypes.c_int32),
+        ("cells_wanted", ctypes.c_void_p),
+    ]
+
+
+class PlanResult(ctypes.Structure):
+    """MistPlanResult (include/mist_plan.h)."""
+    _fields_ = [
+        ("n_groups", ctypes.c_int32), ("n_batches", ctypes.c_int32),
+        ("max_scout_rows", ctypes.c_int32), ("max_group_keys", ctypes.c_int32),
+        ("total_rows", ctypes.c_int64), ("n_space_rows", ctypes.c_int64),
+    ]
+
+
+_PLAN_SIGNATURES = {
+    "mist_sizeof_plan_request": (ctypes.c_int, []),
+    "mist_plan_groups": (
+        ctypes.c_int,
+        [ctypes.POINTER(PlanRequest), _VP, ctypes.c_int32, _VP, _VP, _VP, _VP, _VP, _VP, _VP,
+         ctypes.POINTER(PlanResult)]),
+}
+
 _MIP_SIGNATURES = {
     "mist_sizeof_mip_shape": (ctypes.c_int, []),
     "mist_mip_stage_samples": (
@@ -344,7 +420,7 @@ def load():
 
     lib = ctypes.CDLL(LIB_PATH)
     for name, (restype, argtypes) in {**_SIGNATURES, **_DP_SIGNATURES, **_MIP_SIGNATURES,
-                                      **_INTER_SIGNATURES}.items():
+                                      **_INTER_SIGNATURES, **_PLAN_SIGNATURES}.items():
         fn = getattr(lib, name)
         fn.restype = restype
         fn.argtypes = argtypes
@@ -368,6 +444,10 @@ def load():
         raise MistLibraryError(
             f"MistMipBatchItem layout mismatch: C {lib.mist_sizeof_mip_batch_item()} vs ctypes "
             f"{ctypes.sizeof(MipBatchItem)}")
+    if lib.mist_sizeof_plan_request() != ctypes.sizeof(PlanRequest):
+        raise MistLibraryError(
+            f"MistPlanRequest layout mismatch: C {lib.mist_sizeof_plan_request()} vs ctypes "
+            f"{ctypes.sizeof(PlanRequest)}")
     if lib.mist_sizeof_group() != GROUP_DTYPE.itemsize:
         raise MistLibraryError(
             f"MistGroupDesc layout mismatch: C {lib.mist_sizeof_group()} vs numpy {GROUP_DTYPE.itemsize}"

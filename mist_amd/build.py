@@ -10,7 +10,7 @@ import subprocess
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 REPO_DIR = os.path.dirname(PKG_DIR)
 LIB_PATH = os.path.join(PKG_DIR, "libmist_search.so")
-SOURCES = [os.path.join(PKG_DIR, "csrc", name) for name in ("mist_search.hip", "mist_dp.hip", "mist_mip.hip", "mist_inter.hip")]
+SOURCES = [os.path.join(PKG_DIR, "csrc", name) for name in ("mist_search.hip", "mist_dp.hip", "mist_mip.hip", "mist_inter.hip", "mist_plan.hip")]
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
     "-O3",

@@ -10,6 +10,8 @@ fields and layouts as the reference (:59-82); numpy copies are made lazily on fi
 from __future__ import annotations
 
 import ctypes
+import os
+from collections.abc import Mapping
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence, Tuple
 
@@ -202,6 +204,53 @@ class IntraStageTunerOutput:
         )
 
 
+class _PlanSpaces(Mapping):
+    """``(t, g, q) -> SearchSpace`` over the parallelism rows ``mist_plan_groups`` returns; a
+    space is made when it is asked for (a search decodes a handful of its 240)."""
+
+    def __init__(self, shape, offsets, rows, lists):
+        self._shape, self._offsets, self._rows, self._lists = shape, offsets, rows, lists
+        self._made: Dict[Tuple[int, int, int], SearchSpace] = {}
+
+    def __getitem__(self, key):
+        space = self._made.get(key)
+        if space is None:
+            t, g, q = key
+            T, Gn, Qn = self._shape
+            if not (0 <= t < T and 0 <= g < Gn and 0 <= q < Qn):
+                raise KeyError(key)
+            entry = (t * Gn + g) * Qn + q
+            wo, go, oo, ao, pair_wo, pair_go = self._lists
+            par = self._rows[self._offsets[entry]:self._offsets[entry + 1]]
+            space = self._made[key] = SearchSpace(par=par, wo=wo, go=go, oo=oo, ao=ao,
+                                                  pair_wo=pair_wo, pair_go=pair_go)
+        return space
+
+    def __iter__(self):
+        T, Gn, Qn = self._shape
+        return ((t, g, q) for t in range(T) for g in range(Gn) for q in range(Qn))
+
+    def __len__(self):
+        T, Gn, Qn = self._shape
+        return T * Gn * Qn
+
+
+class _SpacesOfEntry(Mapping):
+    """The ``(g, q) -> SearchSpace`` view of one tensor-parallel entry ``t`` of a plan's spaces."""
+
+    def __init__(self, spaces, t: int):
+        self._spaces, self._t = spaces, t
+
+    def __getitem__(self, key):
+        return self._spaces[(self._t, key[0], key[1])]
+
+    def __iter__(self):
+        return ((g, q) for (t, g, q) in self._spaces if t == self._t)
+
+    def __len__(self):
+        return sum(1 for _ in iter(self))
+
+
 class IntraStageTuner:
     """Reference: ``IntraStageTuner`` (mist/analyzer/intra_tuning.py:84-282).  ``layer_tables``
     replaces the three ``LayerInfo`` arguments."""
@@ -258,8 +307,126 @@ class IntraStageTuner:
 
     # ------------------------------------------------------------------ host side
     def prepare(self):
-        """Builds the group descriptors and the launch decomposition (host only, no GPU)."""
+        """Builds the group descriptors and the launch decomposition (host only, no GPU): in the
+        library (``mist_plan_groups``) for plans on the closed-form layer tables, in python
+        otherwise and when ``MIST_PYTHON_PLAN_BUILDER`` is set; the two give the same bytes."""
         _lib.load()  # the tile sizes of the decomposition are the library's
+        built = None
+        if not os.environ.get("MIST_PYTHON_PLAN_BUILDER"):
+            built = self._build_groups_native()
+        if built is None:
+            built = self._build_groups_python()
+        return self._finish_plan(*built)
+
+    def _cells_wanted_of(self, G, mesh):
+        """``cells_wanted`` of a (G, mesh) as ``(smallest layer count, largest, number of
+        pre-saved micro-batch values)`` or None when the caller reads nothing of it."""
+        wanted = self.cells_wanted(G, mesh)
+        if wanted is None:
+            return None
+        l_min, l_max, p_count = wanted
+        l_min, l_max = max(int(l_min), 1), min(int(l_max), self.num_layers)
+        if l_min > l_max or p_count < 1:
+            return None
+        return l_min, l_max, int(p_count)
+
+    def _build_groups_native(self):
+        """The groups of this call from ``mist_plan_groups``, or None when the plan is outside
+        what it covers or fails one of its checks (the python builder then words the error)."""
+        cfg, tables, L = self.config, self.layer_tables, self.num_layers
+        if type(tables) is not LayerTables:
+            return None  # latencies from an operator database: python look-ups
+        Gs, Q = self.gradient_accumulation_steps_candidates, self.device_mesh_candidates
+        factory = SearchSpaceFactory(cfg, tables.constraint)
+        wo, go, oo, ao, pair_wo, pair_go = factory.lists
+        pp_mode = _lib.PLAN_PP_MODES.get(cfg.tuning.pre_post_strategy)
+        ints = [*Gs, *(n for n, _ in Q), *(m for _, m in Q), *factory.batch_sizes, L,
+                cfg.training.global_batch_size, cfg.model.num_attention_heads,
+                cfg.training.max_sequence_length, *(t for t in self.tp_sizes if t is not None)]
+        if (pp_mode is None or (pp_mode == _lib.PLAN_PP_MODES["preset"] and cfg.strategy is None)
+                or len(self.tp_sizes) > _lib.PLAN_MAX_LIST or len(Gs) > _lib.PLAN_MAX_LIST
+                or len(Q) > _lib.MAX_MESH or len(factory.batch_sizes) > _lib.PLAN_MAX_BATCH_SIZES
+                or len(factory.flag_choices) > _lib.PLAN_MAX_LIST
+                or not all(isinstance(v, (int, np.integer)) and 0 < v < 2**31 for v in ints)):
+            return None
+        req = _lib.PlanRequest()
+        lay = req.layers
+        lay.hidden, lay.heads, lay.kv_heads, lay.ffn = tables.h, tables.heads, tables.kv_heads, tables.ffn
+        lay.vocab, lay.seq_len, lay.norm_params = tables.vocab, tables.s, tables.norm_params
+        lay.opt_mult, lay.bytes_per_param = tables.opt_mult, tables.bytes_per_param
+        lay.peak_flops, lay.hbm_bw = tables.peak_flops, tables.hbm_bw
+        for i, name in enumerate(_lib.PLAN_OP_CLASSES):
+            lay.efficiency[i][0], lay.efficiency[i][1] = tables.eff[name]
+        lay.flash, lay.gated, lay.abs_pos, lay.tied = tables.flash, tables.gated, tables.abs_pos, tables.tied
+        if len(tables.gpu_gpu_comm_params) != 32 or len(cfg.hardware.gpu_gpu_comm_params) != 32:
+            return None
+        if tuple(tables.gpu_gpu_comm_params) != tuple(cfg.hardware.gpu_gpu_comm_params):
+            return None
+        req.gpu_gpu[:] = [float(x) for x in cfg.hardware.gpu_gpu_comm_params]
+        req.memory_capacity_gb = cfg.hardware.memory_capacity
+        req.wo[:len(wo)], req.go[:len(go)], req.oo[:len(oo)], req.ao[:len(ao)] = wo, go, oo, ao
+        req.n_wo, req.n_go, req.n_oo, req.n_ao, req.n_pair = len(wo), len(go), len(oo), len(ao), len(pair_wo)
+        ctypes.memmove(req.pair_wo, pair_wo.ctypes.data, len(pair_wo))
+        ctypes.memmove(req.pair_go, pair_go.ctypes.data, len(pair_go))
+        if pp_mode == _lib.PLAN_PP_MODES["preset"]:
+            preset = [float(x) for x in cfg.strategy.pre_post_strategy_array]
+            if len(preset) != 10 or any(x != int(x) for x in preset[1:3]):
+                return None
+            req.pp_preset[:] = preset
+        req.pp_mode = pp_mode
+        req.scout_tight_fraction = SCOUT_TIGHT_FRACTION
+        req.global_batch_size = cfg.training.global_batch_size
+        req.workspace_rows = max(ROW_TERMS_BUDGET_BYTES // (8 * _lib.ROW_TERMS), 1)
+        req.model_heads, req.model_seq_len = cfg.model.num_attention_heads, cfg.training.max_sequence_length
+        req.model_flash = bool(cfg.model.use_flash_attn)
+        req.num_layers, req.max_pre_saved = L, self.max_possible_pre_saved_micro_batches
+        req.evaluate_all_p, req.exhaustive = bool(self.evaluate_all_p), bool(self.exhaustive)
+        req.n_tp, req.n_grad_accum, req.n_mesh = len(self.tp_sizes), len(Gs), len(Q)
+        req.tp_size[:req.n_tp] = [0 if t is None else t for t in self.tp_sizes]
+        req.grad_accum[:req.n_grad_accum] = Gs
+        req.mesh_n[:req.n_mesh] = [n for n, _ in Q]
+        req.mesh_m[:req.n_mesh] = [m for _, m in Q]
+        req.n_batch_sizes = len(factory.batch_sizes)
+        req.batch_size[:req.n_batch_sizes] = factory.batch_sizes
+        req.zero_2_and_3, req.disable_tp, req.check_shapes = factory.zero_2_and_3, factory.disable_tp, 1
+        req.n_flag_choices = len(factory.flag_choices)
+        for i, flags in enumerate(factory.flag_choices):
+            req.flag_choice[i][:] = flags
+        req.target_reduce_waves, req.scout_min_stages = TARGET_REDUCE_WAVES, SCOUT_MIN_STAGES
+        req.scout_min_pairs, req.scout_pairs = SCOUT_MIN_PAIRS, SCOUT_PAIRS
+        req.scout_pair_span, req.scout_tight_pairs = SCOUT_PAIR_SPAN, SCOUT_TIGHT_PAIRS
+        wanted = None
+        if self.cells_wanted is not None:
+            wanted = np.full((len(Gs), len(Q), 3), -1, dtype=np.int32)
+            for g, G in enumerate(Gs):
+                for q, mesh in enumerate(Q):
+                    cells = self._cells_wanted_of(G, mesh)
+                    if cells is not None:
+                        wanted[g, q] = cells
+            req.cells_wanted = wanted.ctypes.data
+        entries = req.n_tp * req.n_grad_accum * req.n_mesh
+        groups = np.zeros(entries, dtype=_lib.GROUP_DTYPE)
+        space_offset = np.empty(entries + 1, dtype=np.int64)
+        space_rows = np.empty((entries * _lib.MAX_PAR, 6), dtype=np.float64)
+        group_of_entry = np.empty(entries, dtype=np.int32)
+        prefixes = np.empty((4, entries + 1), dtype=np.int32)
+        result = _lib.PlanResult()
+        ptr = lambda a: ctypes.c_void_p(a.ctypes.data)
+        rc = _lib.load().mist_plan_groups(
+            ctypes.byref(req), ptr(groups), entries, ptr(space_offset), ptr(space_rows),
+            ptr(group_of_entry), ptr(prefixes[0]), ptr(prefixes[1]), ptr(prefixes[2]), ptr(prefixes[3]),
+            ctypes.byref(result))
+        if rc == _lib.PLAN_UNSUPPORTED:
+            return None
+        _lib.check(rc, "mist_plan_groups")
+        n = result.n_groups
+        spaces = _PlanSpaces((req.n_tp, req.n_grad_accum, req.n_mesh), space_offset,
+                             space_rows[:result.n_space_rows], factory.lists)
+        bounds = [(int(prefixes[3, i]), int(prefixes[3, i + 1])) for i in range(result.n_batches)]
+        return (groups[:n], spaces, prefixes[0, :n + 1], prefixes[1, :n + 1], prefixes[2, :n + 1], bounds,
+                result.max_scout_rows, result.max_group_keys)
+
+    def _build_groups_python(self):
         cfg, L = self.config, self.num_layers
         Gs, Q = self.gradient_accumulation_steps_candidates, self.device_mesh_candidates
         P = self.max_possible_pre_saved_micro_batches
@@ -284,14 +451,11 @@ class IntraStageTuner:
                         num_p = P + 1
                     window = (0, -(-n_pairs // _lib.LC_TILE))
                     if self.cells_wanted is not None:
-                        wanted = self.cells_wanted(G, (n, m))
+                        wanted = self._cells_wanted_of(G, (n, m))
                         if wanted is None:
                             continue
                         l_min, l_max, p_count = wanted
-                        l_min, l_max = max(int(l_min), 1), min(int(l_max), L)
-                        if l_min > l_max or p_count < 1:
-                            continue
-                        num_p = min(num_p, int(p_count))
+                        num_p = min(num_p, p_count)
                         # pairs are numbered l-major: index(l, c) = l (l + 1) / 2 - 1 + c
                         first = (l_min * (l_min + 1) // 2 - 1) // _lib.LC_TILE
                         last = (l_max * (l_max + 1) // 2 - 1 + l_max) // _lib.LC_TILE
@@ -302,12 +466,14 @@ class IntraStageTuner:
         builder.fill_many(groups, pending)
         builder.validate(groups)
 
+        bounds = self._batch_bounds(groups["n_rows"]) if len(pending) else []
+        max_scout_rows = max_group_keys = 0
         if len(pending):
             groups["lc_tile_begin"] = [w[0] for w in tile_window]
             n_lc_tiles = np.array([w[1] for w in tile_window], dtype=np.int64)
             n_p_tiles = -(-groups["num_p"] // _lib.P_TILE)
             # the row chunks are sized per batch of groups (one reduce launch each, see below)
-            for first, last in self._batch_bounds(groups["n_rows"]):
+            for first, last in bounds:
                 sel = slice(first, last)
                 tile_rows = int(np.sum(groups["n_rows"][sel] * n_lc_tiles[sel] * n_p_tiles[sel]))
                 rows_per_chunk = -(-tile_rows // max(TARGET_REDUCE_WAVES * 64 // _lib.LC_TILE, 1))
@@ -345,6 +511,10 @@ class IntraStageTuner:
             scout_blocks = n_lc_tiles * _lib.SCOUT_SPLIT * n_p_tiles
             if not np.any(groups["scout_stride"] > 0):
                 scout_blocks[:] = 0
+            scouted = groups["scout_stride"] > 0
+            gathered = groups["n_par"] * groups["n_oo"] * groups["n_ao"] * groups["scout_stride"]
+            max_scout_rows = int(gathered[scouted].max()) if scouted.any() else 0
+            max_group_keys = int(n_keys.max())
         else:
             terms_blocks = reduce_blocks = scout_blocks = np.zeros(0, dtype=np.int64)
         terms_prefix = np.concatenate(([0], np.cumsum(terms_blocks))).astype(np.int64)
@@ -352,20 +522,30 @@ class IntraStageTuner:
         scout_prefix = np.concatenate(([0], np.cumsum(scout_blocks))).astype(np.int64)
         if terms_prefix[-1] >= 2**31 or reduce_prefix[-1] + scout_prefix[-1] >= 2**31:
             raise ValueError("launch decomposition exceeds 2**31 workgroups")
+        return (groups, spaces, terms_prefix, reduce_prefix, scout_prefix, bounds, max_scout_rows,
+                max_group_keys)
+
+    def _finish_plan(self, groups, spaces, terms_prefix, reduce_prefix, scout_prefix, bounds,
+                     max_scout_rows, max_group_keys):
+        cfg, L = self.config, self.num_layers
+        Gs, Q = self.gradient_accumulation_steps_candidates, self.device_mesh_candidates
+        P = self.max_possible_pre_saved_micro_batches
         problem = make_problem(cfg, L, P + 1, self.sample_size, len(self.tp_sizes) * len(Gs), len(Q))
-        if len(pending):
-            scouted = groups["scout_stride"] > 0
-            gathered = groups["n_par"] * groups["n_oo"] * groups["n_ao"] * groups["scout_stride"]
-            problem["max_scout_rows"] = int(gathered[scouted].max()) if scouted.any() else 0
-            problem["max_group_keys"] = int(n_keys.max())
+        if len(groups):
+            problem["max_scout_rows"] = max_scout_rows
+            problem["max_group_keys"] = max_group_keys
+        n_keys = groups["n_par"].astype(np.int64) * groups["n_ao"] * groups["n_pair"]
         # Batches of consecutive groups under the workspace bound: each holds its own copy of the
         # descriptors with row offsets that start at 0 and its own workgroup prefixes.
         batches = []
-        for first, last in self._batch_bounds(groups["n_rows"]) if len(pending) else []:
+        for first, last in bounds:
             rows = int(groups["n_rows"][first:last].sum())
-            sub = groups[first:last].copy()
-            sub["row_offset"] -= groups["row_offset"][first]
-            sub["key_offset"] -= groups["key_offset"][first]
+            if first == 0:
+                sub = groups[:last]  # offsets start at 0 already
+            else:
+                sub = groups[first:last].copy()
+                sub["row_offset"] -= groups["row_offset"][first]
+                sub["key_offset"] -= groups["key_offset"][first]
             rebase = lambda prefix: (prefix[first:last + 1] - prefix[first]).astype(np.int32)
             batches.append(dict(
                 first=first, last=last, groups=sub, total_rows=rows,
@@ -377,7 +557,7 @@ class IntraStageTuner:
             problem=problem, groups=groups, spaces=spaces, batches=batches,
             terms_prefix=terms_prefix.astype(np.int32), reduce_prefix=reduce_prefix.astype(np.int32),
             scout_prefix=scout_prefix.astype(np.int32),
-            total_rows=int(groups["n_rows"].sum()) if len(pending) else 0,
+            total_rows=int(groups["n_rows"].sum()) if len(groups) else 0,
         )
 
     @staticmethod
@@ -568,7 +748,7 @@ class IntraStageTuner:
                 delta=[x[t * Gn:(t + 1) * Gn] for x in tables.delta],
                 index=[x[t * Gn:(t + 1) * Gn] for x in tables.index],
             )
-            spaces = {(g, q): sp for (tt, g, q), sp in plan["spaces"].items() if tt == t}
+            spaces = _SpacesOfEntry(plan["spaces"], t)
             outs.append(IntraStageTunerOutput(
                 self.gradient_accumulation_steps_candidates, self.device_mesh_candidates, view,
                 spaces, self.sample_slots, batch=tables, batch_index=t,

@@ -68,14 +68,22 @@ def test_interference_table_and_ratios_match_oracle():
     (dict(hardware__num_nodes=2, hardware__num_gpus_per_node=4, training__global_batch_size=64,
           tuning__pre_post_strategy="intra-node-tp-without-ore"), 4),
 ])
-def test_group_descriptors_bit_exact_against_oracle(overrides, tp):
+@pytest.mark.parametrize("builder", ["library", "python"])
+def test_group_descriptors_bit_exact_against_oracle(monkeypatch, overrides, tp, builder):
     """Every per-group scalar and per-(b, tp) table value that is handed to the kernels equals
-    what the oracle derives for the same group, bit for bit."""
+    what the oracle derives for the same group, bit for bit: from the plan builder in the
+    library (``mist_plan_groups``, the default) and from the python builder."""
+    if builder == "python":
+        monkeypatch.setenv("MIST_PYTHON_PLAN_BUILDER", "1")
+    else:
+        monkeypatch.delenv("MIST_PYTHON_PLAN_BUILDER", raising=False)
     cfg, tables = tiny_plan(1, layers=4, **overrides)
     hw = cfg.hardware
     meshes = _get_device_mesh_candidates(hw.num_nodes, hw.num_gpus_per_node, False)
     Gs = _get_grad_accumu_steps_candidates(cfg.training.global_batch_size)
     tuner = IntraStageTuner(tables, 4, meshes, Gs, tp, cfg, sample_size=1, device="cpu")
+    if builder == "library":
+        assert tuner._build_groups_native() is not None, "the library's builder declined the plan"
     plan = tuner.prepare()
     assert len(plan["groups"]) > 0
     P = _lib.PAR
@@ -113,6 +121,155 @@ def test_group_descriptors_bit_exact_against_oracle(overrides, tp):
     prob = plan["problem"][0]
     assert prob["mem_cap_mb"] == cfg.hardware.memory_capacity * (1 << 30) / (1 << 20)
     assert prob["num_layers"] == 4 and prob["sample_size"] == 1
+
+
+def _same_plans(a, b):
+    """Two ``IntraStageTuner.prepare()`` results hold the same bytes (padding aside)."""
+    def same_records(x, y):
+        assert x.dtype == y.dtype and x.shape == y.shape
+        for name in x.dtype.names:
+            assert np.ascontiguousarray(x[name]).tobytes() == np.ascontiguousarray(y[name]).tobytes(), name
+
+    same_records(a["groups"], b["groups"])
+    same_records(a["problem"], b["problem"])
+    for key in ("terms_prefix", "reduce_prefix", "scout_prefix"):
+        assert a[key].dtype == b[key].dtype and np.array_equal(a[key], b[key]), key
+    assert a["total_rows"] == b["total_rows"] and len(a["batches"]) == len(b["batches"])
+    for x, y in zip(a["batches"], b["batches"]):
+        assert x.keys() == y.keys()
+        for key in x:
+            if key == "groups":
+                same_records(x[key], y[key])
+            elif isinstance(x[key], np.ndarray):
+                assert x[key].dtype == y[key].dtype and np.array_equal(x[key], y[key]), key
+            else:
+                assert x[key] == y[key], key
+    assert list(a["spaces"]) == list(b["spaces"])
+    for key in a["spaces"]:
+        sa, sb = a["spaces"][key], b["spaces"][key]
+        assert sa.par.shape == sb.par.shape and np.array_equal(sa.par, sb.par), key
+        assert (sa.wo, sa.go, sa.oo, sa.ao) == (sb.wo, sb.go, sb.oo, sb.ao)
+        assert np.array_equal(sa.pair_wo, sb.pair_wo) and np.array_equal(sa.pair_go, sb.pair_go)
+        assert sa.n_rows == sb.n_rows
+
+
+def _both_builders(cfg, tables, tp="all", **kw):
+    hw, L = cfg.hardware, cfg.model.num_hidden_layers
+    meshes = _get_device_mesh_candidates(hw.num_nodes, hw.num_gpus_per_node, False)
+    Gs = _get_grad_accumu_steps_candidates(cfg.training.global_batch_size)
+    cells_wanted = kw.pop("cells_wanted", None)
+    evaluate_all_p = kw.pop("evaluate_all_p", False)
+    tuner = IntraStageTuner(tables, L, meshes, Gs, tp_candidates(cfg) if tp == "all" else tp, cfg,
+                            sample_size=kw.pop("sample_size", 1), device="cpu", **kw)
+    tuner.cells_wanted, tuner.evaluate_all_p = cells_wanted, evaluate_all_p
+    native = tuner._build_groups_native()
+    assert native is not None, "the library's builder declined the plan"
+    return tuner._finish_plan(*native), tuner._finish_plan(*tuner._build_groups_python())
+
+
+@pytest.mark.parametrize("plan", [1, 2, 3, 4, 5])
+@pytest.mark.parametrize("kw", [dict(), dict(exhaustive=True), dict(tp=None), dict(tp=2),
+                                dict(evaluate_all_p=True, sample_size=30)],
+                         ids=["all tp", "exhaustive", "tp latched", "tp 2", "every p"])
+def test_plan_builder_of_the_library_equals_the_python_builder(plan, kw):
+    """``mist_plan_groups`` against the python host side it replaces on the five benchmark plans
+    (GPT with absolute positions and plain MLP, LLaMA with gated MLP, RMSNorm and grouped kv
+    heads; 1 to 10 batches of groups): every field of every group descriptor, the problem
+    record, the workgroup prefixes, the batches and every search space, byte for byte."""
+    cfg, tables = load_plan(plan)
+    got, want = _both_builders(cfg, tables, **dict(kw))
+    assert len(got["groups"]) > 0
+    _same_plans(got, want)
+
+
+@pytest.mark.parametrize("overrides", [
+    dict(model__use_flash_attn=False),
+    dict(model__use_flash_attn=False, model__mlp_type="gated_mlp", model__normalization="rmsnorm",
+         model__position_embedding_type="rotary", model__tie_word_embeddings=True),
+    dict(tuning__pre_post_strategy="intra-node-tp-with-ore"),
+    dict(tuning__pre_post_strategy="intra-node-tp-without-ore", hardware__num_nodes=2,
+         hardware__num_gpus_per_node=4, training__global_batch_size=64),
+    dict(hardware__num_nodes=4, hardware__num_gpus_per_node=8, training__global_batch_size=96),
+    dict(tuning__zero_2_and_3_enabled=False, hardware__num_gpus_per_node=8, training__global_batch_size=48),
+    dict(tuning__state_offloading_enabled=False),
+    dict(tuning__activation_offloading_enabled=False, disable_wo_tuning=True, fixed_oo_ratio=0.5),
+    dict(disable_tp_tuning=True, hardware__num_gpus_per_node=4),
+    dict(hardware__memory_capacity=0.5),
+    dict(training__params_dtype="float32"),
+    dict(training__optimizer_name="sgd", hardware__num_gpus_per_node=8),
+    dict(model__num_attention_heads=12, model__hidden_size=1536, hardware__num_gpus_per_node=8,
+         training__global_batch_size=32),   # heads do not split over tp 8
+], ids=lambda o: ",".join(f"{k.split('__')[-1]}={v}" for k, v in o.items())[:60])
+def test_plan_builder_of_the_library_on_plan_variants(overrides):
+    cfg, tables = tiny_plan(1, layers=10, **overrides)
+    _same_plans(*_both_builders(cfg, tables))
+    _same_plans(*_both_builders(cfg, tables, tp=None))
+
+
+def test_plan_builder_of_the_library_with_cell_windows():
+    """Callers that read a range of layer counts only (``cells_wanted``): same groups left out,
+    same tile windows and pre-saved micro-batch counts."""
+    from mist_amd.inter_tuning_mip import cells_wanted
+
+    for plan in (2, 3):
+        cfg, tables = load_plan(plan)
+        hw = cfg.hardware
+        wanted = cells_wanted(cfg.model.num_hidden_layers, hw.num_nodes, hw.num_gpus_per_node)
+        got, want = _both_builders(cfg, tables, cells_wanted=wanted, sample_size=30)
+        assert 0 < len(got["groups"])
+        assert got["groups"]["lc_tile_begin"].max() > 0
+        _same_plans(got, want)
+    _same_plans(*_both_builders(cfg, tables, cells_wanted=lambda G, mesh: None))
+    _same_plans(*_both_builders(cfg, tables, cells_wanted=lambda G, mesh: (3, 2, 1) if G > 4 else (0, 99, 2)))
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_plan_builder_of_the_library_on_random_configurations(seed):
+    """Seeded random model shapes, cluster shapes, batch sizes, efficiencies and communication
+    parameters: the builder in the library and the python builder write the same plan."""
+    rng = np.random.default_rng(7700 + seed)
+    heads = int(rng.choice([8, 16, 32, 40, 64]))
+    gg = []
+    for _ in range(16):
+        gg += [float(rng.uniform(8, 500)), float(rng.uniform(2e-6, 8e-5))]
+    nodes, gpus_per_node = int(rng.choice([1, 2, 4, 16])), int(rng.choice([1, 2, 4, 8]))
+    overrides = dict(
+        model__num_attention_heads=heads, model__hidden_size=heads * int(rng.choice([64, 96, 128])),
+        model__num_heads_kv=int(rng.choice([heads, max(heads // 4, 1), 8])) if seed % 2 else None,
+        model__mlp_type=str(rng.choice(["mlp", "gated_mlp"])),
+        model__normalization=str(rng.choice(["layernorm", "rmsnorm"])),
+        model__position_embedding_type=str(rng.choice(["absolute", "rotary"])),
+        model__tie_word_embeddings=bool(rng.integers(0, 2)),
+        model__use_flash_attn=bool(rng.integers(0, 2)),
+        training__max_sequence_length=int(rng.choice([512, 2048, 4096, 3000])),
+        training__global_batch_size=nodes * gpus_per_node * int(rng.choice([1, 2, 4, 16])) * int(rng.choice([1, 1, 1, 3])),
+        hardware__num_nodes=nodes, hardware__num_gpus_per_node=gpus_per_node,
+        hardware__memory_capacity=float(rng.uniform(2.0, 90.0)),
+        hardware__gpu_gpu_comm_params=gg,
+        tuning__pre_post_strategy=str(rng.choice(["dp", "intra-node-tp-with-ore", "intra-node-tp-without-ore"])),
+        synthetic=dict(seed=int(rng.integers(0, 1000)), peak_tflops=float(rng.uniform(100, 2500)),
+                       hbm_gbps=float(rng.uniform(900, 8000))),
+    )
+    cfg, tables = tiny_plan(1, layers=int(rng.integers(2, 40)), **overrides)
+    got, want = _both_builders(cfg, tables)
+    # (a factor of three in the batch size leaves no data-parallel size that divides the devices)
+    assert len(got["groups"]) > 0 or cfg.training.global_batch_size % 3 == 0
+    _same_plans(got, want)
+    _same_plans(*_both_builders(cfg, tables, tp=None, exhaustive=True))
+
+
+def test_plans_outside_the_library_builder_go_through_the_python_builder():
+    """What ``mist_plan_groups`` declines (here: a collective over three devices, which the
+    alpha-beta tables do not hold) is built, and its error worded, by the python host side."""
+    cfg, tables = tiny_plan(1, layers=4, hardware__num_gpus_per_node=6, training__global_batch_size=24,
+                            tuning__pre_post_strategy="dp")
+    meshes = [(1, 1), (1, 2), (1, 6)]
+    Gs = _get_grad_accumu_steps_candidates(cfg.training.global_batch_size)
+    tuner = IntraStageTuner(tables, 4, meshes, Gs, [1], cfg, sample_size=1, device="cpu")
+    assert tuner._build_groups_native() is None
+    assert b"communication group size" in _lib.load().mist_last_error()
+    with pytest.raises(ValueError, match="communication group size"):
+        tuner.prepare()
 
 
 @pytest.mark.parametrize("plan", [2, 5])
@@ -318,7 +475,7 @@ def test_mip_layer_candidates_match_oracle():
 
 def _declared_functions():
     names = []
-    for header in ("mist_search.h", "mist_dp.h", "mist_mip.h", "mist_inter.h"):
+    for header in ("mist_search.h", "mist_dp.h", "mist_mip.h", "mist_inter.h", "mist_plan.h"):
         text = open(os.path.join(REPO, "include", header)).read()
         text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
         names += re.findall(r"\b(mist_[a-z0-9_]+)\s*\(", text)

@@ -223,7 +223,17 @@ struct Search {
   int64_t launches = 0, fetches = 0, selected = 0, thresholds_run = 0, round_trips = 0,
           left_to_host = 0;
 
-  size_t path_ints(int f) const { return (size_t)shapes[f].max_stages * 4; }
+  // Stage counts the next run of a single family goes up to (0 = all of the shape's).  The
+  // back-pointer run of a winner whose scan result has s stages stops there: the recurrence of
+  // the stage counts 1..s is the same, no smaller count reaches its sum (the first count wins
+  // ties), so the result and the back-pointers on its path are those of the full run.
+  int stage_limit = 0;
+  MistDpShape shape_of(int f) const {
+    MistDpShape shape = shapes[f];
+    if (n_families == 1 && stage_limit > 0) shape.max_stages = std::min(shape.max_stages, stage_limit);
+    return shape;
+  }
+  size_t path_ints(int f) const { return (size_t)shape_of(f).max_stages * 4; }
   // ints in front of family f's partitions in the path buffers of a batch of n instances
   size_t path_offset(int f, int n) const {
     size_t at = 0;
@@ -276,20 +286,21 @@ struct Search {
       float *d_out = ws->d_out.as<float>() + (size_t)f * 3 * n;
       int32_t *d_argmin = want_path ? ws->d_argmin.as<int32_t>() : nullptr;  // no fill: the
                                                      // walk reads what the DP wrote
-      if (int rc = mist_dp_run(&shapes[f], &costs[f], d_in, d_g, n, mode,
+      const MistDpShape shape = shape_of(f);
+      if (int rc = mist_dp_run(&shape, &costs[f], d_in, d_g, n, mode,
                                reinterpret_cast<int32_t *>(d_out), d_out + n, d_out + 2 * n,
                                d_argmin, ws->d_scratch.as<float>(), stream))
         return rc;
       if (want_path) {
         int32_t *d_path = ws->d_path.as<int32_t>() + path_offset(f, n);
-        if (int rc = mist_dp_backtrack(&shapes[f], d_argmin, reinterpret_cast<int32_t *>(d_out), n,
+        if (int rc = mist_dp_backtrack(&shape, d_argmin, reinterpret_cast<int32_t *>(d_out), n,
                                        d_path, stream))
           return rc;
         if (strategy) {
-          const int cells = n * shapes[f].max_stages;
+          const int cells = n * shape.max_stages;
           hipLaunchKernelGGL(strategy_rows_kernel, dim3((cells + 63) / 64), dim3(64), 0, stream,
                              *strategy, d_path, reinterpret_cast<int32_t *>(d_out), d_g, n,
-                             shapes[f].max_stages, ws->d_rows.as<int32_t>() + path_offset(f, n) / 4);
+                             shape.max_stages, ws->d_rows.as<int32_t>() + path_offset(f, n) / 4);
           MIST_HIP_CHECK(hipGetLastError());
         }
       }
@@ -321,13 +332,16 @@ struct Search {
     return (double)h[n + i] + ((double)G - 1.0) * (double)h[2 * n + i];
   }
   // smallest family total (the first family wins ties); *family = the one that attains it
-  double total(int i, int n, int G, int *family = nullptr, const float *out = nullptr) const {
+  double total(int i, int n, int G, int *family = nullptr, const float *out = nullptr,
+               int *stages = nullptr) const {
     double best = kInf;
     for (int f = 0; f < n_families; ++f) {
       const double c = total_of(f, i, n, G, out);
       if (c < best) {
         best = c;
         if (family) *family = f;
+        if (stages)
+          std::memcpy(stages, (out ? out : ws->h_out.as<float>()) + (size_t)f * 3 * n + i, sizeof(int));
       }
     }
     return best;
@@ -582,6 +596,7 @@ struct Scan {
   Window *w = nullptr;
   size_t pos = 0, have_lo = 0;
   std::vector<double> cost;  // DP outcome per computed threshold, inf = infeasible
+  std::vector<int> stages;   // ... and the stage count of its partition
   int limit = kFirstChunk;
   size_t n_kept() const { return w ? w->kept.size() : 0; }
 };
@@ -810,7 +825,7 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
     std::vector<Scan> scans;
     size_t current = 0;
     double best_cost = kInf;
-    int best_g = -1;
+    int best_g = -1, best_stages = 0;
     float best_t = 0.0f;
   };
   std::vector<Chain> chains(n_instances);
@@ -830,9 +845,12 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
       // G grows as after any request
       const int idx = t * n_grad_accum + i, n_first = first_batch[idx];
       const int at = on_device ? S.ws->h_meta.as<int32_t>()[8 * idx + 7] : 0;
-      for (int k = 0; k < n_first; ++k)
+      for (int k = 0; k < n_first; ++k) {
+        int stages = 0;
         sc.cost.push_back(S.total(at + k, n_flat * kFirstChunk, sc.G, nullptr,
-                                  S.ws->h_out_first.as<float>()));
+                                  S.ws->h_out_first.as<float>(), &stages));
+        sc.stages.push_back(stages);
+      }
       if (n_first > 0) sc.limit = std::min(kMaxChunk, sc.limit * 4);
     }
   }
@@ -849,7 +867,8 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
     return pos < sc.n_kept();
   };
   // advances the sequential scan as far as the computed results allow; true = this G is done
-  auto replay = [&](Scan &sc, double &best_cost, bool &improved, float &best_t) -> bool {
+  auto replay = [&](Scan &sc, double &best_cost, bool &improved, float &best_t,
+                    int &best_stages) -> bool {
     for (;;) {
       if (!reach(sc, sc.pos, best_cost)) return true;
       if (sc.w->scaled[sc.pos] >= best_cost) return true;  // inter_tuning.py:196-197
@@ -858,6 +877,7 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
       if (c < best_cost) {
         best_cost = c;
         best_t = sc.w->kept[sc.pos];
+        best_stages = sc.stages[sc.pos - sc.have_lo];
         improved = true;
       }
       ++sc.pos;
@@ -890,11 +910,13 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
         Scan &sc = ch.scans[ch.current];
         bool improved = false;
         float best_t = ch.best_t;
-        const bool finished = replay(sc, ch.best_cost, improved, best_t);
+        int best_stages = ch.best_stages;
+        const bool finished = replay(sc, ch.best_cost, improved, best_t, best_stages);
         if (rc_inner) return rc_inner;
         if (improved) {
           ch.best_g = (int)ch.current;
           ch.best_t = best_t;
+          ch.best_stages = best_stages;
         }
         if (!finished) break;
         ++ch.current;
@@ -934,7 +956,11 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
     int off = 0;
     for (const Span &sp : spans) {
       Scan &sc = chains[sp.t].scans[sp.i];
-      for (int k = 0; k < sp.n; ++k) sc.cost.push_back(S.total(off + k, n, req_G[off + k]));
+      for (int k = 0; k < sp.n; ++k) {
+        int stages = 0;
+        sc.cost.push_back(S.total(off + k, n, req_G[off + k], nullptr, nullptr, &stages));
+        sc.stages.push_back(stages);
+      }
       off += sp.n;
     }
   }
@@ -962,10 +988,13 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
   if (!winners.empty()) {
     std::vector<int32_t> g;
     std::vector<float> tm;
+    int most_stages = 0;
     for (int t : winners) {
       g.push_back(rows[t * n_grad_accum + chains[t].best_g]);
       tm.push_back(chains[t].best_t);
+      most_stages = std::max(most_stages, chains[t].best_stages);
     }
+    S.stage_limit = most_stages;  // no winner has more stages than this
     if (int rc = S.run(g, tm, MIST_DP_THRESHOLD, true)) return rc;
     const int n = (int)winners.size();
     for (int k = 0; k < n; ++k) {

@@ -93,6 +93,21 @@ int mist_mip_solve(const MistMipShape *shape, int grad_accum, double best_cost,
                    const float *t_stable, const float *t_delta, const uint8_t *keep,
                    double *out_cost, int32_t *out_layers, int32_t *out_slot);
 
+/* mist_mip_solve over the problems of whole searches (inter_stage_tune, inter_tuning_mip.py:
+ * 131-214: for every G, for every stage count, one assignment bounded by the best cost so far,
+ * which starts at MIST_MIP_MAX_VALUE; a strictly smaller cost replaces it).  `n_chains`
+ * searches (one per tensor-parallel candidate) of `items_per_chain` problems each, chain c's
+ * problems at items[c * items_per_chain ...] in the reference's order; problem i of every chain
+ * runs with grad_accum[i]; each problem's samples lie at its out_offset in the three HOST
+ * arrays (the layout mist_mip_stage_samples_batch writes).  Chains are solved on a thread each.
+ * Per chain: out_cost (MIST_MIP_MAX_VALUE when no problem has an assignment below it), out_item
+ * (index of the winning problem inside the chain, -1 = none), out_layers / out_slot
+ * [chain][num_layers], the winner's first num_stages entries. */
+int mist_mip_solve_chains(const MistMipBatchItem *items, const int32_t *grad_accum,
+                          int items_per_chain, int n_chains, const float *t_stable,
+                          const float *t_delta, const uint8_t *keep, double *out_cost,
+                          int32_t *out_item, int32_t *out_layers, int32_t *out_slot);
+
 #ifdef __cplusplus
 }
 #endif

@@ -283,6 +283,19 @@ class MipBatchItem(ctypes.Structure):
                 ("first_block", ctypes.c_int32), ("reserved", ctypes.c_int32)]
 
 
+# MistMipBatchItem as a numpy record: a search fills the items of all its problems column-wise
+MIP_ITEM_DTYPE = np.dtype(
+    [
+        ("num_layers", "<i4"), ("p_dim", "<i4"), ("sample_size", "<i4"), ("num_stages", "<i4"),
+        ("layers_min", "<i4"), ("layers_max", "<i4"), ("ckpt_mode", "<i4"), ("fixed_ckpt", "<i4"),
+        ("stable", "<u8", (4,)), ("delta", "<u8", (4,)),
+        ("out_offset", "<i8"), ("first_block", "<i4"), ("reserved", "<i4"),
+    ],
+    align=True,
+)
+assert MIP_ITEM_DTYPE.itemsize == ctypes.sizeof(MipBatchItem)
+
+
 class StrategyIndex(ctypes.Structure):
     """``MistStrategyIndex`` of include/mist_inter.h."""
 
@@ -395,6 +408,8 @@ _MIP_SIGNATURES = {
     "mist_sizeof_mip_batch_item": (ctypes.c_int, []),
     "mist_mip_stage_samples_batch": (
         ctypes.c_int, [_VP, _VP, ctypes.c_int, _VP, _VP, _VP, _VP, _VP, _VP]),
+    "mist_mip_solve_chains": (
+        ctypes.c_int, [_VP, _VP, ctypes.c_int, ctypes.c_int, _VP, _VP, _VP, _VP, _VP, _VP, _VP]),
     "mist_mip_solve": (
         ctypes.c_int,
         [ctypes.POINTER(MipShape), ctypes.c_int, ctypes.c_double, _VP, _VP, _VP,

@@ -16,6 +16,7 @@
 #include <cmath>
 #include <cstdint>
 #include <limits>
+#include <thread>
 #include <vector>
 
 #include "mist_common.h"
@@ -310,6 +311,66 @@ int mist_mip_solve(const MistMipShape *shape, int grad_accum, double best_cost,
     }
   }
   return best < inf ? 1 : 0;
+}
+
+int mist_mip_solve_chains(const MistMipBatchItem *items, const int32_t *grad_accum,
+                          int items_per_chain, int n_chains, const float *t_stable,
+                          const float *t_delta, const uint8_t *keep, double *out_cost,
+                          int32_t *out_item, int32_t *out_layers, int32_t *out_slot) {
+  if (!items || !grad_accum || !t_stable || !t_delta || !keep || !out_cost || !out_item || !out_layers ||
+      !out_slot)
+    return fail(MIST_E_INVALID, "null pointer");
+  if (items_per_chain < 1 || n_chains < 1)
+    return fail(MIST_E_INVALID, "%d chains of %d problems", n_chains, items_per_chain);
+  int L = 0;
+  for (int64_t i = 0; i < (int64_t)items_per_chain * n_chains; ++i) {
+    if (int rc = check_mip_shape(&items[i].shape)) return rc;
+    if (grad_accum[i % items_per_chain] < 1)
+      return fail(MIST_E_INVALID, "grad_accum %d < 1", grad_accum[i % items_per_chain]);
+    if (i > 0 && items[i].shape.num_layers != L)
+      return fail(MIST_E_INVALID, "problem %lld has %d layers, problem 0 has %d", (long long)i,
+                  items[i].shape.num_layers, L);
+    L = items[i].shape.num_layers;
+  }
+  // One chain = the problems of one search in the reference's order: the bound of a problem is
+  // the best cost of those before it (inter_tuning_mip.py:131-214).  Chains do not depend on
+  // each other: a thread each.
+  std::vector<int> status((size_t)n_chains, 0);
+  auto run_chain = [&](int c) {
+    double best_cost = (double)MIST_MIP_MAX_VALUE;
+    int best_item = -1;
+    std::vector<int32_t> layers((size_t)L), slots((size_t)L);
+    for (int i = 0; i < items_per_chain; ++i) {
+      const MistMipBatchItem &item = items[(int64_t)c * items_per_chain + i];
+      double cost = 0.0;
+      const int rc = mist_mip_solve(&item.shape, grad_accum[i], best_cost, t_stable + item.out_offset,
+                                    t_delta + item.out_offset, keep + item.out_offset, &cost,
+                                    layers.data(), slots.data());
+      if (rc < 0) {
+        status[c] = rc;
+        return;
+      }
+      if (rc == 1 && cost < best_cost) {
+        best_cost = cost;
+        best_item = i;
+        std::copy(layers.begin(), layers.begin() + item.shape.num_stages, out_layers + (int64_t)c * L);
+        std::copy(slots.begin(), slots.begin() + item.shape.num_stages, out_slot + (int64_t)c * L);
+      }
+    }
+    out_cost[c] = best_cost;
+    out_item[c] = best_item;
+  };
+  if (n_chains == 1) {
+    run_chain(0);
+  } else {
+    std::vector<std::thread> workers;
+    for (int c = 0; c < n_chains; ++c) workers.emplace_back(run_chain, c);
+    for (std::thread &w : workers) w.join();
+  }
+  for (int c = 0; c < n_chains; ++c)
+    if (status[c] < 0)  // (every argument the solver checks was checked above)
+      return fail(status[c], "the solver of chain %d rejected its arguments", c);
+  return 0;
 }
 
 }  // extern "C"

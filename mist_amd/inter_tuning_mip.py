@@ -69,16 +69,6 @@ def cells_wanted(num_layers: int, num_nodes: int, num_gpus_per_node: int, layers
     return wanted
 
 
-class _Problem:
-    """One (G, S) assignment problem: its shape and where its samples lie in the batch buffers."""
-
-    __slots__ = ("G", "g", "S", "mesh", "q", "shape", "offset", "count")
-
-    def __init__(self, G, g, S, mesh, q, shape, offset, count):
-        self.G, self.g, self.S, self.mesh, self.q = G, g, S, mesh, q
-        self.shape, self.offset, self.count = shape, offset, count
-
-
 def _ckpt_mode(config) -> Tuple[int, int]:
     """inter_tuning_mip.py:471-489."""
     if config.tuning.activation_checkpointing_tuning_enabled:
@@ -87,65 +77,6 @@ def _ckpt_mode(config) -> Tuple[int, int]:
     if fixed is not None:
         return _lib.MIP_CKPT_FIXED, int(fixed)
     return _lib.MIP_CKPT_FULL, 0
-
-
-def stage_samples(results: IntraStageTunerOutput, problems: List[_Problem]):
-    """Launches ``mist_mip_stage_samples`` for every problem and returns the host copies
-    ``(t_stable, t_delta, index, keep)`` of the concatenated outputs."""
-    lib = _lib.load()
-    tables = results.device
-    dev = tables.stable[0].device
-    total = sum(p.count for p in problems)
-    P = tables.stable[0].shape[-1]
-    with torch.cuda.device(dev):
-        ratios = torch.from_numpy(alpha_ratios(P)).to(dev)
-        t_stable = torch.empty(max(total, 1), dtype=torch.float32, device=dev)
-        t_delta = torch.empty(max(total, 1), dtype=torch.float32, device=dev)
-        index = torch.empty(max(total, 1), dtype=torch.int32, device=dev)
-        keep = torch.empty(max(total, 1), dtype=torch.uint8, device=dev)
-        stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
-        live = [p for p in problems if p.count > 0]
-        if live:
-            # every problem in one launch: the rows are a few hundred candidates each, and one
-            # launch per problem (~220 for a 32-layer plan) left the GPU to one wavefront per row
-            items = (_lib.MipBatchItem * len(live))()
-            first_block = 0
-            for item, p in zip(items, live):
-                item.shape = p.shape
-                for v in range(4):
-                    item.tables.stable[v] = tables.stable[v][p.g, p.q].data_ptr()
-                    item.tables.delta[v] = tables.delta[v][p.g, p.q].data_ptr()
-                item.out_offset, item.first_block = p.offset, first_block
-                first_block += p.count // P
-            d_items = torch.frombuffer(bytearray(bytes(items)), dtype=torch.uint8).to(dev)
-            rc = lib.mist_mip_stage_samples_batch(
-                ctypes.byref(items), d_items.data_ptr(), len(live), ratios.data_ptr(),
-                t_stable.data_ptr(), t_delta.data_ptr(), index.data_ptr(), keep.data_ptr(), stream)
-            _lib.check(rc, "mist_mip_stage_samples_batch")
-        return (t_stable.cpu().numpy(), t_delta.cpu().numpy(), index.cpu().numpy(),
-                keep.cpu().numpy())
-
-
-def solve(problem: _Problem, best_cost: float, t_stable, t_delta, keep):
-    """``mist_mip_solve`` on one problem's slice of the host arrays.  Returns ``(cost, layers,
-    slots)`` or ``(inf, None, None)``."""
-    lib = _lib.load()
-    S = problem.S
-    lo, hi = problem.offset, problem.offset + problem.count
-    ts = np.ascontiguousarray(t_stable[lo:hi])
-    td = np.ascontiguousarray(t_delta[lo:hi])
-    kp = np.ascontiguousarray(keep[lo:hi])
-    cost = ctypes.c_double()
-    layers = np.zeros(S, dtype=np.int32)
-    slots = np.zeros(S, dtype=np.int32)
-    rc = lib.mist_mip_solve(
-        ctypes.byref(problem.shape), int(problem.G), float(best_cost), ts.ctypes.data,
-        td.ctypes.data, kp.ctypes.data, ctypes.byref(cost), layers.ctypes.data, slots.ctypes.data)
-    if rc < 0:
-        _lib.check(rc, "mist_mip_solve")
-    if rc == 0:
-        return float("inf"), None, None
-    return cost.value, layers, slots
 
 
 def _variant_cell(num_layers, g, q, p, l0, l1, ckpt, slot):
@@ -160,6 +91,169 @@ def _variant_cell(num_layers, g, q, p, l0, l1, ckpt, slot):
     return 0, (g, q, p, l - 1, ckpt, slot)
 
 
+def _problems(num_layers, num_nodes, num_gpus_per_node, grad_accum_candidates, g_index, q_index,
+              P1, P, mode, fixed, offset_layers):
+    """The (G, S) assignment problems of one search in the reference's order
+    (inter_tuning_mip.py:131-214) that have a layer count to sample, as ``MIP_ITEM_DTYPE``
+    records without table pointers and offsets, with ``G``, table row ``g``, mesh index ``q``
+    and mesh of each."""
+    rows = []
+    for G in grad_accum_candidates:
+        for S in range(1, num_layers + 1):
+            if num_nodes * num_gpus_per_node % S != 0:
+                continue
+            mesh = _uniform_device_mesh_partition(S, num_nodes, num_gpus_per_node)
+            if mesh is None or mesh not in q_index:
+                continue
+            lo, hi = layer_candidates(num_layers, S, G, offset_layers)
+            if hi >= lo:
+                rows.append((G, g_index[G], S, mesh, q_index[mesh], lo, hi))
+    items = np.zeros(len(rows), dtype=_lib.MIP_ITEM_DTYPE)
+    items["num_layers"], items["p_dim"], items["sample_size"] = num_layers, P1, P
+    items["ckpt_mode"], items["fixed_ckpt"] = mode, fixed
+    if rows:
+        items["num_stages"] = [r[2] for r in rows]
+        items["layers_min"] = [r[5] for r in rows]
+        items["layers_max"] = [r[6] for r in rows]
+    return items, rows
+
+
+def inter_stage_tune_batch(
+    num_layers: int,
+    num_nodes: int,
+    num_gpus_per_node: int,
+    device_mesh_candidates: List[Tuple[int, int]],
+    gradient_accumulation_steps_candidates: List[int],
+    results_list: List[IntraStageTunerOutput],
+    config,
+    stats: Optional[dict] = None,
+    only_best_solution: bool = False,
+) -> List[Tuple[float, Optional[List[Any]]]]:
+    """``inter_stage_tune`` for several intra-stage results at once (the tensor-parallel
+    candidates of one ``tune`` call, tables on one device): each is searched as if it were alone
+    (its own bound, from ``MAX_VALUE`` down); the policy samples of all their problems come from
+    one launch and one copy, the assignments are solved by one library call (a thread per
+    search).  ``only_best_solution``: the strategy rows are read back for the first entry with
+    the smallest cost only, the others come back as ``(cost, None)``."""
+    lib = _lib.load()
+    first = results_list[0]
+    for res in results_list:
+        if not isinstance(res, IntraStageTunerOutput):
+            raise TypeError(
+                f"intra_stage_results must be an instance of IntraStageTunerOutput, got {type(res)}")
+        _, Q, P1, L, _, P = res.device.stable[0].shape
+        if L != num_layers:
+            raise ValueError(f"tables hold {L} layers, the search asks for {num_layers}")
+        if tuple(res.sample_slots) != tuple(range(P)):
+            raise ValueError(
+                f"the assignment needs every sample of the intra-stage tables; computed slots: "
+                f"{tuple(res.sample_slots)} of {P}")
+        if P > _lib.MIP_MAX_SAMPLES:
+            raise ValueError(f"sample_size {P} exceeds {_lib.MIP_MAX_SAMPLES}")
+        if (res.device.stable[0].shape != first.device.stable[0].shape
+                or res.gradient_accumulation_steps_candidates != first.gradient_accumulation_steps_candidates
+                or res.device_mesh_candidates != first.device_mesh_candidates
+                or res.device.stable[0].device != first.device.stable[0].device):
+            raise ValueError("the results of one batch must share table shape, candidates and device")
+    _, Q, P1, L, _, P = first.device.stable[0].shape
+    g_index = {g: i for i, g in enumerate(first.gradient_accumulation_steps_candidates)}
+    q_index = {q: i for i, q in enumerate(first.device_mesh_candidates)}
+    mode, fixed = _ckpt_mode(config)
+    offset_layers = int(getattr(config.tuning, "layers_offset", 2))
+    n_res = len(results_list)
+
+    t0 = time.perf_counter()
+    one, rows = _problems(num_layers, num_nodes, num_gpus_per_node, gradient_accumulation_steps_candidates,
+                          g_index, q_index, P1, P, mode, fixed, offset_layers)
+    n_items = len(rows)
+    if n_items == 0:
+        return [(float("inf"), None)] * n_res
+    # every search's problems one after the other: offsets continue through the whole list
+    items = np.tile(one, n_res)
+    blocks = (one["num_stages"] * (one["layers_max"] - one["layers_min"] + 1)).astype(np.int64)
+    blocks = np.tile(blocks, n_res)
+    first_block = np.concatenate(([0], np.cumsum(blocks)[:-1]))
+    items["first_block"], items["out_offset"] = first_block, first_block * P
+    total = int(blocks.sum()) * P
+    cell = np.array([r[1] for r in rows], dtype=np.int64) * Q + np.array([r[4] for r in rows], dtype=np.int64)
+    for t, res in enumerate(results_list):
+        part = items[t * n_items:(t + 1) * n_items]
+        for v in range(4):
+            for name, tabs in (("stable", res.device.stable), ("delta", res.device.delta)):
+                tab = tabs[v]
+                assert tab.is_contiguous() and tab.dtype == torch.float64
+                part[name][:, v] = tab.data_ptr() + cell * (tab.stride(1) * 8)
+    dev = first.device.stable[0].device
+    with torch.cuda.device(dev):
+        ratios = torch.from_numpy(alpha_ratios(P)).to(dev)
+        # t_stable, t_delta (float32), index (int32), keep (uint8) of every problem in one buffer
+        out = torch.empty(13 * total, dtype=torch.uint8, device=dev)
+        d_items = torch.from_numpy(items.view(np.uint8).reshape(-1)).to(dev)
+        rc = lib.mist_mip_stage_samples_batch(
+            ctypes.c_void_p(items.ctypes.data), d_items.data_ptr(), len(items), ratios.data_ptr(),
+            out.data_ptr(), out.data_ptr() + 4 * total, out.data_ptr() + 8 * total,
+            out.data_ptr() + 12 * total, ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream))
+        _lib.check(rc, "mist_mip_stage_samples_batch")
+        host = out.cpu().numpy()
+    t_stable, t_delta = host[:4 * total].view(np.float32), host[4 * total:8 * total].view(np.float32)
+    index, keep = host[8 * total:12 * total].view(np.int32), host[12 * total:]
+    t1 = time.perf_counter()
+
+    G_of = np.array([r[0] for r in rows], dtype=np.int32)
+    cost = np.empty(n_res, dtype=np.float64)
+    winner = np.empty(n_res, dtype=np.int32)
+    layers = np.zeros((n_res, L), dtype=np.int32)
+    slots = np.zeros((n_res, L), dtype=np.int32)
+    ptr = lambda a: ctypes.c_void_p(a.ctypes.data)
+    rc = lib.mist_mip_solve_chains(ptr(items), ptr(G_of), n_items, n_res, ptr(t_stable), ptr(t_delta),
+                                   ptr(keep), ptr(cost), ptr(winner), ptr(layers), ptr(slots))
+    _lib.check(rc, "mist_mip_solve_chains")
+    t2 = time.perf_counter()
+    if stats is not None:
+        stats["mip_problems"] = stats.get("mip_problems", 0) + len(items)
+        stats["mip_samples_s"] = stats.get("mip_samples_s", 0.0) + (t1 - t0)
+        stats["mip_solve_s"] = stats.get("mip_solve_s", 0.0) + (t2 - t1)
+
+    found = [t for t in range(n_res) if winner[t] >= 0]
+    wanted = found
+    if only_best_solution and found:
+        wanted = [min(found, key=lambda t: cost[t])]  # the first of equals (tune_one_case.py:394-398)
+    out_list: List[Tuple[float, Optional[List[Any]]]] = []
+    requests, where = [], []
+    for t, res in enumerate(results_list):
+        if winner[t] < 0:
+            out_list.append((float("inf"), None))
+            continue
+        if t not in wanted:
+            out_list.append((float(cost[t]), None))
+            continue
+        G, g, S, mesh, q, lo, hi = rows[int(winner[t])]
+        item = items[t * n_items + int(winner[t])]
+        nl = hi - lo + 1
+        solution: List[Any] = [G, []]
+        covered = 0
+        for i in range(S):
+            j, a = int(layers[t, i]), int(slots[t, i])
+            n = int(index[int(item["out_offset"]) + (i * nl + (j - lo)) * P + a])
+            if mode == _lib.MIP_CKPT_TUNED:
+                ckpt, policy = n // P, n % P          # inter_tuning_mip.py:507-509
+            else:
+                ckpt, policy = (fixed if mode == _lib.MIP_CKPT_FIXED else j), n
+            l0, l1 = covered, covered + j - 1
+            covered += j
+            variant, cell_at = _variant_cell(num_layers, g, q, S - i - 1, l0, l1, ckpt, policy)
+            requests.append((res, variant, cell_at))
+            where.append((len(out_list), i))
+            solution[1].append(((l0, l1), mesh, ckpt, policy))
+        out_list.append((float(cost[t]), solution))
+    for (at, i), row in zip(where, IntraStageTunerOutput.solutions_at(requests)):  # one read-back
+        row = row.tolist()
+        row[:6] = [int(v) for v in row[:6]]
+        stages = out_list[at][1][1]
+        stages[i] = (stages[i], tuple(row))
+    return out_list
+
+
 def inter_stage_tune(
     num_layers: int,
     num_nodes: int,
@@ -172,78 +266,10 @@ def inter_stage_tune(
 ) -> Tuple[float, Optional[List[Any]]]:
     """Reference signature (inter_tuning_mip.py:87-95).  Returns ``(best_cost, [G, [(((l0, l1),
     (n, m), ckpt, policy), strategy_row), ...per stage]])`` or ``(inf, None)``."""
-    res = intra_stage_results
-    if not isinstance(res, IntraStageTunerOutput):
+    if not isinstance(intra_stage_results, IntraStageTunerOutput):
         raise TypeError(
-            f"intra_stage_results must be an instance of IntraStageTunerOutput, got {type(res)}")
-    tables = res.device
-    _, _, P1, L, _, P = tables.stable[0].shape
-    if L != num_layers:
-        raise ValueError(f"tables hold {L} layers, the search asks for {num_layers}")
-    if tuple(res.sample_slots) != tuple(range(P)):
-        raise ValueError(
-            f"the assignment needs every sample of the intra-stage tables; computed slots: "
-            f"{tuple(res.sample_slots)} of {P}")
-    if P > _lib.MIP_MAX_SAMPLES:
-        raise ValueError(f"sample_size {P} exceeds {_lib.MIP_MAX_SAMPLES}")
-    g_index = {g: i for i, g in enumerate(res.gradient_accumulation_steps_candidates)}
-    q_index = {q: i for i, q in enumerate(res.device_mesh_candidates)}
-    mode, fixed = _ckpt_mode(config)
-    offset_layers = int(getattr(config.tuning, "layers_offset", 2))
-
-    t0 = time.perf_counter()
-    problems: List[_Problem] = []
-    cursor = 0
-    for G in gradient_accumulation_steps_candidates:
-        for S in range(1, num_layers + 1):
-            if num_nodes * num_gpus_per_node % S != 0:
-                continue
-            mesh = _uniform_device_mesh_partition(S, num_nodes, num_gpus_per_node)
-            if mesh is None or mesh not in q_index:
-                continue
-            lo, hi = layer_candidates(num_layers, S, G, offset_layers)
-            shape = _lib.MipShape(num_layers=L, p_dim=P1, sample_size=P, num_stages=S,
-                                  layers_min=lo, layers_max=hi, ckpt_mode=mode, fixed_ckpt=fixed)
-            count = S * max(hi - lo + 1, 0) * P
-            problems.append(_Problem(G, g_index[G], S, mesh, q_index[mesh], shape, cursor, count))
-            cursor += count
-    t_stable, t_delta, index, keep = stage_samples(res, problems)
-    t1 = time.perf_counter()
-
-    best_cost, best = MAX_VALUE, None
-    for prob in problems:  # in the reference's order: best_cost tightens as it goes
-        if prob.count == 0:
-            continue
-        cost, layers, slots = solve(prob, best_cost, t_stable, t_delta, keep)
-        if cost < best_cost:
-            best_cost, best = cost, (prob, layers, slots)
-    t2 = time.perf_counter()
-    if stats is not None:
-        stats["mip_problems"] = stats.get("mip_problems", 0) + len(problems)
-        stats["mip_samples_s"] = stats.get("mip_samples_s", 0.0) + (t1 - t0)
-        stats["mip_solve_s"] = stats.get("mip_solve_s", 0.0) + (t2 - t1)
-    if best is None:
-        return float("inf"), None
-
-    prob, layers, slots = best
-    nl = prob.shape.layers_max - prob.shape.layers_min + 1
-    solution: List[Any] = [prob.G, []]
-    requests = []
-    covered = 0
-    for i in range(prob.S):
-        j, a = int(layers[i]), int(slots[i])
-        n = int(index[prob.offset + (i * nl + (j - prob.shape.layers_min)) * P + a])
-        if mode == _lib.MIP_CKPT_TUNED:
-            ckpt, policy = n // P, n % P          # inter_tuning_mip.py:507-509
-        else:
-            ckpt, policy = (fixed if mode == _lib.MIP_CKPT_FIXED else j), n
-        l0, l1 = covered, covered + j - 1
-        covered += j
-        variant, cell = _variant_cell(num_layers, prob.g, prob.q, prob.S - i - 1, l0, l1, ckpt, policy)
-        requests.append((res, variant, cell))
-        solution[1].append(((l0, l1), prob.mesh, ckpt, policy))
-    for i, row in enumerate(IntraStageTunerOutput.solutions_at(requests)):  # one read-back
-        row = row.tolist()
-        row[:6] = [int(v) for v in row[:6]]
-        solution[1][i] = (solution[1][i], tuple(row))
-    return best_cost, solution
+            f"intra_stage_results must be an instance of IntraStageTunerOutput, got "
+            f"{type(intra_stage_results)}")
+    return inter_stage_tune_batch(
+        num_layers, num_nodes, num_gpus_per_node, device_mesh_candidates,
+        gradient_accumulation_steps_candidates, [intra_stage_results], config, stats)[0]

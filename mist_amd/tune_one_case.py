@@ -36,7 +36,7 @@ from .inter_tuning import inter_stage_tune, inter_stage_tune_batch
 from .inter_tuning_uniform import inter_stage_tune as inter_stage_tune_uniform
 from .inter_tuning_uniform_device import inter_stage_tune_batch_uniform_device
 from .inter_tuning_mip import cells_wanted as mip_cells_wanted
-from .inter_tuning_mip import inter_stage_tune as inter_stage_tune_mip
+from .inter_tuning_mip import inter_stage_tune_batch as inter_stage_tune_batch_mip
 from .intra_tuning import SAMPLE_SIZE, IntraStageTuner, intra_stage_tune
 from .layer_tables import LayerTables
 from .node_database import layer_tables_for
@@ -135,9 +135,10 @@ def _uniform_device_pp_mip(mist_config, device, stats):
         results = tuner.tune_all()
         t1 = time.perf_counter()
         stats["intra_s"] = stats.get("intra_s", 0.0) + (t1 - t0)
-        for r in results:
-            cost, solution = inter_stage_tune_mip(
-                L, hw.num_nodes, hw.num_gpus_per_node, meshes, Gs, r, mist_config, stats=stats)
+        # (the strategy rows are read back for the batch's first best candidate only)
+        for cost, solution in inter_stage_tune_batch_mip(
+                L, hw.num_nodes, hw.num_gpus_per_node, meshes, Gs, results, mist_config, stats=stats,
+                only_best_solution=True):
             if cost < best_cost:
                 best_cost, best_solution = cost, solution
         stats["inter_s"] = stats.get("inter_s", 0.0) + (time.perf_counter() - t1)

@@ -309,3 +309,89 @@ def test_tables_restricted_to_the_cells_the_assignment_reads(monkeypatch, plan, 
         results[all_cells] = tune_one_case.tune(cfg)
     assert results[False] == results[True]
     assert results[False][1] is not None
+
+
+@pytest.mark.parametrize("plan, samples, overrides", [
+    (2, 3, {}),
+    (1, 30, {}),
+    (1, 4, dict(model__num_hidden_layers=9, hardware__num_nodes=2, hardware__num_gpus_per_node=4,
+                training__global_batch_size=32, hardware__memory_capacity=10.0)),
+    (1, 3, dict(model__num_hidden_layers=6, hardware__memory_capacity=0.2)),  # nothing fits
+])
+def test_batched_search_equals_one_search_per_candidate(plan, samples, overrides):
+    """``inter_stage_tune_batch`` (all tensor-parallel candidates of a plan: one sampling launch,
+    one copy, ``mist_mip_solve_chains`` with a thread per candidate) against ``inter_stage_tune``
+    on each candidate alone and against a python loop over ``mist_mip_solve`` with the
+    reference's running bound; with ``only_best_solution`` the strategy of the first best
+    candidate only."""
+    from mist_amd import _lib
+    from mist_amd.config import tp_candidates
+    from mist_amd.inter_tuning_mip import inter_stage_tune, inter_stage_tune_batch
+    from mist_amd.intra_tuning import IntraStageTuner
+    from mist_amd.search_space import _get_device_mesh_candidates, _get_grad_accumu_steps_candidates
+
+    cfg, tables = load_plan(plan, tuning__tuning_granularity="uniform-device-pp-mip",
+                            tuning__sample_size=samples, **overrides)
+    hw, L = cfg.hardware, cfg.model.num_hidden_layers
+    meshes = _get_device_mesh_candidates(hw.num_nodes, hw.num_gpus_per_node, False)
+    Gs = _get_grad_accumu_steps_candidates(cfg.training.global_batch_size)
+    results = IntraStageTuner(tables, L, meshes, Gs, tp_candidates(cfg), cfg, sample_size=samples).tune_all()
+    args = (L, hw.num_nodes, hw.num_gpus_per_node, meshes, Gs)
+    stats = {}
+    together = inter_stage_tune_batch(*args, results, cfg, stats=stats)
+    alone = [inter_stage_tune(*args, r, cfg) for r in results]
+    assert together == alone
+    assert stats["mip_problems"] % len(results) == 0
+    best_only = inter_stage_tune_batch(*args, results, cfg, only_best_solution=True)
+    found = [i for i, (_, sol) in enumerate(alone) if sol is not None]
+    keep = min(found, key=lambda i: alone[i][0]) if found else None
+    assert best_only == [(cost, sol if i == keep else None) for i, (cost, sol) in enumerate(alone)]
+    assert (keep is None) == (overrides.get("hardware__memory_capacity") == 0.2)
+
+    # the chains solver against the single-problem solver driven by the reference's loop
+    rng = np.random.default_rng(5)
+    P, n_chains = samples, 3
+    shapes = [(S, lo, hi) for S, lo, hi in [(1, L, L), (2, max(L // 2 - 2, 1), L // 2 + 2), (3, 1, L - 2),
+                                            (2, 1, L - 1)] if hi >= lo]
+    items = np.zeros(n_chains * len(shapes), dtype=_lib.MIP_ITEM_DTYPE)
+    items["num_layers"], items["p_dim"], items["sample_size"] = L, 4, P
+    cursor = 0
+    for k in range(len(items)):
+        S, lo, hi = shapes[k % len(shapes)]
+        items["num_stages"][k], items["layers_min"][k], items["layers_max"][k] = S, lo, hi
+        items["out_offset"][k] = cursor
+        cursor += S * (hi - lo + 1) * P
+    t_stable = (np.round(rng.uniform(0.1, 2.0, cursor) * 16) / 16).astype(np.float32)  # ties
+    t_delta = (np.round(rng.uniform(0.0, 3.0, cursor) * 8) / 8).astype(np.float32)
+    keep_flags = (rng.random(cursor) < 0.8).astype(np.uint8)
+    G_of = np.array([1, 4, 16, 64][:len(shapes)], dtype=np.int32)
+    lib = _lib.load()
+    ptr = lambda a: ctypes.c_void_p(a.ctypes.data)
+    cost = np.empty(n_chains)
+    winner = np.empty(n_chains, dtype=np.int32)
+    layers = np.zeros((n_chains, L), dtype=np.int32)
+    slots = np.zeros((n_chains, L), dtype=np.int32)
+    _lib.check(lib.mist_mip_solve_chains(ptr(items), ptr(G_of), len(shapes), n_chains, ptr(t_stable),
+                                         ptr(t_delta), ptr(keep_flags), ptr(cost), ptr(winner),
+                                         ptr(layers), ptr(slots)), "mist_mip_solve_chains")
+    for c in range(n_chains):
+        best_cost, best = float(_lib.MIP_MAX_VALUE), None
+        for i in range(len(shapes)):
+            item = items[c * len(shapes) + i]
+            S, at = int(item["num_stages"]), int(item["out_offset"])
+            shape = _lib.MipShape(num_layers=L, p_dim=4, sample_size=P, num_stages=S,
+                                  layers_min=int(item["layers_min"]), layers_max=int(item["layers_max"]))
+            one_cost = ctypes.c_double()
+            one_layers, one_slots = np.zeros(S, dtype=np.int32), np.zeros(S, dtype=np.int32)
+            rc = lib.mist_mip_solve(ctypes.byref(shape), int(G_of[i]), best_cost, ptr(t_stable[at:]),
+                                    ptr(t_delta[at:]), ptr(keep_flags[at:]), ctypes.byref(one_cost),
+                                    ptr(one_layers), ptr(one_slots))
+            assert rc >= 0
+            if rc == 1 and one_cost.value < best_cost:
+                best_cost, best = one_cost.value, (i, one_layers, one_slots)
+        assert cost[c] == best_cost
+        assert winner[c] == (best[0] if best else -1)
+        if best:
+            S = len(best[1])
+            assert np.array_equal(layers[c, :S], best[1]) and np.array_equal(slots[c, :S], best[2])
+    assert (winner >= 0).any()

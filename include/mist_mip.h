@@ -93,6 +93,22 @@ int mist_mip_solve(const MistMipShape *shape, int grad_accum, double best_cost,
                    const float *t_stable, const float *t_delta, const uint8_t *keep,
                    double *out_cost, int32_t *out_layers, int32_t *out_slot);
 
+/* Pre-fill of the intra-stage tables for a caller that reads the cells of the stage assignment
+ * only (the reference allocates whole tables of +inf, mist/analyzer/intra_tuning.py:127-166; an
+ * assignment with 30 samples per cell reads a sixth of them): costs +inf and row indices -1 in
+ * the table rows of n_regions regions, every other cell is left as it is.
+ * regions[n_regions][6] (HOST, and the same array in DEVICE memory as d_regions) =
+ *   (table row g, mesh q, smallest layer count, largest layer count, number of pre-saved
+ *    micro-batch values p = 0.., first workgroup of the region);
+ * a region covers, for its layer counts l, all ckpt counts and samples of variants 0 and 1 at
+ * every p below its count (at most p_dim), of variant 2, and of variant 3 when its largest layer
+ * count is num_layers; region i + 1 starts at the first workgroup of region i plus its rows
+ * (2 * p values * layer counts + layer counts [+ 1]).  Table extents as in MistOutTables:
+ * [num_table_rows][num_mesh][p_dim][L][L+1][sample_size] etc. */
+int mist_mip_prefill_cells(int num_layers, int p_dim, int sample_size, int num_mesh,
+                           int num_table_rows, const int32_t *regions, const int32_t *d_regions,
+                           int n_regions, const MistOutTables *tables, void *stream);
+
 /* mist_mip_solve over the problems of whole searches (inter_stage_tune, inter_tuning_mip.py:
  * 131-214: for every G, for every stage count, one assignment bounded by the best cost so far,
  * which starts at MIST_MIP_MAX_VALUE; a strictly smaller cost replaces it).  `n_chains`

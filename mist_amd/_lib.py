@@ -408,6 +408,9 @@ _MIP_SIGNATURES = {
     "mist_sizeof_mip_batch_item": (ctypes.c_int, []),
     "mist_mip_stage_samples_batch": (
         ctypes.c_int, [_VP, _VP, ctypes.c_int, _VP, _VP, _VP, _VP, _VP, _VP]),
+    "mist_mip_prefill_cells": (
+        ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _VP, _VP,
+                       ctypes.c_int, ctypes.POINTER(OutTables), _VP]),
     "mist_mip_solve_chains": (
         ctypes.c_int, [_VP, _VP, ctypes.c_int, ctypes.c_int, _VP, _VP, _VP, _VP, _VP, _VP, _VP]),
     "mist_mip_solve": (

@@ -136,6 +136,46 @@ __global__ __launch_bounds__(kSampleLanes) void stage_samples_batch_kernel(
                     out_stable + o, out_delta + o, out_index + o, out_keep + o);
 }
 
+// One workgroup per table row (a (variant, pre-saved micro-batches, layer count) of a region, all
+// its ckpt counts and samples): costs +inf, row indices -1.
+__global__ __launch_bounds__(256) void prefill_cells_kernel(const int32_t *__restrict__ regions,
+                                                            int n_regions, int L, int P1, int S,
+                                                            int Q, const MistOutTables tables) {
+  int lo = 0, hi = n_regions - 1;
+  const int block = blockIdx.x;
+  while (lo < hi) {  // last region whose first row is <= block
+    const int mid = (lo + hi + 1) >> 1;
+    if (regions[6 * mid + 5] <= block) lo = mid;
+    else hi = mid - 1;
+  }
+  const int32_t *r = regions + 6 * lo;
+  const int64_t g = r[0], q = r[1];
+  const int l_min = r[2], nl = r[3] - r[2] + 1, pc = min(r[4], P1);
+  int row = block - r[5];
+  const int64_t cells = (int64_t)(L + 1) * S;
+  int v;
+  int64_t at;
+  if (row < 2 * pc * nl) {
+    v = row / (pc * nl);
+    row -= v * pc * nl;
+    const int p = row / nl, l = l_min + row % nl;
+    at = (((g * Q + q) * P1 + p) * L + (l - 1)) * cells;
+  } else if (row < 2 * pc * nl + nl) {
+    v = 2;
+    at = ((g * Q + q) * L + (l_min + row - 2 * pc * nl - 1)) * cells;
+  } else {
+    v = 3;
+    at = (g * Q + q) * cells;
+  }
+  double *__restrict__ stable = tables.stable[v] + at, *__restrict__ delta = tables.delta[v] + at;
+  int32_t *__restrict__ index = tables.index[v] + at;
+  for (int64_t e = threadIdx.x; e < cells; e += blockDim.x) {
+    stable[e] = INFINITY;
+    delta[e] = INFINITY;
+    index[e] = -1;
+  }
+}
+
 int check_mip_shape(const MistMipShape *s) {
   if (!s) return fail(MIST_E_INVALID, "null MistMipShape");
   if (s->num_layers < 1 || s->num_stages < 1 || s->num_stages > s->num_layers)
@@ -311,6 +351,35 @@ int mist_mip_solve(const MistMipShape *shape, int grad_accum, double best_cost,
     }
   }
   return best < inf ? 1 : 0;
+}
+
+int mist_mip_prefill_cells(int num_layers, int p_dim, int sample_size, int num_mesh,
+                           int num_table_rows, const int32_t *regions, const int32_t *d_regions,
+                           int n_regions, const MistOutTables *tables, void *stream) {
+  if (!regions || !d_regions || !tables) return fail(MIST_E_INVALID, "null pointer");
+  if (n_regions < 1) return fail(MIST_E_INVALID, "n_regions %d < 1", n_regions);
+  if (num_layers < 1 || p_dim < 1 || sample_size < 1 || num_mesh < 1 || num_table_rows < 1)
+    return fail(MIST_E_INVALID, "table extents must be positive");
+  for (int v = 0; v < 4; ++v)
+    if (!tables->stable[v] || !tables->delta[v] || !tables->index[v])
+      return fail(MIST_E_INVALID, "null table of variant %d", v);
+  int64_t rows = 0;
+  for (int i = 0; i < n_regions; ++i) {
+    const int32_t *r = regions + 6 * i;
+    if (r[0] < 0 || r[0] >= num_table_rows || r[1] < 0 || r[1] >= num_mesh)
+      return fail(MIST_E_INVALID, "region %d: table row %d / mesh %d outside the tables", i, r[0], r[1]);
+    if (r[2] < 1 || r[3] > num_layers || r[2] > r[3] || r[4] < 1)
+      return fail(MIST_E_INVALID, "region %d: layer counts %d..%d, %d pre-saved micro-batch values", i,
+                  r[2], r[3], r[4]);
+    if (r[5] != rows) return fail(MIST_E_INVALID, "region %d: first row does not continue the list", i);
+    const int64_t nl = r[3] - r[2] + 1, pc = std::min(r[4], p_dim);
+    rows += 2 * pc * nl + nl + (r[3] == num_layers ? 1 : 0);
+  }
+  if (rows >= (int64_t)1 << 31) return fail(MIST_E_INVALID, "too many rows for one launch");
+  hipLaunchKernelGGL(prefill_cells_kernel, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream,
+                     d_regions, n_regions, num_layers, p_dim, sample_size, num_mesh, *tables);
+  MIST_HIP_CHECK(hipGetLastError());
+  return 0;
 }
 
 int mist_mip_solve_chains(const MistMipBatchItem *items, const int32_t *grad_accum,

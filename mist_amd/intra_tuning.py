@@ -302,6 +302,11 @@ class IntraStageTuner:
         # ckpt) pairs that hold them evaluated; every other cell keeps its pre-filled inf / -1.
         # The evaluated cells are the same as without it.
         self.cells_wanted = None
+        # True (with ``cells_wanted``): the output tables are pre-filled (+inf / -1) in the cells
+        # ``cells_wanted`` names only, whatever else they hold is undefined - for a caller that
+        # reads nothing else (the stage assignment; with 30 samples the fill of the whole tables
+        # is a tenth of its search)
+        self.prefill_wanted_cells_only = False
         self.results: Optional[IntraStageTunerOutput] = None
         self.stats: Dict[str, float] = {}
 
@@ -311,12 +316,30 @@ class IntraStageTuner:
         library (``mist_plan_groups``) for plans on the closed-form layer tables, in python
         otherwise and when ``MIST_PYTHON_PLAN_BUILDER`` is set; the two give the same bytes."""
         _lib.load()  # the tile sizes of the decomposition are the library's
+        wanted = self._wanted_cells()
         built = None
         if not os.environ.get("MIST_PYTHON_PLAN_BUILDER"):
-            built = self._build_groups_native()
+            built = self._build_groups_native(wanted)
         if built is None:
-            built = self._build_groups_python()
-        return self._finish_plan(*built)
+            built = self._build_groups_python(wanted)
+        plan = self._finish_plan(*built)
+        plan["wanted"] = wanted
+        return plan
+
+    def _wanted_cells(self) -> Optional[np.ndarray]:
+        """``cells_wanted`` of every (G, mesh) as int32 ``[G][mesh][3]`` = (smallest layer count,
+        largest, number of pre-saved micro-batch values), -1s where nothing is read; None without
+        ``cells_wanted``."""
+        if self.cells_wanted is None:
+            return None
+        Gs, Q = self.gradient_accumulation_steps_candidates, self.device_mesh_candidates
+        wanted = np.full((len(Gs), len(Q), 3), -1, dtype=np.int32)
+        for g, G in enumerate(Gs):
+            for q, mesh in enumerate(Q):
+                cells = self._cells_wanted_of(G, mesh)
+                if cells is not None:
+                    wanted[g, q] = cells
+        return wanted
 
     def _cells_wanted_of(self, G, mesh):
         """``cells_wanted`` of a (G, mesh) as ``(smallest layer count, largest, number of
@@ -330,7 +353,7 @@ class IntraStageTuner:
             return None
         return l_min, l_max, int(p_count)
 
-    def _build_groups_native(self):
+    def _build_groups_native(self, wanted: Optional[np.ndarray] = None):
         """The groups of this call from ``mist_plan_groups``, or None when the plan is outside
         what it covers or fails one of its checks (the python builder then words the error)."""
         cfg, tables, L = self.config, self.layer_tables, self.num_layers
@@ -395,14 +418,9 @@ class IntraStageTuner:
         req.target_reduce_waves, req.scout_min_stages = TARGET_REDUCE_WAVES, SCOUT_MIN_STAGES
         req.scout_min_pairs, req.scout_pairs = SCOUT_MIN_PAIRS, SCOUT_PAIRS
         req.scout_pair_span, req.scout_tight_pairs = SCOUT_PAIR_SPAN, SCOUT_TIGHT_PAIRS
-        wanted = None
-        if self.cells_wanted is not None:
-            wanted = np.full((len(Gs), len(Q), 3), -1, dtype=np.int32)
-            for g, G in enumerate(Gs):
-                for q, mesh in enumerate(Q):
-                    cells = self._cells_wanted_of(G, mesh)
-                    if cells is not None:
-                        wanted[g, q] = cells
+        if wanted is None:
+            wanted = self._wanted_cells()
+        if wanted is not None:
             req.cells_wanted = wanted.ctypes.data
         entries = req.n_tp * req.n_grad_accum * req.n_mesh
         groups = np.zeros(entries, dtype=_lib.GROUP_DTYPE)
@@ -426,7 +444,7 @@ class IntraStageTuner:
         return (groups[:n], spaces, prefixes[0, :n + 1], prefixes[1, :n + 1], prefixes[2, :n + 1], bounds,
                 result.max_scout_rows, result.max_group_keys)
 
-    def _build_groups_python(self):
+    def _build_groups_python(self, wanted: Optional[np.ndarray] = None):
         cfg, L = self.config, self.num_layers
         Gs, Q = self.gradient_accumulation_steps_candidates, self.device_mesh_candidates
         P = self.max_possible_pre_saved_micro_batches
@@ -437,6 +455,8 @@ class IntraStageTuner:
         B = cfg.training.global_batch_size
         n_pairs = L * (L + 1) // 2 + L
         tile_window = []  # per group: first tile of its (layers, ckpt) pairs and how many
+        if wanted is None:
+            wanted = self._wanted_cells()
         for t, tp_size in enumerate(self.tp_sizes):
             for g, G in enumerate(Gs):
                 for q, (n, m) in enumerate(Q):
@@ -450,11 +470,10 @@ class IntraStageTuner:
                     if self.evaluate_all_p:
                         num_p = P + 1
                     window = (0, -(-n_pairs // _lib.LC_TILE))
-                    if self.cells_wanted is not None:
-                        wanted = self._cells_wanted_of(G, (n, m))
-                        if wanted is None:
+                    if wanted is not None:
+                        l_min, l_max, p_count = (int(x) for x in wanted[g, q])
+                        if l_min < 0:
                             continue
-                        l_min, l_max, p_count = wanted
                         num_p = min(num_p, p_count)
                         # pairs are numbered l-major: index(l, c) = l (l + 1) / 2 - 1 + c
                         first = (l_min * (l_min + 1) // 2 - 1) // _lib.LC_TILE
@@ -575,7 +594,9 @@ class IntraStageTuner:
             first = last
         return bounds
 
-    def allocate_tables(self) -> DeviceTables:
+    def allocate_tables(self, plan: Optional[dict] = None) -> DeviceTables:
+        """Output tables, pre-filled with +inf / -1: all of them, or (``plan`` of a tuner with
+        ``prefill_wanted_cells_only``) the cells ``cells_wanted`` names."""
         Gn = len(self.tp_sizes) * len(self.gradient_accumulation_steps_candidates)
         Qn = len(self.device_mesh_candidates)
         P1, L, S = self.max_possible_pre_saved_micro_batches + 1, self.num_layers, self.sample_size
@@ -584,12 +605,39 @@ class IntraStageTuner:
         # one allocation and one fill per element type; the tables are views of it
         sizes = [int(np.prod(s)) for s in shapes]
         starts = np.concatenate([[0], np.cumsum(sizes)])
-        costs = torch.full((2 * int(starts[-1]),), float("inf"), dtype=torch.float64, device=dev)
-        index = torch.full((int(starts[-1]),), -1, dtype=torch.int32, device=dev)
         def views(flat, base):
             return [flat[base + int(starts[v]):base + int(starts[v + 1])].view(shapes[v]) for v in range(4)]
-        return DeviceTables(stable=views(costs, 0), delta=views(costs, int(starts[-1])),
-                            index=views(index, 0))
+        wanted = plan.get("wanted") if plan is not None and self.prefill_wanted_cells_only else None
+        if wanted is None:
+            costs = torch.full((2 * int(starts[-1]),), float("inf"), dtype=torch.float64, device=dev)
+            index = torch.full((int(starts[-1]),), -1, dtype=torch.int32, device=dev)
+            return DeviceTables(stable=views(costs, 0), delta=views(costs, int(starts[-1])),
+                                index=views(index, 0))
+        costs = torch.empty((2 * int(starts[-1]),), dtype=torch.float64, device=dev)
+        index = torch.empty((int(starts[-1]),), dtype=torch.int32, device=dev)
+        tables = DeviceTables(stable=views(costs, 0), delta=views(costs, int(starts[-1])),
+                              index=views(index, 0))
+        g, q = np.nonzero(wanted[:, :, 0] >= 0)
+        if len(g):
+            n_g = wanted.shape[0]
+            one = np.zeros((len(g), 6), dtype=np.int32)
+            one[:, 0], one[:, 1], one[:, 2:5] = g, q, wanted[g, q]
+            regions = np.tile(one, (len(self.tp_sizes), 1))
+            regions[:, 0] += np.repeat(np.arange(len(self.tp_sizes), dtype=np.int32) * n_g, len(g))
+            nl = (regions[:, 3] - regions[:, 2] + 1).astype(np.int64)
+            rows = 2 * np.minimum(regions[:, 4], P1) * nl + nl + (regions[:, 3] == L)
+            first = np.concatenate(([0], np.cumsum(rows)[:-1]))
+            if int(rows.sum()) >= 2**31:
+                raise ValueError("the cells to pre-fill exceed one launch")
+            regions[:, 5] = first
+            d_regions = torch.from_numpy(regions.reshape(-1)).to(dev)
+            struct = tables.as_struct()
+            rc = _lib.load().mist_mip_prefill_cells(
+                L, P1, S, Qn, Gn, ctypes.c_void_p(regions.ctypes.data), d_regions.data_ptr(),
+                len(regions), ctypes.byref(struct),
+                ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream))
+            _lib.check(rc, "mist_mip_prefill_cells")
+        return tables
 
     # ------------------------------------------------------------------ device side
     def upload(self, plan) -> dict:
@@ -759,7 +807,7 @@ class IntraStageTuner:
         """Device part only: fresh output tables + kernel launches for an uploaded plan; one
         output per tp size, all resident in the same tables."""
         with torch.cuda.device(self.device):
-            tables = self.allocate_tables()
+            tables = self.allocate_tables(plan)
             tables.grad_accum = dev_plan.get("grad_accum")
             self.launch(plan, dev_plan, tables)
         return self._outputs(plan, tables)

@@ -132,6 +132,7 @@ def _uniform_device_pp_mip(mist_config, device, stats):
         if not MIP_EVALUATE_ALL_CELLS:
             tuner.cells_wanted = mip_cells_wanted(
                 L, hw.num_nodes, hw.num_gpus_per_node, int(getattr(tuning, "layers_offset", 2)))
+            tuner.prefill_wanted_cells_only = True  # nothing else of the tables is read below
         results = tuner.tune_all()
         t1 = time.perf_counter()
         stats["intra_s"] = stats.get("intra_s", 0.0) + (t1 - t0)

@@ -395,3 +395,66 @@ def test_batched_search_equals_one_search_per_candidate(plan, samples, overrides
             S = len(best[1])
             assert np.array_equal(layers[c, :S], best[1]) and np.array_equal(slots[c, :S], best[2])
     assert (winner >= 0).any()
+
+
+@pytest.mark.parametrize("plan, samples, overrides", [
+    (1, 30, {}),
+    (2, 3, {}),
+    (1, 4, dict(model__num_hidden_layers=9, hardware__num_nodes=2, hardware__num_gpus_per_node=4,
+                training__global_batch_size=32, hardware__memory_capacity=1.5)),  # some cells fit nothing
+])
+def test_tables_prefilled_in_the_cells_the_assignment_reads_only(plan, samples, overrides):
+    """``IntraStageTuner.prefill_wanted_cells_only`` (what ``tune`` sets for this granularity):
+    the tables come from unfilled memory, holding a poison value here, and only the cells
+    ``cells_wanted`` names are pre-filled; all of those - every ckpt count, sample and pre-saved
+    micro-batch value the assignment can index, with or without a feasible strategy - equal the
+    tables of a tuner that fills everything, and so does the search on them."""
+    import torch
+
+    from mist_amd.inter_tuning_mip import cells_wanted, inter_stage_tune_batch
+    from mist_amd.intra_tuning import IntraStageTuner
+    from mist_amd.search_space import _get_device_mesh_candidates, _get_grad_accumu_steps_candidates
+    from mist_amd.tune_one_case import tp_candidates
+
+    cfg, tables = load_plan(plan, tuning__tuning_granularity="uniform-device-pp-mip",
+                            tuning__sample_size=samples, **overrides)
+    hw, L = cfg.hardware, cfg.model.num_hidden_layers
+    meshes = _get_device_mesh_candidates(hw.num_nodes, hw.num_gpus_per_node, False)
+    Gs = _get_grad_accumu_steps_candidates(cfg.training.global_batch_size)
+    tps = tp_candidates(cfg)
+    full_results = IntraStageTuner(tables, L, meshes, Gs, tps, cfg, sample_size=samples).tune_all()
+    full = full_results[0].batch
+    n_cost, n_index = 2 * sum(t.numel() for t in full.stable), sum(t.numel() for t in full.index)
+    # the caching allocator hands the blocks of these two back to the next tables of that size
+    poison = [torch.full((n_cost,), 0.125, dtype=torch.float64, device="cuda"),
+              torch.full((n_index,), 7, dtype=torch.int32, device="cuda")]
+    torch.cuda.synchronize()
+    del poison
+    tuner = IntraStageTuner(tables, L, meshes, Gs, tps, cfg, sample_size=samples)
+    wanted = tuner.cells_wanted = cells_wanted(L, hw.num_nodes, hw.num_gpus_per_node)
+    tuner.prefill_wanted_cells_only = True
+    part_results = tuner.tune_all()
+    part = part_results[0].batch
+    P1 = full.stable[0].shape[2]
+    n_read = n_infeasible = 0
+    for t in range(len(tps)):
+        for g, G in enumerate(Gs):
+            for q, mesh in enumerate(meshes):
+                w = wanted(G, mesh)
+                if w is None:
+                    continue
+                row, (lo, hi, p_count) = t * len(Gs) + g, w
+                lo, hi, p_count = max(lo, 1), min(hi, L), min(p_count, P1)
+                for name in ("stable", "delta", "index"):
+                    a, b = getattr(full, name), getattr(part, name)
+                    for v in (0, 1):
+                        assert torch.equal(a[v][row, q, :p_count, lo - 1:hi], b[v][row, q, :p_count, lo - 1:hi])
+                    assert torch.equal(a[2][row, q, lo - 1:hi], b[2][row, q, lo - 1:hi])
+                    if hi == L:
+                        assert torch.equal(a[3][row, q], b[3][row, q])
+                n_read += 1
+                n_infeasible += int((full.index[0][row, q, :p_count, lo - 1:hi] == -1).any())
+    assert n_read > 0 and n_infeasible > 0
+    assert not torch.equal(full.index[0], part.index[0]), "the poison did not reach the tables: nothing tested"
+    args = (L, hw.num_nodes, hw.num_gpus_per_node, meshes, Gs)
+    assert inter_stage_tune_batch(*args, part_results, cfg) == inter_stage_tune_batch(*args, full_results, cfg)

@@ -237,6 +237,27 @@ int mist_eval_reduce_samples(const MistProblem *problem, const MistGroupDesc *d_
                              int main_batch, double *d_partial_cost, int32_t *d_partial_index,
                              const MistOutTables *tables, void *stream);
 
+/* mist_row_terms + mist_eval_reduce_samples for ALL n_samples ratios of a tuner call (any
+ * number; batches of `sample_batch` <= MIST_MAX_SAMPLE_BATCH, main launches of `main_batch` <=
+ * sample_batch samples), with the small launches moved out of the way of the large ones: the
+ * scout pass of the first batch runs on the library's second stream beside the row terms of the
+ * rows it does not gather (as in mist_intra_stage_eval), and the scout pass of batch b + 1 beside
+ * the main launches of batch b, into the other of two scout regions.  Same tables as the calls
+ * it replaces (reference: the S samples of one compute_indices call per group,
+ * mist/utils/pareto.py:124-144).  `ratios` and `sample_index` are HOST arrays of n_samples.
+ * d_partial_cost / d_partial_index: [main_batch * n_reduce_blocks + 2 * sample_batch *
+ * n_scout_blocks] slabs.  Without a scout pass (n_scout_blocks == 0 or
+ * problem->max_scout_rows == 0) the calls it replaces run one after the other on `stream`. */
+int mist_intra_stage_eval_samples(const MistProblem *problem, const MistGroupDesc *d_groups,
+                                  int n_groups, const int32_t *d_terms_block_prefix,
+                                  int n_terms_blocks, const int32_t *d_reduce_block_prefix,
+                                  int n_reduce_blocks, const int32_t *d_scout_prefix,
+                                  int n_scout_blocks, double *d_row_terms, double *d_stage_floor,
+                                  double *d_key_terms, double *d_partial_cost,
+                                  int32_t *d_partial_index, const double *ratios,
+                                  const int32_t *sample_index, int n_samples, int sample_batch,
+                                  int main_batch, const MistOutTables *tables, void *stream);
+
 /* mist_eval_reduce with every cell evaluated: each (row, layers, ckpt) through the latency and
  * memory model and each pre-saved micro-batch value through the reference's feasibility test
  * (batched_module_analyzer.py:2218-3106, pareto.py:124-144 as written, cell by cell), no scout

@@ -133,6 +133,12 @@ _SIGNATURES = {
         [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, _VP, _VP, _VP,
          ctypes.c_int, ctypes.c_int, _VP, _VP, ctypes.POINTER(OutTables), _VP],
     ),
+    "mist_intra_stage_eval_samples": (
+        ctypes.c_int,
+        [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, ctypes.c_int,
+         _VP, _VP, _VP, _VP, _VP, _VP, _VP, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+         ctypes.POINTER(OutTables), _VP],
+    ),
     "mist_eval_reduce_exhaustive": (
         ctypes.c_int,
         [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, ctypes.c_double, _VP, _VP, _VP],

@@ -2359,8 +2359,9 @@ int mist_finalize(const MistProblem *problem, const MistGroupDesc *d_groups, int
 namespace {
 struct OverlapStreams {
   hipStream_t side = nullptr;
-  hipEvent_t rows_ready = nullptr, scout_done = nullptr;
+  hipEvent_t rows_ready = nullptr, scout_done = nullptr, main_done = nullptr;
 };
+std::mutex g_enqueue_lock;  // one call's records and waits on the shared events are a unit
 int overlap_streams(OverlapStreams **out) {
   static std::mutex lock;
   static OverlapStreams known[64];
@@ -2373,6 +2374,7 @@ int overlap_streams(OverlapStreams **out) {
     MIST_HIP_CHECK(hipStreamCreateWithFlags(&s.side, hipStreamNonBlocking));  // default priority
     MIST_HIP_CHECK(hipEventCreateWithFlags(&s.rows_ready, hipEventDisableTiming));
     MIST_HIP_CHECK(hipEventCreateWithFlags(&s.scout_done, hipEventDisableTiming));
+    MIST_HIP_CHECK(hipEventCreateWithFlags(&s.main_done, hipEventDisableTiming));
   }
   *out = &s;
   return 0;
@@ -2404,8 +2406,7 @@ int mist_intra_stage_eval(const MistProblem *problem, const MistGroupDesc *d_gro
     if (int rc = overlap_streams(&os)) return rc;
     // the second stream and its events are shared by all callers: one call's records and waits
     // are enqueued as a unit
-    static std::mutex enqueue_lock;
-    std::lock_guard<std::mutex> enqueue_guard(enqueue_lock);
+    std::lock_guard<std::mutex> enqueue_guard(g_enqueue_lock);
     hipStream_t main_stream = (hipStream_t)stream;
     const unsigned scout_term_blocks = (unsigned)((problem->max_scout_rows + kTermsBlock - 1) / kTermsBlock);
     hipLaunchKernelGGL((row_terms_kernel<1, false>), dim3(scout_term_blocks, n_groups),
@@ -2453,6 +2454,124 @@ int mist_intra_stage_eval(const MistProblem *problem, const MistGroupDesc *d_gro
     return rc;
   return mist_finalize(problem, d_groups, n_groups, d_reduce_block_prefix, d_row_terms,
                        d_partial_cost, d_partial_index, sample_index, tables, stream);
+}
+
+int mist_intra_stage_eval_samples(const MistProblem *problem, const MistGroupDesc *d_groups,
+                                  int n_groups, const int32_t *d_terms_block_prefix,
+                                  int n_terms_blocks, const int32_t *d_reduce_block_prefix,
+                                  int n_reduce_blocks, const int32_t *d_scout_prefix,
+                                  int n_scout_blocks, double *d_row_terms, double *d_stage_floor,
+                                  double *d_key_terms, double *d_partial_cost,
+                                  int32_t *d_partial_index, const double *ratios,
+                                  const int32_t *sample_index, int n_samples, int sample_batch,
+                                  int main_batch, const MistOutTables *tables, void *stream) {
+  if (!ratios || !sample_index || n_samples < 1)
+    return fail(MIST_E_INVALID, "n_samples %d < 1 or null sample lists", n_samples);
+  if (sample_batch < 1 || sample_batch > MIST_MAX_SAMPLE_BATCH)
+    return fail(MIST_E_INVALID, "sample_batch %d outside [1, %d]", sample_batch, MIST_MAX_SAMPLE_BATCH);
+  if (main_batch < 1 || main_batch > sample_batch)
+    return fail(MIST_E_INVALID, "main_batch %d outside [1, sample_batch = %d]", main_batch, sample_batch);
+  const bool overlap = n_scout_blocks > 0 && problem != nullptr && problem->max_scout_rows > 0 &&
+                       n_groups > 0 && n_groups <= 65535;
+  if (!overlap) {
+    if (int rc = mist_row_terms(problem, d_groups, n_groups, d_terms_block_prefix, n_terms_blocks,
+                                d_row_terms, d_stage_floor, d_key_terms, stream))
+      return rc;
+    for (int first = 0; first < n_samples; first += sample_batch) {
+      const int count = std::min(sample_batch, n_samples - first);
+      if (int rc = mist_eval_reduce_samples(problem, d_groups, n_groups, d_reduce_block_prefix,
+                                            n_reduce_blocks, d_scout_prefix, n_scout_blocks,
+                                            d_row_terms, d_stage_floor, ratios + first,
+                                            sample_index + first, count, std::min(main_batch, count),
+                                            d_partial_cost, d_partial_index, tables, stream))
+        return rc;
+    }
+    return 0;
+  }
+  // Stream order: [terms of the gathered rows] -> side stream: scout pass of the first batch of
+  // samples || this stream: all other row terms -> per batch b: side stream: scout pass of batch
+  // b + 1 (into the other scout region, once the main launches of batch b - 1, which read it,
+  // are through) || this stream: main launches and finalize of batch b.
+  if (int rc = check_reduce_arguments(problem, d_groups, n_groups, d_reduce_block_prefix,
+                                      n_reduce_blocks, d_scout_prefix, n_scout_blocks, d_row_terms,
+                                      d_stage_floor, d_partial_cost, d_partial_index))
+    return rc;
+  if (!d_terms_block_prefix || n_terms_blocks <= 0)
+    return fail(MIST_E_INVALID, "null / empty row-term decomposition");
+  if (int rc = check_factors(problem)) return rc;
+  for (int i = 0; i < n_samples; ++i)
+    if (!(ratios[i] >= 0.0)) return fail(MIST_E_INVALID, "ratio %d must be non-negative", i);
+  OverlapStreams *os = nullptr;
+  if (int rc = overlap_streams(&os)) return rc;
+  std::lock_guard<std::mutex> enqueue_guard(g_enqueue_lock);
+  hipStream_t main_stream = (hipStream_t)stream;
+  const int n_batches = (n_samples + sample_batch - 1) / sample_batch;
+  const int64_t main_slabs = (int64_t)main_batch * n_reduce_blocks;
+  const int64_t scout_slabs = (int64_t)sample_batch * n_scout_blocks;
+  auto batch_ratios = [&](int b, int *count) {
+    RatioList list = {};
+    const int first = b * sample_batch;
+    *count = std::min(sample_batch, n_samples - first);
+    for (int i = 0; i < *count; ++i) list.r[i] = ratios[first + i];
+    return list;
+  };
+  auto scout_of = [&](int b) -> int {  // on the side stream
+    int count = 0;
+    const RatioList list = batch_ratios(b, &count);
+    if (int rc = launch_scout(problem, d_groups, n_groups, d_reduce_block_prefix, n_reduce_blocks,
+                              d_scout_prefix, n_scout_blocks, d_row_terms, d_stage_floor, list, count,
+                              main_slabs + (b % 2) * scout_slabs, d_partial_cost, d_partial_index,
+                              os->side))
+      return rc;
+    MIST_HIP_CHECK(hipEventRecord(os->scout_done, os->side));
+    return 0;
+  };
+  const unsigned scout_term_blocks = (unsigned)((problem->max_scout_rows + kTermsBlock - 1) / kTermsBlock);
+  hipLaunchKernelGGL((row_terms_kernel<1, false>), dim3(scout_term_blocks, n_groups),
+                     dim3(kTermsBlock), 0, main_stream, *problem, d_groups, n_groups,
+                     d_terms_block_prefix, d_row_terms, d_stage_floor, nullptr);
+  MIST_HIP_CHECK(hipGetLastError());
+  MIST_HIP_CHECK(hipEventRecord(os->rows_ready, main_stream));
+  MIST_HIP_CHECK(hipStreamWaitEvent(os->side, os->rows_ready, 0));
+  if (int rc = scout_of(0)) return rc;
+  bool from_keys = false;
+  if (int rc = launch_key_terms(problem, d_groups, n_groups, d_key_terms, main_stream, &from_keys))
+    return rc;
+  if (from_keys)
+    hipLaunchKernelGGL((row_terms_kernel<2, true>), dim3(n_terms_blocks), dim3(kTermsBlock), 0,
+                       main_stream, *problem, d_groups, n_groups, d_terms_block_prefix, d_row_terms,
+                       d_stage_floor, d_key_terms);
+  else
+    hipLaunchKernelGGL((row_terms_kernel<2, false>), dim3(n_terms_blocks), dim3(kTermsBlock), 0,
+                       main_stream, *problem, d_groups, n_groups, d_terms_block_prefix, d_row_terms,
+                       d_stage_floor, nullptr);
+  MIST_HIP_CHECK(hipGetLastError());
+  for (int b = 0; b < n_batches; ++b) {
+    // (a wait takes the event's latest record at the time of the call: the scout pass of batch b)
+    MIST_HIP_CHECK(hipStreamWaitEvent(main_stream, os->scout_done, 0));
+    if (b + 1 < n_batches) {
+      if (b >= 1) MIST_HIP_CHECK(hipStreamWaitEvent(os->side, os->main_done, 0));  // batch b - 1
+      if (int rc = scout_of(b + 1)) return rc;
+    }
+    int count = 0;
+    const RatioList list = batch_ratios(b, &count);
+    for (int first = 0; first < count; first += main_batch) {
+      const int n = std::min(main_batch, count - first);
+      hipLaunchKernelGGL(eval_reduce_kernel, dim3(xcd_padded_grid(n_reduce_blocks), n),
+                         dim3(MIST_LC_TILE), 0, main_stream, *problem, d_groups, n_groups,
+                         d_reduce_block_prefix, n_reduce_blocks, d_scout_prefix, 0, d_row_terms,
+                         d_stage_floor, list, first, main_slabs + (b % 2) * scout_slabs, d_partial_cost,
+                         d_partial_index);
+      MIST_HIP_CHECK(hipGetLastError());
+      if (int rc = launch_finalize(problem, d_groups, n_groups, d_reduce_block_prefix, d_row_terms,
+                                   d_partial_cost, d_partial_index,
+                                   sample_index + b * sample_batch + first, n, n_reduce_blocks, tables,
+                                   stream))
+        return rc;
+    }
+    MIST_HIP_CHECK(hipEventRecord(os->main_done, main_stream));
+  }
+  return 0;
 }
 
 int mist_row_diagnostics(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,

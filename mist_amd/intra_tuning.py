@@ -668,7 +668,9 @@ class IntraStageTuner:
         slab_bytes = _lib.SLOTS * _lib.LC_TILE * 12
         most = max([b["n_reduce_blocks"] for b in batches] + [1])
         self._main_batch = int(max(1, min(self._sample_batch, MAIN_BATCH_SLAB_BYTES // (most * slab_bytes))))
-        n_slabs = max([self._main_batch * b["n_reduce_blocks"] + self._sample_batch * b["n_scout_blocks"]
+        # (two scout regions: the scout pass of the next batch of samples runs beside the main
+        # launches of the current one)
+        n_slabs = max([self._main_batch * b["n_reduce_blocks"] + 2 * self._sample_batch * b["n_scout_blocks"]
                        for b in batches] + [1])
         def workspace():
             return dict(
@@ -744,22 +746,17 @@ class IntraStageTuner:
                     _ptr(w["partial_cost"]), _ptr(w["partial_index"]), stream)
 
             if events is None and not self.exhaustive and len(self.sample_slots) > 1:
-                _lib.check(lib.mist_row_terms(
+                slots = np.array(self.sample_slots, dtype=np.int32)
+                all_ratios = np.ascontiguousarray(ratios[slots], dtype=np.float64)
+                rc = lib.mist_intra_stage_eval_samples(
                     prob_ptr, _ptr(d["groups"]), d["n_groups"], _ptr(d["terms_prefix"]),
-                    d["n_terms_blocks"], _ptr(w["row_terms"]), _ptr(w["stage_floor"]),
-                    _ptr(w["key_terms"]), stream), "mist_row_terms")
-                for first in range(0, len(self.sample_slots), self._sample_batch):
-                    slots = np.array(self.sample_slots[first:first + self._sample_batch], dtype=np.int32)
-                    batch_ratios = np.ascontiguousarray(ratios[slots], dtype=np.float64)
-                    rc = lib.mist_eval_reduce_samples(
-                        prob_ptr, _ptr(d["groups"]), d["n_groups"], _ptr(d["reduce_prefix"]),
-                        d["n_reduce_blocks"], _ptr(d["scout_prefix"]), d["n_scout_blocks"],
-                        _ptr(w["row_terms"]), _ptr(w["stage_floor"]),
-                        ctypes.c_void_p(batch_ratios.ctypes.data), ctypes.c_void_p(slots.ctypes.data),
-                        len(slots), min(self._main_batch, len(slots)), _ptr(w["partial_cost"]),
-                        _ptr(w["partial_index"]),
-                        ctypes.byref(out), stream)
-                    _lib.check(rc, "mist_eval_reduce_samples")
+                    d["n_terms_blocks"], _ptr(d["reduce_prefix"]), d["n_reduce_blocks"],
+                    _ptr(d["scout_prefix"]), d["n_scout_blocks"], _ptr(w["row_terms"]),
+                    _ptr(w["stage_floor"]), _ptr(w["key_terms"]), _ptr(w["partial_cost"]),
+                    _ptr(w["partial_index"]), ctypes.c_void_p(all_ratios.ctypes.data),
+                    ctypes.c_void_p(slots.ctypes.data), len(slots), self._sample_batch,
+                    min(self._main_batch, self._sample_batch), ctypes.byref(out), stream)
+                _lib.check(rc, "mist_intra_stage_eval_samples")
                 continue
             for i, slot in enumerate(self.sample_slots):
                 if events is None and not self.exhaustive:

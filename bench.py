@@ -293,6 +293,10 @@ def main():
     ap.add_argument("--only-plan", default=None, metavar="YAML",
                     help="profiling aid: run --steps search steps of this plan of mist_amd/configs "
                          "with resident descriptors, print their time and exit (no bench line)")
+    ap.add_argument("--only-mip", default=None, metavar="YAML",
+                    help="profiling aid: --steps calls of tune() on this plan of mist_amd/configs with "
+                         "the uniform-device-pp-mip granularity and 30 samples per cell, print their "
+                         "time and exit (no bench line)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU only (got --gpus {args.gpus}): the search runs on a "
@@ -325,6 +329,23 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps(dict(plan=args.only_plan, steps=args.steps, cost=cost,
                               ms_per_step=1e3 * (time.perf_counter() - t0) / args.steps, **search.counts())))
+        return
+
+    if args.only_mip:
+        import yaml
+
+        with open(os.path.join(REPO, "mist_amd", "configs", args.only_mip)) as f:
+            raw = yaml.safe_load(f)
+        raw["tuning"].update(tuning_granularity="uniform-device-pp-mip", sample_size=30)
+        for _ in range(max(args.warmup, 1)):
+            tune(MistConfig(raw))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            cost, solution = tune(MistConfig(raw))
+        torch.cuda.synchronize()
+        print(json.dumps(dict(plan=args.only_mip, steps=args.steps, cost=cost, sample_size=30,
+                              ms_per_tune=1e3 * (time.perf_counter() - t0) / args.steps)))
         return
 
     cfg = MistConfig.from_yaml(PLAN)

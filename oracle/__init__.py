@@ -25,8 +25,8 @@ mathematics fixes (hand-computed cells typed as literals, closed forms, invarian
 on tiny inputs, numpy library routines); see tests/test_known_answer_cells.py and
 tests/test_oracle_*.py.  What none of those can pin is marked "parity unpinned" at the function:
 (1) numba ``fastmath`` contraction / reassociation of ``alpha/(1-alpha)*x + y`` for sample sizes
-above one (``stage_loop.c`` has a build with the fused form; on every group of the two smaller
-benchmark plans with 30 samples it picks the same rows), (2) numpy-1.24 legacy scalar promotion
+above one (``stage_loop.c`` has a build with the fused form; on every group of the three
+smaller benchmark plans with 30 samples it picks the same rows), (2) numpy-1.24 legacy scalar promotion
 in the two scalar expressions of the inter-stage scan, which are restated with explicit float64
 casts.
 """

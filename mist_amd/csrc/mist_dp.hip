@@ -1059,7 +1059,16 @@ __global__ __launch_bounds__(kDpPlaneThreads) void dp_plane_kernel(
       }
       fetch(task_k(round + 1));
       __builtin_amdgcn_wave_barrier();
-      DpBest w[kDpPlaneCols];
+      // Running winner per column, lean: the value and (mesh << 8 | end layer) of the candidate
+      // that set it; an unreachable successor (+inf) never compares below the winner, and the
+      // admissibility of the candidate is the same for every lane (tested once, below).
+      float best[kDpPlaneCols];
+      int best_at[kDpPlaneCols];
+#pragma unroll
+      for (int j = 0; j < kDpPlaneCols; ++j) {
+        best[j] = INFINITY;
+        best_at[j] = -1;
+      }
       for (int q = 0; q < Q; ++q) {
         const int nm = shape.mesh_n[q] * shape.mesh_m[q];
         const int i_first = max(k, reach_q[2 * q] - 1);
@@ -1087,17 +1096,29 @@ __global__ __launch_bounds__(kDpPlaneThreads) void dp_plane_kernel(
 #pragma unroll
             for (int j = 0; j < kDpPlaneCols; ++j)
               prev[j] = lane_ok[j] ? col[j][(i + 1) * W] : INFINITY;
+            const int at = (q << 8) | i;
 #pragma unroll
-            for (int j = 0; j < kDpPlaneCols; ++j)
-              dp_consider<kBottleneck>(w[j], t_max, q, i, prev[j], rmin);
+            for (int j = 0; j < kDpPlaneCols; ++j) {
+              const float target = kBottleneck ? fmaxf(rmin, prev[j]) : rmin + prev[j];
+              const bool better = target < best[j];
+              best[j] = better ? target : best[j];
+              best_at[j] = better ? at : best_at[j];
+            }
           }
         }
       }
       __builtin_amdgcn_wave_barrier();
+      DpBest w[kDpPlaneCols];
 #pragma unroll
       for (int j = 0; j < kDpPlaneCols; ++j) {
         if (!col_ok[j]) continue;
         const int d = d_of[j];
+        if (best_at[j] >= 0) {
+          w[j].best = best[j];
+          w[j].arg_q = best_at[j] >> 8;
+          w[j].arg_i = best_at[j] & 255;
+          w[j].best_rmin = my_rows[w[j].arg_q * width + (w[j].arg_i - k)];
+        }
         dp_finish_winner<kBottleneck>(w[j], shape, tabs, off, t_max, p, k, d, f_lds, m_prev);
         const int e = k * W + d;
         f_cur[e] = w[j].best;
@@ -1581,7 +1602,8 @@ int mist_dp_run(const MistDpShape *shape, const MistDpCosts *costs, const float 
       ((size_t)plane + 6 * (size_t)(shape->num_devices + 1) + 2 * (size_t)shape->num_mesh +
        (size_t)(kDpPlaneThreads / 64) * shape->num_mesh * shape->num_layers) * sizeof(float);
   const bool plane_shape_ok = shape->num_devices <= 64 * kDpPlaneCols &&
-                              shape->num_mesh * shape->num_layers <= 64 * kDpPlaneLoads;
+                              shape->num_mesh * shape->num_layers <= 64 * kDpPlaneLoads &&
+                              shape->num_layers <= 256;  // (mesh << 8 | end layer) of a winner
   const bool plane_possible = costs->stage_min != nullptr && shape->free_devices == 0 &&
                               plane_shape_ok && plane_lds <= plane_lds_limit(mode);
   if (force_plane && !plane_possible)

@@ -474,20 +474,27 @@ __device__ __host__ __forceinline__ int dp_triangle_row(int L, int k) {
 // Running winner of one state's scan.  The reference visits (q, i) in ascending order and
 // replaces on a strict "<".  A state reachable only through an unreachable successor cannot
 // improve (inf + c is never < best); skipping it changes nothing.
+constexpr int kDpNoCandidate = 0x7fffffff;
 struct DpBest {
   float best = INFINITY, best_m = 0.0f, best_rmin = 0.0f;
+  int order = kDpNoCandidate;  // q * L + i of the candidate that set `best`: its place in the visit
   int arg_i = -1, arg_q = -1, arg_j = -1;
+  // mesh and end layer of the winner, once the scan is over
+  __device__ __forceinline__ void resolve(int L) {
+    arg_q = order == kDpNoCandidate ? -1 : order / L;
+    arg_i = order == kDpNoCandidate ? -1 : order % L;
+  }
 };
+// One candidate, without a branch: an unreachable successor (+inf) gives a target of +inf, which
+// is never below the winner's.
 template <bool kBottleneck>
-__device__ __forceinline__ void dp_consider(DpBest &w, float t_max, int q, int i, float prev,
+__device__ __forceinline__ void dp_consider(DpBest &w, float t_max, int order, float prev,
                                             float rmin) {
-  if (prev == INFINITY || !(rmin <= t_max)) return;
   const float target = kBottleneck ? fmaxf(rmin, prev) : rmin + prev;
-  if (!(target < w.best)) return;
-  w.best = target;
-  w.best_rmin = rmin;
-  w.arg_i = i;
-  w.arg_q = q;
+  const bool better = rmin <= t_max && target < w.best;
+  w.best = better ? target : w.best;
+  w.best_rmin = better ? rmin : w.best_rmin;
+  w.order = better ? order : w.order;
 }
 
 // The winner's ckpt count and stage maximum: the first j attaining the sum is the entry the
@@ -624,13 +631,13 @@ __device__ __forceinline__ void dp_scan_state(DpBest &w, const MistDpShape &shap
           rmin[u] = prev[u] == INFINITY ? INFINITY : row_min(q, i0 + u);
 #pragma unroll
         for (int u = 0; u < kDpBatch; ++u)
-          dp_consider<kBottleneck>(w, t_max, q, i0 + u, prev[u], rmin[u]);
+          dp_consider<kBottleneck>(w, t_max, q * L + i0 + u, prev[u], rmin[u]);
       }
     } else {
       for (int i = i_first + member; i <= i_last; i += kDpTeam) {
         const float prev = f_prev[(i + 1) * W + (d - nm)];
         if (prev == INFINITY) continue;
-        dp_consider<kBottleneck>(w, t_max, q, i, prev, row_min(q, i));
+        dp_consider<kBottleneck>(w, t_max, q * L + i, prev, row_min(q, i));
       }
     }
   }
@@ -696,26 +703,26 @@ __global__ __launch_bounds__(kDpThreads) void dp_step_kernel(
         [&](int q, int i) {
           return relaid != nullptr ? relaid[q * tri + i] : dp_row_min(shape, tabs, off, p, k, q, i);
         });
-    if constexpr (kDpTeam == 1)
+    if constexpr (kDpTeam == 1) {
+      w.resolve(L);
       dp_finish_winner<kBottleneck>(w, shape, tabs, off, t_max, p, k, d, f_prev, m_prev);
+    }
   }
   // Team reduction: the winner is the first candidate that attains the minimum, i.e. the
   // lexicographic minimum of (target, q, i).  Each lane holds that minimum over its own
   // candidates.
   if constexpr (kDpTeam > 1) {
-    int order = w.arg_i >= 0 ? w.arg_q * L + w.arg_i : 0x7fffffff;
 #pragma unroll
     for (int step = 1; step < kDpTeam; step <<= 1) {
       const float o_best = __shfl_xor(w.best, step);
       const float o_rmin = __shfl_xor(w.best_rmin, step);
-      const int o_order = __shfl_xor(order, step);
-      const bool take = o_best < w.best || (o_best == w.best && o_order < order);
+      const int o_order = __shfl_xor(w.order, step);
+      const bool take = o_best < w.best || (o_best == w.best && o_order < w.order);
       w.best = take ? o_best : w.best;
       w.best_rmin = take ? o_rmin : w.best_rmin;
-      order = take ? o_order : order;
+      w.order = take ? o_order : w.order;
     }
-    w.arg_q = order == 0x7fffffff ? -1 : order / L;
-    w.arg_i = order == 0x7fffffff ? -1 : order % L;
+    w.resolve(L);
     if (!real || member != 0) return;
     if (live) dp_finish_winner<kBottleneck>(w, shape, tabs, off, t_max, p, k, d, f_prev, m_prev);
   }
@@ -866,6 +873,7 @@ __global__ __launch_bounds__(kDpFusedThreads) void dp_fused_kernel(
                                         i_first = max(i_first, a[0]);
                                         i_last = min(i_last, a[1]);
                                       });
+        w.resolve(L);
         dp_finish_winner<kBottleneck>(w, shape, tabs, off, t_max, p, k, d, f_prev, m_prev);
       }
       f_cur[e] = w.best;

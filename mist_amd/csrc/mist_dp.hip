@@ -43,8 +43,9 @@ constexpr int kDpBatch = 4;  // end layers whose reads a lane of the one-lane-pe
 // Table rows (fixed g, mesh, p, layers) hold the L+1 ckpt entries: cost = (float)stable +
 // (float)delta / G, and alongside its running minimum pmin[j] = min(cost[0..j]).  A workgroup
 // takes as many whole rows as fit its 256 lanes, one lane per entry, so that loads and stores
-// are contiguous; the running minimum is read back from LDS.  Rows longer than the workgroup
-// are walked in passes of 256 entries with the minimum of the earlier passes carried along.
+// are contiguous; the running minimum is a segmented scan (wavefront shuffles, LDS between the
+// wavefronts a row spans).  Rows longer than the workgroup are walked in passes of 256 entries
+// with the minimum of the earlier passes carried along.
 // Most cells of a plan hold no strategy (no group for that (g, mesh), or nothing fits): their
 // row index is -1 and their costs +inf, so with the index table (may be null) the 16 bytes of
 // such a cell's costs are not read.
@@ -77,15 +78,23 @@ __global__ __launch_bounds__(256) void cost_table_kernel(const double *__restric
       }
       out[i] = c;
     }
-    lds[threadIdx.x] = c;
-    __syncthreads();
-    if (live) {
-      float run = carry;
-      for (int a = threadIdx.x - j0; a <= (int)threadIdx.x; ++a) run = fminf(run, lds[a]);
-      pmin[i] = run;
+    // running minimum over the row's lanes of this pass: inside a wavefront by shuffles that stop
+    // at the row's first lane, then the part of the row that lies in earlier wavefronts (their
+    // last lanes hold it)
+    float run = c;
+    const int lane = threadIdx.x & 63;
+#pragma unroll
+    for (int step = 1; step < 64; step <<= 1) {
+      const float other = __shfl_up(run, step);
+      if (lane >= step && j0 >= step) run = fminf(run, other);
     }
-    if (base + seg < row_len)  // only rows longer than one pass
-      for (int a = 0; a < seg; ++a) carry = fminf(carry, lds[threadIdx.x - j0 + a]);
+    lds[threadIdx.x] = run;
+    __syncthreads();
+    const int row_first = (int)threadIdx.x - j0;
+    for (int at = (int)(threadIdx.x & ~63u) - 1; at >= row_first; at -= 64) run = fminf(run, lds[at]);
+    if (live) pmin[i] = fminf(run, carry);
+    if (base + seg < row_len)  // only rows longer than one pass: then the row is the workgroup
+      carry = fminf(carry, fminf(fminf(lds[63], lds[127]), fminf(lds[191], lds[255])));
     __syncthreads();
   }
 }

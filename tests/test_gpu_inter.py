@@ -1046,3 +1046,30 @@ def test_search_on_random_tables_equals_the_reference_scan(monkeypatch, seed, L,
     finite = [i for i, (_, sol) in enumerate(want) if sol is not None]
     keep = min(finite, key=lambda i: want[i][0]) if finite else None
     assert got == [(cost, sol if i == keep else None) for i, (cost, sol) in enumerate(want)]
+
+
+@pytest.mark.parametrize("L, P1, quantum, inf_frac", [(8, 3, 1 / 16, 0.3), (40, 2, None, 0.1), (80, 2, 1 / 4, 0.5),
+                                                      (130, 2, None, 0.0)])
+def test_cost_tables_and_running_minima_equal_numpy(L, P1, quantum, inf_frac):
+    """``mist_dp_cost_tables``: float32 cost = float32(stable) + float32(delta) / G of the sample
+    slot, +inf where the cell holds no strategy, and beside it the running minimum over the ckpt
+    counts of each table row - rows of 9 to 131 entries, i.e. several rows per wavefront up to a
+    row across three wavefronts - against numpy on random tables with ties."""
+    from mist_amd.inter_tuning import _DpRunner
+
+    rng = np.random.default_rng(L)
+    meshes, Gs, S, slot = [(1, 1), (1, 2), (1, 4)], [1, 2, 8], 2, 1
+    ours, theirs = _synthetic_results(rng, 2, Gs, meshes, L, P1, S, quantum or 1 / 1024, inf_frac,
+                                      structured=False)
+    runner = _DpRunner(ours[0], L, 4, meshes, slot)
+    G_of_row = np.tile(np.array(Gs, dtype=np.float32), 2)
+    names = ("costs_stable", "costs_stable_with_pre", "costs_stable_with_post", "costs_stable_no_pp")
+    for v, name in enumerate(names):
+        stable = np.concatenate([getattr(t, name)[..., slot] for t in theirs])
+        delta = np.concatenate([getattr(t, name.replace("stable", "delta"))[..., slot] for t in theirs])
+        with np.errstate(invalid="ignore"):
+            want = (stable + delta / G_of_row.reshape((-1,) + (1,) * (stable.ndim - 1))).astype(np.float32)
+        got, got_min = runner.cost[v].cpu().numpy(), runner.pmin[v].cpu().numpy()
+        assert np.array_equal(got.view(np.int32), want.view(np.int32)), name
+        assert np.array_equal(got_min.view(np.int32), np.minimum.accumulate(want, axis=-1).view(np.int32)), name
+        assert np.isfinite(want).any() and np.isinf(want).any() or inf_frac == 0.0

@@ -22,7 +22,7 @@ from __future__ import annotations
 
 import ctypes
 import time
-from typing import List, Optional, Tuple
+from typing import Dict, List, Optional, Tuple
 
 import numpy as np
 import torch
@@ -795,11 +795,17 @@ def _native_search(runner: _DpRunner, results_list, rows, Gs, n_g, g_index, q_in
         _, inter = _DpRunner._partition_of(float(cost[t]), fam, int(n_stages[t]), path[t, :fam.S_max])
         G = Gs[int(best_g[t])]
         spaces = results_list[t].spaces
-        solution = [G, []]
-        for i, ((l0, l1), (n, m), ckpt) in enumerate(inter):
-            row = spaces[(g_index[G], q_index[(n, m)])].decode(np.array(int(strategy_row[t, i]))).tolist()
-            row[:6] = [int(x) for x in row[:6]]
-            solution[1].append((((l0, l1), (n, m), ckpt, 0), tuple(row)))
+        solution = [G, [None] * len(inter)]
+        # the stages of a partition mostly share a mesh: one decode per search space
+        by_space: Dict[Tuple[int, int], List[int]] = {}
+        for i, (_, mesh, _) in enumerate(inter):
+            by_space.setdefault((g_index[G], q_index[mesh]), []).append(i)
+        for key, stages in by_space.items():
+            rows = spaces[key].decode(strategy_row[t, stages].astype(np.int64)).tolist()
+            for i, row in zip(stages, rows):
+                row[:6] = [int(x) for x in row[:6]]
+                (l0, l1), mesh, ckpt = inter[i]
+                solution[1][i] = (((l0, l1), mesh, ckpt, 0), tuple(row))
         out.append((float(cost[t]), solution))
     if stats is not None:
         stats["dp_search_s"] = stats.get("dp_search_s", 0.0) + (t_1 - t_0)

@@ -72,17 +72,16 @@ struct Buffer {
 };
 
 struct Workspace {
-  Buffer d_in, d_out, d_scratch, d_req, d_counts, d_values, d_request, d_argmin, d_path, d_rows,
-      d_grad;
-  Buffer h_in, h_out, h_req, h_counts, h_values, h_request, h_path, h_rows, h_grad;
+  Buffer d_in, d_out, d_scratch, d_req, d_counts, d_values, d_request, d_argmin, d_grad;
+  Buffer h_in, h_out, h_req, h_counts, h_values, h_request, h_grad;
   // windows and first scan batch decided on the device
-  Buffer d_win_values, d_win_counts, d_kept, d_meta, d_inst_t, d_inst_row, d_out_first;
-  Buffer h_kept, h_meta, h_out_first;
+  // (requests, window descriptions, DP outputs and kept thresholds in one buffer: one copy back)
+  Buffer d_win_values, d_win_counts, d_inst_t, d_inst_row, d_first;
+  Buffer h_first;
   int select_capacity = 1 << 18;
   Workspace() {
     h_in.pinned = h_out.pinned = h_req.pinned = h_counts.pinned = h_values.pinned =
-        h_request.pinned = h_path.pinned = h_rows.pinned = h_grad.pinned = h_kept.pinned =
-            h_meta.pinned = h_out_first.pinned = true;
+        h_request.pinned = h_grad.pinned = h_first.pinned = true;
   }
 };
 
@@ -242,19 +241,26 @@ struct Search {
   }
 
   // DP instances (g_index[i], tmax[i]) of every family -> ws->h_out as [family][3][n] (best_s
-  // bits, best_sum, stage_max); with `want_path` also the partitions (ws->h_path, family after
+  // bits, best_sum, stage_max); with `want_path` also the partitions (h_path, family after
   // family) and, when strategy tables were given, the strategy rows of their stages
-  // (ws->h_rows, same order without the factor 4).  `sync` false leaves the copies of the
+  // (h_rows, same order without the factor 4).  `sync` false leaves the copies of the
   // outputs queued on the stream for the caller to wait for.
   int run(const std::vector<int32_t> &g_index, const std::vector<float> &tmax, int mode,
           bool want_path, bool sync = true) {
     const int n = (int)tmax.size();
     if (n == 0) return 0;
     const size_t n_out = (size_t)3 * n * n_families;
+    // the partitions and their strategy rows lie behind the outputs: one copy back
+    const size_t n_path = path_offset(n_families, n);
+    const size_t n_back = n_out + (want_path ? n_path + n_path / 4 : 0);
     if (int rc = ws->h_in.reserve(sizeof(float) * 2 * n)) return rc;
     if (int rc = ws->d_in.reserve(sizeof(float) * 2 * n)) return rc;
-    if (int rc = ws->d_out.reserve(sizeof(float) * n_out)) return rc;
-    if (int rc = ws->h_out.reserve(sizeof(float) * n_out)) return rc;
+    if (int rc = ws->d_out.reserve(sizeof(float) * n_back)) return rc;
+    if (int rc = ws->h_out.reserve(sizeof(float) * n_back)) return rc;
+    int32_t *d_paths = reinterpret_cast<int32_t *>(ws->d_out.as<float>() + n_out);
+    int32_t *d_strategy_rows = d_paths + n_path;
+    h_path = reinterpret_cast<const int32_t *>(ws->h_out.as<float>() + n_out);
+    h_rows = h_path + n_path;
     int64_t n_scratch = 1;
     size_t slab = 0;
     for (int f = 0; f < n_families; ++f) {
@@ -265,14 +271,8 @@ struct Search {
                                 (shapes[f].num_devices + 1) * 4);
     }
     if (int rc = ws->d_scratch.reserve(sizeof(float) * (size_t)n_scratch)) return rc;
-    const size_t n_path = path_offset(n_families, n);
-    if (want_path) {
+    if (want_path)
       if (int rc = ws->d_argmin.reserve(sizeof(int32_t) * slab * n)) return rc;
-      if (int rc = ws->d_path.reserve(sizeof(int32_t) * n_path)) return rc;
-      if (int rc = ws->h_path.reserve(sizeof(int32_t) * n_path)) return rc;
-      if (int rc = ws->d_rows.reserve(sizeof(int32_t) * n_path / 4)) return rc;
-      if (int rc = ws->h_rows.reserve(sizeof(int32_t) * n_path / 4)) return rc;
-    }
     float *h_in = ws->h_in.as<float>();
     std::memcpy(h_in, tmax.data(), sizeof(float) * n);
     std::memcpy(h_in + n, g_index.data(), sizeof(int32_t) * n);
@@ -292,7 +292,7 @@ struct Search {
                                d_argmin, ws->d_scratch.as<float>(), stream))
         return rc;
       if (want_path) {
-        int32_t *d_path = ws->d_path.as<int32_t>() + path_offset(f, n);
+        int32_t *d_path = d_paths + path_offset(f, n);
         if (int rc = mist_dp_backtrack(&shape, d_argmin, reinterpret_cast<int32_t *>(d_out), n,
                                        d_path, stream))
           return rc;
@@ -300,19 +300,12 @@ struct Search {
           const int cells = n * shape.max_stages;
           hipLaunchKernelGGL(strategy_rows_kernel, dim3((cells + 63) / 64), dim3(64), 0, stream,
                              *strategy, d_path, reinterpret_cast<int32_t *>(d_out), d_g, n,
-                             shape.max_stages, ws->d_rows.as<int32_t>() + path_offset(f, n) / 4);
+                             shape.max_stages, d_strategy_rows + path_offset(f, n) / 4);
           MIST_HIP_CHECK(hipGetLastError());
         }
       }
     }
-    if (want_path) {
-      MIST_HIP_CHECK(hipMemcpyAsync(ws->h_path.ptr, ws->d_path.ptr, sizeof(int32_t) * n_path,
-                                    hipMemcpyDeviceToHost, stream));
-      if (strategy)
-        MIST_HIP_CHECK(hipMemcpyAsync(ws->h_rows.ptr, ws->d_rows.ptr, sizeof(int32_t) * n_path / 4,
-                                      hipMemcpyDeviceToHost, stream));
-    }
-    MIST_HIP_CHECK(hipMemcpyAsync(ws->h_out.ptr, ws->d_out.ptr, sizeof(float) * n_out,
+    MIST_HIP_CHECK(hipMemcpyAsync(ws->h_out.ptr, ws->d_out.ptr, sizeof(float) * n_back,
                                   hipMemcpyDeviceToHost, stream));
     launches += n_families;
     thresholds_run += (int64_t)n * n_families;
@@ -392,28 +385,34 @@ struct Search {
 
   // The same, and the windows and the first scan batch with it (mist_dp_windows_first_batch +
   // the threshold DP of its instances for every family): one round trip.  Afterwards
-  // ws->h_out holds the bottleneck DP's outputs, ws->h_req the requests ([4][n]: row, lo, hi,
-  // smallest feasible threshold), ws->h_meta the windows' descriptions ([n][8]), ws->h_kept
-  // their kept thresholds and ws->h_out_first the DP outputs of the batch
-  // ([family][3][n * first_chunk]; the instances of window r start at h_meta[r][7]).
+  // ws->h_out holds the bottleneck DP's outputs; first_req the requests ([4][n]: row, lo, hi,
+  // smallest feasible threshold), first_meta the windows' descriptions ([n][8]), first_kept
+  // their kept thresholds and first_out the DP outputs of the batch
+  // ([family][3][n * first_chunk]; the instances of window r start at first_meta[r][7]).
+  const float *first_req = nullptr, *first_kept = nullptr, *first_out = nullptr;
+  const int32_t *first_meta = nullptr;
+  // partitions and strategy rows of the last run with `want_path` (behind its outputs in ws->h_out)
+  const int32_t *h_path = nullptr, *h_rows = nullptr;
   int bottleneck_windows_first_batch(const std::vector<int32_t> &rows, const int32_t *grad_accum,
                                      int n_grad_accum, int window_capacity, int first_chunk) {
     const int n = (int)rows.size(), n_inst = n * first_chunk;
     if (int rc = ws->h_grad.reserve(sizeof(int32_t) * n_grad_accum)) return rc;
     if (int rc = ws->d_grad.reserve(sizeof(int32_t) * n_grad_accum)) return rc;
-    if (int rc = ws->h_req.reserve(sizeof(float) * 4 * n)) return rc;
-    if (int rc = ws->d_req.reserve(sizeof(float) * 4 * n)) return rc;
     if (int rc = ws->d_win_values.reserve(sizeof(float) * (size_t)n * window_capacity)) return rc;
     if (int rc = ws->d_win_counts.reserve(sizeof(int32_t) * (2 + 2 * (size_t)n))) return rc;
-    if (int rc = ws->d_kept.reserve(sizeof(float) * kKeptCapacity)) return rc;
-    if (int rc = ws->h_kept.reserve(sizeof(float) * kKeptCapacity)) return rc;
-    if (int rc = ws->d_meta.reserve(sizeof(int32_t) * 8 * n)) return rc;
-    if (int rc = ws->h_meta.reserve(sizeof(int32_t) * 8 * n)) return rc;
     if (int rc = ws->d_inst_t.reserve(sizeof(float) * n_inst)) return rc;
     if (int rc = ws->d_inst_row.reserve(sizeof(int32_t) * n_inst)) return rc;
     const size_t n_out = (size_t)3 * n_inst * n_families;
-    if (int rc = ws->d_out_first.reserve(sizeof(float) * n_out)) return rc;
-    if (int rc = ws->h_out_first.reserve(sizeof(float) * n_out)) return rc;
+    // one buffer of 4-byte words: [requests 4 n][descriptions 8 n][outputs n_out][kept thresholds]
+    const size_t at_meta = (size_t)4 * n, at_out = at_meta + (size_t)8 * n, at_kept = at_out + n_out;
+    const size_t words = at_kept + kKeptCapacity;
+    if (int rc = ws->d_first.reserve(sizeof(float) * words)) return rc;
+    if (int rc = ws->h_first.reserve(sizeof(float) * words)) return rc;
+    float *d_first = ws->d_first.as<float>(), *h_first = ws->h_first.as<float>();
+    first_req = h_first;
+    first_meta = reinterpret_cast<const int32_t *>(h_first + at_meta);
+    first_out = h_first + at_out;
+    first_kept = h_first + at_kept;
     // the state planes of the batch are the larger need: sized before anything is queued
     int64_t n_scratch = 1;
     for (int f = 0; f < n_families; ++f) {
@@ -427,7 +426,7 @@ struct Search {
                                   hipMemcpyHostToDevice, stream));
     const std::vector<float> zeros(n, 0.0f);
     if (int rc = run(rows, zeros, MIST_DP_BOTTLENECK, false, /*sync=*/false)) return rc;
-    float *d_req = ws->d_req.as<float>();
+    float *d_req = d_first;
     hipLaunchKernelGGL(window_request_kernel, dim3((n + 63) / 64), dim3(64), 0, stream,
                        ws->d_out.as<float>(), n_families, n,
                        reinterpret_cast<const int32_t *>(ws->d_in.as<float>() + n),
@@ -436,35 +435,29 @@ struct Search {
     if (int rc = mist_dp_windows_first_batch(
             select_costs, n, reinterpret_cast<int32_t *>(d_req), d_req + n, d_req + 2 * n,
             d_req + 3 * n, kGap, window_capacity, first_chunk, ws->d_win_values.as<float>(),
-            ws->d_win_counts.as<int32_t>(), ws->d_kept.as<float>(), kKeptCapacity,
-            ws->d_meta.as<int32_t>(), ws->d_inst_t.as<float>(), ws->d_inst_row.as<int32_t>(), stream))
+            ws->d_win_counts.as<int32_t>(), d_first + at_kept, kKeptCapacity,
+            reinterpret_cast<int32_t *>(d_first + at_meta), ws->d_inst_t.as<float>(),
+            ws->d_inst_row.as<int32_t>(), stream))
       return rc;
     for (int f = 0; f < n_families; ++f) {
-      float *d_out = ws->d_out_first.as<float>() + (size_t)f * 3 * n_inst;
+      float *d_out = d_first + at_out + (size_t)f * 3 * n_inst;
       if (int rc = mist_dp_run(&shapes[f], &costs[f], ws->d_inst_t.as<float>(),
                                ws->d_inst_row.as<int32_t>(), n_inst, MIST_DP_THRESHOLD,
                                reinterpret_cast<int32_t *>(d_out), d_out + n_inst, d_out + 2 * n_inst,
                                nullptr, ws->d_scratch.as<float>(), stream))
         return rc;
     }
-    MIST_HIP_CHECK(hipMemcpyAsync(ws->h_req.ptr, ws->d_req.ptr, sizeof(float) * 4 * n,
-                                  hipMemcpyDeviceToHost, stream));
-    MIST_HIP_CHECK(hipMemcpyAsync(ws->h_meta.ptr, ws->d_meta.ptr, sizeof(int32_t) * 8 * n,
-                                  hipMemcpyDeviceToHost, stream));
-    MIST_HIP_CHECK(hipMemcpyAsync(ws->h_kept.ptr, ws->d_kept.ptr, sizeof(float) * kKeptHead,
-                                  hipMemcpyDeviceToHost, stream));
-    MIST_HIP_CHECK(hipMemcpyAsync(ws->h_out_first.ptr, ws->d_out_first.ptr, sizeof(float) * n_out,
+    MIST_HIP_CHECK(hipMemcpyAsync(h_first, d_first, sizeof(float) * (at_kept + kKeptHead),
                                   hipMemcpyDeviceToHost, stream));
     MIST_HIP_CHECK(hipStreamSynchronize(stream));
     ++round_trips;
     // kept thresholds beyond the part that travelled with the rest
-    const int32_t *meta = ws->h_meta.as<int32_t>();
+    const int32_t *meta = first_meta;
     int64_t kept_end = 0;
     for (int r = 0; r < n; ++r)
       if (meta[8 * r + 2] == 0) kept_end = std::max<int64_t>(kept_end, (int64_t)meta[8 * r + 4] + meta[8 * r + 3]);
     if (kept_end > kKeptHead) {
-      MIST_HIP_CHECK(hipMemcpyAsync(ws->h_kept.as<float>() + kKeptHead,
-                                    ws->d_kept.as<float>() + kKeptHead,
+      MIST_HIP_CHECK(hipMemcpyAsync(h_first + at_kept + kKeptHead, d_first + at_kept + kKeptHead,
                                     sizeof(float) * (size_t)(kept_end - kKeptHead),
                                     hipMemcpyDeviceToHost, stream));
       MIST_HIP_CHECK(hipStreamSynchronize(stream));
@@ -754,9 +747,9 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
     if (int rc = S.bottleneck_windows_first_batch(flat_rows, grad_accum, n_grad_accum,
                                                   window_capacity, kFirstChunk))
       return rc;
-    const float *req = S.ws->h_req.as<float>();
-    const int32_t *meta = S.ws->h_meta.as<int32_t>();
-    const float *kept = S.ws->h_kept.as<float>();
+    const float *req = S.first_req;
+    const int32_t *meta = S.first_meta;
+    const float *kept = S.first_kept;
     std::vector<int> undecided;
     std::vector<int32_t> u_rows;
     std::vector<float> u_lo, u_hi;
@@ -844,11 +837,11 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
       // below would have asked for first (kFirstChunk from sc.pos on), the next request of this
       // G grows as after any request
       const int idx = t * n_grad_accum + i, n_first = first_batch[idx];
-      const int at = on_device ? S.ws->h_meta.as<int32_t>()[8 * idx + 7] : 0;
+      const int at = on_device ? S.first_meta[8 * idx + 7] : 0;
       for (int k = 0; k < n_first; ++k) {
         int stages = 0;
         sc.cost.push_back(S.total(at + k, n_flat * kFirstChunk, sc.G, nullptr,
-                                  S.ws->h_out_first.as<float>(), &stages));
+                                  S.first_out, &stages));
         sc.stages.push_back(stages);
       }
       if (n_first > 0) sc.limit = std::min(kMaxChunk, sc.limit * 4);
@@ -1009,10 +1002,10 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
       const size_t per = S.path_ints(family), at = S.path_offset(family, n) + (size_t)k * per;
       out_family[t] = family;
       out_stages[t] = best_s;
-      std::memcpy(out_path + (size_t)t * S_max * 4, S.ws->h_path.as<int32_t>() + at,
+      std::memcpy(out_path + (size_t)t * S_max * 4, S.h_path + at,
                   sizeof(int32_t) * per);
       if (strategy)
-        std::memcpy(out_rows + (size_t)t * S_max, S.ws->h_rows.as<int32_t>() + at / 4,
+        std::memcpy(out_rows + (size_t)t * S_max, S.h_rows + at / 4,
                     sizeof(int32_t) * per / 4);
     }
   }

@@ -594,6 +594,48 @@ def test_argument_checks_reject_before_any_launch():
     items[1].tables.delta[2] = None
     assert batch(2) == -1 and b"null table" in lib.mist_last_error()
     assert batch(0) == -1
+    # the chains of assignment problems, the pre-fill of the cells an assignment reads, the
+    # all-samples entry point and the plan builder check their arguments the same way
+    items[1].tables.delta[2] = 4096
+    G_of = np.array([4, 0], dtype=np.int32)
+    out_f, out_i = np.zeros(16), np.zeros(16, dtype=np.int32)
+    hp = lambda a: ctypes.c_void_p(a.ctypes.data)
+    chains = lambda per_chain, n_chains, G=G_of: lib.mist_mip_solve_chains(
+        ctypes.byref(items), hp(G), per_chain, n_chains, fake, fake, fake, hp(out_f), hp(out_i), hp(out_i), hp(out_i))
+    assert chains(0, 1) == -1 and chains(2, 0) == -1
+    assert chains(2, 1) == -1 and b"grad_accum" in lib.mist_last_error()
+    assert lib.mist_mip_solve_chains(ctypes.byref(items), hp(G_of), 1, 1, None, fake, fake, hp(out_f),
+                                     hp(out_i), hp(out_i), hp(out_i)) == -1
+    regions = np.array([[0, 0, 2, 4, 3, 0], [1, 1, 1, 8, 2, 21]], dtype=np.int32)
+    prefill = lambda r, n=2, L=8: lib.mist_mip_prefill_cells(L, 4, 3, 2, 2, hp(r), fake, n, ctypes.byref(some_tables), None)
+    assert prefill(regions) == -1 and b"null table" in lib.mist_last_error()
+    for v in range(4):
+        some_tables.stable[v] = some_tables.delta[v] = some_tables.index[v] = 4096
+    bad = regions.copy()
+    bad[1, 5] = 20
+    assert prefill(bad) == -1 and b"does not continue" in lib.mist_last_error()
+    bad = regions.copy()
+    bad[0, 1] = 2
+    assert prefill(bad) == -1 and b"outside the tables" in lib.mist_last_error()
+    bad = regions.copy()
+    bad[1, 3] = 9
+    assert prefill(bad) == -1 and b"layer counts" in lib.mist_last_error()
+    assert prefill(regions, n=0) == -1
+    all_samples = lambda n, sample_batch, main_batch, r=rp: lib.mist_intra_stage_eval_samples(
+        pp, fake, 1, fake, 1, fake, 1, None, 0, fake, fake, fake, fake, fake, r, sp_, n, sample_batch,
+        main_batch, ctypes.byref(some_tables), None)
+    assert all_samples(0, 1, 1) == -1 and all_samples(2, 0, 1) == -1
+    assert all_samples(2, _lib.MAX_SAMPLE_BATCH + 1, 1) == -1 and b"sample_batch" in lib.mist_last_error()
+    assert all_samples(2, 2, 3) == -1 and b"main_batch" in lib.mist_last_error()
+    assert all_samples(2, 2, 1, None) == -1
+    request, result = _lib.PlanRequest(), _lib.PlanResult()
+    groups = np.zeros(4, dtype=_lib.GROUP_DTYPE)
+    words = np.zeros(64, dtype=np.int64)
+    plan = lambda req, capacity: lib.mist_plan_groups(
+        req, hp(groups), capacity, hp(words), hp(words), hp(words), hp(words), hp(words), hp(words),
+        hp(words), ctypes.byref(result))
+    assert plan(None, 4) == -1 and b"null" in lib.mist_last_error()
+    assert plan(ctypes.byref(request), 4) == _lib.PLAN_UNSUPPORTED and b"list lengths" in lib.mist_last_error()
 
 
 def test_window_begin_matches_numpy_formulation():

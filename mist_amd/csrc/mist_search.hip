@@ -1865,23 +1865,22 @@ __global__ __launch_bounds__(256) void finalize_kernel(
   // blockIdx.y: 0..p_dim-1 base, p_dim..2*p_dim-1 with_pre, 2*p_dim with_post, 2*p_dim+1 no_pp
   const int P1 = prob.p_dim;
   const int slot = blockIdx.y;
-  if (pair_idx >= n_pairs) return;
   int variant, p;
   if (slot < P1) { variant = 0; p = slot; }
   else if (slot < 2 * P1) { variant = 1; p = slot - P1; }
   else { variant = 2 + (slot - 2 * P1); p = 0; }
   if (p >= g->num_p) return;
-  const PairIndex pc = decode_pair(pair_idx);
+  // A wavefront = the 64 pairs of one tile (the workgroup starts at a multiple of 256 pairs):
+  // what follows up to the chunk loop is the same for all its lanes.  The group's tiles are a
+  // window of the pair list; cells outside were not evaluated.
+  const int lc_tile = pair_idx / MIST_LC_TILE - g->lc_tile_begin, lane = pair_idx % MIST_LC_TILE;
+  if (lc_tile < 0 || lc_tile >= g->n_lc_tiles) return;
+  const PairIndex pc = decode_pair(min(pair_idx, n_pairs - 1));
   const int l = pc.l, c = pc.c;
   // Cells the reference never writes (batched_module_analyzer.py:3021-3023 rebinds the layer
   // mask inside the p == 0 branch, so it also governs base / with_pre for p >= 1; :3103).
-  if (variant <= 1 && p >= 1 && c == l - 1) return;
-  if (variant == 2 && c == l - 1) return;
-  if (variant == 3 && (l != L || c == L - 1)) return;
-
-  // the group's tiles are a window of the pair list; cells outside were not evaluated
-  const int lc_tile = pair_idx / MIST_LC_TILE - g->lc_tile_begin, lane = pair_idx % MIST_LC_TILE;
-  if (lc_tile < 0 || lc_tile >= g->n_lc_tiles) return;
+  const bool written = pair_idx < n_pairs && !(variant <= 1 && p >= 1 && c == l - 1) &&
+                       !(variant == 2 && c == l - 1) && !(variant == 3 && (l != L || c == L - 1));
   const int p_tile = p / MIST_P_TILE;
   int kslot;
   if (variant == 0) kslot = p % MIST_P_TILE;
@@ -1892,14 +1891,28 @@ __global__ __launch_bounds__(256) void finalize_kernel(
       (int64_t)m * n_blocks + (int64_t)block_prefix[gi] + (lc_tile * g->n_p_tiles + p_tile);
   double best = INFINITY;
   int32_t best_row = -1;
-  for (int ch = 0; ch < g->n_chunks; ++ch) {
-    const int64_t slab_at = (first_block + (int64_t)ch * n_tiles) * kSlots * MIST_LC_TILE;
-    if (ch > 0 && partial_index[slab_at] == kSlabUnchanged) continue;  // holds the seeds only
-    const int64_t at = slab_at + (int64_t)kslot * MIST_LC_TILE + lane;
-    const double cost = partial_cost[at];
-    const int32_t row = partial_index[at];
-    take_min(best, best_row, row >= 0, cost, row);
+  // Most chunks leave their seeds as they are and write a mark instead of a slab: the marks of
+  // 64 chunks are read at once, a lane each, and only the slabs that were written are visited
+  // (in chunk order, as a walk over all chunks would).
+  for (int ch0 = 0; ch0 < g->n_chunks; ch0 += 64) {
+    const int ch_mine = ch0 + (int)(threadIdx.x & 63);
+    bool has_slab = false;
+    if (ch_mine < g->n_chunks)
+      has_slab = ch_mine == 0 ||
+                 partial_index[(first_block + (int64_t)ch_mine * n_tiles) * kSlots * MIST_LC_TILE] !=
+                     kSlabUnchanged;
+    unsigned long long todo = __ballot(has_slab);
+    while (todo != 0) {
+      const int ch = ch0 + __ffsll(todo) - 1;
+      todo &= todo - 1;
+      const int64_t at = (first_block + (int64_t)ch * n_tiles) * kSlots * MIST_LC_TILE +
+                         (int64_t)kslot * MIST_LC_TILE + lane;
+      const double cost = partial_cost[at];
+      const int32_t row = partial_index[at];
+      take_min(best, best_row, row >= 0, cost, row);
+    }
   }
+  if (!written) return;
 
   double stable = INFINITY, delta = INFINITY;
   if (best_row >= 0) {

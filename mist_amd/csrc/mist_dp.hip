@@ -49,19 +49,29 @@ constexpr int kDpBatch = 4;  // end layers whose reads a lane of the one-lane-pe
 // Most cells of a plan hold no strategy (no group for that (g, mesh), or nothing fits): their
 // row index is -1 and their costs +inf, so with the index table (may be null) the 16 bytes of
 // such a cell's costs are not read.
-__global__ __launch_bounds__(256) void cost_table_kernel(const double *__restrict__ stable,
-                                                         const double *__restrict__ delta,
-                                                         const int32_t *__restrict__ index,
+// The four tables of a call (base, with_pre, with_post, no_pp) go through one launch: table v
+// owns the workgroups first_block[v] .. first_block[v + 1] - 1.
+struct CostTableJob {
+  const double *stable[4], *delta[4];
+  const int32_t *index[4];
+  float *out[4], *pmin[4];
+  int64_t n_rows[4], rows_per_g[4];
+  unsigned first_block[5];
+};
+__global__ __launch_bounds__(256) void cost_table_kernel(const CostTableJob job,
                                                          const int32_t *__restrict__ grad_accum,
-                                                         int64_t n_rows, int64_t rows_per_g,
-                                                         int row_len, int sample_size, int slot,
-                                                         float *__restrict__ out,
-                                                         float *__restrict__ pmin) {
+                                                         int row_len, int sample_size, int slot) {
   __shared__ float lds[256];
+  const int v = (blockIdx.x >= job.first_block[1]) + (blockIdx.x >= job.first_block[2]) +
+                (blockIdx.x >= job.first_block[3]);
+  const double *__restrict__ stable = job.stable[v], *__restrict__ delta = job.delta[v];
+  const int32_t *__restrict__ index = job.index[v];
+  float *__restrict__ out = job.out[v], *__restrict__ pmin = job.pmin[v];
+  const int64_t n_rows = job.n_rows[v], rows_per_g = job.rows_per_g[v];
   const int seg = min(row_len, 256);  // entries of a row per pass
   const int rows_here = 256 / seg;
   const int local_row = threadIdx.x / seg, j0 = threadIdx.x % seg;
-  const int64_t r = (int64_t)blockIdx.x * rows_here + local_row;
+  const int64_t r = (int64_t)(blockIdx.x - job.first_block[v]) * rows_here + local_row;
   const bool live_row = local_row < rows_here && r < n_rows;
   const float G = live_row ? (float)grad_accum[r / rows_per_g] : 1.0f;
   float carry = INFINITY;
@@ -1401,18 +1411,27 @@ int mist_dp_cost_tables(const MistProblem *problem, const MistOutTables *tables,
     return fail(MIST_E_INVALID, "bad problem extents");
   if (slot < 0 || slot >= S) return fail(MIST_E_INVALID, "slot %d outside [0, %d)", slot, (int)S);
   const int64_t rows_per_g[4] = {Q * P1 * L, Q * P1 * L, Q * L, Q};
+  const int64_t rows_per_block = 256 / std::min<int64_t>(L + 1, 256);
+  CostTableJob job = {};
+  int64_t blocks = 0;
   for (int v = 0; v < 4; ++v) {
     if (!tables->stable[v] || !tables->delta[v] || !d_out[v] || !d_out_pmin[v])
       return fail(MIST_E_INVALID, "table %d is null", v);
-    const int64_t n = Gn * rows_per_g[v];
-    const int64_t rows_per_block = 256 / std::min<int64_t>(L + 1, 256);
-    hipLaunchKernelGGL(cost_table_kernel,
-                       dim3((unsigned)((n + rows_per_block - 1) / rows_per_block)), dim3(256), 0,
-                       (hipStream_t)stream, tables->stable[v], tables->delta[v], tables->index[v],
-                       d_grad_accum, n,
-                       rows_per_g[v], (int)(L + 1), (int)S, slot, d_out[v], d_out_pmin[v]);
-    MIST_HIP_CHECK(hipGetLastError());
+    job.stable[v] = tables->stable[v];
+    job.delta[v] = tables->delta[v];
+    job.index[v] = tables->index[v];
+    job.out[v] = d_out[v];
+    job.pmin[v] = d_out_pmin[v];
+    job.n_rows[v] = Gn * rows_per_g[v];
+    job.rows_per_g[v] = rows_per_g[v];
+    job.first_block[v] = (unsigned)blocks;
+    blocks += (job.n_rows[v] + rows_per_block - 1) / rows_per_block;
   }
+  if (blocks >= (int64_t)1 << 31) return fail(MIST_E_INVALID, "cost tables too large for one launch");
+  job.first_block[4] = (unsigned)blocks;
+  hipLaunchKernelGGL(cost_table_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, job,
+                     d_grad_accum, (int)(L + 1), (int)S, slot);
+  MIST_HIP_CHECK(hipGetLastError());
   return 0;
 }
 

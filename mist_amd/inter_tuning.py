@@ -74,11 +74,14 @@ class _DpRunner:
         problem["num_layers"], problem["p_dim"], problem["sample_size"] = L, P1, S
         problem["num_grad_accum"], problem["num_mesh"] = Gn, Q
         with torch.cuda.device(self.device):
-            self.cost = [
-                torch.empty(tuple(t.shape[:-1]), dtype=torch.float32, device=self.device)
-                for t in dev_tabs.stable
-            ]
-            self.pmin = [torch.empty_like(t) for t in self.cost]
+            # the four cost tables and their running minima: one allocation, eight views
+            shapes = [tuple(t.shape[:-1]) for t in dev_tabs.stable]
+            sizes = [int(np.prod(sh)) for sh in shapes]
+            flat = torch.empty(2 * sum(sizes), dtype=torch.float32, device=self.device)
+            starts = np.concatenate(([0], np.cumsum(sizes + sizes))).tolist()
+            views = [flat[starts[i]:starts[i + 1]].view(shapes[i % 4]) for i in range(8)]
+            self.cost, self.pmin = views[:4], views[4:]
+            self._per_q = [sizes[v] // (Gn * Q) for v in range(4)]  # elements per (g, mesh)
             d_G = getattr(dev_tabs, "grad_accum", None)
             if d_G is None or d_G.numel() != Gn:
                 d_G = torch.tensor(Gs, dtype=torch.int32, device=self.device)
@@ -114,12 +117,12 @@ class _DpRunner:
 
     def _costs_struct(self, q: int = 0):
         """Table pointers starting at mesh ``q`` (strides between g unchanged)."""
-        per_q = [self.cost[v][0, 0].numel() for v in range(4)]
+        per_q = self._per_q
         ptrs = [t.data_ptr() + 4 * q * per_q[v] for v, t in enumerate(self.cost)]
         ptrs += [t.data_ptr() + 4 * q * per_q[v] for v, t in enumerate(self.pmin)]
         cs = _lib.DpCosts(*ptrs)
         for v in range(4):
-            cs.g_stride[v] = self.cost[v][0].numel()
+            cs.g_stride[v] = per_q[v] * self.Q
         return cs
 
     def _prepare_stage_minima(self, fam: _DpFamily) -> None:

@@ -594,50 +594,73 @@ class IntraStageTuner:
             first = last
         return bounds
 
-    def allocate_tables(self, plan: Optional[dict] = None) -> DeviceTables:
-        """Output tables, pre-filled with +inf / -1: all of them, or (``plan`` of a tuner with
-        ``prefill_wanted_cells_only``) the cells ``cells_wanted`` names."""
+    def _table_layout(self):
+        """Shapes of the four variants' tables and where each starts in the flat allocations."""
         Gn = len(self.tp_sizes) * len(self.gradient_accumulation_steps_candidates)
         Qn = len(self.device_mesh_candidates)
         P1, L, S = self.max_possible_pre_saved_micro_batches + 1, self.num_layers, self.sample_size
         shapes = [(Gn, Qn, P1, L, L + 1, S), (Gn, Qn, P1, L, L + 1, S), (Gn, Qn, L, L + 1, S), (Gn, Qn, L + 1, S)]
-        dev = self.device
-        # one allocation and one fill per element type; the tables are views of it
-        sizes = [int(np.prod(s)) for s in shapes]
-        starts = np.concatenate([[0], np.cumsum(sizes)])
-        def views(flat, base):
-            return [flat[base + int(starts[v]):base + int(starts[v + 1])].view(shapes[v]) for v in range(4)]
+        starts = [0]
+        for shape in shapes:
+            starts.append(starts[-1] + int(np.prod(shape)))
+        return shapes, starts
+
+    def _allocate_flat(self, plan: Optional[dict] = None):
+        """The output tables as two flat allocations (float64 costs: stable then delta; int32
+        row indices) with their pre-fill queued on the current stream, and the ``MistOutTables``
+        of pointers into them.  Pre-filled with +inf / -1: everywhere, or (``plan`` of a tuner
+        with ``prefill_wanted_cells_only``) in the cells ``cells_wanted`` names."""
+        shapes, starts = self._table_layout()
+        total, dev = starts[-1], self.device
         wanted = plan.get("wanted") if plan is not None and self.prefill_wanted_cells_only else None
         if wanted is None:
-            costs = torch.full((2 * int(starts[-1]),), float("inf"), dtype=torch.float64, device=dev)
-            index = torch.full((int(starts[-1]),), -1, dtype=torch.int32, device=dev)
-            return DeviceTables(stable=views(costs, 0), delta=views(costs, int(starts[-1])),
-                                index=views(index, 0))
-        costs = torch.empty((2 * int(starts[-1]),), dtype=torch.float64, device=dev)
-        index = torch.empty((int(starts[-1]),), dtype=torch.int32, device=dev)
-        tables = DeviceTables(stable=views(costs, 0), delta=views(costs, int(starts[-1])),
-                              index=views(index, 0))
-        g, q = np.nonzero(wanted[:, :, 0] >= 0)
-        if len(g):
-            n_g = wanted.shape[0]
-            one = np.zeros((len(g), 6), dtype=np.int32)
-            one[:, 0], one[:, 1], one[:, 2:5] = g, q, wanted[g, q]
-            regions = np.tile(one, (len(self.tp_sizes), 1))
-            regions[:, 0] += np.repeat(np.arange(len(self.tp_sizes), dtype=np.int32) * n_g, len(g))
-            nl = (regions[:, 3] - regions[:, 2] + 1).astype(np.int64)
-            rows = 2 * np.minimum(regions[:, 4], P1) * nl + nl + (regions[:, 3] == L)
-            first = np.concatenate(([0], np.cumsum(rows)[:-1]))
-            if int(rows.sum()) >= 2**31:
-                raise ValueError("the cells to pre-fill exceed one launch")
-            regions[:, 5] = first
-            d_regions = torch.from_numpy(regions.reshape(-1)).to(dev)
-            struct = tables.as_struct()
-            rc = _lib.load().mist_mip_prefill_cells(
-                L, P1, S, Qn, Gn, ctypes.c_void_p(regions.ctypes.data), d_regions.data_ptr(),
-                len(regions), ctypes.byref(struct),
-                ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream))
-            _lib.check(rc, "mist_mip_prefill_cells")
-        return tables
+            # one allocation and one fill per element type
+            costs = torch.full((2 * total,), float("inf"), dtype=torch.float64, device=dev)
+            index = torch.full((total,), -1, dtype=torch.int32, device=dev)
+        else:
+            costs = torch.empty((2 * total,), dtype=torch.float64, device=dev)
+            index = torch.empty((total,), dtype=torch.int32, device=dev)
+        struct = _lib.OutTables()
+        cost_ptr, index_ptr = costs.data_ptr(), index.data_ptr()
+        for v in range(4):
+            struct.stable[v] = cost_ptr + 8 * starts[v]
+            struct.delta[v] = cost_ptr + 8 * (total + starts[v])
+            struct.index[v] = index_ptr + 4 * starts[v]
+        if wanted is not None:
+            Gn, Qn, P1, L, _, S = shapes[0]
+            g, q = np.nonzero(wanted[:, :, 0] >= 0)
+            if len(g):
+                n_g = wanted.shape[0]
+                one = np.zeros((len(g), 6), dtype=np.int32)
+                one[:, 0], one[:, 1], one[:, 2:5] = g, q, wanted[g, q]
+                regions = np.tile(one, (len(self.tp_sizes), 1))
+                regions[:, 0] += np.repeat(np.arange(len(self.tp_sizes), dtype=np.int32) * n_g, len(g))
+                nl = (regions[:, 3] - regions[:, 2] + 1).astype(np.int64)
+                rows = 2 * np.minimum(regions[:, 4], P1) * nl + nl + (regions[:, 3] == L)
+                first = np.concatenate(([0], np.cumsum(rows)[:-1]))
+                if int(rows.sum()) >= 2**31:
+                    raise ValueError("the cells to pre-fill exceed one launch")
+                regions[:, 5] = first
+                d_regions = torch.from_numpy(regions.reshape(-1)).to(dev)
+                rc = _lib.load().mist_mip_prefill_cells(
+                    L, P1, S, Qn, Gn, ctypes.c_void_p(regions.ctypes.data), d_regions.data_ptr(),
+                    len(regions), ctypes.byref(struct),
+                    ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream))
+                _lib.check(rc, "mist_mip_prefill_cells")
+        return costs, index, struct
+
+    def _table_views(self, costs: torch.Tensor, index: torch.Tensor) -> DeviceTables:
+        shapes, starts = self._table_layout()
+        total = starts[-1]
+        def views(flat, base):
+            return [flat[base + starts[v]:base + starts[v + 1]].view(shapes[v]) for v in range(4)]
+        return DeviceTables(stable=views(costs, 0), delta=views(costs, total), index=views(index, 0))
+
+    def allocate_tables(self, plan: Optional[dict] = None) -> DeviceTables:
+        """Output tables, pre-filled with +inf / -1: all of them, or (``plan`` of a tuner with
+        ``prefill_wanted_cells_only``) the cells ``cells_wanted`` names."""
+        costs, index, _ = self._allocate_flat(plan)
+        return self._table_views(costs, index)
 
     # ------------------------------------------------------------------ device side
     def upload(self, plan) -> dict:
@@ -699,8 +722,9 @@ class IntraStageTuner:
                 "n_terms_blocks", "n_reduce_blocks", "n_scout_blocks")})
         return out
 
-    def launch(self, plan, dev_plan, tables: DeviceTables, events: Optional[list] = None) -> None:
-        """Enqueues the kernels for every requested sample on the current stream.  With
+    def launch(self, plan, dev_plan, tables, events: Optional[list] = None) -> None:
+        """Enqueues the kernels for every requested sample on the current stream; ``tables`` are
+        the output tables (``DeviceTables``) or the ``MistOutTables`` of their pointers.  With
         ``events`` (a list) the three kernels are launched through their own entry points and
         ``(name, start_event, end_event)`` triples recorded on that stream are appended."""
         if not dev_plan["batches"]:
@@ -713,7 +737,7 @@ class IntraStageTuner:
             streams.append(side)
             side.wait_stream(current)  # the tables are filled on the current stream
         ratios = alpha_ratios(self.sample_size)
-        out = tables.as_struct()
+        out = tables.as_struct() if isinstance(tables, DeviceTables) else tables
         prob_ptr = ctypes.c_void_p(plan["problem"].ctypes.data)
 
         def timed(name, call):
@@ -804,9 +828,11 @@ class IntraStageTuner:
         """Device part only: fresh output tables + kernel launches for an uploaded plan; one
         output per tp size, all resident in the same tables."""
         with torch.cuda.device(self.device):
-            tables = self.allocate_tables(plan)
+            costs, index, struct = self._allocate_flat(plan)
+            self.launch(plan, dev_plan, struct)
+            # (the tensor views of the tables are made while the kernels run)
+            tables = self._table_views(costs, index)
             tables.grad_accum = dev_plan.get("grad_accum")
-            self.launch(plan, dev_plan, tables)
         return self._outputs(plan, tables)
 
     def tune_all(self) -> List[IntraStageTunerOutput]:

@@ -331,6 +331,82 @@ def test_randomized_tune_end_to_end_matches_oracle(seed):
     assert got == want
 
 
+RANDOM_PLAN_SEEDS = [0, 3, 5, 6, 27, 40, 42, 44, 48, 54, 57, 58, 63, 65, 77, 84, 97, 109, 119, 128, 180, 195, 216, 250]
+
+
+def _random_plan(seed):
+    """A seeded random plan over what a configuration file can vary: model shape (hidden size,
+    heads, kv heads, gated MLP, norm, position embedding, tied embeddings, sequence length),
+    cluster shape with slow or fast links between nodes, memory capacity, batch size, offload
+    ratio lists, the tuning switches, the fixed / disabled offload ratios, the pre / post layer
+    strategy, every tuning granularity and several sample sizes."""
+    rng = np.random.default_rng(190000 + seed)
+    slow = bool(rng.integers(0, 3) > 0)
+    gg = []
+    for entry in range(16):
+        lo, hi = (8, 500) if (entry < 4 or not slow) else (0.3, 6)  # entries 4..15: several nodes
+        if slow and entry < 4 and rng.integers(0, 2):
+            lo, hi = 2, 20
+        gg += [float(rng.uniform(lo, hi)), float(rng.uniform(2e-6, 8e-5))]
+    nodes, gpn = [(1, 2), (1, 4), (2, 2), (2, 4), (1, 8), (4, 2), (2, 8)][int(rng.integers(0, 7))]
+    granularity = str(rng.choice(["inter-stage", "inter-stage", "uniform-device-pp", "uniform-pp",
+                                  "uniform-device-pp-mip", "uniform-device-pp-mip"]))
+    samples = 1 if granularity != "uniform-device-pp-mip" else int(rng.choice([1, 2, 3, 5]))
+    ratios = [float(x) for x in np.linspace(0, 1, int(rng.choice([2, 3, 5])))]
+    hidden, heads = int(rng.choice([1024, 2048, 2048, 4096])), int(rng.choice([8, 16, 32]))
+    overrides = dict(
+        hardware__gpu_gpu_comm_params=gg,
+        hardware__interference_model_params=[float(x) for x in rng.uniform(1.0, 3.0, size=28)],
+        hardware__cpu_gpu_comm_params=[float(rng.uniform(20, 55)), float(rng.uniform(5e-6, 2e-5))],
+        hardware__gpu_cpu_comm_params=[float(rng.uniform(20, 55)), float(rng.uniform(5e-6, 2e-5))],
+        hardware__memory_capacity=float(rng.choice([2.5, 3.0, 5.0, 8.0, 12.0, 40.0])),
+        hardware__num_nodes=nodes, hardware__num_gpus_per_node=gpn,
+        training__global_batch_size=int(rng.choice([8, 16, 32, 64, 24, 48])),
+        training__max_sequence_length=int(rng.choice([1024, 2048, 4096])),
+        tuning__tuning_granularity=granularity, tuning__sample_size=samples,
+        tuning__zero_2_and_3_enabled=bool(rng.integers(0, 2)),
+        tuning__activation_checkpointing_tuning_enabled=bool(rng.integers(0, 4) > 0),
+        tuning__state_offloading_enabled=bool(rng.integers(0, 4) > 0),
+        tuning__activation_offloading_enabled=bool(rng.integers(0, 4) > 0),
+        tuning__pre_post_strategy=str(rng.choice(["dp", "intra-node-tp-with-ore", "intra-node-tp-without-ore"])),
+        tuning__search_space__offloading_ratio_candidates=ratios,
+        tuning__search_space__sparse_offloading_ratio_candidates=ratios,
+        tuning__search_space__batch_size_candidates=[1, 2, 3, 4, 6, 8],
+        model__use_flash_attn=bool(rng.integers(0, 2)),
+        model__hidden_size=hidden, model__num_attention_heads=heads,
+        model__intermediate_size=int(hidden * rng.choice([2, 4])),
+        model__mlp_type=str(rng.choice(["mlp", "gated_mlp"])),
+        model__normalization=str(rng.choice(["layernorm", "rmsnorm"])),
+        model__position_embedding_type=str(rng.choice(["absolute", "rope"])),
+        model__tie_word_embeddings=bool(rng.integers(0, 2)),
+        model__num_heads_kv=(None if rng.integers(0, 2) else int(heads // rng.choice([1, 2, 4]))),
+        enable_advanced_opt_in_first_block=bool(rng.integers(0, 2)),
+        disable_tp_tuning=bool(rng.integers(0, 5) == 0),
+    )
+    for key in ("disable_wo_tuning", "disable_go_tuning", "disable_oo_tuning"):
+        if rng.integers(0, 4) == 0:
+            overrides[key] = True
+    if rng.integers(0, 5) == 0:
+        overrides["fixed_ao_ratio"] = float(rng.choice(ratios))
+    if rng.integers(0, 6) == 0:
+        overrides["fixed_oo_ratio"] = float(rng.choice(ratios))
+    return tiny_plan(1, layers=int(rng.integers(6, 14)), **overrides)
+
+
+@pytest.mark.parametrize("seed", RANDOM_PLAN_SEEDS)
+def test_randomized_plans_of_every_granularity_match_oracle(seed):
+    """Cost and strategy of random plans equal the oracle's.  The seeds were picked by what the
+    oracle answers: mostly pipelines of two to four stages, some single stages, some plans that
+    fit nowhere."""
+    from mist_amd.tune_one_case import tune
+    from oracle.tune import tune as oracle_tune
+
+    cfg, tables = _random_plan(seed)
+    got = tune(cfg)
+    want = oracle_tune(cfg, tables)
+    assert got == want
+
+
 def test_plan1_end_to_end():
     from mist_amd.tune_one_case import tune
     from oracle.tune import tune as oracle_tune

@@ -130,9 +130,11 @@ int mist_dp_select_candidates(const MistDpCosts *costs, int n_requests, const in
  * per request sorts them, finds the start of the walk as mist_dp_window_begin does (the fetch is
  * never open below) for the smallest feasible threshold d_start[r] (+inf: nothing feasible, the
  * request is skipped), walks them with the gap rule and appends the kept thresholds, ascending,
- * to d_kept; the first `first_chunk` kept thresholds at or above d_start[r] become DP instances,
- * appended to d_inst_tmax / d_inst_row[n_requests * first_chunk] (row -1 in the unused tail:
- * mist_dp_run skips such instances and reports them infeasible).
+ * to d_kept; of the n_avail kept thresholds at or above d_start[r], min(first_chunk, n_avail)
+ * become DP instances, instance k at the mist_dp_first_batch_index(k, ...)-th of them: all if
+ * they fit, else the first `first_lead` ones and the rest of the batch spread evenly up to the
+ * last one.  The instances are appended to d_inst_tmax / d_inst_row[n_requests * first_chunk]
+ * (row -1 in the unused tail: mist_dp_run skips such instances and reports them infeasible).
  *   window_capacity : candidates a request may select (a power of two in [128, 8192])
  *   d_values[n_requests][window_capacity], d_counts[2 + 2 n_requests] : work space
  *   d_meta[n_requests][8] : selected, candidates above d_hi[r], status, kept, offset of the
@@ -144,10 +146,13 @@ int mist_dp_select_candidates(const MistDpCosts *costs, int n_requests, const in
  * (mist_dp_select_candidates + mist_dp_window_begin). */
 int mist_dp_windows_first_batch(const MistDpCosts *costs, int n_requests, const int32_t *d_rows,
                                 const float *d_lo, const float *d_hi, const float *d_start,
-                                double gap, int window_capacity, int first_chunk, float *d_values,
-                                int32_t *d_counts, float *d_kept, int kept_capacity,
-                                int32_t *d_meta, float *d_inst_tmax, int32_t *d_inst_row,
-                                void *stream);
+                                double gap, int window_capacity, int first_chunk, int first_lead,
+                                float *d_values, int32_t *d_counts, float *d_kept,
+                                int kept_capacity, int32_t *d_meta, float *d_inst_tmax,
+                                int32_t *d_inst_row, void *stream);
+/* Host function: index (among the n_avail kept thresholds of a window from its first feasible
+ * one on) of instance k of that window's first scan batch; -1 for k outside the batch. */
+int mist_dp_first_batch_index(int k, int n_avail, int first_chunk, int first_lead);
 
 /* Runs n_tmax DP instances at once: one launch per stage count with a thread (or a team of
  * lanes) per (instance, start layer, devices) state, or, for large batches whose state planes fit

@@ -217,7 +217,9 @@ _DP_SIGNATURES = {
     "mist_dp_windows_first_batch": (
         ctypes.c_int,
         [ctypes.POINTER(DpCosts), ctypes.c_int, _VP, _VP, _VP, _VP, ctypes.c_double, ctypes.c_int,
-         ctypes.c_int, _VP, _VP, _VP, ctypes.c_int, _VP, _VP, _VP, _VP]),
+         ctypes.c_int, ctypes.c_int, _VP, _VP, _VP, ctypes.c_int, _VP, _VP, _VP, _VP]),
+    "mist_dp_first_batch_index": (
+        ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "mist_dp_window_begin": (
         ctypes.c_int,
         [_VP, ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_float, ctypes.c_double, _VP]),

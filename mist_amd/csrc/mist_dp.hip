@@ -231,6 +231,18 @@ __host__ __device__ inline int window_walk_start(const float *ascending, int n, 
   return first;
 }
 
+// Which kept threshold (counted from the first one at or above the smallest feasible threshold)
+// instance k of a window's first scan batch runs, when n_avail of them are there: all of them if
+// they fit the batch; else the first `first_lead` ones, then the rest of the batch spread evenly
+// up to the window's last one (probes: the stage-cost sum at a later threshold bounds the sums at
+// every earlier one from below, which lets the scan pass thresholds that cannot improve its best).
+__host__ __device__ __forceinline__ int dp_first_batch_index(int k, int n_avail, int first_chunk,
+                                                             int first_lead) {
+  if (n_avail <= first_chunk || k < first_lead || first_lead >= first_chunk) return k;
+  const int spread = first_chunk - first_lead;
+  return first_lead + (int)(((int64_t)(k - first_lead + 1) * (n_avail - first_lead)) / spread) - 1;
+}
+
 constexpr int kWindowThreads = 1024;
 // status of a window walked on the device (meta[r][2])
 constexpr int kWindowOk = 0, kWindowNone = 1, kWindowOverflow = 2, kWindowNoStart = 3,
@@ -239,9 +251,9 @@ constexpr int kWindowOk = 0, kWindowNone = 1, kWindowOverflow = 2, kWindowNoStar
 // One workgroup per request of a per-request candidate selection: sorts the request's values
 // (bitonic, in LDS), walks them with the gap rule from the certain start below `start[r]` (the
 // smallest feasible threshold; +inf = nothing feasible, the request is skipped), appends the kept
-// thresholds to one list (kept_out, cursor in counts[0]) and lays out the first scan batch: the
-// first `first_chunk` kept thresholds at or above start[r] as DP instances, appended to
-// inst_tmax / inst_row (cursor in counts[1 + 2 n_requests]; the caller pre-fills inst_row with
+// thresholds to one list (kept_out, cursor in counts[0]) and lays out the first scan batch: up to
+// `first_chunk` kept thresholds at or above start[r] (dp_first_batch_index) as DP instances,
+// appended to inst_tmax / inst_row (cursor in counts[1 + 2 n_requests]; the caller pre-fills inst_row with
 // -1, so that the live instances are the first workgroups of the DP launch and the empty slots
 // its tail).
 // meta[r][8] = (selected, above hi, status, kept, offset in kept_out, kept below start, instances,
@@ -256,9 +268,9 @@ constexpr int kWindowOk = 0, kWindowNone = 1, kWindowOverflow = 2, kWindowNoStar
 __global__ __launch_bounds__(kWindowThreads) void window_walk_kernel(
     const float *__restrict__ values, int capacity, int32_t *__restrict__ counts,
     const int32_t *__restrict__ rows, const float *__restrict__ lo,
-    const float *__restrict__ start, double gap, int first_chunk, float *__restrict__ kept_out,
-    int kept_capacity, int32_t *__restrict__ meta, float *__restrict__ inst_tmax,
-    int32_t *__restrict__ inst_row) {
+    const float *__restrict__ start, double gap, int first_chunk, int first_lead,
+    float *__restrict__ kept_out, int kept_capacity, int32_t *__restrict__ meta,
+    float *__restrict__ inst_tmax, int32_t *__restrict__ inst_row) {
   extern __shared__ float win_lds[];
   float *v = win_lds;                                               // [capacity]
   uint8_t *keep = reinterpret_cast<uint8_t *>(win_lds + capacity);  // [capacity]
@@ -384,11 +396,15 @@ __global__ __launch_bounds__(kWindowThreads) void window_walk_kernel(
     for (int i = i0; i < i1; ++i) {
       if (!keep[i]) continue;
       kept_out[kept_base + at] = v[i];
-      if (at >= pos && at < pos + first_chunk) {
-        inst_tmax[inst_base + at - pos] = v[i];
-        inst_row[inst_base + at - pos] = rows[r];
-      }
       ++at;
+    }
+  }
+  __syncthreads();  // (the workgroup's own writes to kept_out are visible to it behind the barrier)
+  if (status == kWindowOk) {
+    for (int k = tid; k < n_inst; k += blockDim.x) {
+      inst_tmax[inst_base + k] =
+          kept_out[kept_base + pos + dp_first_batch_index(k, n_kept - pos, first_chunk, first_lead)];
+      inst_row[inst_base + k] = rows[r];
     }
   }
   if (tid == 0) {
@@ -1535,12 +1551,17 @@ int mist_dp_select_candidates(const MistDpCosts *costs, int n_requests, const in
   return 0;
 }
 
+int mist_dp_first_batch_index(int k, int n_avail, int first_chunk, int first_lead) {
+  if (k < 0 || first_chunk < 1 || first_lead < 1 || k >= std::min(first_chunk, n_avail)) return -1;
+  return dp_first_batch_index(k, n_avail, first_chunk, first_lead);
+}
+
 int mist_dp_windows_first_batch(const MistDpCosts *costs, int n_requests, const int32_t *d_rows,
                                 const float *d_lo, const float *d_hi, const float *d_start,
-                                double gap, int window_capacity, int first_chunk, float *d_values,
-                                int32_t *d_counts, float *d_kept, int kept_capacity,
-                                int32_t *d_meta, float *d_inst_tmax, int32_t *d_inst_row,
-                                void *stream) {
+                                double gap, int window_capacity, int first_chunk, int first_lead,
+                                float *d_values, int32_t *d_counts, float *d_kept,
+                                int kept_capacity, int32_t *d_meta, float *d_inst_tmax,
+                                int32_t *d_inst_row, void *stream) {
   if (!costs || !costs->costs || !costs->costs_pre || !costs->costs_post)
     return fail(MIST_E_INVALID, "null cost tables");
   if (n_requests <= 0 || n_requests > 65535)
@@ -1553,6 +1574,7 @@ int mist_dp_windows_first_batch(const MistDpCosts *costs, int n_requests, const 
   if (first_chunk < 1 || kept_capacity < 1 || (int64_t)n_requests * first_chunk > 65535)
     return fail(MIST_E_INVALID, "first_chunk %d x %d requests outside [1, 65535] / empty kept list",
                 first_chunk, n_requests);
+  if (first_lead < 1) return fail(MIST_E_INVALID, "first_lead %d < 1", first_lead);
   hipStream_t st = (hipStream_t)stream;
   MIST_HIP_CHECK(hipMemsetAsync(d_counts, 0, sizeof(int32_t) * (2 + 2 * (size_t)n_requests), st));
   MIST_HIP_CHECK(hipMemsetAsync(d_inst_row, 0xFF, sizeof(int32_t) * (size_t)n_requests * first_chunk, st));
@@ -1564,8 +1586,8 @@ int mist_dp_windows_first_batch(const MistDpCosts *costs, int n_requests, const 
   MIST_HIP_CHECK(hipGetLastError());
   const size_t lds = (size_t)window_capacity * (sizeof(float) + sizeof(uint8_t));
   hipLaunchKernelGGL(window_walk_kernel, dim3(n_requests), dim3(kWindowThreads), lds, st, d_values,
-                     window_capacity, d_counts, d_rows, d_lo, d_start, gap, first_chunk, d_kept,
-                     kept_capacity, d_meta, d_inst_tmax, d_inst_row);
+                     window_capacity, d_counts, d_rows, d_lo, d_start, gap, first_chunk, first_lead,
+                     d_kept, kept_capacity, d_meta, d_inst_tmax, d_inst_row);
   MIST_HIP_CHECK(hipGetLastError());
   return 0;
 }

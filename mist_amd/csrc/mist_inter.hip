@@ -39,7 +39,10 @@ using mist::fail;
 
 namespace {
 
-constexpr int kFirstChunk = 48;   // thresholds per G in the first speculative batch
+constexpr int kFirstChunk = 48;   // thresholds per G in the first speculative batch ...
+constexpr int kFirstLead = 16;    // ... of a window longer than that: the first ones, the rest spread
+constexpr int kProbes = 16;       // thresholds spread over what a later request does not reach
+constexpr double kFloorSlack = 1e-6;  // relative slack of the bound that lets the scan pass thresholds
 constexpr int kMaxChunk = 4096;   // most thresholds per G in one batch
 constexpr double kGap = 1e-6;     // inter_tuning.py:177
 constexpr int kSelectHead = 1 << 16;  // selected candidates that travel with the counts of a fetch
@@ -326,10 +329,14 @@ struct Search {
   }
   // smallest family total (the first family wins ties); *family = the one that attains it
   double total(int i, int n, int G, int *family = nullptr, const float *out = nullptr,
-               int *stages = nullptr) const {
+               int *stages = nullptr, double *min_sum = nullptr) const {
     double best = kInf;
+    if (min_sum) *min_sum = kInf;
     for (int f = 0; f < n_families; ++f) {
       const double c = total_of(f, i, n, G, out);
+      if (min_sum && c < kInf)  // smallest stage-cost sum of any family that is feasible here
+        *min_sum = std::min(*min_sum,
+                            (double)((out ? out : ws->h_out.as<float>()) + (size_t)f * 3 * n)[n + i]);
       if (c < best) {
         best = c;
         if (family) *family = f;
@@ -434,7 +441,8 @@ struct Search {
     MIST_HIP_CHECK(hipGetLastError());
     if (int rc = mist_dp_windows_first_batch(
             select_costs, n, reinterpret_cast<int32_t *>(d_req), d_req + n, d_req + 2 * n,
-            d_req + 3 * n, kGap, window_capacity, first_chunk, ws->d_win_values.as<float>(),
+            d_req + 3 * n, kGap, window_capacity, first_chunk, kFirstLead,
+            ws->d_win_values.as<float>(),
             ws->d_win_counts.as<int32_t>(), d_first + at_kept, kKeptCapacity,
             reinterpret_cast<int32_t *>(d_first + at_meta), ws->d_inst_t.as<float>(),
             ws->d_inst_row.as<int32_t>(), stream))
@@ -584,14 +592,35 @@ struct Search {
 };
 
 // Replay state of inter_stage_tune_with_fixed_grad_accumu (inter_tuning.py:163-217) for one G.
+//
+// The reference runs the DP at every kept threshold below best / G.  Most of those runs change
+// nothing, and for many that can be told from the outcome at a LATER threshold j: the DP at
+// threshold i returns the partition the DP at i - 1 returned unless that one uses a stage cost
+// above threshold i - 1 (same visiting order, strict "<": the first best candidate of a state
+// among more candidates, if it is one of the fewer, is the first best among those too), and the
+// same partition gives the same total, which is no improvement.  A partition that is new at i
+// has a stage above threshold i - 1 and stage costs that sum to no less than the smallest sum at
+// j >= i (the admissible costs only grow with the threshold; float32 adds are monotone), so its
+// total is at least sum(j) + (G - 1) threshold(i - 1).  While that is no smaller than the running
+// best, no threshold up to j improves it and the scan passes them without their outcomes.
+struct Outcome {
+  double cost = kInf;  // total of the DP's partition, inf = infeasible
+  double sum = kInf;   // smallest stage-cost sum of a feasible family
+  int stages = 0;
+};
 struct Scan {
   int G = 1;
   Window *w = nullptr;
-  size_t pos = 0, have_lo = 0;
-  std::vector<double> cost;  // DP outcome per computed threshold, inf = infeasible
-  std::vector<int> stages;   // ... and the stage count of its partition
+  size_t pos = 0;    // next threshold the sequential scan looks at
+  size_t first = 0;  // the first one at or above the smallest feasible threshold
+  std::map<size_t, Outcome> known;  // DP outcomes by index of the kept threshold
   int limit = kFirstChunk;
   size_t n_kept() const { return w ? w->kept.size() : 0; }
+  // lower bound of the total of any improvement at thresholds pos..j, from the sum at j
+  double floor_total(size_t at, double sum_later) const {
+    const double prev = at > first ? (double)w->kept[at - 1] : (double)w->start_value;
+    return (sum_later + (double)(G - 1) * prev) * (1.0 - kFloorSlack);
+  }
 };
 
 }  // namespace
@@ -832,17 +861,16 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
       if (sc.w)
         sc.pos = (size_t)(std::lower_bound(w.kept.begin(), w.kept.end(), w.start_value) -
                           w.kept.begin());
-      sc.have_lo = sc.pos;  // everything below is infeasible: the scan passes it unchanged
+      sc.first = sc.pos;  // everything below is infeasible: the scan passes it unchanged
       // the results of the first batch, when the device has run it: the thresholds the scan
-      // below would have asked for first (kFirstChunk from sc.pos on), the next request of this
-      // G grows as after any request
+      // below would have asked for first, the next request of this G grows as after any request
       const int idx = t * n_grad_accum + i, n_first = first_batch[idx];
       const int at = on_device ? S.first_meta[8 * idx + 7] : 0;
+      const int n_avail = (int)(sc.n_kept() - sc.first);
       for (int k = 0; k < n_first; ++k) {
-        int stages = 0;
-        sc.cost.push_back(S.total(at + k, n_flat * kFirstChunk, sc.G, nullptr,
-                                  S.first_out, &stages));
-        sc.stages.push_back(stages);
+        Outcome o;
+        o.cost = S.total(at + k, n_flat * kFirstChunk, sc.G, nullptr, S.first_out, &o.stages, &o.sum);
+        sc.known[sc.first + (size_t)mist_dp_first_batch_index(k, n_avail, kFirstChunk, kFirstLead)] = o;
       }
       if (n_first > 0) sc.limit = std::min(kMaxChunk, sc.limit * 4);
     }
@@ -865,36 +893,86 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
     for (;;) {
       if (!reach(sc, sc.pos, best_cost)) return true;
       if (sc.w->scaled[sc.pos] >= best_cost) return true;  // inter_tuning.py:196-197
-      if (sc.pos >= sc.have_lo + sc.cost.size()) return false;  // needs more DP results
-      const double c = sc.cost[sc.pos - sc.have_lo];
-      if (c < best_cost) {
-        best_cost = c;
+      const auto later = sc.known.lower_bound(sc.pos);
+      if (later != sc.known.end() && sc.floor_total(sc.pos, later->second.sum) >= best_cost) {
+        sc.pos = later->first + 1;  // nothing up to there improves the best
+        continue;
+      }
+      if (later == sc.known.end() || later->first != sc.pos) return false;  // needs more DP results
+      const Outcome &o = later->second;
+      if (o.cost < best_cost) {
+        best_cost = o.cost;
         best_t = sc.w->kept[sc.pos];
-        best_stages = sc.stages[sc.pos - sc.have_lo];
+        best_stages = o.stages;
         improved = true;
       }
       ++sc.pos;
     }
   };
-  // dry run of replay under the bound `best_cost`: true if the computed results do not suffice
-  auto runs_out = [&](Scan &sc, double best_cost) -> bool {
+  // Dry run of replay under the bound `best_cost` (the running best when this G is reached is no
+  // larger, so the true scan passes no fewer thresholds): the thresholds whose outcomes it would
+  // miss, at most sc.limit of them (it goes on as if they improved nothing), and, if it stops at
+  // that limit, kProbes more spread over what it did not get to.  A scan without any outcome
+  // asks for its first batch (mist_dp_first_batch_index over everything below the bound).
+  auto wanted = [&](Scan &sc, double best_cost, std::vector<size_t> *out) {
+    out->clear();
+    if (!sc.w) return;
+    auto stop_of = [&](double bound) {
+      return (size_t)(std::lower_bound(sc.w->scaled.begin(), sc.w->scaled.end(), bound) -
+                      sc.w->scaled.begin());
+    };
+    if (sc.known.empty()) {
+      reach(sc, sc.pos + (size_t)kFirstChunk, best_cost);
+      if (rc_inner) return;
+      const size_t stop = stop_of(best_cost);
+      if (stop <= sc.pos) return;
+      const int n_avail = (int)(stop - sc.pos), n = std::min(kFirstChunk, n_avail);
+      for (int k = 0; k < n; ++k)
+        out->push_back(sc.pos + (size_t)mist_dp_first_batch_index(k, n_avail, kFirstChunk, kFirstLead));
+      return;
+    }
     size_t pos = sc.pos;
-    const size_t hi = sc.have_lo + sc.cost.size();
+    int budget = sc.limit;
+    bool cut = false;
     while (reach(sc, pos, best_cost)) {
-      if (sc.w->scaled[pos] >= best_cost) return false;
-      if (pos >= hi) return true;
-      best_cost = std::min(best_cost, sc.cost[pos - sc.have_lo]);
+      if (sc.w->scaled[pos] >= best_cost) break;
+      const auto later = sc.known.lower_bound(pos);
+      if (later != sc.known.end() && sc.floor_total(pos, later->second.sum) >= best_cost) {
+        pos = later->first + 1;
+        continue;
+      }
+      if (later != sc.known.end() && later->first == pos) {
+        best_cost = std::min(best_cost, later->second.cost);
+      } else {
+        if (budget == 0) {
+          cut = true;
+          break;
+        }
+        out->push_back(pos);
+        --budget;
+      }
       ++pos;
     }
-    return false;
+    if (rc_inner || !cut) return;
+    const size_t stop = stop_of(best_cost);
+    size_t last = 0;
+    for (int k = 0; k < kProbes && stop > pos; ++k) {
+      const size_t step = ((size_t)(k + 1) * (stop - pos)) / kProbes;
+      if (step == 0) continue;
+      const size_t at = pos + step - 1;
+      if ((k > 0 && at <= last) || sc.known.count(at)) continue;
+      out->push_back(at);
+      last = at;
+    }
   };
   struct Span {
-    int t, i, n;
+    int t, i, first, n;  // the indices of the span: req_at[first .. first + n)
   };
   for (;;) {
     std::vector<int32_t> req_g;
     std::vector<float> req_t;
     std::vector<int> req_G;
+    std::vector<size_t> req_at, ask;
     std::vector<Span> spans;
     bool all_done = true;
     for (int t = 0; t < n_instances; ++t) {
@@ -917,28 +995,17 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
       if (ch.current < ch.scans.size()) all_done = false;
       for (size_t i = ch.current; i < ch.scans.size(); ++i) {
         Scan &sc = ch.scans[i];
-        if (i > ch.current && !runs_out(sc, ch.best_cost)) {
-          if (rc_inner) return rc_inner;
-          continue;
-        }
+        wanted(sc, ch.best_cost, &ask);
         if (rc_inner) return rc_inner;
+        if (ask.empty()) continue;
         // the range grows fourfold every time the same G asks again
-        const size_t a = sc.have_lo + sc.cost.size();
-        reach(sc, a + sc.limit, ch.best_cost);
-        if (rc_inner) return rc_inner;
-        size_t stop = 0;
-        if (sc.w)
-          stop = (size_t)(std::lower_bound(sc.w->scaled.begin(), sc.w->scaled.end(), ch.best_cost) -
-                          sc.w->scaled.begin());
-        const size_t b = std::max(a, std::min(stop, a + sc.limit));
-        if (b > a) {
-          sc.limit = std::min(kMaxChunk, sc.limit * 4);
-          for (size_t k = a; k < b; ++k) {
-            req_g.push_back(rows[t * n_grad_accum + (int)i]);
-            req_t.push_back(sc.w->kept[k]);
-            req_G.push_back(sc.G);
-          }
-          spans.push_back(Span{t, (int)i, (int)(b - a)});
+        sc.limit = std::min(kMaxChunk, sc.limit * 4);
+        spans.push_back(Span{t, (int)i, (int)req_at.size(), (int)ask.size()});
+        for (size_t at : ask) {
+          req_g.push_back(rows[t * n_grad_accum + (int)i]);
+          req_t.push_back(sc.w->kept[at]);
+          req_G.push_back(sc.G);
+          req_at.push_back(at);
         }
       }
     }
@@ -946,15 +1013,13 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
     if (spans.empty()) return fail(MIST_E_INVALID, "inter-stage scan made no progress");
     if (int rc = S.run(req_g, req_t, MIST_DP_THRESHOLD, false)) return rc;
     const int n = (int)req_t.size();
-    int off = 0;
     for (const Span &sp : spans) {
       Scan &sc = chains[sp.t].scans[sp.i];
-      for (int k = 0; k < sp.n; ++k) {
-        int stages = 0;
-        sc.cost.push_back(S.total(off + k, n, req_G[off + k], nullptr, nullptr, &stages));
-        sc.stages.push_back(stages);
+      for (int k = sp.first; k < sp.first + sp.n; ++k) {
+        Outcome o;
+        o.cost = S.total(k, n, req_G[k], nullptr, nullptr, &o.stages, &o.sum);
+        sc.known[req_at[k]] = o;
       }
-      off += sp.n;
     }
   }
 

@@ -10,7 +10,9 @@ ties are the reference's.  Exact shortcuts: (1) thresholds below the smallest fe
 not run one by one; that point comes from one bottleneck (min-max) DP per G (an infeasible
 run changes nothing in the reference's scan); (2) thresholds are computed ahead speculatively
 under a bound on the running best that the sequential scan is certain to have reached, and the
-replay asks for more wherever it runs out, so a wrong guess costs time, never correctness.
+replay asks for more wherever it runs out, so a wrong guess costs time, never correctness;
+(3) thresholds that cannot improve the running best are passed without their outcomes, by a
+lower bound of their totals from the stage-cost sum at a later threshold (``_Scan``).
 
 The reference's DP reads ``costs / costs_with_pre / ...`` fields that its intra tuner no longer
 emits; the cost tables are built from the stable / delta tables as
@@ -20,6 +22,7 @@ accepts them.
 """
 from __future__ import annotations
 
+import bisect
 import ctypes
 import time
 from typing import Dict, List, Optional, Tuple
@@ -30,7 +33,10 @@ import torch
 from . import _lib
 from .intra_tuning import IntraStageTunerOutput
 
-FIRST_CHUNK = 48  # thresholds per G in the first speculative scan launch
+FIRST_CHUNK = 48  # thresholds per G in the first speculative scan launch ...
+FIRST_LEAD = 16   # ... of a window longer than that: the first ones, the rest spread up to its last
+PROBES = 16       # thresholds spread over what a later request does not reach
+FLOOR_SLACK = 1e-6  # relative slack of the bound that lets the scan pass thresholds
 MAX_CHUNK = 4096  # most thresholds per G in one launch
 GAP = 1e-6        # inter_tuning.py:177
 _SELECT_HEAD = 1 << 16  # selected candidates read back together with their counts
@@ -484,15 +490,27 @@ class _Window:
 
 class _Scan:
     """Replay state of ``inter_stage_tune_with_fixed_grad_accumu`` (inter_tuning.py:163-217) for
-    one G: ``pos`` = next threshold the sequential scan would look at, ``results`` = DP outcomes
-    already computed for tmax[lo : lo + len]."""
+    one G: ``pos`` = next threshold the sequential scan would look at, ``known`` = DP outcomes
+    (total, smallest family sum) by index of the kept threshold.
 
-    def __init__(self, G: int, window: Optional[_Window], first: int):
+    The reference runs the DP at every kept threshold below ``best / G``.  Most of those runs
+    change nothing, and for many that can be told from the outcome at a LATER threshold j: the
+    DP at threshold i returns the partition the DP at i - 1 returned unless that one uses a
+    stage cost above threshold i - 1 (same visiting order, strict "<"), and the same partition
+    gives the same total, which is no improvement.  A partition that is new at i has a stage
+    above threshold i - 1 and stage costs that sum to no less than the smallest sum at j >= i
+    (the admissible costs only grow with the threshold; float32 adds are monotone), so its total
+    is at least ``sum(j) + (G - 1) * threshold(i - 1)``.  While that is no smaller than the
+    running best, no threshold up to j improves it and the scan passes them."""
+
+    def __init__(self, G: int, window: Optional[_Window], first: int, first_index=None):
         self.G, self.window = G, window
         self.pos = first          # everything below is infeasible: the scan passes it unchanged
-        self.have_lo = first
-        self.cost = np.empty(0, dtype=np.float64)  # DP outcome per computed threshold, inf = infeasible
+        self.first = first
+        self.known: Dict[int, Tuple[float, float]] = {}
+        self.keys: List[int] = []  # sorted indices of ``known``
         self.limit = FIRST_CHUNK
+        self.first_index = first_index  # mist_dp_first_batch_index
 
     @property
     def tmax(self) -> np.ndarray:
@@ -510,66 +528,80 @@ class _Scan:
             w.extend(best_cost)
         return pos < len(self.tmax)
 
-    def wanted(self, best_cost: float) -> Tuple[int, int]:
-        """Index range [a, b) of thresholds to compute next under the bound ``best_cost``; the
-        range grows fourfold every time the same G asks again."""
-        a = self.have_lo + len(self.cost)
-        self._reach(a + self.limit, best_cost)
-        stop = int(np.searchsorted(self.scaled, best_cost, side="left"))
-        b = max(a, min(stop, a + self.limit))
-        if b > a:
-            self.limit = min(MAX_CHUNK, self.limit * 4)
-        return a, b
+    def _floor_total(self, at: int, sum_later: float) -> float:
+        """Lower bound of the total of any improvement at thresholds ``at``..j, from the sum at j."""
+        prev = float(self.tmax[at - 1]) if at > self.first else float(self.window.start_value)
+        return (sum_later + (self.G - 1) * prev) * (1.0 - FLOOR_SLACK)
 
-    def runs_out(self, best_cost: float) -> bool:
+    def _later(self, pos: int) -> Optional[int]:
+        k = bisect.bisect_left(self.keys, pos)
+        return self.keys[k] if k < len(self.keys) else None
+
+    def wanted(self, best_cost: float) -> List[int]:
         """Dry run of ``replay`` under the bound ``best_cost`` (the true running best when this G
-        is reached is no larger, so the true scan stops no later): True if the computed results
-        would not suffice."""
-        pos, hi = self.pos, self.have_lo + len(self.cost)
-        end = min(hi, len(self.scaled))
-        if pos < end:  # the part that is materialised and computed, as plain python floats
-            scaled = self.scaled[pos:end].tolist()
-            cost = self.cost[pos - self.have_lo:end - self.have_lo].tolist()
-            for s, c in zip(scaled, cost):
-                if s >= best_cost:
-                    return False
-                if c < best_cost:
-                    best_cost = c
-            pos = end
+        is reached is no larger, so the true scan passes no fewer thresholds): the thresholds
+        whose outcomes it would miss, at most ``limit`` of them (it goes on as if they improved
+        nothing), and, if it stops at that limit, ``PROBES`` more spread over what it did not get
+        to.  A scan without any outcome asks for its first batch."""
+        if self.window is None:
+            return []
+        if not self.known:
+            self._reach(self.pos + FIRST_CHUNK, best_cost)
+            stop = int(np.searchsorted(self.scaled, best_cost, side="left"))
+            if stop <= self.pos:
+                return []
+            n_avail = stop - self.pos
+            return [self.pos + self.first_index(k, n_avail, FIRST_CHUNK, FIRST_LEAD)
+                    for k in range(min(FIRST_CHUNK, n_avail))]
+        out, pos, budget, cut = [], self.pos, self.limit, False
         while self._reach(pos, best_cost):
             if self.scaled[pos] >= best_cost:
-                return False
-            if pos >= hi:
-                return True
-            best_cost = min(best_cost, float(self.cost[pos - self.have_lo]))
+                break
+            later = self._later(pos)
+            if later is not None and self._floor_total(pos, self.known[later][1]) >= best_cost:
+                pos = later + 1
+                continue
+            if later == pos:
+                best_cost = min(best_cost, self.known[pos][0])
+            else:
+                if budget == 0:
+                    cut = True
+                    break
+                out.append(pos)
+                budget -= 1
             pos += 1
-        return False
+        if cut:
+            stop = int(np.searchsorted(self.scaled, best_cost, side="left"))
+            last = 0
+            for k in range(PROBES):
+                if stop <= pos:
+                    break
+                at = pos + ((k + 1) * (stop - pos)) // PROBES - 1
+                if at < pos or (k > 0 and at <= last) or at in self.known:
+                    continue
+                out.append(at)
+                last = at
+        return out
 
-    def add(self, cost: np.ndarray):
-        self.cost = np.concatenate([self.cost, cost])
+    def add(self, at: List[int], cost: np.ndarray, sums: np.ndarray):
+        for i, c, s in zip(at, cost.tolist(), sums.tolist()):
+            if i not in self.known:
+                bisect.insort(self.keys, i)
+            self.known[i] = (c, s)
 
     def replay(self, best_cost: float, best_t):
         """Advances the sequential scan as far as the computed results allow.  Returns
         (best_cost, best_t, finished)."""
-        hi = self.have_lo + len(self.cost)
-        end = min(hi, len(self.scaled))
-        if self.pos < end:  # the part that is materialised and computed, as plain python floats
-            first = self.pos
-            scaled = self.scaled[first:end].tolist()
-            cost = self.cost[first - self.have_lo:end - self.have_lo].tolist()
-            for j, (s, c) in enumerate(zip(scaled, cost)):
-                if s >= best_cost:  # inter_tuning.py:196-197
-                    self.pos = first + j
-                    return best_cost, best_t, True
-                if c < best_cost:
-                    best_cost, best_t = c, self.tmax[first + j]
-            self.pos = end
         while self._reach(self.pos, best_cost):
-            if self.scaled[self.pos] >= best_cost:
+            if self.scaled[self.pos] >= best_cost:  # inter_tuning.py:196-197
                 return best_cost, best_t, True
-            if self.pos >= hi:
+            later = self._later(self.pos)
+            if later is not None and self._floor_total(self.pos, self.known[later][1]) >= best_cost:
+                self.pos = later + 1  # nothing up to there improves the best
+                continue
+            if later != self.pos:
                 return best_cost, best_t, False     # needs more DP results
-            cost = float(self.cost[self.pos - self.have_lo])
+            cost = self.known[self.pos][0]
             if cost < best_cost:
                 best_cost, best_t = cost, self.tmax[self.pos]
             self.pos += 1
@@ -662,12 +694,12 @@ def _search(runner: _DpRunner, rows: np.ndarray, Gs: List[int], stats: Optional[
         for i, G in enumerate(Gs):
             w = windows[t * len(Gs) + i]
             start = int(np.searchsorted(w.kept, w.start_value, side="left")) if w is not None else 0
-            scans.append(_Scan(G, w, start))
+            scans.append(_Scan(G, w, start, runner.lib.mist_dp_first_batch_index))
         chains.append(dict(scans=scans, current=0, best=(float("inf"), None, None)))
 
     # Speculative batches + sequential replay (see the module docstring).
     while True:
-        req_g, req_t, req_G, req_span = [], [], [], []
+        req_g, req_t, req_G, req_span = [], [], [], []  # (spans: instance, G index, threshold indices)
         for t, ch in enumerate(chains):
             scans = ch["scans"]
             best_cost, best_G, best_t = ch["best"]
@@ -682,23 +714,23 @@ def _search(runner: _DpRunner, rows: np.ndarray, Gs: List[int], stats: Optional[
             ch["best"] = (best_cost, best_G, best_t)
             for i in range(ch["current"], len(scans)):
                 sc = scans[i]
-                if i > ch["current"] and not sc.runs_out(best_cost):
-                    continue
-                a, b = sc.wanted(best_cost)
-                if b > a:
-                    req_g.append(np.full(b - a, rows[t, i], dtype=np.int32))
-                    req_t.append(sc.tmax[a:b])
-                    req_G.append(np.full(b - a, sc.G, dtype=np.int64))
-                    req_span.append((t, i, b - a))
+                at = sc.wanted(best_cost)
+                if at:
+                    # the range grows fourfold every time the same G asks again
+                    sc.limit = min(MAX_CHUNK, sc.limit * 4)
+                    req_g.append(np.full(len(at), rows[t, i], dtype=np.int32))
+                    req_t.append(sc.tmax[at])
+                    req_G.append(np.full(len(at), sc.G, dtype=np.int64))
+                    req_span.append((t, i, at))
         if all(ch["current"] == len(ch["scans"]) for ch in chains):
             break
         if not req_span:
             raise RuntimeError("inter-stage scan made no progress")  # cannot happen: guards a hang
-        cost, _, _ = runner.evaluate(np.concatenate(req_g), np.concatenate(req_t), np.concatenate(req_G))
+        cost, _, sums = runner.evaluate(np.concatenate(req_g), np.concatenate(req_t), np.concatenate(req_G))
         off = 0
-        for t, i, n in req_span:
-            chains[t]["scans"][i].add(cost[off:off + n])
-            off += n
+        for t, i, at in req_span:
+            chains[t]["scans"][i].add(at, cost[off:off + len(at)], sums[off:off + len(at)])
+            off += len(at)
     t_2 = time.perf_counter()
     if stats is not None:
         stats["dp_thresholds_s"] = stats.get("dp_thresholds_s", 0.0) + (t_1 - t_0)

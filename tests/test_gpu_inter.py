@@ -696,12 +696,14 @@ def test_candidate_selection_of_wide_windows_matches_numpy():
             assert above == int((hg > b).sum())
 
 
-@pytest.mark.parametrize("capacity, first_chunk", [(8192, 48), (256, 7)])
-def test_windows_walked_on_the_device_equal_the_host_walk(capacity, first_chunk):
+@pytest.mark.parametrize("capacity, first_chunk, first_lead", [(8192, 48, 16), (256, 7, 7), (8192, 12, 3)])
+def test_windows_walked_on_the_device_equal_the_host_walk(capacity, first_chunk, first_lead):
     """``mist_dp_windows_first_batch`` (per-request selection, sort, start of the walk, gap walk
     and first scan batch on the GPU) against the host route it replaces (numpy filter of the
     same tables, ``mist_dp_window_begin``): kept thresholds, their number below the smallest
-    feasible threshold, the batch's instances and every status - windows of several widths
+    feasible threshold, the batch's instances (all of a short window; of a long one the first
+    ``first_lead`` thresholds and the rest of the batch spread evenly up to its last one) and
+    every status - windows of several widths
     around the real smallest feasible thresholds of the GPT-7B plan, a window whose start cannot
     be certain, an empty one, a skipped request, and (small capacity) windows that overflow."""
     import ctypes
@@ -763,7 +765,7 @@ def test_windows_walked_on_the_device_equal_the_host_walk(capacity, first_chunk)
     with torch.cuda.device(dev):
         rc = lib.mist_dp_windows_first_batch(
             ctypes.byref(runner._all_costs), n, d_rows.data_ptr(), d_lo.data_ptr(), d_hi.data_ptr(),
-            d_start.data_ptr(), GAP, capacity, first_chunk, d_values.data_ptr(), d_counts.data_ptr(),
+            d_start.data_ptr(), GAP, capacity, first_chunk, first_lead, d_values.data_ptr(), d_counts.data_ptr(),
             d_kept.data_ptr(), kept_capacity, d_meta.data_ptr(), d_inst_t.data_ptr(),
             d_inst_row.data_ptr(), None)
         _lib.check(rc, "mist_dp_windows_first_batch")
@@ -774,7 +776,7 @@ def test_windows_walked_on_the_device_equal_the_host_walk(capacity, first_chunk)
     inst_row = d_inst_row.cpu().numpy()
 
     host = runner.candidates_between(rows, lo, hi)
-    seen, used = set(), []
+    seen, used, spread = set(), [], 0
     for r in range(n):
         values, above = host[r]
         n_sel, n_above, status, n_kept, base, pos, n_inst, inst_at = (int(x) for x in meta[r])
@@ -805,10 +807,22 @@ def test_windows_walked_on_the_device_equal_the_host_walk(capacity, first_chunk)
         assert n_kept == len(kept) and np.array_equal(kept_all[base:base + n_kept], kept)
         assert pos == int(np.searchsorted(kept, start[r], side="left"))
         assert n_inst == min(first_chunk, n_kept - pos) > 0
-        assert np.array_equal(inst_t[inst_at:inst_at + n_inst], kept[pos:pos + n_inst])
+        n_avail = n_kept - pos
+        picked = [lib.mist_dp_first_batch_index(k, n_avail, first_chunk, first_lead) for k in range(n_inst)]
+        if n_avail <= first_chunk or first_lead >= first_chunk:
+            assert picked == list(range(n_inst))
+        else:
+            spread += 1
+            assert picked[:first_lead] == list(range(first_lead)) and picked[-1] == n_avail - 1
+            assert all(a < b for a, b in zip(picked, picked[1:]))
+            steps = np.diff(picked[first_lead - 1:])
+            assert steps.max() - steps.min() <= 1
+        assert lib.mist_dp_first_batch_index(n_inst, n_avail, first_chunk, first_lead) == -1
+        assert np.array_equal(inst_t[inst_at:inst_at + n_inst], kept[pos:][picked])
         assert np.all(inst_row[inst_at:inst_at + n_inst] == rows[r])
         used.append((inst_at, n_inst))
     assert {0, 1, 3, 4} <= seen and (capacity > 1024 or 2 in seen)
+    assert spread > 0 or first_lead >= first_chunk
     # the instances of all windows lie behind one another from slot 0 on, the rest is empty
     used.sort()
     assert used[0][0] == 0 and all(a + k == b for (a, k), (b, _) in zip(used, used[1:]))

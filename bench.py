@@ -391,7 +391,8 @@ def main():
         assert (e2e_cost, e2e_solution) == (cost, solution)
     tune_end_to_end_s = sorted(e2e)[len(e2e) // 2]
 
-    # Roofline of the dominant kernel, measured with events on the launch stream.
+    # Roofline of the dominant kernel, measured with events on the launch stream.  (The plan's
+    # problem record is as the steps above left it: with the stage-cost estimate of tune().)
     def time_kernels(tuner, plan, dev_plan, reps):
         ms = {}
         for rep in range(reps + 1):
@@ -512,6 +513,12 @@ def main():
         "sustained": {"seconds": args.sustain_s, "steps": len(sustained), "median_ms_per_step": sustained_ms,
                       "candidates_per_s": counts["candidates"] / (sustained_ms * 1e-3)},
         "dp_thresholds_per_step": stats.get("dp_thresholds", 0) / args.steps,
+        # tune() lets the intra-stage kernels skip stage costs its search cannot use, from an
+        # estimate of the best cost that the scout pass leaves; a step whose result the estimate
+        # does not cover is evaluated again without it (none expected here)
+        "stage_cost_estimate": (float(search.dev_plan["incumbent"].item())
+                                if "incumbent" in search.dev_plan else None),
+        "stage_cost_cutoff_retries": stats.get("stage_cost_cutoff_retries", 0),
         "best_cost": cost,
         "best_solution": repr(solution),
         "roofline": roofline,

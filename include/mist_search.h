@@ -95,6 +95,24 @@ typedef struct MistProblem {
                             * terms and the scout pass one after the other) */
   int32_t max_group_keys;  /* largest n_par * n_ao * n_pair of the call's groups; 0 = unknown
                             * (mist_row_terms then evaluates every row on its own) */
+  /* Optional (NULL = none; sample_size 1 only, where a cell's objective is its stage cost): one
+   * double in device memory, an estimate of the cost of the best pipeline the caller's
+   * inter-stage search returns (+inf before the first call).  The scout pass lowers it to the
+   * cost of the best partition into equal stages on equal meshes that its seeds allow; the main
+   * launch then does not look for stage costs above
+   *     bound(G) = incumbent / G * (1 + mist_incumbent_slack()).
+   * A cell whose minimum is not above bound(G) holds its minimum and row as always; any other
+   * cell holds some value above it (a seed, or +inf / -1), not necessarily its minimum.
+   * A search that scans thresholds t with t * G < best (inter_tuning.py:196-197) and returns a
+   * cost below incumbent * (1 + slack) * (1 - 1e-5) has read the same values, in the same order,
+   * as from the full tables: every threshold that can lead to such a cost lies below bound(G),
+   * where the tables agree, and every partition with a stage above it costs more.  A caller
+   * whose search returns more than that evaluates again without the incumbent. */
+  double *stage_cost_incumbent;
+  int32_t incumbent_num_devices; /* devices of the cluster: stages = this / (n * m of the group) */
+  int32_t incumbent_ckpt_rule;   /* ckpt counts the search admits for a stage that ends at layer
+                                  * i with l layers: 0 = 0..min(l, L - i) (inter_tuning.py:315),
+                                  * 1 = 0..l, 2 = l only (inter_tuning_uniform_device.py:400-404) */
 } MistProblem;
 
 /* One (gradient-accumulation steps, device mesh) group = one call of the reference's
@@ -153,6 +171,7 @@ typedef struct MistOutTables {
 const char *mist_version(void);
 const char *mist_last_error(void);
 int mist_sizeof_problem(void);
+double mist_incumbent_slack(void); /* see MistProblem.stage_cost_incumbent */
 int mist_sizeof_group(void);
 int mist_reduce_p_tile(void); /* MIST_P_TILE the library was built with */
 int mist_reduce_lc_tile(void); /* MIST_LC_TILE the library was built with */

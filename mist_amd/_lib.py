@@ -61,6 +61,9 @@ PROBLEM_DTYPE = np.dtype(
         ("adv_first_block", "<i4"),
         ("max_scout_rows", "<i4"),
         ("max_group_keys", "<i4"),
+        ("stage_cost_incumbent", "<u8"),
+        ("incumbent_num_devices", "<i4"),
+        ("incumbent_ckpt_rule", "<i4"),
     ],
     align=True,
 )
@@ -110,6 +113,7 @@ _SIGNATURES = {
     "mist_version": (ctypes.c_char_p, []),
     "mist_last_error": (ctypes.c_char_p, []),
     "mist_sizeof_problem": (ctypes.c_int, []),
+    "mist_incumbent_slack": (ctypes.c_double, []),
     "mist_sizeof_group": (ctypes.c_int, []),
     "mist_reduce_p_tile": (ctypes.c_int, []),
     "mist_reduce_stage_rows": (ctypes.c_int, []),

@@ -41,6 +41,7 @@ using mist::fail;
 constexpr int kTermsBlock = 128;  // rows per workgroup of the row-term kernel
 constexpr int kStageRows = 64;    // rows staged through LDS per step of the reduce kernel
 constexpr int kSlots = 2 * MIST_P_TILE + 2;  // per-thread running minima: base, with_pre, post, no_pp
+constexpr double kIncumbentSlack = 0.25;  // relative room above MistProblem.stage_cost_incumbent / G
 // Stage summaries (written with the row terms, read by the reduce kernel): per stage of
 // kStageRows workspace rows the term-wise minimum of the latency and memory columns and the
 // maximum of MIST_T_OUT, kStageFloorPitch doubles per stage.
@@ -1097,6 +1098,11 @@ __device__ __forceinline__ void reduce_block(
   const float G32 = (float)g->grad_accum;
   const double inv_G64 = 1.0 / G64;
   const float inv_G32 = 1.0f / G32;
+  // Stage costs the caller's search can use at all (MistProblem.stage_cost_incumbent): rows above
+  // it are not looked for.  (The scout pass, whose seeds the incumbent comes from, has none.)
+  const double cutoff = range.gathered != 0 || prob.stage_cost_incumbent == nullptr || prob.sample_size != 1
+                            ? (double)INFINITY
+                            : *prob.stage_cost_incumbent * inv_G64 * (1.0 + kIncumbentSlack);
   const double pre_saved = g->pre_saved, pre_sas = g->pre_states_and_saved;
   const double pre_states = g->pre_states;
   const double post_states = g->post_states, post_fwd_peak = g->post_fwd_peak;
@@ -1265,10 +1271,10 @@ __device__ __forceinline__ void reduce_block(
     constexpr bool kCommit = decltype(commit_tag)::value;
     double x, d, cost_base, bound;
     objective(t, x, d, cost_base, bound);
-    const bool cand_b = cost_base <= top_b || fin_b < n_tile;
-    const bool want_pre = bound <= top_p || fin_p < n_tile;
-    const bool want_post = do_post && bound <= best_post;
-    const bool want_pp = do_nopp && bound <= best_pp;
+    const bool cand_b = (cost_base <= top_b || fin_b < n_tile) && cost_base <= cutoff;
+    const bool want_pre = (bound <= top_p || fin_p < n_tile) && bound <= cutoff;
+    const bool want_post = do_post && bound <= fmin(best_post, cutoff);
+    const bool want_pp = do_nopp && bound <= fmin(best_pp, cutoff);
     if (!(cand_b || want_pre || want_post || want_pp)) return false;
 
     double cost_pre = INFINITY, cost_post = INFINITY, cost_pp = INFINITY;
@@ -1298,9 +1304,9 @@ __device__ __forceinline__ void reduce_block(
 #pragma unroll
       for (int j = 0; j < MIST_P_TILE; ++j) lo_p += best_p[j] < cost_pre ? 1 : 0;
     }
-    bool need_b = cand_b && lo_b < n_tile, need_p = want_pre && lo_p < n_tile;
-    bool need_post = want_post && cost_post <= best_post;
-    bool need_pp = want_pp && cost_pp <= best_pp;
+    bool need_b = cand_b && lo_b < n_tile, need_p = want_pre && lo_p < n_tile && cost_pre <= cutoff;
+    bool need_post = want_post && cost_post <= fmin(best_post, cutoff);
+    bool need_pp = want_pp && cost_pp <= fmin(best_pp, cutoff);
     if (!(need_b || need_p || need_post || need_pp)) return false;
 
     const LaneMemory mem = lane_memory(t);
@@ -1417,11 +1423,11 @@ __device__ __forceinline__ void reduce_block(
         (ratio * (lds_min[kStageMinOpb] + (k.pp_wre ? nag_min : 0.0) + (k.pp_gre ? nrs_min : 0.0)) +
          div_G((k.pp_wre ? 0.0 : nag_min) + (k.pp_gre ? 0.0 : nrs_min))) * (1.0 - kSlack);
     {
-      const double loose_b = fin_b < n_tile ? (double)INFINITY : top_b;
-      const double loose_p = fin_p < n_tile ? (double)INFINITY : top_p;
+      const double loose_b = fmin(fin_b < n_tile ? (double)INFINITY : top_b, cutoff);
+      const double loose_p = fmin(fin_p < n_tile ? (double)INFINITY : top_p, cutoff);
       double loose_o = below(loose_p, off_pre);
-      if (do_post) loose_o = fmax(loose_o, below(best_post, off_post + stage_post));
-      if (do_nopp) loose_o = fmax(loose_o, below(best_pp, off_pp + stage_post));
+      if (do_post) loose_o = fmax(loose_o, below(fmin(best_post, cutoff), off_post + stage_post));
+      if (do_nopp) loose_o = fmax(loose_o, below(fmin(best_pp, cutoff), off_pp + stage_post));
       if (!__any(active && (floor_cost <= loose_b || floor_bound <= loose_o))) continue;
     }
 
@@ -1437,6 +1443,8 @@ __device__ __forceinline__ void reduce_block(
       thr_b = j < cnt_b ? best_b[j] : thr_b;
       thr_p = j < cnt_p ? best_p[j] : thr_p;
     }
+    thr_b = fmin(thr_b, cutoff);
+    thr_p = fmin(thr_p, cutoff);
     // One threshold for the three composite objectives, expressed for `bound` (objective()):
     // each of them exceeds `bound` by at least its group-wide offset.
     double thr_o = below(thr_p, off_pre);
@@ -1451,12 +1459,12 @@ __device__ __forceinline__ void reduce_block(
       const double pf_post = fmax(f_in, peak_f + post_states);
       const double pb_post = fmax(b_in, peak_b - lds_min[kStageMaxOut] + post_states) + post_output;
       if (fmax(pf_post, pb_post) * floor_mem.mf_pp <= cap)
-        thr_o = fmax(thr_o, below(best_post, off_post + stage_post));
+        thr_o = fmax(thr_o, below(fmin(best_post, cutoff), off_post + stage_post));
       if (do_nopp) {
         const double pf_pp = pf_post + pre_states + pre_saved;
         const double pb_pp = pb_post + pre_states + pre_saved;
         if (fmax(pf_pp, pb_pp) * lds_min[MIST_T_MF] <= cap)
-          thr_o = fmax(thr_o, below(best_pp, off_pp + stage_post));
+          thr_o = fmax(thr_o, below(fmin(best_pp, cutoff), off_pp + stage_post));
       }
     }
 
@@ -1822,6 +1830,87 @@ __global__ __launch_bounds__(MIST_LC_TILE, MIST_EXHAUSTIVE_MIN_WAVES) void eval_
                             lds_terms, lds_row, partial_cost + block * slab, partial_index + block * slab);
 }
 
+// Cost of the best pipeline of equal stages on equal meshes that the scout pass's seeds allow
+// (sample 0 of a call with one sample, whose objective is the stage cost): group (G, mesh (n, m))
+// offers S = devices / (n m) stages of L / S layers each, the first one from the with_pre table
+// at S - 1 pre-saved micro-batches, the last one from the with_post table, those between from
+// the base table, a single one from the no_pp table, each at its cheapest admissible ckpt count
+// (rule of the caller's search, MistProblem.incumbent_ckpt_rule); the cost is the sum of the
+// stage costs + (G - 1) x the largest, as the search forms it (inter_tuning.py:342).  Seeds are
+// minima over some rows, so the finished tables hold no larger values; the search that reads
+// them returns no more than this unless its scan never tries the thresholds of that pipeline
+// (a single-stage cost is no threshold candidate of the reference, and its gap rule drops
+// some), which is why the caller checks its result against the bound that was used.
+// Workgroup = group, one wavefront; lowers *incumbent.
+__global__ __launch_bounds__(64) void incumbent_kernel(
+    const MistProblem prob, const MistGroupDesc *__restrict__ groups,
+    const int32_t *__restrict__ scout_prefix, int64_t scout_base,
+    const double *__restrict__ partial_cost, const int32_t *__restrict__ partial_index) {
+  const MistGroupDesc *g = groups + blockIdx.x;
+  if (g->scout_stride <= 0) return;
+  const int L = prob.num_layers, D = prob.incumbent_num_devices;
+  const int nm = g->num_nodes * g->num_gpus_per_node;
+  if (nm <= 0 || D % nm != 0) return;
+  const int S = D / nm;
+  if (S < 1 || S > L || L % S != 0 || S - 1 >= g->num_p) return;
+  // (the per-mesh search goes up to min(devices, layers) / 2 stages, inter_tuning.py:279-281)
+  if (prob.incumbent_ckpt_rule == 0 && S > (D < L ? D : L) / 2) return;
+  const int l = L / S;
+  const int64_t slab = (int64_t)kSlots * MIST_LC_TILE;
+  // cheapest seed of the stage's (l, c) cells, c = 0..c_last, in slot `slot` of p tile `p_tile`
+  auto cheapest = [&](int slot, int p_tile, int c_last) {
+    double best = INFINITY;
+    for (int c = threadIdx.x; c <= c_last; c += 64) {
+      const int pair = l * (l + 1) / 2 - 1 + c;
+      const int lc_tile = pair / MIST_LC_TILE - g->lc_tile_begin;
+      if (lc_tile < 0 || lc_tile >= g->n_lc_tiles) continue;
+      const int64_t at = (scout_base + scout_prefix[blockIdx.x] +
+                          (int64_t)(lc_tile * g->n_p_tiles + p_tile) * kScoutSplit) * slab +
+                         slot * MIST_LC_TILE + pair % MIST_LC_TILE;
+      if (partial_index[at] >= 0) best = fmin(best, partial_cost[at]);
+    }
+    for (int step = 32; step > 0; step >>= 1) best = fmin(best, __shfl_xor(best, step));
+    return best;
+  };
+  auto c_last_of = [&](int end_layer) {
+    return prob.incumbent_ckpt_rule == 0 ? min(l, L - end_layer) : l;
+  };
+  double sum = 0.0, largest = 0.0;
+  for (int s = 0; s < S; ++s) {
+    const int p = S - 1 - s, end_layer = (s + 1) * l - 1;
+    int slot;
+    if (S == 1) slot = 2 * MIST_P_TILE + 1;
+    else if (s == 0) slot = MIST_P_TILE + p % MIST_P_TILE;
+    else if (s == S - 1) slot = 2 * MIST_P_TILE;
+    else slot = p % MIST_P_TILE;
+    const int p_tile = (S == 1 || s == S - 1) ? 0 : p / MIST_P_TILE;
+    double cost;
+    if (prob.incumbent_ckpt_rule == 2) {  // every layer of the stage checkpointed
+      cost = INFINITY;
+      if (threadIdx.x == 0) {
+        const int pair = l * (l + 1) / 2 - 1 + l;
+        const int lc_tile = pair / MIST_LC_TILE - g->lc_tile_begin;
+        if (lc_tile >= 0 && lc_tile < g->n_lc_tiles) {
+          const int64_t at = (scout_base + scout_prefix[blockIdx.x] +
+                              (int64_t)(lc_tile * g->n_p_tiles + p_tile) * kScoutSplit) * slab +
+                             slot * MIST_LC_TILE + pair % MIST_LC_TILE;
+          if (partial_index[at] >= 0) cost = partial_cost[at];
+        }
+      }
+      cost = __shfl(cost, 0);
+    } else {
+      cost = cheapest(slot, p_tile, c_last_of(end_layer));
+    }
+    sum += cost;
+    largest = fmax(largest, cost);
+  }
+  const double total = sum + (double)(g->grad_accum - 1) * largest;
+  // costs are not negative, and non-negative doubles order like their bit patterns
+  if (threadIdx.x == 0 && total >= 0.0 && total < INFINITY)
+    atomicMin(reinterpret_cast<unsigned long long *>(prob.stage_cost_incumbent),
+              (unsigned long long)__double_as_longlong(total));
+}
+
 // Combines the slabs of the kScoutSplit scout workgroups of every tile into the first of them,
 // so that each chunk of the main launch reads one slab of seeds instead of kScoutSplit.
 // Workgroup = tile; the scout slabs of tile t are scout_base + t * kScoutSplit + k.
@@ -2129,6 +2218,16 @@ int check_factors(const MistProblem *problem) {
 int check_common(const void *d_problem, const void *d_groups, int n_groups) {
   if (!d_problem || !d_groups) return fail(MIST_E_INVALID, "null problem / group pointer");
   if (n_groups <= 0) return fail(MIST_E_INVALID, "n_groups must be positive, got %d", n_groups);
+  const MistProblem *problem = static_cast<const MistProblem *>(d_problem);
+  if (problem->stage_cost_incumbent != nullptr) {
+    if (problem->sample_size != 1)
+      return fail(MIST_E_INVALID, "a stage-cost incumbent needs sample_size 1, got %d",
+                  problem->sample_size);
+    if (problem->incumbent_num_devices < 1 || problem->incumbent_ckpt_rule < 0 ||
+        problem->incumbent_ckpt_rule > 2)
+      return fail(MIST_E_INVALID, "stage-cost incumbent with %d devices, ckpt rule %d",
+                  problem->incumbent_num_devices, problem->incumbent_ckpt_rule);
+  }
   return 0;
 }
 
@@ -2141,6 +2240,7 @@ const char *mist_last_error(void) { return g_last_error; }
 int mist_sizeof_problem(void) { return (int)sizeof(MistProblem); }
 int mist_sizeof_group(void) { return (int)sizeof(MistGroupDesc); }
 int mist_reduce_p_tile(void) { return MIST_P_TILE; }
+double mist_incumbent_slack(void) { return kIncumbentSlack; }
 
 // key_terms_kernel over every group when the caller gave a key-term workspace and the bound the
 // grid needs; *launched tells whether the row-term kernel can read key terms.
@@ -2214,6 +2314,11 @@ static int launch_scout(const MistProblem *problem, const MistGroupDesc *d_group
     hipLaunchKernelGGL(merge_scout_kernel, dim3(n_scout_blocks / kScoutSplit, n_samples), dim3(256),
                        0, (hipStream_t)stream, scout_base, n_scout_blocks, d_partial_cost,
                        d_partial_index);
+    MIST_HIP_CHECK(hipGetLastError());
+  }
+  if (problem->stage_cost_incumbent != nullptr && n_samples == 1) {
+    hipLaunchKernelGGL(incumbent_kernel, dim3(n_groups), dim3(64), 0, (hipStream_t)stream, *problem,
+                       d_groups, scout_prefix, scout_base, d_partial_cost, d_partial_index);
     MIST_HIP_CHECK(hipGetLastError());
   }
   return 0;

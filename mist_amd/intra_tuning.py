@@ -824,9 +824,26 @@ class IntraStageTuner:
             ))
         return outs
 
-    def run_prepared(self, plan, dev_plan) -> List[IntraStageTunerOutput]:
+    def run_prepared(self, plan, dev_plan,
+                     stage_cost_cutoff: Optional[dict] = None) -> List[IntraStageTunerOutput]:
         """Device part only: fresh output tables + kernel launches for an uploaded plan; one
-        output per tp size, all resident in the same tables."""
+        output per tp size, all resident in the same tables.
+
+        ``stage_cost_cutoff`` (``num_devices``, ``ckpt_rule``; one sample only) is for a caller
+        whose inter-stage search is all that reads the tables: the scout pass turns its seeds
+        into an upper bound of the best pipeline cost (``MistProblem.stage_cost_incumbent``),
+        and the main launch does not look for stage costs that no threshold of that search can
+        admit.  Cells above that bound then hold some value above it, not their minimum."""
+        problem = plan["problem"]
+        problem["stage_cost_incumbent"] = 0
+        if stage_cost_cutoff is not None and self.sample_size == 1 and not self.exhaustive:
+            with torch.cuda.device(self.device):
+                if "incumbent" not in dev_plan:
+                    dev_plan["incumbent"] = torch.empty(1, dtype=torch.float64, device=self.device)
+                dev_plan["incumbent"].fill_(float("inf"))
+            problem["stage_cost_incumbent"] = dev_plan["incumbent"].data_ptr()
+            problem["incumbent_num_devices"] = int(stage_cost_cutoff["num_devices"])
+            problem["incumbent_ckpt_rule"] = int(stage_cost_cutoff["ckpt_rule"])
         with torch.cuda.device(self.device):
             costs, index, struct = self._allocate_flat(plan)
             self.launch(plan, dev_plan, struct)

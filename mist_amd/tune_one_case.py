@@ -31,6 +31,7 @@ import numpy as np
 import torch
 import yaml
 
+from . import _lib
 from .config import OFFLOADING_RATIO_CANDIDATES, MistConfig, tp_candidates
 from .inter_tuning import inter_stage_tune, inter_stage_tune_batch
 from .inter_tuning_uniform import inter_stage_tune as inter_stage_tune_uniform
@@ -175,6 +176,21 @@ class PreparedSearch:
         self.plan = self.tuner.prepare()
         with torch.cuda.device(self.tuner.device):
             self.dev_plan = self.tuner.upload(self.plan)
+        # The searches that scan thresholds below best / G (inter_tuning.py:196-197) never admit
+        # a stage cost above that: the intra-stage kernels need not find the minima of such
+        # cells (IntraStageTuner.run_prepared), given an estimate of the best cost.  ``run``
+        # checks the search's result against the estimate that was used and evaluates again
+        # without it if the result is not below.  ckpt counts a stage may use, as those
+        # searches restrict them: inter_tuning.py:315; inter_tuning_uniform_device.py:400-404.
+        self.stage_cost_cutoff = None
+        self._incumbent_host = self._incumbent_read = None
+        if sample_size == 1 and not exhaustive and os.environ.get("MIST_NO_STAGE_COST_CUTOFF") is None:
+            devices = hw.num_nodes * hw.num_gpus_per_node
+            if self.granularity == "inter-stage":
+                self.stage_cost_cutoff = dict(num_devices=devices, ckpt_rule=0)
+            elif self.granularity == "uniform-device-pp":
+                rule = 1 if tuning.activation_checkpointing_tuning_enabled else 2
+                self.stage_cost_cutoff = dict(num_devices=devices, ckpt_rule=rule)
 
     def counts(self) -> Dict[str, int]:
         """Search-space sizes: strategy rows, candidates = rows * (L + 1), base-variant cells
@@ -195,7 +211,16 @@ class PreparedSearch:
         stats = {} if stats is None else stats
         hw = self.config.hardware
         t0 = time.perf_counter()
-        results = self.tuner.run_prepared(self.plan, self.dev_plan)
+        cutoff = self.stage_cost_cutoff
+        results = self.tuner.run_prepared(self.plan, self.dev_plan, cutoff)
+        if cutoff is not None:
+            # the estimate the kernels ended with travels to the host behind them
+            with torch.cuda.device(self.tuner.device):
+                if self._incumbent_host is None:
+                    self._incumbent_host = torch.empty(1, dtype=torch.float64, pin_memory=True)
+                    self._incumbent_read = torch.cuda.Event()
+                self._incumbent_host.copy_(self.dev_plan["incumbent"], non_blocking=True)
+                self._incumbent_read.record()
         if split_timing:
             torch.cuda.synchronize(self.tuner.device)
         t1 = time.perf_counter()
@@ -220,6 +245,19 @@ class PreparedSearch:
         for cost, solution in outcomes:  # tune_one_case.py:228-231: the first best tp wins
             if cost < best_cost:
                 best_cost, best_solution = cost, solution
+        if cutoff is not None:
+            self._incumbent_read.synchronize()
+            estimate = float(self._incumbent_host[0])
+            # Below this cost the search has read nothing but cells that hold their minima
+            # (MistProblem.stage_cost_incumbent); an infinite estimate left every cell exact.
+            safe_below = estimate * (1.0 + _lib.load().mist_incumbent_slack()) * (1.0 - 1e-5)
+            if np.isfinite(estimate) and not best_cost < safe_below:
+                stats["stage_cost_cutoff_retries"] = stats.get("stage_cost_cutoff_retries", 0) + 1
+                self.stage_cost_cutoff = None
+                try:
+                    return self.run(stats, split_timing)
+                finally:
+                    self.stage_cost_cutoff = cutoff
         return best_cost, best_solution
 
 

@@ -407,6 +407,80 @@ def test_randomized_plans_of_every_granularity_match_oracle(seed):
     assert got == want
 
 
+def _realistic_plan(seed):
+    """Seeded random plan at realistic sizes (8-64 layers, 2-128 devices, the GPT-7B or LLaMA-13B
+    offload grid, random link / copy / interference parameters, capacities from "nothing fits"
+    to "everything fits") for a search that scans thresholds: per-mesh or uniform-device."""
+    rng = np.random.default_rng(333000 + seed)
+    slow = bool(rng.integers(0, 2))
+    gg = []
+    for entry in range(16):
+        lo, hi = (8, 500) if (entry < 4 or not slow) else (0.5, 20)
+        gg += [float(rng.uniform(lo, hi)), float(rng.uniform(2e-6, 8e-5))]
+    nodes, gpn = int(rng.choice([1, 2, 4, 8, 16])), int(rng.choice([2, 4, 8]))
+    L = int(rng.integers(8, 65))
+    granularity = str(rng.choice(["inter-stage", "inter-stage", "uniform-device-pp"]))
+    overrides = dict(
+        model__num_hidden_layers=L,
+        hardware__gpu_gpu_comm_params=gg,
+        hardware__cpu_gpu_comm_params=[float(rng.uniform(5, 60)), float(rng.uniform(2e-6, 3e-5))],
+        hardware__gpu_cpu_comm_params=[float(rng.uniform(5, 60)), float(rng.uniform(2e-6, 3e-5))],
+        hardware__interference_model_params=[float(x) for x in rng.uniform(1.0, 4.0, size=28)],
+        hardware__memory_capacity=float(np.exp(rng.uniform(np.log(3.0), np.log(300.0)))),
+        hardware__num_nodes=nodes, hardware__num_gpus_per_node=gpn,
+        training__global_batch_size=int(rng.choice([64, 128, 256, 512, 96, 384])),
+        model__use_flash_attn=bool(rng.integers(2)),
+        enable_advanced_opt_in_first_block=bool(rng.integers(2)),
+        tuning__pre_post_strategy=str(rng.choice(["dp", "intra-node-tp-with-ore", "intra-node-tp-without-ore"])),
+        tuning__zero_2_and_3_enabled=bool(rng.integers(0, 4) > 0),
+        tuning__activation_checkpointing_tuning_enabled=bool(rng.integers(0, 4) > 0),
+        tuning__state_offloading_enabled=bool(rng.integers(0, 5) > 0),
+        tuning__activation_offloading_enabled=bool(rng.integers(0, 5) > 0),
+        tuning__tuning_granularity=granularity,
+        synthetic__seed=int(rng.integers(1 << 20)),
+    )
+    return load_plan(int(rng.choice([2, 2, 3])), **overrides)[0]
+
+
+def _tune_with_and_without_estimate(cfg):
+    from mist_amd.tune_one_case import PreparedSearch
+
+    search = PreparedSearch(cfg)
+    assert search.stage_cost_cutoff is not None
+    stats = {}
+    got = search.run(stats)
+    estimate = float(search.dev_plan["incumbent"].item())
+    search.stage_cost_cutoff = None
+    want = search.run()
+    assert got == want
+    return want, estimate, stats.get("stage_cost_cutoff_retries", 0)
+
+
+@pytest.mark.parametrize("plan, overrides", [
+    (1, {}), (2, {}), (3, {}), (4, {}), (5, {}),
+    (2, dict(tuning__tuning_granularity="uniform-device-pp")),
+    (3, dict(tuning__tuning_granularity="uniform-device-pp", tuning__activation_checkpointing_tuning_enabled=False)),
+])
+def test_tune_of_the_benchmark_plans_with_a_stage_cost_estimate(plan, overrides):
+    """``tune`` lets the intra-stage kernels skip stage costs its search cannot use
+    (``PreparedSearch.stage_cost_cutoff``): same cost, partition and strategies as the search on
+    the full tables, for every benchmark plan, without a second evaluation; the scout pass of
+    the large plans does produce an estimate."""
+    (cost, solution), estimate, retries = _tune_with_and_without_estimate(load_plan(plan, **overrides)[0])
+    assert solution is not None and retries == 0
+    assert plan == 1 or (np.isfinite(estimate) and cost < estimate * 1.25)
+
+
+@pytest.mark.parametrize("seed", [1, 6, 7, 3, 31, 34, 47, 89, 149, 252, 315, 499, 144, 785, 972, 985, 2088, 3887, 823, 1000])
+def test_tune_of_random_plans_with_a_stage_cost_estimate(seed):
+    """The same on random plans.  The estimate comes from pipelines of equal stages that the
+    reference's scan does not always try (785 ... 3887: it lies below the result; 823 and 1000:
+    so far below that the result is not covered and ``tune`` evaluates again without it)."""
+    _, estimate, retries = _tune_with_and_without_estimate(_realistic_plan(seed))
+    assert retries == (1 if seed in (823, 1000) else 0)
+    assert seed == 144 or np.isfinite(estimate)  # (144: nothing fits)
+
+
 def test_plan1_end_to_end():
     from mist_amd.tune_one_case import tune
     from oracle.tune import tune as oracle_tune

@@ -178,6 +178,49 @@ def test_scout_pass_leaves_results_unchanged(monkeypatch, min_stages, min_pairs)
     _compare(cfg, tables, 2)
 
 
+@pytest.mark.parametrize("plan, rule", [(2, 0), (3, 0), (2, 1), (3, 2)])
+def test_tables_under_a_stage_cost_estimate(plan, rule):
+    """``run_prepared`` with ``stage_cost_cutoff``: the scout pass leaves an estimate of the best
+    pipeline cost, and with bound(G) = estimate / G * (1 + slack) every cell whose minimum is not
+    above the bound holds the same row and costs as without the estimate; every other cell holds
+    a value above the bound or nothing."""
+    import torch
+
+    from mist_amd import _lib
+    from mist_amd.tune_one_case import PreparedSearch
+
+    cfg, _ = load_plan(plan)
+    hw = cfg.hardware
+    search = PreparedSearch(cfg)
+    tuner = search.tuner
+    full = tuner.run_prepared(search.plan, search.dev_plan)[0].batch
+    assert int(search.plan["problem"]["stage_cost_incumbent"][0]) == 0
+    cut = tuner.run_prepared(search.plan, search.dev_plan,
+                             dict(num_devices=hw.num_nodes * hw.num_gpus_per_node, ckpt_rule=rule))[0].batch
+    estimate = float(search.dev_plan["incumbent"].item())
+    assert np.isfinite(estimate) and estimate > 0
+    slack = _lib.load().mist_incumbent_slack()
+    G = torch.tensor(search.Gs * len(tuner.tp_sizes), dtype=torch.float64, device=full.stable[0].device)
+    n_open = n_closed = 0
+    for v in range(4):
+        shape = [-1] + [1] * (full.stable[v].dim() - 1)
+        bound = (estimate * (1.0 + slack) / G).view(shape)
+        cost = lambda t: torch.where(t.index[v] >= 0,
+                                     t.stable[v].float().double() + t.delta[v].float().double() / G.view(shape),
+                                     torch.full_like(t.stable[v], float("inf")))
+        exact, got = cost(full), cost(cut)
+        below = exact <= bound * (1.0 - 1e-6)
+        assert torch.equal(cut.index[v][below], full.index[v][below])
+        assert torch.equal(cut.stable[v][below], full.stable[v][below])
+        assert torch.equal(cut.delta[v][below], full.delta[v][below])
+        above = exact > bound * (1.0 + 1e-6)
+        assert bool((got[above] > (bound.expand_as(got))[above] * (1.0 - 1e-6)).all())
+        assert bool((got >= exact).all())
+        n_open += int(below.sum())
+        n_closed += int((above & (cut.index[v] != full.index[v])).sum())
+    assert n_open > 1000 and n_closed > 1000  # the estimate closes cells, and leaves many open
+
+
 @pytest.mark.parametrize("waves, scout", [(1 << 22, 1), (1 << 22, 0), (1, 1)])
 def test_row_chunking_leaves_results_unchanged(monkeypatch, waves, scout):
     """Groups cut into the smallest row chunks (256 rows: many chunks per tile, most of which

@@ -962,7 +962,7 @@ __device__ __forceinline__ void take_min(double &best, int32_t &best_row, bool f
 #define MIST_REDUCE_MIN_WAVES 2
 #endif
 #ifndef MIST_SCOUT_SPLIT
-#define MIST_SCOUT_SPLIT 2
+#define MIST_SCOUT_SPLIT 4
 #endif
 constexpr int kScoutSplit = MIST_SCOUT_SPLIT;  // scout workgroups per (group, (l, c) tile, p tile)
 constexpr int32_t kSlabUnchanged = -2;  // first row index of a slab that was not written (rows are >= -1)
@@ -1841,8 +1841,9 @@ __global__ __launch_bounds__(MIST_LC_TILE, MIST_EXHAUSTIVE_MIN_WAVES) void eval_
 // them returns no more than this unless its scan never tries the thresholds of that pipeline
 // (a single-stage cost is no threshold candidate of the reference, and its gap rule drops
 // some), which is why the caller checks its result against the bound that was used.
-// Workgroup = group, one wavefront; lowers *incumbent.
-__global__ __launch_bounds__(64) void incumbent_kernel(
+// Workgroup = group, its wavefronts take the stages in turn; lowers *incumbent.
+constexpr int kIncumbentWaves = 4;
+__global__ __launch_bounds__(64 * kIncumbentWaves) void incumbent_kernel(
     const MistProblem prob, const MistGroupDesc *__restrict__ groups,
     const int32_t *__restrict__ scout_prefix, int64_t scout_base,
     const double *__restrict__ partial_cost, const int32_t *__restrict__ partial_index) {
@@ -1860,7 +1861,7 @@ __global__ __launch_bounds__(64) void incumbent_kernel(
   // cheapest seed of the stage's (l, c) cells, c = 0..c_last, in slot `slot` of p tile `p_tile`
   auto cheapest = [&](int slot, int p_tile, int c_last) {
     double best = INFINITY;
-    for (int c = threadIdx.x; c <= c_last; c += 64) {
+    for (int c = threadIdx.x & 63; c <= c_last; c += 64) {
       const int pair = l * (l + 1) / 2 - 1 + c;
       const int lc_tile = pair / MIST_LC_TILE - g->lc_tile_begin;
       if (lc_tile < 0 || lc_tile >= g->n_lc_tiles) continue;
@@ -1875,8 +1876,10 @@ __global__ __launch_bounds__(64) void incumbent_kernel(
   auto c_last_of = [&](int end_layer) {
     return prob.incumbent_ckpt_rule == 0 ? min(l, L - end_layer) : l;
   };
+  __shared__ double wave_sum[kIncumbentWaves], wave_largest[kIncumbentWaves];
+  const int wave = threadIdx.x >> 6;
   double sum = 0.0, largest = 0.0;
-  for (int s = 0; s < S; ++s) {
+  for (int s = wave; s < S; s += kIncumbentWaves) {
     const int p = S - 1 - s, end_layer = (s + 1) * l - 1;
     int slot;
     if (S == 1) slot = 2 * MIST_P_TILE + 1;
@@ -1887,7 +1890,7 @@ __global__ __launch_bounds__(64) void incumbent_kernel(
     double cost;
     if (prob.incumbent_ckpt_rule == 2) {  // every layer of the stage checkpointed
       cost = INFINITY;
-      if (threadIdx.x == 0) {
+      if ((threadIdx.x & 63) == 0) {
         const int pair = l * (l + 1) / 2 - 1 + l;
         const int lc_tile = pair / MIST_LC_TILE - g->lc_tile_begin;
         if (lc_tile >= 0 && lc_tile < g->n_lc_tiles) {
@@ -1903,6 +1906,17 @@ __global__ __launch_bounds__(64) void incumbent_kernel(
     }
     sum += cost;
     largest = fmax(largest, cost);
+  }
+  if ((threadIdx.x & 63) == 0) {
+    wave_sum[wave] = sum;
+    wave_largest[wave] = largest;
+  }
+  __syncthreads();
+  sum = 0.0;
+  largest = 0.0;
+  for (int w = 0; w < kIncumbentWaves; ++w) {
+    sum += wave_sum[w];
+    largest = fmax(largest, wave_largest[w]);
   }
   const double total = sum + (double)(g->grad_accum - 1) * largest;
   // costs are not negative, and non-negative doubles order like their bit patterns
@@ -2317,7 +2331,8 @@ static int launch_scout(const MistProblem *problem, const MistGroupDesc *d_group
     MIST_HIP_CHECK(hipGetLastError());
   }
   if (problem->stage_cost_incumbent != nullptr && n_samples == 1) {
-    hipLaunchKernelGGL(incumbent_kernel, dim3(n_groups), dim3(64), 0, (hipStream_t)stream, *problem,
+    hipLaunchKernelGGL(incumbent_kernel, dim3(n_groups), dim3(64 * kIncumbentWaves), 0,
+                       (hipStream_t)stream, *problem,
                        d_groups, scout_prefix, scout_base, d_partial_cost, d_partial_index);
     MIST_HIP_CHECK(hipGetLastError());
   }

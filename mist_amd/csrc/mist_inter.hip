@@ -18,7 +18,8 @@
 // mist_dp_window_begin, and a window it cannot decide sends the search down the host route).
 // How far a window is fetched or how many thresholds a batch speculates on
 // only changes the work done, never the outcome: the replay consumes DP results in the
-// reference's order with its stop rule and its strict "<".
+// reference's order with its stop rule and its strict "<", and passes without a DP run only
+// the thresholds at which the reference's run provably changes nothing (struct Scan).
 #include <hip/hip_runtime.h>
 
 #include <algorithm>

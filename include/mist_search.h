@@ -99,7 +99,8 @@ typedef struct MistProblem {
    * double in device memory, an estimate of the cost of the best pipeline the caller's
    * inter-stage search returns (+inf before the first call).  The scout pass lowers it to the
    * cost of the best partition into equal stages on equal meshes that its seeds allow; the main
-   * launch then does not look for stage costs above
+   * launch (and the scout pass itself, with the value it finds) then does not look for stage
+   * costs above
    *     bound(G) = incumbent / G * (1 + mist_incumbent_slack()).
    * A cell whose minimum is not above bound(G) holds its minimum and row as always; any other
    * cell holds some value above it (a seed, or +inf / -1), not necessarily its minimum.
@@ -113,6 +114,13 @@ typedef struct MistProblem {
   int32_t incumbent_ckpt_rule;   /* ckpt counts the search admits for a stage that ends at layer
                                   * i with l layers: 0 = 0..min(l, L - i) (inter_tuning.py:315),
                                   * 1 = 0..l, 2 = l only (inter_tuning_uniform_device.py:400-404) */
+  int32_t incumbent_first_estimate; /* != 0: before its scout pass the call forms a first estimate
+                                  * of the same pipeline cost from about a thousand rows per
+                                  * group, and the scout pass, too, leaves out stage costs above
+                                  * bound(G) of the estimate it finds in place.  For the first call
+                                  * after the incumbent was set to +inf; later calls of the same
+                                  * search (further groups) read what the earlier ones left. */
+  int32_t reserved0;
 } MistProblem;
 
 /* One (gradient-accumulation steps, device mesh) group = one call of the reference's

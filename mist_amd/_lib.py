@@ -64,6 +64,8 @@ PROBLEM_DTYPE = np.dtype(
         ("stage_cost_incumbent", "<u8"),
         ("incumbent_num_devices", "<i4"),
         ("incumbent_ckpt_rule", "<i4"),
+        ("incumbent_first_estimate", "<i4"),
+        ("reserved0", "<i4"),
     ],
     align=True,
 )

@@ -1099,8 +1099,9 @@ __device__ __forceinline__ void reduce_block(
   const double inv_G64 = 1.0 / G64;
   const float inv_G32 = 1.0f / G32;
   // Stage costs the caller's search can use at all (MistProblem.stage_cost_incumbent): rows above
-  // it are not looked for.  (The scout pass, whose seeds the incumbent comes from, has none.)
-  const double cutoff = range.gathered != 0 || prob.stage_cost_incumbent == nullptr || prob.sample_size != 1
+  // it are not looked for.  (The scout pass reads the first estimate, which a few rows gave
+  // before it; the main launch reads the one the scout's seeds gave.)
+  const double cutoff = prob.stage_cost_incumbent == nullptr || prob.sample_size != 1
                             ? (double)INFINITY
                             : *prob.stage_cost_incumbent * inv_G64 * (1.0 + kIncumbentSlack);
   const double pre_saved = g->pre_saved, pre_sas = g->pre_states_and_saved;
@@ -1830,6 +1831,21 @@ __global__ __launch_bounds__(MIST_LC_TILE, MIST_EXHAUSTIVE_MIN_WAVES) void eval_
                             lds_terms, lds_row, partial_cost + block * slab, partial_index + block * slab);
 }
 
+// The equal-stage pipeline a group offers to the stage-cost estimates: S stages of L / S layers
+// on the group's mesh, or 0 when the devices or the layers do not divide, the group has too few
+// pre-saved micro-batch values, or the caller's search does not go that deep.
+__device__ __forceinline__ int incumbent_stage_count(const MistProblem &prob,
+                                                     const MistGroupDesc *__restrict__ g) {
+  const int L = prob.num_layers, D = prob.incumbent_num_devices;
+  const int nm = g->num_nodes * g->num_gpus_per_node;
+  if (nm <= 0 || D % nm != 0) return 0;
+  const int S = D / nm;
+  if (S < 1 || S > L || L % S != 0 || S - 1 >= g->num_p) return 0;
+  // (the per-mesh search goes up to min(devices, layers) / 2 stages, inter_tuning.py:279-281)
+  if (prob.incumbent_ckpt_rule == 0 && S > (D < L ? D : L) / 2) return 0;
+  return S;
+}
+
 // Cost of the best pipeline of equal stages on equal meshes that the scout pass's seeds allow
 // (sample 0 of a call with one sample, whose objective is the stage cost): group (G, mesh (n, m))
 // offers S = devices / (n m) stages of L / S layers each, the first one from the with_pre table
@@ -1849,13 +1865,9 @@ __global__ __launch_bounds__(64 * kIncumbentWaves) void incumbent_kernel(
     const double *__restrict__ partial_cost, const int32_t *__restrict__ partial_index) {
   const MistGroupDesc *g = groups + blockIdx.x;
   if (g->scout_stride <= 0) return;
-  const int L = prob.num_layers, D = prob.incumbent_num_devices;
-  const int nm = g->num_nodes * g->num_gpus_per_node;
-  if (nm <= 0 || D % nm != 0) return;
-  const int S = D / nm;
-  if (S < 1 || S > L || L % S != 0 || S - 1 >= g->num_p) return;
-  // (the per-mesh search goes up to min(devices, layers) / 2 stages, inter_tuning.py:279-281)
-  if (prob.incumbent_ckpt_rule == 0 && S > (D < L ? D : L) / 2) return;
+  const int L = prob.num_layers;
+  const int S = incumbent_stage_count(prob, g);
+  if (S == 0) return;
   const int l = L / S;
   const int64_t slab = (int64_t)kSlots * MIST_LC_TILE;
   // cheapest seed of the stage's (l, c) cells, c = 0..c_last, in slot `slot` of p tile `p_tile`
@@ -1920,6 +1932,131 @@ __global__ __launch_bounds__(64 * kIncumbentWaves) void incumbent_kernel(
   }
   const double total = sum + (double)(g->grad_accum - 1) * largest;
   // costs are not negative, and non-negative doubles order like their bit patterns
+  if (threadIdx.x == 0 && total >= 0.0 && total < INFINITY)
+    atomicMin(reinterpret_cast<unsigned long long *>(prob.stage_cost_incumbent),
+              (unsigned long long)__double_as_longlong(total));
+}
+
+// First estimate of the same pipeline cost, formed before the scout pass so that the scout pass
+// can already leave out stage costs the caller's search cannot use.  Each group evaluates about
+// kEstimateRows of its gathered rows - every parallelism row of every scout pair without
+// activation / optimizer offloading first, then with the next ratios - for the layer count
+// l = L / S and every ckpt count, exactly as the tables would (same latency and memory code as
+// the evaluate-every-cell kernel, same cells kept: c == l - 1 only at p == 0 of the base /
+// with_pre tables), and keeps per stage of the pipeline the cheapest feasible cost.  Minima over
+// fewer rows than the scout pass sees, so the estimate is no smaller than the scout's.
+// Grid (kEstimateSplit, group); workgroup k writes its S minima to doubles [k S, (k + 1) S) of
+// the group's first scout slab (free until the scout pass writes it).
+constexpr int kEstimateSplit = 16;
+constexpr int kEstimateRows = 1024;
+constexpr int kEstimateMaxStages = 256;
+static_assert(kEstimateSplit * kEstimateMaxStages <= kScoutSplit * kSlots * MIST_LC_TILE,
+              "the partial minima of a group fit the scout slabs of one tile");
+__device__ __forceinline__ bool estimate_runs(const MistProblem &prob, const MistGroupDesc *g,
+                                              const int32_t *__restrict__ scout_prefix, int gi,
+                                              int *stages) {
+  if (g->scout_stride <= 0 || scout_prefix[gi + 1] - scout_prefix[gi] < kScoutSplit) return false;
+  *stages = incumbent_stage_count(prob, g);
+  return *stages > 0 && *stages <= kEstimateMaxStages;
+}
+
+__global__ __launch_bounds__(256) void estimate_stage_minima_kernel(
+    const MistProblem prob, const MistGroupDesc *__restrict__ groups,
+    const int32_t *__restrict__ scout_prefix, int64_t scout_base,
+    const double *__restrict__ row_terms, double ratio, double *__restrict__ partial_cost) {
+  const int gi = (int)blockIdx.y;
+  const MistGroupDesc *g = groups + gi;
+  int S;
+  if (!estimate_runs(prob, g, scout_prefix, gi, &S)) return;
+  const int L = prob.num_layers, l = L / S, rule = prob.incumbent_ckpt_rule;
+  __shared__ unsigned long long stage_min[kEstimateMaxStages];
+  const unsigned long long kInf = (unsigned long long)__double_as_longlong((double)INFINITY);
+  for (int st = threadIdx.x; st < S; st += blockDim.x) stage_min[st] = kInf;
+  __syncthreads();
+  const int n_tail = g->n_oo * g->n_ao;
+  const int64_t per_pair = (int64_t)g->n_par * n_tail;
+  const int64_t per_tail = (int64_t)g->n_par * max(g->scout_stride, 1);
+  const int64_t n_tails = min((int64_t)n_tail, max((int64_t)1, (int64_t)kEstimateRows / per_tail));
+  const int64_t n_items = per_tail * n_tails * (l + 1);
+  const GroupConsts k = group_consts(g);
+  const double cap = prob.mem_cap_mb;
+  const double G64 = (double)g->grad_accum;
+  const float G32 = (float)g->grad_accum;
+  const double *__restrict__ src = row_terms + g->row_offset * MIST_ROW_TERMS;
+  auto offer = [&](int st, bool ok, double cost) {
+    // costs are not negative, and non-negative doubles order like their bit patterns
+    if (ok && cost >= 0.0 && cost < INFINITY)
+      atomicMin(&stage_min[st], (unsigned long long)__double_as_longlong(cost));
+  };
+  for (int64_t item = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; item < n_items;
+       item += (int64_t)gridDim.x * blockDim.x) {
+    const int c = (int)(item % (l + 1));
+    const int64_t q = item / (l + 1);
+    const int64_t tail = q / per_tail, rest = q - tail * per_tail;
+    const int64_t pair = rest / g->n_par, par = rest - pair * g->n_par;
+    if (rule == 2 && c != l) continue;  // every layer of a stage checkpointed
+    if (c == l - 1) continue;  // kept at p == 0 of base / with_pre only, which no stage below reads
+    const double *__restrict__ t =
+        src + gathered_position(g, pair * per_pair + par * n_tail + tail) * MIST_ROW_TERMS;
+    const CellLatency lat = cell_latency<true>(t, l, c, k);
+    const LaneMemory mem = cell_memory(t, l, c);
+    // largest ckpt count of the stage that ends with layer end_layer (rule of the caller's search)
+    auto c_last = [&](int st) { return rule == 0 ? min(l, L - ((st + 1) * l - 1)) : l; };
+    double peak_f, peak_b;
+    mem.peaks(0, peak_f, peak_b);
+    const double f_in = mem.fwd_states + g->post_states + mem.mod_saved + g->post_fwd_peak + mem.gcb;
+    const double b_in = mem.bwd_states + g->post_states + mem.mod_saved + g->post_bwd_peak +
+                        (c == 0 ? t[MIST_T_RD] : 0.0) + mem.gcb;
+    const double pf_post = fmax(f_in, peak_f + g->post_states);
+    const double pb_post = fmax(b_in, peak_b - mem.out + g->post_states) + g->post_output;
+    if (S == 1) {  // single stage: the no_pp table
+      const double pf_pp = pf_post + g->pre_states + g->pre_saved;
+      const double pb_pp = pb_post + g->pre_states + g->pre_saved;
+      offer(0, c <= c_last(0) && fmax(pf_pp, pb_pp) * t[MIST_T_MF] <= cap,
+            ratio * lat.spp + lat.dpp / G64);
+      continue;
+    }
+    // first stage: with_pre table at S - 1 pre-saved micro-batches
+    offer(0, c <= c_last(0) && mem.feasible_pre(S - 1, cap, g->pre_saved, g->pre_states_and_saved),
+          ratio * lat.sp + lat.dpre / G64);
+    // last stage: with_post table
+    offer(S - 1, c <= c_last(S - 1) && fmax(pf_post, pb_post) * mem.mf_pp <= cap,
+          ratio * lat.spost + lat.dpost / G64);
+    // stages between: base table at S - 1 - st pre-saved micro-batches
+    const double cost_base = ratio * (double)lat.x + (double)(lat.d / G32);
+    for (int st = 1; st < S - 1; ++st)
+      offer(st, c <= c_last(st) && mem.feasible_base(S - 1 - st, cap), cost_base);
+  }
+  __syncthreads();
+  const int64_t slab = (int64_t)kSlots * MIST_LC_TILE;
+  double *out = partial_cost + (scout_base + scout_prefix[gi]) * slab + (int64_t)blockIdx.x * S;
+  for (int st = threadIdx.x; st < S; st += blockDim.x)
+    out[st] = __longlong_as_double((long long)stage_min[st]);
+}
+
+// Sum of a group's stage minima + (G - 1) x the largest (inter_tuning.py:342) into *incumbent.
+__global__ __launch_bounds__(64) void estimate_combine_kernel(
+    const MistProblem prob, const MistGroupDesc *__restrict__ groups,
+    const int32_t *__restrict__ scout_prefix, int64_t scout_base,
+    const double *__restrict__ partial_cost) {
+  const int gi = (int)blockIdx.x;
+  const MistGroupDesc *g = groups + gi;
+  int S;
+  if (!estimate_runs(prob, g, scout_prefix, gi, &S)) return;
+  const int64_t slab = (int64_t)kSlots * MIST_LC_TILE;
+  const double *in = partial_cost + (scout_base + scout_prefix[gi]) * slab;
+  double sum = 0.0, largest = 0.0;
+  for (int st = threadIdx.x; st < S; st += 64) {
+    double best = INFINITY;
+    for (int k = 0; k < kEstimateSplit; ++k) best = fmin(best, in[(int64_t)k * S + st]);
+    sum += best;
+    largest = fmax(largest, best);
+  }
+  for (int step = 32; step > 0; step >>= 1) {
+    sum += __shfl_xor(sum, step);
+    largest = fmax(largest, __shfl_xor(largest, step));
+  }
+  const double total = sum + (double)(g->grad_accum - 1) * largest;
   if (threadIdx.x == 0 && total >= 0.0 && total < INFINITY)
     atomicMin(reinterpret_cast<unsigned long long *>(prob.stage_cost_incumbent),
               (unsigned long long)__double_as_longlong(total));
@@ -2319,6 +2456,17 @@ static int launch_scout(const MistProblem *problem, const MistGroupDesc *d_group
   if (n_scout_blocks % kScoutSplit != 0)
     return fail(MIST_E_INVALID, "n_scout_blocks %d is not a multiple of the scout split %d",
                 n_scout_blocks, kScoutSplit);
+  if (problem->stage_cost_incumbent != nullptr && problem->incumbent_first_estimate != 0 &&
+      n_samples == 1 && n_groups <= 65535) {
+    // a first estimate from a few rows, so that the scout pass itself runs under a bound
+    hipLaunchKernelGGL(estimate_stage_minima_kernel, dim3(kEstimateSplit, n_groups), dim3(256), 0,
+                       (hipStream_t)stream, *problem, d_groups, scout_prefix, scout_base,
+                       d_row_terms, ratios.r[0], d_partial_cost);
+    MIST_HIP_CHECK(hipGetLastError());
+    hipLaunchKernelGGL(estimate_combine_kernel, dim3(n_groups), dim3(64), 0, (hipStream_t)stream,
+                       *problem, d_groups, scout_prefix, scout_base, d_partial_cost);
+    MIST_HIP_CHECK(hipGetLastError());
+  }
   hipLaunchKernelGGL(eval_reduce_kernel, dim3(xcd_padded_grid(n_scout_blocks), n_samples),
                      dim3(MIST_LC_TILE), 0, (hipStream_t)stream, *problem, d_groups, n_groups,
                      d_block_prefix, n_blocks, scout_prefix, 1, d_row_terms, d_stage_floor, ratios,

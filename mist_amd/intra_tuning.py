@@ -756,6 +756,9 @@ class IntraStageTuner:
             # workspace is reused in stream order)
             stream = ctypes.c_void_p(streams[bi % len(streams)].cuda_stream)
             w = dev_plan["workspaces"][bi % len(dev_plan["workspaces"])]
+            # (the structure is read when a call is made: only the first batch of a search forms
+            # a first estimate, the others find the estimates of the batches before them)
+            plan["problem"]["incumbent_first_estimate"] = 1 if bi == 0 else 0
 
             def reduce_call(slot):
                 if self.exhaustive:

@@ -248,6 +248,22 @@ int mist_eval_reduce(const MistProblem *problem, const MistGroupDesc *d_groups, 
                      const double *d_row_terms, const double *d_stage_floor, double ratio,
                      double *d_partial_cost, int32_t *d_partial_index, void *stream);
 
+/* First estimate of MistProblem.stage_cost_incumbent, the step mist_eval_reduce takes before its
+ * scout pass when problem->incumbent_first_estimate is set: for every group with a scout pass
+ * whose mesh divides the cluster into S equal stages of L / S layers, about a thousand of its
+ * scout rows (every parallelism row of every scout pair, activation / optimizer ratios from the
+ * first on) are evaluated at that layer count for every ckpt count the caller's search admits
+ * (same cells, latencies and memory tests as the tables: batched_module_analyzer.py:2165-2216,
+ * 2755-2834, 2866-2923, 2946-3106), the cheapest feasible cost of each stage is kept, and
+ * sum + (G - 1) * largest (inter_tuning.py:342) lowers *stage_cost_incumbent.  Needs the row terms
+ * of the scout rows (mist_row_terms).  Scratch: the first 4096 doubles of each such group's scout
+ * slabs, d_partial_cost + (n_blocks + d_scout_prefix[group]) slabs, which a later scout pass
+ * overwrites. */
+int mist_stage_cost_first_estimate(const MistProblem *problem, const MistGroupDesc *d_groups,
+                                   int n_groups, const int32_t *d_scout_prefix, int n_blocks,
+                                   const double *d_row_terms, double ratio, double *d_partial_cost,
+                                   void *stream);
+
 /* mist_eval_reduce + mist_finalize for n_samples <= MIST_MAX_SAMPLE_BATCH ratios of the same
  * row terms (reference: the S samples of one compute_indices call, mist/utils/pareto.py:124-144):
  * the scout passes of all samples run as ONE launch (a single one fills a tenth of the GPU), then

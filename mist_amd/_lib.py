@@ -134,6 +134,10 @@ _SIGNATURES = {
         [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, _VP, ctypes.c_double,
          _VP, _VP, _VP],
     ),
+    "mist_stage_cost_first_estimate": (
+        ctypes.c_int,
+        [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, ctypes.c_double, _VP, _VP],
+    ),
     "mist_eval_reduce_samples": (
         ctypes.c_int,
         [_VP, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, ctypes.c_int, _VP, _VP, _VP, _VP,

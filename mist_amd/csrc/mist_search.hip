@@ -2447,6 +2447,20 @@ int64_t mist_stage_floor_doubles(int64_t total_rows, int n_groups) {
   return (total_rows / kStageRows + n_groups + 1) * kStageFloorPitch;
 }
 
+static int launch_first_estimate(const MistProblem *problem, const MistGroupDesc *d_groups,
+                                 int n_groups, const int32_t *scout_prefix, int64_t scout_base,
+                                 const double *d_row_terms, double ratio, double *d_partial_cost,
+                                 void *stream) {
+  hipLaunchKernelGGL(estimate_stage_minima_kernel, dim3(kEstimateSplit, n_groups), dim3(256), 0,
+                     (hipStream_t)stream, *problem, d_groups, scout_prefix, scout_base, d_row_terms,
+                     ratio, d_partial_cost);
+  MIST_HIP_CHECK(hipGetLastError());
+  hipLaunchKernelGGL(estimate_combine_kernel, dim3(n_groups), dim3(64), 0, (hipStream_t)stream,
+                     *problem, d_groups, scout_prefix, scout_base, d_partial_cost);
+  MIST_HIP_CHECK(hipGetLastError());
+  return 0;
+}
+
 // Scout launch + slab merge for n_samples ratios at once (grid.y = sample).
 static int launch_scout(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,
                         const int32_t *d_block_prefix, int n_blocks, const int32_t *scout_prefix,
@@ -2457,16 +2471,11 @@ static int launch_scout(const MistProblem *problem, const MistGroupDesc *d_group
     return fail(MIST_E_INVALID, "n_scout_blocks %d is not a multiple of the scout split %d",
                 n_scout_blocks, kScoutSplit);
   if (problem->stage_cost_incumbent != nullptr && problem->incumbent_first_estimate != 0 &&
-      n_samples == 1 && n_groups <= 65535) {
+      n_samples == 1 && n_groups <= 65535)
     // a first estimate from a few rows, so that the scout pass itself runs under a bound
-    hipLaunchKernelGGL(estimate_stage_minima_kernel, dim3(kEstimateSplit, n_groups), dim3(256), 0,
-                       (hipStream_t)stream, *problem, d_groups, scout_prefix, scout_base,
-                       d_row_terms, ratios.r[0], d_partial_cost);
-    MIST_HIP_CHECK(hipGetLastError());
-    hipLaunchKernelGGL(estimate_combine_kernel, dim3(n_groups), dim3(64), 0, (hipStream_t)stream,
-                       *problem, d_groups, scout_prefix, scout_base, d_partial_cost);
-    MIST_HIP_CHECK(hipGetLastError());
-  }
+    if (int rc = launch_first_estimate(problem, d_groups, n_groups, scout_prefix, scout_base,
+                                       d_row_terms, ratios.r[0], d_partial_cost, stream))
+      return rc;
   hipLaunchKernelGGL(eval_reduce_kernel, dim3(xcd_padded_grid(n_scout_blocks), n_samples),
                      dim3(MIST_LC_TILE), 0, (hipStream_t)stream, *problem, d_groups, n_groups,
                      d_block_prefix, n_blocks, scout_prefix, 1, d_row_terms, d_stage_floor, ratios,
@@ -2526,6 +2535,22 @@ int mist_eval_reduce(const MistProblem *problem, const MistGroupDesc *d_groups, 
                      d_partial_cost, d_partial_index);
   MIST_HIP_CHECK(hipGetLastError());
   return 0;
+}
+
+int mist_stage_cost_first_estimate(const MistProblem *problem, const MistGroupDesc *d_groups,
+                                   int n_groups, const int32_t *d_scout_prefix, int n_blocks,
+                                   const double *d_row_terms, double ratio, double *d_partial_cost,
+                                   void *stream) {
+  if (int rc = check_common(problem, d_groups, n_groups)) return rc;
+  if (!d_scout_prefix || !d_row_terms || !d_partial_cost)
+    return fail(MIST_E_INVALID, "null workspace pointer");
+  if (n_blocks < 0) return fail(MIST_E_INVALID, "n_blocks must not be negative, got %d", n_blocks);
+  if (problem->stage_cost_incumbent == nullptr)
+    return fail(MIST_E_INVALID, "no stage-cost incumbent to lower");
+  if (n_groups > 65535) return fail(MIST_E_INVALID, "at most 65535 groups per call, got %d", n_groups);
+  if (!(ratio >= 0.0)) return fail(MIST_E_INVALID, "ratio must be non-negative");
+  return launch_first_estimate(problem, d_groups, n_groups, d_scout_prefix, (int64_t)n_blocks,
+                               d_row_terms, ratio, d_partial_cost, stream);
 }
 
 static int launch_finalize(const MistProblem *problem, const MistGroupDesc *d_groups, int n_groups,

@@ -221,6 +221,89 @@ def test_tables_under_a_stage_cost_estimate(plan, rule):
     assert n_open > 1000 and n_closed > 1000  # the estimate closes cells, and leaves many open
 
 
+def _best_equal_stage_pipeline(full, Gs, meshes, L, D, rule):
+    """Cheapest pipeline of S = D / (n m) equal stages on one mesh that the finished tables hold
+    (first stage from with_pre at S - 1 pre-saved micro-batches, last from with_post, those
+    between from base, a single one from no_pp; ckpt counts by the search's rule), as
+    sum + (G - 1) x largest stage cost."""
+    import torch
+
+    def costs(v, G):
+        c = full.stable[v] + (full.delta[v].float() / G.float()).double() if v == 0 else full.stable[v] + full.delta[v] / G
+        return torch.where(full.index[v] >= 0, c, torch.full_like(c, float("inf")))[..., 0]
+
+    G = torch.tensor(Gs, dtype=torch.float64, device=full.stable[0].device)
+    base, pre, post, nopp = (costs(v, G.view([-1] + [1] * (full.stable[v].dim() - 1))) for v in range(4))
+    best = float("inf")
+    for q, (n, m) in enumerate(meshes):
+        if D % (n * m):
+            continue
+        S = D // (n * m)
+        if S > L or L % S or S - 1 >= base.shape[2] or (rule == 0 and S > min(D, L) // 2):
+            continue
+        l = L // S
+
+        def cheapest(cells, s):  # cells: [g, c]
+            c_last = min(l, L - ((s + 1) * l - 1)) if rule == 0 else l
+            return (cells[:, l:l + 1] if rule == 2 else cells[:, :c_last + 1]).min(dim=1).values
+
+        if S == 1:
+            stages = [cheapest(nopp[:, q], 0)]
+        else:
+            stages = [cheapest(pre[:, q, S - 1, l - 1], 0)]
+            stages += [cheapest(base[:, q, S - 1 - s, l - 1], s) for s in range(1, S - 1)]
+            stages += [cheapest(post[:, q, l - 1], S - 1)]
+        stages = torch.stack(stages)
+        largest = stages.max(dim=0).values
+        usable = torch.isfinite(largest)  # (G = 1: 0 x inf)
+        if bool(usable.any()):
+            total = stages.sum(dim=0)[usable] + (G[usable] - 1.0) * largest[usable]
+            best = min(best, float(total.min()))
+    return best
+
+
+@pytest.mark.parametrize("plan, rule", [(2, 0), (3, 0), (5, 0), (2, 1), (3, 2)])
+def test_first_stage_cost_estimate_is_a_pipeline_the_tables_hold(plan, rule):
+    """``mist_stage_cost_first_estimate`` alone: what it leaves in the incumbent is the cost of an
+    equal-stage pipeline made of real rows, so it is no smaller than the best such pipeline of
+    the finished tables (and than the estimate the scout pass's seeds give afterwards), and on the
+    benchmark plans it is close enough to it to bound the scout pass."""
+    import torch
+
+    from mist_amd import _lib
+    from mist_amd.intra_tuning import _ptr, alpha_ratios
+    from mist_amd.tune_one_case import PreparedSearch
+
+    cfg, _ = load_plan(plan)
+    hw, L = cfg.hardware, cfg.model.num_hidden_layers
+    D = hw.num_nodes * hw.num_gpus_per_node
+    search = PreparedSearch(cfg)
+    tuner = search.tuner
+    full = tuner.run_prepared(search.plan, search.dev_plan)[0].batch
+    assert len(search.dev_plan["batches"]) == 1  # the workspace holds the row terms of every group
+    d, w = search.dev_plan["batches"][0], search.dev_plan["workspaces"][0]
+    first = torch.full((1,), float("inf"), dtype=torch.float64, device=full.stable[0].device)
+    problem = search.plan["problem"].copy()
+    problem["stage_cost_incumbent"] = first.data_ptr()
+    problem["incumbent_num_devices"] = D
+    problem["incumbent_ckpt_rule"] = rule
+    lib = _lib.load()
+    rc = lib.mist_stage_cost_first_estimate(
+        ctypes.c_void_p(problem.ctypes.data), _ptr(d["groups"]), d["n_groups"], _ptr(d["scout_prefix"]),
+        d["n_reduce_blocks"], _ptr(w["row_terms"]), float(alpha_ratios(1)[0]), _ptr(w["partial_cost"]),
+        ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    _lib.check(rc, "mist_stage_cost_first_estimate")
+    first = float(first.item())
+    tuner.run_prepared(search.plan, search.dev_plan, dict(num_devices=D, ckpt_rule=rule))
+    after_scout = float(search.dev_plan["incumbent"].item())
+    in_tables = _best_equal_stage_pipeline(full, search.Gs * len(tuner.tp_sizes),
+                                           tuner.device_mesh_candidates, L, D, rule)
+    print(f"plan {plan} rule {rule}: first {first!r} after the scout pass {after_scout!r} tables {in_tables!r}")
+    assert np.isfinite(first)
+    assert in_tables <= after_scout * (1 + 1e-12) and after_scout <= first
+    assert first <= in_tables * 1.1
+
+
 @pytest.mark.parametrize("waves, scout", [(1 << 22, 1), (1 << 22, 0), (1, 1)])
 def test_row_chunking_leaves_results_unchanged(monkeypatch, waves, scout):
     """Groups cut into the smallest row chunks (256 rows: many chunks per tile, most of which

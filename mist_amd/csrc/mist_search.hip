@@ -2721,13 +2721,8 @@ int mist_intra_stage_eval(const MistProblem *problem, const MistGroupDesc *d_gro
     MIST_HIP_CHECK(hipGetLastError());
     MIST_HIP_CHECK(hipEventRecord(os->rows_ready, main_stream));
     MIST_HIP_CHECK(hipStreamWaitEvent(os->side, os->rows_ready, 0));
-    RatioList ratios = {};
-    ratios.r[0] = ratio;
-    if (int rc = launch_scout(problem, d_groups, n_groups, d_reduce_block_prefix, n_reduce_blocks,
-                              d_scout_prefix, n_scout_blocks, d_row_terms, d_stage_floor, ratios, 1,
-                              n_reduce_blocks, d_partial_cost, d_partial_index, os->side))
-      return rc;
-    MIST_HIP_CHECK(hipEventRecord(os->scout_done, os->side));
+    // (the other row terms are queued first: the scout pass is five launches, and this stream
+    // would idle while they are made)
     bool from_keys = false;
     if (int rc = launch_key_terms(problem, d_groups, n_groups, d_key_terms, main_stream, &from_keys))
       return rc;
@@ -2740,6 +2735,13 @@ int mist_intra_stage_eval(const MistProblem *problem, const MistGroupDesc *d_gro
                          main_stream, *problem, d_groups, n_groups, d_terms_block_prefix, d_row_terms,
                          d_stage_floor, nullptr);
     MIST_HIP_CHECK(hipGetLastError());
+    RatioList ratios = {};
+    ratios.r[0] = ratio;
+    if (int rc = launch_scout(problem, d_groups, n_groups, d_reduce_block_prefix, n_reduce_blocks,
+                              d_scout_prefix, n_scout_blocks, d_row_terms, d_stage_floor, ratios, 1,
+                              n_reduce_blocks, d_partial_cost, d_partial_index, os->side))
+      return rc;
+    MIST_HIP_CHECK(hipEventRecord(os->scout_done, os->side));
     MIST_HIP_CHECK(hipStreamWaitEvent(main_stream, os->scout_done, 0));
     hipLaunchKernelGGL(eval_reduce_kernel, dim3(xcd_padded_grid(n_reduce_blocks)), dim3(MIST_LC_TILE),
                        0, main_stream, *problem, d_groups, n_groups, d_reduce_block_prefix,

@@ -448,7 +448,7 @@ def main():
             r["valu_busy_frac"] = counters["SQ_ACTIVE_INST_VALU"][which] * 4 / (1024 * 2.4e9 * sec)
         return r, executed
 
-    roofline, executed = roofline_of("eval_reduce_kernel (scout + main launch of one call)", "pruned",
+    roofline, executed = roofline_of("eval_reduce_kernel (first estimate, scout and main launch of one call)", "pruned",
                                      kernel_ms["eval_reduce"])
     # achieved = what the pruned kernel EXECUTES (it skips most cells exactly); the reference's
     # per-cell formulas over the same time are reported as pruning_gain (> 1 by design)

@@ -78,6 +78,38 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
                                      int32_t *out_stages, int32_t *out_path, int32_t *out_rows,
                                      int64_t *out_stats, void *stream);
 
+/* mist_inter_stage_search_families over tables that hold their values only up to a limit per G
+ * (the tables an intra-stage call with MistProblem.stage_cost_incumbent leaves: a cell whose
+ * minimum is not above estimate / G * (1 + mist_incumbent_slack()) holds it, any other cell
+ * holds something above).  No counterpart in the reference: it is the reference's scan
+ * (inter_tuning.py:163-217) made safe for such tables.
+ *   host_estimate : one double in (pinned) HOST memory that holds the estimate once the work
+ *                   queued on `stream` before this call has run (the search reads it after its
+ *                   first synchronisation); +inf = the tables are complete, plain search
+ *   limit_factor  : limit(G) = *host_estimate * limit_factor / G, at or below which every cell
+ *                   the DP reads holds its value ((1 + slack) shortened by a few float32 ulps)
+ *   out_unresolved: HOST.  The scan tries no threshold at or above limit(G), and one DP run per
+ *                   (instance, G) at limit(G) itself travels with its first batch of requests:
+ *                   the number of (instance, G) pairs for which that run finds a partition
+ *                   cheaper than the running best the scan of G ended with.  Zero, and a
+ *                   returned cost below estimate * limit_factor, means the result is what the
+ *                   scan over the complete tables returns: thresholds above limit(G) can then
+ *                   only produce partitions with a stage above limit(G), which cost more than
+ *                   estimate * limit_factor, or partitions the scan already has.  Otherwise the
+ *                   reference's scan may find such a partition at a threshold above limit(G)
+ *                   (its threshold candidates leave out single-stage costs and those its gap
+ *                   rule drops), which these tables cannot tell: evaluate again on complete
+ *                   tables. */
+int mist_inter_stage_search_bounded(int n_families, const MistDpShape *shapes,
+                                    const MistDpCosts *costs, const MistDpCosts *select_costs,
+                                    const MistStrategyIndex *strategy, int n_instances,
+                                    int n_grad_accum, const int32_t *rows,
+                                    const int32_t *grad_accum, int only_best_path, double *out_cost,
+                                    int32_t *out_g, float *out_tmax, int32_t *out_family,
+                                    int32_t *out_stages, int32_t *out_path, int32_t *out_rows,
+                                    int64_t *out_stats, void *stream, const double *host_estimate,
+                                    double limit_factor, int32_t *out_unresolved);
+
 #ifdef __cplusplus
 }
 #endif

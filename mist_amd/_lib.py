@@ -340,6 +340,11 @@ _INTER_SIGNATURES = {
         [ctypes.c_int, _VP, _VP, ctypes.POINTER(DpCosts), ctypes.POINTER(StrategyIndex),
          ctypes.c_int, ctypes.c_int, _VP, _VP, ctypes.c_int,
          _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP]),
+    "mist_inter_stage_search_bounded": (
+        ctypes.c_int,
+        [ctypes.c_int, _VP, _VP, ctypes.POINTER(DpCosts), ctypes.POINTER(StrategyIndex),
+         ctypes.c_int, ctypes.c_int, _VP, _VP, ctypes.c_int,
+         _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, ctypes.c_double, _VP]),
 }
 
 PLAN_MAX_LIST = 32

@@ -616,6 +616,9 @@ struct Scan {
   size_t first = 0;  // the first one at or above the smallest feasible threshold
   std::map<size_t, Outcome> known;  // DP outcomes by index of the kept threshold
   int limit = kFirstChunk;
+  // thresholds t with t * G >= cap are not tried (kInf: the reference's stop rule alone): the
+  // caller's tables hold their values only up to cap / G
+  double cap = kInf;
   size_t n_kept() const { return w ? w->kept.size() : 0; }
   // lower bound of the total of any improvement at thresholds pos..j, from the sum at j
   double floor_total(size_t at, double sum_later) const {
@@ -630,14 +633,16 @@ extern "C" {
 
 int mist_sizeof_strategy_index(void) { return (int)sizeof(MistStrategyIndex); }
 
-int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
-                                     const MistDpCosts *costs, const MistDpCosts *select_costs,
-                                     const MistStrategyIndex *strategy, int n_instances,
-                                     int n_grad_accum, const int32_t *rows,
-                                     const int32_t *grad_accum, int only_best_path, double *out_cost,
-                                     int32_t *out_g, float *out_tmax, int32_t *out_family,
-                                     int32_t *out_stages, int32_t *out_path, int32_t *out_rows,
-                                     int64_t *out_stats, void *stream_) {
+static int search_families(int n_families, const MistDpShape *shapes,
+                           const MistDpCosts *costs, const MistDpCosts *select_costs,
+                           const MistStrategyIndex *strategy, int n_instances,
+                           int n_grad_accum, const int32_t *rows,
+                           const int32_t *grad_accum, int only_best_path, double *out_cost,
+                           int32_t *out_g, float *out_tmax, int32_t *out_family,
+                           int32_t *out_stages, int32_t *out_path, int32_t *out_rows,
+                           int64_t *out_stats, void *stream_, const double *host_estimate,
+                           double limit_factor, int32_t *out_unresolved) {
+  if (out_unresolved) *out_unresolved = 0;
   if (!shapes || !costs || !select_costs || !rows || !grad_accum || !out_cost || !out_g ||
       !out_tmax || !out_family || !out_stages || !out_path)
     return fail(MIST_E_INVALID, "null pointer argument");
@@ -851,6 +856,18 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
     int best_g = -1, best_stages = 0;
     float best_t = 0.0f;
   };
+  // Exact part of the caller's tables (a search over tables that hold their values up to
+  // limit(G) = estimate * limit_factor / G only): the estimate has arrived with the first round
+  // trip (it was copied on this stream before the search was called).
+  std::vector<float> limit_t(n_grad_accum, std::numeric_limits<float>::infinity());
+  const bool bounded = host_estimate != nullptr && std::isfinite(*host_estimate);
+  if (bounded)
+    for (int i = 0; i < n_grad_accum; ++i)
+      limit_t[i] = (float)(*host_estimate * limit_factor / (double)grad_accum[i]);
+  // per (instance, G): the running best when the scan of G ended, and the cost of the best
+  // partition whose stages all lie within limit(G)
+  std::vector<double> best_after(bounded ? n_flat : 0, kInf), within_limit(bounded ? n_flat : 0, kInf);
+  bool within_limit_known = !bounded;
   std::vector<Chain> chains(n_instances);
   for (int t = 0; t < n_instances; ++t) {
     chains[t].scans.resize(n_grad_accum);
@@ -858,6 +875,7 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
       Scan &sc = chains[t].scans[i];
       Window &w = windows[t * n_grad_accum + i];
       sc.G = grad_accum[i];
+      if (bounded) sc.cap = (double)limit_t[i] * (double)grad_accum[i];
       sc.w = w.exists ? &w : nullptr;
       if (sc.w)
         sc.pos = (size_t)(std::lower_bound(w.kept.begin(), w.kept.end(), w.start_value) -
@@ -880,6 +898,7 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
   // makes sure threshold `pos` is materialised if the scan can get there
   auto reach = [&](Scan &sc, size_t pos, double best_cost) -> bool {
     Window *w = sc.w;
+    best_cost = std::min(best_cost, sc.cap);
     while (w && pos >= w->kept.size() && !w->covers(best_cost)) {
       if (int rc = S.extend(w, best_cost)) {
         rc_inner = rc;
@@ -893,7 +912,7 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
                     int &best_stages) -> bool {
     for (;;) {
       if (!reach(sc, sc.pos, best_cost)) return true;
-      if (sc.w->scaled[sc.pos] >= best_cost) return true;  // inter_tuning.py:196-197
+      if (sc.w->scaled[sc.pos] >= std::min(best_cost, sc.cap)) return true;  // inter_tuning.py:196-197
       const auto later = sc.known.lower_bound(sc.pos);
       if (later != sc.known.end() && sc.floor_total(sc.pos, later->second.sum) >= best_cost) {
         sc.pos = later->first + 1;  // nothing up to there improves the best
@@ -925,7 +944,7 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
     if (sc.known.empty()) {
       reach(sc, sc.pos + (size_t)kFirstChunk, best_cost);
       if (rc_inner) return;
-      const size_t stop = stop_of(best_cost);
+      const size_t stop = stop_of(std::min(best_cost, sc.cap));
       if (stop <= sc.pos) return;
       const int n_avail = (int)(stop - sc.pos), n = std::min(kFirstChunk, n_avail);
       for (int k = 0; k < n; ++k)
@@ -936,7 +955,7 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
     int budget = sc.limit;
     bool cut = false;
     while (reach(sc, pos, best_cost)) {
-      if (sc.w->scaled[pos] >= best_cost) break;
+      if (sc.w->scaled[pos] >= std::min(best_cost, sc.cap)) break;
       const auto later = sc.known.lower_bound(pos);
       if (later != sc.known.end() && sc.floor_total(pos, later->second.sum) >= best_cost) {
         pos = later->first + 1;
@@ -955,7 +974,7 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
       ++pos;
     }
     if (rc_inner || !cut) return;
-    const size_t stop = stop_of(best_cost);
+    const size_t stop = stop_of(std::min(best_cost, sc.cap));
     size_t last = 0;
     for (int k = 0; k < kProbes && stop > pos; ++k) {
       const size_t step = ((size_t)(k + 1) * (stop - pos)) / kProbes;
@@ -991,6 +1010,7 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
           ch.best_stages = best_stages;
         }
         if (!finished) break;
+        if (bounded) best_after[t * n_grad_accum + (int)ch.current] = ch.best_cost;
         ++ch.current;
       }
       if (ch.current < ch.scans.size()) all_done = false;
@@ -1010,10 +1030,27 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
         }
       }
     }
-    if (all_done) break;
-    if (spans.empty()) return fail(MIST_E_INVALID, "inter-stage scan made no progress");
+    if (all_done && within_limit_known) break;
+    if (spans.empty() && within_limit_known)
+      return fail(MIST_E_INVALID, "inter-stage scan made no progress");
+    // the DP at limit(G) of every (instance, G) with a window travels with the first batch
+    const int n_scan_requests = (int)req_t.size();
+    std::vector<int> limit_of;
+    if (!within_limit_known)
+      for (int i = 0; i < n_flat; ++i)
+        if (windows[i].exists) {
+          limit_of.push_back(i);
+          req_g.push_back(flat_rows[i]);
+          req_t.push_back(limit_t[i % n_grad_accum]);
+        }
+    if (req_t.empty()) break;  // (nothing feasible anywhere)
     if (int rc = S.run(req_g, req_t, MIST_DP_THRESHOLD, false)) return rc;
     const int n = (int)req_t.size();
+    for (size_t k = 0; k < limit_of.size(); ++k)
+      within_limit[limit_of[k]] = S.total(n_scan_requests + (int)k, n,
+                                          grad_accum[limit_of[k] % n_grad_accum], nullptr, nullptr,
+                                          nullptr, nullptr);
+    within_limit_known = true;
     for (const Span &sp : spans) {
       Scan &sc = chains[sp.t].scans[sp.i];
       for (int k = sp.first; k < sp.first + sp.n; ++k) {
@@ -1023,6 +1060,14 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
       }
     }
   }
+
+  // A partition inside the exact part of the tables that is cheaper than what the scan of its G
+  // ended with was admissible at no threshold the scan tried: the reference may or may not find
+  // it at a threshold above limit(G), which these tables cannot tell.  (One that costs
+  // estimate * limit_factor or more changes nothing the scan does below the limits.)
+  if (bounded && out_unresolved)
+    for (int i = 0; i < n_flat; ++i)
+      if (within_limit[i] < std::min(best_after[i], *host_estimate * limit_factor)) ++*out_unresolved;
 
   // ---- results and the partitions of the winners ----
   std::vector<int> winners;
@@ -1084,6 +1129,37 @@ int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
     out_stats[5] = S.left_to_host;
   }
   return 0;
+}
+
+int mist_inter_stage_search_families(int n_families, const MistDpShape *shapes,
+                                     const MistDpCosts *costs, const MistDpCosts *select_costs,
+                                     const MistStrategyIndex *strategy, int n_instances,
+                                     int n_grad_accum, const int32_t *rows,
+                                     const int32_t *grad_accum, int only_best_path, double *out_cost,
+                                     int32_t *out_g, float *out_tmax, int32_t *out_family,
+                                     int32_t *out_stages, int32_t *out_path, int32_t *out_rows,
+                                     int64_t *out_stats, void *stream) {
+  return search_families(n_families, shapes, costs, select_costs, strategy, n_instances,
+                         n_grad_accum, rows, grad_accum, only_best_path, out_cost, out_g, out_tmax,
+                         out_family, out_stages, out_path, out_rows, out_stats, stream, nullptr, 0.0,
+                         nullptr);
+}
+
+int mist_inter_stage_search_bounded(int n_families, const MistDpShape *shapes,
+                                    const MistDpCosts *costs, const MistDpCosts *select_costs,
+                                    const MistStrategyIndex *strategy, int n_instances,
+                                    int n_grad_accum, const int32_t *rows,
+                                    const int32_t *grad_accum, int only_best_path, double *out_cost,
+                                    int32_t *out_g, float *out_tmax, int32_t *out_family,
+                                    int32_t *out_stages, int32_t *out_path, int32_t *out_rows,
+                                    int64_t *out_stats, void *stream, const double *host_estimate,
+                                    double limit_factor, int32_t *out_unresolved) {
+  if (!host_estimate || !out_unresolved) return fail(MIST_E_INVALID, "null pointer argument");
+  if (!(limit_factor > 0.0)) return fail(MIST_E_INVALID, "limit_factor must be positive");
+  return search_families(n_families, shapes, costs, select_costs, strategy, n_instances,
+                         n_grad_accum, rows, grad_accum, only_best_path, out_cost, out_g, out_tmax,
+                         out_family, out_stages, out_path, out_rows, out_stats, stream,
+                         host_estimate, limit_factor, out_unresolved);
 }
 
 int mist_inter_stage_search(const MistDpShape *shape, const MistDpCosts *costs, int n_instances,

@@ -782,7 +782,7 @@ def _solutions(runner: _DpRunner, results_list, bests, n_g, g_index, q_index, nu
 
 
 def _native_search(runner: _DpRunner, results_list, rows, Gs, n_g, g_index, q_index, num_layers,
-                   slot, only_best, stats):
+                   slot, only_best, stats, table_limit=None):
     """The search of ``_search`` + the partitions and strategy rows of ``_solutions`` in one
     library call (``mist_inter_stage_search_families``: the same steps without the interpreter
     between the dependent GPU batches, for the per-mesh family or the uniform-device families
@@ -806,17 +806,28 @@ def _native_search(runner: _DpRunner, results_list, rows, Gs, n_g, g_index, q_in
     strategy_row = np.empty((n_inst, s_max), dtype=np.int32)
     counters = np.zeros(6, dtype=np.int64)
     t_0 = time.perf_counter()
+    arguments = [
+        len(fams), ctypes.c_void_p(shapes.ctypes.data), ctypes.cast(costs, ctypes.c_void_p),
+        ctypes.byref(select), ctypes.byref(runner.strategy_index), n_inst, len(Gs),
+        ctypes.c_void_p(rows.ctypes.data), ctypes.c_void_p(G_arr.ctypes.data),
+        1 if only_best else 0, ctypes.c_void_p(cost.ctypes.data),
+        ctypes.c_void_p(best_g.ctypes.data), ctypes.c_void_p(best_t.ctypes.data),
+        ctypes.c_void_p(family.ctypes.data), ctypes.c_void_p(n_stages.ctypes.data),
+        ctypes.c_void_p(path.ctypes.data), ctypes.c_void_p(strategy_row.ctypes.data),
+        ctypes.c_void_p(counters.ctypes.data), _stream(runner.device)]
+    unresolved = np.zeros(1, dtype=np.int32)
     with torch.cuda.device(runner.device):
-        rc = runner.lib.mist_inter_stage_search_families(
-            len(fams), ctypes.c_void_p(shapes.ctypes.data), ctypes.cast(costs, ctypes.c_void_p),
-            ctypes.byref(select), ctypes.byref(runner.strategy_index), n_inst, len(Gs),
-            ctypes.c_void_p(rows.ctypes.data), ctypes.c_void_p(G_arr.ctypes.data),
-            1 if only_best else 0, ctypes.c_void_p(cost.ctypes.data),
-            ctypes.c_void_p(best_g.ctypes.data), ctypes.c_void_p(best_t.ctypes.data),
-            ctypes.c_void_p(family.ctypes.data), ctypes.c_void_p(n_stages.ctypes.data),
-            ctypes.c_void_p(path.ctypes.data), ctypes.c_void_p(strategy_row.ctypes.data),
-            ctypes.c_void_p(counters.ctypes.data), _stream(runner.device))
+        if table_limit is None:
+            rc = runner.lib.mist_inter_stage_search_families(*arguments)
+        else:
+            # the tables hold their values up to estimate * factor / G only (``table_limit`` =
+            # the estimate as a pinned host tensor that the stream fills, and the factor)
+            rc = runner.lib.mist_inter_stage_search_bounded(
+                *arguments, ctypes.c_void_p(table_limit[0].data_ptr()), float(table_limit[1]),
+                ctypes.c_void_p(unresolved.ctypes.data))
     _lib.check(rc, "mist_inter_stage_search_families")
+    if stats is not None:
+        stats["dp_unresolved"] = stats.get("dp_unresolved", 0) + int(unresolved[0])
     t_1 = time.perf_counter()
     out = []
     for t in range(n_inst):
@@ -864,6 +875,7 @@ def inter_stage_tune_batch(
     stats: Optional[dict] = None,
     uniform_device: Optional[dict] = None,
     only_best_solution: bool = False,
+    table_limit=None,
 ):
     """``inter_stage_tune`` for several intra-stage results at once (the tensor-parallel
     candidates of one ``tune`` call).  Each entry is searched exactly as if it were alone (its
@@ -871,7 +883,13 @@ def inter_stage_tune_batch(
     ``(best_cost, best_solution)``.  ``uniform_device`` (``num_nodes``, ``num_gpus_per_node``,
     ``ckpt_tuning``) selects the recurrence of inter_tuning_uniform_device.py instead.
     ``only_best_solution``: a caller that keeps the best entry only (``tune``) gets the partition
-    and strategies of that entry; the other entries come back as ``(cost, None)``."""
+    and strategies of that entry; the other entries come back as ``(cost, None)``.
+    ``table_limit`` (pinned host tensor with an estimate, factor): the tables hold their values
+    up to ``estimate * factor / G`` only (``IntraStageTuner.run_prepared`` with a stage-cost
+    cutoff); the search then stays below that limit and ``stats['dp_unresolved']`` counts the
+    (entry, G) pairs whose result is not certain to be the reference's (library search only)."""
+    if table_limit is not None and not (NATIVE_SEARCH and _same_batch(results_list)):
+        raise ValueError("tables with a limit need the library's search over one batch of tables")
     for r in results_list:
         if not isinstance(r, IntraStageTunerOutput):
             raise TypeError(
@@ -903,7 +921,7 @@ def inter_stage_tune_batch(
     t_0 = time.perf_counter()
     if NATIVE_SEARCH:
         out = _native_search(runner, results_list, rows, Gs, n_g, g_index, q_index, num_layers, slot,
-                             only_best_solution, stats)
+                             only_best_solution, stats, table_limit)
         if stats is not None:
             stats["dp_setup_s"] = stats.get("dp_setup_s", 0.0) + (t_0 - t_start)
         return out

@@ -34,6 +34,7 @@ def inter_stage_tune_batch_uniform_device(
     slot: int = 0,
     stats: Optional[dict] = None,
     only_best_solution: bool = False,
+    table_limit=None,
 ):
     """All tensor-parallel candidates of one ``tune`` call in one batch of launches."""
     uniform = dict(
@@ -43,7 +44,7 @@ def inter_stage_tune_batch_uniform_device(
     return inter_stage_tune_batch(
         num_layers, num_nodes * num_gpus_per_node, device_mesh_candidates,
         gradient_accumulation_steps_candidates, results_list, slot, stats, uniform_device=uniform,
-        only_best_solution=only_best_solution,
+        only_best_solution=only_best_solution, table_limit=table_limit,
     )
 
 

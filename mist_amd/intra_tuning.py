@@ -758,7 +758,8 @@ class IntraStageTuner:
             w = dev_plan["workspaces"][bi % len(dev_plan["workspaces"])]
             # (the structure is read when a call is made: only the first batch of a search forms
             # a first estimate, the others find the estimates of the batches before them)
-            plan["problem"]["incumbent_first_estimate"] = 1 if bi == 0 else 0
+            plan["problem"]["incumbent_first_estimate"] = (
+                1 if bi == 0 and os.environ.get("MIST_NO_FIRST_ESTIMATE") is None else 0)
 
             def reduce_call(slot):
                 if self.exhaustive:

@@ -32,6 +32,7 @@ import torch
 import yaml
 
 from . import _lib
+from . import inter_tuning as _inter_tuning
 from .config import OFFLOADING_RATIO_CANDIDATES, MistConfig, tp_candidates
 from .inter_tuning import inter_stage_tune, inter_stage_tune_batch
 from .inter_tuning_uniform import inter_stage_tune as inter_stage_tune_uniform
@@ -211,7 +212,8 @@ class PreparedSearch:
         stats = {} if stats is None else stats
         hw = self.config.hardware
         t0 = time.perf_counter()
-        cutoff = self.stage_cost_cutoff
+        # (tables with a limit are searched by the library's driver only)
+        cutoff = self.stage_cost_cutoff if _inter_tuning.NATIVE_SEARCH else None
         results = self.tuner.run_prepared(self.plan, self.dev_plan, cutoff)
         if cutoff is not None:
             # the estimate the kernels ended with travels to the host behind them
@@ -224,15 +226,21 @@ class PreparedSearch:
         if split_timing:
             torch.cuda.synchronize(self.tuner.device)
         t1 = time.perf_counter()
+        # The tables hold their values up to estimate * limit_factor / G: the search stays below
+        # that and reports where this leaves its result uncertain.
+        limit_factor = (1.0 + _lib.load().mist_incumbent_slack()) * (1.0 - 1e-5)
+        table_limit = None if cutoff is None else (self._incumbent_host, limit_factor)
+        unresolved_before = stats.get("dp_unresolved", 0)
         if self.granularity == "inter-stage":
             outcomes = inter_stage_tune_batch(
                 self.L, hw.num_nodes * hw.num_gpus_per_node, self.meshes, self.Gs, results, slot=0, stats=stats,
                 only_best_solution=True,  # the loop below keeps the first best entry only
+                table_limit=table_limit,
             )
         elif self.granularity == "uniform-device-pp":
             outcomes = inter_stage_tune_batch_uniform_device(
                 self.L, hw.num_nodes, hw.num_gpus_per_node, self.meshes, self.Gs, results,
-                self.config, slot=0, stats=stats, only_best_solution=True,
+                self.config, slot=0, stats=stats, only_best_solution=True, table_limit=table_limit,
             )
         else:
             outcomes = [
@@ -250,8 +258,9 @@ class PreparedSearch:
             estimate = float(self._incumbent_host[0])
             # Below this cost the search has read nothing but cells that hold their minima
             # (MistProblem.stage_cost_incumbent); an infinite estimate left every cell exact.
-            safe_below = estimate * (1.0 + _lib.load().mist_incumbent_slack()) * (1.0 - 1e-5)
-            if np.isfinite(estimate) and not best_cost < safe_below:
+            safe_below = estimate * limit_factor
+            unresolved = stats.get("dp_unresolved", 0) - unresolved_before
+            if np.isfinite(estimate) and (unresolved > 0 or not best_cost < safe_below):
                 stats["stage_cost_cutoff_retries"] = stats.get("stage_cost_cutoff_retries", 0) + 1
                 self.stage_cost_cutoff = None
                 try:

@@ -104,11 +104,13 @@ typedef struct MistProblem {
    *     bound(G) = incumbent / G * (1 + mist_incumbent_slack()).
    * A cell whose minimum is not above bound(G) holds its minimum and row as always; any other
    * cell holds some value above it (a seed, or +inf / -1), not necessarily its minimum.
-   * A search that scans thresholds t with t * G < best (inter_tuning.py:196-197) and returns a
-   * cost below incumbent * (1 + slack) * (1 - 1e-5) has read the same values, in the same order,
-   * as from the full tables: every threshold that can lead to such a cost lies below bound(G),
-   * where the tables agree, and every partition with a stage above it costs more.  A caller
-   * whose search returns more than that evaluates again without the incumbent. */
+   * The reference's scan tries thresholds t with t * G < best (inter_tuning.py:196-197), so
+   * below limit(G) = incumbent * (1 + slack) * (1 - 1e-5) / G it reads the same values, in the
+   * same order, as from the full tables; what it does above that limit on the full tables these
+   * tables cannot tell.  mist_inter_stage_search_bounded (mist_inter.h) is the search for them:
+   * it stays below the limit and reports when that leaves the result uncertain, in which case
+   * (or when the result is not below incumbent * (1 + slack) * (1 - 1e-5)) the caller
+   * evaluates again without the incumbent. */
   double *stage_cost_incumbent;
   int32_t incumbent_num_devices; /* devices of the cluster: stages = this / (n * m of the group) */
   int32_t incumbent_ckpt_rule;   /* ckpt counts the search admits for a stage that ends at layer

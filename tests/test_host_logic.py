@@ -498,6 +498,7 @@ def test_library_loads_and_exports_every_declared_symbol():
 def test_argument_checks_reject_before_any_launch():
     """Host-side validation paths of the C ABI (no GPU needed: they return before launching)."""
     lib = _lib.load()
+    hp = lambda a: ctypes.c_void_p(a.ctypes.data)
     assert lib.mist_row_terms(None, None, 1, None, 1, None, None, None, None) == -1
     assert b"null" in lib.mist_last_error()
     prob = make_problem(load_plan(1)[0], 4, 2, 1, 4, 2)
@@ -573,6 +574,22 @@ def test_argument_checks_reject_before_any_launch():
     free["free_devices"], free["num_devices"], free["num_mesh"] = 1, 0, 1
     assert search(ctypes.c_void_p(free.ctypes.data), 1, 1, op) == -1
     assert b"per-mesh" in lib.mist_last_error()
+    # the search over tables with a limit needs the estimate, a factor and the counter
+    host_estimate, unresolved = np.full(1, np.inf), np.zeros(1, dtype=np.int32)
+    bounded = lambda est, factor, out: lib.mist_inter_stage_search_bounded(
+        1, so, ctypes.byref(costs), ctypes.byref(costs), None, 1, 1, op, op, 0, fake, fake, fake, fake,
+        fake, fake, None, None, None, est, factor, out)
+    assert bounded(None, 1.25, hp(unresolved)) == -1 and bounded(hp(host_estimate), 1.25, None) == -1
+    assert bounded(hp(host_estimate), 0.0, hp(unresolved)) == -1 and b"limit_factor" in lib.mist_last_error()
+    # the first stage-cost estimate: workspace pointers, an incumbent to lower, a ratio
+    estimate = lambda problem, prefix=fake, ratio=1.0: lib.mist_stage_cost_first_estimate(
+        problem, fake, 1, prefix, 4, fake, ratio, fake, None)
+    assert estimate(pp) == -1 and b"incumbent" in lib.mist_last_error()
+    with_incumbent = prob.copy()
+    with_incumbent["stage_cost_incumbent"], with_incumbent["incumbent_num_devices"] = 4096, 8
+    wp = ctypes.c_void_p(with_incumbent.ctypes.data)
+    assert estimate(wp, None) == -1 and estimate(wp, fake, -1.0) == -1 and b"ratio" in lib.mist_last_error()
+    assert estimate(None) == -1
     # re-laid row minima: max_stages * Q * L (L + 1) / 2 floats per g
     assert lib.mist_dp_stage_minima_floats(sp) == 4 * 2 * (80 * 81 // 2)
     assert lib.mist_dp_stage_minima_floats(ctypes.c_void_p(np.zeros(1, dtype=_lib.DP_SHAPE_DTYPE).ctypes.data)) == -1

@@ -1036,9 +1036,12 @@ static int search_families(int n_families, const MistDpShape *shapes,
     // the DP at limit(G) of every (instance, G) with a window travels with the first batch
     const int n_scan_requests = (int)req_t.size();
     std::vector<int> limit_of;
+    // (no partition of a pair costs less than G x its smallest feasible threshold: a pair for
+    // which that is not below estimate * limit_factor has nothing to report)
     if (!within_limit_known)
       for (int i = 0; i < n_flat; ++i)
-        if (windows[i].exists) {
+        if (windows[i].exists && (double)windows[i].start_value * (double)windows[i].G <
+                                     *host_estimate * limit_factor) {
           limit_of.push_back(i);
           req_g.push_back(flat_rows[i]);
           req_t.push_back(limit_t[i % n_grad_accum]);

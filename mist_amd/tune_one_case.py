@@ -180,8 +180,10 @@ class PreparedSearch:
         # The searches that scan thresholds below best / G (inter_tuning.py:196-197) never admit
         # a stage cost above that: the intra-stage kernels need not find the minima of such
         # cells (IntraStageTuner.run_prepared), given an estimate of the best cost.  ``run``
-        # checks the search's result against the estimate that was used and evaluates again
-        # without it if the result is not below.  ckpt counts a stage may use, as those
+        # searches such tables below the limit up to which they are exact
+        # (mist_inter_stage_search_bounded) and evaluates again without the estimate if that
+        # search reports a partition it may have missed or its result is not below the limit
+        # of the estimate that was used.  ckpt counts a stage may use, as those
         # searches restrict them: inter_tuning.py:315; inter_tuning_uniform_device.py:400-404.
         self.stage_cost_cutoff = None
         self._incumbent_host = self._incumbent_read = None

@@ -519,6 +519,9 @@ def main():
         "stage_cost_estimate": (float(search.dev_plan["incumbent"].item())
                                 if "incumbent" in search.dev_plan else None),
         "stage_cost_cutoff_retries": stats.get("stage_cost_cutoff_retries", 0),
+        # (tp, G) pairs of the timed steps whose partition inside the limit of the tables under
+        # the estimate the search could not rule out (each makes a step evaluate twice)
+        "dp_unresolved": stats.get("dp_unresolved", 0),
         "best_cost": cost,
         "best_solution": repr(solution),
         "roofline": roofline,
